@@ -1,0 +1,255 @@
+// C ABI: device shim, host index math and operator entry points.
+#include <hip/hip_runtime.h>
+
+#include <new>
+
+#include "core/fixed_dim.h"
+#include "device/ctx.h"
+
+using altius::DeviceCtx;
+using altius::FixedDimensions;
+
+struct ahip_ctx {
+    DeviceCtx d;
+};
+
+namespace {
+
+int global_fail(int code, const std::string &msg) {
+    altius::set_global_error(msg);
+    return code;
+}
+
+int global_check(hipError_t e, const char *what) {
+    if (e == hipSuccess) return AHIP_OK;
+    altius::set_global_error(std::string(what) + ": " + hipGetErrorString(e));
+    return e == hipErrorOutOfMemory ? AHIP_ERR_OOM : AHIP_ERR_HIP;
+}
+
+int create_ctx(int device, hipStream_t stream, bool own_stream, ahip_ctx **out) {
+    if (!out) return global_fail(AHIP_ERR_ARG, "ahip_init: null output pointer");
+    *out = nullptr;
+    int n = 0;
+    int rc = global_check(hipGetDeviceCount(&n), "hipGetDeviceCount");
+    if (rc) return rc;
+    if (device < 0 || device >= n) return global_fail(AHIP_ERR_ARG, "ahip_init: no such device");
+    rc = global_check(hipSetDevice(device), "hipSetDevice");
+    if (rc) return rc;
+    ahip_ctx *c = new (std::nothrow) ahip_ctx();
+    if (!c) return global_fail(AHIP_ERR_OOM, "ahip_init: out of host memory");
+    c->d.device = device;
+    if (own_stream) {
+        rc = global_check(hipStreamCreateWithFlags(&c->d.stream, hipStreamNonBlocking), "hipStreamCreate");
+        if (rc) {
+            delete c;
+            return rc;
+        }
+        c->d.owns_stream = true;
+    } else {
+        c->d.stream = stream;
+    }
+    void *scratch = nullptr;
+    rc = global_check(hipMalloc(&scratch, altius::SCRATCH_FLOATS * sizeof(float)), "hipMalloc(scratch)");
+    if (rc) {
+        if (c->d.owns_stream) (void)hipStreamDestroy(c->d.stream);
+        delete c;
+        return rc;
+    }
+    c->d.scratch = static_cast<float *>(scratch);
+    c->d.scratch_floats = altius::SCRATCH_FLOATS;
+    *out = c;
+    return AHIP_OK;
+}
+
+}  // namespace
+
+#define REQUIRE_CTX(ctx, name)                                                       \
+    do {                                                                             \
+        if (!(ctx)) return global_fail(AHIP_ERR_ARG, name ": null context");         \
+        if (hipSetDevice((ctx)->d.device) != hipSuccess)                             \
+            return (ctx)->d.fail(AHIP_ERR_HIP, name ": hipSetDevice failed");        \
+    } while (0)
+
+extern "C" {
+
+int ahip_init(int device, ahip_ctx **ctx) { return create_ctx(device, nullptr, true, ctx); }
+
+int ahip_init_on_stream(int device, void *hip_stream, ahip_ctx **ctx) {
+    return create_ctx(device, static_cast<hipStream_t>(hip_stream), false, ctx);
+}
+
+int ahip_destroy(ahip_ctx *ctx) {
+    if (!ctx) return AHIP_OK;
+    int rc = AHIP_OK;
+    if (hipSetDevice(ctx->d.device) == hipSuccess) {
+        (void)hipStreamSynchronize(ctx->d.stream);
+        if (ctx->d.scratch) rc = global_check(hipFree(ctx->d.scratch), "hipFree(scratch)");
+        if (ctx->d.owns_stream) (void)hipStreamDestroy(ctx->d.stream);
+    }
+    delete ctx;
+    return rc;
+}
+
+const char *ahip_last_error(ahip_ctx *ctx) { return ctx ? ctx->d.last_error.c_str() : altius::global_error(); }
+
+int ahip_device_count(void) {
+    int n = 0;
+    int rc = global_check(hipGetDeviceCount(&n), "hipGetDeviceCount");
+    return rc ? -rc : n;
+}
+
+int ahip_malloc(ahip_ctx *ctx, size_t bytes, void **dptr) {
+    REQUIRE_CTX(ctx, "ahip_malloc");
+    if (!dptr) return ctx->d.fail(AHIP_ERR_ARG, "ahip_malloc: null output pointer");
+    *dptr = nullptr;
+    if (bytes == 0) return AHIP_OK;
+    return ctx->d.check(hipMalloc(dptr, bytes), "hipMalloc");
+}
+
+int ahip_free(ahip_ctx *ctx, void *dptr) {
+    REQUIRE_CTX(ctx, "ahip_free");
+    if (!dptr) return AHIP_OK;
+    return ctx->d.check(hipFree(dptr), "hipFree");
+}
+
+int ahip_h2d_async(ahip_ctx *ctx, void *dst, const void *src, size_t bytes) {
+    REQUIRE_CTX(ctx, "ahip_h2d_async");
+    if (bytes == 0) return AHIP_OK;
+    if (!dst || !src) return ctx->d.fail(AHIP_ERR_ARG, "ahip_h2d_async: null pointer");
+    return ctx->d.check(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->d.stream), "hipMemcpyAsync(H2D)");
+}
+
+int ahip_d2h_async(ahip_ctx *ctx, void *dst, const void *src, size_t bytes) {
+    REQUIRE_CTX(ctx, "ahip_d2h_async");
+    if (bytes == 0) return AHIP_OK;
+    if (!dst || !src) return ctx->d.fail(AHIP_ERR_ARG, "ahip_d2h_async: null pointer");
+    return ctx->d.check(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->d.stream), "hipMemcpyAsync(D2H)");
+}
+
+int ahip_d2d_async(ahip_ctx *ctx, void *dst, const void *src, size_t bytes) {
+    REQUIRE_CTX(ctx, "ahip_d2d_async");
+    if (bytes == 0) return AHIP_OK;
+    if (!dst || !src) return ctx->d.fail(AHIP_ERR_ARG, "ahip_d2d_async: null pointer");
+    return ctx->d.check(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->d.stream), "hipMemcpyAsync(D2D)");
+}
+
+int ahip_memset_async(ahip_ctx *ctx, void *dst, int byte_value, size_t bytes) {
+    REQUIRE_CTX(ctx, "ahip_memset_async");
+    if (bytes == 0) return AHIP_OK;
+    if (!dst) return ctx->d.fail(AHIP_ERR_ARG, "ahip_memset_async: null pointer");
+    return ctx->d.check(hipMemsetAsync(dst, byte_value, bytes, ctx->d.stream), "hipMemsetAsync");
+}
+
+int ahip_sync(ahip_ctx *ctx) {
+    REQUIRE_CTX(ctx, "ahip_sync");
+    return ctx->d.check(hipStreamSynchronize(ctx->d.stream), "hipStreamSynchronize");
+}
+
+int ahip_host_alloc(ahip_ctx *ctx, size_t bytes, void **hptr) {
+    REQUIRE_CTX(ctx, "ahip_host_alloc");
+    if (!hptr) return ctx->d.fail(AHIP_ERR_ARG, "ahip_host_alloc: null output pointer");
+    *hptr = nullptr;
+    if (bytes == 0) return AHIP_OK;
+    return ctx->d.check(hipHostMalloc(hptr, bytes, hipHostMallocDefault), "hipHostMalloc");
+}
+
+int ahip_host_free(ahip_ctx *ctx, void *hptr) {
+    REQUIRE_CTX(ctx, "ahip_host_free");
+    if (!hptr) return AHIP_OK;
+    return ctx->d.check(hipHostFree(hptr), "hipHostFree");
+}
+
+int ahip_event_create(ahip_ctx *ctx, void **event) {
+    REQUIRE_CTX(ctx, "ahip_event_create");
+    if (!event) return ctx->d.fail(AHIP_ERR_ARG, "ahip_event_create: null output pointer");
+    hipEvent_t e;
+    int rc = ctx->d.check(hipEventCreate(&e), "hipEventCreate");
+    if (rc) return rc;
+    *event = e;
+    return AHIP_OK;
+}
+
+int ahip_event_record(ahip_ctx *ctx, void *event) {
+    REQUIRE_CTX(ctx, "ahip_event_record");
+    if (!event) return ctx->d.fail(AHIP_ERR_ARG, "ahip_event_record: null event");
+    return ctx->d.check(hipEventRecord(static_cast<hipEvent_t>(event), ctx->d.stream), "hipEventRecord");
+}
+
+int ahip_event_synchronize(ahip_ctx *ctx, void *event) {
+    REQUIRE_CTX(ctx, "ahip_event_synchronize");
+    if (!event) return ctx->d.fail(AHIP_ERR_ARG, "ahip_event_synchronize: null event");
+    return ctx->d.check(hipEventSynchronize(static_cast<hipEvent_t>(event)), "hipEventSynchronize");
+}
+
+int ahip_event_elapsed_ms(ahip_ctx *ctx, void *start, void *stop, float *ms) {
+    REQUIRE_CTX(ctx, "ahip_event_elapsed_ms");
+    if (!start || !stop || !ms) return ctx->d.fail(AHIP_ERR_ARG, "ahip_event_elapsed_ms: null argument");
+    return ctx->d.check(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)),
+                        "hipEventElapsedTime");
+}
+
+int ahip_event_destroy(ahip_ctx *ctx, void *event) {
+    REQUIRE_CTX(ctx, "ahip_event_destroy");
+    if (!event) return AHIP_OK;
+    return ctx->d.check(hipEventDestroy(static_cast<hipEvent_t>(event)), "hipEventDestroy");
+}
+
+// ---- host index math -------------------------------------------------------
+
+int ahip_broadcast_shape(int a_rank, const int64_t *a_dims, int b_rank, const int64_t *b_dims, int *out_rank,
+                         int64_t *out_dims) {
+    if (a_rank < 0 || b_rank < 0 || (a_rank && !a_dims) || (b_rank && !b_dims) || !out_rank || !out_dims)
+        return global_fail(AHIP_ERR_ARG, "ahip_broadcast_shape: invalid argument");
+    FixedDimensions a = FixedDimensions::from_i64(a_dims, (size_t)a_rank);
+    FixedDimensions b = FixedDimensions::from_i64(b_dims, (size_t)b_rank);
+    auto r = a.broadcast(b);
+    if (!r)
+        return global_fail(AHIP_ERR_SHAPE, "cannot broadcast " + a.to_string() + " with " + b.to_string());
+    *out_rank = (int)r->len();
+    for (size_t i = 0; i < r->len(); i++) out_dims[i] = (int64_t)(*r)[i];
+    return AHIP_OK;
+}
+
+int ahip_strides_for_broadcasting(int from_rank, const int64_t *from_dims, int to_rank, const int64_t *to_dims,
+                                  int64_t *out_strides) {
+    if (from_rank < 0 || to_rank < 0 || (from_rank && !from_dims) || (to_rank && (!to_dims || !out_strides)))
+        return global_fail(AHIP_ERR_ARG, "ahip_strides_for_broadcasting: invalid argument");
+    FixedDimensions from = FixedDimensions::from_i64(from_dims, (size_t)from_rank);
+    FixedDimensions to = FixedDimensions::from_i64(to_dims, (size_t)to_rank);
+    auto r = from.strides_for_broadcasting_to(to);
+    if (!r)
+        return global_fail(AHIP_ERR_SHAPE, "cannot broadcast " + from.to_string() + " to " + to.to_string());
+    for (size_t i = 0; i < r->len(); i++) out_strides[i] = (int64_t)(*r)[i];
+    return AHIP_OK;
+}
+
+// ---- operators --------------------------------------------------------------
+
+int ahip_binary(ahip_ctx *ctx, int op, float *out, const float *a, const float *b, int rank,
+                const int64_t *out_dims, const int64_t *a_strides, const int64_t *b_strides) {
+    REQUIRE_CTX(ctx, "ahip_binary");
+    return altius::launch_binary(ctx->d, op, out, a, b, rank, out_dims, a_strides, b_strides);
+}
+
+int ahip_unary(ahip_ctx *ctx, int op, float *out, const float *in, size_t n, float alpha, float beta) {
+    REQUIRE_CTX(ctx, "ahip_unary");
+    return altius::launch_unary(ctx->d, op, out, in, n, alpha, beta);
+}
+
+int ahip_softmax_lastaxis(ahip_ctx *ctx, float *out, const float *in, size_t rows, size_t len) {
+    REQUIRE_CTX(ctx, "ahip_softmax_lastaxis");
+    return altius::launch_softmax(ctx->d, out, in, rows, len);
+}
+
+int ahip_layernorm_lastaxis(ahip_ctx *ctx, float *out, const float *in, const float *gamma, const float *beta,
+                            size_t rows, size_t len, float eps) {
+    REQUIRE_CTX(ctx, "ahip_layernorm_lastaxis");
+    return altius::launch_layernorm(ctx->d, out, in, gamma, beta, rows, len, eps);
+}
+
+int ahip_reduce(ahip_ctx *ctx, int kind, float *out, const float *in, size_t outer, size_t reduce, size_t inner) {
+    REQUIRE_CTX(ctx, "ahip_reduce");
+    return altius::launch_reduce(ctx->d, kind, out, in, outer, reduce, inner);
+}
+
+}  // extern "C"

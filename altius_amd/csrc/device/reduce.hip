@@ -1,0 +1,307 @@
+// ReduceMean / ReduceMax for gfx950 over an [outer, reduce, inner] view.
+//
+//   inner == 1 (reduced axes are the trailing ones):
+//     short or many rows  -> one wavefront per row, lanes stride through the
+//                            row (16-byte loads when rows stay aligned), lane
+//                            butterfly at the end;
+//     long rows           -> a grid of 256-thread blocks per row, each block
+//                            reducing a contiguous chunk through LDS; with more
+//                            than one chunk per row the partials go to the
+//                            context's scratch buffer and a second, tiny launch
+//                            folds them.
+//   inner > 1 (e.g. axis 1 of [256,768,197]):
+//     lanes own output columns, so a wave reads whole contiguous input rows;
+//     the 8 waves of a block interleave over the reduced axis and combine
+//     through LDS; the reduced axis can additionally be split over blocks,
+//     again through the scratch buffer.
+//
+// Reference: crates/session_interpreter/src/session.rs:1292-1340.  ReduceMean
+// multiplies the sum by the f32 reciprocal of the reduced length, as the
+// reference does (session.rs:1331,1338).  Max is order-independent and exact;
+// sums are accumulated in a different order than the reference's 8 strided
+// accumulators.
+
+#include "common.h"
+#include "ctx.h"
+
+namespace altius {
+namespace {
+
+using namespace dev;
+
+constexpr int ROW_BLOCK = 256;
+constexpr int ROW_WAVES = ROW_BLOCK / WAVE;
+
+template <class OP> __device__ __forceinline__ float fold4(float acc, const float4 &v) {
+    acc = OP::apply(acc, v.x);
+    acc = OP::apply(acc, v.y);
+    acc = OP::apply(acc, v.z);
+    acc = OP::apply(acc, v.w);
+    return acc;
+}
+
+// Accumulates x[begin..end) strided over `nthreads` lanes starting at `tid`.
+// VEC == 4 requires x + begin 16-byte aligned; the range length may be ragged.
+template <class OP, int VEC>
+__device__ __forceinline__ float strided_fold(const float *__restrict__ x, size_t begin, size_t end, int tid,
+                                              int nthreads) {
+    float acc0 = OP::identity(), acc1 = OP::identity(), acc2 = OP::identity(), acc3 = OP::identity();
+    if (VEC == 4) {
+        const float4 *x4 = reinterpret_cast<const float4 *>(x + begin);
+        const size_t n4 = (end - begin) >> 2;
+        size_t i = tid;
+        for (; i + 3 * (size_t)nthreads < n4; i += 4 * (size_t)nthreads) {
+            const float4 a = x4[i];
+            const float4 b = x4[i + nthreads];
+            const float4 c = x4[i + 2 * (size_t)nthreads];
+            const float4 d = x4[i + 3 * (size_t)nthreads];
+            acc0 = fold4<OP>(acc0, a);
+            acc1 = fold4<OP>(acc1, b);
+            acc2 = fold4<OP>(acc2, c);
+            acc3 = fold4<OP>(acc3, d);
+        }
+        for (; i < n4; i += nthreads) acc0 = fold4<OP>(acc0, x4[i]);
+        for (size_t j = begin + (n4 << 2) + tid; j < end; j += nthreads) acc1 = OP::apply(acc1, x[j]);
+    } else {
+        size_t i = begin + tid;
+        for (; i + 3 * (size_t)nthreads < end; i += 4 * (size_t)nthreads) {
+            const float a = x[i];
+            const float b = x[i + nthreads];
+            const float c = x[i + 2 * (size_t)nthreads];
+            const float d = x[i + 3 * (size_t)nthreads];
+            acc0 = OP::apply(acc0, a);
+            acc1 = OP::apply(acc1, b);
+            acc2 = OP::apply(acc2, c);
+            acc3 = OP::apply(acc3, d);
+        }
+        for (; i < end; i += nthreads) acc0 = OP::apply(acc0, x[i]);
+    }
+    return OP::apply(OP::apply(acc0, acc1), OP::apply(acc2, acc3));
+}
+
+template <class OP, int VEC, bool SCALE>
+__global__ __launch_bounds__(ROW_BLOCK) void reduce_rows_wave(float *__restrict__ out,
+                                                              const float *__restrict__ in, size_t outer,
+                                                              size_t red, float scale) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const size_t row = (size_t)blockIdx.x * ROW_WAVES + (threadIdx.x >> 6);
+    if (row >= outer) return;
+    float acc = strided_fold<OP, VEC>(in + row * red, 0, red, lane, WAVE);
+    acc = wave_reduce<OP>(acc);
+    if (lane == 0) out[row] = SCALE ? acc * scale : acc;
+}
+
+// grid = (splits, outer).  Block (s, o) folds chunk s of row o into
+// dst[o * splits + s].
+template <class OP, int VEC, bool SCALE>
+__global__ __launch_bounds__(ROW_BLOCK) void reduce_rows_block(float *__restrict__ dst,
+                                                               const float *__restrict__ in, size_t red,
+                                                               size_t chunk, float scale) {
+    __shared__ float lds[ROW_WAVES];
+    const size_t o = blockIdx.y, s = blockIdx.x;
+    const size_t begin = s * chunk;
+    size_t end = begin + chunk;
+    if (end > red) end = red;
+    float acc = OP::identity();
+    if (begin < end) acc = strided_fold<OP, VEC>(in + o * red, begin, end, threadIdx.x, ROW_BLOCK);
+    acc = block_reduce<OP, ROW_WAVES>(acc, lds);
+    if (threadIdx.x == 0) dst[o * gridDim.x + s] = SCALE ? acc * scale : acc;
+}
+
+// ---------------------------------------------------------------------------
+// inner > 1
+// ---------------------------------------------------------------------------
+constexpr int COL_BLOCK = 512;
+constexpr int COL_WAVES = COL_BLOCK / WAVE;
+constexpr int ROW_UNROLL = 4;
+
+// grid = (outer * splits, column tiles).  Block (o*splits + s, t) folds rows
+// [s*chunk, (s+1)*chunk) of slab o for columns [t*64*CPL, (t+1)*64*CPL) into
+// dst[(o*splits + s) * inner + column].
+template <class OP, int CPL, bool SCALE>
+__global__ __launch_bounds__(COL_BLOCK) void reduce_cols(float *__restrict__ dst, const float *__restrict__ in,
+                                                         uint32_t red, uint32_t inner, uint32_t splits,
+                                                         uint32_t chunk, float scale) {
+    __shared__ float lds[COL_WAVES][CPL * WAVE];
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x >> 6;
+    const uint32_t o = blockIdx.x / splits, s = blockIdx.x % splits;
+    const uint32_t c0 = blockIdx.y * (CPL * WAVE) + lane;
+    const uint32_t r_begin = s * chunk;
+    uint32_t r_end = r_begin + chunk;
+    if (r_end > red) r_end = red;
+    const float *slab = in + (size_t)o * red * inner;
+
+    float acc[CPL];
+#pragma unroll
+    for (int j = 0; j < CPL; j++) acc[j] = OP::identity();
+
+    uint32_t r = r_begin + wave;
+    for (; r + (ROW_UNROLL - 1) * COL_WAVES < r_end; r += ROW_UNROLL * COL_WAVES) {
+        float v[ROW_UNROLL][CPL];
+#pragma unroll
+        for (int u = 0; u < ROW_UNROLL; u++) {
+            const float *row = slab + (size_t)(r + u * COL_WAVES) * inner;
+#pragma unroll
+            for (int j = 0; j < CPL; j++) {
+                const uint32_t c = c0 + j * WAVE;
+                v[u][j] = c < inner ? row[c] : OP::identity();
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < ROW_UNROLL; u++)
+#pragma unroll
+            for (int j = 0; j < CPL; j++) acc[j] = OP::apply(acc[j], v[u][j]);
+    }
+    for (; r < r_end; r += COL_WAVES) {
+        const float *row = slab + (size_t)r * inner;
+#pragma unroll
+        for (int j = 0; j < CPL; j++) {
+            const uint32_t c = c0 + j * WAVE;
+            if (c < inner) acc[j] = OP::apply(acc[j], row[c]);
+        }
+    }
+
+#pragma unroll
+    for (int j = 0; j < CPL; j++) lds[wave][j * WAVE + lane] = acc[j];
+    __syncthreads();
+    for (int t = threadIdx.x; t < CPL * WAVE; t += COL_BLOCK) {
+        float a = OP::identity();
+#pragma unroll
+        for (int w = 0; w < COL_WAVES; w++) a = OP::apply(a, lds[w][t]);
+        const uint32_t c = blockIdx.y * (CPL * WAVE) + t;
+        if (c < inner) dst[(size_t)blockIdx.x * inner + c] = SCALE ? a * scale : a;
+    }
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+constexpr size_t MAX_GRID_X = 0x7FFFFFFFu;
+constexpr size_t MAX_GRID_Y = 65535;
+
+template <class OP, bool SCALE>
+void rows_wave_launch(hipStream_t s, float *out, const float *in, size_t outer, size_t red, float scale) {
+    const bool vec4 = (red % 4 == 0) && aligned16(in);
+    const size_t blocks = (outer + ROW_WAVES - 1) / ROW_WAVES;
+    if (vec4)
+        hipLaunchKernelGGL((reduce_rows_wave<OP, 4, SCALE>), dim3((unsigned)blocks), dim3(ROW_BLOCK), 0, s, out,
+                           in, outer, red, scale);
+    else
+        hipLaunchKernelGGL((reduce_rows_wave<OP, 1, SCALE>), dim3((unsigned)blocks), dim3(ROW_BLOCK), 0, s, out,
+                           in, outer, red, scale);
+}
+
+template <class OP, bool SCALE>
+void rows_block_launch(hipStream_t s, float *dst, const float *in, size_t outer, size_t red, size_t splits,
+                       size_t chunk, float scale) {
+    // Chunks start 16-byte aligned when the row pitch and the chunk length are multiples of 4.
+    const bool vec4 = aligned16(in) && (red % 4 == 0 || outer == 1) && (chunk % 4 == 0);
+    const dim3 grid((unsigned)splits, (unsigned)outer);
+    if (vec4)
+        hipLaunchKernelGGL((reduce_rows_block<OP, 4, SCALE>), grid, dim3(ROW_BLOCK), 0, s, dst, in, red, chunk,
+                           scale);
+    else
+        hipLaunchKernelGGL((reduce_rows_block<OP, 1, SCALE>), grid, dim3(ROW_BLOCK), 0, s, dst, in, red, chunk,
+                           scale);
+}
+
+template <class OP, bool SCALE>
+void cols_launch(hipStream_t s, float *dst, const float *in, size_t outer, size_t red, size_t inner,
+                 size_t splits, size_t chunk, float scale) {
+    const size_t cpl = inner <= 64 ? 1 : inner <= 128 ? 2 : 4;
+    const size_t tiles = (inner + cpl * WAVE - 1) / (cpl * WAVE);
+    const dim3 grid((unsigned)(outer * splits), (unsigned)tiles);
+    const dim3 block(COL_BLOCK);
+    if (cpl == 1)
+        hipLaunchKernelGGL((reduce_cols<OP, 1, SCALE>), grid, block, 0, s, dst, in, (uint32_t)red,
+                           (uint32_t)inner, (uint32_t)splits, (uint32_t)chunk, scale);
+    else if (cpl == 2)
+        hipLaunchKernelGGL((reduce_cols<OP, 2, SCALE>), grid, block, 0, s, dst, in, (uint32_t)red,
+                           (uint32_t)inner, (uint32_t)splits, (uint32_t)chunk, scale);
+    else
+        hipLaunchKernelGGL((reduce_cols<OP, 4, SCALE>), grid, block, 0, s, dst, in, (uint32_t)red,
+                           (uint32_t)inner, (uint32_t)splits, (uint32_t)chunk, scale);
+}
+
+template <class OP, bool SCALE>
+int reduce_impl(DeviceCtx &ctx, float *out, const float *in, size_t outer, size_t red, size_t inner,
+                float scale) {
+    hipStream_t s = ctx.stream;
+    if (inner == 1) {
+        if (red <= 4096 || outer >= 65536) {
+            if ((outer + ROW_WAVES - 1) / ROW_WAVES > MAX_GRID_X)
+                return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: too many rows for one launch");
+            rows_wave_launch<OP, SCALE>(s, out, in, outer, red, scale);
+            return ctx.check(hipGetLastError(), "reduce rows (wave) launch");
+        }
+        if (outer > MAX_GRID_Y) return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: too many rows for one launch");
+        // Aim for a few thousand blocks; every block gets at least 4096 elements.
+        size_t splits = 1;
+        if (outer < 1024) {
+            splits = (4096 + outer - 1) / outer;
+            const size_t max_splits = (red + 4095) / 4096;
+            if (splits > max_splits) splits = max_splits;
+            if (splits < 1) splits = 1;
+        }
+        size_t chunk = (red + splits - 1) / splits;
+        chunk = (chunk + 1023) / 1024 * 1024;
+        splits = (red + chunk - 1) / chunk;
+        if (splits == 1) {
+            rows_block_launch<OP, SCALE>(s, out, in, outer, red, 1, chunk, scale);
+            return ctx.check(hipGetLastError(), "reduce rows (block) launch");
+        }
+        if (outer * splits > ctx.scratch_floats)
+            return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: scratch buffer too small");
+        rows_block_launch<OP, false>(s, ctx.scratch, in, outer, red, splits, chunk, 1.0f);
+        rows_wave_launch<OP, SCALE>(s, out, ctx.scratch, outer, splits, scale);
+        return ctx.check(hipGetLastError(), "reduce rows (two-stage) launch");
+    }
+
+    // inner > 1
+    if (red >= ((size_t)1 << 32) || inner >= ((size_t)1 << 31))
+        return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: axis extent exceeds 32-bit index range");
+    const size_t cpl = inner <= 64 ? 1 : inner <= 128 ? 2 : 4;
+    const size_t tiles = (inner + cpl * WAVE - 1) / (cpl * WAVE);
+    if (tiles > MAX_GRID_Y) return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: inner extent too large");
+    size_t splits = 1;
+    const size_t blocks = outer * tiles;
+    if (blocks < 1024 && red >= 64) {
+        splits = (1024 + blocks - 1) / blocks;
+        const size_t max_splits = red / 32;  // at least 32 rows (4 per wave) per block
+        if (splits > max_splits) splits = max_splits;
+        if (splits < 1) splits = 1;
+    }
+    size_t chunk = (red + splits - 1) / splits;
+    splits = (red + chunk - 1) / chunk;
+    if (outer * splits > MAX_GRID_X)
+        return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: outer extent too large for one launch");
+    if (splits == 1) {
+        cols_launch<OP, SCALE>(s, out, in, outer, red, inner, 1, chunk, scale);
+        return ctx.check(hipGetLastError(), "reduce cols launch");
+    }
+    if (outer * splits * inner > ctx.scratch_floats) {
+        // Not enough scratch for the partials: do it in one stage.
+        cols_launch<OP, SCALE>(s, out, in, outer, red, inner, 1, red, scale);
+        return ctx.check(hipGetLastError(), "reduce cols launch");
+    }
+    cols_launch<OP, false>(s, ctx.scratch, in, outer, red, inner, splits, chunk, 1.0f);
+    cols_launch<OP, SCALE>(s, out, ctx.scratch, outer, splits, inner, 1, splits, scale);
+    return ctx.check(hipGetLastError(), "reduce cols (two-stage) launch");
+}
+
+}  // namespace
+
+int launch_reduce(DeviceCtx &ctx, int kind, float *out, const float *in, size_t outer, size_t red,
+                  size_t inner) {
+    if (kind != AHIP_REDUCE_MEAN && kind != AHIP_REDUCE_MAX) return ctx.fail(AHIP_ERR_ARG, "reduce: unknown kind");
+    if (outer == 0 || inner == 0) return AHIP_OK;
+    if (red == 0) return ctx.fail(AHIP_ERR_ARG, "reduce: empty reduced axis");
+    if (!out || !in) return ctx.fail(AHIP_ERR_ARG, "reduce: null tensor pointer");
+    if (kind == AHIP_REDUCE_MEAN) {
+        const float r_axis_len = 1.0f / (float)red;
+        return reduce_impl<SumOp, true>(ctx, out, in, outer, red, inner, r_axis_len);
+    }
+    return reduce_impl<MaxOp, false>(ctx, out, in, outer, red, inner, 1.0f);
+}
+
+}  // namespace altius

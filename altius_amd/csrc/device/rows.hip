@@ -1,0 +1,290 @@
+// Softmax and LayerNormalization over the last axis for gfx950.
+//
+// Rows of up to 1024 elements: one 64-lane wavefront per row, the row held in
+// registers (read once, written once), max / sum reductions as lane butterflies.
+// Lane l owns elements (l + 64*k)*VEC .. +VEC-1, so every load instruction of
+// the wave covers one contiguous 256-byte (VEC=1) or 1-KiB (VEC=4) span.
+// Longer rows: one 256-thread block per row, streaming the row from memory
+// (L2-resident after the first pass) with LDS-staged block reductions.
+//
+// Reference arithmetic:
+//   Softmax  crates/session_interpreter/src/session.rs:990-1026,
+//            crates/session_interpreter/src/fast_math.rs:102-187
+//   LayerNorm crates/session_interpreter/src/session.rs:1433-1486
+// The per-element values follow the reference bit for bit; the row sums are
+// accumulated in a different order (lane butterfly instead of 8 strided
+// accumulators), which moves results by a few ulp.
+
+#include "common.h"
+#include "ctx.h"
+#include "math.h"
+
+#include <math.h>
+
+namespace altius {
+namespace {
+
+using namespace dev;
+
+constexpr int BLOCK = 256;
+constexpr int WAVES_PER_BLOCK = BLOCK / WAVE;
+
+// Register image of one row spread over a wavefront.
+template <int VEC, int NCH> struct RowRegs {
+    float v[NCH * VEC];
+
+    // Loads the row; slots past `len` are set to `fill`.
+    __device__ __forceinline__ void load(const float *__restrict__ row, int len, int lane, float fill) {
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            const int e = (lane + WAVE * k) * VEC;
+            if (VEC == 4) {
+                if (e < len) {
+                    const float4 t = *reinterpret_cast<const float4 *>(row + e);
+                    v[k * VEC + 0] = t.x;
+                    v[k * VEC + 1 % VEC] = t.y;
+                    v[k * VEC + 2 % VEC] = t.z;
+                    v[k * VEC + 3 % VEC] = t.w;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < VEC; j++) v[k * VEC + j] = fill;
+                }
+            } else {
+                v[k] = e < len ? row[e] : fill;
+            }
+        }
+    }
+    __device__ __forceinline__ void store(float *__restrict__ row, int len, int lane) const {
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            const int e = (lane + WAVE * k) * VEC;
+            if (e < len) {
+                if (VEC == 4) {
+                    float4 t;
+                    t.x = v[k * VEC + 0];
+                    t.y = v[k * VEC + 1 % VEC];
+                    t.z = v[k * VEC + 2 % VEC];
+                    t.w = v[k * VEC + 3 % VEC];
+                    *reinterpret_cast<float4 *>(row + e) = t;
+                } else {
+                    row[e] = v[k];
+                }
+            }
+        }
+    }
+    // Element index of slot s, for per-column operands.
+    static __device__ __forceinline__ int index(int lane, int s) {
+        return (lane + WAVE * (s / VEC)) * VEC + (s % VEC);
+    }
+};
+
+// ---------------------------------------------------------------------------
+// Softmax
+// ---------------------------------------------------------------------------
+template <int VEC, int NCH>
+__global__ __launch_bounds__(BLOCK) void softmax_wave(float *__restrict__ out, const float *__restrict__ in,
+                                                      size_t rows, int len) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const size_t row = (size_t)blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float *x = in + row * (size_t)len;
+    float *o = out + row * (size_t)len;
+
+    RowRegs<VEC, NCH> r;
+    const float nan = __builtin_nanf("");
+    r.load(x, len, lane, nan);
+
+    float mx = nan;  // fold(NAN, max): NaN elements are ignored
+#pragma unroll
+    for (int s = 0; s < NCH * VEC; s++) mx = nanmax(r.v[s], mx);
+    mx = wave_reduce<MaxOp>(mx);
+
+    float sum = 0.0f;
+#pragma unroll
+    for (int s = 0; s < NCH * VEC; s++) {
+        const bool valid = RowRegs<VEC, NCH>::index(lane, s) < len;
+        const float e = softmax_exp(r.v[s], mx);
+        r.v[s] = e;
+        sum += valid ? e : 0.0f;
+    }
+    sum = wave_reduce<SumOp>(sum);
+    const float recip = 1.0f / sum;
+#pragma unroll
+    for (int s = 0; s < NCH * VEC; s++) r.v[s] *= recip;
+    r.store(o, len, lane);
+}
+
+// One block per row, any length: max pass, sum pass, write pass.
+__global__ __launch_bounds__(BLOCK) void softmax_block_stream(float *__restrict__ out,
+                                                              const float *__restrict__ in, size_t len) {
+    __shared__ float lds[WAVES_PER_BLOCK];
+    const float *x = in + (size_t)blockIdx.x * len;
+    float *o = out + (size_t)blockIdx.x * len;
+    const float nan = __builtin_nanf("");
+
+    float mx = nan;
+    for (size_t i = threadIdx.x; i < len; i += BLOCK) mx = nanmax(x[i], mx);
+    mx = block_reduce<MaxOp, WAVES_PER_BLOCK>(mx, lds);
+
+    float sum = 0.0f;
+    for (size_t i = threadIdx.x; i < len; i += BLOCK) sum += softmax_exp(x[i], mx);
+    sum = block_reduce<SumOp, WAVES_PER_BLOCK>(sum, lds);
+    const float recip = 1.0f / sum;
+
+    for (size_t i = threadIdx.x; i < len; i += BLOCK) o[i] = softmax_exp(x[i], mx) * recip;
+}
+
+// ---------------------------------------------------------------------------
+// LayerNormalization
+// ---------------------------------------------------------------------------
+template <int VEC, int NCH>
+__global__ __launch_bounds__(BLOCK) void layernorm_wave(float *__restrict__ out, const float *__restrict__ in,
+                                                        const float *__restrict__ gamma,
+                                                        const float *__restrict__ beta, size_t rows, int len,
+                                                        float eps) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const size_t row = (size_t)blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float *x = in + row * (size_t)len;
+    float *o = out + row * (size_t)len;
+
+    RowRegs<VEC, NCH> r;
+    r.load(x, len, lane, 0.0f);
+
+    const float inv_n = 1.0f / (float)len;
+    float sum = 0.0f;
+#pragma unroll
+    for (int s = 0; s < NCH * VEC; s++) sum += r.v[s];
+    const float mean = wave_reduce<SumOp>(sum) * inv_n;
+
+    float ss = 0.0f;
+#pragma unroll
+    for (int s = 0; s < NCH * VEC; s++) {
+        const bool valid = RowRegs<VEC, NCH>::index(lane, s) < len;
+        const float d = r.v[s] - mean;
+        r.v[s] = d;
+        ss += valid ? d * d : 0.0f;
+    }
+    ss = wave_reduce<SumOp>(ss);
+    const float inv_std = 1.0f / sqrtf(__builtin_fmaf(ss, inv_n, eps));
+
+    RowRegs<VEC, NCH> g, b;
+    g.load(gamma, len, lane, 0.0f);
+    b.load(beta, len, lane, 0.0f);
+#pragma unroll
+    for (int s = 0; s < NCH * VEC; s++) r.v[s] = __builtin_fmaf(r.v[s] * inv_std, g.v[s], b.v[s]);
+    r.store(o, len, lane);
+}
+
+__global__ __launch_bounds__(BLOCK) void layernorm_block_stream(float *__restrict__ out,
+                                                                const float *__restrict__ in,
+                                                                const float *__restrict__ gamma,
+                                                                const float *__restrict__ beta, size_t len,
+                                                                float eps) {
+    __shared__ float lds[WAVES_PER_BLOCK];
+    const float *x = in + (size_t)blockIdx.x * len;
+    float *o = out + (size_t)blockIdx.x * len;
+    const float inv_n = 1.0f / (float)len;
+
+    float sum = 0.0f;
+    for (size_t i = threadIdx.x; i < len; i += BLOCK) sum += x[i];
+    const float mean = block_reduce<SumOp, WAVES_PER_BLOCK>(sum, lds) * inv_n;
+
+    float ss = 0.0f;
+    for (size_t i = threadIdx.x; i < len; i += BLOCK) {
+        const float d = x[i] - mean;
+        ss += d * d;
+    }
+    ss = block_reduce<SumOp, WAVES_PER_BLOCK>(ss, lds);
+    const float inv_std = 1.0f / sqrtf(__builtin_fmaf(ss, inv_n, eps));
+
+    for (size_t i = threadIdx.x; i < len; i += BLOCK)
+        o[i] = __builtin_fmaf((x[i] - mean) * inv_std, gamma[i], beta[i]);
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Picks the register layout for a wave-per-row kernel: VEC=4 when rows stay
+// 16-byte aligned, and the smallest chunk count that covers the row.
+template <template <int, int> class Launcher, class... Args>
+bool dispatch_wave(bool vec4, size_t len, Args... args) {
+    if (vec4) {
+        const size_t chunks = (len / 4 + WAVE - 1) / WAVE;
+        switch (chunks) {
+        case 1: Launcher<4, 1>::go(args...); return true;
+        case 2: Launcher<4, 2>::go(args...); return true;
+        case 3: Launcher<4, 3>::go(args...); return true;
+        case 4: Launcher<4, 4>::go(args...); return true;
+        }
+        return false;
+    }
+    const size_t chunks = (len + WAVE - 1) / WAVE;
+    if (chunks <= 1) { Launcher<1, 1>::go(args...); return true; }
+    if (chunks <= 2) { Launcher<1, 2>::go(args...); return true; }
+    if (chunks <= 4) { Launcher<1, 4>::go(args...); return true; }
+    if (chunks <= 8) { Launcher<1, 8>::go(args...); return true; }
+    if (chunks <= 12) { Launcher<1, 12>::go(args...); return true; }
+    if (chunks <= 16) { Launcher<1, 16>::go(args...); return true; }
+    return false;
+}
+
+template <int VEC, int NCH> struct SoftmaxLauncher {
+    static void go(hipStream_t s, float *out, const float *in, size_t rows, int len) {
+        const size_t blocks = (rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+        hipLaunchKernelGGL((softmax_wave<VEC, NCH>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, rows,
+                           len);
+    }
+};
+
+template <int VEC, int NCH> struct LayerNormLauncher {
+    static void go(hipStream_t s, float *out, const float *in, const float *gamma, const float *beta,
+                   size_t rows, int len, float eps) {
+        const size_t blocks = (rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+        hipLaunchKernelGGL((layernorm_wave<VEC, NCH>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in,
+                           gamma, beta, rows, len, eps);
+    }
+};
+
+constexpr size_t MAX_WAVE_ROW = 1024;
+constexpr size_t MAX_GRID = 0x7FFFFFFFu;
+
+}  // namespace
+
+int launch_softmax(DeviceCtx &ctx, float *out, const float *in, size_t rows, size_t len) {
+    if (rows == 0 || len == 0) return AHIP_OK;
+    if (!out || !in) return ctx.fail(AHIP_ERR_ARG, "softmax: null tensor pointer");
+    if (len <= MAX_WAVE_ROW) {
+        if ((rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK > MAX_GRID)
+            return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: too many rows for one launch");
+        const bool vec4 = (len % 4 == 0) && aligned16(out) && aligned16(in);
+        if (!dispatch_wave<SoftmaxLauncher>(vec4, len, ctx.stream, out, in, rows, (int)len))
+            return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: no wave layout for this row length");
+    } else {
+        if (rows > MAX_GRID) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: too many rows for one launch");
+        hipLaunchKernelGGL(softmax_block_stream, dim3((unsigned)rows), dim3(BLOCK), 0, ctx.stream, out, in,
+                           len);
+    }
+    return ctx.check(hipGetLastError(), "softmax launch");
+}
+
+int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *gamma, const float *beta,
+                     size_t rows, size_t len, float eps) {
+    if (rows == 0 || len == 0) return AHIP_OK;
+    if (!out || !in || !gamma || !beta) return ctx.fail(AHIP_ERR_ARG, "layernorm: null tensor pointer");
+    if (len <= MAX_WAVE_ROW) {
+        if ((rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK > MAX_GRID)
+            return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: too many rows for one launch");
+        const bool vec4 =
+            (len % 4 == 0) && aligned16(out) && aligned16(in) && aligned16(gamma) && aligned16(beta);
+        if (!dispatch_wave<LayerNormLauncher>(vec4, len, ctx.stream, out, in, gamma, beta, rows, (int)len,
+                                              eps))
+            return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: no wave layout for this row length");
+    } else {
+        if (rows > MAX_GRID) return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: too many rows for one launch");
+        hipLaunchKernelGGL(layernorm_block_stream, dim3((unsigned)rows), dim3(BLOCK), 0, ctx.stream, out, in,
+                           gamma, beta, len, eps);
+    }
+    return ctx.check(hipGetLastError(), "layernorm launch");
+}
+
+}  // namespace altius

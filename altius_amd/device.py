@@ -1,0 +1,215 @@
+"""Python handles over the device part of the C ABI: a context (device + stream),
+device buffers, events, and the operator kernels on device-resident tensors.
+
+Everything here is a thin call into libaltius_hip.so; no arithmetic happens in
+Python.
+"""
+import ctypes
+
+import numpy as np
+
+from . import _lib
+from ._lib import check, i64_array
+
+ADD, SUB, MUL, DIV, POW = 0, 1, 2, 3, 4
+SQRT, ERF, GELU, SIGMOID, HARDSIGMOID, RELU = 0, 1, 2, 3, 4, 5
+REDUCE_MEAN, REDUCE_MAX = 0, 1
+
+
+def broadcast_shape(a_dims, b_dims):
+    """fixed_dim::broadcast through the C ABI; raises AltiusHipError(Shape) if incompatible."""
+    L = _lib.lib()
+    rank = ctypes.c_int(0)
+    out = (ctypes.c_int64 * max(len(a_dims), len(b_dims), 1))()
+    check(L.ahip_broadcast_shape(len(a_dims), i64_array(a_dims), len(b_dims), i64_array(b_dims),
+                                 ctypes.byref(rank), out))
+    return [int(out[i]) for i in range(rank.value)]
+
+
+def strides_for_broadcasting(from_dims, to_dims):
+    """Tensor::strides_for_broadcasting through the C ABI."""
+    L = _lib.lib()
+    out = (ctypes.c_int64 * max(len(to_dims), 1))()
+    check(L.ahip_strides_for_broadcasting(len(from_dims), i64_array(from_dims), len(to_dims),
+                                          i64_array(to_dims), out))
+    return [int(out[i]) for i in range(len(to_dims))]
+
+
+class DeviceBuffer:
+    """A device allocation owned by a Context."""
+
+    def __init__(self, ctx, nbytes):
+        self.ctx = ctx
+        self.nbytes = int(nbytes)
+        p = ctypes.c_void_p()
+        check(ctx.L.ahip_malloc(ctx.handle, self.nbytes, ctypes.byref(p)), ctx.handle)
+        self.ptr = p.value or 0
+
+    def free(self):
+        if self.ptr and self.ctx.handle:
+            check(self.ctx.L.ahip_free(self.ctx.handle, self.ptr), self.ctx.handle)
+        self.ptr = 0
+
+    def offset(self, nbytes):
+        return self.ptr + int(nbytes)
+
+
+class Context:
+    """One device + one stream.  Not thread-safe; create one per thread."""
+
+    def __init__(self, device=0):
+        self.L = _lib.lib()
+        h = ctypes.c_void_p()
+        check(self.L.ahip_init(int(device), ctypes.byref(h)))
+        self.handle = h
+        self._buffers = []
+
+    def close(self):
+        if self.handle:
+            for b in self._buffers:
+                b.free()
+            self._buffers = []
+            self.L.ahip_destroy(self.handle)
+            self.handle = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    # --- memory ---------------------------------------------------------
+    def alloc(self, nbytes):
+        b = DeviceBuffer(self, nbytes)
+        self._buffers.append(b)
+        return b
+
+    def free(self, buf):
+        buf.free()
+        self._buffers = [b for b in self._buffers if b is not buf]
+
+    def upload(self, array):
+        """Copies a numpy array to a new device buffer."""
+        a = np.ascontiguousarray(array)
+        buf = self.alloc(max(a.nbytes, 4))
+        if a.nbytes:
+            check(self.L.ahip_h2d_async(self.handle, buf.ptr, a.ctypes.data, a.nbytes), self.handle)
+            self.sync()
+        return buf
+
+    def download(self, buf, shape, dtype=np.float32, offset_bytes=0):
+        out = np.empty(shape, dtype=dtype)
+        if out.nbytes:
+            check(self.L.ahip_d2h_async(self.handle, out.ctypes.data, buf.ptr + offset_bytes, out.nbytes),
+                  self.handle)
+        self.sync()
+        return out
+
+    def sync(self):
+        check(self.L.ahip_sync(self.handle), self.handle)
+
+    # --- events -----------------------------------------------------------
+    def event(self):
+        e = ctypes.c_void_p()
+        check(self.L.ahip_event_create(self.handle, ctypes.byref(e)), self.handle)
+        return e
+
+    def record(self, event):
+        check(self.L.ahip_event_record(self.handle, event), self.handle)
+
+    def elapsed_ms(self, start, stop):
+        check(self.L.ahip_event_synchronize(self.handle, stop), self.handle)
+        ms = ctypes.c_float(0)
+        check(self.L.ahip_event_elapsed_ms(self.handle, start, stop, ctypes.byref(ms)), self.handle)
+        return ms.value
+
+    def destroy_event(self, event):
+        check(self.L.ahip_event_destroy(self.handle, event), self.handle)
+
+    # --- kernels on raw device pointers -----------------------------------
+    def binary_raw(self, op, out_ptr, a_ptr, b_ptr, out_dims, a_strides, b_strides):
+        check(self.L.ahip_binary(self.handle, op, out_ptr, a_ptr, b_ptr, len(out_dims), i64_array(out_dims),
+                                 i64_array(a_strides), i64_array(b_strides)), self.handle)
+
+    def unary_raw(self, op, out_ptr, in_ptr, n, alpha=0.0, beta=0.0):
+        check(self.L.ahip_unary(self.handle, op, out_ptr, in_ptr, n, alpha, beta), self.handle)
+
+    def softmax_raw(self, out_ptr, in_ptr, rows, length):
+        check(self.L.ahip_softmax_lastaxis(self.handle, out_ptr, in_ptr, rows, length), self.handle)
+
+    def layernorm_raw(self, out_ptr, in_ptr, gamma_ptr, beta_ptr, rows, length, eps):
+        check(self.L.ahip_layernorm_lastaxis(self.handle, out_ptr, in_ptr, gamma_ptr, beta_ptr, rows, length,
+                                             eps), self.handle)
+
+    def reduce_raw(self, kind, out_ptr, in_ptr, outer, red, inner):
+        check(self.L.ahip_reduce(self.handle, kind, out_ptr, in_ptr, outer, red, inner), self.handle)
+
+    # --- convenience: numpy in, numpy out (upload, one kernel, download) ----
+    def binary(self, op, a, b):
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        b = np.ascontiguousarray(b, dtype=np.float32)
+        out_dims = broadcast_shape(a.shape, b.shape)
+        a_str = strides_for_broadcasting(a.shape, out_dims)
+        b_str = strides_for_broadcasting(b.shape, out_dims)
+        n = int(np.prod(out_dims, dtype=np.int64)) if out_dims else 1
+        da, db = self.upload(a), self.upload(b)
+        do = self.alloc(max(n * 4, 4))
+        try:
+            self.binary_raw(op, do.ptr, da.ptr, db.ptr, out_dims, a_str, b_str)
+            return self.download(do, out_dims)
+        finally:
+            for x in (da, db, do):
+                self.free(x)
+
+    def unary(self, op, x, alpha=0.0, beta=0.0):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        dx = self.upload(x)
+        do = self.alloc(max(x.nbytes, 4))
+        try:
+            self.unary_raw(op, do.ptr, dx.ptr, x.size, alpha, beta)
+            return self.download(do, x.shape)
+        finally:
+            self.free(dx)
+            self.free(do)
+
+    def softmax(self, x):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        length = x.shape[-1]
+        rows = x.size // length if length else 0
+        dx = self.upload(x)
+        do = self.alloc(max(x.nbytes, 4))
+        try:
+            self.softmax_raw(do.ptr, dx.ptr, rows, length)
+            return self.download(do, x.shape)
+        finally:
+            self.free(dx)
+            self.free(do)
+
+    def layer_norm(self, x, gamma, beta, eps=1e-5):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        gamma = np.ascontiguousarray(gamma, dtype=np.float32)
+        beta = np.ascontiguousarray(beta, dtype=np.float32)
+        length = x.shape[-1]
+        assert gamma.size == length and beta.size == length
+        rows = x.size // length if length else 0
+        dx, dg, db = self.upload(x), self.upload(gamma), self.upload(beta)
+        do = self.alloc(max(x.nbytes, 4))
+        try:
+            self.layernorm_raw(do.ptr, dx.ptr, dg.ptr, db.ptr, rows, length, eps)
+            return self.download(do, x.shape)
+        finally:
+            for t in (dx, dg, db, do):
+                self.free(t)
+
+    def reduce(self, kind, x, outer, red, inner):
+        """Reduces the middle axis of x viewed as [outer, red, inner]; returns [outer, inner]."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        assert x.size == outer * red * inner
+        dx = self.upload(x)
+        do = self.alloc(max(outer * inner * 4, 4))
+        try:
+            self.reduce_raw(kind, do.ptr, dx.ptr, outer, red, inner)
+            return self.download(do, (outer, inner))
+        finally:
+            self.free(dx)
+            self.free(do)

@@ -1,0 +1,132 @@
+/*
+ * CPU oracle for the altius interpreter tensor kernels.
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  It is a C++ restatement,
+ * written from the reference's source text, of the arithmetic that
+ * altius_session_interpreter::InterpreterSession performs for the broadcast
+ * binary ops, the unary ops, ReduceMean/ReduceMax, Softmax and
+ * LayerNormalization.  Only tests, the smoke check and the CPU-baseline leg of
+ * the benchmark may load it; the shipped library never links or calls it.
+ *
+ * Every function below cites the reference file:line it follows (paths are
+ * relative to the reference checkout root).
+ *
+ * Parity status per function (what pins the restatement without running the
+ * reference, which needs a Rust nightly toolchain that is not available):
+ *   - orc_broadcast / orc_strides_for_broadcasting: pinned by the reference's
+ *     own unit tests (crates/core/src/fixed_dim.rs:192-245) and by
+ *     numpy.broadcast_to on the shape list of
+ *     crates/altius_py/tests/test_ops_bin.py.
+ *   - Add/Sub/Mul/Div, Sqrt, Relu, HardSigmoid, Pow(x,2): IEEE-754 closed forms,
+ *     pinned bit-exactly against numpy float32 / float64-emulated fma.
+ *   - Softmax, Sigmoid, Gelu: formulas are fully in-tree
+ *     (crates/session_interpreter/src/fast_math.rs); pinned against exact
+ *     softmax / logistic / tanh-GELU at the reference's own test tolerance and
+ *     by invariants (rows sum to 1, symmetry, monotonicity, saturation).
+ *   - ReduceMean, LayerNormalization: pinned against float64 two-pass formulas
+ *     and by known-answer vectors whose result depends on the 8-lane strided
+ *     accumulation order (crates/session_interpreter/src/session.rs:1028-1055).
+ *   - ReduceMax: order-independent, pinned by brute force.
+ *   - orc_unary(ORC_ERF): PARITY UNPINNED.  The reference calls
+ *     fastapprox::faster::erf from the crate fastapprox 0.3.1 (Cargo.lock:978),
+ *     whose source is not vendored.  The restatement follows the published
+ *     algorithm of that crate (a port of Paul Mineiro's fastapprox "fasterpow2"
+ *     / "fastererfc"); only the loose bounds the reference's own test states
+ *     (|erf - exact| <= 1e-1, crates/altius_py/tests/test_ops_elemwise.py:129-152)
+ *     are checked.
+ *   - Shapes the reference interpreter has no kernel for (axis ReduceMax,
+ *     multi-axis / non-rank-3 ReduceMean, general-broadcast Pow) are computed
+ *     per the ONNX definition with the same accumulation primitives; the
+ *     functions report that through *no_reference_kernel.
+ */
+#ifndef ALTIUS_ORACLE_H
+#define ALTIUS_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum orc_binary_op { ORC_ADD = 0, ORC_SUB = 1, ORC_MUL = 2, ORC_DIV = 3, ORC_POW = 4 };
+
+enum orc_unary_op {
+    ORC_SQRT = 0,
+    ORC_ERF = 1,
+    ORC_GELU = 2,
+    ORC_SIGMOID = 3,
+    ORC_HARDSIGMOID = 4,
+    ORC_RELU = 5
+};
+
+enum orc_reduce_kind { ORC_REDUCE_MEAN = 0, ORC_REDUCE_MAX = 1 };
+
+/* Return codes. */
+#define ORC_OK 0
+#define ORC_ERR_BROADCAST 1    /* shapes cannot be broadcast (reference: unwrap() on None -> panic) */
+#define ORC_ERR_UNSUPPORTED 2  /* the reference has no kernel (assert/todo!() panic) and strict mode was asked */
+#define ORC_ERR_ARG 3
+
+/* crates/core/src/fixed_dim.rs:26-28 */
+int orc_is_scalar(int rank, const int64_t *dims);
+
+/* crates/core/src/fixed_dim.rs:112-136.  out_dims must hold max(rank) entries. */
+int orc_broadcast(int n_shapes, const int *ranks, const int64_t *const *dims, int *out_rank,
+                  int64_t *out_dims);
+
+/* crates/core/src/tensor.rs:369-406 == crates/core/src/fixed_dim.rs:64-101.
+ * out_strides holds to_rank entries, in elements. */
+int orc_strides_for_broadcasting(int from_rank, const int64_t *from_dims, int to_rank,
+                                 const int64_t *to_dims, int64_t *out_strides);
+
+/* crates/core/src/tensor.rs:554-560 */
+void orc_compute_strides(int rank, const int64_t *dims, int64_t *out_strides);
+
+/* crates/core/src/analysis/shape.rs:354-411 (ReduceMax / ReduceMean output dims).
+ * kind selects the arm: ReduceMax with no axes reduces every axis, ReduceMean
+ * with no axes reduces none. */
+int orc_reduce_shape(int kind, int rank, const int64_t *dims, int n_axes, const int64_t *axes,
+                     int keep_dims, int *out_rank, int64_t *out_dims);
+
+/* crates/session_interpreter/src/session.rs:384-526 (Add/Sub/Mul/Div) and
+ * 566-606 (Pow).  `out` has the broadcast shape.  threads follows ThreadCtx
+ * (crates/session_interpreter/src/thread.rs): only the equal-dims path is
+ * threaded.  strict != 0 returns ORC_ERR_UNSUPPORTED where the reference
+ * panics (rank-1 general path, Pow with a non-scalar, non-equal exponent). */
+int orc_binary(int op, const float *a, int a_rank, const int64_t *a_dims, const float *b, int b_rank,
+               const int64_t *b_dims, float *out, int threads, int strict,
+               int *no_reference_kernel);
+
+/* session.rs:608-619 (Sqrt), 796-803 (Relu), 805-812 (HardSigmoid),
+ * 823-838 + fast_math.rs:281-355 (Gelu), 905-922 + fast_math.rs:189-279
+ * (Sigmoid), 924-931 (Erf -> fastapprox::faster::erf).
+ * alpha/beta are HardSigmoid's attributes, ignored by the other ops. */
+int orc_unary(int op, const float *in, float *out, size_t n, float alpha, float beta, int threads);
+
+/* session.rs:990-1026 + fast_math.rs:102-187.  Last axis only. */
+int orc_softmax(const float *in, float *out, size_t rows, size_t len, int threads);
+
+/* session.rs:1433-1486, 1028-1055.  Last axis only; scale/bias hold len values. */
+int orc_layer_norm(const float *in, const float *scale, const float *bias, float *out, size_t rows,
+                   size_t len, float eps, int threads);
+
+/* session.rs:1292-1340.  The reference implements exactly two cases:
+ * ReduceMean over axis 2 of a rank-3 tensor with keepdims, and ReduceMax over
+ * all axes without keepdims.  Other contiguous axis groups are computed per the
+ * ONNX definition (and *no_reference_kernel is set); strict != 0 refuses them.
+ * *saw_nan is set when ReduceMax meets a NaN (the reference panics there). */
+int orc_reduce(int kind, const float *in, int rank, const int64_t *dims, int n_axes,
+               const int64_t *axes, int keep_dims, float *out, int strict,
+               int *no_reference_kernel, int *saw_nan);
+
+/* The accumulation primitives on their own, for known-answer tests.
+ * session.rs:1028-1040 and 1042-1055. */
+float orc_fast_sum(const float *x, size_t n);
+float orc_fast_sum_squares(const float *x, size_t n);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif

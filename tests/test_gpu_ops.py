@@ -1,0 +1,296 @@
+"""Parity of the HIP kernels with the CPU oracle, called through the C ABI.
+
+Bars (BASELINE.json): bit-exact for Add/Sub/Mul/Div, Sqrt, Relu, HardSigmoid,
+Pow(x, 2), ReduceMax and all broadcast indexing; 1e-5 relative / 1e-6 absolute
+for everything whose row sums are accumulated in a different order than the
+reference's 8-lane accumulators (Softmax, LayerNormalization, ReduceMean).
+The element-wise approximations (Gelu, Sigmoid, Erf) are deterministic
+per-element formulas and are held to bit equality as well.
+"""
+import numpy as np
+import pytest
+
+from altius_amd import device as D
+from altius_amd import synth
+from conftest import assert_bits_equal, assert_close
+
+pytestmark = pytest.mark.gpu
+
+BIN = {"Add": (D.ADD, 0), "Sub": (D.SUB, 1), "Mul": (D.MUL, 2), "Div": (D.DIV, 3)}
+
+# Shape pairs of the reference's own binary-op tests
+# (crates/altius_py/tests/test_ops_bin.py:11-140, crates/session_interpreter/tests/op_bin.rs:62-76)
+# plus the benchmark configurations' broadcast patterns at reduced batch.
+BIN_SHAPES = [
+    ([1, 2], [1, 2]),
+    ([3, 1, 10], [3, 1, 10]),
+    ([1, 2, 3, 4, 5, 6, 7], [1, 2, 3, 4, 5, 6, 7]),
+    ([16, 3, 224, 224], [16, 3, 224, 224]),
+    ([1, 3, 28, 28], [3, 1, 1]),
+    ([1, 12, 9, 9], [1, 1, 1, 9]),
+    ([4, 1, 2], [3, 1]),
+    ([3, 28, 28], [3, 28, 1]),
+    ([3, 15, 15], [15]),
+    ([3, 28, 28], [1]),
+    ([1], [3, 28, 28]),
+    ([3, 28, 28], []),
+    ([1, 197, 768], [768]),            # cfg0
+    ([4, 12, 197, 197], [4, 1, 1, 197]),  # cfg4 mask pattern
+    ([8, 197, 768], [8, 197, 1]),      # cfg2 Sub/Div
+    ([8, 576, 7, 7], [8, 576, 1, 1]),  # cfg3 squeeze-excite
+    ([5, 1, 7, 1, 3], [1, 6, 1, 2, 3]),  # two-sided, rank 5
+    ([2, 3, 4, 5, 6, 7], [7]),
+    ([1, 1, 1], [1]),
+    ([7], [7]),
+    ([1023], [1023]),
+    ([2, 0, 3], [3]),                  # empty
+]
+
+
+@pytest.mark.parametrize("name", list(BIN))
+@pytest.mark.parametrize("sa,sb", BIN_SHAPES)
+def test_binary_bit_exact(ctx, oracle, case, name, sa, sb):
+    case(f"binary {name} {sa} {sb}")
+    op, oop = BIN[name]
+    a = synth.uniform(11, sa) + np.float32(0.25)
+    b = synth.uniform(12, sb) + np.float32(0.25)
+    expected = oracle.binary(oop, a, b)
+    actual = ctx.binary(op, a, b)
+    assert_bits_equal(actual, expected, f"{name} {sa} {sb}")
+    # The oracle itself agrees with numpy's IEEE arithmetic and broadcasting.
+    ref = {"Add": a + b, "Sub": a - b, "Mul": a * b, "Div": a / b}[name]
+    assert_bits_equal(expected, ref.astype(np.float32), f"oracle vs numpy {name}")
+
+
+def test_binary_known_answer(ctx, case):
+    """[1,3,...,15] + [2,4,...,16] = [3,7,...,31] (crates/session/tests/ort.rs:17-25)."""
+    case("binary KAT")
+    a = np.arange(1, 16, 2, dtype=np.float32)
+    b = np.arange(2, 17, 2, dtype=np.float32)
+    assert ctx.binary(D.ADD, a, b).tolist() == [3, 7, 11, 15, 19, 23, 27, 31]
+
+
+def test_binary_special_values(ctx, oracle, case):
+    case("binary special values")
+    s = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 3.4e38, 1e-38, 2.5],
+                 dtype=np.float32)
+    a = np.repeat(s, len(s)).reshape(len(s), len(s))
+    b = np.tile(s, len(s)).reshape(len(s), len(s))
+    for name, (op, oop) in BIN.items():
+        with np.errstate(all="ignore"):
+            assert_bits_equal(ctx.binary(op, a, b), oracle.binary(oop, a, b), f"special {name}")
+
+
+def test_binary_unaligned_pointers(ctx, oracle, case):
+    """Operands at addresses that are not 16-byte aligned take the scalar kernels."""
+    case("binary unaligned")
+    n = 4099
+    a = synth.normal(21, (n + 1,))
+    b = synth.normal(22, (n + 3,))
+    da, db = ctx.upload(a), ctx.upload(b)
+    do = ctx.alloc((n + 1) * 4)
+    ctx.binary_raw(D.MUL, do.ptr + 4, da.ptr + 4, db.ptr + 12, [n], [1], [1])
+    got = ctx.download(do, (n,), offset_bytes=4)
+    assert_bits_equal(got, a[1:] * b[3:], "unaligned flat")
+    # strided with unaligned pieces: [17, 5] * [5]
+    x = synth.normal(23, (17 * 5 + 1,))
+    y = synth.normal(24, (5 + 1,))
+    dx, dy = ctx.upload(x), ctx.upload(y)
+    ctx.binary_raw(D.ADD, do.ptr + 4, dx.ptr + 4, dy.ptr + 4, [17, 5], [5, 1], [0, 1])
+    got = ctx.download(do, (17, 5), offset_bytes=4)
+    assert_bits_equal(got, x[1:].reshape(17, 5) + y[1:], "unaligned strided")
+    for t in (da, db, do, dx, dy):
+        ctx.free(t)
+
+
+def test_binary_broadcast_mismatch_is_an_error(ctx, case):
+    """[1,3,28,28] + [3,1,2] cannot broadcast (test_ops_bin.py:31-40): an error value, not an abort."""
+    case("binary mismatch")
+    from altius_amd._lib import AltiusHipError, ERR_SHAPE
+
+    with pytest.raises(AltiusHipError) as e:
+        ctx.binary(D.ADD, np.zeros([1, 3, 28, 28], np.float32), np.zeros([3, 1, 2], np.float32))
+    assert e.value.code == ERR_SHAPE
+
+
+@pytest.mark.parametrize("sa,sb", [([1, 2], [1, 2]), ([1, 2, 3, 4, 5, 6, 7], [1, 2, 3, 4, 5, 6, 7]),
+                                   ([128, 3, 8, 8], [128, 3, 8, 8]), ([128, 3, 8, 8], [1]),
+                                   ([8, 197, 768], [])])
+def test_pow(ctx, oracle, case, sa, sb):
+    """Pow shapes of test_ops_bin.py:123-140.  powf is a libm call on both sides."""
+    case(f"pow {sa} {sb}")
+    a = synth.uniform(31, sa) + np.float32(0.5)
+    b = synth.uniform(32, sb) * np.float32(3.0)
+    assert_close(ctx.binary(D.POW, a, b), oracle.binary(4, a, b), what=f"pow {sa} {sb}")
+
+
+def test_pow_square_is_exact(ctx, oracle, case):
+    """Pow(x, 2) with a scalar exponent is x*x (session.rs:588-591): bit-exact."""
+    case("pow square")
+    x = synth.normal(33, (8, 197, 768))
+    for two in (np.array(2.0, np.float32), np.array([2.0], np.float32)):
+        got = ctx.binary(D.POW, x, two)
+        assert_bits_equal(got, x * x, "pow(x,2)")
+        assert_bits_equal(got, oracle.binary(4, x, two), "pow(x,2) vs oracle")
+
+
+UNARY = {
+    "Sqrt": (D.SQRT, 0),
+    "Erf": (D.ERF, 1),
+    "Gelu": (D.GELU, 2),
+    "Sigmoid": (D.SIGMOID, 3),
+    "HardSigmoid": (D.HARDSIGMOID, 4),
+    "Relu": (D.RELU, 5),
+}
+
+
+@pytest.mark.parametrize("name", list(UNARY))
+@pytest.mark.parametrize("shape", [[1, 2], [3, 1, 28, 28], [3, 1, 7, 7], [1, 2, 3], [4, 197, 3072], [1], [0], [4097]])
+def test_unary_bit_exact(ctx, oracle, case, name, shape):
+    """Shapes of crates/altius_py/tests/test_ops_elemwise.py:22-152 plus cfg3 at reduced batch."""
+    case(f"unary {name} {shape}")
+    op, oop = UNARY[name]
+    x = synth.normal(41, shape, std=2.0)
+    if name == "Sqrt":
+        x = np.abs(x)
+    alpha, beta = (1.0 / 6.0, 0.5) if name == "HardSigmoid" else (0.0, 0.0)
+    expected = oracle.unary(oop, x, alpha, beta)
+    actual = ctx.unary(op, x, alpha, beta)
+    assert_bits_equal(actual, expected, f"{name} {shape}")
+
+
+@pytest.mark.parametrize("name", list(UNARY))
+def test_unary_special_values(ctx, oracle, case, name):
+    case(f"unary special {name}")
+    op, oop = UNARY[name]
+    x = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 3.4e38, -3.4e38, 1e-38,
+                  88.0, -88.0, 89.0, -104.0, 104.0, 9.0, -9.0, 10.0, 38.0, 39.0, 50.0, -50.0, 0.5, 6.0, -6.0],
+                 dtype=np.float32)
+    with np.errstate(all="ignore"):
+        expected = oracle.unary(oop, x, 0.2, 0.5)
+    actual = ctx.unary(op, x, 0.2, 0.5)
+    # Relu of -0.0: the reference leaves the sign of the zero unspecified.
+    assert_bits_equal(actual, expected, f"special {name}", zero_sign_free=(name == "Relu"))
+
+
+def test_hardsigmoid_default_attributes(ctx, oracle, case):
+    """ONNX defaults alpha=0.2, beta=0.5 (crates/core/src/onnx/load.rs:321-324)."""
+    case("hardsigmoid defaults")
+    x = synth.normal(42, (3, 1, 28, 28), std=3.0)
+    got = ctx.unary(D.HARDSIGMOID, x, 0.2, 0.5)
+    assert_bits_equal(got, oracle.unary(4, x, 0.2, 0.5), "hardsigmoid")
+    exact = np.clip(np.float64(np.float32(0.2)) * x.astype(np.float64) + 0.5, 0, 1).astype(np.float32)
+    assert_bits_equal(got, exact, "hardsigmoid vs float64 fma")
+
+
+SOFTMAX_SHAPES = [[1, 2, 3], [3, 28, 28], [16, 512, 512], [2, 12, 197, 197], [5, 1], [7, 64], [3, 65], [9, 256],
+                  [3, 1000], [2, 1024], [3, 1025], [2, 4096], [2, 5000], [1, 70001]]
+
+
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
+def test_softmax(ctx, oracle, case, shape):
+    """Shapes of test_ops_elemwise.py:107-126 plus row lengths around every kernel boundary."""
+    case(f"softmax {shape}")
+    x = synth.normal(51, shape)
+    got = ctx.softmax(x)
+    assert_close(got, oracle.softmax(x), what=f"softmax {shape}")
+    np.testing.assert_allclose(got.sum(-1, dtype=np.float64), 1.0, atol=2e-6)
+
+
+def test_softmax_masked_rows(ctx, oracle, case):
+    """cfg4: scores + mask(-1e4) then Softmax; masked entries underflow to exact zeros or denormals."""
+    case("softmax masked")
+    c = synth.cfg4(batch=2)
+    z = c["scores"] + c["mask"]
+    got = ctx.softmax(z)
+    exp = oracle.softmax(z)
+    assert_close(got, exp, what="masked softmax")
+    masked = np.broadcast_to(c["mask"], z.shape) != 0
+    assert masked.any() and np.all(got[masked] < 1e-30)
+    # Fully masked and constant rows, huge and tiny magnitudes, NaN in a row.
+    x = np.zeros((6, 197), np.float32)
+    x[0] = -1e4
+    x[1] = 3.0
+    x[2, ::2] = 1e30
+    x[3, 5] = -np.inf
+    x[4] = synth.normal(52, (197,)) * 1e-30
+    x[5, 7] = np.nan
+    with np.errstate(all="ignore"):
+        assert_close(ctx.softmax(x), oracle.softmax(x), what="softmax edge rows")
+
+
+LN_SHAPES = [[1, 20, 10], [2, 197, 768], [3, 5, 197], [4, 1], [5, 64], [3, 1024], [2, 1028], [2, 4100], [3, 3072]]
+
+
+@pytest.mark.parametrize("shape", LN_SHAPES)
+def test_layernorm(ctx, oracle, case, shape):
+    """[1,20,10] is the reference's test (crates/altius_py/tests/test_ops_norm.py:16-18)."""
+    case(f"layernorm {shape}")
+    x = synth.normal(61, shape, mean=0.3, std=1.7)
+    g = synth.normal(62, (shape[-1],), mean=1.0, std=0.02)
+    b = synth.normal(63, (shape[-1],), mean=0.0, std=0.02)
+    got = ctx.layer_norm(x, g, b, 1e-5)
+    assert_close(got, oracle.layer_norm(x, g, b, 1e-5), what=f"layernorm {shape}")
+    # and the textbook formula at the reference's own tolerance (test_ops_norm.py:86)
+    xd = x.astype(np.float64)
+    ref = (xd - xd.mean(-1, keepdims=True)) / np.sqrt(xd.var(-1, keepdims=True) + 1e-5) * g + b
+    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5)
+
+
+REDUCE_CASES = [
+    # (shape, axes, keepdims)
+    ([1, 50, 70], [-1], True),         # test_ops_reduce.py:10-18
+    ([8, 4, 5, 5], [2, 3], True),      # test_ops_reduce.py:21-30
+    ([8, 197, 768], [-1], True),       # cfg2
+    ([8, 576, 7, 7], [2, 3], True),    # cfg3 squeeze-excite
+    ([4, 768, 197], [1], False),       # cfg4 pattern
+    ([4, 768, 197], [1], True),
+    ([3, 10, 5000], [2], True),        # long rows, wave path limit
+    ([2, 3, 70000], [2], False),       # long rows, block path
+    ([1, 2000000], [1], False),        # split rows through scratch
+    ([5, 33, 2], [1], False),          # narrow inner
+    ([2, 100, 300], [1], False),       # several column tiles
+    ([2, 4000, 64], [1], False),       # split columns through scratch
+    ([7, 1, 9], [1], True),
+    ([6, 5], [0], False),
+]
+
+
+@pytest.mark.parametrize("shape,axes,keep", REDUCE_CASES)
+def test_reduce_mean(ctx, oracle, case, shape, axes, keep):
+    case(f"reduce_mean {shape} {axes}")
+    x = synth.normal(71, shape, mean=0.5)
+    exp = oracle.reduce(0, x, axes, keep)
+    ax = sorted(a % len(shape) for a in axes)
+    outer = int(np.prod(shape[:ax[0]], dtype=np.int64))
+    red = int(np.prod(shape[ax[0]:ax[-1] + 1], dtype=np.int64))
+    inner = int(np.prod(shape[ax[-1] + 1:], dtype=np.int64))
+    got = ctx.reduce(D.REDUCE_MEAN, x, outer, red, inner).reshape(exp.shape)
+    assert_close(got, exp, what=f"reduce_mean {shape}")
+    np.testing.assert_allclose(got, x.astype(np.float64).mean(tuple(ax), keepdims=keep), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("shape,axes,keep", REDUCE_CASES)
+def test_reduce_max_bit_exact(ctx, oracle, case, shape, axes, keep):
+    case(f"reduce_max {shape} {axes}")
+    x = synth.normal(72, shape)
+    exp = oracle.reduce(1, x, axes, keep)
+    ax = sorted(a % len(shape) for a in axes)
+    outer = int(np.prod(shape[:ax[0]], dtype=np.int64))
+    red = int(np.prod(shape[ax[0]:ax[-1] + 1], dtype=np.int64))
+    inner = int(np.prod(shape[ax[-1] + 1:], dtype=np.int64))
+    got = ctx.reduce(D.REDUCE_MAX, x, outer, red, inner).reshape(exp.shape)
+    assert_bits_equal(got, exp, f"reduce_max {shape}")
+    assert_bits_equal(got, x.max(tuple(ax), keepdims=keep), "reduce_max vs numpy")
+
+
+@pytest.mark.parametrize("shape", [[1, 50, 70], [3, 1000, 1000], [1], [5]])
+def test_reduce_max_all_axes(ctx, oracle, case, shape):
+    """The one ReduceMax the reference implements: every axis, keepdims=0 (test_ops_reduce.py:33-41)."""
+    case(f"reduce_max all {shape}")
+    x = synth.normal(73, shape)
+    info = {}
+    exp = oracle.reduce(1, x, [], False, strict=True, info=info)
+    assert not info["no_reference_kernel"]
+    got = ctx.reduce(D.REDUCE_MAX, x, 1, x.size, 1).reshape(exp.shape)
+    assert_bits_equal(got, exp, f"reduce_max all {shape}")

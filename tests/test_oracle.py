@@ -1,0 +1,364 @@
+"""Pins the CPU oracle without the reference (which needs a Rust toolchain that is
+not available): the reference's own unit tests and known answers, IEEE closed
+forms, exact rational arithmetic on samples, invariants of the approximated
+functions at the reference's own test tolerances, and known-answer vectors whose
+result depends on the accumulation order.  No GPU needed.
+"""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+from scipy.special import erf as exact_erf
+
+from altius_amd import synth
+from conftest import assert_bits_equal
+
+
+def round_f32(q: Fraction) -> np.float32:
+    """Correctly rounded (nearest-even) float32 of an exact rational."""
+    if q == 0:
+        return np.float32(0.0)
+    c = np.float32(float(q))
+    cands = {c, np.nextafter(c, np.float32(np.inf)), np.nextafter(c, np.float32(-np.inf))}
+    best = None
+    for x in cands:
+        if not np.isfinite(x):
+            continue
+        d = abs(Fraction(float(x)) - q)
+        key = (d, int(np.float32(x).view(np.uint32)) & 1)  # ties: even mantissa
+        if best is None or key < best[0]:
+            best = (key, np.float32(x))
+    return best[1]
+
+
+# ---- shapes and broadcasting ---------------------------------------------------
+
+def test_broadcast_reference_unit_tests(oracle):
+    """crates/core/src/fixed_dim.rs:192-245 (broadcast_1 .. broadcast_7)."""
+    assert oracle.broadcast([1]) == [1]
+    assert oracle.broadcast([1], [4, 1]) == [4, 1]
+    assert oracle.broadcast([4, 1], [1]) == [4, 1]
+    assert oracle.broadcast([10, 20, 30], [10, 20]) is None  # broadcast_4 panics
+    assert oracle.broadcast([1, 3, 3], [5, 1, 3, 3]) == [5, 1, 3, 3]
+    assert oracle.broadcast([1, 3, 1], [5, 3, 10]) == [5, 3, 10]
+    assert oracle.broadcast([1, 3, 4, 4], [3, 1, 1]) == [1, 3, 4, 4]
+
+
+def test_is_scalar(oracle):
+    """crates/core/src/fixed_dim.rs:26-28."""
+    assert oracle.is_scalar([])
+    assert oracle.is_scalar([1])
+    assert oracle.is_scalar([0])
+    assert not oracle.is_scalar([2])
+    assert not oracle.is_scalar([1, 1])
+
+
+PAIRS = [
+    ([1, 3, 28, 28], [3, 1, 1]), ([1, 12, 9, 9], [1, 1, 1, 9]), ([4, 1, 2], [3, 1]), ([3, 28, 28], [3, 28, 1]),
+    ([3, 15, 15], [15]), ([3, 28, 28], [1]), ([1, 197, 768], [768]), ([256, 12, 197, 197], [256, 1, 1, 197]),
+    ([32, 197, 768], [32, 197, 1]), ([32, 576, 7, 7], [32, 576, 1, 1]), ([5, 1, 7, 1, 3], [1, 6, 1, 2, 3]),
+    ([2, 3], []), ([1, 1], [1]), ([7], [7]),
+]
+
+
+@pytest.mark.parametrize("a,b", PAIRS)
+def test_broadcast_and_strides_match_numpy(oracle, a, b):
+    """Shape list of crates/altius_py/tests/test_ops_bin.py plus the benchmark configurations."""
+    out = oracle.broadcast(a, b)
+    assert tuple(out) == np.broadcast_shapes(tuple(a), tuple(b))
+    if int(np.prod(out, dtype=np.int64)) > 4_000_000:  # same pattern, smaller batch, for the index check
+        a, b = [2] + a[1:], [2] + b[1:]
+        out = oracle.broadcast(a, b)
+    for src in (a, b):
+        got = oracle.strides_for_broadcasting(src, out)
+        # Read a tensor of index values through those strides: must equal numpy's broadcast.
+        idx = np.arange(int(np.prod(src, dtype=np.int64)) if src else 1, dtype=np.int64).reshape(src)
+        want = np.broadcast_to(idx, out)
+        coords = np.indices(out).reshape(len(out), -1)
+        flat = (np.array(got, dtype=np.int64)[:, None] * coords).sum(0) if out else np.zeros(1, np.int64)
+        assert np.array_equal(idx.reshape(-1)[flat].reshape(out), want)
+
+
+def test_stride_of_matching_unit_axis_is_kept(oracle):
+    """An input extent of 1 that meets an output extent of 1 keeps its real stride (tensor.rs:391-392)."""
+    assert oracle.strides_for_broadcasting([256, 1, 1, 197], [256, 12, 197, 197]) == [197, 0, 0, 1]
+    assert oracle.strides_for_broadcasting([768], [1, 197, 768]) == [0, 0, 1]
+    assert oracle.strides_for_broadcasting([3, 1, 5], [3, 1, 5]) == [5, 5, 1]
+    assert oracle.strides_for_broadcasting([3, 1, 2], [1, 3, 28, 28]) is None
+    assert oracle.strides_for_broadcasting([2, 3, 4], [3, 4]) is None
+    assert oracle.compute_strides([256, 12, 197, 197]) == [465708, 38809, 197, 1]
+
+
+def test_reduce_shapes(oracle):
+    """crates/core/src/analysis/shape.rs:354-411."""
+    assert oracle.reduce_shape(1, [1, 50, 70], [], False) == [1]          # ReduceMax, all axes -> [1]
+    assert oracle.reduce_shape(1, [1, 50, 70], [], True) == [1, 1, 1]
+    assert oracle.reduce_shape(1, [256, 768, 197], [1], False) == [256, 197]
+    assert oracle.reduce_shape(1, [256, 768, 197], [1], True) == [256, 1, 197]
+    assert oracle.reduce_shape(0, [1, 50, 70], [-1], True) == [1, 50, 1]
+    assert oracle.reduce_shape(0, [8, 4, 5, 5], [2, 3], True) == [8, 4, 1, 1]
+    assert oracle.reduce_shape(0, [8, 4, 5, 5], [2, 3], False) == [8, 4]
+    assert oracle.reduce_shape(0, [2, 3], [], True) == [2, 3]             # ReduceMean without axes reduces nothing
+
+
+# ---- binary ops ----------------------------------------------------------------
+
+def test_add_known_answer(oracle):
+    """crates/session/tests/ort.rs:17-25."""
+    a = np.arange(1, 16, 2, dtype=np.float32)
+    b = np.arange(2, 17, 2, dtype=np.float32)
+    assert oracle.binary(0, a, b).tolist() == [3, 7, 11, 15, 19, 23, 27, 31]
+
+
+@pytest.mark.parametrize("a,b", PAIRS + [([1, 2], [1, 2]), ([3, 1, 10], [3, 1, 10]), ([16, 3, 32, 32], [16, 3, 32, 32])])
+def test_binary_matches_ieee(oracle, a, b):
+    """Expected values as crates/session_interpreter/tests/op_bin.rs:41-46 computes them: x op y."""
+    if int(np.prod(a, dtype=np.int64)) > 4_000_000:
+        a, b = [2] + a[1:], [2] + b[1:]
+    x = synth.uniform(1, a) + np.float32(0.1)
+    y = synth.uniform(2, b) + np.float32(0.1)
+    for op, ref in ((0, x + y), (1, x - y), (2, x * y), (3, x / y)):
+        for threads in (1, 4):
+            assert_bits_equal(oracle.binary(op, x, y, threads=threads), ref.astype(np.float32), f"op {op}")
+
+
+def test_binary_errors(oracle):
+    from oracle import ERR_BROADCAST, ERR_UNSUPPORTED, OracleError
+
+    with pytest.raises(OracleError) as e:  # test_ops_bin.py:31-40 (xfail in the reference)
+        oracle.binary(0, np.zeros([1, 3, 28, 28], np.float32), np.zeros([3, 1, 2], np.float32))
+    assert e.value.code == ERR_BROADCAST
+    with pytest.raises(OracleError) as e:  # Pow with a non-scalar, non-equal exponent: todo!() (session.rs:601)
+        oracle.binary(4, np.ones([3, 4], np.float32), np.ones([4], np.float32), strict=True)
+    assert e.value.code == ERR_UNSUPPORTED
+    info = {}
+    out = oracle.binary(4, np.full([3, 4], 3, np.float32), np.full([4], 2, np.float32), info=info)
+    assert info["no_reference_kernel"] and np.all(out == 9)
+
+
+def test_pow(oracle):
+    x = synth.uniform(3, [128, 3, 8, 8]) + np.float32(0.5)
+    assert_bits_equal(oracle.binary(4, x, np.array([2.0], np.float32)), x * x, "pow 2")
+    y = synth.uniform(4, [128, 3, 8, 8]) * 3
+    np.testing.assert_allclose(oracle.binary(4, x, y), np.power(x.astype(np.float64), y), rtol=2e-7)
+    np.testing.assert_allclose(oracle.binary(4, x, np.array([1.7], np.float32)),
+                               np.power(x.astype(np.float64), np.float32(1.7)), rtol=2e-7)
+
+
+# ---- unary ops -----------------------------------------------------------------
+
+def test_sqrt_relu_closed_forms(oracle):
+    x = synth.normal(5, [3, 1, 28, 28], std=3.0)
+    assert_bits_equal(oracle.unary(0, np.abs(x)), np.sqrt(np.abs(x)), "sqrt")
+    assert_bits_equal(oracle.unary(5, x), np.maximum(x, 0), "relu")
+    s = np.array([np.nan, -np.inf, np.inf, -0.0, 0.0, -1e-45], np.float32)
+    assert oracle.unary(5, s).tolist() == [0.0, 0.0, np.inf, 0.0, 0.0, 0.0]  # NaN.max(0.0) == 0.0 in Rust
+
+
+def test_hardsigmoid_is_fma_then_clamp(oracle):
+    """session.rs:810: alpha.mul_add(x, beta).clamp(0, 1), one rounding; checked in exact arithmetic."""
+    x = synth.normal(6, [600], std=3.0)
+    for alpha, beta in ((np.float32(0.2), np.float32(0.5)), (np.float32(1.0 / 6.0), np.float32(0.5))):
+        got = oracle.unary(4, x, alpha, beta)
+        want = np.array(
+            [min(max(round_f32(Fraction(float(alpha)) * Fraction(float(v)) + Fraction(float(beta))), np.float32(0)),
+                 np.float32(1)) for v in x], dtype=np.float32)
+        assert_bits_equal(got, want, "hardsigmoid")
+    assert np.isnan(oracle.unary(4, np.array([np.nan], np.float32), 0.2, 0.5)[0])  # clamp keeps NaN
+
+
+def test_sigmoid_against_exact(oracle):
+    """Reference tolerance: numpy default allclose (test_ops_elemwise.py:61-83)."""
+    x = synth.normal(7, [3, 1, 28, 28], std=4.0)
+    got = oracle.unary(3, x)
+    want = 1.0 / (1.0 + np.exp(-x.astype(np.float64)))
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-8)
+    # saturation, symmetry, monotonicity
+    s = oracle.unary(3, np.array([-200, -104, -50, 0, 50, 89, 200], np.float32))
+    assert 0 <= s[0] < 1e-38 and s[0] == s[1]   # input clamped at -103.97: exp overflows or nearly does
+    assert s[3] == 0.5 and s[5] == 1.0 and s[6] == 1.0
+    grid = np.linspace(-30, 30, 20001, dtype=np.float32)
+    g = oracle.unary(3, grid)
+    assert np.all(np.diff(g) >= -1e-7)
+    np.testing.assert_allclose(g + g[::-1], 1.0, atol=3e-7)
+    for t in (2, 3, 8):
+        assert_bits_equal(oracle.unary(3, x, threads=t), got, "sigmoid threads")
+
+
+def test_gelu_is_the_tanh_form(oracle):
+    """fast_math.rs:281-355: 0.5x(1+tanh(x(B+Cx^2))) with a rational tanh."""
+    x = synth.normal(8, [4, 197, 64], std=2.0)
+    got = oracle.unary(2, x)
+    xd = x.astype(np.float64)
+    tanh_gelu = 0.5 * xd * (1 + np.tanh(np.sqrt(2 / np.pi) * (xd + 0.044715 * xd ** 3)))
+    np.testing.assert_allclose(got, tanh_gelu, rtol=0, atol=1e-6)
+    erf_gelu = 0.5 * xd * (1 + exact_erf(xd / np.sqrt(2)))
+    np.testing.assert_allclose(got, erf_gelu, rtol=1e-5, atol=1e-1)  # the reference's bar (test_ops_elemwise.py:169-185)
+    assert np.max(np.abs(got - erf_gelu)) < 1e-3
+    s = oracle.unary(2, np.array([0.0, -20.0, 20.0, -9.0, 9.0], np.float32))
+    assert s[0] == 0 and abs(s[1]) < 1e-6 and s[2] == 20.0
+    for t in (2, 8):
+        assert_bits_equal(oracle.unary(2, x, threads=t), got, "gelu threads")
+
+
+def test_erf_loose_bounds(oracle):
+    """PARITY UNPINNED at the bit level (fastapprox is not vendored); only the reference's own
+    bound is checked: |erf - exact| <= 1e-1 (test_ops_elemwise.py:129-152)."""
+    x = np.linspace(-4, 4, 4001, dtype=np.float32)
+    got = oracle.unary(1, x)
+    assert np.max(np.abs(got - exact_erf(x.astype(np.float64)))) < 1e-1
+    assert abs(oracle.unary(1, np.zeros(1, np.float32))[0]) < 0.03
+    assert np.all(np.diff(got) >= -1e-6)
+    assert got[0] < -0.99 and got[-1] > 0.99
+
+
+# ---- accumulation order ----------------------------------------------------------
+
+def test_fast_sum_order_known_answers(oracle):
+    """session.rs:1028-1055: 8 strided accumulators, ordered lane sum, then the tail.
+    2^24 absorbs a lone +1 but not +2, so only that order gives these answers."""
+    x = np.ones(16, np.float32)
+    x[0] = 2.0 ** 24
+    # lane 0: 2^24 + 1 -> 2^24; lanes 1..7: 2 each; ordered: 2^24 + 2*7
+    assert oracle.fast_sum(x) == np.float32(2.0 ** 24 + 14)
+    # a sequential sum would give 2^24, a pairwise one 2^24 + 14 or 16: order matters here
+    assert np.float32(2.0 ** 24) + np.float32(1) == np.float32(2.0 ** 24)
+    # tail is summed on its own, then added: 2^24 + (1+1+1) = 2^24 + 3 -> rounds to even 2^24 + 4
+    y = np.zeros(11, np.float32)
+    y[0] = 2.0 ** 24
+    y[8:] = 1.0
+    assert oracle.fast_sum(y) == np.float32(2.0 ** 24 + 4)
+    # lanes are summed in order 0..7: (2^24 + 1) + 1 ... stays 2^24, then + 2^24*... use lane order
+    z = np.zeros(8, np.float32)
+    z[0] = 2.0 ** 24
+    z[1:] = 1.0
+    assert oracle.fast_sum(z) == np.float32(2.0 ** 24)       # ordered: each +1 is absorbed
+    assert oracle.fast_sum(z[::-1].copy()) == np.float32(2.0 ** 24 + 8)  # 7 first, then 2^24+7 -> 2^24+8
+    # squares
+    w = np.ones(16, np.float32)
+    w[0] = 4096.0
+    assert oracle.fast_sum_squares(w) == np.float32(2.0 ** 24 + 14)
+    # integers sum exactly in any order: every element is counted once
+    v = np.arange(1, 1000, dtype=np.float32)
+    assert oracle.fast_sum(v) == 999 * 1000 / 2
+    assert oracle.fast_sum(np.zeros(0, np.float32)) == 0
+
+
+# ---- Softmax ---------------------------------------------------------------------
+
+@pytest.mark.parametrize("shape", [[1, 2, 3], [3, 28, 28], [8, 512, 512], [2, 12, 197, 197], [5, 1], [3, 8], [3, 9]])
+def test_softmax_against_exact(oracle, shape):
+    """Reference tolerance: numpy default allclose vs the exact softmax (test_ops_elemwise.py:107-126)."""
+    x = synth.uniform(9, shape) if shape[0] != 2 else synth.normal(9, shape)
+    got = oracle.softmax(x)
+    xd = x.astype(np.float64)
+    e = np.exp(xd - xd.max(-1, keepdims=True))
+    np.testing.assert_allclose(got, e / e.sum(-1, keepdims=True), rtol=1e-5, atol=1e-8)
+    np.testing.assert_allclose(got.sum(-1, dtype=np.float64), 1.0, atol=1e-6)
+    for t in (2, 8):
+        assert_bits_equal(oracle.softmax(x, threads=t), got, "softmax threads")
+
+
+def test_softmax_edges(oracle):
+    x = np.zeros((5, 197), np.float32)
+    x[0] = -1e4                      # a constant row is uniform
+    x[1, 3] = 50.0                   # one dominant logit
+    x[2] = synth.attention_mask(10, (197,))
+    x[3, 0] = np.nan                 # NaN is skipped by the max, and max(NaN - m, -88.4) is -88.4: it becomes 0
+    x[4, :] = -np.inf
+    with np.errstate(all="ignore"):
+        s = oracle.softmax(x)
+    np.testing.assert_allclose(s[0], 1 / 197, rtol=1e-6)
+    assert s[1, 3] == 1.0 and np.all(s[1, :3] < 1e-20)
+    masked = x[2] != 0
+    assert masked.any() and np.all(s[2][masked] == 0) and abs(s[2].sum() - 1) < 1e-6
+    assert s[3, 0] < 1e-37 and not np.isnan(s[3]).any()
+    np.testing.assert_allclose(s[3, 1:], 1 / 196, rtol=1e-6)
+    assert np.all(np.isnan(s[4]))    # -inf - -inf = NaN
+
+
+# ---- LayerNormalization / ReduceMean / ReduceMax -------------------------------------
+
+@pytest.mark.parametrize("shape", [[1, 20, 10], [4, 197, 768], [3, 5, 197], [2, 1], [3, 7]])
+def test_layernorm_against_two_pass(oracle, shape):
+    """Reference tolerance rtol 1e-4 / atol 1e-5 (test_ops_norm.py:86); scale/bias shaped [1,1,n] there."""
+    x = synth.uniform(11, shape)
+    g = synth.uniform(12, [1] * (len(shape) - 1) + [shape[-1]])
+    b = synth.uniform(13, [1] * (len(shape) - 1) + [shape[-1]])
+    got = oracle.layer_norm(x, g, b, 1e-5)
+    xd = x.astype(np.float64)
+    want = (xd - xd.mean(-1, keepdims=True)) / np.sqrt(xd.var(-1, keepdims=True) + 1e-5) * g + b
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-5)
+    if shape[-1] > 1:
+        np.testing.assert_allclose(got, want, rtol=2e-6, atol=2e-6)
+    for t in (2, 8):
+        assert_bits_equal(oracle.layer_norm(x, g, b, 1e-5, threads=t), got, "layernorm threads")
+
+
+def test_layernorm_constant_row_gives_bias(oracle):
+    x = np.full((2, 64), 3.25, np.float32)
+    b = synth.normal(14, (64,))
+    assert_bits_equal(oracle.layer_norm(x, np.ones(64, np.float32), b, 1e-5), np.broadcast_to(b, (2, 64)), "ln const")
+
+
+def test_reduce_mean(oracle):
+    from oracle import ERR_UNSUPPORTED, OracleError
+
+    x = synth.uniform(15, [1, 50, 70])
+    info = {}
+    got = oracle.reduce(0, x, [-1], True, strict=True, info=info)   # the reference's kernel
+    assert not info["no_reference_kernel"] and got.shape == (1, 50, 1)
+    np.testing.assert_allclose(got, x.astype(np.float64).mean(-1, keepdims=True), rtol=1e-6)
+    # sum * (1/len), not sum / len (session.rs:1331,1338)
+    row = x[0, 0]
+    assert got[0, 0, 0] == oracle.fast_sum(row) * (np.float32(1.0) / np.float32(70))
+    y = synth.uniform(16, [8, 4, 5, 5])
+    with pytest.raises(OracleError) as e:                           # interpreter asserts rank 3, axis 2
+        oracle.reduce(0, y, [2, 3], True, strict=True)
+    assert e.value.code == ERR_UNSUPPORTED
+    got = oracle.reduce(0, y, [2, 3], True, info=info)              # clang-backend semantics (translator.rs:2757-2787)
+    assert info["no_reference_kernel"] and got.shape == (8, 4, 1, 1)
+    np.testing.assert_allclose(got, y.astype(np.float64).mean((2, 3), keepdims=True), rtol=1e-6)
+    z = synth.uniform(17, [4, 30, 7])
+    np.testing.assert_allclose(oracle.reduce(0, z, [1], False), z.astype(np.float64).mean(1), rtol=1e-6)
+
+
+def test_reduce_max(oracle):
+    from oracle import ERR_UNSUPPORTED, OracleError
+
+    x = synth.normal(18, [1, 50, 70])
+    info = {}
+    got = oracle.reduce(1, x, [], False, strict=True, info=info)    # the reference's kernel
+    assert not info["no_reference_kernel"] and got.shape == (1,) and got[0] == x.max()
+    y = synth.normal(19, [4, 768, 197])
+    with pytest.raises(OracleError) as e:                           # asserts axes.is_empty() (session.rs:1295)
+        oracle.reduce(1, y, [1], False, strict=True)
+    assert e.value.code == ERR_UNSUPPORTED
+    assert_bits_equal(oracle.reduce(1, y, [1], False, info=info), y.max(1), "axis max")
+    assert info["no_reference_kernel"]
+    assert_bits_equal(oracle.reduce(1, y, [1], True), y.max(1, keepdims=True), "axis max keepdims")
+    # max_by(partial_cmp) returns the last of equal maxima (+-0); NaN is reported
+    assert np.signbit(oracle.reduce(1, np.array([0.0, -0.0], np.float32), [], False)[0])
+    assert not np.signbit(oracle.reduce(1, np.array([-0.0, 0.0], np.float32), [], False)[0])
+    oracle.reduce(1, np.array([1.0, np.nan], np.float32), [], False, info=info)
+    assert info["saw_nan"]
+
+
+# ---- frozen vectors ---------------------------------------------------------------
+
+def test_golden_vectors(oracle):
+    """Small seeded inputs with the outputs this oracle produced when it was pinned by the checks
+    above (tests/golden/make_golden.py): guards the oracle against later edits."""
+    import os
+
+    path = os.path.join(os.path.dirname(__file__), "golden", "oracle_vectors.npz")
+    g = np.load(path)
+    x, y, gamma, beta = g["x"], g["y"], g["gamma"], g["beta"]
+    assert_bits_equal(oracle.binary(3, x, y), g["div"], "golden div")
+    for name, op in (("erf", 1), ("gelu", 2), ("sigmoid", 3)):
+        assert_bits_equal(oracle.unary(op, x), g[name], f"golden {name}")
+    assert_bits_equal(oracle.unary(4, x, 1.0 / 6.0, 0.5), g["hardsigmoid"], "golden hardsigmoid")
+    assert_bits_equal(oracle.softmax(x), g["softmax"], "golden softmax")
+    assert_bits_equal(oracle.layer_norm(x, gamma, beta, 1e-5), g["layernorm"], "golden layernorm")
+    assert_bits_equal(oracle.reduce(0, x, [-1], True), g["reduce_mean"], "golden reduce_mean")
+    assert_bits_equal(oracle.reduce(1, x, [1], False), g["reduce_max_axis1"], "golden reduce_max")
