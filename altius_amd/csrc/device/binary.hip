@@ -41,45 +41,31 @@ struct OpPowScalarExp {
 constexpr int BLOCK = 256;
 
 // ---------------------------------------------------------------------------
-// Flat kernel: both operands are FULL or SCALAR.  UNROLL float4 per lane,
-// block-contiguous so that a block's accesses stay coalesced.
+// Flat kernel: both operands are FULL or SCALAR.  One float4 per lane.
 // ---------------------------------------------------------------------------
-template <class OP, int MA, int MB, int UNROLL>
+template <class OP, int MA, int MB, bool NT>
 __global__ __launch_bounds__(BLOCK) void binary_flat_vec4(float *__restrict__ out,
                                                           const float *__restrict__ a,
                                                           const float *__restrict__ b, size_t n) {
     const size_t n4 = n >> 2;
-    const size_t base = (size_t)blockIdx.x * (BLOCK * UNROLL) + threadIdx.x;
+    const size_t i = (size_t)blockIdx.x * BLOCK + threadIdx.x;
     float sa = 0.f, sb = 0.f;
     if (MA == SCALAR) sa = a[0];
     if (MB == SCALAR) sb = b[0];
-    float4 va[UNROLL], vb[UNROLL];
-#pragma unroll
-    for (int u = 0; u < UNROLL; u++) {
-        const size_t i = base + (size_t)u * BLOCK;
-        if (i < n4) {
-            if (MA == FULL) va[u] = reinterpret_cast<const float4 *>(a)[i];
-            if (MB == FULL) vb[u] = reinterpret_cast<const float4 *>(b)[i];
-        }
-    }
-#pragma unroll
-    for (int u = 0; u < UNROLL; u++) {
-        const size_t i = base + (size_t)u * BLOCK;
-        if (i < n4) {
-            float4 x = MA == FULL ? va[u] : make_float4(sa, sa, sa, sa);
-            float4 y = MB == FULL ? vb[u] : make_float4(sb, sb, sb, sb);
-            float4 r;
-            r.x = OP::f(x.x, y.x);
-            r.y = OP::f(x.y, y.y);
-            r.z = OP::f(x.z, y.z);
-            r.w = OP::f(x.w, y.w);
-            reinterpret_cast<float4 *>(out)[i] = r;
-        }
+    if (i < n4) {
+        const float4 x = MA == FULL ? load4<NT>(a + 4 * i) : make_float4(sa, sa, sa, sa);
+        const float4 y = MB == FULL ? load4<NT>(b + 4 * i) : make_float4(sb, sb, sb, sb);
+        float4 r;
+        r.x = OP::f(x.x, y.x);
+        r.y = OP::f(x.y, y.y);
+        r.z = OP::f(x.z, y.z);
+        r.w = OP::f(x.w, y.w);
+        store4<NT>(out + 4 * i, r);
     }
     // The last (n % 4) elements.
     if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
-        const size_t i = (n4 << 2) + threadIdx.x;
-        out[i] = OP::f(MA == FULL ? a[i] : sa, MB == FULL ? b[i] : sb);
+        const size_t j = (n4 << 2) + threadIdx.x;
+        out[j] = OP::f(MA == FULL ? a[j] : sa, MB == FULL ? b[j] : sb);
     }
 }
 
@@ -96,9 +82,16 @@ __global__ __launch_bounds__(BLOCK) void binary_flat_scalar(float *__restrict__ 
 // ---------------------------------------------------------------------------
 // Strided kernel.
 // ---------------------------------------------------------------------------
+// Division of an index below 2^31 by a fixed divisor as multiply-high, add,
+// shift (the divisor's magic numbers are computed once on the host).
+struct FastDiv {
+    uint32_t d, mul, shift;
+    __device__ __forceinline__ uint32_t div(uint32_t n) const { return (__umulhi(n, mul) + n) >> shift; }
+};
+
 struct Geom {
     // Axis 0 is the innermost (fastest) output axis.
-    uint32_t dims[MAX_RANK];
+    FastDiv dims[MAX_RANK];
     uint32_t a_str[MAX_RANK];
     uint32_t b_str[MAX_RANK];
     int mode_a, mode_b;  // Mode
@@ -107,43 +100,56 @@ struct Geom {
     int a_vec, b_vec;
 };
 
-template <int RANK> struct Cursor {
-    uint32_t c[RANK];
-    uint32_t a_off, b_off;
-
-    __device__ __forceinline__ void init(const Geom &g, uint32_t flat) {
-        a_off = 0;
-        b_off = 0;
-#pragma unroll
-        for (int d = 0; d < RANK; d++) {
-            const uint32_t q = flat / g.dims[d];
-            c[d] = flat - q * g.dims[d];
-            flat = q;
-            a_off += c[d] * g.a_str[d];
-            b_off += c[d] * g.b_str[d];
-        }
-    }
-    // Advances by one output element.
-    __device__ __forceinline__ void next(const Geom &g) {
-        c[0]++;
-        a_off += g.a_str[0];
-        b_off += g.b_str[0];
-        if (c[0] == g.dims[0]) {
-#pragma unroll
-            for (int d = 0; d < RANK - 1; d++) {
-                if (c[d] != g.dims[d]) break;
-                c[d] = 0;
-                a_off -= g.dims[d] * g.a_str[d];
-                b_off -= g.dims[d] * g.b_str[d];
-                c[d + 1]++;
-                a_off += g.a_str[d + 1];
-                b_off += g.b_str[d + 1];
-            }
-        }
+// Offsets of one operand for VEC consecutive output elements that start at
+// column c0 of a row: elements past the end of the row continue in the next
+// row (VEC <= innermost extent, so at most one row change).
+template <int VEC> struct Span {
+    uint32_t row, next;  // operand offset of column 0 of this row / of the next row
+    __device__ __forceinline__ uint32_t at(int j, uint32_t c0, uint32_t d0, uint32_t s0) const {
+        const uint32_t c = c0 + j;
+        return c >= d0 ? next + (c - d0) * s0 : row + c * s0;
     }
 };
 
-template <class OP, int RANK, int VEC>
+// 16 bytes from an address that is only 4-byte aligned (global memory allows it).
+struct __attribute__((packed, aligned(4))) Float4U {
+    float x, y, z, w;
+};
+
+// Reads VEC consecutive output elements' worth of one operand.
+template <int VEC, bool NT>
+__device__ __forceinline__ void fetch(float (&v)[VEC], const float *__restrict__ p, int mode, int vec_ok,
+                                      const Span<VEC> &sp, uint32_t c0, uint32_t d0, uint32_t s0, uint32_t i0,
+                                      uint32_t n, bool whole, bool same_row) {
+    if (mode == FULL) {
+        if (VEC == 4 && whole) {
+            const float4 t = load4<NT>(p + i0);
+            v[0] = t.x; v[1 % VEC] = t.y; v[2 % VEC] = t.z; v[3 % VEC] = t.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC; j++) v[j] = i0 + j < n ? p[i0 + j] : 0.f;
+        }
+    } else if (mode == SCALAR) {
+        const float s = p[0];
+#pragma unroll
+        for (int j = 0; j < VEC; j++) v[j] = s;
+    } else if (VEC == 4 && vec_ok) {  // aligned, and no row change inside the four elements
+        const float4 t = *reinterpret_cast<const float4 *>(p + sp.row + c0);
+        v[0] = t.x; v[1 % VEC] = t.y; v[2 % VEC] = t.z; v[3 % VEC] = t.w;
+    } else if (VEC == 4 && whole && same_row && s0 == 1) {
+        const Float4U t = *reinterpret_cast<const Float4U *>(p + sp.row + c0);
+        v[0] = t.x; v[1 % VEC] = t.y; v[2 % VEC] = t.z; v[3 % VEC] = t.w;
+    } else if (VEC == 4 && whole && same_row && s0 == 0) {
+        const float s = p[sp.row];
+#pragma unroll
+        for (int j = 0; j < VEC; j++) v[j] = s;
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) v[j] = i0 + j < n ? p[sp.at(j, c0, d0, s0)] : 0.f;
+    }
+}
+
+template <class OP, int RANK, int VEC, bool NT>
 __global__ __launch_bounds__(BLOCK) void binary_strided(float *__restrict__ out,
                                                         const float *__restrict__ a,
                                                         const float *__restrict__ b, uint32_t n,
@@ -154,72 +160,40 @@ __global__ __launch_bounds__(BLOCK) void binary_strided(float *__restrict__ out,
     const uint32_t i0 = t * VEC;
     const bool whole = i0 + VEC <= n;
 
-    Cursor<RANK> cur;
-    cur.init(g, i0);
+    // Coordinates of element i0; row offsets of both operands; the same for the next row.
+    const uint32_t d0 = g.dims[0].d;
+    uint32_t q = g.dims[0].div(i0);
+    const uint32_t c0 = i0 - q * d0;
+    Span<VEC> sa, sb;
+    sa.row = sb.row = 0;
+    sa.next = sb.next = 0;
+    bool carry = true;  // the next row increments axis 1, and further axes while they wrap
+#pragma unroll
+    for (int d = 1; d < RANK; d++) {
+        uint32_t c;
+        if (d < RANK - 1) {
+            const uint32_t q2 = g.dims[d].div(q);
+            c = q - q2 * g.dims[d].d;
+            q = q2;
+        } else {
+            c = q;
+        }
+        sa.row += c * g.a_str[d];
+        sb.row += c * g.b_str[d];
+        uint32_t cn = c;
+        if (carry) {
+            cn = c + 1;
+            carry = cn == g.dims[d].d && d < RANK - 1;
+            if (carry) cn = 0;
+        }
+        sa.next += cn * g.a_str[d];
+        sb.next += cn * g.b_str[d];
+    }
+    const bool same_row = c0 + VEC <= d0;
 
     float x[VEC], y[VEC];
-    const bool same_row = cur.c[0] + VEC <= g.dims[0];
-
-    // Operand a.
-    if (g.mode_a == FULL) {
-        if (VEC == 4 && whole) {
-            const float4 v = *reinterpret_cast<const float4 *>(a + i0);
-            x[0] = v.x; x[1 % VEC] = v.y; x[2 % VEC] = v.z; x[3 % VEC] = v.w;
-        } else {
-#pragma unroll
-            for (int j = 0; j < VEC; j++) x[j] = i0 + j < n ? a[i0 + j] : 0.f;
-        }
-    } else if (g.mode_a == SCALAR) {
-        const float s = a[0];
-#pragma unroll
-        for (int j = 0; j < VEC; j++) x[j] = s;
-    }
-    // Operand b.
-    if (g.mode_b == FULL) {
-        if (VEC == 4 && whole) {
-            const float4 v = *reinterpret_cast<const float4 *>(b + i0);
-            y[0] = v.x; y[1 % VEC] = v.y; y[2 % VEC] = v.z; y[3 % VEC] = v.w;
-        } else {
-#pragma unroll
-            for (int j = 0; j < VEC; j++) y[j] = i0 + j < n ? b[i0 + j] : 0.f;
-        }
-    } else if (g.mode_b == SCALAR) {
-        const float s = b[0];
-#pragma unroll
-        for (int j = 0; j < VEC; j++) y[j] = s;
-    }
-    // Strided operands.
-    if (g.mode_a == STRIDED || g.mode_b == STRIDED) {
-        if (VEC == 4 && whole && same_row) {
-            if (g.mode_a == STRIDED) {
-                if (g.a_vec) {
-                    const float4 v = *reinterpret_cast<const float4 *>(a + cur.a_off);
-                    x[0] = v.x; x[1 % VEC] = v.y; x[2 % VEC] = v.z; x[3 % VEC] = v.w;
-                } else {
-#pragma unroll
-                    for (int j = 0; j < VEC; j++) x[j] = a[cur.a_off + j * g.a_str[0]];
-                }
-            }
-            if (g.mode_b == STRIDED) {
-                if (g.b_vec) {
-                    const float4 v = *reinterpret_cast<const float4 *>(b + cur.b_off);
-                    y[0] = v.x; y[1 % VEC] = v.y; y[2 % VEC] = v.z; y[3 % VEC] = v.w;
-                } else {
-#pragma unroll
-                    for (int j = 0; j < VEC; j++) y[j] = b[cur.b_off + j * g.b_str[0]];
-                }
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < VEC; j++) {
-                if (i0 + j < n) {
-                    if (g.mode_a == STRIDED) x[j] = a[cur.a_off];
-                    if (g.mode_b == STRIDED) y[j] = b[cur.b_off];
-                    if (j + 1 < VEC) cur.next(g);
-                }
-            }
-        }
-    }
+    fetch<VEC, NT>(x, a, g.mode_a, g.a_vec, sa, c0, d0, g.a_str[0], i0, n, whole, same_row);
+    fetch<VEC, NT>(y, b, g.mode_b, g.b_vec, sb, c0, d0, g.b_str[0], i0, n, whole, same_row);
 
     if (VEC == 4 && whole) {
         float4 r;
@@ -227,7 +201,7 @@ __global__ __launch_bounds__(BLOCK) void binary_strided(float *__restrict__ out,
         r.y = OP::f(x[1 % VEC], y[1 % VEC]);
         r.z = OP::f(x[2 % VEC], y[2 % VEC]);
         r.w = OP::f(x[3 % VEC], y[3 % VEC]);
-        *reinterpret_cast<float4 *>(out + i0) = r;
+        store4<NT>(out + i0, r);
     } else {
 #pragma unroll
         for (int j = 0; j < VEC; j++)
@@ -235,53 +209,69 @@ __global__ __launch_bounds__(BLOCK) void binary_strided(float *__restrict__ out,
     }
 }
 
+FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f;
+    f.d = d;
+    uint32_t shift = 0;
+    while (shift < 32 && ((uint64_t)1 << shift) < d) shift++;
+    const uint64_t one = 1;
+    f.mul = (uint32_t)(((one << 32) * ((one << shift) - d)) / d + 1);
+    f.shift = shift;
+    return f;
+}
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <class OP, int MA, int MB>
-void flat_dispatch(hipStream_t s, float *out, const float *a, const float *b, size_t n, bool vec) {
+void flat_dispatch(hipStream_t s, float *out, const float *a, const float *b, size_t n, bool vec, bool nt) {
     if (vec) {
-        constexpr int UNROLL = 4;
-        const size_t n4 = n >> 2;
-        size_t blocks = (n4 + (size_t)BLOCK * UNROLL - 1) / ((size_t)BLOCK * UNROLL);
+        size_t blocks = ((n >> 2) + BLOCK - 1) / BLOCK;
         if (blocks == 0) blocks = 1;
-        hipLaunchKernelGGL((binary_flat_vec4<OP, MA, MB, UNROLL>), dim3((unsigned)blocks), dim3(BLOCK),
-                           0, s, out, a, b, n);
+        if (nt)
+            hipLaunchKernelGGL((binary_flat_vec4<OP, MA, MB, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s,
+                               out, a, b, n);
+        else
+            hipLaunchKernelGGL((binary_flat_vec4<OP, MA, MB, false>), dim3((unsigned)blocks), dim3(BLOCK), 0, s,
+                               out, a, b, n);
     } else {
         const size_t blocks = (n + BLOCK - 1) / BLOCK;
-        hipLaunchKernelGGL((binary_flat_scalar<OP, MA, MB>), dim3((unsigned)blocks), dim3(BLOCK), 0, s,
-                           out, a, b, n);
+        hipLaunchKernelGGL((binary_flat_scalar<OP, MA, MB>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, a,
+                           b, n);
     }
 }
 
 template <class OP>
-void flat_launch(hipStream_t s, int ma, int mb, float *out, const float *a, const float *b, size_t n,
-                 bool vec) {
-    if (ma == FULL && mb == FULL) flat_dispatch<OP, FULL, FULL>(s, out, a, b, n, vec);
-    else if (ma == FULL && mb == SCALAR) flat_dispatch<OP, FULL, SCALAR>(s, out, a, b, n, vec);
-    else if (ma == SCALAR && mb == FULL) flat_dispatch<OP, SCALAR, FULL>(s, out, a, b, n, vec);
-    else flat_dispatch<OP, SCALAR, SCALAR>(s, out, a, b, n, vec);
+void flat_launch(hipStream_t s, int ma, int mb, float *out, const float *a, const float *b, size_t n, bool vec,
+                 bool nt) {
+    if (ma == FULL && mb == FULL) flat_dispatch<OP, FULL, FULL>(s, out, a, b, n, vec, nt);
+    else if (ma == FULL && mb == SCALAR) flat_dispatch<OP, FULL, SCALAR>(s, out, a, b, n, vec, nt);
+    else if (ma == SCALAR && mb == FULL) flat_dispatch<OP, SCALAR, FULL>(s, out, a, b, n, vec, nt);
+    else flat_dispatch<OP, SCALAR, SCALAR>(s, out, a, b, n, vec, nt);
 }
 
 template <class OP, int RANK>
-void strided_dispatch(hipStream_t s, float *out, const float *a, const float *b, uint32_t n,
-                      const Geom &g, bool vec) {
+void strided_dispatch(hipStream_t s, float *out, const float *a, const float *b, uint32_t n, const Geom &g,
+                      bool vec, bool nt) {
     if (vec) {
         const uint32_t nvec = (n + 3) / 4;
-        hipLaunchKernelGGL((binary_strided<OP, RANK, 4>), dim3((nvec + BLOCK - 1) / BLOCK), dim3(BLOCK),
-                           0, s, out, a, b, n, g);
+        const dim3 grid((nvec + BLOCK - 1) / BLOCK);
+        if (nt)
+            hipLaunchKernelGGL((binary_strided<OP, RANK, 4, true>), grid, dim3(BLOCK), 0, s, out, a, b, n, g);
+        else
+            hipLaunchKernelGGL((binary_strided<OP, RANK, 4, false>), grid, dim3(BLOCK), 0, s, out, a, b, n, g);
     } else {
-        hipLaunchKernelGGL((binary_strided<OP, RANK, 1>), dim3((n + BLOCK - 1) / BLOCK), dim3(BLOCK), 0,
+        hipLaunchKernelGGL((binary_strided<OP, RANK, 1, false>), dim3((n + BLOCK - 1) / BLOCK), dim3(BLOCK), 0,
                            s, out, a, b, n, g);
     }
 }
 
 template <class OP>
 void strided_launch(hipStream_t s, int rank, float *out, const float *a, const float *b, uint32_t n,
-                    const Geom &g, bool vec) {
-    if (rank <= 2) strided_dispatch<OP, 2>(s, out, a, b, n, g, vec);
-    else if (rank == 3) strided_dispatch<OP, 3>(s, out, a, b, n, g, vec);
-    else if (rank == 4) strided_dispatch<OP, 4>(s, out, a, b, n, g, vec);
-    else strided_dispatch<OP, MAX_RANK>(s, out, a, b, n, g, vec);
+                    const Geom &g, bool vec, bool nt) {
+    if (rank <= 2) strided_dispatch<OP, 2>(s, out, a, b, n, g, vec, nt);
+    else if (rank == 3) strided_dispatch<OP, 3>(s, out, a, b, n, g, vec, nt);
+    else if (rank == 4) strided_dispatch<OP, 4>(s, out, a, b, n, g, vec, nt);
+    else strided_dispatch<OP, MAX_RANK>(s, out, a, b, n, g, vec, nt);
 }
 
 }  // namespace
@@ -342,16 +332,18 @@ int launch_binary(DeviceCtx &ctx, int op, float *out, const float *a, const floa
     const bool square = op == AHIP_POW && mb == SCALAR && ma != SCALAR;
 
     hipStream_t s = ctx.stream;
+    if (total > ((size_t)1 << 38)) return ctx.fail(AHIP_ERR_UNSUPPORTED, "binary: more than 2^38 elements");
+    const bool nt = ctx.streaming(total * sizeof(float));
     if (ma != STRIDED && mb != STRIDED) {
         const bool vec = aligned16(out) && (ma != FULL || aligned16(a)) && (mb != FULL || aligned16(b));
         switch (op) {
-        case AHIP_ADD: flat_launch<OpAdd>(s, ma, mb, out, a, b, total, vec); break;
-        case AHIP_SUB: flat_launch<OpSub>(s, ma, mb, out, a, b, total, vec); break;
-        case AHIP_MUL: flat_launch<OpMul>(s, ma, mb, out, a, b, total, vec); break;
-        case AHIP_DIV: flat_launch<OpDiv>(s, ma, mb, out, a, b, total, vec); break;
+        case AHIP_ADD: flat_launch<OpAdd>(s, ma, mb, out, a, b, total, vec, nt); break;
+        case AHIP_SUB: flat_launch<OpSub>(s, ma, mb, out, a, b, total, vec, nt); break;
+        case AHIP_MUL: flat_launch<OpMul>(s, ma, mb, out, a, b, total, vec, nt); break;
+        case AHIP_DIV: flat_launch<OpDiv>(s, ma, mb, out, a, b, total, vec, nt); break;
         case AHIP_POW:
-            if (square) flat_launch<OpPowScalarExp>(s, ma, mb, out, a, b, total, vec);
-            else flat_launch<OpPow>(s, ma, mb, out, a, b, total, vec);
+            if (square) flat_launch<OpPowScalarExp>(s, ma, mb, out, a, b, total, vec, nt);
+            else flat_launch<OpPow>(s, ma, mb, out, a, b, total, vec, nt);
             break;
         }
         return ctx.check(hipGetLastError(), "binary flat launch");
@@ -369,18 +361,18 @@ int launch_binary(DeviceCtx &ctx, int op, float *out, const float *a, const floa
 
     Geom g;
     for (int d = 0; d < MAX_RANK; d++) {
-        g.dims[d] = 1;
+        g.dims[d] = make_fastdiv(1);
         g.a_str[d] = g.b_str[d] = 0;
     }
     for (int d = 0; d < r; d++) {  // reverse: innermost first
-        g.dims[d] = (uint32_t)dims[r - 1 - d];
+        g.dims[d] = make_fastdiv((uint32_t)dims[r - 1 - d]);
         g.a_str[d] = (uint32_t)as[r - 1 - d];
         g.b_str[d] = (uint32_t)bs[r - 1 - d];
     }
     g.mode_a = ma;
     g.mode_b = mb;
     auto vec_ok = [&](const float *p, const uint32_t *st) {
-        if (!aligned16(p) || st[0] != 1 || (g.dims[0] & 3)) return 0;
+        if (!aligned16(p) || st[0] != 1 || (g.dims[0].d & 3)) return 0;
         for (int d = 1; d < r; d++)
             if (st[d] & 3) return 0;
         return 1;
@@ -395,24 +387,26 @@ int launch_binary(DeviceCtx &ctx, int op, float *out, const float *a, const floa
         const size_t o1 = o0 + rows_per_launch < outer ? o0 + rows_per_launch : outer;
         const uint32_t n = (uint32_t)((o1 - o0) * inner_elems);
         Geom gl = g;
-        gl.dims[r - 1] = (uint32_t)(o1 - o0);
+        gl.dims[r - 1] = make_fastdiv((uint32_t)(o1 - o0));
         float *po = out + o0 * inner_elems;
         const float *pa = a + o0 * (size_t)as[0];
         const float *pb = b + o0 * (size_t)bs[0];
-        const bool vec = aligned16(po) && (ma != FULL || aligned16(pa)) && (mb != FULL || aligned16(pb));
+        // Four elements per lane need an innermost extent of at least 4 (one row change at most).
+        const bool vec = aligned16(po) && (ma != FULL || aligned16(pa)) && (mb != FULL || aligned16(pb)) &&
+                         gl.dims[0].d >= 4;
         if (!vec) gl.a_vec = gl.b_vec = 0;
         else {
             gl.a_vec = g.a_vec && aligned16(pa);
             gl.b_vec = g.b_vec && aligned16(pb);
         }
         switch (op) {
-        case AHIP_ADD: strided_launch<OpAdd>(s, r, po, pa, pb, n, gl, vec); break;
-        case AHIP_SUB: strided_launch<OpSub>(s, r, po, pa, pb, n, gl, vec); break;
-        case AHIP_MUL: strided_launch<OpMul>(s, r, po, pa, pb, n, gl, vec); break;
-        case AHIP_DIV: strided_launch<OpDiv>(s, r, po, pa, pb, n, gl, vec); break;
+        case AHIP_ADD: strided_launch<OpAdd>(s, r, po, pa, pb, n, gl, vec, nt); break;
+        case AHIP_SUB: strided_launch<OpSub>(s, r, po, pa, pb, n, gl, vec, nt); break;
+        case AHIP_MUL: strided_launch<OpMul>(s, r, po, pa, pb, n, gl, vec, nt); break;
+        case AHIP_DIV: strided_launch<OpDiv>(s, r, po, pa, pb, n, gl, vec, nt); break;
         case AHIP_POW:
-            if (square) strided_launch<OpPowScalarExp>(s, r, po, pa, pb, n, gl, vec);
-            else strided_launch<OpPow>(s, r, po, pa, pb, n, gl, vec);
+            if (square) strided_launch<OpPowScalarExp>(s, r, po, pa, pb, n, gl, vec, nt);
+            else strided_launch<OpPow>(s, r, po, pa, pb, n, gl, vec, nt);
             break;
         }
     }

@@ -21,7 +21,11 @@ struct DeviceCtx {
     // Partial results of two-stage reductions (device memory, owned).
     float *scratch = nullptr;
     size_t scratch_floats = 0;
+    // Tensors of at least this many bytes are streamed with non-temporal accesses.
+    size_t nt_threshold_bytes = (size_t)128 << 20;
     std::string last_error;
+
+    bool streaming(size_t bytes) const { return bytes >= nt_threshold_bytes; }
 
     int fail(int code, const std::string &msg);
     int check(hipError_t e, const char *what);

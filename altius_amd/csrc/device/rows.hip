@@ -20,6 +20,7 @@
 #include "math.h"
 
 #include <math.h>
+#include <stdlib.h>
 
 namespace altius {
 namespace {
@@ -112,6 +113,104 @@ __global__ __launch_bounds__(BLOCK) void softmax_wave(float *__restrict__ out, c
 #pragma unroll
     for (int s = 0; s < NCH * VEC; s++) r.v[s] *= recip;
     r.store(o, len, lane);
+}
+
+// Rows whose length is not a multiple of 4 (197 tokens, say) start at addresses
+// that are only 4-byte aligned, and a wave per row would leave a quarter of its
+// lanes idle in the last chunk.  This kernel decouples the two layouts through
+// LDS.  One wavefront per block takes a group of G consecutive rows (G a
+// multiple of 4, so the group is a 16-byte aligned, contiguous span):
+//   1. the span is copied to LDS with 16-byte loads, every lane busy;
+//   2. rows are processed from LDS with SUB = 16, 32 or 64 lanes per row
+//      (64/SUB rows at a time), NCH chunks per lane, max and sum all-reduced
+//      inside each lane group with DPP rotations; results overwrite the row;
+//   3. the span is written back with 16-byte stores.
+// With SUB*NCH just above the row length nearly every lane slot of the
+// arithmetic does useful work (197 -> 16 x 13 = 208 slots).
+constexpr int STAGE = 16;                            // float4 per lane staged through registers
+constexpr size_t LDS_GROUP_FLOATS = STAGE * WAVE * 4;  // so a group holds at most 4096 floats
+
+template <int SUB, int NCH>
+__global__ __launch_bounds__(WAVE) void softmax_lds(float *__restrict__ out, const float *__restrict__ in,
+                                                    size_t rows, int len, int group_rows, int nt) {
+    extern __shared__ __align__(16) float lds[];
+    const int lane = threadIdx.x;
+    const size_t row0 = (size_t)blockIdx.x * group_rows;
+    const int nrows = rows - row0 < (size_t)group_rows ? (int)(rows - row0) : group_rows;
+    const int n = nrows * len;
+    const int n4 = n >> 2;
+    const float *src = in + row0 * (size_t)len;
+    float *dst = out + row0 * (size_t)len;
+
+    // All of the group's loads are issued before the first LDS write, so one
+    // wave keeps up to STAGE KiB in flight.
+    float4 stage[STAGE];
+    if (nt) {
+#pragma unroll
+        for (int u = 0; u < STAGE; u++)
+            if (lane + WAVE * u < n4) stage[u] = load4<true>(src + 4 * (lane + WAVE * u));
+    } else {
+#pragma unroll
+        for (int u = 0; u < STAGE; u++)
+            if (lane + WAVE * u < n4) stage[u] = load4<false>(src + 4 * (lane + WAVE * u));
+    }
+#pragma unroll
+    for (int u = 0; u < STAGE; u++)
+        if (lane + WAVE * u < n4) *reinterpret_cast<float4 *>(lds + 4 * (lane + WAVE * u)) = stage[u];
+    for (int i = (n4 << 2) + lane; i < n; i += WAVE) lds[i] = src[i];  // ragged end of the last group
+    __syncthreads();
+
+    constexpr int RPP = WAVE / SUB;  // rows per pass
+    const int s = lane & (SUB - 1);
+    const int rr = lane / SUB;
+    const float nan = __builtin_nanf("");
+    for (int r0 = 0; r0 < nrows; r0 += RPP) {
+        int r = r0 + rr;
+        const bool active = r < nrows;
+        if (!active) r = nrows - 1;  // idle lane groups recompute the last row and store nothing
+        float *row = lds + r * len + s;
+
+        float x[NCH];
+        float mx = nan;
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            const bool full = SUB * (k + 1) <= len;  // uniform
+            x[k] = (full || s + SUB * k < len) ? row[SUB * k] : nan;
+            mx = nanmax(x[k], mx);
+        }
+        mx = subwave_allreduce<MaxOp, SUB>(mx);
+
+        float sum = 0.0f;
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            const bool full = SUB * (k + 1) <= len;
+            const float e = softmax_exp(x[k], mx);
+            x[k] = e;
+            sum += (full || s + SUB * k < len) ? e : 0.0f;
+        }
+        sum = subwave_allreduce<SumOp, SUB>(sum);
+        const float recip = 1.0f / sum;
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            const bool full = SUB * (k + 1) <= len;
+            if (active && (full || s + SUB * k < len)) row[SUB * k] = x[k] * recip;
+        }
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int u = 0; u < STAGE; u++)
+        if (lane + WAVE * u < n4) stage[u] = *reinterpret_cast<const float4 *>(lds + 4 * (lane + WAVE * u));
+    if (nt) {
+#pragma unroll
+        for (int u = 0; u < STAGE; u++)
+            if (lane + WAVE * u < n4) store4<true>(dst + 4 * (lane + WAVE * u), stage[u]);
+    } else {
+#pragma unroll
+        for (int u = 0; u < STAGE; u++)
+            if (lane + WAVE * u < n4) store4<false>(dst + 4 * (lane + WAVE * u), stage[u]);
+    }
+    for (int i = (n4 << 2) + lane; i < n; i += WAVE) dst[i] = lds[i];
 }
 
 // One block per row, any length: max pass, sum pass, write pass.
@@ -245,6 +344,40 @@ template <int VEC, int NCH> struct LayerNormLauncher {
     }
 };
 
+// Launches softmax_lds with the lane-group width and chunk count that waste the
+// fewest lane slots for this row length (len <= 1024).
+template <int SUB> bool softmax_lds_launch_nch(int nch, dim3 grid, size_t shmem, hipStream_t s, float *out,
+                                               const float *in, size_t rows, int len, int g, int nt) {
+#define ALTIUS_CASE(N)                                                                                         \
+    case N:                                                                                                    \
+        hipLaunchKernelGGL((softmax_lds<SUB, N>), grid, dim3(WAVE), shmem, s, out, in, rows, len, g, nt);      \
+        return true;
+    switch (nch) {
+        ALTIUS_CASE(1) ALTIUS_CASE(2) ALTIUS_CASE(3) ALTIUS_CASE(4) ALTIUS_CASE(5) ALTIUS_CASE(6) ALTIUS_CASE(7)
+        ALTIUS_CASE(8) ALTIUS_CASE(9) ALTIUS_CASE(10) ALTIUS_CASE(11) ALTIUS_CASE(12) ALTIUS_CASE(13)
+        ALTIUS_CASE(14) ALTIUS_CASE(15) ALTIUS_CASE(16)
+    }
+#undef ALTIUS_CASE
+    return false;
+}
+
+bool softmax_lds_launch(hipStream_t s, float *out, const float *in, size_t rows, size_t len, bool nt) {
+    // Rows per group: a multiple of 4 (16-byte aligned groups, whole passes), about 12 KiB of LDS.
+    static const size_t target = getenv("AHIP_EXP_GROUP_FLOATS") ? (size_t)atoi(getenv("AHIP_EXP_GROUP_FLOATS")) : 3200;
+    size_t g = target / len / 4 * 4;
+    if (g < 4) g = 4;  // len <= 1024, so 4 rows still fit LDS_GROUP_FLOATS
+    if (g > 512) g = 512;
+    static_assert(4 * 1024 <= LDS_GROUP_FLOATS, "a group of 4 rows must fit the staging registers");
+    const size_t groups = (rows + g - 1) / g;
+    if (groups > 0x7FFFFFFFu) return false;
+    const dim3 grid((unsigned)groups);
+    const size_t shmem = g * len * sizeof(float);
+    const int L = (int)len, G = (int)g, NT = nt ? 1 : 0;
+    if (len <= 256) return softmax_lds_launch_nch<16>((L + 15) / 16, grid, shmem, s, out, in, rows, L, G, NT);
+    if (len <= 512) return softmax_lds_launch_nch<32>((L + 31) / 32, grid, shmem, s, out, in, rows, L, G, NT);
+    return softmax_lds_launch_nch<64>((L + 63) / 64, grid, shmem, s, out, in, rows, L, G, NT);
+}
+
 constexpr size_t MAX_WAVE_ROW = 1024;
 constexpr size_t MAX_GRID = 0x7FFFFFFFu;
 
@@ -256,9 +389,18 @@ int launch_softmax(DeviceCtx &ctx, float *out, const float *in, size_t rows, siz
     if (len <= MAX_WAVE_ROW) {
         if ((rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK > MAX_GRID)
             return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: too many rows for one launch");
-        const bool vec4 = (len % 4 == 0) && aligned16(out) && aligned16(in);
-        if (!dispatch_wave<SoftmaxLauncher>(vec4, len, ctx.stream, out, in, rows, (int)len))
+        const bool aligned = aligned16(out) && aligned16(in);
+        const bool vec4 = (len % 4 == 0) && aligned;
+        // A wave per row with 16-byte accesses is ideal when the row fills (most of) the wave's
+        // 256-element chunks; otherwise go through LDS, which needs aligned buffers only.
+        const size_t slots = (len + 255) / 256 * 256;
+        const bool wave_fits = vec4 && len * 4 >= slots * 3;
+        if (aligned && !wave_fits) {
+            if (!softmax_lds_launch(ctx.stream, out, in, rows, len, ctx.streaming(rows * len * sizeof(float))))
+                return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: too many rows for one launch");
+        } else if (!dispatch_wave<SoftmaxLauncher>(vec4, len, ctx.stream, out, in, rows, (int)len)) {
             return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: no wave layout for this row length");
+        }
     } else {
         if (rows > MAX_GRID) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: too many rows for one launch");
         hipLaunchKernelGGL(softmax_block_stream, dim3((unsigned)rows), dim3(BLOCK), 0, ctx.stream, out, in,

@@ -1,6 +1,6 @@
 // Flat unary ops (Sqrt/Erf/Gelu/Sigmoid/HardSigmoid/Relu) for gfx950.
-// One 16-byte load and one 16-byte store per lane and step, UNROLL steps per
-// lane, block-contiguous.  Per-element formulas are in math.h.
+// One 16-byte load and one 16-byte store per lane.  Per-element formulas are in
+// math.h.
 //
 // Reference: crates/session_interpreter/src/session.rs:608-619, 796-838,
 // 905-931 and crates/session_interpreter/src/fast_math.rs.
@@ -28,32 +28,25 @@ struct FHardSigmoid {
 
 constexpr int BLOCK = 256;
 
-template <class F, int UNROLL>
+// One float4 per lane: on this part a streaming kernel is fastest with the
+// smallest per-lane footprint and the occupancy that comes with it.
+template <class F, bool NT>
 __global__ __launch_bounds__(BLOCK) void unary_vec4(float *__restrict__ out, const float *__restrict__ in,
                                                     size_t n, F f) {
     const size_t n4 = n >> 2;
-    const size_t base = (size_t)blockIdx.x * (BLOCK * UNROLL) + threadIdx.x;
-    float4 v[UNROLL];
-#pragma unroll
-    for (int u = 0; u < UNROLL; u++) {
-        const size_t i = base + (size_t)u * BLOCK;
-        if (i < n4) v[u] = reinterpret_cast<const float4 *>(in)[i];
-    }
-#pragma unroll
-    for (int u = 0; u < UNROLL; u++) {
-        const size_t i = base + (size_t)u * BLOCK;
-        if (i < n4) {
-            float4 r;
-            r.x = f(v[u].x);
-            r.y = f(v[u].y);
-            r.z = f(v[u].z);
-            r.w = f(v[u].w);
-            reinterpret_cast<float4 *>(out)[i] = r;
-        }
+    const size_t i = (size_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (i < n4) {
+        const float4 v = load4<NT>(in + 4 * i);
+        float4 r;
+        r.x = f(v.x);
+        r.y = f(v.y);
+        r.z = f(v.z);
+        r.w = f(v.w);
+        store4<NT>(out + 4 * i, r);
     }
     if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
-        const size_t i = (n4 << 2) + threadIdx.x;
-        out[i] = f(in[i]);
+        const size_t j = (n4 << 2) + threadIdx.x;
+        out[j] = f(in[j]);
     }
 }
 
@@ -64,13 +57,15 @@ __global__ __launch_bounds__(BLOCK) void unary_scalar(float *__restrict__ out, c
     if (i < n) out[i] = f(in[i]);
 }
 
-template <class F> void launch(hipStream_t s, float *out, const float *in, size_t n, F f) {
+template <class F> void launch(hipStream_t s, float *out, const float *in, size_t n, F f, bool nt) {
     const bool vec = ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(in)) & 15u) == 0;
     if (vec) {
-        constexpr int UNROLL = 4;
-        size_t blocks = ((n >> 2) + (size_t)BLOCK * UNROLL - 1) / ((size_t)BLOCK * UNROLL);
+        size_t blocks = ((n >> 2) + BLOCK - 1) / BLOCK;
         if (blocks == 0) blocks = 1;
-        hipLaunchKernelGGL((unary_vec4<F, UNROLL>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, n, f);
+        if (nt)
+            hipLaunchKernelGGL((unary_vec4<F, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, n, f);
+        else
+            hipLaunchKernelGGL((unary_vec4<F, false>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, n, f);
     } else {
         hipLaunchKernelGGL((unary_scalar<F>), dim3((unsigned)((n + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, s,
                            out, in, n, f);
@@ -83,14 +78,15 @@ int launch_unary(DeviceCtx &ctx, int op, float *out, const float *in, size_t n, 
     if (op < AHIP_SQRT || op > AHIP_RELU) return ctx.fail(AHIP_ERR_ARG, "unary: unknown op");
     if (n == 0) return AHIP_OK;
     if (!out || !in) return ctx.fail(AHIP_ERR_ARG, "unary: null tensor pointer");
-    if (n > ((size_t)1 << 40)) return ctx.fail(AHIP_ERR_UNSUPPORTED, "unary: more than 2^40 elements");
+    if (n > ((size_t)1 << 38)) return ctx.fail(AHIP_ERR_UNSUPPORTED, "unary: more than 2^38 elements");
+    const bool nt = ctx.streaming(n * sizeof(float));
     switch (op) {
-    case AHIP_SQRT: launch(ctx.stream, out, in, n, FSqrt{}); break;
-    case AHIP_ERF: launch(ctx.stream, out, in, n, FErf{}); break;
-    case AHIP_GELU: launch(ctx.stream, out, in, n, FGelu{}); break;
-    case AHIP_SIGMOID: launch(ctx.stream, out, in, n, FSigmoid{}); break;
-    case AHIP_HARDSIGMOID: launch(ctx.stream, out, in, n, FHardSigmoid{alpha, beta}); break;
-    case AHIP_RELU: launch(ctx.stream, out, in, n, FRelu{}); break;
+    case AHIP_SQRT: launch(ctx.stream, out, in, n, FSqrt{}, nt); break;
+    case AHIP_ERF: launch(ctx.stream, out, in, n, FErf{}, nt); break;
+    case AHIP_GELU: launch(ctx.stream, out, in, n, FGelu{}, nt); break;
+    case AHIP_SIGMOID: launch(ctx.stream, out, in, n, FSigmoid{}, nt); break;
+    case AHIP_HARDSIGMOID: launch(ctx.stream, out, in, n, FHardSigmoid{alpha, beta}, nt); break;
+    case AHIP_RELU: launch(ctx.stream, out, in, n, FRelu{}, nt); break;
     }
     return ctx.check(hipGetLastError(), "unary launch");
 }

@@ -1,0 +1,273 @@
+#!/usr/bin/env python3
+"""Benchmark of the interpreter tensor kernels on one MI355X.
+
+Workload (BASELINE.json configs[4], the configuration the >= 70 %-of-HBM target is quoted on):
+one "step" is one pass of the four kernels over device-resident fp32 inputs
+
+    Add      scores[256,12,197,197] + mask[256,1,1,197]
+    Softmax  over the last axis of that sum
+    ReduceMax over axis 1 of [256,768,197]
+    Div      [256,197,768] / scalar
+
+`value` is the whole step's algorithmic bytes (every tensor read or written once) divided by
+the step time, in GB/s.  Per-kernel times are measured with HIP events on the stream the
+kernels run on; `roofline` describes the slowest kernel of the step.  The CPU baseline is the
+oracle (a C++ restatement of the reference interpreter's kernels) timed on this machine's host
+cores on a reduced batch of the same workload.
+
+Prints one JSON line on stdout; a per-kernel table goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def ensure_built():
+    from altius_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        from altius_amd import build
+
+        log("libaltius_hip.so missing: building")
+        build.build()
+
+
+class Op:
+    """One kernel launch on fixed device buffers, with its algorithmic byte count."""
+
+    def __init__(self, name, nbytes, launchers):
+        self.name = name
+        self.nbytes = nbytes
+        self.launchers = launchers  # one closure per rotated buffer set
+        self.i = 0
+
+    def launch(self):
+        self.launchers[self.i % len(self.launchers)]()
+        self.i += 1
+
+
+def build_cfg4(ctx, D, synth, batch, rotate_bytes):
+    """Uploads configs[4] at the given batch and returns the four ops of a step."""
+    c = synth.cfg4(batch=batch)
+    ops = []
+
+    def copies(nbytes_per_set):
+        return max(1, min(4, int(np.ceil(rotate_bytes / max(nbytes_per_set, 1)))))
+
+    # Add (mask)
+    scores, mask = c["scores"], c["mask"]
+    out_dims = list(scores.shape)
+    a_str = D.strides_for_broadcasting(scores.shape, out_dims)
+    b_str = D.strides_for_broadcasting(mask.shape, out_dims)
+    d_scores = ctx.upload(scores)
+    d_mask = ctx.upload(mask)
+    d_sum = ctx.alloc(scores.nbytes)
+    add_bytes = 2 * scores.nbytes + mask.nbytes
+    ops.append(Op("Add(mask) [%d,12,197,197]+[%d,1,1,197]" % (batch, batch), add_bytes,
+                  [lambda: ctx.binary_raw(D.ADD, d_sum.ptr, d_scores.ptr, d_mask.ptr, out_dims, a_str, b_str)]))
+
+    # Softmax on the sum
+    d_prob = ctx.alloc(scores.nbytes)
+    rows = scores.size // 197
+    ops.append(Op("Softmax(-1) [%d,12,197,197]" % batch, 2 * scores.nbytes,
+                  [lambda: ctx.softmax_raw(d_prob.ptr, d_sum.ptr, rows, 197)]))
+
+    # ReduceMax over axis 1; inputs rotated so that repeated launches do not hit the Infinity Cache
+    x = c["rmax_in"]
+    rmax_bytes = x.nbytes + batch * 197 * 4
+    d_out = ctx.alloc(batch * 197 * 4)
+    ins = [ctx.upload(x) for _ in range(copies(rmax_bytes))]
+    ops.append(Op("ReduceMax(axis=1) [%d,768,197]" % batch, rmax_bytes,
+                  [(lambda p=b.ptr: ctx.reduce_raw(D.REDUCE_MAX, d_out.ptr, p, batch, 768, 197)) for b in ins]))
+
+    # Div by a scalar
+    y = c["div_in"]
+    d_scalar = ctx.upload(np.array([c["div_scalar"]], np.float32))
+    div_bytes = 2 * y.nbytes + 4
+    n_sets = copies(div_bytes)
+    ins = [ctx.upload(y) for _ in range(n_sets)]
+    outs = [ctx.alloc(y.nbytes) for _ in range(n_sets)]
+    dims = list(y.shape)
+    ys = D.strides_for_broadcasting(y.shape, dims)
+    ss = D.strides_for_broadcasting([], dims)
+    ops.append(Op("Div(scalar) [%d,197,768]" % batch, div_bytes,
+                  [(lambda i=i: ctx.binary_raw(D.DIV, outs[i].ptr, ins[i].ptr, d_scalar.ptr, dims, ys, ss))
+                   for i in range(n_sets)]))
+    return ops, c
+
+
+def time_kernel(ctx, op, iters, warmup):
+    """Average duration of one launch, in ms, from HIP events around `iters` back-to-back launches."""
+    for _ in range(warmup):
+        op.launch()
+    start, stop = ctx.event(), ctx.event()
+    ctx.sync()
+    ctx.record(start)
+    for _ in range(iters):
+        op.launch()
+    ctx.record(stop)
+    ms = ctx.elapsed_ms(start, stop) / iters
+    ctx.destroy_event(start)
+    ctx.destroy_event(stop)
+    return ms
+
+
+def cpu_baseline(synth, batch_full, sample_batch, threads):
+    """Times the oracle on a reduced batch of the same step; returns GB/s and per-op seconds."""
+    import oracle as O
+
+    O.lib()
+    c = synth.cfg4(batch=sample_batch)
+    times = {}
+    total_bytes = 0
+
+    def timed(name, nbytes, fn, reps=2):
+        nonlocal total_bytes
+        best = float("inf")
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            best = min(best, time.perf_counter() - t0)
+        times[name] = best
+        total_bytes += nbytes
+
+    scores, mask = c["scores"], c["mask"]
+    z = {}
+    timed("Add", 2 * scores.nbytes + mask.nbytes, lambda: z.__setitem__("z", O.binary(O.ADD, scores, mask, threads=threads)))
+    out = np.empty_like(scores)
+    timed("Softmax", 2 * scores.nbytes, lambda: O.softmax(z["z"], threads=threads, out=out))
+    x = c["rmax_in"]
+    timed("ReduceMax", x.nbytes + sample_batch * 197 * 4, lambda: O.reduce(O.REDUCE_MAX, x, [1], False))
+    y = c["div_in"]
+    s = np.array(c["div_scalar"], np.float32)
+    timed("Div", 2 * y.nbytes + 4, lambda: O.binary(O.DIV, y, s, threads=threads))
+    total_s = sum(times.values())
+    return total_bytes / total_s / 1e9, times
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=256, help="batch of configs[4] (256 = the named workload)")
+    ap.add_argument("--kernel-iters", type=int, default=50, help="launches per kernel for the per-kernel timing")
+    ap.add_argument("--cpu-sample-batch", type=int, default=32, help="batch of the CPU baseline sample")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", type=str, default="", help="run only kernels whose name contains this text (profiling)")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        log("bench.py: this build runs on one GPU only (the path shards without communication; "
+            "see DESIGN.md); run with --gpus 1")
+        sys.exit(2)
+
+    ensure_built()
+    from altius_amd import device as D
+    from altius_amd import synth
+
+    ctx = D.Context(0)
+    ops, _ = build_cfg4(ctx, D, synth, args.batch, rotate_bytes=600e6)
+    if args.only:
+        ops = [o for o in ops if args.only.lower() in o.name.lower()]
+    ctx.sync()
+
+    # --- whole step: W warm-up steps, then exactly K timed steps --------------------------------
+    for _ in range(args.warmup):
+        for o in ops:
+            o.launch()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        for o in ops:
+            o.launch()
+    ctx.sync()
+    step_s = (time.perf_counter() - t0) / args.steps
+    step_bytes = sum(o.nbytes for o in ops)
+    value = step_bytes / step_s / 1e9
+
+    # --- per kernel, HIP events on the kernels' stream -----------------------------------------
+    rows = []
+    for o in ops:
+        ms = time_kernel(ctx, o, args.kernel_iters, 5)
+        gbps = o.nbytes / (ms * 1e-3) / 1e9
+        rows.append({"kernel": o.name, "bytes": o.nbytes, "us": ms * 1e3, "GBps": gbps,
+                     "pct_hbm_peak": 100.0 * gbps / HBM_PEAK_GBPS})
+    log("%-44s %14s %10s %10s %8s" % ("kernel", "alg. bytes", "us/call", "GB/s", "% peak"))
+    for r in rows:
+        log("%-44s %14d %10.1f %10.1f %8.1f" % (r["kernel"], r["bytes"], r["us"], r["GBps"], r["pct_hbm_peak"]))
+    dom = max(rows, key=lambda r: r["us"])
+
+    result = {
+        "metric": "per-op HBM GB/s and % of MI355X peak; us/call vs CPU interpreter",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[4]: Add(mask)+Softmax on [%d,12,197,197], ReduceMax(axis=1) on [%d,768,197], "
+                        "Div(scalar) on [%d,197,768]; one step = the four kernels once" % ((args.batch,) * 3),
+            "batch": args.batch,
+            "step_bytes": step_bytes,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": dom["kernel"],
+            "achieved": round(dom["GBps"], 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "us_per_launch": round(dom["us"], 2),
+            "algorithmic_bytes": dom["bytes"],
+        },
+        "per_kernel": [{k: (round(v, 2) if isinstance(v, float) else v) for k, v in r.items()} for r in rows],
+    }
+
+    if not args.no_cpu:
+        threads = min(16, os.cpu_count() or 1)
+        gbps_n, t_n = cpu_baseline(synth, args.batch, args.cpu_sample_batch, threads)
+        gbps_1, t_1 = cpu_baseline(synth, args.batch, args.cpu_sample_batch, 1)
+        scale = args.batch / args.cpu_sample_batch
+        log("CPU oracle, batch %d sample (x%.0f for the full step): %d threads %.2f GB/s, 1 thread %.2f GB/s"
+            % (args.cpu_sample_batch, scale, threads, gbps_n, gbps_1))
+        for k in t_n:
+            log("  %-10s %d threads %9.1f us   1 thread %9.1f us  (scaled to batch %d)"
+                % (k, threads, t_n[k] * scale * 1e6, t_1[k] * scale * 1e6, args.batch))
+        result["cpu_baseline"] = {
+            "value": round(gbps_n, 2),
+            "unit": "GB/s",
+            "cores": threads,
+            "kind": "port",
+            "sample": "same four kernels at batch %d of %d (1/%d of the step), best of 2 runs; "
+                      "1 thread: %.2f GB/s" % (args.cpu_sample_batch, args.batch, int(scale), gbps_1),
+            "single_thread_value": round(gbps_1, 2),
+            "us_per_kernel_scaled": {k: round(v * scale * 1e6, 1) for k, v in t_n.items()},
+        }
+
+    ctx.close()
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()
