@@ -174,6 +174,93 @@ __global__ __launch_bounds__(COL_BLOCK) void reduce_cols(float *__restrict__ dst
     }
 }
 
+// The same reduction with 16-byte loads, for inner extents up to 256 that are
+// not multiples of 4 (197, say), where rows are only 4-byte aligned.  Four
+// consecutive rows are `inner` float4 that start 16-byte aligned, and because
+// the group is exactly four rows long, float4 number f of every group holds the
+// same four (row-in-group, column) positions.  So a lane accumulates float4
+// number lane + 64k of group after group element by element, and only at the end
+// do the 4*inner accumulators go through LDS, where column c collects positions
+// c, c + inner, c + 2*inner, c + 3*inner of every wave.  Rows left over when the
+// reduced extent is not a multiple of 4 are folded in by the last split.
+// grid = (outer * splits); dynamic LDS = COL_WAVES * 4 * inner floats.
+template <class OP, int NCH, bool SCALE, bool NT>
+__global__ __launch_bounds__(COL_BLOCK) void reduce_cols_flat4(float *__restrict__ dst,
+                                                               const float *__restrict__ in, uint32_t red,
+                                                               uint32_t inner, uint32_t splits,
+                                                               uint32_t groups_per_split, float scale) {
+    extern __shared__ __align__(16) float lds4[];
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x >> 6;
+    const uint32_t o = blockIdx.x / splits, s = blockIdx.x % splits;
+    const uint32_t ngroups = red >> 2;
+    const uint32_t g_begin = s * groups_per_split;
+    uint32_t g_end = g_begin + groups_per_split;
+    if (g_end > ngroups) g_end = ngroups;
+    const float *slab = in + (size_t)o * red * inner;
+    const size_t group_floats = (size_t)4 * inner;
+
+    float4 acc[NCH];
+#pragma unroll
+    for (int k = 0; k < NCH; k++) acc[k] = make_float4(OP::identity(), OP::identity(), OP::identity(), OP::identity());
+
+    uint32_t g = g_begin + wave;
+    for (; g + COL_WAVES < g_end; g += 2 * COL_WAVES) {  // two groups in flight
+        const float *p0 = slab + g * group_floats;
+        const float *p1 = p0 + COL_WAVES * group_floats;
+        float4 v0[NCH], v1[NCH];
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            const uint32_t f = lane + WAVE * k;
+            if (f < inner) {
+                v0[k] = load4<NT>(p0 + 4 * f);
+                v1[k] = load4<NT>(p1 + 4 * f);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            const uint32_t f = lane + WAVE * k;
+            if (f < inner) {
+                acc[k].x = OP::apply(OP::apply(acc[k].x, v0[k].x), v1[k].x);
+                acc[k].y = OP::apply(OP::apply(acc[k].y, v0[k].y), v1[k].y);
+                acc[k].z = OP::apply(OP::apply(acc[k].z, v0[k].z), v1[k].z);
+                acc[k].w = OP::apply(OP::apply(acc[k].w, v0[k].w), v1[k].w);
+            }
+        }
+    }
+    for (; g < g_end; g += COL_WAVES) {
+        const float *p0 = slab + g * group_floats;
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            const uint32_t f = lane + WAVE * k;
+            if (f < inner) {
+                const float4 v = load4<NT>(p0 + 4 * f);
+                acc[k].x = OP::apply(acc[k].x, v.x);
+                acc[k].y = OP::apply(acc[k].y, v.y);
+                acc[k].z = OP::apply(acc[k].z, v.z);
+                acc[k].w = OP::apply(acc[k].w, v.w);
+            }
+        }
+    }
+
+    float *mine = lds4 + (size_t)wave * group_floats;
+#pragma unroll
+    for (int k = 0; k < NCH; k++) {
+        const uint32_t f = lane + WAVE * k;
+        if (f < inner) *reinterpret_cast<float4 *>(mine + 4 * f) = acc[k];
+    }
+    __syncthreads();
+    for (uint32_t c = threadIdx.x; c < inner; c += COL_BLOCK) {
+        float a = OP::identity();
+        for (int w = 0; w < COL_WAVES; w++)
+#pragma unroll
+            for (int p = 0; p < 4; p++) a = OP::apply(a, lds4[w * group_floats + p * inner + c]);
+        if (s == splits - 1)
+            for (uint32_t r = ngroups << 2; r < red; r++) a = OP::apply(a, slab[(size_t)r * inner + c]);
+        dst[(size_t)blockIdx.x * inner + c] = SCALE ? a * scale : a;
+    }
+}
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 constexpr size_t MAX_GRID_X = 0x7FFFFFFFu;
@@ -224,6 +311,30 @@ void cols_launch(hipStream_t s, float *dst, const float *in, size_t outer, size_
 }
 
 template <class OP, bool SCALE>
+void cols_flat4_launch(hipStream_t s, float *dst, const float *in, size_t outer, size_t red, size_t inner,
+                       size_t splits, size_t groups_per_split, float scale, bool nt) {
+    const dim3 grid((unsigned)(outer * splits));
+    const dim3 block(COL_BLOCK);
+    const size_t shmem = (size_t)COL_WAVES * 4 * inner * sizeof(float);
+    const int nch = (int)((inner + WAVE - 1) / WAVE);
+#define ALTIUS_LAUNCH(N, T)                                                                                    \
+    hipLaunchKernelGGL((reduce_cols_flat4<OP, N, SCALE, T>), grid, block, shmem, s, dst, in, (uint32_t)red,    \
+                       (uint32_t)inner, (uint32_t)splits, (uint32_t)groups_per_split, scale)
+    if (nt) {
+        if (nch == 1) ALTIUS_LAUNCH(1, true);
+        else if (nch == 2) ALTIUS_LAUNCH(2, true);
+        else if (nch == 3) ALTIUS_LAUNCH(3, true);
+        else ALTIUS_LAUNCH(4, true);
+    } else {
+        if (nch == 1) ALTIUS_LAUNCH(1, false);
+        else if (nch == 2) ALTIUS_LAUNCH(2, false);
+        else if (nch == 3) ALTIUS_LAUNCH(3, false);
+        else ALTIUS_LAUNCH(4, false);
+    }
+#undef ALTIUS_LAUNCH
+}
+
+template <class OP, bool SCALE>
 int reduce_impl(DeviceCtx &ctx, float *out, const float *in, size_t outer, size_t red, size_t inner,
                 float scale) {
     hipStream_t s = ctx.stream;
@@ -260,6 +371,31 @@ int reduce_impl(DeviceCtx &ctx, float *out, const float *in, size_t outer, size_
     // inner > 1
     if (red >= ((size_t)1 << 32) || inner >= ((size_t)1 << 31))
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: axis extent exceeds 32-bit index range");
+    // Unaligned rows of moderate width: the 16-byte flat variant.
+    if (inner % 4 != 0 && inner <= 256 && red >= 16 && aligned16(in) && (outer == 1 || (red * inner) % 4 == 0)) {
+        const size_t groups = red / 4;
+        size_t fsplits = 1;
+        if (outer < 1024) {
+            fsplits = (1024 + outer - 1) / outer;
+            const size_t max_splits = groups / 16 > 0 ? groups / 16 : 1;  // two groups per wave at least
+            if (fsplits > max_splits) fsplits = max_splits;
+        }
+        size_t gps = (groups + fsplits - 1) / fsplits;
+        fsplits = (groups + gps - 1) / gps;
+        const bool nt = ctx.streaming(outer * red * inner * sizeof(float));
+        if (outer * fsplits <= MAX_GRID_X) {
+            if (fsplits == 1) {
+                cols_flat4_launch<OP, SCALE>(s, out, in, outer, red, inner, 1, gps, scale, nt);
+                return ctx.check(hipGetLastError(), "reduce cols (flat4) launch");
+            }
+            if (outer * fsplits * inner <= ctx.scratch_floats) {
+                cols_flat4_launch<OP, false>(s, ctx.scratch, in, outer, red, inner, fsplits, gps, 1.0f, nt);
+                cols_launch<OP, SCALE>(s, out, ctx.scratch, outer, fsplits, inner, 1, fsplits, scale);
+                return ctx.check(hipGetLastError(), "reduce cols (flat4, two-stage) launch");
+            }
+        }
+    }
+
     const size_t cpl = inner <= 64 ? 1 : inner <= 128 ? 2 : 4;
     const size_t tiles = (inner + cpl * WAVE - 1) / (cpl * WAVE);
     if (tiles > MAX_GRID_Y) return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: inner extent too large");

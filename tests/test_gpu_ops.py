@@ -253,6 +253,12 @@ REDUCE_CASES = [
     ([2, 4000, 64], [1], False),       # split columns through scratch
     ([7, 1, 9], [1], True),
     ([6, 5], [0], False),
+    ([1, 18, 197], [1], False),        # 16-byte flat column kernel with two left-over rows
+    ([1, 17, 5], [1], False),          # the same, one left-over row, one wave of columns
+    ([2, 100, 30], [1], True),         # flat kernel, aligned slabs
+    ([3, 17, 5], [1], False),          # unaligned slabs: dword column kernel
+    ([2, 2049, 255], [1], False),      # flat kernel split over blocks, odd row count
+    ([300, 64, 6], [1], False),
 ]
 
 
