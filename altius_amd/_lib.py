@@ -75,6 +75,68 @@ def _declare(L):
     f("ahip_reduce", [c_void_p, c_int, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t])
 
 
+class OpAttrs(ctypes.Structure):
+    """ahip_op_attrs"""
+
+    _fields_ = [
+        ("axis", c_int64),
+        ("axes", c_int64 * MAX_RANK),
+        ("n_axes", ctypes.c_int32),
+        ("keep_dims", ctypes.c_int32),
+        ("alpha", c_float),
+        ("beta", c_float),
+        ("epsilon", c_float),
+        ("stash_type", c_int64),
+    ]
+
+
+def _declare_graph(L):
+    def f(name, argtypes, restype=c_int):
+        fn = getattr(L, name)
+        fn.argtypes = argtypes
+        fn.restype = restype
+
+    c_double = ctypes.c_double
+    f("ahip_op_attrs_default", [P(OpAttrs)], None)
+    f("ahip_op_name", [c_int], c_char_p)
+    f("ahip_model_new", [c_int64, P(c_void_p)])
+    f("ahip_model_clone", [c_void_p, P(c_void_p)])
+    f("ahip_model_free", [c_void_p], None)
+    f("ahip_model_new_value", [c_void_p, c_char_p, P(c_int64)])
+    f("ahip_model_new_value_shaped", [c_void_p, c_char_p, c_int, c_int, P(c_int64), P(c_int64)])
+    f("ahip_model_add_initializer", [c_void_p, c_int64, c_int, c_int, P(c_int64), c_void_p, c_size_t])
+    f("ahip_model_add_node", [c_void_p, c_int, P(OpAttrs), c_char_p, c_int, P(c_int64), c_int, P(c_int64), P(c_int64)])
+    f("ahip_model_add_input", [c_void_p, c_int64])
+    f("ahip_model_add_output", [c_void_p, c_int64])
+    f("ahip_model_lookup_named_value", [c_void_p, c_char_p, P(c_int64)])
+    f("ahip_model_graph_io", [c_void_p, c_int, P(c_int64), c_int, P(c_int)])
+    f("ahip_model_topo_sort", [c_void_p, P(c_int64), c_int, P(c_int)])
+    f("ahip_model_node_info", [c_void_p, c_int64, P(c_int), P(OpAttrs), P(c_int), P(c_int64), P(c_int), P(c_int64), c_int])
+    f("ahip_model_infer_value_shape", [c_void_p, c_int64, P(c_int), P(c_int), P(c_int64)])
+    f("ahip_model_execution_plan", [c_void_p, P(c_int64), P(c_int), c_int, P(c_int64), c_int, P(c_int), P(c_int)])
+    for name in ("ahip_fuse_layer_norm", "ahip_fuse_gelu", "ahip_fuse_fast_gelu", "ahip_eliminate_identity"):
+        f(name, [c_void_p, P(c_int)])
+    f("ahip_tensor_new", [c_int, c_int, P(c_int64), c_void_p, c_size_t, P(c_void_p)])
+    f("ahip_tensor_free", [c_void_p], None)
+    f("ahip_tensor_elem_type", [c_void_p])
+    f("ahip_tensor_rank", [c_void_p])
+    f("ahip_tensor_dims", [c_void_p, P(c_int64), c_int])
+    f("ahip_tensor_nbytes", [c_void_p], c_size_t)
+    f("ahip_tensor_data", [c_void_p], c_void_p)
+    f("ahip_session_builder_new", [c_void_p, P(c_void_p)])
+    f("ahip_session_builder_free", [c_void_p], None)
+    f("ahip_session_builder_with_intra_op_num_threads", [c_void_p, c_size_t])
+    f("ahip_session_builder_with_profiling_enabled", [c_void_p, c_int])
+    f("ahip_session_builder_with_device", [c_void_p, c_int])
+    f("ahip_session_builder_build", [c_void_p, P(c_void_p)])
+    f("ahip_session_free", [c_void_p], None)
+    f("ahip_session_run", [c_void_p, c_int, P(c_void_p), c_int, P(c_void_p), P(c_int)])
+    f("ahip_session_model", [c_void_p], c_void_p)
+    f("ahip_session_profile", [c_void_p, c_int, P(c_char_p), P(c_double), P(c_int)])
+    f("ahip_session_last_run_ms", [c_void_p, P(c_double)])
+    f("ahip_session_device_allocations", [c_void_p, P(c_size_t)])
+
+
 def lib():
     """The loaded library.  Raises if it has not been built."""
     global _lib
@@ -86,6 +148,7 @@ def lib():
             )
         L = ctypes.CDLL(LIB_PATH)
         _declare(L)
+        _declare_graph(L)
         _lib = L
     return _lib
 

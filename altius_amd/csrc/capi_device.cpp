@@ -29,34 +29,14 @@ int global_check(hipError_t e, const char *what) {
 int create_ctx(int device, hipStream_t stream, bool own_stream, ahip_ctx **out) {
     if (!out) return global_fail(AHIP_ERR_ARG, "ahip_init: null output pointer");
     *out = nullptr;
-    int n = 0;
-    int rc = global_check(hipGetDeviceCount(&n), "hipGetDeviceCount");
-    if (rc) return rc;
-    if (device < 0 || device >= n) return global_fail(AHIP_ERR_ARG, "ahip_init: no such device");
-    rc = global_check(hipSetDevice(device), "hipSetDevice");
-    if (rc) return rc;
     ahip_ctx *c = new (std::nothrow) ahip_ctx();
     if (!c) return global_fail(AHIP_ERR_OOM, "ahip_init: out of host memory");
-    c->d.device = device;
-    if (own_stream) {
-        rc = global_check(hipStreamCreateWithFlags(&c->d.stream, hipStreamNonBlocking), "hipStreamCreate");
-        if (rc) {
-            delete c;
-            return rc;
-        }
-        c->d.owns_stream = true;
-    } else {
-        c->d.stream = stream;
-    }
-    void *scratch = nullptr;
-    rc = global_check(hipMalloc(&scratch, altius::SCRATCH_FLOATS * sizeof(float)), "hipMalloc(scratch)");
+    std::string err;
+    const int rc = altius::create_device_ctx(device, stream, own_stream, &c->d, &err);
     if (rc) {
-        if (c->d.owns_stream) (void)hipStreamDestroy(c->d.stream);
         delete c;
-        return rc;
+        return global_fail(rc, "ahip_init: " + err);
     }
-    c->d.scratch = static_cast<float *>(scratch);
-    c->d.scratch_floats = altius::SCRATCH_FLOATS;
     *out = c;
     return AHIP_OK;
 }
@@ -80,14 +60,9 @@ int ahip_init_on_stream(int device, void *hip_stream, ahip_ctx **ctx) {
 
 int ahip_destroy(ahip_ctx *ctx) {
     if (!ctx) return AHIP_OK;
-    int rc = AHIP_OK;
-    if (hipSetDevice(ctx->d.device) == hipSuccess) {
-        (void)hipStreamSynchronize(ctx->d.stream);
-        if (ctx->d.scratch) rc = global_check(hipFree(ctx->d.scratch), "hipFree(scratch)");
-        if (ctx->d.owns_stream) (void)hipStreamDestroy(ctx->d.stream);
-    }
+    altius::destroy_device_ctx(&ctx->d);
     delete ctx;
-    return rc;
+    return AHIP_OK;
 }
 
 const char *ahip_last_error(ahip_ctx *ctx) { return ctx ? ctx->d.last_error.c_str() : altius::global_error(); }

@@ -1,0 +1,397 @@
+// C ABI: graph IR, analysis, fusion passes, host tensors and the session.
+#include <cstring>
+#include <new>
+#include <string>
+
+#include "../../include/altius_hip.h"
+#include "core/model.h"
+#include "core/optimize.h"
+#include "core/shape.h"
+#include "device/ctx.h"
+#include "session/hip_session.h"
+#include "session/plan.h"
+
+using namespace altius;
+
+struct ahip_model {
+    Model m;
+};
+struct ahip_tensor {
+    Tensor t;
+};
+struct ahip_session_builder {
+    Model model;
+    size_t threads = 1;
+    bool profiling = false;
+    int device = 0;
+};
+struct ahip_session {
+    std::unique_ptr<HipSession> s;
+    ahip_model view;  // what ahip_session_model hands out (a copy of the session's model)
+    std::vector<std::pair<std::string, double>> profile;
+};
+
+namespace {
+
+int fail(int code, const std::string &msg) {
+    set_global_error(msg);
+    return code;
+}
+
+bool valid_elem_type(int t) { return t >= AHIP_BOOL && t <= AHIP_I64; }
+
+Op op_from_c(int kind, const ahip_op_attrs *a) {
+    Op op(static_cast<OpKind>(kind));
+    ahip_op_attrs d;
+    ahip_op_attrs_default(&d);
+    if (!a) a = &d;
+    op.axis = a->axis;
+    op.axes.assign(a->axes, a->axes + (a->n_axes < 0 ? 0 : a->n_axes > AHIP_MAX_RANK ? AHIP_MAX_RANK : a->n_axes));
+    op.keep_dims = a->keep_dims != 0;
+    op.alpha = a->alpha;
+    op.beta = a->beta;
+    op.epsilon = a->epsilon;
+    op.stash_type = a->stash_type;
+    return op;
+}
+
+void op_to_c(const Op &op, ahip_op_attrs *a) {
+    ahip_op_attrs_default(a);
+    a->axis = op.axis;
+    a->n_axes = (int32_t)std::min<size_t>(op.axes.size(), AHIP_MAX_RANK);
+    for (int i = 0; i < a->n_axes; i++) a->axes[i] = op.axes[i];
+    a->keep_dims = op.keep_dims ? 1 : 0;
+    a->alpha = op.alpha;
+    a->beta = op.beta;
+    a->epsilon = op.epsilon;
+    a->stash_type = op.stash_type;
+}
+
+bool valid_value(const ahip_model *m, int64_t id) { return id >= 0 && (size_t)id < m->m.graph.values.size(); }
+
+template <class F> int run_pass(ahip_model *model, int *count, F pass, const char *name) {
+    if (!model) return fail(AHIP_ERR_ARG, std::string(name) + ": null model");
+    const size_t n = pass(model->m);
+    if (count) *count = (int)n;
+    return AHIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+void ahip_op_attrs_default(ahip_op_attrs *a) {
+    if (!a) return;
+    std::memset(a, 0, sizeof(*a));
+    a->axis = -1;
+    a->n_axes = 0;
+    a->keep_dims = 1;
+    a->alpha = 0.2f;
+    a->beta = 0.5f;
+    a->epsilon = 1e-5f;
+    a->stash_type = 1;
+}
+
+const char *ahip_op_name(int op_kind) { return op_kind_name(static_cast<OpKind>(op_kind)); }
+
+int ahip_model_new(int64_t opset_version, ahip_model **model) {
+    if (!model) return fail(AHIP_ERR_ARG, "ahip_model_new: null output pointer");
+    *model = new (std::nothrow) ahip_model();
+    if (!*model) return fail(AHIP_ERR_OOM, "ahip_model_new: out of host memory");
+    (*model)->m.opset_version = opset_version;
+    return AHIP_OK;
+}
+
+int ahip_model_clone(const ahip_model *model, ahip_model **copy) {
+    if (!model || !copy) return fail(AHIP_ERR_ARG, "ahip_model_clone: null argument");
+    *copy = new (std::nothrow) ahip_model(*model);
+    if (!*copy) return fail(AHIP_ERR_OOM, "ahip_model_clone: out of host memory");
+    return AHIP_OK;
+}
+
+void ahip_model_free(ahip_model *model) { delete model; }
+
+int ahip_model_new_value(ahip_model *model, const char *name, int64_t *value_id) {
+    if (!model || !value_id) return fail(AHIP_ERR_ARG, "ahip_model_new_value: null argument");
+    *value_id = (int64_t)(name ? model->m.graph.values.new_val_named(name) : model->m.graph.values.new_val());
+    return AHIP_OK;
+}
+
+int ahip_model_new_value_shaped(ahip_model *model, const char *name, int elem_type, int rank, const int64_t *dims,
+                                int64_t *value_id) {
+    if (!model || !value_id || rank < 0 || (rank && !dims) || !valid_elem_type(elem_type))
+        return fail(AHIP_ERR_ARG, "ahip_model_new_value_shaped: invalid argument");
+    std::vector<Dimension> d;
+    for (int i = 0; i < rank; i++)
+        d.push_back(dims[i] < 0 ? Dimension::Dynamic("dim" + std::to_string(i)) : Dimension::Fixed((size_t)dims[i]));
+    TypedShape ts{Dimensions(std::move(d)), static_cast<TensorElemType>(elem_type)};
+    *value_id = (int64_t)model->m.graph.values.new_val_named_and_shaped(name ? name : "", std::move(ts));
+    return AHIP_OK;
+}
+
+int ahip_model_add_initializer(ahip_model *model, int64_t value_id, int elem_type, int rank, const int64_t *dims,
+                               const void *data, size_t nbytes) {
+    if (!model || rank < 0 || (rank && !dims) || !valid_elem_type(elem_type) || !valid_value(model, value_id))
+        return fail(AHIP_ERR_ARG, "ahip_model_add_initializer: invalid argument");
+    for (int i = 0; i < rank; i++)
+        if (dims[i] < 0) return fail(AHIP_ERR_ARG, "ahip_model_add_initializer: negative dimension");
+    FixedDimensions fd = FixedDimensions::from_i64(dims, (size_t)rank);
+    const TensorElemType ty = static_cast<TensorElemType>(elem_type);
+    if (nbytes != fd.total_elems() * elem_size(ty) || (nbytes && !data))
+        return fail(AHIP_ERR_ARG, "ahip_model_add_initializer: data size does not match the shape");
+    model->m.graph.inits[(ValueId)value_id] = Tensor::from_raw(std::move(fd), ty, data, nbytes);
+    return AHIP_OK;
+}
+
+int ahip_model_add_node(ahip_model *model, int op_kind, const ahip_op_attrs *attrs, const char *name, int n_inputs,
+                        const int64_t *inputs, int n_outputs, const int64_t *outputs, int64_t *node_id) {
+    if (!model || op_kind < 0 || op_kind >= AHIP_OP_COUNT || n_inputs < 0 || n_outputs < 0 ||
+        (n_inputs && !inputs) || (n_outputs && !outputs))
+        return fail(AHIP_ERR_ARG, "ahip_model_add_node: invalid argument");
+    Node node(op_from_c(op_kind, attrs));
+    if (name) node.with_name(name);
+    for (int i = 0; i < n_inputs; i++) {
+        if (!valid_value(model, inputs[i])) return fail(AHIP_ERR_ARG, "ahip_model_add_node: unknown input value");
+        node.with_in((ValueId)inputs[i]);
+    }
+    for (int i = 0; i < n_outputs; i++) {
+        if (!valid_value(model, outputs[i])) return fail(AHIP_ERR_ARG, "ahip_model_add_node: unknown output value");
+        node.with_out((ValueId)outputs[i]);
+    }
+    const NodeId id = model->m.graph.add_node(std::move(node));
+    if (node_id) *node_id = (int64_t)id;
+    return AHIP_OK;
+}
+
+int ahip_model_add_input(ahip_model *model, int64_t value_id) {
+    if (!model || !valid_value(model, value_id)) return fail(AHIP_ERR_ARG, "ahip_model_add_input: invalid argument");
+    model->m.graph.inputs.push_back((ValueId)value_id);
+    return AHIP_OK;
+}
+
+int ahip_model_add_output(ahip_model *model, int64_t value_id) {
+    if (!model || !valid_value(model, value_id)) return fail(AHIP_ERR_ARG, "ahip_model_add_output: invalid argument");
+    model->m.graph.outputs.push_back((ValueId)value_id);
+    return AHIP_OK;
+}
+
+int ahip_model_lookup_named_value(const ahip_model *model, const char *name, int64_t *value_id) {
+    if (!model || !name || !value_id) return fail(AHIP_ERR_ARG, "ahip_model_lookup_named_value: null argument");
+    auto id = model->m.lookup_named_value(name);
+    if (!id) return fail(AHIP_ERR_ARG, std::string("no value named '") + name + "'");
+    *value_id = (int64_t)*id;
+    return AHIP_OK;
+}
+
+int ahip_model_graph_io(const ahip_model *model, int which, int64_t *value_ids, int capacity, int *n) {
+    if (!model || !n || (which != 0 && which != 1) || capacity < 0 || (capacity && !value_ids))
+        return fail(AHIP_ERR_ARG, "ahip_model_graph_io: invalid argument");
+    const auto &v = which == 0 ? model->m.graph.inputs : model->m.graph.outputs;
+    *n = (int)v.size();
+    for (int i = 0; i < capacity && i < (int)v.size(); i++) value_ids[i] = (int64_t)v[i];
+    return AHIP_OK;
+}
+
+int ahip_model_topo_sort(const ahip_model *model, int64_t *node_ids, int capacity, int *n) {
+    if (!model || !n || capacity < 0 || (capacity && !node_ids))
+        return fail(AHIP_ERR_ARG, "ahip_model_topo_sort: invalid argument");
+    const auto order = model->m.topo_sort_nodes();
+    *n = (int)order.size();
+    for (int i = 0; i < capacity && i < (int)order.size(); i++) node_ids[i] = (int64_t)order[i];
+    return AHIP_OK;
+}
+
+int ahip_model_node_info(const ahip_model *model, int64_t node_id, int *op_kind, ahip_op_attrs *attrs, int *n_inputs,
+                         int64_t *inputs, int *n_outputs, int64_t *outputs, int io_capacity) {
+    if (!model || node_id < 0 || (size_t)node_id >= model->m.graph.nodes.size() || io_capacity < 0)
+        return fail(AHIP_ERR_ARG, "ahip_model_node_info: invalid argument");
+    const Node &node = model->m.graph.nodes[(size_t)node_id];
+    if (op_kind) *op_kind = (int)node.op.kind;
+    if (attrs) op_to_c(node.op, attrs);
+    if (n_inputs) *n_inputs = (int)node.inputs.size();
+    if (n_outputs) *n_outputs = (int)node.outputs.size();
+    if (inputs)
+        for (int i = 0; i < io_capacity && i < (int)node.inputs.size(); i++) inputs[i] = (int64_t)node.inputs[i];
+    if (outputs)
+        for (int i = 0; i < io_capacity && i < (int)node.outputs.size(); i++) outputs[i] = (int64_t)node.outputs[i];
+    return AHIP_OK;
+}
+
+int ahip_model_infer_value_shape(const ahip_model *model, int64_t value_id, int *elem_type, int *rank,
+                                 int64_t *dims) {
+    if (!model || !rank || !dims || !valid_value(model, value_id))
+        return fail(AHIP_ERR_ARG, "ahip_model_infer_value_shape: invalid argument");
+    std::map<ValueId, TypedFixedShape> shapes;
+    ShapeError err;
+    if (!infer_shapes(model->m, nullptr, &shapes, &err)) return fail(AHIP_ERR_SHAPE, err.message);
+    auto it = shapes.find((ValueId)value_id);
+    if (it == shapes.end()) return fail(AHIP_ERR_ARG, "the shape of this value is not known before run time");
+    if (it->second.dims.len() > AHIP_MAX_RANK) return fail(AHIP_ERR_UNSUPPORTED, "rank above AHIP_MAX_RANK");
+    if (elem_type) *elem_type = (int)it->second.elem_ty;
+    *rank = (int)it->second.dims.len();
+    for (size_t i = 0; i < it->second.dims.len(); i++) dims[i] = (int64_t)it->second.dims[i];
+    return AHIP_OK;
+}
+
+int ahip_model_execution_plan(const ahip_model *model, int64_t *node_ids, int *free_offsets, int node_capacity,
+                              int64_t *free_vals, int free_capacity, int *n_nodes, int *n_free) {
+    if (!model || !n_nodes || !n_free || node_capacity < 0 || free_capacity < 0)
+        return fail(AHIP_ERR_ARG, "ahip_model_execution_plan: invalid argument");
+    const auto plan = create_execution_plan(model->m);
+    int nf = 0;
+    for (size_t i = 0; i < plan.size(); i++) {
+        if ((int)i < node_capacity) {
+            if (node_ids) node_ids[i] = (int64_t)plan[i].node_id;
+            if (free_offsets) free_offsets[i] = nf;
+        }
+        for (ValueId v : plan[i].free_vals) {
+            if (nf < free_capacity && free_vals) free_vals[nf] = (int64_t)v;
+            nf++;
+        }
+    }
+    if (free_offsets && (int)plan.size() <= node_capacity) free_offsets[plan.size()] = nf;
+    *n_nodes = (int)plan.size();
+    *n_free = nf;
+    return AHIP_OK;
+}
+
+int ahip_fuse_layer_norm(ahip_model *model, int *count) { return run_pass(model, count, fuse_layer_norm, "ahip_fuse_layer_norm"); }
+int ahip_fuse_gelu(ahip_model *model, int *count) { return run_pass(model, count, fuse_gelu, "ahip_fuse_gelu"); }
+int ahip_fuse_fast_gelu(ahip_model *model, int *count) { return run_pass(model, count, fuse_fast_gelu, "ahip_fuse_fast_gelu"); }
+int ahip_eliminate_identity(ahip_model *model, int *count) { return run_pass(model, count, eliminate_identity, "ahip_eliminate_identity"); }
+
+// ---- tensors -----------------------------------------------------------------------
+
+int ahip_tensor_new(int elem_type, int rank, const int64_t *dims, const void *data, size_t nbytes,
+                    ahip_tensor **tensor) {
+    if (!tensor || rank < 0 || (rank && !dims) || !valid_elem_type(elem_type))
+        return fail(AHIP_ERR_ARG, "ahip_tensor_new: invalid argument");
+    for (int i = 0; i < rank; i++)
+        if (dims[i] < 0) return fail(AHIP_ERR_ARG, "ahip_tensor_new: negative dimension");
+    FixedDimensions fd = FixedDimensions::from_i64(dims, (size_t)rank);
+    const TensorElemType ty = static_cast<TensorElemType>(elem_type);
+    const size_t want = fd.total_elems() * elem_size(ty);
+    if (data && nbytes != want) return fail(AHIP_ERR_ARG, "ahip_tensor_new: data size does not match the shape");
+    ahip_tensor *t = new (std::nothrow) ahip_tensor();
+    if (!t) return fail(AHIP_ERR_OOM, "ahip_tensor_new: out of host memory");
+    t->t = data ? Tensor::from_raw(std::move(fd), ty, data, want) : Tensor::zeros_of_type(ty, std::move(fd));
+    *tensor = t;
+    return AHIP_OK;
+}
+
+void ahip_tensor_free(ahip_tensor *tensor) { delete tensor; }
+int ahip_tensor_elem_type(const ahip_tensor *tensor) { return tensor ? (int)tensor->t.elem_ty() : -1; }
+int ahip_tensor_rank(const ahip_tensor *tensor) { return tensor ? (int)tensor->t.dims().len() : -1; }
+int ahip_tensor_dims(const ahip_tensor *tensor, int64_t *dims, int capacity) {
+    if (!tensor || capacity < 0 || (capacity && !dims)) return fail(AHIP_ERR_ARG, "ahip_tensor_dims: invalid argument");
+    const auto &d = tensor->t.dims();
+    for (int i = 0; i < capacity && i < (int)d.len(); i++) dims[i] = (int64_t)d[i];
+    return AHIP_OK;
+}
+size_t ahip_tensor_nbytes(const ahip_tensor *tensor) { return tensor ? tensor->t.nbytes() : 0; }
+const void *ahip_tensor_data(const ahip_tensor *tensor) { return tensor ? tensor->t.data_as_bytes() : nullptr; }
+
+// ---- session ---------------------------------------------------------------------------
+
+int ahip_session_builder_new(const ahip_model *model, ahip_session_builder **builder) {
+    if (!model || !builder) return fail(AHIP_ERR_ARG, "ahip_session_builder_new: null argument");
+    ahip_session_builder *b = new (std::nothrow) ahip_session_builder();
+    if (!b) return fail(AHIP_ERR_OOM, "ahip_session_builder_new: out of host memory");
+    b->model = model->m;
+    *builder = b;
+    return AHIP_OK;
+}
+
+void ahip_session_builder_free(ahip_session_builder *builder) { delete builder; }
+
+int ahip_session_builder_with_intra_op_num_threads(ahip_session_builder *builder, size_t n) {
+    if (!builder) return fail(AHIP_ERR_ARG, "null builder");
+    builder->threads = n;
+    return AHIP_OK;
+}
+
+int ahip_session_builder_with_profiling_enabled(ahip_session_builder *builder, int enable) {
+    if (!builder) return fail(AHIP_ERR_ARG, "null builder");
+    builder->profiling = enable != 0;
+    return AHIP_OK;
+}
+
+int ahip_session_builder_with_device(ahip_session_builder *builder, int device) {
+    if (!builder) return fail(AHIP_ERR_ARG, "null builder");
+    builder->device = device;
+    return AHIP_OK;
+}
+
+int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **session) {
+    if (!builder || !session) return fail(AHIP_ERR_ARG, "ahip_session_builder_build: null argument");
+    *session = nullptr;
+    HipSessionBuilder b(builder->model);
+    b.with_intra_op_num_threads(builder->threads).with_profiling_enabled(builder->profiling).with_device(builder->device);
+    SessionError err;
+    std::unique_ptr<HipSession> s = b.build(&err);
+    if (!s) return fail(err.code(), err.to_string());
+    ahip_session *out = new (std::nothrow) ahip_session();
+    if (!out) return fail(AHIP_ERR_OOM, "ahip_session_builder_build: out of host memory");
+    out->view.m = s->model();
+    out->s = std::move(s);
+    *session = out;
+    return AHIP_OK;
+}
+
+void ahip_session_free(ahip_session *session) { delete session; }
+
+int ahip_session_run(ahip_session *session, int n_inputs, const ahip_tensor *const *inputs, int output_capacity,
+                     ahip_tensor **outputs, int *n_outputs) {
+    if (!session || n_inputs < 0 || (n_inputs && !inputs) || output_capacity < 0 || (output_capacity && !outputs) ||
+        !n_outputs)
+        return fail(AHIP_ERR_ARG, "ahip_session_run: invalid argument");
+    std::vector<Tensor> in;
+    for (int i = 0; i < n_inputs; i++) {
+        if (!inputs[i]) return fail(AHIP_ERR_ARG, "ahip_session_run: null input tensor");
+        in.push_back(inputs[i]->t);  // shares the bytes, no copy
+    }
+    std::vector<Tensor> out;
+    SessionError err;
+    if (!session->s->run(in, &out, &err)) return fail(err.code(), err.to_string());
+    *n_outputs = (int)out.size();
+    if ((int)out.size() > output_capacity) return fail(AHIP_ERR_ARG, "ahip_session_run: output capacity too small");
+    for (size_t i = 0; i < out.size(); i++) {
+        ahip_tensor *t = new (std::nothrow) ahip_tensor();
+        if (!t) {
+            for (size_t j = 0; j < i; j++) delete outputs[j];
+            return fail(AHIP_ERR_OOM, "ahip_session_run: out of host memory");
+        }
+        t->t = std::move(out[i]);
+        outputs[i] = t;
+    }
+    session->profile.assign(session->s->last_profile().begin(), session->s->last_profile().end());
+    return AHIP_OK;
+}
+
+const ahip_model *ahip_session_model(const ahip_session *session) { return session ? &session->view : nullptr; }
+
+int ahip_session_profile(const ahip_session *session, int index, const char **op_name, double *ms, int *count) {
+    if (!session) return fail(AHIP_ERR_ARG, "ahip_session_profile: null session");
+    if (count) *count = (int)session->profile.size();
+    if (index < 0 || index >= (int)session->profile.size()) {
+        if (op_name || ms) return fail(AHIP_ERR_ARG, "ahip_session_profile: index out of range");
+        return AHIP_OK;
+    }
+    if (op_name) *op_name = session->profile[index].first.c_str();
+    if (ms) *ms = session->profile[index].second;
+    return AHIP_OK;
+}
+
+int ahip_session_last_run_ms(const ahip_session *session, double *ms) {
+    if (!session || !ms) return fail(AHIP_ERR_ARG, "ahip_session_last_run_ms: null argument");
+    *ms = session->s->last_run_ms();
+    return AHIP_OK;
+}
+
+int ahip_session_device_allocations(const ahip_session *session, size_t *count) {
+    if (!session || !count) return fail(AHIP_ERR_ARG, "ahip_session_device_allocations: null argument");
+    *count = session->s->device_allocations();
+    return AHIP_OK;
+}
+
+}  // extern "C"

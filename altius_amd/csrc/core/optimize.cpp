@@ -1,0 +1,255 @@
+#include "optimize.h"
+
+#include <algorithm>
+
+namespace altius {
+
+namespace {
+
+using Users = std::map<ValueId, std::set<NodeId>>;
+
+// The user of `value` whose operator is `kind`, if any.
+std::optional<NodeId> user_of_kind(const Model &m, const Users &users, ValueId value, OpKind kind) {
+    auto it = users.find(value);
+    if (it == users.end()) return std::nullopt;
+    for (NodeId id : it->second)
+        if (m.graph.nodes[id].op.kind == kind) return id;
+    return std::nullopt;
+}
+
+const Tensor *init_of(const Model &m, ValueId v) {
+    auto it = m.graph.inits.find(v);
+    return it == m.graph.inits.end() ? nullptr : &it->second;
+}
+
+// The initializer is f32, has at least one element and its first element equals `want`.
+bool init_first_is(const Model &m, ValueId v, float want) {
+    const Tensor *t = init_of(m, v);
+    return t && t->elem_ty() == TensorElemType::F32 && t->nbytes() >= sizeof(float) && t->data_f32()[0] == want;
+}
+
+bool init_allclose(const Model &m, ValueId v, float want) {
+    const Tensor *t = init_of(m, v);
+    return t && t->allclose_f32({want});
+}
+
+// Points every reader of `from` (nodes and graph outputs) at `to`.
+void replace_value(Model &m, const Users &users, ValueId from, ValueId to) {
+    auto it = users.find(from);
+    if (it != users.end())
+        for (NodeId u : it->second)
+            for (ValueId &in : m.graph.nodes[u].inputs)
+                if (in == from) in = to;
+    for (ValueId &out : m.graph.outputs)
+        if (out == from) out = to;
+}
+
+}  // namespace
+
+size_t fuse_layer_norm(Model &model) {
+    const auto users = model.get_value_users();
+    struct Match {
+        ValueId data, end, scale, bias;
+        float epsilon;
+    };
+    std::vector<Match> matches;
+    std::vector<NodeId> doomed;
+
+    for (NodeId mean_id : model.topo_sort_nodes()) {
+        const Node &mean = model.graph.nodes[mean_id];
+        if (mean.op.kind != OpKind::ReduceMean || mean.outputs.empty() || mean.inputs.empty()) continue;
+        static const OpKind chain[] = {OpKind::Sub,  OpKind::Pow, OpKind::ReduceMean, OpKind::Add,
+                                       OpKind::Sqrt, OpKind::Div, OpKind::Mul,        OpKind::Add};
+        std::vector<NodeId> ids{mean_id};
+        ValueId cur = mean.outputs[0];
+        bool ok = true;
+        for (OpKind k : chain) {
+            auto next = user_of_kind(model, users, cur, k);
+            if (!next || model.graph.nodes[*next].outputs.empty()) {
+                ok = false;
+                break;
+            }
+            ids.push_back(*next);
+            cur = model.graph.nodes[*next].outputs[0];
+        }
+        if (!ok) continue;
+        const Node &add = model.graph.nodes[ids[4]];
+        const Node &mul = model.graph.nodes[ids[7]];
+        const Node &add2 = model.graph.nodes[ids[8]];
+        if (add.inputs.size() < 2 || mul.inputs.size() < 2 || add2.inputs.size() < 2) continue;
+        const Tensor *eps = init_of(model, add.inputs[1]);
+        if (!eps || eps->elem_ty() != TensorElemType::F32 || eps->nbytes() < sizeof(float)) continue;
+        matches.push_back({mean.inputs[0], add2.outputs[0], mul.inputs[1], add2.inputs[1], eps->data_f32()[0]});
+        doomed.insert(doomed.end(), ids.begin(), ids.end());
+    }
+
+    for (const Match &m : matches) {
+        const ValueId ln_out = model.graph.values.new_val();
+        Node ln(Op::layer_normalization(-1, m.epsilon, 1));
+        ln.with_in(m.data).with_in(m.scale).with_in(m.bias).with_out(ln_out);
+        model.graph.add_node(std::move(ln));
+        replace_value(model, users, m.end, ln_out);
+    }
+    for (NodeId id : doomed) model.graph.nodes[id].deleted = true;
+    model.remove_unnecessary_nodes();
+    return matches.size();
+}
+
+size_t fuse_gelu(Model &model) {
+    const auto users = model.get_value_users();
+    struct Match {
+        ValueId start, end;
+    };
+    std::vector<Match> matches;
+    std::vector<NodeId> doomed;
+
+    for (NodeId div_id : model.topo_sort_nodes()) {
+        const Node &div = model.graph.nodes[div_id];
+        if (div.op.kind != OpKind::Div || div.inputs.size() < 2 || div.outputs.empty()) continue;
+        if (!init_allclose(model, div.inputs[1], 1.4142099618911743f)) continue;
+        const ValueId x = div.inputs[0];
+
+        auto erf_id = user_of_kind(model, users, div.outputs[0], OpKind::Erf);
+        if (!erf_id) continue;
+        const Node &erf = model.graph.nodes[*erf_id];
+
+        auto add_id = user_of_kind(model, users, erf.outputs[0], OpKind::Add);
+        if (!add_id) continue;
+        const Node &add = model.graph.nodes[*add_id];
+        if (add.inputs.size() < 2) continue;
+        const ValueId add_other = add.inputs[0] == erf.outputs[0] ? add.inputs[1] : add.inputs[0];
+        if (!init_first_is(model, add_other, 1.0f)) continue;
+
+        auto mul1_id = user_of_kind(model, users, add.outputs[0], OpKind::Mul);
+        if (!mul1_id) continue;
+        const Node &mul1 = model.graph.nodes[*mul1_id];
+        if (mul1.inputs.size() < 2) continue;
+        const ValueId mul1_other = mul1.inputs[0] == add.outputs[0] ? mul1.inputs[1] : mul1.inputs[0];
+        if (mul1_other != x) continue;
+
+        auto mul2_id = user_of_kind(model, users, mul1.outputs[0], OpKind::Mul);
+        if (!mul2_id) continue;
+        const Node &mul2 = model.graph.nodes[*mul2_id];
+        if (mul2.inputs.size() < 2) continue;
+        const ValueId mul2_other = mul2.inputs[0] == mul1.outputs[0] ? mul2.inputs[1] : mul2.inputs[0];
+        if (!init_first_is(model, mul2_other, 0.5f)) continue;
+
+        matches.push_back({x, mul2.outputs[0]});
+        for (NodeId id : {div_id, *erf_id, *add_id, *mul1_id, *mul2_id}) doomed.push_back(id);
+    }
+
+    for (const Match &m : matches) {
+        const ValueId gelu_out = model.graph.values.new_val();
+        Node gelu{Op(OpKind::Gelu)};
+        gelu.with_in(m.start).with_out(gelu_out);
+        model.graph.add_node(std::move(gelu));
+        replace_value(model, users, m.end, gelu_out);
+    }
+    for (NodeId id : doomed) model.graph.nodes[id].deleted = true;
+    model.remove_unnecessary_nodes();
+    return matches.size();
+}
+
+size_t fuse_fast_gelu(Model &model) {
+    const auto users = model.get_value_users();
+    const auto parents = model.get_value_parents();
+    struct Match {
+        ValueId start, end;
+    };
+    std::vector<Match> matches;
+    std::vector<NodeId> doomed;
+
+    // The single user of `v`, required to have operator `kind`.
+    auto sole_user = [&](ValueId v, OpKind kind) -> std::optional<NodeId> {
+        auto it = users.find(v);
+        if (it == users.end() || it->second.size() != 1) return std::nullopt;
+        const NodeId id = *it->second.begin();
+        if (model.graph.nodes[id].op.kind != kind) return std::nullopt;
+        return id;
+    };
+
+    for (NodeId src_id : model.topo_sort_nodes()) {
+        const Node &src = model.graph.nodes[src_id];
+        if (src.outputs.size() != 1) continue;
+        const ValueId x = src.outputs[0];
+
+        auto pow_id = user_of_kind(model, users, x, OpKind::Pow);
+        if (!pow_id) continue;
+        const Node &pow = model.graph.nodes[*pow_id];
+        if (pow.inputs.size() < 2 || !init_first_is(model, pow.inputs[1], 3.0f)) continue;
+
+        auto mul1_id = sole_user(pow.outputs[0], OpKind::Mul);
+        if (!mul1_id) continue;
+        const Node &mul1 = model.graph.nodes[*mul1_id];
+        if (mul1.inputs.size() < 2 || !init_allclose(model, mul1.inputs[1], 0.044714998453855515f)) continue;
+
+        auto add1_id = sole_user(mul1.outputs[0], OpKind::Add);
+        if (!add1_id) continue;
+        const Node &add1 = model.graph.nodes[*add1_id];
+        if (add1.inputs.empty() || add1.inputs[0] != x) continue;
+
+        auto mul2_id = sole_user(add1.outputs[0], OpKind::Mul);
+        if (!mul2_id) continue;
+        const Node &mul2 = model.graph.nodes[*mul2_id];
+        if (mul2.inputs.size() < 2 || !init_allclose(model, mul2.inputs[1], 0.7978845834732056f)) continue;
+
+        auto tanh_id = sole_user(mul2.outputs[0], OpKind::Tanh);
+        if (!tanh_id) continue;
+        const Node &tanh = model.graph.nodes[*tanh_id];
+
+        auto add2_id = sole_user(tanh.outputs[0], OpKind::Add);
+        if (!add2_id) continue;
+        const Node &add2 = model.graph.nodes[*add2_id];
+        if (add2.inputs.size() < 2 || !init_first_is(model, add2.inputs[1], 1.0f)) continue;
+
+        auto mul3_id = sole_user(add2.outputs[0], OpKind::Mul);
+        if (!mul3_id) continue;
+        const Node &mul3 = model.graph.nodes[*mul3_id];
+        if (mul3.inputs.size() < 2 || mul3.inputs[1] != add2.outputs[0]) continue;
+
+        auto mul4_parent = parents.find(mul3.inputs[0]);
+        if (mul4_parent == parents.end()) continue;
+        const NodeId mul4_id = mul4_parent->second;
+        const Node &mul4 = model.graph.nodes[mul4_id];
+        if (mul4.op.kind != OpKind::Mul || mul4.inputs.size() < 2 || mul4.inputs[0] != x) continue;
+        if (!init_first_is(model, mul4.inputs[1], 0.5f)) continue;
+        auto mul4_users = users.find(mul4.outputs[0]);
+        if (mul4_users == users.end() || mul4_users->second.size() != 1) continue;
+
+        matches.push_back({x, mul3.outputs[0]});
+        for (NodeId id : {*pow_id, *mul1_id, *add1_id, *mul2_id, *tanh_id, *add2_id, *mul3_id, mul4_id})
+            doomed.push_back(id);
+    }
+
+    for (const Match &m : matches) {
+        const ValueId gelu_out = model.graph.values.new_val();
+        Node gelu{Op(OpKind::Gelu)};
+        gelu.with_in(m.start).with_out(gelu_out);
+        model.graph.add_node(std::move(gelu));
+        replace_value(model, users, m.end, gelu_out);
+    }
+    for (NodeId id : doomed) model.graph.nodes[id].deleted = true;
+    model.remove_unnecessary_nodes();
+    return matches.size();
+}
+
+size_t eliminate_identity(Model &model) {
+    const auto users = model.get_value_users();
+    size_t count = 0;
+    for (NodeId id : model.topo_sort_nodes()) {
+        Node &node = model.graph.nodes[id];
+        if (node.op.kind != OpKind::Identity || node.inputs.size() != 1 || node.outputs.size() != 1) continue;
+        const ValueId in = node.inputs[0], out = node.outputs[0];
+        auto it = users.find(out);
+        if (it == users.end()) continue;  // feeds a graph output (or nothing): kept
+        for (NodeId u : it->second)
+            for (ValueId &v : model.graph.nodes[u].inputs)
+                if (v == out) v = in;
+        node.deleted = true;
+        count++;
+    }
+    model.remove_unnecessary_nodes();
+    return count;
+}
+
+}  // namespace altius

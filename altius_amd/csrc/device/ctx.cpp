@@ -21,4 +21,49 @@ int DeviceCtx::check(hipError_t e, const char *what) {
     return e == hipErrorOutOfMemory ? AHIP_ERR_OOM : AHIP_ERR_HIP;
 }
 
+int create_device_ctx(int device, hipStream_t stream, bool own_stream, DeviceCtx *ctx, std::string *error) {
+    auto fail = [&](hipError_t e, const char *what) {
+        if (error) *error = std::string(what) + ": " + hipGetErrorString(e);
+        return e == hipErrorOutOfMemory ? AHIP_ERR_OOM : AHIP_ERR_HIP;
+    };
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) return fail(e, "hipGetDeviceCount");
+    if (device < 0 || device >= n) {
+        if (error) *error = "no such device: " + std::to_string(device);
+        return AHIP_ERR_ARG;
+    }
+    e = hipSetDevice(device);
+    if (e != hipSuccess) return fail(e, "hipSetDevice");
+    ctx->device = device;
+    if (own_stream) {
+        // Default priority; non-blocking with respect to the legacy default stream.
+        e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+        if (e != hipSuccess) return fail(e, "hipStreamCreate");
+        ctx->owns_stream = true;
+    } else {
+        ctx->stream = stream;
+        ctx->owns_stream = false;
+    }
+    void *scratch = nullptr;
+    e = hipMalloc(&scratch, SCRATCH_FLOATS * sizeof(float));
+    if (e != hipSuccess) {
+        if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+        ctx->stream = nullptr;
+        return fail(e, "hipMalloc(scratch)");
+    }
+    ctx->scratch = static_cast<float *>(scratch);
+    ctx->scratch_floats = SCRATCH_FLOATS;
+    return AHIP_OK;
+}
+
+void destroy_device_ctx(DeviceCtx *ctx) {
+    if (hipSetDevice(ctx->device) != hipSuccess) return;
+    (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->scratch) (void)hipFree(ctx->scratch);
+    ctx->scratch = nullptr;
+    if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+    ctx->stream = nullptr;
+}
+
 }  // namespace altius

@@ -35,6 +35,10 @@ struct DeviceCtx {
 void set_global_error(const std::string &msg);
 const char *global_error();
 
+// Creates / tears down a context (stream + scratch buffer) on `device`.
+int create_device_ctx(int device, hipStream_t stream, bool own_stream, DeviceCtx *ctx, std::string *error);
+void destroy_device_ctx(DeviceCtx *ctx);
+
 constexpr int MAX_RANK = 8;
 constexpr size_t SCRATCH_FLOATS = 1u << 20;  // 4 MiB
 

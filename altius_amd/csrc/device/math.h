@@ -76,10 +76,9 @@ __device__ __forceinline__ float sigmoid_elem(float x) {
     return 1.0f / (1.0f + p);
 }
 
-// Op::Gelu (fast_math.rs:304-323): tanh form with a 13/6-degree rational tanh.
-__device__ __forceinline__ float gelu_elem(float i) {
-    constexpr float B = 0.7978845608028654f;
-    constexpr float C = 0.035677408136300125f;
+// The 13/6-degree rational tanh shared by Op::Tanh (session.rs:860-877) and
+// Op::Gelu (fast_math.rs:306-322), applied to an already clamped argument.
+__device__ __forceinline__ float rational_tanh(float v) {
     constexpr float ALPHA_13 = -2.76076847742355e-16f;
     constexpr float ALPHA_11 = 2.00018790482477e-13f;
     constexpr float ALPHA_9 = -8.60467152213735e-11f;
@@ -91,9 +90,6 @@ __device__ __forceinline__ float gelu_elem(float i) {
     constexpr float BETA_4 = 1.18534705686654e-04f;
     constexpr float BETA_2 = 2.26843463243900e-03f;
     constexpr float BETA_0 = 4.89352518554385e-03f;
-
-    float v = i * (C * i * i + B);
-    v = rclamp(v, -9.0f, 9.0f);
     float v2 = v * v;
     float p = __builtin_fmaf(v2, ALPHA_13, ALPHA_11);
     p = __builtin_fmaf(p, v2, ALPHA_9);
@@ -105,8 +101,19 @@ __device__ __forceinline__ float gelu_elem(float i) {
     float q = __builtin_fmaf(v2, BETA_6, BETA_4);
     q = __builtin_fmaf(q, v2, BETA_2);
     q = __builtin_fmaf(q, v2, BETA_0);
-    float o = p / q;
-    return (o + 1.0f) * (i * 0.5f);
+    return p / q;
+}
+
+// Op::Tanh (session.rs:840-903).
+__device__ __forceinline__ float tanh_elem(float x) { return rational_tanh(rclamp(x, -9.0f, 9.0f)); }
+
+// Op::Gelu (fast_math.rs:304-323): 0.5x(1 + tanh(x(B + Cx^2))); the inner
+// product is plain multiplies and an add, no fma.
+__device__ __forceinline__ float gelu_elem(float i) {
+    constexpr float B = 0.7978845608028654f;
+    constexpr float C = 0.035677408136300125f;
+    const float v = rclamp(i * (C * i * i + B), -9.0f, 9.0f);
+    return (rational_tanh(v) + 1.0f) * (i * 0.5f);
 }
 
 // Op::Erf: fastapprox::faster::erf (crate fastapprox 0.3.1; call site

@@ -20,6 +20,7 @@ struct FSqrt { __device__ __forceinline__ float operator()(float x) const { retu
 struct FErf { __device__ __forceinline__ float operator()(float x) const { return erf_elem(x); } };
 struct FGelu { __device__ __forceinline__ float operator()(float x) const { return gelu_elem(x); } };
 struct FSigmoid { __device__ __forceinline__ float operator()(float x) const { return sigmoid_elem(x); } };
+struct FTanh { __device__ __forceinline__ float operator()(float x) const { return tanh_elem(x); } };
 struct FRelu { __device__ __forceinline__ float operator()(float x) const { return relu_elem(x); } };
 struct FHardSigmoid {
     float alpha, beta;
@@ -75,7 +76,7 @@ template <class F> void launch(hipStream_t s, float *out, const float *in, size_
 }  // namespace
 
 int launch_unary(DeviceCtx &ctx, int op, float *out, const float *in, size_t n, float alpha, float beta) {
-    if (op < AHIP_SQRT || op > AHIP_RELU) return ctx.fail(AHIP_ERR_ARG, "unary: unknown op");
+    if (op < AHIP_SQRT || op > AHIP_TANH) return ctx.fail(AHIP_ERR_ARG, "unary: unknown op");
     if (n == 0) return AHIP_OK;
     if (!out || !in) return ctx.fail(AHIP_ERR_ARG, "unary: null tensor pointer");
     if (n > ((size_t)1 << 38)) return ctx.fail(AHIP_ERR_UNSUPPORTED, "unary: more than 2^38 elements");
@@ -87,6 +88,7 @@ int launch_unary(DeviceCtx &ctx, int op, float *out, const float *in, size_t n, 
     case AHIP_SIGMOID: launch(ctx.stream, out, in, n, FSigmoid{}, nt); break;
     case AHIP_HARDSIGMOID: launch(ctx.stream, out, in, n, FHardSigmoid{alpha, beta}, nt); break;
     case AHIP_RELU: launch(ctx.stream, out, in, n, FRelu{}, nt); break;
+    case AHIP_TANH: launch(ctx.stream, out, in, n, FTanh{}, nt); break;
     }
     return ctx.check(hipGetLastError(), "unary launch");
 }

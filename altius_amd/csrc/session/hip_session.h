@@ -1,0 +1,132 @@
+// The session: same construction and run interface as the reference's
+// InterpreterSessionBuilder / InterpreterSession
+// (crates/session_interpreter/src/builder.rs:12-66, session.rs:49-134), with the
+// kernels running on an MI355X and tensors resident in device memory between nodes.
+//
+//   HipSessionBuilder(model).with_intra_op_num_threads(n).with_profiling_enabled(b).build()
+//   session.run(inputs) -> outputs        inputs/outputs are host Tensors, positional
+//   session.model()
+//
+// Failures come back as a SessionError value; nothing panics or aborts.
+#pragma once
+
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../core/model.h"
+#include "../core/shape.h"
+#include "../device/ctx.h"
+#include "plan.h"
+
+namespace altius {
+
+// altius_session::SessionError (crates/session/src/lib.rs:14-35): Shape and Message
+// keep their meaning; Hip stands for failures of the device runtime.
+struct SessionError {
+    enum Kind { Shape, Message, Hip, OutOfMemory, Argument } kind = Message;
+    std::string message;
+    int code() const;  // the AHIP_ERR_* code of this kind
+    std::string to_string() const;
+};
+
+// Device memory reused between nodes and runs: freed blocks are kept in
+// size-bucketed lists and handed out again, so a steady-state run allocates nothing.
+class BufferPool {
+public:
+    explicit BufferPool(DeviceCtx *ctx) : ctx_(ctx) {}
+    ~BufferPool();
+    int acquire(size_t bytes, void **ptr, size_t *bucket);
+    void release(void *ptr, size_t bucket);
+    void trim();  // returns every cached block to the device
+    size_t bytes_reserved() const { return reserved_; }
+    size_t device_allocations() const { return allocations_; }
+
+private:
+    static size_t bucket_of(size_t bytes);
+    DeviceCtx *ctx_;
+    std::map<size_t, std::vector<void *>> free_;
+    size_t reserved_ = 0;
+    size_t allocations_ = 0;
+};
+
+struct DeviceTensor {
+    FixedDimensions dims;
+    TensorElemType elem_ty = TensorElemType::F32;
+    void *ptr = nullptr;
+    size_t bucket = 0;    // pool bucket, 0 when not pooled
+    bool pooled = false;  // owned by the run (returned to the pool when freed)
+    size_t nbytes() const { return dims.total_elems() * elem_size(elem_ty); }
+};
+
+class HipSession {
+public:
+    ~HipSession();
+    HipSession(const HipSession &) = delete;
+    HipSession &operator=(const HipSession &) = delete;
+
+    const Model &model() const { return model_; }
+
+    // Binds inputs[i] to graph.inputs[i], runs every node of the plan on the
+    // device, and returns graph.outputs in order.  Calls are serialised.
+    bool run(const std::vector<Tensor> &inputs, std::vector<Tensor> *outputs, SessionError *err);
+
+    // Per-operator device time of the last run, in milliseconds (filled when
+    // profiling is enabled), keyed by Op::name().
+    const std::map<std::string, double> &last_profile() const { return profile_; }
+    double last_run_ms() const { return last_run_ms_; }
+    size_t device_allocations() const { return pool_->device_allocations(); }
+    const std::vector<NodeExecutionPlan> &execution_plan() const { return plan_; }
+    const InferredShapes &inferred_shapes() const { return inferred_; }
+
+private:
+    friend class HipSessionBuilder;
+    HipSession() = default;
+
+    bool run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, SessionError *err);
+    void release(DeviceTensor &t);
+
+    Model model_;
+    std::vector<NodeExecutionPlan> plan_;
+    InferredShapes inferred_;
+    bool enable_profiling_ = false;
+    size_t intra_op_num_threads_ = 1;
+    DeviceCtx ctx_;
+    std::unique_ptr<BufferPool> pool_;
+    std::map<ValueId, DeviceTensor> inits_;  // uploaded once at build
+    std::map<std::string, double> profile_;
+    double last_run_ms_ = 0;
+    std::mutex mutex_;
+};
+
+class HipSessionBuilder {
+public:
+    explicit HipSessionBuilder(Model model) : model_(std::move(model)) {}
+    // Accepted for interface parity; the device kernels do not use host threads.
+    HipSessionBuilder &with_intra_op_num_threads(size_t n) {
+        intra_op_num_threads_ = n;
+        return *this;
+    }
+    HipSessionBuilder &with_profiling_enabled(bool enable) {
+        enable_profiling_ = enable;
+        return *this;
+    }
+    // Not in the reference: which GPU to run on (default 0).
+    HipSessionBuilder &with_device(int device) {
+        device_ = device;
+        return *this;
+    }
+    // Infers shapes, builds the execution plan, creates the device context and
+    // uploads the initializers.  Returns nullptr and fills *err on failure.
+    std::unique_ptr<HipSession> build(SessionError *err);
+
+private:
+    Model model_;
+    size_t intra_op_num_threads_ = 1;
+    bool enable_profiling_ = false;
+    int device_ = 0;
+};
+
+}  // namespace altius

@@ -12,7 +12,7 @@ from . import _lib
 from ._lib import check, i64_array
 
 ADD, SUB, MUL, DIV, POW = 0, 1, 2, 3, 4
-SQRT, ERF, GELU, SIGMOID, HARDSIGMOID, RELU = 0, 1, 2, 3, 4, 5
+SQRT, ERF, GELU, SIGMOID, HARDSIGMOID, RELU, TANH = 0, 1, 2, 3, 4, 5, 6
 REDUCE_MEAN, REDUCE_MAX = 0, 1
 
 
@@ -90,7 +90,7 @@ class Context:
 
     def upload(self, array):
         """Copies a numpy array to a new device buffer."""
-        a = np.ascontiguousarray(array)
+        a = np.asarray(array, order="C")
         buf = self.alloc(max(a.nbytes, 4))
         if a.nbytes:
             check(self.L.ahip_h2d_async(self.handle, buf.ptr, a.ctypes.data, a.nbytes), self.handle)
@@ -146,8 +146,8 @@ class Context:
 
     # --- convenience: numpy in, numpy out (upload, one kernel, download) ----
     def binary(self, op, a, b):
-        a = np.ascontiguousarray(a, dtype=np.float32)
-        b = np.ascontiguousarray(b, dtype=np.float32)
+        a = np.asarray(a, dtype=np.float32, order="C")
+        b = np.asarray(b, dtype=np.float32, order="C")
         out_dims = broadcast_shape(a.shape, b.shape)
         a_str = strides_for_broadcasting(a.shape, out_dims)
         b_str = strides_for_broadcasting(b.shape, out_dims)
@@ -162,7 +162,7 @@ class Context:
                 self.free(x)
 
     def unary(self, op, x, alpha=0.0, beta=0.0):
-        x = np.ascontiguousarray(x, dtype=np.float32)
+        x = np.asarray(x, dtype=np.float32, order="C")
         dx = self.upload(x)
         do = self.alloc(max(x.nbytes, 4))
         try:
@@ -173,7 +173,7 @@ class Context:
             self.free(do)
 
     def softmax(self, x):
-        x = np.ascontiguousarray(x, dtype=np.float32)
+        x = np.asarray(x, dtype=np.float32, order="C")
         length = x.shape[-1]
         rows = x.size // length if length else 0
         dx = self.upload(x)
@@ -186,9 +186,9 @@ class Context:
             self.free(do)
 
     def layer_norm(self, x, gamma, beta, eps=1e-5):
-        x = np.ascontiguousarray(x, dtype=np.float32)
-        gamma = np.ascontiguousarray(gamma, dtype=np.float32)
-        beta = np.ascontiguousarray(beta, dtype=np.float32)
+        x = np.asarray(x, dtype=np.float32, order="C")
+        gamma = np.asarray(gamma, dtype=np.float32, order="C")
+        beta = np.asarray(beta, dtype=np.float32, order="C")
         length = x.shape[-1]
         assert gamma.size == length and beta.size == length
         rows = x.size // length if length else 0
@@ -203,7 +203,7 @@ class Context:
 
     def reduce(self, kind, x, outer, red, inner):
         """Reduces the middle axis of x viewed as [outer, red, inner]; returns [outer, inner]."""
-        x = np.ascontiguousarray(x, dtype=np.float32)
+        x = np.asarray(x, dtype=np.float32, order="C")
         assert x.size == outer * red * inner
         dx = self.upload(x)
         do = self.alloc(max(outer * inner * 4, 4))

@@ -1,0 +1,91 @@
+"""HipSessionBuilder / HipSession: the MI355X stand-in for altius's
+InterpreterSessionBuilder / InterpreterSession, over the C ABI."""
+import ctypes
+
+import numpy as np
+
+from . import _lib
+from ._lib import check
+from .graph import Model, Tensor
+
+
+class HipSession:
+    def __init__(self, handle):
+        self.L = _lib.lib()
+        self.handle = handle
+
+    def __del__(self):
+        self.close()
+
+    def close(self):
+        if getattr(self, "handle", None):
+            self.L.ahip_session_free(self.handle)
+            self.handle = None
+
+    def model(self):
+        """A borrowed view of the session's model (valid while the session lives)."""
+        return Model(_handle=ctypes.c_void_p(self.L.ahip_session_model(self.handle)), _borrowed=True)
+
+    def run(self, inputs):
+        """inputs: numpy arrays or Tensors, positional in graph.inputs order.  Returns numpy arrays
+        in graph.outputs order."""
+        tensors = [t if isinstance(t, Tensor) else Tensor.from_numpy(t) for t in inputs]
+        arr = (ctypes.c_void_p * max(len(tensors), 1))(*[t.handle for t in tensors])
+        cap = 16
+        outs = (ctypes.c_void_p * cap)()
+        n = ctypes.c_int()
+        check(self.L.ahip_session_run(self.handle, len(tensors), arr, cap, outs, ctypes.byref(n)))
+        return [Tensor(ctypes.c_void_p(outs[i])).numpy() for i in range(n.value)]
+
+    def profile(self):
+        """{op name: device milliseconds} of the last run (profiling enabled)."""
+        count = ctypes.c_int()
+        check(self.L.ahip_session_profile(self.handle, -1, None, None, ctypes.byref(count)))
+        out = {}
+        for i in range(count.value):
+            name, ms = ctypes.c_char_p(), ctypes.c_double()
+            check(self.L.ahip_session_profile(self.handle, i, ctypes.byref(name), ctypes.byref(ms), None))
+            out[name.value.decode()] = ms.value
+        return out
+
+    def last_run_ms(self):
+        ms = ctypes.c_double()
+        check(self.L.ahip_session_last_run_ms(self.handle, ctypes.byref(ms)))
+        return ms.value
+
+    def device_allocations(self):
+        c = ctypes.c_size_t()
+        check(self.L.ahip_session_device_allocations(self.handle, ctypes.byref(c)))
+        return c.value
+
+
+class HipSessionBuilder:
+    """HipSessionBuilder(model).with_intra_op_num_threads(n).with_profiling_enabled(b).build()"""
+
+    def __init__(self, model):
+        self.L = _lib.lib()
+        h = ctypes.c_void_p()
+        check(self.L.ahip_session_builder_new(model.handle, ctypes.byref(h)))
+        self.handle = h
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            self.L.ahip_session_builder_free(self.handle)
+            self.handle = None
+
+    def with_intra_op_num_threads(self, n):
+        check(self.L.ahip_session_builder_with_intra_op_num_threads(self.handle, n))
+        return self
+
+    def with_profiling_enabled(self, enable):
+        check(self.L.ahip_session_builder_with_profiling_enabled(self.handle, int(bool(enable))))
+        return self
+
+    def with_device(self, device):
+        check(self.L.ahip_session_builder_with_device(self.handle, device))
+        return self
+
+    def build(self):
+        s = ctypes.c_void_p()
+        check(self.L.ahip_session_builder_build(self.handle, ctypes.byref(s)))
+        return HipSession(s)

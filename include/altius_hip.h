@@ -119,7 +119,8 @@ enum ahip_unary_op {
     AHIP_GELU = 2,        /* compute_gelu, session.rs:823-838 + fast_math.rs:281-355 */
     AHIP_SIGMOID = 3,     /* compute_sigmoid, session.rs:905-922 + fast_math.rs:189-279 */
     AHIP_HARDSIGMOID = 4, /* compute_hard_sigmoid, session.rs:805-812 (alpha, beta) */
-    AHIP_RELU = 5         /* compute_relu, session.rs:796-803 */
+    AHIP_RELU = 5,        /* compute_relu, session.rs:796-803 */
+    AHIP_TANH = 6         /* compute_tanh, session.rs:840-903, 933-938 (rational tanh) */
 };
 
 /* Flat element-wise op over n elements.  alpha/beta are read by HardSigmoid only. */
@@ -145,6 +146,147 @@ enum ahip_reduce_kind { AHIP_REDUCE_MEAN = 0, AHIP_REDUCE_MAX = 1 };
  * panics on NaN). */
 int ahip_reduce(ahip_ctx *ctx, int kind, float *out, const float *in, size_t outer, size_t reduce,
                 size_t inner);
+
+/* ------------------------------------------------------------------------
+ * Graph IR: the same Model / Graph / Node / Value / Op structure as
+ * altius_core (crates/core/src/model.rs:13-17, graph.rs:9-16, node.rs:7-14,
+ * value.rs:9-13, op.rs:7-57), built through handles.  Value and node ids are
+ * indices into the model's arenas.  None of these functions needs a device;
+ * their error text is read with ahip_last_error(NULL).
+ * ---------------------------------------------------------------------- */
+
+typedef struct ahip_model ahip_model;
+typedef struct ahip_tensor ahip_tensor;
+typedef struct ahip_session_builder ahip_session_builder;
+typedef struct ahip_session ahip_session;
+
+/* TensorElemType (crates/core/src/tensor.rs:47-53) */
+enum ahip_elem_type { AHIP_BOOL = 0, AHIP_F32 = 1, AHIP_I32 = 2, AHIP_I64 = 3 };
+
+/* Op (crates/core/src/op.rs:7-57), same variants in the same order.  The
+ * session executes the kinds marked (*); the others are representable so that
+ * any altius graph can be described, and fail at build or run time with
+ * AHIP_ERR_UNSUPPORTED, as the reference's unimplemented kernels do
+ * (session.rs:200-245). */
+enum ahip_op_kind {
+    AHIP_OP_IDENTITY = 0 /* (*) */, AHIP_OP_CONV2D, AHIP_OP_ADD /* (*) */, AHIP_OP_SUB /* (*) */,
+    AHIP_OP_MUL /* (*) */, AHIP_OP_DIV /* (*) */, AHIP_OP_POW /* (*) */, AHIP_OP_GREATER,
+    AHIP_OP_SQRT /* (*) */, AHIP_OP_RELU /* (*) */, AHIP_OP_GELU /* (*) */, AHIP_OP_LEAKYRELU,
+    AHIP_OP_SIGMOID /* (*) */, AHIP_OP_ERF /* (*) */, AHIP_OP_TANH /* (*) */, AHIP_OP_CLIP, AHIP_OP_WHERE,
+    AHIP_OP_SOFTMAX /* (*) */, AHIP_OP_CAST, AHIP_OP_MAXPOOL, AHIP_OP_GLOBALAVERAGEPOOL, AHIP_OP_RESHAPE,
+    AHIP_OP_FLATTEN, AHIP_OP_RESIZE, AHIP_OP_CONCAT, AHIP_OP_TRANSPOSE, AHIP_OP_SQUEEZE, AHIP_OP_UNSQUEEZE,
+    AHIP_OP_REDUCEMIN, AHIP_OP_REDUCEMAX /* (*) */, AHIP_OP_REDUCEMEAN /* (*) */, AHIP_OP_ROUND, AHIP_OP_EXP,
+    AHIP_OP_EXPAND, AHIP_OP_RANGE, AHIP_OP_LOOP, AHIP_OP_TILE, AHIP_OP_SPLIT, AHIP_OP_SLICE, AHIP_OP_GATHER,
+    AHIP_OP_SHAPE, AHIP_OP_NONMAXSUPPRESSION, AHIP_OP_MATMUL, AHIP_OP_GEMM, AHIP_OP_BATCHNORMALIZATION,
+    AHIP_OP_LAYERNORMALIZATION /* (*) */, AHIP_OP_HARDSIGMOID /* (*) */, AHIP_OP_CONSTANT,
+    AHIP_OP_FUSEDELEMWISE, AHIP_OP_COUNT
+};
+
+/* Attributes of the executable operators (op.rs:84-99, 143-162, 195-200). */
+typedef struct ahip_op_attrs {
+    int64_t axis;                /* Softmax, LayerNormalization */
+    int64_t axes[AHIP_MAX_RANK]; /* ReduceMax, ReduceMean */
+    int32_t n_axes;
+    int32_t keep_dims;           /* ReduceMax, ReduceMean */
+    float alpha;                 /* HardSigmoid */
+    float beta;                  /* HardSigmoid */
+    float epsilon;               /* LayerNormalization */
+    int64_t stash_type;          /* LayerNormalization */
+} ahip_op_attrs;
+
+/* Fills the ONNX defaults the reference's loader applies
+ * (crates/core/src/onnx/load.rs:185-187, 277-288, 321-324, 340-344):
+ * axis -1, no axes, keep_dims 1, alpha 0.2, beta 0.5, epsilon 1e-5, stash_type 1. */
+void ahip_op_attrs_default(ahip_op_attrs *attrs);
+const char *ahip_op_name(int op_kind); /* Op::name (op.rs:324-376) */
+
+int ahip_model_new(int64_t opset_version, ahip_model **model);
+int ahip_model_clone(const ahip_model *model, ahip_model **copy);
+void ahip_model_free(ahip_model *model);
+/* ValueArena::new_val / new_val_named (value.rs:19-31); name may be NULL. */
+int ahip_model_new_value(ahip_model *model, const char *name, int64_t *value_id);
+/* ValueArena::new_val_named_and_shaped (value.rs:33-42); a negative dim is a dynamic one. */
+int ahip_model_new_value_shaped(ahip_model *model, const char *name, int elem_type, int rank,
+                                const int64_t *dims, int64_t *value_id);
+/* graph.inits.insert (graph.rs:13); data is copied, nbytes must match the shape. */
+int ahip_model_add_initializer(ahip_model *model, int64_t value_id, int elem_type, int rank,
+                               const int64_t *dims, const void *data, size_t nbytes);
+/* Graph::add_node (graph.rs:18-22); attrs may be NULL for the defaults, name may be NULL. */
+int ahip_model_add_node(ahip_model *model, int op_kind, const ahip_op_attrs *attrs, const char *name,
+                        int n_inputs, const int64_t *inputs, int n_outputs, const int64_t *outputs,
+                        int64_t *node_id);
+int ahip_model_add_input(ahip_model *model, int64_t value_id);   /* graph.inputs.push */
+int ahip_model_add_output(ahip_model *model, int64_t value_id);  /* graph.outputs.push */
+/* Model::lookup_named_value (model.rs:19-28); AHIP_ERR_ARG when no value has that name. */
+int ahip_model_lookup_named_value(const ahip_model *model, const char *name, int64_t *value_id);
+/* which = 0: graph.inputs, 1: graph.outputs.  *n gets the full count even beyond capacity. */
+int ahip_model_graph_io(const ahip_model *model, int which, int64_t *value_ids, int capacity, int *n);
+/* Model::topo_sort_nodes (model.rs:62-101). */
+int ahip_model_topo_sort(const ahip_model *model, int64_t *node_ids, int capacity, int *n);
+/* Reads one node back.  inputs/outputs hold io_capacity entries each. */
+int ahip_model_node_info(const ahip_model *model, int64_t node_id, int *op_kind, ahip_op_attrs *attrs,
+                         int *n_inputs, int64_t *inputs, int *n_outputs, int64_t *outputs, int io_capacity);
+/* infer_shapes (crates/core/src/analysis/shape.rs:659-692) and the shape it finds for one
+ * value.  AHIP_ERR_SHAPE if inference fails, AHIP_ERR_ARG if that value's shape stays unknown. */
+int ahip_model_infer_value_shape(const ahip_model *model, int64_t value_id, int *elem_type, int *rank,
+                                 int64_t *dims);
+/* create_execution_plan (crates/session/src/plan.rs:14-58): node ids in execution order,
+ * and for node i the values freed after it: free_vals[free_offsets[i] .. free_offsets[i+1]).
+ * free_offsets holds node_capacity + 1 entries. */
+int ahip_model_execution_plan(const ahip_model *model, int64_t *node_ids, int *free_offsets,
+                              int node_capacity, int64_t *free_vals, int free_capacity, int *n_nodes,
+                              int *n_free);
+
+/* Fusion passes (crates/core/src/optimize/{layer_norm_fusion,gelu_fusion,fast_gelu_fusion,
+ * identity_elim}.rs).  *count (may be NULL) gets the number of rewrites. */
+int ahip_fuse_layer_norm(ahip_model *model, int *count);
+int ahip_fuse_gelu(ahip_model *model, int *count);
+int ahip_fuse_fast_gelu(ahip_model *model, int *count);
+int ahip_eliminate_identity(ahip_model *model, int *count);
+
+/* Host tensors (crates/core/src/tensor.rs:61-76).  data is copied; NULL data gives zeros. */
+int ahip_tensor_new(int elem_type, int rank, const int64_t *dims, const void *data, size_t nbytes,
+                    ahip_tensor **tensor);
+void ahip_tensor_free(ahip_tensor *tensor);
+int ahip_tensor_elem_type(const ahip_tensor *tensor);
+int ahip_tensor_rank(const ahip_tensor *tensor);
+int ahip_tensor_dims(const ahip_tensor *tensor, int64_t *dims, int capacity);
+size_t ahip_tensor_nbytes(const ahip_tensor *tensor);
+const void *ahip_tensor_data(const ahip_tensor *tensor);
+
+/* ------------------------------------------------------------------------
+ * Session: InterpreterSessionBuilder / InterpreterSession
+ * (crates/session_interpreter/src/builder.rs:18-66, session.rs:61-134).
+ * ---------------------------------------------------------------------- */
+
+/* InterpreterSessionBuilder::new(model); the model is copied. */
+int ahip_session_builder_new(const ahip_model *model, ahip_session_builder **builder);
+void ahip_session_builder_free(ahip_session_builder *builder);
+/* with_intra_op_num_threads: accepted for parity, device kernels use no host threads. */
+int ahip_session_builder_with_intra_op_num_threads(ahip_session_builder *builder, size_t n);
+int ahip_session_builder_with_profiling_enabled(ahip_session_builder *builder, int enable);
+/* Not in the reference: the GPU to run on (default 0). */
+int ahip_session_builder_with_device(ahip_session_builder *builder, int device);
+/* build(): shape inference (AHIP_ERR_SHAPE on failure), execution plan, device context,
+ * upload of the initializers.  The builder stays valid and must still be freed. */
+int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **session);
+
+void ahip_session_free(ahip_session *session);
+/* run(inputs): inputs are bound to graph.inputs in order; outputs come back in
+ * graph.outputs order as new tensors the caller frees.  *n_outputs gets their
+ * number; AHIP_ERR_ARG if output_capacity is too small.  Calls on one session
+ * are serialised internally. */
+int ahip_session_run(ahip_session *session, int n_inputs, const ahip_tensor *const *inputs,
+                     int output_capacity, ahip_tensor **outputs, int *n_outputs);
+/* model(): a borrowed handle, valid while the session lives. */
+const ahip_model *ahip_session_model(const ahip_session *session);
+/* Per-operator device time of the last run when profiling is enabled
+ * (session.rs:117-125, 251-255): entry `index` of `*count` entries. */
+int ahip_session_profile(const ahip_session *session, int index, const char **op_name, double *ms,
+                         int *count);
+int ahip_session_last_run_ms(const ahip_session *session, double *ms);
+/* Number of hipMalloc calls the session's buffer pool has made so far. */
+int ahip_session_device_allocations(const ahip_session *session, size_t *count);
 
 #ifdef __cplusplus
 }

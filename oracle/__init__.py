@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
 ADD, SUB, MUL, DIV, POW = 0, 1, 2, 3, 4
-SQRT, ERF, GELU, SIGMOID, HARDSIGMOID, RELU = 0, 1, 2, 3, 4, 5
+SQRT, ERF, GELU, SIGMOID, HARDSIGMOID, RELU, TANH = 0, 1, 2, 3, 4, 5, 6
 REDUCE_MEAN, REDUCE_MAX = 0, 1
 
 OK, ERR_BROADCAST, ERR_UNSUPPORTED, ERR_ARG = 0, 1, 2, 3
@@ -58,7 +58,7 @@ def _fptr(a):
 
 
 def _f32(a):
-    a = np.ascontiguousarray(a, dtype=np.float32)
+    a = np.asarray(a, dtype=np.float32, order="C")
     return a
 
 

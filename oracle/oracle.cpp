@@ -285,6 +285,35 @@ inline float gelu_elem(float i) {
     return (o + 1.0f) * (i * 0.5f);
 }
 
+// One element of tanh (session.rs:860-877 / 883-902): the same 13/6-degree
+// rational function fast_gelu uses, on the clamped input itself.
+inline float tanh_elem(float x) {
+    const float ALPHA_13 = -2.76076847742355e-16f;
+    const float ALPHA_11 = 2.00018790482477e-13f;
+    const float ALPHA_9 = -8.60467152213735e-11f;
+    const float ALPHA_7 = 5.12229709037114e-08f;
+    const float ALPHA_5 = 1.48572235717979e-05f;
+    const float ALPHA_3 = 6.37261928875436e-04f;
+    const float ALPHA_1 = 4.89352455891786e-03f;
+    const float BETA_6 = 1.19825839466702e-06f;
+    const float BETA_4 = 1.18534705686654e-04f;
+    const float BETA_2 = 2.26843463243900e-03f;
+    const float BETA_0 = 4.89352518554385e-03f;
+    float v = rclamp(x, -9.0f, 9.0f);
+    float v2 = v * v;
+    float p = fmaf(v2, ALPHA_13, ALPHA_11);
+    p = fmaf(p, v2, ALPHA_9);
+    p = fmaf(p, v2, ALPHA_7);
+    p = fmaf(p, v2, ALPHA_5);
+    p = fmaf(p, v2, ALPHA_3);
+    p = fmaf(p, v2, ALPHA_1);
+    p = p * v;
+    float q = fmaf(v2, BETA_6, BETA_4);
+    q = fmaf(q, v2, BETA_2);
+    q = fmaf(q, v2, BETA_0);
+    return p / q;
+}
+
 void fast_gelu(float *out, const float *in, size_t len) {
     for (size_t i = 0; i < len; i++) out[i] = gelu_elem(in[i]);
 }
@@ -621,6 +650,9 @@ int orc_unary(int op, const float *in, float *out, size_t n, float alpha, float 
         return ORC_OK;
     case ORC_HARDSIGMOID:  // session.rs:805-812
         for (size_t i = 0; i < n; i++) out[i] = rclamp(fmaf(alpha, in[i], beta), 0.0f, 1.0f);
+        return ORC_OK;
+    case ORC_TANH:  // session.rs:933-938
+        for (size_t i = 0; i < n; i++) out[i] = tanh_elem(in[i]);
         return ORC_OK;
     case ORC_ERF:  // session.rs:924-931
         for (size_t i = 0; i < n; i++) out[i] = faster_erf(in[i]);

@@ -19,7 +19,7 @@
  *     crates/altius_py/tests/test_ops_bin.py.
  *   - Add/Sub/Mul/Div, Sqrt, Relu, HardSigmoid, Pow(x,2): IEEE-754 closed forms,
  *     pinned bit-exactly against numpy float32 / float64-emulated fma.
- *   - Softmax, Sigmoid, Gelu: formulas are fully in-tree
+ *   - Softmax, Sigmoid, Gelu, Tanh: formulas are fully in-tree
  *     (crates/session_interpreter/src/fast_math.rs); pinned against exact
  *     softmax / logistic / tanh-GELU at the reference's own test tolerance and
  *     by invariants (rows sum to 1, symmetry, monotonicity, saturation).
@@ -57,7 +57,8 @@ enum orc_unary_op {
     ORC_GELU = 2,
     ORC_SIGMOID = 3,
     ORC_HARDSIGMOID = 4,
-    ORC_RELU = 5
+    ORC_RELU = 5,
+    ORC_TANH = 6
 };
 
 enum orc_reduce_kind { ORC_REDUCE_MEAN = 0, ORC_REDUCE_MAX = 1 };
@@ -100,7 +101,7 @@ int orc_binary(int op, const float *a, int a_rank, const int64_t *a_dims, const 
 
 /* session.rs:608-619 (Sqrt), 796-803 (Relu), 805-812 (HardSigmoid),
  * 823-838 + fast_math.rs:281-355 (Gelu), 905-922 + fast_math.rs:189-279
- * (Sigmoid), 924-931 (Erf -> fastapprox::faster::erf).
+ * (Sigmoid), 924-931 (Erf -> fastapprox::faster::erf), 840-903 + 933-938 (Tanh).
  * alpha/beta are HardSigmoid's attributes, ignored by the other ops. */
 int orc_unary(int op, const float *in, float *out, size_t n, float alpha, float beta, int threads);
 

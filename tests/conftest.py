@@ -68,8 +68,8 @@ def assert_close(actual, expected, rtol=RTOL, atol=ATOL, what=""):
 
 def assert_bits_equal(actual, expected, what="", zero_sign_free=False):
     """Bit-for-bit equality of two float32 arrays (NaN payloads excepted)."""
-    actual = np.ascontiguousarray(actual, dtype=np.float32)
-    expected = np.ascontiguousarray(expected, dtype=np.float32)
+    actual = np.asarray(actual, dtype=np.float32, order="C")
+    expected = np.asarray(expected, dtype=np.float32, order="C")
     assert actual.shape == expected.shape, f"{what}: shape {actual.shape} vs {expected.shape}"
     a = actual.view(np.uint32)
     e = expected.view(np.uint32)

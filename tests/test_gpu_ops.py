@@ -141,6 +141,7 @@ UNARY = {
     "Sigmoid": (D.SIGMOID, 3),
     "HardSigmoid": (D.HARDSIGMOID, 4),
     "Relu": (D.RELU, 5),
+    "Tanh": (D.TANH, 6),
 }
 
 

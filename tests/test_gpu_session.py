@@ -1,0 +1,305 @@
+"""The session on the GPU: graphs built the way the reference's tests build them
+(crates/session_interpreter/tests/op_bin.rs:27-37), run through HipSessionBuilder / HipSession,
+and compared with the CPU oracle applied node by node.  Covers every benchmark configuration at
+reduced batch, the fused-vs-unfused comparisons, and the error paths."""
+import numpy as np
+import pytest
+
+import oracle as O
+from altius_amd import synth
+from altius_amd._lib import ERR_ARG, ERR_SHAPE, ERR_UNSUPPORTED, AltiusHipError
+from altius_amd.graph import F32, I64, Model, Op
+from altius_amd.session import HipSessionBuilder
+from conftest import assert_bits_equal, assert_close
+from test_host import erf_gelu_chain, layer_norm_chain
+
+pytestmark = pytest.mark.gpu
+
+
+def binary_model(op):
+    """x, y -> op -> z with no declared shapes, exactly as op_bin.rs:27-37 builds it."""
+    m = Model()
+    x, y, z = m.new_val_named("x"), m.new_val_named("y"), m.new_val_named("z")
+    m.add_node(op, [x, y], [z])
+    m.add_input(x)
+    m.add_input(y)
+    m.add_output(z)
+    return m
+
+
+@pytest.mark.parametrize("shape", [[1, 2], [3, 1, 10], [16, 3, 224, 224]])
+@pytest.mark.parametrize("name,op,fn", [("add", Op.Add, np.add), ("sub", Op.Sub, np.subtract),
+                                        ("mul", Op.Mul, np.multiply), ("div", Op.Div, np.divide)])
+def test_op_bin(case, name, op, fn, shape):
+    """test_op_{add,sub,mul,div}_{1,2,3} (op_bin.rs:62-76); expected = x op y (op_bin.rs:41-46),
+    tolerance 1e-5/1e-5 there, bit equality here."""
+    case(f"session op_bin {name} {shape}")
+    sess = HipSessionBuilder(binary_model(op)).build()
+    x = synth.uniform(42, shape)
+    y = synth.uniform(43, shape) + np.float32(1e-3)
+    (z,) = sess.run([x, y])
+    assert_bits_equal(z, fn(x, y), f"{name} {shape}")
+
+
+def test_run_time_shape_inference_with_broadcast(case):
+    """Inputs without declared shapes are inferred at run time (session.rs:149-158)."""
+    case("session run-time shapes")
+    sess = HipSessionBuilder(binary_model(Op.Mul)).build()
+    for sa, sb in (([3, 15, 15], [15]), ([4, 1, 2], [3, 1]), ([2, 3], [])):
+        a, b = synth.normal(1, sa), synth.normal(2, sb)
+        (z,) = sess.run([a, b])
+        assert_bits_equal(z, a * b, f"{sa}*{sb}")
+
+
+def test_cfg0_bias_add(case):
+    case("session cfg0")
+    c = synth.cfg0()
+    m = Model()
+    a = m.new_val_named_and_shaped("a", c["a"].shape)
+    b = m.new_initializer(c["b"], "bias")
+    z = m.new_val_named("z")
+    m.add_node(Op.Add, [a, b], [z])
+    m.add_input(a)
+    m.add_output(z)
+    sess = HipSessionBuilder(m).build()
+    (out,) = sess.run([c["a"]])
+    assert_bits_equal(out, O.binary(O.ADD, c["a"], c["b"]), "cfg0")
+
+
+def test_cfg1_softmax_and_layernorm(case):
+    case("session cfg1")
+    c = synth.cfg1(batch=2)
+    m = Model()
+    s = m.new_val_named_and_shaped("scores", c["scores"].shape)
+    x = m.new_val_named_and_shaped("x", c["x"].shape)
+    g = m.new_initializer(c["gamma"])
+    b = m.new_initializer(c["beta"])
+    p, y = m.new_val_named("p"), m.new_val_named("y")
+    m.add_node(Op.Softmax, [s], [p], axis=-1)
+    m.add_node(Op.LayerNormalization, [x, g, b], [y], axis=-1, epsilon=c["eps"])
+    m.add_input(s)
+    m.add_input(x)
+    m.add_output(p)
+    m.add_output(y)
+    sess = HipSessionBuilder(m).with_profiling_enabled(True).build()
+    p_out, y_out = sess.run([c["scores"], c["x"]])
+    assert_close(p_out, O.softmax(c["scores"]), what="cfg1 softmax")
+    assert_close(y_out, O.layer_norm(c["x"], c["gamma"], c["beta"], c["eps"]), what="cfg1 layernorm")
+    prof = sess.profile()
+    assert set(prof) == {"Softmax", "LayerNormalization"} and all(v > 0 for v in prof.values())
+    assert sess.last_run_ms() > 0
+
+
+def oracle_ln_chain(x, gamma, beta, eps):
+    mean = O.reduce(O.REDUCE_MEAN, x, [-1], True)
+    d = O.binary(O.SUB, x, mean)
+    sq = O.binary(O.POW, d, np.array(2.0, np.float32))
+    var = O.reduce(O.REDUCE_MEAN, sq, [-1], True)
+    ve = O.binary(O.ADD, var, np.array(eps, np.float32))
+    sd = O.unary(O.SQRT, ve)
+    n = O.binary(O.DIV, d, sd)
+    return O.binary(O.ADD, O.binary(O.MUL, n, gamma), beta)
+
+
+def test_cfg2_unfused_chain_and_fused_layernorm(case):
+    """The 9-node chain against the oracle's 9 steps, then the same model after fuse_layer_norm against
+    the oracle's LayerNormalization; the two results agree to fp32 rounding of the two formulas."""
+    case("session cfg2")
+    c = synth.cfg2(batch=4)
+    m = Model()
+    x = m.new_val_named_and_shaped("x", c["x"].shape)
+    out, _, _ = layer_norm_chain(m, x, c["gamma"], c["beta"], eps=float(c["eps"]))
+    m.add_input(x)
+    m.add_output(out)
+    fused = m.clone()
+    assert fused.fuse_layer_norm() == 1 and [n["op_name"] for n in fused.nodes()] == ["LayerNormalization"]
+
+    sess = HipSessionBuilder(m).build()
+    (unfused_out,) = sess.run([c["x"]])
+    assert_close(unfused_out, oracle_ln_chain(c["x"], c["gamma"], c["beta"], c["eps"]), what="cfg2 chain")
+    allocs = sess.device_allocations()
+    (again,) = sess.run([c["x"]])
+    assert_bits_equal(again, unfused_out, "second run")
+    assert sess.device_allocations() == allocs        # steady state: the pool serves every buffer
+
+    fsess = HipSessionBuilder(fused).build()
+    (fused_out,) = fsess.run([c["x"]])
+    assert_close(fused_out, O.layer_norm(c["x"], c["gamma"], c["beta"], float(c["eps"])), what="cfg2 fused")
+    np.testing.assert_allclose(fused_out, unfused_out, rtol=1e-4, atol=1e-5)
+
+
+def test_cfg3_gelu_unfused_and_fused(case):
+    """Div -> Erf -> Add -> Mul -> Mul against the oracle's chain (approximate erf), and after fuse_gelu
+    against the oracle's Gelu (tanh form): each path matches its own reference path."""
+    case("session cfg3 gelu")
+    c = synth.cfg3(batch=2)
+    m = Model()
+    x = m.new_val_named_and_shaped("x", c["x"].shape)
+    out = erf_gelu_chain(m, x, sqrt2=float(c["sqrt2"]))
+    m.add_input(x)
+    m.add_output(out)
+    fused = m.clone()
+    assert fused.fuse_gelu() == 1
+
+    (got,) = HipSessionBuilder(m).build().run([c["x"]])
+    t = O.binary(O.DIV, c["x"], np.array(c["sqrt2"], np.float32))
+    t = O.binary(O.ADD, O.unary(O.ERF, t), np.array(1.0, np.float32))
+    want = O.binary(O.MUL, O.binary(O.MUL, c["x"], t), np.array(0.5, np.float32))
+    assert_bits_equal(got, want, "cfg3 erf chain")
+
+    (gf,) = HipSessionBuilder(fused).build().run([c["x"]])
+    assert_bits_equal(gf, O.unary(O.GELU, c["x"]), "cfg3 fused gelu")
+    assert np.max(np.abs(gf - got)) < 5e-2     # the two reference paths differ by the erf approximation
+
+
+def test_cfg3_squeeze_excite(case):
+    """ReduceMean over H,W -> HardSigmoid(1/6, 0.5) -> Mul back onto NCHW.  The reference interpreter
+    has no kernel for the two-axis mean; the oracle computes it per the ONNX definition."""
+    case("session cfg3 squeeze-excite")
+    c = synth.cfg3(batch=4)
+    m = Model()
+    x = m.new_val_named_and_shaped("se", c["se"].shape)
+    s, h, y = m.new_val(), m.new_val(), m.new_val_named("y")
+    m.add_node(Op.ReduceMean, [x], [s], axes=[2, 3], keep_dims=True)
+    m.add_node(Op.HardSigmoid, [s], [h], alpha=float(c["alpha"]), beta=float(c["beta"]))
+    m.add_node(Op.Mul, [x, h], [y])
+    m.add_input(x)
+    m.add_output(y)
+    (got,) = HipSessionBuilder(m).build().run([c["se"]])
+    info = {}
+    mean = O.reduce(O.REDUCE_MEAN, c["se"], [2, 3], True, info=info)
+    assert info["no_reference_kernel"] and mean.shape == (4, 576, 1, 1)
+    want = O.binary(O.MUL, c["se"], O.unary(O.HARDSIGMOID, mean, c["alpha"], c["beta"]))
+    assert_close(got, want, what="cfg3 squeeze-excite")
+
+
+def test_cfg4_pipeline(case):
+    case("session cfg4")
+    c = synth.cfg4(batch=4)
+    m = Model()
+    s = m.new_val_named_and_shaped("scores", c["scores"].shape)
+    mask = m.new_val_named_and_shaped("mask", c["mask"].shape)
+    r = m.new_val_named_and_shaped("r", c["rmax_in"].shape)
+    d = m.new_val_named_and_shaped("d", c["div_in"].shape)
+    k = m.new_initializer(np.array(c["div_scalar"], np.float32))
+    z, p, mx, q = (m.new_val() for _ in range(4))
+    m.add_node(Op.Add, [s, mask], [z])
+    m.add_node(Op.Softmax, [z], [p], axis=-1)
+    m.add_node(Op.ReduceMax, [r], [mx], axes=[1], keep_dims=False)
+    m.add_node(Op.Div, [d, k], [q])
+    for v in (s, mask, r, d):
+        m.add_input(v)
+    for v in (p, mx, q):
+        m.add_output(v)
+    p_out, mx_out, q_out = HipSessionBuilder(m).build().run([c["scores"], c["mask"], c["rmax_in"], c["div_in"]])
+    assert_close(p_out, O.softmax(O.binary(O.ADD, c["scores"], c["mask"])), what="cfg4 softmax")
+    assert mx_out.shape == (4, 197)
+    assert_bits_equal(mx_out, O.reduce(O.REDUCE_MAX, c["rmax_in"], [1], False), "cfg4 reducemax")
+    assert_bits_equal(q_out, O.binary(O.DIV, c["div_in"], np.array(c["div_scalar"], np.float32)), "cfg4 div")
+
+
+def test_reference_reduce_kernels(case):
+    """The two reductions the reference implements: ReduceMean(axis 2 of rank 3, keepdims) and
+    ReduceMax(all axes, keepdims=0) (crates/altius_py/tests/test_ops_reduce.py:10-41)."""
+    case("session reference reductions")
+    x = synth.uniform(7, [1, 50, 70])
+    for op, kind, kw, shape in ((Op.ReduceMean, O.REDUCE_MEAN, dict(axes=[-1], keep_dims=True), [1, 50, 1]),
+                                (Op.ReduceMax, O.REDUCE_MAX, dict(axes=[], keep_dims=False), [1])):
+        m = Model()
+        a = m.new_val_named_and_shaped("x", x.shape)
+        y = m.new_val_named("y")
+        m.add_node(op, [a], [y], **kw)
+        m.add_input(a)
+        m.add_output(y)
+        (got,) = HipSessionBuilder(m).build().run([x])
+        info = {}
+        want = O.reduce(kind, x, kw["axes"], kw["keep_dims"], strict=True, info=info)
+        assert list(got.shape) == shape and not info["no_reference_kernel"]
+        assert_close(got, want, what=f"reduce {op}")
+
+
+def test_identity_and_sigmoid_sqrt_relu_tanh(case):
+    case("session unary chain")
+    x = synth.normal(9, [3, 1, 28, 28], std=2.0)
+    m = Model()
+    a = m.new_val_named_and_shaped("x", x.shape)
+    v = [m.new_val() for _ in range(6)]
+    m.add_node(Op.Identity, [a], [v[0]])
+    m.add_node(Op.Sigmoid, [v[0]], [v[1]])
+    m.add_node(Op.Sqrt, [v[1]], [v[2]])
+    m.add_node(Op.Tanh, [v[2]], [v[3]])
+    m.add_node(Op.ReLU, [a], [v[4]])
+    m.add_node(Op.Identity, [v[4]], [v[5]])
+    m.add_input(a)
+    m.add_output(v[3])
+    m.add_output(v[5])
+    assert m.eliminate_identity() == 1   # the one feeding a graph output stays
+    got1, got2 = HipSessionBuilder(m).build().run([x])
+    assert_bits_equal(got1, O.unary(O.TANH, O.unary(O.SQRT, O.unary(O.SIGMOID, x))), "sigmoid-sqrt-tanh")
+    assert_bits_equal(got2, O.unary(O.RELU, x), "relu-identity")
+
+
+def test_errors_come_back_as_values(case):
+    case("session errors")
+    # an operator this backend has no kernel for: refused when the session is built
+    m = Model()
+    a = m.new_val_named_and_shaped("a", [2, 3])
+    c = m.new_val()
+    m.add_node(Op.Clip, [a], [c])
+    m.add_input(a)
+    m.add_output(c)
+    with pytest.raises(AltiusHipError) as e:
+        HipSessionBuilder(m).build()
+    assert e.value.code == ERR_SHAPE and "Clip" in e.value.message
+
+    # ... and at run time when shapes were not known at build time (session.rs:200)
+    m = Model()
+    a, c = m.new_val_named("a"), m.new_val()
+    m.add_node(Op.Clip, [a], [c])
+    m.add_input(a)
+    m.add_output(c)
+    sess = HipSessionBuilder(m).build()
+    with pytest.raises(AltiusHipError) as e:
+        sess.run([np.zeros([2, 3], np.float32)])
+    assert "Clip" in e.value.message
+
+    sess = HipSessionBuilder(binary_model(Op.Add)).build()
+    with pytest.raises(AltiusHipError) as e:   # shapes that do not broadcast (test_ops_bin.py:31-40)
+        sess.run([np.zeros([1, 3, 28, 28], np.float32), np.zeros([3, 1, 2], np.float32)])
+    assert e.value.code == ERR_SHAPE
+    with pytest.raises(AltiusHipError) as e:   # too few inputs
+        sess.run([np.zeros([2], np.float32)])
+    assert e.value.code == ERR_ARG
+    with pytest.raises(AltiusHipError) as e:   # not f32
+        sess.run([np.zeros([2], np.int64), np.zeros([2], np.int64)])
+    assert e.value.code == ERR_UNSUPPORTED
+    # the session is still usable after errors
+    (z,) = sess.run([np.ones([2], np.float32), np.ones([2], np.float32)])
+    assert z.tolist() == [2.0, 2.0]
+
+    # Softmax / LayerNormalization over an axis that is not the last (session.rs:999, 1444-1447)
+    for op, extra in ((Op.Softmax, []), (Op.LayerNormalization, [np.ones(3, np.float32), np.ones(3, np.float32)])):
+        m = Model()
+        a = m.new_val_named_and_shaped("a", [2, 3, 4])
+        ins = [a] + [m.new_initializer(t) for t in extra]
+        c = m.new_val()
+        m.add_node(op, ins, [c], axis=1)
+        m.add_input(a)
+        m.add_output(c)
+        sess = HipSessionBuilder(m).build()
+        with pytest.raises(AltiusHipError) as e:
+            sess.run([np.zeros([2, 3, 4], np.float32)])
+        assert e.value.code == ERR_UNSUPPORTED
+
+    with pytest.raises(AltiusHipError):        # no such GPU
+        HipSessionBuilder(binary_model(Op.Add)).with_device(99).build()
+
+
+def test_session_model_accessor_and_threads_option(case):
+    case("session model()")
+    m = binary_model(Op.Sub)
+    sess = HipSessionBuilder(m).with_intra_op_num_threads(16).build()
+    view = sess.model()
+    assert [n["op_name"] for n in view.nodes()] == ["Sub"] and view.inputs == m.inputs
+    (z,) = sess.run([np.full([5], 3, np.float32), np.full([5], 1, np.float32)])
+    assert z.tolist() == [2.0] * 5

@@ -1,0 +1,340 @@
+"""Host-side logic behind the C ABI, no GPU needed: the library loads and exports every
+symbol the header declares, broadcasting index math, graph IR, topological order, execution
+plan, shape inference and the fusion passes.  Expectations come from the reference's own unit
+tests and from the documented behaviour of its functions (cited per test)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from altius_amd import _lib
+from altius_amd import device as D
+from altius_amd._lib import ERR_ARG, ERR_SHAPE, AltiusHipError
+from altius_amd.graph import F32, I64, Model, Op, Tensor
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "altius_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    names = set(re.findall(r"\b(ahip_[a-z0-9_]+)\s*\(", header))
+    assert len(names) >= 60
+    L = ctypes.CDLL(_lib.LIB_PATH)
+    missing = [n for n in sorted(names) if not hasattr(L, n)]
+    assert not missing, f"declared but not exported: {missing}"
+
+
+def test_no_cpu_fallback_when_library_is_missing(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libaltius_hip.so"))
+    with pytest.raises(ImportError):
+        _lib.lib()
+
+
+def test_broadcast_reference_unit_tests():
+    """crates/core/src/fixed_dim.rs:192-245."""
+    assert D.broadcast_shape([1], [1]) == [1]
+    assert D.broadcast_shape([1], [4, 1]) == [4, 1]
+    assert D.broadcast_shape([4, 1], [1]) == [4, 1]
+    with pytest.raises(AltiusHipError) as e:
+        D.broadcast_shape([10, 20, 30], [10, 20])
+    assert e.value.code == ERR_SHAPE
+    assert D.broadcast_shape([1, 3, 3], [5, 1, 3, 3]) == [5, 1, 3, 3]
+    assert D.broadcast_shape([1, 3, 1], [5, 3, 10]) == [5, 3, 10]
+    assert D.broadcast_shape([1, 3, 4, 4], [3, 1, 1]) == [1, 3, 4, 4]
+    assert D.broadcast_shape([], []) == []
+
+
+@pytest.mark.parametrize("a,b", [
+    ([1, 3, 28, 28], [3, 1, 1]), ([1, 12, 9, 9], [1, 1, 1, 9]), ([4, 1, 2], [3, 1]), ([3, 28, 28], [3, 28, 1]),
+    ([3, 15, 15], [15]), ([3, 28, 28], [1]), ([1, 197, 768], [768]), ([256, 12, 197, 197], [256, 1, 1, 197]),
+    ([32, 197, 768], [32, 197, 1]), ([32, 576, 7, 7], [32, 576, 1, 1]), ([5, 1, 7, 1, 3], [1, 6, 1, 2, 3]), ([2, 3], []),
+])
+def test_strides_agree_with_oracle_and_numpy(oracle, a, b):
+    """Tensor::strides_for_broadcasting (crates/core/src/tensor.rs:369-406): integer, must be exact."""
+    out = D.broadcast_shape(a, b)
+    assert tuple(out) == np.broadcast_shapes(tuple(a), tuple(b))
+    for src in (a, b):
+        assert D.strides_for_broadcasting(src, out) == oracle.strides_for_broadcasting(src, out)
+    assert D.strides_for_broadcasting([256, 1, 1, 197], [256, 12, 197, 197]) == [197, 0, 0, 1]
+    with pytest.raises(AltiusHipError):
+        D.strides_for_broadcasting([3, 1, 2], [1, 3, 28, 28])
+
+
+def chain_model():
+    """x -> Relu -> Sigmoid -> (Add with x) -> out, plus a side branch that is a second output."""
+    m = Model()
+    x = m.new_val_named_and_shaped("x", [2, 3])
+    a, b, c, d = (m.new_val_named(n) for n in "abcd")
+    n_add = m.add_node(Op.Add, [b, x], [c], name="add")     # added first: order must come from the data flow
+    n_relu = m.add_node(Op.ReLU, [x], [a], name="relu")
+    n_sig = m.add_node(Op.Sigmoid, [a], [b], name="sigmoid")
+    n_sqrt = m.add_node(Op.Sqrt, [a], [d], name="sqrt")
+    m.add_input(x)
+    m.add_output(c)
+    m.add_output(d)
+    return m, (x, a, b, c, d), (n_add, n_relu, n_sig, n_sqrt)
+
+
+def test_graph_round_trip_and_named_lookup():
+    m, (x, a, b, c, d), (n_add, n_relu, n_sig, n_sqrt) = chain_model()
+    assert m.inputs == [x] and m.outputs == [c, d]
+    assert m.lookup_named_value("b") == b and m.lookup_named_value("nope") is None
+    node = m.node(n_add)
+    assert node["op_name"] == "Add" and node["inputs"] == [b, x] and node["outputs"] == [c]
+    assert [_lib.lib().ahip_op_name(i).decode() for i in (Op.ReLU, Op.LayerNormalization, Op.FusedElemwise)] == [
+        "ReLU", "LayerNormalization", "FusedElemwise"]  # Op::name (crates/core/src/op.rs:324-376)
+
+
+def test_topological_order_and_execution_plan():
+    """create_execution_plan (crates/session/src/plan.rs:14-58): each value is freed after its last
+    reader; graph outputs are never freed."""
+    m, (x, a, b, c, d), (n_add, n_relu, n_sig, n_sqrt) = chain_model()
+    order = m.topo_sort_nodes()
+    assert sorted(order) == sorted([n_add, n_relu, n_sig, n_sqrt])
+    pos = {n: i for i, n in enumerate(order)}
+    assert pos[n_relu] < pos[n_sig] < pos[n_add] and pos[n_relu] < pos[n_sqrt]
+    plan = m.execution_plan()
+    assert [n for n, _ in plan] == order
+    frees = {n: f for n, f in plan}
+    last_reader_of_a = n_sig if pos[n_sig] > pos[n_sqrt] else n_sqrt
+    assert frees[last_reader_of_a] == [a]
+    assert frees[n_add] == [b]
+    assert all(v not in (c, d, x) for f in frees.values() for v in f)
+
+
+def test_shape_inference():
+    """crates/core/src/analysis/shape.rs:89-94, 354-411, 590-611."""
+    m = Model(opset_version=13)
+    x = m.new_val_named_and_shaped("x", [4, 12, 197, 197])
+    mask = m.new_val_named_and_shaped("mask", [4, 1, 1, 197])
+    y = m.new_val_named_and_shaped("y", [4, 768, 197])
+    s, p, r1, r2, r3, r4 = (m.new_val() for _ in range(6))
+    m.add_node(Op.Add, [x, mask], [s])
+    m.add_node(Op.Softmax, [s], [p], axis=-1)
+    m.add_node(Op.ReduceMax, [y], [r1], axes=[1], keep_dims=False)
+    m.add_node(Op.ReduceMax, [y], [r2], axes=[], keep_dims=False)
+    m.add_node(Op.ReduceMean, [y], [r3], axes=[-1], keep_dims=True)
+    m.add_node(Op.ReduceMean, [y], [r4], axes=[], keep_dims=True)
+    for v in (x, mask, y):
+        m.add_input(v)
+    assert m.infer_value_shape(s) == ([4, 12, 197, 197], F32)
+    assert m.infer_value_shape(p) == ([4, 12, 197, 197], F32)
+    assert m.infer_value_shape(r1) == ([4, 197], F32)
+    assert m.infer_value_shape(r2) == ([1], F32)            # full reduction without keepdims -> [1]
+    assert m.infer_value_shape(r3) == ([4, 768, 1], F32)
+    assert m.infer_value_shape(r4) == ([4, 768, 197], F32)  # ReduceMean without axes reduces nothing
+
+
+def test_shape_inference_errors_are_values_not_aborts():
+    m = Model()
+    a = m.new_val_named_and_shaped("a", [1, 3, 28, 28])
+    b = m.new_val_named_and_shaped("b", [3, 1, 2])
+    c = m.new_val()
+    m.add_node(Op.Add, [a, b], [c])
+    m.add_input(a)
+    m.add_input(b)
+    with pytest.raises(AltiusHipError) as e:  # the reference unwrap()s None here and panics
+        m.infer_value_shape(c)
+    assert e.value.code == ERR_SHAPE and "broadcast" in e.value.message
+
+    m = Model()
+    a = m.new_val_named_and_shaped("a", [None, 3])  # dynamic dimension: "Must be fixed dimension" (shape.rs:675)
+    c = m.new_val()
+    m.add_node(Op.ReLU, [a], [c])
+    m.add_input(a)
+    with pytest.raises(AltiusHipError) as e:
+        m.infer_value_shape(c)
+    assert e.value.code == ERR_SHAPE
+
+    m = Model()
+    a = m.new_val_named("a")  # no declared shape: nodes are skipped, inferred at run time (shape.rs:704-706)
+    c = m.new_val()
+    m.add_node(Op.ReLU, [a], [c])
+    m.add_input(a)
+    with pytest.raises(AltiusHipError) as e:
+        m.infer_value_shape(c)
+    assert e.value.code == ERR_ARG
+
+    m = Model(opset_version=18)  # ReduceMax asserts opset <= 13 (shape.rs:355)
+    a = m.new_val_named_and_shaped("a", [2, 3])
+    c = m.new_val()
+    m.add_node(Op.ReduceMax, [a], [c], axes=[1])
+    m.add_input(a)
+    with pytest.raises(AltiusHipError):
+        m.infer_value_shape(c)
+
+    m = Model()
+    a = m.new_val_named_and_shaped("a", [2, 3])
+    c = m.new_val()
+    m.add_node(Op.MatMul, [a, a], [c])  # outside this backend
+    m.add_input(a)
+    with pytest.raises(AltiusHipError) as e:
+        m.infer_value_shape(c)
+    assert "MatMul" in e.value.message
+
+
+def layer_norm_chain(m, x, gamma, beta, eps=1e-5):
+    """The 9-node chain ONNX exporters emit for LayerNorm (crates/core/src/optimize/layer_norm_fusion.rs:9-16)."""
+    two = m.new_initializer(np.array(2.0, np.float32))
+    e = m.new_initializer(np.array(eps, np.float32))
+    g = m.new_initializer(gamma)
+    b = m.new_initializer(beta)
+    v = [m.new_val() for _ in range(9)]
+    m.add_node(Op.ReduceMean, [x], [v[0]], axes=[-1], keep_dims=True)
+    m.add_node(Op.Sub, [x, v[0]], [v[1]])
+    m.add_node(Op.Pow, [v[1], two], [v[2]])
+    m.add_node(Op.ReduceMean, [v[2]], [v[3]], axes=[-1], keep_dims=True)
+    m.add_node(Op.Add, [v[3], e], [v[4]])
+    m.add_node(Op.Sqrt, [v[4]], [v[5]])
+    m.add_node(Op.Div, [v[1], v[5]], [v[6]])
+    m.add_node(Op.Mul, [v[6], g], [v[7]])
+    m.add_node(Op.Add, [v[7], b], [v[8]])
+    return v[8], g, b
+
+
+def test_fuse_layer_norm():
+    m = Model()
+    x = m.new_val_named_and_shaped("x", [2, 5, 8])
+    out, g, b = layer_norm_chain(m, x, np.ones(8, np.float32), np.zeros(8, np.float32), eps=1e-6)
+    tail = m.new_val()
+    m.add_node(Op.ReLU, [out], [tail])
+    m.add_input(x)
+    m.add_output(tail)
+    assert len(m.nodes()) == 10
+    assert m.fuse_layer_norm() == 1
+    nodes = m.nodes()
+    assert [n["op_name"] for n in nodes] == ["LayerNormalization", "ReLU"]
+    ln = nodes[0]
+    assert ln["inputs"] == [x, g, b] and ln["axis"] == -1 and ln["stash_type"] == 1
+    assert ln["epsilon"] == np.float32(1e-6)               # taken from the Add's initializer (:128)
+    assert nodes[1]["inputs"] == ln["outputs"]             # the chain's reader now reads the fused node
+    assert m.fuse_layer_norm() == 0
+
+    # the chain's result as a graph output: the output is rewired (layer_norm_fusion.rs:141-145)
+    m = Model()
+    x = m.new_val_named_and_shaped("x", [2, 8])
+    out, _, _ = layer_norm_chain(m, x, np.ones(8, np.float32), np.zeros(8, np.float32))
+    m.add_input(x)
+    m.add_output(out)
+    assert m.fuse_layer_norm() == 1
+    (ln,) = m.nodes()
+    assert m.outputs == ln["outputs"]
+
+    # a chain that stops early is left alone
+    m = Model()
+    x = m.new_val_named_and_shaped("x", [2, 8])
+    a, b2 = m.new_val(), m.new_val()
+    m.add_node(Op.ReduceMean, [x], [a], axes=[-1])
+    m.add_node(Op.Sub, [x, a], [b2])
+    m.add_input(x)
+    m.add_output(b2)
+    assert m.fuse_layer_norm() == 0 and len(m.nodes()) == 2
+
+
+def erf_gelu_chain(m, x, sqrt2=1.4142135):
+    c = m.new_initializer(np.array(sqrt2, np.float32))
+    one = m.new_initializer(np.array(1.0, np.float32))
+    half = m.new_initializer(np.array(0.5, np.float32))
+    v = [m.new_val() for _ in range(5)]
+    m.add_node(Op.Div, [x, c], [v[0]])
+    m.add_node(Op.Erf, [v[0]], [v[1]])
+    m.add_node(Op.Add, [v[1], one], [v[2]])
+    m.add_node(Op.Mul, [x, v[2]], [v[3]])
+    m.add_node(Op.Mul, [v[3], half], [v[4]])
+    return v[4]
+
+
+def test_fuse_gelu():
+    """crates/core/src/optimize/gelu_fusion.rs:12-82."""
+    m = Model()
+    x = m.new_val_named_and_shaped("x", [1, 2, 3])
+    out = erf_gelu_chain(m, x)
+    m.add_input(x)
+    m.add_output(out)
+    assert m.fuse_gelu() == 1
+    (g,) = m.nodes()
+    assert g["op_name"] == "Gelu" and g["inputs"] == [x] and m.outputs == g["outputs"]
+
+    m = Model()  # a divisor that is not sqrt(2) within 1e-5: no fusion (:18-24)
+    x = m.new_val_named_and_shaped("x", [1, 2, 3])
+    out = erf_gelu_chain(m, x, sqrt2=1.5)
+    m.add_input(x)
+    m.add_output(out)
+    assert m.fuse_gelu() == 0 and len(m.nodes()) == 5
+
+
+def test_fuse_fast_gelu():
+    """crates/core/src/optimize/fast_gelu_fusion.rs:5-190: the tanh form with x produced by a node."""
+    m = Model()
+    x0 = m.new_val_named_and_shaped("x0", [2, 4])
+    x = m.new_val()
+    m.add_node(Op.ReLU, [x0], [x])
+    three = m.new_initializer(np.array(3.0, np.float32))
+    c1 = m.new_initializer(np.array(0.044715, np.float32))
+    c2 = m.new_initializer(np.array(0.7978845608, np.float32))
+    one = m.new_initializer(np.array(1.0, np.float32))
+    half = m.new_initializer(np.array(0.5, np.float32))
+    v = [m.new_val() for _ in range(8)]
+    m.add_node(Op.Pow, [x, three], [v[0]])
+    m.add_node(Op.Mul, [v[0], c1], [v[1]])
+    m.add_node(Op.Add, [x, v[1]], [v[2]])
+    m.add_node(Op.Mul, [v[2], c2], [v[3]])
+    m.add_node(Op.Tanh, [v[3]], [v[4]])
+    m.add_node(Op.Add, [v[4], one], [v[5]])
+    m.add_node(Op.Mul, [x, half], [v[6]])
+    m.add_node(Op.Mul, [v[6], v[5]], [v[7]])
+    tail = m.new_val()
+    m.add_node(Op.Sqrt, [v[7]], [tail])
+    m.add_input(x0)
+    m.add_output(tail)
+    assert m.fuse_fast_gelu() == 1
+    names = [n["op_name"] for n in m.nodes()]
+    assert names == ["ReLU", "Gelu", "Sqrt"]
+    gelu = m.nodes()[1]
+    assert gelu["inputs"] == [x] and m.nodes()[2]["inputs"] == gelu["outputs"]
+
+
+def test_eliminate_identity():
+    """crates/core/src/optimize/identity_elim.rs:5-45: readers are rewired; an Identity feeding a graph
+    output stays."""
+    m = Model()
+    x = m.new_val_named_and_shaped("x", [3])
+    a, b, c = m.new_val(), m.new_val(), m.new_val()
+    m.add_node(Op.Identity, [x], [a])
+    m.add_node(Op.ReLU, [a], [b])
+    m.add_node(Op.Identity, [b], [c])
+    m.add_input(x)
+    m.add_output(c)
+    assert m.eliminate_identity() == 1
+    nodes = m.nodes()
+    assert [n["op_name"] for n in nodes] == ["ReLU", "Identity"] and nodes[0]["inputs"] == [x]
+
+
+def test_argument_errors():
+    m = Model()
+    x = m.new_val()
+    L = _lib.lib()
+    assert L.ahip_model_add_input(m.handle, 999) == ERR_ARG
+    assert L.ahip_model_add_node(m.handle, 999, None, None, 0, None, 0, None, None) == ERR_ARG
+    bad = (ctypes.c_int64 * 1)(42)
+    assert L.ahip_model_add_node(m.handle, Op.ReLU, None, None, 1, bad, 0, None, None) == ERR_ARG
+    assert b"unknown input" in L.ahip_last_error(None)
+    with pytest.raises(AltiusHipError):  # initializer whose byte count does not match its shape
+        check_dims = (ctypes.c_int64 * 1)(4)
+        data = np.zeros(3, np.float32)
+        _lib.check(L.ahip_model_add_initializer(m.handle, x, F32, 1, check_dims, data.ctypes.data, data.nbytes))
+    assert L.ahip_session_builder_new(None, None) == ERR_ARG
+    assert L.ahip_tensor_new(7, 0, None, None, 0, None) == ERR_ARG
+
+
+def test_host_tensor_round_trip():
+    for arr in (np.arange(24, dtype=np.float32).reshape(2, 3, 4), np.array(5, np.int64), np.zeros((0, 3), np.float32)):
+        t = Tensor.from_numpy(arr)
+        assert t.dims == list(arr.shape)
+        back = t.numpy()
+        assert back.dtype == arr.dtype and np.array_equal(back, arr)
+    assert Tensor.from_numpy(np.array([1, 2], np.int64)).elem_ty == I64

@@ -201,6 +201,20 @@ def test_gelu_is_the_tanh_form(oracle):
         assert_bits_equal(oracle.unary(2, x, threads=t), got, "gelu threads")
 
 
+def test_tanh_rational(oracle):
+    """session.rs:840-903: rational tanh on [-9, 9]; Gelu is built on the same function."""
+    half = np.linspace(0, 12, 2401, dtype=np.float32)
+    x = np.concatenate([-half[::-1], half])
+    got = oracle.unary(6, x)
+    np.testing.assert_allclose(got, np.tanh(x.astype(np.float64)), rtol=0, atol=5e-7)
+    assert got[0] == -1.0 and got[-1] == 1.0 and oracle.unary(6, np.zeros(1, np.float32))[0] == 0
+    assert_bits_equal(got, -got[::-1], "tanh odd")
+    # Gelu(x) == (tanh(x(B + Cx^2)) + 1) * (x/2) with the same rounding steps
+    B, C = np.float32(0.7978845608028654), np.float32(0.035677408136300125)
+    inner = x * (C * x * x + B)
+    assert_bits_equal(oracle.unary(2, x), (oracle.unary(6, inner) + np.float32(1)) * (x * np.float32(0.5)), "gelu via tanh")
+
+
 def test_erf_loose_bounds(oracle):
     """PARITY UNPINNED at the bit level (fastapprox is not vendored); only the reference's own
     bound is checked: |erf - exact| <= 1e-1 (test_ops_elemwise.py:129-152)."""
