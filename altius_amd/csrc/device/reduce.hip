@@ -183,9 +183,12 @@ __global__ __launch_bounds__(COL_BLOCK) void reduce_cols(float *__restrict__ dst
 // do the 4*inner accumulators go through LDS, where column c collects positions
 // c, c + inner, c + 2*inner, c + 3*inner of every wave.  Rows left over when the
 // reduced extent is not a multiple of 4 are folded in by the last split.
-// grid = (outer * splits); dynamic LDS = COL_WAVES * 4 * inner floats.
+// grid = (outer * splits); dynamic LDS = FLAT_WAVES * 4 * inner floats.
+constexpr int FLAT_BLOCK = 1024;
+constexpr int FLAT_WAVES = FLAT_BLOCK / WAVE;
+
 template <class OP, int NCH, bool SCALE, bool NT>
-__global__ __launch_bounds__(COL_BLOCK) void reduce_cols_flat4(float *__restrict__ dst,
+__global__ __launch_bounds__(FLAT_BLOCK) void reduce_cols_flat4(float *__restrict__ dst,
                                                                const float *__restrict__ in, uint32_t red,
                                                                uint32_t inner, uint32_t splits,
                                                                uint32_t groups_per_split, float scale) {
@@ -205,9 +208,9 @@ __global__ __launch_bounds__(COL_BLOCK) void reduce_cols_flat4(float *__restrict
     for (int k = 0; k < NCH; k++) acc[k] = make_float4(OP::identity(), OP::identity(), OP::identity(), OP::identity());
 
     uint32_t g = g_begin + wave;
-    for (; g + COL_WAVES < g_end; g += 2 * COL_WAVES) {  // two groups in flight
+    for (; g + FLAT_WAVES < g_end; g += 2 * FLAT_WAVES) {  // two groups in flight
         const float *p0 = slab + g * group_floats;
-        const float *p1 = p0 + COL_WAVES * group_floats;
+        const float *p1 = p0 + FLAT_WAVES * group_floats;
         float4 v0[NCH], v1[NCH];
 #pragma unroll
         for (int k = 0; k < NCH; k++) {
@@ -228,7 +231,7 @@ __global__ __launch_bounds__(COL_BLOCK) void reduce_cols_flat4(float *__restrict
             }
         }
     }
-    for (; g < g_end; g += COL_WAVES) {
+    for (; g < g_end; g += FLAT_WAVES) {
         const float *p0 = slab + g * group_floats;
 #pragma unroll
         for (int k = 0; k < NCH; k++) {
@@ -250,9 +253,9 @@ __global__ __launch_bounds__(COL_BLOCK) void reduce_cols_flat4(float *__restrict
         if (f < inner) *reinterpret_cast<float4 *>(mine + 4 * f) = acc[k];
     }
     __syncthreads();
-    for (uint32_t c = threadIdx.x; c < inner; c += COL_BLOCK) {
+    for (uint32_t c = threadIdx.x; c < inner; c += FLAT_BLOCK) {
         float a = OP::identity();
-        for (int w = 0; w < COL_WAVES; w++)
+        for (int w = 0; w < FLAT_WAVES; w++)
 #pragma unroll
             for (int p = 0; p < 4; p++) a = OP::apply(a, lds4[w * group_floats + p * inner + c]);
         if (s == splits - 1)
@@ -314,8 +317,8 @@ template <class OP, bool SCALE>
 void cols_flat4_launch(hipStream_t s, float *dst, const float *in, size_t outer, size_t red, size_t inner,
                        size_t splits, size_t groups_per_split, float scale, bool nt) {
     const dim3 grid((unsigned)(outer * splits));
-    const dim3 block(COL_BLOCK);
-    const size_t shmem = (size_t)COL_WAVES * 4 * inner * sizeof(float);
+    const dim3 block(FLAT_BLOCK);
+    const size_t shmem = (size_t)FLAT_WAVES * 4 * inner * sizeof(float);
     const int nch = (int)((inner + WAVE - 1) / WAVE);
 #define ALTIUS_LAUNCH(N, T)                                                                                    \
     hipLaunchKernelGGL((reduce_cols_flat4<OP, N, SCALE, T>), grid, block, shmem, s, dst, in, (uint32_t)red,    \
@@ -374,10 +377,12 @@ int reduce_impl(DeviceCtx &ctx, float *out, const float *in, size_t outer, size_
     // Unaligned rows of moderate width: the 16-byte flat variant.
     if (inner % 4 != 0 && inner <= 256 && red >= 16 && aligned16(in) && (outer == 1 || (red * inner) % 4 == 0)) {
         const size_t groups = red / 4;
+        // One 16-wave block per slab fills the chip once there are about as many slabs as CUs;
+        // with fewer slabs the reduced axis is split over blocks and a second launch folds the parts.
         size_t fsplits = 1;
-        if (outer < 1024) {
-            fsplits = (1024 + outer - 1) / outer;
-            const size_t max_splits = groups / 16 > 0 ? groups / 16 : 1;  // two groups per wave at least
+        if (outer < 192) {
+            fsplits = (512 + outer - 1) / outer;
+            const size_t max_splits = groups / 32 > 0 ? groups / 32 : 1;  // two groups per wave at least
             if (fsplits > max_splits) fsplits = max_splits;
         }
         size_t gps = (groups + fsplits - 1) / fsplits;

@@ -105,6 +105,9 @@ class Context:
         self.sync()
         return out
 
+    def memset(self, buf, byte_value):
+        check(self.L.ahip_memset_async(self.handle, buf.ptr, byte_value, buf.nbytes), self.handle)
+
     def sync(self):
         check(self.L.ahip_sync(self.handle), self.handle)
 
