@@ -20,7 +20,6 @@
 #include "math.h"
 
 #include <math.h>
-#include <stdlib.h>
 
 namespace altius {
 namespace {
@@ -117,24 +116,36 @@ __global__ __launch_bounds__(BLOCK) void softmax_wave(float *__restrict__ out, c
 
 // Rows whose length is not a multiple of 4 (197 tokens, say) start at addresses
 // that are only 4-byte aligned, and a wave per row would leave a quarter of its
-// lanes idle in the last chunk.  This kernel decouples the two layouts through
-// LDS.  One wavefront per block takes a group of G consecutive rows (G a
-// multiple of 4, so the group is a 16-byte aligned, contiguous span):
-//   1. the span is copied to LDS with 16-byte loads, every lane busy;
+// lanes idle in the last chunk.  This kernel decouples the memory layout from
+// the compute layout through LDS.  A block of 16 wavefronts takes a group of
+// consecutive rows whose span starts and ends on a 128-byte boundary (32 rows
+// when the length is odd), so no cache line is shared between blocks or between
+// the load/store instructions of different waves:
+//   1. the span is copied to LDS with 16-byte loads, thread t taking float4
+//      t and t + 1024; both loads are issued before the first LDS write.
+//      Measured on this part: copy bandwidth falls with the number of loads a
+//      wave issues back to back (6.6 TB/s at 1-2, 6.1 at 4, 5.5 at 13) and with
+//      spans that share cache lines between waves, hence wide blocks, shallow
+//      bursts and line-aligned groups;
 //   2. rows are processed from LDS with SUB = 16, 32 or 64 lanes per row
-//      (64/SUB rows at a time), NCH chunks per lane, max and sum all-reduced
-//      inside each lane group with DPP rotations; results overwrite the row;
+//      (64/SUB rows per wave pass, passes dealt round-robin to the waves), NCH
+//      chunks per lane, max and sum all-reduced inside each lane group with DPP
+//      rotations; results overwrite the row in LDS;
 //   3. the span is written back with 16-byte stores.
 // With SUB*NCH just above the row length nearly every lane slot of the
 // arithmetic does useful work (197 -> 16 x 13 = 208 slots).
-constexpr int STAGE = 16;                            // float4 per lane staged through registers
-constexpr size_t LDS_GROUP_FLOATS = STAGE * WAVE * 4;  // so a group holds at most 4096 floats
+constexpr int LDS_BLOCK = 1024;
+constexpr int LDS_WAVES = LDS_BLOCK / WAVE;
+constexpr int STAGE_LDS = 2;                                         // float4 per lane staged through registers
+constexpr size_t LDS_GROUP_FLOATS = (size_t)STAGE_LDS * LDS_BLOCK * 4;  // 8192 floats = 32 KiB of LDS at most
 
-template <int SUB, int NCH>
-__global__ __launch_bounds__(WAVE) void softmax_lds(float *__restrict__ out, const float *__restrict__ in,
-                                                    size_t rows, int len, int group_rows, int nt) {
+template <int SUB, int NCH, bool NT>
+__global__ __launch_bounds__(LDS_BLOCK) void softmax_lds(float *__restrict__ out, const float *__restrict__ in,
+                                                         size_t rows, int len, int group_rows) {
     extern __shared__ __align__(16) float lds[];
-    const int lane = threadIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1);
+    const int wave = tid >> 6;
     const size_t row0 = (size_t)blockIdx.x * group_rows;
     const int nrows = rows - row0 < (size_t)group_rows ? (int)(rows - row0) : group_rows;
     const int n = nrows * len;
@@ -142,75 +153,84 @@ __global__ __launch_bounds__(WAVE) void softmax_lds(float *__restrict__ out, con
     const float *src = in + row0 * (size_t)len;
     float *dst = out + row0 * (size_t)len;
 
-    // All of the group's loads are issued before the first LDS write, so one
-    // wave keeps up to STAGE KiB in flight.
-    float4 stage[STAGE];
-    if (nt) {
+    // Whether float4 number tid + 1024u exists is decided per block (scalar branch) except for the
+    // one partially filled step.
+    float4 stage[STAGE_LDS];
 #pragma unroll
-        for (int u = 0; u < STAGE; u++)
-            if (lane + WAVE * u < n4) stage[u] = load4<true>(src + 4 * (lane + WAVE * u));
-    } else {
-#pragma unroll
-        for (int u = 0; u < STAGE; u++)
-            if (lane + WAVE * u < n4) stage[u] = load4<false>(src + 4 * (lane + WAVE * u));
+    for (int u = 0; u < STAGE_LDS; u++) {
+        const float *p = src + 4 * (tid + LDS_BLOCK * u);
+        if (LDS_BLOCK * (u + 1) <= n4) {
+            stage[u] = load4<NT>(p);
+        } else if (LDS_BLOCK * u < n4) {
+            if (tid + LDS_BLOCK * u < n4) stage[u] = load4<NT>(p);
+        }
     }
 #pragma unroll
-    for (int u = 0; u < STAGE; u++)
-        if (lane + WAVE * u < n4) *reinterpret_cast<float4 *>(lds + 4 * (lane + WAVE * u)) = stage[u];
-    for (int i = (n4 << 2) + lane; i < n; i += WAVE) lds[i] = src[i];  // ragged end of the last group
+    for (int u = 0; u < STAGE_LDS; u++) {
+        float *q = lds + 4 * (tid + LDS_BLOCK * u);
+        if (LDS_BLOCK * (u + 1) <= n4) {
+            *reinterpret_cast<float4 *>(q) = stage[u];
+        } else if (LDS_BLOCK * u < n4) {
+            if (tid + LDS_BLOCK * u < n4) *reinterpret_cast<float4 *>(q) = stage[u];
+        }
+    }
+    for (int i = (n4 << 2) + tid; i < n; i += LDS_BLOCK) lds[i] = src[i];  // ragged end of the last group
     __syncthreads();
 
-    constexpr int RPP = WAVE / SUB;  // rows per pass
+    constexpr int RPP = WAVE / SUB;  // rows per wave pass
+    constexpr int LAST = NCH - 1;    // NCH == ceil(len / SUB): only the last chunk can be partial
     const int s = lane & (SUB - 1);
     const int rr = lane / SUB;
+    const bool last_valid = s + SUB * LAST < len;
     const float nan = __builtin_nanf("");
-    for (int r0 = 0; r0 < nrows; r0 += RPP) {
-        int r = r0 + rr;
-        const bool active = r < nrows;
-        if (!active) r = nrows - 1;  // idle lane groups recompute the last row and store nothing
+    for (int r0 = wave * RPP; r0 < nrows; r0 += LDS_WAVES * RPP) {
+        // Lane groups past the end of a ragged last group redo its last row: they compute and
+        // store the same values as the group that owns it.
+        const int r = r0 + rr < nrows ? r0 + rr : nrows - 1;
         float *row = lds + r * len + s;
 
         float x[NCH];
-        float mx = nan;
 #pragma unroll
-        for (int k = 0; k < NCH; k++) {
-            const bool full = SUB * (k + 1) <= len;  // uniform
-            x[k] = (full || s + SUB * k < len) ? row[SUB * k] : nan;
-            mx = nanmax(x[k], mx);
-        }
+        for (int k = 0; k < LAST; k++) x[k] = row[SUB * k];
+        x[LAST] = last_valid ? row[SUB * LAST] : nan;
+        float mx = nan;  // fold(NAN, max): NaN elements are ignored
+#pragma unroll
+        for (int k = 0; k < NCH; k++) mx = nanmax(x[k], mx);
         mx = subwave_allreduce<MaxOp, SUB>(mx);
 
         float sum = 0.0f;
 #pragma unroll
         for (int k = 0; k < NCH; k++) {
-            const bool full = SUB * (k + 1) <= len;
-            const float e = softmax_exp(x[k], mx);
-            x[k] = e;
-            sum += (full || s + SUB * k < len) ? e : 0.0f;
+            x[k] = softmax_exp(x[k], mx);
+            sum += (k < LAST || last_valid) ? x[k] : 0.0f;
         }
         sum = subwave_allreduce<SumOp, SUB>(sum);
         const float recip = 1.0f / sum;
 #pragma unroll
-        for (int k = 0; k < NCH; k++) {
-            const bool full = SUB * (k + 1) <= len;
-            if (active && (full || s + SUB * k < len)) row[SUB * k] = x[k] * recip;
-        }
+        for (int k = 0; k < LAST; k++) row[SUB * k] = x[k] * recip;
+        if (last_valid) row[SUB * LAST] = x[LAST] * recip;
     }
     __syncthreads();
 
 #pragma unroll
-    for (int u = 0; u < STAGE; u++)
-        if (lane + WAVE * u < n4) stage[u] = *reinterpret_cast<const float4 *>(lds + 4 * (lane + WAVE * u));
-    if (nt) {
-#pragma unroll
-        for (int u = 0; u < STAGE; u++)
-            if (lane + WAVE * u < n4) store4<true>(dst + 4 * (lane + WAVE * u), stage[u]);
-    } else {
-#pragma unroll
-        for (int u = 0; u < STAGE; u++)
-            if (lane + WAVE * u < n4) store4<false>(dst + 4 * (lane + WAVE * u), stage[u]);
+    for (int u = 0; u < STAGE_LDS; u++) {
+        const float *q = lds + 4 * (tid + LDS_BLOCK * u);
+        if (LDS_BLOCK * (u + 1) <= n4) {
+            stage[u] = *reinterpret_cast<const float4 *>(q);
+        } else if (LDS_BLOCK * u < n4) {
+            if (tid + LDS_BLOCK * u < n4) stage[u] = *reinterpret_cast<const float4 *>(q);
+        }
     }
-    for (int i = (n4 << 2) + lane; i < n; i += WAVE) dst[i] = lds[i];
+#pragma unroll
+    for (int u = 0; u < STAGE_LDS; u++) {
+        float *p = dst + 4 * (tid + LDS_BLOCK * u);
+        if (LDS_BLOCK * (u + 1) <= n4) {
+            store4<NT>(p, stage[u]);
+        } else if (LDS_BLOCK * u < n4) {
+            if (tid + LDS_BLOCK * u < n4) store4<NT>(p, stage[u]);
+        }
+    }
+    for (int i = (n4 << 2) + tid; i < n; i += LDS_BLOCK) dst[i] = lds[i];
 }
 
 // One block per row, any length: max pass, sum pass, write pass.
@@ -345,37 +365,72 @@ template <int VEC, int NCH> struct LayerNormLauncher {
 };
 
 // Launches softmax_lds with the lane-group width and chunk count that waste the
-// fewest lane slots for this row length (len <= 1024).
-template <int SUB> bool softmax_lds_launch_nch(int nch, dim3 grid, size_t shmem, hipStream_t s, float *out,
-                                               const float *in, size_t rows, int len, int g, int nt) {
-#define ALTIUS_CASE(N)                                                                                         \
-    case N:                                                                                                    \
-        hipLaunchKernelGGL((softmax_lds<SUB, N>), grid, dim3(WAVE), shmem, s, out, in, rows, len, g, nt);      \
-        return true;
-    switch (nch) {
-        ALTIUS_CASE(1) ALTIUS_CASE(2) ALTIUS_CASE(3) ALTIUS_CASE(4) ALTIUS_CASE(5) ALTIUS_CASE(6) ALTIUS_CASE(7)
-        ALTIUS_CASE(8) ALTIUS_CASE(9) ALTIUS_CASE(10) ALTIUS_CASE(11) ALTIUS_CASE(12) ALTIUS_CASE(13)
-        ALTIUS_CASE(14) ALTIUS_CASE(15) ALTIUS_CASE(16)
+// fewest lane slots for this row length (len <= 1024): 16 lanes per row up to
+// 256 elements, 32 up to 512, 64 above.
+template <int SUB, int NCH>
+void softmax_lds_go(bool nt, dim3 grid, size_t shmem, hipStream_t s, float *out, const float *in, size_t rows,
+                    int len, int g) {
+    if (nt)
+        hipLaunchKernelGGL((softmax_lds<SUB, NCH, true>), grid, dim3(LDS_BLOCK), shmem, s, out, in, rows, len, g);
+    else
+        hipLaunchKernelGGL((softmax_lds<SUB, NCH, false>), grid, dim3(LDS_BLOCK), shmem, s, out, in, rows, len, g);
+}
+
+size_t gcd_size(size_t a, size_t b) {
+    while (b) {
+        const size_t t = a % b;
+        a = b;
+        b = t;
     }
-#undef ALTIUS_CASE
-    return false;
+    return a;
+}
+
+// Rows per block: the smallest count whose span is a whole number of 128-byte lines (or of
+// 64/32/16 bytes when that would not fit), repeated up to the LDS budget.
+size_t softmax_lds_group_rows(size_t len) {
+    for (size_t align_floats = 32; align_floats >= 4; align_floats /= 2) {
+        const size_t base = align_floats / gcd_size(len, align_floats);
+        if (base * len <= LDS_GROUP_FLOATS) {
+            size_t m = LDS_GROUP_FLOATS / (base * len);
+            const size_t max_rows = 1024;
+            if (base * m > max_rows) m = max_rows / base > 0 ? max_rows / base : 1;
+            return base * m;
+        }
+    }
+    return 4;  // unreachable for len <= 1024: 4 rows are at most 4096 floats
 }
 
 bool softmax_lds_launch(hipStream_t s, float *out, const float *in, size_t rows, size_t len, bool nt) {
-    // Rows per group: a multiple of 4 (16-byte aligned groups, whole passes), about 12 KiB of LDS.
-    static const size_t target = getenv("AHIP_EXP_GROUP_FLOATS") ? (size_t)atoi(getenv("AHIP_EXP_GROUP_FLOATS")) : 3200;
-    size_t g = target / len / 4 * 4;
-    if (g < 4) g = 4;  // len <= 1024, so 4 rows still fit LDS_GROUP_FLOATS
-    if (g > 512) g = 512;
-    static_assert(4 * 1024 <= LDS_GROUP_FLOATS, "a group of 4 rows must fit the staging registers");
+    static_assert(4 * 1024 <= LDS_GROUP_FLOATS, "four rows of the longest supported length must fit");
+    const size_t g = softmax_lds_group_rows(len);
     const size_t groups = (rows + g - 1) / g;
     if (groups > 0x7FFFFFFFu) return false;
     const dim3 grid((unsigned)groups);
     const size_t shmem = g * len * sizeof(float);
-    const int L = (int)len, G = (int)g, NT = nt ? 1 : 0;
-    if (len <= 256) return softmax_lds_launch_nch<16>((L + 15) / 16, grid, shmem, s, out, in, rows, L, G, NT);
-    if (len <= 512) return softmax_lds_launch_nch<32>((L + 31) / 32, grid, shmem, s, out, in, rows, L, G, NT);
-    return softmax_lds_launch_nch<64>((L + 63) / 64, grid, shmem, s, out, in, rows, L, G, NT);
+    const int L = (int)len, G = (int)g;
+#define ALTIUS_GO(SUB, N)                                                    \
+    case N:                                                                  \
+        softmax_lds_go<SUB, N>(nt, grid, shmem, s, out, in, rows, L, G);     \
+        return true;
+    if (len <= 256) {
+        switch ((L + 15) / 16) {
+            ALTIUS_GO(16, 1) ALTIUS_GO(16, 2) ALTIUS_GO(16, 3) ALTIUS_GO(16, 4) ALTIUS_GO(16, 5) ALTIUS_GO(16, 6)
+            ALTIUS_GO(16, 7) ALTIUS_GO(16, 8) ALTIUS_GO(16, 9) ALTIUS_GO(16, 10) ALTIUS_GO(16, 11)
+            ALTIUS_GO(16, 12) ALTIUS_GO(16, 13) ALTIUS_GO(16, 14) ALTIUS_GO(16, 15) ALTIUS_GO(16, 16)
+        }
+    } else if (len <= 512) {
+        switch ((L + 31) / 32) {
+            ALTIUS_GO(32, 9) ALTIUS_GO(32, 10) ALTIUS_GO(32, 11) ALTIUS_GO(32, 12) ALTIUS_GO(32, 13)
+            ALTIUS_GO(32, 14) ALTIUS_GO(32, 15) ALTIUS_GO(32, 16)
+        }
+    } else {
+        switch ((L + 63) / 64) {
+            ALTIUS_GO(64, 9) ALTIUS_GO(64, 10) ALTIUS_GO(64, 11) ALTIUS_GO(64, 12) ALTIUS_GO(64, 13)
+            ALTIUS_GO(64, 14) ALTIUS_GO(64, 15) ALTIUS_GO(64, 16)
+        }
+    }
+#undef ALTIUS_GO
+    return false;
 }
 
 constexpr size_t MAX_WAVE_ROW = 1024;
