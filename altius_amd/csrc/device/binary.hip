@@ -209,6 +209,76 @@ __global__ __launch_bounds__(BLOCK) void binary_strided(float *__restrict__ out,
     }
 }
 
+// ---------------------------------------------------------------------------
+// Row-broadcast kernel: out[n][r][c] = full[n][r][c] op small[n][c] (an attention
+// mask [N,1,1,C] on scores [N,H,S,C], a bias [C] on [.., C]).  The block's one or
+// two rows of the small operand are staged in LDS, so the only global traffic per
+// lane is one 16-byte load and one 16-byte store, as in a plain copy; gathering
+// the small operand from global memory instead costs as many L1 accesses as the
+// main stream.
+// ---------------------------------------------------------------------------
+struct RowBcast {
+    FastDiv rc;     // R * C: elements per outer index
+    FastDiv c;      // C: row length
+    uint32_t n;     // number of outer indices (rows of the small operand)
+    uint32_t total; // N * R * C
+};
+
+template <class OP, bool SMALL_IS_A, bool NT>
+__global__ __launch_bounds__(BLOCK) void binary_rowbcast(float *__restrict__ out, const float *__restrict__ full,
+                                                         const float *__restrict__ small, const RowBcast g) {
+    extern __shared__ float rows_lds[];  // two rows of C floats
+    const uint32_t C = g.c.d;
+    const uint32_t block_start = blockIdx.x * (BLOCK * 4);
+    const uint32_t n_first = g.rc.div(block_start);  // uniform
+    // The 16-byte load of the dense operand goes out first, so its latency covers the staging of
+    // the small operand and the index arithmetic.
+    const uint32_t i0 = block_start + threadIdx.x * 4;
+    const bool whole = i0 + 4 <= g.total;
+    float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (whole) x = load4<NT>(full + i0);
+    {
+        // Row n_first, and the next one only if this block really reaches into it.
+        uint32_t block_last = block_start + BLOCK * 4 - 1;
+        if (block_last >= g.total) block_last = g.total - 1;
+        const uint32_t want = g.rc.div(block_last) != n_first ? 2 * C : C;
+        const float *src = small + (size_t)n_first * C;
+        for (uint32_t i = threadIdx.x; i < want; i += BLOCK) rows_lds[i] = src[i];
+    }
+    __syncthreads();
+
+    if (i0 >= g.total) return;
+    const uint32_t n = g.rc.div(i0);
+    const uint32_t rem = i0 - n * g.rc.d;            // offset inside outer index n
+    const uint32_t row = g.c.div(rem);
+    const uint32_t c0 = rem - row * C;               // column of element 0
+    const uint32_t base = (n - n_first) * C;         // LDS offset of row n
+
+    float y[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        uint32_t c = c0 + j, b = base;
+        if (c >= C) {                                // next row of the output ...
+            c -= C;
+            if (rem + j >= g.rc.d) b += C;           // ... which may belong to the next outer index
+        }
+        y[j] = rows_lds[b + c];
+    }
+    if (whole) {
+        float4 r;
+        r.x = SMALL_IS_A ? OP::f(y[0], x.x) : OP::f(x.x, y[0]);
+        r.y = SMALL_IS_A ? OP::f(y[1], x.y) : OP::f(x.y, y[1]);
+        r.z = SMALL_IS_A ? OP::f(y[2], x.z) : OP::f(x.z, y[2]);
+        r.w = SMALL_IS_A ? OP::f(y[3], x.w) : OP::f(x.w, y[3]);
+        store4<NT>(out + i0, r);
+    } else {
+        for (int j = 0; j < 4 && i0 + j < g.total; j++) {
+            const float xs = full[i0 + j];
+            out[i0 + j] = SMALL_IS_A ? OP::f(y[j], xs) : OP::f(xs, y[j]);
+        }
+    }
+}
+
 FastDiv make_fastdiv(uint32_t d) {
     FastDiv f;
     f.d = d;
@@ -272,6 +342,20 @@ void strided_launch(hipStream_t s, int rank, float *out, const float *a, const f
     else if (rank == 3) strided_dispatch<OP, 3>(s, out, a, b, n, g, vec, nt);
     else if (rank == 4) strided_dispatch<OP, 4>(s, out, a, b, n, g, vec, nt);
     else strided_dispatch<OP, MAX_RANK>(s, out, a, b, n, g, vec, nt);
+}
+
+template <class OP>
+void rowbcast_launch(hipStream_t s, bool small_is_a, bool nt, float *out, const float *full, const float *small,
+                     const RowBcast &g) {
+    const dim3 grid((g.total + BLOCK * 4 - 1) / (BLOCK * 4));
+    const size_t shmem = (size_t)2 * g.c.d * sizeof(float);
+    if (small_is_a) {
+        if (nt) hipLaunchKernelGGL((binary_rowbcast<OP, true, true>), grid, dim3(BLOCK), shmem, s, out, full, small, g);
+        else hipLaunchKernelGGL((binary_rowbcast<OP, true, false>), grid, dim3(BLOCK), shmem, s, out, full, small, g);
+    } else {
+        if (nt) hipLaunchKernelGGL((binary_rowbcast<OP, false, true>), grid, dim3(BLOCK), shmem, s, out, full, small, g);
+        else hipLaunchKernelGGL((binary_rowbcast<OP, false, false>), grid, dim3(BLOCK), shmem, s, out, full, small, g);
+    }
 }
 
 }  // namespace
@@ -358,6 +442,39 @@ int launch_binary(DeviceCtx &ctx, int op, float *out, const float *a, const floa
     for (int i = 0; i < r; i++)
         if ((uint64_t)as[i] >= LIMIT || (uint64_t)bs[i] >= LIMIT)
             return ctx.fail(AHIP_ERR_UNSUPPORTED, "binary: operand stride exceeds 2^31 elements");
+
+    // One operand dense, the other a row per outer index: [N,R,C] op [N,1,C] (strides [C,0,1]) or
+    // [R,C] op [C] (strides [0,1]).
+    {
+        const int64_t *ss = ma == STRIDED ? as : bs;  // strides of the small operand
+        const int other = ma == STRIDED ? mb : ma;
+        const bool pattern3 = r == 3 && ss[0] == dims[2] && ss[1] == 0 && ss[2] == 1;
+        const bool pattern2 = r == 2 && ss[0] == 0 && ss[1] == 1;
+        const int64_t C = dims[r - 1];
+        // A block covers BLOCK*4 consecutive elements and stages two rows of the small operand, so
+        // an outer index must span at least that many elements.
+        const bool two_rows_suffice = pattern2 || (r == 3 && dims[1] * dims[2] >= BLOCK * 4);
+        if (other == FULL && (pattern3 || pattern2) && two_rows_suffice && C >= 4 && C <= 512 && total < LIMIT &&
+            aligned16(out) &&
+            aligned16(ma == STRIDED ? b : a)) {
+            RowBcast rb;
+            rb.c = make_fastdiv((uint32_t)C);
+            rb.rc = make_fastdiv((uint32_t)(pattern3 ? dims[1] * dims[2] : dims[0] * dims[1]));
+            rb.n = pattern3 ? (uint32_t)dims[0] : 1u;
+            rb.total = (uint32_t)total;
+            const bool small_is_a = ma == STRIDED;
+            const float *full = small_is_a ? b : a;
+            const float *small = small_is_a ? a : b;
+            switch (op) {
+            case AHIP_ADD: rowbcast_launch<OpAdd>(s, small_is_a, nt, out, full, small, rb); break;
+            case AHIP_SUB: rowbcast_launch<OpSub>(s, small_is_a, nt, out, full, small, rb); break;
+            case AHIP_MUL: rowbcast_launch<OpMul>(s, small_is_a, nt, out, full, small, rb); break;
+            case AHIP_DIV: rowbcast_launch<OpDiv>(s, small_is_a, nt, out, full, small, rb); break;
+            case AHIP_POW: rowbcast_launch<OpPow>(s, small_is_a, nt, out, full, small, rb); break;
+            }
+            return ctx.check(hipGetLastError(), "binary row-broadcast launch");
+        }
+    }
 
     Geom g;
     for (int d = 0; d < MAX_RANK; d++) {

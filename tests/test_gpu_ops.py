@@ -44,6 +44,11 @@ BIN_SHAPES = [
     ([7], [7]),
     ([1023], [1023]),
     ([2, 0, 3], [3]),                  # empty
+    ([3, 40, 30], [3, 1, 30]),         # row broadcast staged in LDS, blocks spanning two outer indices
+    ([3, 1, 30], [3, 40, 30]),         # the same with the operands swapped
+    ([5, 2, 6], [5, 1, 6]),            # row broadcast too short for the LDS kernel
+    ([2, 3, 1031], [1031]),            # bias with an odd length
+    ([7, 5], [5]),
 ]
 
 
