@@ -174,92 +174,94 @@ __global__ __launch_bounds__(COL_BLOCK) void reduce_cols(float *__restrict__ dst
     }
 }
 
-// The same reduction with 16-byte loads, for inner extents up to 256 that are
-// not multiples of 4 (197, say), where rows are only 4-byte aligned.  Four
-// consecutive rows are `inner` float4 that start 16-byte aligned, and because
-// the group is exactly four rows long, float4 number f of every group holds the
-// same four (row-in-group, column) positions.  So a lane accumulates float4
-// number lane + 64k of group after group element by element, and only at the end
-// do the 4*inner accumulators go through LDS, where column c collects positions
-// c, c + inner, c + 2*inner, c + 3*inner of every wave.  Rows left over when the
-// reduced extent is not a multiple of 4 are folded in by the last split.
-// grid = (outer * splits); dynamic LDS = FLAT_WAVES * 4 * inner floats.
-constexpr int FLAT_BLOCK = 1024;
-constexpr int FLAT_WAVES = FLAT_BLOCK / WAVE;
+// The same reduction with 16-byte loads even when rows are only 4-byte aligned
+// (inner = 197, say).  A "span" is P consecutive rows, P chosen so that a span is
+// a whole number of 128-byte lines (32 rows when inner is odd).  Because every
+// span is exactly P rows long, float4 number j of every span holds the same four
+// (row-in-span, column) positions, so thread t accumulates float4 t, t + 1024, ...
+// of span after span element by element, and only at the end do the P*inner
+// accumulators go through LDS, where column c collects positions c, c + inner,
+// c + 2*inner, ...  The loads of the next span are issued before the current one
+// is folded in, so each wave has U to 2*U 16-byte loads in flight on whole,
+// line-aligned 1-KiB pieces.  Rows left over when the reduced extent is
+// not a multiple of P are folded in at the end by the last split.
+// grid = (outer * splits); dynamic LDS = P * inner floats.
+constexpr int SPAN_BLOCK = 1024;
 
-template <class OP, int NCH, bool SCALE, bool NT>
-__global__ __launch_bounds__(FLAT_BLOCK) void reduce_cols_flat4(float *__restrict__ dst,
-                                                               const float *__restrict__ in, uint32_t red,
-                                                               uint32_t inner, uint32_t splits,
-                                                               uint32_t groups_per_split, float scale) {
-    extern __shared__ __align__(16) float lds4[];
-    const int lane = threadIdx.x & (WAVE - 1);
-    const int wave = threadIdx.x >> 6;
+template <class OP, int U, bool SCALE, bool NT>
+__global__ __launch_bounds__(SPAN_BLOCK) void reduce_cols_span(float *__restrict__ dst, const float *__restrict__ in,
+                                                               uint32_t red, uint32_t inner, uint32_t span_rows,
+                                                               uint32_t splits, uint32_t spans_per_split, float scale) {
+    extern __shared__ __align__(16) float span_lds[];
+    const uint32_t tid = threadIdx.x;
     const uint32_t o = blockIdx.x / splits, s = blockIdx.x % splits;
-    const uint32_t ngroups = red >> 2;
-    const uint32_t g_begin = s * groups_per_split;
-    uint32_t g_end = g_begin + groups_per_split;
-    if (g_end > ngroups) g_end = ngroups;
+    const uint32_t span_floats = span_rows * inner;
+    const uint32_t nf4 = span_floats >> 2;
+    const uint32_t nspans = red / span_rows;
+    const uint32_t sp_begin = s * spans_per_split;
+    uint32_t sp_end = sp_begin + spans_per_split;
+    if (sp_end > nspans) sp_end = nspans;
     const float *slab = in + (size_t)o * red * inner;
-    const size_t group_floats = (size_t)4 * inner;
 
-    float4 acc[NCH];
+    float4 acc[U];
 #pragma unroll
-    for (int k = 0; k < NCH; k++) acc[k] = make_float4(OP::identity(), OP::identity(), OP::identity(), OP::identity());
+    for (int u = 0; u < U; u++) acc[u] = make_float4(OP::identity(), OP::identity(), OP::identity(), OP::identity());
 
-    uint32_t g = g_begin + wave;
-    for (; g + FLAT_WAVES < g_end; g += 2 * FLAT_WAVES) {  // two groups in flight
-        const float *p0 = slab + g * group_floats;
-        const float *p1 = p0 + FLAT_WAVES * group_floats;
-        float4 v0[NCH], v1[NCH];
+    // Software pipeline: the loads of span i+1 are in flight while span i is folded in.  Lanes
+    // whose float4 index lies past the span re-read its last float4 instead of being masked off:
+    // straight-line code lets the loads of the next span overtake the wait for the current one.
+    uint32_t off[U];
 #pragma unroll
-        for (int k = 0; k < NCH; k++) {
-            const uint32_t f = lane + WAVE * k;
-            if (f < inner) {
-                v0[k] = load4<NT>(p0 + 4 * f);
-                v1[k] = load4<NT>(p1 + 4 * f);
-            }
+    for (int u = 0; u < U; u++) {
+        const uint32_t j = tid + SPAN_BLOCK * u;
+        off[u] = 4 * (j < nf4 ? j : nf4 - 1);
+    }
+    auto load_span = [&](uint32_t sp, float4 (&v)[U]) {
+        const float *p = slab + (size_t)sp * span_floats;
+#pragma unroll
+        for (int u = 0; u < U; u++) v[u] = load4<NT>(p + off[u]);
+    };
+    auto fold_span = [&](const float4 (&v)[U]) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            acc[u].x = OP::apply(acc[u].x, v[u].x);
+            acc[u].y = OP::apply(acc[u].y, v[u].y);
+            acc[u].z = OP::apply(acc[u].z, v[u].z);
+            acc[u].w = OP::apply(acc[u].w, v[u].w);
         }
-#pragma unroll
-        for (int k = 0; k < NCH; k++) {
-            const uint32_t f = lane + WAVE * k;
-            if (f < inner) {
-                acc[k].x = OP::apply(OP::apply(acc[k].x, v0[k].x), v1[k].x);
-                acc[k].y = OP::apply(OP::apply(acc[k].y, v0[k].y), v1[k].y);
-                acc[k].z = OP::apply(OP::apply(acc[k].z, v0[k].z), v1[k].z);
-                acc[k].w = OP::apply(OP::apply(acc[k].w, v0[k].w), v1[k].w);
-            }
+    };
+    // The loop body has no conditional loads, so the wait before each fold can allow exactly
+    // the U younger loads to stay in flight.
+    if (sp_begin < sp_end) {
+        float4 va[U], vb[U];
+        uint32_t sp = sp_begin;
+        load_span(sp, va);
+        for (; sp + 2 < sp_end; sp += 2) {  // va holds span sp
+            load_span(sp + 1, vb);
+            fold_span(va);
+            load_span(sp + 2, va);
+            fold_span(vb);
+        }
+        if (sp + 1 < sp_end) {
+            load_span(sp + 1, vb);
+            fold_span(va);
+            fold_span(vb);
+        } else {
+            fold_span(va);
         }
     }
-    for (; g < g_end; g += FLAT_WAVES) {
-        const float *p0 = slab + g * group_floats;
-#pragma unroll
-        for (int k = 0; k < NCH; k++) {
-            const uint32_t f = lane + WAVE * k;
-            if (f < inner) {
-                const float4 v = load4<NT>(p0 + 4 * f);
-                acc[k].x = OP::apply(acc[k].x, v.x);
-                acc[k].y = OP::apply(acc[k].y, v.y);
-                acc[k].z = OP::apply(acc[k].z, v.z);
-                acc[k].w = OP::apply(acc[k].w, v.w);
-            }
-        }
-    }
 
-    float *mine = lds4 + (size_t)wave * group_floats;
 #pragma unroll
-    for (int k = 0; k < NCH; k++) {
-        const uint32_t f = lane + WAVE * k;
-        if (f < inner) *reinterpret_cast<float4 *>(mine + 4 * f) = acc[k];
+    for (int u = 0; u < U; u++) {
+        const uint32_t j = tid + SPAN_BLOCK * u;
+        if (j < nf4) *reinterpret_cast<float4 *>(span_lds + 4 * j) = acc[u];
     }
     __syncthreads();
-    for (uint32_t c = threadIdx.x; c < inner; c += FLAT_BLOCK) {
+    for (uint32_t c = tid; c < inner; c += SPAN_BLOCK) {
         float a = OP::identity();
-        for (int w = 0; w < FLAT_WAVES; w++)
-#pragma unroll
-            for (int p = 0; p < 4; p++) a = OP::apply(a, lds4[w * group_floats + p * inner + c]);
+        for (uint32_t p = 0; p < span_rows; p++) a = OP::apply(a, span_lds[p * inner + c]);
         if (s == splits - 1)
-            for (uint32_t r = ngroups << 2; r < red; r++) a = OP::apply(a, slab[(size_t)r * inner + c]);
+            for (uint32_t r = nspans * span_rows; r < red; r++) a = OP::apply(a, slab[(size_t)r * inner + c]);
         dst[(size_t)blockIdx.x * inner + c] = SCALE ? a * scale : a;
     }
 }
@@ -314,27 +316,34 @@ void cols_launch(hipStream_t s, float *dst, const float *in, size_t outer, size_
 }
 
 template <class OP, bool SCALE>
-void cols_flat4_launch(hipStream_t s, float *dst, const float *in, size_t outer, size_t red, size_t inner,
-                       size_t splits, size_t groups_per_split, float scale, bool nt) {
+void cols_span_launch(hipStream_t s, float *dst, const float *in, size_t outer, size_t red, size_t inner,
+                      size_t span_rows, size_t splits, size_t spans_per_split, float scale, bool nt) {
     const dim3 grid((unsigned)(outer * splits));
-    const dim3 block(FLAT_BLOCK);
-    const size_t shmem = (size_t)FLAT_WAVES * 4 * inner * sizeof(float);
-    const int nch = (int)((inner + WAVE - 1) / WAVE);
-#define ALTIUS_LAUNCH(N, T)                                                                                    \
-    hipLaunchKernelGGL((reduce_cols_flat4<OP, N, SCALE, T>), grid, block, shmem, s, dst, in, (uint32_t)red,    \
-                       (uint32_t)inner, (uint32_t)splits, (uint32_t)groups_per_split, scale)
+    const dim3 block(SPAN_BLOCK);
+    const size_t shmem = span_rows * inner * sizeof(float);
+    const int u = (int)((span_rows * inner / 4 + SPAN_BLOCK - 1) / SPAN_BLOCK);
+#define ALTIUS_LAUNCH(N, T)                                                                                   \
+    hipLaunchKernelGGL((reduce_cols_span<OP, N, SCALE, T>), grid, block, shmem, s, dst, in, (uint32_t)red,    \
+                       (uint32_t)inner, (uint32_t)span_rows, (uint32_t)splits, (uint32_t)spans_per_split, scale)
     if (nt) {
-        if (nch == 1) ALTIUS_LAUNCH(1, true);
-        else if (nch == 2) ALTIUS_LAUNCH(2, true);
-        else if (nch == 3) ALTIUS_LAUNCH(3, true);
+        if (u <= 1) ALTIUS_LAUNCH(1, true);
+        else if (u == 2) ALTIUS_LAUNCH(2, true);
         else ALTIUS_LAUNCH(4, true);
     } else {
-        if (nch == 1) ALTIUS_LAUNCH(1, false);
-        else if (nch == 2) ALTIUS_LAUNCH(2, false);
-        else if (nch == 3) ALTIUS_LAUNCH(3, false);
+        if (u <= 1) ALTIUS_LAUNCH(1, false);
+        else if (u == 2) ALTIUS_LAUNCH(2, false);
         else ALTIUS_LAUNCH(4, false);
     }
 #undef ALTIUS_LAUNCH
+}
+
+size_t gcd_size(size_t a, size_t b) {
+    while (b) {
+        const size_t t = a % b;
+        a = b;
+        b = t;
+    }
+    return a;
 }
 
 template <class OP, bool SCALE>
@@ -374,29 +383,32 @@ int reduce_impl(DeviceCtx &ctx, float *out, const float *in, size_t outer, size_
     // inner > 1
     if (red >= ((size_t)1 << 32) || inner >= ((size_t)1 << 31))
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: axis extent exceeds 32-bit index range");
-    // Unaligned rows of moderate width: the 16-byte flat variant.
-    if (inner % 4 != 0 && inner <= 256 && red >= 16 && aligned16(in) && (outer == 1 || (red * inner) % 4 == 0)) {
-        const size_t groups = red / 4;
-        // One 16-wave block per slab fills the chip once there are about as many slabs as CUs;
-        // with fewer slabs the reduced axis is split over blocks and a second launch folds the parts.
-        size_t fsplits = 1;
-        if (outer < 192) {
-            fsplits = (512 + outer - 1) / outer;
-            const size_t max_splits = groups / 32 > 0 ? groups / 32 : 1;  // two groups per wave at least
-            if (fsplits > max_splits) fsplits = max_splits;
-        }
-        size_t gps = (groups + fsplits - 1) / fsplits;
-        fsplits = (groups + gps - 1) / gps;
-        const bool nt = ctx.streaming(outer * red * inner * sizeof(float));
-        if (outer * fsplits <= MAX_GRID_X) {
-            if (fsplits == 1) {
-                cols_flat4_launch<OP, SCALE>(s, out, in, outer, red, inner, 1, gps, scale, nt);
-                return ctx.check(hipGetLastError(), "reduce cols (flat4) launch");
+    // Rows that are not multiples of 16 bytes, moderate width: the span variant with 16-byte loads.
+    if (inner % 4 != 0 && inner <= 1024 && aligned16(in) && (outer == 1 || (red * inner) % 4 == 0)) {
+        const size_t span_rows = 32 / gcd_size(inner, 32);  // smallest P with P * inner * 4 bytes a multiple of 128
+        const size_t nspans = red / span_rows;
+        if (span_rows * inner <= (size_t)4 * 4 * SPAN_BLOCK && nspans >= 4) {
+            // One 16-wave block per slab fills the chip once there are about as many slabs as CUs;
+            // with fewer slabs the reduced axis is split over blocks and a second launch folds the parts.
+            size_t fsplits = 1;
+            if (outer < 192) {
+                fsplits = (512 + outer - 1) / outer;
+                const size_t max_splits = nspans / 4 > 0 ? nspans / 4 : 1;
+                if (fsplits > max_splits) fsplits = max_splits;
             }
-            if (outer * fsplits * inner <= ctx.scratch_floats) {
-                cols_flat4_launch<OP, false>(s, ctx.scratch, in, outer, red, inner, fsplits, gps, 1.0f, nt);
-                cols_launch<OP, SCALE>(s, out, ctx.scratch, outer, fsplits, inner, 1, fsplits, scale);
-                return ctx.check(hipGetLastError(), "reduce cols (flat4, two-stage) launch");
+            size_t sps = (nspans + fsplits - 1) / fsplits;
+            fsplits = (nspans + sps - 1) / sps;
+            const bool nt = ctx.streaming(outer * red * inner * sizeof(float));
+            if (outer * fsplits <= MAX_GRID_X) {
+                if (fsplits == 1) {
+                    cols_span_launch<OP, SCALE>(s, out, in, outer, red, inner, span_rows, 1, sps, scale, nt);
+                    return ctx.check(hipGetLastError(), "reduce cols (span) launch");
+                }
+                if (outer * fsplits * inner <= ctx.scratch_floats) {
+                    cols_span_launch<OP, false>(s, ctx.scratch, in, outer, red, inner, span_rows, fsplits, sps, 1.0f, nt);
+                    cols_launch<OP, SCALE>(s, out, ctx.scratch, outer, fsplits, inner, 1, fsplits, scale);
+                    return ctx.check(hipGetLastError(), "reduce cols (span, two-stage) launch");
+                }
             }
         }
     }

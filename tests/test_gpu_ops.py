@@ -265,6 +265,9 @@ REDUCE_CASES = [
     ([3, 17, 5], [1], False),          # unaligned slabs: dword column kernel
     ([2, 2049, 255], [1], False),      # flat kernel split over blocks, odd row count
     ([300, 64, 6], [1], False),
+    ([3, 640, 7], [1], False),         # span kernel, one float4 step per thread
+    ([1, 4099, 33], [1], False),       # span kernel split over blocks, three left-over rows
+    ([2, 130, 1023], [1], True),       # span kernel at its widest (four float4 steps per thread)
 ]
 
 
