@@ -66,6 +66,10 @@ def _declare(L):
     f("ahip_event_synchronize", [c_void_p, c_void_p])
     f("ahip_event_elapsed_ms", [c_void_p, c_void_p, c_void_p, P(c_float)])
     f("ahip_event_destroy", [c_void_p, c_void_p])
+    f("ahip_module_load", [c_void_p, c_void_p, c_size_t, P(c_void_p)])
+    f("ahip_module_unload", [c_void_p, c_void_p])
+    f("ahip_launch", [c_void_p, c_void_p, c_char_p, P(ctypes.c_uint32), P(ctypes.c_uint32), ctypes.c_uint32,
+                      P(c_void_p)])
     f("ahip_broadcast_shape", [c_int, P(c_int64), c_int, P(c_int64), P(c_int), P(c_int64)])
     f("ahip_strides_for_broadcasting", [c_int, P(c_int64), c_int, P(c_int64), P(c_int64)])
     f("ahip_binary", [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, P(c_int64), P(c_int64), P(c_int64)])
@@ -123,6 +127,9 @@ def _declare_graph(L):
     f("ahip_tensor_dims", [c_void_p, P(c_int64), c_int])
     f("ahip_tensor_nbytes", [c_void_p], c_size_t)
     f("ahip_tensor_data", [c_void_p], c_void_p)
+    f("ahip_tensor_data_mut", [c_void_p], c_void_p)
+    f("ahip_host_pool_stats", [P(c_size_t), P(c_size_t), P(c_size_t), P(c_size_t)])
+    f("ahip_host_pool_trim", [], c_size_t)
     f("ahip_session_builder_new", [c_void_p, P(c_void_p)])
     f("ahip_session_builder_free", [c_void_p], None)
     f("ahip_session_builder_with_intra_op_num_threads", [c_void_p, c_size_t])

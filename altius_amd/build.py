@@ -13,6 +13,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "libaltius_hip.so")
+MODULE_SRC_DIR = os.path.join(CSRC, "modules")  # stand-alone code objects, not linked into the library
+MODULE_DIR = os.path.join(HERE, "modules")
 
 ARCH = "gfx950"
 
@@ -47,7 +49,23 @@ def hipcc():
 def sources():
     src = sorted(glob.glob(os.path.join(CSRC, "**", "*.hip"), recursive=True))
     src += sorted(glob.glob(os.path.join(CSRC, "**", "*.cpp"), recursive=True))
-    return src
+    return [s for s in src if not s.startswith(MODULE_SRC_DIR + os.sep)]
+
+
+def module_path(name):
+    """Path of the code object built from csrc/modules/<name>.hip."""
+    return os.path.join(MODULE_DIR, name + ".hsaco")
+
+
+def _compile_module(src, force):
+    out = module_path(os.path.splitext(os.path.basename(src))[0])
+    if not force and os.path.exists(out) and os.path.getmtime(out) >= os.path.getmtime(src):
+        return out
+    cmd = [hipcc(), "--genco"] + COMMON_FLAGS + DEVICE_FLAGS + [src, "-o", out]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc --genco failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
+    return out
 
 
 def _obj_path(src):
@@ -91,6 +109,8 @@ def build(force=False, jobs=None):
     jobs = jobs or min(8, os.cpu_count() or 1)
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(lambda s: _compile(s, force), src))
+        os.makedirs(MODULE_DIR, exist_ok=True)
+        list(ex.map(lambda s: _compile_module(s, force), sorted(glob.glob(os.path.join(MODULE_SRC_DIR, "*.hip")))))
     cmd = [hipcc(), "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", LIB_PATH] + objs
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:

@@ -1,7 +1,10 @@
 // C ABI: device shim, host index math and operator entry points.
 #include <hip/hip_runtime.h>
 
+#include <cstring>
 #include <new>
+#include <string>
+#include <unordered_map>
 
 #include "core/fixed_dim.h"
 #include "device/ctx.h"
@@ -167,6 +170,82 @@ int ahip_event_destroy(ahip_ctx *ctx, void *event) {
     REQUIRE_CTX(ctx, "ahip_event_destroy");
     if (!event) return AHIP_OK;
     return ctx->d.check(hipEventDestroy(static_cast<hipEvent_t>(event)), "hipEventDestroy");
+}
+
+// ---- code objects loaded at run time -----------------------------------------
+
+struct ahip_module {
+    hipModule_t mod = nullptr;
+    int device = 0;
+    std::unordered_map<std::string, hipFunction_t> functions;
+};
+
+int ahip_module_load(ahip_ctx *ctx, const void *image, size_t bytes, ahip_module **module) {
+    REQUIRE_CTX(ctx, "ahip_module_load");
+    if (!module) return ctx->d.fail(AHIP_ERR_ARG, "ahip_module_load: null output pointer");
+    *module = nullptr;
+    if (!image || bytes < 8) return ctx->d.fail(AHIP_ERR_ARG, "ahip_module_load: empty image");
+    const unsigned char *p = static_cast<const unsigned char *>(image);
+    const bool elf = p[0] == 0x7f && p[1] == 'E' && p[2] == 'L' && p[3] == 'F';
+    const bool bundle = bytes >= 24 && std::memcmp(p, "__CLANG_OFFLOAD_BUNDLE__", 24) == 0;
+    if (!elf && !bundle)
+        return ctx->d.fail(AHIP_ERR_ARG, "ahip_module_load: image is neither an ELF code object nor an offload bundle");
+    ahip_module *m = new (std::nothrow) ahip_module();
+    if (!m) return ctx->d.fail(AHIP_ERR_OOM, "ahip_module_load: out of host memory");
+    m->device = ctx->d.device;
+    // The runtime reads the image through the pointer only during this call.
+    const int rc = ctx->d.check(hipModuleLoadData(&m->mod, image), "hipModuleLoadData");
+    if (rc) {
+        delete m;
+        return rc;
+    }
+    *module = m;
+    return AHIP_OK;
+}
+
+int ahip_module_unload(ahip_ctx *ctx, ahip_module *module) {
+    REQUIRE_CTX(ctx, "ahip_module_unload");
+    if (!module) return AHIP_OK;
+    if (module->device != ctx->d.device)
+        return ctx->d.fail(AHIP_ERR_ARG, "ahip_module_unload: module belongs to another device");
+    // Kernels of the module may still be queued on the stream.
+    int rc = ctx->d.check(hipStreamSynchronize(ctx->d.stream), "hipStreamSynchronize");
+    const int rc2 = ctx->d.check(hipModuleUnload(module->mod), "hipModuleUnload");
+    delete module;
+    return rc ? rc : rc2;
+}
+
+int ahip_launch(ahip_ctx *ctx, ahip_module *module, const char *kernel, const uint32_t grid[3],
+                const uint32_t block[3], uint32_t shared_bytes, void **args) {
+    REQUIRE_CTX(ctx, "ahip_launch");
+    if (!module || !kernel || !grid || !block)
+        return ctx->d.fail(AHIP_ERR_ARG, "ahip_launch: null module, kernel name, grid or block");
+    if (module->device != ctx->d.device)
+        return ctx->d.fail(AHIP_ERR_ARG, "ahip_launch: module belongs to another device");
+    const uint64_t threads = (uint64_t)block[0] * block[1] * block[2];
+    if (threads == 0 || threads > 1024 || block[0] > 1024 || block[1] > 1024 || block[2] > 1024)
+        return ctx->d.fail(AHIP_ERR_ARG, "ahip_launch: a block holds 1 to 1024 threads");
+    if (grid[0] == 0 || grid[1] == 0 || grid[2] == 0 || grid[1] > 65535u || grid[2] > 65535u ||
+        (uint64_t)grid[0] * block[0] > 0xffffffffull)
+        return ctx->d.fail(AHIP_ERR_ARG, "ahip_launch: grid extent out of range");
+    if (shared_bytes > 160u * 1024u)
+        return ctx->d.fail(AHIP_ERR_ARG, "ahip_launch: more than 160 KiB of shared memory per block");
+    hipFunction_t fn = nullptr;
+    auto it = module->functions.find(kernel);
+    if (it != module->functions.end()) {
+        fn = it->second;
+    } else {
+        const hipError_t e = hipModuleGetFunction(&fn, module->mod, kernel);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return ctx->d.fail(AHIP_ERR_ARG, std::string("ahip_launch: no kernel named '") + kernel +
+                                                 "' in the module (" + hipGetErrorString(e) + ")");
+        }
+        module->functions.emplace(kernel, fn);
+    }
+    return ctx->d.check(hipModuleLaunchKernel(fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                                              shared_bytes, ctx->d.stream, args, nullptr),
+                        "hipModuleLaunchKernel");
 }
 
 // ---- host index math -------------------------------------------------------

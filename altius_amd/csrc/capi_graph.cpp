@@ -8,6 +8,7 @@
 #include "core/optimize.h"
 #include "core/shape.h"
 #include "device/ctx.h"
+#include "device/host_pool.h"
 #include "session/hip_session.h"
 #include "session/plan.h"
 
@@ -274,10 +275,29 @@ int ahip_tensor_new(int elem_type, int rank, const int64_t *dims, const void *da
     if (data && nbytes != want) return fail(AHIP_ERR_ARG, "ahip_tensor_new: data size does not match the shape");
     ahip_tensor *t = new (std::nothrow) ahip_tensor();
     if (!t) return fail(AHIP_ERR_OOM, "ahip_tensor_new: out of host memory");
-    t->t = data ? Tensor::from_raw(std::move(fd), ty, data, want) : Tensor::zeros_of_type(ty, std::move(fd));
+    // Tensors made here are the ones handed to ahip_session_run: pinned storage when a device is there.
+    t->t = data ? Tensor::from_raw(std::move(fd), ty, data, want, altius::pinned_host_block)
+                : Tensor::zeros_of_type(ty, std::move(fd), altius::pinned_host_block);
+    if (!t->t.has_data()) {
+        delete t;
+        return fail(AHIP_ERR_OOM, "ahip_tensor_new: out of host memory");
+    }
     *tensor = t;
     return AHIP_OK;
 }
+
+void *ahip_tensor_data_mut(ahip_tensor *tensor) { return tensor ? tensor->t.data_as_bytes_mut() : nullptr; }
+
+int ahip_host_pool_stats(size_t *live_bytes, size_t *cached_bytes, size_t *pinned_allocations, size_t *reuses) {
+    const altius::HostPoolStats st = altius::host_pool_stats();
+    if (live_bytes) *live_bytes = st.live_bytes;
+    if (cached_bytes) *cached_bytes = st.cached_bytes;
+    if (pinned_allocations) *pinned_allocations = st.pinned_allocations;
+    if (reuses) *reuses = st.reuses;
+    return AHIP_OK;
+}
+
+size_t ahip_host_pool_trim(void) { return altius::host_pool_trim(); }
 
 void ahip_tensor_free(ahip_tensor *tensor) { delete tensor; }
 int ahip_tensor_elem_type(const ahip_tensor *tensor) { return tensor ? (int)tensor->t.elem_ty() : -1; }

@@ -20,7 +20,7 @@ const char *op_kind_name(OpKind k) {
 
 bool Tensor::allclose_f32(const std::vector<float> &other) const {
     if (elem_ty_ != TensorElemType::F32) return false;
-    const size_t n = data_->size() / sizeof(float);
+    const size_t n = data_->size / sizeof(float);
     if (n != other.size()) return false;
     const float *x = data_f32();
     for (size_t i = 0; i < n; i++) {

@@ -3,6 +3,8 @@
 #include <algorithm>
 #include <chrono>
 
+#include "../device/host_pool.h"
+
 namespace altius {
 
 int SessionError::code() const {
@@ -267,7 +269,12 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
             destroy_events();
             return fail(err, SessionError::Message, "run: graph output was not produced");
         }
-        Tensor t = Tensor::uninit_of_type(d->elem_ty, d->dims);
+        Tensor t = Tensor::uninit_of_type(d->elem_ty, d->dims, pinned_host_block);
+        if (!t.has_data()) {
+            cleanup();
+            destroy_events();
+            return fail(err, SessionError::OutOfMemory, "run: out of host memory for an output tensor");
+        }
         if (d->nbytes()) {
             int rc = ctx_.check(hipMemcpyAsync(t.data_as_bytes_mut(), d->ptr, d->nbytes(), hipMemcpyDeviceToHost,
                                                ctx_.stream),

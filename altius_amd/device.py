@@ -129,6 +129,25 @@ class Context:
     def destroy_event(self, event):
         check(self.L.ahip_event_destroy(self.handle, event), self.handle)
 
+    # --- code objects loaded at run time ----------------------------------
+    def load_module(self, image):
+        """Loads a gfx950 code object (bytes) and returns its handle."""
+        buf = ctypes.create_string_buffer(bytes(image), max(1, len(image)))
+        m = ctypes.c_void_p()
+        check(self.L.ahip_module_load(self.handle, ctypes.cast(buf, ctypes.c_void_p), len(image), ctypes.byref(m)),
+              self.handle)
+        return m
+
+    def unload_module(self, module):
+        check(self.L.ahip_module_unload(self.handle, module), self.handle)
+
+    def launch(self, module, kernel, grid, block, args, shared_bytes=0):
+        """Launches `kernel` of `module`; args are ctypes values (c_void_p, c_float, c_uint64 ...)."""
+        u3 = ctypes.c_uint32 * 3
+        ptrs = (ctypes.c_void_p * max(1, len(args)))(*[ctypes.cast(ctypes.pointer(a), ctypes.c_void_p) for a in args])
+        check(self.L.ahip_launch(self.handle, module, kernel.encode(), u3(*grid), u3(*block), shared_bytes, ptrs),
+              self.handle)
+
     # --- kernels on raw device pointers -----------------------------------
     def binary_raw(self, op, out_ptr, a_ptr, b_ptr, out_dims, a_strides, b_strides):
         check(self.L.ahip_binary(self.handle, op, out_ptr, a_ptr, b_ptr, len(out_dims), i64_array(out_dims),

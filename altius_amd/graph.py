@@ -100,10 +100,40 @@ class Tensor:
             ctypes.memmove(out.ctypes.data, L.ahip_tensor_data(self.handle), n)
         return out
 
+    def view(self):
+        """The tensor's own bytes as a numpy array, without a copy.  The array keeps this Tensor
+        alive; writing through it fills the tensor in place (Tensor::data_mut)."""
+        L = _lib.lib()
+        n = L.ahip_tensor_nbytes(self.handle)
+        dtype = _NP_OF[self.elem_ty]
+        if n == 0:
+            return np.empty(self.dims, dtype=dtype)
+        raw = (ctypes.c_ubyte * n).from_address(L.ahip_tensor_data_mut(self.handle))
+        raw._tensor = self  # the buffer object owns a reference to the tensor
+        return np.frombuffer(raw, dtype=dtype).reshape(self.dims)
+
+    @classmethod
+    def zeros(cls, dims, elem_ty=1):
+        """A zero-filled tensor of the given shape (fill it through view())."""
+        h = ctypes.c_void_p()
+        check(_lib.lib().ahip_tensor_new(elem_ty, len(dims), i64_array(dims), None, 0, ctypes.byref(h)))
+        return cls(h)
+
     def __del__(self):
         if getattr(self, "handle", None):
             _lib.lib().ahip_tensor_free(self.handle)
             self.handle = None
+
+
+def host_pool_stats():
+    """(live_bytes, cached_bytes, pinned_allocations, reuses) of the pinned pool behind host tensors."""
+    v = [ctypes.c_size_t() for _ in range(4)]
+    check(_lib.lib().ahip_host_pool_stats(*[ctypes.byref(x) for x in v]))
+    return tuple(x.value for x in v)
+
+
+def host_pool_trim():
+    return _lib.lib().ahip_host_pool_trim()
 
 
 class Model:

@@ -26,16 +26,17 @@ class HipSession:
         """A borrowed view of the session's model (valid while the session lives)."""
         return Model(_handle=ctypes.c_void_p(self.L.ahip_session_model(self.handle)), _borrowed=True)
 
-    def run(self, inputs):
+    def run(self, inputs, copy=True):
         """inputs: numpy arrays or Tensors, positional in graph.inputs order.  Returns numpy arrays
-        in graph.outputs order."""
+        in graph.outputs order; with copy=False they are views of the output tensors' own memory."""
         tensors = [t if isinstance(t, Tensor) else Tensor.from_numpy(t) for t in inputs]
         arr = (ctypes.c_void_p * max(len(tensors), 1))(*[t.handle for t in tensors])
         cap = 16
         outs = (ctypes.c_void_p * cap)()
         n = ctypes.c_int()
         check(self.L.ahip_session_run(self.handle, len(tensors), arr, cap, outs, ctypes.byref(n)))
-        return [Tensor(ctypes.c_void_p(outs[i])).numpy() for i in range(n.value)]
+        tensors_out = [Tensor(ctypes.c_void_p(outs[i])) for i in range(n.value)]
+        return [t.numpy() if copy else t.view() for t in tensors_out]
 
     def profile(self):
         """{op name: device milliseconds} of the last run (profiling enabled)."""

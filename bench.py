@@ -109,6 +109,128 @@ def build_cfg4(ctx, D, synth, batch, rotate_bytes):
     return ops, c
 
 
+def build_other_configs(ctx, D, synth, rotate_bytes=600e6, max_sets=48):
+    """Kernels of configs[0..3] at their BASELINE.json shapes (parity-test shapes, reported as a table
+    only).  Buffers are rotated over enough copies that repeated launches miss the 256 MB cache."""
+    ops = []
+
+    def sets(nbytes):
+        return max(1, min(max_sets, int(np.ceil(rotate_bytes / max(nbytes, 1)))))
+
+    def binary(name, op, a, b):
+        out_dims = D.broadcast_shape(a.shape, b.shape)
+        n = int(np.prod(out_dims))
+        nbytes = a.nbytes + b.nbytes + 4 * n
+        a_str, b_str = D.strides_for_broadcasting(a.shape, out_dims), D.strides_for_broadcasting(b.shape, out_dims)
+        k = sets(nbytes)
+        da = [ctx.upload(a) for _ in range(k)]
+        db = ctx.upload(b) if b.nbytes < (1 << 20) else None
+        dbs = [db] * k if db else [ctx.upload(b) for _ in range(k)]
+        do = [ctx.alloc(4 * n) for _ in range(k)]
+        ops.append(Op(name, nbytes, [(lambda i=i: ctx.binary_raw(op, do[i].ptr, da[i].ptr, dbs[i].ptr, out_dims, a_str, b_str))
+                                     for i in range(k)]))
+
+    def unary(name, op, x, alpha=0.0, beta=0.0):
+        k = sets(2 * x.nbytes)
+        dx = [ctx.upload(x) for _ in range(k)]
+        do = [ctx.alloc(x.nbytes) for _ in range(k)]
+        ops.append(Op(name, 2 * x.nbytes, [(lambda i=i: ctx.unary_raw(op, do[i].ptr, dx[i].ptr, x.size, alpha, beta))
+                                           for i in range(k)]))
+
+    def softmax(name, x):
+        k = sets(2 * x.nbytes)
+        dx = [ctx.upload(x) for _ in range(k)]
+        do = [ctx.alloc(x.nbytes) for _ in range(k)]
+        rows, length = x.size // x.shape[-1], x.shape[-1]
+        ops.append(Op(name, 2 * x.nbytes, [(lambda i=i: ctx.softmax_raw(do[i].ptr, dx[i].ptr, rows, length)) for i in range(k)]))
+
+    def layer_norm(name, x, gamma, beta, eps):
+        nbytes = 2 * x.nbytes + gamma.nbytes + beta.nbytes
+        k = sets(nbytes)
+        dx = [ctx.upload(x) for _ in range(k)]
+        do = [ctx.alloc(x.nbytes) for _ in range(k)]
+        dg, db = ctx.upload(gamma), ctx.upload(beta)
+        rows, length = x.size // x.shape[-1], x.shape[-1]
+        ops.append(Op(name, nbytes, [(lambda i=i: ctx.layernorm_raw(do[i].ptr, dx[i].ptr, dg.ptr, db.ptr, rows, length, eps))
+                                     for i in range(k)]))
+
+    def reduce(name, kind, x, outer, red, inner):
+        nbytes = x.nbytes + 4 * outer * inner
+        k = sets(nbytes)
+        dx = [ctx.upload(x) for _ in range(k)]
+        do = [ctx.alloc(4 * outer * inner) for _ in range(k)]
+        ops.append(Op(name, nbytes, [(lambda i=i: ctx.reduce_raw(kind, do[i].ptr, dx[i].ptr, outer, red, inner))
+                                     for i in range(k)]))
+
+    c0 = synth.cfg0()
+    binary("cfg0 Add [1,197,768]+[768]", D.ADD, c0["a"], c0["b"])
+    c1 = synth.cfg1()
+    softmax("cfg1 Softmax [8,12,197,197]", c1["scores"])
+    layer_norm("cfg1 LayerNorm [8,197,768]", c1["x"], c1["gamma"], c1["beta"], float(c1["eps"]))
+    c2 = synth.cfg2()
+    x = c2["x"]
+    mean = np.zeros((32, 197, 1), np.float32)
+    layer_norm("cfg2 LayerNorm (fused) [32,197,768]", x, c2["gamma"], c2["beta"], float(c2["eps"]))
+    reduce("cfg2 ReduceMean(-1) [32,197,768]", D.REDUCE_MEAN, x, 32 * 197, 768, 1)
+    binary("cfg2 Sub [32,197,768]-[32,197,1]", D.SUB, x, mean)
+    binary("cfg2 Pow(.,2) [32,197,768]", D.POW, x, np.array(2.0, np.float32))
+    binary("cfg2 Div [32,197,768]/[32,197,1]", D.DIV, x, mean + np.float32(1.5))
+    binary("cfg2 Mul gamma [32,197,768]*[768]", D.MUL, x, c2["gamma"])
+    c3 = synth.cfg3()
+    unary("cfg3 Gelu [32,197,3072]", D.GELU, c3["x"])
+    unary("cfg3 Erf [32,197,3072]", D.ERF, c3["x"])
+    binary("cfg3 Mul [32,197,3072]*[32,197,3072]", D.MUL, c3["x"], c3["x"])
+    se = c3["se"]
+    reduce("cfg3 ReduceMean(H,W) [32,576,7,7]", D.REDUCE_MEAN, se, 32 * 576, 49, 1)
+    unary("cfg3 HardSigmoid [32,576,1,1]", D.HARDSIGMOID, np.zeros((32, 576, 1, 1), np.float32), 1.0 / 6.0, 0.5)
+    binary("cfg3 Mul [32,576,7,7]*[32,576,1,1]", D.MUL, se, np.ones((32, 576, 1, 1), np.float32))
+    return ops
+
+
+def session_table(synth):
+    """Whole `run()` calls on host tensors (upload, kernels, download) for the graph-level configurations,
+    with the device-only share from the session's own per-op events."""
+    from altius_amd import graphs
+    from altius_amd.graph import Tensor
+    from altius_amd.session import HipSessionBuilder
+
+    rows = []
+
+    def measure(name, model, x, alg_bytes):
+        sess = HipSessionBuilder(model).with_profiling_enabled(True).build()
+        best_run, best_dev = float("inf"), float("inf")
+        t_in = Tensor.from_numpy(x)              # the caller's host tensor, as the reference's run() takes it
+        for _ in range(5):
+            outs = sess.run([t_in], copy=False)
+            best_run = min(best_run, sess.last_run_ms())
+            best_dev = min(best_dev, sum(sess.profile().values()))
+            del outs                             # output tensors dropped, as a caller would after use
+        rows.append({"graph": name, "algorithmic_bytes": alg_bytes, "kernels_us": round(best_dev * 1e3, 1),
+                     "run_ms_with_pcie": round(best_run, 3),
+                     "kernels_GBps": round(alg_bytes / (best_dev * 1e-3) / 1e9, 1)})
+        sess.close()
+
+    c2 = synth.cfg2()
+    X, r = c2["x"].nbytes, 32 * 197 * 4
+    chain = graphs.single_input_model(c2["x"].shape, lambda m, x: graphs.layer_norm_chain(
+        m, x, c2["gamma"], c2["beta"], float(c2["eps"]))[0])
+    fused = chain.clone()
+    fused.fuse_layer_norm()
+    measure("cfg2 LayerNorm chain, 9 nodes", chain, c2["x"], 12 * X + 8 * r + 2 * 768 * 4 + 8)
+    measure("cfg2 after fuse_layer_norm, 1 node", fused, c2["x"], 2 * X + 2 * 768 * 4)
+    c3 = synth.cfg3()
+    X = c3["x"].nbytes
+    chain = graphs.single_input_model(c3["x"].shape, lambda m, x: graphs.erf_gelu_chain(m, x, float(c3["sqrt2"])))
+    fused = chain.clone()
+    fused.fuse_gelu()
+    measure("cfg3 erf-GELU chain, 5 nodes", chain, c3["x"], 11 * X + 12)
+    measure("cfg3 after fuse_gelu, 1 node", fused, c3["x"], 2 * X)
+    se = c3["se"]
+    model = graphs.single_input_model(se.shape, lambda m, x: graphs.squeeze_excite(m, x, c3["alpha"], c3["beta"]))
+    measure("cfg3 squeeze-excite, 3 nodes", model, se, 3 * se.nbytes + 4 * 32 * 576 * 4)
+    return rows
+
+
 def calibration_op(ctx, D):
     """A copy-shaped kernel of known traffic (Relu over 477 MB in, 477 MB out) used to scale the
     FETCH_SIZE / WRITE_SIZE counters of a profiling run."""
@@ -195,6 +317,8 @@ def main():
     ap.add_argument("--only", type=str, default="", help="run only kernels whose name contains this text (profiling)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a copy-shaped Relu of known size (scales rocprof byte counters)")
+    ap.add_argument("--all-configs", action="store_true",
+                    help="also time the kernels and graphs of configs[0..3] (table on stderr, 'other_configs' in the JSON)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -271,6 +395,20 @@ def main():
         },
         "per_kernel": [{k: (round(v, 2) if isinstance(v, float) else v) for k, v in r.items()} for r in rows],
     }
+
+    if args.all_configs:
+        others = []
+        for o in build_other_configs(ctx, D, synth):
+            ms = time_kernel(ctx, o, args.kernel_iters, 5)
+            gbps = o.nbytes / (ms * 1e-3) / 1e9
+            others.append({"kernel": o.name, "bytes": o.nbytes, "us": round(ms * 1e3, 2), "GBps": round(gbps, 1),
+                           "pct_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 1)})
+            log("%-44s %14d %10.2f %10.1f %8.1f" % (o.name, o.nbytes, ms * 1e3, gbps, 100.0 * gbps / HBM_PEAK_GBPS))
+        graphs_rows = session_table(synth)
+        for r in graphs_rows:
+            log("%-40s kernels %9.1f us (%7.1f GB/s)   run() incl. PCIe %9.3f ms"
+                % (r["graph"], r["kernels_us"], r["kernels_GBps"], r["run_ms_with_pcie"]))
+        result["other_configs"] = {"kernels": others, "graphs": graphs_rows}
 
     if not args.no_cpu:
         threads = min(16, os.cpu_count() or 1)

@@ -80,6 +80,22 @@ int ahip_event_synchronize(ahip_ctx *ctx, void *event);
 int ahip_event_elapsed_ms(ahip_ctx *ctx, void *start, void *stop, float *ms);
 int ahip_event_destroy(ahip_ctx *ctx, void *event);
 
+/* Code objects built elsewhere (hipcc --genco --offload-arch=gfx950) and loaded
+ * at run time, then launched by kernel name on the context's stream.  Same role
+ * as the reference's ClangSession, which dlopen()s a compiled model and calls
+ * its exported entry (crates/session_clang/src/builder.rs:44-76,
+ * crates/session_clang/src/session.rs:46-56).  image points to `bytes` bytes
+ * of a gfx950 code object (raw or clang offload bundle); it may be freed after
+ * the call.  grid counts BLOCKS per dimension; args[i] points to the i-th
+ * kernel argument.  Unknown kernel names and launch shapes the device cannot
+ * run (block of more than 1024 threads, zero extent, shared memory beyond
+ * 160 KiB) are refused with AHIP_ERR_ARG before anything is launched. */
+typedef struct ahip_module ahip_module;
+int ahip_module_load(ahip_ctx *ctx, const void *image, size_t bytes, ahip_module **module);
+int ahip_module_unload(ahip_ctx *ctx, ahip_module *module);
+int ahip_launch(ahip_ctx *ctx, ahip_module *module, const char *kernel, const uint32_t grid[3],
+                const uint32_t block[3], uint32_t shared_bytes, void **args);
+
 /* ------------------------------------------------------------------------
  * Host-side index math (no device needed).
  * ---------------------------------------------------------------------- */
@@ -244,7 +260,10 @@ int ahip_fuse_gelu(ahip_model *model, int *count);
 int ahip_fuse_fast_gelu(ahip_model *model, int *count);
 int ahip_eliminate_identity(ahip_model *model, int *count);
 
-/* Host tensors (crates/core/src/tensor.rs:61-76).  data is copied; NULL data gives zeros. */
+/* Host tensors (crates/core/src/tensor.rs:61-76).  data is copied; NULL data gives zeros.
+ * Storage of 64 KiB and more is pinned (page-locked) host memory from a process-wide pool when
+ * a device is present, so that ahip_session_run moves it over PCIe by DMA; a freed tensor's
+ * block is kept for the next tensor of its size class. */
 int ahip_tensor_new(int elem_type, int rank, const int64_t *dims, const void *data, size_t nbytes,
                     ahip_tensor **tensor);
 void ahip_tensor_free(ahip_tensor *tensor);
@@ -253,6 +272,15 @@ int ahip_tensor_rank(const ahip_tensor *tensor);
 int ahip_tensor_dims(const ahip_tensor *tensor, int64_t *dims, int capacity);
 size_t ahip_tensor_nbytes(const ahip_tensor *tensor);
 const void *ahip_tensor_data(const ahip_tensor *tensor);
+/* Writable view of the same bytes, to fill a tensor made with NULL data in place
+ * (Tensor::data_mut, crates/core/src/tensor.rs:318). */
+void *ahip_tensor_data_mut(ahip_tensor *tensor);
+
+/* The pinned pool behind host tensors: bytes handed out, bytes cached for reuse, page-locking
+ * allocations made so far and requests served from the cache (any pointer may be NULL).
+ * ahip_host_pool_trim frees the cached blocks and returns the number of bytes freed. */
+int ahip_host_pool_stats(size_t *live_bytes, size_t *cached_bytes, size_t *pinned_allocations, size_t *reuses);
+size_t ahip_host_pool_trim(void);
 
 /* ------------------------------------------------------------------------
  * Session: InterpreterSessionBuilder / InterpreterSession

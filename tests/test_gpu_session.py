@@ -8,10 +8,10 @@ import pytest
 import oracle as O
 from altius_amd import synth
 from altius_amd._lib import ERR_ARG, ERR_SHAPE, ERR_UNSUPPORTED, AltiusHipError
-from altius_amd.graph import F32, I64, Model, Op
+from altius_amd.graph import F32, I64, Model, Op, Tensor, host_pool_stats, host_pool_trim
+from altius_amd.graphs import erf_gelu_chain, layer_norm_chain
 from altius_amd.session import HipSessionBuilder
 from conftest import assert_bits_equal, assert_close
-from test_host import erf_gelu_chain, layer_norm_chain
 
 pytestmark = pytest.mark.gpu
 
@@ -303,3 +303,39 @@ def test_session_model_accessor_and_threads_option(case):
     assert [n["op_name"] for n in view.nodes()] == ["Sub"] and view.inputs == m.inputs
     (z,) = sess.run([np.full([5], 3, np.float32), np.full([5], 1, np.float32)])
     assert z.tolist() == [2.0] * 5
+
+
+def test_io_tensors_live_in_recycled_pinned_memory(case):
+    """Inputs made through the C ABI and outputs made by run() are pinned blocks from the pool;
+    in steady state a run page-locks nothing new."""
+    case("session pinned I/O")
+    c = synth.cfg2(batch=2)
+    x = c["x"]                                   # 1.2 MB
+    m = Model()
+    xin = m.new_val_named_and_shaped("x", x.shape)
+    y = m.new_val()
+    m.add_node(Op.LayerNormalization, [xin, m.new_initializer(c["gamma"]), m.new_initializer(c["beta"])], [y],
+               axis=-1, epsilon=1e-5, stash_type=1)
+    m.add_input(xin)
+    m.add_output(y)
+    sess = HipSessionBuilder(m).build()
+    want = O.layer_norm(x, c["gamma"], c["beta"], 1e-5)
+    host_pool_trim()
+    base = host_pool_stats()
+    t = Tensor.from_numpy(x)
+    assert host_pool_stats()[0] > base[0] and host_pool_stats()[2] == base[2] + 1     # one page-locked block
+    (out,) = sess.run([t], copy=False)
+    assert_close(out, want, what="pinned run")
+    assert host_pool_stats()[2] == base[2] + 2                                         # input + output
+    del out
+    for _ in range(3):
+        (out,) = sess.run([t], copy=False)
+        assert_close(out, want, what="pinned run, recycled output")
+        del out
+    st = host_pool_stats()
+    assert st[2] == base[2] + 2 and st[3] >= base[3] + 3                               # nothing new, 3 reuses
+    del t
+    assert host_pool_stats()[0] == base[0]
+    assert host_pool_trim() >= 2 * x.nbytes and host_pool_stats()[1] == 0
+    (out,) = sess.run([x])                                                             # still works after a trim
+    assert_close(out, want, what="after trim")

@@ -12,7 +12,8 @@ import pytest
 from altius_amd import _lib
 from altius_amd import device as D
 from altius_amd._lib import ERR_ARG, ERR_SHAPE, AltiusHipError
-from altius_amd.graph import F32, I64, Model, Op, Tensor
+from altius_amd.graph import F32, I64, Model, Op, Tensor, host_pool_stats, host_pool_trim
+from altius_amd.graphs import erf_gelu_chain, layer_norm_chain
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -177,25 +178,6 @@ def test_shape_inference_errors_are_values_not_aborts():
     assert "MatMul" in e.value.message
 
 
-def layer_norm_chain(m, x, gamma, beta, eps=1e-5):
-    """The 9-node chain ONNX exporters emit for LayerNorm (crates/core/src/optimize/layer_norm_fusion.rs:9-16)."""
-    two = m.new_initializer(np.array(2.0, np.float32))
-    e = m.new_initializer(np.array(eps, np.float32))
-    g = m.new_initializer(gamma)
-    b = m.new_initializer(beta)
-    v = [m.new_val() for _ in range(9)]
-    m.add_node(Op.ReduceMean, [x], [v[0]], axes=[-1], keep_dims=True)
-    m.add_node(Op.Sub, [x, v[0]], [v[1]])
-    m.add_node(Op.Pow, [v[1], two], [v[2]])
-    m.add_node(Op.ReduceMean, [v[2]], [v[3]], axes=[-1], keep_dims=True)
-    m.add_node(Op.Add, [v[3], e], [v[4]])
-    m.add_node(Op.Sqrt, [v[4]], [v[5]])
-    m.add_node(Op.Div, [v[1], v[5]], [v[6]])
-    m.add_node(Op.Mul, [v[6], g], [v[7]])
-    m.add_node(Op.Add, [v[7], b], [v[8]])
-    return v[8], g, b
-
-
 def test_fuse_layer_norm():
     m = Model()
     x = m.new_val_named_and_shaped("x", [2, 5, 8])
@@ -233,19 +215,6 @@ def test_fuse_layer_norm():
     m.add_input(x)
     m.add_output(b2)
     assert m.fuse_layer_norm() == 0 and len(m.nodes()) == 2
-
-
-def erf_gelu_chain(m, x, sqrt2=1.4142135):
-    c = m.new_initializer(np.array(sqrt2, np.float32))
-    one = m.new_initializer(np.array(1.0, np.float32))
-    half = m.new_initializer(np.array(0.5, np.float32))
-    v = [m.new_val() for _ in range(5)]
-    m.add_node(Op.Div, [x, c], [v[0]])
-    m.add_node(Op.Erf, [v[0]], [v[1]])
-    m.add_node(Op.Add, [v[1], one], [v[2]])
-    m.add_node(Op.Mul, [x, v[2]], [v[3]])
-    m.add_node(Op.Mul, [v[3], half], [v[4]])
-    return v[4]
 
 
 def test_fuse_gelu():
@@ -329,6 +298,10 @@ def test_argument_errors():
         _lib.check(L.ahip_model_add_initializer(m.handle, x, F32, 1, check_dims, data.ctypes.data, data.nbytes))
     assert L.ahip_session_builder_new(None, None) == ERR_ARG
     assert L.ahip_tensor_new(7, 0, None, None, 0, None) == ERR_ARG
+    # device entry points refuse a null context before touching the runtime
+    assert L.ahip_module_load(None, None, 0, None) == ERR_ARG
+    assert L.ahip_launch(None, None, b"k", None, None, 0, None) == ERR_ARG
+    assert b"null context" in L.ahip_last_error(None)
 
 
 def test_host_tensor_round_trip():
@@ -338,3 +311,29 @@ def test_host_tensor_round_trip():
         back = t.numpy()
         assert back.dtype == arr.dtype and np.array_equal(back, arr)
     assert Tensor.from_numpy(np.array([1, 2], np.int64)).elem_ty == I64
+
+
+def test_host_tensor_views_and_pool_without_a_device():
+    """Large tensors ask the pinned pool first; the pool's counters never go backwards and the
+    bytes are the same whichever memory holds them.  view() aliases the tensor's own storage."""
+    before = host_pool_stats()
+    a = np.arange(1 << 18, dtype=np.float32).reshape(512, 512)      # 1 MiB: above the pool's threshold
+    t = Tensor.from_numpy(a)
+    v = t.view()
+    assert v.shape == (512, 512) and np.array_equal(v, a)
+    v[0, 0] = 42.0                                                  # Tensor::data_mut
+    assert t.numpy()[0, 0] == 42.0 and a[0, 0] == 0.0               # the tensor holds a copy of `a`
+    z = Tensor.zeros([3, 5])
+    assert z.dims == [3, 5] and not z.view().any()
+    z.view()[:] = 7
+    assert np.all(z.numpy() == 7)
+    live = host_pool_stats()[0]
+    del v, t
+    after = host_pool_stats()
+    assert after[0] <= live and after[2] >= before[2] and after[3] >= before[3]
+    host_pool_trim()
+    assert host_pool_stats()[1] == 0
+    keep = Tensor.from_numpy(a).view()                              # the view keeps its tensor alive
+    import gc
+    gc.collect()
+    assert np.array_equal(keep, a)
