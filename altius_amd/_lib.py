@@ -9,7 +9,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libaltius_hip.so")
 
-OK, ERR_HIP, ERR_ARG, ERR_SHAPE, ERR_UNSUPPORTED, ERR_OOM = 0, 1, 2, 3, 4, 5
+OK, ERR_HIP, ERR_ARG, ERR_SHAPE, ERR_UNSUPPORTED, ERR_OOM, ERR_IO = 0, 1, 2, 3, 4, 5, 6
 MAX_RANK = 8
 
 c_int = ctypes.c_int
@@ -38,6 +38,7 @@ _CODE_NAMES = {
     ERR_SHAPE: "Shape",
     ERR_UNSUPPORTED: "Message",
     ERR_OOM: "OOM",
+    ERR_IO: "Io",
 }
 
 
@@ -116,6 +117,24 @@ def _declare_graph(L):
     f("ahip_model_graph_io", [c_void_p, c_int, P(c_int64), c_int, P(c_int)])
     f("ahip_model_topo_sort", [c_void_p, P(c_int64), c_int, P(c_int)])
     f("ahip_model_node_info", [c_void_p, c_int64, P(c_int), P(OpAttrs), P(c_int), P(c_int64), P(c_int), P(c_int64), c_int])
+    f("ahip_model_load_onnx", [c_char_p, P(c_void_p)])
+    f("ahip_model_load_onnx_buffer", [c_void_p, c_size_t, P(c_void_p)])
+    f("ahip_model_opset_version", [c_void_p], c_int64)
+    f("ahip_model_num_values", [c_void_p], c_int64)
+    f("ahip_model_num_nodes", [c_void_p], c_int64)
+    f("ahip_model_value_info", [c_void_p, c_int64, P(c_char_p), P(c_int), P(c_int), P(c_int64), c_int])
+    f("ahip_model_initializer", [c_void_p, c_int64, P(c_void_p)])
+    f("ahip_model_node_name", [c_void_p, c_int64], c_char_p)
+    f("ahip_node_set_attr_int", [c_void_p, c_int64, c_char_p, c_int64])
+    f("ahip_node_set_attr_float", [c_void_p, c_int64, c_char_p, c_float])
+    f("ahip_node_set_attr_ints", [c_void_p, c_int64, c_char_p, P(c_int64), c_int])
+    f("ahip_node_set_attr_string", [c_void_p, c_int64, c_char_p, c_char_p])
+    f("ahip_node_set_attr_tensor", [c_void_p, c_int64, c_char_p, c_void_p])
+    f("ahip_node_get_attr_int", [c_void_p, c_int64, c_char_p, P(c_int64)])
+    f("ahip_node_get_attr_float", [c_void_p, c_int64, c_char_p, P(c_float)])
+    f("ahip_node_get_attr_ints", [c_void_p, c_int64, c_char_p, P(c_int64), c_int, P(c_int)])
+    f("ahip_node_get_attr_string", [c_void_p, c_int64, c_char_p, c_char_p, c_int, P(c_int)])
+    f("ahip_node_get_attr_tensor", [c_void_p, c_int64, c_char_p, P(c_void_p)])
     f("ahip_model_infer_value_shape", [c_void_p, c_int64, P(c_int), P(c_int), P(c_int64)])
     f("ahip_model_execution_plan", [c_void_p, P(c_int64), P(c_int), c_int, P(c_int64), c_int, P(c_int), P(c_int)])
     for name in ("ahip_fuse_layer_norm", "ahip_fuse_gelu", "ahip_fuse_fast_gelu", "ahip_eliminate_identity"):

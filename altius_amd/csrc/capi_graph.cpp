@@ -9,6 +9,7 @@
 #include "core/shape.h"
 #include "device/ctx.h"
 #include "device/host_pool.h"
+#include "onnx/load.h"
 #include "session/hip_session.h"
 #include "session/plan.h"
 
@@ -41,11 +42,15 @@ int fail(int code, const std::string &msg) {
 
 bool valid_elem_type(int t) { return t >= AHIP_BOOL && t <= AHIP_I64; }
 
-Op op_from_c(int kind, const ahip_op_attrs *a) {
+Op op_from_c(int kind, const ahip_op_attrs *a, int64_t opset_version) {
     Op op(static_cast<OpKind>(kind));
-    ahip_op_attrs d;
-    ahip_op_attrs_default(&d);
-    if (!a) a = &d;
+    if (!a) {
+        // No attribute block: the operator starts from the defaults the ONNX loader gives it
+        // (Gemm alpha = beta = 1, LeakyRelu alpha = 0.01, Flatten axis = 1, ...).
+        const char *onnx = onnx_type_of(op.kind);
+        if (onnx) op_from_onnx_type(onnx, opset_version, &op);
+        return op;
+    }
     op.axis = a->axis;
     op.axes.assign(a->axes, a->axes + (a->n_axes < 0 ? 0 : a->n_axes > AHIP_MAX_RANK ? AHIP_MAX_RANK : a->n_axes));
     op.keep_dims = a->keep_dims != 0;
@@ -149,7 +154,7 @@ int ahip_model_add_node(ahip_model *model, int op_kind, const ahip_op_attrs *att
     if (!model || op_kind < 0 || op_kind >= AHIP_OP_COUNT || n_inputs < 0 || n_outputs < 0 ||
         (n_inputs && !inputs) || (n_outputs && !outputs))
         return fail(AHIP_ERR_ARG, "ahip_model_add_node: invalid argument");
-    Node node(op_from_c(op_kind, attrs));
+    Node node(op_from_c(op_kind, attrs, model->m.opset_version));
     if (name) node.with_name(name);
     for (int i = 0; i < n_inputs; i++) {
         if (!valid_value(model, inputs[i])) return fail(AHIP_ERR_ARG, "ahip_model_add_node: unknown input value");
@@ -253,6 +258,169 @@ int ahip_model_execution_plan(const ahip_model *model, int64_t *node_ids, int *f
     if (free_offsets && (int)plan.size() <= node_capacity) free_offsets[plan.size()] = nf;
     *n_nodes = (int)plan.size();
     *n_free = nf;
+    return AHIP_OK;
+}
+
+// ---- ONNX loader, value / node inspection, attributes by name ------------------------------
+
+namespace {
+
+int load_error_code(const ModelLoadError &e) {
+    switch (e.kind) {
+    case ModelLoadError::Io: return AHIP_ERR_IO;
+    case ModelLoadError::Todo: return AHIP_ERR_UNSUPPORTED;
+    default: return AHIP_ERR_ARG;
+    }
+}
+
+Node *live_node(ahip_model *m, int64_t id) {
+    if (!m || id < 0 || (size_t)id >= m->m.graph.nodes.size() || m->m.graph.nodes[(size_t)id].deleted) return nullptr;
+    return &m->m.graph.nodes[(size_t)id];
+}
+const Node *live_node_c(const ahip_model *m, int64_t id) { return live_node(const_cast<ahip_model *>(m), id); }
+
+int no_attr(const char *fn, const Node &n, const char *name) {
+    return fail(AHIP_ERR_ARG, std::string(fn) + ": " + n.op.name() + " has no attribute '" + name + "' of that kind");
+}
+
+}  // namespace
+
+int ahip_model_load_onnx(const char *path, ahip_model **model) {
+    if (!path || !model) return fail(AHIP_ERR_ARG, "ahip_model_load_onnx: null argument");
+    *model = nullptr;
+    ahip_model *m = new (std::nothrow) ahip_model();
+    if (!m) return fail(AHIP_ERR_OOM, "ahip_model_load_onnx: out of host memory");
+    ModelLoadError e;
+    if (!load_onnx(path, &m->m, &e)) {
+        delete m;
+        return fail(load_error_code(e), e.to_string());
+    }
+    *model = m;
+    return AHIP_OK;
+}
+
+int ahip_model_load_onnx_buffer(const void *data, size_t bytes, ahip_model **model) {
+    if (!model || (!data && bytes)) return fail(AHIP_ERR_ARG, "ahip_model_load_onnx_buffer: null argument");
+    *model = nullptr;
+    ahip_model *m = new (std::nothrow) ahip_model();
+    if (!m) return fail(AHIP_ERR_OOM, "ahip_model_load_onnx_buffer: out of host memory");
+    ModelLoadError e;
+    if (!load_onnx_from_buffer(data, bytes, &m->m, &e)) {
+        delete m;
+        return fail(load_error_code(e), e.to_string());
+    }
+    *model = m;
+    return AHIP_OK;
+}
+
+int64_t ahip_model_opset_version(const ahip_model *model) { return model ? model->m.opset_version : -1; }
+int64_t ahip_model_num_values(const ahip_model *model) { return model ? (int64_t)model->m.graph.values.size() : -1; }
+int64_t ahip_model_num_nodes(const ahip_model *model) { return model ? (int64_t)model->m.graph.nodes.size() : -1; }
+
+int ahip_model_value_info(const ahip_model *model, int64_t value_id, const char **name, int *elem_type, int *rank,
+                          int64_t *dims, int dims_capacity) {
+    if (!model || !valid_value(model, value_id) || dims_capacity < 0 || (dims_capacity && !dims))
+        return fail(AHIP_ERR_ARG, "ahip_model_value_info: invalid argument");
+    const Value &v = model->m.graph.values[(ValueId)value_id];
+    if (name) *name = v.name ? v.name->c_str() : nullptr;
+    if (!v.shape) {
+        if (rank) *rank = -1;
+        return AHIP_OK;
+    }
+    if (elem_type) *elem_type = (int)v.shape->elem_ty;
+    const auto &dv = v.shape->dims.as_vec();
+    if (rank) *rank = (int)dv.size();
+    for (int i = 0; i < dims_capacity && i < (int)dv.size(); i++) dims[i] = dv[(size_t)i].fixed ? (int64_t)dv[(size_t)i].value : -1;
+    return AHIP_OK;
+}
+
+int ahip_model_initializer(const ahip_model *model, int64_t value_id, ahip_tensor **tensor) {
+    if (!model || !tensor || !valid_value(model, value_id)) return fail(AHIP_ERR_ARG, "ahip_model_initializer: invalid argument");
+    auto it = model->m.graph.inits.find((ValueId)value_id);
+    if (it == model->m.graph.inits.end()) return fail(AHIP_ERR_ARG, "ahip_model_initializer: the value has no initializer");
+    ahip_tensor *t = new (std::nothrow) ahip_tensor();
+    if (!t) return fail(AHIP_ERR_OOM, "ahip_model_initializer: out of host memory");
+    t->t = it->second;  // shares the bytes
+    *tensor = t;
+    return AHIP_OK;
+}
+
+const char *ahip_model_node_name(const ahip_model *model, int64_t node_id) {
+    const Node *n = live_node_c(model, node_id);
+    return n && n->name ? n->name->c_str() : nullptr;
+}
+
+int ahip_node_set_attr_int(ahip_model *model, int64_t node_id, const char *name, int64_t value) {
+    Node *n = live_node(model, node_id);
+    if (!n || !name) return fail(AHIP_ERR_ARG, "ahip_node_set_attr_int: invalid argument");
+    return n->op.set_int(name, value) ? AHIP_OK : no_attr("ahip_node_set_attr_int", *n, name);
+}
+int ahip_node_set_attr_float(ahip_model *model, int64_t node_id, const char *name, float value) {
+    Node *n = live_node(model, node_id);
+    if (!n || !name) return fail(AHIP_ERR_ARG, "ahip_node_set_attr_float: invalid argument");
+    return n->op.set_float(name, value) ? AHIP_OK : no_attr("ahip_node_set_attr_float", *n, name);
+}
+int ahip_node_set_attr_ints(ahip_model *model, int64_t node_id, const char *name, const int64_t *values, int count) {
+    Node *n = live_node(model, node_id);
+    if (!n || !name || count < 0 || (count && !values)) return fail(AHIP_ERR_ARG, "ahip_node_set_attr_ints: invalid argument");
+    return n->op.set_ints(name, std::vector<int64_t>(values, values + count)) ? AHIP_OK
+                                                                               : no_attr("ahip_node_set_attr_ints", *n, name);
+}
+int ahip_node_set_attr_string(ahip_model *model, int64_t node_id, const char *name, const char *value) {
+    Node *n = live_node(model, node_id);
+    if (!n || !name || !value) return fail(AHIP_ERR_ARG, "ahip_node_set_attr_string: invalid argument");
+    return n->op.set_string(name, value) ? AHIP_OK : no_attr("ahip_node_set_attr_string", *n, name);
+}
+int ahip_node_set_attr_tensor(ahip_model *model, int64_t node_id, const char *name, const ahip_tensor *value) {
+    Node *n = live_node(model, node_id);
+    if (!n || !name || !value) return fail(AHIP_ERR_ARG, "ahip_node_set_attr_tensor: invalid argument");
+    if (n->op.kind != OpKind::Constant || std::string(name) != "value") return no_attr("ahip_node_set_attr_tensor", *n, name);
+    n->op.value = std::make_shared<Tensor>(value->t);
+    return AHIP_OK;
+}
+int ahip_node_get_attr_int(const ahip_model *model, int64_t node_id, const char *name, int64_t *value) {
+    const Node *n = live_node_c(model, node_id);
+    if (!n || !name || !value) return fail(AHIP_ERR_ARG, "ahip_node_get_attr_int: invalid argument");
+    return n->op.get_int(name, value) ? AHIP_OK : no_attr("ahip_node_get_attr_int", *n, name);
+}
+int ahip_node_get_attr_float(const ahip_model *model, int64_t node_id, const char *name, float *value) {
+    const Node *n = live_node_c(model, node_id);
+    if (!n || !name || !value) return fail(AHIP_ERR_ARG, "ahip_node_get_attr_float: invalid argument");
+    return n->op.get_float(name, value) ? AHIP_OK : no_attr("ahip_node_get_attr_float", *n, name);
+}
+int ahip_node_get_attr_ints(const ahip_model *model, int64_t node_id, const char *name, int64_t *values, int capacity,
+                            int *count) {
+    const Node *n = live_node_c(model, node_id);
+    if (!n || !name || capacity < 0 || (capacity && !values)) return fail(AHIP_ERR_ARG, "ahip_node_get_attr_ints: invalid argument");
+    std::vector<int64_t> v;
+    if (!n->op.get_ints(name, &v)) return no_attr("ahip_node_get_attr_ints", *n, name);
+    for (int i = 0; i < capacity && i < (int)v.size(); i++) values[i] = v[(size_t)i];
+    if (count) *count = (int)v.size();
+    return AHIP_OK;
+}
+int ahip_node_get_attr_string(const ahip_model *model, int64_t node_id, const char *name, char *value, int capacity,
+                              int *length) {
+    const Node *n = live_node_c(model, node_id);
+    if (!n || !name || capacity < 0 || (capacity && !value)) return fail(AHIP_ERR_ARG, "ahip_node_get_attr_string: invalid argument");
+    std::string v;
+    if (!n->op.get_string(name, &v)) return no_attr("ahip_node_get_attr_string", *n, name);
+    if (capacity > 0) {
+        const size_t k = std::min<size_t>(v.size(), (size_t)capacity - 1);
+        std::memcpy(value, v.data(), k);
+        value[k] = 0;
+    }
+    if (length) *length = (int)v.size();
+    return AHIP_OK;
+}
+int ahip_node_get_attr_tensor(const ahip_model *model, int64_t node_id, const char *name, ahip_tensor **value) {
+    const Node *n = live_node_c(model, node_id);
+    if (!n || !name || !value) return fail(AHIP_ERR_ARG, "ahip_node_get_attr_tensor: invalid argument");
+    if (n->op.kind != OpKind::Constant || std::string(name) != "value" || !n->op.value)
+        return no_attr("ahip_node_get_attr_tensor", *n, name);
+    ahip_tensor *t = new (std::nothrow) ahip_tensor();
+    if (!t) return fail(AHIP_ERR_OOM, "ahip_node_get_attr_tensor: out of host memory");
+    t->t = *n->op.value;
+    *value = t;
     return AHIP_OK;
 }
 

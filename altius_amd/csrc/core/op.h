@@ -1,11 +1,14 @@
 // Operator kinds and attributes of the graph IR.
 // Mirrors altius_core::op::Op (crates/core/src/op.rs:7-57): the same 49 kinds in the
 // same order, so a graph built for the interpreter names the same operators here.
-// Attributes are kept for the operators this backend executes.
+// Every attribute the reference's loader reads is kept (op.rs:59-218), under one struct.
 #pragma once
 
 #include <stdint.h>
 
+#include <memory>
+#include <optional>
+#include <string>
 #include <vector>
 
 #include "tensor.h"
@@ -39,6 +42,26 @@ struct Op {
     int64_t stash_type = 1;
     // Cast.to
     TensorElemType to = TensorElemType::F32;
+    // Conv2d / MaxPool (op.rs:59-83)
+    std::string auto_pad;
+    std::vector<int64_t> dilations, kernel_shape, strides, padding;
+    int64_t group = 1;
+    // Transpose.perm, Split.split (op.rs:127-130, 165-168)
+    std::vector<int64_t> perm, split;
+    // Gemm (op.rs:183-188); alpha / beta above
+    bool trans_a = false, trans_b = false;
+    // BatchNormalization (op.rs:190-195); epsilon above
+    float momentum = 1e-5f;
+    bool training_mode = false;
+    // Shape (op.rs:177-181)
+    int64_t start = 0;
+    std::optional<int64_t> end;
+    // Resize (op.rs:113-121)
+    std::string coordinate_transformation_mode, mode, nearest_mode;
+    float cubic_coeff_a = -0.75f, extrapolation_value = 0.0f;
+    int64_t exclude_outside = 0;
+    // Constant.value (op.rs:206-210)
+    std::shared_ptr<Tensor> value;
 
     Op() = default;
     explicit Op(OpKind k) : kind(k) {}
@@ -75,6 +98,28 @@ struct Op {
     }
 
     const char *name() const { return op_kind_name(kind); }
+
+    // Attribute access by ONNX attribute name ("axis", "perm", "kernel_shape", "transB", ...): the
+    // one vocabulary shared by the ONNX loader and the C ABI.  Setters return false for a name
+    // this operator kind does not carry.
+    bool set_int(const std::string &name, int64_t v);
+    bool set_float(const std::string &name, float v);
+    bool set_ints(const std::string &name, const std::vector<int64_t> &v);
+    bool set_string(const std::string &name, const std::string &v);
+    bool get_int(const std::string &name, int64_t *v) const;
+    bool get_float(const std::string &name, float *v) const;
+    bool get_ints(const std::string &name, std::vector<int64_t> *v) const;
+    bool get_string(const std::string &name, std::string *v) const;
 };
+
+// The operator a freshly loaded ONNX node of this type starts from: kind plus the defaults the
+// reference's loader applies for absent attributes (crates/core/src/onnx/load.rs:171-361).
+// Returns false for an op_type the reference does not know.
+bool op_from_onnx_type(const std::string &op_type, int64_t opset_version, Op *op);
+// Attributes the reference's loader insists on (`get_attribute(..)?`): missing ones are an error.
+std::vector<std::string> required_onnx_attributes(const Op &op, int64_t opset_version);
+// ONNX op_type string of a kind ("Relu" for ReLU, "Conv" for Conv2d, ...); nullptr for kinds
+// that have no ONNX spelling (Gelu, FusedElemwise).
+const char *onnx_type_of(OpKind k);
 
 }  // namespace altius

@@ -193,13 +193,108 @@ class Model:
         return v.value if rc == 0 else None
 
     # --- nodes --------------------------------------------------------------------
+    _ATTR_ALIASES = {"keep_dims": "keepdims", "trans_a": "transA", "trans_b": "transB", "padding": "pads"}
+
     def add_node(self, op_kind, inputs, outputs, name=None, **attrs):
-        a = make_attrs(**attrs)
+        """Attributes go by their ONNX names (axis, axes, keepdims, perm, kernel_shape, transB, to, ...;
+        keep_dims / trans_a / trans_b / padding are accepted spellings of the reference's field names).
+        Absent ones keep the defaults the ONNX loader applies."""
         nid = ctypes.c_int64()
-        check(self.L.ahip_model_add_node(self.handle, op_kind, ctypes.byref(a), name.encode() if name else None,
+        check(self.L.ahip_model_add_node(self.handle, op_kind, None, name.encode() if name else None,
                                          len(inputs), i64_array(inputs), len(outputs), i64_array(outputs),
                                          ctypes.byref(nid)))
+        for key, value in attrs.items():
+            self.set_attr(nid.value, self._ATTR_ALIASES.get(key, key), value)
         return nid.value
+
+    def set_attr(self, node_id, name, value):
+        n = name.encode()
+        if isinstance(value, Tensor):
+            check(self.L.ahip_node_set_attr_tensor(self.handle, node_id, n, value.handle))
+        elif isinstance(value, np.ndarray):
+            t = Tensor.from_numpy(value)
+            check(self.L.ahip_node_set_attr_tensor(self.handle, node_id, n, t.handle))
+        elif isinstance(value, str):
+            check(self.L.ahip_node_set_attr_string(self.handle, node_id, n, value.encode()))
+        elif isinstance(value, (list, tuple)):
+            check(self.L.ahip_node_set_attr_ints(self.handle, node_id, n, i64_array(value), len(value)))
+        elif isinstance(value, (bool, int, np.integer)):
+            check(self.L.ahip_node_set_attr_int(self.handle, node_id, n, int(value)))
+        elif isinstance(value, (float, np.floating)):
+            check(self.L.ahip_node_set_attr_float(self.handle, node_id, n, float(value)))
+        else:
+            raise TypeError(f"attribute {name}: unsupported value {value!r}")
+
+    def get_attr(self, node_id, name, kind):
+        """kind: 'int', 'float', 'ints', 'string' or 'tensor'."""
+        n = name.encode()
+        if kind == "int":
+            v = ctypes.c_int64()
+            check(self.L.ahip_node_get_attr_int(self.handle, node_id, n, ctypes.byref(v)))
+            return v.value
+        if kind == "float":
+            v = ctypes.c_float()
+            check(self.L.ahip_node_get_attr_float(self.handle, node_id, n, ctypes.byref(v)))
+            return v.value
+        if kind == "ints":
+            c = ctypes.c_int()
+            check(self.L.ahip_node_get_attr_ints(self.handle, node_id, n, None, 0, ctypes.byref(c)))
+            buf = (ctypes.c_int64 * max(c.value, 1))()
+            check(self.L.ahip_node_get_attr_ints(self.handle, node_id, n, buf, c.value, ctypes.byref(c)))
+            return [int(buf[i]) for i in range(c.value)]
+        if kind == "string":
+            c = ctypes.c_int()
+            check(self.L.ahip_node_get_attr_string(self.handle, node_id, n, None, 0, ctypes.byref(c)))
+            buf = ctypes.create_string_buffer(c.value + 1)
+            check(self.L.ahip_node_get_attr_string(self.handle, node_id, n, buf, c.value + 1, ctypes.byref(c)))
+            return buf.value.decode()
+        if kind == "tensor":
+            h = ctypes.c_void_p()
+            check(self.L.ahip_node_get_attr_tensor(self.handle, node_id, n, ctypes.byref(h)))
+            return Tensor(h).numpy()
+        raise ValueError(kind)
+
+    # --- ONNX files (altius_core::onnx::load_onnx) ----------------------------------------------
+    @classmethod
+    def load_onnx(cls, path):
+        h = ctypes.c_void_p()
+        check(_lib.lib().ahip_model_load_onnx(str(path).encode(), ctypes.byref(h)))
+        return cls(_handle=h)
+
+    @classmethod
+    def load_onnx_from_buffer(cls, data):
+        data = bytes(data)
+        buf = ctypes.create_string_buffer(data, max(1, len(data)))
+        h = ctypes.c_void_p()
+        check(_lib.lib().ahip_model_load_onnx_buffer(ctypes.cast(buf, ctypes.c_void_p), len(data), ctypes.byref(h)))
+        return cls(_handle=h)
+
+    @property
+    def opset_version(self):
+        return self.L.ahip_model_opset_version(self.handle)
+
+    def num_values(self):
+        return self.L.ahip_model_num_values(self.handle)
+
+    def value_info(self, value_id):
+        """(name or None, elem type or None, dims or None); dynamic dimensions read -1."""
+        name, ty, rank = ctypes.c_char_p(), ctypes.c_int(), ctypes.c_int()
+        dims = (ctypes.c_int64 * 16)()
+        check(self.L.ahip_model_value_info(self.handle, value_id, ctypes.byref(name), ctypes.byref(ty),
+                                           ctypes.byref(rank), dims, 16))
+        nm = name.value.decode() if name.value is not None else None
+        if rank.value < 0:
+            return nm, None, None
+        return nm, ty.value, [int(dims[i]) for i in range(rank.value)]
+
+    def initializer(self, value_id):
+        h = ctypes.c_void_p()
+        check(self.L.ahip_model_initializer(self.handle, value_id, ctypes.byref(h)))
+        return Tensor(h).numpy()
+
+    def node_name(self, node_id):
+        n = self.L.ahip_model_node_name(self.handle, node_id)
+        return n.decode() if n is not None else None
 
     def add_input(self, value_id):
         check(self.L.ahip_model_add_input(self.handle, value_id))

@@ -38,6 +38,7 @@ extern "C" {
 #define AHIP_ERR_UNSUPPORTED 4 /* SessionError::Message: no kernel for this op / shape / dtype
                                   (crates/session/src/lib.rs:32-34) */
 #define AHIP_ERR_OOM 5         /* device allocation failed */
+#define AHIP_ERR_IO 6          /* ModelLoadError::Io: a model file could not be read */
 
 #define AHIP_MAX_RANK 8
 
@@ -227,7 +228,9 @@ int ahip_model_new_value_shaped(ahip_model *model, const char *name, int elem_ty
 /* graph.inits.insert (graph.rs:13); data is copied, nbytes must match the shape. */
 int ahip_model_add_initializer(ahip_model *model, int64_t value_id, int elem_type, int rank,
                                const int64_t *dims, const void *data, size_t nbytes);
-/* Graph::add_node (graph.rs:18-22); attrs may be NULL for the defaults, name may be NULL. */
+/* Graph::add_node (graph.rs:18-22); name may be NULL.  With attrs == NULL the operator starts
+ * from the defaults the ONNX loader applies to its kind (load.rs:171-361) and is then refined with
+ * ahip_node_set_attr_*; a non-NULL block sets the seven fields of ahip_op_attrs as given. */
 int ahip_model_add_node(ahip_model *model, int op_kind, const ahip_op_attrs *attrs, const char *name,
                         int n_inputs, const int64_t *inputs, int n_outputs, const int64_t *outputs,
                         int64_t *node_id);
@@ -252,6 +255,47 @@ int ahip_model_infer_value_shape(const ahip_model *model, int64_t value_id, int 
 int ahip_model_execution_plan(const ahip_model *model, int64_t *node_ids, int *free_offsets,
                               int node_capacity, int64_t *free_vals, int free_capacity, int *n_nodes,
                               int *n_free);
+
+/* ONNX files (crates/core/src/onnx/load.rs:55-63: load_onnx, load_onnx_from_buffer).  The
+ * decoder reads the protobuf wire format itself; values are created in the reference's order
+ * (initializers, graph inputs, graph outputs, then node inputs/outputs as met).  Errors mirror
+ * ModelLoadError (load.rs:25-53): AHIP_ERR_IO for the file, AHIP_ERR_ARG for a malformed or
+ * graph-less model, a missing required attribute or value type/shape, AHIP_ERR_UNSUPPORTED for
+ * operators, element types and opset domains the reference does not load. */
+int ahip_model_load_onnx(const char *path, ahip_model **model);
+int ahip_model_load_onnx_buffer(const void *data, size_t bytes, ahip_model **model);
+int64_t ahip_model_opset_version(const ahip_model *model);
+int64_t ahip_model_num_values(const ahip_model *model);
+int64_t ahip_model_num_nodes(const ahip_model *model);
+/* One value: its name (NULL if unnamed; valid until the model changes), and its declared shape:
+ * *rank is -1 when none is declared, dynamic dimensions read -1.  Any output pointer may be NULL. */
+int ahip_model_value_info(const ahip_model *model, int64_t value_id, const char **name, int *elem_type,
+                          int *rank, int64_t *dims, int dims_capacity);
+/* A copy of the initializer bound to a value (graph.inits); AHIP_ERR_ARG if it has none. */
+int ahip_model_initializer(const ahip_model *model, int64_t value_id, ahip_tensor **tensor);
+/* Node name (NULL if unnamed). */
+const char *ahip_model_node_name(const ahip_model *model, int64_t node_id);
+
+/* Operator attributes by their ONNX names ("axis", "axes", "keepdims", "perm", "split", "to",
+ * "kernel_shape", "strides", "pads", "dilations", "group", "auto_pad", "alpha", "beta",
+ * "transA", "transB", "epsilon", "momentum", "training_mode", "stash_type", "start", "end",
+ * "mode", "nearest_mode", "coordinate_transformation_mode", "cubic_coeff_a", "exclude_outside",
+ * "extrapolation_value", "value"): every field of the attribute structs in op.rs:59-218.
+ * AHIP_ERR_ARG when the node's operator does not carry an attribute of that name and kind. */
+int ahip_node_set_attr_int(ahip_model *model, int64_t node_id, const char *name, int64_t value);
+int ahip_node_set_attr_float(ahip_model *model, int64_t node_id, const char *name, float value);
+int ahip_node_set_attr_ints(ahip_model *model, int64_t node_id, const char *name, const int64_t *values, int n);
+int ahip_node_set_attr_string(ahip_model *model, int64_t node_id, const char *name, const char *value);
+int ahip_node_set_attr_tensor(ahip_model *model, int64_t node_id, const char *name, const ahip_tensor *value);
+int ahip_node_get_attr_int(const ahip_model *model, int64_t node_id, const char *name, int64_t *value);
+int ahip_node_get_attr_float(const ahip_model *model, int64_t node_id, const char *name, float *value);
+/* *n gets the full count even beyond capacity. */
+int ahip_node_get_attr_ints(const ahip_model *model, int64_t node_id, const char *name, int64_t *values,
+                            int capacity, int *n);
+/* Copies at most capacity-1 characters and a terminator; *n gets the full length. */
+int ahip_node_get_attr_string(const ahip_model *model, int64_t node_id, const char *name, char *value,
+                              int capacity, int *n);
+int ahip_node_get_attr_tensor(const ahip_model *model, int64_t node_id, const char *name, ahip_tensor **value);
 
 /* Fusion passes (crates/core/src/optimize/{layer_norm_fusion,gelu_fusion,fast_gelu_fusion,
  * identity_elim}.rs).  *count (may be NULL) gets the number of rewrites. */
