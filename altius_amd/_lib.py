@@ -67,6 +67,15 @@ def _declare(L):
     f("ahip_event_synchronize", [c_void_p, c_void_p])
     f("ahip_event_elapsed_ms", [c_void_p, c_void_p, c_void_p, P(c_float)])
     f("ahip_event_destroy", [c_void_p, c_void_p])
+    f("ahip_copy_strided", [c_void_p, c_void_p, c_void_p, c_int, c_int, P(c_int64), P(c_int64), P(c_int64)])
+    f("ahip_transpose", [c_void_p, c_void_p, c_void_p, c_int, c_int, P(c_int64), P(c_int64)])
+    f("ahip_gather", [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_size_t, c_size_t, c_size_t, c_size_t])
+    f("ahip_where", [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, P(c_int64), P(c_int64), P(c_int64),
+                     P(c_int64)])
+    f("ahip_greater", [c_void_p, c_void_p, c_void_p, c_void_p, c_int, P(c_int64), P(c_int64), P(c_int64)])
+    f("ahip_cast", [c_void_p, c_void_p, c_void_p, c_int, c_int, c_size_t])
+    f("ahip_batchnorm", [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t,
+                         c_float])
     f("ahip_module_load", [c_void_p, c_void_p, c_size_t, P(c_void_p)])
     f("ahip_module_unload", [c_void_p, c_void_p])
     f("ahip_launch", [c_void_p, c_void_p, c_char_p, P(ctypes.c_uint32), P(ctypes.c_uint32), ctypes.c_uint32,

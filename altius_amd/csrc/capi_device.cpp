@@ -120,7 +120,8 @@ int ahip_memset_async(ahip_ctx *ctx, void *dst, int byte_value, size_t bytes) {
 
 int ahip_sync(ahip_ctx *ctx) {
     REQUIRE_CTX(ctx, "ahip_sync");
-    return ctx->d.check(hipStreamSynchronize(ctx->d.stream), "hipStreamSynchronize");
+    const int rc = ctx->d.check(hipStreamSynchronize(ctx->d.stream), "hipStreamSynchronize");
+    return rc ? rc : altius::check_device_flags(ctx->d);
 }
 
 int ahip_host_alloc(ahip_ctx *ctx, size_t bytes, void **hptr) {
@@ -304,6 +305,53 @@ int ahip_layernorm_lastaxis(ahip_ctx *ctx, float *out, const float *in, const fl
 int ahip_reduce(ahip_ctx *ctx, int kind, float *out, const float *in, size_t outer, size_t reduce, size_t inner) {
     REQUIRE_CTX(ctx, "ahip_reduce");
     return altius::launch_reduce(ctx->d, kind, out, in, outer, reduce, inner);
+}
+
+int ahip_copy_strided(ahip_ctx *ctx, void *out, const void *in, int elem_size, int rank, const int64_t *dims,
+                      const int64_t *out_strides, const int64_t *in_strides) {
+    REQUIRE_CTX(ctx, "ahip_copy_strided");
+    if (rank > 0 && (!dims || !out_strides || !in_strides)) return ctx->d.fail(AHIP_ERR_ARG, "ahip_copy_strided: null shape");
+    return altius::launch_copy_strided(ctx->d, out, in, elem_size, rank, dims, out_strides, in_strides);
+}
+
+int ahip_transpose(ahip_ctx *ctx, void *out, const void *in, int elem_size, int rank, const int64_t *in_dims,
+                   const int64_t *perm) {
+    REQUIRE_CTX(ctx, "ahip_transpose");
+    if (rank > 0 && (!in_dims || !perm)) return ctx->d.fail(AHIP_ERR_ARG, "ahip_transpose: null shape");
+    return altius::launch_transpose(ctx->d, out, in, elem_size, rank, in_dims, perm);
+}
+
+int ahip_gather(ahip_ctx *ctx, void *out, const void *data, const void *indices, int index_size, int elem_size,
+                size_t outer, size_t axis_len, size_t n_indices, size_t inner) {
+    REQUIRE_CTX(ctx, "ahip_gather");
+    ctx->d.flags_armed = true;
+    return altius::launch_gather(ctx->d, out, data, indices, index_size, elem_size, outer, axis_len, n_indices, inner,
+                                 ctx->d.flags);
+}
+
+int ahip_where(ahip_ctx *ctx, void *out, const void *cond, const void *x, const void *y, int elem_size, int rank,
+               const int64_t *dims, const int64_t *cond_strides, const int64_t *x_strides, const int64_t *y_strides) {
+    REQUIRE_CTX(ctx, "ahip_where");
+    if (rank > 0 && (!dims || !cond_strides || !x_strides || !y_strides)) return ctx->d.fail(AHIP_ERR_ARG, "ahip_where: null shape");
+    return altius::launch_where(ctx->d, out, cond, x, y, elem_size, rank, dims, cond_strides, x_strides, y_strides);
+}
+
+int ahip_greater(ahip_ctx *ctx, void *out, const float *a, const float *b, int rank, const int64_t *dims,
+                 const int64_t *a_strides, const int64_t *b_strides) {
+    REQUIRE_CTX(ctx, "ahip_greater");
+    if (rank > 0 && (!dims || !a_strides || !b_strides)) return ctx->d.fail(AHIP_ERR_ARG, "ahip_greater: null shape");
+    return altius::launch_greater(ctx->d, static_cast<uint8_t *>(out), a, b, rank, dims, a_strides, b_strides);
+}
+
+int ahip_cast(ahip_ctx *ctx, void *out, const void *in, int from_elem_type, int to_elem_type, size_t n) {
+    REQUIRE_CTX(ctx, "ahip_cast");
+    return altius::launch_cast(ctx->d, out, in, from_elem_type, to_elem_type, n);
+}
+
+int ahip_batchnorm(ahip_ctx *ctx, float *out, const float *x, const float *scale, const float *bias, const float *mean,
+                   const float *var, size_t n, size_t c, size_t hw, float epsilon) {
+    REQUIRE_CTX(ctx, "ahip_batchnorm");
+    return altius::launch_batchnorm(ctx->d, out, x, scale, bias, mean, var, n, c, hw, epsilon);
 }
 
 }  // extern "C"

@@ -82,12 +82,8 @@ __global__ __launch_bounds__(BLOCK) void binary_flat_scalar(float *__restrict__ 
 // ---------------------------------------------------------------------------
 // Strided kernel.
 // ---------------------------------------------------------------------------
-// Division of an index below 2^31 by a fixed divisor as multiply-high, add,
-// shift (the divisor's magic numbers are computed once on the host).
-struct FastDiv {
-    uint32_t d, mul, shift;
-    __device__ __forceinline__ uint32_t div(uint32_t n) const { return (__umulhi(n, mul) + n) >> shift; }
-};
+using dev::FastDiv;
+using dev::make_fastdiv;
 
 struct Geom {
     // Axis 0 is the innermost (fastest) output axis.
@@ -277,17 +273,6 @@ __global__ __launch_bounds__(BLOCK) void binary_rowbcast(float *__restrict__ out
             out[i0 + j] = SMALL_IS_A ? OP::f(y[j], xs) : OP::f(xs, y[j]);
         }
     }
-}
-
-FastDiv make_fastdiv(uint32_t d) {
-    FastDiv f;
-    f.d = d;
-    uint32_t shift = 0;
-    while (shift < 32 && ((uint64_t)1 << shift) < d) shift++;
-    const uint64_t one = 1;
-    f.mul = (uint32_t)(((one << 32) * ((one << shift) - d)) / d + 1);
-    f.shift = shift;
-    return f;
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -38,6 +38,24 @@ template <bool NT> __device__ __forceinline__ void store4(float *p, const float4
     }
 }
 
+// Division of an index below 2^31 by a fixed divisor as multiply-high, add, shift (the
+// divisor's magic numbers are computed once on the host).
+struct FastDiv {
+    uint32_t d, mul, shift;
+    __device__ __forceinline__ uint32_t div(uint32_t n) const { return (__umulhi(n, mul) + n) >> shift; }
+};
+
+inline FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f;
+    f.d = d;
+    uint32_t shift = 0;
+    while (shift < 32 && ((uint64_t)1 << shift) < d) shift++;
+    const uint64_t one = 1;
+    f.mul = (uint32_t)(((one << 32) * ((one << shift) - d)) / d + 1);
+    f.shift = shift;
+    return f;
+}
+
 // The non-NaN operand wins (f32::max in the reference).
 __device__ __forceinline__ float nanmax(float a, float b) { return fmaxf(a, b); }
 

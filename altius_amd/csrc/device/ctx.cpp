@@ -54,7 +54,32 @@ int create_device_ctx(int device, hipStream_t stream, bool own_stream, DeviceCtx
     }
     ctx->scratch = static_cast<float *>(scratch);
     ctx->scratch_floats = SCRATCH_FLOATS;
+    void *flags = nullptr;
+    e = hipMalloc(&flags, 256);
+    if (e == hipSuccess) e = hipMemset(flags, 0, 256);
+    if (e != hipSuccess) {
+        if (flags) (void)hipFree(flags);
+        (void)hipFree(scratch);
+        ctx->scratch = nullptr;
+        if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+        ctx->stream = nullptr;
+        return fail(e, "hipMalloc(flags)");
+    }
+    ctx->flags = static_cast<int *>(flags);
+    ctx->flags_armed = false;
     return AHIP_OK;
+}
+
+int check_device_flags(DeviceCtx &ctx) {
+    if (!ctx.flags_armed) return AHIP_OK;
+    ctx.flags_armed = false;
+    int raised = 0;
+    int rc = ctx.check(hipMemcpy(&raised, ctx.flags, sizeof(int), hipMemcpyDeviceToHost), "hipMemcpy(flags)");
+    if (rc) return rc;
+    if (!raised) return AHIP_OK;
+    rc = ctx.check(hipMemset(ctx.flags, 0, sizeof(int)), "hipMemset(flags)");
+    if (rc) return rc;
+    return ctx.fail(AHIP_ERR_ARG, "Gather: an index is outside the gathered axis");
 }
 
 void destroy_device_ctx(DeviceCtx *ctx) {
@@ -62,6 +87,8 @@ void destroy_device_ctx(DeviceCtx *ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     ctx->scratch = nullptr;
+    if (ctx->flags) (void)hipFree(ctx->flags);
+    ctx->flags = nullptr;
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
     ctx->stream = nullptr;
 }

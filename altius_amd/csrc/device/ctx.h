@@ -21,6 +21,10 @@ struct DeviceCtx {
     // Partial results of two-stage reductions (device memory, owned).
     float *scratch = nullptr;
     size_t scratch_floats = 0;
+    // Error flags kernels raise (device memory, one int: Gather's index check); read back by
+    // check_device_flags after a synchronisation, only when a kernel that can raise one has run.
+    int *flags = nullptr;
+    bool flags_armed = false;
     // Tensors of at least this many bytes are streamed with non-temporal accesses.
     size_t nt_threshold_bytes = (size_t)128 << 20;
     std::string last_error;
@@ -38,6 +42,8 @@ const char *global_error();
 // Creates / tears down a context (stream + scratch buffer) on `device`.
 int create_device_ctx(int device, hipStream_t stream, bool own_stream, DeviceCtx *ctx, std::string *error);
 void destroy_device_ctx(DeviceCtx *ctx);
+// After the stream has been synchronised: reports and clears an error flag raised by a kernel.
+int check_device_flags(DeviceCtx &ctx);
 
 constexpr int MAX_RANK = 8;
 constexpr size_t SCRATCH_FLOATS = 1u << 20;  // 4 MiB
@@ -51,5 +57,22 @@ int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *g
                      const float *beta, size_t rows, size_t len, float eps);
 int launch_reduce(DeviceCtx &ctx, int kind, float *out, const float *in, size_t outer, size_t red,
                   size_t inner);
+
+
+// Data movement (movement.hip).  Strides are in elements; elem_size in bytes (1, 4 or 8).
+int launch_copy_strided(DeviceCtx &ctx, void *out, const void *in, int elem_size, int rank, const int64_t *dims,
+                        const int64_t *out_strides, const int64_t *in_strides);
+int launch_transpose(DeviceCtx &ctx, void *out, const void *in, int elem_size, int rank, const int64_t *in_dims,
+                     const int64_t *perm);
+// *bad_flag (device memory, zeroed by the caller) becomes 1 if an index is out of range.
+int launch_gather(DeviceCtx &ctx, void *out, const void *data, const void *indices, int index_size, int elem_size,
+                  size_t outer, size_t axis_len, size_t n_idx, size_t inner, int *bad_flag);
+int launch_where(DeviceCtx &ctx, void *out, const void *cond, const void *x, const void *y, int elem_size, int rank,
+                 const int64_t *dims, const int64_t *c_strides, const int64_t *x_strides, const int64_t *y_strides);
+int launch_greater(DeviceCtx &ctx, uint8_t *out, const float *a, const float *b, int rank, const int64_t *dims,
+                   const int64_t *a_strides, const int64_t *b_strides);
+int launch_cast(DeviceCtx &ctx, void *out, const void *in, int from_type, int to_type, size_t n);
+int launch_batchnorm(DeviceCtx &ctx, float *out, const float *x, const float *scale, const float *bias, const float *mean,
+                     const float *var, size_t n, size_t c, size_t hw, float eps);
 
 }  // namespace altius

@@ -142,5 +142,13 @@ __device__ __forceinline__ float hard_sigmoid_elem(float x, float alpha, float b
 // Op::ReLU (session.rs:801): x.max(0.0); NaN -> 0.0.
 __device__ __forceinline__ float relu_elem(float x) { return x > 0.0f ? x : 0.0f; }
 
+
+// Op::LeakyReLU (session.rs:819): alpha * x below zero, x otherwise (NaN and -0.0 pass through).
+__device__ __forceinline__ float leaky_relu_elem(float x, float alpha) { return x < 0.0f ? alpha * x : x; }
+
+// Op::Clip: min(max(x, lo), hi) as ONNX defines it; the reference interpreter has no kernel
+// (session.rs:201).  NaN stays NaN.
+__device__ __forceinline__ float clip_elem(float x, float lo, float hi) { return x != x ? x : rclamp(x, lo, hi); }
+
 }  // namespace dev
 }  // namespace altius

@@ -1,0 +1,580 @@
+// Data-movement kernels: strided copies (Transpose, Slice, Concat, Split, Expand, Tile), a tiled
+// transpose for permutations that move the innermost axis, Gather, Where, Cast, Greater and
+// BatchNormalization.  Counterparts in the reference interpreter:
+// crates/session_interpreter/src/session.rs:1134-1278 (concat, transpose), 1488-1598 (split, slice,
+// gather), 940-988 (where), 1350-1378 (cast), 1380-1431 (batch normalisation), 541-562 (greater).
+// All of them move each byte once: the roofline is HBM bandwidth, the care goes into keeping both
+// the read and the write side coalesced.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <vector>
+
+#include "common.h"
+#include "ctx.h"
+
+namespace altius {
+
+namespace {
+
+using dev::FastDiv;
+using dev::make_fastdiv;
+
+constexpr int BLOCK = 256;
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- generic strided copy --------------------------------------------------------------------
+// Logical index space dims[0..rank) (axis 0 innermost here); element `idx` is read at
+// sum(idx[d] * in_str[d]) and written at sum(idx[d] * out_str[d]).  Either side may be dense,
+// windowed (Concat / Split / Slice), permuted (Transpose) or repeated (stride 0: Expand, Tile).
+struct CopyGeom {
+    FastDiv dims[MAX_RANK];
+    uint32_t in_str[MAX_RANK];
+    uint32_t out_str[MAX_RANK];
+    int rank;
+};
+
+// T is the storage unit: 1, 4, 8 or 16 bytes (16 = four 4-byte elements moved together when the
+// innermost axis is contiguous on both sides and everything is 16-byte aligned).
+template <class T>
+__global__ __launch_bounds__(BLOCK) void copy_strided(T *__restrict__ out, const T *__restrict__ in, CopyGeom g,
+                                                      uint32_t total) {
+    const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= total) return;
+    uint32_t rest = i, src = 0, dst = 0;
+#pragma unroll
+    for (int d = 0; d < MAX_RANK; d++) {
+        if (d < g.rank) {
+            const uint32_t q = g.dims[d].div(rest);
+            const uint32_t r = rest - q * g.dims[d].d;
+            src += r * g.in_str[d];
+            dst += r * g.out_str[d];
+            rest = q;
+        }
+    }
+    out[dst] = in[src];
+}
+
+// ---- tiled transpose -------------------------------------------------------------------------
+// For permutations whose output-innermost axis is not the input-innermost axis.  View the tensor
+// as [batch..., R, ..., C, ...] where C is the input's contiguous axis and R the axis that becomes
+// contiguous in the output.  A block moves a TILE x TILE patch of (R, C) through LDS: rows of the
+// patch are read along C (coalesced), columns are written along R (coalesced).  The remaining axes
+// are enumerated by blockIdx.z through the same index decomposition as copy_strided.
+constexpr int TILE = 64;
+
+struct TransGeom {
+    uint32_t r_len, c_len;          // extents of R and C
+    uint32_t r_in_str, c_out_str;   // stride of R in the input, of C in the output (both sides' other stride is 1)
+    FastDiv bdims[MAX_RANK];        // the remaining axes (any order; innermost first)
+    uint32_t b_in_str[MAX_RANK];
+    uint32_t b_out_str[MAX_RANK];
+    int brank;
+};
+
+template <class T>
+__global__ __launch_bounds__(BLOCK) void transpose_tiled(T *__restrict__ out, const T *__restrict__ in, TransGeom g) {
+    __shared__ T tile[TILE][TILE + 1];
+    uint32_t rest = blockIdx.z, src0 = 0, dst0 = 0;
+#pragma unroll
+    for (int d = 0; d < MAX_RANK; d++) {
+        if (d < g.brank) {
+            const uint32_t q = g.bdims[d].div(rest);
+            const uint32_t r = rest - q * g.bdims[d].d;
+            src0 += r * g.b_in_str[d];
+            dst0 += r * g.b_out_str[d];
+            rest = q;
+        }
+    }
+    const uint32_t c0 = blockIdx.x * TILE, r0 = blockIdx.y * TILE;
+    const uint32_t tx = threadIdx.x & (TILE - 1), ty = threadIdx.x / TILE;  // 64 x 4
+    // read: lane tx walks C, ty (+4k) walks R
+#pragma unroll 4
+    for (int k = 0; k < TILE; k += BLOCK / TILE) {
+        const uint32_t r = r0 + ty + k, c = c0 + tx;
+        if (r < g.r_len && c < g.c_len) tile[ty + k][tx] = in[src0 + r * g.r_in_str + c];
+    }
+    __syncthreads();
+    // write: lane tx walks R, ty (+4k) walks C
+#pragma unroll 4
+    for (int k = 0; k < TILE; k += BLOCK / TILE) {
+        const uint32_t c = c0 + ty + k, r = r0 + tx;
+        if (r < g.r_len && c < g.c_len) out[dst0 + c * g.c_out_str + r] = tile[tx][ty + k];
+    }
+}
+
+// ---- gather ----------------------------------------------------------------------------------
+// out[o, j, :] = data[o, idx[j], :] with `inner` contiguous elements per row; negative indices
+// count from the end (ONNX).  Out-of-range indices read row 0 and raise the flag in *bad.
+template <class T, class I>
+__global__ __launch_bounds__(BLOCK) void gather_rows(T *__restrict__ out, const T *__restrict__ data,
+                                                     const I *__restrict__ idx, uint32_t axis_len, uint32_t n_idx,
+                                                     FastDiv inner, FastDiv idx_div, uint32_t total,
+                                                     int *__restrict__ bad) {
+    const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= total) return;
+    const uint32_t row = inner.div(i);        // o * n_idx + j
+    const uint32_t col = i - row * inner.d;
+    const uint32_t o = idx_div.div(row);
+    const uint32_t j = row - o * idx_div.d;
+    long long k = (long long)idx[j];
+    if (k < 0) k += axis_len;
+    if (k < 0 || k >= (long long)axis_len) {
+        *bad = 1;
+        k = 0;
+    }
+    out[i] = data[((size_t)o * axis_len + (size_t)k) * inner.d + col];
+}
+
+// ---- where -----------------------------------------------------------------------------------
+struct WhereGeom {
+    FastDiv dims[MAX_RANK];
+    uint32_t c_str[MAX_RANK], x_str[MAX_RANK], y_str[MAX_RANK];
+    int rank;
+};
+
+template <class T>
+__global__ __launch_bounds__(BLOCK) void where_strided(T *__restrict__ out, const uint8_t *__restrict__ cond,
+                                                       const T *__restrict__ x, const T *__restrict__ y, WhereGeom g,
+                                                       uint32_t total) {
+    const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= total) return;
+    uint32_t rest = i, ci = 0, xi = 0, yi = 0;
+#pragma unroll
+    for (int d = 0; d < MAX_RANK; d++) {
+        if (d < g.rank) {
+            const uint32_t q = g.dims[d].div(rest);
+            const uint32_t r = rest - q * g.dims[d].d;
+            ci += r * g.c_str[d];
+            xi += r * g.x_str[d];
+            yi += r * g.y_str[d];
+            rest = q;
+        }
+    }
+    out[i] = cond[ci] ? x[xi] : y[yi];
+}
+
+// ---- greater ---------------------------------------------------------------------------------
+struct CmpGeom {
+    FastDiv dims[MAX_RANK];
+    uint32_t a_str[MAX_RANK], b_str[MAX_RANK];
+    int rank;
+};
+
+__global__ __launch_bounds__(BLOCK) void greater_strided(uint8_t *__restrict__ out, const float *__restrict__ a,
+                                                         const float *__restrict__ b, CmpGeom g, uint32_t total) {
+    const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= total) return;
+    uint32_t rest = i, ai = 0, bi = 0;
+#pragma unroll
+    for (int d = 0; d < MAX_RANK; d++) {
+        if (d < g.rank) {
+            const uint32_t q = g.dims[d].div(rest);
+            const uint32_t r = rest - q * g.dims[d].d;
+            ai += r * g.a_str[d];
+            bi += r * g.b_str[d];
+            rest = q;
+        }
+    }
+    out[i] = a[ai] > b[bi] ? 1 : 0;
+}
+
+// ---- cast ------------------------------------------------------------------------------------
+// Rust `as` semantics (session.rs:1350-1378): int -> float rounds to nearest, float -> int
+// truncates and saturates with NaN -> 0, wider -> narrower int wraps, anything -> bool is != 0.
+template <class To, class From> __device__ __forceinline__ To cast_one(From v) { return (To)v; }
+template <> __device__ __forceinline__ int32_t cast_one<int32_t, float>(float v) {
+    if (v != v) return 0;
+    if (v >= 2147483648.0f) return INT32_MAX;
+    if (v <= -2147483648.0f) return INT32_MIN;
+    return (int32_t)v;
+}
+template <> __device__ __forceinline__ long long cast_one<long long, float>(float v) {
+    if (v != v) return 0;
+    if (v >= 9223372036854775808.0f) return INT64_MAX;
+    if (v <= -9223372036854775808.0f) return INT64_MIN;
+    return (long long)v;
+}
+struct BoolTag {
+    uint8_t v;
+};
+template <class From> __device__ __forceinline__ uint8_t to_bool(From v) { return v != (From)0 ? 1 : 0; }
+
+template <class To, class From, bool TO_BOOL>
+__global__ __launch_bounds__(BLOCK) void cast_flat(To *__restrict__ out, const From *__restrict__ in, size_t n) {
+    const size_t i = (size_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= n) return;
+    if (TO_BOOL)
+        out[i] = (To)to_bool<From>(in[i]);
+    else
+        out[i] = cast_one<To, From>(in[i]);
+}
+
+// ---- batch normalisation ---------------------------------------------------------------------
+// y = ((x - mean[c]) / sqrt(var[c] + eps)) * scale[c] + bias[c] on NCHW, in the reference's
+// operation order (session.rs:1424-1427): true division, no fused multiply-add.
+template <int VEC>
+__global__ __launch_bounds__(BLOCK) void batchnorm_nchw(float *__restrict__ out, const float *__restrict__ x,
+                                                        const float *__restrict__ scale, const float *__restrict__ bias,
+                                                        const float *__restrict__ mean, const float *__restrict__ var,
+                                                        FastDiv hw, FastDiv ch, uint32_t total, float eps) {
+    const uint32_t i = (blockIdx.x * BLOCK + threadIdx.x) * VEC;
+    if (i >= total) return;
+    const uint32_t plane = hw.div(i);  // n * C + c ; VEC divides H*W, so the VEC elements share a plane
+    const uint32_t c = plane - ch.div(plane) * ch.d;
+    const float m = mean[c], d = sqrtf(var[c] + eps), s = scale[c], b = bias[c];
+    if (VEC == 4) {
+        const float4 v = *reinterpret_cast<const float4 *>(x + i);
+        float4 r;
+        r.x = ((v.x - m) / d) * s + b;
+        r.y = ((v.y - m) / d) * s + b;
+        r.z = ((v.z - m) / d) * s + b;
+        r.w = ((v.w - m) / d) * s + b;
+        *reinterpret_cast<float4 *>(out + i) = r;
+    } else {
+        out[i] = ((x[i] - m) / d) * s + b;
+    }
+}
+
+struct Vec16 {
+    uint32_t a, b, c, d;
+};
+
+int fits32(DeviceCtx &ctx, size_t total, const char *what) {
+    if (total >= ((size_t)1 << 31)) return ctx.fail(AHIP_ERR_UNSUPPORTED, std::string(what) + ": more than 2^31 elements");
+    return AHIP_OK;
+}
+
+template <class T>
+void launch_copy(hipStream_t s, void *out, const void *in, const CopyGeom &g, uint32_t total) {
+    hipLaunchKernelGGL((copy_strided<T>), dim3((total + BLOCK - 1) / BLOCK), dim3(BLOCK), 0, s, static_cast<T *>(out),
+                       static_cast<const T *>(in), g, total);
+}
+
+}  // namespace
+
+int launch_copy_strided(DeviceCtx &ctx, void *out, const void *in, int elem_size, int rank, const int64_t *dims,
+                        const int64_t *out_strides, const int64_t *in_strides) {
+    if (rank < 0 || rank > MAX_RANK) return ctx.fail(AHIP_ERR_ARG, "copy: rank must be 0..8");
+    if (elem_size != 1 && elem_size != 4 && elem_size != 8) return ctx.fail(AHIP_ERR_ARG, "copy: element size must be 1, 4 or 8");
+    // Drop size-1 axes, then merge neighbours that are contiguous on both sides.
+    std::vector<int64_t> d, so, si;
+    size_t total = 1;
+    for (int i = 0; i < rank; i++) {
+        if (dims[i] < 0 || out_strides[i] < 0 || in_strides[i] < 0) return ctx.fail(AHIP_ERR_ARG, "copy: negative extent or stride");
+        total *= (size_t)dims[i];
+        if (dims[i] == 1) continue;
+        d.push_back(dims[i]);
+        so.push_back(out_strides[i]);
+        si.push_back(in_strides[i]);
+    }
+    if (total == 0) return AHIP_OK;
+    if (!out || !in) return ctx.fail(AHIP_ERR_ARG, "copy: null pointer");
+    for (size_t i = d.size(); i-- > 1;) {
+        // axis i-1 (outer) and i (inner) merge when outer stride == inner stride * inner extent on both sides
+        if (so[i - 1] == so[i] * d[i] && si[i - 1] == si[i] * d[i]) {
+            d[i - 1] *= d[i];
+            so[i - 1] = so[i];
+            si[i - 1] = si[i];
+            d.erase(d.begin() + i);
+            so.erase(so.begin() + i);
+            si.erase(si.begin() + i);
+        }
+    }
+    if (int rc = fits32(ctx, total, "copy")) return rc;
+    size_t max_in = 0, max_out = 0;
+    for (size_t i = 0; i < d.size(); i++) {
+        max_in += (size_t)(d[i] - 1) * (size_t)si[i];
+        max_out += (size_t)(d[i] - 1) * (size_t)so[i];
+    }
+    if (max_in >= ((size_t)1 << 31) || max_out >= ((size_t)1 << 31))
+        return ctx.fail(AHIP_ERR_UNSUPPORTED, "copy: an operand spans more than 2^31 elements");
+    if (d.empty()) {
+        d.push_back(1);
+        so.push_back(1);
+        si.push_back(1);
+    }
+    // 16-byte units when the innermost axis is contiguous on both sides and everything lines up.
+    int unit = elem_size;
+    if (elem_size == 4 && so.back() == 1 && si.back() == 1 && d.back() % 4 == 0 && aligned16(out) && aligned16(in)) {
+        bool ok = true;
+        for (size_t i = 0; i + 1 < d.size(); i++) ok = ok && so[i] % 4 == 0 && si[i] % 4 == 0;
+        if (ok) {
+            unit = 16;
+            d.back() /= 4;
+            for (size_t i = 0; i + 1 < d.size(); i++) {
+                so[i] /= 4;
+                si[i] /= 4;
+            }
+            total /= 4;
+        }
+    }
+    CopyGeom g;
+    g.rank = (int)d.size();
+    for (int i = 0; i < MAX_RANK; i++) {
+        g.dims[i] = make_fastdiv(1);
+        g.in_str[i] = g.out_str[i] = 0;
+    }
+    for (int i = 0; i < g.rank; i++) {  // innermost first
+        const size_t j = d.size() - 1 - (size_t)i;
+        g.dims[i] = make_fastdiv((uint32_t)d[j]);
+        g.in_str[i] = (uint32_t)si[j];
+        g.out_str[i] = (uint32_t)so[j];
+    }
+    switch (unit) {
+    case 1: launch_copy<uint8_t>(ctx.stream, out, in, g, (uint32_t)total); break;
+    case 4: launch_copy<uint32_t>(ctx.stream, out, in, g, (uint32_t)total); break;
+    case 8: launch_copy<uint64_t>(ctx.stream, out, in, g, (uint32_t)total); break;
+    default: launch_copy<uint4>(ctx.stream, out, in, g, (uint32_t)total); break;
+    }
+    return ctx.check(hipGetLastError(), "copy_strided launch");
+}
+
+int launch_transpose(DeviceCtx &ctx, void *out, const void *in, int elem_size, int rank, const int64_t *in_dims,
+                     const int64_t *perm) {
+    if (rank < 0 || rank > MAX_RANK) return ctx.fail(AHIP_ERR_ARG, "transpose: rank must be 0..8");
+    if (elem_size != 1 && elem_size != 4 && elem_size != 8) return ctx.fail(AHIP_ERR_ARG, "transpose: element size must be 1, 4 or 8");
+    bool seen[MAX_RANK] = {};
+    for (int i = 0; i < rank; i++) {
+        if (perm[i] < 0 || perm[i] >= rank || seen[perm[i]]) return ctx.fail(AHIP_ERR_ARG, "transpose: perm must name every axis once");
+        seen[perm[i]] = true;
+        if (in_dims[i] < 0) return ctx.fail(AHIP_ERR_ARG, "transpose: negative extent");
+    }
+    // Strides of the input, then the logical (output-ordered) view: out axis i reads input axis perm[i].
+    int64_t in_str[MAX_RANK], od[MAX_RANK], os[MAX_RANK], is[MAX_RANK];
+    int64_t acc = 1;
+    for (int i = rank - 1; i >= 0; i--) {
+        in_str[i] = acc;
+        acc *= in_dims[i];
+    }
+    const size_t total = (size_t)acc;
+    if (total == 0) return AHIP_OK;
+    if (!out || !in) return ctx.fail(AHIP_ERR_ARG, "transpose: null pointer");
+    acc = 1;
+    for (int i = rank - 1; i >= 0; i--) {
+        od[i] = in_dims[perm[i]];
+        is[i] = in_str[perm[i]];
+        os[i] = acc;
+        acc *= od[i];
+    }
+    // Collapse: drop size-1 axes and merge output-adjacent axes that are also adjacent in the input.
+    std::vector<int64_t> d, so, si;
+    for (int i = 0; i < rank; i++) {
+        if (od[i] == 1) continue;
+        d.push_back(od[i]);
+        so.push_back(os[i]);
+        si.push_back(is[i]);
+    }
+    for (size_t i = d.size(); i-- > 1;) {
+        if (si[i - 1] == si[i] * d[i]) {  // output strides are dense by construction
+            d[i - 1] *= d[i];
+            so[i - 1] = so[i];
+            si[i - 1] = si[i];
+            d.erase(d.begin() + i);
+            so.erase(so.begin() + i);
+            si.erase(si.begin() + i);
+        }
+    }
+    if (int rc = fits32(ctx, total, "transpose")) return rc;
+    // The innermost output axis is contiguous in the input too (or nothing is left to permute):
+    // rows of `d.back()` elements move whole -> strided copy, 16 bytes at a time when it lines up.
+    if (d.size() <= 1 || si.back() == 1) {
+        const int r = (int)d.size();
+        return launch_copy_strided(ctx, out, in, elem_size, r, d.data(), so.data(), si.data());
+    }
+    // Tiled path: C = the axis with input stride 1, R = the innermost output axis.
+    size_t c_axis = d.size();
+    for (size_t i = 0; i < d.size(); i++)
+        if (si[i] == 1) c_axis = i;
+    if (c_axis == d.size()) return ctx.fail(AHIP_ERR_ARG, "transpose: no contiguous input axis");  // cannot happen for a dense input
+    TransGeom g;
+    g.r_len = (uint32_t)d.back();
+    g.r_in_str = (uint32_t)si.back();
+    g.c_len = (uint32_t)d[c_axis];
+    g.c_out_str = (uint32_t)so[c_axis];
+    g.brank = 0;
+    size_t batches = 1;
+    for (int i = 0; i < MAX_RANK; i++) {
+        g.bdims[i] = make_fastdiv(1);
+        g.b_in_str[i] = g.b_out_str[i] = 0;
+    }
+    for (size_t i = d.size() - 1; i-- > 0;) {  // innermost of the rest first
+        if (i == c_axis) continue;
+        g.bdims[g.brank] = make_fastdiv((uint32_t)d[i]);
+        g.b_in_str[g.brank] = (uint32_t)si[i];
+        g.b_out_str[g.brank] = (uint32_t)so[i];
+        g.brank++;
+        batches *= (size_t)d[i];
+    }
+    const size_t gx = (g.c_len + TILE - 1) / TILE, gy = (g.r_len + TILE - 1) / TILE;
+    if (gy > 65535 || batches > 65535) {
+        // Grid limits: fall back to the one-element-per-thread copy (still correct, reads uncoalesced).
+        return launch_copy_strided(ctx, out, in, elem_size, (int)d.size(), d.data(), so.data(), si.data());
+    }
+    const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batches);
+    switch (elem_size) {
+    case 1:
+        hipLaunchKernelGGL((transpose_tiled<uint8_t>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint8_t *>(out),
+                           static_cast<const uint8_t *>(in), g);
+        break;
+    case 4:
+        hipLaunchKernelGGL((transpose_tiled<uint32_t>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint32_t *>(out),
+                           static_cast<const uint32_t *>(in), g);
+        break;
+    default:
+        hipLaunchKernelGGL((transpose_tiled<uint64_t>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint64_t *>(out),
+                           static_cast<const uint64_t *>(in), g);
+        break;
+    }
+    return ctx.check(hipGetLastError(), "transpose_tiled launch");
+}
+
+int launch_gather(DeviceCtx &ctx, void *out, const void *data, const void *indices, int index_size, int elem_size,
+                  size_t outer, size_t axis_len, size_t n_idx, size_t inner, int *bad_flag) {
+    if (elem_size != 1 && elem_size != 4 && elem_size != 8) return ctx.fail(AHIP_ERR_ARG, "gather: element size must be 1, 4 or 8");
+    if (index_size != 4 && index_size != 8) return ctx.fail(AHIP_ERR_ARG, "gather: indices must be i32 or i64");
+    const size_t total = outer * n_idx * inner;
+    if (total == 0) return AHIP_OK;
+    if (axis_len == 0) return ctx.fail(AHIP_ERR_SHAPE, "gather: the gathered axis is empty");
+    if (!out || !data || !indices || !bad_flag) return ctx.fail(AHIP_ERR_ARG, "gather: null pointer");
+    if (int rc = fits32(ctx, std::max(total, outer * axis_len * inner), "gather")) return rc;
+    const FastDiv in = make_fastdiv((uint32_t)inner), nd = make_fastdiv((uint32_t)n_idx);
+    const dim3 grid((unsigned)((total + BLOCK - 1) / BLOCK));
+#define GATHER(T, I)                                                                                                   \
+    hipLaunchKernelGGL((gather_rows<T, I>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<T *>(out),                  \
+                       static_cast<const T *>(data), static_cast<const I *>(indices), (uint32_t)axis_len,             \
+                       (uint32_t)n_idx, in, nd, (uint32_t)total, bad_flag)
+    if (index_size == 8) {
+        if (elem_size == 1) GATHER(uint8_t, long long);
+        else if (elem_size == 4) GATHER(uint32_t, long long);
+        else GATHER(uint64_t, long long);
+    } else {
+        if (elem_size == 1) GATHER(uint8_t, int);
+        else if (elem_size == 4) GATHER(uint32_t, int);
+        else GATHER(uint64_t, int);
+    }
+#undef GATHER
+    return ctx.check(hipGetLastError(), "gather launch");
+}
+
+int launch_where(DeviceCtx &ctx, void *out, const void *cond, const void *x, const void *y, int elem_size, int rank,
+                 const int64_t *dims, const int64_t *c_strides, const int64_t *x_strides, const int64_t *y_strides) {
+    if (rank < 0 || rank > MAX_RANK) return ctx.fail(AHIP_ERR_ARG, "where: rank must be 0..8");
+    if (elem_size != 1 && elem_size != 4 && elem_size != 8) return ctx.fail(AHIP_ERR_ARG, "where: element size must be 1, 4 or 8");
+    size_t total = 1;
+    for (int i = 0; i < rank; i++) {
+        if (dims[i] < 0) return ctx.fail(AHIP_ERR_ARG, "where: negative extent");
+        total *= (size_t)dims[i];
+    }
+    if (total == 0) return AHIP_OK;
+    if (!out || !cond || !x || !y) return ctx.fail(AHIP_ERR_ARG, "where: null pointer");
+    if (int rc = fits32(ctx, total, "where")) return rc;
+    WhereGeom g;
+    g.rank = rank;
+    for (int i = 0; i < MAX_RANK; i++) {
+        g.dims[i] = make_fastdiv(1);
+        g.c_str[i] = g.x_str[i] = g.y_str[i] = 0;
+    }
+    for (int i = 0; i < rank; i++) {
+        const int j = rank - 1 - i;
+        g.dims[i] = make_fastdiv((uint32_t)dims[j]);
+        g.c_str[i] = (uint32_t)c_strides[j];
+        g.x_str[i] = (uint32_t)x_strides[j];
+        g.y_str[i] = (uint32_t)y_strides[j];
+    }
+    const dim3 grid((unsigned)((total + BLOCK - 1) / BLOCK));
+    const uint8_t *c = static_cast<const uint8_t *>(cond);
+    switch (elem_size) {
+    case 1:
+        hipLaunchKernelGGL((where_strided<uint8_t>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint8_t *>(out), c,
+                           static_cast<const uint8_t *>(x), static_cast<const uint8_t *>(y), g, (uint32_t)total);
+        break;
+    case 4:
+        hipLaunchKernelGGL((where_strided<uint32_t>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint32_t *>(out), c,
+                           static_cast<const uint32_t *>(x), static_cast<const uint32_t *>(y), g, (uint32_t)total);
+        break;
+    default:
+        hipLaunchKernelGGL((where_strided<uint64_t>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint64_t *>(out), c,
+                           static_cast<const uint64_t *>(x), static_cast<const uint64_t *>(y), g, (uint32_t)total);
+        break;
+    }
+    return ctx.check(hipGetLastError(), "where launch");
+}
+
+int launch_greater(DeviceCtx &ctx, uint8_t *out, const float *a, const float *b, int rank, const int64_t *dims,
+                   const int64_t *a_strides, const int64_t *b_strides) {
+    if (rank < 0 || rank > MAX_RANK) return ctx.fail(AHIP_ERR_ARG, "greater: rank must be 0..8");
+    size_t total = 1;
+    for (int i = 0; i < rank; i++) {
+        if (dims[i] < 0) return ctx.fail(AHIP_ERR_ARG, "greater: negative extent");
+        total *= (size_t)dims[i];
+    }
+    if (total == 0) return AHIP_OK;
+    if (!out || !a || !b) return ctx.fail(AHIP_ERR_ARG, "greater: null pointer");
+    if (int rc = fits32(ctx, total, "greater")) return rc;
+    CmpGeom g;
+    g.rank = rank;
+    for (int i = 0; i < MAX_RANK; i++) {
+        g.dims[i] = make_fastdiv(1);
+        g.a_str[i] = g.b_str[i] = 0;
+    }
+    for (int i = 0; i < rank; i++) {
+        const int j = rank - 1 - i;
+        g.dims[i] = make_fastdiv((uint32_t)dims[j]);
+        g.a_str[i] = (uint32_t)a_strides[j];
+        g.b_str[i] = (uint32_t)b_strides[j];
+    }
+    hipLaunchKernelGGL(greater_strided, dim3((unsigned)((total + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, ctx.stream, out, a, b,
+                       g, (uint32_t)total);
+    return ctx.check(hipGetLastError(), "greater launch");
+}
+
+int launch_cast(DeviceCtx &ctx, void *out, const void *in, int from_type, int to_type, size_t n) {
+    if (n == 0) return AHIP_OK;
+    if (!out || !in) return ctx.fail(AHIP_ERR_ARG, "cast: null pointer");
+    const dim3 grid((unsigned)((n + BLOCK - 1) / BLOCK));
+    if (grid.x == 0 || (n + BLOCK - 1) / BLOCK > 0x7fffffffull) return ctx.fail(AHIP_ERR_UNSUPPORTED, "cast: too many elements");
+#define CAST(TO, FROM, B)                                                                                              \
+    hipLaunchKernelGGL((cast_flat<TO, FROM, B>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<TO *>(out),            \
+                       static_cast<const FROM *>(in), n)
+    const int F = AHIP_F32, I4 = AHIP_I32, I8 = AHIP_I64, BO = AHIP_BOOL;
+    if (from_type == to_type) {
+        const size_t bytes = n * (from_type == BO ? 1 : from_type == I8 ? 8 : 4);
+        return ctx.check(hipMemcpyAsync(out, in, bytes, hipMemcpyDeviceToDevice, ctx.stream), "hipMemcpyAsync(cast)");
+    }
+    if (from_type == F && to_type == I4) CAST(int32_t, float, false);
+    else if (from_type == F && to_type == I8) CAST(long long, float, false);
+    else if (from_type == F && to_type == BO) CAST(uint8_t, float, true);
+    else if (from_type == I4 && to_type == F) CAST(float, int32_t, false);
+    else if (from_type == I4 && to_type == I8) CAST(long long, int32_t, false);
+    else if (from_type == I4 && to_type == BO) CAST(uint8_t, int32_t, true);
+    else if (from_type == I8 && to_type == F) CAST(float, long long, false);
+    else if (from_type == I8 && to_type == I4) CAST(int32_t, long long, false);
+    else if (from_type == I8 && to_type == BO) CAST(uint8_t, long long, true);
+    else if (from_type == BO && to_type == F) CAST(float, uint8_t, false);
+    else if (from_type == BO && to_type == I4) CAST(int32_t, uint8_t, false);
+    else if (from_type == BO && to_type == I8) CAST(long long, uint8_t, false);
+    else return ctx.fail(AHIP_ERR_ARG, "cast: unknown element type");
+#undef CAST
+    return ctx.check(hipGetLastError(), "cast launch");
+}
+
+int launch_batchnorm(DeviceCtx &ctx, float *out, const float *x, const float *scale, const float *bias, const float *mean,
+                     const float *var, size_t n, size_t c, size_t hw, float eps) {
+    const size_t total = n * c * hw;
+    if (total == 0) return AHIP_OK;
+    if (!out || !x || !scale || !bias || !mean || !var) return ctx.fail(AHIP_ERR_ARG, "batchnorm: null pointer");
+    if (int rc = fits32(ctx, total, "batchnorm")) return rc;
+    const FastDiv fhw = make_fastdiv((uint32_t)hw), fc = make_fastdiv((uint32_t)c);
+    if (hw % 4 == 0 && aligned16(out) && aligned16(x)) {
+        hipLaunchKernelGGL((batchnorm_nchw<4>), dim3((unsigned)((total / 4 + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, ctx.stream,
+                           out, x, scale, bias, mean, var, fhw, fc, (uint32_t)total, eps);
+    } else {
+        hipLaunchKernelGGL((batchnorm_nchw<1>), dim3((unsigned)((total + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, ctx.stream, out,
+                           x, scale, bias, mean, var, fhw, fc, (uint32_t)total, eps);
+    }
+    return ctx.check(hipGetLastError(), "batchnorm launch");
+}
+
+}  // namespace altius

@@ -446,7 +446,8 @@ int reduce_impl(DeviceCtx &ctx, float *out, const float *in, size_t outer, size_
 
 int launch_reduce(DeviceCtx &ctx, int kind, float *out, const float *in, size_t outer, size_t red,
                   size_t inner) {
-    if (kind != AHIP_REDUCE_MEAN && kind != AHIP_REDUCE_MAX) return ctx.fail(AHIP_ERR_ARG, "reduce: unknown kind");
+    if (kind != AHIP_REDUCE_MEAN && kind != AHIP_REDUCE_MAX && kind != AHIP_REDUCE_SUM)
+        return ctx.fail(AHIP_ERR_ARG, "reduce: unknown kind");
     if (outer == 0 || inner == 0) return AHIP_OK;
     if (red == 0) return ctx.fail(AHIP_ERR_ARG, "reduce: empty reduced axis");
     if (!out || !in) return ctx.fail(AHIP_ERR_ARG, "reduce: null tensor pointer");
@@ -454,6 +455,7 @@ int launch_reduce(DeviceCtx &ctx, int kind, float *out, const float *in, size_t 
         const float r_axis_len = 1.0f / (float)red;
         return reduce_impl<SumOp, true>(ctx, out, in, outer, red, inner, r_axis_len);
     }
+    if (kind == AHIP_REDUCE_SUM) return reduce_impl<SumOp, false>(ctx, out, in, outer, red, inner, 1.0f);
     return reduce_impl<MaxOp, false>(ctx, out, in, outer, red, inner, 1.0f);
 }
 

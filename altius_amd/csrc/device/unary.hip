@@ -27,6 +27,19 @@ struct FHardSigmoid {
     __device__ __forceinline__ float operator()(float x) const { return hard_sigmoid_elem(x, alpha, beta); }
 };
 
+struct FLeakyRelu {
+    float alpha;
+    __device__ __forceinline__ float operator()(float x) const { return leaky_relu_elem(x, alpha); }
+};
+struct FClip {
+    float lo, hi;
+    __device__ __forceinline__ float operator()(float x) const { return clip_elem(x, lo, hi); }
+};
+// Exp and Round have no kernel in the reference interpreter (session.rs:219-224): correctly
+// rounded-to-1-ulp expf, and round-half-to-even as ONNX defines Round.
+struct FExp { __device__ __forceinline__ float operator()(float x) const { return expf(x); } };
+struct FRound { __device__ __forceinline__ float operator()(float x) const { return rintf(x); } };
+
 constexpr int BLOCK = 256;
 
 // One float4 per lane: on this part a streaming kernel is fastest with the
@@ -76,7 +89,7 @@ template <class F> void launch(hipStream_t s, float *out, const float *in, size_
 }  // namespace
 
 int launch_unary(DeviceCtx &ctx, int op, float *out, const float *in, size_t n, float alpha, float beta) {
-    if (op < AHIP_SQRT || op > AHIP_TANH) return ctx.fail(AHIP_ERR_ARG, "unary: unknown op");
+    if (op < AHIP_SQRT || op > AHIP_CLIP) return ctx.fail(AHIP_ERR_ARG, "unary: unknown op");
     if (n == 0) return AHIP_OK;
     if (!out || !in) return ctx.fail(AHIP_ERR_ARG, "unary: null tensor pointer");
     if (n > ((size_t)1 << 38)) return ctx.fail(AHIP_ERR_UNSUPPORTED, "unary: more than 2^38 elements");
@@ -89,6 +102,10 @@ int launch_unary(DeviceCtx &ctx, int op, float *out, const float *in, size_t n, 
     case AHIP_HARDSIGMOID: launch(ctx.stream, out, in, n, FHardSigmoid{alpha, beta}, nt); break;
     case AHIP_RELU: launch(ctx.stream, out, in, n, FRelu{}, nt); break;
     case AHIP_TANH: launch(ctx.stream, out, in, n, FTanh{}, nt); break;
+    case AHIP_LEAKYRELU: launch(ctx.stream, out, in, n, FLeakyRelu{alpha}, nt); break;
+    case AHIP_EXP: launch(ctx.stream, out, in, n, FExp{}, nt); break;
+    case AHIP_ROUND: launch(ctx.stream, out, in, n, FRound{}, nt); break;
+    case AHIP_CLIP: launch(ctx.stream, out, in, n, FClip{alpha, beta}, nt); break;
     }
     return ctx.check(hipGetLastError(), "unary launch");
 }

@@ -12,8 +12,10 @@ from . import _lib
 from ._lib import check, i64_array
 
 ADD, SUB, MUL, DIV, POW = 0, 1, 2, 3, 4
-SQRT, ERF, GELU, SIGMOID, HARDSIGMOID, RELU, TANH = 0, 1, 2, 3, 4, 5, 6
-REDUCE_MEAN, REDUCE_MAX = 0, 1
+SQRT, ERF, GELU, SIGMOID, HARDSIGMOID, RELU, TANH, LEAKYRELU, EXP, ROUND, CLIP = range(11)
+REDUCE_MEAN, REDUCE_MAX, REDUCE_SUM = 0, 1, 2
+BOOL, F32, I32, I64 = 0, 1, 2, 3
+_ELEM_OF = {np.dtype(np.bool_): BOOL, np.dtype(np.float32): F32, np.dtype(np.int32): I32, np.dtype(np.int64): I64}
 
 
 def broadcast_shape(a_dims, b_dims):
@@ -235,3 +237,112 @@ class Context:
         finally:
             self.free(dx)
             self.free(do)
+
+
+    # --- data movement: numpy in, numpy out -------------------------------------------------------
+    def _upload_any(self, a):
+        a = np.asarray(a, order="C")
+        if a.dtype not in _ELEM_OF:
+            raise TypeError(f"unsupported dtype {a.dtype}")
+        return a, self.upload(a)
+
+    def copy_strided(self, x, dims, out_strides, in_strides, out_shape, in_offset=0, out_offset=0, out_init=None):
+        """One ahip_copy_strided over a fresh (or given) output array; offsets are in elements."""
+        x, dx = self._upload_any(x)
+        out = np.zeros(out_shape, x.dtype) if out_init is None else np.asarray(out_init, dtype=x.dtype, order="C")
+        do = self.upload(out) if out.size else self.alloc(4)
+        try:
+            isz = x.dtype.itemsize
+            check(self.L.ahip_copy_strided(self.handle, do.ptr + out_offset * isz, dx.ptr + in_offset * isz, isz, len(dims),
+                                           i64_array(dims), i64_array(out_strides), i64_array(in_strides)), self.handle)
+            return self.download(do, out.shape, x.dtype)
+        finally:
+            self.free(dx)
+            self.free(do)
+
+    def transpose(self, x, perm):
+        x, dx = self._upload_any(x)
+        shape = [x.shape[p] for p in perm]
+        do = self.alloc(max(x.nbytes, 4))
+        try:
+            check(self.L.ahip_transpose(self.handle, do.ptr, dx.ptr, x.dtype.itemsize, x.ndim, i64_array(x.shape),
+                                        i64_array(perm)), self.handle)
+            return self.download(do, shape, x.dtype)
+        finally:
+            self.free(dx)
+            self.free(do)
+
+    def gather(self, data, indices, axis=0):
+        data, dd = self._upload_any(data)
+        idx = np.asarray(indices, order="C")
+        if idx.dtype not in (np.int32, np.int64):
+            idx = idx.astype(np.int64)
+        di = self.upload(idx)
+        ax = axis + data.ndim if axis < 0 else axis
+        shape = data.shape[:ax] + idx.shape + data.shape[ax + 1:]
+        outer = int(np.prod(data.shape[:ax], dtype=np.int64))
+        inner = int(np.prod(data.shape[ax + 1:], dtype=np.int64))
+        do = self.alloc(max(int(np.prod(shape, dtype=np.int64)) * data.dtype.itemsize, 4))
+        try:
+            check(self.L.ahip_gather(self.handle, do.ptr, dd.ptr, di.ptr, idx.dtype.itemsize, data.dtype.itemsize, outer,
+                                     data.shape[ax], idx.size, inner), self.handle)
+            return self.download(do, shape, data.dtype)      # download synchronises: a bad index raises here
+        finally:
+            for b in (dd, di, do):
+                self.free(b)
+
+    def where(self, cond, x, y):
+        cond = np.asarray(cond, dtype=np.bool_, order="C")
+        x, dx = self._upload_any(x)
+        y = np.asarray(y, dtype=x.dtype, order="C")
+        dc, dy = self.upload(cond), self.upload(y)
+        dims = list(np.broadcast_shapes(cond.shape, x.shape, y.shape))
+        st = [strides_for_broadcasting(a.shape, dims) for a in (cond, x, y)]
+        n = int(np.prod(dims, dtype=np.int64))
+        do = self.alloc(max(n * x.dtype.itemsize, 4))
+        try:
+            check(self.L.ahip_where(self.handle, do.ptr, dc.ptr, dx.ptr, dy.ptr, x.dtype.itemsize, len(dims), i64_array(dims),
+                                    i64_array(st[0]), i64_array(st[1]), i64_array(st[2])), self.handle)
+            return self.download(do, dims, x.dtype)
+        finally:
+            for b in (dc, dx, dy, do):
+                self.free(b)
+
+    def greater(self, a, b):
+        a = np.asarray(a, dtype=np.float32, order="C")
+        b = np.asarray(b, dtype=np.float32, order="C")
+        dims = list(np.broadcast_shapes(a.shape, b.shape))
+        da, db = self.upload(a), self.upload(b)
+        n = int(np.prod(dims, dtype=np.int64))
+        do = self.alloc(max(n, 4))
+        try:
+            check(self.L.ahip_greater(self.handle, do.ptr, da.ptr, db.ptr, len(dims), i64_array(dims),
+                                      i64_array(strides_for_broadcasting(a.shape, dims)),
+                                      i64_array(strides_for_broadcasting(b.shape, dims))), self.handle)
+            return self.download(do, dims, np.bool_)
+        finally:
+            for x in (da, db, do):
+                self.free(x)
+
+    def cast(self, x, to_dtype):
+        x, dx = self._upload_any(x)
+        to_dtype = np.dtype(to_dtype)
+        do = self.alloc(max(x.size * to_dtype.itemsize, 4))
+        try:
+            check(self.L.ahip_cast(self.handle, do.ptr, dx.ptr, _ELEM_OF[x.dtype], _ELEM_OF[to_dtype], x.size), self.handle)
+            return self.download(do, x.shape, to_dtype)
+        finally:
+            self.free(dx)
+            self.free(do)
+
+    def batchnorm(self, x, scale, bias, mean, var, eps=1e-5):
+        arrs = [np.asarray(a, dtype=np.float32, order="C") for a in (x, scale, bias, mean, var)]
+        n, c, h, w = arrs[0].shape
+        bufs = [self.upload(a) for a in arrs]
+        do = self.alloc(max(arrs[0].nbytes, 4))
+        try:
+            check(self.L.ahip_batchnorm(self.handle, do.ptr, *[b.ptr for b in bufs], n, c, h * w, eps), self.handle)
+            return self.download(do, arrs[0].shape)
+        finally:
+            for b in bufs + [do]:
+                self.free(b)

@@ -137,10 +137,15 @@ enum ahip_unary_op {
     AHIP_SIGMOID = 3,     /* compute_sigmoid, session.rs:905-922 + fast_math.rs:189-279 */
     AHIP_HARDSIGMOID = 4, /* compute_hard_sigmoid, session.rs:805-812 (alpha, beta) */
     AHIP_RELU = 5,        /* compute_relu, session.rs:796-803 */
-    AHIP_TANH = 6         /* compute_tanh, session.rs:840-903, 933-938 (rational tanh) */
+    AHIP_TANH = 6,        /* compute_tanh, session.rs:840-903, 933-938 (rational tanh) */
+    AHIP_LEAKYRELU = 7,   /* compute_leaky_relu, session.rs:814-821 (alpha) */
+    AHIP_EXP = 8,         /* no reference kernel (session.rs:224): expf */
+    AHIP_ROUND = 9,       /* no reference kernel (session.rs:219-223): round half to even (ONNX Round) */
+    AHIP_CLIP = 10        /* no reference kernel (session.rs:201): clamp to [alpha, beta] (ONNX Clip) */
 };
 
-/* Flat element-wise op over n elements.  alpha/beta are read by HardSigmoid only. */
+/* Flat element-wise op over n elements.  alpha/beta are read by HardSigmoid (alpha, beta),
+ * LeakyRelu (alpha) and Clip (alpha = min, beta = max). */
 int ahip_unary(ahip_ctx *ctx, int op, float *out, const float *in, size_t n, float alpha,
                float beta);
 
@@ -153,7 +158,11 @@ int ahip_softmax_lastaxis(ahip_ctx *ctx, float *out, const float *in, size_t row
 int ahip_layernorm_lastaxis(ahip_ctx *ctx, float *out, const float *in, const float *gamma,
                             const float *beta, size_t rows, size_t len, float eps);
 
-enum ahip_reduce_kind { AHIP_REDUCE_MEAN = 0, AHIP_REDUCE_MAX = 1 };
+enum ahip_reduce_kind {
+    AHIP_REDUCE_MEAN = 0, /* sum * (1 / len) */
+    AHIP_REDUCE_MAX = 1,
+    AHIP_REDUCE_SUM = 2   /* plain sum: GlobalAveragePool divides it by H*W afterwards (session.rs:265-297) */
+};
 
 /* compute_reduce_mean / compute_reduce_max (session.rs:1292-1340), generalised
  * to any contiguous run of reduced axes: the input is viewed as
@@ -163,6 +172,38 @@ enum ahip_reduce_kind { AHIP_REDUCE_MEAN = 0, AHIP_REDUCE_MAX = 1 };
  * panics on NaN). */
 int ahip_reduce(ahip_ctx *ctx, int kind, float *out, const float *in, size_t outer, size_t reduce,
                 size_t inner);
+
+/* Data movement.  Element sizes are in bytes (1 = Bool, 4 = F32 / I32, 8 = I64); strides in
+ * elements.  All of these move each byte once and accept any rank up to 8.
+ *
+ * ahip_copy_strided: element idx of the index space dims[rank] is read at sum(idx*in_strides)
+ * and written at sum(idx*out_strides).  With a dense output it is Slice (offset base pointer,
+ * strides scaled by the steps), Expand and Tile (stride 0) or a Transpose; with a dense input
+ * and a windowed output it is one operand of Concat; Split is the reverse
+ * (compute_concat / compute_split / compute_slice, session.rs:1134-1177, 1488-1558).
+ * ahip_transpose: compute_transpose (session.rs:1179-1278); perm as in Op::Transpose.
+ * ahip_gather: out[o, j, :] = data[o, indices[j], :] for outer x n_indices rows of `inner`
+ * elements (compute_gather, session.rs:1560-1598, any index count); indices are i32 or i64
+ * (index_size 4 or 8), negative ones count from the end.  An index out of range reads row 0
+ * and makes the next ahip_sync on this context fail with AHIP_ERR_ARG.
+ * ahip_where: out = cond ? x : y with broadcast strides (compute_where, session.rs:940-988).
+ * ahip_greater: out (bool) = a > b (compute_greater, session.rs:541-562; any broadcast).
+ * ahip_cast: Rust `as` between Bool / F32 / I32 / I64 (compute_cast, session.rs:1350-1378).
+ * ahip_batchnorm: ((x - mean[c]) / sqrt(var[c] + eps)) * scale[c] + bias[c] on [n, c, hw]
+ * (compute_batch_normalization, session.rs:1380-1431). */
+int ahip_copy_strided(ahip_ctx *ctx, void *out, const void *in, int elem_size, int rank, const int64_t *dims,
+                      const int64_t *out_strides, const int64_t *in_strides);
+int ahip_transpose(ahip_ctx *ctx, void *out, const void *in, int elem_size, int rank, const int64_t *in_dims,
+                   const int64_t *perm);
+int ahip_gather(ahip_ctx *ctx, void *out, const void *data, const void *indices, int index_size, int elem_size,
+                size_t outer, size_t axis_len, size_t n_indices, size_t inner);
+int ahip_where(ahip_ctx *ctx, void *out, const void *cond, const void *x, const void *y, int elem_size, int rank,
+               const int64_t *dims, const int64_t *cond_strides, const int64_t *x_strides, const int64_t *y_strides);
+int ahip_greater(ahip_ctx *ctx, void *out, const float *a, const float *b, int rank, const int64_t *dims,
+                 const int64_t *a_strides, const int64_t *b_strides);
+int ahip_cast(ahip_ctx *ctx, void *out, const void *in, int from_elem_type, int to_elem_type, size_t n);
+int ahip_batchnorm(ahip_ctx *ctx, float *out, const float *x, const float *scale, const float *bias, const float *mean,
+                   const float *var, size_t n, size_t c, size_t hw, float epsilon);
 
 /* ------------------------------------------------------------------------
  * Graph IR: the same Model / Graph / Node / Value / Op structure as

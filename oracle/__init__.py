@@ -197,3 +197,143 @@ def fast_sum(x):
 def fast_sum_squares(x):
     x = _f32(x)
     return np.float32(lib().orc_fast_sum_squares(_fptr(x), ctypes.c_size_t(x.size)))
+
+
+# ---- data movement and the remaining element-wise kernels ---------------------------------------
+
+_TYPE_OF = {np.dtype(np.bool_): 0, np.dtype(np.float32): 1, np.dtype(np.int32): 2, np.dtype(np.int64): 3}
+_NP_OF = {0: np.bool_, 1: np.float32, 2: np.int32, 3: np.int64}
+
+
+def _c(a):
+    return np.asarray(a, order="C")
+
+
+def _vp(a):
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+def _note(info, noref):
+    if info is not None:
+        info["no_reference_kernel"] = bool(noref.value)
+
+
+def transpose(x, perm):
+    x = _c(x)
+    out = np.empty([x.shape[p] for p in perm], dtype=x.dtype)
+    d, r = _dims(x.shape)
+    pm, _ = _dims(perm)
+    rc = lib().orc_transpose(_vp(x), _vp(out), x.dtype.itemsize, r, d, pm)
+    if rc != OK:
+        raise OracleError(rc, "transpose")
+    return out
+
+
+def gather(data, indices, axis=0, strict=False, info=None):
+    data = _c(data)
+    idx = np.asarray(indices, dtype=np.int64, order="C")
+    ax = axis + data.ndim if axis < 0 else axis
+    out = np.empty(data.shape[:ax] + idx.shape + data.shape[ax + 1:], dtype=data.dtype)
+    d, r = _dims(data.shape)
+    i_d, i_r = _dims(idx.shape)
+    noref = ctypes.c_int(0)
+    rc = lib().orc_gather(_vp(data), data.dtype.itemsize, r, d, axis, idx.ctypes.data_as(ctypes.POINTER(ctypes.c_int64)),
+                          i_r, i_d, _vp(out), int(bool(strict)), ctypes.byref(noref))
+    _note(info, noref)
+    if rc != OK:
+        raise OracleError(rc, "gather")
+    return out
+
+
+def split(x, parts, axis, strict=False, info=None):
+    x = _c(x)
+    ax = axis + x.ndim if axis < 0 else axis
+    outs = []
+    for p in parts:
+        shape = list(x.shape)
+        shape[ax] = int(p)
+        outs.append(np.empty(shape, dtype=x.dtype))
+    ptrs = (ctypes.c_void_p * len(outs))(*[o.ctypes.data for o in outs])
+    d, r = _dims(x.shape)
+    ps, n = _dims(parts)
+    noref = ctypes.c_int(0)
+    rc = lib().orc_split(_vp(x), x.dtype.itemsize, r, d, axis, n, ps, ptrs, int(bool(strict)), ctypes.byref(noref))
+    _note(info, noref)
+    if rc != OK:
+        raise OracleError(rc, "split")
+    return outs
+
+
+def where(cond, x, y, strict=False, info=None):
+    cond = np.asarray(cond, dtype=np.bool_, order="C")
+    x, y = _f32(x), _f32(y)
+    out = np.empty(np.broadcast_shapes(cond.shape, x.shape, y.shape), dtype=np.float32)
+    cd, cr = _dims(cond.shape)
+    xd, xr = _dims(x.shape)
+    yd, yr = _dims(y.shape)
+    noref = ctypes.c_int(0)
+    rc = lib().orc_where(cond.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)), cr, cd, _fptr(x), xr, xd, _fptr(y), yr, yd,
+                         _fptr(out), int(bool(strict)), ctypes.byref(noref))
+    _note(info, noref)
+    if rc != OK:
+        raise OracleError(rc, "where")
+    return out
+
+
+def greater(a, b, strict=False, info=None):
+    a, b = _f32(a), _f32(b)
+    out = np.empty(np.broadcast_shapes(a.shape, b.shape), dtype=np.bool_)
+    ad, ar = _dims(a.shape)
+    bd, br = _dims(b.shape)
+    noref = ctypes.c_int(0)
+    rc = lib().orc_greater(_fptr(a), ar, ad, _fptr(b), br, bd, out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)),
+                           int(bool(strict)), ctypes.byref(noref))
+    _note(info, noref)
+    if rc != OK:
+        raise OracleError(rc, "greater")
+    return out
+
+
+def cast(x, to_dtype, strict=False, info=None):
+    x = _c(x)
+    to_dtype = np.dtype(to_dtype)
+    out = np.empty(x.shape, dtype=to_dtype)
+    noref = ctypes.c_int(0)
+    rc = lib().orc_cast(_vp(x), _TYPE_OF[x.dtype], _vp(out), _TYPE_OF[to_dtype], ctypes.c_size_t(x.size), int(bool(strict)),
+                        ctypes.byref(noref))
+    _note(info, noref)
+    if rc != OK:
+        raise OracleError(rc, "cast")
+    return out
+
+
+def batchnorm(x, scale, bias, mean, var, eps=1e-5):
+    x, scale, bias, mean, var = (_f32(v) for v in (x, scale, bias, mean, var))
+    n, c, h, w = x.shape
+    out = np.empty_like(x)
+    sz = ctypes.c_size_t
+    rc = lib().orc_batchnorm(_fptr(x), _fptr(scale), _fptr(bias), _fptr(mean), _fptr(var), _fptr(out), sz(n), sz(c), sz(h),
+                             sz(w), ctypes.c_float(eps))
+    if rc != OK:
+        raise OracleError(rc, "batchnorm")
+    return out
+
+
+def global_average_pool(x):
+    x = _f32(x)
+    n, c, h, w = x.shape
+    out = np.empty((n, c, 1, 1), dtype=np.float32)
+    sz = ctypes.c_size_t
+    rc = lib().orc_global_average_pool(_fptr(x), _fptr(out), sz(n), sz(c), sz(h), sz(w))
+    if rc != OK:
+        raise OracleError(rc, "global_average_pool")
+    return out
+
+
+def leaky_relu(x, alpha=0.01):
+    x = _f32(x)
+    out = np.empty_like(x)
+    rc = lib().orc_leaky_relu(_fptr(x), _fptr(out), ctypes.c_size_t(x.size), ctypes.c_float(alpha))
+    if rc != OK:
+        raise OracleError(rc, "leaky_relu")
+    return out

@@ -7,6 +7,7 @@
 
 #include "oracle.h"
 
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <condition_variable>
@@ -809,6 +810,262 @@ int orc_reduce(int kind, const float *in, int rank, const int64_t *dims, int n_a
         return ORC_OK;
     }
     return ORC_ERR_ARG;
+}
+
+// ---- data movement (session.rs:940-988, 1134-1278, 1350-1431, 1488-1598) ----------------------
+
+static size_t total_of(int rank, const int64_t *dims) {
+    size_t n = 1;
+    for (int i = 0; i < rank; i++) n *= (size_t)dims[i];
+    return n;
+}
+
+// compute_transpose: blocks = the run of trailing axes with perm[i] == i; every other axis is
+// walked by an odometer whose digit i advances the source by the input stride of perm[i].
+int orc_transpose(const void *in, void *out, int elem_size, int rank, const int64_t *in_dims, const int64_t *perm) {
+    if (rank < 0 || rank > 16 || elem_size <= 0) return ORC_ERR_ARG;
+    std::vector<int64_t> in_str((size_t)rank), out_dims((size_t)rank), new_str((size_t)rank);
+    int64_t acc = 1;
+    for (int i = rank - 1; i >= 0; i--) {
+        in_str[(size_t)i] = acc;
+        acc *= in_dims[i];
+    }
+    for (int i = 0; i < rank; i++) {
+        if (perm[i] < 0 || perm[i] >= rank) return ORC_ERR_ARG;
+        out_dims[(size_t)i] = in_dims[perm[i]];
+        new_str[(size_t)i] = in_str[(size_t)perm[i]];
+    }
+    size_t num_blocks = 1, block = 1;
+    int reduced = 0;
+    bool suffix = true;
+    for (int i = rank - 1; i >= 0; i--) {
+        const int axis = (int)perm[i];
+        if (suffix && axis == i) {
+            block *= (size_t)in_dims[axis];
+        } else {
+            suffix = false;
+            num_blocks *= (size_t)in_dims[axis];
+            reduced++;
+        }
+    }
+    if (num_blocks * block == 0) return ORC_OK;
+    const char *src = static_cast<const char *>(in);
+    char *dst = static_cast<char *>(out);
+    std::vector<size_t> index((size_t)reduced, 0);
+    size_t src_idx = 0;
+    for (size_t b = 0; b < num_blocks; b++) {
+        std::memcpy(dst + b * block * (size_t)elem_size, src + src_idx * (size_t)elem_size, block * (size_t)elem_size);
+        // next_index (session.rs:1188-1216)
+        for (int pos = reduced - 1; pos >= 0; pos--) {
+            src_idx += (size_t)new_str[(size_t)pos];
+            index[(size_t)pos]++;
+            if (index[(size_t)pos] < (size_t)out_dims[(size_t)pos]) break;
+            src_idx -= (size_t)new_str[(size_t)pos] * index[(size_t)pos];
+            index[(size_t)pos] = 0;
+        }
+    }
+    return ORC_OK;
+}
+
+int orc_gather(const void *data, int elem_size, int rank, const int64_t *dims, int axis, const int64_t *indices,
+               int idx_rank, const int64_t *idx_dims, void *out, int strict, int *no_reference_kernel) {
+    if (axis < 0) axis += rank;
+    if (axis < 0 || axis >= rank) return ORC_ERR_ARG;
+    const bool scalar = orc_is_scalar(idx_rank, idx_dims) != 0;
+    bool leading_ones = true;
+    for (int i = 0; i < axis; i++) leading_ones = leading_ones && dims[i] == 1;
+    const bool ref = (scalar && leading_ones) || (!scalar && idx_rank == 2 && idx_dims[0] == 1 && axis == 0 && rank == 2);
+    if (no_reference_kernel) *no_reference_kernel = ref ? 0 : 1;
+    if (!ref && strict) return ORC_ERR_UNSUPPORTED;
+    size_t outer = 1, inner = 1;
+    for (int i = 0; i < axis; i++) outer *= (size_t)dims[i];
+    for (int i = axis + 1; i < rank; i++) inner *= (size_t)dims[i];
+    const size_t axis_len = (size_t)dims[axis], n_idx = total_of(idx_rank, idx_dims);
+    const char *src = static_cast<const char *>(data);
+    char *dst = static_cast<char *>(out);
+    const size_t row = inner * (size_t)elem_size;
+    for (size_t o = 0; o < outer; o++)
+        for (size_t j = 0; j < n_idx; j++) {
+            int64_t k = indices[j];
+            if (k < 0) k += (int64_t)axis_len;
+            if (k < 0 || k >= (int64_t)axis_len) return ORC_ERR_ARG;
+            std::memcpy(dst + (o * n_idx + j) * row, src + (o * axis_len + (size_t)k) * row, row);
+        }
+    return ORC_OK;
+}
+
+int orc_split(const void *in, int elem_size, int rank, const int64_t *dims, int axis, int n_parts,
+              const int64_t *parts, void *const *outs, int strict, int *no_reference_kernel) {
+    if (axis < 0) axis += rank;
+    if (axis < 0 || axis >= rank) return ORC_ERR_ARG;
+    const bool ref = axis == rank - 1;  // assert_eq!(axis, inputs[0].dims().len() - 1)
+    if (no_reference_kernel) *no_reference_kernel = ref ? 0 : 1;
+    if (!ref && strict) return ORC_ERR_UNSUPPORTED;
+    size_t outer = 1, inner = 1;
+    for (int i = 0; i < axis; i++) outer *= (size_t)dims[i];
+    for (int i = axis + 1; i < rank; i++) inner *= (size_t)dims[i];
+    const size_t axis_len = (size_t)dims[axis];
+    const char *src = static_cast<const char *>(in);
+    // session.rs:1500-1511: walk the rows of the split axis, dealing each part to its output.
+    std::vector<size_t> offset((size_t)n_parts, 0);
+    for (size_t o = 0; o < outer; o++) {
+        size_t s = 0;
+        for (int p = 0; p < n_parts; p++) {
+            const size_t bytes = (size_t)parts[p] * inner * (size_t)elem_size;
+            std::memcpy(static_cast<char *>(outs[p]) + offset[(size_t)p], src + (o * axis_len + s) * inner * (size_t)elem_size, bytes);
+            offset[(size_t)p] += bytes;
+            s += (size_t)parts[p];
+        }
+        if (s != axis_len) return ORC_ERR_ARG;
+    }
+    return ORC_OK;
+}
+
+int orc_where(const uint8_t *cond, int c_rank, const int64_t *c_dims, const float *x, int x_rank, const int64_t *x_dims,
+              const float *y, int y_rank, const int64_t *y_dims, float *out, int strict, int *no_reference_kernel) {
+    const bool same_cy = c_rank == y_rank && std::equal(c_dims, c_dims + c_rank, y_dims);
+    const bool p1 = same_cy && orc_is_scalar(x_rank, x_dims);
+    const bool p2 = orc_is_scalar(y_rank, y_dims) && x_rank == 4 && c_rank == 4 && c_dims[0] == 1 && c_dims[1] == 1;
+    if (no_reference_kernel) *no_reference_kernel = (p1 || p2) ? 0 : 1;
+    if (p1) {  // session.rs:947-956
+        const size_t n = total_of(c_rank, c_dims);
+        for (size_t i = 0; i < n; i++) out[i] = cond[i] ? x[0] : y[i];
+        return ORC_OK;
+    }
+    if (p2 && c_dims[2] == x_dims[2] && c_dims[3] == x_dims[3]) {  // session.rs:958-987
+        const size_t plane = (size_t)(x_dims[2] * x_dims[3]), planes = (size_t)(x_dims[0] * x_dims[1]);
+        for (size_t p = 0; p < planes; p++)
+            for (size_t i = 0; i < plane; i++) out[p * plane + i] = cond[i] ? x[p * plane + i] : y[0];
+        return ORC_OK;
+    }
+    if (no_reference_kernel) *no_reference_kernel = 1;
+    if (strict) return ORC_ERR_UNSUPPORTED;
+    const int ranks[3] = {c_rank, x_rank, y_rank};
+    const int64_t *shapes[3] = {c_dims, x_dims, y_dims};
+    int out_rank = 0;
+    int64_t out_dims[16], cs[16], xs[16], ys[16];
+    if (orc_broadcast(3, ranks, shapes, &out_rank, out_dims)) return ORC_ERR_BROADCAST;
+    if (orc_strides_for_broadcasting(c_rank, c_dims, out_rank, out_dims, cs) ||
+        orc_strides_for_broadcasting(x_rank, x_dims, out_rank, out_dims, xs) ||
+        orc_strides_for_broadcasting(y_rank, y_dims, out_rank, out_dims, ys))
+        return ORC_ERR_BROADCAST;
+    const size_t n = total_of(out_rank, out_dims);
+    std::vector<int64_t> idx((size_t)out_rank, 0);
+    for (size_t i = 0; i < n; i++) {
+        int64_t ci = 0, xi = 0, yi = 0;
+        for (int d = 0; d < out_rank; d++) {
+            ci += idx[(size_t)d] * cs[d];
+            xi += idx[(size_t)d] * xs[d];
+            yi += idx[(size_t)d] * ys[d];
+        }
+        out[i] = cond[ci] ? x[xi] : y[yi];
+        for (int d = out_rank - 1; d >= 0; d--) {
+            if (++idx[(size_t)d] < out_dims[d]) break;
+            idx[(size_t)d] = 0;
+        }
+    }
+    return ORC_OK;
+}
+
+int orc_greater(const float *a, int a_rank, const int64_t *a_dims, const float *b, int b_rank, const int64_t *b_dims,
+                uint8_t *out, int strict, int *no_reference_kernel) {
+    const bool ref = orc_is_scalar(b_rank, b_dims) != 0;
+    if (no_reference_kernel) *no_reference_kernel = ref ? 0 : 1;
+    if (ref) {
+        const size_t n = total_of(a_rank, a_dims);
+        for (size_t i = 0; i < n; i++) out[i] = a[i] > b[0] ? 1 : 0;
+        return ORC_OK;
+    }
+    if (strict) return ORC_ERR_UNSUPPORTED;
+    const int ranks[2] = {a_rank, b_rank};
+    const int64_t *shapes[2] = {a_dims, b_dims};
+    int out_rank = 0;
+    int64_t out_dims[16], as[16], bs[16];
+    if (orc_broadcast(2, ranks, shapes, &out_rank, out_dims)) return ORC_ERR_BROADCAST;
+    if (orc_strides_for_broadcasting(a_rank, a_dims, out_rank, out_dims, as) ||
+        orc_strides_for_broadcasting(b_rank, b_dims, out_rank, out_dims, bs))
+        return ORC_ERR_BROADCAST;
+    const size_t n = total_of(out_rank, out_dims);
+    std::vector<int64_t> idx((size_t)out_rank, 0);
+    for (size_t i = 0; i < n; i++) {
+        int64_t ai = 0, bi = 0;
+        for (int d = 0; d < out_rank; d++) {
+            ai += idx[(size_t)d] * as[d];
+            bi += idx[(size_t)d] * bs[d];
+        }
+        out[i] = a[ai] > b[bi] ? 1 : 0;
+        for (int d = out_rank - 1; d >= 0; d--) {
+            if (++idx[(size_t)d] < out_dims[d]) break;
+            idx[(size_t)d] = 0;
+        }
+    }
+    return ORC_OK;
+}
+
+// Rust `as`: float -> int truncates toward zero, saturates, NaN -> 0; int -> narrower int wraps.
+static int32_t f32_as_i32(float v) {
+    if (v != v) return 0;
+    if (v >= 2147483648.0f) return INT32_MAX;
+    if (v <= -2147483648.0f) return INT32_MIN;
+    return (int32_t)v;
+}
+static int64_t f32_as_i64(float v) {
+    if (v != v) return 0;
+    if (v >= 9223372036854775808.0f) return INT64_MAX;
+    if (v <= -9223372036854775808.0f) return INT64_MIN;
+    return (int64_t)v;
+}
+
+int orc_cast(const void *in, int from, void *out, int to, size_t n, int strict, int *no_reference_kernel) {
+    enum { B = 0, F = 1, I4 = 2, I8 = 3 };
+    const bool ref = (from == I4 && to == F) || (from == I8 && to == I4) || (from == I8 && to == F) || (from == F && to == B);
+    if (no_reference_kernel) *no_reference_kernel = ref ? 0 : 1;
+    if (!ref && strict) return ORC_ERR_UNSUPPORTED;
+    for (size_t i = 0; i < n; i++) {
+        int64_t iv = 0;
+        float fv = 0;
+        switch (from) {
+        case B: iv = static_cast<const uint8_t *>(in)[i] ? 1 : 0; fv = (float)iv; break;
+        case F: fv = static_cast<const float *>(in)[i]; break;
+        case I4: iv = static_cast<const int32_t *>(in)[i]; fv = (float)iv; break;
+        case I8: iv = static_cast<const int64_t *>(in)[i]; fv = (float)iv; break;
+        default: return ORC_ERR_ARG;
+        }
+        switch (to) {
+        case B: static_cast<uint8_t *>(out)[i] = from == F ? (fv != 0.0f) : (iv != 0); break;
+        case F: static_cast<float *>(out)[i] = fv; break;
+        case I4: static_cast<int32_t *>(out)[i] = from == F ? f32_as_i32(fv) : (int32_t)(uint32_t)(uint64_t)iv; break;
+        case I8: static_cast<int64_t *>(out)[i] = from == F ? f32_as_i64(fv) : iv; break;
+        default: return ORC_ERR_ARG;
+        }
+    }
+    return ORC_OK;
+}
+
+int orc_batchnorm(const float *x, const float *scale, const float *bias, const float *mean, const float *var, float *out,
+                  size_t n, size_t c, size_t h, size_t w, float eps) {
+    for (size_t in_ = 0; in_ < n; in_++)
+        for (size_t ch = 0; ch < c; ch++)
+            for (size_t i = 0; i < h * w; i++) {
+                const size_t off = (in_ * c + ch) * h * w + i;
+                out[off] = ((x[off] - mean[ch]) / std::sqrt(var[ch] + eps)) * scale[ch] + bias[ch];
+            }
+    return ORC_OK;
+}
+
+int orc_global_average_pool(const float *x, float *out, size_t n, size_t c, size_t h, size_t w) {
+    const size_t area = h * w;
+    for (size_t p = 0; p < n * c; p++) {
+        float sum = 0.0f;  // Iterator::sum::<f32>() folds from 0.0 in order
+        for (size_t i = 0; i < area; i++) sum += x[p * area + i];
+        out[p] = sum / (float)area;
+    }
+    return ORC_OK;
+}
+
+int orc_leaky_relu(const float *x, float *out, size_t n, float alpha) {
+    for (size_t i = 0; i < n; i++) out[i] = x[i] < 0.0f ? alpha * x[i] : x[i];
+    return ORC_OK;
 }
 
 float orc_fast_sum(const float *x, size_t n) { return fast_sum(x, n); }

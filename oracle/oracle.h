@@ -123,6 +123,49 @@ int orc_reduce(int kind, const float *in, int rank, const int64_t *dims, int n_a
 
 /* The accumulation primitives on their own, for known-answer tests.
  * session.rs:1028-1040 and 1042-1055. */
+/* ---- data movement and the remaining element-wise kernels (round out a transformer block) ----
+ * Element sizes are in bytes; the movement kernels copy opaque elements of 1, 4 or 8 bytes. */
+
+/* compute_transpose (session.rs:1179-1278): the suffix of axes the permutation leaves in place
+ * forms a block that is copied whole; the blocks are enumerated with an odometer over the
+ * permuted strides.  PINNED by numpy.transpose (bit equality). */
+int orc_transpose(const void *in, void *out, int elem_size, int rank, const int64_t *in_dims, const int64_t *perm);
+
+/* compute_gather (session.rs:1560-1598).  The reference takes a scalar index (all axes before
+ * `axis` of extent 1) or indices of shape [1, n] with axis 0; strict = 1 reports anything else
+ * as ORC_ERR_UNSUPPORTED, strict = 0 computes the ONNX definition.  PINNED by numpy.take. */
+int orc_gather(const void *data, int elem_size, int rank, const int64_t *dims, int axis, const int64_t *indices,
+               int idx_rank, const int64_t *idx_dims, void *out, int strict, int *no_reference_kernel);
+
+/* compute_split (session.rs:1488-1512): last axis only in the reference (strict); any axis otherwise.
+ * outs[i] receives part i.  PINNED by numpy.split. */
+int orc_split(const void *in, int elem_size, int rank, const int64_t *dims, int axis, int n_parts,
+              const int64_t *parts, void *const *outs, int strict, int *no_reference_kernel);
+
+/* compute_where (session.rs:940-988): the reference's two patterns (cond.dims == y.dims with
+ * scalar x; 4-d cond [1,1,h,w] over x [n,c,h,w] with scalar y), else by NumPy broadcasting.
+ * PINNED by numpy.where. */
+int orc_where(const uint8_t *cond, int c_rank, const int64_t *c_dims, const float *x, int x_rank, const int64_t *x_dims,
+              const float *y, int y_rank, const int64_t *y_dims, float *out, int strict, int *no_reference_kernel);
+
+/* compute_greater (session.rs:541-562): scalar right-hand side in the reference. */
+int orc_greater(const float *a, int a_rank, const int64_t *a_dims, const float *b, int b_rank, const int64_t *b_dims,
+                uint8_t *out, int strict, int *no_reference_kernel);
+
+/* compute_cast (session.rs:1350-1378): Rust `as`.  Element types: 0 Bool, 1 F32, 2 I32, 3 I64.
+ * The reference implements i32->f32, i64->i32, i64->f32 and f32->bool. */
+int orc_cast(const void *in, int from_type, void *out, int to_type, size_t n, int strict, int *no_reference_kernel);
+
+/* compute_batch_normalization (session.rs:1380-1431), NCHW, inference mode. */
+int orc_batchnorm(const float *x, const float *scale, const float *bias, const float *mean, const float *var, float *out,
+                  size_t n, size_t c, size_t h, size_t w, float eps);
+
+/* compute_gavg_pool (session.rs:265-297): sequential sum of each H*W plane divided by H*W. */
+int orc_global_average_pool(const float *x, float *out, size_t n, size_t c, size_t h, size_t w);
+
+/* compute_leaky_relu (session.rs:814-821). */
+int orc_leaky_relu(const float *x, float *out, size_t n, float alpha);
+
 float orc_fast_sum(const float *x, size_t n);
 float orc_fast_sum_squares(const float *x, size_t n);
 

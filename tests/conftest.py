@@ -67,7 +67,17 @@ def assert_close(actual, expected, rtol=RTOL, atol=ATOL, what=""):
 
 
 def assert_bits_equal(actual, expected, what="", zero_sign_free=False):
-    """Bit-for-bit equality of two float32 arrays (NaN payloads excepted)."""
+    """Bit-for-bit equality of two float32 arrays (NaN payloads excepted); exact equality of
+    values and element type for integer and bool arrays."""
+    if np.asarray(expected).dtype.kind in "iub" or np.asarray(actual).dtype.kind in "iub":
+        actual, expected = np.asarray(actual), np.asarray(expected)
+        assert actual.dtype == expected.dtype, f"{what}: dtype {actual.dtype} vs {expected.dtype}"
+        assert actual.shape == expected.shape, f"{what}: shape {actual.shape} vs {expected.shape}"
+        if not np.array_equal(actual, expected):
+            bad = np.argwhere(actual != expected)
+            i = tuple(bad[0])
+            raise AssertionError(f"{what}: {len(bad)} of {actual.size} elements differ; first at {i}: {actual[i]} vs {expected[i]}")
+        return
     actual = np.asarray(actual, dtype=np.float32, order="C")
     expected = np.asarray(expected, dtype=np.float32, order="C")
     assert actual.shape == expected.shape, f"{what}: shape {actual.shape} vs {expected.shape}"

@@ -376,3 +376,108 @@ def test_golden_vectors(oracle):
     assert_bits_equal(oracle.layer_norm(x, gamma, beta, 1e-5), g["layernorm"], "golden layernorm")
     assert_bits_equal(oracle.reduce(0, x, [-1], True), g["reduce_mean"], "golden reduce_mean")
     assert_bits_equal(oracle.reduce(1, x, [1], False), g["reduce_max_axis1"], "golden reduce_max")
+
+
+# ---- data movement: the restated reference algorithms against numpy's own routines -----------------
+
+def test_transpose_matches_numpy(oracle):
+    rng = np.random.default_rng(5)
+    for shape, perm in [((2, 3, 4, 5), (0, 2, 1, 3)), ((2, 3, 4, 5), (3, 2, 1, 0)), ((6, 7), (1, 0)), ((2, 3, 4), (0, 1, 2)),
+                        ((2, 12, 197, 64), (0, 1, 3, 2)), ((1, 5, 1, 3), (2, 0, 3, 1)), ((4,), (0,)), ((0, 3), (1, 0))]:
+        for dt in (np.float32, np.int64, np.bool_):
+            x = (rng.standard_normal(shape) * 100).astype(dt)
+            got = oracle.transpose(x, perm)
+            assert got.shape == tuple(shape[p] for p in perm) and np.array_equal(got, np.transpose(x, perm))
+
+
+def test_gather_split_where_greater_match_numpy(oracle):
+    rng = np.random.default_rng(6)
+    d = rng.standard_normal((5, 6, 7)).astype(np.float32)
+    info = {}
+    # the reference's two patterns ...
+    e = rng.standard_normal((30, 8)).astype(np.float32)
+    idx = np.array([[3, 0, 29, 3]], np.int64)
+    assert np.array_equal(oracle.gather(e, idx, 0, strict=True, info=info), np.take(e, idx, axis=0)) and not info["no_reference_kernel"]
+    one = rng.standard_normal((1, 1, 9, 4)).astype(np.float32)
+    assert np.array_equal(oracle.gather(one, np.array(5, np.int64), 2, strict=True), np.take(one, 5, axis=2))
+    # ... and the ONNX definition beyond them
+    for axis, ix in [(0, [2, 2, 4]), (1, [[0, 5], [3, 3]]), (2, -1), (-2, [-6, 5])]:
+        got = oracle.gather(d, np.array(ix, np.int64), axis, info=info)
+        assert np.array_equal(got, np.take(d, np.array(ix), axis=axis)) and info["no_reference_kernel"]
+    with pytest.raises(oracle.OracleError):
+        oracle.gather(d, np.array([7], np.int64), 1)                      # out of range
+    with pytest.raises(oracle.OracleError):
+        oracle.gather(d, np.array([1, 2], np.int64), 1, strict=True)     # not one of the reference's patterns
+
+    x = rng.standard_normal((3, 4, 12)).astype(np.float32)
+    parts = oracle.split(x, [2, 4, 6], 2, strict=True)
+    for got, want in zip(parts, np.split(x, [2, 6], axis=2)):
+        assert np.array_equal(got, want)
+    for got, want in zip(oracle.split(x, [1, 3], 1), np.split(x, [1], axis=1)):
+        assert np.array_equal(got, want)
+    with pytest.raises(oracle.OracleError):
+        oracle.split(x, [1, 3], 1, strict=True)                           # the reference splits the last axis only
+
+    y = rng.standard_normal((2, 3, 5, 5)).astype(np.float32)
+    c = rng.random((2, 3, 5, 5)) > 0.5
+    assert np.array_equal(oracle.where(c, np.float32(-1e9), y, strict=True), np.where(c, np.float32(-1e9), y))
+    c2 = rng.random((1, 1, 5, 5)) > 0.5
+    assert np.array_equal(oracle.where(c2, y, np.float32(0.5), strict=True), np.where(c2, y, np.float32(0.5)))
+    c3 = rng.random((3, 1, 5)) > 0.5
+    assert np.array_equal(oracle.where(c3, y, y[:, :1] * 2, info=info), np.where(c3, y, y[:, :1] * 2)) and info["no_reference_kernel"]
+
+    assert np.array_equal(oracle.greater(y, np.float32(0.1), strict=True), y > np.float32(0.1))
+    assert np.array_equal(oracle.greater(y, y[:, :, :1], info=info), y > y[:, :, :1]) and info["no_reference_kernel"]
+    assert not oracle.greater(np.array([np.nan, 1.0], np.float32), np.float32(np.nan)).any()
+
+
+def test_cast_is_rusts_as(oracle):
+    info = {}
+    i32 = np.array([0, 1, -1, 2**31 - 1, -2**31, 16777217], np.int32)
+    assert np.array_equal(oracle.cast(i32, np.float32, strict=True), i32.astype(np.float32))               # round to nearest
+    i64 = np.array([0, -1, 2**31, 2**32 + 5, -2**63, 2**63 - 1, 2**53 + 1], np.int64)
+    assert np.array_equal(oracle.cast(i64, np.int32, strict=True), i64.astype(np.int32))                    # wraps
+    assert np.array_equal(oracle.cast(i64, np.float32, strict=True), i64.astype(np.float32))
+    f = np.array([0.0, -0.0, 1e-30, np.nan, np.inf, -3.5], np.float32)
+    assert oracle.cast(f, np.bool_, strict=True).tolist() == [False, False, True, True, True, True]         # x != 0.0
+    # beyond the reference's four arms: float -> int truncates, saturates, NaN -> 0
+    g = np.array([1.9, -1.9, 3e9, -3e9, np.nan, np.inf, -np.inf, 2147483520.0], np.float32)
+    assert oracle.cast(g, np.int32, info=info).tolist() == [1, -1, 2**31 - 1, -2**31, 0, 2**31 - 1, -2**31, 2147483520]
+    assert info["no_reference_kernel"]
+    assert oracle.cast(np.array([1e19, -1e19, 2.5, np.nan], np.float32), np.int64).tolist() == [2**63 - 1, -2**63, 2, 0]
+    assert oracle.cast(np.array([True, False]), np.float32).tolist() == [1.0, 0.0]
+    with pytest.raises(oracle.OracleError):
+        oracle.cast(g, np.int32, strict=True)
+
+
+def test_batchnorm_gavgpool_leakyrelu(oracle):
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((2, 3, 4, 5)).astype(np.float32)
+    scale, bias, mean = (rng.standard_normal(3).astype(np.float32) for _ in range(3))
+    var = rng.random(3).astype(np.float32) + np.float32(0.1)
+    eps = np.float32(1e-5)
+    got = oracle.batchnorm(x, scale, bias, mean, var, eps)
+    v = lambda a: a.reshape(1, 3, 1, 1)
+    want = ((x - v(mean)) / np.sqrt(v(var) + eps)) * v(scale) + v(bias)                   # the same fp32 steps, in numpy
+    assert np.array_equal(got, want)
+    exact = (x.astype(np.float64) - v(mean)) / np.sqrt(v(var).astype(np.float64) + 1e-5) * v(scale) + v(bias)
+    np.testing.assert_allclose(got, exact, rtol=1e-5, atol=1e-6)
+    # statistics taken from the data itself normalise it
+    m, s2 = x.mean((0, 2, 3)), x.var((0, 2, 3))
+    n = oracle.batchnorm(x, np.ones(3, np.float32), np.zeros(3, np.float32), m, s2, 0.0)
+    assert np.abs(n.mean((0, 2, 3))).max() < 1e-6 and np.abs(n.var((0, 2, 3)) - 1).max() < 1e-5
+
+    p = oracle.global_average_pool(x)
+    assert p.shape == (2, 3, 1, 1)
+    seq = np.zeros((2, 3), np.float32)
+    for i in range(4):
+        for j in range(5):
+            seq = seq + x[:, :, i, j]                                                      # the reference's left-to-right sum
+    assert np.array_equal(p[:, :, 0, 0], seq / np.float32(20))
+    ints = rng.integers(-8, 9, size=(2, 2, 7, 7)).astype(np.float32)
+    assert np.array_equal(oracle.global_average_pool(ints)[:, :, 0, 0], ints.sum((2, 3)) / np.float32(49))
+
+    z = np.array([-2.0, -0.0, 0.0, 3.0, np.nan, -np.inf], np.float32)
+    got = oracle.leaky_relu(z, 0.1)
+    assert np.array_equal(got[:4], np.array([np.float32(0.1) * np.float32(-2.0), -0.0, 0.0, 3.0], np.float32))
+    assert np.isnan(got[4]) and got[5] == -np.inf and np.signbit(got[1])
