@@ -112,6 +112,18 @@ public:
         return from_raw(std::move(dims), ty, nullptr, bytes, alloc);
     }
 
+    // The same bytes under another shape of as many elements (Tensor::copy_data_from shares the
+    // buffer in the reference too, tensor.rs:340-342); an empty tensor if the counts differ.
+    Tensor reshaped(FixedDimensions dims) const {
+        Tensor t;
+        if (dims.total_elems() != dims_.total_elems()) return t;
+        t.stride_ = dims.strides();
+        t.dims_ = std::move(dims);
+        t.elem_ty_ = elem_ty_;
+        t.data_ = data_;
+        return t;
+    }
+
     const FixedDimensions &dims() const { return dims_; }
     const FixedDimensions &strides() const { return stride_; }
     TensorElemType elem_ty() const { return elem_ty_; }

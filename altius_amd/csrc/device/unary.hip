@@ -37,6 +37,11 @@ struct FClip {
 };
 // Exp and Round have no kernel in the reference interpreter (session.rs:219-224): correctly
 // rounded-to-1-ulp expf, and round-half-to-even as ONNX defines Round.
+// x / alpha with a true division: the second half of GlobalAveragePool (sum / area, session.rs:291).
+struct FDivBy {
+    float d;
+    __device__ __forceinline__ float operator()(float x) const { return x / d; }
+};
 struct FExp { __device__ __forceinline__ float operator()(float x) const { return expf(x); } };
 struct FRound { __device__ __forceinline__ float operator()(float x) const { return rintf(x); } };
 
@@ -89,7 +94,7 @@ template <class F> void launch(hipStream_t s, float *out, const float *in, size_
 }  // namespace
 
 int launch_unary(DeviceCtx &ctx, int op, float *out, const float *in, size_t n, float alpha, float beta) {
-    if (op < AHIP_SQRT || op > AHIP_CLIP) return ctx.fail(AHIP_ERR_ARG, "unary: unknown op");
+    if (op < AHIP_SQRT || op > AHIP_DIV_BY) return ctx.fail(AHIP_ERR_ARG, "unary: unknown op");
     if (n == 0) return AHIP_OK;
     if (!out || !in) return ctx.fail(AHIP_ERR_ARG, "unary: null tensor pointer");
     if (n > ((size_t)1 << 38)) return ctx.fail(AHIP_ERR_UNSUPPORTED, "unary: more than 2^38 elements");
@@ -106,6 +111,7 @@ int launch_unary(DeviceCtx &ctx, int op, float *out, const float *in, size_t n, 
     case AHIP_EXP: launch(ctx.stream, out, in, n, FExp{}, nt); break;
     case AHIP_ROUND: launch(ctx.stream, out, in, n, FRound{}, nt); break;
     case AHIP_CLIP: launch(ctx.stream, out, in, n, FClip{alpha, beta}, nt); break;
+    case AHIP_DIV_BY: launch(ctx.stream, out, in, n, FDivBy{alpha}, nt); break;
     }
     return ctx.check(hipGetLastError(), "unary launch");
 }

@@ -2,8 +2,10 @@
 
 #include <algorithm>
 #include <chrono>
+#include <limits>
 
 #include "../device/host_pool.h"
+#include "host_eval.h"
 
 namespace altius {
 
@@ -123,31 +125,17 @@ std::unique_ptr<HipSession> HipSessionBuilder::build(SessionError *err) {
     }
     s->pool_.reset(new BufferPool(&s->ctx_));
 
-    // Initializers live on the device for the lifetime of the session.
+    // Initializers live on the device for the lifetime of the session; their host contents stay
+    // reachable for shape inference and shape arithmetic.
     for (const auto &kv : s->model_.graph.inits) {
         const Tensor &t = kv.second;
-        DeviceTensor d;
-        d.dims = t.dims();
-        d.elem_ty = t.elem_ty();
-        const size_t bytes = d.nbytes();
-        if (t.nbytes() != bytes) {
+        if (t.nbytes() != t.dims().total_elems() * elem_size(t.elem_ty())) {
             fail(err, SessionError::Argument, "initializer data does not match its shape");
             return nullptr;
         }
-        rc = s->pool_->acquire(bytes, &d.ptr, &d.bucket);
-        if (rc) {
-            fail_code(err, rc, s->ctx_.last_error);
-            return nullptr;
-        }
-        if (bytes) {
-            rc = s->ctx_.check(hipMemcpyAsync(d.ptr, t.data_as_bytes(), bytes, hipMemcpyHostToDevice, s->ctx_.stream),
-                               "hipMemcpyAsync(initializer)");
-            if (rc) {
-                fail_code(err, rc, s->ctx_.last_error);
-                return nullptr;
-            }
-        }
-        s->inits_[kv.first] = d;
+        DeviceTensor d;
+        if (!s->upload(t, &d, err)) return nullptr;
+        s->inits_[kv.first] = std::move(d);
     }
     rc = s->ctx_.check(hipStreamSynchronize(s->ctx_.stream), "hipStreamSynchronize(build)");
     if (rc) {
@@ -163,21 +151,53 @@ HipSession::~HipSession() {
     if (pool_) {
         (void)hipSetDevice(ctx_.device);
         (void)hipStreamSynchronize(ctx_.stream);
-        for (auto &kv : inits_) pool_->release(kv.second.ptr, kv.second.bucket);
-        inits_.clear();
+        inits_.clear();  // blocks go back to the pool before it is destroyed
         pool_.reset();
         destroy_device_ctx(&ctx_);
     }
 }
 
-void HipSession::release(DeviceTensor &t) {
-    if (t.pooled && t.ptr) pool_->release(t.ptr, t.bucket);
-    t.ptr = nullptr;
-    t.pooled = false;
+bool HipSession::allocate(const TypedFixedShape &shape, DeviceTensor *out, SessionError *err) {
+    out->dims = shape.dims;
+    out->elem_ty = shape.elem_ty;
+    out->host.reset();
+    auto block = std::make_shared<DeviceBlock>();
+    const int rc = pool_->acquire(out->nbytes(), &block->ptr, &block->bucket);
+    if (rc) return fail_code(err, rc, ctx_.last_error);
+    block->pool = pool_.get();
+    out->ptr = block->ptr;
+    out->block = std::move(block);
+    return true;
+}
+
+bool HipSession::upload(const Tensor &t, DeviceTensor *out, SessionError *err) {
+    if (!allocate(TypedFixedShape{t.dims(), t.elem_ty()}, out, err)) return false;
+    if (out->nbytes()) {
+        const int rc = ctx_.check(hipMemcpyAsync(out->ptr, t.data_as_bytes(), out->nbytes(), hipMemcpyHostToDevice, ctx_.stream),
+                                  "hipMemcpyAsync(upload)");
+        if (rc) return fail_code(err, rc, ctx_.last_error);
+    }
+    out->host = std::make_shared<const Tensor>(t);  // shares the bytes; keeps them alive while the copy is in flight
+    return true;
+}
+
+bool HipSession::fetch_host(DeviceTensor *t, SessionError *err) {
+    if (t->host) return true;
+    Tensor h = Tensor::uninit_of_type(t->elem_ty, t->dims);
+    if (!h.has_data()) return fail(err, SessionError::OutOfMemory, "out of host memory");
+    if (t->nbytes()) {
+        int rc = ctx_.check(hipMemcpyAsync(h.data_as_bytes_mut(), t->ptr, t->nbytes(), hipMemcpyDeviceToHost, ctx_.stream),
+                            "hipMemcpyAsync(shape operand)");
+        if (!rc) rc = ctx_.check(hipStreamSynchronize(ctx_.stream), "hipStreamSynchronize(shape operand)");
+        if (rc) return fail_code(err, rc, ctx_.last_error);
+    }
+    t->host = std::make_shared<const Tensor>(std::move(h));
+    return true;
 }
 
 bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *outputs, SessionError *err) {
     std::lock_guard<std::mutex> lock(mutex_);
+    const auto t0 = std::chrono::steady_clock::now();
     if (!outputs) return fail(err, SessionError::Argument, "run: null output vector");
     outputs->clear();
     profile_.clear();
@@ -188,71 +208,48 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
                         std::to_string(g.inputs.size()));
     if (hipSetDevice(ctx_.device) != hipSuccess) return fail(err, SessionError::Hip, "hipSetDevice failed");
 
-    const auto t0 = std::chrono::steady_clock::now();
     std::map<ValueId, DeviceTensor> values;
-    auto cleanup = [&]() {
-        (void)hipStreamSynchronize(ctx_.stream);  // nothing still reads a block that goes back to the pool
-        for (auto &kv : values) release(kv.second);
+    std::vector<hipEvent_t> events;
+    // Nothing may still read a block when it goes back to the pool for another run, and input
+    // tensors must outlive their uploads: every exit path synchronises first.
+    auto finish = [&](bool ok) {
+        (void)hipStreamSynchronize(ctx_.stream);
+        for (auto e : events) (void)hipEventDestroy(e);
+        values.clear();
+        return ok;
     };
 
     // Upload the inputs (positional, session.rs:81-83).
     for (size_t i = 0; i < g.inputs.size(); i++) {
         const Tensor &t = inputs[i];
-        if (!t.has_data()) {
-            cleanup();
-            return fail(err, SessionError::Argument, "run: input " + std::to_string(i) + " has no data");
-        }
+        if (!t.has_data()) return finish(fail(err, SessionError::Argument, "run: input " + std::to_string(i) + " has no data"));
         DeviceTensor d;
-        d.dims = t.dims();
-        d.elem_ty = t.elem_ty();
-        int rc = pool_->acquire(d.nbytes(), &d.ptr, &d.bucket);
-        if (rc) {
-            cleanup();
-            return fail_code(err, rc, ctx_.last_error);
-        }
-        d.pooled = true;
-        values[g.inputs[i]] = d;
-        if (d.nbytes()) {
-            rc = ctx_.check(hipMemcpyAsync(d.ptr, t.data_as_bytes(), d.nbytes(), hipMemcpyHostToDevice, ctx_.stream),
-                            "hipMemcpyAsync(input)");
-            if (rc) {
-                cleanup();
-                return fail_code(err, rc, ctx_.last_error);
-            }
-        }
+        if (!upload(t, &d, err)) return finish(false);
+        // Only small integer inputs keep their host view (shape arithmetic may read them).
+        if (t.elem_ty() == TensorElemType::F32 || t.dims().total_elems() > 4096) d.host.reset();
+        values[g.inputs[i]] = std::move(d);
     }
 
     // One event per node boundary when profiling.
-    std::vector<hipEvent_t> events;
     if (enable_profiling_) {
         events.resize(plan_.size() + 1);
-        for (auto &e : events) {
-            if (hipEventCreate(&e) != hipSuccess) {
-                cleanup();
-                return fail(err, SessionError::Hip, "hipEventCreate failed");
+        for (size_t i = 0; i < events.size(); i++) {
+            if (hipEventCreate(&events[i]) != hipSuccess) {
+                events.resize(i);
+                return finish(fail(err, SessionError::Hip, "hipEventCreate failed"));
             }
         }
         (void)hipEventRecord(events[0], ctx_.stream);
     }
-    auto destroy_events = [&]() {
-        for (auto e : events) (void)hipEventDestroy(e);
-    };
 
     // The hot loop (session.rs:86-92).
     for (size_t i = 0; i < plan_.size(); i++) {
-        if (!run_node(plan_[i].node_id, values, err)) {
-            cleanup();
-            destroy_events();
-            return false;
-        }
+        if (!run_node(plan_[i].node_id, values, err)) return finish(false);
         if (enable_profiling_) (void)hipEventRecord(events[i + 1], ctx_.stream);
-        for (ValueId v : plan_[i].free_vals) {
-            auto it = values.find(v);
-            if (it != values.end()) {
-                release(it->second);  // stream order makes immediate reuse safe
-                values.erase(it);
-            }
-        }
+        // Stream order makes immediate reuse safe.  A value that is also a graph output stays: the
+        // plan lists it when another node reads it, but it is still owed to the caller.
+        for (ValueId v : plan_[i].free_vals)
+            if (std::find(g.outputs.begin(), g.outputs.end(), v) == g.outputs.end()) values.erase(v);
     }
 
     // Download the outputs (session.rs:127-133).
@@ -264,34 +261,21 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
             auto ii = inits_.find(v);
             if (ii != inits_.end()) d = &ii->second;
         }
-        if (!d) {
-            cleanup();
-            destroy_events();
-            return fail(err, SessionError::Message, "run: graph output was not produced");
-        }
+        if (!d) return finish(fail(err, SessionError::Message, "run: graph output was not produced"));
         Tensor t = Tensor::uninit_of_type(d->elem_ty, d->dims, pinned_host_block);
-        if (!t.has_data()) {
-            cleanup();
-            destroy_events();
-            return fail(err, SessionError::OutOfMemory, "run: out of host memory for an output tensor");
-        }
+        if (!t.has_data()) return finish(fail(err, SessionError::OutOfMemory, "run: out of host memory for an output tensor"));
         if (d->nbytes()) {
-            int rc = ctx_.check(hipMemcpyAsync(t.data_as_bytes_mut(), d->ptr, d->nbytes(), hipMemcpyDeviceToHost,
-                                               ctx_.stream),
-                                "hipMemcpyAsync(output)");
-            if (rc) {
-                cleanup();
-                destroy_events();
-                return fail_code(err, rc, ctx_.last_error);
-            }
+            const int rc = ctx_.check(hipMemcpyAsync(t.data_as_bytes_mut(), d->ptr, d->nbytes(), hipMemcpyDeviceToHost, ctx_.stream),
+                                      "hipMemcpyAsync(output)");
+            if (rc) return finish(fail_code(err, rc, ctx_.last_error));
         }
         outputs->push_back(std::move(t));
     }
     int rc = ctx_.check(hipStreamSynchronize(ctx_.stream), "hipStreamSynchronize(run)");
+    if (!rc) rc = check_device_flags(ctx_);
     if (rc) {
-        cleanup();
-        destroy_events();
-        return fail_code(err, rc, ctx_.last_error);
+        outputs->clear();
+        return finish(fail_code(err, rc, ctx_.last_error));
     }
     if (enable_profiling_) {
         for (size_t i = 0; i < plan_.size(); i++) {
@@ -299,19 +283,35 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
             if (hipEventElapsedTime(&ms, events[i], events[i + 1]) == hipSuccess)
                 profile_[model_.graph.nodes[plan_[i].node_id].op.name()] += ms;
         }
-        destroy_events();
     }
-    for (auto &kv : values) release(kv.second);
+    finish(true);
     last_run_ms_ = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     return true;
 }
+
+namespace {
+
+bool is_alias_op(OpKind k) {
+    return k == OpKind::Reshape || k == OpKind::Flatten || k == OpKind::Squeeze || k == OpKind::Unsqueeze;
+}
+
+// [outer, axis, inner] view of `dims` around `axis`.
+void split_at(const FixedDimensions &dims, size_t axis, size_t *outer, size_t *len, size_t *inner) {
+    *outer = *inner = 1;
+    for (size_t i = 0; i < axis; i++) *outer *= dims[i];
+    *len = dims[axis];
+    for (size_t i = axis + 1; i < dims.len(); i++) *inner *= dims[i];
+}
+
+}  // namespace
 
 bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, SessionError *err) {
     const Node &node = model_.graph.nodes[id];
     const std::string opname = node.op.name();
 
-    // Inputs: run-time values first, then initializers.
-    std::vector<const DeviceTensor *> in;
+    // Inputs: run-time values first, then initializers.  An input whose value is never produced
+    // and carries the empty name is an omitted optional input (the reference binds a dummy tensor).
+    std::vector<DeviceTensor *> in;
     for (ValueId v : node.inputs) {
         auto it = values.find(v);
         if (it != values.end()) {
@@ -319,11 +319,21 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
             continue;
         }
         auto ii = inits_.find(v);
-        if (ii == inits_.end()) return fail(err, SessionError::Message, opname + ": an input value is missing");
-        in.push_back(&ii->second);
+        if (ii != inits_.end()) {
+            in.push_back(&ii->second);
+            continue;
+        }
+        const auto &name = model_.graph.values[v].name;
+        if (name && name->empty()) {
+            in.push_back(nullptr);
+            continue;
+        }
+        return fail(err, SessionError::Message, opname + ": an input value is missing");
     }
+    if (node.outputs.empty()) return fail(err, SessionError::Message, opname + ": node without outputs");
 
-    // Output shapes: inferred at build time if possible, else now (session.rs:149-158).
+    // Output shapes: inferred at build time if possible, else now (session.rs:149-158).  Operands
+    // whose contents decide a shape are read from their host copy, fetched on demand.
     Op op = node.op;
     std::vector<TypedFixedShape> shapes;
     auto cached = inferred_.find(id);
@@ -331,109 +341,233 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
         op = cached->second.first;
         shapes = cached->second.second;
     } else {
-        std::vector<Tensor> meta;
-        meta.reserve(in.size());
-        for (auto *d : in) meta.push_back(Tensor::empty_of_type(d->elem_ty, d->dims));
-        std::vector<const Tensor *> ptrs;
-        for (auto &m : meta) ptrs.push_back(&m);
-        ShapeError serr;
-        if (!compute_output_shapes(model_, op, ptrs, node.outputs.size(), &shapes, &serr))
-            return fail(err, SessionError::Shape, serr.message);
+        static const Tensor absent;
+        for (int attempt = 0;; attempt++) {
+            std::vector<Tensor> meta;
+            meta.reserve(in.size());
+            for (auto *d : in) meta.push_back(!d ? absent : d->host ? *d->host : Tensor::empty_of_type(d->elem_ty, d->dims));
+            std::vector<const Tensor *> ptrs;
+            for (auto &m : meta) ptrs.push_back(&m);
+            ShapeError serr;
+            op = node.op;
+            if (compute_output_shapes(model_, op, ptrs, node.outputs.size(), &shapes, &serr)) break;
+            if (!serr.needs_data || attempt > 0) return fail(err, SessionError::Shape, serr.message);
+            // Read back the small operands (shape vectors, Resize scales) and try once more.
+            for (size_t i = 1; i < in.size(); i++)
+                if (in[i] && !in[i]->host && in[i]->dims.total_elems() <= 4096 && !fetch_host(in[i], err)) return false;
+        }
     }
-    if (shapes.size() < node.outputs.size() || node.outputs.empty())
-        return fail(err, SessionError::Message, opname + ": output count mismatch");
+    if (shapes.size() < node.outputs.size()) return fail(err, SessionError::Message, opname + ": output count mismatch");
 
-    // Every kernel here computes in fp32.
-    for (auto *d : in)
-        if (d->elem_ty != TensorElemType::F32)
-            return fail(err, SessionError::Message,
-                        opname + ": input type " + elem_name(d->elem_ty) + " is not supported (f32 only)");
+    std::vector<DeviceTensor> outs;
 
-    // Allocate the output, pre-sized, contents unspecified (session.rs:159-162).
-    DeviceTensor out;
-    out.dims = shapes[0].dims;
-    out.elem_ty = shapes[0].elem_ty;
-    int rc = pool_->acquire(out.nbytes(), &out.ptr, &out.bucket);
-    if (rc) return fail_code(err, rc, ctx_.last_error);
-    out.pooled = true;
-    float *o = static_cast<float *>(out.ptr);
-    auto f = [](const DeviceTensor *d) { return static_cast<const float *>(d->ptr); };
-    auto bail = [&](SessionError::Kind k, const std::string &msg) {
-        release(out);
-        return fail(err, k, msg);
+    // Reshape family: the output is the input's memory under another shape.
+    if (is_alias_op(op.kind) && in[0]) {
+        DeviceTensor o = *in[0];
+        o.dims = shapes[0].dims;
+        if (in[0]->host) {
+            Tensor h = in[0]->host->reshaped(shapes[0].dims);
+            o.host = h.has_data() || shapes[0].dims.total_elems() == 0 ? std::make_shared<const Tensor>(std::move(h)) : nullptr;
+        }
+        outs.push_back(std::move(o));
+    } else {
+        // Shape arithmetic: integer tensors whose operands the host already knows (or can read back
+        // cheaply) are computed there and uploaded; Shape and Constant always are.
+        bool on_host = false;
+        if (host_evaluable(op)) {
+            const bool int_out = shapes[0].elem_ty != TensorElemType::F32;
+            bool small = shapes[0].dims.total_elems() <= 4096;
+            bool ints_in = true;
+            for (auto *d : in)
+                if (d) {
+                    small = small && d->dims.total_elems() <= 4096;
+                    ints_in = ints_in && d->elem_ty != TensorElemType::F32;
+                }
+            if (op.kind == OpKind::Shape || op.kind == OpKind::Constant) {
+                on_host = true;
+            } else if (small && ints_in && (int_out || op.kind == OpKind::Cast)) {
+                on_host = true;
+                for (auto *d : in)
+                    if (d && !fetch_host(d, err)) return false;
+            }
+        }
+        if (on_host) {
+            std::vector<const Tensor *> hin;
+            static const Tensor no_data;
+            for (auto *d : in) hin.push_back(!d ? nullptr : d->host ? d->host.get() : &no_data);
+            // Shape reads only the dims of its operand.
+            std::vector<Tensor> dims_only;
+            if (op.kind == OpKind::Shape && in[0] && !in[0]->host) {
+                dims_only.push_back(Tensor::empty_of_type(in[0]->elem_ty, in[0]->dims));
+                hin[0] = &dims_only[0];
+            }
+            std::vector<Tensor> results;
+            std::string msg;
+            if (!evaluate_on_host(model_, op, hin, shapes, &results, &msg)) return fail(err, SessionError::Message, msg);
+            for (const Tensor &t : results) {
+                DeviceTensor d;
+                if (!upload(t, &d, err)) return false;
+                outs.push_back(std::move(d));
+            }
+        } else if (!run_device_op(node, op, in, shapes, &outs, err)) {
+            return false;
+        }
+    }
+    for (size_t i = 0; i < node.outputs.size() && i < outs.size(); i++) values[node.outputs[i]] = std::move(outs[i]);
+    return true;
+}
+
+bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector<DeviceTensor *> &in,
+                               const std::vector<TypedFixedShape> &shapes, std::vector<DeviceTensor> *outs, SessionError *err) {
+    const std::string opname = op.name();
+    auto need = [&](size_t n) {
+        if (in.size() >= n) {
+            bool all = true;
+            for (size_t i = 0; i < n; i++) all = all && in[i];
+            if (all) return true;
+        }
+        return fail(err, SessionError::Message, opname + ": expected " + std::to_string(n) + " inputs");
     };
+    auto need_f32 = [&](std::initializer_list<size_t> which) {
+        for (size_t i : which)
+            if (in[i]->elem_ty != TensorElemType::F32)
+                return fail(err, SessionError::Message,
+                            opname + ": input type " + elem_name(in[i]->elem_ty) + " is not supported (f32 only)");
+        return true;
+    };
+    auto f = [](const DeviceTensor *d) { return static_cast<const float *>(d->ptr); };
+    auto esize = [](const DeviceTensor *d) { return (int)elem_size(d->elem_ty); };
+    auto i64v = [](const FixedDimensions &d) {
+        std::vector<int64_t> v;
+        for (auto x : d.as_vec()) v.push_back((int64_t)x);
+        return v;
+    };
+    auto done = [&](int rc) { return rc ? fail_code(err, rc, ctx_.last_error) : true; };
+
+    // Split produces one tensor per part; everything else one output.
+    if (op.kind == OpKind::Split) {
+        if (!need(1)) return false;
+        const size_t rank = in[0]->dims.len();
+        const size_t axis = (size_t)(op.axis < 0 ? op.axis + (int64_t)rank : op.axis);
+        const std::vector<int64_t> in_str = i64v(in[0]->dims.strides());
+        size_t start = 0;
+        for (size_t p = 0; p < node.outputs.size(); p++) {
+            DeviceTensor o;
+            if (!allocate(shapes[p], &o, err)) return false;
+            const std::vector<int64_t> d = i64v(o.dims), os = i64v(o.dims.strides());
+            const char *src = static_cast<const char *>(in[0]->ptr) + start * (size_t)in_str[axis] * (size_t)esize(in[0]);
+            if (!done(launch_copy_strided(ctx_, o.ptr, src, esize(in[0]), (int)rank, d.data(), os.data(), in_str.data()))) return false;
+            start += o.dims[axis];
+            outs->push_back(std::move(o));
+        }
+        return true;
+    }
+
+    DeviceTensor out;
+    if (!allocate(shapes[0], &out, err)) return false;
+    float *o = static_cast<float *>(out.ptr);
+    const size_t n_out = out.dims.total_elems();
+    int rc = AHIP_OK;
 
     switch (op.kind) {
     case OpKind::Identity:
+        if (!need(1)) return false;
         if (out.nbytes())
-            rc = ctx_.check(hipMemcpyAsync(out.ptr, in[0]->ptr, out.nbytes(), hipMemcpyDeviceToDevice, ctx_.stream),
-                            "hipMemcpyAsync(Identity)");
+            rc = ctx_.check(hipMemcpyAsync(out.ptr, in[0]->ptr, out.nbytes(), hipMemcpyDeviceToDevice, ctx_.stream), "hipMemcpyAsync(Identity)");
         break;
     case OpKind::Add:
     case OpKind::Sub:
     case OpKind::Mul:
     case OpKind::Div:
     case OpKind::Pow: {
+        if (!need(2) || !need_f32({0, 1})) return false;
         auto as = in[0]->dims.strides_for_broadcasting_to(out.dims);
         auto bs = in[1]->dims.strides_for_broadcasting_to(out.dims);
-        if (!as || !bs) return bail(SessionError::Shape, opname + ": operands do not broadcast to the output shape");
-        const size_t rank = out.dims.len();
-        if (rank > (size_t)MAX_RANK) return bail(SessionError::Message, opname + ": rank above 8 is not supported");
-        int64_t dims[MAX_RANK], sa[MAX_RANK], sb[MAX_RANK];
-        for (size_t i = 0; i < rank; i++) {
-            dims[i] = (int64_t)out.dims[i];
-            sa[i] = (int64_t)(*as)[i];
-            sb[i] = (int64_t)(*bs)[i];
-        }
+        if (!as || !bs) return fail(err, SessionError::Shape, opname + ": operands do not broadcast to the output shape");
+        if (out.dims.len() > (size_t)MAX_RANK) return fail(err, SessionError::Message, opname + ": rank above 8 is not supported");
+        const std::vector<int64_t> dims = i64v(out.dims), sa = i64v(*as), sb = i64v(*bs);
         const int bop = op.kind == OpKind::Add   ? AHIP_ADD
                         : op.kind == OpKind::Sub ? AHIP_SUB
                         : op.kind == OpKind::Mul ? AHIP_MUL
                         : op.kind == OpKind::Div ? AHIP_DIV
                                                  : AHIP_POW;
-        rc = launch_binary(ctx_, bop, o, f(in[0]), f(in[1]), (int)rank, dims, sa, sb);
+        rc = launch_binary(ctx_, bop, o, f(in[0]), f(in[1]), (int)dims.size(), dims.data(), sa.data(), sb.data());
         break;
     }
-    case OpKind::Sqrt: rc = launch_unary(ctx_, AHIP_SQRT, o, f(in[0]), out.dims.total_elems(), 0, 0); break;
-    case OpKind::ReLU: rc = launch_unary(ctx_, AHIP_RELU, o, f(in[0]), out.dims.total_elems(), 0, 0); break;
-    case OpKind::Gelu: rc = launch_unary(ctx_, AHIP_GELU, o, f(in[0]), out.dims.total_elems(), 0, 0); break;
-    case OpKind::Sigmoid: rc = launch_unary(ctx_, AHIP_SIGMOID, o, f(in[0]), out.dims.total_elems(), 0, 0); break;
-    case OpKind::Erf: rc = launch_unary(ctx_, AHIP_ERF, o, f(in[0]), out.dims.total_elems(), 0, 0); break;
-    case OpKind::Tanh: rc = launch_unary(ctx_, AHIP_TANH, o, f(in[0]), out.dims.total_elems(), 0, 0); break;
+    case OpKind::Sqrt:
+    case OpKind::ReLU:
+    case OpKind::Gelu:
+    case OpKind::Sigmoid:
+    case OpKind::Erf:
+    case OpKind::Tanh:
+    case OpKind::Exp:
+    case OpKind::Round:
     case OpKind::HardSigmoid:
-        rc = launch_unary(ctx_, AHIP_HARDSIGMOID, o, f(in[0]), out.dims.total_elems(), op.alpha, op.beta);
+    case OpKind::LeakyReLU: {
+        if (!need(1) || !need_f32({0})) return false;
+        int uop = AHIP_SQRT;
+        float a = 0, b = 0;
+        switch (op.kind) {
+        case OpKind::Sqrt: uop = AHIP_SQRT; break;
+        case OpKind::ReLU: uop = AHIP_RELU; break;
+        case OpKind::Gelu: uop = AHIP_GELU; break;
+        case OpKind::Sigmoid: uop = AHIP_SIGMOID; break;
+        case OpKind::Erf: uop = AHIP_ERF; break;
+        case OpKind::Tanh: uop = AHIP_TANH; break;
+        case OpKind::Exp: uop = AHIP_EXP; break;
+        case OpKind::Round: uop = AHIP_ROUND; break;
+        case OpKind::HardSigmoid: uop = AHIP_HARDSIGMOID; a = op.alpha; b = op.beta; break;
+        default: uop = AHIP_LEAKYRELU; a = op.alpha; break;
+        }
+        rc = launch_unary(ctx_, uop, o, f(in[0]), n_out, a, b);
         break;
+    }
+    case OpKind::Clip: {  // bounds are optional scalar inputs (opset >= 11); the host needs their values
+        if (!need(1) || !need_f32({0})) return false;
+        float lo = -std::numeric_limits<float>::infinity(), hi = std::numeric_limits<float>::infinity();
+        for (size_t k = 1; k <= 2; k++) {
+            if (k >= in.size() || !in[k] || in[k]->dims.total_elems() == 0) continue;
+            if (in[k]->elem_ty != TensorElemType::F32 || in[k]->dims.total_elems() != 1)
+                return fail(err, SessionError::Message, "Clip: bounds must be f32 scalars");
+            if (!fetch_host(in[k], err)) return false;
+            (k == 1 ? lo : hi) = *in[k]->host->data_f32();
+        }
+        rc = launch_unary(ctx_, AHIP_CLIP, o, f(in[0]), n_out, lo, hi);
+        break;
+    }
     case OpKind::Softmax: {
+        if (!need(1) || !need_f32({0})) return false;
         const size_t rank = in[0]->dims.len();
-        if (rank == 0) return bail(SessionError::Message, "Softmax: rank-0 input");
+        if (rank == 0) return fail(err, SessionError::Message, "Softmax: rank-0 input");
         if (!(op.axis == -1 || op.axis == (int64_t)rank - 1))  // session.rs:999
-            return bail(SessionError::Message, "Softmax: only the last axis is supported");
+            return fail(err, SessionError::Message, "Softmax: only the last axis is supported");
         const size_t len = in[0]->dims[rank - 1];
-        rc = launch_softmax(ctx_, o, f(in[0]), len ? out.dims.total_elems() / len : 0, len);
+        rc = launch_softmax(ctx_, o, f(in[0]), len ? n_out / len : 0, len);
         break;
     }
     case OpKind::LayerNormalization: {
+        if (!need(3) || !need_f32({0, 1, 2})) return false;
         const size_t rank = in[0]->dims.len();
-        if (rank == 0) return bail(SessionError::Message, "LayerNormalization: rank-0 input");
+        if (rank == 0) return fail(err, SessionError::Message, "LayerNormalization: rank-0 input");
         if (!(op.axis == -1 || op.axis == (int64_t)rank - 1))
-            return bail(SessionError::Message, "LayerNormalization: Axis must be the last dimension.");
-        if (op.stash_type != 1) return bail(SessionError::Message, "LayerNormalization: Stash type must be 1.");
+            return fail(err, SessionError::Message, "LayerNormalization: Axis must be the last dimension.");
+        if (op.stash_type != 1) return fail(err, SessionError::Message, "LayerNormalization: Stash type must be 1.");
         const size_t len = in[0]->dims[rank - 1];
         if (in[1]->dims.total_elems() != len || in[2]->dims.total_elems() != len)
-            return bail(SessionError::Shape, "LayerNormalization: scale and bias must hold one value per column");
-        rc = launch_layernorm(ctx_, o, f(in[0]), f(in[1]), f(in[2]), len ? out.dims.total_elems() / len : 0, len,
-                              op.epsilon);
+            return fail(err, SessionError::Shape, "LayerNormalization: scale and bias must hold one value per column");
+        rc = launch_layernorm(ctx_, o, f(in[0]), f(in[1]), f(in[2]), len ? n_out / len : 0, len, op.epsilon);
         break;
     }
     case OpKind::ReduceMean:
     case OpKind::ReduceMax: {
+        if (!need(1) || !need_f32({0})) return false;
         const FixedDimensions &d = in[0]->dims;
         const size_t rank = d.len();
         std::vector<size_t> axes;
         if (op.axes.empty()) {
             if (op.kind == OpKind::ReduceMean) {  // nothing is reduced: the output is the input
                 if (out.nbytes())
-                    rc = ctx_.check(hipMemcpyAsync(out.ptr, in[0]->ptr, out.nbytes(), hipMemcpyDeviceToDevice,
-                                                   ctx_.stream),
+                    rc = ctx_.check(hipMemcpyAsync(out.ptr, in[0]->ptr, out.nbytes(), hipMemcpyDeviceToDevice, ctx_.stream),
                                     "hipMemcpyAsync(ReduceMean)");
                 break;
             }
@@ -446,27 +580,159 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
             std::sort(axes.begin(), axes.end());
             axes.erase(std::unique(axes.begin(), axes.end()), axes.end());
             for (size_t i = 1; i < axes.size(); i++)
-                if (axes[i] != axes[i - 1] + 1)
-                    return bail(SessionError::Message, opname + ": reduced axes must be adjacent");
+                if (axes[i] != axes[i - 1] + 1) return fail(err, SessionError::Message, opname + ": reduced axes must be adjacent");
             for (size_t i = 0; i < axes.front(); i++) outer *= d[i];
             for (size_t i = axes.front(); i <= axes.back(); i++) red *= d[i];
             for (size_t i = axes.back() + 1; i < rank; i++) inner *= d[i];
         }
-        rc = launch_reduce(ctx_, op.kind == OpKind::ReduceMean ? AHIP_REDUCE_MEAN : AHIP_REDUCE_MAX, o, f(in[0]),
-                           outer, red, inner);
+        rc = launch_reduce(ctx_, op.kind == OpKind::ReduceMean ? AHIP_REDUCE_MEAN : AHIP_REDUCE_MAX, o, f(in[0]), outer, red, inner);
         break;
     }
-    default:
-        return bail(SessionError::Message, opname + ": Kernel not implemented");
+    case OpKind::GlobalAveragePool: {  // sum of each H*W plane, then a true division by H*W (session.rs:265-297)
+        if (!need(1) || !need_f32({0})) return false;
+        const FixedDimensions &d = in[0]->dims;
+        const size_t planes = d[0] * d[1], area = d[2] * d[3];
+        if (area == 0) return fail(err, SessionError::Shape, "GlobalAveragePool: empty plane");
+        rc = launch_reduce(ctx_, AHIP_REDUCE_SUM, o, f(in[0]), planes, area, 1);
+        if (!rc) rc = launch_unary(ctx_, AHIP_DIV_BY, o, o, planes, (float)area, 0);
+        break;
     }
-    if (rc) {
-        release(out);
-        return fail_code(err, rc, ctx_.last_error);
+    case OpKind::BatchNormalization: {
+        if (!need(5) || !need_f32({0, 1, 2, 3, 4})) return false;
+        if (op.training_mode) return fail(err, SessionError::Message, "BatchNormalization: Training mode is not supported.");
+        const FixedDimensions &d = in[0]->dims;
+        if (d.len() < 2) return fail(err, SessionError::Message, "BatchNormalization: input rank must be at least 2");
+        const size_t c = d[1];
+        for (size_t k = 1; k < 5; k++)
+            if (in[k]->dims.total_elems() != c) return fail(err, SessionError::Shape, "BatchNormalization: one value per channel is needed");
+        size_t hw = 1;
+        for (size_t i = 2; i < d.len(); i++) hw *= d[i];
+        rc = launch_batchnorm(ctx_, o, f(in[0]), f(in[1]), f(in[2]), f(in[3]), f(in[4]), d[0], c, hw, op.epsilon);
+        break;
     }
-    // A node may be listed with more outputs than this backend produces; only the first is bound.
-    auto old = values.find(node.outputs[0]);
-    if (old != values.end()) release(old->second);
-    values[node.outputs[0]] = out;
+    case OpKind::Transpose: {
+        if (!need(1)) return false;
+        const std::vector<int64_t> d = i64v(in[0]->dims);
+        rc = launch_transpose(ctx_, out.ptr, in[0]->ptr, esize(in[0]), (int)d.size(), d.data(), op.perm.data());
+        break;
+    }
+    case OpKind::Concat: {
+        if (!need(1)) return false;
+        const size_t rank = out.dims.len();
+        const size_t axis = (size_t)(op.axis < 0 ? op.axis + (int64_t)rank : op.axis);
+        const std::vector<int64_t> out_str = i64v(out.dims.strides());
+        size_t at = 0;
+        for (auto *t : in) {
+            if (!t) return fail(err, SessionError::Message, "Concat: an input value is missing");
+            if (t->elem_ty != out.elem_ty) return fail(err, SessionError::Message, "Concat: inputs differ in element type");
+            const std::vector<int64_t> d = i64v(t->dims), is = i64v(t->dims.strides());
+            char *dst = static_cast<char *>(out.ptr) + at * (size_t)out_str[axis] * (size_t)esize(t);
+            rc = launch_copy_strided(ctx_, dst, t->ptr, esize(t), (int)rank, d.data(), out_str.data(), is.data());
+            if (rc) break;
+            at += t->dims[axis];
+        }
+        break;
+    }
+    case OpKind::Slice: {
+        if (!need(3)) return false;
+        std::vector<int64_t> starts, ends, axes, steps;
+        auto read = [&](size_t k, std::vector<int64_t> *v) {
+            if (k >= in.size() || !in[k] || in[k]->dims.total_elems() == 0) return true;
+            if (!fetch_host(in[k], err)) return false;
+            const Tensor &t = *in[k]->host;
+            const size_t n = t.dims().total_elems();
+            for (size_t i = 0; i < n; i++)
+                v->push_back(t.elem_ty() == TensorElemType::I64 ? reinterpret_cast<const int64_t *>(t.data_as_bytes())[i]
+                                                                 : (int64_t)reinterpret_cast<const int32_t *>(t.data_as_bytes())[i]);
+            return true;
+        };
+        if (!read(1, &starts) || !read(2, &ends) || !read(3, &axes) || !read(4, &steps)) return false;
+        if (axes.empty())
+            for (size_t i = 0; i < starts.size(); i++) axes.push_back((int64_t)i);
+        if (steps.empty()) steps.assign(starts.size(), 1);
+        const FixedDimensions &d = in[0]->dims;
+        std::vector<int64_t> in_str = i64v(d.strides());
+        const std::vector<int64_t> base_str = in_str;
+        size_t base = 0;
+        for (size_t i = 0; i < starts.size(); i++) {
+            const size_t ax = (size_t)(axes[i] < 0 ? axes[i] + (int64_t)d.len() : axes[i]);
+            const int64_t n = (int64_t)d[ax];
+            int64_t s = starts[i] < 0 ? starts[i] + n : starts[i];
+            s = std::min(std::max<int64_t>(s, 0), n);
+            base += (size_t)s * (size_t)base_str[ax];
+            in_str[ax] = base_str[ax] * steps[i];
+        }
+        const std::vector<int64_t> od = i64v(out.dims), os = i64v(out.dims.strides());
+        const char *src = static_cast<const char *>(in[0]->ptr) + base * (size_t)esize(in[0]);
+        rc = launch_copy_strided(ctx_, out.ptr, src, esize(in[0]), (int)od.size(), od.data(), os.data(), in_str.data());
+        break;
+    }
+    case OpKind::Expand: {
+        if (!need(1)) return false;
+        auto is = in[0]->dims.strides_for_broadcasting_to(out.dims);
+        if (!is) return fail(err, SessionError::Shape, "Expand: the input does not broadcast to the output shape");
+        const std::vector<int64_t> od = i64v(out.dims), os = i64v(out.dims.strides()), ist = i64v(*is);
+        rc = launch_copy_strided(ctx_, out.ptr, in[0]->ptr, esize(in[0]), (int)od.size(), od.data(), os.data(), ist.data());
+        break;
+    }
+    case OpKind::Tile: {  // each axis becomes (repeat, extent) with stride 0 on the repeat
+        if (!need(1)) return false;
+        const FixedDimensions &d = in[0]->dims;
+        if (d.len() * 2 > (size_t)MAX_RANK) return fail(err, SessionError::Message, "Tile: rank above 4 is not supported");
+        std::vector<int64_t> dims, os, is;
+        const std::vector<int64_t> in_str = i64v(d.strides()), out_str = i64v(out.dims.strides());
+        for (size_t i = 0; i < d.len(); i++) {
+            const int64_t reps = d[i] ? (int64_t)(out.dims[i] / d[i]) : 0;
+            dims.push_back(reps);
+            os.push_back(out_str[i] * (int64_t)d[i]);
+            is.push_back(0);
+            dims.push_back((int64_t)d[i]);
+            os.push_back(out_str[i]);
+            is.push_back(in_str[i]);
+        }
+        rc = launch_copy_strided(ctx_, out.ptr, in[0]->ptr, esize(in[0]), (int)dims.size(), dims.data(), os.data(), is.data());
+        break;
+    }
+    case OpKind::Gather: {
+        if (!need(2)) return false;
+        if (in[1]->elem_ty != TensorElemType::I64 && in[1]->elem_ty != TensorElemType::I32)
+            return fail(err, SessionError::Message, "Gather: indices must be i32 or i64");
+        const size_t rank = in[0]->dims.len();
+        const size_t axis = (size_t)(op.axis < 0 ? op.axis + (int64_t)rank : op.axis);
+        size_t outer, len, inner;
+        split_at(in[0]->dims, axis, &outer, &len, &inner);
+        ctx_.flags_armed = true;
+        rc = launch_gather(ctx_, out.ptr, in[0]->ptr, in[1]->ptr, esize(in[1]), esize(in[0]), outer, len, in[1]->dims.total_elems(), inner,
+                           ctx_.flags);
+        break;
+    }
+    case OpKind::Where: {
+        if (!need(3)) return false;
+        if (in[0]->elem_ty != TensorElemType::Bool) return fail(err, SessionError::Message, "Where: the condition must be bool");
+        if (in[1]->elem_ty != in[2]->elem_ty) return fail(err, SessionError::Message, "Where: x and y differ in element type");
+        auto cs = in[0]->dims.strides_for_broadcasting_to(out.dims), xs = in[1]->dims.strides_for_broadcasting_to(out.dims),
+             ys = in[2]->dims.strides_for_broadcasting_to(out.dims);
+        if (!cs || !xs || !ys) return fail(err, SessionError::Shape, "Where: operands do not broadcast to the output shape");
+        const std::vector<int64_t> d = i64v(out.dims), c = i64v(*cs), x = i64v(*xs), y = i64v(*ys);
+        rc = launch_where(ctx_, out.ptr, in[0]->ptr, in[1]->ptr, in[2]->ptr, esize(in[1]), (int)d.size(), d.data(), c.data(), x.data(), y.data());
+        break;
+    }
+    case OpKind::Greater: {
+        if (!need(2) || !need_f32({0, 1})) return false;
+        auto as = in[0]->dims.strides_for_broadcasting_to(out.dims), bs = in[1]->dims.strides_for_broadcasting_to(out.dims);
+        if (!as || !bs) return fail(err, SessionError::Shape, "Greater: operands do not broadcast to the output shape");
+        const std::vector<int64_t> d = i64v(out.dims), a = i64v(*as), b = i64v(*bs);
+        rc = launch_greater(ctx_, static_cast<uint8_t *>(out.ptr), f(in[0]), f(in[1]), (int)d.size(), d.data(), a.data(), b.data());
+        break;
+    }
+    case OpKind::Cast:
+        if (!need(1)) return false;
+        rc = launch_cast(ctx_, out.ptr, in[0]->ptr, (int)in[0]->elem_ty, (int)out.elem_ty, n_out);
+        break;
+    default: return fail(err, SessionError::Message, opname + ": Kernel not implemented");
+    }
+    if (rc) return fail_code(err, rc, ctx_.last_error);
+    outs->push_back(std::move(out));
     return true;
 }
 

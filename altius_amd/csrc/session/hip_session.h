@@ -52,12 +52,29 @@ private:
     size_t allocations_ = 0;
 };
 
+// A block of pooled device memory; goes back to its pool when the last tensor using it is dropped.
+struct DeviceBlock {
+    BufferPool *pool = nullptr;
+    void *ptr = nullptr;
+    size_t bucket = 0;
+    DeviceBlock() = default;
+    DeviceBlock(const DeviceBlock &) = delete;
+    DeviceBlock &operator=(const DeviceBlock &) = delete;
+    ~DeviceBlock() {
+        if (pool && ptr) pool->release(ptr, bucket);
+    }
+};
+
 struct DeviceTensor {
     FixedDimensions dims;
     TensorElemType elem_ty = TensorElemType::F32;
     void *ptr = nullptr;
-    size_t bucket = 0;    // pool bucket, 0 when not pooled
-    bool pooled = false;  // owned by the run (returned to the pool when freed)
+    // Keeps the memory alive.  Reshape / Flatten / Squeeze / Unsqueeze / Identity outputs share
+    // their input's block (the reference shares the buffer the same way, tensor.rs:340-342).
+    std::shared_ptr<DeviceBlock> block;
+    // The contents on the host, when they are known there: initializers and the small integer
+    // tensors of shape arithmetic.  Shape inference and the host evaluator read these.
+    std::shared_ptr<const Tensor> host;
     size_t nbytes() const { return dims.total_elems() * elem_size(elem_ty); }
 };
 
@@ -86,7 +103,14 @@ private:
     HipSession() = default;
 
     bool run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, SessionError *err);
-    void release(DeviceTensor &t);
+    // A fresh pooled tensor of the given shape (contents unspecified).
+    bool allocate(const TypedFixedShape &shape, DeviceTensor *out, SessionError *err);
+    // Uploads a host tensor into a fresh pooled tensor that remembers its host contents.
+    bool upload(const Tensor &t, DeviceTensor *out, SessionError *err);
+    // Makes t.host available by reading a small tensor back (synchronises the stream).
+    bool fetch_host(DeviceTensor *t, SessionError *err);
+    bool run_device_op(const Node &node, const Op &op, const std::vector<DeviceTensor *> &in,
+                       const std::vector<TypedFixedShape> &shapes, std::vector<DeviceTensor> *outs, SessionError *err);
 
     Model model_;
     std::vector<NodeExecutionPlan> plan_;

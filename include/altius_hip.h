@@ -141,7 +141,8 @@ enum ahip_unary_op {
     AHIP_LEAKYRELU = 7,   /* compute_leaky_relu, session.rs:814-821 (alpha) */
     AHIP_EXP = 8,         /* no reference kernel (session.rs:224): expf */
     AHIP_ROUND = 9,       /* no reference kernel (session.rs:219-223): round half to even (ONNX Round) */
-    AHIP_CLIP = 10        /* no reference kernel (session.rs:201): clamp to [alpha, beta] (ONNX Clip) */
+    AHIP_CLIP = 10,       /* no reference kernel (session.rs:201): clamp to [alpha, beta] (ONNX Clip) */
+    AHIP_DIV_BY = 11      /* x / alpha: the division by H*W of compute_gavg_pool (session.rs:291) */
 };
 
 /* Flat element-wise op over n elements.  alpha/beta are read by HardSigmoid (alpha, beta),
