@@ -104,6 +104,59 @@ __global__ __launch_bounds__(BLOCK) void transpose_tiled(T *__restrict__ out, co
     }
 }
 
+// Batched transpose of small matrices that are contiguous on both sides (attention's K^T:
+// [.., 197, 64] -> [.., 64, 197]).  One block moves one whole r_len x c_len matrix: it reads the
+// matrix as one contiguous span, scatters it into LDS transposed, and writes the result as one
+// contiguous span, so both global sides run at full 16-byte width whatever the extents are.
+// The LDS row pitch is odd, which keeps the transposed stores conflict-free.
+template <class T, int VEC>
+__global__ __launch_bounds__(BLOCK) void transpose_small(T *__restrict__ out, const T *__restrict__ in, uint32_t r_len,
+                                                         uint32_t c_len, uint32_t pitch, FastDiv cdiv, FastDiv rdiv) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T *lds = reinterpret_cast<T *>(smem_raw);  // [c_len][pitch], element (c, r) at c * pitch + r
+    const uint32_t n = r_len * c_len;
+    const T *src = in + (size_t)blockIdx.x * n;
+    T *dst = out + (size_t)blockIdx.x * n;
+    for (uint32_t i = threadIdx.x * VEC; i < n; i += BLOCK * VEC) {
+        T v[VEC];
+        if (VEC == 4) {
+            const uint4 t = *reinterpret_cast<const uint4 *>(src + i);
+            v[0] = (T)t.x; v[1 % VEC] = (T)t.y; v[2 % VEC] = (T)t.z; v[3 % VEC] = (T)t.w;
+        } else {
+            v[0] = src[i];
+        }
+        uint32_t r = cdiv.div(i), c = i - r * c_len;  // input is [r][c]
+#pragma unroll
+        for (int k = 0; k < VEC; k++) {
+            lds[c * pitch + r] = v[k];
+            if (++c == c_len) {
+                c = 0;
+                r++;
+            }
+        }
+    }
+    __syncthreads();
+    for (uint32_t i = threadIdx.x * VEC; i < n; i += BLOCK * VEC) {
+        uint32_t c = rdiv.div(i), r = i - c * r_len;  // output is [c][r]
+        T v[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; k++) {
+            v[k] = lds[c * pitch + r];
+            if (++r == r_len) {
+                r = 0;
+                c++;
+            }
+        }
+        if (VEC == 4) {
+            uint4 t;
+            t.x = (uint32_t)v[0]; t.y = (uint32_t)v[1 % VEC]; t.z = (uint32_t)v[2 % VEC]; t.w = (uint32_t)v[3 % VEC];
+            *reinterpret_cast<uint4 *>(dst + i) = t;
+        } else {
+            dst[i] = v[0];
+        }
+    }
+}
+
 // ---- gather ----------------------------------------------------------------------------------
 // out[o, j, :] = data[o, idx[j], :] with `inner` contiguous elements per row; negative indices
 // count from the end (ONNX).  Out-of-range indices read row 0 and raise the flag in *bad.
@@ -406,6 +459,44 @@ int launch_transpose(DeviceCtx &ctx, void *out, const void *in, int elem_size, i
         g.b_out_str[g.brank] = (uint32_t)so[i];
         g.brank++;
         batches *= (size_t)d[i];
+    }
+    // A short R or C axis wastes most of a 64 x 64 tile; one element per thread in output order
+    // keeps the writes dense and the reads in runs of r_len-strided segments.
+    if (g.r_len < 16 || g.c_len < 16)
+        return launch_copy_strided(ctx, out, in, elem_size, (int)d.size(), d.data(), so.data(), si.data());
+    // Whole small matrices, contiguous on both sides: one block each through LDS.
+    {
+        const size_t n = (size_t)g.r_len * g.c_len;
+        const uint32_t pitch = g.r_len | 1u;
+        const size_t lds_bytes = (size_t)g.c_len * pitch * (size_t)elem_size;
+        if (g.r_in_str == g.c_len && g.c_out_str == g.r_len && lds_bytes <= 64 * 1024 && n >= 1024 && batches <= 0x7fffffffull) {
+            // every other axis must step over whole matrices: true by construction after collapsing
+            // when C and R are the two innermost axes of both sides
+            bool whole = c_axis + 2 == d.size();
+            size_t expect = n;
+            for (size_t i = c_axis; whole && i-- > 0;) {
+                whole = si[i] == (int64_t)expect && so[i] == (int64_t)expect;
+                expect *= (size_t)d[i];
+            }
+            if (whole) {
+                const FastDiv cdiv = make_fastdiv(g.c_len), rdiv = make_fastdiv(g.r_len);
+                const dim3 grid((unsigned)batches);
+                const bool vec = elem_size == 4 && n % 4 == 0 && aligned16(out) && aligned16(in);
+                if (elem_size == 4 && vec)
+                    hipLaunchKernelGGL((transpose_small<uint32_t, 4>), grid, dim3(BLOCK), lds_bytes, ctx.stream,
+                                       static_cast<uint32_t *>(out), static_cast<const uint32_t *>(in), g.r_len, g.c_len, pitch, cdiv, rdiv);
+                else if (elem_size == 4)
+                    hipLaunchKernelGGL((transpose_small<uint32_t, 1>), grid, dim3(BLOCK), lds_bytes, ctx.stream,
+                                       static_cast<uint32_t *>(out), static_cast<const uint32_t *>(in), g.r_len, g.c_len, pitch, cdiv, rdiv);
+                else if (elem_size == 8)
+                    hipLaunchKernelGGL((transpose_small<uint64_t, 1>), grid, dim3(BLOCK), lds_bytes, ctx.stream,
+                                       static_cast<uint64_t *>(out), static_cast<const uint64_t *>(in), g.r_len, g.c_len, pitch, cdiv, rdiv);
+                else
+                    hipLaunchKernelGGL((transpose_small<uint8_t, 1>), grid, dim3(BLOCK), lds_bytes, ctx.stream,
+                                       static_cast<uint8_t *>(out), static_cast<const uint8_t *>(in), g.r_len, g.c_len, pitch, cdiv, rdiv);
+                return ctx.check(hipGetLastError(), "transpose_small launch");
+            }
+        }
     }
     const size_t gx = (g.c_len + TILE - 1) / TILE, gy = (g.r_len + TILE - 1) / TILE;
     if (gy > 65535 || batches > 65535) {
