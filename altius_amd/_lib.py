@@ -76,6 +76,8 @@ def _declare(L):
     f("ahip_cast", [c_void_p, c_void_p, c_void_p, c_int, c_int, c_size_t])
     f("ahip_batchnorm", [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t,
                          c_float])
+    f("ahip_gemm", [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p] + [c_size_t] * 4 + [c_int, c_int] + [c_size_t] * 8
+      + [c_float, c_float])
     f("ahip_module_load", [c_void_p, c_void_p, c_size_t, P(c_void_p)])
     f("ahip_module_unload", [c_void_p, c_void_p])
     f("ahip_launch", [c_void_p, c_void_p, c_char_p, P(ctypes.c_uint32), P(ctypes.c_uint32), ctypes.c_uint32,

@@ -354,4 +354,13 @@ int ahip_batchnorm(ahip_ctx *ctx, float *out, const float *x, const float *scale
     return altius::launch_batchnorm(ctx->d, out, x, scale, bias, mean, var, n, c, hw, epsilon);
 }
 
+int ahip_gemm(ahip_ctx *ctx, float *c, const float *a, const float *b, const float *c0, size_t batch, size_t m, size_t n,
+              size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t a_batch_stride,
+              size_t b_batch_stride, size_t c_batch_stride, size_t c0_row_stride, size_t c0_col_stride, float alpha,
+              float beta) {
+    REQUIRE_CTX(ctx, "ahip_gemm");
+    return altius::launch_gemm(ctx->d, c, a, b, c0, batch, m, n, k, trans_a, trans_b, lda, ldb, ldc, a_batch_stride,
+                               b_batch_stride, c_batch_stride, c0_row_stride, c0_col_stride, alpha, beta);
+}
+
 }  // extern "C"

@@ -75,4 +75,13 @@ int launch_cast(DeviceCtx &ctx, void *out, const void *in, int from_type, int to
 int launch_batchnorm(DeviceCtx &ctx, float *out, const float *x, const float *scale, const float *bias, const float *mean,
                      const float *var, size_t n, size_t c, size_t hw, float eps);
 
+// C[b] = alpha * op(A[b]) * op(B[b]) + beta * C0 for b in [0, batch) (matmul.hip).  op(X) is X or its
+// transpose; lda / ldb / ldc are row pitches of the stored matrices; batch strides in elements
+// (0 = one matrix shared by all batches); C0 may be null, and is read at
+// c0[i * c0_row_stride + j * c0_col_stride] (strides of 0 broadcast a row vector or a scalar).
+int launch_gemm(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t batch, size_t m, size_t n,
+                size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t a_batch_stride,
+                size_t b_batch_stride, size_t c_batch_stride, size_t c0_row_stride, size_t c0_col_stride, float alpha,
+                float beta);
+
 }  // namespace altius

@@ -1,0 +1,228 @@
+// fp32 matrix multiplication on the matrix cores: C = alpha * op(A) * op(B) + beta * C0, batched
+// with broadcast batch strides.  Counterparts in the reference: compute_mat_mul
+// (crates/session_interpreter/src/session.rs:621-684) and compute_gemm (686-794), both of which
+// call sgemm (crates/session_interpreter/src/gemm.rs: the `matrixmultiply` crate or CBLAS).
+//
+// This is the one MFMA-bound kernel of the library.  A 256-thread block (4 wavefronts in a 2 x 2
+// grid) owns a 128 x 128 tile of C; each wavefront accumulates a 64 x 64 sub-tile in four
+// 32 x 32 accumulators with v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate: 256 flop per cycle
+// per CU, 157 Tflop/s on the part).  K advances 16 at a time through double-buffered LDS tiles
+// stored k-major ([k][m] and [k][n], pitch 132 floats) so that a fragment read is 32 consecutive
+// floats per half-wave and the transposing store of a k-contiguous operand spreads over all banks.
+// The global loads of tile t+1 are issued before the MFMA loop of tile t and land in LDS after it:
+// one barrier per K tile.
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "ctx.h"
+
+namespace altius {
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128, BN = 128, BK = 16;
+constexpr int PITCH = BM + 4;  // floats; (4k + m) mod 64 is a bijection over a transposing store's lanes
+constexpr int THREADS = 256;
+
+struct GemmArgs {
+    const float *a, *b, *c0;
+    float *c;
+    uint32_t m, n, k;
+    // Element (i, kk) of op(A) is a[i * a_rs + kk * a_cs]; (kk, j) of op(B) is b[kk * b_rs + j * b_cs].
+    // One of the two strides of each operand is 1.
+    uint32_t a_rs, a_cs, b_rs, b_cs;
+    uint32_t ldc;
+    // C0 (Gemm's third input) is read as c0[i * c0_rs + j * c0_cs]; either stride may be 0.
+    uint32_t c0_rs, c0_cs;
+    uint64_t a_bs, b_bs, c_bs;  // batch strides in elements (0 = shared by every batch)
+    float alpha, beta;
+    int a_vec, b_vec;  // 16-byte loads are legal for this operand (alignment of base, strides, batch stride)
+};
+
+// Loads this thread's share of a BK x 128 operand tile into registers.
+// K_CONTIG: the operand's k axis is the contiguous one (A without transA, B with transB).
+// `mn` is the tile's first row (A) or column (B), `lim` the extent of that axis.
+template <bool K_CONTIG>
+__device__ __forceinline__ void load_tile(float4 (&r)[2], const float *__restrict__ p, uint32_t mn0, uint32_t lim,
+                                          uint32_t k0, uint32_t kdim, uint32_t s_mn, uint32_t s_k, int vec, int tid) {
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int f = tid + THREADS * u;
+        uint32_t mn, kk;
+        if (K_CONTIG) {  // 128 rows of 16 floats: 4 float4 per row
+            mn = mn0 + (f >> 2);
+            kk = k0 + ((f & 3) << 2);
+        } else {  // 16 rows of 128 floats: 32 float4 per row
+            kk = k0 + (f >> 5);
+            mn = mn0 + ((f & 31) << 2);
+        }
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (K_CONTIG) {
+            if (mn < lim) {
+                const float *q = p + (size_t)mn * s_mn + kk;
+                if (vec && kk + 3 < kdim) {
+                    v = *reinterpret_cast<const float4 *>(q);
+                } else {
+                    if (kk < kdim) v.x = q[0];
+                    if (kk + 1 < kdim) v.y = q[1];
+                    if (kk + 2 < kdim) v.z = q[2];
+                    if (kk + 3 < kdim) v.w = q[3];
+                }
+            }
+        } else {
+            if (kk < kdim) {
+                const float *q = p + (size_t)kk * s_k + mn;
+                if (vec && mn + 3 < lim) {
+                    v = *reinterpret_cast<const float4 *>(q);
+                } else {
+                    if (mn < lim) v.x = q[0];
+                    if (mn + 1 < lim) v.y = q[1];
+                    if (mn + 2 < lim) v.z = q[2];
+                    if (mn + 3 < lim) v.w = q[3];
+                }
+            }
+        }
+        r[u] = v;
+    }
+}
+
+// Stores the registers into the k-major LDS tile [BK][PITCH].
+template <bool K_CONTIG> __device__ __forceinline__ void store_tile(float *__restrict__ t, const float4 (&r)[2], int tid) {
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int f = tid + THREADS * u;
+        if (K_CONTIG) {
+            const int mn = f >> 2, kk = (f & 3) << 2;
+            t[(kk + 0) * PITCH + mn] = r[u].x;
+            t[(kk + 1) * PITCH + mn] = r[u].y;
+            t[(kk + 2) * PITCH + mn] = r[u].z;
+            t[(kk + 3) * PITCH + mn] = r[u].w;
+        } else {
+            const int kk = f >> 5, mn = (f & 31) << 2;
+            *reinterpret_cast<float4 *>(t + kk * PITCH + mn) = r[u];
+        }
+    }
+}
+
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(THREADS) void gemm_f32_mfma(GemmArgs g) {
+    __shared__ __align__(16) float As[2][BK * PITCH];
+    __shared__ __align__(16) float Bs[2][BK * PITCH];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const float *a = g.a + (size_t)blockIdx.z * g.a_bs;
+    const float *b = g.b + (size_t)blockIdx.z * g.b_bs;
+    // Strides of the tile's mn axis and k axis for each operand.
+    const uint32_t a_smn = g.a_rs, a_sk = g.a_cs, b_smn = g.b_cs, b_sk = g.b_rs;
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    float4 ra[2], rb[2];
+    load_tile<A_KC>(ra, a, m0, g.m, 0, g.k, a_smn, a_sk, g.a_vec, tid);
+    load_tile<B_KC>(rb, b, n0, g.n, 0, g.k, b_smn, b_sk, g.b_vec, tid);
+    store_tile<A_KC>(As[0], ra, tid);
+    store_tile<B_KC>(Bs[0], rb, tid);
+    __syncthreads();
+
+    const uint32_t nk = (g.k + BK - 1) / BK;
+    const int lr = lane & 31, lk = lane >> 5;
+    for (uint32_t kt = 0; kt < nk; kt++) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < nk;
+        if (more) {
+            load_tile<A_KC>(ra, a, m0, g.m, (kt + 1) * BK, g.k, a_smn, a_sk, g.a_vec, tid);
+            load_tile<B_KC>(rb, b, n0, g.n, (kt + 1) * BK, g.k, b_smn, b_sk, g.b_vec, tid);
+        }
+        const float *at = As[cur] + wm * 64 + lr;
+        const float *bt = Bs[cur] + wn * 64 + lr;
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 2) {
+            const float a0 = at[(kk + lk) * PITCH], a1 = at[(kk + lk) * PITCH + 32];
+            const float b0 = bt[(kk + lk) * PITCH], b1 = bt[(kk + lk) * PITCH + 32];
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+        }
+        if (more) {
+            store_tile<A_KC>(As[cur ^ 1], ra, tid);
+            store_tile<B_KC>(Bs[cur ^ 1], rb, tid);
+        }
+        __syncthreads();
+    }
+
+    // Accumulator r of lane l is C[8 * (r / 4) + 4 * (l / 32) + r % 4][l % 32] of its 32 x 32 tile.
+    float *c = g.c + (size_t)blockIdx.z * g.c_bs;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const uint32_t col = n0 + wn * 64 + j * 32 + lr;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const uint32_t row = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * lk + (r & 3);
+                if (row < g.m && col < g.n) {
+                    float v = g.alpha * acc[i][j][r];
+                    if (g.c0) v += g.beta * g.c0[(size_t)row * g.c0_rs + (size_t)col * g.c0_cs];
+                    c[(size_t)row * g.ldc + col] = v;
+                }
+            }
+        }
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+
+int launch_gemm(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t batch, size_t m, size_t n,
+                size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t a_batch_stride,
+                size_t b_batch_stride, size_t c_batch_stride, size_t c0_row_stride, size_t c0_col_stride, float alpha,
+                float beta) {
+    if (batch == 0 || m == 0 || n == 0) return AHIP_OK;
+    if (!c || (k && (!a || !b))) return ctx.fail(AHIP_ERR_ARG, "gemm: null pointer");
+    const size_t lim = (size_t)1 << 31;
+    if (m >= lim || n >= lim || k >= lim || lda >= lim || ldb >= lim || ldc >= lim || m * ldc >= ((size_t)1 << 40))
+        return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm: extent above 2^31");
+    const size_t gy = (m + BM - 1) / BM, gx = (n + BN - 1) / BN;
+    if (gy > 65535 || batch > 65535) return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm: more than 65535 row tiles or batches");
+    GemmArgs g;
+    g.a = a;
+    g.b = b;
+    g.c0 = (c0 && beta != 0.0f) ? c0 : nullptr;
+    g.c = c;
+    g.m = (uint32_t)m;
+    g.n = (uint32_t)n;
+    g.k = (uint32_t)k;
+    g.a_rs = trans_a ? 1u : (uint32_t)lda;
+    g.a_cs = trans_a ? (uint32_t)lda : 1u;
+    g.b_rs = trans_b ? 1u : (uint32_t)ldb;
+    g.b_cs = trans_b ? (uint32_t)ldb : 1u;
+    g.ldc = (uint32_t)ldc;
+    g.c0_rs = (uint32_t)c0_row_stride;
+    g.c0_cs = (uint32_t)c0_col_stride;
+    g.a_bs = a_batch_stride;
+    g.b_bs = b_batch_stride;
+    g.c_bs = c_batch_stride;
+    g.alpha = alpha;
+    g.beta = beta;
+    g.a_vec = aligned16(a) && lda % 4 == 0 && a_batch_stride % 4 == 0;
+    g.b_vec = aligned16(b) && ldb % 4 == 0 && b_batch_stride % 4 == 0;
+    const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch);
+    const bool a_kc = !trans_a, b_kc = trans_b != 0;
+    if (a_kc && b_kc) hipLaunchKernelGGL((gemm_f32_mfma<true, true>), grid, dim3(THREADS), 0, ctx.stream, g);
+    else if (a_kc) hipLaunchKernelGGL((gemm_f32_mfma<true, false>), grid, dim3(THREADS), 0, ctx.stream, g);
+    else if (b_kc) hipLaunchKernelGGL((gemm_f32_mfma<false, true>), grid, dim3(THREADS), 0, ctx.stream, g);
+    else hipLaunchKernelGGL((gemm_f32_mfma<false, false>), grid, dim3(THREADS), 0, ctx.stream, g);
+    return ctx.check(hipGetLastError(), "gemm launch");
+}
+
+}  // namespace altius

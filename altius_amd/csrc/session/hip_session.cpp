@@ -729,6 +729,43 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
         if (!need(1)) return false;
         rc = launch_cast(ctx_, out.ptr, in[0]->ptr, (int)in[0]->elem_ty, (int)out.elem_ty, n_out);
         break;
+    case OpKind::MatMul: {  // compute_mat_mul (session.rs:621-684), with NumPy broadcasting of the batch axes
+        if (!need(2) || !need_f32({0, 1})) return false;
+        const FixedDimensions &a = in[0]->dims, &b = in[1]->dims;
+        const size_t m = a[a.len() - 2], k = a[a.len() - 1], n = b[b.len() - 1];
+        size_t a_batch = 1, b_batch = 1, batch = 1;
+        for (size_t i = 0; i + 2 < a.len(); i++) a_batch *= a[i];
+        for (size_t i = 0; i + 2 < b.len(); i++) b_batch *= b[i];
+        for (size_t i = 0; i + 2 < out.dims.len(); i++) batch *= out.dims[i];
+        if (b_batch == 1 && a_batch == batch) {
+            // [.., m, k] x [k, n]: one tall sgemm, as the reference does (session.rs:653-660)
+            rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), nullptr, 1, batch * m, n, k, 0, 0, k, n, n, 0, 0, 0, 0, 0, 1.0f, 0.0f);
+        } else if ((a_batch == batch || a_batch == 1) && (b_batch == batch || b_batch == 1)) {
+            rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), nullptr, batch, m, n, k, 0, 0, k, n, n, a_batch == 1 ? 0 : m * k,
+                             b_batch == 1 ? 0 : k * n, m * n, 0, 0, 1.0f, 0.0f);
+        } else {
+            return fail(err, SessionError::Message, "MatMul: batch axes that broadcast against each other partially are not supported");
+        }
+        break;
+    }
+    case OpKind::Gemm: {  // compute_gemm (session.rs:686-794)
+        if (!need(2) || !need_f32({0, 1})) return false;
+        const FixedDimensions &a = in[0]->dims, &b = in[1]->dims;
+        const size_t m = op.trans_a ? a[1] : a[0], k = op.trans_a ? a[0] : a[1], n = op.trans_b ? b[0] : b[1];
+        const float *c0 = nullptr;
+        size_t rs = 0, cs = 0;
+        if (in.size() > 2 && in[2]) {
+            if (in[2]->elem_ty != TensorElemType::F32) return fail(err, SessionError::Message, "Gemm: C must be f32");
+            auto st = in[2]->dims.strides_for_broadcasting_to(out.dims);
+            if (!st) return fail(err, SessionError::Shape, "Gemm: C does not broadcast to the output");
+            rs = (*st)[0];
+            cs = (*st)[1];
+            c0 = f(in[2]);
+        }
+        rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), c0, 1, m, n, k, op.trans_a, op.trans_b, a[1], b[1], n, 0, 0, 0, rs, cs, op.alpha,
+                         c0 ? op.beta : 0.0f);
+        break;
+    }
     default: return fail(err, SessionError::Message, opname + ": Kernel not implemented");
     }
     if (rc) return fail_code(err, rc, ctx_.last_error);

@@ -346,3 +346,59 @@ class Context:
         finally:
             for b in bufs + [do]:
                 self.free(b)
+
+    # --- matrix multiplication -------------------------------------------------------------------
+    def gemm_raw(self, c_ptr, a_ptr, b_ptr, c0_ptr, batch, m, n, k, trans_a=False, trans_b=False, lda=None, ldb=None,
+                 ldc=None, a_bs=0, b_bs=0, c_bs=0, c0_rs=0, c0_cs=0, alpha=1.0, beta=0.0):
+        lda = lda if lda is not None else (m if trans_a else k)
+        ldb = ldb if ldb is not None else (k if trans_b else n)
+        ldc = ldc if ldc is not None else n
+        check(self.L.ahip_gemm(self.handle, c_ptr, a_ptr, b_ptr, c0_ptr, batch, m, n, k, int(trans_a), int(trans_b), lda,
+                               ldb, ldc, a_bs, b_bs, c_bs, c0_rs, c0_cs, alpha, beta), self.handle)
+
+    def matmul(self, a, b):
+        """numpy.matmul semantics for operands of rank >= 2 (batch axes broadcast)."""
+        a = np.asarray(a, dtype=np.float32, order="C")
+        b = np.asarray(b, dtype=np.float32, order="C")
+        m, k, n = a.shape[-2], a.shape[-1], b.shape[-1]
+        batch_shape = np.broadcast_shapes(a.shape[:-2], b.shape[:-2])
+        batch = int(np.prod(batch_shape, dtype=np.int64))
+        # batched operands are made dense over the broadcast batch unless they are a single shared matrix
+        def prep(x):
+            if x.ndim == 2 or int(np.prod(x.shape[:-2], dtype=np.int64)) == 1:
+                return np.ascontiguousarray(x.reshape(x.shape[-2:])), 0
+            full = np.ascontiguousarray(np.broadcast_to(x, batch_shape + x.shape[-2:]))
+            return full, x.shape[-2] * x.shape[-1]
+        a2, a_bs = prep(a)
+        b2, b_bs = prep(b)
+        da, db = self.upload(a2), self.upload(b2)
+        dc = self.alloc(max(batch * m * n * 4, 4))
+        try:
+            self.gemm_raw(dc.ptr, da.ptr, db.ptr, None, batch, m, n, k, a_bs=a_bs, b_bs=b_bs, c_bs=m * n)
+            return self.download(dc, batch_shape + (m, n))
+        finally:
+            for x in (da, db, dc):
+                self.free(x)
+
+    def gemm(self, a, b, c=None, alpha=1.0, beta=1.0, trans_a=False, trans_b=False):
+        a = np.asarray(a, dtype=np.float32, order="C")
+        b = np.asarray(b, dtype=np.float32, order="C")
+        m, k = (a.shape[1], a.shape[0]) if trans_a else a.shape
+        n = b.shape[0] if trans_b else b.shape[1]
+        da, db = self.upload(a), self.upload(b)
+        dc0, rs, cs = None, 0, 0
+        if c is not None:
+            c = np.asarray(c, dtype=np.float32, order="C")
+            dc0 = self.upload(c)
+            if c.ndim == 2:
+                rs, cs = (c.shape[1] if c.shape[0] != 1 else 0), (1 if c.shape[1] != 1 else 0)
+            elif c.ndim == 1:
+                rs, cs = 0, (1 if c.shape[0] != 1 else 0)
+        dout = self.alloc(max(m * n * 4, 4))
+        try:
+            self.gemm_raw(dout.ptr, da.ptr, db.ptr, dc0.ptr if dc0 else None, 1, m, n, k, trans_a, trans_b, c0_rs=rs,
+                          c0_cs=cs, alpha=alpha, beta=beta)
+            return self.download(dout, (m, n))
+        finally:
+            for x in (da, db, dout) + ((dc0,) if dc0 else ()):
+                self.free(x)

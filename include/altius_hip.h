@@ -206,6 +206,18 @@ int ahip_cast(ahip_ctx *ctx, void *out, const void *in, int from_elem_type, int 
 int ahip_batchnorm(ahip_ctx *ctx, float *out, const float *x, const float *scale, const float *bias, const float *mean,
                    const float *var, size_t n, size_t c, size_t hw, float epsilon);
 
+/* C[b] = alpha * op(A[b]) * op(B[b]) + beta * C0, b in [0, batch): sgemm as compute_mat_mul and
+ * compute_gemm call it (crates/session_interpreter/src/session.rs:621-794, gemm.rs:3-52), on the
+ * matrix cores in fp32.  op(X) = X or its transpose (trans_a / trans_b); A is stored m x k (k x m
+ * when transposed) with row pitch lda, B k x n (n x k) with row pitch ldb, C m x n with row pitch
+ * ldc.  Batch strides are in elements; 0 shares one matrix between all batches (MatMul of
+ * [b, m, k] by [k, n]).  c0 may be NULL; it is read at c0[i * c0_row_stride + j * c0_col_stride],
+ * so (0, 1) broadcasts a bias row and (n, 1) reads a full matrix (Gemm's third input). */
+int ahip_gemm(ahip_ctx *ctx, float *c, const float *a, const float *b, const float *c0, size_t batch, size_t m,
+              size_t n, size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t a_batch_stride,
+              size_t b_batch_stride, size_t c_batch_stride, size_t c0_row_stride, size_t c0_col_stride, float alpha,
+              float beta);
+
 /* ------------------------------------------------------------------------
  * Graph IR: the same Model / Graph / Node / Value / Op structure as
  * altius_core (crates/core/src/model.rs:13-17, graph.rs:9-16, node.rs:7-14,

@@ -337,3 +337,36 @@ def leaky_relu(x, alpha=0.01):
     if rc != OK:
         raise OracleError(rc, "leaky_relu")
     return out
+
+
+def matmul(a, b):
+    """compute_mat_mul (session.rs:621-684): numpy.matmul shapes, one sgemm per batch item."""
+    a, b = _f32(a), _f32(b)
+    m, k, n = a.shape[-2], a.shape[-1], b.shape[-1]
+    batch_shape = np.broadcast_shapes(a.shape[:-2], b.shape[:-2])
+    af = np.ascontiguousarray(np.broadcast_to(a, batch_shape + (m, k))).reshape(-1, m, k)
+    bf = np.ascontiguousarray(np.broadcast_to(b, batch_shape + (k, n))).reshape(-1, k, n)
+    out = np.zeros((af.shape[0], m, n), dtype=np.float32)
+    sz = ctypes.c_size_t
+    for i in range(af.shape[0]):
+        rc = lib().orc_sgemm(0, 0, sz(m), sz(k), sz(n), ctypes.c_float(1.0), _fptr(af[i]), sz(k), _fptr(bf[i]), sz(n),
+                             ctypes.c_float(0.0), _fptr(out[i]), sz(n))
+        if rc != OK:
+            raise OracleError(rc, "matmul")
+    return out.reshape(batch_shape + (m, n))
+
+
+def gemm(a, b, c=None, alpha=1.0, beta=1.0, trans_a=False, trans_b=False):
+    """compute_gemm (session.rs:686-794): C is copied (bias rows repeated) into the output, then sgemm."""
+    a, b = _f32(a), _f32(b)
+    m, k = (a.shape[1], a.shape[0]) if trans_a else a.shape
+    n = b.shape[0] if trans_b else b.shape[1]
+    out = np.zeros((m, n), dtype=np.float32)
+    if c is not None:
+        out[:] = np.broadcast_to(_f32(c), (m, n))
+    sz = ctypes.c_size_t
+    rc = lib().orc_sgemm(int(trans_a), int(trans_b), sz(m), sz(k), sz(n), ctypes.c_float(alpha), _fptr(a), sz(a.shape[1]),
+                         _fptr(b), sz(b.shape[1]), ctypes.c_float(beta if c is not None else 0.0), _fptr(out), sz(n))
+    if rc != OK:
+        raise OracleError(rc, "gemm")
+    return out

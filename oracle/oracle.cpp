@@ -1068,6 +1068,32 @@ int orc_leaky_relu(const float *x, float *out, size_t n, float alpha) {
     return ORC_OK;
 }
 
+int orc_sgemm(int trans_a, int trans_b, size_t m, size_t k, size_t n, float alpha, const float *a, size_t lda,
+              const float *b, size_t ldb, float beta, float *c, size_t ldc) {
+    const size_t KC = 256;
+    if (k == 0) {
+        for (size_t i = 0; i < m; i++)
+            for (size_t j = 0; j < n; j++) c[i * ldc + j] = beta == 0.0f ? 0.0f : beta * c[i * ldc + j];
+        return ORC_OK;
+    }
+    for (size_t k0 = 0; k0 < k; k0 += KC) {
+        const size_t k1 = std::min(k, k0 + KC);
+        const float bt = k0 == 0 ? beta : 1.0f;
+        for (size_t i = 0; i < m; i++)
+            for (size_t j = 0; j < n; j++) {
+                float ab = 0.0f;
+                for (size_t p = k0; p < k1; p++) {
+                    const float av = trans_a ? a[p * lda + i] : a[i * lda + p];
+                    const float bv = trans_b ? b[j * ldb + p] : b[p * ldb + j];
+                    ab = std::fma(av, bv, ab);
+                }
+                float &cv = c[i * ldc + j];
+                cv = bt == 0.0f ? alpha * ab : bt * cv + alpha * ab;
+            }
+    }
+    return ORC_OK;
+}
+
 float orc_fast_sum(const float *x, size_t n) { return fast_sum(x, n); }
 float orc_fast_sum_squares(const float *x, size_t n) { return fast_sum_squares(x, n); }
 

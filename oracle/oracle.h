@@ -166,6 +166,17 @@ int orc_global_average_pool(const float *x, float *out, size_t n, size_t c, size
 /* compute_leaky_relu (session.rs:814-821). */
 int orc_leaky_relu(const float *x, float *out, size_t n, float alpha);
 
+/* sgemm as compute_mat_mul / compute_gemm call it (session.rs:621-794 through gemm.rs:3-52):
+ * C = alpha * op(A) * op(B) + beta * C, row-major, C pre-filled by the caller (Gemm copies its
+ * third input in, session.rs:703-718).  The arithmetic lives in the `matrixmultiply` crate
+ * (0.3.10, Cargo.lock:1538-1541; not vendored) or CBLAS.  PARITY UNPINNED at the bit level: the
+ * order of accumulation restated here is the crate's published design (k in panels of 256, one
+ * fused multiply-add per product inside a panel, alpha and beta applied when a panel is added
+ * to C); the reference's own tests bound it by numpy.allclose against onnxruntime
+ * (test_ops_matmul.py:66, test_ops_gemm.py). */
+int orc_sgemm(int trans_a, int trans_b, size_t m, size_t k, size_t n, float alpha, const float *a, size_t lda,
+              const float *b, size_t ldb, float beta, float *c, size_t ldc);
+
 float orc_fast_sum(const float *x, size_t n);
 float orc_fast_sum_squares(const float *x, size_t n);
 

@@ -1,0 +1,154 @@
+"""MatMul / Gemm on the matrix cores, through the C ABI and the session.  The accumulation order of a
+GEMM is implementation-defined (the reference's own lives in the matrixmultiply crate), so parity is
+what the mathematics fixes: exact results on integer-valued operands, the forward error bound
+|C - exact| <= K * 2^-24 * |A||B| on random ones (and numpy.allclose, the reference's own test bar,
+against the oracle), every tile-edge case, transposes, alpha / beta / bias, batch broadcasting."""
+import numpy as np
+import pytest
+
+import oracle as O
+from altius_amd.graph import Model, Op
+from altius_amd.session import HipSessionBuilder
+from conftest import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+RNG = np.random.default_rng(31)
+
+
+def ints(*shape):
+    return RNG.integers(-4, 5, size=shape).astype(np.float32)
+
+
+def check_bound(got, a, b, what):
+    exact = np.matmul(a.astype(np.float64), b.astype(np.float64))
+    k = a.shape[-1]
+    bound = (k + 2) * 2.0 ** -24 * np.matmul(np.abs(a).astype(np.float64), np.abs(b).astype(np.float64)) + 1e-30
+    err = np.abs(got.astype(np.float64) - exact)
+    assert got.shape == exact.shape, f"{what}: shape {got.shape} vs {exact.shape}"
+    assert np.all(err <= bound), f"{what}: error {err.max():.3e} beyond the bound (worst ratio {np.max(err / bound):.2f})"
+    assert np.allclose(got, O.matmul(a, b), rtol=1e-5, atol=1e-5 * np.sqrt(k)), f"{what}: differs from the oracle"
+
+
+SHAPES = [((5, 10), (10, 15)), ((3, 5, 10), (10, 15)), ((3, 5, 10), (3, 10, 15)), ((1, 5, 10), (10, 15)),       # test_ops_matmul.py
+          ((128, 16), (16, 128)), ((129, 17), (17, 127)), ((1, 1), (1, 1)), ((64, 300), (300, 64)), ((257, 33), (33, 130)),
+          ((2, 197, 768), (768, 2304)), ((2, 12, 197, 64), (2, 12, 64, 197)), ((2, 12, 197, 197), (2, 12, 197, 64)),
+          ((1, 6, 3, 4), (1, 6, 4, 5)), ((7, 1, 9, 8), (8, 11)), ((4, 20, 31), (1, 31, 6)), ((300, 7), (7, 3))]
+
+
+@pytest.mark.parametrize("sa,sb", SHAPES)
+def test_matmul_exact_on_integers_and_bounded_on_reals(ctx, case, sa, sb):
+    case(f"matmul {sa} x {sb}")
+    a, b = ints(*sa), ints(*sb)
+    want = np.matmul(a.astype(np.float64), b.astype(np.float64)).astype(np.float32)
+    assert_bits_equal(ctx.matmul(a, b), want, "integer operands")
+    assert_bits_equal(O.matmul(a, b), want, "oracle agrees")
+    a, b = RNG.standard_normal(sa).astype(np.float32), RNG.standard_normal(sb).astype(np.float32)
+    check_bound(ctx.matmul(a, b), a, b, "random operands")
+
+
+def test_matmul_each_product_lands_in_its_place(ctx, case):
+    """Unit vectors pick single entries: C = A[:, p] (outer) B[q, :] catches a transposed or permuted fragment."""
+    case("matmul placement")
+    m, k, n = 70, 37, 90
+    a = np.zeros((m, k), np.float32)
+    b = np.zeros((k, n), np.float32)
+    a[:, 5] = np.arange(1, m + 1)
+    b[5, :] = np.arange(1, n + 1) * 1000
+    assert_bits_equal(ctx.matmul(a, b), np.outer(np.arange(1, m + 1), np.arange(1, n + 1) * 1000).astype(np.float32), "outer product")
+    eye = np.eye(150, dtype=np.float32)
+    x = RNG.standard_normal((150, 150)).astype(np.float32)
+    assert_bits_equal(ctx.matmul(eye, x), x, "identity on the left")
+    assert_bits_equal(ctx.matmul(x, eye), x, "identity on the right")
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_gemm(ctx, case, ta, tb):
+    case(f"gemm transA={ta} transB={tb}")
+    for m, k, n in [(5, 10, 15), (130, 70, 129), (64, 64, 64), (3, 1, 2)]:
+        a, b = ints(*((k, m) if ta else (m, k))), ints(*((n, k) if tb else (k, n)))
+        for c in (None, ints(n), ints(m, n), ints(1, n), ints(m, 1), ints(1)):
+            got = ctx.gemm(a, b, c, alpha=2.0, beta=3.0, trans_a=ta, trans_b=tb)
+            assert_bits_equal(got, O.gemm(a, b, c, alpha=2.0, beta=3.0, trans_a=ta, trans_b=tb), f"gemm {m}x{k}x{n} c={None if c is None else c.shape}")
+        ar, br = a + RNG.standard_normal(a.shape).astype(np.float32), b + RNG.standard_normal(b.shape).astype(np.float32)
+        got = ctx.gemm(ar, br, None, trans_a=ta, trans_b=tb)
+        check_bound(got, ar.T if ta else ar, br.T if tb else br, "random gemm")
+
+
+def test_unaligned_operands_take_the_scalar_loads(ctx, case):
+    case("gemm on unaligned pointers / odd pitches")
+    a, b = ints(33, 21), ints(21, 19)                 # pitches 21 and 19: no 16-byte rows
+    assert_bits_equal(ctx.matmul(a, b), a @ b, "odd pitches")
+    da = ctx.upload(np.concatenate([np.zeros(1, np.float32), ints(64 * 32)]))
+    db = ctx.upload(np.concatenate([np.zeros(3, np.float32), ints(32 * 48)]))
+    dc = ctx.alloc(64 * 48 * 4 + 4)
+    ctx.gemm_raw(dc.ptr + 4, da.ptr + 4, db.ptr + 12, None, 1, 64, 48, 32)
+    A = ctx.download(da, (64 * 32 + 1,))[1:].reshape(64, 32)
+    B = ctx.download(db, (32 * 48 + 3,))[3:].reshape(32, 48)
+    assert_bits_equal(ctx.download(dc, (64 * 48 + 1,))[1:].reshape(64, 48), A @ B, "offset bases")
+    for x in (da, db, dc):
+        ctx.free(x)
+
+
+def test_attention_block_through_the_session(case):
+    """LayerNorm -> qkv MatMul + bias -> split -> heads -> QK^T * scale -> Softmax -> PV -> merge -> proj + residual,
+    against the same chain on the oracle."""
+    case("session: one attention block")
+    B, T, H, NH = 2, 50, 64, 4
+    D = H // NH
+    x = RNG.standard_normal((B, T, H)).astype(np.float32)
+    g, be = RNG.standard_normal(H).astype(np.float32), RNG.standard_normal(H).astype(np.float32)
+    wqkv, bqkv = (RNG.standard_normal((H, 3 * H)) * 0.1).astype(np.float32), RNG.standard_normal(3 * H).astype(np.float32)
+    wo, bo = (RNG.standard_normal((H, H)) * 0.1).astype(np.float32), RNG.standard_normal(H).astype(np.float32)
+    m = Model(opset_version=13)
+    v = m.new_val_named_and_shaped("x", x.shape)
+    I = lambda a: m.new_initializer(np.asarray(a))
+    n = lambda: m.new_val()
+    ln, qkv, qkvb, q, k, vv = n(), n(), n(), n(), n(), n()
+    m.add_node(Op.LayerNormalization, [v, I(g), I(be)], [ln], axis=-1, epsilon=1e-5)
+    m.add_node(Op.MatMul, [ln, I(wqkv)], [qkv])
+    m.add_node(Op.Add, [qkv, I(bqkv)], [qkvb])
+    m.add_node(Op.Split, [qkvb, I(np.array([H, H, H], np.int64))], [q, k, vv], axis=2)
+    heads = []
+    for t in (q, k, vv):
+        r, tr = n(), n()
+        m.add_node(Op.Reshape, [t, I(np.array([B, T, NH, D], np.int64))], [r])
+        m.add_node(Op.Transpose, [r], [tr], perm=[0, 2, 1, 3])
+        heads.append(tr)
+    kt, s, ss, p, ctxv, ct, cm, proj, pb, y = (n() for _ in range(10))
+    m.add_node(Op.Transpose, [heads[1]], [kt], perm=[0, 1, 3, 2])
+    m.add_node(Op.MatMul, [heads[0], kt], [s])
+    m.add_node(Op.Mul, [s, I(np.array(1.0 / np.sqrt(D), np.float32))], [ss])
+    m.add_node(Op.Softmax, [ss], [p], axis=-1)
+    m.add_node(Op.MatMul, [p, heads[2]], [ctxv])
+    m.add_node(Op.Transpose, [ctxv], [ct], perm=[0, 2, 1, 3])
+    m.add_node(Op.Reshape, [ct, I(np.array([B, T, H], np.int64))], [cm])
+    m.add_node(Op.MatMul, [cm, I(wo)], [proj])
+    m.add_node(Op.Add, [proj, I(bo)], [pb])
+    m.add_node(Op.Add, [v, pb], [y])
+    m.add_input(v)
+    m.add_output(y)
+    (got,) = HipSessionBuilder(m).build().run([x])
+
+    l = O.layer_norm(x, g, be, 1e-5)
+    qkv_ = O.binary(O.ADD, O.matmul(l, wqkv), bqkv)
+    qh, kh, vh = (np.ascontiguousarray(t.reshape(B, T, NH, D).transpose(0, 2, 1, 3)) for t in np.split(qkv_, 3, axis=2))
+    sc = O.binary(O.MUL, O.matmul(qh, np.ascontiguousarray(kh.transpose(0, 1, 3, 2))), np.array(1.0 / np.sqrt(D), np.float32))
+    pr = O.softmax(sc)
+    cv = np.ascontiguousarray(O.matmul(pr, vh).transpose(0, 2, 1, 3)).reshape(B, T, H)
+    want = O.binary(O.ADD, x, O.binary(O.ADD, O.matmul(cv, wo), bo))
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
+
+
+def test_gemm_head_through_the_session(case):
+    case("session: Gemm classifier head")
+    x, w, b = RNG.standard_normal((8, 768)).astype(np.float32), (RNG.standard_normal((1000, 768)) * 0.05).astype(np.float32), ints(1000)
+    m = Model()
+    v = m.new_val_named_and_shaped("x", x.shape)
+    y = m.new_val()
+    m.add_node(Op.Gemm, [v, m.new_initializer(w), m.new_initializer(b)], [y], transB=1)
+    m.add_input(v)
+    m.add_output(y)
+    (got,) = HipSessionBuilder(m).build().run([x])
+    assert np.allclose(got, O.gemm(x, w, b, trans_b=True), rtol=1e-5, atol=1e-4)
+    check_bound(got - b, x, w.T, "gemm head")

@@ -481,3 +481,26 @@ def test_batchnorm_gavgpool_leakyrelu(oracle):
     got = oracle.leaky_relu(z, 0.1)
     assert np.array_equal(got[:4], np.array([np.float32(0.1) * np.float32(-2.0), -0.0, 0.0, 3.0], np.float32))
     assert np.isnan(got[4]) and got[5] == -np.inf and np.signbit(got[1])
+
+
+def test_sgemm_against_exact_products(oracle):
+    """Accumulation order is the unpinned part; what the mathematics fixes is checked: exact results on
+    integer-valued operands (every order gives the same sum), the forward error bound on random ones,
+    transposes as index swaps, alpha / beta / bias as in compute_gemm."""
+    rng = np.random.default_rng(9)
+    for shape_a, shape_b in [((5, 10), (10, 15)), ((3, 5, 10), (10, 15)), ((3, 5, 10), (3, 10, 15)), ((1, 4, 7, 300), (1, 4, 300, 9))]:
+        a = rng.integers(-4, 5, size=shape_a).astype(np.float32)
+        b = rng.integers(-4, 5, size=shape_b).astype(np.float32)
+        assert np.array_equal(oracle.matmul(a, b), np.matmul(a.astype(np.float64), b.astype(np.float64)).astype(np.float32))
+    a, b = rng.standard_normal((33, 700)).astype(np.float32), rng.standard_normal((700, 21)).astype(np.float32)
+    exact = a.astype(np.float64) @ b.astype(np.float64)
+    bound = 700 * 2.0 ** -24 * (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64))
+    assert np.all(np.abs(oracle.matmul(a, b) - exact) <= bound)
+    ai = rng.integers(-3, 4, size=(6, 4)).astype(np.float32)
+    bi = rng.integers(-3, 4, size=(5, 6)).astype(np.float32)
+    ci = rng.integers(-3, 4, size=(5,)).astype(np.float32)
+    want = 2.0 * (ai.T.astype(np.float64) @ bi.T.astype(np.float64)) + 3.0 * ci
+    assert np.array_equal(oracle.gemm(ai, bi, ci, alpha=2.0, beta=3.0, trans_a=True, trans_b=True), want.astype(np.float32))
+    full = rng.integers(-3, 4, size=(4, 5)).astype(np.float32)
+    assert np.array_equal(oracle.gemm(ai.T.copy(), bi.T.copy(), full), (ai.T @ bi.T + full))
+    assert np.array_equal(oracle.gemm(ai.T.copy(), bi.T.copy()), ai.T @ bi.T)         # no C: beta has nothing to scale
