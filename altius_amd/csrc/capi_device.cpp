@@ -363,4 +363,21 @@ int ahip_gemm(ahip_ctx *ctx, float *c, const float *a, const float *b, const flo
                                b_batch_stride, c_batch_stride, c0_row_stride, c0_col_stride, alpha, beta);
 }
 
+int ahip_conv2d(ahip_ctx *ctx, float *out, const float *x, const float *w, const float *bias, float *col, size_t batch,
+                size_t c, size_t ih, size_t iw, size_t oc, size_t oh, size_t ow, size_t kh, size_t kw, size_t stride_h,
+                size_t stride_w, size_t dilation_h, size_t dilation_w, size_t pad_top, size_t pad_left, size_t group) {
+    REQUIRE_CTX(ctx, "ahip_conv2d");
+    if (!kh || !kw || !stride_h || !stride_w || !dilation_h || !dilation_w)
+        return ctx->d.fail(AHIP_ERR_ARG, "ahip_conv2d: kernel, stride and dilation must be positive");
+    return altius::launch_conv2d(ctx->d, out, x, w, bias, col, batch, c, ih, iw, oc, oh, ow, kh, kw, stride_h, stride_w,
+                                 dilation_h, dilation_w, pad_top, pad_left, group);
+}
+
+int ahip_maxpool(ahip_ctx *ctx, float *out, const float *x, size_t planes, size_t ih, size_t iw, size_t oh, size_t ow,
+                 size_t kh, size_t kw, size_t stride_h, size_t stride_w, size_t pad_top, size_t pad_left) {
+    REQUIRE_CTX(ctx, "ahip_maxpool");
+    if (!kh || !kw || !stride_h || !stride_w) return ctx->d.fail(AHIP_ERR_ARG, "ahip_maxpool: kernel and stride must be positive");
+    return altius::launch_maxpool(ctx->d, out, x, planes, ih, iw, oh, ow, kh, kw, stride_h, stride_w, pad_top, pad_left);
+}
+
 }  // extern "C"

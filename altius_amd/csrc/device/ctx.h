@@ -84,4 +84,15 @@ int launch_gemm(DeviceCtx &ctx, float *c, const float *a, const float *b, const 
                 size_t b_batch_stride, size_t c_batch_stride, size_t c0_row_stride, size_t c0_col_stride, float alpha,
                 float beta);
 
+// col[b][c][fy][fx][oh][ow] for a convolution (movement.hip); maxpool over [planes, ih, iw].
+int launch_im2col(DeviceCtx &ctx, float *col, const float *x, size_t batch, size_t c, size_t ih, size_t iw, size_t oh,
+                  size_t ow, size_t kh, size_t kw, size_t sh, size_t sw, size_t dh, size_t dw, size_t pad_t, size_t pad_l);
+int launch_maxpool(DeviceCtx &ctx, float *out, const float *x, size_t planes, size_t ih, size_t iw, size_t oh, size_t ow,
+                   size_t kh, size_t kw, size_t sh, size_t sw, size_t pad_t, size_t pad_l);
+// Conv2d = im2col + one batched GEMM per group (conv2d.cpp).  `col` is caller-provided scratch of
+// batch * c * kh * kw * oh * ow floats; bias may be null.
+int launch_conv2d(DeviceCtx &ctx, float *out, const float *x, const float *w, const float *bias, float *col, size_t batch,
+                  size_t c, size_t ih, size_t iw, size_t oc, size_t oh, size_t ow, size_t kh, size_t kw, size_t sh, size_t sw,
+                  size_t dh, size_t dw, size_t pad_t, size_t pad_l, size_t group);
+
 }  // namespace altius

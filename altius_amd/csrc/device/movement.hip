@@ -290,6 +290,67 @@ __global__ __launch_bounds__(BLOCK) void batchnorm_nchw(float *__restrict__ out,
     }
 }
 
+// ---- im2col and max pooling -------------------------------------------------------------------
+// col[b][c][fy][fx][oh][ow] = x[b][c][oh*sh - pad_t + fy*dh][ow*sw - pad_l + fx*dw], zero outside the
+// image: the layout the reference builds (conv2d.rs:82-150, 213-333), K-major so that the
+// convolution is W[oc, K] x col[K, oh*ow] per image and group.
+struct ConvGeom {
+    FastDiv ow, oh, kw, kh, c;
+    uint32_t ih, iw, sh, sw, dh, dw, pad_t, pad_l;
+};
+
+__global__ __launch_bounds__(BLOCK) void im2col_kernel(float *__restrict__ col, const float *__restrict__ x, ConvGeom g,
+                                                       uint32_t total) {
+    const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= total) return;
+    uint32_t r = i;
+    uint32_t q = g.ow.div(r);
+    const uint32_t ow = r - q * g.ow.d;
+    r = q;
+    q = g.oh.div(r);
+    const uint32_t oh = r - q * g.oh.d;
+    r = q;
+    q = g.kw.div(r);
+    const uint32_t fx = r - q * g.kw.d;
+    r = q;
+    q = g.kh.div(r);
+    const uint32_t fy = r - q * g.kh.d;
+    const uint32_t plane = q;  // b * C + c
+    const int y = (int)(oh * g.sh + fy * g.dh) - (int)g.pad_t;
+    const int xx = (int)(ow * g.sw + fx * g.dw) - (int)g.pad_l;
+    float v = 0.0f;
+    if (y >= 0 && y < (int)g.ih && xx >= 0 && xx < (int)g.iw) v = x[((size_t)plane * g.ih + (uint32_t)y) * g.iw + (uint32_t)xx];
+    col[i] = v;
+}
+
+// compute_max_pool (session.rs:324-382): the window is clipped to the image, NaN never wins
+// (f32::max), and a window that holds nothing (or only f32::MIN) yields 0.0.
+__global__ __launch_bounds__(BLOCK) void maxpool_kernel(float *__restrict__ out, const float *__restrict__ x, FastDiv ow,
+                                                        FastDiv oh, uint32_t ih, uint32_t iw, uint32_t kh, uint32_t kw,
+                                                        uint32_t sh, uint32_t sw, uint32_t pad_t, uint32_t pad_l,
+                                                        uint32_t total) {
+    const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= total) return;
+    uint32_t q = ow.div(i);
+    const uint32_t ox = i - q * ow.d;
+    const uint32_t plane = oh.div(q);
+    const uint32_t oy = q - plane * oh.d;
+    const int y0 = (int)(oy * sh) - (int)pad_t, x0 = (int)(ox * sw) - (int)pad_l;
+    const float lowest = -3.40282347e+38f;  // f32::MIN
+    float m = lowest;
+    const float *p = x + (size_t)plane * ih * iw;
+    for (uint32_t fy = 0; fy < kh; fy++) {
+        const int y = y0 + (int)fy;
+        if (y < 0 || y >= (int)ih) continue;
+        for (uint32_t fx = 0; fx < kw; fx++) {
+            const int xx = x0 + (int)fx;
+            if (xx < 0 || xx >= (int)iw) continue;
+            m = fmaxf(p[(uint32_t)y * iw + (uint32_t)xx], m);
+        }
+    }
+    out[i] = m == lowest ? 0.0f : m;
+}
+
 struct Vec16 {
     uint32_t a, b, c, d;
 };
@@ -666,6 +727,43 @@ int launch_batchnorm(DeviceCtx &ctx, float *out, const float *x, const float *sc
                            x, scale, bias, mean, var, fhw, fc, (uint32_t)total, eps);
     }
     return ctx.check(hipGetLastError(), "batchnorm launch");
+}
+
+int launch_im2col(DeviceCtx &ctx, float *col, const float *x, size_t batch, size_t c, size_t ih, size_t iw, size_t oh,
+                  size_t ow, size_t kh, size_t kw, size_t sh, size_t sw, size_t dh, size_t dw, size_t pad_t, size_t pad_l) {
+    const size_t total = batch * c * kh * kw * oh * ow;
+    if (total == 0) return AHIP_OK;
+    if (!col || !x) return ctx.fail(AHIP_ERR_ARG, "im2col: null pointer");
+    if (int rc = fits32(ctx, std::max(total, batch * c * ih * iw), "im2col")) return rc;
+    ConvGeom g;
+    g.ow = make_fastdiv((uint32_t)ow);
+    g.oh = make_fastdiv((uint32_t)oh);
+    g.kw = make_fastdiv((uint32_t)kw);
+    g.kh = make_fastdiv((uint32_t)kh);
+    g.c = make_fastdiv((uint32_t)c);
+    g.ih = (uint32_t)ih;
+    g.iw = (uint32_t)iw;
+    g.sh = (uint32_t)sh;
+    g.sw = (uint32_t)sw;
+    g.dh = (uint32_t)dh;
+    g.dw = (uint32_t)dw;
+    g.pad_t = (uint32_t)pad_t;
+    g.pad_l = (uint32_t)pad_l;
+    hipLaunchKernelGGL(im2col_kernel, dim3((unsigned)((total + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, ctx.stream, col, x, g,
+                       (uint32_t)total);
+    return ctx.check(hipGetLastError(), "im2col launch");
+}
+
+int launch_maxpool(DeviceCtx &ctx, float *out, const float *x, size_t planes, size_t ih, size_t iw, size_t oh, size_t ow,
+                   size_t kh, size_t kw, size_t sh, size_t sw, size_t pad_t, size_t pad_l) {
+    const size_t total = planes * oh * ow;
+    if (total == 0) return AHIP_OK;
+    if (!out || !x) return ctx.fail(AHIP_ERR_ARG, "maxpool: null pointer");
+    if (int rc = fits32(ctx, std::max(total, planes * ih * iw), "maxpool")) return rc;
+    hipLaunchKernelGGL(maxpool_kernel, dim3((unsigned)((total + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, ctx.stream, out, x,
+                       make_fastdiv((uint32_t)ow), make_fastdiv((uint32_t)oh), (uint32_t)ih, (uint32_t)iw, (uint32_t)kh,
+                       (uint32_t)kw, (uint32_t)sh, (uint32_t)sw, (uint32_t)pad_t, (uint32_t)pad_l, (uint32_t)total);
+    return ctx.check(hipGetLastError(), "maxpool launch");
 }
 
 }  // namespace altius

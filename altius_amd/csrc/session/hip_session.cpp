@@ -729,6 +729,34 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
         if (!need(1)) return false;
         rc = launch_cast(ctx_, out.ptr, in[0]->ptr, (int)in[0]->elem_ty, (int)out.elem_ty, n_out);
         break;
+    case OpKind::Conv2d: {  // conv2d::compute (conv2d.rs:26-211)
+        if (!need(2) || !need_f32({0, 1})) return false;
+        const FixedDimensions &x = in[0]->dims, &w = in[1]->dims;
+        if (x.len() != 4 || w.len() != 4 || op.padding.size() != 4) return fail(err, SessionError::Shape, "Conv2d: four-dimensional input, weight and padding are needed");
+        const size_t group = (size_t)op.group;
+        if (group == 0 || x[1] % group || w[0] % group || w[1] != x[1] / group || w[2] != (size_t)op.kernel_shape[0] || w[3] != (size_t)op.kernel_shape[1])
+            return fail(err, SessionError::Shape, "Conv2d: weight " + w.to_string() + " does not fit input " + x.to_string() + " with group " + std::to_string(group));
+        const float *bias = nullptr;
+        if (in.size() > 2 && in[2]) {
+            if (in[2]->elem_ty != TensorElemType::F32 || in[2]->dims.total_elems() != w[0]) return fail(err, SessionError::Shape, "Conv2d: bias must hold one f32 per output channel");
+            bias = f(in[2]);
+        }
+        DeviceTensor col;
+        const size_t oh = out.dims[2], ow = out.dims[3];
+        if (!allocate(TypedFixedShape{FixedDimensions({x[0], x[1], w[2], w[3], oh, ow}), TensorElemType::F32}, &col, err)) return false;
+        rc = launch_conv2d(ctx_, o, f(in[0]), f(in[1]), bias, static_cast<float *>(col.ptr), x[0], x[1], x[2], x[3], w[0], oh, ow, w[2], w[3],
+                           (size_t)op.strides[0], (size_t)op.strides[1], (size_t)op.dilations[0], (size_t)op.dilations[1],
+                           (size_t)op.padding[0], (size_t)op.padding[1], group);
+        break;  // `col` goes back to the pool here; stream order keeps it intact until the GEMMs have read it
+    }
+    case OpKind::MaxPool: {  // compute_max_pool (session.rs:324-382)
+        if (!need(1) || !need_f32({0})) return false;
+        const FixedDimensions &x = in[0]->dims;
+        if (x.len() != 4 || op.padding.size() != 4) return fail(err, SessionError::Shape, "MaxPool: four-dimensional input and padding are needed");
+        rc = launch_maxpool(ctx_, o, f(in[0]), x[0] * x[1], x[2], x[3], out.dims[2], out.dims[3], (size_t)op.kernel_shape[0],
+                            (size_t)op.kernel_shape[1], (size_t)op.strides[0], (size_t)op.strides[1], (size_t)op.padding[0], (size_t)op.padding[1]);
+        break;
+    }
     case OpKind::MatMul: {  // compute_mat_mul (session.rs:621-684), with NumPy broadcasting of the batch axes
         if (!need(2) || !need_f32({0, 1})) return false;
         const FixedDimensions &a = in[0]->dims, &b = in[1]->dims;

@@ -402,3 +402,37 @@ class Context:
         finally:
             for x in (da, db, dout) + ((dc0,) if dc0 else ()):
                 self.free(x)
+
+    def conv2d(self, x, w, bias=None, strides=(1, 1), pads=(0, 0, 0, 0), dilations=(1, 1), group=1):
+        x = np.asarray(x, dtype=np.float32, order="C")
+        w = np.asarray(w, dtype=np.float32, order="C")
+        b, c, ih, iw = x.shape
+        oc, _, kh, kw = w.shape
+        oh = (ih + pads[0] + pads[2] - dilations[0] * (kh - 1) - 1) // strides[0] + 1
+        ow = (iw + pads[1] + pads[3] - dilations[1] * (kw - 1) - 1) // strides[1] + 1
+        dx, dw = self.upload(x), self.upload(w)
+        db = self.upload(np.asarray(bias, dtype=np.float32)) if bias is not None else None
+        dcol = self.alloc(max(b * c * kh * kw * oh * ow * 4, 4))
+        do = self.alloc(max(b * oc * oh * ow * 4, 4))
+        try:
+            check(self.L.ahip_conv2d(self.handle, do.ptr, dx.ptr, dw.ptr, db.ptr if db else None, dcol.ptr, b, c, ih, iw, oc, oh, ow,
+                                     kh, kw, strides[0], strides[1], dilations[0], dilations[1], pads[0], pads[1], group), self.handle)
+            return self.download(do, (b, oc, oh, ow))
+        finally:
+            for t in (dx, dw, dcol, do) + ((db,) if db else ()):
+                self.free(t)
+
+    def max_pool(self, x, kernel, strides, pads=(0, 0, 0, 0)):
+        x = np.asarray(x, dtype=np.float32, order="C")
+        b, c, ih, iw = x.shape
+        oh = (ih + pads[0] + pads[2] - kernel[0]) // strides[0] + 1
+        ow = (iw + pads[1] + pads[3] - kernel[1]) // strides[1] + 1
+        dx = self.upload(x)
+        do = self.alloc(max(b * c * oh * ow * 4, 4))
+        try:
+            check(self.L.ahip_maxpool(self.handle, do.ptr, dx.ptr, b * c, ih, iw, oh, ow, kernel[0], kernel[1], strides[0], strides[1],
+                                      pads[0], pads[1]), self.handle)
+            return self.download(do, (b, c, oh, ow))
+        finally:
+            self.free(dx)
+            self.free(do)

@@ -218,6 +218,17 @@ int ahip_gemm(ahip_ctx *ctx, float *c, const float *a, const float *b, const flo
               size_t b_batch_stride, size_t c_batch_stride, size_t c0_row_stride, size_t c0_col_stride, float alpha,
               float beta);
 
+/* Conv2d on NCHW (crates/session_interpreter/src/conv2d.rs:26-211): im2col into `col`
+ * (scratch of batch*c*kh*kw*oh*ow floats, the reference's layout [b][c][kh][kw][oh][ow]) and one
+ * batched GEMM per group.  w is [oc, c/group, kh, kw]; bias ([oc]) may be NULL.  oh / ow are the
+ * output extents the caller inferred (shape.rs:38-88).
+ * MaxPool (compute_max_pool, session.rs:324-382) over [planes, ih, iw] -> [planes, oh, ow]. */
+int ahip_conv2d(ahip_ctx *ctx, float *out, const float *x, const float *w, const float *bias, float *col, size_t batch,
+                size_t c, size_t ih, size_t iw, size_t oc, size_t oh, size_t ow, size_t kh, size_t kw, size_t stride_h,
+                size_t stride_w, size_t dilation_h, size_t dilation_w, size_t pad_top, size_t pad_left, size_t group);
+int ahip_maxpool(ahip_ctx *ctx, float *out, const float *x, size_t planes, size_t ih, size_t iw, size_t oh, size_t ow,
+                 size_t kh, size_t kw, size_t stride_h, size_t stride_w, size_t pad_top, size_t pad_left);
+
 /* ------------------------------------------------------------------------
  * Graph IR: the same Model / Graph / Node / Value / Op structure as
  * altius_core (crates/core/src/model.rs:13-17, graph.rs:9-16, node.rs:7-14,

@@ -370,3 +370,38 @@ def gemm(a, b, c=None, alpha=1.0, beta=1.0, trans_a=False, trans_b=False):
     if rc != OK:
         raise OracleError(rc, "gemm")
     return out
+
+
+def _conv_out(n, k, s, p0, p1, d=1):
+    return (n + p0 + p1 - d * (k - 1) - 1) // s + 1
+
+
+def conv2d(x, w, bias=None, strides=(1, 1), pads=(0, 0, 0, 0), dilations=(1, 1), group=1):
+    x, w = _f32(x), _f32(w)
+    b, c, ih, iw = x.shape
+    oc, _, kh, kw = w.shape
+    oh = _conv_out(ih, kh, strides[0], pads[0], pads[2], dilations[0])
+    ow = _conv_out(iw, kw, strides[1], pads[1], pads[3], dilations[1])
+    out = np.empty((b, oc, oh, ow), dtype=np.float32)
+    bias_arr = _f32(bias) if bias is not None else None
+    sz = ctypes.c_size_t
+    rc = lib().orc_conv2d(_fptr(x), _fptr(w), _fptr(bias_arr) if bias_arr is not None else None, _fptr(out), sz(b), sz(c), sz(ih),
+                          sz(iw), sz(oc), sz(oh), sz(ow), sz(kh), sz(kw), sz(strides[0]), sz(strides[1]), sz(dilations[0]),
+                          sz(dilations[1]), sz(pads[0]), sz(pads[1]), sz(group))
+    if rc != OK:
+        raise OracleError(rc, "conv2d")
+    return out
+
+
+def max_pool(x, kernel, strides, pads=(0, 0, 0, 0)):
+    x = _f32(x)
+    b, c, ih, iw = x.shape
+    oh = _conv_out(ih, kernel[0], strides[0], pads[0], pads[2])
+    ow = _conv_out(iw, kernel[1], strides[1], pads[1], pads[3])
+    out = np.empty((b, c, oh, ow), dtype=np.float32)
+    sz = ctypes.c_size_t
+    rc = lib().orc_max_pool(_fptr(x), _fptr(out), sz(b * c), sz(ih), sz(iw), sz(oh), sz(ow), sz(kernel[0]), sz(kernel[1]),
+                            sz(strides[0]), sz(strides[1]), sz(pads[0]), sz(pads[1]))
+    if rc != OK:
+        raise OracleError(rc, "max_pool")
+    return out

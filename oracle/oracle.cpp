@@ -1094,6 +1094,54 @@ int orc_sgemm(int trans_a, int trans_b, size_t m, size_t k, size_t n, float alph
     return ORC_OK;
 }
 
+int orc_conv2d(const float *x, const float *w, const float *bias, float *out, size_t batch, size_t c, size_t ih, size_t iw,
+               size_t oc, size_t oh, size_t ow, size_t kh, size_t kw, size_t sh, size_t sw, size_t dh, size_t dw, size_t pad_t,
+               size_t pad_l, size_t group) {
+    if (group == 0 || c % group || oc % group) return ORC_ERR_ARG;
+    const size_t ohw = oh * ow, cg = c / group, ocg = oc / group, k = cg * kh * kw;
+    for (size_t b = 0; b < batch; b++)  // conv2d.rs:63-80
+        for (size_t o = 0; o < oc; o++)
+            for (size_t i = 0; i < ohw; i++) out[(b * oc + o) * ohw + i] = bias ? bias[o] : 0.0f;
+    std::vector<float> col(batch * c * kh * kw * ohw);
+    for (size_t b = 0; b < batch; b++)
+        for (size_t ch = 0; ch < c; ch++)
+            for (size_t fy = 0; fy < kh; fy++)
+                for (size_t fx = 0; fx < kw; fx++)
+                    for (size_t y = 0; y < oh; y++)
+                        for (size_t xo = 0; xo < ow; xo++) {
+                            const long iy = (long)(y * sh + fy * dh) - (long)pad_t, ix = (long)(xo * sw + fx * dw) - (long)pad_l;
+                            const bool in = iy >= 0 && iy < (long)ih && ix >= 0 && ix < (long)iw;
+                            col[((((b * c + ch) * kh + fy) * kw + fx) * oh + y) * ow + xo] =
+                                in ? x[((b * c + ch) * ih + (size_t)iy) * iw + (size_t)ix] : 0.0f;
+                        }
+    // conv2d.rs:152-210: chunks of col (per image and group) against the weights of the group, cycling.
+    for (size_t b = 0; b < batch; b++)
+        for (size_t g = 0; g < group; g++)
+            orc_sgemm(0, 0, ocg, k, ohw, 1.0f, w + g * ocg * k, k, col.data() + (b * group + g) * k * ohw, ohw, 1.0f,
+                      out + (b * group + g) * ocg * ohw, ohw);
+    return ORC_OK;
+}
+
+int orc_max_pool(const float *x, float *out, size_t planes, size_t ih, size_t iw, size_t oh, size_t ow, size_t kh, size_t kw,
+                 size_t sh, size_t sw, size_t pad_t, size_t pad_l) {
+    const float lowest = -3.40282347e+38f;
+    for (size_t p = 0; p < planes; p++)
+        for (size_t ay = 0; ay < oh; ay++)
+            for (size_t ax = 0; ax < ow; ax++) {
+                const long y = (long)(ay * sh) - (long)pad_t, xx = (long)(ax * sw) - (long)pad_l;
+                float m = lowest;
+                for (size_t fy = 0; fy < kh; fy++)
+                    for (size_t fx = 0; fx < kw; fx++) {
+                        const long oy = y + (long)fy, ox = xx + (long)fx;
+                        if (oy < 0 || oy >= (long)ih || ox < 0 || ox >= (long)iw) continue;
+                        const float v = x[(p * ih + (size_t)oy) * iw + (size_t)ox];
+                        m = std::fmax(v, m);  // f32::max: NaN loses
+                    }
+                out[(p * oh + ay) * ow + ax] = m == lowest ? 0.0f : m;
+            }
+    return ORC_OK;
+}
+
 float orc_fast_sum(const float *x, size_t n) { return fast_sum(x, n); }
 float orc_fast_sum_squares(const float *x, size_t n) { return fast_sum_squares(x, n); }
 

@@ -177,6 +177,18 @@ int orc_leaky_relu(const float *x, float *out, size_t n, float alpha);
 int orc_sgemm(int trans_a, int trans_b, size_t m, size_t k, size_t n, float alpha, const float *a, size_t lda,
               const float *b, size_t ldb, float beta, float *c, size_t ldc);
 
+/* conv2d::compute (conv2d.rs:26-211): bias fill, im2col into [b][c][kh][kw][oh][ow], then per image
+ * and group out += W_g * col_g through sgemm (accumulation order as orc_sgemm: unpinned at the bit
+ * level).  pads = [top, left, bottom, right].  PINNED against the direct definition of the
+ * convolution (exact on integer-valued data, forward error bound otherwise). */
+int orc_conv2d(const float *x, const float *w, const float *bias, float *out, size_t batch, size_t c, size_t ih, size_t iw,
+               size_t oc, size_t oh, size_t ow, size_t kh, size_t kw, size_t sh, size_t sw, size_t dh, size_t dw, size_t pad_t,
+               size_t pad_l, size_t group);
+
+/* compute_max_pool (session.rs:324-382). */
+int orc_max_pool(const float *x, float *out, size_t planes, size_t ih, size_t iw, size_t oh, size_t ow, size_t kh, size_t kw,
+                 size_t sh, size_t sw, size_t pad_t, size_t pad_l);
+
 float orc_fast_sum(const float *x, size_t n);
 float orc_fast_sum_squares(const float *x, size_t n);
 

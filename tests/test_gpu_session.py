@@ -265,13 +265,13 @@ def test_errors_come_back_as_values(case):
     # shapes are fine but there is no kernel: SessionError::Message, as the reference reports it
     m = Model()
     a, c = m.new_val_named_and_shaped("a", [1, 1, 4, 4]), m.new_val()
-    m.add_node(Op.MaxPool, [a], [c], kernel_shape=[2, 2], strides=[2, 2])
+    m.add_node(Op.ReduceMin, [a], [c], axes=[1])
     m.add_input(a)
     m.add_output(c)
     sess = HipSessionBuilder(m).build()
     with pytest.raises(AltiusHipError) as e:
         sess.run([np.zeros([1, 1, 4, 4], np.float32)])
-    assert e.value.code == ERR_UNSUPPORTED and "MaxPool: Kernel not implemented" in e.value.message
+    assert e.value.code == ERR_UNSUPPORTED and "ReduceMin: Kernel not implemented" in e.value.message   # session.rs:209-213
 
     sess = HipSessionBuilder(binary_model(Op.Add)).build()
     with pytest.raises(AltiusHipError) as e:   # shapes that do not broadcast (test_ops_bin.py:31-40)

@@ -504,3 +504,74 @@ def test_sgemm_against_exact_products(oracle):
     full = rng.integers(-3, 4, size=(4, 5)).astype(np.float32)
     assert np.array_equal(oracle.gemm(ai.T.copy(), bi.T.copy(), full), (ai.T @ bi.T + full))
     assert np.array_equal(oracle.gemm(ai.T.copy(), bi.T.copy()), ai.T @ bi.T)         # no C: beta has nothing to scale
+
+
+def direct_conv(x, w, bias, strides, pads, dilations, group):
+    """The definition of the cross-correlation, in float64."""
+    b, c, ih, iw = x.shape
+    oc, cg, kh, kw = w.shape
+    xp = np.zeros((b, c, ih + pads[0] + pads[2], iw + pads[1] + pads[3]))
+    xp[:, :, pads[0]:pads[0] + ih, pads[1]:pads[1] + iw] = x
+    oh = (xp.shape[2] - dilations[0] * (kh - 1) - 1) // strides[0] + 1
+    ow = (xp.shape[3] - dilations[1] * (kw - 1) - 1) // strides[1] + 1
+    out = np.zeros((b, oc, oh, ow))
+    ocg = oc // group
+    for o in range(oc):
+        g = o // ocg
+        for ci in range(cg):
+            for fy in range(kh):
+                for fx in range(kw):
+                    patch = xp[:, g * cg + ci, fy * dilations[0]:fy * dilations[0] + oh * strides[0]:strides[0],
+                               fx * dilations[1]:fx * dilations[1] + ow * strides[1]:strides[1]]
+                    out[:, o] += float(w[o, ci, fy, fx]) * patch
+        if bias is not None:
+            out[:, o] += float(bias[o])
+    return out
+
+
+CONV_CASES = [
+    dict(x=(2, 3, 32, 32), w=(8, 3, 16, 16), strides=(16, 16)),                                       # patch embedding
+    dict(x=(1, 4, 9, 11), w=(6, 4, 3, 3), pads=(1, 1, 1, 1)),
+    dict(x=(2, 4, 10, 9), w=(6, 4, 3, 5), pads=(0, 2, 1, 3), strides=(2, 1)),
+    dict(x=(1, 2, 12, 12), w=(4, 2, 3, 3), dilations=(2, 2), pads=(2, 2, 2, 2)),
+    dict(x=(2, 6, 8, 8), w=(6, 1, 3, 3), pads=(1, 1, 1, 1), group=6),                                 # depthwise
+    dict(x=(1, 8, 7, 7), w=(4, 4, 1, 1), group=2),
+    dict(x=(1, 3, 5, 5), w=(2, 3, 5, 5)),                                                             # no padding, stride 1 (conv2d.rs:90-112)
+]
+
+
+@pytest.mark.parametrize("case_", CONV_CASES)
+def test_conv2d_against_the_definition(oracle, case_):
+    rng = np.random.default_rng(13)
+    kw = {k: v for k, v in case_.items() if k not in ("x", "w")}
+    args = dict(strides=(1, 1), pads=(0, 0, 0, 0), dilations=(1, 1), group=1)
+    args.update(kw)
+    x = rng.integers(-3, 4, size=case_["x"]).astype(np.float32)
+    w = rng.integers(-3, 4, size=case_["w"]).astype(np.float32)
+    bias = rng.integers(-3, 4, size=case_["w"][0]).astype(np.float32)
+    for b in (bias, None):
+        assert np.array_equal(oracle.conv2d(x, w, b, **args), direct_conv(x, w, b, **args).astype(np.float32))
+    xr, wr = rng.standard_normal(case_["x"]).astype(np.float32), rng.standard_normal(case_["w"]).astype(np.float32)
+    k = int(np.prod(case_["w"][1:]))
+    exact = direct_conv(xr, wr, bias, **args)
+    bound = (k + 2) * 2.0 ** -24 * direct_conv(np.abs(xr), np.abs(wr), np.abs(bias), **args)
+    assert np.all(np.abs(oracle.conv2d(xr, wr, bias, **args) - exact) <= bound)
+
+
+def test_max_pool_against_sliding_windows(oracle):
+    rng = np.random.default_rng(14)
+    x = rng.standard_normal((2, 3, 9, 10)).astype(np.float32)
+    for kernel, strides, pads in [((2, 2), (2, 2), (0, 0, 0, 0)), ((3, 3), (2, 2), (1, 1, 1, 1)), ((3, 2), (1, 3), (0, 1, 2, 0))]:
+        got = oracle.max_pool(x, kernel, strides, pads)
+        xp = np.full((2, 3, 9 + pads[0] + pads[2], 10 + pads[1] + pads[3]), -np.inf, np.float32)
+        xp[:, :, pads[0]:pads[0] + 9, pads[1]:pads[1] + 10] = x
+        oh, ow = got.shape[2:]
+        want = np.empty_like(got)
+        for i in range(oh):
+            for j in range(ow):
+                want[:, :, i, j] = xp[:, :, i * strides[0]:i * strides[0] + kernel[0], j * strides[1]:j * strides[1] + kernel[1]].max((2, 3))
+        assert np.array_equal(got, want)
+    nan = x.copy()
+    nan[0, 0, 0, 0] = np.nan
+    assert not np.isnan(oracle.max_pool(nan, (2, 2), (2, 2))).any()                                      # f32::max drops NaN
+    assert np.array_equal(oracle.max_pool(np.full((1, 1, 2, 2), np.finfo(np.float32).min, np.float32), (2, 2), (2, 2)), [[[[0.0]]]])
