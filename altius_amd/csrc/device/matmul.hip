@@ -44,19 +44,19 @@ struct GemmArgs {
 // Loads this thread's share of a BK x 128 operand tile into registers.
 // K_CONTIG: the operand's k axis is the contiguous one (A without transA, B with transB).
 // `mn` is the tile's first row (A) or column (B), `lim` the extent of that axis.
-template <bool K_CONTIG>
-__device__ __forceinline__ void load_tile(float4 (&r)[2], const float *__restrict__ p, uint32_t mn0, uint32_t lim,
+template <bool K_CONTIG, int WIDTH>
+__device__ __forceinline__ void load_tile(float4 (&r)[WIDTH / 64], const float *__restrict__ p, uint32_t mn0, uint32_t lim,
                                           uint32_t k0, uint32_t kdim, uint32_t s_mn, uint32_t s_k, int vec, int tid) {
 #pragma unroll
-    for (int u = 0; u < 2; u++) {
+    for (int u = 0; u < WIDTH / 64; u++) {
         const int f = tid + THREADS * u;
         uint32_t mn, kk;
-        if (K_CONTIG) {  // 128 rows of 16 floats: 4 float4 per row
+        if (K_CONTIG) {  // WIDTH rows of 16 floats: 4 float4 per row
             mn = mn0 + (f >> 2);
             kk = k0 + ((f & 3) << 2);
-        } else {  // 16 rows of 128 floats: 32 float4 per row
-            kk = k0 + (f >> 5);
-            mn = mn0 + ((f & 31) << 2);
+        } else {  // 16 rows of WIDTH floats: WIDTH / 4 float4 per row
+            kk = k0 + f / (WIDTH / 4);
+            mn = mn0 + ((f % (WIDTH / 4)) << 2);
         }
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
         if (K_CONTIG) {
@@ -89,9 +89,10 @@ __device__ __forceinline__ void load_tile(float4 (&r)[2], const float *__restric
 }
 
 // Stores the registers into the k-major LDS tile [BK][PITCH].
-template <bool K_CONTIG> __device__ __forceinline__ void store_tile(float *__restrict__ t, const float4 (&r)[2], int tid) {
+template <bool K_CONTIG, int WIDTH>
+__device__ __forceinline__ void store_tile(float *__restrict__ t, const float4 (&r)[WIDTH / 64], int tid) {
 #pragma unroll
-    for (int u = 0; u < 2; u++) {
+    for (int u = 0; u < WIDTH / 64; u++) {
         const int f = tid + THREADS * u;
         if (K_CONTIG) {
             const int mn = f >> 2, kk = (f & 3) << 2;
@@ -100,37 +101,40 @@ template <bool K_CONTIG> __device__ __forceinline__ void store_tile(float *__res
             t[(kk + 2) * PITCH + mn] = r[u].z;
             t[(kk + 3) * PITCH + mn] = r[u].w;
         } else {
-            const int kk = f >> 5, mn = (f & 31) << 2;
+            const int kk = f / (WIDTH / 4), mn = (f % (WIDTH / 4)) << 2;
             *reinterpret_cast<float4 *>(t + kk * PITCH + mn) = r[u];
         }
     }
 }
 
-template <bool A_KC, bool B_KC>
+// TN = 128: wavefronts in a 2 x 2 grid, 64 x 64 each.  TN = 64 (narrow outputs such as attention's
+// P x V with 64 columns): wavefronts stacked 4 x 1, 32 x 64 each.
+template <bool A_KC, bool B_KC, int TN>
 __global__ __launch_bounds__(THREADS) void gemm_f32_mfma(GemmArgs g) {
+    constexpr int WI = TN == 128 ? 2 : 1;  // 32-row MFMA tiles per wavefront
     __shared__ __align__(16) float As[2][BK * PITCH];
     __shared__ __align__(16) float Bs[2][BK * PITCH];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int wm = TN == 128 ? wave >> 1 : wave, wn = TN == 128 ? wave & 1 : 0;
+    const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * TN;
     const float *a = g.a + (size_t)blockIdx.z * g.a_bs;
     const float *b = g.b + (size_t)blockIdx.z * g.b_bs;
     // Strides of the tile's mn axis and k axis for each operand.
     const uint32_t a_smn = g.a_rs, a_sk = g.a_cs, b_smn = g.b_cs, b_sk = g.b_rs;
 
-    floatx16 acc[2][2];
+    floatx16 acc[WI][2];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < WI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    float4 ra[2], rb[2];
-    load_tile<A_KC>(ra, a, m0, g.m, 0, g.k, a_smn, a_sk, g.a_vec, tid);
-    load_tile<B_KC>(rb, b, n0, g.n, 0, g.k, b_smn, b_sk, g.b_vec, tid);
-    store_tile<A_KC>(As[0], ra, tid);
-    store_tile<B_KC>(Bs[0], rb, tid);
+    float4 ra[BM / 64], rb[TN / 64];
+    load_tile<A_KC, BM>(ra, a, m0, g.m, 0, g.k, a_smn, a_sk, g.a_vec, tid);
+    load_tile<B_KC, TN>(rb, b, n0, g.n, 0, g.k, b_smn, b_sk, g.b_vec, tid);
+    store_tile<A_KC, BM>(As[0], ra, tid);
+    store_tile<B_KC, TN>(Bs[0], rb, tid);
     __syncthreads();
 
     const uint32_t nk = (g.k + BK - 1) / BK;
@@ -139,23 +143,26 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_mfma(GemmArgs g) {
         const int cur = kt & 1;
         const bool more = kt + 1 < nk;
         if (more) {
-            load_tile<A_KC>(ra, a, m0, g.m, (kt + 1) * BK, g.k, a_smn, a_sk, g.a_vec, tid);
-            load_tile<B_KC>(rb, b, n0, g.n, (kt + 1) * BK, g.k, b_smn, b_sk, g.b_vec, tid);
+            load_tile<A_KC, BM>(ra, a, m0, g.m, (kt + 1) * BK, g.k, a_smn, a_sk, g.a_vec, tid);
+            load_tile<B_KC, TN>(rb, b, n0, g.n, (kt + 1) * BK, g.k, b_smn, b_sk, g.b_vec, tid);
         }
-        const float *at = As[cur] + wm * 64 + lr;
+        const float *at = As[cur] + wm * (32 * WI) + lr;
         const float *bt = Bs[cur] + wn * 64 + lr;
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 2) {
-            const float a0 = at[(kk + lk) * PITCH], a1 = at[(kk + lk) * PITCH + 32];
+            float av[WI];
+#pragma unroll
+            for (int i = 0; i < WI; i++) av[i] = at[(kk + lk) * PITCH + 32 * i];
             const float b0 = bt[(kk + lk) * PITCH], b1 = bt[(kk + lk) * PITCH + 32];
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < WI; i++) {
+                acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], b0, acc[i][0], 0, 0, 0);
+                acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], b1, acc[i][1], 0, 0, 0);
+            }
         }
         if (more) {
-            store_tile<A_KC>(As[cur ^ 1], ra, tid);
-            store_tile<B_KC>(Bs[cur ^ 1], rb, tid);
+            store_tile<A_KC, BM>(As[cur ^ 1], ra, tid);
+            store_tile<B_KC, TN>(Bs[cur ^ 1], rb, tid);
         }
         __syncthreads();
     }
@@ -163,13 +170,13 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_mfma(GemmArgs g) {
     // Accumulator r of lane l is C[8 * (r / 4) + 4 * (l / 32) + r % 4][l % 32] of its 32 x 32 tile.
     float *c = g.c + (size_t)blockIdx.z * g.c_bs;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < WI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const uint32_t col = n0 + wn * 64 + j * 32 + lr;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const uint32_t row = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * lk + (r & 3);
+                const uint32_t row = m0 + wm * (32 * WI) + i * 32 + 8 * (r >> 2) + 4 * lk + (r & 3);
                 if (row < g.m && col < g.n) {
                     float v = g.alpha * acc[i][j][r];
                     if (g.c0) v += g.beta * g.c0[(size_t)row * g.c0_rs + (size_t)col * g.c0_cs];
@@ -192,7 +199,10 @@ int launch_gemm(DeviceCtx &ctx, float *c, const float *a, const float *b, const 
     const size_t lim = (size_t)1 << 31;
     if (m >= lim || n >= lim || k >= lim || lda >= lim || ldb >= lim || ldc >= lim || m * ldc >= ((size_t)1 << 40))
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm: extent above 2^31");
-    const size_t gy = (m + BM - 1) / BM, gx = (n + BN - 1) / BN;
+    // The narrow tile when it leaves fewer idle columns (n = 64: 64 instead of 128 computed).
+    const bool narrow = n <= 64 || (n < 512 && n % 128 != 0 && n % 128 <= 64);
+    const size_t tn = narrow ? 64 : BN;
+    const size_t gy = (m + BM - 1) / BM, gx = (n + tn - 1) / tn;
     if (gy > 65535 || batch > 65535) return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm: more than 65535 row tiles or batches");
     GemmArgs g;
     g.a = a;
@@ -218,10 +228,19 @@ int launch_gemm(DeviceCtx &ctx, float *c, const float *a, const float *b, const 
     g.b_vec = aligned16(b) && ldb % 4 == 0 && b_batch_stride % 4 == 0;
     const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch);
     const bool a_kc = !trans_a, b_kc = trans_b != 0;
-    if (a_kc && b_kc) hipLaunchKernelGGL((gemm_f32_mfma<true, true>), grid, dim3(THREADS), 0, ctx.stream, g);
-    else if (a_kc) hipLaunchKernelGGL((gemm_f32_mfma<true, false>), grid, dim3(THREADS), 0, ctx.stream, g);
-    else if (b_kc) hipLaunchKernelGGL((gemm_f32_mfma<false, true>), grid, dim3(THREADS), 0, ctx.stream, g);
-    else hipLaunchKernelGGL((gemm_f32_mfma<false, false>), grid, dim3(THREADS), 0, ctx.stream, g);
+#define GEMM(AK, BK_, TN_) hipLaunchKernelGGL((gemm_f32_mfma<AK, BK_, TN_>), grid, dim3(THREADS), 0, ctx.stream, g)
+    if (narrow) {
+        if (a_kc && b_kc) GEMM(true, true, 64);
+        else if (a_kc) GEMM(true, false, 64);
+        else if (b_kc) GEMM(false, true, 64);
+        else GEMM(false, false, 64);
+    } else {
+        if (a_kc && b_kc) GEMM(true, true, 128);
+        else if (a_kc) GEMM(true, false, 128);
+        else if (b_kc) GEMM(false, true, 128);
+        else GEMM(false, false, 128);
+    }
+#undef GEMM
     return ctx.check(hipGetLastError(), "gemm launch");
 }
 

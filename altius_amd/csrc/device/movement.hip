@@ -591,6 +591,21 @@ int launch_gather(DeviceCtx &ctx, void *out, const void *data, const void *indic
     if (axis_len == 0) return ctx.fail(AHIP_ERR_SHAPE, "gather: the gathered axis is empty");
     if (!out || !data || !indices || !bad_flag) return ctx.fail(AHIP_ERR_ARG, "gather: null pointer");
     if (int rc = fits32(ctx, std::max(total, outer * axis_len * inner), "gather")) return rc;
+    // Rows of whole 16-byte units move as such (embedding rows, class tokens).
+    if (elem_size == 4 && inner % 4 == 0 && aligned16(out) && aligned16(data)) {
+        const FastDiv in4 = make_fastdiv((uint32_t)(inner / 4)), nd4 = make_fastdiv((uint32_t)n_idx);
+        const uint32_t total4 = (uint32_t)(total / 4);
+        const dim3 grid4((total4 + BLOCK - 1) / BLOCK);
+        if (index_size == 8)
+            hipLaunchKernelGGL((gather_rows<uint4, long long>), grid4, dim3(BLOCK), 0, ctx.stream, static_cast<uint4 *>(out),
+                               static_cast<const uint4 *>(data), static_cast<const long long *>(indices), (uint32_t)axis_len,
+                               (uint32_t)n_idx, in4, nd4, total4, bad_flag);
+        else
+            hipLaunchKernelGGL((gather_rows<uint4, int>), grid4, dim3(BLOCK), 0, ctx.stream, static_cast<uint4 *>(out),
+                               static_cast<const uint4 *>(data), static_cast<const int *>(indices), (uint32_t)axis_len,
+                               (uint32_t)n_idx, in4, nd4, total4, bad_flag);
+        return ctx.check(hipGetLastError(), "gather launch");
+    }
     const FastDiv in = make_fastdiv((uint32_t)inner), nd = make_fastdiv((uint32_t)n_idx);
     const dim3 grid((unsigned)((total + BLOCK - 1) / BLOCK));
 #define GATHER(T, I)                                                                                                   \

@@ -231,6 +231,57 @@ def session_table(synth):
     return rows
 
 
+def build_next_rows(ctx, D, batch=256):
+    """The operators either side of the hot path (data movement, MatMul) at ViT-B/16 shapes for the given
+    batch: (name, bytes, flops, launcher).  Device buffers are left uninitialised where contents do not matter."""
+    from altius_amd._lib import check, i64_array
+
+    L, h = ctx.L, ctx.handle
+    rows = []
+    T, H, NH, DH = 197, 768, 12, 64
+
+    def transpose(name, shape, perm):
+        n = int(np.prod(shape))
+        a, b = ctx.alloc(n * 4), ctx.alloc(n * 4)
+        rows.append((name, 8 * n, 0, lambda: check(L.ahip_transpose(h, b.ptr, a.ptr, 4, len(shape), i64_array(shape), i64_array(perm)), h)))
+
+    transpose("Transpose split heads [%d,197,12,64]->(0,2,1,3)" % batch, (batch, T, NH, DH), (0, 2, 1, 3))
+    transpose("Transpose K^T [%d,12,197,64]->(0,1,3,2)" % batch, (batch, NH, T, DH), (0, 1, 3, 2))
+    n = batch * T * 3 * H
+    qkv = ctx.alloc(n * 4)
+    parts = [ctx.alloc(n * 4 // 3) for _ in range(3)]
+
+    def split():
+        for i, o in enumerate(parts):
+            check(L.ahip_copy_strided(h, o.ptr, qkv.ptr + H * 4 * i, 4, 2, i64_array([batch * T, H]), i64_array([H, 1]),
+                                      i64_array([3 * H, 1])), h)
+
+    rows.append(("Split qkv [%d,197,2304] -> 3 x 768" % batch, 8 * n, 0, split))
+    V, S = 50257, batch * 128
+    table, out = ctx.alloc(V * H * 4), ctx.alloc(S * H * 4)
+    ids = ctx.upload(np.random.default_rng(0).integers(0, V, size=S).astype(np.int64))
+    rows.append(("Gather [50257,768] x %d ids" % S, 2 * S * H * 4 + S * 8, 0,
+                 lambda: check(L.ahip_gather(h, out.ptr, table.ptr, ids.ptr, 8, 4, 1, V, S, H), h)))
+
+    def gemm(name, b, m, n_, k, a_bs, b_bs):
+        a = ctx.alloc((b if a_bs else 1) * m * k * 4)
+        w = ctx.alloc((b if b_bs else 1) * k * n_ * 4)
+        c = ctx.alloc(b * m * n_ * 4)
+        ctx.memset(a, 0x3c)
+        ctx.memset(w, 0x3c)
+        nbytes = 4 * ((b if a_bs else 1) * m * k + (b if b_bs else 1) * k * n_ + b * m * n_)
+        rows.append((name, nbytes, 2.0 * b * m * n_ * k,
+                     lambda: ctx.gemm_raw(c.ptr, a.ptr, w.ptr, None, b, m, n_, k, a_bs=a_bs, b_bs=b_bs, c_bs=m * n_)))
+
+    M = batch * T
+    gemm("MatMul qkv [%d,768]x[768,2304]" % M, 1, M, 3 * H, H, 0, 0)
+    gemm("MatMul fc1 [%d,768]x[768,3072]" % M, 1, M, 4 * H, H, 0, 0)
+    gemm("MatMul fc2 [%d,3072]x[3072,768]" % M, 1, M, H, 4 * H, 0, 0)
+    gemm("MatMul QK^T %d x [197,64]x[64,197]" % (batch * NH), batch * NH, T, T, DH, T * DH, DH * T)
+    gemm("MatMul PV %d x [197,197]x[197,64]" % (batch * NH), batch * NH, T, DH, T, T * T, T * DH)
+    return rows
+
+
 def calibration_op(ctx, D):
     """A copy-shaped kernel of known traffic (Relu over 477 MB in, 477 MB out) used to scale the
     FETCH_SIZE / WRITE_SIZE counters of a profiling run."""
@@ -319,6 +370,8 @@ def main():
                     help="also run a copy-shaped Relu of known size (scales rocprof byte counters)")
     ap.add_argument("--all-configs", action="store_true",
                     help="also time the kernels and graphs of configs[0..3] (table on stderr, 'other_configs' in the JSON)")
+    ap.add_argument("--next-rows", action="store_true",
+                    help="also time the data-movement and MatMul kernels at ViT-B/16 shapes ('next_rows' in the JSON)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -409,6 +462,25 @@ def main():
             log("%-40s kernels %9.1f us (%7.1f GB/s)   run() incl. PCIe %9.3f ms"
                 % (r["graph"], r["kernels_us"], r["kernels_GBps"], r["run_ms_with_pcie"]))
         result["other_configs"] = {"kernels": others, "graphs": graphs_rows}
+
+    if args.next_rows:
+        MFMA_F32_PEAK = 157.3  # TFLOP/s, dense fp32 matrix cores
+        nxt = []
+        for name, nbytes, flops, fn in build_next_rows(ctx, D, args.batch):
+            o = Op(name, nbytes, [fn])
+            ms = time_kernel(ctx, o, max(10, args.kernel_iters // 2), 3)
+            row = {"kernel": name, "us": round(ms * 1e3, 1), "bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1)}
+            if flops:
+                row.update({"bound": "mfma", "TFLOPs": round(flops / ms / 1e9, 1),
+                            "frac_of_peak": round(flops / ms / 1e9 / MFMA_F32_PEAK, 3)})
+                log("%-48s %10.1f us %8.1f TFLOP/s (%4.1f %% of %.1f)" % (name, ms * 1e3, flops / ms / 1e9,
+                                                                         100 * flops / ms / 1e9 / MFMA_F32_PEAK, MFMA_F32_PEAK))
+            else:
+                row.update({"bound": "hbm", "frac_of_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 3)})
+                log("%-48s %10.1f us %8.1f GB/s    (%4.1f %% of 8000)" % (name, ms * 1e3, nbytes / ms / 1e6,
+                                                                        100 * nbytes / ms / 1e6 / HBM_PEAK_GBPS))
+            nxt.append(row)
+        result["next_rows"] = nxt
 
     if not args.no_cpu:
         threads = min(16, os.cpu_count() or 1)
