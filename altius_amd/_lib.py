@@ -80,6 +80,7 @@ def _declare(L):
       + [c_float, c_float])
     f("ahip_conv2d", [c_void_p] * 6 + [c_size_t] * 16)
     f("ahip_maxpool", [c_void_p] * 3 + [c_size_t] * 11)
+    f("ahip_resize", [c_void_p] * 3 + [c_size_t] * 5 + [c_int])
     f("ahip_module_load", [c_void_p, c_void_p, c_size_t, P(c_void_p)])
     f("ahip_module_unload", [c_void_p, c_void_p])
     f("ahip_launch", [c_void_p, c_void_p, c_char_p, P(ctypes.c_uint32), P(ctypes.c_uint32), ctypes.c_uint32,

@@ -380,4 +380,10 @@ int ahip_maxpool(ahip_ctx *ctx, float *out, const float *x, size_t planes, size_
     return altius::launch_maxpool(ctx->d, out, x, planes, ih, iw, oh, ow, kh, kw, stride_h, stride_w, pad_top, pad_left);
 }
 
+int ahip_resize(ahip_ctx *ctx, float *out, const float *x, size_t planes, size_t ih, size_t iw, size_t oh, size_t ow,
+                int nearest) {
+    REQUIRE_CTX(ctx, "ahip_resize");
+    return altius::launch_resize(ctx->d, out, x, planes, ih, iw, oh, ow, nearest);
+}
+
 }  // extern "C"

@@ -95,4 +95,8 @@ int launch_conv2d(DeviceCtx &ctx, float *out, const float *x, const float *w, co
                   size_t c, size_t ih, size_t iw, size_t oc, size_t oh, size_t ow, size_t kh, size_t kw, size_t sh, size_t sw,
                   size_t dh, size_t dw, size_t pad_t, size_t pad_l, size_t group);
 
+// Resize on [planes, ih, iw] -> [planes, oh, ow]: nearest, or the reference's bilinear blend (movement.hip).
+int launch_resize(DeviceCtx &ctx, float *out, const float *x, size_t planes, size_t ih, size_t iw, size_t oh, size_t ow,
+                  int nearest);
+
 }  // namespace altius

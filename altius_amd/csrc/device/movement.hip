@@ -351,6 +351,40 @@ __global__ __launch_bounds__(BLOCK) void maxpool_kernel(float *__restrict__ out,
     out[i] = m == lowest ? 0.0f : m;
 }
 
+// ---- resize ----------------------------------------------------------------------------------
+// compute_resize (session.rs:1056-1132) on NCHW: "nearest" takes x[(h / scale) as usize][(w / scale) as usize];
+// every other mode is the reference's bilinear blend with half-pixel centres clamped at 0.  The
+// reference derives one scale from the heights and uses it for both axes; here each axis has its own
+// (identical whenever the two agree, which is the only case in which the reference stays in bounds).
+template <bool NEAREST>
+__global__ __launch_bounds__(BLOCK) void resize_kernel(float *__restrict__ out, const float *__restrict__ x, FastDiv ow,
+                                                       FastDiv oh, uint32_t ih, uint32_t iw, float scale_h, float scale_w,
+                                                       uint32_t total) {
+    const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= total) return;
+    uint32_t q = ow.div(i);
+    const uint32_t w = i - q * ow.d;
+    const uint32_t plane = oh.div(q);
+    const uint32_t h = q - plane * oh.d;
+    const float *p = x + (size_t)plane * ih * iw;
+    if (NEAREST) {
+        uint32_t y = (uint32_t)((float)h / scale_h), xx = (uint32_t)((float)w / scale_w);
+        y = y < ih ? y : ih - 1;
+        xx = xx < iw ? xx : iw - 1;
+        out[i] = p[y * iw + xx];
+    } else {
+        const float ihf = fmaxf((float)h / scale_h - 0.5f, 0.0f), iwf = fmaxf((float)w / scale_w - 0.5f, 0.0f);
+        const uint32_t y = (uint32_t)ihf, xx = (uint32_t)iwf;
+        const uint32_t y0 = y < ih - 1 ? y : ih - 1, y1 = y + 1 < ih - 1 ? y + 1 : ih - 1;
+        const uint32_t x0 = xx < iw - 1 ? xx : iw - 1, x1 = xx + 1 < iw - 1 ? xx + 1 : iw - 1;
+        const float v00 = p[y0 * iw + x0], v01 = p[y0 * iw + x1], v10 = p[y1 * iw + x0], v11 = p[y1 * iw + x1];
+        const float fy = ihf - (float)y, fx = iwf - (float)xx;
+        const float hd = v00 + (v10 - v00) * fy;
+        const float hw = v01 + (v11 - v01) * fy;
+        out[i] = hd + (hw - hd) * fx;
+    }
+}
+
 struct Vec16 {
     uint32_t a, b, c, d;
 };
@@ -779,6 +813,24 @@ int launch_maxpool(DeviceCtx &ctx, float *out, const float *x, size_t planes, si
                        make_fastdiv((uint32_t)ow), make_fastdiv((uint32_t)oh), (uint32_t)ih, (uint32_t)iw, (uint32_t)kh,
                        (uint32_t)kw, (uint32_t)sh, (uint32_t)sw, (uint32_t)pad_t, (uint32_t)pad_l, (uint32_t)total);
     return ctx.check(hipGetLastError(), "maxpool launch");
+}
+
+int launch_resize(DeviceCtx &ctx, float *out, const float *x, size_t planes, size_t ih, size_t iw, size_t oh, size_t ow,
+                  int nearest) {
+    const size_t total = planes * oh * ow;
+    if (total == 0) return AHIP_OK;
+    if (ih == 0 || iw == 0) return ctx.fail(AHIP_ERR_SHAPE, "resize: empty input plane");
+    if (!out || !x) return ctx.fail(AHIP_ERR_ARG, "resize: null pointer");
+    if (int rc = fits32(ctx, std::max(total, planes * ih * iw), "resize")) return rc;
+    const float sh = (float)oh / (float)ih, sw = (float)ow / (float)iw;
+    const dim3 grid((unsigned)((total + BLOCK - 1) / BLOCK));
+    if (nearest)
+        hipLaunchKernelGGL((resize_kernel<true>), grid, dim3(BLOCK), 0, ctx.stream, out, x, make_fastdiv((uint32_t)ow),
+                           make_fastdiv((uint32_t)oh), (uint32_t)ih, (uint32_t)iw, sh, sw, (uint32_t)total);
+    else
+        hipLaunchKernelGGL((resize_kernel<false>), grid, dim3(BLOCK), 0, ctx.stream, out, x, make_fastdiv((uint32_t)ow),
+                           make_fastdiv((uint32_t)oh), (uint32_t)ih, (uint32_t)iw, sh, sw, (uint32_t)total);
+    return ctx.check(hipGetLastError(), "resize launch");
 }
 
 }  // namespace altius

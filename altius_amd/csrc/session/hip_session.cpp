@@ -757,6 +757,14 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
                             (size_t)op.kernel_shape[1], (size_t)op.strides[0], (size_t)op.strides[1], (size_t)op.padding[0], (size_t)op.padding[1]);
         break;
     }
+    case OpKind::Resize: {  // compute_resize (session.rs:1056-1132): batch and channels keep their extents
+        if (!need(1) || !need_f32({0})) return false;
+        const FixedDimensions &x = in[0]->dims;
+        if (x.len() != 4 || out.dims[0] != x[0] || out.dims[1] != x[1])
+            return fail(err, SessionError::Message, "Resize: only the two spatial axes of an NCHW tensor can be resized");
+        rc = launch_resize(ctx_, o, f(in[0]), x[0] * x[1], x[2], x[3], out.dims[2], out.dims[3], op.mode == "nearest");
+        break;
+    }
     case OpKind::MatMul: {  // compute_mat_mul (session.rs:621-684), with NumPy broadcasting of the batch axes
         if (!need(2) || !need_f32({0, 1})) return false;
         const FixedDimensions &a = in[0]->dims, &b = in[1]->dims;

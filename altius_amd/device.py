@@ -436,3 +436,15 @@ class Context:
         finally:
             self.free(dx)
             self.free(do)
+
+    def resize(self, x, out_hw, nearest=True):
+        x = np.asarray(x, dtype=np.float32, order="C")
+        b, c, ih, iw = x.shape
+        dx = self.upload(x)
+        do = self.alloc(max(b * c * out_hw[0] * out_hw[1] * 4, 4))
+        try:
+            check(self.L.ahip_resize(self.handle, do.ptr, dx.ptr, b * c, ih, iw, out_hw[0], out_hw[1], int(nearest)), self.handle)
+            return self.download(do, (b, c, out_hw[0], out_hw[1]))
+        finally:
+            self.free(dx)
+            self.free(do)

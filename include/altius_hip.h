@@ -228,6 +228,11 @@ int ahip_conv2d(ahip_ctx *ctx, float *out, const float *x, const float *w, const
                 size_t stride_w, size_t dilation_h, size_t dilation_w, size_t pad_top, size_t pad_left, size_t group);
 int ahip_maxpool(ahip_ctx *ctx, float *out, const float *x, size_t planes, size_t ih, size_t iw, size_t oh, size_t ow,
                  size_t kh, size_t kw, size_t stride_h, size_t stride_w, size_t pad_top, size_t pad_left);
+/* compute_resize (session.rs:1056-1132) over [planes, ih, iw] -> [planes, oh, ow]: nearest != 0 takes
+ * x[(h / scale) as usize][(w / scale) as usize], otherwise the reference's bilinear blend (its only
+ * other mode).  scale = output extent / input extent, per axis. */
+int ahip_resize(ahip_ctx *ctx, float *out, const float *x, size_t planes, size_t ih, size_t iw, size_t oh, size_t ow,
+                int nearest);
 
 /* ------------------------------------------------------------------------
  * Graph IR: the same Model / Graph / Node / Value / Op structure as

@@ -405,3 +405,14 @@ def max_pool(x, kernel, strides, pads=(0, 0, 0, 0)):
     if rc != OK:
         raise OracleError(rc, "max_pool")
     return out
+
+
+def resize(x, out_hw, nearest=True):
+    x = _f32(x)
+    b, c, ih, iw = x.shape
+    out = np.empty((b, c, out_hw[0], out_hw[1]), dtype=np.float32)
+    sz = ctypes.c_size_t
+    rc = lib().orc_resize(_fptr(x), _fptr(out), sz(b * c), sz(ih), sz(iw), sz(out_hw[0]), sz(out_hw[1]), int(bool(nearest)))
+    if rc != OK:
+        raise OracleError(rc, "resize")
+    return out

@@ -1142,6 +1142,34 @@ int orc_max_pool(const float *x, float *out, size_t planes, size_t ih, size_t iw
     return ORC_OK;
 }
 
+int orc_resize(const float *x, float *out, size_t planes, size_t ih, size_t iw, size_t oh, size_t ow, int nearest) {
+    if (ih == 0 || iw == 0) return ORC_ERR_ARG;
+    const float sh = (float)oh / (float)ih, sw = (float)ow / (float)iw;
+    for (size_t p = 0; p < planes; p++) {
+        const float *in = x + p * ih * iw;
+        float *o = out + p * oh * ow;
+        for (size_t h = 0; h < oh; h++)
+            for (size_t w = 0; w < ow; w++) {
+                if (nearest) {  // session.rs:1078-1090
+                    size_t y = (size_t)((float)h / sh), xx = (size_t)((float)w / sw);
+                    y = std::min(y, ih - 1);
+                    xx = std::min(xx, iw - 1);
+                    o[h * ow + w] = in[y * iw + xx];
+                } else {  // session.rs:1099-1121
+                    const float ihf = std::fmax((float)h / sh - 0.5f, 0.0f), iwf = std::fmax((float)w / sw - 0.5f, 0.0f);
+                    const size_t y = (size_t)ihf, xx = (size_t)iwf;
+                    const size_t y0 = std::min(y, ih - 1), y1 = std::min(y + 1, ih - 1);
+                    const size_t x0 = std::min(xx, iw - 1), x1 = std::min(xx + 1, iw - 1);
+                    const float v00 = in[y0 * iw + x0], v01 = in[y0 * iw + x1], v10 = in[y1 * iw + x0], v11 = in[y1 * iw + x1];
+                    const float hd = v00 + (v10 - v00) * (ihf - (float)y);
+                    const float hw = v01 + (v11 - v01) * (ihf - (float)y);
+                    o[h * ow + w] = hd + (hw - hd) * (iwf - (float)xx);
+                }
+            }
+    }
+    return ORC_OK;
+}
+
 float orc_fast_sum(const float *x, size_t n) { return fast_sum(x, n); }
 float orc_fast_sum_squares(const float *x, size_t n) { return fast_sum_squares(x, n); }
 

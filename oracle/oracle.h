@@ -189,6 +189,10 @@ int orc_conv2d(const float *x, const float *w, const float *bias, float *out, si
 int orc_max_pool(const float *x, float *out, size_t planes, size_t ih, size_t iw, size_t oh, size_t ow, size_t kh, size_t kw,
                  size_t sh, size_t sw, size_t pad_t, size_t pad_l);
 
+/* compute_resize (session.rs:1056-1132): nearest or the reference's bilinear blend; one scale per
+ * axis (the reference uses the height's scale for both, identical whenever they agree). */
+int orc_resize(const float *x, float *out, size_t planes, size_t ih, size_t iw, size_t oh, size_t ow, int nearest);
+
 float orc_fast_sum(const float *x, size_t n);
 float orc_fast_sum_squares(const float *x, size_t n);
 

@@ -78,3 +78,24 @@ def test_vit_patch_embedding_and_cnn_stem_through_the_session(case):
     conv = direct_conv(x2, w2, None, (2, 2), (1, 1, 1, 1), (1, 1), 1).astype(np.float32)
     assert conv.shape == (1, 8, 8, 9)
     assert_bits_equal(got, O.max_pool(np.maximum(conv, 0), (2, 2), (2, 2)), "cnn stem")
+
+
+def test_resize(ctx, case):
+    case("resize")
+    x = RNG.standard_normal((2, 3, 13, 17)).astype(np.float32)
+    for out_hw in [(26, 34), (13, 17), (39, 51), (20, 25), (6, 8), (1, 1)]:
+        for nearest in (True, False):
+            assert_bits_equal(ctx.resize(x, out_hw, nearest), O.resize(x, out_hw, nearest), f"resize {out_hw} nearest={nearest}")
+    # through the session, with `scales` (3 inputs) and with `sizes` (4 inputs)
+    for extra, mode in (([np.zeros(0, np.float32), np.array([1, 1, 2, 2], np.float32)], "nearest"),
+                        ([np.zeros(0, np.float32), np.zeros(0, np.float32), np.array([2, 3, 30, 40], np.int64)], "linear")):
+        m = Model(opset_version=13)
+        v = m.new_val_named_and_shaped("x", x.shape)
+        y = m.new_val()
+        m.add_node(Op.Resize, [v] + [m.new_initializer(e) for e in extra], [y], mode=mode, coordinate_transformation_mode="asymmetric",
+                   nearest_mode="floor")
+        m.add_input(v)
+        m.add_output(y)
+        (got,) = HipSessionBuilder(m).build().run([x])
+        want = O.resize(x, (26, 34), True) if mode == "nearest" else O.resize(x, (30, 40), False)
+        assert_bits_equal(got, want, f"session resize {mode}")

@@ -575,3 +575,26 @@ def test_max_pool_against_sliding_windows(oracle):
     nan[0, 0, 0, 0] = np.nan
     assert not np.isnan(oracle.max_pool(nan, (2, 2), (2, 2))).any()                                      # f32::max drops NaN
     assert np.array_equal(oracle.max_pool(np.full((1, 1, 2, 2), np.finfo(np.float32).min, np.float32), (2, 2), (2, 2)), [[[[0.0]]]])
+
+
+def test_resize_closed_forms(oracle):
+    rng = np.random.default_rng(15)
+    x = rng.standard_normal((2, 3, 5, 7)).astype(np.float32)
+    # nearest with an integer factor repeats pixels; factor 1 is the identity for both modes
+    assert np.array_equal(oracle.resize(x, (10, 14), nearest=True), x.repeat(2, axis=2).repeat(2, axis=3))
+    assert np.array_equal(oracle.resize(x, (15, 21), nearest=True), x.repeat(3, axis=2).repeat(3, axis=3))
+    assert np.array_equal(oracle.resize(x, (5, 7), nearest=True), x)
+    # downscaling by 2 keeps every other pixel: (h / 0.5) as usize = 2h
+    assert np.array_equal(oracle.resize(np.ascontiguousarray(x[:, :, :4, :6]), (2, 3), nearest=True), x[:, :, 0:4:2, 0:6:2])
+    # bilinear reproduces an affine image away from the clamped border: value at output pixel h is
+    # the input sampled at max(h / s - 0.5, 0)
+    yy, xx = np.meshgrid(np.arange(6, dtype=np.float32), np.arange(8, dtype=np.float32), indexing="ij")
+    ramp = (3 * yy - 2 * xx + 1).reshape(1, 1, 6, 8)
+    got = oracle.resize(ramp, (12, 16), nearest=False)[0, 0]
+    sy = np.minimum(np.maximum(np.arange(12) / 2 - 0.5, 0), 5)
+    sx = np.minimum(np.maximum(np.arange(16) / 2 - 0.5, 0), 7)
+    np.testing.assert_allclose(got, 3 * sy[:, None] - 2 * sx[None, :] + 1, rtol=0, atol=1e-5)
+    # a constant image stays constant, and the blend never leaves the range of its four neighbours
+    assert np.array_equal(oracle.resize(np.full((1, 1, 4, 4), 2.5, np.float32), (9, 9), nearest=False), np.full((1, 1, 9, 9), 2.5, np.float32))
+    up = oracle.resize(x, (13, 17), nearest=False)
+    assert up.min() >= x.min() - 1e-6 and up.max() <= x.max() + 1e-6
