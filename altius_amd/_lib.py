@@ -168,12 +168,15 @@ def _declare_graph(L):
     f("ahip_session_builder_with_intra_op_num_threads", [c_void_p, c_size_t])
     f("ahip_session_builder_with_profiling_enabled", [c_void_p, c_int])
     f("ahip_session_builder_with_device", [c_void_p, c_int])
+    f("ahip_session_builder_with_graph_replay", [c_void_p, c_int])
+    f("ahip_session_graph_replays", [c_void_p, P(c_size_t)])
     f("ahip_session_builder_build", [c_void_p, P(c_void_p)])
     f("ahip_session_free", [c_void_p], None)
     f("ahip_session_run", [c_void_p, c_int, P(c_void_p), c_int, P(c_void_p), P(c_int)])
     f("ahip_session_model", [c_void_p], c_void_p)
     f("ahip_session_profile", [c_void_p, c_int, P(c_char_p), P(c_double), P(c_int)])
     f("ahip_session_last_run_ms", [c_void_p, P(c_double)])
+    f("ahip_session_last_device_ms", [c_void_p, P(c_double)])
     f("ahip_session_device_allocations", [c_void_p, P(c_size_t)])
 
 

@@ -26,6 +26,7 @@ struct ahip_session_builder {
     size_t threads = 1;
     bool profiling = false;
     int device = 0;
+    bool graph_replay = false;
 };
 struct ahip_session {
     std::unique_ptr<HipSession> s;
@@ -510,11 +511,23 @@ int ahip_session_builder_with_device(ahip_session_builder *builder, int device) 
     return AHIP_OK;
 }
 
+int ahip_session_builder_with_graph_replay(ahip_session_builder *builder, int enable) {
+    if (!builder) return fail(AHIP_ERR_ARG, "null builder");
+    builder->graph_replay = enable != 0;
+    return AHIP_OK;
+}
+
+int ahip_session_graph_replays(const ahip_session *session, size_t *count) {
+    if (!session || !count) return fail(AHIP_ERR_ARG, "ahip_session_graph_replays: null argument");
+    *count = session->s->graph_replays();
+    return AHIP_OK;
+}
+
 int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **session) {
     if (!builder || !session) return fail(AHIP_ERR_ARG, "ahip_session_builder_build: null argument");
     *session = nullptr;
     HipSessionBuilder b(builder->model);
-    b.with_intra_op_num_threads(builder->threads).with_profiling_enabled(builder->profiling).with_device(builder->device);
+    b.with_intra_op_num_threads(builder->threads).with_profiling_enabled(builder->profiling).with_device(builder->device).with_graph_replay(builder->graph_replay);
     SessionError err;
     std::unique_ptr<HipSession> s = b.build(&err);
     if (!s) return fail(err.code(), err.to_string());
@@ -567,6 +580,12 @@ int ahip_session_profile(const ahip_session *session, int index, const char **op
     }
     if (op_name) *op_name = session->profile[index].first.c_str();
     if (ms) *ms = session->profile[index].second;
+    return AHIP_OK;
+}
+
+int ahip_session_last_device_ms(const ahip_session *session, double *ms) {
+    if (!session || !ms) return fail(AHIP_ERR_ARG, "ahip_session_last_device_ms: null argument");
+    *ms = session->s->last_device_ms();
     return AHIP_OK;
 }
 

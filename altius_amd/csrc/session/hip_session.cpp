@@ -62,7 +62,10 @@ size_t BufferPool::bucket_of(size_t bytes) {
     return (bytes + unit - 1) / unit * unit;
 }
 
-BufferPool::~BufferPool() { trim(); }
+BufferPool::~BufferPool() {
+    hold_ = false;
+    trim();
+}
 
 int BufferPool::acquire(size_t bytes, void **ptr, size_t *bucket) {
     const size_t b = bucket_of(bytes);
@@ -93,6 +96,7 @@ void BufferPool::release(void *ptr, size_t bucket) {
 }
 
 void BufferPool::trim() {
+    if (hold_) return;
     for (auto &kv : free_) {
         for (void *p : kv.second) {
             (void)hipFree(p);
@@ -109,6 +113,7 @@ std::unique_ptr<HipSession> HipSessionBuilder::build(SessionError *err) {
     s->model_ = std::move(model_);
     s->enable_profiling_ = enable_profiling_;
     s->intra_op_num_threads_ = intra_op_num_threads_;
+    s->graph_replay_ = graph_replay_ && !enable_profiling_;
 
     ShapeError serr;
     if (!infer_shapes(s->model_, &s->inferred_, nullptr, &serr)) {
@@ -124,6 +129,10 @@ std::unique_ptr<HipSession> HipSessionBuilder::build(SessionError *err) {
         return nullptr;
     }
     s->pool_.reset(new BufferPool(&s->ctx_));
+    if (hipEventCreate(&s->span_begin_) != hipSuccess || hipEventCreate(&s->span_end_) != hipSuccess) {
+        fail(err, SessionError::Hip, "hipEventCreate failed");
+        return nullptr;
+    }
 
     // Initializers live on the device for the lifetime of the session; their host contents stay
     // reachable for shape inference and shape arithmetic.
@@ -151,6 +160,9 @@ HipSession::~HipSession() {
     if (pool_) {
         (void)hipSetDevice(ctx_.device);
         (void)hipStreamSynchronize(ctx_.stream);
+        drop_graphs();
+        if (span_begin_) (void)hipEventDestroy(span_begin_);
+        if (span_end_) (void)hipEventDestroy(span_end_);
         inits_.clear();  // blocks go back to the pool before it is destroyed
         pool_.reset();
         destroy_device_ctx(&ctx_);
@@ -183,6 +195,10 @@ bool HipSession::upload(const Tensor &t, DeviceTensor *out, SessionError *err) {
 
 bool HipSession::fetch_host(DeviceTensor *t, SessionError *err) {
     if (t->host) return true;
+    if (capturing_) {  // a read-back would synchronise the capturing stream
+        capture_refused_ = true;
+        return fail(err, SessionError::Message, "graph capture: a node needs tensor contents on the host");
+    }
     Tensor h = Tensor::uninit_of_type(t->elem_ty, t->dims);
     if (!h.has_data()) return fail(err, SessionError::OutOfMemory, "out of host memory");
     if (t->nbytes()) {
@@ -207,6 +223,23 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
                     "run: " + std::to_string(inputs.size()) + " inputs given, the graph has " +
                         std::to_string(g.inputs.size()));
     if (hipSetDevice(ctx_.device) != hipSuccess) return fail(err, SessionError::Hip, "hipSetDevice failed");
+
+    if (graph_replay_) {
+        std::string key;
+        for (size_t i = 0; i < g.inputs.size(); i++)
+            key += std::to_string((int)inputs[i].elem_ty()) + inputs[i].dims().to_string() + ";";
+        auto it = graphs_.find(key);
+        if (it == graphs_.end() && eager_runs_[key] >= 1) {
+            if (!try_capture(key, inputs, err)) return false;
+            it = graphs_.find(key);
+        }
+        if (it != graphs_.end() && !it->second.unusable) {
+            if (!replay(it->second, inputs, outputs, err)) return false;
+            last_run_ms_ = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+            return true;
+        }
+        eager_runs_[key]++;
+    }
 
     std::map<ValueId, DeviceTensor> values;
     std::vector<hipEvent_t> events;
@@ -243,6 +276,7 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
     }
 
     // The hot loop (session.rs:86-92).
+    (void)hipEventRecord(span_begin_, ctx_.stream);
     for (size_t i = 0; i < plan_.size(); i++) {
         if (!run_node(plan_[i].node_id, values, err)) return finish(false);
         if (enable_profiling_) (void)hipEventRecord(events[i + 1], ctx_.stream);
@@ -251,6 +285,8 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
         for (ValueId v : plan_[i].free_vals)
             if (std::find(g.outputs.begin(), g.outputs.end(), v) == g.outputs.end()) values.erase(v);
     }
+
+    (void)hipEventRecord(span_end_, ctx_.stream);
 
     // Download the outputs (session.rs:127-133).
     for (ValueId v : g.outputs) {
@@ -277,6 +313,8 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
         outputs->clear();
         return finish(fail_code(err, rc, ctx_.last_error));
     }
+    float span_ms = 0;
+    last_device_ms_ = hipEventElapsedTime(&span_ms, span_begin_, span_end_) == hipSuccess ? span_ms : 0;
     if (enable_profiling_) {
         for (size_t i = 0; i < plan_.size(); i++) {
             float ms = 0;
@@ -286,6 +324,120 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
     }
     finish(true);
     last_run_ms_ = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+    return true;
+}
+
+void HipSession::drop_graphs() {
+    for (auto &kv : graphs_)
+        if (kv.second.exec) (void)hipGraphExecDestroy(kv.second.exec);
+    graphs_.clear();
+    if (pool_) pool_->hold_memory(false);
+}
+
+// Records the node loop for these input shapes.  Returns false only for errors that should fail
+// the run; a refused capture marks the signature unusable and returns true.
+bool HipSession::try_capture(const std::string &key, const std::vector<Tensor> &inputs, SessionError *err) {
+    const Graph &g = model_.graph;
+    CapturedRun run;
+    std::map<ValueId, DeviceTensor> values;
+    for (size_t i = 0; i < g.inputs.size(); i++) {
+        DeviceTensor d;
+        if (!allocate(TypedFixedShape{inputs[i].dims(), inputs[i].elem_ty()}, &d, err)) return false;
+        run.inputs.push_back(d);
+        values[g.inputs[i]] = d;
+    }
+    if (hipStreamBeginCapture(ctx_.stream, hipStreamCaptureModeRelaxed) != hipSuccess) {
+        (void)hipGetLastError();
+        graphs_[key].unusable = true;
+        return true;
+    }
+    capturing_ = true;
+    capture_refused_ = false;
+    ctx_.flags_armed = false;
+    bool ok = true;
+    SessionError local;
+    for (size_t i = 0; i < plan_.size() && ok; i++) {
+        ok = run_node(plan_[i].node_id, values, &local);
+        if (!ok) break;
+        for (ValueId v : plan_[i].free_vals)
+            if (std::find(g.outputs.begin(), g.outputs.end(), v) == g.outputs.end()) values.erase(v);
+    }
+    capturing_ = false;
+    hipGraph_t graph = nullptr;
+    const hipError_t end = hipStreamEndCapture(ctx_.stream, &graph);
+    run.has_gather = ctx_.flags_armed;
+    ctx_.flags_armed = false;
+    // A capture that had to grow the pool recorded kernels against fresh blocks: still valid, the
+    // blocks stay in the pool.  A capture that failed for any reason leaves the eager path in charge.
+    if (ok && end == hipSuccess && graph) {
+        for (ValueId v : g.outputs) {
+            auto it = values.find(v);
+            const DeviceTensor *d = it != values.end() ? &it->second : nullptr;
+            if (!d) {
+                auto ii = inits_.find(v);
+                if (ii != inits_.end()) d = &ii->second;
+            }
+            if (!d) {
+                ok = false;
+                break;
+            }
+            run.outputs.push_back(*d);  // holds the block: the recorded kernels write here on every replay
+        }
+    }
+    if (ok && end == hipSuccess && graph && hipGraphInstantiate(&run.exec, graph, nullptr, nullptr, 0) == hipSuccess) {
+        (void)hipGraphDestroy(graph);
+        graphs_[key] = std::move(run);
+        pool_->hold_memory(true);
+        return true;
+    }
+    (void)hipGetLastError();
+    if (graph) (void)hipGraphDestroy(graph);
+    if (!ok && !capture_refused_) {  // a real error (unsupported operator, bad shapes): report it as the eager run would
+        if (err) *err = local;
+        return false;
+    }
+    graphs_[key].unusable = true;
+    return true;
+}
+
+bool HipSession::replay(CapturedRun &run, const std::vector<Tensor> &inputs, std::vector<Tensor> *outputs, SessionError *err) {
+    int rc = AHIP_OK;
+    for (size_t i = 0; i < run.inputs.size(); i++)
+        if (!inputs[i].has_data()) return fail(err, SessionError::Argument, "run: input " + std::to_string(i) + " has no data");
+    for (size_t i = 0; i < run.inputs.size() && !rc; i++)
+        if (run.inputs[i].nbytes())
+            rc = ctx_.check(hipMemcpyAsync(run.inputs[i].ptr, inputs[i].data_as_bytes(), run.inputs[i].nbytes(), hipMemcpyHostToDevice,
+                                           ctx_.stream),
+                            "hipMemcpyAsync(input)");
+    (void)hipEventRecord(span_begin_, ctx_.stream);
+    if (!rc) rc = ctx_.check(hipGraphLaunch(run.exec, ctx_.stream), "hipGraphLaunch");
+    (void)hipEventRecord(span_end_, ctx_.stream);
+    for (size_t i = 0; i < run.outputs.size() && !rc; i++) {
+        Tensor t = Tensor::uninit_of_type(run.outputs[i].elem_ty, run.outputs[i].dims, pinned_host_block);
+        if (!t.has_data()) {
+            (void)hipStreamSynchronize(ctx_.stream);
+            outputs->clear();
+            return fail(err, SessionError::OutOfMemory, "run: out of host memory for an output tensor");
+        }
+        if (run.outputs[i].nbytes())
+            rc = ctx_.check(hipMemcpyAsync(t.data_as_bytes_mut(), run.outputs[i].ptr, run.outputs[i].nbytes(), hipMemcpyDeviceToHost,
+                                           ctx_.stream),
+                            "hipMemcpyAsync(output)");
+        outputs->push_back(std::move(t));
+    }
+    const int rs = ctx_.check(hipStreamSynchronize(ctx_.stream), "hipStreamSynchronize(run)");
+    if (!rc) rc = rs;
+    if (!rc && run.has_gather) {
+        ctx_.flags_armed = true;
+        rc = check_device_flags(ctx_);
+    }
+    if (rc) {
+        outputs->clear();
+        return fail_code(err, rc, ctx_.last_error);
+    }
+    float span_ms = 0;
+    last_device_ms_ = hipEventElapsedTime(&span_ms, span_begin_, span_end_) == hipSuccess ? span_ms : 0;
+    graph_replays_++;
     return true;
 }
 
@@ -340,6 +492,9 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
     if (cached != inferred_.end()) {
         op = cached->second.first;
         shapes = cached->second.second;
+    } else if (capturing_) {
+        capture_refused_ = true;
+        return fail(err, SessionError::Message, "graph capture: a node's shape is not known before the run");
     } else {
         static const Tensor absent;
         for (int attempt = 0;; attempt++) {
@@ -390,6 +545,10 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
                 for (auto *d : in)
                     if (d && !fetch_host(d, err)) return false;
             }
+        }
+        if (on_host && capturing_) {
+            capture_refused_ = true;
+            return fail(err, SessionError::Message, "graph capture: a node is evaluated on the host");
         }
         if (on_host) {
             std::vector<const Tensor *> hin;

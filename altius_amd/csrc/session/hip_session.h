@@ -40,7 +40,9 @@ public:
     ~BufferPool();
     int acquire(size_t bytes, void **ptr, size_t *bucket);
     void release(void *ptr, size_t bucket);
-    void trim();  // returns every cached block to the device
+    void trim();  // returns every cached block to the device (a no-op while trimming is held off)
+    // Recorded HIP graphs address cached blocks directly: while one exists nothing may be freed.
+    void hold_memory(bool hold) { hold_ = hold; }
     size_t bytes_reserved() const { return reserved_; }
     size_t device_allocations() const { return allocations_; }
 
@@ -50,6 +52,7 @@ private:
     std::map<size_t, std::vector<void *>> free_;
     size_t reserved_ = 0;
     size_t allocations_ = 0;
+    bool hold_ = false;
 };
 
 // A block of pooled device memory; goes back to its pool when the last tensor using it is dropped.
@@ -94,7 +97,12 @@ public:
     // profiling is enabled), keyed by Op::name().
     const std::map<std::string, double> &last_profile() const { return profile_; }
     double last_run_ms() const { return last_run_ms_; }
+    // Device time of the last run's kernels alone (between the uploads and the downloads), from two
+    // events on the session's stream.
+    double last_device_ms() const { return last_device_ms_; }
     size_t device_allocations() const { return pool_->device_allocations(); }
+    // Runs served by replaying a captured HIP graph since the session was built.
+    size_t graph_replays() const { return graph_replays_; }
     const std::vector<NodeExecutionPlan> &execution_plan() const { return plan_; }
     const InferredShapes &inferred_shapes() const { return inferred_; }
 
@@ -112,6 +120,20 @@ private:
     bool run_device_op(const Node &node, const Op &op, const std::vector<DeviceTensor *> &in,
                        const std::vector<TypedFixedShape> &shapes, std::vector<DeviceTensor> *outs, SessionError *err);
 
+    // A run recorded as a HIP graph for one set of input shapes: replaying it issues every kernel
+    // of the plan with one launch.  The graph refers to pool blocks by address, which stays valid
+    // because the pool never returns memory to the device while a graph exists.
+    struct CapturedRun {
+        hipGraphExec_t exec = nullptr;
+        std::vector<DeviceTensor> inputs;   // persistent device copies of the graph inputs
+        std::vector<DeviceTensor> outputs;  // where the recorded kernels leave the graph outputs
+        bool has_gather = false;
+        bool unusable = false;              // capture was tried and refused; run eagerly from now on
+    };
+    bool try_capture(const std::string &key, const std::vector<Tensor> &inputs, SessionError *err);
+    bool replay(CapturedRun &run, const std::vector<Tensor> &inputs, std::vector<Tensor> *outputs, SessionError *err);
+    void drop_graphs();
+
     Model model_;
     std::vector<NodeExecutionPlan> plan_;
     InferredShapes inferred_;
@@ -122,7 +144,15 @@ private:
     std::map<ValueId, DeviceTensor> inits_;  // uploaded once at build
     std::map<std::string, double> profile_;
     double last_run_ms_ = 0;
+    double last_device_ms_ = 0;
+    hipEvent_t span_begin_ = nullptr, span_end_ = nullptr;  // bracket the kernels of a run
     std::mutex mutex_;
+    bool graph_replay_ = false;
+    bool capturing_ = false;        // a stream capture is in progress: nothing may synchronise
+    bool capture_refused_ = false;  // a node needed the host during capture
+    std::map<std::string, CapturedRun> graphs_;
+    std::map<std::string, int> eager_runs_;  // per input signature: eager runs so far (the pool is warm after one)
+    size_t graph_replays_ = 0;
 };
 
 class HipSessionBuilder {
@@ -135,6 +165,14 @@ public:
     }
     HipSessionBuilder &with_profiling_enabled(bool enable) {
         enable_profiling_ = enable;
+        return *this;
+    }
+    // Not in the reference: record each distinct input-shape signature as a HIP graph on its second
+    // run and replay it afterwards (one launch per run instead of one per node).  Off by default.
+    // Graphs whose shapes or operands need the host during the run, and profiled sessions, keep
+    // running node by node.
+    HipSessionBuilder &with_graph_replay(bool enable) {
+        graph_replay_ = enable;
         return *this;
     }
     // Not in the reference: which GPU to run on (default 0).
@@ -151,6 +189,7 @@ private:
     size_t intra_op_num_threads_ = 1;
     bool enable_profiling_ = false;
     int device_ = 0;
+    bool graph_replay_ = false;
 };
 
 }  // namespace altius

@@ -54,6 +54,17 @@ class HipSession:
         check(self.L.ahip_session_last_run_ms(self.handle, ctypes.byref(ms)))
         return ms.value
 
+    def last_device_ms(self):
+        """Device time of the last run's kernels alone (uploads and downloads excluded)."""
+        ms = ctypes.c_double()
+        check(self.L.ahip_session_last_device_ms(self.handle, ctypes.byref(ms)))
+        return ms.value
+
+    def graph_replays(self):
+        c = ctypes.c_size_t()
+        check(self.L.ahip_session_graph_replays(self.handle, ctypes.byref(c)))
+        return c.value
+
     def device_allocations(self):
         c = ctypes.c_size_t()
         check(self.L.ahip_session_device_allocations(self.handle, ctypes.byref(c)))
@@ -80,6 +91,11 @@ class HipSessionBuilder:
 
     def with_profiling_enabled(self, enable):
         check(self.L.ahip_session_builder_with_profiling_enabled(self.handle, int(bool(enable))))
+        return self
+
+    def with_graph_replay(self, enable=True):
+        """Record each input-shape signature as a HIP graph on its second run and replay it afterwards."""
+        check(self.L.ahip_session_builder_with_graph_replay(self.handle, int(bool(enable))))
         return self
 
     def with_device(self, device):

@@ -197,18 +197,24 @@ def session_table(synth):
     rows = []
 
     def measure(name, model, x, alg_bytes):
-        sess = HipSessionBuilder(model).with_profiling_enabled(True).build()
-        best_run, best_dev = float("inf"), float("inf")
         t_in = Tensor.from_numpy(x)              # the caller's host tensor, as the reference's run() takes it
-        for _ in range(5):
-            outs = sess.run([t_in], copy=False)
-            best_run = min(best_run, sess.last_run_ms())
-            best_dev = min(best_dev, sum(sess.profile().values()))
-            del outs                             # output tensors dropped, as a caller would after use
-        rows.append({"graph": name, "algorithmic_bytes": alg_bytes, "kernels_us": round(best_dev * 1e3, 1),
-                     "run_ms_with_pcie": round(best_run, 3),
-                     "kernels_GBps": round(alg_bytes / (best_dev * 1e-3) / 1e9, 1)})
-        sess.close()
+        row = {"graph": name, "algorithmic_bytes": alg_bytes}
+        # Node by node, then with the run recorded as a HIP graph and replayed (one launch per run).
+        for key, replay in (("kernels_us", False), ("kernels_us_graph_replay", True)):
+            sess = HipSessionBuilder(model.clone()).with_graph_replay(replay).build()
+            best_run, best_dev = float("inf"), float("inf")
+            for _ in range(7):
+                outs = sess.run([t_in], copy=False)
+                best_run = min(best_run, sess.last_run_ms())
+                best_dev = min(best_dev, sess.last_device_ms())
+                del outs                         # output tensors dropped, as a caller would after use
+            if replay:
+                assert sess.graph_replays() == 6, sess.graph_replays()
+            row[key] = round(best_dev * 1e3, 1)
+            row["run_ms_with_pcie" + ("_graph_replay" if replay else "")] = round(best_run, 3)
+            sess.close()
+        row["kernels_GBps"] = round(alg_bytes / (row["kernels_us_graph_replay"] * 1e-6) / 1e9, 1)
+        rows.append(row)
 
     c2 = synth.cfg2()
     X, r = c2["x"].nbytes, 32 * 197 * 4
@@ -459,8 +465,9 @@ def main():
             log("%-44s %14d %10.2f %10.1f %8.1f" % (o.name, o.nbytes, ms * 1e3, gbps, 100.0 * gbps / HBM_PEAK_GBPS))
         graphs_rows = session_table(synth)
         for r in graphs_rows:
-            log("%-40s kernels %9.1f us (%7.1f GB/s)   run() incl. PCIe %9.3f ms"
-                % (r["graph"], r["kernels_us"], r["kernels_GBps"], r["run_ms_with_pcie"]))
+            log("%-40s kernels %8.1f us, as one HIP graph %8.1f us (%7.1f GB/s)   run() incl. PCIe %8.3f / %8.3f ms"
+                % (r["graph"], r["kernels_us"], r["kernels_us_graph_replay"], r["kernels_GBps"], r["run_ms_with_pcie"],
+                   r["run_ms_with_pcie_graph_replay"]))
         result["other_configs"] = {"kernels": others, "graphs": graphs_rows}
 
     if args.next_rows:

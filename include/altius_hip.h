@@ -409,6 +409,11 @@ int ahip_session_builder_with_intra_op_num_threads(ahip_session_builder *builder
 int ahip_session_builder_with_profiling_enabled(ahip_session_builder *builder, int enable);
 /* Not in the reference: the GPU to run on (default 0). */
 int ahip_session_builder_with_device(ahip_session_builder *builder, int device);
+/* Not in the reference: with enable != 0 the session records the kernels of a run as a HIP graph
+ * the second time it sees a set of input shapes and replays that graph afterwards (one launch per
+ * run instead of one per node).  Results are those of the node-by-node run.  Graphs whose shapes
+ * or operands need the host during the run, and profiled sessions, keep running node by node. */
+int ahip_session_builder_with_graph_replay(ahip_session_builder *builder, int enable);
 /* build(): shape inference (AHIP_ERR_SHAPE on failure), execution plan, device context,
  * upload of the initializers.  The builder stays valid and must still be freed. */
 int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **session);
@@ -427,8 +432,13 @@ const ahip_model *ahip_session_model(const ahip_session *session);
 int ahip_session_profile(const ahip_session *session, int index, const char **op_name, double *ms,
                          int *count);
 int ahip_session_last_run_ms(const ahip_session *session, double *ms);
+/* Not in the reference: device time of the last run's kernels alone (between the uploads and the
+ * downloads), measured by two events on the session's stream. */
+int ahip_session_last_device_ms(const ahip_session *session, double *ms);
 /* Number of hipMalloc calls the session's buffer pool has made so far. */
 int ahip_session_device_allocations(const ahip_session *session, size_t *count);
+/* Runs served by replaying a recorded HIP graph so far. */
+int ahip_session_graph_replays(const ahip_session *session, size_t *count);
 
 #ifdef __cplusplus
 }
