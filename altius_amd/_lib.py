@@ -173,6 +173,14 @@ def _declare_graph(L):
     f("ahip_session_builder_build", [c_void_p, P(c_void_p)])
     f("ahip_session_free", [c_void_p], None)
     f("ahip_session_run", [c_void_p, c_int, P(c_void_p), c_int, P(c_void_p), P(c_int)])
+    f("ahip_session_run_device", [c_void_p, c_int, P(c_void_p), P(c_int), P(c_int), P(P(c_int64)), c_int, P(c_void_p), P(c_int)])
+    f("ahip_session_synchronize", [c_void_p])
+    f("ahip_device_tensor_free", [c_void_p], None)
+    f("ahip_device_tensor_ptr", [c_void_p], c_void_p)
+    f("ahip_device_tensor_elem_type", [c_void_p])
+    f("ahip_device_tensor_rank", [c_void_p])
+    f("ahip_device_tensor_dims", [c_void_p, P(c_int64), c_int])
+    f("ahip_device_tensor_nbytes", [c_void_p], c_size_t)
     f("ahip_session_model", [c_void_p], c_void_p)
     f("ahip_session_profile", [c_void_p, c_int, P(c_char_p), P(c_double), P(c_int)])
     f("ahip_session_last_run_ms", [c_void_p, P(c_double)])

@@ -29,9 +29,17 @@ struct ahip_session_builder {
     bool graph_replay = false;
 };
 struct ahip_session {
-    std::unique_ptr<HipSession> s;
+    std::shared_ptr<HipSession> s;  // shared with the device tensors the session has handed out
     ahip_model view;  // what ahip_session_model hands out (a copy of the session's model)
     std::vector<std::pair<std::string, double>> profile;
+};
+
+struct ahip_device_tensor {
+    DeviceTensor t;
+    std::shared_ptr<HipSession> owner;  // keeps the pool (and the device context) alive
+    ~ahip_device_tensor() {
+        if (owner) owner->release(&t);
+    }
 };
 
 namespace {
@@ -566,6 +574,66 @@ int ahip_session_run(ahip_session *session, int n_inputs, const ahip_tensor *con
         outputs[i] = t;
     }
     session->profile.assign(session->s->last_profile().begin(), session->s->last_profile().end());
+    return AHIP_OK;
+}
+
+int ahip_session_run_device(ahip_session *session, int n_inputs, const void *const *device_ptrs, const int *elem_types,
+                            const int *ranks, const int64_t *const *dims, int output_capacity,
+                            ahip_device_tensor **outputs, int *n_outputs) {
+    if (!session || n_inputs < 0 || (n_inputs && (!device_ptrs || !elem_types || !ranks || !dims)) || output_capacity < 0 ||
+        (output_capacity && !outputs) || !n_outputs)
+        return fail(AHIP_ERR_ARG, "ahip_session_run_device: invalid argument");
+    std::vector<DeviceTensor> in(n_inputs);
+    for (int i = 0; i < n_inputs; i++) {
+        if (!valid_elem_type(elem_types[i])) return fail(AHIP_ERR_ARG, "ahip_session_run_device: unknown element type");
+        if (ranks[i] < 0 || ranks[i] > AHIP_MAX_RANK || (ranks[i] && !dims[i]))
+            return fail(AHIP_ERR_ARG, "ahip_session_run_device: bad rank or null dims");
+        for (int k = 0; k < ranks[i]; k++)
+            if (dims[i][k] < 0) return fail(AHIP_ERR_ARG, "ahip_session_run_device: negative dimension");
+        in[i].dims = FixedDimensions::from_i64(dims[i], (size_t)ranks[i]);
+        in[i].elem_ty = static_cast<TensorElemType>(elem_types[i]);
+        in[i].ptr = const_cast<void *>(device_ptrs[i]);
+    }
+    std::vector<DeviceTensor> out;
+    SessionError err;
+    if (!session->s->run_device(in, &out, &err)) return fail(err.code(), err.to_string());
+    *n_outputs = (int)out.size();
+    auto drop_all = [&](size_t made) {
+        for (size_t j = 0; j < made; j++) delete outputs[j];
+        for (auto &t : out) session->s->release(&t);
+    };
+    if ((int)out.size() > output_capacity) {
+        drop_all(0);
+        return fail(AHIP_ERR_ARG, "ahip_session_run_device: output capacity too small");
+    }
+    for (size_t i = 0; i < out.size(); i++) {
+        ahip_device_tensor *t = new (std::nothrow) ahip_device_tensor();
+        if (!t) {
+            drop_all(i);
+            return fail(AHIP_ERR_OOM, "ahip_session_run_device: out of host memory");
+        }
+        t->t = std::move(out[i]);
+        t->owner = session->s;
+        outputs[i] = t;
+    }
+    return AHIP_OK;
+}
+
+int ahip_session_synchronize(ahip_session *session) {
+    if (!session) return fail(AHIP_ERR_ARG, "ahip_session_synchronize: null session");
+    SessionError err;
+    if (!session->s->synchronize(&err)) return fail(err.code(), err.to_string());
+    return AHIP_OK;
+}
+
+void ahip_device_tensor_free(ahip_device_tensor *tensor) { delete tensor; }
+void *ahip_device_tensor_ptr(const ahip_device_tensor *tensor) { return tensor ? tensor->t.ptr : nullptr; }
+int ahip_device_tensor_elem_type(const ahip_device_tensor *tensor) { return tensor ? (int)tensor->t.elem_ty : -1; }
+int ahip_device_tensor_rank(const ahip_device_tensor *tensor) { return tensor ? (int)tensor->t.dims.len() : -1; }
+size_t ahip_device_tensor_nbytes(const ahip_device_tensor *tensor) { return tensor ? tensor->t.nbytes() : 0; }
+int ahip_device_tensor_dims(const ahip_device_tensor *tensor, int64_t *dims, int capacity) {
+    if (!tensor || capacity < 0 || (capacity && !dims)) return fail(AHIP_ERR_ARG, "ahip_device_tensor_dims: invalid argument");
+    for (int i = 0; i < capacity && i < (int)tensor->t.dims.len(); i++) dims[i] = (int64_t)tensor->t.dims[i];
     return AHIP_OK;
 }
 

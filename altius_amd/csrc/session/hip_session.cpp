@@ -211,6 +211,18 @@ bool HipSession::fetch_host(DeviceTensor *t, SessionError *err) {
     return true;
 }
 
+// The shapes cached at build time were derived from the declared input shapes: kernels sized by
+// them must never see a tensor of another extent.
+bool HipSession::check_input(size_t i, TensorElemType elem_ty, const FixedDimensions &dims, SessionError *err) const {
+    const auto &declared = model_.graph.values[model_.graph.inputs[i]].shape;
+    if (!declared) return true;
+    const auto fixed = declared->dims.as_fixed_dims();
+    if (fixed && *fixed == dims && declared->elem_ty == elem_ty) return true;
+    return fail(err, SessionError::Shape,
+                "run: input " + std::to_string(i) + " is " + elem_name(elem_ty) + dims.to_string() +
+                    " but the graph declares " + elem_name(declared->elem_ty) + (fixed ? fixed->to_string() : "a dynamic shape"));
+}
+
 bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *outputs, SessionError *err) {
     std::lock_guard<std::mutex> lock(mutex_);
     const auto t0 = std::chrono::steady_clock::now();
@@ -223,6 +235,8 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
                     "run: " + std::to_string(inputs.size()) + " inputs given, the graph has " +
                         std::to_string(g.inputs.size()));
     if (hipSetDevice(ctx_.device) != hipSuccess) return fail(err, SessionError::Hip, "hipSetDevice failed");
+    for (size_t i = 0; i < g.inputs.size(); i++)
+        if (!check_input(i, inputs[i].elem_ty(), inputs[i].dims(), err)) return false;
 
     if (graph_replay_) {
         std::string key;
@@ -325,6 +339,77 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
     finish(true);
     last_run_ms_ = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     return true;
+}
+
+bool HipSession::run_device(const std::vector<DeviceTensor> &inputs, std::vector<DeviceTensor> *outputs, SessionError *err) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    const auto t0 = std::chrono::steady_clock::now();
+    if (!outputs) return fail(err, SessionError::Argument, "run_device: null output vector");
+    outputs->clear();
+    profile_.clear();
+    const Graph &g = model_.graph;
+    if (inputs.size() < g.inputs.size())
+        return fail(err, SessionError::Argument,
+                    "run_device: " + std::to_string(inputs.size()) + " inputs given, the graph has " +
+                        std::to_string(g.inputs.size()));
+    if (hipSetDevice(ctx_.device) != hipSuccess) return fail(err, SessionError::Hip, "hipSetDevice failed");
+
+    std::map<ValueId, DeviceTensor> values;
+    for (size_t i = 0; i < g.inputs.size(); i++) {
+        if (!inputs[i].ptr && inputs[i].nbytes())
+            return fail(err, SessionError::Argument, "run_device: input " + std::to_string(i) + " has no device pointer");
+        if (!check_input(i, inputs[i].elem_ty, inputs[i].dims, err)) return false;
+        DeviceTensor d;
+        d.dims = inputs[i].dims;
+        d.elem_ty = inputs[i].elem_ty;
+        d.ptr = inputs[i].ptr;  // the caller's memory: no block, never returned to the pool
+        values[g.inputs[i]] = std::move(d);
+    }
+    // A failed run leaves nothing behind; blocks released while kernels are still queued are only
+    // handed to later work on the same stream.
+    (void)hipEventRecord(span_begin_, ctx_.stream);
+    for (size_t i = 0; i < plan_.size(); i++) {
+        if (!run_node(plan_[i].node_id, values, err)) return false;
+        for (ValueId v : plan_[i].free_vals)
+            if (std::find(g.outputs.begin(), g.outputs.end(), v) == g.outputs.end()) values.erase(v);
+    }
+    (void)hipEventRecord(span_end_, ctx_.stream);
+    for (ValueId v : g.outputs) {
+        const DeviceTensor *d = nullptr;
+        auto it = values.find(v);
+        if (it != values.end()) d = &it->second;
+        else {
+            auto ii = inits_.find(v);
+            if (ii != inits_.end()) d = &ii->second;
+        }
+        if (!d) {
+            outputs->clear();
+            return fail(err, SessionError::Message, "run_device: graph output was not produced");
+        }
+        outputs->push_back(*d);
+    }
+    span_pending_ = true;
+    last_run_ms_ = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+    return true;
+}
+
+bool HipSession::synchronize(SessionError *err) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    if (hipSetDevice(ctx_.device) != hipSuccess) return fail(err, SessionError::Hip, "hipSetDevice failed");
+    int rc = ctx_.check(hipStreamSynchronize(ctx_.stream), "hipStreamSynchronize");
+    if (!rc) rc = check_device_flags(ctx_);
+    if (rc) return fail_code(err, rc, ctx_.last_error);
+    if (span_pending_) {
+        span_pending_ = false;
+        float span_ms = 0;
+        last_device_ms_ = hipEventElapsedTime(&span_ms, span_begin_, span_end_) == hipSuccess ? span_ms : 0;
+    }
+    return true;
+}
+
+void HipSession::release(DeviceTensor *t) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    *t = DeviceTensor();
 }
 
 void HipSession::drop_graphs() {

@@ -93,6 +93,18 @@ public:
     // device, and returns graph.outputs in order.  Calls are serialised.
     bool run(const std::vector<Tensor> &inputs, std::vector<Tensor> *outputs, SessionError *err);
 
+    // Not in the reference: the same run on tensors that already live on the session's GPU.
+    // inputs[i] describes caller-owned device memory (ptr, dims, element type; no block), read in
+    // stream order: it must hold its data before the call and stay valid until synchronize().
+    // Outputs are device tensors whose memory belongs to the session's pool (or, for an output
+    // that is a reshaped view of an input, the caller's own pointer); they hold results once
+    // synchronize() has returned.  Nothing crosses PCIe and the call does not wait for the GPU.
+    bool run_device(const std::vector<DeviceTensor> &inputs, std::vector<DeviceTensor> *outputs, SessionError *err);
+    // Waits for the session's stream and reports errors that kernels leave in device flags.
+    bool synchronize(SessionError *err);
+    // Drops a tensor run_device() returned; its block goes back to the pool for later nodes.
+    void release(DeviceTensor *t);
+
     // Per-operator device time of the last run, in milliseconds (filled when
     // profiling is enabled), keyed by Op::name().
     const std::map<std::string, double> &last_profile() const { return profile_; }
@@ -130,6 +142,7 @@ private:
         bool has_gather = false;
         bool unusable = false;              // capture was tried and refused; run eagerly from now on
     };
+    bool check_input(size_t i, TensorElemType elem_ty, const FixedDimensions &dims, SessionError *err) const;
     bool try_capture(const std::string &key, const std::vector<Tensor> &inputs, SessionError *err);
     bool replay(CapturedRun &run, const std::vector<Tensor> &inputs, std::vector<Tensor> *outputs, SessionError *err);
     void drop_graphs();
@@ -145,6 +158,7 @@ private:
     std::map<std::string, double> profile_;
     double last_run_ms_ = 0;
     double last_device_ms_ = 0;
+    bool span_pending_ = false;  // run_device() recorded the span; synchronize() reads it
     hipEvent_t span_begin_ = nullptr, span_end_ = nullptr;  // bracket the kernels of a run
     std::mutex mutex_;
     bool graph_replay_ = false;

@@ -6,7 +6,43 @@ import numpy as np
 
 from . import _lib
 from ._lib import check
-from .graph import Model, Tensor
+from .graph import _ELEM_OF, _NP_OF, Model, Tensor
+
+
+class DeviceTensor:
+    """An output of HipSession.run_device: memory on the session's GPU, released by free() (or when
+    the object is dropped)."""
+
+    def __init__(self, handle):
+        self.L = _lib.lib()
+        self.handle = handle
+
+    def __del__(self):
+        self.free()
+
+    def free(self):
+        if getattr(self, "handle", None):
+            self.L.ahip_device_tensor_free(self.handle)
+            self.handle = None
+
+    @property
+    def ptr(self):
+        return self.L.ahip_device_tensor_ptr(self.handle) or 0
+
+    @property
+    def shape(self):
+        rank = self.L.ahip_device_tensor_rank(self.handle)
+        dims = (ctypes.c_int64 * max(rank, 1))()
+        check(self.L.ahip_device_tensor_dims(self.handle, dims, rank))
+        return tuple(dims[i] for i in range(rank))
+
+    @property
+    def dtype(self):
+        return np.dtype(_NP_OF[self.L.ahip_device_tensor_elem_type(self.handle)])
+
+    @property
+    def nbytes(self):
+        return self.L.ahip_device_tensor_nbytes(self.handle)
 
 
 class HipSession:
@@ -37,6 +73,25 @@ class HipSession:
         check(self.L.ahip_session_run(self.handle, len(tensors), arr, cap, outs, ctypes.byref(n)))
         tensors_out = [Tensor(ctypes.c_void_p(outs[i])) for i in range(n.value)]
         return [t.numpy() if copy else t.view() for t in tensors_out]
+
+    def run_device(self, inputs):
+        """inputs: (device pointer, shape, numpy dtype) triples, positional in graph.inputs order, on the
+        session's GPU.  Enqueues the plan and returns DeviceTensors without waiting for the GPU; call
+        synchronize() before reading them from another stream or copying them out."""
+        n_in = len(inputs)
+        ptrs = (ctypes.c_void_p * max(n_in, 1))(*[int(p) for p, _, _ in inputs])
+        elem = (ctypes.c_int * max(n_in, 1))(*[_ELEM_OF[np.dtype(dt)] for _, _, dt in inputs])
+        ranks = (ctypes.c_int * max(n_in, 1))(*[len(shape) for _, shape, _ in inputs])
+        dim_arrays = [(ctypes.c_int64 * max(len(shape), 1))(*[int(d) for d in shape]) for _, shape, _ in inputs]
+        dims = (ctypes.POINTER(ctypes.c_int64) * max(n_in, 1))(*[ctypes.cast(a, ctypes.POINTER(ctypes.c_int64)) for a in dim_arrays])
+        cap = 16
+        outs = (ctypes.c_void_p * cap)()
+        n = ctypes.c_int()
+        check(self.L.ahip_session_run_device(self.handle, n_in, ptrs, elem, ranks, dims, cap, outs, ctypes.byref(n)))
+        return [DeviceTensor(ctypes.c_void_p(outs[i])) for i in range(n.value)]
+
+    def synchronize(self):
+        check(self.L.ahip_session_synchronize(self.handle))
 
     def profile(self):
         """{op name: device milliseconds} of the last run (profiling enabled)."""

@@ -425,6 +425,29 @@ void ahip_session_free(ahip_session *session);
  * are serialised internally. */
 int ahip_session_run(ahip_session *session, int n_inputs, const ahip_tensor *const *inputs,
                      int output_capacity, ahip_tensor **outputs, int *n_outputs);
+/* Not in the reference (its tensors are host memory): the same run on tensors that already live on
+ * the session's GPU, so that nothing crosses PCIe.  Input i is `device_ptrs[i]`, caller-owned device
+ * memory holding a dense row-major tensor of `elem_types[i]` (ahip_elem_type) and `dims[i][0..ranks[i])`.
+ * The call enqueues the whole plan on the session's stream and returns without waiting: inputs are
+ * read in stream order (they must hold their data before the call and stay valid until
+ * ahip_session_synchronize), and the outputs hold their results once ahip_session_synchronize has
+ * returned.  Outputs are device tensors in graph-output order; their memory belongs to the session's
+ * pool, except that an output which is a reshaped view of an input is the caller's own pointer.
+ * Free each with ahip_device_tensor_free (before or after the session; the pool lives until both
+ * are gone).  A recorded HIP graph is not used on this path. */
+typedef struct ahip_device_tensor ahip_device_tensor;
+int ahip_session_run_device(ahip_session *session, int n_inputs, const void *const *device_ptrs,
+                            const int *elem_types, const int *ranks, const int64_t *const *dims,
+                            int output_capacity, ahip_device_tensor **outputs, int *n_outputs);
+/* Waits for everything the session has enqueued; reports errors kernels leave in device flags
+ * (an out-of-range Gather index) as AHIP_ERR_ARG. */
+int ahip_session_synchronize(ahip_session *session);
+void ahip_device_tensor_free(ahip_device_tensor *tensor);
+void *ahip_device_tensor_ptr(const ahip_device_tensor *tensor);
+int ahip_device_tensor_elem_type(const ahip_device_tensor *tensor);
+int ahip_device_tensor_rank(const ahip_device_tensor *tensor);
+int ahip_device_tensor_dims(const ahip_device_tensor *tensor, int64_t *dims, int capacity);
+size_t ahip_device_tensor_nbytes(const ahip_device_tensor *tensor);
 /* model(): a borrowed handle, valid while the session lives. */
 const ahip_model *ahip_session_model(const ahip_session *session);
 /* Per-operator device time of the last run when profiling is enabled
