@@ -42,6 +42,17 @@ _CODE_NAMES = {
 }
 
 
+class FusedStep(ctypes.Structure):
+    """ahip_fused_step"""
+    _fields_ = [("is_unary", c_int), ("op", c_int), ("lhs", c_int), ("rhs", c_int), ("alpha", c_float), ("beta", c_float),
+                ("pow_scalar_exponent", c_int)]
+
+
+FUSED_ACC = -1
+FUSED_MAX_INPUTS = 6
+FUSED_MAX_STEPS = 16
+
+
 def _declare(L):
     def f(name, argtypes, restype=c_int):
         fn = getattr(L, name)
@@ -89,6 +100,8 @@ def _declare(L):
     f("ahip_strides_for_broadcasting", [c_int, P(c_int64), c_int, P(c_int64), P(c_int64)])
     f("ahip_binary", [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, P(c_int64), P(c_int64), P(c_int64)])
     f("ahip_unary", [c_void_p, c_int, c_void_p, c_void_p, c_size_t, c_float, c_float])
+    f("ahip_fused_use_compiled_chains", [c_void_p, c_int])
+    f("ahip_fused_elemwise", [c_void_p, c_void_p, c_int, P(c_int64), c_int, P(c_void_p), P(P(c_int64)), c_int, P(FusedStep)])
     f("ahip_softmax_lastaxis", [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t])
     f("ahip_layernorm_lastaxis", [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_float])
     f("ahip_reduce", [c_void_p, c_int, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t])
@@ -153,6 +166,7 @@ def _declare_graph(L):
     f("ahip_model_execution_plan", [c_void_p, P(c_int64), P(c_int), c_int, P(c_int64), c_int, P(c_int), P(c_int)])
     for name in ("ahip_fuse_layer_norm", "ahip_fuse_gelu", "ahip_fuse_fast_gelu", "ahip_eliminate_identity"):
         f(name, [c_void_p, P(c_int)])
+    f("ahip_fuse_elemwise_ops", [c_void_p, c_int, P(c_int)])
     f("ahip_tensor_new", [c_int, c_int, P(c_int64), c_void_p, c_size_t, P(c_void_p)])
     f("ahip_tensor_free", [c_void_p], None)
     f("ahip_tensor_elem_type", [c_void_p])

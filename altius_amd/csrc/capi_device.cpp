@@ -291,6 +291,18 @@ int ahip_unary(ahip_ctx *ctx, int op, float *out, const float *in, size_t n, flo
     return altius::launch_unary(ctx->d, op, out, in, n, alpha, beta);
 }
 
+int ahip_fused_elemwise(ahip_ctx *ctx, float *out, int rank, const int64_t *out_dims, int n_inputs, const float *const *inputs,
+                        const int64_t *const *input_strides, int n_steps, const ahip_fused_step *steps) {
+    REQUIRE_CTX(ctx, "ahip_fused_elemwise");
+    return altius::launch_fused_elemwise(ctx->d, out, rank, out_dims, n_inputs, inputs, input_strides, n_steps, steps);
+}
+
+int ahip_fused_use_compiled_chains(ahip_ctx *ctx, int enable) {
+    REQUIRE_CTX(ctx, "ahip_fused_use_compiled_chains");
+    ctx->d.fused_static_chains = enable != 0;
+    return AHIP_OK;
+}
+
 int ahip_softmax_lastaxis(ahip_ctx *ctx, float *out, const float *in, size_t rows, size_t len) {
     REQUIRE_CTX(ctx, "ahip_softmax_lastaxis");
     return altius::launch_softmax(ctx->d, out, in, rows, len);

@@ -192,6 +192,10 @@ bool Op::get_string(const std::string &n, std::string *v) const {
         *v = mode;
     } else if (n == "nearest_mode" && kind == OpKind::Resize) {
         *v = nearest_mode;
+    } else if (n == "chain" && kind == OpKind::FusedElemwise && fused) {
+        // Not an ONNX attribute: the fused operators' names in order, comma-separated, for inspection.
+        v->clear();
+        for (const auto &step : fused->chain) *v += (v->empty() ? "" : ",") + std::string(step.op.name());
     } else {
         return false;
     }

@@ -26,6 +26,8 @@ enum class OpKind : int {
 
 const char *op_kind_name(OpKind k);
 
+struct FusedElemwise;
+
 struct Op {
     OpKind kind = OpKind::Identity;
 
@@ -62,6 +64,8 @@ struct Op {
     int64_t exclude_outside = 0;
     // Constant.value (op.rs:206-210)
     std::shared_ptr<Tensor> value;
+    // FusedElemwise (op.rs:213-217)
+    std::shared_ptr<const FusedElemwise> fused;
 
     Op() = default;
     explicit Op(OpKind k) : kind(k) {}
@@ -98,6 +102,16 @@ struct Op {
     }
 
     const char *name() const { return op_kind_name(kind); }
+    // Op::is_elemwise (op.rs:387-412): the operators fuse_elemwise_ops chains together.
+    bool is_elemwise() const {
+        switch (kind) {
+        case OpKind::Add: case OpKind::Sub: case OpKind::Mul: case OpKind::Div: case OpKind::Pow: case OpKind::Greater:
+        case OpKind::Sqrt: case OpKind::ReLU: case OpKind::LeakyReLU: case OpKind::HardSigmoid:
+            return true;
+        default:
+            return false;
+        }
+    }
 
     // Attribute access by ONNX attribute name ("axis", "perm", "kernel_shape", "transB", ...): the
     // one vocabulary shared by the ONNX loader and the C ABI.  Setters return false for a name
@@ -110,6 +124,18 @@ struct Op {
     bool get_float(const std::string &name, float *v) const;
     bool get_ints(const std::string &name, std::vector<int64_t> *v) const;
     bool get_string(const std::string &name, std::string *v) const;
+};
+
+// The payload of Op::FusedElemwise (op.rs:213-217): the value ids the fused node reads, in the order
+// of its inputs, and the operators it stands for with the value ids they were wired with.  Every
+// step but the first reads the output of the step before it.
+struct FusedElemwise {
+    struct Step {
+        Op op;
+        std::vector<size_t> inputs, outputs;  // ValueIds
+    };
+    std::vector<size_t> input_map;
+    std::vector<Step> chain;
 };
 
 // The operator a freshly loaded ONNX node of this type starts from: kind plus the defaults the

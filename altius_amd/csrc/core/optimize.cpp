@@ -1,5 +1,7 @@
 #include "optimize.h"
 
+#include "shape.h"
+
 #include <algorithm>
 
 namespace altius {
@@ -250,6 +252,129 @@ size_t eliminate_identity(Model &model) {
     }
     model.remove_unnecessary_nodes();
     return count;
+}
+
+namespace {
+
+bool extended_elemwise(const Op &op) {
+    switch (op.kind) {
+    case OpKind::Add: case OpKind::Sub: case OpKind::Mul: case OpKind::Div: case OpKind::Pow:
+    case OpKind::Sqrt: case OpKind::ReLU: case OpKind::LeakyReLU: case OpKind::HardSigmoid:
+    case OpKind::Erf: case OpKind::Gelu: case OpKind::Sigmoid: case OpKind::Tanh: case OpKind::Exp: case OpKind::Round:
+        return true;
+    default:
+        return false;
+    }
+}
+
+}  // namespace
+
+bool fuse_elemwise_ops(Model &model, ElemwiseFusionRule rule, size_t *count, std::string *err) {
+    if (count) *count = 0;
+    const std::vector<NodeId> order = model.topo_sort_nodes();
+    const auto users = model.get_value_users();
+    const auto parents = model.get_value_parents();
+    std::map<ValueId, TypedFixedShape> shapes;
+    ShapeError serr;
+    if (!infer_shapes(model, nullptr, &shapes, &serr)) {
+        if (err) *err = serr.message;
+        return false;
+    }
+    const auto &outs = model.graph.outputs;
+    auto is_graph_output = [&](ValueId v) { return std::find(outs.begin(), outs.end(), v) != outs.end(); };
+    auto shape_of = [&](ValueId v) -> const TypedFixedShape * {
+        auto it = shapes.find(v);
+        return it == shapes.end() ? nullptr : &it->second;
+    };
+    auto f32_known = [&](ValueId v) {
+        const TypedFixedShape *s = shape_of(v);
+        return s && s->elem_ty == TensorElemType::F32;
+    };
+    const bool extended = rule == ElemwiseFusionRule::ExtendedRule;
+    constexpr size_t MAX_STEPS = 16, MAX_OPERANDS = 6;
+
+    std::vector<std::vector<NodeId>> chains;
+    std::set<NodeId> visited;
+    for (NodeId start : order) {
+        if (visited.count(start)) continue;
+        std::vector<NodeId> chain;
+        std::set<ValueId> operands;  // distinct values the chain reads from outside (extended rule's limit)
+        std::optional<NodeId> last;
+        NodeId cur = start;
+        for (;;) {
+            const Node &node = model.graph.nodes[cur];
+            bool fusible = node.outputs.size() == 1 && !node.inputs.empty() && !visited.count(cur);
+            std::set<ValueId> more = operands;
+            if (fusible && !extended) {
+                fusible = node.op.is_elemwise();
+                for (ValueId in : node.inputs) {
+                    if (!fusible) break;
+                    auto p = parents.find(in);
+                    fusible = p == parents.end() || !last || p->second == *last;
+                }
+                if (fusible && last) {
+                    const Node &prev = model.graph.nodes[*last];
+                    fusible = prev.inputs.size() == 2 && prev.outputs[0] == node.inputs[0];
+                    if (fusible && node.inputs.size() == 2) {
+                        const TypedFixedShape *a = shape_of(node.inputs[1]), *b = shape_of(prev.inputs[1]);
+                        fusible = a && b && a->dims == b->dims && a->elem_ty == b->elem_ty;
+                    } else if (fusible) {
+                        fusible = node.inputs.size() == 1;
+                    }
+                }
+            } else if (fusible) {
+                fusible = extended_elemwise(node.op) && node.inputs.size() <= 2 && f32_known(node.outputs[0]) &&
+                          chain.size() < MAX_STEPS;
+                bool reads_prev = !last;
+                for (ValueId in : node.inputs) {
+                    if (!fusible) break;
+                    if (last && in == model.graph.nodes[*last].outputs[0]) {
+                        reads_prev = true;
+                        continue;
+                    }
+                    fusible = f32_known(in);
+                    more.insert(in);
+                }
+                fusible = fusible && reads_prev && more.size() <= MAX_OPERANDS;
+            }
+            if (!fusible) break;
+            chain.push_back(cur);
+            operands = std::move(more);
+            last = cur;
+            auto u = users.find(node.outputs[0]);
+            if (u == users.end() || u->second.size() != 1 || is_graph_output(node.outputs[0])) break;
+            cur = *u->second.begin();
+        }
+        if (chain.size() > 1) {
+            visited.insert(chain.begin(), chain.end());
+            chains.push_back(std::move(chain));
+        }
+    }
+
+    for (const auto &chain : chains) {
+        auto fused = std::make_shared<FusedElemwise>();
+        std::optional<NodeId> prev;
+        for (NodeId id : chain) {
+            const Node &node = model.graph.nodes[id];
+            for (ValueId in : node.inputs) {
+                if (prev && model.graph.nodes[*prev].outputs[0] == in) continue;
+                if (std::find(fused->input_map.begin(), fused->input_map.end(), in) == fused->input_map.end())
+                    fused->input_map.push_back(in);
+            }
+            fused->chain.push_back({node.op, node.inputs, node.outputs});
+            prev = id;
+        }
+        Op op(OpKind::FusedElemwise);
+        const std::vector<ValueId> ins = fused->input_map;
+        op.fused = std::move(fused);
+        Node node(std::move(op));
+        node.with_ins(ins).with_out(model.graph.nodes[chain.back()].outputs[0]);
+        model.graph.add_node(std::move(node));
+        for (NodeId id : chain) model.graph.nodes[id].deleted = true;
+    }
+    model.remove_unnecessary_nodes();
+    if (count) *count = chains.size();
+    return true;
 }
 
 }  // namespace altius

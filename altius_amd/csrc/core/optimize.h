@@ -4,6 +4,8 @@
 // number of subgraphs it rewrote.
 #pragma once
 
+#include <string>
+
 #include "model.h"
 
 namespace altius {
@@ -25,5 +27,24 @@ size_t fuse_fast_gelu(Model &model);
 // Rewires the users of every Identity node to its input and drops the node; an
 // Identity that feeds a graph output is kept.
 size_t eliminate_identity(Model &model);
+
+// Chains of element-wise operators => one FusedElemwise node (crates/core/src/optimize/elemwise_fusion.rs:12-138).
+//
+// ReferenceRule restates the reference's pass: operators of Op::is_elemwise with one output; a node
+// continues a chain when its first input is the previous node's output, that output has no other
+// reader, the previous node is binary, its remaining inputs are not produced by other nodes, and (if
+// it is binary) its second operand has the shape of the previous node's second operand.
+//
+// ExtendedRule is this backend's own: the previous result may be any operand (also both), the other
+// operands may be any values computed outside the chain with any shapes that broadcast, and the
+// approximated unary functions (Erf, Gelu, Sigmoid, Tanh, Exp, Round) count as element-wise, as long as
+// every tensor involved is f32 with a known shape, the chain has at most 16 steps and reads at most 6
+// distinct values.  Greater is left out (its result is not f32).
+//
+// Under both rules a value that is also a graph output ends the chain (the reference would drop such an
+// output).  Needs every shape it looks at to be inferable; returns false with *err set when shape
+// inference fails.  *count receives the number of chains fused.
+enum class ElemwiseFusionRule { ReferenceRule = 0, ExtendedRule = 1 };
+bool fuse_elemwise_ops(Model &model, ElemwiseFusionRule rule, size_t *count, std::string *err);
 
 }  // namespace altius

@@ -159,6 +159,36 @@ bool compute_output_shapes(const Model &model, Op &op, const std::vector<const T
         out->push_back({inputs[0]->dims(), inputs[0]->elem_ty()});
         return true;
     }
+    case OpKind::FusedElemwise: {  // shape.rs:616-650: the chain's steps one after the other
+        if (!op.fused || op.fused->chain.empty()) return fail(err, "FusedElemwise: empty chain");
+        const FusedElemwise &f = *op.fused;
+        if (!need_inputs(f.input_map.size())) return false;
+        std::map<size_t, const Tensor *> outer;
+        for (size_t i = 0; i < f.input_map.size(); i++) outer[f.input_map[i]] = inputs[i];
+        Tensor prev;
+        bool have_prev = false;
+        size_t prev_id = 0;
+        std::vector<TypedFixedShape> step_out;
+        for (const auto &step : f.chain) {
+            if (step.outputs.size() != 1) return fail(err, "FusedElemwise: a step must have one output");
+            std::vector<const Tensor *> ins;
+            for (size_t v : step.inputs) {
+                auto it = outer.find(v);
+                if (it != outer.end()) ins.push_back(it->second);
+                else if (have_prev && v == prev_id) ins.push_back(&prev);
+                else return fail(err, "FusedElemwise: a step reads a value that is neither an input nor the previous result");
+            }
+            Op step_op = step.op;
+            step_out.clear();
+            if (!compute_output_shapes(model, step_op, ins, 1, &step_out, err)) return false;
+            if (step_out.empty()) return fail(err, "FusedElemwise: a step produced no shape");
+            prev = Tensor::empty_of_type(step_out[0].elem_ty, step_out[0].dims);
+            have_prev = true;
+            prev_id = step.outputs[0];
+        }
+        out->push_back(step_out[0]);
+        return true;
+    }
     case OpKind::Cast: {  // shape.rs:612-615
         if (!need_inputs(1)) return false;
         out->push_back({inputs[0]->dims(), op.to});

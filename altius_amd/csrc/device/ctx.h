@@ -27,6 +27,9 @@ struct DeviceCtx {
     bool flags_armed = false;
     // Tensors of at least this many bytes are streamed with non-temporal accesses.
     size_t nt_threshold_bytes = (size_t)128 << 20;
+    // Chains of element-wise steps that were instantiated at compile time run as straight-line code;
+    // switched off, every chain takes the interpreting kernel (tests compare the two).
+    bool fused_static_chains = true;
     std::string last_error;
 
     bool streaming(size_t bytes) const { return bytes >= nt_threshold_bytes; }
@@ -52,6 +55,10 @@ int launch_binary(DeviceCtx &ctx, int op, float *out, const float *a, const floa
                   const int64_t *out_dims, const int64_t *a_strides, const int64_t *b_strides);
 int launch_unary(DeviceCtx &ctx, int op, float *out, const float *in, size_t n, float alpha,
                  float beta);
+// A chain of element-wise steps in one kernel (fused.hip); AHIP_ERR_UNSUPPORTED when the geometry
+// needs the operator-by-operator route.
+int launch_fused_elemwise(DeviceCtx &ctx, float *out, int rank, const int64_t *out_dims, int n_inputs, const float *const *inputs,
+                          const int64_t *const *input_strides, int n_steps, const ahip_fused_step *steps);
 int launch_softmax(DeviceCtx &ctx, float *out, const float *in, size_t rows, size_t len);
 int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *gamma,
                      const float *beta, size_t rows, size_t len, float eps);

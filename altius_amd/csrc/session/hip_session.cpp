@@ -661,6 +661,149 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
     return true;
 }
 
+// Op::FusedElemwise: the whole chain in one kernel when its operands fit the kernel's geometry and
+// every step has a step code there; otherwise the steps run one after the other through their own
+// kernels, which gives the same bits.
+bool HipSession::run_fused_elemwise(const Node &node, const Op &op, const std::vector<DeviceTensor *> &in,
+                                    const std::vector<TypedFixedShape> &shapes, std::vector<DeviceTensor> *outs, SessionError *err) {
+    if (!op.fused || op.fused->chain.empty()) return fail(err, SessionError::Message, "FusedElemwise: empty chain");
+    const FusedElemwise &f = *op.fused;
+    if (in.size() < f.input_map.size()) return fail(err, SessionError::Message, "FusedElemwise: too few inputs");
+    for (size_t i = 0; i < f.input_map.size(); i++)
+        if (!in[i]) return fail(err, SessionError::Message, "FusedElemwise: an input value is missing");
+    auto outer_index = [&](ValueId v) -> int {
+        for (size_t i = 0; i < f.input_map.size(); i++)
+            if (f.input_map[i] == v) return (int)i;
+        return -1;
+    };
+
+    // Translate the chain into the kernel's steps while following the shapes operator by operator
+    // (Pow's scalar-exponent path depends on the operand extents of its own node).
+    std::vector<ahip_fused_step> steps;
+    bool one_kernel = f.input_map.size() <= AHIP_FUSED_MAX_INPUTS && f.chain.size() <= AHIP_FUSED_MAX_STEPS &&
+                      shapes[0].elem_ty == TensorElemType::F32 && shapes[0].dims.len() <= (size_t)MAX_RANK;
+    for (size_t i = 0; i < f.input_map.size() && one_kernel; i++) one_kernel = in[i]->elem_ty == TensorElemType::F32;
+    FixedDimensions prev_dims;
+    ValueId prev_id = 0;
+    for (size_t t = 0; t < f.chain.size() && one_kernel; t++) {
+        const auto &step = f.chain[t];
+        ahip_fused_step s{};
+        std::vector<FixedDimensions> operand_dims;
+        int sel[2] = {AHIP_FUSED_ACC, AHIP_FUSED_ACC};
+        if (step.inputs.empty() || step.inputs.size() > 2 || step.outputs.size() != 1) {
+            one_kernel = false;
+            break;
+        }
+        for (size_t k = 0; k < step.inputs.size(); k++) {
+            const int idx = outer_index(step.inputs[k]);
+            if (idx >= 0) {
+                sel[k] = idx;
+                operand_dims.push_back(in[idx]->dims);
+            } else if (t > 0 && step.inputs[k] == prev_id) {
+                operand_dims.push_back(prev_dims);
+            } else {
+                return fail(err, SessionError::Message, "FusedElemwise: a step reads a value that is neither an input nor the previous result");
+            }
+        }
+        s.lhs = sel[0];
+        s.rhs = sel[1];
+        switch (step.op.kind) {
+        case OpKind::Add: s.op = AHIP_ADD; break;
+        case OpKind::Sub: s.op = AHIP_SUB; break;
+        case OpKind::Mul: s.op = AHIP_MUL; break;
+        case OpKind::Div: s.op = AHIP_DIV; break;
+        case OpKind::Pow: s.op = AHIP_POW; break;
+        case OpKind::Sqrt: s.is_unary = 1; s.op = AHIP_SQRT; break;
+        case OpKind::ReLU: s.is_unary = 1; s.op = AHIP_RELU; break;
+        case OpKind::Gelu: s.is_unary = 1; s.op = AHIP_GELU; break;
+        case OpKind::Sigmoid: s.is_unary = 1; s.op = AHIP_SIGMOID; break;
+        case OpKind::Erf: s.is_unary = 1; s.op = AHIP_ERF; break;
+        case OpKind::Tanh: s.is_unary = 1; s.op = AHIP_TANH; break;
+        case OpKind::Exp: s.is_unary = 1; s.op = AHIP_EXP; break;
+        case OpKind::Round: s.is_unary = 1; s.op = AHIP_ROUND; break;
+        case OpKind::HardSigmoid: s.is_unary = 1; s.op = AHIP_HARDSIGMOID; s.alpha = step.op.alpha; s.beta = step.op.beta; break;
+        case OpKind::LeakyReLU: s.is_unary = 1; s.op = AHIP_LEAKYRELU; s.alpha = step.op.alpha; break;
+        default: one_kernel = false; break;  // Greater, or anything without a step code
+        }
+        if (!one_kernel) break;
+        if ((s.is_unary != 0) != (step.inputs.size() == 1)) {
+            one_kernel = false;
+            break;
+        }
+        if (s.is_unary) {
+            prev_dims = operand_dims[0];
+        } else {
+            auto b = operand_dims[0].broadcast(operand_dims[1]);
+            if (!b) return fail(err, SessionError::Shape, std::string("FusedElemwise: ") + step.op.name() + " operands do not broadcast");
+            // launch_binary's rule: one exponent for a base of more than one element.
+            s.pow_scalar_exponent = s.op == AHIP_POW && operand_dims[1].total_elems() == 1 && operand_dims[0].total_elems() > 1;
+            prev_dims = *b;
+        }
+        prev_id = step.outputs[0];
+        steps.push_back(s);
+    }
+    if (one_kernel && prev_dims != shapes[0].dims) one_kernel = false;
+
+    if (one_kernel) {
+        DeviceTensor out;
+        if (!allocate(shapes[0], &out, err)) return false;
+        std::vector<std::vector<int64_t>> strides(f.input_map.size());
+        std::vector<const int64_t *> stride_ptrs;
+        std::vector<const float *> ptrs;
+        for (size_t i = 0; i < f.input_map.size(); i++) {
+            auto st = in[i]->dims.strides_for_broadcasting_to(out.dims);
+            if (!st) return fail(err, SessionError::Shape, "FusedElemwise: an operand does not broadcast to the output shape");
+            for (auto x : st->as_vec()) strides[i].push_back((int64_t)x);
+            stride_ptrs.push_back(strides[i].data());
+            ptrs.push_back(static_cast<const float *>(in[i]->ptr));
+        }
+        std::vector<int64_t> dims;
+        for (auto x : out.dims.as_vec()) dims.push_back((int64_t)x);
+        const int rc = launch_fused_elemwise(ctx_, static_cast<float *>(out.ptr), (int)dims.size(), dims.data(), (int)ptrs.size(), ptrs.data(),
+                                             stride_ptrs.data(), (int)steps.size(), steps.data());
+        if (rc == AHIP_OK) {
+            outs->push_back(std::move(out));
+            return true;
+        }
+        if (rc != AHIP_ERR_UNSUPPORTED) return fail_code(err, rc, ctx_.last_error);
+        // geometry the kernel does not take: fall through to the operator-by-operator route
+    }
+
+    DeviceTensor prev;
+    bool have_prev = false;
+    prev_id = 0;
+    for (const auto &step : f.chain) {
+        if (step.outputs.size() != 1) return fail(err, SessionError::Message, "FusedElemwise: a step must have one output");
+        std::vector<DeviceTensor *> ins;
+        std::vector<Tensor> meta;
+        meta.reserve(step.inputs.size());
+        for (ValueId v : step.inputs) {
+            const int idx = outer_index(v);
+            if (idx >= 0) ins.push_back(in[idx]);
+            else if (have_prev && v == prev_id) ins.push_back(&prev);
+            else return fail(err, SessionError::Message, "FusedElemwise: a step reads a value that is neither an input nor the previous result");
+            meta.push_back(Tensor::empty_of_type(ins.back()->elem_ty, ins.back()->dims));
+        }
+        std::vector<const Tensor *> meta_ptrs;
+        for (auto &m : meta) meta_ptrs.push_back(&m);
+        Op step_op = step.op;
+        std::vector<TypedFixedShape> step_shapes;
+        ShapeError serr;
+        if (!compute_output_shapes(model_, step_op, meta_ptrs, 1, &step_shapes, &serr)) return fail(err, SessionError::Shape, serr.message);
+        Node step_node(step_op);
+        step_node.inputs = step.inputs;
+        step_node.outputs = step.outputs;
+        std::vector<DeviceTensor> step_outs;
+        if (!run_device_op(step_node, step_op, ins, step_shapes, &step_outs, err)) return false;
+        if (step_outs.empty()) return fail(err, SessionError::Message, "FusedElemwise: a step produced nothing");
+        prev = std::move(step_outs[0]);  // the previous intermediate goes back to the pool; stream order keeps it readable
+        have_prev = true;
+        prev_id = step.outputs[0];
+    }
+    outs->push_back(std::move(prev));
+    return true;
+}
+
 bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector<DeviceTensor *> &in,
                                const std::vector<TypedFixedShape> &shapes, std::vector<DeviceTensor> *outs, SessionError *err) {
     const std::string opname = op.name();
@@ -687,6 +830,8 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
         return v;
     };
     auto done = [&](int rc) { return rc ? fail_code(err, rc, ctx_.last_error) : true; };
+
+    if (op.kind == OpKind::FusedElemwise) return run_fused_elemwise(node, op, in, shapes, outs, err);
 
     // Split produces one tensor per part; everything else one output.
     if (op.kind == OpKind::Split) {

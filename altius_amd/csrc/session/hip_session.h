@@ -129,6 +129,8 @@ private:
     bool upload(const Tensor &t, DeviceTensor *out, SessionError *err);
     // Makes t.host available by reading a small tensor back (synchronises the stream).
     bool fetch_host(DeviceTensor *t, SessionError *err);
+    bool run_fused_elemwise(const Node &node, const Op &op, const std::vector<DeviceTensor *> &in,
+                            const std::vector<TypedFixedShape> &shapes, std::vector<DeviceTensor> *outs, SessionError *err);
     bool run_device_op(const Node &node, const Op &op, const std::vector<DeviceTensor *> &in,
                        const std::vector<TypedFixedShape> &shapes, std::vector<DeviceTensor> *outs, SessionError *err);
 

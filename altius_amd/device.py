@@ -196,6 +196,37 @@ class Context:
             self.free(dx)
             self.free(do)
 
+    def fused_use_compiled_chains(self, enable):
+        """False: every chain takes the interpreting kernel, also those the library has compiled code for."""
+        check(self.L.ahip_fused_use_compiled_chains(self.handle, int(bool(enable))), self.handle)
+
+    def fused_elemwise(self, inputs, steps):
+        """A chain of element-wise steps in one kernel.  inputs: f32 arrays that broadcast to a common shape;
+        steps: (kind, op, lhs, rhs[, alpha, beta, pow_scalar_exponent]) with kind "b" (binary, op = ADD..POW) or
+        "u" (unary, op = SQRT..), lhs / rhs an index into inputs or _lib.FUSED_ACC.  Returns the last step's
+        result at the broadcast shape."""
+        arrays = [np.asarray(a, dtype=np.float32, order="C") for a in inputs]
+        shape = np.broadcast_shapes(*[a.shape for a in arrays])
+        bufs = [self.upload(a) for a in arrays]
+        n = int(np.prod(shape, dtype=np.int64))
+        out = self.alloc(max(n * 4, 4))
+        stride_arrays = [i64_array(strides_for_broadcasting(a.shape, shape)) if len(shape) else i64_array([0]) for a in arrays]
+        strides = (ctypes.POINTER(ctypes.c_int64) * len(arrays))(
+            *[ctypes.cast(s, ctypes.POINTER(ctypes.c_int64)) for s in stride_arrays])
+        ptrs = (ctypes.c_void_p * len(arrays))(*[b.ptr for b in bufs])
+        c_steps = (_lib.FusedStep * len(steps))()
+        for i, st in enumerate(steps):
+            kind, op, lhs, rhs = st[:4]
+            extra = list(st[4:]) + [0.0, 0.0, 0][len(st) - 4:]
+            c_steps[i] = _lib.FusedStep(1 if kind == "u" else 0, op, lhs, rhs, extra[0], extra[1], int(extra[2]))
+        try:
+            check(self.L.ahip_fused_elemwise(self.handle, out.ptr, len(shape), i64_array(shape) if len(shape) else None,
+                                             len(arrays), ptrs, strides, len(steps), c_steps), self.handle)
+            return self.download(out, shape)
+        finally:
+            for b in bufs + [out]:
+                self.free(b)
+
     def softmax(self, x):
         x = np.asarray(x, dtype=np.float32, order="C")
         length = x.shape[-1]

@@ -332,6 +332,7 @@ class Model:
         check(self.L.ahip_model_node_info(self.handle, node_id, ctypes.byref(kind), ctypes.byref(a),
                                           ctypes.byref(nin), ins, ctypes.byref(nout), outs, io_capacity))
         return {
+            "id": node_id,
             "op": kind.value,
             "op_name": op_name(kind.value),
             "inputs": [int(ins[i]) for i in range(min(nin.value, io_capacity))],
@@ -384,3 +385,18 @@ class Model:
 
     def eliminate_identity(self):
         return self._pass(self.L.ahip_eliminate_identity)
+
+    def fuse_elemwise_ops(self, extended=False):
+        """Chains of element-wise operators -> FusedElemwise nodes; the reference's rule, or this backend's
+        wider one with extended=True.  Returns the number of chains fused."""
+        c = ctypes.c_int()
+        check(self.L.ahip_fuse_elemwise_ops(self.handle, 1 if extended else 0, ctypes.byref(c)))
+        return c.value
+
+    def fused_chain(self, node_id):
+        """Operator names of a FusedElemwise node, in order."""
+        n = ctypes.c_int()
+        check(self.L.ahip_node_get_attr_string(self.handle, node_id, b"chain", None, 0, ctypes.byref(n)))
+        buf = ctypes.create_string_buffer(n.value + 1)
+        check(self.L.ahip_node_get_attr_string(self.handle, node_id, b"chain", buf, n.value + 1, None))
+        return buf.value.decode().split(",")

@@ -238,6 +238,9 @@ def session_table(synth, dev_ctx):
     fused.fuse_layer_norm()
     measure("cfg2 LayerNorm chain, 9 nodes", chain, c2["x"], 12 * X + 8 * r + 2 * 768 * 4 + 8)
     measure("cfg2 after fuse_layer_norm, 1 node", fused, c2["x"], 2 * X + 2 * 768 * 4)
+    ew = chain.clone()
+    ew.fuse_elemwise_ops(extended=True)        # ReduceMean, Sub, Pow, ReduceMean, FusedElemwise[Add,Sqrt,Div,Mul,Add]
+    measure("cfg2 chain after fuse_elemwise_ops, 5 nodes", ew, c2["x"], 8 * X + 4 * r + 2 * 768 * 4 + 8)
     c3 = synth.cfg3()
     X = c3["x"].nbytes
     chain = graphs.single_input_model(c3["x"].shape, lambda m, x: graphs.erf_gelu_chain(m, x, float(c3["sqrt2"])))
@@ -245,6 +248,9 @@ def session_table(synth, dev_ctx):
     fused.fuse_gelu()
     measure("cfg3 erf-GELU chain, 5 nodes", chain, c3["x"], 11 * X + 12)
     measure("cfg3 after fuse_gelu, 1 node", fused, c3["x"], 2 * X)
+    ew = chain.clone()
+    ew.fuse_elemwise_ops(extended=True)        # one FusedElemwise with the bits of the 5-node chain
+    measure("cfg3 chain after fuse_elemwise_ops, 1 node", ew, c3["x"], 2 * X + 12)
     se = c3["se"]
     model = graphs.single_input_model(se.shape, lambda m, x: graphs.squeeze_excite(m, x, c3["alpha"], c3["beta"]))
     measure("cfg3 squeeze-excite, 3 nodes", model, se, 3 * se.nbytes + 4 * 32 * 576 * 4)

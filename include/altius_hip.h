@@ -150,6 +150,38 @@ enum ahip_unary_op {
 int ahip_unary(ahip_ctx *ctx, int op, float *out, const float *in, size_t n, float alpha,
                float beta);
 
+/* A chain of element-wise operators in one pass: Op::FusedElemwise (crates/core/src/op.rs:213-217),
+ * which the reference emits in crates/core/src/optimize/elemwise_fusion.rs and runs only on its
+ * code-generating backend (crates/session_clang/src/translator.rs:975-1143; the interpreter has no
+ * kernel, session.rs:246).  Step t computes acc = op(lhs, rhs) (binary) or acc = op(lhs) (unary) for
+ * every output element; an operand is inputs[k] broadcast to the output with input_strides[k] (from
+ * ahip_strides_for_broadcasting) or AHIP_FUSED_ACC, the previous step's result; the last acc is the
+ * output.  Each step applies exactly the per-element function of ahip_binary / ahip_unary, so the
+ * result has the bits of the unfused chain.  pow_scalar_exponent selects the reference's
+ * scalar-exponent Pow path (a*a when the exponent equals 2; session.rs:585-598), which the unfused
+ * kernel takes when the exponent tensor has one element and the base has more.
+ * AHIP_ERR_UNSUPPORTED (nothing launched) when the operands need more than three merged axes, or
+ * there are more than AHIP_FUSED_MAX_INPUTS operands or AHIP_FUSED_MAX_STEPS steps: run the chain
+ * operator by operator then. */
+#define AHIP_FUSED_MAX_INPUTS 6
+#define AHIP_FUSED_MAX_STEPS 16
+#define AHIP_FUSED_ACC (-1)
+typedef struct ahip_fused_step {
+    int is_unary;            /* 0: op is an ahip_binary_op, 1: op is an ahip_unary_op */
+    int op;
+    int lhs, rhs;            /* index into inputs[] or AHIP_FUSED_ACC; rhs is ignored by unary steps */
+    float alpha, beta;       /* parameters of unary steps (HardSigmoid, LeakyRelu, Clip) */
+    int pow_scalar_exponent; /* AHIP_POW only */
+} ahip_fused_step;
+int ahip_fused_elemwise(ahip_ctx *ctx, float *out, int rank, const int64_t *out_dims, int n_inputs,
+                        const float *const *inputs, const int64_t *const *input_strides, int n_steps,
+                        const ahip_fused_step *steps);
+/* ahip_fused_elemwise runs a chain through a kernel compiled for exactly that chain when the library
+ * has one (the exporter's erf-GELU, the LayerNorm tail, scale-and-shift, bias + Relu, x * Sigmoid(x),
+ * x * HardSigmoid(x)) and through a kernel that interprets the steps otherwise; both give the same bits.
+ * enable = 0 sends every chain of this context to the interpreting kernel (default 1). */
+int ahip_fused_use_compiled_chains(ahip_ctx *ctx, int enable);
+
 /* compute_softmax over the last axis (session.rs:990-1026 + fast_math.rs:102-187):
  * `rows` rows of `len` contiguous elements. */
 int ahip_softmax_lastaxis(ahip_ctx *ctx, float *out, const float *in, size_t rows, size_t len);
@@ -373,6 +405,19 @@ int ahip_fuse_layer_norm(ahip_model *model, int *count);
 int ahip_fuse_gelu(ahip_model *model, int *count);
 int ahip_fuse_fast_gelu(ahip_model *model, int *count);
 int ahip_eliminate_identity(ahip_model *model, int *count);
+/* fuse_elemwise_ops (crates/core/src/optimize/elemwise_fusion.rs:12-138): chains of element-wise
+ * operators become one FusedElemwise node each, which the session runs as one kernel
+ * (ahip_fused_elemwise) with the bits of the unfused chain.  AHIP_FUSE_REFERENCE_RULE restates the
+ * reference's conditions (operators of Op::is_elemwise; the previous result must be the first operand of
+ * the next node, the previous node binary, second operands of equal shape).  AHIP_FUSE_EXTENDED_RULE is
+ * this backend's own: the previous result may be either operand, other operands may have any
+ * broadcastable shape and come from anywhere outside the chain, and Erf / Gelu / Sigmoid / Tanh / Exp /
+ * Round count as element-wise; f32 tensors of known shape only, at most 16 steps and 6 operands per chain.
+ * Under both rules a value that is also a graph output ends its chain.  AHIP_ERR_SHAPE when shape
+ * inference fails (the reference returns ShapeError).  The node's operators can be read back with
+ * ahip_node_get_attr_string(model, node, "chain", ...) as a comma-separated list of names. */
+enum ahip_fuse_rule { AHIP_FUSE_REFERENCE_RULE = 0, AHIP_FUSE_EXTENDED_RULE = 1 };
+int ahip_fuse_elemwise_ops(ahip_model *model, int rule, int *count);
 
 /* Host tensors (crates/core/src/tensor.rs:61-76).  data is copied; NULL data gives zeros.
  * Storage of 64 KiB and more is pinned (page-locked) host memory from a process-wide pool when

@@ -337,3 +337,122 @@ def test_host_tensor_views_and_pool_without_a_device():
     import gc
     gc.collect()
     assert np.array_equal(keep, a)
+
+
+def _ln_chain_model(shape=(2, 5, 8)):
+    m = Model()
+    x = m.new_val_named_and_shaped("x", list(shape))
+    out, g, b = layer_norm_chain(m, x, np.ones(shape[-1], np.float32), np.zeros(shape[-1], np.float32))
+    m.add_input(x)
+    m.add_output(out)
+    return m, x, out, g, b
+
+
+def test_fuse_elemwise_ops_reference_rule():
+    """crates/core/src/optimize/elemwise_fusion.rs:12-138 on the exporter's LayerNorm chain: Add(eps) -> Sqrt
+    fuse (Sqrt is unary and reads the Add), Mul(gamma) -> Add(beta) fuse (second operands of equal shape);
+    Sub feeds two readers, Pow feeds a ReduceMean, Div's second operand [2,5,1] differs from gamma's [8]."""
+    m, x, out, g, b = _ln_chain_model()
+    assert m.fuse_elemwise_ops() == 2
+    nodes = m.nodes()
+    assert [n["op_name"] for n in nodes] == ["ReduceMean", "Sub", "Pow", "ReduceMean", "FusedElemwise", "Div", "FusedElemwise"]
+    assert m.fused_chain(nodes[4]["id"]) == ["Add", "Sqrt"] and m.fused_chain(nodes[6]["id"]) == ["Mul", "Add"]
+    # inputs of the fused node = the chain's outside operands in order of first use (:95-112), output = the last node's
+    assert nodes[6]["inputs"] == [nodes[5]["outputs"][0], g, b] and nodes[6]["outputs"] == [out] == m.outputs
+    assert len(nodes[4]["inputs"]) == 2 and nodes[5]["inputs"][1] == nodes[4]["outputs"][0]
+    assert m.infer_value_shape(out) == ([2, 5, 8], F32)     # shape.rs:616-650 walks the chain
+    assert m.fuse_elemwise_ops() == 0                        # FusedElemwise itself is not element-wise (op.rs:387-412)
+
+    # a unary node ends a chain: the node after it would need a binary predecessor (:44)
+    m = Model()
+    x = m.new_val_named_and_shaped("x", [4, 4])
+    v = [m.new_val() for _ in range(3)]
+    m.add_node(Op.Add, [x, x], [v[0]])
+    m.add_node(Op.Sqrt, [v[0]], [v[1]])
+    m.add_node(Op.ReLU, [v[1]], [v[2]])
+    m.add_input(x)
+    m.add_output(v[2])
+    assert m.fuse_elemwise_ops() == 1
+    assert [n["op_name"] for n in m.nodes()] == ["FusedElemwise", "ReLU"]
+
+    # the approximated functions are not element-wise for the reference (op.rs:400-409): nothing to fuse
+    m = Model()
+    x = m.new_val_named_and_shaped("x", [3, 7])
+    out = erf_gelu_chain(m, x)
+    m.add_input(x)
+    m.add_output(out)
+    assert m.fuse_elemwise_ops() == 0 and len(m.nodes()) == 5
+
+
+def test_fuse_elemwise_ops_extended_rule():
+    m = Model()
+    x = m.new_val_named_and_shaped("x", [3, 7])
+    out = erf_gelu_chain(m, x)
+    m.add_input(x)
+    m.add_output(out)
+    assert m.fuse_elemwise_ops(extended=True) == 1
+    (n,) = m.nodes()
+    assert m.fused_chain(n["id"]) == ["Div", "Erf", "Add", "Mul", "Mul"]
+    assert n["inputs"][0] == x and len(n["inputs"]) == 4 and n["outputs"] == m.outputs   # x, sqrt 2, 1, 0.5: x only once
+    assert m.infer_value_shape(out) == ([3, 7], F32)
+    assert [p[0] for p in m.execution_plan()] == [n["id"]]
+
+    # The LayerNorm chain: Add(eps) -> Sqrt -> Div(d, .) -> Mul(gamma) -> Add(beta) is one chain, the square root
+    # being the SECOND operand of the Div; its [2,5,1] intermediates are computed at the output's extent.
+    m, x, out, g, b = _ln_chain_model()
+    assert m.fuse_elemwise_ops(extended=True) == 1
+    nodes = m.nodes()
+    assert [n["op_name"] for n in nodes] == ["ReduceMean", "Sub", "Pow", "ReduceMean", "FusedElemwise"]
+    assert m.fused_chain(nodes[4]["id"]) == ["Add", "Sqrt", "Div", "Mul", "Add"]
+    assert nodes[4]["inputs"][0] == nodes[3]["outputs"][0] and nodes[4]["inputs"][2:] == [nodes[1]["outputs"][0], g, b]
+    assert m.infer_value_shape(out) == ([2, 5, 8], F32)
+
+    # a value that is also a graph output ends its chain; an integer tensor is never fused
+    m = Model()
+    x = m.new_val_named_and_shaped("x", [4])
+    i = m.new_val_named_and_shaped("i", [4], I64)
+    a, b2, c, d = (m.new_val() for _ in range(4))
+    m.add_node(Op.Sqrt, [x], [a])
+    m.add_node(Op.ReLU, [a], [b2])
+    m.add_node(Op.Tanh, [b2], [c])
+    m.add_node(Op.Add, [i, i], [d])
+    m.add_input(x)
+    m.add_input(i)
+    for o in (a, c, d):
+        m.add_output(o)
+    assert m.fuse_elemwise_ops(extended=True) == 1
+    assert sorted(n["op_name"] for n in m.nodes()) == ["Add", "FusedElemwise", "Sqrt"]
+
+    # chains are cut at 16 steps and at 6 distinct outside operands
+    m = Model()
+    x = m.new_val_named_and_shaped("x", [8])
+    cur = x
+    for _ in range(20):
+        nxt = m.new_val()
+        m.add_node(Op.ReLU, [cur], [nxt])
+        cur = nxt
+    m.add_input(x)
+    m.add_output(cur)
+    assert m.fuse_elemwise_ops(extended=True) == 2
+    assert [len(m.fused_chain(n["id"])) for n in m.nodes()] == [16, 4]
+    m = Model()
+    x = m.new_val_named_and_shaped("x", [8])
+    cur = x
+    for k in range(9):
+        nxt = m.new_val()
+        m.add_node(Op.Add, [cur, m.new_initializer(np.full(8, k, np.float32))], [nxt])
+        cur = nxt
+    m.add_input(x)
+    m.add_output(cur)
+    assert m.fuse_elemwise_ops(extended=True) == 2
+    assert [len(n["inputs"]) for n in m.nodes()] == [6, 5]   # x + 5 constants, then the first result + 4 constants
+
+    with pytest.raises(AltiusHipError) as e:                  # shape inference fails -> ShapeError, as in the reference
+        m = Model()
+        p, q, r = m.new_val_named_and_shaped("p", [2, 3]), m.new_val_named_and_shaped("q", [4]), m.new_val()
+        m.add_node(Op.Add, [p, q], [r])
+        m.add_input(p)
+        m.add_input(q)
+        m.add_output(r)
+        m.fuse_elemwise_ops()
+    assert e.value.code == ERR_SHAPE
