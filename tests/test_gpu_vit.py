@@ -148,3 +148,38 @@ def test_vit_from_onnx_bytes(case):
     np.testing.assert_allclose(plain, oracle_vit(image, params, fused=False), rtol=2e-4, atol=2e-4)
     # the two reference paths differ only by their GELU approximations
     assert np.max(np.abs(plain - logits)) < 0.2
+
+
+def test_inference_session_like_altius_py(case, tmp_path):
+    """altius_py.InferenceSession(path).run(None, {name: array}) (crates/altius_py/altius_py/__init__.py:4-30) with
+    the rewrite pipeline of altius_py.session (crates/altius_py/src/lib.rs:52-62) on this backend."""
+    case("InferenceSession on a ViT file")
+    from altius_amd.inference import InferenceSession, load, session
+
+    data, params = make_vit()
+    path = tmp_path / "vit.onnx"
+    path.write_bytes(data)
+    image = rnd(B, 3, IMG, IMG)
+    sess = InferenceSession(str(path), enable_profile=True)
+    (logits,) = sess.run(None, {"image": image})
+    np.testing.assert_allclose(logits, oracle_vit(image, params, fused=True), rtol=2e-4, atol=2e-4)
+    assert "LayerNormalization" in sess.session.profile()
+    with pytest.raises(RuntimeError, match="not found"):
+        sess.run(None, {"picture": image})
+    with pytest.raises(RuntimeError, match="Unknown backend"):
+        session(load(str(path)), backend="cuda")
+
+
+def test_elementwise_fusion_keeps_the_bits_of_the_plain_graph(case):
+    """The exporter's graph with only fuse_elemwise_ops applied: fewer nodes, the same logits bit for bit."""
+    case("ViT with element-wise chains fused")
+    data, _ = make_vit()
+    image = rnd(B, 3, IMG, IMG)
+    plain = Model.load_onnx_from_buffer(data)
+    fused = plain.clone()
+    n = fused.fuse_elemwise_ops(extended=True)
+    ops = [k["op_name"] for k in fused.nodes()]
+    assert n >= 3 * LAYERS + 1 and ops.count("FusedElemwise") == n and "Erf" not in ops
+    (want,) = HipSessionBuilder(plain).build().run([image])
+    (got,) = HipSessionBuilder(fused).build().run([image])
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
