@@ -308,6 +308,12 @@ int ahip_softmax_lastaxis(ahip_ctx *ctx, float *out, const float *in, size_t row
     return altius::launch_softmax(ctx->d, out, in, rows, len);
 }
 
+int ahip_softmax_lastaxis_prologue(ahip_ctx *ctx, float *out, const float *in, size_t rows, size_t len, int scale_op, float scale,
+                                   const float *mask, size_t rows_per_mask) {
+    REQUIRE_CTX(ctx, "ahip_softmax_lastaxis_prologue");
+    return altius::launch_softmax_prologue(ctx->d, out, in, rows, len, scale_op, scale, mask, rows_per_mask);
+}
+
 int ahip_layernorm_lastaxis(ahip_ctx *ctx, float *out, const float *in, const float *gamma, const float *beta,
                             size_t rows, size_t len, float eps) {
     REQUIRE_CTX(ctx, "ahip_layernorm_lastaxis");

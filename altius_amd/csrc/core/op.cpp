@@ -52,6 +52,14 @@ bool Op::set_int(const std::string &n, int64_t v) {
 }
 
 bool Op::get_int(const std::string &n, int64_t *v) const {
+    if (kind == OpKind::Softmax && n == "prologue_scale") {
+        *v = prologue_scale;
+        return true;
+    }
+    if (kind == OpKind::Softmax && n == "prologue_mask") {
+        *v = prologue_mask ? 1 : 0;
+        return true;
+    }
     if (n == "axis" && is(kind, {OpKind::Softmax, OpKind::LayerNormalization, OpKind::Concat, OpKind::Flatten,
                                  OpKind::Gather, OpKind::Split})) {
         *v = axis;

@@ -66,6 +66,11 @@ struct Op {
     std::shared_ptr<Tensor> value;
     // FusedElemwise (op.rs:213-217)
     std::shared_ptr<const FusedElemwise> fused;
+    // Not in the reference: a Softmax that absorbed the Mul / Div by one value and the mask Add in front
+    // of it (fuse_softmax_prologue).  Its inputs are then x, the scale value if prologue_scale != 0
+    // (1: x * scale, 2: x / scale), and the mask if prologue_mask.
+    int prologue_scale = 0;
+    bool prologue_mask = false;
 
     Op() = default;
     explicit Op(OpKind k) : kind(k) {}

@@ -377,4 +377,100 @@ bool fuse_elemwise_ops(Model &model, ElemwiseFusionRule rule, size_t *count, std
     return true;
 }
 
+size_t fuse_softmax_prologue(Model &model) {
+    const auto users = model.get_value_users();
+    const auto parents = model.get_value_parents();
+    std::map<ValueId, TypedFixedShape> shapes;
+    ShapeError serr;
+    if (!infer_shapes(model, nullptr, &shapes, &serr)) return 0;
+    const auto &outs = model.graph.outputs;
+    auto single_use = [&](ValueId v) {
+        auto u = users.find(v);
+        return u != users.end() && u->second.size() == 1 && std::find(outs.begin(), outs.end(), v) == outs.end();
+    };
+    auto dims_of = [&](ValueId v) -> const FixedDimensions * {
+        auto it = shapes.find(v);
+        return it == shapes.end() || it->second.elem_ty != TensorElemType::F32 ? nullptr : &it->second.dims;
+    };
+    auto one_value_init = [&](ValueId v) {
+        const Tensor *t = init_of(model, v);
+        return t && t->elem_ty() == TensorElemType::F32 && t->dims().total_elems() == 1 && t->nbytes() == sizeof(float);
+    };
+    // Constant along every axis but the first and the last, and not growing x.
+    auto mask_fits = [&](const FixedDimensions &m, const FixedDimensions &x) {
+        if (x.len() < 1 || m.len() > x.len() || m.len() == 0) return false;
+        const size_t off = x.len() - m.len();
+        for (size_t i = 0; i < m.len(); i++) {
+            const size_t xi = i + off;
+            if (xi == x.len() - 1) {
+                if (m[i] != x[xi]) return false;
+            } else if (xi == 0) {
+                if (m[i] != x[xi] && m[i] != 1) return false;
+            } else if (m[i] != 1) {
+                return false;
+            }
+        }
+        return true;
+    };
+
+    size_t count = 0;
+    std::vector<NodeId> doomed;
+    for (NodeId sid : model.topo_sort_nodes()) {
+        Node &sm = model.graph.nodes[sid];
+        if (sm.op.kind != OpKind::Softmax || sm.inputs.size() != 1 || sm.op.prologue_scale || sm.op.prologue_mask) continue;
+        const FixedDimensions *xd = dims_of(sm.inputs[0]);
+        if (!xd || xd->len() == 0 || !(sm.op.axis == -1 || sm.op.axis == (int64_t)xd->len() - 1)) continue;
+
+        ValueId x = sm.inputs[0];
+        std::optional<ValueId> mask, scale;
+        int scale_code = 0;
+        std::vector<NodeId> absorbed;
+        // the mask Add, directly in front of the Softmax
+        auto p = parents.find(x);
+        if (p != parents.end() && single_use(x)) {
+            const Node &add = model.graph.nodes[p->second];
+            if (add.op.kind == OpKind::Add && add.inputs.size() == 2 && add.outputs.size() == 1) {
+                for (int side = 0; side < 2 && !mask; side++) {
+                    const ValueId data = add.inputs[side], m = add.inputs[1 - side];
+                    const FixedDimensions *dd = dims_of(data), *md = dims_of(m);
+                    if (dd && md && *dd == *xd && mask_fits(*md, *xd)) {
+                        mask = m;
+                        x = data;
+                        absorbed.push_back(p->second);
+                    }
+                }
+            }
+        }
+        // the scale, in front of that
+        p = parents.find(x);
+        if (p != parents.end() && single_use(x)) {
+            const Node &sc = model.graph.nodes[p->second];
+            if ((sc.op.kind == OpKind::Mul || sc.op.kind == OpKind::Div) && sc.inputs.size() == 2 && sc.outputs.size() == 1) {
+                const bool mul = sc.op.kind == OpKind::Mul;
+                for (int side = 0; side < (mul ? 2 : 1) && !scale; side++) {  // x / c only; c * x or x * c
+                    const ValueId data = sc.inputs[side], c = sc.inputs[1 - side];
+                    const FixedDimensions *dd = dims_of(data);
+                    if (dd && *dd == *xd && one_value_init(c)) {
+                        scale = c;
+                        scale_code = mul ? 1 : 2;
+                        x = data;
+                        absorbed.push_back(p->second);
+                    }
+                }
+            }
+        }
+        if (!mask && !scale) continue;
+        sm.inputs.assign(1, x);
+        if (scale) sm.inputs.push_back(*scale);
+        if (mask) sm.inputs.push_back(*mask);
+        sm.op.prologue_scale = scale_code;
+        sm.op.prologue_mask = mask.has_value();
+        doomed.insert(doomed.end(), absorbed.begin(), absorbed.end());
+        count++;
+    }
+    for (NodeId id : doomed) model.graph.nodes[id].deleted = true;
+    if (count) model.remove_unnecessary_nodes();
+    return count;
+}
+
 }  // namespace altius

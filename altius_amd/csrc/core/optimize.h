@@ -44,6 +44,14 @@ size_t eliminate_identity(Model &model);
 // Under both rules a value that is also a graph output ends the chain (the reference would drop such an
 // output).  Needs every shape it looks at to be inferable; returns false with *err set when shape
 // inference fails.  *count receives the number of chains fused.
+// Not in the reference.  [Mul | Div by a one-element f32 initializer] -> [Add of a mask] -> Softmax(last axis)
+// => one Softmax node with inputs (x, scale?, mask?) and Op::prologue_scale / prologue_mask set, which the
+// session runs as one kernel with the bits of the separate nodes.  Either prologue operator may be absent (not
+// both); intermediates must have no other reader and must not be graph outputs; the mask must be f32 of
+// known shape, broadcast onto x without changing x's shape, and constant along every axis but the first and
+// the last ([N,1,1,C], [1,1,1,C], [C]).  Returns the number of Softmax nodes rewritten.
+size_t fuse_softmax_prologue(Model &model);
+
 enum class ElemwiseFusionRule { ReferenceRule = 0, ExtendedRule = 1 };
 bool fuse_elemwise_ops(Model &model, ElemwiseFusionRule rule, size_t *count, std::string *err);
 

@@ -60,6 +60,10 @@ int launch_unary(DeviceCtx &ctx, int op, float *out, const float *in, size_t n, 
 int launch_fused_elemwise(DeviceCtx &ctx, float *out, int rank, const int64_t *out_dims, int n_inputs, const float *const *inputs,
                           const int64_t *const *input_strides, int n_steps, const ahip_fused_step *steps);
 int launch_softmax(DeviceCtx &ctx, float *out, const float *in, size_t rows, size_t len);
+// Softmax of (in [*|/] scale) + mask over the last axis; scale_op 0 none / 1 multiply / 2 divide, mask (may be
+// null) holds rows / rows_per_mask rows of len values.  AHIP_ERR_UNSUPPORTED when the geometry needs separate kernels.
+int launch_softmax_prologue(DeviceCtx &ctx, float *out, const float *in, size_t rows, size_t len, int scale_op, float scale,
+                            const float *mask, size_t rows_per_mask);
 int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *gamma,
                      const float *beta, size_t rows, size_t len, float eps);
 int launch_reduce(DeviceCtx &ctx, int kind, float *out, const float *in, size_t outer, size_t red,

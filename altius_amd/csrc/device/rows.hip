@@ -81,9 +81,22 @@ template <int VEC, int NCH> struct RowRegs {
 // ---------------------------------------------------------------------------
 // Softmax
 // ---------------------------------------------------------------------------
-template <int VEC, int NCH>
+// What may happen to the scores on their way into Softmax, in this order: a multiplication or
+// division by one value (the 1/sqrt(d) of attention), then the addition of a mask that holds one
+// row per `rows_per_mask` consecutive score rows ([N,1,1,C] onto [N,H,R,C]: H*R rows).  Each is the
+// single IEEE operation the stand-alone Mul / Div / Add kernel performs, so Softmax sees the same
+// bits; what disappears is one pass over the scores per operation.
+struct SoftmaxPrologue {
+    int scale_code;  // 0: none, 1: x * scale, 2: x / scale
+    float scale;
+    const float *mask;  // null: none
+    uint32_t rows_per_mask;
+    uint32_t mask_rows;
+};
+
+template <int VEC, int NCH, bool PRO>
 __global__ __launch_bounds__(BLOCK) void softmax_wave(float *__restrict__ out, const float *__restrict__ in,
-                                                      size_t rows, int len) {
+                                                      size_t rows, int len, const SoftmaxPrologue pro) {
     const int lane = threadIdx.x & (WAVE - 1);
     const size_t row = (size_t)blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
     if (row >= rows) return;
@@ -93,6 +106,23 @@ __global__ __launch_bounds__(BLOCK) void softmax_wave(float *__restrict__ out, c
     RowRegs<VEC, NCH> r;
     const float nan = __builtin_nanf("");
     r.load(x, len, lane, nan);
+    if (PRO) {
+        // The mask row is shared by rows_per_mask score rows: it comes from the caches, and its load
+        // is issued before the scores are looked at.
+        RowRegs<VEC, NCH> m;
+        if (pro.mask) m.load(pro.mask + (size_t)((uint32_t)row / pro.rows_per_mask) * len, len, lane, 0.0f);
+        if (pro.scale_code == 1) {
+#pragma unroll
+            for (int s = 0; s < NCH * VEC; s++) r.v[s] = r.v[s] * pro.scale;
+        } else if (pro.scale_code == 2) {
+#pragma unroll
+            for (int s = 0; s < NCH * VEC; s++) r.v[s] = r.v[s] / pro.scale;
+        }
+        if (pro.mask) {
+#pragma unroll
+            for (int s = 0; s < NCH * VEC; s++) r.v[s] = r.v[s] + m.v[s];  // slots past the row stay NaN
+        }
+    }
 
     float mx = nan;  // fold(NAN, max): NaN elements are ignored
 #pragma unroll
@@ -139,9 +169,9 @@ constexpr int LDS_WAVES = LDS_BLOCK / WAVE;
 constexpr int STAGE_LDS = 2;                                         // float4 per lane staged through registers
 constexpr size_t LDS_GROUP_FLOATS = (size_t)STAGE_LDS * LDS_BLOCK * 4;  // 8192 floats = 32 KiB of LDS at most
 
-template <int SUB, int NCH, bool NT>
+template <int SUB, int NCH, bool NT, bool PRO>
 __global__ __launch_bounds__(LDS_BLOCK) void softmax_lds(float *__restrict__ out, const float *__restrict__ in,
-                                                         size_t rows, int len, int group_rows) {
+                                                         size_t rows, int len, int group_rows, const SoftmaxPrologue pro) {
     extern __shared__ __align__(16) float lds[];
     const int tid = threadIdx.x;
     const int lane = tid & (WAVE - 1);
@@ -175,6 +205,19 @@ __global__ __launch_bounds__(LDS_BLOCK) void softmax_lds(float *__restrict__ out
         }
     }
     for (int i = (n4 << 2) + tid; i < n; i += LDS_BLOCK) lds[i] = src[i];  // ragged end of the last group
+    // The group's rows use at most two consecutive mask rows (the host checks rows_per_mask >=
+    // group_rows); they go to LDS behind the scores, once per block.
+    float *mask_lds = lds + (size_t)group_rows * len;
+    uint32_t second_mask_from = 0xFFFFFFFFu;  // first row of the group (block-relative) that uses the second mask row
+    if (PRO && pro.mask) {
+        const uint32_t m0 = (uint32_t)(row0 / pro.rows_per_mask);
+        const size_t boundary = (size_t)(m0 + 1) * pro.rows_per_mask;  // first score row of mask row m0 + 1
+        const bool two = boundary < row0 + (size_t)nrows;
+        if (two) second_mask_from = (uint32_t)(boundary - row0);
+        const int count = two ? 2 * len : len;
+        const float *m = pro.mask + (size_t)m0 * len;
+        for (int i = tid; i < count; i += LDS_BLOCK) mask_lds[i] = m[i];
+    }
     __syncthreads();
 
     constexpr int RPP = WAVE / SUB;  // rows per wave pass
@@ -193,6 +236,21 @@ __global__ __launch_bounds__(LDS_BLOCK) void softmax_lds(float *__restrict__ out
 #pragma unroll
         for (int k = 0; k < LAST; k++) x[k] = row[SUB * k];
         x[LAST] = last_valid ? row[SUB * LAST] : nan;
+        if (PRO) {
+            if (pro.scale_code == 1) {
+#pragma unroll
+                for (int k = 0; k < NCH; k++) x[k] = x[k] * pro.scale;
+            } else if (pro.scale_code == 2) {
+#pragma unroll
+                for (int k = 0; k < NCH; k++) x[k] = x[k] / pro.scale;
+            }
+            if (pro.mask) {
+                const float *mrow = mask_lds + ((uint32_t)r >= second_mask_from ? len : 0) + s;
+#pragma unroll
+                for (int k = 0; k < LAST; k++) x[k] = x[k] + mrow[SUB * k];
+                if (last_valid) x[LAST] = x[LAST] + mrow[SUB * LAST];
+            }
+        }
         float mx = nan;  // fold(NAN, max): NaN elements are ignored
 #pragma unroll
         for (int k = 0; k < NCH; k++) mx = nanmax(x[k], mx);
@@ -348,10 +406,13 @@ bool dispatch_wave(bool vec4, size_t len, Args... args) {
 }
 
 template <int VEC, int NCH> struct SoftmaxLauncher {
-    static void go(hipStream_t s, float *out, const float *in, size_t rows, int len) {
+    static void go(hipStream_t s, float *out, const float *in, size_t rows, int len, const SoftmaxPrologue *pro) {
         const size_t blocks = (rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-        hipLaunchKernelGGL((softmax_wave<VEC, NCH>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, rows,
-                           len);
+        if (pro)
+            hipLaunchKernelGGL((softmax_wave<VEC, NCH, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, rows, len, *pro);
+        else
+            hipLaunchKernelGGL((softmax_wave<VEC, NCH, false>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, rows, len,
+                               SoftmaxPrologue{0, 0.0f, nullptr, 1, 0});
     }
 };
 
@@ -369,11 +430,18 @@ template <int VEC, int NCH> struct LayerNormLauncher {
 // 256 elements, 32 up to 512, 64 above.
 template <int SUB, int NCH>
 void softmax_lds_go(bool nt, dim3 grid, size_t shmem, hipStream_t s, float *out, const float *in, size_t rows,
-                    int len, int g) {
-    if (nt)
-        hipLaunchKernelGGL((softmax_lds<SUB, NCH, true>), grid, dim3(LDS_BLOCK), shmem, s, out, in, rows, len, g);
-    else
-        hipLaunchKernelGGL((softmax_lds<SUB, NCH, false>), grid, dim3(LDS_BLOCK), shmem, s, out, in, rows, len, g);
+                    int len, int g, const SoftmaxPrologue *pro) {
+    const SoftmaxPrologue none{0, 0.0f, nullptr, 1, 0};
+    if (pro) {
+        if (nt)
+            hipLaunchKernelGGL((softmax_lds<SUB, NCH, true, true>), grid, dim3(LDS_BLOCK), shmem, s, out, in, rows, len, g, *pro);
+        else
+            hipLaunchKernelGGL((softmax_lds<SUB, NCH, false, true>), grid, dim3(LDS_BLOCK), shmem, s, out, in, rows, len, g, *pro);
+    } else if (nt) {
+        hipLaunchKernelGGL((softmax_lds<SUB, NCH, true, false>), grid, dim3(LDS_BLOCK), shmem, s, out, in, rows, len, g, none);
+    } else {
+        hipLaunchKernelGGL((softmax_lds<SUB, NCH, false, false>), grid, dim3(LDS_BLOCK), shmem, s, out, in, rows, len, g, none);
+    }
 }
 
 size_t gcd_size(size_t a, size_t b) {
@@ -400,17 +468,26 @@ size_t softmax_lds_group_rows(size_t len) {
     return 4;  // unreachable for len <= 1024: 4 rows are at most 4096 floats
 }
 
-bool softmax_lds_launch(hipStream_t s, float *out, const float *in, size_t rows, size_t len, bool nt) {
+bool softmax_lds_launch(hipStream_t s, float *out, const float *in, size_t rows, size_t len, bool nt,
+                        const SoftmaxPrologue *pro = nullptr) {
     static_assert(4 * 1024 <= LDS_GROUP_FLOATS, "four rows of the longest supported length must fit");
-    const size_t g = softmax_lds_group_rows(len);
+    size_t g = softmax_lds_group_rows(len);
+    // A group may straddle one boundary between mask rows, not more: with a mask, groups are cut
+    // down to a line-aligned row count that does not exceed the rows of one mask row.
+    if (pro && pro->mask && pro->rows_per_mask < g) {
+        size_t base = 32 / gcd_size(len, 32);
+        while (base > 1 && base > pro->rows_per_mask) base /= 2;  // fall back to 64-, 32-, 16-byte aligned groups
+        g = pro->rows_per_mask / base * base;
+        if (g == 0) return false;
+    }
     const size_t groups = (rows + g - 1) / g;
     if (groups > 0x7FFFFFFFu) return false;
     const dim3 grid((unsigned)groups);
-    const size_t shmem = g * len * sizeof(float);
+    const size_t shmem = (g * len + (pro && pro->mask ? 2 * len : 0)) * sizeof(float);
     const int L = (int)len, G = (int)g;
 #define ALTIUS_GO(SUB, N)                                                    \
     case N:                                                                  \
-        softmax_lds_go<SUB, N>(nt, grid, shmem, s, out, in, rows, L, G);     \
+        softmax_lds_go<SUB, N>(nt, grid, shmem, s, out, in, rows, L, G, pro); \
         return true;
     if (len <= 256) {
         switch ((L + 15) / 16) {
@@ -453,7 +530,7 @@ int launch_softmax(DeviceCtx &ctx, float *out, const float *in, size_t rows, siz
         if (aligned && !wave_fits) {
             if (!softmax_lds_launch(ctx.stream, out, in, rows, len, ctx.streaming(rows * len * sizeof(float))))
                 return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: too many rows for one launch");
-        } else if (!dispatch_wave<SoftmaxLauncher>(vec4, len, ctx.stream, out, in, rows, (int)len)) {
+        } else if (!dispatch_wave<SoftmaxLauncher>(vec4, len, ctx.stream, out, in, rows, (int)len, (const SoftmaxPrologue *)nullptr)) {
             return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: no wave layout for this row length");
         }
     } else {
@@ -462,6 +539,32 @@ int launch_softmax(DeviceCtx &ctx, float *out, const float *in, size_t rows, siz
                            len);
     }
     return ctx.check(hipGetLastError(), "softmax launch");
+}
+
+int launch_softmax_prologue(DeviceCtx &ctx, float *out, const float *in, size_t rows, size_t len, int scale_op, float scale,
+                            const float *mask, size_t rows_per_mask) {
+    if (scale_op < 0 || scale_op > 2) return ctx.fail(AHIP_ERR_ARG, "softmax: scale_op must be 0 (none), 1 (multiply) or 2 (divide)");
+    if (rows == 0 || len == 0) return AHIP_OK;
+    if (!out || !in) return ctx.fail(AHIP_ERR_ARG, "softmax: null tensor pointer");
+    if (mask && (rows_per_mask == 0 || rows % rows_per_mask != 0))
+        return ctx.fail(AHIP_ERR_ARG, "softmax: the row count must be a multiple of rows_per_mask");
+    if (scale_op == 0 && !mask) return launch_softmax(ctx, out, in, rows, len);
+    // The same kernel choice as launch_softmax, so that the row sums are accumulated in the same order and
+    // the result has the bits of the separate operators.  Unaligned tensors and rows beyond 1024 elements
+    // are left to the caller's operator-by-operator route.
+    if (len > MAX_WAVE_ROW || !aligned16(out) || !aligned16(in) || rows >= ((size_t)1 << 32) || rows_per_mask >= ((size_t)1 << 32))
+        return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax prologue: needs 16-byte aligned tensors and rows of at most 1024 elements");
+    SoftmaxPrologue pro{scale_op, scale, mask, (uint32_t)(mask ? rows_per_mask : 1), (uint32_t)(mask ? rows / rows_per_mask : 0)};
+    const size_t slots = (len + 255) / 256 * 256;
+    const bool wave_fits = len % 4 == 0 && len * 4 >= slots * 3;
+    if (wave_fits) {
+        if (mask && !aligned16(mask)) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax prologue: the mask must be 16-byte aligned");
+        if ((rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK > MAX_GRID || !dispatch_wave<SoftmaxLauncher>(true, len, ctx.stream, out, in, rows, (int)len, (const SoftmaxPrologue *)&pro))
+            return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax prologue: too many rows for one launch");
+    } else if (!softmax_lds_launch(ctx.stream, out, in, rows, len, ctx.streaming(rows * len * sizeof(float)), &pro)) {
+        return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax prologue: too many rows for one launch");
+    }
+    return ctx.check(hipGetLastError(), "softmax (prologue) launch");
 }
 
 int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *gamma, const float *beta,

@@ -931,7 +931,52 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
         if (!(op.axis == -1 || op.axis == (int64_t)rank - 1))  // session.rs:999
             return fail(err, SessionError::Message, "Softmax: only the last axis is supported");
         const size_t len = in[0]->dims[rank - 1];
-        rc = launch_softmax(ctx_, o, f(in[0]), len ? n_out / len : 0, len);
+        const size_t rows = len ? n_out / len : 0;
+        if (!op.prologue_scale && !op.prologue_mask) {
+            rc = launch_softmax(ctx_, o, f(in[0]), rows, len);
+            break;
+        }
+        // Softmax that absorbed its scale and mask (fuse_softmax_prologue): inputs x, scale?, mask?.
+        const size_t n_in = 1 + (op.prologue_scale ? 1 : 0) + (op.prologue_mask ? 1 : 0);
+        if (!need(n_in)) return false;
+        DeviceTensor *scale_t = op.prologue_scale ? in[1] : nullptr;
+        DeviceTensor *mask_t = op.prologue_mask ? in[n_in - 1] : nullptr;
+        float scale = 1.0f;
+        if (scale_t) {
+            if (scale_t->elem_ty != TensorElemType::F32 || scale_t->dims.total_elems() != 1)
+                return fail(err, SessionError::Shape, "Softmax: the absorbed scale must be one f32 value");
+            if (!fetch_host(scale_t, err)) return false;
+            scale = scale_t->host->data_f32()[0];
+        }
+        size_t rows_per_mask = 0;
+        if (mask_t) {
+            if (mask_t->elem_ty != TensorElemType::F32) return fail(err, SessionError::Message, "Softmax: the absorbed mask must be f32");
+            const size_t m_elems = mask_t->dims.total_elems();
+            if (len == 0 || m_elems % len != 0 || m_elems == 0 || rows % (m_elems / len) != 0 ||
+                (m_elems / len != 1 && m_elems / len != in[0]->dims[0]))
+                return fail(err, SessionError::Shape, "Softmax: the absorbed mask does not fit the scores");
+            rows_per_mask = rows / (m_elems / len);
+        }
+        rc = launch_softmax_prologue(ctx_, o, f(in[0]), rows, len, op.prologue_scale, scale, mask_t ? f(mask_t) : nullptr, rows_per_mask);
+        if (rc == AHIP_ERR_UNSUPPORTED) {
+            // Geometry the one-kernel route does not take: the same operators one after the other, in place.
+            const std::vector<int64_t> xd = i64v(out.dims), xs = i64v(out.dims.strides());
+            const std::vector<int64_t> zero(xd.size(), 0);
+            const float *cur = f(in[0]);
+            rc = AHIP_OK;
+            if (scale_t) {
+                rc = launch_binary(ctx_, op.prologue_scale == 1 ? AHIP_MUL : AHIP_DIV, o, cur, f(scale_t), (int)xd.size(), xd.data(), xs.data(), zero.data());
+                cur = o;
+            }
+            if (!rc && mask_t) {
+                auto ms = mask_t->dims.strides_for_broadcasting_to(out.dims);
+                if (!ms) return fail(err, SessionError::Shape, "Softmax: the absorbed mask does not broadcast to the scores");
+                const std::vector<int64_t> msv = i64v(*ms);
+                rc = launch_binary(ctx_, AHIP_ADD, o, cur, f(mask_t), (int)xd.size(), xd.data(), xs.data(), msv.data());
+                cur = o;
+            }
+            if (!rc) rc = launch_softmax(ctx_, o, cur, rows, len);
+        }
         break;
     }
     case OpKind::LayerNormalization: {

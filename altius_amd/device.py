@@ -240,6 +240,29 @@ class Context:
             self.free(dx)
             self.free(do)
 
+    def softmax_prologue(self, x, scale_op=0, scale=1.0, mask=None):
+        """softmax((x [*|/] scale) + mask) in one kernel; scale_op 0 none, 1 multiply, 2 divide; mask holds
+        x.size / (mask rows * length) consecutive rows of x per mask row."""
+        x = np.asarray(x, dtype=np.float32, order="C")
+        length = x.shape[-1]
+        rows = x.size // length if length else 0
+        dx = self.upload(x)
+        do = self.alloc(max(x.nbytes, 4))
+        dm, rpm = None, 0
+        if mask is not None:
+            mask = np.asarray(mask, dtype=np.float32, order="C")
+            assert mask.shape[-1] == length and rows % (mask.size // length) == 0
+            rpm = rows // (mask.size // length)
+            dm = self.upload(mask)
+        try:
+            check(self.L.ahip_softmax_lastaxis_prologue(self.handle, do.ptr, dx.ptr, rows, length, scale_op, float(scale),
+                                                        dm.ptr if dm else None, rpm), self.handle)
+            return self.download(do, x.shape)
+        finally:
+            for b in (dx, do, dm):
+                if b is not None:
+                    self.free(b)
+
     def layer_norm(self, x, gamma, beta, eps=1e-5):
         x = np.asarray(x, dtype=np.float32, order="C")
         gamma = np.asarray(gamma, dtype=np.float32, order="C")

@@ -386,6 +386,10 @@ class Model:
     def eliminate_identity(self):
         return self._pass(self.L.ahip_eliminate_identity)
 
+    def fuse_softmax_prologue(self):
+        """[Mul | Div by a constant] -> [Add mask] -> Softmax becomes one Softmax node with inputs (x, scale?, mask?)."""
+        return self._pass(self.L.ahip_fuse_softmax_prologue)
+
     def fuse_elemwise_ops(self, extended=False):
         """Chains of element-wise operators -> FusedElemwise nodes; the reference's rule, or this backend's
         wider one with extended=True.  Returns the number of chains fused."""

@@ -185,6 +185,15 @@ int ahip_fused_use_compiled_chains(ahip_ctx *ctx, int enable);
 /* compute_softmax over the last axis (session.rs:990-1026 + fast_math.rs:102-187):
  * `rows` rows of `len` contiguous elements. */
 int ahip_softmax_lastaxis(ahip_ctx *ctx, float *out, const float *in, size_t rows, size_t len);
+/* Not in the reference: Softmax that applies, while it loads the scores, the two operators exporters put in
+ * front of it in attention -- Mul or Div by one value (scale_op 1 or 2, 0 for none), then Add of a mask
+ * that holds one row of `len` values per `rows_per_mask` consecutive rows (mask may be NULL; [N,1,1,C] onto
+ * [N,H,R,C] has rows_per_mask = H*R, one row for all has rows_per_mask = rows).  Each is the one IEEE
+ * operation ahip_binary performs, so the result has the bits of Mul/Div -> Add -> Softmax run one after the
+ * other, without their two passes over the scores.  AHIP_ERR_UNSUPPORTED (nothing launched) for tensors that
+ * are not 16-byte aligned or rows longer than 1024: run the operators one after the other then. */
+int ahip_softmax_lastaxis_prologue(ahip_ctx *ctx, float *out, const float *in, size_t rows, size_t len,
+                                   int scale_op, float scale, const float *mask, size_t rows_per_mask);
 
 /* compute_layer_normalization over the last axis (session.rs:1433-1486).
  * gamma and beta hold `len` values each. */
@@ -416,6 +425,12 @@ int ahip_eliminate_identity(ahip_model *model, int *count);
  * Under both rules a value that is also a graph output ends its chain.  AHIP_ERR_SHAPE when shape
  * inference fails (the reference returns ShapeError).  The node's operators can be read back with
  * ahip_node_get_attr_string(model, node, "chain", ...) as a comma-separated list of names. */
+/* Not in the reference: [Mul | Div by a one-element f32 initializer] -> [Add of a mask that is constant along
+ * every axis but the first and the last] -> Softmax(last axis) becomes one Softmax node with inputs
+ * (x, scale?, mask?), run as one kernel (ahip_softmax_lastaxis_prologue) with the bits of the separate nodes.
+ * Readable afterwards as the integer attributes "prologue_scale" (0 none, 1 multiply, 2 divide) and
+ * "prologue_mask" of the Softmax node. */
+int ahip_fuse_softmax_prologue(ahip_model *model, int *count);
 enum ahip_fuse_rule { AHIP_FUSE_REFERENCE_RULE = 0, AHIP_FUSE_EXTENDED_RULE = 1 };
 int ahip_fuse_elemwise_ops(ahip_model *model, int rule, int *count);
 

@@ -12,6 +12,7 @@ import pytest
 
 from altius_amd import device as D
 from altius_amd import synth
+from altius_amd._lib import ERR_ARG, ERR_UNSUPPORTED, AltiusHipError
 from conftest import assert_bits_equal, assert_close
 
 pytestmark = pytest.mark.gpu
@@ -309,3 +310,39 @@ def test_reduce_max_all_axes(ctx, oracle, case, shape):
     assert not info["no_reference_kernel"]
     got = ctx.reduce(D.REDUCE_MAX, x, 1, x.size, 1).reshape(exp.shape)
     assert_bits_equal(got, exp, f"reduce_max all {shape}")
+
+
+@pytest.mark.parametrize("shape,mask_shape", [((4, 12, 197, 197), (4, 1, 1, 197)), ((3, 2, 40, 50), (3, 1, 1, 50)),
+                                              ((2, 3, 33, 64), (1, 1, 1, 64)), ((2, 2048, 7), (2, 1, 7)), ((5, 64, 7), (5, 1, 7)), ((6, 3, 9), (6, 1, 9)), ((96, 100), None), ((2, 3, 40, 512), (1, 1, 1, 512)), ((4, 2, 16, 1024), (4, 1, 1, 1024)), ((64, 256), None)])
+@pytest.mark.parametrize("scale_op", [0, 1, 2])
+def test_softmax_with_scale_and_mask_prologue(case, ctx, oracle, shape, mask_shape, scale_op):
+    """softmax((x [*|/] c) + mask) in one kernel has the bits of the oracle's Mul/Div, Add and Softmax one after
+    the other when the kernel's lane layout sums each row in the same order as its plain Softmax -- checked here
+    against this backend's own three kernels bit for bit, and against the oracle's chain at the parity bar."""
+    case(f"softmax prologue {shape} mask {mask_shape} scale_op {scale_op}")
+    if scale_op == 0 and mask_shape is None:
+        pytest.skip("nothing to fuse")
+    x = synth.normal(5, list(shape))
+    mask = None if mask_shape is None else synth.attention_mask(6, list(mask_shape), p_masked=0.2)
+    c = np.float32(0.125) if scale_op == 1 else np.float32(7.9)
+    got = ctx.softmax_prologue(x, scale_op, c, mask)
+    z_gpu, z_cpu = x, x
+    if scale_op:
+        op_g, op_o = (D.MUL, oracle.MUL) if scale_op == 1 else (D.DIV, oracle.DIV)
+        z_gpu, z_cpu = ctx.binary(op_g, z_gpu, np.array(c, np.float32)), oracle.binary(op_o, z_cpu, np.array(c, np.float32))
+    if mask is not None:
+        z_gpu, z_cpu = ctx.binary(D.ADD, z_gpu, mask), oracle.binary(oracle.ADD, z_cpu, mask)
+    assert_bits_equal(z_gpu, z_cpu, "the prologue's operators alone")
+    assert_bits_equal(got, ctx.softmax(z_gpu), "fused vs three kernels")
+    assert_close(got, oracle.softmax(z_cpu), what="fused vs oracle chain")
+
+
+def test_softmax_prologue_refusals(case, ctx):
+    case("softmax prologue: geometry the kernel does not take")
+    x = synth.normal(1, [64, 16])
+    with pytest.raises(AltiusHipError) as e:      # rows longer than the LDS kernel handles
+        ctx.softmax_prologue(synth.normal(3, [4, 2048]), 1, 0.5, None)
+    assert e.value.code == ERR_UNSUPPORTED
+    with pytest.raises(AltiusHipError) as e:
+        ctx.softmax_prologue(x, 3, 0.5, None)
+    assert e.value.code == ERR_ARG

@@ -351,3 +351,46 @@ def test_io_tensors_live_in_recycled_pinned_memory(case):
     assert host_pool_trim() >= 2 * x.nbytes and host_pool_stats()[1] == 0
     (out,) = sess.run([x])                                                             # still works after a trim
     assert_close(out, want, what="after trim")
+
+
+@pytest.mark.parametrize("shape,mask_shape,scale_kind", [
+    ((4, 12, 197, 197), (4, 1, 1, 197), None),          # configs[4]: Add(mask) -> Softmax
+    ((2, 12, 197, 197), (2, 1, 1, 197), "Div"),         # scores / sqrt(d) + mask
+    ((2, 4, 17, 17), None, "Mul"),                      # the ViT test graph's scale only
+    ((3, 2, 5, 2048), (3, 1, 1, 2048), "Mul"),          # rows too long for the one-kernel route: separate kernels, same result
+    ((2, 3, 40, 512), (1, 1, 1, 512), "Div"),           # one mask row for everything
+])
+def test_softmax_with_absorbed_scale_and_mask(case, shape, mask_shape, scale_kind):
+    """fuse_softmax_prologue: one Softmax node in place of [Mul|Div] -> [Add mask] -> Softmax, with the bits of
+    the three nodes run one after the other."""
+    case(f"session softmax prologue {shape} {mask_shape} {scale_kind}")
+    m = Model()
+    x = m.new_val_named_and_shaped("scores", list(shape))
+    cur = x
+    inputs = [synth.normal(61, list(shape))]
+    if scale_kind:
+        nxt = m.new_val()
+        m.add_node(Op.Div if scale_kind == "Div" else Op.Mul, [cur, m.new_initializer(np.array(8.0 if scale_kind == "Div" else 0.125, np.float32))], [nxt])
+        cur = nxt
+    m.add_input(x)
+    if mask_shape is not None:
+        mv = m.new_val_named_and_shaped("mask", list(mask_shape))
+        nxt = m.new_val()
+        m.add_node(Op.Add, [cur, mv], [nxt])
+        cur = nxt
+        m.add_input(mv)
+        inputs.append(synth.attention_mask(62, list(mask_shape), p_masked=0.2))
+    p = m.new_val_named("p")
+    m.add_node(Op.Softmax, [cur], [p], axis=-1)
+    m.add_output(p)
+    fused = m.clone()
+    assert fused.fuse_softmax_prologue() == 1 and [n["op_name"] for n in fused.nodes()] == ["Softmax"]
+    (want,) = HipSessionBuilder(m).build().run(inputs)
+    (got,) = HipSessionBuilder(fused).build().run(inputs)
+    assert_bits_equal(got, want, "one node vs three")
+    z = inputs[0]
+    if scale_kind:
+        z = O.binary(O.DIV if scale_kind == "Div" else O.MUL, z, np.array(8.0 if scale_kind == "Div" else 0.125, np.float32))
+    if mask_shape is not None:
+        z = O.binary(O.ADD, z, inputs[1])
+    assert_close(got, O.softmax(z), what="vs oracle chain")

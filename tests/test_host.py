@@ -456,3 +456,64 @@ def test_fuse_elemwise_ops_extended_rule():
         m.add_output(r)
         m.fuse_elemwise_ops()
     assert e.value.code == ERR_SHAPE
+
+
+def _attention_tail(x_shape, mask_shape, scale_kind="Div", mask_first=False, swap_scale=False):
+    m = Model()
+    x = m.new_val_named_and_shaped("scores", list(x_shape))
+    cur = x
+    c = None
+    if scale_kind:
+        c = m.new_initializer(np.array(8.0, np.float32))
+        nxt = m.new_val()
+        m.add_node(Op.Div if scale_kind == "Div" else Op.Mul, [c, cur] if swap_scale else [cur, c], [nxt])
+        cur = nxt
+    mask = None
+    if mask_shape is not None:
+        mask = m.new_val_named_and_shaped("mask", list(mask_shape))
+        nxt = m.new_val()
+        m.add_node(Op.Add, [mask, cur] if mask_first else [cur, mask], [nxt])
+        cur = nxt
+        m.add_input(mask)
+    p = m.new_val_named("p")
+    m.add_node(Op.Softmax, [cur], [p], axis=-1)
+    m.add_input(x)
+    m.add_output(p)
+    return m, x, c, mask
+
+
+def test_fuse_softmax_prologue():
+    def attr(m, node, name):
+        v = ctypes.c_int64()
+        _lib.check(m.L.ahip_node_get_attr_int(m.handle, node["id"], name.encode(), ctypes.byref(v)))
+        return v.value
+
+    m, x, c, mask = _attention_tail([2, 4, 9, 9], [2, 1, 1, 9])
+    assert m.fuse_softmax_prologue() == 1
+    (sm,) = m.nodes()
+    assert sm["op_name"] == "Softmax" and sm["inputs"] == [x, c, mask] and sm["outputs"] == m.outputs
+    assert attr(m, sm, "prologue_scale") == 2 and attr(m, sm, "prologue_mask") == 1
+    assert m.infer_value_shape(m.outputs[0]) == ([2, 4, 9, 9], F32)
+    assert m.fuse_softmax_prologue() == 0
+
+    m, x, c, mask = _attention_tail([2, 4, 9, 9], [9], scale_kind="Mul", mask_first=True, swap_scale=True)   # c * x, mask + .
+    assert m.fuse_softmax_prologue() == 1
+    (sm,) = m.nodes()
+    assert sm["inputs"] == [x, c, mask] and attr(m, sm, "prologue_scale") == 1
+
+    m, x, c, mask = _attention_tail([2, 4, 9, 9], None, scale_kind="Mul")                                    # scale only
+    assert m.fuse_softmax_prologue() == 1 and m.nodes()[0]["inputs"] == [x, c]
+    m, x, c, mask = _attention_tail([2, 4, 9, 9], [1, 1, 1, 9], scale_kind=None)                             # mask only
+    assert m.fuse_softmax_prologue() == 1 and m.nodes()[0]["inputs"] == [x, mask]
+
+    # left alone: c / x is not a scale; a mask that varies along a middle axis; a mask that grows the scores;
+    # an intermediate that is also a graph output
+    m, *_ = _attention_tail([2, 4, 9, 9], None, scale_kind="Div", swap_scale=True)
+    assert m.fuse_softmax_prologue() == 0 and len(m.nodes()) == 2
+    m, *_ = _attention_tail([2, 4, 9, 9], [2, 4, 1, 9], scale_kind=None)
+    assert m.fuse_softmax_prologue() == 0
+    m, *_ = _attention_tail([1, 4, 9, 9], [2, 1, 1, 9], scale_kind=None)
+    assert m.fuse_softmax_prologue() == 0
+    m, x, c, mask = _attention_tail([2, 4, 9, 9], None, scale_kind="Mul")
+    m.add_output(m.nodes()[0]["outputs"][0])
+    assert m.fuse_softmax_prologue() == 0
