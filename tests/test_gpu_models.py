@@ -1,0 +1,201 @@
+"""Two more whole graphs as ONNX bytes, of the families the reference's scripts run
+(crates/altius_py/mobilenet.py, bert.py): a MobileNetV3-style CNN (stem Conv + BatchNorm + hard-swish,
+inverted-residual blocks with depthwise Conv and squeeze-excite, GlobalAveragePool, classifier Gemm)
+and a BERT-style encoder layer (embedding Gather, the exporter's mask arithmetic
+(1 - mask) * -10000 through Unsqueeze / Cast / Sub / Mul, scaled and masked attention, LayerNorm
+chains, erf-GELU).  Each is loaded, rewritten by the session pipeline of altius_py
+(crates/altius_py/src/lib.rs:52-62) and compared with the same computation carried out node by node
+with the CPU oracle, whose Gelu / LayerNormalization are the fused operators' formulas."""
+import os
+
+import numpy as np
+import pytest
+
+import onnx_writer as W
+import oracle as O
+from altius_amd.graph import Model
+from altius_amd.inference import InferenceSession, session
+from altius_amd.session import HipSessionBuilder
+
+pytestmark = pytest.mark.gpu
+
+RNG = np.random.default_rng(77)
+
+
+def rnd(*shape, scale=1.0, shift=0.0):
+    return (RNG.standard_normal(shape) * scale + shift).astype(np.float32)
+
+
+class G:
+    def __init__(self):
+        self.nodes, self.inits, self.n = [], [], 0
+
+    def c(self, array):
+        name = f"c{len(self.inits)}"
+        self.inits.append(W.tensor(name, np.asarray(array)))
+        return name
+
+    def op(self, op_type, inputs, **attrs):
+        out = f"v{self.n}"
+        self.n += 1
+        self.nodes.append(W.node(op_type, inputs, [out], **attrs))
+        return out
+
+
+# ---- MobileNetV3-style ---------------------------------------------------------------------------------
+def hard_swish_nodes(g, x):
+    return g.op("Mul", [x, g.op("HardSigmoid", [x], alpha=1.0 / 6.0, beta=0.5)])
+
+
+def hard_swish_oracle(x):
+    return O.binary(O.MUL, x, O.unary(O.HARDSIGMOID, x, np.float32(1.0 / 6.0), 0.5))
+
+
+def make_mobilenet(batch=2, classes=10):
+    p = {"stem_w": rnd(16, 3, 3, 3, scale=0.2), "stem_bn": [rnd(16, shift=1.0, scale=0.1), rnd(16, scale=0.1), rnd(16, scale=0.1),
+                                                            np.abs(rnd(16)) + np.float32(0.5)],
+         "blocks": [], "head_w": rnd(classes, 24, scale=0.2), "head_b": rnd(classes, scale=0.1)}
+    g = G()
+    x = g.op("Conv", ["image", g.c(p["stem_w"])], kernel_shape=[3, 3], strides=[2, 2], pads=[1, 1, 1, 1])
+    x = g.op("BatchNormalization", [x] + [g.c(t) for t in p["stem_bn"]], epsilon=1e-5)
+    x = hard_swish_nodes(g, x)
+    cin = 16
+    for cexp, cout, stride, k in ((32, 16, 1, 3), (48, 24, 2, 5)):
+        blk = {"exp_w": rnd(cexp, cin, 1, 1, scale=0.2), "exp_b": rnd(cexp, scale=0.1),
+               "dw_w": rnd(cexp, 1, k, k, scale=0.2), "dw_b": rnd(cexp, scale=0.1),
+               "se1_w": rnd(cexp // 4, cexp, 1, 1, scale=0.2), "se1_b": rnd(cexp // 4, scale=0.1),
+               "se2_w": rnd(cexp, cexp // 4, 1, 1, scale=0.2), "se2_b": rnd(cexp, scale=0.1),
+               "proj_w": rnd(cout, cexp, 1, 1, scale=0.2), "proj_b": rnd(cout, scale=0.1), "stride": stride, "k": k,
+               "residual": stride == 1 and cin == cout}
+        p["blocks"].append(blk)
+        y = hard_swish_nodes(g, g.op("Conv", [x, g.c(blk["exp_w"]), g.c(blk["exp_b"])], kernel_shape=[1, 1]))
+        y = g.op("Conv", [y, g.c(blk["dw_w"]), g.c(blk["dw_b"])], kernel_shape=[k, k], strides=[stride, stride],
+                 pads=[k // 2] * 4, group=cexp)
+        y = g.op("Relu", [y])
+        s = g.op("GlobalAveragePool", [y])
+        s = g.op("Relu", [g.op("Conv", [s, g.c(blk["se1_w"]), g.c(blk["se1_b"])], kernel_shape=[1, 1])])
+        s = g.op("HardSigmoid", [g.op("Conv", [s, g.c(blk["se2_w"]), g.c(blk["se2_b"])], kernel_shape=[1, 1])], alpha=1.0 / 6.0, beta=0.5)
+        y = g.op("Mul", [y, s])
+        y = g.op("Conv", [y, g.c(blk["proj_w"]), g.c(blk["proj_b"])], kernel_shape=[1, 1])
+        x = g.op("Add", [x, y]) if blk["residual"] else y
+        cin = cout
+    x = g.op("Flatten", [g.op("GlobalAveragePool", [x])], axis=1)
+    logits = g.op("Gemm", [x, g.c(p["head_w"]), g.c(p["head_b"])], transB=1)
+    g.nodes.append(W.node("Identity", [logits], ["logits"]))
+    data = W.model(W.graph(g.nodes, g.inits, [W.value_info("image", W.FLOAT, [batch, 3, 32, 32])],
+                           [W.value_info("logits", W.FLOAT, [batch, classes])]), opsets=(("", 13),))
+    return data, p
+
+
+def oracle_mobilenet(image, p):
+    x = O.conv2d(image, p["stem_w"], None, strides=(2, 2), pads=(1, 1, 1, 1))
+    x = hard_swish_oracle(O.batchnorm(x, *p["stem_bn"], eps=1e-5))
+    for b in p["blocks"]:
+        y = hard_swish_oracle(O.conv2d(x, b["exp_w"], b["exp_b"]))
+        k = b["k"]
+        y = O.unary(O.RELU, O.conv2d(y, b["dw_w"], b["dw_b"], strides=(b["stride"],) * 2, pads=(k // 2,) * 4, group=y.shape[1]))
+        s = O.global_average_pool(y)
+        s = O.unary(O.RELU, O.conv2d(s, b["se1_w"], b["se1_b"]))
+        s = O.unary(O.HARDSIGMOID, O.conv2d(s, b["se2_w"], b["se2_b"]), np.float32(1.0 / 6.0), 0.5)
+        y = O.conv2d(O.binary(O.MUL, y, s), b["proj_w"], b["proj_b"])
+        x = O.binary(O.ADD, x, y) if b["residual"] else y
+    pooled = O.global_average_pool(x).reshape(x.shape[0], -1)
+    return O.gemm(pooled, p["head_w"], p["head_b"], trans_b=True)
+
+
+def test_mobilenet_style_cnn(case, tmp_path):
+    case("MobileNetV3-style CNN from ONNX bytes")
+    data, p = make_mobilenet()
+    image = rnd(2, 3, 32, 32)
+    want = oracle_mobilenet(image, p)
+    model = Model.load_onnx_from_buffer(data)
+    (plain,) = HipSessionBuilder(model).build().run([image])
+    np.testing.assert_allclose(plain, want, rtol=2e-4, atol=2e-4)
+    # the session pipeline: hard-swish and squeeze-excite pairs become FusedElemwise nodes, same bits
+    sess = session(model, enable_profiling=True)
+    (logits,) = sess.run({"image": image})
+    assert "FusedElemwise" in sess.profile()
+    assert np.array_equal(logits.view(np.uint32), plain.view(np.uint32))
+    path = os.path.join(tmp_path, "mobilenet.onnx")
+    with open(path, "wb") as f:
+        f.write(data)
+    (again,) = InferenceSession(path).run(None, {"image": image})
+    assert np.array_equal(again, logits)
+
+
+# ---- BERT-style --------------------------------------------------------------------------------------
+B, T, H, NH, FF, VOCAB = 2, 24, 64, 4, 128, 50
+DH = H // NH
+
+
+def make_bert():
+    p = {"tok": rnd(VOCAB, H, scale=0.5), "pos": rnd(T, H, scale=0.1), "ln0": (rnd(H, shift=1.0, scale=0.1), rnd(H, scale=0.1)),
+         "wq": rnd(H, H, scale=0.1), "bq": rnd(H, scale=0.1), "wk": rnd(H, H, scale=0.1), "bk": rnd(H, scale=0.1),
+         "wv": rnd(H, H, scale=0.1), "bv": rnd(H, scale=0.1), "wo": rnd(H, H, scale=0.1), "bo": rnd(H, scale=0.1),
+         "ln1": (rnd(H, shift=1.0, scale=0.1), rnd(H, scale=0.1)), "w1": rnd(H, FF, scale=0.1), "b1": rnd(FF, scale=0.1),
+         "w2": rnd(FF, H, scale=0.1), "b2": rnd(H, scale=0.1), "ln2": (rnd(H, shift=1.0, scale=0.1), rnd(H, scale=0.1))}
+    g = G()
+    f = lambda v: g.c(np.array(v, np.float32))
+
+    def layer_norm(x, gamma, beta):
+        mean = g.op("ReduceMean", [x], axes=[-1])
+        d = g.op("Sub", [x, mean])
+        var = g.op("ReduceMean", [g.op("Pow", [d, f(2.0)])], axes=[-1])
+        return g.op("Add", [g.op("Mul", [g.op("Div", [d, g.op("Sqrt", [g.op("Add", [var, f(1e-12)])])]), g.c(gamma)]), g.c(beta)])
+
+    def linear(x, w, b):
+        return g.op("Add", [g.op("MatMul", [x, g.c(w)]), g.c(b)])
+
+    def heads(x):
+        return g.op("Transpose", [g.op("Reshape", [x, g.c(np.array([B, T, NH, DH], np.int64))])], perm=[0, 2, 1, 3])
+
+    x = g.op("Add", [g.op("Gather", [g.c(p["tok"]), "input_ids"], axis=0), g.c(p["pos"])])
+    x = layer_norm(x, *p["ln0"])
+    # (1 - mask[:, None, None, :]) * -10000, the way exporters write it
+    m = g.op("Cast", [g.op("Unsqueeze", ["attention_mask"], axes=[1, 2])], to=W.FLOAT)
+    m = g.op("Mul", [g.op("Sub", [f(1.0), m]), f(-10000.0)])
+    q, k, v = heads(linear(x, p["wq"], p["bq"])), heads(linear(x, p["wk"], p["bk"])), heads(linear(x, p["wv"], p["bv"]))
+    s = g.op("MatMul", [q, g.op("Transpose", [k], perm=[0, 1, 3, 2])])
+    s = g.op("Softmax", [g.op("Add", [g.op("Div", [s, f(np.sqrt(DH))]), m])], axis=-1)
+    a = g.op("Reshape", [g.op("Transpose", [g.op("MatMul", [s, v])], perm=[0, 2, 1, 3]), g.c(np.array([B, T, H], np.int64))])
+    x = layer_norm(g.op("Add", [x, linear(a, p["wo"], p["bo"])]), *p["ln1"])
+    h = linear(x, p["w1"], p["b1"])
+    h = g.op("Mul", [g.op("Mul", [h, g.op("Add", [g.op("Erf", [g.op("Div", [h, f(1.4142135)])]), f(1.0)])]), f(0.5)])
+    x = layer_norm(g.op("Add", [x, linear(h, p["w2"], p["b2"])]), *p["ln2"])
+    g.nodes.append(W.node("Identity", [x], ["hidden"]))
+    data = W.model(W.graph(g.nodes, g.inits, [W.value_info("input_ids", W.INT64, [B, T]), W.value_info("attention_mask", W.INT64, [B, T])],
+                           [W.value_info("hidden", W.FLOAT, [B, T, H])]), opsets=(("", 11),))
+    return data, p
+
+
+def oracle_bert(ids, mask, p):
+    s = lambda v: np.array(v, np.float32)
+    ln = lambda x, gb: O.layer_norm(x, gb[0], gb[1], 1e-12)
+    lin = lambda x, w, b: O.binary(O.ADD, O.matmul(x, w), b)
+    heads = lambda x: O.transpose(x.reshape(B, T, NH, DH), (0, 2, 1, 3))
+    x = ln(O.binary(O.ADD, p["tok"][ids], p["pos"]), p["ln0"])
+    m = O.binary(O.MUL, O.binary(O.SUB, s(1.0), mask[:, None, None, :].astype(np.float32)), s(-10000.0))
+    q, k, v = heads(lin(x, p["wq"], p["bq"])), heads(lin(x, p["wk"], p["bk"])), heads(lin(x, p["wv"], p["bv"]))
+    sc = O.binary(O.ADD, O.binary(O.DIV, O.matmul(q, O.transpose(k, (0, 1, 3, 2))), s(np.sqrt(DH))), m)
+    a = O.transpose(O.matmul(O.softmax(sc), v), (0, 2, 1, 3)).reshape(B, T, H)
+    x = ln(O.binary(O.ADD, x, lin(a, p["wo"], p["bo"])), p["ln1"])
+    h = lin(x, p["w1"], p["b1"])
+    x = ln(O.binary(O.ADD, x, lin(O.unary(O.GELU, h), p["w2"], p["b2"])), p["ln2"])
+    return x
+
+
+def test_bert_style_encoder_layer(case):
+    case("BERT-style encoder layer from ONNX bytes")
+    data, p = make_bert()
+    ids = RNG.integers(0, VOCAB, size=(B, T)).astype(np.int64)
+    mask = np.ones((B, T), np.int64)
+    mask[0, 17:] = 0
+    mask[1, 9:] = 0
+    model = Model.load_onnx_from_buffer(data)
+    sess = session(model, enable_profiling=True)
+    (hidden,) = sess.run({"input_ids": ids, "attention_mask": mask})
+    np.testing.assert_allclose(hidden, oracle_bert(ids, mask, p), rtol=3e-4, atol=3e-4)
+    ops = set(sess.profile())
+    assert {"LayerNormalization", "FusedElemwise", "Softmax", "Gather", "MatMul"} <= ops
+    # the scale and the mask went into the Softmax, the erf chain became Gelu, and Gelu joined its bias Add
+    assert not ops & {"Div", "Erf", "Gelu", "Pow", "Sqrt"}
