@@ -13,7 +13,7 @@
 // round trip through memory between the steps.
 //
 // Two executors share the program format.  Chains that models actually contain (the exporter's
-// erf-GELU, the tail of its LayerNorm, scale-and-shift, bias + activation, x * sigmoid(x)) are also
+// erf-GELU, the tail of its LayerNorm, scale-and-shift, bias + activation or residual, x * sigmoid(x)) are also
 // instantiated at compile time: the host compares the program with each instantiated signature and,
 // on a match, launches straight-line code that runs at the speed of a copy.  Everything else goes to
 // the interpreting kernel, whose per-step dispatch costs scalar-unit time.
@@ -220,6 +220,10 @@ using NormaliseScaleShiftChain = Chain<3, 4, S<C_DIV, 0, 3>, S<C_MUL, ACC, 1>, S
 using MulAddChain = Chain<3, 3, S<C_MUL, 0, 1>, S<C_ADD, ACC, 2>>;
 // x + b -> Relu (bias or residual, then the activation)
 using AddReluChain = Chain<2, 2, S<C_ADD, 0, 1>, S<C_RELU, ACC>>;
+// x + b -> Gelu (a linear layer's bias, then the fused activation)
+using AddGeluChain = Chain<2, 2, S<C_ADD, 0, 1>, S<C_GELU, ACC>>;
+// x + b + r (bias, then the residual)
+using AddAddChain = Chain<3, 3, S<C_ADD, 0, 1>, S<C_ADD, ACC, 2>>;
 // x * Sigmoid(x)
 using SiluChain = Chain<1, 1, S<C_SIGMOID, 0>, S<C_MUL, ACC, 0>>;
 // x * HardSigmoid(x)  (hard swish)
@@ -447,7 +451,8 @@ int launch_fused_elemwise(DeviceCtx &ctx, float *out, int rank, const int64_t *o
         const bool fixed = ctx.fused_static_chains &&
                            (try_static<ErfGeluChain>(s, grid, nt, out, prog) || try_static<LayerNormTailChain>(s, grid, nt, out, prog) ||
                             try_static<NormaliseScaleShiftChain>(s, grid, nt, out, prog) || try_static<MulAddChain>(s, grid, nt, out, prog) ||
-                            try_static<AddReluChain>(s, grid, nt, out, prog) || try_static<SiluChain>(s, grid, nt, out, prog) ||
+                            try_static<AddReluChain>(s, grid, nt, out, prog) || try_static<AddGeluChain>(s, grid, nt, out, prog) ||
+                            try_static<AddAddChain>(s, grid, nt, out, prog) || try_static<SiluChain>(s, grid, nt, out, prog) ||
                             try_static<HardSwishChain>(s, grid, nt, out, prog));
         if (!fixed) launch_vec4<AnyChain>(s, grid, nt, out, prog);
     } else {

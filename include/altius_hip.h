@@ -177,7 +177,7 @@ int ahip_fused_elemwise(ahip_ctx *ctx, float *out, int rank, const int64_t *out_
                         const float *const *inputs, const int64_t *const *input_strides, int n_steps,
                         const ahip_fused_step *steps);
 /* ahip_fused_elemwise runs a chain through a kernel compiled for exactly that chain when the library
- * has one (the exporter's erf-GELU, the LayerNorm tail, scale-and-shift, bias + Relu, x * Sigmoid(x),
+ * has one (the exporter's erf-GELU, the LayerNorm tail, scale-and-shift, bias + Relu or Gelu or residual, x * Sigmoid(x),
  * x * HardSigmoid(x)) and through a kernel that interprets the steps otherwise; both give the same bits.
  * enable = 0 sends every chain of this context to the interpreting kernel (default 1). */
 int ahip_fused_use_compiled_chains(ahip_ctx *ctx, int enable);

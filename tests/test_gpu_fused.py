@@ -131,6 +131,8 @@ def test_compiled_chains_equal_the_interpreter(case, ctx):
         "normalise, scale, shift": ([x, var, g, b], [("b", D.DIV, 0, 1), ("b", D.MUL, ACC, 2), ("b", D.ADD, 3, ACC)]),
         "mul add": ([x, g, y], [("b", D.MUL, 0, 1), ("b", D.ADD, ACC, 2)]),
         "add relu": ([x, b], [("b", D.ADD, 0, 1), ("u", D.RELU, ACC, 0)]),
+        "add gelu": ([x, b], [("b", D.ADD, 0, 1), ("u", D.GELU, ACC, 0)]),
+        "add add": ([x, b, y], [("b", D.ADD, 0, 1), ("b", D.ADD, 2, ACC)]),
         "silu": ([x], [("u", D.SIGMOID, 0, 0), ("b", D.MUL, 0, ACC)]),
         "hard swish": ([x], [("u", D.HARDSIGMOID, 0, 0, 1 / 6, 0.5), ("b", D.MUL, ACC, 0)]),
     }
