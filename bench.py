@@ -408,8 +408,9 @@ def main():
     args = ap.parse_args()
 
     if args.gpus != 1:
-        log("bench.py: this build runs on one GPU only (the path shards without communication; "
-            "see DESIGN.md); run with --gpus 1")
+        log("bench.py: this build runs on one GPU only (every operator on the path is independent along the batch "
+            "axis, so more GPUs would each run the same kernels on a slice of the batch, without communication); "
+            "run with --gpus 1")
         sys.exit(2)
 
     ensure_built()
