@@ -394,3 +394,39 @@ def test_softmax_with_absorbed_scale_and_mask(case, shape, mask_shape, scale_kin
     if mask_shape is not None:
         z = O.binary(O.ADD, z, inputs[1])
     assert_close(got, O.softmax(z), what="vs oracle chain")
+
+
+def test_run_from_several_threads(case):
+    """InterpreterSession::run takes &self and may be called from several threads at once (per-thread value maps,
+    session.rs:52-58).  Here concurrent calls on one session are serialised internally, and sessions of different
+    threads run side by side on their own streams; every call must return its own inputs' result."""
+    import threading
+
+    case("session: concurrent run() calls")
+    c = synth.cfg2(batch=1)
+    m = Model()
+    x = m.new_val_named_and_shaped("x", c["x"].shape)
+    out, _, _ = layer_norm_chain(m, x, c["gamma"], c["beta"], eps=float(c["eps"]))
+    m.add_input(x)
+    m.add_output(out)
+    shared = HipSessionBuilder(m).build()
+    inputs = [synth.normal(300 + i, c["x"].shape, std=1.0 + i) for i in range(4)]
+    want = [oracle_ln_chain(v, c["gamma"], c["beta"], c["eps"]) for v in inputs]
+    errors = []
+
+    def worker(i, own_session):
+        try:
+            sess = HipSessionBuilder(m.clone()).build() if own_session else shared
+            for _ in range(8):
+                (got,) = sess.run([inputs[i]])
+                assert_close(got, want[i], what=f"thread {i}")
+        except Exception as e:  # noqa: BLE001 - reported below, in the main thread
+            errors.append((i, repr(e)))
+
+    for own in (False, True):
+        threads = [threading.Thread(target=worker, args=(i, own)) for i in range(4)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+    assert not errors, errors
