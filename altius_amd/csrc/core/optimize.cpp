@@ -473,4 +473,41 @@ size_t fuse_softmax_prologue(Model &model) {
     return count;
 }
 
+size_t fuse_matmul_bias(Model &model) {
+    const auto users = model.get_value_users();
+    std::map<ValueId, TypedFixedShape> shapes;
+    ShapeError serr;
+    if (!infer_shapes(model, nullptr, &shapes, &serr)) return 0;
+    const auto &outs = model.graph.outputs;
+    size_t count = 0;
+    std::vector<NodeId> doomed;
+    for (NodeId mid : model.topo_sort_nodes()) {
+        Node &mm = model.graph.nodes[mid];
+        if (mm.op.kind != OpKind::MatMul || mm.inputs.size() != 2 || mm.outputs.size() != 1) continue;
+        const ValueId prod = mm.outputs[0];
+        auto u = users.find(prod);
+        if (u == users.end() || u->second.size() != 1 || std::find(outs.begin(), outs.end(), prod) != outs.end()) continue;
+        const NodeId aid = *u->second.begin();
+        const Node &add = model.graph.nodes[aid];
+        if (add.op.kind != OpKind::Add || add.inputs.size() != 2 || add.outputs.size() != 1 || add.inputs[0] == add.inputs[1]) continue;
+        const ValueId bias = add.inputs[0] == prod ? add.inputs[1] : add.inputs[0];
+        auto ps = shapes.find(prod), bs = shapes.find(bias), os = shapes.find(add.outputs[0]);
+        if (ps == shapes.end() || bs == shapes.end() || os == shapes.end()) continue;
+        if (ps->second.elem_ty != TensorElemType::F32 || bs->second.elem_ty != TensorElemType::F32) continue;
+        const FixedDimensions &pd = ps->second.dims, &bd = bs->second.dims;
+        if (pd.len() < 2 || os->second.dims != pd || bd.len() == 0 || bd.len() > pd.len()) continue;
+        // one value per column: the last extent equals N, every other extent is 1
+        bool row_vector = bd[bd.len() - 1] == pd[pd.len() - 1];
+        for (size_t i = 0; i + 1 < bd.len(); i++) row_vector = row_vector && bd[i] == 1;
+        if (!row_vector) continue;
+        mm.inputs.push_back(bias);
+        mm.outputs[0] = add.outputs[0];
+        doomed.push_back(aid);
+        count++;
+    }
+    for (NodeId id : doomed) model.graph.nodes[id].deleted = true;
+    if (count) model.remove_unnecessary_nodes();
+    return count;
+}
+
 }  // namespace altius

@@ -52,6 +52,12 @@ size_t eliminate_identity(Model &model);
 // the last ([N,1,1,C], [1,1,1,C], [C]).  Returns the number of Softmax nodes rewritten.
 size_t fuse_softmax_prologue(Model &model);
 
+// Not in the reference.  MatMul(x, W) -> Add(., b) with b one value per output column (shape [N], [1, N], ...),
+// the product having no other reader: the MatMul node takes b as a third input and the session adds it in the
+// product's epilogue -- the same single addition per element, without the extra pass over the output.
+// Returns the number of MatMul nodes rewritten.
+size_t fuse_matmul_bias(Model &model);
+
 enum class ElemwiseFusionRule { ReferenceRule = 0, ExtendedRule = 1 };
 bool fuse_elemwise_ops(Model &model, ElemwiseFusionRule rule, size_t *count, std::string *err);
 

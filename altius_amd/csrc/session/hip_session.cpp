@@ -1207,12 +1207,21 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
         for (size_t i = 0; i + 2 < a.len(); i++) a_batch *= a[i];
         for (size_t i = 0; i + 2 < b.len(); i++) b_batch *= b[i];
         for (size_t i = 0; i + 2 < out.dims.len(); i++) batch *= out.dims[i];
+        // A third input is a bias row absorbed by fuse_matmul_bias: added in the epilogue (1 * acc + 1 * bias,
+        // the one addition the separate Add performs).
+        const float *bias = nullptr;
+        if (in.size() > 2 && in[2]) {
+            if (in[2]->elem_ty != TensorElemType::F32 || in[2]->dims.total_elems() != n)
+                return fail(err, SessionError::Shape, "MatMul: the absorbed bias must hold one f32 value per output column");
+            bias = f(in[2]);
+        }
+        const float beta = bias ? 1.0f : 0.0f;
         if (b_batch == 1 && a_batch == batch) {
             // [.., m, k] x [k, n]: one tall sgemm, as the reference does (session.rs:653-660)
-            rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), nullptr, 1, batch * m, n, k, 0, 0, k, n, n, 0, 0, 0, 0, 0, 1.0f, 0.0f);
+            rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), bias, 1, batch * m, n, k, 0, 0, k, n, n, 0, 0, 0, 0, 1, 1.0f, beta);
         } else if ((a_batch == batch || a_batch == 1) && (b_batch == batch || b_batch == 1)) {
-            rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), nullptr, batch, m, n, k, 0, 0, k, n, n, a_batch == 1 ? 0 : m * k,
-                             b_batch == 1 ? 0 : k * n, m * n, 0, 0, 1.0f, 0.0f);
+            rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), bias, batch, m, n, k, 0, 0, k, n, n, a_batch == 1 ? 0 : m * k,
+                             b_batch == 1 ? 0 : k * n, m * n, 0, 1, 1.0f, beta);
         } else {
             return fail(err, SessionError::Message, "MatMul: batch axes that broadcast against each other partially are not supported");
         }

@@ -386,6 +386,10 @@ class Model:
     def eliminate_identity(self):
         return self._pass(self.L.ahip_eliminate_identity)
 
+    def fuse_matmul_bias(self):
+        """MatMul -> Add(bias row) becomes a MatMul node with the bias as third input."""
+        return self._pass(self.L.ahip_fuse_matmul_bias)
+
     def fuse_softmax_prologue(self):
         """[Mul | Div by a constant] -> [Add mask] -> Softmax becomes one Softmax node with inputs (x, scale?, mask?)."""
         return self._pass(self.L.ahip_fuse_softmax_prologue)

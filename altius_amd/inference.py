@@ -42,7 +42,7 @@ class _NamedSession:
 def session(model, enable_profiling=False, intra_op_num_threads=1, backend="hip", device=0):
     """altius_py.session (lib.rs:44-88): the same rewrite pipeline -- fuse_layer_norm, fuse_gelu, fuse_fast_gelu,
     element-wise fusion for the backend that has a kernel for it (the reference: "cpu"; here: "hip", with the wider
-    rule, after the scale and mask in front of each Softmax have been folded into it), eliminate_identity -- then the session builder.  The model object is left untouched, as in the
+    rule, after the scale and mask in front of each Softmax and the bias row behind each MatMul have been folded into them), eliminate_identity -- then the session builder.  The model object is left untouched, as in the
     reference (it takes a clone)."""
     if backend != "hip":
         raise RuntimeError(f"Unknown backend: {backend}")
@@ -51,6 +51,7 @@ def session(model, enable_profiling=False, intra_op_num_threads=1, backend="hip"
     m.fuse_gelu()
     m.fuse_fast_gelu()
     m.fuse_softmax_prologue()
+    m.fuse_matmul_bias()
     m.fuse_elemwise_ops(extended=True)
     m.eliminate_identity()
     builder = HipSessionBuilder(m).with_profiling_enabled(enable_profiling).with_intra_op_num_threads(intra_op_num_threads)

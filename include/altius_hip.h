@@ -431,6 +431,10 @@ int ahip_eliminate_identity(ahip_model *model, int *count);
  * Readable afterwards as the integer attributes "prologue_scale" (0 none, 1 multiply, 2 divide) and
  * "prologue_mask" of the Softmax node. */
 int ahip_fuse_softmax_prologue(ahip_model *model, int *count);
+/* Not in the reference: MatMul(x, W) -> Add(., b), b holding one value per output column and the product having
+ * no other reader, becomes a MatMul node with b as third input; the session adds it in the product's epilogue
+ * (the same single addition per element, without the extra pass over the output). */
+int ahip_fuse_matmul_bias(ahip_model *model, int *count);
 enum ahip_fuse_rule { AHIP_FUSE_REFERENCE_RULE = 0, AHIP_FUSE_EXTENDED_RULE = 1 };
 int ahip_fuse_elemwise_ops(ahip_model *model, int rule, int *count);
 

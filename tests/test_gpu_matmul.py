@@ -152,3 +152,31 @@ def test_gemm_head_through_the_session(case):
     (got,) = HipSessionBuilder(m).build().run([x])
     assert np.allclose(got, O.gemm(x, w, b, trans_b=True), rtol=1e-5, atol=1e-4)
     check_bound(got - b, x, w.T, "gemm head")
+
+
+@pytest.mark.parametrize("x_shape,w_shape", [([5, 10], [10, 15]), ([3, 197, 64], [64, 192]), ([2, 3, 50, 32], [2, 3, 32, 70]),
+                                             ([4, 300, 256], [256, 130])])
+def test_matmul_with_absorbed_bias_has_the_bits_of_matmul_then_add(case, x_shape, w_shape):
+    """fuse_matmul_bias: the bias row goes into the product's epilogue as acc + bias, the one addition the
+    separate Add node performs."""
+    from altius_amd.graph import Model, Op
+    from altius_amd.session import HipSessionBuilder
+
+    case(f"matmul + bias {x_shape} x {w_shape}")
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(x_shape).astype(np.float32)
+    w = (rng.standard_normal(w_shape) * 0.1).astype(np.float32)
+    b = rng.standard_normal(w_shape[-1]).astype(np.float32)
+    m = Model()
+    vx = m.new_val_named_and_shaped("x", x_shape)
+    p, y = m.new_val(), m.new_val()
+    m.add_node(Op.MatMul, [vx, m.new_initializer(w)], [p])
+    m.add_node(Op.Add, [p, m.new_initializer(b)], [y])
+    m.add_input(vx)
+    m.add_output(y)
+    fused = m.clone()
+    assert fused.fuse_matmul_bias() == 1 and len(fused.nodes()) == 1
+    (want,) = HipSessionBuilder(m).build().run([x])
+    (got,) = HipSessionBuilder(fused).build().run([x])
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    np.testing.assert_allclose(got, np.matmul(x.astype(np.float64), w.astype(np.float64)) + b, rtol=1e-4, atol=1e-4)

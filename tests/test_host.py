@@ -517,3 +517,34 @@ def test_fuse_softmax_prologue():
     m, x, c, mask = _attention_tail([2, 4, 9, 9], None, scale_kind="Mul")
     m.add_output(m.nodes()[0]["outputs"][0])
     assert m.fuse_softmax_prologue() == 0
+
+
+def test_fuse_matmul_bias():
+    def build(x_shape, w_shape, b_shape, bias_first=False, extra_reader=False):
+        m = Model()
+        x = m.new_val_named_and_shaped("x", x_shape)
+        w = m.new_initializer(np.zeros(w_shape, np.float32))
+        b = m.new_initializer(np.zeros(b_shape, np.float32))
+        p, y = m.new_val(), m.new_val_named("y")
+        m.add_node(Op.MatMul, [x, w], [p])
+        m.add_node(Op.Add, [b, p] if bias_first else [p, b], [y])
+        m.add_input(x)
+        m.add_output(y)
+        if extra_reader:
+            z = m.new_val()
+            m.add_node(Op.ReLU, [p], [z])
+            m.add_output(z)
+        return m, x, w, b, y
+
+    for x_shape, w_shape, b_shape, first in (([5, 10], [10, 15], [15], False), ([3, 5, 10], [10, 15], [1, 15], True),
+                                             ([2, 3, 5, 10], [2, 3, 10, 15], [1, 1, 1, 15], False)):
+        m, x, w, b, y = build(x_shape, w_shape, b_shape, first)
+        assert m.fuse_matmul_bias() == 1
+        (mm,) = m.nodes()
+        assert mm["op_name"] == "MatMul" and mm["inputs"] == [x, w, b] and mm["outputs"] == [y] == m.outputs
+        assert m.infer_value_shape(y)[0] == x_shape[:-1] + [15]
+        assert m.fuse_matmul_bias() == 0
+    # left alone: a bias that is not one value per column, a product with a second reader
+    assert build([5, 10], [10, 15], [5, 1])[0].fuse_matmul_bias() == 0
+    assert build([5, 10], [10, 15], [5, 15])[0].fuse_matmul_bias() == 0
+    assert build([5, 10], [10, 15], [15], extra_reader=True)[0].fuse_matmul_bias() == 0
