@@ -13,6 +13,8 @@
 // one barrier per K tile.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "common.h"
 #include "ctx.h"
 
@@ -44,7 +46,9 @@ struct GemmArgs {
 // Loads this thread's share of a BK x 128 operand tile into registers.
 // K_CONTIG: the operand's k axis is the contiguous one (A without transA, B with transB).
 // `mn` is the tile's first row (A) or column (B), `lim` the extent of that axis.
-template <bool K_CONTIG, int WIDTH>
+// INSIDE: the whole tile lies inside the operand and 16-byte loads are legal (decided per block and
+// K tile, a scalar branch): no per-lane bounds checks.
+template <bool K_CONTIG, int WIDTH, bool INSIDE>
 __device__ __forceinline__ void load_tile(float4 (&r)[WIDTH / 64], const float *__restrict__ p, uint32_t mn0, uint32_t lim,
                                           uint32_t k0, uint32_t kdim, uint32_t s_mn, uint32_t s_k, int vec, int tid) {
 #pragma unroll
@@ -57,6 +61,10 @@ __device__ __forceinline__ void load_tile(float4 (&r)[WIDTH / 64], const float *
         } else {  // 16 rows of WIDTH floats: WIDTH / 4 float4 per row
             kk = k0 + f / (WIDTH / 4);
             mn = mn0 + ((f % (WIDTH / 4)) << 2);
+        }
+        if (INSIDE) {
+            r[u] = *reinterpret_cast<const float4 *>(K_CONTIG ? p + (size_t)mn * s_mn + kk : p + (size_t)kk * s_k + mn);
+            continue;
         }
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
         if (K_CONTIG) {
@@ -130,42 +138,56 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_mfma(GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    float4 ra[BM / 64], rb[TN / 64];
-    load_tile<A_KC, BM>(ra, a, m0, g.m, 0, g.k, a_smn, a_sk, g.a_vec, tid);
-    load_tile<B_KC, TN>(rb, b, n0, g.n, 0, g.k, b_smn, b_sk, g.b_vec, tid);
-    store_tile<A_KC, BM>(As[0], ra, tid);
-    store_tile<B_KC, TN>(Bs[0], rb, tid);
-    __syncthreads();
-
-    const uint32_t nk = (g.k + BK - 1) / BK;
+    // Blocks whose tiles lie inside both operands run a loop without any bounds check on all K tiles
+    // but a ragged last one; the choice is made once per block (a scalar branch around the whole loop),
+    // so the interior loop is straight-line code between its barriers.
+    const bool inside = g.a_vec && g.b_vec && m0 + BM <= g.m && n0 + TN <= g.n;
     const int lr = lane & 31, lk = lane >> 5;
-    for (uint32_t kt = 0; kt < nk; kt++) {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < nk;
-        if (more) {
-            load_tile<A_KC, BM>(ra, a, m0, g.m, (kt + 1) * BK, g.k, a_smn, a_sk, g.a_vec, tid);
-            load_tile<B_KC, TN>(rb, b, n0, g.n, (kt + 1) * BK, g.k, b_smn, b_sk, g.b_vec, tid);
-        }
-        const float *at = As[cur] + wm * (32 * WI) + lr;
-        const float *bt = Bs[cur] + wn * 64 + lr;
-#pragma unroll
-        for (int kk = 0; kk < BK; kk += 2) {
-            float av[WI];
-#pragma unroll
-            for (int i = 0; i < WI; i++) av[i] = at[(kk + lk) * PITCH + 32 * i];
-            const float b0 = bt[(kk + lk) * PITCH], b1 = bt[(kk + lk) * PITCH + 32];
-#pragma unroll
-            for (int i = 0; i < WI; i++) {
-                acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], b0, acc[i][0], 0, 0, 0);
-                acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], b1, acc[i][1], 0, 0, 0);
+    auto main_loop = [&](auto inside_tag) {
+        constexpr bool INSIDE = decltype(inside_tag)::value;
+        float4 ra[BM / 64], rb[TN / 64];
+        auto load = [&](uint32_t k0) {
+            if (INSIDE && k0 + BK <= g.k) {
+                load_tile<A_KC, BM, true>(ra, a, m0, g.m, k0, g.k, a_smn, a_sk, 1, tid);
+                load_tile<B_KC, TN, true>(rb, b, n0, g.n, k0, g.k, b_smn, b_sk, 1, tid);
+            } else {
+                load_tile<A_KC, BM, false>(ra, a, m0, g.m, k0, g.k, a_smn, a_sk, g.a_vec, tid);
+                load_tile<B_KC, TN, false>(rb, b, n0, g.n, k0, g.k, b_smn, b_sk, g.b_vec, tid);
             }
-        }
-        if (more) {
-            store_tile<A_KC, BM>(As[cur ^ 1], ra, tid);
-            store_tile<B_KC, TN>(Bs[cur ^ 1], rb, tid);
-        }
+        };
+        load(0);
+        store_tile<A_KC, BM>(As[0], ra, tid);
+        store_tile<B_KC, TN>(Bs[0], rb, tid);
         __syncthreads();
-    }
+
+        const uint32_t nk = (g.k + BK - 1) / BK;
+        for (uint32_t kt = 0; kt < nk; kt++) {
+            const int cur = kt & 1;
+            const bool more = kt + 1 < nk;
+            if (more) load((kt + 1) * BK);
+            const float *at = As[cur] + wm * (32 * WI) + lr;
+            const float *bt = Bs[cur] + wn * 64 + lr;
+#pragma unroll
+            for (int kk = 0; kk < BK; kk += 2) {
+                float av[WI];
+#pragma unroll
+                for (int i = 0; i < WI; i++) av[i] = at[(kk + lk) * PITCH + 32 * i];
+                const float b0 = bt[(kk + lk) * PITCH], b1 = bt[(kk + lk) * PITCH + 32];
+#pragma unroll
+                for (int i = 0; i < WI; i++) {
+                    acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], b0, acc[i][0], 0, 0, 0);
+                    acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], b1, acc[i][1], 0, 0, 0);
+                }
+            }
+            if (more) {
+                store_tile<A_KC, BM>(As[cur ^ 1], ra, tid);
+                store_tile<B_KC, TN>(Bs[cur ^ 1], rb, tid);
+            }
+            __syncthreads();
+        }
+    };
+    if (inside) main_loop(std::true_type{});
+    else main_loop(std::false_type{});
 
     // Accumulator r of lane l is C[8 * (r / 4) + 4 * (l / 32) + r % 4][l % 32] of its 32 x 32 tile.
     float *c = g.c + (size_t)blockIdx.z * g.c_bs;

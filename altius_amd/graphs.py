@@ -57,3 +57,44 @@ def single_input_model(shape, body):
     m.add_input(x)
     m.add_output(out)
     return m
+
+
+def vit_encoder(batch, layers=12, hidden=768, heads=12, mlp=3072, tokens=197, classes=1000, seed=0):
+    """A ViT-B/16-shaped encoder stack the way exporters write it (9-node LayerNorm chains, MatMul + Add, head
+    split by Reshape / Transpose, QK^T, Mul by 1/sqrt(d), Softmax, 5-node erf-GELU chains), a final LayerNorm,
+    the class token and a Gemm head, with random weights.  Input: embedded tokens [batch, tokens, hidden]."""
+    rng = np.random.default_rng(seed)
+    w = lambda *shape, scale=0.02: (rng.standard_normal(shape) * scale).astype(np.float32)
+    m = Model(opset_version=13)
+    x = m.new_val_named_and_shaped("tokens", [batch, tokens, hidden])
+    m.add_input(x)
+    d = hidden // heads
+    i64 = lambda *v: m.new_initializer(np.array(v, np.int64))
+
+    def node(op, inputs, **attrs):
+        out = m.new_val()
+        m.add_node(op, inputs, [out], **attrs)
+        return out
+
+    def linear(v, n_in, n_out):
+        return node(Op.Add, [node(Op.MatMul, [v, m.new_initializer(w(n_in, n_out))]), m.new_initializer(w(n_out))])
+
+    def norm(v):
+        return layer_norm_chain(m, v, 1 + w(hidden), w(hidden), eps=1e-6)[0]
+
+    cur = x
+    for _ in range(layers):
+        qkv = linear(norm(cur), hidden, 3 * hidden)
+        parts = [m.new_val() for _ in range(3)]
+        m.add_node(Op.Split, [qkv, i64(hidden, hidden, hidden)], parts, axis=2)
+        q, k, v = (node(Op.Transpose, [node(Op.Reshape, [p, i64(batch, tokens, heads, d)])], perm=[0, 2, 1, 3]) for p in parts)
+        s = node(Op.MatMul, [q, node(Op.Transpose, [k], perm=[0, 1, 3, 2])])
+        s = node(Op.Softmax, [node(Op.Mul, [s, m.new_initializer(np.array(d ** -0.5, np.float32))])], axis=-1)
+        a = node(Op.Reshape, [node(Op.Transpose, [node(Op.MatMul, [s, v])], perm=[0, 2, 1, 3]), i64(batch, tokens, hidden)])
+        cur = node(Op.Add, [cur, linear(a, hidden, hidden)])
+        h = erf_gelu_chain(m, linear(norm(cur), hidden, mlp))
+        cur = node(Op.Add, [cur, linear(h, mlp, hidden)])
+    cls = node(Op.Gather, [norm(cur), m.new_initializer(np.array(0, np.int64))], axis=1)
+    logits = node(Op.Gemm, [cls, m.new_initializer(w(classes, hidden)), m.new_initializer(w(classes))], trans_b=True)
+    m.add_output(logits)
+    return m

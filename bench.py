@@ -264,6 +264,42 @@ def session_table(synth, dev_ctx):
     return rows
 
 
+def vit_table(batch, layers=12):
+    """Whole-model device time (kernels only, input already uploaded by run()) of a ViT-B/16-shaped encoder for
+    three versions of the same graph, with the per-operator split of each from a profiled run."""
+    from altius_amd import graphs
+    from altius_amd.graph import Tensor
+    from altius_amd.session import HipSessionBuilder
+
+    base = graphs.vit_encoder(batch, layers=layers)
+    x = Tensor.from_numpy(np.random.default_rng(1).standard_normal((batch, 197, 768)).astype(np.float32))
+    versions = []
+    versions.append(("as exported", base))
+    ref = base.clone()
+    ref.fuse_layer_norm(), ref.fuse_gelu(), ref.fuse_fast_gelu(), ref.eliminate_identity()
+    versions.append(("reference rewrites (fuse_layer_norm, fuse_gelu)", ref))
+    ours = ref.clone()
+    ours.fuse_softmax_prologue(), ours.fuse_matmul_bias(), ours.fuse_elemwise_ops(extended=True)
+    versions.append(("+ softmax prologue, matmul bias, element-wise chains", ours))
+    rows = []
+    for name, model in versions:
+        sess = HipSessionBuilder(model).build()
+        best = float("inf")
+        for _ in range(4):
+            outs = sess.run([x], copy=False)
+            best = min(best, sess.last_device_ms())
+            del outs
+        sess.close()
+        prof = HipSessionBuilder(model).with_profiling_enabled(True).build()
+        for _ in range(2):
+            outs = prof.run([x], copy=False)
+            del outs
+        split = {k: round(v, 3) for k, v in sorted(prof.profile().items(), key=lambda kv: -kv[1])}
+        prof.close()
+        rows.append({"graph": name, "nodes": len(model.nodes()), "device_ms": round(best, 3), "per_op_ms": split})
+    return rows
+
+
 def build_next_rows(ctx, D, batch=256):
     """The operators either side of the hot path (data movement, MatMul) at ViT-B/16 shapes for the given
     batch: (name, bytes, flops, launcher).  Device buffers are left uninitialised where contents do not matter."""
@@ -405,6 +441,9 @@ def main():
                     help="also time the kernels and graphs of configs[0..3] (table on stderr, 'other_configs' in the JSON)")
     ap.add_argument("--next-rows", action="store_true",
                     help="also time the data-movement and MatMul kernels at ViT-B/16 shapes ('next_rows' in the JSON)")
+    ap.add_argument("--vit", type=int, default=0, metavar="BATCH",
+                    help="also run a ViT-B/16-shaped encoder (12 layers, exporter-style graph, random weights) at this batch: "
+                         "device time per forward as exported, after the reference's rewrites, and after this backend's ('vit' in the JSON)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -499,6 +538,13 @@ def main():
                 % (r["graph"], r["kernels_us"], r["kernels_us_graph_replay"], r["kernels_GBps"], r["run_device_us"],
                    r["run_ms_with_pcie"]))
         result["other_configs"] = {"kernels": others, "graphs": graphs_rows}
+
+    if args.vit:
+        vit_rows = vit_table(args.vit)
+        for r in vit_rows:
+            top = ", ".join("%s %.2f" % kv for kv in list(r["per_op_ms"].items())[:8])
+            log("ViT-B/16 encoder, batch %d, %-58s %4d nodes %9.3f ms   (%s)" % (args.vit, r["graph"], r["nodes"], r["device_ms"], top))
+        result["vit"] = {"batch": args.vit, "layers": 12, "rows": vit_rows}
 
     if args.next_rows:
         MFMA_F32_PEAK = 157.3  # TFLOP/s, dense fp32 matrix cores
