@@ -48,10 +48,11 @@ def ensure_built():
 class Op:
     """One kernel launch on fixed device buffers, with its algorithmic byte count."""
 
-    def __init__(self, name, nbytes, launchers):
+    def __init__(self, name, nbytes, launchers, cpu=None):
         self.name = name
         self.nbytes = nbytes
         self.launchers = launchers  # one closure per rotated buffer set
+        self.cpu = cpu              # cpu(threads): the same operator on the CPU oracle (test infrastructure, timed beside)
         self.i = 0
 
     def launch(self):
@@ -118,7 +119,10 @@ def build_cfg4(ctx, D, synth, batch, rotate_bytes):
 
 def build_other_configs(ctx, D, synth, rotate_bytes=600e6, max_sets=48):
     """Kernels of configs[0..3] at their BASELINE.json shapes (parity-test shapes, reported as a table
-    only).  Buffers are rotated over enough copies that repeated launches miss the 256 MB cache."""
+    only).  Buffers are rotated over enough copies that repeated launches miss the 256 MB cache.  Each
+    operator also carries the same call on the CPU oracle, timed beside it by the caller."""
+    import oracle as O
+
     ops = []
 
     def sets(nbytes):
@@ -135,21 +139,22 @@ def build_other_configs(ctx, D, synth, rotate_bytes=600e6, max_sets=48):
         dbs = [db] * k if db else [ctx.upload(b) for _ in range(k)]
         do = [ctx.alloc(4 * n) for _ in range(k)]
         ops.append(Op(name, nbytes, [(lambda i=i: ctx.binary_raw(op, do[i].ptr, da[i].ptr, dbs[i].ptr, out_dims, a_str, b_str))
-                                     for i in range(k)]))
+                                     for i in range(k)], cpu=lambda threads: O.binary(op, a, b, threads=threads)))
 
     def unary(name, op, x, alpha=0.0, beta=0.0):
         k = sets(2 * x.nbytes)
         dx = [ctx.upload(x) for _ in range(k)]
         do = [ctx.alloc(x.nbytes) for _ in range(k)]
         ops.append(Op(name, 2 * x.nbytes, [(lambda i=i: ctx.unary_raw(op, do[i].ptr, dx[i].ptr, x.size, alpha, beta))
-                                           for i in range(k)]))
+                                           for i in range(k)], cpu=lambda threads: O.unary(op, x, alpha, beta, threads=threads)))
 
     def softmax(name, x):
         k = sets(2 * x.nbytes)
         dx = [ctx.upload(x) for _ in range(k)]
         do = [ctx.alloc(x.nbytes) for _ in range(k)]
         rows, length = x.size // x.shape[-1], x.shape[-1]
-        ops.append(Op(name, 2 * x.nbytes, [(lambda i=i: ctx.softmax_raw(do[i].ptr, dx[i].ptr, rows, length)) for i in range(k)]))
+        ops.append(Op(name, 2 * x.nbytes, [(lambda i=i: ctx.softmax_raw(do[i].ptr, dx[i].ptr, rows, length)) for i in range(k)],
+                      cpu=lambda threads: O.softmax(x, threads=threads)))
 
     def layer_norm(name, x, gamma, beta, eps):
         nbytes = 2 * x.nbytes + gamma.nbytes + beta.nbytes
@@ -159,15 +164,15 @@ def build_other_configs(ctx, D, synth, rotate_bytes=600e6, max_sets=48):
         dg, db = ctx.upload(gamma), ctx.upload(beta)
         rows, length = x.size // x.shape[-1], x.shape[-1]
         ops.append(Op(name, nbytes, [(lambda i=i: ctx.layernorm_raw(do[i].ptr, dx[i].ptr, dg.ptr, db.ptr, rows, length, eps))
-                                     for i in range(k)]))
+                                     for i in range(k)], cpu=lambda threads: O.layer_norm(x, gamma, beta, eps, threads=threads)))
 
-    def reduce(name, kind, x, outer, red, inner):
+    def reduce(name, kind, x, outer, red, inner, axes):
         nbytes = x.nbytes + 4 * outer * inner
         k = sets(nbytes)
         dx = [ctx.upload(x) for _ in range(k)]
         do = [ctx.alloc(4 * outer * inner) for _ in range(k)]
         ops.append(Op(name, nbytes, [(lambda i=i: ctx.reduce_raw(kind, do[i].ptr, dx[i].ptr, outer, red, inner))
-                                     for i in range(k)]))
+                                     for i in range(k)], cpu=lambda threads: O.reduce(kind, x, axes, True)))  # single-threaded in the reference
 
     c0 = synth.cfg0()
     binary("cfg0 Add [1,197,768]+[768]", D.ADD, c0["a"], c0["b"])
@@ -178,7 +183,7 @@ def build_other_configs(ctx, D, synth, rotate_bytes=600e6, max_sets=48):
     x = c2["x"]
     mean = np.zeros((32, 197, 1), np.float32)
     layer_norm("cfg2 LayerNorm (fused) [32,197,768]", x, c2["gamma"], c2["beta"], float(c2["eps"]))
-    reduce("cfg2 ReduceMean(-1) [32,197,768]", D.REDUCE_MEAN, x, 32 * 197, 768, 1)
+    reduce("cfg2 ReduceMean(-1) [32,197,768]", D.REDUCE_MEAN, x, 32 * 197, 768, 1, [-1])
     binary("cfg2 Sub [32,197,768]-[32,197,1]", D.SUB, x, mean)
     binary("cfg2 Pow(.,2) [32,197,768]", D.POW, x, np.array(2.0, np.float32))
     binary("cfg2 Div [32,197,768]/[32,197,1]", D.DIV, x, mean + np.float32(1.5))
@@ -188,7 +193,7 @@ def build_other_configs(ctx, D, synth, rotate_bytes=600e6, max_sets=48):
     unary("cfg3 Erf [32,197,3072]", D.ERF, c3["x"])
     binary("cfg3 Mul [32,197,3072]*[32,197,3072]", D.MUL, c3["x"], c3["x"])
     se = c3["se"]
-    reduce("cfg3 ReduceMean(H,W) [32,576,7,7]", D.REDUCE_MEAN, se, 32 * 576, 49, 1)
+    reduce("cfg3 ReduceMean(H,W) [32,576,7,7]", D.REDUCE_MEAN, se, 32 * 576, 49, 1, [2, 3])
     unary("cfg3 HardSigmoid [32,576,1,1]", D.HARDSIGMOID, np.zeros((32, 576, 1, 1), np.float32), 1.0 / 6.0, 0.5)
     binary("cfg3 Mul [32,576,7,7]*[32,576,1,1]", D.MUL, se, np.ones((32, 576, 1, 1), np.float32))
     return ops
@@ -526,12 +531,25 @@ def main():
 
     if args.all_configs:
         others = []
+        log("%-44s %14s %10s %10s %8s %14s %14s" % ("kernel", "alg. bytes", "us/call", "GB/s", "% peak", "CPU 16 thr us", "CPU 1 thr us"))
         for o in build_other_configs(ctx, D, synth):
             ms = time_kernel(ctx, o, args.kernel_iters, 5)
             gbps = o.nbytes / (ms * 1e-3) / 1e9
-            others.append({"kernel": o.name, "bytes": o.nbytes, "us": round(ms * 1e3, 2), "GBps": round(gbps, 1),
-                           "pct_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 1)})
-            log("%-44s %14d %10.2f %10.1f %8.1f" % (o.name, o.nbytes, ms * 1e3, gbps, 100.0 * gbps / HBM_PEAK_GBPS))
+            row = {"kernel": o.name, "bytes": o.nbytes, "us": round(ms * 1e3, 2), "GBps": round(gbps, 1),
+                   "pct_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 1)}
+            cpu_us = {}
+            if not args.no_cpu and o.cpu:
+                for threads in (16, 1):               # the CPU oracle on the host cores, best of 2 calls
+                    best = float("inf")
+                    for _ in range(2):
+                        t0 = time.perf_counter()
+                        o.cpu(threads)
+                        best = min(best, time.perf_counter() - t0)
+                    cpu_us[threads] = best * 1e6
+                row["cpu_us_16_threads"], row["cpu_us_1_thread"] = round(cpu_us[16], 1), round(cpu_us[1], 1)
+            others.append(row)
+            log("%-44s %14d %10.2f %10.1f %8.1f %14s %14s" % (o.name, o.nbytes, ms * 1e3, gbps, 100.0 * gbps / HBM_PEAK_GBPS,
+                                                               "%.1f" % cpu_us[16] if cpu_us else "-", "%.1f" % cpu_us[1] if cpu_us else "-"))
         graphs_rows = session_table(synth, ctx)
         for r in graphs_rows:
             log("%-36s kernels %7.1f us, as one HIP graph %7.1f us (%7.1f GB/s)  run_device() wall %7.1f us  run() incl. PCIe %7.3f ms"
