@@ -166,7 +166,7 @@ def _declare_graph(L):
     f("ahip_model_infer_value_shape", [c_void_p, c_int64, P(c_int), P(c_int), P(c_int64)])
     f("ahip_model_execution_plan", [c_void_p, P(c_int64), P(c_int), c_int, P(c_int64), c_int, P(c_int), P(c_int)])
     for name in ("ahip_fuse_layer_norm", "ahip_fuse_gelu", "ahip_fuse_fast_gelu", "ahip_eliminate_identity", "ahip_fuse_softmax_prologue",
-                 "ahip_fuse_matmul_bias"):
+                 "ahip_fuse_matmul_bias", "ahip_fuse_transpose_matmul"):
         f(name, [c_void_p, P(c_int)])
     f("ahip_fuse_elemwise_ops", [c_void_p, c_int, P(c_int)])
     f("ahip_tensor_new", [c_int, c_int, P(c_int64), c_void_p, c_size_t, P(c_void_p)])

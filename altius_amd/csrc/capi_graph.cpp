@@ -437,6 +437,7 @@ int ahip_fuse_layer_norm(ahip_model *model, int *count) { return run_pass(model,
 int ahip_fuse_gelu(ahip_model *model, int *count) { return run_pass(model, count, fuse_gelu, "ahip_fuse_gelu"); }
 int ahip_fuse_fast_gelu(ahip_model *model, int *count) { return run_pass(model, count, fuse_fast_gelu, "ahip_fuse_fast_gelu"); }
 int ahip_eliminate_identity(ahip_model *model, int *count) { return run_pass(model, count, eliminate_identity, "ahip_eliminate_identity"); }
+int ahip_fuse_transpose_matmul(ahip_model *model, int *count) { return run_pass(model, count, fuse_transpose_matmul, "ahip_fuse_transpose_matmul"); }
 int ahip_fuse_matmul_bias(ahip_model *model, int *count) { return run_pass(model, count, fuse_matmul_bias, "ahip_fuse_matmul_bias"); }
 int ahip_fuse_softmax_prologue(ahip_model *model, int *count) { return run_pass(model, count, fuse_softmax_prologue, "ahip_fuse_softmax_prologue"); }
 int ahip_fuse_elemwise_ops(ahip_model *model, int rule, int *count) {

@@ -60,6 +60,10 @@ bool Op::get_int(const std::string &n, int64_t *v) const {
         *v = prologue_mask ? 1 : 0;
         return true;
     }
+    if (kind == OpKind::MatMul && (n == "transA" || n == "transB")) {  // set by fuse_transpose_matmul
+        *v = (n == "transA" ? trans_a : trans_b) ? 1 : 0;
+        return true;
+    }
     if (n == "axis" && is(kind, {OpKind::Softmax, OpKind::LayerNormalization, OpKind::Concat, OpKind::Flatten,
                                  OpKind::Gather, OpKind::Split})) {
         *v = axis;

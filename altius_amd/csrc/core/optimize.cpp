@@ -510,4 +510,49 @@ size_t fuse_matmul_bias(Model &model) {
     return count;
 }
 
+size_t fuse_transpose_matmul(Model &model) {
+    const auto users = model.get_value_users();
+    const auto parents = model.get_value_parents();
+    const auto &outs = model.graph.outputs;
+    auto swaps_last_two = [](const std::vector<int64_t> &perm) {
+        const size_t r = perm.size();
+        if (r < 2 || r > 4) return false;
+        for (size_t i = 0; i + 2 < r; i++)
+            if (perm[i] != (int64_t)i) return false;
+        return perm[r - 2] == (int64_t)r - 1 && perm[r - 1] == (int64_t)r - 2;
+    };
+    size_t count = 0;
+    std::set<NodeId> maybe_dead;
+    for (NodeId mid : model.topo_sort_nodes()) {
+        Node &mm = model.graph.nodes[mid];
+        if (mm.op.kind != OpKind::MatMul || mm.inputs.size() < 2) continue;
+        bool changed = false;
+        for (int side = 0; side < 2; side++) {
+            auto p = parents.find(mm.inputs[side]);
+            if (p == parents.end()) continue;
+            const Node &tr = model.graph.nodes[p->second];
+            if (tr.op.kind != OpKind::Transpose || tr.inputs.size() != 1 || !swaps_last_two(tr.op.perm)) continue;
+            bool &flag = side == 0 ? mm.op.trans_a : mm.op.trans_b;
+            mm.inputs[side] = tr.inputs[0];
+            flag = !flag;
+            maybe_dead.insert(p->second);
+            changed = true;
+        }
+        if (changed) count++;
+    }
+    // A folded Transpose goes away when nothing else reads it.
+    if (count) {
+        const auto now = model.get_value_users();
+        for (NodeId id : maybe_dead) {
+            const ValueId out = model.graph.nodes[id].outputs[0];
+            auto u = now.find(out);
+            const bool read = u != now.end() && !u->second.empty();
+            if (!read && std::find(outs.begin(), outs.end(), out) == outs.end()) model.graph.nodes[id].deleted = true;
+        }
+        model.remove_unnecessary_nodes();
+    }
+    (void)users;
+    return count;
+}
+
 }  // namespace altius

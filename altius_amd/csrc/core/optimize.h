@@ -58,6 +58,13 @@ size_t fuse_softmax_prologue(Model &model);
 // Returns the number of MatMul nodes rewritten.
 size_t fuse_matmul_bias(Model &model);
 
+// Transpose of the last two axes (perm [1,0], [0,2,1] or [0,1,3,2]) in front of a MatMul operand is folded into
+// the product: the MatMul node reads the untransposed tensor and carries trans_a / trans_b.  The reference has
+// this pass switched off (crates/core/src/optimize/transpose_fusion.rs:10-104 emits a Gemm its interpreter cannot
+// run on batched operands, mod.rs:7); here the MatMul kernel takes the flags.  Unlike the reference's draft, a
+// Transpose that has other readers is kept for them.  Returns the number of MatMul nodes rewritten.
+size_t fuse_transpose_matmul(Model &model);
+
 enum class ElemwiseFusionRule { ReferenceRule = 0, ExtendedRule = 1 };
 bool fuse_elemwise_ops(Model &model, ElemwiseFusionRule rule, size_t *count, std::string *err);
 

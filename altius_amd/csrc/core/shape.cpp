@@ -527,7 +527,9 @@ bool compute_output_shapes(const Model &model, Op &op, const std::vector<const T
         if (!need_inputs(2)) return false;
         const FixedDimensions &a = inputs[0]->dims(), &b = inputs[1]->dims();
         if (a.len() < 2 || b.len() < 2) return fail(err, "MatMul: operands must have at least two dimensions");
-        const size_t m = a[a.len() - 2], k = a[a.len() - 1], k2 = b[b.len() - 2], n = b[b.len() - 1];
+        // trans_a / trans_b are set by fuse_transpose_matmul only: the stored operand is the transposed one.
+        const size_t m = op.trans_a ? a[a.len() - 1] : a[a.len() - 2], k = op.trans_a ? a[a.len() - 2] : a[a.len() - 1];
+        const size_t k2 = op.trans_b ? b[b.len() - 1] : b[b.len() - 2], n = op.trans_b ? b[b.len() - 2] : b[b.len() - 1];
         if (k != k2) return fail(err, "MatMul: A shape: " + a.to_string() + ", B shape: " + b.to_string());
         std::vector<FixedDimension> ab(a.as_vec().begin(), a.as_vec().end() - 2), bb(b.as_vec().begin(), b.as_vec().end() - 2);
         auto batch = FixedDimensions(ab).broadcast(FixedDimensions(bb));

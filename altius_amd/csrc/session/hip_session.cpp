@@ -1202,7 +1202,11 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
     case OpKind::MatMul: {  // compute_mat_mul (session.rs:621-684), with NumPy broadcasting of the batch axes
         if (!need(2) || !need_f32({0, 1})) return false;
         const FixedDimensions &a = in[0]->dims, &b = in[1]->dims;
-        const size_t m = a[a.len() - 2], k = a[a.len() - 1], n = b[b.len() - 1];
+        // trans_a / trans_b (fuse_transpose_matmul): the stored operand is the transposed one.
+        const int ta = op.trans_a ? 1 : 0, tb = op.trans_b ? 1 : 0;
+        const size_t lda = a[a.len() - 1], ldb = b[b.len() - 1];
+        const size_t m = ta ? a[a.len() - 1] : a[a.len() - 2], k = ta ? a[a.len() - 2] : a[a.len() - 1];
+        const size_t n = tb ? b[b.len() - 2] : b[b.len() - 1];
         size_t a_batch = 1, b_batch = 1, batch = 1;
         for (size_t i = 0; i + 2 < a.len(); i++) a_batch *= a[i];
         for (size_t i = 0; i + 2 < b.len(); i++) b_batch *= b[i];
@@ -1216,11 +1220,11 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
             bias = f(in[2]);
         }
         const float beta = bias ? 1.0f : 0.0f;
-        if (b_batch == 1 && a_batch == batch) {
+        if (b_batch == 1 && a_batch == batch && !ta) {
             // [.., m, k] x [k, n]: one tall sgemm, as the reference does (session.rs:653-660)
-            rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), bias, 1, batch * m, n, k, 0, 0, k, n, n, 0, 0, 0, 0, 1, 1.0f, beta);
+            rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), bias, 1, batch * m, n, k, 0, tb, lda, ldb, n, 0, 0, 0, 0, 1, 1.0f, beta);
         } else if ((a_batch == batch || a_batch == 1) && (b_batch == batch || b_batch == 1)) {
-            rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), bias, batch, m, n, k, 0, 0, k, n, n, a_batch == 1 ? 0 : m * k,
+            rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), bias, batch, m, n, k, ta, tb, lda, ldb, n, a_batch == 1 ? 0 : m * k,
                              b_batch == 1 ? 0 : k * n, m * n, 0, 1, 1.0f, beta);
         } else {
             return fail(err, SessionError::Message, "MatMul: batch axes that broadcast against each other partially are not supported");

@@ -386,6 +386,10 @@ class Model:
     def eliminate_identity(self):
         return self._pass(self.L.ahip_eliminate_identity)
 
+    def fuse_transpose_matmul(self):
+        """A Transpose of the last two axes feeding a MatMul operand becomes a flag of the product."""
+        return self._pass(self.L.ahip_fuse_transpose_matmul)
+
     def fuse_matmul_bias(self):
         """MatMul -> Add(bias row) becomes a MatMul node with the bias as third input."""
         return self._pass(self.L.ahip_fuse_matmul_bias)

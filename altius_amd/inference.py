@@ -52,6 +52,7 @@ def session(model, enable_profiling=False, intra_op_num_threads=1, backend="hip"
     m.fuse_fast_gelu()
     m.fuse_softmax_prologue()
     m.fuse_matmul_bias()
+    m.fuse_transpose_matmul()
     m.fuse_elemwise_ops(extended=True)
     m.eliminate_identity()
     builder = HipSessionBuilder(m).with_profiling_enabled(enable_profiling).with_intra_op_num_threads(intra_op_num_threads)

@@ -284,8 +284,8 @@ def vit_table(batch, layers=12):
     ref.fuse_layer_norm(), ref.fuse_gelu(), ref.fuse_fast_gelu(), ref.eliminate_identity()
     versions.append(("reference rewrites (fuse_layer_norm, fuse_gelu)", ref))
     ours = ref.clone()
-    ours.fuse_softmax_prologue(), ours.fuse_matmul_bias(), ours.fuse_elemwise_ops(extended=True)
-    versions.append(("+ softmax prologue, matmul bias, element-wise chains", ours))
+    ours.fuse_softmax_prologue(), ours.fuse_matmul_bias(), ours.fuse_transpose_matmul(), ours.fuse_elemwise_ops(extended=True)
+    versions.append(("+ softmax prologue, matmul bias / transposes, element-wise chains", ours))
     rows = []
     for name, model in versions:
         sess = HipSessionBuilder(model).build()

@@ -435,6 +435,11 @@ int ahip_fuse_softmax_prologue(ahip_model *model, int *count);
  * no other reader, becomes a MatMul node with b as third input; the session adds it in the product's epilogue
  * (the same single addition per element, without the extra pass over the output). */
 int ahip_fuse_matmul_bias(ahip_model *model, int *count);
+/* fuse_transpose_matmul (crates/core/src/optimize/transpose_fusion.rs:10-104; switched off in the reference,
+ * mod.rs:7, because its interpreter cannot run the node it emits): a Transpose of the last two axes in front of a
+ * MatMul operand is folded into the product.  The MatMul node then reads the untransposed tensor and reports
+ * "transA" / "transB" through ahip_node_get_attr_int; a Transpose with other readers stays for them. */
+int ahip_fuse_transpose_matmul(ahip_model *model, int *count);
 enum ahip_fuse_rule { AHIP_FUSE_REFERENCE_RULE = 0, AHIP_FUSE_EXTENDED_RULE = 1 };
 int ahip_fuse_elemwise_ops(ahip_model *model, int rule, int *count);
 

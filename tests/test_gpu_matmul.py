@@ -180,3 +180,37 @@ def test_matmul_with_absorbed_bias_has_the_bits_of_matmul_then_add(case, x_shape
     (got,) = HipSessionBuilder(fused).build().run([x])
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     np.testing.assert_allclose(got, np.matmul(x.astype(np.float64), w.astype(np.float64)) + b, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("a_shape,b_shape,ta,tb", [([2, 12, 197, 64], [2, 12, 197, 64], False, True), ([6, 5], [4, 6], True, True),
+                                                   ([3, 40, 70], [3, 40, 33], True, False), ([4, 50, 32], [64, 32], False, True)])
+def test_transposes_folded_into_the_product(case, a_shape, b_shape, ta, tb):
+    """fuse_transpose_matmul: MatMul on the untransposed tensors with trans flags against Transpose -> MatMul; the
+    accumulation order does not change, so the bits do not either."""
+    case(f"matmul with folded transposes {a_shape} {b_shape} ta={ta} tb={tb}")
+    rng = np.random.default_rng(8)
+    a = rng.standard_normal(a_shape).astype(np.float32)
+    b = rng.standard_normal(b_shape).astype(np.float32)
+    swap = lambda r: list(range(r - 2)) + [r - 1, r - 2]
+    m = Model()
+    va, vb = m.new_val_named_and_shaped("a", a_shape), m.new_val_named_and_shaped("b", b_shape)
+    xa, xb = va, vb
+    if ta:
+        xa = m.new_val()
+        m.add_node(Op.Transpose, [va], [xa], perm=swap(len(a_shape)))
+    if tb:
+        xb = m.new_val()
+        m.add_node(Op.Transpose, [vb], [xb], perm=swap(len(b_shape)))
+    y = m.new_val()
+    m.add_node(Op.MatMul, [xa, xb], [y])
+    m.add_input(va)
+    m.add_input(vb)
+    m.add_output(y)
+    fused = m.clone()
+    assert fused.fuse_transpose_matmul() == 1 and [n["op_name"] for n in fused.nodes()] == ["MatMul"]
+    (want,) = HipSessionBuilder(m).build().run([a, b])
+    (got,) = HipSessionBuilder(fused).build().run([a, b])
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    A = np.swapaxes(a, -1, -2) if ta else a
+    Bm = np.swapaxes(b, -1, -2) if tb else b
+    np.testing.assert_allclose(got, np.matmul(A.astype(np.float64), Bm.astype(np.float64)), rtol=1e-4, atol=1e-4)

@@ -548,3 +548,54 @@ def test_fuse_matmul_bias():
     assert build([5, 10], [10, 15], [5, 1])[0].fuse_matmul_bias() == 0
     assert build([5, 10], [10, 15], [5, 15])[0].fuse_matmul_bias() == 0
     assert build([5, 10], [10, 15], [15], extra_reader=True)[0].fuse_matmul_bias() == 0
+
+
+def test_fuse_transpose_matmul():
+    """crates/core/src/optimize/transpose_fusion.rs:33-62: perms [1,0], [0,2,1], [0,1,3,2] on either operand."""
+    def attr(m, node, name):
+        v = ctypes.c_int64()
+        _lib.check(m.L.ahip_node_get_attr_int(m.handle, node["id"], name.encode(), ctypes.byref(v)))
+        return v.value
+
+    m = Model()
+    q = m.new_val_named_and_shaped("q", [2, 3, 7, 4])
+    k = m.new_val_named_and_shaped("k", [2, 3, 7, 4])
+    kt, s, other = m.new_val(), m.new_val_named("s"), m.new_val_named("other")
+    m.add_node(Op.Transpose, [k], [kt], perm=[0, 1, 3, 2])
+    m.add_node(Op.MatMul, [q, kt], [s])
+    m.add_input(q)
+    m.add_input(k)
+    m.add_output(s)
+    keep = m.clone()
+    assert m.fuse_transpose_matmul() == 1
+    (mm,) = m.nodes()
+    assert mm["op_name"] == "MatMul" and mm["inputs"] == [q, k] and attr(m, mm, "transB") == 1 and attr(m, mm, "transA") == 0
+    assert m.infer_value_shape(s) == ([2, 3, 7, 7], F32)
+    assert m.fuse_transpose_matmul() == 0
+
+    # a Transpose with a second reader stays for it; a permutation that moves other axes is not folded
+    t2 = keep.new_val()
+    keep.add_node(Op.ReLU, [kt], [t2])
+    keep.add_output(t2)
+    assert keep.fuse_transpose_matmul() == 1
+    assert sorted(n["op_name"] for n in keep.nodes()) == ["MatMul", "ReLU", "Transpose"]
+    m = Model()
+    a = m.new_val_named_and_shaped("a", [5, 2, 6])
+    at, w, y = m.new_val(), m.new_initializer(np.zeros([2, 5, 3], np.float32)), m.new_val()
+    m.add_node(Op.Transpose, [a], [at], perm=[1, 2, 0])
+    m.add_node(Op.MatMul, [at, w], [y])
+    m.add_input(a)
+    m.add_output(y)
+    assert m.fuse_transpose_matmul() == 0
+    # both operands, rank 2
+    m = Model()
+    a, b = m.new_val_named_and_shaped("a", [6, 5]), m.new_val_named_and_shaped("b", [4, 6])
+    at, bt, y = m.new_val(), m.new_val(), m.new_val()
+    m.add_node(Op.Transpose, [a], [at], perm=[1, 0])
+    m.add_node(Op.Transpose, [b], [bt], perm=[1, 0])
+    m.add_node(Op.MatMul, [at, bt], [y])
+    m.add_input(a)
+    m.add_input(b)
+    m.add_output(y)
+    assert m.fuse_transpose_matmul() == 1 and len(m.nodes()) == 1
+    assert m.infer_value_shape(y) == ([5, 4], F32)
