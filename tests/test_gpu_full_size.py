@@ -85,3 +85,25 @@ def test_cfg3_gelu_and_mean_full(ctx, case):
     assert_bits_equal(twice, mean * np.float32(2), "mean(2x) = 2 mean(x)")
     neg = ctx.reduce(D.REDUCE_MEAN, -se, 32 * 576, 49, 1).reshape(mean.shape)
     assert_bits_equal(neg, -mean, "mean(-x) = -mean(x)")
+
+
+def test_cfg4_masked_softmax_in_one_kernel(ctx, case, cfg4):
+    """Add(mask) + Softmax fused at the full configs[4] size: the bits of the two kernels, on all 605 184 rows."""
+    case("full cfg4 Add(mask)+Softmax in one kernel [256,12,197,197]")
+    scores, mask = cfg4["scores"], cfg4["mask"]
+    fused = ctx.softmax_prologue(scores, 0, 1.0, mask)
+    assert_bits_equal(fused, ctx.softmax(ctx.binary(D.ADD, scores, mask)), "fused vs Add then Softmax")
+
+
+def test_cfg3_erf_gelu_chain_in_one_kernel(ctx, case):
+    """The 5-node erf-GELU chain as one FusedElemwise kernel at the full configs[3] size, against the oracle's chain."""
+    from altius_amd._lib import FUSED_ACC as ACC
+
+    case("full cfg3 erf-GELU chain in one kernel [32,197,3072]")
+    c = synth.cfg3(batch=32)
+    x = c["x"]
+    s = lambda v: np.array(v, np.float32)
+    steps = [("b", D.DIV, 0, 1), ("u", D.ERF, ACC, 0), ("b", D.ADD, ACC, 2), ("b", D.MUL, 0, ACC), ("b", D.MUL, ACC, 3)]
+    got = ctx.fused_elemwise([x, s(c["sqrt2"]), s(1.0), s(0.5)], steps)
+    t = O.binary(O.ADD, O.unary(O.ERF, O.binary(O.DIV, x, s(c["sqrt2"]), threads=THREADS), threads=THREADS), s(1.0), threads=THREADS)
+    assert_bits_equal(got, O.binary(O.MUL, O.binary(O.MUL, x, t, threads=THREADS), s(0.5), threads=THREADS), "fused chain vs oracle chain")
