@@ -89,6 +89,9 @@ def _declare(L):
                          c_float])
     f("ahip_gemm", [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p] + [c_size_t] * 4 + [c_int, c_int] + [c_size_t] * 8
       + [c_float, c_float])
+    f("ahip_gemm_set_algorithm", [c_void_p, c_int])
+    f("ahip_gemm_register_constant", [c_void_p, c_void_p, c_size_t])
+    f("ahip_gemm_unregister_constant", [c_void_p, c_void_p])
     f("ahip_conv2d", [c_void_p] * 6 + [c_size_t] * 16)
     f("ahip_maxpool", [c_void_p] * 3 + [c_size_t] * 11)
     f("ahip_resize", [c_void_p] * 3 + [c_size_t] * 5 + [c_int])
@@ -185,6 +188,7 @@ def _declare_graph(L):
     f("ahip_session_builder_with_profiling_enabled", [c_void_p, c_int])
     f("ahip_session_builder_with_device", [c_void_p, c_int])
     f("ahip_session_builder_with_graph_replay", [c_void_p, c_int])
+    f("ahip_session_builder_with_gemm_algorithm", [c_void_p, c_int])
     f("ahip_session_graph_replays", [c_void_p, P(c_size_t)])
     f("ahip_session_builder_build", [c_void_p, P(c_void_p)])
     f("ahip_session_free", [c_void_p], None)

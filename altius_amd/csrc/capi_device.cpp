@@ -381,6 +381,24 @@ int ahip_gemm(ahip_ctx *ctx, float *c, const float *a, const float *b, const flo
                                b_batch_stride, c_batch_stride, c0_row_stride, c0_col_stride, alpha, beta);
 }
 
+int ahip_gemm_set_algorithm(ahip_ctx *ctx, int algorithm) {
+    REQUIRE_CTX(ctx, "ahip_gemm_set_algorithm");
+    if (algorithm != AHIP_GEMM_AUTO && algorithm != AHIP_GEMM_FP32 && algorithm != AHIP_GEMM_BF16X3)
+        return ctx->d.fail(AHIP_ERR_ARG, "ahip_gemm_set_algorithm: unknown algorithm");
+    ctx->d.gemm_algorithm = algorithm;
+    return AHIP_OK;
+}
+
+int ahip_gemm_register_constant(ahip_ctx *ctx, const void *ptr, size_t bytes) {
+    REQUIRE_CTX(ctx, "ahip_gemm_register_constant");
+    return altius::gemm_register_constant(ctx->d, ptr, bytes);
+}
+
+int ahip_gemm_unregister_constant(ahip_ctx *ctx, const void *ptr) {
+    REQUIRE_CTX(ctx, "ahip_gemm_unregister_constant");
+    return altius::gemm_unregister_constant(ctx->d, ptr);
+}
+
 int ahip_conv2d(ahip_ctx *ctx, float *out, const float *x, const float *w, const float *bias, float *col, size_t batch,
                 size_t c, size_t ih, size_t iw, size_t oc, size_t oh, size_t ow, size_t kh, size_t kw, size_t stride_h,
                 size_t stride_w, size_t dilation_h, size_t dilation_w, size_t pad_top, size_t pad_left, size_t group) {

@@ -27,6 +27,7 @@ struct ahip_session_builder {
     bool profiling = false;
     int device = 0;
     bool graph_replay = false;
+    int gemm_algorithm = AHIP_GEMM_AUTO;
 };
 struct ahip_session {
     std::shared_ptr<HipSession> s;  // shared with the device tensors the session has handed out
@@ -537,6 +538,14 @@ int ahip_session_builder_with_graph_replay(ahip_session_builder *builder, int en
     return AHIP_OK;
 }
 
+int ahip_session_builder_with_gemm_algorithm(ahip_session_builder *builder, int algorithm) {
+    if (!builder) return fail(AHIP_ERR_ARG, "null builder");
+    if (algorithm != AHIP_GEMM_AUTO && algorithm != AHIP_GEMM_FP32 && algorithm != AHIP_GEMM_BF16X3)
+        return fail(AHIP_ERR_ARG, "ahip_session_builder_with_gemm_algorithm: unknown algorithm");
+    builder->gemm_algorithm = algorithm;
+    return AHIP_OK;
+}
+
 int ahip_session_graph_replays(const ahip_session *session, size_t *count) {
     if (!session || !count) return fail(AHIP_ERR_ARG, "ahip_session_graph_replays: null argument");
     *count = session->s->graph_replays();
@@ -547,7 +556,7 @@ int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **ses
     if (!builder || !session) return fail(AHIP_ERR_ARG, "ahip_session_builder_build: null argument");
     *session = nullptr;
     HipSessionBuilder b(builder->model);
-    b.with_intra_op_num_threads(builder->threads).with_profiling_enabled(builder->profiling).with_device(builder->device).with_graph_replay(builder->graph_replay);
+    b.with_intra_op_num_threads(builder->threads).with_profiling_enabled(builder->profiling).with_device(builder->device).with_graph_replay(builder->graph_replay).with_gemm_algorithm(builder->gemm_algorithm);
     SessionError err;
     std::unique_ptr<HipSession> s = b.build(&err);
     if (!s) return fail(err.code(), err.to_string());

@@ -85,6 +85,7 @@ int check_device_flags(DeviceCtx &ctx) {
 void destroy_device_ctx(DeviceCtx *ctx) {
     if (hipSetDevice(ctx->device) != hipSuccess) return;
     (void)hipStreamSynchronize(ctx->stream);
+    gemm_release_all(*ctx);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     ctx->scratch = nullptr;
     if (ctx->flags) (void)hipFree(ctx->flags);

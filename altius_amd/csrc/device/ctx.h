@@ -7,10 +7,26 @@
 #include <stdint.h>
 
 #include <string>
+#include <vector>
 
 #include "../../../include/altius_hip.h"
 
 namespace altius {
+
+// A device buffer whose contents the caller has declared immutable (weights), and the bf16 planes the
+// split GEMM has derived from an operand inside such a buffer.
+struct ConstantBuffer {
+    const void *ptr;
+    size_t bytes;
+};
+struct PackedOperand {
+    const void *owner;  // the ConstantBuffer the operand lies in
+    const void *src;
+    size_t rows, k, ld;
+    bool k_contig;
+    void *planes;
+    size_t bytes;
+};
 
 // One context = one device + one stream.  All work issued through a context is
 // ordered on that stream.  A context is not thread-safe; use one per thread.
@@ -30,6 +46,15 @@ struct DeviceCtx {
     // Chains of element-wise steps that were instantiated at compile time run as straight-line code;
     // switched off, every chain takes the interpreting kernel (tests compare the two).
     bool fused_static_chains = true;
+    // Which kernel large single-batch fp32 products take (AHIP_GEMM_*).
+    int gemm_algorithm = AHIP_GEMM_AUTO;
+    // bf16 planes of the run-time operands of the split GEMM (device memory, owned, grows on demand;
+    // the generation counts reallocations so that holders of recorded launches can tell).
+    void *gemm_ws = nullptr;
+    size_t gemm_ws_bytes = 0;
+    uint64_t gemm_ws_generation = 0;
+    std::vector<ConstantBuffer> gemm_constants;
+    std::vector<PackedOperand> gemm_packed;
     std::string last_error;
 
     bool streaming(size_t bytes) const { return bytes >= nt_threshold_bytes; }
@@ -94,6 +119,20 @@ int launch_gemm(DeviceCtx &ctx, float *c, const float *a, const float *b, const 
                 size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t a_batch_stride,
                 size_t b_batch_stride, size_t c_batch_stride, size_t c0_row_stride, size_t c0_col_stride, float alpha,
                 float beta);
+
+// The same product for one batch through three bf16 planes per operand and six bf16 MFMAs per fp32
+// product (gemm_split.hip): as accurate as an fp32 multiply-add chain, about 1.6 times the fp32 matrix
+// cores' rate on large shapes.  launch_gemm takes this route by itself according to ctx.gemm_algorithm.
+int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t m, size_t n, size_t k,
+                      int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t c0_row_stride, size_t c0_col_stride,
+                      float alpha, float beta);
+// Large and tile-filling enough for the split kernel to win (the AHIP_GEMM_AUTO rule).
+bool gemm_split_worthwhile(size_t m, size_t n, size_t k);
+// Declares [ptr, ptr + bytes) immutable until unregistered: operands inside it are split once and the
+// planes kept.  Unregistering frees them (after synchronising the stream).
+int gemm_register_constant(DeviceCtx &ctx, const void *ptr, size_t bytes);
+int gemm_unregister_constant(DeviceCtx &ctx, const void *ptr);
+void gemm_release_all(DeviceCtx &ctx);
 
 // col[b][c][fy][fx][oh][ow] for a convolution (movement.hip); maxpool over [planes, ih, iw].
 int launch_im2col(DeviceCtx &ctx, float *col, const float *x, size_t batch, size_t c, size_t ih, size_t iw, size_t oh,

@@ -1,0 +1,502 @@
+// fp32 matrix multiplication on the bf16 matrix cores: every fp32 operand value x is written as
+// x = h0 + h1 + h2 with three bf16 numbers (8 + 8 + 8 significand bits: the sum is exact), and
+//   a * b = a0 b0 + (a0 b1 + a1 b0) + (a0 b2 + a1 b1 + a2 b0) + [a1 b2 + a2 b1 + a2 b2]
+// is accumulated in fp32 by six v_mfma_f32_32x32x16_bf16 per tile and k step; the bracket, below
+// 2^-23 |a b| with random signs, is dropped.  Against a float64 product the result is as close as
+// a chain of fp32 fused multiply-adds (the reference's sgemm, crates/session_interpreter/src/gemm.rs:3-52,
+// called by compute_mat_mul and compute_gemm, session.rs:621-794), and six bf16 MFMAs cost 6 / 16 of
+// one fp32 MFMA per product.
+//
+// Two kernels.  split_planes turns an operand into three planes stored [plane][k / 8][row][8]
+// (16-byte chunks: 8 consecutive k of one row), rows and k padded with zeros to whole tiles, so
+// that both the GEMM's global reads and its LDS layout are plain contiguous copies.  gemm_bf16x3
+// computes a 256 x 256 tile of C per 512-thread block (8 wavefronts, 64 x 128 each) in k steps of
+// 16 through three LDS buffers that are filled by direct global->LDS loads issued two steps ahead;
+// one barrier per step.  The epilogue transposes the accumulators through LDS so that C is written
+// in whole 512-byte row segments.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+
+#include "common.h"
+#include "ctx.h"
+
+namespace altius {
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// ---------------------------------------------------------------- operand -> three bf16 planes
+
+__device__ __forceinline__ uint32_t round_bf16(uint32_t u) { return (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u; }
+
+// The upper halves of three floats whose sum is x.  Round-to-nearest at each step keeps the
+// residuals small and sign-symmetric; each residual is exact (it has at most 16, then 8 significant
+// bits).  A value that would round up to infinity is truncated instead; infinities and NaNs stay in
+// the first plane alone.
+__device__ __forceinline__ void split3(float x, uint32_t &h0, uint32_t &h1, uint32_t &h2) {
+    const uint32_t u = __float_as_uint(x);
+    const bool finite = (u & 0x7f800000u) != 0x7f800000u;
+    uint32_t r0 = round_bf16(u);
+    if ((r0 & 0x7f800000u) == 0x7f800000u) {
+        r0 = u & 0xffff0000u;
+        if (!finite && (u & 0x007fffffu)) r0 |= 0x00400000u;  // a NaN whose payload sat in the low half
+    }
+    const float e1 = finite ? x - __uint_as_float(r0) : 0.0f;
+    const uint32_t r1 = round_bf16(__float_as_uint(e1));
+    const float e2 = e1 - __uint_as_float(r1);
+    const uint32_t r2 = round_bf16(__float_as_uint(e2));
+    h0 = r0 >> 16;
+    h1 = r1 >> 16;
+    h2 = r2 >> 16;
+}
+
+__device__ __forceinline__ void store_planes(u32x4 *__restrict__ planes, const float (&v)[8], uint32_t row, uint32_t kg, uint32_t rp,
+                                             uint32_t kgs) {
+    uint32_t h[3][8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) split3(v[j], h[0][j], h[1][j], h[2][j]);
+#pragma unroll
+    for (int p = 0; p < 3; p++) {
+        u32x4 o;
+        o.x = h[p][0] | (h[p][1] << 16);
+        o.y = h[p][2] | (h[p][3] << 16);
+        o.z = h[p][4] | (h[p][5] << 16);
+        o.w = h[p][6] | (h[p][7] << 16);
+        planes[((size_t)p * kgs + kg) * rp + row] = o;
+    }
+}
+
+// Any strides: element (row, k) is src[row * s_r + k * s_k].  Consecutive lanes take consecutive rows,
+// which is the contiguous direction of an operand stored k-major (A transposed, B as given).
+__global__ __launch_bounds__(256) void split_planes(const float *__restrict__ src, u32x4 *__restrict__ planes, uint32_t rows, uint32_t k,
+                                                    size_t s_r, size_t s_k, uint32_t rp, uint32_t kgs) {
+    const uint32_t row = blockIdx.x * 64 + (threadIdx.x & 63);
+    const uint32_t kg = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (kg >= kgs) return;
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint32_t kk = kg * 8 + j;
+        v[j] = (row < rows && kk < k) ? src[(size_t)row * s_r + (size_t)kk * s_k] : 0.0f;
+    }
+    store_planes(planes, v, row, kg, rp, kgs);
+}
+
+// Rows contiguous in k and 16-byte aligned: four adjacent lanes read 128 contiguous bytes of a row,
+// sixteen rows per wavefront; each (plane, k group) store of a wavefront is 256 contiguous bytes.
+__global__ __launch_bounds__(256) void split_planes_rows(const float *__restrict__ src, u32x4 *__restrict__ planes, uint32_t rows,
+                                                         uint32_t k, size_t s_r, uint32_t rp, uint32_t kgs) {
+    const uint32_t row = blockIdx.x * 64 + (threadIdx.x >> 2);
+    const uint32_t kg = blockIdx.y * 4 + (threadIdx.x & 3);
+    if (kg >= kgs) return;
+    float v[8];
+    const uint32_t k0 = kg * 8;
+    if (row < rows && k0 + 8 <= k) {
+        const f32x4 lo = *reinterpret_cast<const f32x4 *>(src + (size_t)row * s_r + k0);
+        const f32x4 hi = *reinterpret_cast<const f32x4 *>(src + (size_t)row * s_r + k0 + 4);
+        v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = (row < rows && k0 + j < k) ? src[(size_t)row * s_r + k0 + j] : 0.0f;
+    }
+    store_planes(planes, v, row, kg, rp, kgs);
+}
+
+// ---------------------------------------------------------------- the product
+
+constexpr int TM = 256, TN = 256, THREADS = 512;
+
+// One k step of 16 (two k groups of 8) of both operand tiles.
+struct Stage {
+    u32x4 a[3][2][TM];
+    u32x4 b[3][2][TN];
+};
+constexpr uint32_t PLANE_BYTES = 2 * 256 * 16;  // distance between two planes of one operand inside a Stage
+static_assert(sizeof(Stage) == 6 * PLANE_BYTES, "Stage layout");
+
+struct SplitGemmArgs {
+    const u32x4 *ap, *bp;  // planes of op(A) (rows = m) and of op(B) transposed (rows = n)
+    float *c;
+    const float *c0;
+    uint32_t m, n, mp, np, kgs, ldc;
+    uint32_t c0_rs, c0_cs;
+    float alpha, beta;
+    uint32_t tiles_n, tiles, chunk;
+    int c_vec;    // 16-byte stores into C are aligned
+    int c_stream;  // C is large: write it with non-temporal stores
+};
+
+typedef __attribute__((address_space(3))) void *lds_ptr;
+typedef const __attribute__((address_space(1))) void *global_ptr;
+
+// Wavefront w fills rows [64 (w & 3), +64) of k group (w >> 2) of all three planes of both operands:
+// six loads of 1 KiB, each lane's 16 bytes landing at consecutive LDS addresses.
+__device__ __forceinline__ void issue(Stage &s, const u32x4 *ga, const u32x4 *gb, size_t a_plane, size_t b_plane, int sub) {
+#pragma unroll
+    for (int p = 0; p < 3; p++) {
+        __builtin_amdgcn_global_load_lds((global_ptr)(ga + p * a_plane), (lds_ptr)(&s.a[p][0][0] + sub), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((global_ptr)(gb + p * b_plane), (lds_ptr)(&s.b[p][0][0] + sub), 16, 0, 0);
+    }
+}
+
+// The fragment reads are written as asm: the compiler's wait-count pass drains every outstanding
+// global->LDS load before an LDS read that it cannot prove independent of them, which would undo
+// the two-steps-ahead prefetch.  The "+v" operands of the waits tie each use to its wait.
+#define DS_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off) : "memory")
+#define MFMA(A, B, C) C = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, A), __builtin_bit_cast(bf16x8, B), C, 0, 0, 0)
+
+// Smallest terms first.
+__device__ __forceinline__ void six(const u32x4 (&a)[3], const u32x4 (&b)[3], floatx16 &c) {
+    MFMA(a[0], b[2], c);
+    MFMA(a[2], b[0], c);
+    MFMA(a[1], b[1], c);
+    MFMA(a[0], b[1], c);
+    MFMA(a[1], b[0], c);
+    MFMA(a[0], b[0], c);
+}
+
+// a_addr / b_addr: LDS byte addresses of this lane's first A / B fragment in the stage.
+__device__ __forceinline__ void compute(uint32_t a_addr, uint32_t b_addr, floatx16 (&acc)[2][4]) {
+    u32x4 a0[3], a1[3], b0[3], b1[3], b2[3], b3[3];
+    DS_READ(a0[0], a_addr, 0);
+    DS_READ(a0[1], a_addr, PLANE_BYTES);
+    DS_READ(a0[2], a_addr, 2 * PLANE_BYTES);
+    DS_READ(b0[0], b_addr, 0);
+    DS_READ(b0[1], b_addr, PLANE_BYTES);
+    DS_READ(b0[2], b_addr, 2 * PLANE_BYTES);
+    DS_READ(a1[0], a_addr, 512);
+    DS_READ(a1[1], a_addr, PLANE_BYTES + 512);
+    DS_READ(a1[2], a_addr, 2 * PLANE_BYTES + 512);
+    DS_READ(b1[0], b_addr, 512);
+    DS_READ(b1[1], b_addr, PLANE_BYTES + 512);
+    DS_READ(b1[2], b_addr, 2 * PLANE_BYTES + 512);
+    asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(a0[0]), "+v"(a0[1]), "+v"(a0[2]), "+v"(b0[0]), "+v"(b0[1]), "+v"(b0[2]));
+    six(a0, b0, acc[0][0]);
+    asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(a1[0]), "+v"(a1[1]), "+v"(a1[2]));
+    six(a1, b0, acc[1][0]);
+    DS_READ(b2[0], b_addr, 1024);
+    DS_READ(b2[1], b_addr, PLANE_BYTES + 1024);
+    DS_READ(b2[2], b_addr, 2 * PLANE_BYTES + 1024);
+    asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(b1[0]), "+v"(b1[1]), "+v"(b1[2]));
+    six(a0, b1, acc[0][1]);
+    six(a1, b1, acc[1][1]);
+    DS_READ(b3[0], b_addr, 1536);
+    DS_READ(b3[1], b_addr, PLANE_BYTES + 1536);
+    DS_READ(b3[2], b_addr, 2 * PLANE_BYTES + 1536);
+    asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(b2[0]), "+v"(b2[1]), "+v"(b2[2]));
+    six(a0, b2, acc[0][2]);
+    six(a1, b2, acc[1][2]);
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(b3[0]), "+v"(b3[1]), "+v"(b3[2]));
+    six(a0, b3, acc[0][3]);
+    six(a1, b3, acc[1][3]);
+}
+
+// Stage t lives in buffer t % 3.  Before stage t is used: this wavefront's six loads of it have
+// landed (those of stage t + 1 may still be in flight), and the barrier says the same of every
+// wavefront and that all of them are done with stage t - 1, whose buffer the loads of stage
+// t + 2 then overwrite.
+__device__ __forceinline__ void step(uint32_t a_addr, uint32_t b_addr, Stage *next2, floatx16 (&acc)[2][4], bool more1, bool more2,
+                                     const u32x4 *ga, const u32x4 *gb, size_t a_plane, size_t b_plane, int sub) {
+    if (more1) asm volatile("s_waitcnt vmcnt(6)\n\ts_barrier" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    if (more2) issue(*next2, ga, gb, a_plane, b_plane, sub);
+    compute(a_addr, b_addr, acc);
+}
+
+__global__ __launch_bounds__(THREADS, 1) void gemm_bf16x3(SplitGemmArgs g) {
+    __shared__ Stage S[3];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1, lr = lane & 31, lk = lane >> 5;
+    // Consecutive block ids are dealt to the eight XCDs in turn; give each XCD (one L2) a contiguous
+    // run of tiles so that the blocks it runs together share operand panels.
+    const uint32_t slot = blockIdx.x >> 3, tile = (blockIdx.x & 7) * g.chunk + slot;
+    if (slot >= g.chunk || tile >= g.tiles) return;
+    const uint32_t m0 = (tile / g.tiles_n) * TM, n0 = (tile % g.tiles_n) * TN;
+    const size_t a_plane = (size_t)g.kgs * g.mp, b_plane = (size_t)g.kgs * g.np;
+
+    floatx16 acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    const uint32_t nst = g.kgs / 2;
+    const uint32_t a_addr = (uint32_t)(uintptr_t)(lds_ptr)&S[0].a[0][lk][wm * 64 + lr];
+    const uint32_t b_addr = (uint32_t)(uintptr_t)(lds_ptr)&S[0].b[0][lk][wn * 128 + lr];
+    const int sub = (wave >> 2) * 256 + (wave & 3) * 64;
+    const u32x4 *ga = g.ap + (size_t)(wave >> 2) * g.mp + m0 + (wave & 3) * 64 + lane;
+    const u32x4 *gb = g.bp + (size_t)(wave >> 2) * g.np + n0 + (wave & 3) * 64 + lane;
+    const size_t a_step = (size_t)2 * g.mp, b_step = (size_t)2 * g.np;
+    issue(S[0], ga, gb, a_plane, b_plane, sub);
+    if (nst > 1) issue(S[1], ga + a_step, gb + b_step, a_plane, b_plane, sub);
+#define STEP(CUR, NEXT2)                                                                                              \
+    {                                                                                                                 \
+        step(a_addr + CUR * (uint32_t)sizeof(Stage), b_addr + CUR * (uint32_t)sizeof(Stage), &S[NEXT2], acc, t + 1 < nst, \
+             t + 2 < nst, ga + (t + 2) * a_step, gb + (t + 2) * b_step, a_plane, b_plane, sub);                          \
+        if (++t >= nst) break;                                                                                        \
+    }
+    for (uint32_t t = 0;;) {
+        STEP(0, 2)
+        STEP(1, 0)
+        STEP(2, 1)
+    }
+#undef STEP
+
+    // Epilogue: each wavefront transposes 32 x 128 of its sub-tile at a time through a private LDS
+    // region (pitch 132 floats), then stores rows of 128 floats, 16 bytes per lane.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    constexpr int EP = 132;
+    float *stage = reinterpret_cast<float *>(&S[0]) + wave * (32 * EP);
+    // A bias row (c0_rs == 0) is the same for every row of the tile: read it once, ahead of the stores.
+    const uint32_t gcol = n0 + wn * 128 + lr * 4;
+    const bool row_bias = g.c0 && g.c0_rs == 0;
+    float bias[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (row_bias) {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            if (gcol + e < g.n) bias[e] = g.c0[(size_t)(gcol + e) * g.c0_cs];
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) stage[(8 * (r >> 2) + 4 * lk + (r & 3)) * EP + j * 32 + lr] = acc[i][j][r];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll 4
+        for (int q = 0; q < 16; q++) {
+            const int row = 2 * q + lk;
+            const f32x4 t = *reinterpret_cast<const f32x4 *>(stage + row * EP + lr * 4);
+            const uint32_t grow = m0 + wm * 64 + i * 32 + row;
+            if (grow >= g.m || gcol >= g.n) continue;
+            float v[4] = {g.alpha * t.x, g.alpha * t.y, g.alpha * t.z, g.alpha * t.w};
+            const bool whole = gcol + 3 < g.n;
+            if (row_bias) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] += g.beta * bias[e];
+            } else if (g.c0) {
+                const float *c0 = g.c0 + (size_t)grow * g.c0_rs + (size_t)gcol * g.c0_cs;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (gcol + e < g.n) v[e] += g.beta * c0[(size_t)e * g.c0_cs];
+            }
+            float *dst = g.c + (size_t)grow * g.ldc + gcol;
+            if (whole && g.c_vec) {
+                const f32x4 o = {v[0], v[1], v[2], v[3]};
+                if (g.c_stream) __builtin_nontemporal_store(o, reinterpret_cast<f32x4 *>(dst));
+                else *reinterpret_cast<f32x4 *>(dst) = o;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (gcol + e < g.n) dst[e] = v[e];
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
+inline size_t round_up(size_t x, size_t q) { return (x + q - 1) / q * q; }
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Geometry of one operand's planes.
+struct PlaneDims {
+    size_t rp, kgs, bytes;
+};
+PlaneDims plane_dims(size_t rows, size_t k) {
+    PlaneDims d;
+    d.rp = round_up(rows, 256);
+    d.kgs = round_up(k, 16) / 8;
+    d.bytes = (size_t)3 * d.kgs * d.rp * 16;
+    return d;
+}
+
+int run_split(DeviceCtx &ctx, void *planes, const float *src, size_t rows, size_t k, size_t ld, bool k_contig) {
+    const PlaneDims d = plane_dims(rows, k);
+    const dim3 grid((unsigned)(d.rp / 64), (unsigned)((d.kgs + 3) / 4));
+    if (k_contig && aligned16(src) && ld % 4 == 0)
+        hipLaunchKernelGGL(split_planes_rows, grid, dim3(256), 0, ctx.stream, src, static_cast<u32x4 *>(planes), (uint32_t)rows,
+                           (uint32_t)k, ld, (uint32_t)d.rp, (uint32_t)d.kgs);
+    else
+        hipLaunchKernelGGL(split_planes, grid, dim3(256), 0, ctx.stream, src, static_cast<u32x4 *>(planes), (uint32_t)rows, (uint32_t)k,
+                           k_contig ? ld : (size_t)1, k_contig ? (size_t)1 : ld, (uint32_t)d.rp, (uint32_t)d.kgs);
+    return ctx.check(hipGetLastError(), "split_planes launch");
+}
+
+// Planes of an operand that lies in a registered constant buffer are made once and kept.
+const void *cached_planes(DeviceCtx &ctx, const float *src, size_t rows, size_t k, size_t ld, bool k_contig, int *rc) {
+    *rc = AHIP_OK;
+    for (const PackedOperand &p : ctx.gemm_packed)
+        if (p.src == src && p.rows == rows && p.k == k && p.ld == ld && p.k_contig == k_contig) return p.planes;
+    const char *lo = reinterpret_cast<const char *>(src);
+    // Last element read: row rows-1 at k-1.
+    const size_t span = k_contig ? ((rows - 1) * ld + k) : ((k - 1) * ld + rows);
+    const ConstantBuffer *owner = nullptr;
+    for (const ConstantBuffer &cb : ctx.gemm_constants) {
+        const char *base = static_cast<const char *>(cb.ptr);
+        if (lo >= base && lo + span * sizeof(float) <= base + cb.bytes) owner = &cb;
+    }
+    if (!owner) return nullptr;
+    const PlaneDims d = plane_dims(rows, k);
+    void *planes = nullptr;
+    if (hipMalloc(&planes, d.bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        *rc = ctx.fail(AHIP_ERR_OOM, "gemm: no memory for the bf16 planes of a constant operand");
+        return nullptr;
+    }
+    *rc = run_split(ctx, planes, src, rows, k, ld, k_contig);
+    if (*rc) {
+        (void)hipFree(planes);
+        return nullptr;
+    }
+    PackedOperand p;
+    p.owner = owner->ptr;
+    p.src = src;
+    p.rows = rows;
+    p.k = k;
+    p.ld = ld;
+    p.k_contig = k_contig;
+    p.planes = planes;
+    p.bytes = d.bytes;
+    ctx.gemm_packed.push_back(p);
+    return planes;
+}
+
+int ensure_workspace(DeviceCtx &ctx, size_t bytes) {
+    if (bytes <= ctx.gemm_ws_bytes) return AHIP_OK;
+    // Work already queued may still read the old buffer.
+    int rc = ctx.check(hipStreamSynchronize(ctx.stream), "hipStreamSynchronize");
+    if (rc) return rc;
+    if (ctx.gemm_ws) (void)hipFree(ctx.gemm_ws);
+    ctx.gemm_ws = nullptr;
+    ctx.gemm_ws_bytes = 0;
+    ctx.gemm_ws_generation++;
+    void *p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return ctx.fail(AHIP_ERR_OOM, "gemm: no memory for the bf16 planes of the operands");
+    }
+    ctx.gemm_ws = p;
+    ctx.gemm_ws_bytes = bytes;
+    return AHIP_OK;
+}
+
+}  // namespace
+
+bool gemm_split_worthwhile(size_t m, size_t n, size_t k) {
+    if (m < 1024 || n < 256 || k < 128) return false;
+    const double useful = (double)m * (double)n / ((double)round_up(m, TM) * (double)round_up(n, TN));
+    return useful >= 0.8 && (double)m * (double)n * (double)k >= 2147483648.0;
+}
+
+int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t m, size_t n, size_t k,
+                      int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t c0_row_stride, size_t c0_col_stride,
+                      float alpha, float beta) {
+    if (m == 0 || n == 0) return AHIP_OK;
+    if (!c || !a || !b || k == 0) return ctx.fail(AHIP_ERR_ARG, "gemm (bf16 x 3): null pointer or k = 0");
+    const size_t lim = (size_t)1 << 31;
+    if (m >= lim - 256 || n >= lim - 256 || k >= lim - 16 || lda >= lim || ldb >= lim || ldc >= lim || c0_row_stride >= lim ||
+        c0_col_stride >= lim)
+        return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm (bf16 x 3): extent above 2^31");
+    const PlaneDims da = plane_dims(m, k), db = plane_dims(n, k);
+    const size_t tiles_n = db.rp / TN, tiles = tiles_n * (da.rp / TM);
+    if (tiles >= lim / 8 || (da.kgs + 3) / 4 > 65535) return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm (bf16 x 3): too many tiles");
+    const bool a_kc = !trans_a, b_kc = trans_b != 0;
+    int rc = AHIP_OK;
+    const void *pa = cached_planes(ctx, a, m, k, lda, a_kc, &rc);
+    if (rc) return rc;
+    const void *pb = cached_planes(ctx, b, n, k, ldb, b_kc, &rc);
+    if (rc) return rc;
+    const size_t a_off = 0, b_off = pa ? 0 : round_up(da.bytes, 256);
+    const size_t need = (pa ? 0 : round_up(da.bytes, 256)) + (pb ? 0 : db.bytes);
+    if (need) {
+        rc = ensure_workspace(ctx, need);
+        if (rc) return rc;
+    }
+    if (!pa) {
+        void *p = static_cast<char *>(ctx.gemm_ws) + a_off;
+        rc = run_split(ctx, p, a, m, k, lda, a_kc);
+        if (rc) return rc;
+        pa = p;
+    }
+    if (!pb) {
+        void *p = static_cast<char *>(ctx.gemm_ws) + b_off;
+        rc = run_split(ctx, p, b, n, k, ldb, b_kc);
+        if (rc) return rc;
+        pb = p;
+    }
+    SplitGemmArgs g;
+    g.ap = static_cast<const u32x4 *>(pa);
+    g.bp = static_cast<const u32x4 *>(pb);
+    g.c = c;
+    g.c0 = (c0 && beta != 0.0f) ? c0 : nullptr;
+    g.m = (uint32_t)m;
+    g.n = (uint32_t)n;
+    g.mp = (uint32_t)da.rp;
+    g.np = (uint32_t)db.rp;
+    g.kgs = (uint32_t)da.kgs;
+    g.ldc = (uint32_t)ldc;
+    g.c0_rs = (uint32_t)c0_row_stride;
+    g.c0_cs = (uint32_t)c0_col_stride;
+    g.alpha = alpha;
+    g.beta = beta;
+    g.tiles_n = (uint32_t)tiles_n;
+    g.tiles = (uint32_t)tiles;
+    g.chunk = (uint32_t)((tiles + 7) / 8);
+    g.c_vec = aligned16(c) && ldc % 4 == 0;
+    g.c_stream = ctx.streaming(m * n * sizeof(float));
+    hipLaunchKernelGGL(gemm_bf16x3, dim3(g.chunk * 8), dim3(THREADS), 0, ctx.stream, g);
+    return ctx.check(hipGetLastError(), "gemm (bf16 x 3) launch");
+}
+
+int gemm_register_constant(DeviceCtx &ctx, const void *ptr, size_t bytes) {
+    if (!ptr || !bytes) return ctx.fail(AHIP_ERR_ARG, "gemm_register_constant: null buffer");
+    for (ConstantBuffer &cb : ctx.gemm_constants)
+        if (cb.ptr == ptr) {
+            cb.bytes = bytes;
+            return AHIP_OK;
+        }
+    ctx.gemm_constants.push_back(ConstantBuffer{ptr, bytes});
+    return AHIP_OK;
+}
+
+int gemm_unregister_constant(DeviceCtx &ctx, const void *ptr) {
+    auto it = std::find_if(ctx.gemm_constants.begin(), ctx.gemm_constants.end(), [&](const ConstantBuffer &cb) { return cb.ptr == ptr; });
+    if (it == ctx.gemm_constants.end()) return AHIP_OK;
+    ctx.gemm_constants.erase(it);
+    bool any = false;
+    for (const PackedOperand &p : ctx.gemm_packed) any = any || p.owner == ptr;
+    if (!any) return AHIP_OK;
+    // Kernels that read the planes may still be queued.
+    int rc = ctx.check(hipStreamSynchronize(ctx.stream), "hipStreamSynchronize");
+    for (size_t i = 0; i < ctx.gemm_packed.size();) {
+        if (ctx.gemm_packed[i].owner == ptr) {
+            (void)hipFree(ctx.gemm_packed[i].planes);
+            ctx.gemm_packed.erase(ctx.gemm_packed.begin() + (long)i);
+        } else {
+            i++;
+        }
+    }
+    return rc;
+}
+
+void gemm_release_all(DeviceCtx &ctx) {
+    for (PackedOperand &p : ctx.gemm_packed) (void)hipFree(p.planes);
+    ctx.gemm_packed.clear();
+    ctx.gemm_constants.clear();
+    if (ctx.gemm_ws) (void)hipFree(ctx.gemm_ws);
+    ctx.gemm_ws = nullptr;
+    ctx.gemm_ws_bytes = 0;
+}
+
+}  // namespace altius

@@ -218,6 +218,9 @@ int launch_gemm(DeviceCtx &ctx, float *c, const float *a, const float *b, const 
                 float beta) {
     if (batch == 0 || m == 0 || n == 0) return AHIP_OK;
     if (!c || (k && (!a || !b))) return ctx.fail(AHIP_ERR_ARG, "gemm: null pointer");
+    if (batch == 1 && k > 0 &&
+        (ctx.gemm_algorithm == AHIP_GEMM_BF16X3 || (ctx.gemm_algorithm == AHIP_GEMM_AUTO && gemm_split_worthwhile(m, n, k))))
+        return launch_gemm_split(ctx, c, a, b, c0, m, n, k, trans_a, trans_b, lda, ldb, ldc, c0_row_stride, c0_col_stride, alpha, beta);
     const size_t lim = (size_t)1 << 31;
     if (m >= lim || n >= lim || k >= lim || lda >= lim || ldb >= lim || ldc >= lim || m * ldc >= ((size_t)1 << 40))
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm: extent above 2^31");

@@ -128,6 +128,12 @@ std::unique_ptr<HipSession> HipSessionBuilder::build(SessionError *err) {
         fail_code(err, rc, derr);
         return nullptr;
     }
+    if (gemm_algorithm_ != AHIP_GEMM_AUTO && gemm_algorithm_ != AHIP_GEMM_FP32 && gemm_algorithm_ != AHIP_GEMM_BF16X3) {
+        destroy_device_ctx(&s->ctx_);
+        fail(err, SessionError::Argument, "unknown GEMM algorithm");
+        return nullptr;
+    }
+    s->ctx_.gemm_algorithm = gemm_algorithm_;
     s->pool_.reset(new BufferPool(&s->ctx_));
     if (hipEventCreate(&s->span_begin_) != hipSuccess || hipEventCreate(&s->span_end_) != hipSuccess) {
         fail(err, SessionError::Hip, "hipEventCreate failed");
@@ -144,6 +150,7 @@ std::unique_ptr<HipSession> HipSessionBuilder::build(SessionError *err) {
         }
         DeviceTensor d;
         if (!s->upload(t, &d, err)) return nullptr;
+        if (t.elem_ty() == TensorElemType::F32 && d.ptr && d.nbytes()) gemm_register_constant(s->ctx_, d.ptr, d.nbytes());
         s->inits_[kv.first] = std::move(d);
     }
     rc = s->ctx_.check(hipStreamSynchronize(s->ctx_.stream), "hipStreamSynchronize(build)");
@@ -239,6 +246,10 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
         if (!check_input(i, inputs[i].elem_ty(), inputs[i].dims(), err)) return false;
 
     if (graph_replay_) {
+        if (seen_ws_generation_ != ctx_.gemm_ws_generation) {  // the GEMM workspace moved: recorded launches point at the old one
+            drop_graphs();
+            seen_ws_generation_ = ctx_.gemm_ws_generation;
+        }
         std::string key;
         for (size_t i = 0; i < g.inputs.size(); i++)
             key += std::to_string((int)inputs[i].elem_ty()) + inputs[i].dims().to_string() + ";";

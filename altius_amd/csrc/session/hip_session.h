@@ -169,6 +169,7 @@ private:
     std::map<std::string, CapturedRun> graphs_;
     std::map<std::string, int> eager_runs_;  // per input signature: eager runs so far (the pool is warm after one)
     size_t graph_replays_ = 0;
+    uint64_t seen_ws_generation_ = 0;  // recorded launches hold the GEMM workspace's address
 };
 
 class HipSessionBuilder {
@@ -191,6 +192,13 @@ public:
         graph_replay_ = enable;
         return *this;
     }
+    // Not in the reference: the kernel large single-batch MatMul / Gemm products take (AHIP_GEMM_AUTO, the
+    // default, AHIP_GEMM_FP32 or AHIP_GEMM_BF16X3).  Float initializers are declared constant to the
+    // GEMM, so a weight operand's bf16 planes are made on its first use and kept.
+    HipSessionBuilder &with_gemm_algorithm(int algorithm) {
+        gemm_algorithm_ = algorithm;
+        return *this;
+    }
     // Not in the reference: which GPU to run on (default 0).
     HipSessionBuilder &with_device(int device) {
         device_ = device;
@@ -206,6 +214,7 @@ private:
     bool enable_profiling_ = false;
     int device_ = 0;
     bool graph_replay_ = false;
+    int gemm_algorithm_ = AHIP_GEMM_AUTO;
 };
 
 }  // namespace altius

@@ -15,6 +15,7 @@ ADD, SUB, MUL, DIV, POW = 0, 1, 2, 3, 4
 SQRT, ERF, GELU, SIGMOID, HARDSIGMOID, RELU, TANH, LEAKYRELU, EXP, ROUND, CLIP = range(11)
 REDUCE_MEAN, REDUCE_MAX, REDUCE_SUM = 0, 1, 2
 BOOL, F32, I32, I64 = 0, 1, 2, 3
+GEMM_AUTO, GEMM_FP32, GEMM_BF16X3 = 0, 1, 2
 _ELEM_OF = {np.dtype(np.bool_): BOOL, np.dtype(np.float32): F32, np.dtype(np.int32): I32, np.dtype(np.int64): I64}
 
 
@@ -409,6 +410,17 @@ class Context:
         ldc = ldc if ldc is not None else n
         check(self.L.ahip_gemm(self.handle, c_ptr, a_ptr, b_ptr, c0_ptr, batch, m, n, k, int(trans_a), int(trans_b), lda,
                                ldb, ldc, a_bs, b_bs, c_bs, c0_rs, c0_cs, alpha, beta), self.handle)
+
+    def gemm_set_algorithm(self, algorithm):
+        """GEMM_AUTO / GEMM_FP32 / GEMM_BF16X3: the kernel single-batch products take."""
+        check(self.L.ahip_gemm_set_algorithm(self.handle, int(algorithm)), self.handle)
+
+    def gemm_register_constant(self, buf):
+        """Declares a device buffer immutable: the split GEMM keeps the planes of operands inside it."""
+        check(self.L.ahip_gemm_register_constant(self.handle, buf.ptr, buf.nbytes), self.handle)
+
+    def gemm_unregister_constant(self, buf):
+        check(self.L.ahip_gemm_unregister_constant(self.handle, buf.ptr), self.handle)
 
     def matmul(self, a, b):
         """numpy.matmul semantics for operands of rank >= 2 (batch axes broadcast)."""

@@ -153,6 +153,11 @@ class HipSessionBuilder:
         check(self.L.ahip_session_builder_with_graph_replay(self.handle, int(bool(enable))))
         return self
 
+    def with_gemm_algorithm(self, algorithm):
+        """device.GEMM_AUTO (default) / GEMM_FP32 / GEMM_BF16X3 for the large single-batch products."""
+        check(self.L.ahip_session_builder_with_gemm_algorithm(self.handle, int(algorithm)))
+        return self
+
     def with_device(self, device):
         check(self.L.ahip_session_builder_with_device(self.handle, device))
         return self

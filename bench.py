@@ -272,7 +272,7 @@ def session_table(synth, dev_ctx):
 def vit_table(batch, layers=12):
     """Whole-model device time (kernels only, input already uploaded by run()) of a ViT-B/16-shaped encoder for
     three versions of the same graph, with the per-operator split of each from a profiled run."""
-    from altius_amd import graphs
+    from altius_amd import device as D, graphs
     from altius_amd.graph import Tensor
     from altius_amd.session import HipSessionBuilder
 
@@ -286,16 +286,18 @@ def vit_table(batch, layers=12):
     ours = ref.clone()
     ours.fuse_softmax_prologue(), ours.fuse_matmul_bias(), ours.fuse_transpose_matmul(), ours.fuse_elemwise_ops(extended=True)
     versions.append(("+ softmax prologue, matmul bias / transposes, element-wise chains", ours))
+    versions.append(("+ large products on the bf16 matrix cores (three planes per operand)", ours))
     rows = []
-    for name, model in versions:
-        sess = HipSessionBuilder(model).build()
+    for i, (name, model) in enumerate(versions):
+        algo = D.GEMM_AUTO if i == 3 else D.GEMM_FP32
+        sess = HipSessionBuilder(model).with_gemm_algorithm(algo).build()
         best = float("inf")
         for _ in range(4):
             outs = sess.run([x], copy=False)
             best = min(best, sess.last_device_ms())
             del outs
         sess.close()
-        prof = HipSessionBuilder(model).with_profiling_enabled(True).build()
+        prof = HipSessionBuilder(model).with_gemm_algorithm(algo).with_profiling_enabled(True).build()
         for _ in range(2):
             outs = prof.run([x], copy=False)
             del outs
@@ -337,20 +339,31 @@ def build_next_rows(ctx, D, batch=256):
     rows.append(("Gather [50257,768] x %d ids" % S, 2 * S * H * 4 + S * 8, 0,
                  lambda: check(L.ahip_gather(h, out.ptr, table.ptr, ids.ptr, 8, 4, 1, V, S, H), h)))
 
-    def gemm(name, b, m, n_, k, a_bs, b_bs):
-        a = ctx.alloc((b if a_bs else 1) * m * k * 4)
-        w = ctx.alloc((b if b_bs else 1) * k * n_ * 4)
+    rng = np.random.default_rng(5)
+
+    def gemm(name, b, m, n_, k, a_bs, b_bs, algorithms=(("fp32 MFMA", D.GEMM_FP32),)):
+        # random operands: constant ones toggle fewer bits in the matrix cores and run at a higher clock
+        a = ctx.upload(rng.standard_normal(((b if a_bs else 1) * m, k), dtype=np.float32))
+        w = ctx.upload(rng.standard_normal(((b if b_bs else 1) * k, n_), dtype=np.float32) * np.float32(0.03))
         c = ctx.alloc(b * m * n_ * 4)
-        ctx.memset(a, 0x3c)
-        ctx.memset(w, 0x3c)
         nbytes = 4 * ((b if a_bs else 1) * m * k + (b if b_bs else 1) * k * n_ + b * m * n_)
-        rows.append((name, nbytes, 2.0 * b * m * n_ * k,
-                     lambda: ctx.gemm_raw(c.ptr, a.ptr, w.ptr, None, b, m, n_, k, a_bs=a_bs, b_bs=b_bs, c_bs=m * n_)))
+        for label, algo in algorithms:
+            if algo == D.GEMM_BF16X3:
+                ctx.gemm_register_constant(w)  # as a session does for its weights: their planes are made once
+
+            def launch(algo=algo):
+                ctx.gemm_set_algorithm(algo)
+                ctx.gemm_raw(c.ptr, a.ptr, w.ptr, None, b, m, n_, k, a_bs=a_bs, b_bs=b_bs, c_bs=m * n_)
+                ctx.gemm_set_algorithm(D.GEMM_AUTO)
+
+            rows.append(("%s (%s)" % (name, label), nbytes, 2.0 * b * m * n_ * k, launch))
 
     M = batch * T
-    gemm("MatMul qkv [%d,768]x[768,2304]" % M, 1, M, 3 * H, H, 0, 0)
-    gemm("MatMul fc1 [%d,768]x[768,3072]" % M, 1, M, 4 * H, H, 0, 0)
-    gemm("MatMul fc2 [%d,3072]x[3072,768]" % M, 1, M, H, 4 * H, 0, 0)
+    both = (("fp32 MFMA", D.GEMM_FP32), ("bf16 x 3 incl. split of A", D.GEMM_BF16X3))
+    gemm("MatMul qkv [%d,768]x[768,2304]" % M, 1, M, 3 * H, H, 0, 0, both)
+    gemm("MatMul proj [%d,768]x[768,768]" % M, 1, M, H, H, 0, 0, both)
+    gemm("MatMul fc1 [%d,768]x[768,3072]" % M, 1, M, 4 * H, H, 0, 0, both)
+    gemm("MatMul fc2 [%d,3072]x[3072,768]" % M, 1, M, H, 4 * H, 0, 0, both)
     gemm("MatMul QK^T %d x [197,64]x[64,197]" % (batch * NH), batch * NH, T, T, DH, T * DH, DH * T)
     gemm("MatMul PV %d x [197,197]x[197,64]" % (batch * NH), batch * NH, T, DH, T, T * T, T * DH)
     return rows
@@ -572,10 +585,12 @@ def main():
             ms = time_kernel(ctx, o, max(10, args.kernel_iters // 2), 3)
             row = {"kernel": name, "us": round(ms * 1e3, 1), "bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1)}
             if flops:
-                row.update({"bound": "mfma", "TFLOPs": round(flops / ms / 1e9, 1),
-                            "frac_of_peak": round(flops / ms / 1e9 / MFMA_F32_PEAK, 3)})
-                log("%-48s %10.1f us %8.1f TFLOP/s (%4.1f %% of %.1f)" % (name, ms * 1e3, flops / ms / 1e9,
-                                                                         100 * flops / ms / 1e9 / MFMA_F32_PEAK, MFMA_F32_PEAK))
+                # six bf16 MFMAs per fp32 product: the bf16 peak (2500 TFLOP/s dense) over six
+                peak = 2500.0 / 6 if "bf16 x 3" in name else MFMA_F32_PEAK
+                row.update({"bound": "mfma", "TFLOPs": round(flops / ms / 1e9, 1), "peak_TFLOPs": round(peak, 1),
+                            "frac_of_peak": round(flops / ms / 1e9 / peak, 3)})
+                log("%-64s %10.1f us %8.1f TFLOP/s (%4.1f %% of %.1f)" % (name, ms * 1e3, flops / ms / 1e9,
+                                                                         100 * flops / ms / 1e9 / peak, peak))
             else:
                 row.update({"bound": "hbm", "frac_of_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 3)})
                 log("%-48s %10.1f us %8.1f GB/s    (%4.1f %% of 8000)" % (name, ms * 1e3, nbytes / ms / 1e6,

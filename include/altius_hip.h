@@ -259,6 +259,24 @@ int ahip_gemm(ahip_ctx *ctx, float *c, const float *a, const float *b, const flo
               size_t b_batch_stride, size_t c_batch_stride, size_t c0_row_stride, size_t c0_col_stride, float alpha,
               float beta);
 
+/* Which kernel ahip_gemm (and the MatMul / Gemm / Conv2d operators of a session on this context) uses
+ * for a single-batch product.  AHIP_GEMM_FP32: v_mfma_f32_32x32x2_f32 on the operands as they are.
+ * AHIP_GEMM_BF16X3: every operand value is split exactly into three bf16 numbers and six bf16 MFMAs per
+ * product accumulate in fp32 (the terms dropped are below 2^-23 of each product); measured against
+ * float64 it is as close as a chain of fp32 multiply-adds, and about 1.6 times faster on large shapes.
+ * AHIP_GEMM_AUTO (the default): BF16X3 for large products whose C fills whole 256 x 256 tiles, FP32
+ * otherwise.  The reference has one sgemm (gemm.rs:3-52) and no such switch. */
+#define AHIP_GEMM_AUTO 0
+#define AHIP_GEMM_FP32 1
+#define AHIP_GEMM_BF16X3 2
+int ahip_gemm_set_algorithm(ahip_ctx *ctx, int algorithm);
+/* Declares the device buffer [ptr, ptr + bytes) immutable (model weights) until it is unregistered:
+ * AHIP_GEMM_BF16X3 then splits an operand that lies inside it once and keeps the planes (1.5 times the
+ * operand's size) instead of splitting it on every call.  Unregister before freeing or rewriting the
+ * buffer.  No counterpart in the reference, whose sgemm reads fp32 operands directly. */
+int ahip_gemm_register_constant(ahip_ctx *ctx, const void *ptr, size_t bytes);
+int ahip_gemm_unregister_constant(ahip_ctx *ctx, const void *ptr);
+
 /* Conv2d on NCHW (crates/session_interpreter/src/conv2d.rs:26-211): im2col into `col`
  * (scratch of batch*c*kh*kw*oh*ow floats, the reference's layout [b][c][kh][kw][oh][ow]) and one
  * batched GEMM per group.  w is [oc, c/group, kh, kw]; bias ([oc]) may be NULL.  oh / ow are the
@@ -483,6 +501,11 @@ int ahip_session_builder_with_device(ahip_session_builder *builder, int device);
  * run instead of one per node).  Results are those of the node-by-node run.  Graphs whose shapes
  * or operands need the host during the run, and profiled sessions, keep running node by node. */
 int ahip_session_builder_with_graph_replay(ahip_session_builder *builder, int enable);
+/* Not in the reference: the kernel the session's large single-batch MatMul / Gemm products take
+ * (AHIP_GEMM_AUTO, the default, AHIP_GEMM_FP32 or AHIP_GEMM_BF16X3; see ahip_gemm_set_algorithm).  The
+ * session declares its float initializers constant to the GEMM, so the bf16 planes of a weight are
+ * made on its first use and kept until the session is freed. */
+int ahip_session_builder_with_gemm_algorithm(ahip_session_builder *builder, int algorithm);
 /* build(): shape inference (AHIP_ERR_SHAPE on failure), execution plan, device context,
  * upload of the initializers.  The builder stays valid and must still be freed. */
 int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **session);
