@@ -89,6 +89,8 @@ def _declare(L):
                          c_float])
     f("ahip_gemm", [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p] + [c_size_t] * 4 + [c_int, c_int] + [c_size_t] * 8
       + [c_float, c_float])
+    f("ahip_gemm_batch2", [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p] + [c_size_t] * 5 + [c_int, c_int] + [c_size_t] * 3
+      + [P(c_size_t)] * 3 + [c_size_t, c_size_t, c_float, c_float])
     f("ahip_gemm_set_algorithm", [c_void_p, c_int])
     f("ahip_gemm_register_constant", [c_void_p, c_void_p, c_size_t])
     f("ahip_gemm_unregister_constant", [c_void_p, c_void_p])
@@ -189,6 +191,8 @@ def _declare_graph(L):
     f("ahip_session_builder_with_device", [c_void_p, c_int])
     f("ahip_session_builder_with_graph_replay", [c_void_p, c_int])
     f("ahip_session_builder_with_gemm_algorithm", [c_void_p, c_int])
+    f("ahip_session_builder_with_strided_views", [c_void_p, c_int])
+    f("ahip_session_copies_avoided", [c_void_p, P(c_size_t)])
     f("ahip_session_graph_replays", [c_void_p, P(c_size_t)])
     f("ahip_session_builder_build", [c_void_p, P(c_void_p)])
     f("ahip_session_free", [c_void_p], None)

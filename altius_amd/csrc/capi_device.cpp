@@ -381,6 +381,17 @@ int ahip_gemm(ahip_ctx *ctx, float *c, const float *a, const float *b, const flo
                                b_batch_stride, c_batch_stride, c0_row_stride, c0_col_stride, alpha, beta);
 }
 
+int ahip_gemm_batch2(ahip_ctx *ctx, float *c, const float *a, const float *b, const float *c0, size_t batch_outer,
+                     size_t batch_inner, size_t m, size_t n, size_t k, int trans_a, int trans_b, size_t lda, size_t ldb,
+                     size_t ldc, const size_t a_batch_strides[2], const size_t b_batch_strides[2],
+                     const size_t c_batch_strides[2], size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta) {
+    REQUIRE_CTX(ctx, "ahip_gemm_batch2");
+    if (!a_batch_strides || !b_batch_strides || !c_batch_strides) return ctx->d.fail(AHIP_ERR_ARG, "ahip_gemm_batch2: null strides");
+    if (batch_inner == 0) return ctx->d.fail(AHIP_ERR_ARG, "ahip_gemm_batch2: batch_inner is 0");
+    return altius::launch_gemm_batch2(ctx->d, c, a, b, c0, batch_outer, batch_inner, m, n, k, trans_a, trans_b, lda, ldb, ldc,
+                                      a_batch_strides, b_batch_strides, c_batch_strides, c0_row_stride, c0_col_stride, alpha, beta);
+}
+
 int ahip_gemm_set_algorithm(ahip_ctx *ctx, int algorithm) {
     REQUIRE_CTX(ctx, "ahip_gemm_set_algorithm");
     if (algorithm != AHIP_GEMM_AUTO && algorithm != AHIP_GEMM_FP32 && algorithm != AHIP_GEMM_BF16X3)

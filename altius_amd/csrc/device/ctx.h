@@ -120,6 +120,14 @@ int launch_gemm(DeviceCtx &ctx, float *c, const float *a, const float *b, const 
                 size_t b_batch_stride, size_t c_batch_stride, size_t c0_row_stride, size_t c0_col_stride, float alpha,
                 float beta);
 
+// The same with the batch index split in two, z = (z / batch_inner, z % batch_inner), each part with its own
+// stride per operand: operands that are strided views of a larger tensor (the heads of a [b, t, h, d] tensor
+// read in place as b x h matrices of t x d with row pitch h * d) need no copy.
+int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t batch_outer,
+                       size_t batch_inner, size_t m, size_t n, size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc,
+                       const size_t a_batch_strides[2], const size_t b_batch_strides[2], const size_t c_batch_strides[2],
+                       size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta);
+
 // The same product for one batch through three bf16 planes per operand and six bf16 MFMAs per fp32
 // product (gemm_split.hip): as accurate as an fp32 multiply-add chain, about 1.6 times the fp32 matrix
 // cores' rate on large shapes.  launch_gemm takes this route by itself according to ctx.gemm_algorithm.

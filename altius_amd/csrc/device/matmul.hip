@@ -38,7 +38,10 @@ struct GemmArgs {
     uint32_t ldc;
     // C0 (Gemm's third input) is read as c0[i * c0_rs + j * c0_cs]; either stride may be 0.
     uint32_t c0_rs, c0_cs;
-    uint64_t a_bs, b_bs, c_bs;  // batch strides in elements (0 = shared by every batch)
+    // Batch z = blockIdx.z is (z / batch_inner, z % batch_inner); operand X starts at
+    // x + (z / batch_inner) * x_bs + (z % batch_inner) * x_bs2 (strides in elements, 0 = shared).
+    uint64_t a_bs, b_bs, c_bs, a_bs2, b_bs2, c_bs2;
+    uint32_t batch_inner;
     float alpha, beta;
     int a_vec, b_vec;  // 16-byte loads are legal for this operand (alignment of base, strides, batch stride)
 };
@@ -125,8 +128,9 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_mfma(GemmArgs g) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = TN == 128 ? wave >> 1 : wave, wn = TN == 128 ? wave & 1 : 0;
     const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * TN;
-    const float *a = g.a + (size_t)blockIdx.z * g.a_bs;
-    const float *b = g.b + (size_t)blockIdx.z * g.b_bs;
+    const uint32_t zo = blockIdx.z / g.batch_inner, zi = blockIdx.z % g.batch_inner;
+    const float *a = g.a + (size_t)zo * g.a_bs + (size_t)zi * g.a_bs2;
+    const float *b = g.b + (size_t)zo * g.b_bs + (size_t)zi * g.b_bs2;
     // Strides of the tile's mn axis and k axis for each operand.
     const uint32_t a_smn = g.a_rs, a_sk = g.a_cs, b_smn = g.b_cs, b_sk = g.b_rs;
 
@@ -190,7 +194,7 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_mfma(GemmArgs g) {
     else main_loop(std::false_type{});
 
     // Accumulator r of lane l is C[8 * (r / 4) + 4 * (l / 32) + r % 4][l % 32] of its 32 x 32 tile.
-    float *c = g.c + (size_t)blockIdx.z * g.c_bs;
+    float *c = g.c + (size_t)zo * g.c_bs + (size_t)zi * g.c_bs2;
 #pragma unroll
     for (int i = 0; i < WI; i++)
 #pragma unroll
@@ -216,6 +220,16 @@ int launch_gemm(DeviceCtx &ctx, float *c, const float *a, const float *b, const 
                 size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t a_batch_stride,
                 size_t b_batch_stride, size_t c_batch_stride, size_t c0_row_stride, size_t c0_col_stride, float alpha,
                 float beta) {
+    const size_t a_bs[2] = {a_batch_stride, 0}, b_bs[2] = {b_batch_stride, 0}, c_bs[2] = {c_batch_stride, 0};
+    return launch_gemm_batch2(ctx, c, a, b, c0, batch, 1, m, n, k, trans_a, trans_b, lda, ldb, ldc, a_bs, b_bs, c_bs, c0_row_stride,
+                              c0_col_stride, alpha, beta);
+}
+
+int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t batch_outer,
+                       size_t batch_inner, size_t m, size_t n, size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc,
+                       const size_t a_batch_strides[2], const size_t b_batch_strides[2], const size_t c_batch_strides[2],
+                       size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta) {
+    const size_t batch = batch_outer * batch_inner;
     if (batch == 0 || m == 0 || n == 0) return AHIP_OK;
     if (!c || (k && (!a || !b))) return ctx.fail(AHIP_ERR_ARG, "gemm: null pointer");
     if (batch == 1 && k > 0 &&
@@ -247,13 +261,17 @@ int launch_gemm(DeviceCtx &ctx, float *c, const float *a, const float *b, const 
     g.ldc = (uint32_t)ldc;
     g.c0_rs = (uint32_t)c0_row_stride;
     g.c0_cs = (uint32_t)c0_col_stride;
-    g.a_bs = a_batch_stride;
-    g.b_bs = b_batch_stride;
-    g.c_bs = c_batch_stride;
+    g.a_bs = a_batch_strides[0];
+    g.b_bs = b_batch_strides[0];
+    g.c_bs = c_batch_strides[0];
+    g.a_bs2 = a_batch_strides[1];
+    g.b_bs2 = b_batch_strides[1];
+    g.c_bs2 = c_batch_strides[1];
+    g.batch_inner = (uint32_t)batch_inner;
     g.alpha = alpha;
     g.beta = beta;
-    g.a_vec = aligned16(a) && lda % 4 == 0 && a_batch_stride % 4 == 0;
-    g.b_vec = aligned16(b) && ldb % 4 == 0 && b_batch_stride % 4 == 0;
+    g.a_vec = aligned16(a) && lda % 4 == 0 && a_batch_strides[0] % 4 == 0 && a_batch_strides[1] % 4 == 0;
+    g.b_vec = aligned16(b) && ldb % 4 == 0 && b_batch_strides[0] % 4 == 0 && b_batch_strides[1] % 4 == 0;
     const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch);
     const bool a_kc = !trans_a, b_kc = trans_b != 0;
 #define GEMM(AK, BK_, TN_) hipLaunchKernelGGL((gemm_f32_mfma<AK, BK_, TN_>), grid, dim3(THREADS), 0, ctx.stream, g)

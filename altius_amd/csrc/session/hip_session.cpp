@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <chrono>
+#include <functional>
 #include <limits>
 
 #include "../device/host_pool.h"
@@ -121,6 +122,7 @@ std::unique_ptr<HipSession> HipSessionBuilder::build(SessionError *err) {
         return nullptr;
     }
     s->plan_ = create_execution_plan(s->model_);
+    if (strided_views_) s->plan_views();
 
     std::string derr;
     int rc = create_device_ctx(device_, nullptr, true, &s->ctx_, &derr);
@@ -267,6 +269,7 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
     }
 
     std::map<ValueId, DeviceTensor> values;
+    copies_avoided_ = 0;
     std::vector<hipEvent_t> events;
     // Nothing may still read a block when it goes back to the pool for another run, and input
     // tensors must outlive their uploads: every exit path synchronises first.
@@ -317,6 +320,7 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
     for (ValueId v : g.outputs) {
         const DeviceTensor *d = nullptr;
         auto it = values.find(v);
+        if (it != values.end() && !it->second.strides.empty() && !materialize(&it->second, err)) return finish(false);  // never planned; dense for the caller
         if (it != values.end()) d = &it->second;
         else {
             auto ii = inits_.find(v);
@@ -366,6 +370,7 @@ bool HipSession::run_device(const std::vector<DeviceTensor> &inputs, std::vector
     if (hipSetDevice(ctx_.device) != hipSuccess) return fail(err, SessionError::Hip, "hipSetDevice failed");
 
     std::map<ValueId, DeviceTensor> values;
+    copies_avoided_ = 0;
     for (size_t i = 0; i < g.inputs.size(); i++) {
         if (!inputs[i].ptr && inputs[i].nbytes())
             return fail(err, SessionError::Argument, "run_device: input " + std::to_string(i) + " has no device pointer");
@@ -388,6 +393,7 @@ bool HipSession::run_device(const std::vector<DeviceTensor> &inputs, std::vector
     for (ValueId v : g.outputs) {
         const DeviceTensor *d = nullptr;
         auto it = values.find(v);
+        if (it != values.end() && !it->second.strides.empty() && !materialize(&it->second, err)) return false;  // never planned; dense for the caller
         if (it != values.end()) d = &it->second;
         else {
             auto ii = inits_.find(v);
@@ -436,6 +442,7 @@ bool HipSession::try_capture(const std::string &key, const std::vector<Tensor> &
     const Graph &g = model_.graph;
     CapturedRun run;
     std::map<ValueId, DeviceTensor> values;
+    copies_avoided_ = 0;
     for (size_t i = 0; i < g.inputs.size(); i++) {
         DeviceTensor d;
         if (!allocate(TypedFixedShape{inputs[i].dims(), inputs[i].elem_ty()}, &d, err)) return false;
@@ -468,6 +475,7 @@ bool HipSession::try_capture(const std::string &key, const std::vector<Tensor> &
     if (ok && end == hipSuccess && graph) {
         for (ValueId v : g.outputs) {
             auto it = values.find(v);
+            if (it != values.end() && !it->second.strides.empty() && !materialize(&it->second, err)) ok = false;
             const DeviceTensor *d = it != values.end() ? &it->second : nullptr;
             if (!d) {
                 auto ii = inits_.find(v);
@@ -543,6 +551,71 @@ bool is_alias_op(OpKind k) {
     return k == OpKind::Reshape || k == OpKind::Flatten || k == OpKind::Squeeze || k == OpKind::Unsqueeze;
 }
 
+// Operators that read a strided view in place (or pass it on as another view).
+bool reads_views(OpKind k) { return is_alias_op(k) || k == OpKind::MatMul || k == OpKind::Transpose || k == OpKind::Split; }
+
+std::vector<int64_t> dense_strides(const FixedDimensions &dims) {
+    std::vector<int64_t> s(dims.len());
+    int64_t acc = 1;
+    for (size_t i = dims.len(); i-- > 0;) {
+        s[i] = acc;
+        acc *= (int64_t)dims[i];
+    }
+    return s;
+}
+
+std::vector<int64_t> strides_of(const DeviceTensor &t) { return t.strides.empty() ? dense_strides(t.dims) : t.strides; }
+
+// Axes of extent 1 may carry any stride.
+bool is_dense(const FixedDimensions &dims, const std::vector<int64_t> &strides) {
+    const std::vector<int64_t> d = dense_strides(dims);
+    for (size_t i = 0; i < dims.len(); i++)
+        if (dims[i] != 1 && strides[i] != d[i]) return false;
+    return true;
+}
+
+// Strides of the same elements under new_dims, if they exist without a copy (each run of new axes
+// must tile a run of old axes that is itself uniformly strided).
+bool reshape_strides(const FixedDimensions &old_dims, const std::vector<int64_t> &old_strides, const FixedDimensions &new_dims,
+                     std::vector<int64_t> *out) {
+    std::vector<size_t> od;
+    std::vector<int64_t> os;
+    for (size_t i = 0; i < old_dims.len(); i++)
+        if (old_dims[i] != 1) od.push_back(old_dims[i]), os.push_back(old_strides[i]);
+    out->assign(new_dims.len(), 0);
+    size_t oi = 0, ni = 0;
+    while (ni < new_dims.len() && oi < od.size()) {
+        if (new_dims[ni] == 1) {
+            (*out)[ni++] = 1;
+            continue;
+        }
+        size_t np = new_dims[ni], op = od[oi], nj = ni + 1, oj = oi + 1;
+        while (np != op) {
+            if (np < op) {
+                if (nj >= new_dims.len()) return false;
+                np *= new_dims[nj++];
+            } else {
+                if (oj >= od.size()) return false;
+                op *= od[oj++];
+            }
+        }
+        for (size_t q = oi; q + 1 < oj; q++)
+            if (os[q] != (int64_t)od[q + 1] * os[q + 1]) return false;
+        int64_t st = os[oj - 1];
+        for (size_t q = nj; q-- > ni;) {
+            (*out)[q] = st;
+            st *= (int64_t)new_dims[q];
+        }
+        ni = nj;
+        oi = oj;
+    }
+    for (; ni < new_dims.len(); ni++) {
+        if (new_dims[ni] != 1) return false;
+        (*out)[ni] = 1;
+    }
+    return oi == od.size();
+}
+
 // [outer, axis, inner] view of `dims` around `axis`.
 void split_at(const FixedDimensions &dims, size_t axis, size_t *outer, size_t *len, size_t *inner) {
     *outer = *inner = 1;
@@ -552,6 +625,66 @@ void split_at(const FixedDimensions &dims, size_t axis, size_t *outer, size_t *l
 }
 
 }  // namespace
+
+bool HipSession::materialize(DeviceTensor *t, SessionError *err) {
+    if (t->strides.empty()) return true;
+    DeviceTensor dense;
+    if (!allocate(TypedFixedShape{t->dims, t->elem_ty}, &dense, err)) return false;
+    std::vector<int64_t> d;
+    for (auto x : t->dims.as_vec()) d.push_back((int64_t)x);
+    const std::vector<int64_t> os = dense_strides(t->dims);
+    const int rc = launch_copy_strided(ctx_, dense.ptr, t->ptr, (int)elem_size(t->elem_ty), (int)d.size(), d.data(), os.data(),
+                                       t->strides.data());
+    if (rc) return fail_code(err, rc, ctx_.last_error);
+    dense.host = t->host;
+    *t = std::move(dense);
+    return true;
+}
+
+// A Split or Transpose hands out views when everything downstream of it can read them in place:
+// MatMul operands, possibly through reshapes and further transposes.  A MatMul whose only reader is
+// a Transpose that keeps the last axis writes its result directly in that Transpose's layout.
+void HipSession::plan_views() {
+    const auto users = model_.get_value_users();
+    const Graph &g = model_.graph;
+    auto is_output = [&](ValueId v) { return std::find(g.outputs.begin(), g.outputs.end(), v) != g.outputs.end(); };
+    std::function<bool(ValueId, int)> view_ok = [&](ValueId v, int depth) -> bool {
+        if (depth > 8 || is_output(v)) return false;
+        auto it = users.find(v);
+        if (it == users.end() || it->second.empty()) return false;
+        for (NodeId u : it->second) {
+            const Node &n = g.nodes[u];
+            if (n.op.kind == OpKind::MatMul) {
+                if (n.inputs.size() > 2 && n.inputs[2] == v) return false;
+            } else if (is_alias_op(n.op.kind) || n.op.kind == OpKind::Transpose) {
+                if (n.inputs.empty() || n.inputs[0] != v || n.outputs.empty()) return false;
+                for (size_t i = 1; i < n.inputs.size(); i++)
+                    if (n.inputs[i] == v) return false;
+                if (!view_ok(n.outputs[0], depth + 1)) return false;
+            } else {
+                return false;
+            }
+        }
+        return true;
+    };
+    for (const NodeExecutionPlan &step : plan_) {
+        const NodeId id = step.node_id;
+        const Node &n = g.nodes[id];
+        if (n.op.kind == OpKind::Split || n.op.kind == OpKind::Transpose) {
+            bool all = !n.outputs.empty();
+            for (ValueId v : n.outputs) all = all && view_ok(v, 0);
+            if (all) lazy_views_.insert(id);
+        } else if (n.op.kind == OpKind::MatMul && n.outputs.size() == 1 && !is_output(n.outputs[0])) {
+            auto it = users.find(n.outputs[0]);
+            if (it == users.end() || it->second.size() != 1) continue;
+            const Node &t = g.nodes[*it->second.begin()];
+            if (t.op.kind != OpKind::Transpose || t.inputs.size() != 1) continue;
+            const auto &perm = t.op.perm;
+            if (perm.size() < 3 || perm.back() != (int64_t)perm.size() - 1) continue;
+            matmul_out_perm_[id] = perm;
+        }
+    }
+}
 
 bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, SessionError *err) {
     const Node &node = model_.graph.nodes[id];
@@ -579,6 +712,11 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
         return fail(err, SessionError::Message, opname + ": an input value is missing");
     }
     if (node.outputs.empty()) return fail(err, SessionError::Message, opname + ": node without outputs");
+    // Strided views are read in place by the operators that can; every other reader gets a dense
+    // copy, which also replaces the view for whoever reads the value later.
+    if (!reads_views(node.op.kind))
+        for (auto *d : in)
+            if (d && !d->strides.empty() && !materialize(d, err)) return false;
 
     // Output shapes: inferred at build time if possible, else now (session.rs:149-158).  Operands
     // whose contents decide a shape are read from their host copy, fetched on demand.
@@ -614,13 +752,62 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
 
     // Reshape family: the output is the input's memory under another shape.
     if (is_alias_op(op.kind) && in[0]) {
+        std::vector<int64_t> view_strides;
+        if (!in[0]->strides.empty()) {
+            if (!reshape_strides(in[0]->dims, in[0]->strides, shapes[0].dims, &view_strides)) {
+                if (!materialize(in[0], err)) return false;
+                view_strides.clear();
+            } else if (is_dense(shapes[0].dims, view_strides)) {
+                view_strides.clear();
+            }
+        }
         DeviceTensor o = *in[0];
         o.dims = shapes[0].dims;
+        o.strides = view_strides;
         if (in[0]->host) {
             Tensor h = in[0]->host->reshaped(shapes[0].dims);
             o.host = h.has_data() || shapes[0].dims.total_elems() == 0 ? std::make_shared<const Tensor>(std::move(h)) : nullptr;
         }
         outs.push_back(std::move(o));
+    } else if (op.kind == OpKind::Transpose && in[0] && !in[0]->host && (lazy_views_.count(id) || !in[0]->strides.empty())) {
+        // The permuted strides describe the result in place.  Dense again (the Transpose that a MatMul
+        // wrote ahead of): a plain tensor.  Otherwise a view when every reader takes views, else a
+        // strided copy.
+        const std::vector<int64_t> s = strides_of(*in[0]);
+        if (op.perm.size() != s.size()) return fail(err, SessionError::Shape, "Transpose: perm does not match the rank");
+        std::vector<int64_t> ps(s.size());
+        for (size_t i = 0; i < s.size(); i++) ps[i] = s[(size_t)op.perm[i]];
+        if (is_dense(shapes[0].dims, ps) || lazy_views_.count(id)) {
+            copies_avoided_++;
+            DeviceTensor o = *in[0];
+            o.dims = shapes[0].dims;
+            o.strides = is_dense(shapes[0].dims, ps) ? std::vector<int64_t>() : ps;
+            outs.push_back(std::move(o));
+        } else {
+            DeviceTensor o;
+            if (!allocate(shapes[0], &o, err)) return false;
+            std::vector<int64_t> d;
+            for (auto x : o.dims.as_vec()) d.push_back((int64_t)x);
+            const std::vector<int64_t> os = dense_strides(o.dims);
+            const int rc = launch_copy_strided(ctx_, o.ptr, in[0]->ptr, (int)elem_size(o.elem_ty), (int)d.size(), d.data(), os.data(), ps.data());
+            if (rc) return fail_code(err, rc, ctx_.last_error);
+            outs.push_back(std::move(o));
+        }
+    } else if (op.kind == OpKind::Split && in[0] && !in[0]->host && lazy_views_.count(id)) {
+        const size_t rank = in[0]->dims.len();
+        const size_t axis = (size_t)(op.axis < 0 ? op.axis + (int64_t)rank : op.axis);
+        if (axis >= rank) return fail(err, SessionError::Shape, "Split: axis out of range");
+        const std::vector<int64_t> s = strides_of(*in[0]);
+        size_t start = 0;
+        copies_avoided_++;
+        for (size_t p = 0; p < node.outputs.size(); p++) {
+            DeviceTensor o = *in[0];
+            o.dims = shapes[p].dims;
+            o.ptr = static_cast<char *>(in[0]->ptr) + start * (size_t)s[axis] * elem_size(o.elem_ty);
+            o.strides = is_dense(o.dims, s) ? std::vector<int64_t>() : s;
+            start += o.dims[axis];
+            outs.push_back(std::move(o));
+        }
     } else {
         // Shape arithmetic: integer tensors whose operands the host already knows (or can read back
         // cheaply) are computed there and uploaded; Shape and Constant always are.
@@ -664,7 +851,7 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
                 if (!upload(t, &d, err)) return false;
                 outs.push_back(std::move(d));
             }
-        } else if (!run_device_op(node, op, in, shapes, &outs, err)) {
+        } else if (current_node_ = id, !run_device_op(node, op, in, shapes, &outs, err)) {
             return false;
         }
     }
@@ -849,7 +1036,7 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
         if (!need(1)) return false;
         const size_t rank = in[0]->dims.len();
         const size_t axis = (size_t)(op.axis < 0 ? op.axis + (int64_t)rank : op.axis);
-        const std::vector<int64_t> in_str = i64v(in[0]->dims.strides());
+        const std::vector<int64_t> in_str = strides_of(*in[0]);  // a view's own strides
         size_t start = 0;
         for (size_t p = 0; p < node.outputs.size(); p++) {
             DeviceTensor o;
@@ -1212,16 +1399,57 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
     }
     case OpKind::MatMul: {  // compute_mat_mul (session.rs:621-684), with NumPy broadcasting of the batch axes
         if (!need(2) || !need_f32({0, 1})) return false;
-        const FixedDimensions &a = in[0]->dims, &b = in[1]->dims;
-        // trans_a / trans_b (fuse_transpose_matmul): the stored operand is the transposed one.
-        const int ta = op.trans_a ? 1 : 0, tb = op.trans_b ? 1 : 0;
-        const size_t lda = a[a.len() - 1], ldb = b[b.len() - 1];
-        const size_t m = ta ? a[a.len() - 1] : a[a.len() - 2], k = ta ? a[a.len() - 2] : a[a.len() - 1];
-        const size_t n = tb ? b[b.len() - 2] : b[b.len() - 1];
-        size_t a_batch = 1, b_batch = 1, batch = 1;
-        for (size_t i = 0; i + 2 < a.len(); i++) a_batch *= a[i];
-        for (size_t i = 0; i + 2 < b.len(); i++) b_batch *= b[i];
-        for (size_t i = 0; i + 2 < out.dims.len(); i++) batch *= out.dims[i];
+        // An operand may be a strided view (a head of a [b, t, h, d] tensor taken by Split / Reshape /
+        // Transpose without a copy).  Its matrix must have one unit stride; a unit row stride means the
+        // stored matrix is the transposed one.  A view the kernel's addressing cannot express is copied.
+        struct Operand {
+            size_t rows, cols, ld, batch;
+            bool stored_transposed;
+            std::vector<size_t> bdims;
+            std::vector<int64_t> bstr;
+        };
+        auto describe = [&](DeviceTensor *t, Operand *o) -> bool {
+            for (int attempt = 0; attempt < 2; attempt++) {
+                const size_t r = t->dims.len();
+                const std::vector<int64_t> st = strides_of(*t);
+                o->rows = t->dims[r - 2], o->cols = t->dims[r - 1];
+                const int64_t sr = st[r - 2], sc = st[r - 1];
+                bool ok = true;
+                if (sc == 1 || o->cols == 1) {
+                    o->stored_transposed = false;
+                    o->ld = o->rows == 1 ? o->cols : (size_t)sr;
+                    ok = o->ld >= o->cols;
+                } else if (sr == 1 || o->rows == 1) {
+                    o->stored_transposed = true;
+                    o->ld = o->cols == 1 ? o->rows : (size_t)sc;
+                    ok = o->ld >= o->rows;
+                } else {
+                    ok = false;
+                }
+                o->batch = 1;
+                o->bdims.clear(), o->bstr.clear();
+                for (size_t i = 0; i + 2 < r; i++) {
+                    o->batch *= t->dims[i];
+                    o->bdims.push_back(t->dims[i]);
+                    o->bstr.push_back(st[i]);
+                    ok = ok && st[i] >= 0;
+                }
+                if (ok || t->strides.empty()) return ok;
+                if (!materialize(t, err)) return false;
+            }
+            return false;
+        };
+        if (in[0]->dims.len() < 2 || in[1]->dims.len() < 2) return fail(err, SessionError::Shape, "MatMul: operands of rank < 2");
+        Operand A, B;
+        if (!describe(in[0], &A) || !describe(in[1], &B))
+            return fail(err, SessionError::Message, "MatMul: an operand's layout could not be read");
+        // trans_a / trans_b (fuse_transpose_matmul): the logical operand is the transpose of the tensor.
+        const int ta = (op.trans_a ? 1 : 0) ^ (A.stored_transposed ? 1 : 0), tb = (op.trans_b ? 1 : 0) ^ (B.stored_transposed ? 1 : 0);
+        const size_t m = op.trans_a ? A.cols : A.rows, k = op.trans_a ? A.rows : A.cols;
+        const size_t n = op.trans_b ? B.rows : B.cols;
+        size_t batch = 1;
+        std::vector<size_t> bd;
+        for (size_t i = 0; i + 2 < out.dims.len(); i++) batch *= out.dims[i], bd.push_back(out.dims[i]);
         // A third input is a bias row absorbed by fuse_matmul_bias: added in the epilogue (1 * acc + 1 * bias,
         // the one addition the separate Add performs).
         const float *bias = nullptr;
@@ -1231,14 +1459,74 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
             bias = f(in[2]);
         }
         const float beta = bias ? 1.0f : 0.0f;
-        if (b_batch == 1 && a_batch == batch && !ta) {
+        // The result in the layout of the Transpose that reads it (plan_views): the buffer is dense in the
+        // transposed shape, and this node's value is a view of it.
+        std::vector<int64_t> c_str = dense_strides(out.dims);
+        auto pv = matmul_out_perm_.find(current_node_);
+        if (pv != matmul_out_perm_.end() && pv->second.size() == out.dims.len()) {
+            FixedDimensions td = out.dims;
+            for (size_t i = 0; i < td.len(); i++) td[i] = out.dims[(size_t)pv->second[i]];
+            const std::vector<int64_t> ts = dense_strides(td);
+            for (size_t i = 0; i < td.len(); i++) c_str[(size_t)pv->second[i]] = ts[i];
+            if (!is_dense(out.dims, c_str)) out.strides = c_str;
+        }
+        const bool plain = in[0]->strides.empty() && in[1]->strides.empty() && out.strides.empty();
+        if (plain && B.batch == 1 && A.batch == batch && !ta) {
             // [.., m, k] x [k, n]: one tall sgemm, as the reference does (session.rs:653-660)
-            rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), bias, 1, batch * m, n, k, 0, tb, lda, ldb, n, 0, 0, 0, 0, 1, 1.0f, beta);
-        } else if ((a_batch == batch || a_batch == 1) && (b_batch == batch || b_batch == 1)) {
-            rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), bias, batch, m, n, k, ta, tb, lda, ldb, n, a_batch == 1 ? 0 : m * k,
-                             b_batch == 1 ? 0 : k * n, m * n, 0, 1, 1.0f, beta);
-        } else {
+            rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), bias, 1, batch * m, n, k, 0, tb, A.ld, B.ld, n, 0, 0, 0, 0, 1, 1.0f, beta);
+            break;
+        }
+        if (out.dims.len() < 2) return fail(err, SessionError::Shape, "MatMul: result of rank < 2");
+        if (!((A.batch == batch || A.batch == 1) && (B.batch == batch || B.batch == 1)))
             return fail(err, SessionError::Message, "MatMul: batch axes that broadcast against each other partially are not supported");
+        // Batch strides per output batch axis for each operand (0 = shared); a dense operand counts its
+        // matrices in the output's batch order whatever its own leading shape.
+        auto batch_strides = [&](const Operand &x, const DeviceTensor *t, std::vector<int64_t> *s) -> bool {
+            s->assign(bd.size(), 0);
+            if (x.batch == 1) return true;
+            if (t->strides.empty()) {
+                int64_t acc = (int64_t)(x.rows * x.cols);
+                for (size_t i = bd.size(); i-- > 0;) (*s)[i] = acc, acc *= (int64_t)bd[i];
+                return true;
+            }
+            if (x.bdims != bd) return false;
+            *s = x.bstr;
+            return true;
+        };
+        std::vector<int64_t> as, bs;
+        for (int attempt = 0;; attempt++) {
+            const std::vector<int64_t> cs(c_str.begin(), c_str.begin() + (long)bd.size());
+            const size_t ldc = out.dims[out.dims.len() - 2] > 1 ? (size_t)c_str[out.dims.len() - 2] : n;
+            bool ok = batch_strides(A, in[0], &as) && batch_strides(B, in[1], &bs);
+            std::vector<size_t> d = bd;
+            std::vector<int64_t> sa = as, sb = bs, sc = cs;
+            if (ok) {
+                // Drop axes of extent 1, then fold neighbours that every operand strides uniformly.
+                for (size_t i = d.size(); i-- > 0;)
+                    if (d[i] == 1) d.erase(d.begin() + (long)i), sa.erase(sa.begin() + (long)i), sb.erase(sb.begin() + (long)i), sc.erase(sc.begin() + (long)i);
+                for (size_t i = d.size(); i-- > 1;) {
+                    auto folds = [&](const std::vector<int64_t> &v) { return v[i - 1] == (int64_t)d[i] * v[i]; };
+                    if (folds(sa) && folds(sb) && folds(sc)) {
+                        d[i - 1] *= d[i];
+                        sa[i - 1] = sa[i], sb[i - 1] = sb[i], sc[i - 1] = sc[i];
+                        d.erase(d.begin() + (long)i), sa.erase(sa.begin() + (long)i), sb.erase(sb.begin() + (long)i), sc.erase(sc.begin() + (long)i);
+                    }
+                }
+                ok = d.size() <= 2;
+            }
+            if (ok) {
+                while (d.size() < 2) d.push_back(1), sa.push_back(0), sb.push_back(0), sc.push_back(0);
+                const size_t a2[2] = {(size_t)sa[0], (size_t)sa[1]}, b2[2] = {(size_t)sb[0], (size_t)sb[1]}, c2[2] = {(size_t)sc[0], (size_t)sc[1]};
+                rc = launch_gemm_batch2(ctx_, o, f(in[0]), f(in[1]), bias, d[0], d[1], m, n, k, ta, tb, A.ld, B.ld, ldc, a2, b2, c2, 0, 1, 1.0f, beta);
+                break;
+            }
+            // Not expressible: dense copies of the operands and a dense result instead.
+            if (attempt > 0 || (in[0]->strides.empty() && in[1]->strides.empty() && out.strides.empty()))
+                return fail(err, SessionError::Message, "MatMul: more than two independent batch axes");
+            if (!materialize(in[0], err) || !materialize(in[1], err)) return false;
+            if (!describe(in[0], &A) || !describe(in[1], &B)) return fail(err, SessionError::Message, "MatMul: an operand's layout could not be read");
+            out.strides.clear();
+            c_str = dense_strides(out.dims);
         }
         break;
     }

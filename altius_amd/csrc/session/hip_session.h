@@ -11,6 +11,7 @@
 #pragma once
 
 #include <map>
+#include <set>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -78,6 +79,10 @@ struct DeviceTensor {
     // The contents on the host, when they are known there: initializers and the small integer
     // tensors of shape arithmetic.  Shape inference and the host evaluator read these.
     std::shared_ptr<const Tensor> host;
+    // Element strides when the tensor is a strided view of its block (a lazily taken Split part or
+    // Transpose); empty for the usual dense row-major layout.  Only operators that read views in
+    // place ever see one: every other reader gets a dense copy first.
+    std::vector<int64_t> strides;
     size_t nbytes() const { return dims.total_elems() * elem_size(elem_ty); }
 };
 
@@ -114,6 +119,8 @@ public:
     double last_device_ms() const { return last_device_ms_; }
     size_t device_allocations() const { return pool_->device_allocations(); }
     // Runs served by replaying a captured HIP graph since the session was built.
+    // Nodes of the last node-by-node run that produced a view or wrote a following Transpose's layout.
+    size_t copies_avoided() const { return copies_avoided_; }
     size_t graph_replays() const { return graph_replays_; }
     const std::vector<NodeExecutionPlan> &execution_plan() const { return plan_; }
     const InferredShapes &inferred_shapes() const { return inferred_; }
@@ -148,6 +155,11 @@ private:
     bool try_capture(const std::string &key, const std::vector<Tensor> &inputs, SessionError *err);
     bool replay(CapturedRun &run, const std::vector<Tensor> &inputs, std::vector<Tensor> *outputs, SessionError *err);
     void drop_graphs();
+    // Decides at build time which Split / Transpose nodes hand out views and which MatMul nodes
+    // write their result in the layout a following Transpose would produce.
+    void plan_views();
+    // Replaces a view by a dense copy of itself.
+    bool materialize(DeviceTensor *t, SessionError *err);
 
     Model model_;
     std::vector<NodeExecutionPlan> plan_;
@@ -169,7 +181,11 @@ private:
     std::map<std::string, CapturedRun> graphs_;
     std::map<std::string, int> eager_runs_;  // per input signature: eager runs so far (the pool is warm after one)
     size_t graph_replays_ = 0;
-    uint64_t seen_ws_generation_ = 0;  // recorded launches hold the GEMM workspace's address
+    uint64_t seen_ws_generation_ = 0;
+    size_t copies_avoided_ = 0;
+    NodeId current_node_ = 0;  // the node run_device_op is working on
+    std::set<NodeId> lazy_views_;                               // Split / Transpose nodes whose outputs are views
+    std::map<NodeId, std::vector<int64_t>> matmul_out_perm_;    // MatMul nodes -> perm of the Transpose they feed  // recorded launches hold the GEMM workspace's address
 };
 
 class HipSessionBuilder {
@@ -199,6 +215,13 @@ public:
         gemm_algorithm_ = algorithm;
         return *this;
     }
+    // Not in the reference: Split and Transpose nodes whose results only MatMuls read (possibly through
+    // reshapes) hand out strided views instead of copies, and a MatMul read only by a Transpose writes
+    // that Transpose's layout directly (default on; off makes every node copy, as the reference does).
+    HipSessionBuilder &with_strided_views(bool enable) {
+        strided_views_ = enable;
+        return *this;
+    }
     // Not in the reference: which GPU to run on (default 0).
     HipSessionBuilder &with_device(int device) {
         device_ = device;
@@ -215,6 +238,7 @@ private:
     int device_ = 0;
     bool graph_replay_ = false;
     int gemm_algorithm_ = AHIP_GEMM_AUTO;
+    bool strided_views_ = true;
 };
 
 }  // namespace altius

@@ -120,6 +120,12 @@ class HipSession:
         check(self.L.ahip_session_graph_replays(self.handle, ctypes.byref(c)))
         return c.value
 
+    def copies_avoided(self):
+        """Nodes of the last node-by-node run served without their copy (views taken, layouts written in place)."""
+        c = ctypes.c_size_t()
+        check(self.L.ahip_session_copies_avoided(self.handle, ctypes.byref(c)))
+        return c.value
+
     def device_allocations(self):
         c = ctypes.c_size_t()
         check(self.L.ahip_session_device_allocations(self.handle, ctypes.byref(c)))
@@ -156,6 +162,11 @@ class HipSessionBuilder:
     def with_gemm_algorithm(self, algorithm):
         """device.GEMM_AUTO (default) / GEMM_FP32 / GEMM_BF16X3 for the large single-batch products."""
         check(self.L.ahip_session_builder_with_gemm_algorithm(self.handle, int(algorithm)))
+        return self
+
+    def with_strided_views(self, enable=True):
+        """Split / Transpose results that only MatMuls read become views instead of copies (default on)."""
+        check(self.L.ahip_session_builder_with_strided_views(self.handle, int(bool(enable))))
         return self
 
     def with_device(self, device):

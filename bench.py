@@ -287,17 +287,19 @@ def vit_table(batch, layers=12):
     ours.fuse_softmax_prologue(), ours.fuse_matmul_bias(), ours.fuse_transpose_matmul(), ours.fuse_elemwise_ops(extended=True)
     versions.append(("+ softmax prologue, matmul bias / transposes, element-wise chains", ours))
     versions.append(("+ large products on the bf16 matrix cores (three planes per operand)", ours))
+    versions.append(("+ Split / Transpose around the attention products as strided views", ours))
     rows = []
     for i, (name, model) in enumerate(versions):
-        algo = D.GEMM_AUTO if i == 3 else D.GEMM_FP32
-        sess = HipSessionBuilder(model).with_gemm_algorithm(algo).build()
+        algo = D.GEMM_AUTO if i >= 3 else D.GEMM_FP32
+        views = i >= 4
+        sess = HipSessionBuilder(model).with_gemm_algorithm(algo).with_strided_views(views).build()
         best = float("inf")
         for _ in range(4):
             outs = sess.run([x], copy=False)
             best = min(best, sess.last_device_ms())
             del outs
         sess.close()
-        prof = HipSessionBuilder(model).with_gemm_algorithm(algo).with_profiling_enabled(True).build()
+        prof = HipSessionBuilder(model).with_gemm_algorithm(algo).with_strided_views(views).with_profiling_enabled(True).build()
         for _ in range(2):
             outs = prof.run([x], copy=False)
             del outs

@@ -259,6 +259,16 @@ int ahip_gemm(ahip_ctx *ctx, float *c, const float *a, const float *b, const flo
               size_t b_batch_stride, size_t c_batch_stride, size_t c0_row_stride, size_t c0_col_stride, float alpha,
               float beta);
 
+/* ahip_gemm with the batch index split in two: batch z = (z / batch_inner, z % batch_inner), and operand X of
+ * that batch starts at x + (z / batch_inner) * x_batch_strides[0] + (z % batch_inner) * x_batch_strides[1]
+ * (elements; 0 shares).  Lets a product read or write the heads of a [b, t, h, d] tensor in place (b x h
+ * matrices of t x d with row pitch h * d) instead of through a Transpose; the session uses it that way.  The
+ * reference's sgemm call sites always copy (session.rs:1179-1278 Transpose, 621-684 MatMul). */
+int ahip_gemm_batch2(ahip_ctx *ctx, float *c, const float *a, const float *b, const float *c0, size_t batch_outer,
+                     size_t batch_inner, size_t m, size_t n, size_t k, int trans_a, int trans_b, size_t lda, size_t ldb,
+                     size_t ldc, const size_t a_batch_strides[2], const size_t b_batch_strides[2],
+                     const size_t c_batch_strides[2], size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta);
+
 /* Which kernel ahip_gemm (and the MatMul / Gemm / Conv2d operators of a session on this context) uses
  * for a single-batch product.  AHIP_GEMM_FP32: v_mfma_f32_32x32x2_f32 on the operands as they are.
  * AHIP_GEMM_BF16X3: every operand value is split exactly into three bf16 numbers and six bf16 MFMAs per
@@ -506,6 +516,16 @@ int ahip_session_builder_with_graph_replay(ahip_session_builder *builder, int en
  * session declares its float initializers constant to the GEMM, so the bf16 planes of a weight are
  * made on its first use and kept until the session is freed. */
 int ahip_session_builder_with_gemm_algorithm(ahip_session_builder *builder, int algorithm);
+/* Not in the reference, whose Split and Transpose always copy (session.rs:1179-1278, 1488-1548): with enable
+ * != 0 (the default) a Split or Transpose whose result only MatMuls read, possibly through reshapes and further
+ * transposes, hands out a strided view of its input, which the MatMul reads in place (ahip_gemm_batch2), and
+ * a MatMul read only by a Transpose that keeps the last axis writes that Transpose's layout directly.  The
+ * products are the same kernels on the same values: results do not change by a bit.  A view that some other
+ * reader needs, or that the GEMM's addressing cannot express, is copied as before. */
+int ahip_session_builder_with_strided_views(ahip_session_builder *builder, int enable);
+/* Nodes of the last node-by-node run that were served without their copy (views taken, transposed layouts
+ * written in place). */
+int ahip_session_copies_avoided(const ahip_session *session, size_t *count);
 /* build(): shape inference (AHIP_ERR_SHAPE on failure), execution plan, device context,
  * upload of the initializers.  The builder stays valid and must still be freed. */
 int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **session);

@@ -1,0 +1,212 @@
+"""Split / Transpose results that only MatMuls read are strided views, and a MatMul read only by a Transpose
+writes that Transpose's layout: the session with views must give, bit for bit, what the session that copies
+gives (same kernels, same values, other addresses), and both must match NumPy's definition of the graph.
+Also every way a view has to fall back to a copy."""
+import numpy as np
+import pytest
+
+from altius_amd.graph import Model, Op, Tensor
+from altius_amd.session import HipSessionBuilder
+from conftest import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+RNG = np.random.default_rng(2025)
+
+
+def run_both(model, feeds):
+    """Outputs with views and with copies, and how many nodes the first run served without a copy."""
+    outs = []
+    avoided = 0
+    for views in (True, False):
+        sess = HipSessionBuilder(model.clone()).with_strided_views(views).build()
+        for _ in range(2):  # the second run reuses pooled blocks: a stale view would show
+            got = [np.array(t) for t in sess.run([Tensor.from_numpy(x) for x in feeds])]
+        if views:
+            avoided = sess.copies_avoided()
+        else:
+            assert sess.copies_avoided() == 0
+        sess.close()
+        outs.append(got)
+    for a, b in zip(*outs):
+        assert_bits_equal(a, b, "views vs copies")
+    return outs[0], avoided
+
+
+def i64(m, *v):
+    return m.new_initializer(np.array(v, np.int64))
+
+
+def node(m, op, inputs, n_out=1, **attrs):
+    outs = [m.new_val() for _ in range(n_out)]
+    m.add_node(op, inputs, outs, **attrs)
+    return outs[0] if n_out == 1 else outs
+
+
+def attention(batch, tokens, heads, d, fold_kt):
+    """qkv [b, t, 3 h d] -> Split -> Reshape -> Transpose(0,2,1,3) -> QK^T -> Softmax -> PV -> Transpose -> Reshape -> proj."""
+    hd = heads * d
+    m = Model(opset_version=13)
+    x = m.new_val_named_and_shaped("qkv", [batch, tokens, 3 * hd])
+    m.add_input(x)
+    parts = node(m, Op.Split, [x, i64(m, hd, hd, hd)], 3, axis=2)
+    q, k, v = (node(m, Op.Transpose, [node(m, Op.Reshape, [p, i64(m, batch, tokens, heads, d)])], perm=[0, 2, 1, 3]) for p in parts)
+    s = node(m, Op.MatMul, [q, node(m, Op.Transpose, [k], perm=[0, 1, 3, 2])])
+    s = node(m, Op.Softmax, [s], axis=-1)
+    a = node(m, Op.Reshape, [node(m, Op.Transpose, [node(m, Op.MatMul, [s, v])], perm=[0, 2, 1, 3]), i64(m, batch, tokens, hd)])
+    w = (RNG.standard_normal((hd, hd)) * 0.1).astype(np.float32)
+    out = node(m, Op.MatMul, [a, m.new_initializer(w)])
+    m.add_output(out)
+    if fold_kt:
+        m.fuse_transpose_matmul()
+    return m, w
+
+
+def attention_numpy(x, heads, d, w):
+    b, t, _ = x.shape
+    hd = heads * d
+    q, k, v = (x[:, :, i * hd:(i + 1) * hd].reshape(b, t, heads, d).transpose(0, 2, 1, 3).astype(np.float64) for i in range(3))
+    s = q @ k.transpose(0, 1, 3, 2)
+    s = np.exp(s - s.max(-1, keepdims=True))
+    s /= s.sum(-1, keepdims=True)
+    return (s @ v).transpose(0, 2, 1, 3).reshape(b, t, hd) @ w.astype(np.float64)
+
+
+@pytest.mark.parametrize("fold_kt", [False, True])
+@pytest.mark.parametrize("batch,tokens,heads,d", [(2, 197, 12, 64), (3, 50, 4, 32), (1, 7, 1, 8), (4, 33, 3, 20)])
+def test_attention_reads_and_writes_heads_in_place(case, batch, tokens, heads, d, fold_kt):
+    case(f"attention views b={batch} t={tokens} h={heads} d={d} fold_kt={fold_kt}")
+    m, w = attention(batch, tokens, heads, d, fold_kt)
+    x = (RNG.standard_normal((batch, tokens, 3 * heads * d)) * 0.3).astype(np.float32)
+    (got,), avoided = run_both(m, [x])
+    # Split, three head transposes, (the K^T transpose unless folded,) and the merge transpose behind P V
+    assert avoided == (5 if fold_kt else 6), avoided
+    np.testing.assert_allclose(got, attention_numpy(x, heads, d, w), rtol=2e-4, atol=2e-5)
+
+
+def test_view_with_another_reader_is_copied(case):
+    """A part that an element-wise operator also reads is not made a view; its siblings' fate follows (one Split node)."""
+    case("split part read by Add as well")
+    m = Model(opset_version=13)
+    x = m.new_val_named_and_shaped("x", [2, 9, 24])
+    m.add_input(x)
+    a, b = node(m, Op.Split, [x, i64(m, 12, 12)], 2, axis=2)
+    w = RNG.standard_normal((12, 5)).astype(np.float32)
+    y = node(m, Op.MatMul, [a, m.new_initializer(w)])
+    z = node(m, Op.Add, [node(m, Op.MatMul, [b, m.new_initializer(w)]), node(m, Op.ReduceMean, [b], axes=[-1], keep_dims=True)])
+    m.add_output(y)
+    m.add_output(z)
+    xv = RNG.standard_normal((2, 9, 24)).astype(np.float32)
+    (gy, gz), avoided = run_both(m, [xv])
+    assert avoided == 0
+    np.testing.assert_allclose(gy, xv[:, :, :12] @ w, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(gz, xv[:, :, 12:] @ w + xv[:, :, 12:].mean(-1, keepdims=True), rtol=1e-5, atol=1e-5)
+
+
+def test_split_part_that_is_a_graph_output_is_copied(case):
+    case("split part as graph output")
+    m = Model(opset_version=13)
+    x = m.new_val_named_and_shaped("x", [6, 10])
+    m.add_input(x)
+    a, b = node(m, Op.Split, [x, i64(m, 4, 6)], 2, axis=1)
+    w = RNG.standard_normal((4, 3)).astype(np.float32)
+    m.add_output(node(m, Op.MatMul, [a, m.new_initializer(w)]))
+    m.add_output(b)
+    xv = RNG.standard_normal((6, 10)).astype(np.float32)
+    (gy, gb), avoided = run_both(m, [xv])
+    assert avoided == 0
+    np.testing.assert_allclose(gy, xv[:, :4] @ w, rtol=1e-5, atol=1e-5)
+    assert_bits_equal(gb, xv[:, 4:], "second part")
+
+
+@pytest.mark.parametrize("axis", [0, 1, 2])
+def test_split_on_any_axis_feeds_matmul_in_place(case, axis):
+    case(f"split axis {axis} -> matmul")
+    shape = [4, 6, 8]
+    m = Model(opset_version=13)
+    x = m.new_val_named_and_shaped("x", shape)
+    m.add_input(x)
+    half = shape[axis] // 2
+    a, b = node(m, Op.Split, [x, i64(m, half, half)], 2, axis=axis)
+    k = a_shape_last = shape[2] if axis != 2 else half
+    w = RNG.standard_normal((k, 5)).astype(np.float32)
+    m.add_output(node(m, Op.MatMul, [a, m.new_initializer(w)]))
+    m.add_output(node(m, Op.MatMul, [b, m.new_initializer(w)]))
+    xv = RNG.standard_normal(shape).astype(np.float32)
+    (ga, gb), avoided = run_both(m, [xv])
+    assert avoided == 1
+    pa, pb = np.split(xv, 2, axis=axis)
+    np.testing.assert_allclose(ga, pa @ w, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(gb, pb @ w, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("perm,side", [([1, 0], 0), ([1, 0], 1), ([0, 2, 1], 0), ([0, 2, 1], 1), ([1, 0, 2], 0), ([2, 0, 1], 0), ([2, 1, 0], 1)])
+def test_transposed_operand_of_any_permutation(case, perm, side):
+    """A lazy Transpose in front of either operand: unit row stride flips the product's transpose flag, other
+    permutations are read through batch strides or, when no unit stride is left, copied."""
+    case(f"transpose {perm} as operand {side}")
+    shape = [5, 6, 7][:len(perm)]
+    m = Model(opset_version=13)
+    x = m.new_val_named_and_shaped("x", shape)
+    m.add_input(x)
+    t = node(m, Op.Transpose, [x], perm=perm)
+    tshape = [shape[p] for p in perm]
+    if side == 0:
+        other = RNG.standard_normal((tshape[-1], 4)).astype(np.float32)
+        out = node(m, Op.MatMul, [t, m.new_initializer(other)])
+    else:
+        other = RNG.standard_normal((3, tshape[-2])).astype(np.float32)
+        out = node(m, Op.MatMul, [m.new_initializer(other), t])
+    m.add_output(out)
+    xv = RNG.standard_normal(shape).astype(np.float32)
+    (got,), avoided = run_both(m, [xv])
+    assert avoided == 1
+    want = (xv.transpose(perm) @ other) if side == 0 else (other @ xv.transpose(perm))
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
+def test_reshape_that_a_view_cannot_express_copies(case):
+    """Transpose(0,2,1,3) then Reshape that merges the two middle axes: no strides describe it, so the Reshape copies."""
+    case("reshape of a view that needs a copy")
+    m = Model(opset_version=13)
+    x = m.new_val_named_and_shaped("x", [2, 3, 4, 5])
+    m.add_input(x)
+    t = node(m, Op.Transpose, [x], perm=[0, 2, 1, 3])
+    r = node(m, Op.Reshape, [t, i64(m, 2, 12, 5)])
+    w = RNG.standard_normal((5, 6)).astype(np.float32)
+    m.add_output(node(m, Op.MatMul, [r, m.new_initializer(w)]))
+    xv = RNG.standard_normal((2, 3, 4, 5)).astype(np.float32)
+    (got,), _ = run_both(m, [xv])
+    np.testing.assert_allclose(got, xv.transpose(0, 2, 1, 3).reshape(2, 12, 5) @ w, rtol=1e-5, atol=1e-5)
+
+
+def test_three_independent_batch_axes_fall_back(case):
+    """[a, b, c, t, d] heads taken out of the middle: three batch axes that do not fold; the operands are copied."""
+    case("three batch axes")
+    m = Model(opset_version=13)
+    x = m.new_val_named_and_shaped("x", [2, 3, 5, 4, 6])
+    m.add_input(x)
+    t = node(m, Op.Transpose, [x], perm=[2, 1, 0, 3, 4])        # [5, 3, 2, 4, 6]: batch strides 24, 120, 360
+    y = m.new_val_named_and_shaped("y", [5, 3, 2, 6, 7])
+    m.add_input(y)
+    m.add_output(node(m, Op.MatMul, [t, y]))
+    xv = RNG.standard_normal((2, 3, 5, 4, 6)).astype(np.float32)
+    yv = RNG.standard_normal((5, 3, 2, 6, 7)).astype(np.float32)
+    (got,), _ = run_both(m, [xv, yv])
+    np.testing.assert_allclose(got, xv.transpose(2, 1, 0, 3, 4) @ yv, rtol=1e-5, atol=1e-5)
+
+
+def test_matmul_writes_the_layout_of_the_transpose_behind_it(case):
+    case("matmul -> transpose written in place")
+    for perm in ([0, 2, 1, 3], [1, 0, 2, 3], [2, 0, 1, 3], [1, 2, 0, 3]):
+        m = Model(opset_version=13)
+        a = m.new_val_named_and_shaped("a", [2, 3, 9, 4])
+        b = m.new_val_named_and_shaped("b", [2, 3, 4, 6])
+        m.add_input(a)
+        m.add_input(b)
+        t = node(m, Op.Transpose, [node(m, Op.MatMul, [a, b])], perm=perm)
+        m.add_output(node(m, Op.ReLU, [t]))
+        av, bv = RNG.standard_normal((2, 3, 9, 4)).astype(np.float32), RNG.standard_normal((2, 3, 4, 6)).astype(np.float32)
+        (got,), avoided = run_both(m, [av, bv])
+        assert avoided == 1, (perm, avoided)
+        np.testing.assert_allclose(got, np.maximum((av @ bv).transpose(perm), 0), rtol=1e-5, atol=1e-5)
