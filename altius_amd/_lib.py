@@ -91,6 +91,8 @@ def _declare(L):
       + [c_float, c_float])
     f("ahip_gemm_batch2", [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p] + [c_size_t] * 5 + [c_int, c_int] + [c_size_t] * 3
       + [P(c_size_t)] * 3 + [c_size_t, c_size_t, c_float, c_float])
+    f("ahip_gemm_activated", [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p] + [c_size_t] * 3 + [c_int, c_int]
+      + [c_size_t] * 5 + [c_float, c_float])
     f("ahip_gemm_set_algorithm", [c_void_p, c_int])
     f("ahip_gemm_register_constant", [c_void_p, c_void_p, c_size_t])
     f("ahip_gemm_unregister_constant", [c_void_p, c_void_p])

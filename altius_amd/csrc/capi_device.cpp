@@ -392,6 +392,17 @@ int ahip_gemm_batch2(ahip_ctx *ctx, float *c, const float *a, const float *b, co
                                       a_batch_strides, b_batch_strides, c_batch_strides, c0_row_stride, c0_col_stride, alpha, beta);
 }
 
+int ahip_gemm_activated(ahip_ctx *ctx, int a_op, float *c, const float *a, const float *b, const float *c0, size_t m,
+                        size_t n, size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc,
+                        size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta) {
+    REQUIRE_CTX(ctx, "ahip_gemm_activated");
+    if (a_op != AHIP_GELU && a_op != AHIP_RELU) return ctx->d.fail(AHIP_ERR_ARG, "ahip_gemm_activated: a_op must be AHIP_GELU or AHIP_RELU");
+    if (!altius::gemm_takes_split(ctx->d, m, n, k))
+        return ctx->d.fail(AHIP_ERR_UNSUPPORTED, "ahip_gemm_activated: this product does not take the bf16 route");
+    return altius::launch_gemm_split(ctx->d, c, a, b, c0, m, n, k, trans_a, trans_b, lda, ldb, ldc, c0_row_stride, c0_col_stride,
+                                     alpha, beta, a_op);
+}
+
 int ahip_gemm_set_algorithm(ahip_ctx *ctx, int algorithm) {
     REQUIRE_CTX(ctx, "ahip_gemm_set_algorithm");
     if (algorithm != AHIP_GEMM_AUTO && algorithm != AHIP_GEMM_FP32 && algorithm != AHIP_GEMM_BF16X3)

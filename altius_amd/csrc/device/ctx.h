@@ -131,9 +131,12 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
 // The same product for one batch through three bf16 planes per operand and six bf16 MFMAs per fp32
 // product (gemm_split.hip): as accurate as an fp32 multiply-add chain, about 1.6 times the fp32 matrix
 // cores' rate on large shapes.  launch_gemm takes this route by itself according to ctx.gemm_algorithm.
+// a_op: 0, or AHIP_GELU / AHIP_RELU applied to A's values while they are split (C = alpha f(A) B + beta C0).
 int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t m, size_t n, size_t k,
                       int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t c0_row_stride, size_t c0_col_stride,
-                      float alpha, float beta);
+                      float alpha, float beta, int a_op = 0);
+// Whether launch_gemm would send this single-batch product through launch_gemm_split.
+bool gemm_takes_split(const DeviceCtx &ctx, size_t m, size_t n, size_t k);
 // Large and tile-filling enough for the split kernel to win (the AHIP_GEMM_AUTO rule).
 bool gemm_split_worthwhile(size_t m, size_t n, size_t k);
 // Declares [ptr, ptr + bytes) immutable until unregistered: operands inside it are split once and the

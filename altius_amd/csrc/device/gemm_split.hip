@@ -20,6 +20,7 @@
 
 #include "common.h"
 #include "ctx.h"
+#include "math.h"
 
 namespace altius {
 
@@ -55,6 +56,15 @@ __device__ __forceinline__ void split3(float x, uint32_t &h0, uint32_t &h1, uint
     h2 = r2 >> 16;
 }
 
+// An activation applied to the operand's values on their way into the planes (PRE: 0 none, else an AHIP_* unary
+// code): the product reads f(A) without f(A) ever being stored as fp32.
+template <int PRE>
+__device__ __forceinline__ float pre(float x) {
+    if (PRE == AHIP_GELU) return dev::gelu_elem(x);
+    if (PRE == AHIP_RELU) return dev::relu_elem(x);
+    return x;
+}
+
 __device__ __forceinline__ void store_planes(u32x4 *__restrict__ planes, const float (&v)[8], uint32_t row, uint32_t kg, uint32_t rp,
                                              uint32_t kgs) {
     uint32_t h[3][8];
@@ -73,6 +83,7 @@ __device__ __forceinline__ void store_planes(u32x4 *__restrict__ planes, const f
 
 // Any strides: element (row, k) is src[row * s_r + k * s_k].  Consecutive lanes take consecutive rows,
 // which is the contiguous direction of an operand stored k-major (A transposed, B as given).
+template <int PRE>
 __global__ __launch_bounds__(256) void split_planes(const float *__restrict__ src, u32x4 *__restrict__ planes, uint32_t rows, uint32_t k,
                                                     size_t s_r, size_t s_k, uint32_t rp, uint32_t kgs) {
     const uint32_t row = blockIdx.x * 64 + (threadIdx.x & 63);
@@ -82,13 +93,14 @@ __global__ __launch_bounds__(256) void split_planes(const float *__restrict__ sr
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         const uint32_t kk = kg * 8 + j;
-        v[j] = (row < rows && kk < k) ? src[(size_t)row * s_r + (size_t)kk * s_k] : 0.0f;
+        v[j] = (row < rows && kk < k) ? pre<PRE>(src[(size_t)row * s_r + (size_t)kk * s_k]) : 0.0f;
     }
     store_planes(planes, v, row, kg, rp, kgs);
 }
 
 // Rows contiguous in k and 16-byte aligned: four adjacent lanes read 128 contiguous bytes of a row,
 // sixteen rows per wavefront; each (plane, k group) store of a wavefront is 256 contiguous bytes.
+template <int PRE>
 __global__ __launch_bounds__(256) void split_planes_rows(const float *__restrict__ src, u32x4 *__restrict__ planes, uint32_t rows,
                                                          uint32_t k, size_t s_r, uint32_t rp, uint32_t kgs) {
     const uint32_t row = blockIdx.x * 64 + (threadIdx.x >> 2);
@@ -99,10 +111,11 @@ __global__ __launch_bounds__(256) void split_planes_rows(const float *__restrict
     if (row < rows && k0 + 8 <= k) {
         const f32x4 lo = *reinterpret_cast<const f32x4 *>(src + (size_t)row * s_r + k0);
         const f32x4 hi = *reinterpret_cast<const f32x4 *>(src + (size_t)row * s_r + k0 + 4);
-        v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+        v[0] = pre<PRE>(lo.x), v[1] = pre<PRE>(lo.y), v[2] = pre<PRE>(lo.z), v[3] = pre<PRE>(lo.w);
+        v[4] = pre<PRE>(hi.x), v[5] = pre<PRE>(hi.y), v[6] = pre<PRE>(hi.z), v[7] = pre<PRE>(hi.w);
     } else {
 #pragma unroll
-        for (int j = 0; j < 8; j++) v[j] = (row < rows && k0 + j < k) ? src[(size_t)row * s_r + k0 + j] : 0.0f;
+        for (int j = 0; j < 8; j++) v[j] = (row < rows && k0 + j < k) ? pre<PRE>(src[(size_t)row * s_r + k0 + j]) : 0.0f;
     }
     store_planes(planes, v, row, kg, rp, kgs);
 }
@@ -321,15 +334,22 @@ PlaneDims plane_dims(size_t rows, size_t k) {
     return d;
 }
 
-int run_split(DeviceCtx &ctx, void *planes, const float *src, size_t rows, size_t k, size_t ld, bool k_contig) {
-    const PlaneDims d = plane_dims(rows, k);
+template <int PRE>
+void launch_split(DeviceCtx &ctx, void *planes, const float *src, size_t rows, size_t k, size_t ld, bool k_contig, const PlaneDims &d) {
     const dim3 grid((unsigned)(d.rp / 64), (unsigned)((d.kgs + 3) / 4));
     if (k_contig && aligned16(src) && ld % 4 == 0)
-        hipLaunchKernelGGL(split_planes_rows, grid, dim3(256), 0, ctx.stream, src, static_cast<u32x4 *>(planes), (uint32_t)rows,
+        hipLaunchKernelGGL(split_planes_rows<PRE>, grid, dim3(256), 0, ctx.stream, src, static_cast<u32x4 *>(planes), (uint32_t)rows,
                            (uint32_t)k, ld, (uint32_t)d.rp, (uint32_t)d.kgs);
     else
-        hipLaunchKernelGGL(split_planes, grid, dim3(256), 0, ctx.stream, src, static_cast<u32x4 *>(planes), (uint32_t)rows, (uint32_t)k,
-                           k_contig ? ld : (size_t)1, k_contig ? (size_t)1 : ld, (uint32_t)d.rp, (uint32_t)d.kgs);
+        hipLaunchKernelGGL(split_planes<PRE>, grid, dim3(256), 0, ctx.stream, src, static_cast<u32x4 *>(planes), (uint32_t)rows,
+                           (uint32_t)k, k_contig ? ld : (size_t)1, k_contig ? (size_t)1 : ld, (uint32_t)d.rp, (uint32_t)d.kgs);
+}
+
+int run_split(DeviceCtx &ctx, void *planes, const float *src, size_t rows, size_t k, size_t ld, bool k_contig, int pre_op = 0) {
+    const PlaneDims d = plane_dims(rows, k);
+    if (pre_op == AHIP_GELU) launch_split<AHIP_GELU>(ctx, planes, src, rows, k, ld, k_contig, d);
+    else if (pre_op == AHIP_RELU) launch_split<AHIP_RELU>(ctx, planes, src, rows, k, ld, k_contig, d);
+    else launch_split<0>(ctx, planes, src, rows, k, ld, k_contig, d);
     return ctx.check(hipGetLastError(), "split_planes launch");
 }
 
@@ -401,7 +421,9 @@ bool gemm_split_worthwhile(size_t m, size_t n, size_t k) {
 
 int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t m, size_t n, size_t k,
                       int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t c0_row_stride, size_t c0_col_stride,
-                      float alpha, float beta) {
+                      float alpha, float beta, int a_op) {
+    if (a_op != 0 && a_op != AHIP_GELU && a_op != AHIP_RELU)
+        return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm (bf16 x 3): only Gelu and Relu can be folded into the operand split");
     if (m == 0 || n == 0) return AHIP_OK;
     if (!c || !a || !b || k == 0) return ctx.fail(AHIP_ERR_ARG, "gemm (bf16 x 3): null pointer or k = 0");
     const size_t lim = (size_t)1 << 31;
@@ -413,7 +435,7 @@ int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, 
     if (tiles >= lim / 8 || (da.kgs + 3) / 4 > 65535) return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm (bf16 x 3): too many tiles");
     const bool a_kc = !trans_a, b_kc = trans_b != 0;
     int rc = AHIP_OK;
-    const void *pa = cached_planes(ctx, a, m, k, lda, a_kc, &rc);
+    const void *pa = a_op ? nullptr : cached_planes(ctx, a, m, k, lda, a_kc, &rc);  // cached planes hold the plain values
     if (rc) return rc;
     const void *pb = cached_planes(ctx, b, n, k, ldb, b_kc, &rc);
     if (rc) return rc;
@@ -425,7 +447,7 @@ int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, 
     }
     if (!pa) {
         void *p = static_cast<char *>(ctx.gemm_ws) + a_off;
-        rc = run_split(ctx, p, a, m, k, lda, a_kc);
+        rc = run_split(ctx, p, a, m, k, lda, a_kc, a_op);
         if (rc) return rc;
         pa = p;
     }

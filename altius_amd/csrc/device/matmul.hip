@@ -216,6 +216,10 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 }  // namespace
 
+bool gemm_takes_split(const DeviceCtx &ctx, size_t m, size_t n, size_t k) {
+    return k > 0 && (ctx.gemm_algorithm == AHIP_GEMM_BF16X3 || (ctx.gemm_algorithm == AHIP_GEMM_AUTO && gemm_split_worthwhile(m, n, k)));
+}
+
 int launch_gemm(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t batch, size_t m, size_t n,
                 size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t a_batch_stride,
                 size_t b_batch_stride, size_t c_batch_stride, size_t c0_row_stride, size_t c0_col_stride, float alpha,
@@ -232,8 +236,7 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
     const size_t batch = batch_outer * batch_inner;
     if (batch == 0 || m == 0 || n == 0) return AHIP_OK;
     if (!c || (k && (!a || !b))) return ctx.fail(AHIP_ERR_ARG, "gemm: null pointer");
-    if (batch == 1 && k > 0 &&
-        (ctx.gemm_algorithm == AHIP_GEMM_BF16X3 || (ctx.gemm_algorithm == AHIP_GEMM_AUTO && gemm_split_worthwhile(m, n, k))))
+    if (batch == 1 && gemm_takes_split(ctx, m, n, k))
         return launch_gemm_split(ctx, c, a, b, c0, m, n, k, trans_a, trans_b, lda, ldb, ldc, c0_row_stride, c0_col_stride, alpha, beta);
     const size_t lim = (size_t)1 << 31;
     if (m >= lim || n >= lim || k >= lim || lda >= lim || ldb >= lim || ldc >= lim || m * ldc >= ((size_t)1 << 40))

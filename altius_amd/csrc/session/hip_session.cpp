@@ -320,7 +320,7 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
     for (ValueId v : g.outputs) {
         const DeviceTensor *d = nullptr;
         auto it = values.find(v);
-        if (it != values.end() && !it->second.strides.empty() && !materialize(&it->second, err)) return finish(false);  // never planned; dense for the caller
+        if (it != values.end() && (!materialize(&it->second, err) || !apply_pending(&it->second, err))) return finish(false);  // never planned; dense for the caller
         if (it != values.end()) d = &it->second;
         else {
             auto ii = inits_.find(v);
@@ -393,7 +393,7 @@ bool HipSession::run_device(const std::vector<DeviceTensor> &inputs, std::vector
     for (ValueId v : g.outputs) {
         const DeviceTensor *d = nullptr;
         auto it = values.find(v);
-        if (it != values.end() && !it->second.strides.empty() && !materialize(&it->second, err)) return false;  // never planned; dense for the caller
+        if (it != values.end() && (!materialize(&it->second, err) || !apply_pending(&it->second, err))) return false;  // never planned; dense for the caller
         if (it != values.end()) d = &it->second;
         else {
             auto ii = inits_.find(v);
@@ -475,7 +475,7 @@ bool HipSession::try_capture(const std::string &key, const std::vector<Tensor> &
     if (ok && end == hipSuccess && graph) {
         for (ValueId v : g.outputs) {
             auto it = values.find(v);
-            if (it != values.end() && !it->second.strides.empty() && !materialize(&it->second, err)) ok = false;
+            if (it != values.end() && (!materialize(&it->second, err) || !apply_pending(&it->second, err))) ok = false;
             const DeviceTensor *d = it != values.end() ? &it->second : nullptr;
             if (!d) {
                 auto ii = inits_.find(v);
@@ -641,6 +641,18 @@ bool HipSession::materialize(DeviceTensor *t, SessionError *err) {
     return true;
 }
 
+bool HipSession::apply_pending(DeviceTensor *t, SessionError *err) {
+    if (t->pending_op < 0) return true;
+    if (!materialize(t, err)) return false;
+    DeviceTensor done;
+    if (!allocate(TypedFixedShape{t->dims, t->elem_ty}, &done, err)) return false;
+    const int rc = launch_unary(ctx_, t->pending_op, static_cast<float *>(done.ptr), static_cast<const float *>(t->ptr),
+                                t->dims.total_elems(), 0.0f, 0.0f);
+    if (rc) return fail_code(err, rc, ctx_.last_error);
+    *t = std::move(done);
+    return true;
+}
+
 // A Split or Transpose hands out views when everything downstream of it can read them in place:
 // MatMul operands, possibly through reshapes and further transposes.  A MatMul whose only reader is
 // a Transpose that keeps the last axis writes its result directly in that Transpose's layout.
@@ -674,6 +686,16 @@ void HipSession::plan_views() {
             bool all = !n.outputs.empty();
             for (ValueId v : n.outputs) all = all && view_ok(v, 0);
             if (all) lazy_views_.insert(id);
+        } else if ((n.op.kind == OpKind::Gelu || n.op.kind == OpKind::ReLU) && n.outputs.size() == 1 && n.inputs.size() == 1 &&
+                   !is_output(n.outputs[0])) {
+            // The activation between two products: its only reader is a MatMul's first operand.
+            auto it = users.find(n.outputs[0]);
+            if (it == users.end() || it->second.size() != 1) continue;
+            const Node &mm = g.nodes[*it->second.begin()];
+            if (mm.op.kind != OpKind::MatMul || mm.inputs.size() < 2 || mm.inputs[0] != n.outputs[0]) continue;
+            bool elsewhere = false;
+            for (size_t i = 1; i < mm.inputs.size(); i++) elsewhere = elsewhere || mm.inputs[i] == n.outputs[0];
+            if (!elsewhere) deferred_unary_.insert(id);
         } else if (n.op.kind == OpKind::MatMul && n.outputs.size() == 1 && !is_output(n.outputs[0])) {
             auto it = users.find(n.outputs[0]);
             if (it == users.end() || it->second.size() != 1) continue;
@@ -717,6 +739,9 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
     if (!reads_views(node.op.kind))
         for (auto *d : in)
             if (d && !d->strides.empty() && !materialize(d, err)) return false;
+    // An activation still owed is applied by the MatMul that reads the tensor as its first operand, or here.
+    for (size_t i = 0; i < in.size(); i++)
+        if (in[i] && in[i]->pending_op >= 0 && !(node.op.kind == OpKind::MatMul && i == 0) && !apply_pending(in[i], err)) return false;
 
     // Output shapes: inferred at build time if possible, else now (session.rs:149-158).  Operands
     // whose contents decide a shape are read from their host copy, fetched on demand.
@@ -768,6 +793,12 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
             Tensor h = in[0]->host->reshaped(shapes[0].dims);
             o.host = h.has_data() || shapes[0].dims.total_elems() == 0 ? std::make_shared<const Tensor>(std::move(h)) : nullptr;
         }
+        outs.push_back(std::move(o));
+    } else if (deferred_unary_.count(id) && in[0] && !in[0]->host && in[0]->elem_ty == TensorElemType::F32 && in[0]->pending_op < 0) {
+        DeviceTensor o = *in[0];
+        o.dims = shapes[0].dims;
+        o.pending_op = op.kind == OpKind::Gelu ? AHIP_GELU : AHIP_RELU;
+        copies_avoided_++;
         outs.push_back(std::move(o));
     } else if (op.kind == OpKind::Transpose && in[0] && !in[0]->host && (lazy_views_.count(id) || !in[0]->strides.empty())) {
         // The permuted strides describe the result in place.  Dense again (the Transpose that a MatMul
@@ -1440,6 +1471,22 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
             return false;
         };
         if (in[0]->dims.len() < 2 || in[1]->dims.len() < 2) return fail(err, SessionError::Shape, "MatMul: operands of rank < 2");
+        // The activation the first operand still owes is folded into the bf16 route's operand split when this
+        // product is one tall sgemm that takes that route; otherwise it runs now.
+        int a_op = 0;
+        if (in[0]->pending_op >= 0) {
+            const FixedDimensions &ad = in[0]->dims, &bdm = in[1]->dims;
+            size_t rows = 1;
+            for (size_t i = 0; i + 1 < ad.len(); i++) rows *= ad[i];
+            const bool tall = !op.trans_a && bdm.len() == 2 && in[0]->strides.empty() && in[1]->strides.empty() &&
+                              matmul_out_perm_.count(current_node_) == 0;
+            const size_t nn = op.trans_b ? bdm[0] : bdm[1];
+            if (tall && gemm_takes_split(ctx_, rows, nn, ad[ad.len() - 1])) {
+                a_op = in[0]->pending_op;
+            } else if (!apply_pending(in[0], err)) {
+                return false;
+            }
+        }
         Operand A, B;
         if (!describe(in[0], &A) || !describe(in[1], &B))
             return fail(err, SessionError::Message, "MatMul: an operand's layout could not be read");
@@ -1473,9 +1520,11 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
         const bool plain = in[0]->strides.empty() && in[1]->strides.empty() && out.strides.empty();
         if (plain && B.batch == 1 && A.batch == batch && !ta) {
             // [.., m, k] x [k, n]: one tall sgemm, as the reference does (session.rs:653-660)
-            rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), bias, 1, batch * m, n, k, 0, tb, A.ld, B.ld, n, 0, 0, 0, 0, 1, 1.0f, beta);
+            if (a_op) rc = launch_gemm_split(ctx_, o, f(in[0]), f(in[1]), bias, batch * m, n, k, 0, tb, A.ld, B.ld, n, 0, 1, 1.0f, beta, a_op);
+            else rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), bias, 1, batch * m, n, k, 0, tb, A.ld, B.ld, n, 0, 0, 0, 0, 1, 1.0f, beta);
             break;
         }
+        if (a_op) return fail(err, SessionError::Message, "MatMul: an activation was left pending on a product that cannot fold it");
         if (out.dims.len() < 2) return fail(err, SessionError::Shape, "MatMul: result of rank < 2");
         if (!((A.batch == batch || A.batch == 1) && (B.batch == batch || B.batch == 1)))
             return fail(err, SessionError::Message, "MatMul: batch axes that broadcast against each other partially are not supported");

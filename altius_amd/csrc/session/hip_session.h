@@ -83,6 +83,9 @@ struct DeviceTensor {
     // Transpose); empty for the usual dense row-major layout.  Only operators that read views in
     // place ever see one: every other reader gets a dense copy first.
     std::vector<int64_t> strides;
+    // An activation (AHIP_GELU / AHIP_RELU) that has not been applied yet: the tensor holds the
+    // activation's input, and its one reader, a MatMul, applies it while splitting the operand.
+    int pending_op = -1;
     size_t nbytes() const { return dims.total_elems() * elem_size(elem_ty); }
 };
 
@@ -160,6 +163,8 @@ private:
     void plan_views();
     // Replaces a view by a dense copy of itself.
     bool materialize(DeviceTensor *t, SessionError *err);
+    // Runs the activation a tensor still owes (pending_op) into a new buffer.
+    bool apply_pending(DeviceTensor *t, SessionError *err);
 
     Model model_;
     std::vector<NodeExecutionPlan> plan_;
@@ -184,6 +189,7 @@ private:
     uint64_t seen_ws_generation_ = 0;
     size_t copies_avoided_ = 0;
     NodeId current_node_ = 0;  // the node run_device_op is working on
+    std::set<NodeId> deferred_unary_;                           // Gelu / Relu nodes folded into the MatMul that reads them
     std::set<NodeId> lazy_views_;                               // Split / Transpose nodes whose outputs are views
     std::map<NodeId, std::vector<int64_t>> matmul_out_perm_;    // MatMul nodes -> perm of the Transpose they feed  // recorded launches hold the GEMM workspace's address
 };

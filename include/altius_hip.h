@@ -269,6 +269,16 @@ int ahip_gemm_batch2(ahip_ctx *ctx, float *c, const float *a, const float *b, co
                      size_t ldc, const size_t a_batch_strides[2], const size_t b_batch_strides[2],
                      const size_t c_batch_strides[2], size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta);
 
+/* C = alpha * f(op(A)) * op(B) + beta * C0 for one batch, f = AHIP_GELU or AHIP_RELU applied to A's values
+ * while the bf16 route (AHIP_GEMM_BF16X3) splits them: the activation between two products (Gelu between the
+ * two MatMuls of a transformer MLP) costs no pass of its own and f(A) is never stored.  The values multiplied
+ * are exactly those ahip_unary would have written.  AHIP_ERR_UNSUPPORTED, nothing launched, when this
+ * product would not take the bf16 route under the context's algorithm setting (run ahip_unary, then
+ * ahip_gemm).  No counterpart in the reference. */
+int ahip_gemm_activated(ahip_ctx *ctx, int a_op, float *c, const float *a, const float *b, const float *c0, size_t m,
+                        size_t n, size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc,
+                        size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta);
+
 /* Which kernel ahip_gemm (and the MatMul / Gemm / Conv2d operators of a session on this context) uses
  * for a single-batch product.  AHIP_GEMM_FP32: v_mfma_f32_32x32x2_f32 on the operands as they are.
  * AHIP_GEMM_BF16X3: every operand value is split exactly into three bf16 numbers and six bf16 MFMAs per

@@ -210,3 +210,77 @@ def test_matmul_writes_the_layout_of_the_transpose_behind_it(case):
         (got,), avoided = run_both(m, [av, bv])
         assert avoided == 1, (perm, avoided)
         np.testing.assert_allclose(got, np.maximum((av @ bv).transpose(perm), 0), rtol=1e-5, atol=1e-5)
+
+
+# ---- the activation between two products, folded into the second one's operand split ----
+
+from altius_amd import device as D  # noqa: E402
+from altius_amd._lib import ERR_UNSUPPORTED, AltiusHipError, check  # noqa: E402
+
+
+def mlp(rows, hidden, inner, act, second_reader=False):
+    m = Model(opset_version=13)
+    x = m.new_val_named_and_shaped("x", list(rows) + [hidden])
+    m.add_input(x)
+    w1 = (RNG.standard_normal((hidden, inner)) * 0.2).astype(np.float32)
+    w2 = (RNG.standard_normal((inner, hidden)) * 0.2).astype(np.float32)
+    b1 = RNG.standard_normal(inner).astype(np.float32)
+    h = node(m, Op.Add, [node(m, Op.MatMul, [x, m.new_initializer(w1)]), m.new_initializer(b1)])
+    a = node(m, act, [h])
+    m.add_output(node(m, Op.MatMul, [a, m.new_initializer(w2)]))
+    if second_reader:
+        m.add_output(node(m, Op.Sqrt, [node(m, Op.Mul, [a, a])]))
+    m.fuse_matmul_bias()
+    return m, (w1, b1, w2)
+
+
+@pytest.mark.parametrize("act", ["Gelu", "ReLU"])
+@pytest.mark.parametrize("algo", [D.GEMM_BF16X3, D.GEMM_FP32])
+def test_activation_between_two_products(case, act, algo):
+    """With the bf16 route the activation rides on the second product's operand split (no pass, no tensor); with
+    the fp32 route it runs when the product asks for its operand.  Either way the bits are those of the separate
+    operators."""
+    case(f"{act} between two MatMuls, algorithm {algo}")
+    m, (w1, b1, w2) = mlp((3, 50), 40, 72, getattr(Op, act))
+    x = RNG.standard_normal((3, 50, 40)).astype(np.float32)
+    outs = []
+    for views in (True, False):
+        sess = HipSessionBuilder(m.clone()).with_gemm_algorithm(algo).with_strided_views(views).build()
+        outs.append(np.array(sess.run([Tensor.from_numpy(x)])[0]))
+        assert sess.copies_avoided() == (1 if views else 0)
+        sess.close()
+    assert_bits_equal(outs[0], outs[1], "folded vs separate")
+    h = x.astype(np.float64) @ w1 + b1
+    import math
+    a = np.maximum(h, 0) if act == "ReLU" else 0.5 * h * (1 + np.vectorize(math.erf)(h / np.sqrt(2)))
+    np.testing.assert_allclose(outs[0], a @ w2, rtol=2e-3, atol=2e-3)      # the reference's Gelu is the tanh form (fast_gelu)
+
+
+def test_activation_with_a_second_reader_runs_on_its_own(case):
+    case("Gelu read by a MatMul and by an element-wise operator")
+    m, _ = mlp((20,), 16, 24, Op.Gelu, second_reader=True)
+    x = RNG.standard_normal((20, 16)).astype(np.float32)
+    (y, z), avoided = run_both(m, [x])
+    assert avoided == 0
+
+
+def test_gemm_activated_through_the_c_abi(ctx, case):
+    case("ahip_gemm_activated vs ahip_unary + ahip_gemm")
+    m, k, n = 130, 70, 90
+    a = RNG.standard_normal((m, k)).astype(np.float32)
+    b = RNG.standard_normal((k, n)).astype(np.float32)
+    da, db, dc = ctx.upload(a), ctx.upload(b), ctx.alloc(m * n * 4)
+    try:
+        ctx.gemm_set_algorithm(D.GEMM_FP32)
+        with pytest.raises(AltiusHipError) as e:
+            check(ctx.L.ahip_gemm_activated(ctx.handle, D.GELU, dc.ptr, da.ptr, db.ptr, None, m, n, k, 0, 0, k, n, n, 0, 0, 1.0, 0.0), ctx.handle)
+        assert e.value.code == ERR_UNSUPPORTED
+        ctx.gemm_set_algorithm(D.GEMM_BF16X3)
+        for op in (D.GELU, D.RELU):
+            check(ctx.L.ahip_gemm_activated(ctx.handle, op, dc.ptr, da.ptr, db.ptr, None, m, n, k, 0, 0, k, n, n, 0, 0, 1.0, 0.0), ctx.handle)
+            got = ctx.download(dc, (m, n))
+            assert_bits_equal(got, ctx.matmul(ctx.unary(op, a), b), f"op {op}")
+    finally:
+        ctx.gemm_set_algorithm(D.GEMM_AUTO)
+        for x in (da, db, dc):
+            ctx.free(x)
