@@ -42,6 +42,9 @@ struct GemmArgs {
     // x + (z / batch_inner) * x_bs + (z % batch_inner) * x_bs2 (strides in elements, 0 = shared).
     uint64_t a_bs, b_bs, c_bs, a_bs2, b_bs2, c_bs2;
     uint32_t batch_inner;
+    // Single-batch launches are one-dimensional: consecutive block ids go to the eight XCDs in turn, and
+    // each XCD (one L2) is given a contiguous run of tiles, so the blocks it runs together share panels.
+    uint32_t tiles_n, tiles, chunk;  // chunk = 0: the grid is (n tiles, m tiles, batches)
     float alpha, beta;
     int a_vec, b_vec;  // 16-byte loads are legal for this operand (alignment of base, strides, batch stride)
 };
@@ -127,7 +130,13 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_mfma(GemmArgs g) {
     __shared__ __align__(16) float Bs[2][BK * PITCH];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = TN == 128 ? wave >> 1 : wave, wn = TN == 128 ? wave & 1 : 0;
-    const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * TN;
+    uint32_t tile_m = blockIdx.y, tile_n = blockIdx.x;
+    if (g.chunk) {
+        const uint32_t tile = (blockIdx.x & 7) * g.chunk + (blockIdx.x >> 3);
+        if (tile >= g.tiles) return;
+        tile_m = tile / g.tiles_n, tile_n = tile % g.tiles_n;
+    }
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * TN;
     const uint32_t zo = blockIdx.z / g.batch_inner, zi = blockIdx.z % g.batch_inner;
     const float *a = g.a + (size_t)zo * g.a_bs + (size_t)zi * g.a_bs2;
     const float *b = g.b + (size_t)zo * g.b_bs + (size_t)zi * g.b_bs2;
@@ -275,7 +284,10 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
     g.beta = beta;
     g.a_vec = aligned16(a) && lda % 4 == 0 && a_batch_strides[0] % 4 == 0 && a_batch_strides[1] % 4 == 0;
     g.b_vec = aligned16(b) && ldb % 4 == 0 && b_batch_strides[0] % 4 == 0 && b_batch_strides[1] % 4 == 0;
-    const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch);
+    g.tiles_n = (uint32_t)gx;
+    g.tiles = (uint32_t)(gx * gy);
+    g.chunk = batch == 1 && gx * gy >= 64 && gx * gy < lim / 8 ? (uint32_t)((gx * gy + 7) / 8) : 0;
+    const dim3 grid = g.chunk ? dim3(g.chunk * 8) : dim3((unsigned)gx, (unsigned)gy, (unsigned)batch);
     const bool a_kc = !trans_a, b_kc = trans_b != 0;
 #define GEMM(AK, BK_, TN_) hipLaunchKernelGGL((gemm_f32_mfma<AK, BK_, TN_>), grid, dim3(THREADS), 0, ctx.stream, g)
     if (narrow) {
