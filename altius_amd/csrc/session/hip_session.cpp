@@ -270,6 +270,7 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
 
     std::map<ValueId, DeviceTensor> values;
     copies_avoided_ = 0;
+    pending_attn_.clear();
     std::vector<hipEvent_t> events;
     // Nothing may still read a block when it goes back to the pool for another run, and input
     // tensors must outlive their uploads: every exit path synchronises first.
@@ -371,6 +372,7 @@ bool HipSession::run_device(const std::vector<DeviceTensor> &inputs, std::vector
 
     std::map<ValueId, DeviceTensor> values;
     copies_avoided_ = 0;
+    pending_attn_.clear();
     for (size_t i = 0; i < g.inputs.size(); i++) {
         if (!inputs[i].ptr && inputs[i].nbytes())
             return fail(err, SessionError::Argument, "run_device: input " + std::to_string(i) + " has no device pointer");
@@ -443,6 +445,7 @@ bool HipSession::try_capture(const std::string &key, const std::vector<Tensor> &
     CapturedRun run;
     std::map<ValueId, DeviceTensor> values;
     copies_avoided_ = 0;
+    pending_attn_.clear();
     for (size_t i = 0; i < g.inputs.size(); i++) {
         DeviceTensor d;
         if (!allocate(TypedFixedShape{inputs[i].dims(), inputs[i].elem_ty()}, &d, err)) return false;
@@ -643,6 +646,8 @@ bool HipSession::materialize(DeviceTensor *t, SessionError *err) {
 
 bool HipSession::apply_pending(DeviceTensor *t, SessionError *err) {
     if (t->pending_op < 0) return true;
+    if (t->pending_op == PENDING_ATTENTION)
+        return fail(err, SessionError::Message, "internal: a deferred attention product was read by an operator that cannot finish it");
     if (!materialize(t, err)) return false;
     DeviceTensor done;
     if (!allocate(TypedFixedShape{t->dims, t->elem_ty}, &done, err)) return false;
@@ -650,6 +655,168 @@ bool HipSession::apply_pending(DeviceTensor *t, SessionError *err) {
                                 t->dims.total_elems(), 0.0f, 0.0f);
     if (rc) return fail_code(err, rc, ctx_.last_error);
     *t = std::move(done);
+    return true;
+}
+
+bool HipSession::describe_operand(DeviceTensor *t, MatOperand *o, SessionError *err) {
+    for (int attempt = 0; attempt < 2; attempt++) {
+        const size_t r = t->dims.len();
+        const std::vector<int64_t> st = strides_of(*t);
+        o->rows = t->dims[r - 2], o->cols = t->dims[r - 1];
+        const int64_t sr = st[r - 2], sc = st[r - 1];
+        bool ok = true;
+        if (sc == 1 || o->cols == 1) {
+            o->stored_transposed = false;
+            o->ld = o->rows == 1 ? o->cols : (size_t)sr;
+            ok = o->ld >= o->cols;
+        } else if (sr == 1 || o->rows == 1) {
+            o->stored_transposed = true;
+            o->ld = o->cols == 1 ? o->rows : (size_t)sc;
+            ok = o->ld >= o->rows;
+        } else {
+            ok = false;
+        }
+        o->batch = 1;
+        o->bdims.clear(), o->bstr.clear();
+        for (size_t i = 0; i + 2 < r; i++) {
+            o->batch *= t->dims[i];
+            o->bdims.push_back(t->dims[i]);
+            o->bstr.push_back(st[i]);
+            ok = ok && st[i] >= 0;
+        }
+        if (ok) return true;
+        if (t->strides.empty()) break;
+        if (!materialize(t, err)) return false;
+    }
+    return fail(err, SessionError::Message, "MatMul: an operand's layout could not be read");
+}
+
+namespace {
+// Batch strides of an operand over the batch axes bd (extent-1 axes already dropped from both): a dense
+// operand counts its matrices in bd's order whatever its own leading shape.
+bool operand_batch_strides(const std::vector<size_t> &bd, const std::vector<size_t> &own_dims, const std::vector<int64_t> &own_strides,
+                           bool dense, size_t matrix_elems, size_t batch, std::vector<int64_t> *out) {
+    out->assign(bd.size(), 0);
+    if (batch == 1) return true;
+    if (dense) {
+        int64_t acc = (int64_t)matrix_elems;
+        for (size_t i = bd.size(); i-- > 0;) (*out)[i] = acc, acc *= (int64_t)bd[i];
+        return true;
+    }
+    std::vector<size_t> d;
+    std::vector<int64_t> s;
+    for (size_t i = 0; i < own_dims.size(); i++)
+        if (own_dims[i] != 1) d.push_back(own_dims[i]), s.push_back(own_strides[i]);
+    if (d != bd) return false;
+    *out = s;
+    return true;
+}
+bool aligned_operand(const void *p, size_t ld, const std::vector<int64_t> &bs) {
+    bool ok = (reinterpret_cast<uintptr_t>(p) & 15u) == 0 && ld % 4 == 0;
+    for (int64_t s : bs) ok = ok && s % 4 == 0;
+    return ok;
+}
+}  // namespace
+
+// The first product of MatMul -> Softmax -> MatMul: if the one-kernel attention can take it (64-wide heads,
+// at most 256 keys, at most two batch axes, aligned operands), leave a placeholder and remember Q and K.
+bool HipSession::try_defer_attention(const Node &node, const Op &op, const std::vector<DeviceTensor *> &in,
+                                     const std::vector<TypedFixedShape> &shapes, std::vector<DeviceTensor> *outs, SessionError *err) {
+    if (in.size() != 2 || !in[0] || !in[1] || in[0]->elem_ty != TensorElemType::F32 || in[1]->elem_ty != TensorElemType::F32) return true;
+    if (in[0]->dims.len() < 2 || in[1]->dims.len() < 2 || in[0]->pending_op >= 0 || in[1]->pending_op >= 0) return true;
+    PendingAttention pa;
+    if (!describe_operand(in[0], &pa.Q, err) || !describe_operand(in[1], &pa.K, err)) return false;
+    // Q as stored rows [tq, d]; the logical second operand is K^T, so K must be stored as rows [tk, d].
+    const bool q_rows = !((op.trans_a ? 1 : 0) ^ (pa.Q.stored_transposed ? 1 : 0));
+    const bool k_rows = ((op.trans_b ? 1 : 0) ^ (pa.K.stored_transposed ? 1 : 0)) != 0;
+    if (!q_rows || !k_rows) return true;
+    const size_t tq = pa.Q.stored_transposed ? pa.Q.cols : pa.Q.rows, d = pa.Q.stored_transposed ? pa.Q.rows : pa.Q.cols;
+    const size_t tk = pa.K.stored_transposed ? pa.K.cols : pa.K.rows, dk = pa.K.stored_transposed ? pa.K.rows : pa.K.cols;
+    if (d != 64 || dk != 64 || tk == 0 || tk > 256 || tq == 0) return true;
+    const FixedDimensions &od = shapes[0].dims;
+    size_t batch = 1;
+    for (size_t i = 0; i + 2 < od.len(); i++) {
+        batch *= od[i];
+        if (od[i] != 1) pa.bd.push_back(od[i]);
+    }
+    if (pa.bd.size() > 2 || pa.Q.batch != batch || pa.K.batch != batch) return true;
+    std::vector<int64_t> qs, ks;
+    if (!operand_batch_strides(pa.bd, pa.Q.bdims, pa.Q.bstr, in[0]->strides.empty(), tq * d, pa.Q.batch, &qs) ||
+        !operand_batch_strides(pa.bd, pa.K.bdims, pa.K.bstr, in[1]->strides.empty(), tk * d, pa.K.batch, &ks))
+        return true;
+    if (!aligned_operand(in[0]->ptr, pa.Q.ld, qs) || !aligned_operand(in[1]->ptr, pa.K.ld, ks)) return true;
+    pa.Q.bstr = qs, pa.K.bstr = ks;  // now per axis of bd
+    pa.q = *in[0], pa.k = *in[1];
+    pending_attn_[node.outputs[0]] = std::move(pa);
+    DeviceTensor o;
+    o.dims = od;
+    o.elem_ty = TensorElemType::F32;
+    o.pending_op = PENDING_ATTENTION;
+    copies_avoided_++;
+    outs->push_back(std::move(o));
+    return true;
+}
+
+// The second product: O = Softmax(scale(Q K^T)) V in one kernel, into `out` (dense, or in the layout of the
+// Transpose behind this node).
+bool HipSession::run_attention_tail(const Op &op, const std::vector<DeviceTensor *> &in, DeviceTensor *out, SessionError *err) {
+    const Node &node = model_.graph.nodes[current_node_];
+    auto it = pending_attn_.find(node.inputs[0]);
+    if (it == pending_attn_.end()) return fail(err, SessionError::Message, "MatMul: deferred attention operands are missing");
+    PendingAttention pa = std::move(it->second);
+    pending_attn_.erase(it);
+    // Which attention this is (for the scale): the head that names this node as its tail.
+    const AttentionPlan *plan = nullptr;
+    for (const auto &kv : attn_head_)
+        if (kv.second.tail == current_node_) plan = &kv.second;
+    if (!plan) return fail(err, SessionError::Message, "MatMul: no attention plan for this node");
+    if (op.trans_a || in.size() != 2 || !in[1] || in[1]->elem_ty != TensorElemType::F32 || in[1]->dims.len() < 2)
+        return fail(err, SessionError::Message, "MatMul: the second product of an attention has an unexpected form");
+    const size_t tq = pa.Q.stored_transposed ? pa.Q.cols : pa.Q.rows, tk = pa.K.stored_transposed ? pa.K.cols : pa.K.rows;
+    MatOperand V;
+    std::vector<int64_t> vs;
+    for (int attempt = 0;; attempt++) {
+        if (!describe_operand(in[1], &V, err)) return false;
+        const bool v_rows = !((op.trans_b ? 1 : 0) ^ (V.stored_transposed ? 1 : 0));
+        size_t batch = 1;
+        for (size_t x : pa.bd) batch *= x;
+        bool ok = v_rows && V.rows == tk && V.cols == 64 && (V.batch == batch || V.batch == 1) &&
+                  operand_batch_strides(pa.bd, V.bdims, V.bstr, in[1]->strides.empty(), tk * 64, V.batch, &vs) &&
+                  aligned_operand(in[1]->ptr, V.ld, vs);
+        if (ok) break;
+        if (attempt > 0 || in[1]->strides.empty())
+            return fail(err, SessionError::Message, "MatMul: the values of an attention do not fit its keys");
+        if (!materialize(in[1], err)) return false;
+    }
+    // Output strides: dense, or the Transpose's layout behind this node.
+    std::vector<int64_t> c_str = dense_strides(out->dims);
+    auto pv = matmul_out_perm_.find(current_node_);
+    if (pv != matmul_out_perm_.end() && pv->second.size() == out->dims.len()) {
+        FixedDimensions td = out->dims;
+        for (size_t i = 0; i < td.len(); i++) td[i] = out->dims[(size_t)pv->second[i]];
+        const std::vector<int64_t> ts = dense_strides(td);
+        std::vector<int64_t> cand = c_str;
+        for (size_t i = 0; i < td.len(); i++) cand[(size_t)pv->second[i]] = ts[i];
+        bool aligned = true;
+        for (size_t i = 0; i + 1 < cand.size(); i++) aligned = aligned && (out->dims[i] == 1 || cand[i] % 4 == 0);
+        if (aligned && !is_dense(out->dims, cand)) out->strides = c_str = cand;
+    }
+    const size_t rank = out->dims.len();
+    std::vector<int64_t> os;
+    for (size_t i = 0; i + 2 < rank; i++)
+        if (out->dims[i] != 1) os.push_back(c_str[i]);
+    const size_t ldo = out->dims[rank - 2] > 1 ? (size_t)c_str[rank - 2] : 64;
+    auto two = [](const std::vector<int64_t> &s, size_t out2[2]) {
+        out2[0] = s.size() > 0 ? (size_t)s[0] : 0;
+        out2[1] = s.size() > 1 ? (size_t)s[1] : 0;
+    };
+    size_t q2[2], k2[2], v2[2], o2[2];
+    two(pa.Q.bstr, q2), two(pa.K.bstr, k2), two(vs, v2), two(os, o2);
+    const size_t outer = pa.bd.size() > 0 ? pa.bd[0] : 1, inner = pa.bd.size() > 1 ? pa.bd[1] : 1;
+    const int rc = launch_attention(ctx_, static_cast<float *>(out->ptr), static_cast<const float *>(pa.q.ptr),
+                                    static_cast<const float *>(pa.k.ptr), static_cast<const float *>(in[1]->ptr), outer, inner, tq, tk, 64,
+                                    pa.Q.ld, pa.K.ld, V.ld, ldo, q2, k2, v2, o2, plan->scale_op, plan->scale);
+    if (rc) return fail_code(err, rc, ctx_.last_error);
     return true;
 }
 
@@ -699,6 +866,39 @@ void HipSession::plan_views() {
         } else if (n.op.kind == OpKind::MatMul && n.outputs.size() == 1 && !is_output(n.outputs[0])) {
             auto it = users.find(n.outputs[0]);
             if (it == users.end() || it->second.size() != 1) continue;
+            // MatMul -> Softmax(last axis, optional scalar scale, no mask) -> MatMul(first operand): one attention kernel.
+            {
+                const NodeId sid = *it->second.begin();
+                const Node &sm = g.nodes[sid];
+                if (sm.op.kind == OpKind::Softmax && n.inputs.size() == 2 && !sm.inputs.empty() && sm.inputs[0] == n.outputs[0] &&
+                    !sm.op.prologue_mask && sm.outputs.size() == 1 && !is_output(sm.outputs[0])) {
+                    bool last_axis = sm.op.axis == -1;
+                    auto sh = inferred_.find(sid);
+                    if (!last_axis && sh != inferred_.end() && !sh->second.second.empty())
+                        last_axis = sm.op.axis == (int64_t)sh->second.second[0].dims.len() - 1;
+                    AttentionPlan ap;
+                    bool scale_ok = true;
+                    if (sm.op.prologue_scale) {
+                        auto init = sm.inputs.size() > 1 ? g.inits.find(sm.inputs[1]) : g.inits.end();
+                        scale_ok = init != g.inits.end() && init->second.elem_ty() == TensorElemType::F32 &&
+                                   init->second.dims().total_elems() == 1 && init->second.has_data();
+                        if (scale_ok) ap.scale_op = sm.op.prologue_scale, ap.scale = init->second.data_f32()[0];
+                    }
+                    auto su = users.find(sm.outputs[0]);
+                    if (last_axis && scale_ok && su != users.end() && su->second.size() == 1) {
+                        const NodeId tid = *su->second.begin();
+                        const Node &mm = g.nodes[tid];
+                        if (mm.op.kind == OpKind::MatMul && mm.inputs.size() == 2 && mm.inputs[0] == sm.outputs[0] &&
+                            mm.inputs[1] != sm.outputs[0] && !mm.op.trans_a) {
+                            ap.softmax = sid, ap.tail = tid;
+                            attn_head_[id] = ap;
+                            attn_softmax_.insert(sid);
+                            attn_tail_.insert(tid);
+                            continue;
+                        }
+                    }
+                }
+            }
             const Node &t = g.nodes[*it->second.begin()];
             if (t.op.kind != OpKind::Transpose || t.inputs.size() != 1) continue;
             const auto &perm = t.op.perm;
@@ -741,7 +941,9 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
             if (d && !d->strides.empty() && !materialize(d, err)) return false;
     // An activation still owed is applied by the MatMul that reads the tensor as its first operand, or here.
     for (size_t i = 0; i < in.size(); i++)
-        if (in[i] && in[i]->pending_op >= 0 && !(node.op.kind == OpKind::MatMul && i == 0) && !apply_pending(in[i], err)) return false;
+        if (in[i] && in[i]->pending_op >= 0 && !(node.op.kind == OpKind::MatMul && i == 0) &&
+            !(in[i]->pending_op == PENDING_ATTENTION && i == 0 && attn_softmax_.count(id)) && !apply_pending(in[i], err))
+            return false;
 
     // Output shapes: inferred at build time if possible, else now (session.rs:149-158).  Operands
     // whose contents decide a shape are read from their host copy, fetched on demand.
@@ -793,6 +995,17 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
             Tensor h = in[0]->host->reshaped(shapes[0].dims);
             o.host = h.has_data() || shapes[0].dims.total_elems() == 0 ? std::make_shared<const Tensor>(std::move(h)) : nullptr;
         }
+        outs.push_back(std::move(o));
+    } else if (attn_softmax_.count(id) && in[0] && in[0]->pending_op == PENDING_ATTENTION) {
+        // The Softmax of a deferred attention: its work happens in the second product's kernel.
+        auto it = pending_attn_.find(node.inputs[0]);
+        if (it == pending_attn_.end()) return fail(err, SessionError::Message, "Softmax: deferred attention operands are missing");
+        PendingAttention pa = std::move(it->second);
+        pending_attn_.erase(it);
+        pending_attn_[node.outputs[0]] = std::move(pa);
+        DeviceTensor o = *in[0];
+        o.dims = shapes[0].dims;
+        copies_avoided_++;
         outs.push_back(std::move(o));
     } else if (deferred_unary_.count(id) && in[0] && !in[0]->host && in[0]->elem_ty == TensorElemType::F32 && in[0]->pending_op < 0) {
         DeviceTensor o = *in[0];
@@ -1079,6 +1292,12 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
             outs->push_back(std::move(o));
         }
         return true;
+    }
+
+    if (op.kind == OpKind::MatMul && attn_head_.count(current_node_)) {
+        const size_t before = outs->size();
+        if (!try_defer_attention(node, op, in, shapes, outs, err)) return false;
+        if (outs->size() > before) return true;  // deferred; otherwise this product runs as usual
     }
 
     DeviceTensor out;
@@ -1433,44 +1652,11 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
         // An operand may be a strided view (a head of a [b, t, h, d] tensor taken by Split / Reshape /
         // Transpose without a copy).  Its matrix must have one unit stride; a unit row stride means the
         // stored matrix is the transposed one.  A view the kernel's addressing cannot express is copied.
-        struct Operand {
-            size_t rows, cols, ld, batch;
-            bool stored_transposed;
-            std::vector<size_t> bdims;
-            std::vector<int64_t> bstr;
-        };
-        auto describe = [&](DeviceTensor *t, Operand *o) -> bool {
-            for (int attempt = 0; attempt < 2; attempt++) {
-                const size_t r = t->dims.len();
-                const std::vector<int64_t> st = strides_of(*t);
-                o->rows = t->dims[r - 2], o->cols = t->dims[r - 1];
-                const int64_t sr = st[r - 2], sc = st[r - 1];
-                bool ok = true;
-                if (sc == 1 || o->cols == 1) {
-                    o->stored_transposed = false;
-                    o->ld = o->rows == 1 ? o->cols : (size_t)sr;
-                    ok = o->ld >= o->cols;
-                } else if (sr == 1 || o->rows == 1) {
-                    o->stored_transposed = true;
-                    o->ld = o->cols == 1 ? o->rows : (size_t)sc;
-                    ok = o->ld >= o->rows;
-                } else {
-                    ok = false;
-                }
-                o->batch = 1;
-                o->bdims.clear(), o->bstr.clear();
-                for (size_t i = 0; i + 2 < r; i++) {
-                    o->batch *= t->dims[i];
-                    o->bdims.push_back(t->dims[i]);
-                    o->bstr.push_back(st[i]);
-                    ok = ok && st[i] >= 0;
-                }
-                if (ok || t->strides.empty()) return ok;
-                if (!materialize(t, err)) return false;
-            }
-            return false;
-        };
         if (in[0]->dims.len() < 2 || in[1]->dims.len() < 2) return fail(err, SessionError::Shape, "MatMul: operands of rank < 2");
+        if (in[0]->pending_op == PENDING_ATTENTION) {  // the second product of a deferred attention: everything happens here
+            if (!run_attention_tail(op, in, &out, err)) return false;
+            break;
+        }
         // The activation the first operand still owes is folded into the bf16 route's operand split when this
         // product is one tall sgemm that takes that route; otherwise it runs now.
         int a_op = 0;
@@ -1487,9 +1673,8 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
                 return false;
             }
         }
-        Operand A, B;
-        if (!describe(in[0], &A) || !describe(in[1], &B))
-            return fail(err, SessionError::Message, "MatMul: an operand's layout could not be read");
+        MatOperand A, B;
+        if (!describe_operand(in[0], &A, err) || !describe_operand(in[1], &B, err)) return false;
         // trans_a / trans_b (fuse_transpose_matmul): the logical operand is the transpose of the tensor.
         const int ta = (op.trans_a ? 1 : 0) ^ (A.stored_transposed ? 1 : 0), tb = (op.trans_b ? 1 : 0) ^ (B.stored_transposed ? 1 : 0);
         const size_t m = op.trans_a ? A.cols : A.rows, k = op.trans_a ? A.rows : A.cols;
@@ -1530,7 +1715,7 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
             return fail(err, SessionError::Message, "MatMul: batch axes that broadcast against each other partially are not supported");
         // Batch strides per output batch axis for each operand (0 = shared); a dense operand counts its
         // matrices in the output's batch order whatever its own leading shape.
-        auto batch_strides = [&](const Operand &x, const DeviceTensor *t, std::vector<int64_t> *s) -> bool {
+        auto batch_strides = [&](const MatOperand &x, const DeviceTensor *t, std::vector<int64_t> *s) -> bool {
             s->assign(bd.size(), 0);
             if (x.batch == 1) return true;
             if (t->strides.empty()) {
@@ -1573,7 +1758,7 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
             if (attempt > 0 || (in[0]->strides.empty() && in[1]->strides.empty() && out.strides.empty()))
                 return fail(err, SessionError::Message, "MatMul: more than two independent batch axes");
             if (!materialize(in[0], err) || !materialize(in[1], err)) return false;
-            if (!describe(in[0], &A) || !describe(in[1], &B)) return fail(err, SessionError::Message, "MatMul: an operand's layout could not be read");
+            if (!describe_operand(in[0], &A, err) || !describe_operand(in[1], &B, err)) return false;
             out.strides.clear();
             c_str = dense_strides(out.dims);
         }

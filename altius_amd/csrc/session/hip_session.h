@@ -69,6 +69,9 @@ struct DeviceBlock {
     }
 };
 
+// DeviceTensor::pending_op of the placeholder a deferred attention product leaves behind (no memory).
+constexpr int PENDING_ATTENTION = 1000;
+
 struct DeviceTensor {
     FixedDimensions dims;
     TensorElemType elem_ty = TensorElemType::F32;
@@ -163,6 +166,31 @@ private:
     void plan_views();
     // Replaces a view by a dense copy of itself.
     bool materialize(DeviceTensor *t, SessionError *err);
+    // How a MatMul reads an operand that may be a strided view: its last two axes as a matrix with one unit
+    // stride (a unit row stride means the stored matrix is the transposed one), the leading axes as batches.
+    struct MatOperand {
+        size_t rows = 0, cols = 0, ld = 0, batch = 1;
+        bool stored_transposed = false;
+        std::vector<size_t> bdims;
+        std::vector<int64_t> bstr;
+    };
+    // Fills *o; a view the GEMM's addressing cannot express is replaced by a dense copy first.
+    bool describe_operand(DeviceTensor *t, MatOperand *o, SessionError *err);
+    // MatMul -> Softmax -> MatMul as one kernel (plan_views finds the triples): the first MatMul leaves a
+    // placeholder and its operands here, the Softmax passes the placeholder on, the second MatMul launches.
+    struct PendingAttention {
+        DeviceTensor q, k;
+        MatOperand Q, K;
+        std::vector<size_t> bd;  // batch axes (extent-1 axes dropped), at most two
+    };
+    struct AttentionPlan {
+        NodeId softmax, tail;
+        int scale_op = 0;
+        float scale = 1.0f;
+    };
+    bool try_defer_attention(const Node &node, const Op &op, const std::vector<DeviceTensor *> &in,
+                             const std::vector<TypedFixedShape> &shapes, std::vector<DeviceTensor> *outs, SessionError *err);
+    bool run_attention_tail(const Op &op, const std::vector<DeviceTensor *> &in, DeviceTensor *out, SessionError *err);
     // Runs the activation a tensor still owes (pending_op) into a new buffer.
     bool apply_pending(DeviceTensor *t, SessionError *err);
 
@@ -189,6 +217,9 @@ private:
     uint64_t seen_ws_generation_ = 0;
     size_t copies_avoided_ = 0;
     NodeId current_node_ = 0;  // the node run_device_op is working on
+    std::map<NodeId, AttentionPlan> attn_head_;                  // first MatMul of a fusable attention -> the rest
+    std::set<NodeId> attn_softmax_, attn_tail_;
+    std::map<ValueId, PendingAttention> pending_attn_;
     std::set<NodeId> deferred_unary_;                           // Gelu / Relu nodes folded into the MatMul that reads them
     std::set<NodeId> lazy_views_;                               // Split / Transpose nodes whose outputs are views
     std::map<NodeId, std::vector<int64_t>> matmul_out_perm_;    // MatMul nodes -> perm of the Transpose they feed  // recorded launches hold the GEMM workspace's address

@@ -411,6 +411,23 @@ class Context:
         check(self.L.ahip_gemm(self.handle, c_ptr, a_ptr, b_ptr, c0_ptr, batch, m, n, k, int(trans_a), int(trans_b), lda,
                                ldb, ldc, a_bs, b_bs, c_bs, c0_rs, c0_cs, alpha, beta), self.handle)
 
+    def attention(self, q, k, v, scale_op=0, scale=1.0):
+        """Softmax(scale(Q K^T)) V for q [..., tq, 64], k / v [..., tk, 64] (same leading shape), in one kernel."""
+        q, k, v = (np.asarray(x, dtype=np.float32, order="C") for x in (q, k, v))
+        tq, d = q.shape[-2:]
+        tk = k.shape[-2]
+        batch = int(np.prod(q.shape[:-2], dtype=np.int64))
+        dq, dk, dv = self.upload(q), self.upload(k), self.upload(v)
+        do = self.alloc(max(q.nbytes, 4))
+        S = ctypes.c_size_t * 2
+        try:
+            check(self.L.ahip_attention(self.handle, do.ptr, dq.ptr, dk.ptr, dv.ptr, batch, 1, tq, tk, d, d, d, d, d, S(tq * d, 0),
+                                        S(tk * d, 0), S(tk * d, 0), S(tq * d, 0), scale_op, scale), self.handle)
+            return self.download(do, q.shape)
+        finally:
+            for x in (dq, dk, dv, do):
+                self.free(x)
+
     def gemm_set_algorithm(self, algorithm):
         """GEMM_AUTO / GEMM_FP32 / GEMM_BF16X3: the kernel single-batch products take."""
         check(self.L.ahip_gemm_set_algorithm(self.handle, int(algorithm)), self.handle)

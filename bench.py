@@ -287,7 +287,7 @@ def vit_table(batch, layers=12):
     ours.fuse_softmax_prologue(), ours.fuse_matmul_bias(), ours.fuse_transpose_matmul(), ours.fuse_elemwise_ops(extended=True)
     versions.append(("+ softmax prologue, matmul bias / transposes, element-wise chains", ours))
     versions.append(("+ large products on the bf16 matrix cores (three planes per operand)", ours))
-    versions.append(("+ strided views around the attention products, Gelu folded into fc2's operand split", ours))
+    versions.append(("+ strided views, one-kernel attention, Gelu folded into fc2's operand split", ours))
     rows = []
     for i, (name, model) in enumerate(versions):
         algo = D.GEMM_AUTO if i >= 3 else D.GEMM_FP32
@@ -368,6 +368,17 @@ def build_next_rows(ctx, D, batch=256):
     gemm("MatMul fc2 [%d,3072]x[3072,768]" % M, 1, M, H, 4 * H, 0, 0, both)
     gemm("MatMul QK^T %d x [197,64]x[64,197]" % (batch * NH), batch * NH, T, T, DH, T * DH, DH * T)
     gemm("MatMul PV %d x [197,197]x[197,64]" % (batch * NH), batch * NH, T, DH, T, T * T, T * DH)
+    # QK^T -> scale -> Softmax -> PV in one kernel, heads read in place from the [b, t, 3 h d] result of the qkv product
+    # and written as [b, t, h d]
+    import ctypes
+    qkv3 = ctx.upload(rng.standard_normal((batch * T, 3 * H), dtype=np.float32))
+    att = ctx.alloc(batch * T * H * 4)
+    S2 = ctypes.c_size_t * 2
+    ld = 3 * H
+    rows.append(("Attention %d x Softmax(QK^T/8)V [197,64], one kernel" % (batch * NH), 4 * batch * T * 4 * H,
+                 2.0 * batch * NH * (2 * T * T * DH),
+                 lambda: check(L.ahip_attention(h, att.ptr, qkv3.ptr, qkv3.ptr + H * 4, qkv3.ptr + 2 * H * 4, batch, NH, T, T, DH, ld, ld, ld, H,
+                                                S2(T * ld, DH), S2(T * ld, DH), S2(T * ld, DH), S2(T * H, DH), 1, 0.125), h)))
     return rows
 
 

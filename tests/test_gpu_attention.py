@@ -1,0 +1,79 @@
+"""The one-kernel attention (Softmax(scale(Q K^T)) V with the scores in registers), through the C ABI and through
+the session that recognises MatMul -> Softmax -> MatMul.  Pinned by the definition in float64 and by the three
+separate operators (whose Softmax is itself held to the oracle elsewhere): same exp, same normalisation, other
+summation orders.  Unscaled scores of 64-wide N(0,1) vectors reach +-30, where an fp32 rounding of the score
+already moves exp by 3e-5 relative: the bars are 2e-4 relative, 2e-5 absolute."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from altius_amd._lib import ERR_UNSUPPORTED, AltiusHipError, check
+
+pytestmark = pytest.mark.gpu
+
+RNG = np.random.default_rng(99)
+
+
+def reference(q, k, v, scale_op, scale):
+    s = q.astype(np.float64) @ np.swapaxes(k.astype(np.float64), -1, -2)
+    s = s * scale if scale_op == 1 else s / scale if scale_op == 2 else s
+    e = np.exp(s - s.max(-1, keepdims=True))
+    return (e / e.sum(-1, keepdims=True)) @ v.astype(np.float64)
+
+
+@pytest.mark.parametrize("batch,tq,tk", [((2, 3), 197, 197), ((1,), 1, 1), ((4,), 32, 32), ((2,), 33, 31), ((3,), 70, 256), ((1,), 300, 100),
+                                         ((2, 2), 64, 129), ((1,), 257, 224), ((5,), 7, 200)])
+@pytest.mark.parametrize("scale_op", [0, 1, 2])
+def test_attention_matches_its_definition_and_the_separate_operators(ctx, case, batch, tq, tk, scale_op):
+    case(f"attention batch {batch} tq {tq} tk {tk} scale_op {scale_op}")
+    q = RNG.standard_normal(batch + (tq, 64)).astype(np.float32)
+    k = RNG.standard_normal(batch + (tk, 64)).astype(np.float32)
+    v = RNG.standard_normal(batch + (tk, 64)).astype(np.float32)
+    scale = np.float32(0.125) if scale_op == 1 else np.float32(8.0)
+    got = ctx.attention(q, k, v, scale_op, float(scale))
+    np.testing.assert_allclose(got, reference(q, k, v, scale_op, scale), rtol=2e-4, atol=2e-5)
+    s = ctx.matmul(q, np.ascontiguousarray(np.swapaxes(k, -1, -2)))
+    s = s * scale if scale_op == 1 else s / scale if scale_op == 2 else s
+    sep = ctx.matmul(ctx.softmax(s.astype(np.float32)), v)
+    np.testing.assert_allclose(got, sep, rtol=2e-4, atol=2e-5)
+
+
+def test_attention_with_peaked_and_masked_like_scores(ctx, case):
+    """Large score ranges (one key dominating, keys at -1e4 relative) exercise the exp clamp and the row maximum."""
+    case("attention, peaked scores")
+    q = (RNG.standard_normal((2, 50, 64)) * 6).astype(np.float32)
+    k = (RNG.standard_normal((2, 90, 64)) * 6).astype(np.float32)
+    v = RNG.standard_normal((2, 90, 64)).astype(np.float32)
+    got = ctx.attention(q, k, v)
+    np.testing.assert_allclose(got, reference(q, k, v, 0, 1.0), rtol=2e-3, atol=2e-4)
+    rows = got.reshape(-1, 64)
+    assert np.isfinite(rows).all()
+
+
+def test_attention_reads_heads_in_place(ctx, case):
+    """Q, K, V as column blocks of one [b, t, 3 h d] tensor, O written as [b, t, h d]: row pitches and two-level batches."""
+    case("attention on strided heads")
+    b, t, h, d = 2, 45, 3, 64
+    x = RNG.standard_normal((b, t, 3 * h * d)).astype(np.float32)
+    dx, do = ctx.upload(x), ctx.alloc(b * t * h * d * 4)
+    S = ctypes.c_size_t * 2
+    try:
+        ld = 3 * h * d
+        check(ctx.L.ahip_attention(ctx.handle, do.ptr, dx.ptr, dx.ptr + h * d * 4, dx.ptr + 2 * h * d * 4, b, h, t, t, d, ld, ld, ld, h * d,
+                                   S(t * ld, d), S(t * ld, d), S(t * ld, d), S(t * h * d, d), 1, 0.125), ctx.handle)
+        got = ctx.download(do, (b, t, h, d))
+    finally:
+        ctx.free(dx)
+        ctx.free(do)
+    q, k, v = (x[:, :, i * h * d:(i + 1) * h * d].reshape(b, t, h, d).transpose(0, 2, 1, 3) for i in range(3))
+    np.testing.assert_allclose(got.transpose(0, 2, 1, 3), reference(q, k, v, 1, 0.125), rtol=2e-5, atol=2e-6)
+
+
+def test_attention_refuses_what_it_cannot_do(ctx, case):
+    case("attention refusals")
+    for shape_q, shape_k in (((4, 32), (4, 32)), ((4, 64), (300, 64))):
+        q, k = np.zeros(shape_q, np.float32), np.zeros(shape_k, np.float32)
+        with pytest.raises(AltiusHipError) as e:
+            ctx.attention(q, k, k)
+        assert e.value.code == ERR_UNSUPPORTED
