@@ -144,3 +144,32 @@ def test_profiled_session_is_not_recorded(case):
     for _ in range(3):
         sess.run([c["x"]])
     assert sess.graph_replays() == 0 and sess.profile()
+
+
+def test_replay_of_an_encoder_layer_with_views_attention_and_the_bf16_route(case):
+    """A ViT-style encoder layer (two shapes, the second one larger so that the GEMM workspace grows and recorded
+    graphs have to be dropped): strided views, the deferred Gelu, the one-kernel attention and the bf16 GEMM route with
+    its workspace and cached weight planes, eager against replayed, bit for bit, on fresh inputs."""
+    from altius_amd import device as D
+    from altius_amd import graphs
+
+    case("graph replay: encoder layer")
+    sessions = {}
+    for batch in (2, 5):
+        m = graphs.vit_encoder(batch, layers=1, tokens=50, classes=10)
+        m.fuse_layer_norm(), m.fuse_gelu(), m.fuse_softmax_prologue(), m.fuse_matmul_bias(), m.fuse_transpose_matmul()
+        m.fuse_elemwise_ops(extended=True)
+        sessions[batch] = (HipSessionBuilder(m.clone()).with_gemm_algorithm(D.GEMM_BF16X3).build(),
+                           HipSessionBuilder(m).with_gemm_algorithm(D.GEMM_BF16X3).with_graph_replay().build())
+    for i in range(4):
+        for batch, (eager, replayed) in sessions.items():
+            x = synth.normal(50 + i, [batch, 50, 768], std=1.0)
+            (want,) = eager.run([x])
+            (got,) = replayed.run([x])
+            assert_bits_equal(got, want, f"batch {batch} run {i}")
+            assert eager.copies_avoided() >= 8          # Split, 3 head transposes, first product, Softmax, merge transpose, Gelu
+    for eager, replayed in sessions.values():
+        assert replayed.graph_replays() >= 2
+        eager.close()
+        replayed.close()
+
