@@ -36,6 +36,10 @@ int create_device_ctx(int device, hipStream_t stream, bool own_stream, DeviceCtx
     e = hipSetDevice(device);
     if (e != hipSuccess) return fail(e, "hipSetDevice");
     ctx->device = device;
+    {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && cus >= 8) ctx->cus_per_xcd = cus / 8;
+    }
     if (own_stream) {
         // Default priority; non-blocking with respect to the legacy default stream.
         e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);

@@ -53,6 +53,12 @@ struct DeviceCtx {
     void *gemm_ws = nullptr;
     size_t gemm_ws_bytes = 0;
     uint64_t gemm_ws_generation = 0;
+    // Partial sums and arrival counters of tiles the bf16 GEMM cuts along k (device memory, owned).
+    void *gemm_partials = nullptr;
+    size_t gemm_partials_bytes = 0;
+    int *gemm_counters = nullptr;
+    bool gemm_split_k = true;
+    int cus_per_xcd = 0;  // compute units / 8, read when the context is created
     std::vector<ConstantBuffer> gemm_constants;
     std::vector<PackedOperand> gemm_packed;
     std::string last_error;

@@ -123,6 +123,7 @@ __global__ __launch_bounds__(256) void split_planes_rows(const float *__restrict
 // ---------------------------------------------------------------- the product
 
 constexpr int TM = 256, TN = 256, THREADS = 512;
+constexpr size_t GEMM_COUNTERS = 256;  // tiles cut along k per launch: at most 8 XCDs x 31
 
 // One k step of 16 (two k groups of 8) of both operand tiles.
 struct Stage {
@@ -140,6 +141,11 @@ struct SplitGemmArgs {
     uint32_t c0_rs, c0_cs;
     float alpha, beta;
     uint32_t tiles_n, tiles, chunk;
+    // Each XCD's run of `chunk` tiles: the first `full` are whole tiles (one block each); each of the rest is
+    // computed by `sf` blocks over `sf` slices of k, whose partial sums meet in `partials` (see the kernel).
+    uint32_t full, sf;
+    float *partials;
+    int *counters;
     int c_vec;    // 16-byte stores into C are aligned
     int c_stream;  // C is large: write it with non-temporal stores
 };
@@ -227,8 +233,17 @@ __global__ __launch_bounds__(THREADS, 1) void gemm_bf16x3(SplitGemmArgs g) {
     const int wm = wave >> 1, wn = wave & 1, lr = lane & 31, lk = lane >> 5;
     // Consecutive block ids are dealt to the eight XCDs in turn; give each XCD (one L2) a contiguous
     // run of tiles so that the blocks it runs together share operand panels.
-    const uint32_t slot = blockIdx.x >> 3, tile = (blockIdx.x & 7) * g.chunk + slot;
-    if (slot >= g.chunk || tile >= g.tiles) return;
+    // The last, partly filled round of an XCD is cut along k instead: its tiles are computed by sf blocks each,
+    // so that round takes 1 / sf of a tile's time.
+    const uint32_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    uint32_t local = slot, part = 0, nparts = 1;
+    if (slot >= g.full) {
+        local = g.full + (slot - g.full) / g.sf;
+        part = (slot - g.full) % g.sf;
+        nparts = g.sf;
+    }
+    const uint32_t tile = xcd * g.chunk + local;
+    if (local >= g.chunk || tile >= g.tiles) return;
     const uint32_t m0 = (tile / g.tiles_n) * TM, n0 = (tile % g.tiles_n) * TN;
     const size_t a_plane = (size_t)g.kgs * g.mp, b_plane = (size_t)g.kgs * g.np;
 
@@ -240,13 +255,13 @@ __global__ __launch_bounds__(THREADS, 1) void gemm_bf16x3(SplitGemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    const uint32_t nst = g.kgs / 2;
+    const uint32_t all_stages = g.kgs / 2, first = part * all_stages / nparts, nst = (part + 1) * all_stages / nparts - first;
     const uint32_t a_addr = (uint32_t)(uintptr_t)(lds_ptr)&S[0].a[0][lk][wm * 64 + lr];
     const uint32_t b_addr = (uint32_t)(uintptr_t)(lds_ptr)&S[0].b[0][lk][wn * 128 + lr];
     const int sub = (wave >> 2) * 256 + (wave & 3) * 64;
-    const u32x4 *ga = g.ap + (size_t)(wave >> 2) * g.mp + m0 + (wave & 3) * 64 + lane;
-    const u32x4 *gb = g.bp + (size_t)(wave >> 2) * g.np + n0 + (wave & 3) * 64 + lane;
     const size_t a_step = (size_t)2 * g.mp, b_step = (size_t)2 * g.np;
+    const u32x4 *ga = g.ap + first * a_step + (size_t)(wave >> 2) * g.mp + m0 + (wave & 3) * 64 + lane;
+    const u32x4 *gb = g.bp + first * b_step + (size_t)(wave >> 2) * g.np + n0 + (wave & 3) * 64 + lane;
     issue(S[0], ga, gb, a_plane, b_plane, sub);
     if (nst > 1) issue(S[1], ga + a_step, gb + b_step, a_plane, b_plane, sub);
 #define STEP(CUR, NEXT2)                                                                                              \
@@ -261,6 +276,51 @@ __global__ __launch_bounds__(THREADS, 1) void gemm_bf16x3(SplitGemmArgs g) {
         STEP(2, 1)
     }
 #undef STEP
+
+    // A tile cut along k: every block leaves its partial sums in `partials` (register r of thread t at
+    // [r][t]: coalesced), and the block that arrives last adds them up in slice order, so the result does not
+    // depend on who was last, and goes on to the epilogue.  All slices of a tile run on one XCD (one L2).
+    if (nparts > 1) {
+        __shared__ int arrived;
+        const uint32_t idx = xcd * (g.chunk - g.full) + (local - g.full);
+        float *mine = g.partials + ((size_t)idx * nparts + part) * (TM * TN);
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) mine[(size_t)((i * 4 + j) * 16 + r) * THREADS + tid] = acc[i][j][r];
+        // The partial sums only have to reach this XCD's L2, where the other slices' blocks read them: stores
+        // write through the L1, and vmcnt(0) says the L2 has them.  (A device-wide release fence here would
+        // write the whole L2 back, once per wavefront.)
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (tid == 0) arrived = atomicAdd(&g.counters[idx], 1);
+        __syncthreads();
+        if (arrived != (int)nparts - 1) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // nothing stale in this CU's L1
+        if (tid == 0) atomicExch(&g.counters[idx], 0);      // ready for the next launch
+        // Sum in slice order, 64 registers' worth of loads in flight at a time.
+        const float *all = g.partials + (size_t)idx * nparts * (TM * TN) + tid;
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+        for (uint32_t q = 0; q < nparts; q++) {
+            const float *src = all + (size_t)q * (TM * TN);
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                float tmp[64];
+#pragma unroll
+                for (int e = 0; e < 64; e++) tmp[e] = src[(size_t)(i * 64 + e) * THREADS];
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[i][j][r] += tmp[j * 16 + r];
+            }
+        }
+    }
 
     // Epilogue: each wavefront transposes 32 x 128 of its sub-tile at a time through a private LDS
     // region (pitch 132 floats), then stores rows of 128 floats, 16 bytes per lane.
@@ -411,6 +471,35 @@ int ensure_workspace(DeviceCtx &ctx, size_t bytes) {
     return AHIP_OK;
 }
 
+int ensure_partials(DeviceCtx &ctx, size_t bytes) {
+    if (!ctx.gemm_counters) {
+        void *c = nullptr;
+        // Zeroed once, in stream order ahead of the first kernel that counts in it; the kernels leave it zeroed.
+        if (hipMalloc(&c, GEMM_COUNTERS * sizeof(int)) != hipSuccess ||
+            hipMemsetAsync(c, 0, GEMM_COUNTERS * sizeof(int), ctx.stream) != hipSuccess) {
+            (void)hipGetLastError();
+            if (c) (void)hipFree(c);
+            return ctx.fail(AHIP_ERR_OOM, "gemm: no memory for the slice counters");
+        }
+        ctx.gemm_counters = static_cast<int *>(c);
+    }
+    if (bytes <= ctx.gemm_partials_bytes) return AHIP_OK;
+    int rc = ctx.check(hipStreamSynchronize(ctx.stream), "hipStreamSynchronize");
+    if (rc) return rc;
+    if (ctx.gemm_partials) (void)hipFree(ctx.gemm_partials);
+    ctx.gemm_partials = nullptr;
+    ctx.gemm_partials_bytes = 0;
+    ctx.gemm_ws_generation++;
+    void *p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return ctx.fail(AHIP_ERR_OOM, "gemm: no memory for the partial sums of tiles cut along k");
+    }
+    ctx.gemm_partials = p;
+    ctx.gemm_partials_bytes = bytes;
+    return AHIP_OK;
+}
+
 }  // namespace
 
 bool gemm_split_worthwhile(size_t m, size_t n, size_t k) {
@@ -475,9 +564,32 @@ int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, 
     g.tiles_n = (uint32_t)tiles_n;
     g.tiles = (uint32_t)tiles;
     g.chunk = (uint32_t)((tiles + 7) / 8);
+    // An XCD works through its run of tiles one round of `per` blocks at a time (one block per CU).  If the last
+    // round is partly filled, cut each of its tiles along k into as many slices as fill it.
+    const uint32_t per = ctx.cus_per_xcd ? (uint32_t)ctx.cus_per_xcd : 32u, stages = g.kgs / 2;
+    g.full = g.chunk / per * per;
+    g.sf = 1;
+    const uint32_t rem = g.chunk - g.full;
+    if (rem && ctx.gemm_split_k) {
+        uint32_t sf = per / rem;
+        sf = std::min(sf, 8u);
+        sf = std::min(sf, stages / 4);
+        if (sf >= 2 && (size_t)8 * rem <= GEMM_COUNTERS) g.sf = sf;
+    }
+    if (g.sf == 1) g.full = g.chunk;
+    g.partials = nullptr;
+    g.counters = nullptr;
+    if (g.sf > 1) {
+        rc = ensure_partials(ctx, (size_t)8 * (g.chunk - g.full) * g.sf * TM * TN * sizeof(float));
+        if (rc) return rc;
+        g.partials = static_cast<float *>(ctx.gemm_partials);
+        g.counters = ctx.gemm_counters;  // allocated by ensure_partials on first use
+        if (!g.partials || !g.counters) return ctx.fail(AHIP_ERR_HIP, "gemm: the buffers for tiles cut along k are missing");
+    }
+    const uint32_t slots = g.full + (g.chunk - g.full) * g.sf;
     g.c_vec = aligned16(c) && ldc % 4 == 0;
     g.c_stream = ctx.streaming(m * n * sizeof(float));
-    hipLaunchKernelGGL(gemm_bf16x3, dim3(g.chunk * 8), dim3(THREADS), 0, ctx.stream, g);
+    hipLaunchKernelGGL(gemm_bf16x3, dim3(slots * 8), dim3(THREADS), 0, ctx.stream, g);
     return ctx.check(hipGetLastError(), "gemm (bf16 x 3) launch");
 }
 
@@ -519,6 +631,11 @@ void gemm_release_all(DeviceCtx &ctx) {
     if (ctx.gemm_ws) (void)hipFree(ctx.gemm_ws);
     ctx.gemm_ws = nullptr;
     ctx.gemm_ws_bytes = 0;
+    if (ctx.gemm_partials) (void)hipFree(ctx.gemm_partials);
+    ctx.gemm_partials = nullptr;
+    ctx.gemm_partials_bytes = 0;
+    if (ctx.gemm_counters) (void)hipFree(ctx.gemm_counters);
+    ctx.gemm_counters = nullptr;
 }
 
 }  // namespace altius
