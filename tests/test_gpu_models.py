@@ -200,3 +200,94 @@ def test_bert_style_encoder_layer(case):
     # the scale and the mask went into the Softmax, the erf chain became Gelu, the LayerNorm chains one node each,
     # the bias rows went into their products
     assert not ops & {"Div", "Erf", "Pow", "Sqrt", "ReduceMean"}
+
+
+# ---- GPT-2-style -------------------------------------------------------------------------------------
+# The graph `python -m transformers.onnx --model=gpt2` writes (crates/altius_py/gpt2.py:1), one block of it:
+# token and position Gathers, LayerNorm chains, every linear layer as Reshape -> Gemm -> Reshape, one Split of the
+# fused qkv projection, keys transposed straight to [b, h, d, t], Div by sqrt(d), the causal mask as Where over a
+# Slice of a lower-triangular bool buffer, the padding mask added, tanh-GELU written out, the output projection
+# on the transposed token table.
+GB, GT, GH, GNH, GFF, GV, GCTX = 2, 20, 128, 2, 256, 60, 32
+GDH = GH // GNH
+
+
+def make_gpt2():
+    p = {"wte": rnd(GV, GH, scale=0.3), "wpe": rnd(GCTX, GH, scale=0.1), "ln1": (rnd(GH, shift=1.0, scale=0.1), rnd(GH, scale=0.1)),
+         "w_qkv": rnd(GH, 3 * GH, scale=0.08), "b_qkv": rnd(3 * GH, scale=0.05), "w_o": rnd(GH, GH, scale=0.08), "b_o": rnd(GH, scale=0.05),
+         "ln2": (rnd(GH, shift=1.0, scale=0.1), rnd(GH, scale=0.1)), "w_fc": rnd(GH, GFF, scale=0.08), "b_fc": rnd(GFF, scale=0.05),
+         "w_pr": rnd(GFF, GH, scale=0.08), "b_pr": rnd(GH, scale=0.05), "lnf": (rnd(GH, shift=1.0, scale=0.1), rnd(GH, scale=0.1))}
+    g = G()
+    f = lambda v: g.c(np.array(v, np.float32))
+    i64 = lambda *v: g.c(np.array(v, np.int64))
+
+    def layer_norm(x, gamma, beta):
+        mean = g.op("ReduceMean", [x], axes=[-1])
+        d = g.op("Sub", [x, mean])
+        var = g.op("ReduceMean", [g.op("Pow", [d, f(2.0)])], axes=[-1])
+        return g.op("Add", [g.op("Mul", [g.op("Div", [d, g.op("Sqrt", [g.op("Add", [var, f(1e-5)])])]), g.c(gamma)]), g.c(beta)])
+
+    def conv1d(x, w, b, n_in, n_out):  # HF's Conv1D: x.view(-1, n_in) @ w + b, viewed back
+        y = g.op("Gemm", [g.op("Reshape", [x, i64(-1, n_in)]), g.c(w), g.c(b)])
+        return g.op("Reshape", [y, i64(GB, GT, n_out)])
+
+    x = g.op("Add", [g.op("Gather", [g.c(p["wte"]), "input_ids"], axis=0), g.op("Gather", [g.c(p["wpe"]), "position_ids"], axis=0)])
+    h = layer_norm(x, *p["ln1"])
+    qkv = conv1d(h, p["w_qkv"], p["b_qkv"], GH, 3 * GH)
+    parts = [f"qkv{i}" for i in range(3)]
+    g.nodes.append(W.node("Split", [qkv, i64(GH, GH, GH)], parts, axis=2))
+    heads = lambda t, perm: g.op("Transpose", [g.op("Reshape", [t, i64(GB, GT, GNH, GDH)])], perm=perm)
+    q, k, v = heads(parts[0], [0, 2, 1, 3]), heads(parts[1], [0, 2, 3, 1]), heads(parts[2], [0, 2, 1, 3])
+    s = g.op("Div", [g.op("MatMul", [q, k]), f(np.sqrt(GDH))])
+    tril = np.tril(np.ones((1, 1, GCTX, GCTX), np.bool_))
+    causal = g.op("Slice", [g.c(tril), i64(0, 0), i64(GT, GT), i64(2, 3)])
+    s = g.op("Where", [causal, s, f(-1e4)])
+    pad = g.op("Mul", [g.op("Sub", [f(1.0), g.op("Cast", [g.op("Unsqueeze", ["attention_mask", i64(1, 2)])], to=W.FLOAT)]), f(-10000.0)])
+    s = g.op("Softmax", [g.op("Add", [s, pad])], axis=-1)
+    a = g.op("Reshape", [g.op("Transpose", [g.op("MatMul", [s, v])], perm=[0, 2, 1, 3]), i64(GB, GT, GH)])
+    x = g.op("Add", [x, conv1d(a, p["w_o"], p["b_o"], GH, GH)])
+    h = conv1d(layer_norm(x, *p["ln2"]), p["w_fc"], p["b_fc"], GH, GFF)
+    # 0.5 h (1 + tanh(0.79788456 (h + 0.044715 h^3))) as the exporter writes it (fast_gelu_fusion.rs:5-190)
+    inner = g.op("Mul", [g.op("Add", [h, g.op("Mul", [g.op("Pow", [h, f(3.0)]), f(0.044715)])]), f(0.7978845608)])
+    h = g.op("Mul", [g.op("Mul", [h, f(0.5)]), g.op("Add", [g.op("Tanh", [inner]), f(1.0)])])
+    x = g.op("Add", [x, conv1d(h, p["w_pr"], p["b_pr"], GFF, GH)])
+    x = layer_norm(x, *p["lnf"])
+    logits = g.op("MatMul", [x, g.op("Transpose", [g.c(p["wte"])], perm=[1, 0])])
+    g.nodes.append(W.node("Identity", [logits], ["logits"]))
+    data = W.model(W.graph(g.nodes, g.inits,
+                           [W.value_info(nm, W.INT64, [GB, GT]) for nm in ("input_ids", "attention_mask", "position_ids")],
+                           [W.value_info("logits", W.FLOAT, [GB, GT, GV])]), opsets=(("", 13),))
+    return data, p
+
+
+def oracle_gpt2(ids, mask, pos, p):
+    s = lambda v: np.array(v, np.float32)
+    ln = lambda x, gb: O.layer_norm(x, gb[0], gb[1], 1e-5)
+    lin = lambda x, w, b: O.gemm(x.reshape(-1, x.shape[-1]), w, b).reshape(x.shape[:-1] + (w.shape[1],))
+    x = O.binary(O.ADD, p["wte"][ids], p["wpe"][pos])
+    qkv = lin(ln(x, p["ln1"]), p["w_qkv"], p["b_qkv"])
+    q, k, v = (np.ascontiguousarray(t.reshape(GB, GT, GNH, GDH).transpose(0, 2, 1, 3)) for t in np.split(qkv, 3, axis=2))
+    sc = O.binary(O.DIV, O.matmul(q, np.ascontiguousarray(k.transpose(0, 1, 3, 2))), s(np.sqrt(GDH)))
+    sc = np.where(np.tril(np.ones((GT, GT), np.bool_))[None, None], sc, s(-1e4)).astype(np.float32)
+    pad = O.binary(O.MUL, O.binary(O.SUB, s(1.0), mask[:, None, None, :].astype(np.float32)), s(-10000.0))
+    a = O.matmul(O.softmax(O.binary(O.ADD, sc, pad)), v).transpose(0, 2, 1, 3).reshape(GB, GT, GH)
+    x = O.binary(O.ADD, x, lin(np.ascontiguousarray(a), p["w_o"], p["b_o"]))
+    h = O.unary(O.GELU, lin(ln(x, p["ln2"]), p["w_fc"], p["b_fc"]))
+    x = ln(O.binary(O.ADD, x, lin(h, p["w_pr"], p["b_pr"])), p["lnf"])
+    return O.matmul(x, np.ascontiguousarray(p["wte"].T))
+
+
+def test_gpt2_style_decoder_block(case):
+    case("GPT-2-style decoder block from ONNX bytes")
+    data, p = make_gpt2()
+    ids = RNG.integers(0, GV, size=(GB, GT)).astype(np.int64)
+    mask = np.ones((GB, GT), np.int64)
+    mask[1, 13:] = 0
+    pos = np.tile(np.arange(GT, dtype=np.int64), (GB, 1))
+    model = Model.load_onnx_from_buffer(data)
+    sess = session(model, enable_profiling=True)
+    (logits,) = sess.run({"input_ids": ids, "attention_mask": mask, "position_ids": pos})
+    np.testing.assert_allclose(logits, oracle_gpt2(ids, mask, pos, p), rtol=5e-4, atol=5e-4)
+    ops = set(sess.profile())
+    assert {"LayerNormalization", "Gemm", "Where", "Softmax", "Gather", "MatMul", "Gelu"} <= ops
+    assert not ops & {"Tanh", "Pow", "Sqrt", "ReduceMean"}      # the tanh chain became Gelu, the LayerNorm chains one node each
