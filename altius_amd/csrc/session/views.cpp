@@ -1,0 +1,294 @@
+// The session's copy avoidance: strided views (Split / Transpose results that only MatMuls read), operand
+// descriptions for the GEMM, activations deferred into the next product's operand split, and
+// MatMul -> Softmax -> MatMul deferred into the one-kernel attention.  Counterparts in the reference always
+// copy: compute_transpose (crates/session_interpreter/src/session.rs:1179-1278), compute_split (1488-1548),
+// compute_mat_mul (621-684), compute_softmax (990-1026).
+#include <algorithm>
+#include <functional>
+
+#include "views.h"
+
+namespace altius {
+
+using namespace detail;
+
+bool HipSession::materialize(DeviceTensor *t, SessionError *err) {
+    if (t->strides.empty()) return true;
+    DeviceTensor dense;
+    if (!allocate(TypedFixedShape{t->dims, t->elem_ty}, &dense, err)) return false;
+    std::vector<int64_t> d;
+    for (auto x : t->dims.as_vec()) d.push_back((int64_t)x);
+    const std::vector<int64_t> os = dense_strides(t->dims);
+    const int rc = launch_copy_strided(ctx_, dense.ptr, t->ptr, (int)elem_size(t->elem_ty), (int)d.size(), d.data(), os.data(),
+                                       t->strides.data());
+    if (rc) return fail_code(err, rc, ctx_.last_error);
+    dense.host = t->host;
+    *t = std::move(dense);
+    return true;
+}
+
+bool HipSession::apply_pending(DeviceTensor *t, SessionError *err) {
+    if (t->pending_op < 0) return true;
+    if (t->pending_op == PENDING_ATTENTION)
+        return fail(err, SessionError::Message, "internal: a deferred attention product was read by an operator that cannot finish it");
+    if (!materialize(t, err)) return false;
+    DeviceTensor done;
+    if (!allocate(TypedFixedShape{t->dims, t->elem_ty}, &done, err)) return false;
+    const int rc = launch_unary(ctx_, t->pending_op, static_cast<float *>(done.ptr), static_cast<const float *>(t->ptr),
+                                t->dims.total_elems(), 0.0f, 0.0f);
+    if (rc) return fail_code(err, rc, ctx_.last_error);
+    *t = std::move(done);
+    return true;
+}
+
+bool HipSession::describe_operand(DeviceTensor *t, MatOperand *o, SessionError *err) {
+    for (int attempt = 0; attempt < 2; attempt++) {
+        const size_t r = t->dims.len();
+        const std::vector<int64_t> st = strides_of(*t);
+        o->rows = t->dims[r - 2], o->cols = t->dims[r - 1];
+        const int64_t sr = st[r - 2], sc = st[r - 1];
+        bool ok = true;
+        if (sc == 1 || o->cols == 1) {
+            o->stored_transposed = false;
+            o->ld = o->rows == 1 ? o->cols : (size_t)sr;
+            ok = o->ld >= o->cols;
+        } else if (sr == 1 || o->rows == 1) {
+            o->stored_transposed = true;
+            o->ld = o->cols == 1 ? o->rows : (size_t)sc;
+            ok = o->ld >= o->rows;
+        } else {
+            ok = false;
+        }
+        o->batch = 1;
+        o->bdims.clear(), o->bstr.clear();
+        for (size_t i = 0; i + 2 < r; i++) {
+            o->batch *= t->dims[i];
+            o->bdims.push_back(t->dims[i]);
+            o->bstr.push_back(st[i]);
+            ok = ok && st[i] >= 0;
+        }
+        if (ok) return true;
+        if (t->strides.empty()) break;
+        if (!materialize(t, err)) return false;
+    }
+    return fail(err, SessionError::Message, "MatMul: an operand's layout could not be read");
+}
+
+namespace {
+// Batch strides of an operand over the batch axes bd (extent-1 axes already dropped from both): a dense
+// operand counts its matrices in bd's order whatever its own leading shape.
+bool operand_batch_strides(const std::vector<size_t> &bd, const std::vector<size_t> &own_dims, const std::vector<int64_t> &own_strides,
+                           bool dense, size_t matrix_elems, size_t batch, std::vector<int64_t> *out) {
+    out->assign(bd.size(), 0);
+    if (batch == 1) return true;
+    if (dense) {
+        int64_t acc = (int64_t)matrix_elems;
+        for (size_t i = bd.size(); i-- > 0;) (*out)[i] = acc, acc *= (int64_t)bd[i];
+        return true;
+    }
+    std::vector<size_t> d;
+    std::vector<int64_t> s;
+    for (size_t i = 0; i < own_dims.size(); i++)
+        if (own_dims[i] != 1) d.push_back(own_dims[i]), s.push_back(own_strides[i]);
+    if (d != bd) return false;
+    *out = s;
+    return true;
+}
+bool aligned_operand(const void *p, size_t ld, const std::vector<int64_t> &bs) {
+    bool ok = (reinterpret_cast<uintptr_t>(p) & 15u) == 0 && ld % 4 == 0;
+    for (int64_t s : bs) ok = ok && s % 4 == 0;
+    return ok;
+}
+}  // namespace
+
+// The first product of MatMul -> Softmax -> MatMul: if the one-kernel attention can take it (64-wide heads,
+// at most 256 keys, at most two batch axes, aligned operands), leave a placeholder and remember Q and K.
+bool HipSession::try_defer_attention(const Node &node, const Op &op, const std::vector<DeviceTensor *> &in,
+                                     const std::vector<TypedFixedShape> &shapes, std::vector<DeviceTensor> *outs, SessionError *err) {
+    if (in.size() != 2 || !in[0] || !in[1] || in[0]->elem_ty != TensorElemType::F32 || in[1]->elem_ty != TensorElemType::F32) return true;
+    if (in[0]->dims.len() < 2 || in[1]->dims.len() < 2 || in[0]->pending_op >= 0 || in[1]->pending_op >= 0) return true;
+    PendingAttention pa;
+    if (!describe_operand(in[0], &pa.Q, err) || !describe_operand(in[1], &pa.K, err)) return false;
+    // Q as stored rows [tq, d]; the logical second operand is K^T, so K must be stored as rows [tk, d].
+    const bool q_rows = !((op.trans_a ? 1 : 0) ^ (pa.Q.stored_transposed ? 1 : 0));
+    const bool k_rows = ((op.trans_b ? 1 : 0) ^ (pa.K.stored_transposed ? 1 : 0)) != 0;
+    if (!q_rows || !k_rows) return true;
+    const size_t tq = pa.Q.stored_transposed ? pa.Q.cols : pa.Q.rows, d = pa.Q.stored_transposed ? pa.Q.rows : pa.Q.cols;
+    const size_t tk = pa.K.stored_transposed ? pa.K.cols : pa.K.rows, dk = pa.K.stored_transposed ? pa.K.rows : pa.K.cols;
+    if (d != 64 || dk != 64 || tk == 0 || tk > 256 || tq == 0) return true;
+    const FixedDimensions &od = shapes[0].dims;
+    size_t batch = 1;
+    for (size_t i = 0; i + 2 < od.len(); i++) {
+        batch *= od[i];
+        if (od[i] != 1) pa.bd.push_back(od[i]);
+    }
+    if (pa.bd.size() > 2 || pa.Q.batch != batch || pa.K.batch != batch) return true;
+    std::vector<int64_t> qs, ks;
+    if (!operand_batch_strides(pa.bd, pa.Q.bdims, pa.Q.bstr, in[0]->strides.empty(), tq * d, pa.Q.batch, &qs) ||
+        !operand_batch_strides(pa.bd, pa.K.bdims, pa.K.bstr, in[1]->strides.empty(), tk * d, pa.K.batch, &ks))
+        return true;
+    if (!aligned_operand(in[0]->ptr, pa.Q.ld, qs) || !aligned_operand(in[1]->ptr, pa.K.ld, ks)) return true;
+    pa.Q.bstr = qs, pa.K.bstr = ks;  // now per axis of bd
+    pa.q = *in[0], pa.k = *in[1];
+    pending_attn_[node.outputs[0]] = std::move(pa);
+    DeviceTensor o;
+    o.dims = od;
+    o.elem_ty = TensorElemType::F32;
+    o.pending_op = PENDING_ATTENTION;
+    copies_avoided_++;
+    outs->push_back(std::move(o));
+    return true;
+}
+
+// The second product: O = Softmax(scale(Q K^T)) V in one kernel, into `out` (dense, or in the layout of the
+// Transpose behind this node).
+bool HipSession::run_attention_tail(const Op &op, const std::vector<DeviceTensor *> &in, DeviceTensor *out, SessionError *err) {
+    const Node &node = model_.graph.nodes[current_node_];
+    auto it = pending_attn_.find(node.inputs[0]);
+    if (it == pending_attn_.end()) return fail(err, SessionError::Message, "MatMul: deferred attention operands are missing");
+    PendingAttention pa = std::move(it->second);
+    pending_attn_.erase(it);
+    // Which attention this is (for the scale): the head that names this node as its tail.
+    const AttentionPlan *plan = nullptr;
+    for (const auto &kv : attn_head_)
+        if (kv.second.tail == current_node_) plan = &kv.second;
+    if (!plan) return fail(err, SessionError::Message, "MatMul: no attention plan for this node");
+    if (op.trans_a || in.size() != 2 || !in[1] || in[1]->elem_ty != TensorElemType::F32 || in[1]->dims.len() < 2)
+        return fail(err, SessionError::Message, "MatMul: the second product of an attention has an unexpected form");
+    const size_t tq = pa.Q.stored_transposed ? pa.Q.cols : pa.Q.rows, tk = pa.K.stored_transposed ? pa.K.cols : pa.K.rows;
+    MatOperand V;
+    std::vector<int64_t> vs;
+    for (int attempt = 0;; attempt++) {
+        if (!describe_operand(in[1], &V, err)) return false;
+        const bool v_rows = !((op.trans_b ? 1 : 0) ^ (V.stored_transposed ? 1 : 0));
+        size_t batch = 1;
+        for (size_t x : pa.bd) batch *= x;
+        bool ok = v_rows && V.rows == tk && V.cols == 64 && (V.batch == batch || V.batch == 1) &&
+                  operand_batch_strides(pa.bd, V.bdims, V.bstr, in[1]->strides.empty(), tk * 64, V.batch, &vs) &&
+                  aligned_operand(in[1]->ptr, V.ld, vs);
+        if (ok) break;
+        if (attempt > 0 || in[1]->strides.empty())
+            return fail(err, SessionError::Message, "MatMul: the values of an attention do not fit its keys");
+        if (!materialize(in[1], err)) return false;
+    }
+    // Output strides: dense, or the Transpose's layout behind this node.
+    std::vector<int64_t> c_str = dense_strides(out->dims);
+    auto pv = matmul_out_perm_.find(current_node_);
+    if (pv != matmul_out_perm_.end() && pv->second.size() == out->dims.len()) {
+        FixedDimensions td = out->dims;
+        for (size_t i = 0; i < td.len(); i++) td[i] = out->dims[(size_t)pv->second[i]];
+        const std::vector<int64_t> ts = dense_strides(td);
+        std::vector<int64_t> cand = c_str;
+        for (size_t i = 0; i < td.len(); i++) cand[(size_t)pv->second[i]] = ts[i];
+        bool aligned = true;
+        for (size_t i = 0; i + 1 < cand.size(); i++) aligned = aligned && (out->dims[i] == 1 || cand[i] % 4 == 0);
+        if (aligned && !is_dense(out->dims, cand)) out->strides = c_str = cand;
+    }
+    const size_t rank = out->dims.len();
+    std::vector<int64_t> os;
+    for (size_t i = 0; i + 2 < rank; i++)
+        if (out->dims[i] != 1) os.push_back(c_str[i]);
+    const size_t ldo = out->dims[rank - 2] > 1 ? (size_t)c_str[rank - 2] : 64;
+    auto two = [](const std::vector<int64_t> &s, size_t out2[2]) {
+        out2[0] = s.size() > 0 ? (size_t)s[0] : 0;
+        out2[1] = s.size() > 1 ? (size_t)s[1] : 0;
+    };
+    size_t q2[2], k2[2], v2[2], o2[2];
+    two(pa.Q.bstr, q2), two(pa.K.bstr, k2), two(vs, v2), two(os, o2);
+    const size_t outer = pa.bd.size() > 0 ? pa.bd[0] : 1, inner = pa.bd.size() > 1 ? pa.bd[1] : 1;
+    const int rc = launch_attention(ctx_, static_cast<float *>(out->ptr), static_cast<const float *>(pa.q.ptr),
+                                    static_cast<const float *>(pa.k.ptr), static_cast<const float *>(in[1]->ptr), outer, inner, tq, tk, 64,
+                                    pa.Q.ld, pa.K.ld, V.ld, ldo, q2, k2, v2, o2, plan->scale_op, plan->scale);
+    if (rc) return fail_code(err, rc, ctx_.last_error);
+    return true;
+}
+
+// A Split or Transpose hands out views when everything downstream of it can read them in place:
+// MatMul operands, possibly through reshapes and further transposes.  A MatMul whose only reader is
+// a Transpose that keeps the last axis writes its result directly in that Transpose's layout.
+void HipSession::plan_views() {
+    const auto users = model_.get_value_users();
+    const Graph &g = model_.graph;
+    auto is_output = [&](ValueId v) { return std::find(g.outputs.begin(), g.outputs.end(), v) != g.outputs.end(); };
+    std::function<bool(ValueId, int)> view_ok = [&](ValueId v, int depth) -> bool {
+        if (depth > 8 || is_output(v)) return false;
+        auto it = users.find(v);
+        if (it == users.end() || it->second.empty()) return false;
+        for (NodeId u : it->second) {
+            const Node &n = g.nodes[u];
+            if (n.op.kind == OpKind::MatMul) {
+                if (n.inputs.size() > 2 && n.inputs[2] == v) return false;
+            } else if (is_alias_op(n.op.kind) || n.op.kind == OpKind::Transpose) {
+                if (n.inputs.empty() || n.inputs[0] != v || n.outputs.empty()) return false;
+                for (size_t i = 1; i < n.inputs.size(); i++)
+                    if (n.inputs[i] == v) return false;
+                if (!view_ok(n.outputs[0], depth + 1)) return false;
+            } else {
+                return false;
+            }
+        }
+        return true;
+    };
+    for (const NodeExecutionPlan &step : plan_) {
+        const NodeId id = step.node_id;
+        const Node &n = g.nodes[id];
+        if (n.op.kind == OpKind::Split || n.op.kind == OpKind::Transpose) {
+            bool all = !n.outputs.empty();
+            for (ValueId v : n.outputs) all = all && view_ok(v, 0);
+            if (all) lazy_views_.insert(id);
+        } else if ((n.op.kind == OpKind::Gelu || n.op.kind == OpKind::ReLU) && n.outputs.size() == 1 && n.inputs.size() == 1 &&
+                   !is_output(n.outputs[0])) {
+            // The activation between two products: its only reader is a MatMul's first operand.
+            auto it = users.find(n.outputs[0]);
+            if (it == users.end() || it->second.size() != 1) continue;
+            const Node &mm = g.nodes[*it->second.begin()];
+            if (mm.op.kind != OpKind::MatMul || mm.inputs.size() < 2 || mm.inputs[0] != n.outputs[0]) continue;
+            bool elsewhere = false;
+            for (size_t i = 1; i < mm.inputs.size(); i++) elsewhere = elsewhere || mm.inputs[i] == n.outputs[0];
+            if (!elsewhere) deferred_unary_.insert(id);
+        } else if (n.op.kind == OpKind::MatMul && n.outputs.size() == 1 && !is_output(n.outputs[0])) {
+            auto it = users.find(n.outputs[0]);
+            if (it == users.end() || it->second.size() != 1) continue;
+            // MatMul -> Softmax(last axis, optional scalar scale, no mask) -> MatMul(first operand): one attention kernel.
+            {
+                const NodeId sid = *it->second.begin();
+                const Node &sm = g.nodes[sid];
+                if (sm.op.kind == OpKind::Softmax && n.inputs.size() == 2 && !sm.inputs.empty() && sm.inputs[0] == n.outputs[0] &&
+                    !sm.op.prologue_mask && sm.outputs.size() == 1 && !is_output(sm.outputs[0])) {
+                    bool last_axis = sm.op.axis == -1;
+                    auto sh = inferred_.find(sid);
+                    if (!last_axis && sh != inferred_.end() && !sh->second.second.empty())
+                        last_axis = sm.op.axis == (int64_t)sh->second.second[0].dims.len() - 1;
+                    AttentionPlan ap;
+                    bool scale_ok = true;
+                    if (sm.op.prologue_scale) {
+                        auto init = sm.inputs.size() > 1 ? g.inits.find(sm.inputs[1]) : g.inits.end();
+                        scale_ok = init != g.inits.end() && init->second.elem_ty() == TensorElemType::F32 &&
+                                   init->second.dims().total_elems() == 1 && init->second.has_data();
+                        if (scale_ok) ap.scale_op = sm.op.prologue_scale, ap.scale = init->second.data_f32()[0];
+                    }
+                    auto su = users.find(sm.outputs[0]);
+                    if (last_axis && scale_ok && su != users.end() && su->second.size() == 1) {
+                        const NodeId tid = *su->second.begin();
+                        const Node &mm = g.nodes[tid];
+                        if (mm.op.kind == OpKind::MatMul && mm.inputs.size() == 2 && mm.inputs[0] == sm.outputs[0] &&
+                            mm.inputs[1] != sm.outputs[0] && !mm.op.trans_a) {
+                            ap.softmax = sid, ap.tail = tid;
+                            attn_head_[id] = ap;
+                            attn_softmax_.insert(sid);
+                            attn_tail_.insert(tid);
+                            continue;
+                        }
+                    }
+                }
+            }
+            const Node &t = g.nodes[*it->second.begin()];
+            if (t.op.kind != OpKind::Transpose || t.inputs.size() != 1) continue;
+            const auto &perm = t.op.perm;
+            if (perm.size() < 3 || perm.back() != (int64_t)perm.size() - 1) continue;
+            matmul_out_perm_[id] = perm;
+        }
+    }
+}
+
+}  // namespace altius
