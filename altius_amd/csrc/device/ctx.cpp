@@ -1,6 +1,8 @@
 // Device context: error bookkeeping and creation/destruction.
 #include "ctx.h"
 
+#include <cstdlib>
+
 namespace altius {
 
 namespace {
@@ -36,6 +38,9 @@ int create_device_ctx(int device, hipStream_t stream, bool own_stream, DeviceCtx
     e = hipSetDevice(device);
     if (e != hipSuccess) return fail(e, "hipSetDevice");
     ctx->device = device;
+    // AHIP_GEMM_SPLIT_K=0 keeps the bf16 GEMM from cutting an XCD's partly filled last round of tiles along k
+    // (for measurements).
+    if (const char *e = getenv("AHIP_GEMM_SPLIT_K")) ctx->gemm_split_k = atoi(e) != 0;
     {
         int cus = 0;
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && cus >= 8) ctx->cus_per_xcd = cus / 8;
