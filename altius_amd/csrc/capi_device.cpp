@@ -406,13 +406,13 @@ int ahip_gemm_activated(ahip_ctx *ctx, int a_op, float *c, const float *a, const
 int ahip_attention(ahip_ctx *ctx, float *o, const float *q, const float *k, const float *v, size_t batch_outer,
                    size_t batch_inner, size_t tq, size_t tk, size_t d, size_t ldq, size_t ldk, size_t ldv, size_t ldo,
                    const size_t q_batch_strides[2], const size_t k_batch_strides[2], const size_t v_batch_strides[2],
-                   const size_t o_batch_strides[2], int scale_op, float scale) {
+                   const size_t o_batch_strides[2], int scale_op, float scale, const float *mask, size_t mask_outer_stride) {
     REQUIRE_CTX(ctx, "ahip_attention");
     if (!q_batch_strides || !k_batch_strides || !v_batch_strides || !o_batch_strides)
         return ctx->d.fail(AHIP_ERR_ARG, "ahip_attention: null strides");
     if (batch_inner == 0) return ctx->d.fail(AHIP_ERR_ARG, "ahip_attention: batch_inner is 0");
     return altius::launch_attention(ctx->d, o, q, k, v, batch_outer, batch_inner, tq, tk, d, ldq, ldk, ldv, ldo, q_batch_strides,
-                                    k_batch_strides, v_batch_strides, o_batch_strides, scale_op, scale);
+                                    k_batch_strides, v_batch_strides, o_batch_strides, scale_op, scale, mask, mask_outer_stride);
 }
 
 int ahip_gemm_set_algorithm(ahip_ctx *ctx, int algorithm) {

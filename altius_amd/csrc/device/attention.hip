@@ -1,5 +1,5 @@
 // Attention for one (batch, head) per block, without the score tensor ever reaching memory:
-//   O = Softmax(scale(Q K^T)) V,   Q [tq, 64], K [tk, 64], V [tk, 64], tk <= 256,
+//   O = Softmax(scale(Q K^T) + mask) V,   Q [tq, 64], K [tk, 64], V [tk, 64], tk <= 256, mask one value per key,
 // the three operators compute_mat_mul -> compute_softmax -> compute_mat_mul of the reference
 // (crates/session_interpreter/src/session.rs:621-684, 990-1026) on the fp32 matrix cores, with the
 // reference's own exp (fast_math.rs:130-150, dev::softmax_exp) and its reciprocal-multiply
@@ -41,6 +41,9 @@ struct AttnArgs {
     uint32_t batch_inner;
     int scale_op;  // 0 none, 1 scores * scale, 2 scores / scale
     float scale;
+    // Added to the scaled scores, one value per key: mask[(z / batch_inner) * mask_outer_stride + key] (null: none).
+    const float *mask;
+    uint32_t mask_outer_stride;
 };
 
 template <int NT>
@@ -123,6 +126,7 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void attention_d64(AttnArgs g) {
 
     // Softmax over the keys of this lane's query: scale, maximum (NaNs ignored, as the reference's fold does),
     // exp, sum, one reciprocal.  Keys past tk take no part.
+    const float *mask = g.mask ? g.mask + (size_t)zo * g.mask_outer_stride : nullptr;
     float mx = -INFINITY;
 #pragma unroll
     for (int j = 0; j < NT; j++)
@@ -132,6 +136,7 @@ __global__ __launch_bounds__(64 * MAX_WAVES) void attention_d64(AttnArgs g) {
             float x = s[j][r];
             if (g.scale_op == 1) x = x * g.scale;
             else if (g.scale_op == 2) x = x / g.scale;
+            if (mask && key < g.tk) x = x + mask[key];
             s[j][r] = x;
             if (key < g.tk) mx = dev::nanmax(mx, x);
         }
@@ -189,13 +194,15 @@ void launch_nt(DeviceCtx &ctx, const AttnArgs &g, dim3 grid, unsigned threads) {
 
 int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, const float *v, size_t batch_outer, size_t batch_inner,
                      size_t tq, size_t tk, size_t d, size_t ldq, size_t ldk, size_t ldv, size_t ldo, const size_t q_bs[2],
-                     const size_t k_bs[2], const size_t v_bs[2], const size_t o_bs[2], int scale_op, float scale) {
+                     const size_t k_bs[2], const size_t v_bs[2], const size_t o_bs[2], int scale_op, float scale, const float *mask,
+                     size_t mask_outer_stride) {
     const size_t batch = batch_outer * batch_inner;
     if (batch == 0 || tq == 0) return AHIP_OK;
     if (!o || !q || !k || !v) return ctx.fail(AHIP_ERR_ARG, "attention: null pointer");
     if (scale_op < 0 || scale_op > 2) return ctx.fail(AHIP_ERR_ARG, "attention: scale_op must be 0, 1 or 2");
     if (d != (size_t)D || tk == 0 || tk > 256) return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: needs 64-wide heads and 1..256 keys");
     const size_t lim = (size_t)1 << 31;
+    if (mask_outer_stride >= lim) return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: mask stride above 2^31");
     if (tq >= lim || ldq >= lim || ldk >= lim || ldv >= lim || ldo >= lim || batch >= lim)
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: extent above 2^31");
     auto vec_ok = [](const void *p, size_t ld, const size_t bs[2]) { return aligned16(p) && ld % 4 == 0 && bs[0] % 4 == 0 && bs[1] % 4 == 0; };
@@ -211,6 +218,8 @@ int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, c
     g.batch_inner = (uint32_t)batch_inner;
     g.scale_op = scale_op;
     g.scale = scale;
+    g.mask = mask;
+    g.mask_outer_stride = (uint32_t)mask_outer_stride;
     const size_t q_tiles = (tq + 31) / 32;
     const size_t gy = (q_tiles + MAX_WAVES - 1) / MAX_WAVES;
     if (gy > 65535) return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: too many queries");

@@ -134,12 +134,14 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
                        const size_t a_batch_strides[2], const size_t b_batch_strides[2], const size_t c_batch_strides[2],
                        size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta);
 
-// O = Softmax(scale(Q K^T)) V per batch, scores kept in registers (attention.hip).  Q [tq, d], K [tk, d], V [tk, d],
-// O [tq, d] with row pitches ld*; batches as in launch_gemm_batch2; scale_op 0 none / 1 multiply / 2 divide.
+// O = Softmax(scale(Q K^T) + mask) V per batch, scores kept in registers (attention.hip).  Q [tq, d], K [tk, d], V [tk, d],
+// O [tq, d] with row pitches ld*; batches as in launch_gemm_batch2; scale_op 0 none / 1 multiply / 2 divide; mask (may be
+// null) one value per key, read at mask[outer batch * mask_outer_stride + key].
 // AHIP_ERR_UNSUPPORTED (nothing launched) unless d == 64, tk <= 256 and everything is 16-byte aligned.
 int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, const float *v, size_t batch_outer, size_t batch_inner,
                      size_t tq, size_t tk, size_t d, size_t ldq, size_t ldk, size_t ldv, size_t ldo, const size_t q_bs[2],
-                     const size_t k_bs[2], const size_t v_bs[2], const size_t o_bs[2], int scale_op, float scale);
+                     const size_t k_bs[2], const size_t v_bs[2], const size_t o_bs[2], int scale_op, float scale, const float *mask = nullptr,
+                     size_t mask_outer_stride = 0);
 
 // The same product for one batch through three bf16 planes per operand and six bf16 MFMAs per fp32
 // product (gemm_split.hip): as accurate as an fp32 multiply-add chain, about 1.6 times the fp32 matrix

@@ -564,7 +564,8 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
     // An activation still owed is applied by the MatMul that reads the tensor as its first operand, or here.
     for (size_t i = 0; i < in.size(); i++)
         if (in[i] && in[i]->pending_op >= 0 && !(node.op.kind == OpKind::MatMul && i == 0) &&
-            !(in[i]->pending_op == PENDING_ATTENTION && i == 0 && attn_softmax_.count(id)) && !apply_pending(in[i], err))
+            !(in[i]->pending_op == PENDING_ATTENTION && i == 0 && attn_softmax_.count(id)) &&
+            !(in[i]->pending_op == PENDING_ATTENTION ? flush_attention(node.inputs[i], in[i], err) : apply_pending(in[i], err)))
             return false;
 
     // Output shapes: inferred at build time if possible, else now (session.rs:149-158).  Operands
@@ -622,13 +623,43 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
         // The Softmax of a deferred attention: its work happens in the second product's kernel.
         auto it = pending_attn_.find(node.inputs[0]);
         if (it == pending_attn_.end()) return fail(err, SessionError::Message, "Softmax: deferred attention operands are missing");
-        PendingAttention pa = std::move(it->second);
-        pending_attn_.erase(it);
-        pending_attn_[node.outputs[0]] = std::move(pa);
-        DeviceTensor o = *in[0];
-        o.dims = shapes[0].dims;
-        copies_avoided_++;
-        outs.push_back(std::move(o));
+        // An absorbed mask must be one value per key: a single row, or one row per outermost batch.
+        bool fits = true;
+        DeviceTensor *mask_t = nullptr;
+        size_t mask_stride = 0;
+        if (op.prologue_mask) {
+            const size_t n_in = 1 + (op.prologue_scale ? 1 : 0) + 1;
+            mask_t = in.size() >= n_in ? in[n_in - 1] : nullptr;
+            const FixedDimensions &sd = it->second.score_dims;
+            const size_t tk = sd[sd.len() - 1];
+            fits = mask_t && mask_t->elem_ty == TensorElemType::F32 && mask_t->strides.empty() && mask_t->pending_op < 0 &&
+                   (reinterpret_cast<uintptr_t>(mask_t->ptr) & 3u) == 0;
+            const size_t m_elems = fits ? mask_t->dims.total_elems() : 0;
+            if (fits && m_elems == tk) {
+                mask_stride = 0;
+            } else if (fits && !it->second.bd.empty() && m_elems == sd[0] * tk && sd[0] == it->second.bd[0] && mask_t->dims.len() >= 1 &&
+                       mask_t->dims[mask_t->dims.len() - 1] == tk) {
+                mask_stride = tk;
+            } else {
+                fits = false;
+            }
+        }
+        if (fits) {
+            PendingAttention pa = std::move(it->second);
+            pending_attn_.erase(it);
+            if (mask_t) pa.mask = *mask_t, pa.mask_outer_stride = mask_stride;
+            pending_attn_[node.outputs[0]] = std::move(pa);
+            DeviceTensor o = *in[0];
+            o.dims = shapes[0].dims;
+            copies_avoided_++;
+            outs.push_back(std::move(o));
+        } else {
+            // This Softmax is not one the attention kernel can absorb: compute the scores after all and go on as usual.
+            if (!flush_attention(node.inputs[0], in[0], err)) return false;
+            copies_avoided_--;
+            current_node_ = id;
+            if (!run_device_op(node, op, in, shapes, &outs, err)) return false;
+        }
     } else if (deferred_unary_.count(id) && in[0] && !in[0]->host && in[0]->elem_ty == TensorElemType::F32 && in[0]->pending_op < 0) {
         DeviceTensor o = *in[0];
         o.dims = shapes[0].dims;

@@ -182,12 +182,18 @@ private:
         DeviceTensor q, k;
         MatOperand Q, K;
         std::vector<size_t> bd;  // batch axes (extent-1 axes dropped), at most two
+        FixedDimensions score_dims;
+        DeviceTensor mask;       // the Softmax's absorbed mask (one value per key), if any
+        size_t mask_outer_stride = 0;
     };
     struct AttentionPlan {
         NodeId softmax, tail;
         int scale_op = 0;
         float scale = 1.0f;
+        bool has_mask = false;
     };
+    // Undoes a deferral: runs the first product of a pending attention into real scores.
+    bool flush_attention(ValueId scores, DeviceTensor *placeholder, SessionError *err);
     bool try_defer_attention(const Node &node, const Op &op, const std::vector<DeviceTensor *> &in,
                              const std::vector<TypedFixedShape> &shapes, std::vector<DeviceTensor> *outs, SessionError *err);
     bool run_attention_tail(const Op &op, const std::vector<DeviceTensor *> &in, DeviceTensor *out, SessionError *err);

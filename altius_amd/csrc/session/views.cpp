@@ -29,7 +29,7 @@ bool HipSession::materialize(DeviceTensor *t, SessionError *err) {
 
 bool HipSession::apply_pending(DeviceTensor *t, SessionError *err) {
     if (t->pending_op < 0) return true;
-    if (t->pending_op == PENDING_ATTENTION)
+    if (t->pending_op == PENDING_ATTENTION)  // callers that know the value's id flush it instead (flush_attention)
         return fail(err, SessionError::Message, "internal: a deferred attention product was read by an operator that cannot finish it");
     if (!materialize(t, err)) return false;
     DeviceTensor done;
@@ -101,6 +101,30 @@ bool aligned_operand(const void *p, size_t ld, const std::vector<int64_t> &bs) {
 }
 }  // namespace
 
+bool HipSession::flush_attention(ValueId scores, DeviceTensor *placeholder, SessionError *err) {
+    auto it = pending_attn_.find(scores);
+    if (it == pending_attn_.end()) return fail(err, SessionError::Message, "internal: no operands kept for a deferred attention product");
+    PendingAttention pa = std::move(it->second);
+    pending_attn_.erase(it);
+    DeviceTensor out;
+    if (!allocate(TypedFixedShape{pa.score_dims, TensorElemType::F32}, &out, err)) return false;
+    const size_t tq = pa.Q.stored_transposed ? pa.Q.cols : pa.Q.rows, tk = pa.K.stored_transposed ? pa.K.cols : pa.K.rows;
+    auto two = [](const std::vector<int64_t> &s, size_t out2[2]) {
+        out2[0] = s.size() > 0 ? (size_t)s[0] : 0;
+        out2[1] = s.size() > 1 ? (size_t)s[1] : 0;
+    };
+    const size_t outer = pa.bd.size() > 0 ? pa.bd[0] : 1, inner = pa.bd.size() > 1 ? pa.bd[1] : 1;
+    size_t q2[2], k2[2], c2[2] = {inner * tq * tk, pa.bd.size() > 1 ? tq * tk : 0};
+    two(pa.Q.bstr, q2), two(pa.K.bstr, k2);
+    // Q rows [tq, 64] times the transpose of K rows [tk, 64].
+    const int rc = launch_gemm_batch2(ctx_, static_cast<float *>(out.ptr), static_cast<const float *>(pa.q.ptr),
+                                      static_cast<const float *>(pa.k.ptr), nullptr, outer, inner, tq, tk, 64, 0, 1, pa.Q.ld, pa.K.ld, tk, q2,
+                                      k2, c2, 0, 1, 1.0f, 0.0f);
+    if (rc) return fail_code(err, rc, ctx_.last_error);
+    *placeholder = std::move(out);
+    return true;
+}
+
 // The first product of MatMul -> Softmax -> MatMul: if the one-kernel attention can take it (64-wide heads,
 // at most 256 keys, at most two batch axes, aligned operands), leave a placeholder and remember Q and K.
 bool HipSession::try_defer_attention(const Node &node, const Op &op, const std::vector<DeviceTensor *> &in,
@@ -130,6 +154,7 @@ bool HipSession::try_defer_attention(const Node &node, const Op &op, const std::
     if (!aligned_operand(in[0]->ptr, pa.Q.ld, qs) || !aligned_operand(in[1]->ptr, pa.K.ld, ks)) return true;
     pa.Q.bstr = qs, pa.K.bstr = ks;  // now per axis of bd
     pa.q = *in[0], pa.k = *in[1];
+    pa.score_dims = od;
     pending_attn_[node.outputs[0]] = std::move(pa);
     DeviceTensor o;
     o.dims = od;
@@ -198,7 +223,8 @@ bool HipSession::run_attention_tail(const Op &op, const std::vector<DeviceTensor
     const size_t outer = pa.bd.size() > 0 ? pa.bd[0] : 1, inner = pa.bd.size() > 1 ? pa.bd[1] : 1;
     const int rc = launch_attention(ctx_, static_cast<float *>(out->ptr), static_cast<const float *>(pa.q.ptr),
                                     static_cast<const float *>(pa.k.ptr), static_cast<const float *>(in[1]->ptr), outer, inner, tq, tk, 64,
-                                    pa.Q.ld, pa.K.ld, V.ld, ldo, q2, k2, v2, o2, plan->scale_op, plan->scale);
+                                    pa.Q.ld, pa.K.ld, V.ld, ldo, q2, k2, v2, o2, plan->scale_op, plan->scale,
+                                    pa.mask.ptr ? static_cast<const float *>(pa.mask.ptr) : nullptr, pa.mask_outer_stride);
     if (rc) return fail_code(err, rc, ctx_.last_error);
     return true;
 }
@@ -254,12 +280,13 @@ void HipSession::plan_views() {
                 const NodeId sid = *it->second.begin();
                 const Node &sm = g.nodes[sid];
                 if (sm.op.kind == OpKind::Softmax && n.inputs.size() == 2 && !sm.inputs.empty() && sm.inputs[0] == n.outputs[0] &&
-                    !sm.op.prologue_mask && sm.outputs.size() == 1 && !is_output(sm.outputs[0])) {
+                    sm.outputs.size() == 1 && !is_output(sm.outputs[0])) {
                     bool last_axis = sm.op.axis == -1;
                     auto sh = inferred_.find(sid);
                     if (!last_axis && sh != inferred_.end() && !sh->second.second.empty())
                         last_axis = sm.op.axis == (int64_t)sh->second.second[0].dims.len() - 1;
                     AttentionPlan ap;
+                    ap.has_mask = sm.op.prologue_mask != 0;
                     bool scale_ok = true;
                     if (sm.op.prologue_scale) {
                         auto init = sm.inputs.size() > 1 ? g.inits.find(sm.inputs[1]) : g.inits.end();

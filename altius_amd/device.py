@@ -411,8 +411,9 @@ class Context:
         check(self.L.ahip_gemm(self.handle, c_ptr, a_ptr, b_ptr, c0_ptr, batch, m, n, k, int(trans_a), int(trans_b), lda,
                                ldb, ldc, a_bs, b_bs, c_bs, c0_rs, c0_cs, alpha, beta), self.handle)
 
-    def attention(self, q, k, v, scale_op=0, scale=1.0):
-        """Softmax(scale(Q K^T)) V for q [..., tq, 64], k / v [..., tk, 64] (same leading shape), in one kernel."""
+    def attention(self, q, k, v, scale_op=0, scale=1.0, mask=None):
+        """Softmax(scale(Q K^T) + mask) V for q [..., tq, 64], k / v [..., tk, 64] (same leading shape), in one kernel;
+        mask: [tk] (shared) or [q.shape[0], tk] (one row per leading batch)."""
         q, k, v = (np.asarray(x, dtype=np.float32, order="C") for x in (q, k, v))
         tq, d = q.shape[-2:]
         tk = k.shape[-2]
@@ -420,12 +421,19 @@ class Context:
         dq, dk, dv = self.upload(q), self.upload(k), self.upload(v)
         do = self.alloc(max(q.nbytes, 4))
         S = ctypes.c_size_t * 2
+        dm, outer, inner, mstride = None, batch, 1, 0
+        if mask is not None:
+            mask = np.asarray(mask, dtype=np.float32, order="C")
+            dm = self.upload(mask)
+            if mask.ndim == 2:
+                outer, inner, mstride = q.shape[0], batch // q.shape[0], tk
         try:
-            check(self.L.ahip_attention(self.handle, do.ptr, dq.ptr, dk.ptr, dv.ptr, batch, 1, tq, tk, d, d, d, d, d, S(tq * d, 0),
-                                        S(tk * d, 0), S(tk * d, 0), S(tq * d, 0), scale_op, scale), self.handle)
+            check(self.L.ahip_attention(self.handle, do.ptr, dq.ptr, dk.ptr, dv.ptr, outer, inner, tq, tk, d, d, d, d, d,
+                                        S(inner * tq * d, tq * d), S(inner * tk * d, tk * d), S(inner * tk * d, tk * d),
+                                        S(inner * tq * d, tq * d), scale_op, scale, dm.ptr if dm else None, mstride), self.handle)
             return self.download(do, q.shape)
         finally:
-            for x in (dq, dk, dv, do):
+            for x in (dq, dk, dv, do) + ((dm,) if dm else ()):
                 self.free(x)
 
     def gemm_set_algorithm(self, algorithm):

@@ -378,7 +378,7 @@ def build_next_rows(ctx, D, batch=256):
     rows.append(("Attention %d x Softmax(QK^T/8)V [197,64], one kernel" % (batch * NH), 4 * batch * T * 4 * H,
                  2.0 * batch * NH * (2 * T * T * DH),
                  lambda: check(L.ahip_attention(h, att.ptr, qkv3.ptr, qkv3.ptr + H * 4, qkv3.ptr + 2 * H * 4, batch, NH, T, T, DH, ld, ld, ld, H,
-                                                S2(T * ld, DH), S2(T * ld, DH), S2(T * ld, DH), S2(T * H, DH), 1, 0.125), h)))
+                                                S2(T * ld, DH), S2(T * ld, DH), S2(T * ld, DH), S2(T * H, DH), 1, 0.125, None, 0), h)))
     return rows
 
 

@@ -279,19 +279,21 @@ int ahip_gemm_activated(ahip_ctx *ctx, int a_op, float *c, const float *a, const
                         size_t n, size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc,
                         size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta);
 
-/* O = Softmax(scale(Q K^T)) V for batch_outer * batch_inner independent (batch, head) pairs in one kernel: the
- * MatMul -> (Mul | Div by a scalar) -> Softmax(last axis) -> MatMul chain of an attention block
+/* O = Softmax(scale(Q K^T) + mask) V for batch_outer * batch_inner independent (batch, head) pairs in one kernel: the
+ * MatMul -> (Mul | Div by a scalar) -> (Add of a per-key mask) -> Softmax(last axis) -> MatMul chain of an attention block
  * (session.rs:621-684, 990-1026) without the [tq, tk] score tensor ever reaching memory.  Q is [tq, d] with row
  * pitch ldq, K and V [tk, d], O [tq, d]; operand X of batch z starts at x + (z / batch_inner) * x_batch_strides[0]
  * + (z % batch_inner) * x_batch_strides[1] (elements), so heads are read out of a [b, t, h * d] tensor and O is
- * written into one in place.  scale_op: 0 none, 1 scores * scale, 2 scores / scale.  Same exp and
+ * written into one in place.  scale_op: 0 none, 1 scores * scale, 2 scores / scale.  mask (may be NULL): one value per
+ * key, added after the scale, read at mask[(z / batch_inner) * mask_outer_stride + key] (stride 0: one row for all
+ * batches; tk: one row per outer batch, the [b, 1, 1, tk] padding mask of BERT-style graphs).  Same exp and
  * reciprocal-multiply normalisation as ahip_softmax_lastaxis; the two products on the fp32 matrix cores.
  * AHIP_ERR_UNSUPPORTED (nothing launched) unless d == 64, 1 <= tk <= 256 and all pointers, pitches and batch
  * strides are multiples of 16 bytes: run the three operators then.  No counterpart in the reference. */
 int ahip_attention(ahip_ctx *ctx, float *o, const float *q, const float *k, const float *v, size_t batch_outer,
                    size_t batch_inner, size_t tq, size_t tk, size_t d, size_t ldq, size_t ldk, size_t ldv, size_t ldo,
                    const size_t q_batch_strides[2], const size_t k_batch_strides[2], const size_t v_batch_strides[2],
-                   const size_t o_batch_strides[2], int scale_op, float scale);
+                   const size_t o_batch_strides[2], int scale_op, float scale, const float *mask, size_t mask_outer_stride);
 
 /* Which kernel ahip_gemm (and the MatMul / Gemm / Conv2d operators of a session on this context) uses
  * for a single-batch product.  AHIP_GEMM_FP32: v_mfma_f32_32x32x2_f32 on the operands as they are.

@@ -51,6 +51,18 @@ def test_attention_with_peaked_and_masked_like_scores(ctx, case):
     assert np.isfinite(rows).all()
 
 
+def test_attention_with_masks(ctx, case):
+    case("attention with per-key masks")
+    q = RNG.standard_normal((3, 2, 40, 64)).astype(np.float32)
+    k = RNG.standard_normal((3, 2, 70, 64)).astype(np.float32)
+    v = RNG.standard_normal((3, 2, 70, 64)).astype(np.float32)
+    for mask in (np.where(RNG.random(70) < 0.3, -1e4, 0.0).astype(np.float32), np.where(RNG.random((3, 70)) < 0.3, -1e4, 0.0).astype(np.float32)):
+        got = ctx.attention(q, k, v, 2, 8.0, mask=mask)
+        s = q.astype(np.float64) @ np.swapaxes(k.astype(np.float64), -1, -2) / 8.0 + (mask if mask.ndim == 1 else mask[:, None, None, :])
+        e = np.exp(s - s.max(-1, keepdims=True))
+        np.testing.assert_allclose(got, (e / e.sum(-1, keepdims=True)) @ v, rtol=2e-4, atol=2e-5)
+
+
 def test_attention_reads_heads_in_place(ctx, case):
     """Q, K, V as column blocks of one [b, t, 3 h d] tensor, O written as [b, t, h d]: row pitches and two-level batches."""
     case("attention on strided heads")
@@ -61,7 +73,7 @@ def test_attention_reads_heads_in_place(ctx, case):
     try:
         ld = 3 * h * d
         check(ctx.L.ahip_attention(ctx.handle, do.ptr, dx.ptr, dx.ptr + h * d * 4, dx.ptr + 2 * h * d * 4, b, h, t, t, d, ld, ld, ld, h * d,
-                                   S(t * ld, d), S(t * ld, d), S(t * ld, d), S(t * h * d, d), 1, 0.125), ctx.handle)
+                                   S(t * ld, d), S(t * ld, d), S(t * ld, d), S(t * h * d, d), 1, 0.125, None, 0), ctx.handle)
         got = ctx.download(do, (b, t, h, d))
     finally:
         ctx.free(dx)

@@ -295,6 +295,7 @@ def test_gemm_activated_through_the_c_abi(ctx, case):
 # ---- MatMul -> Softmax -> MatMul as one kernel ----
 
 def scaled_attention(batch, tq, tk, heads, d, scale_kind, extra_reader=False, mask=False):
+    # mask: False, "keys" ([b, 1, 1, tk], one value per key and batch), "shared" ([tk]) or "queries" ([b, 1, tq, tk])
     """q [b, h, tq, d], k [b, h, tk, d], v [b, h, tk, d] as inputs; scores scaled by Mul / Div of a scalar (or not)."""
     m = Model(opset_version=13)
     q = m.new_val_named_and_shaped("q", [batch, heads, tq, d])
@@ -308,8 +309,10 @@ def scaled_attention(batch, tq, tk, heads, d, scale_kind, extra_reader=False, ma
     elif scale_kind == "div":
         s = node(m, Op.Div, [s, m.new_initializer(np.array(d ** 0.5, np.float32))])
     if mask:
-        mk = np.where(RNG.random((batch, 1, 1, tk)) < 0.2, np.float32(-1e4), np.float32(0)).astype(np.float32)
+        shape = {"keys": (batch, 1, 1, tk), "shared": (tk,), "queries": (batch, 1, tq, tk)}[mask]
+        mk = np.where(RNG.random(shape) < 0.2, np.float32(-1e4), np.float32(0)).astype(np.float32)
         s = node(m, Op.Add, [s, m.new_initializer(mk)])
+        m.mask_values = mk
     p = node(m, Op.Softmax, [s], axis=-1)
     m.add_output(node(m, Op.MatMul, [p, v]))
     if extra_reader:
@@ -333,7 +336,21 @@ def test_attention_triple_becomes_one_kernel(case, batch, tq, tk, heads, scale_k
     np.testing.assert_allclose(got, (e / e.sum(-1, keepdims=True)) @ v, rtol=2e-4, atol=2e-5)
 
 
-@pytest.mark.parametrize("why", ["more than 256 keys", "narrow heads", "second reader of the probabilities", "masked scores"])
+@pytest.mark.parametrize("mask", ["keys", "shared"])
+def test_attention_with_a_per_key_mask(case, mask):
+    """The padding mask of BERT-style graphs, absorbed by the Softmax and from there by the attention kernel."""
+    case(f"session attention with a {mask} mask")
+    batch, tq, tk, heads = 3, 37, 50, 2
+    m = scaled_attention(batch, tq, tk, heads, 64, "div", mask=mask)
+    q, k, v = (RNG.standard_normal((batch, heads, t, 64)).astype(np.float32) for t in (tq, tk, tk))
+    (got,), avoided = run_both(m, [q, k, v], exact=False)
+    assert avoided == 2, avoided
+    s = q.astype(np.float64) @ k.astype(np.float64).transpose(0, 1, 3, 2) / np.float32(8.0) + m.mask_values
+    e = np.exp(s - s.max(-1, keepdims=True))
+    np.testing.assert_allclose(got, (e / e.sum(-1, keepdims=True)) @ v, rtol=2e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize("why", ["more than 256 keys", "narrow heads", "second reader of the probabilities", "mask per query"])
 def test_attention_triples_that_stay_three_operators(case, why):
     case(f"attention not fused: {why}")
     kw = dict(batch=2, tq=20, tk=40, heads=2, d=64, scale_kind="mul")
@@ -344,7 +361,7 @@ def test_attention_triples_that_stay_three_operators(case, why):
     elif why == "second reader of the probabilities":
         kw["extra_reader"] = True
     else:
-        kw["mask"] = True
+        kw["mask"] = "queries"    # found only when the Softmax runs: the deferred first product is computed after all
     m = scaled_attention(**kw)
     q, k, v = (RNG.standard_normal((kw["batch"], kw["heads"], t, kw["d"])).astype(np.float32) for t in (kw["tq"], kw["tk"], kw["tk"]))
     outs, avoided = run_both(m, [q, k, v])          # bit for bit: nothing may have changed
