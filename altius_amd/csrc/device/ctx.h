@@ -137,7 +137,7 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
 // O = Softmax(scale(Q K^T) + mask) V per batch, scores kept in registers (attention.hip).  Q [tq, d], K [tk, d], V [tk, d],
 // O [tq, d] with row pitches ld*; batches as in launch_gemm_batch2; scale_op 0 none / 1 multiply / 2 divide; mask (may be
 // null) one value per key, read at mask[outer batch * mask_outer_stride + key].
-// AHIP_ERR_UNSUPPORTED (nothing launched) unless d == 64, tk <= 256 and everything is 16-byte aligned.
+// AHIP_ERR_UNSUPPORTED (nothing launched) unless d == 64 and everything is 16-byte aligned.
 int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, const float *v, size_t batch_outer, size_t batch_inner,
                      size_t tq, size_t tk, size_t d, size_t ldq, size_t ldk, size_t ldv, size_t ldo, const size_t q_bs[2],
                      const size_t k_bs[2], const size_t v_bs[2], const size_t o_bs[2], int scale_op, float scale, const float *mask = nullptr,

@@ -126,7 +126,7 @@ bool HipSession::flush_attention(ValueId scores, DeviceTensor *placeholder, Sess
 }
 
 // The first product of MatMul -> Softmax -> MatMul: if the one-kernel attention can take it (64-wide heads,
-// at most 256 keys, at most two batch axes, aligned operands), leave a placeholder and remember Q and K.
+// at most two batch axes, aligned operands), leave a placeholder and remember Q and K.
 bool HipSession::try_defer_attention(const Node &node, const Op &op, const std::vector<DeviceTensor *> &in,
                                      const std::vector<TypedFixedShape> &shapes, std::vector<DeviceTensor> *outs, SessionError *err) {
     if (in.size() != 2 || !in[0] || !in[1] || in[0]->elem_ty != TensorElemType::F32 || in[1]->elem_ty != TensorElemType::F32) return true;
@@ -139,7 +139,7 @@ bool HipSession::try_defer_attention(const Node &node, const Op &op, const std::
     if (!q_rows || !k_rows) return true;
     const size_t tq = pa.Q.stored_transposed ? pa.Q.cols : pa.Q.rows, d = pa.Q.stored_transposed ? pa.Q.rows : pa.Q.cols;
     const size_t tk = pa.K.stored_transposed ? pa.K.cols : pa.K.rows, dk = pa.K.stored_transposed ? pa.K.rows : pa.K.cols;
-    if (d != 64 || dk != 64 || tk == 0 || tk > 256 || tq == 0) return true;
+    if (d != 64 || dk != 64 || tk == 0 || tq == 0) return true;
     const FixedDimensions &od = shapes[0].dims;
     size_t batch = 1;
     for (size_t i = 0; i + 2 < od.len(); i++) {

@@ -288,8 +288,8 @@ int ahip_gemm_activated(ahip_ctx *ctx, int a_op, float *c, const float *a, const
  * key, added after the scale, read at mask[(z / batch_inner) * mask_outer_stride + key] (stride 0: one row for all
  * batches; tk: one row per outer batch, the [b, 1, 1, tk] padding mask of BERT-style graphs).  Same exp and
  * reciprocal-multiply normalisation as ahip_softmax_lastaxis; the two products on the fp32 matrix cores.
- * AHIP_ERR_UNSUPPORTED (nothing launched) unless d == 64, 1 <= tk <= 256 and all pointers, pitches and batch
- * strides are multiples of 16 bytes: run the three operators then.  No counterpart in the reference. */
+ * AHIP_ERR_UNSUPPORTED (nothing launched) unless d == 64 and all pointers, pitches and batch strides are
+ * multiples of 16 bytes: run the three operators then.  Any number of keys (they are streamed 64 at a time).  No counterpart in the reference. */
 int ahip_attention(ahip_ctx *ctx, float *o, const float *q, const float *k, const float *v, size_t batch_outer,
                    size_t batch_inner, size_t tq, size_t tk, size_t d, size_t ldq, size_t ldk, size_t ldv, size_t ldo,
                    const size_t q_batch_strides[2], const size_t k_batch_strides[2], const size_t v_batch_strides[2],

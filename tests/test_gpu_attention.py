@@ -84,8 +84,21 @@ def test_attention_reads_heads_in_place(ctx, case):
 
 def test_attention_refuses_what_it_cannot_do(ctx, case):
     case("attention refusals")
-    for shape_q, shape_k in (((4, 32), (4, 32)), ((4, 64), (300, 64))):
-        q, k = np.zeros(shape_q, np.float32), np.zeros(shape_k, np.float32)
-        with pytest.raises(AltiusHipError) as e:
-            ctx.attention(q, k, k)
-        assert e.value.code == ERR_UNSUPPORTED
+    q = np.zeros((4, 32), np.float32)               # heads that are not 64 wide
+    with pytest.raises(AltiusHipError) as e:
+        ctx.attention(q, q, q)
+    assert e.value.code == ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("tq,tk", [(50, 257), (128, 512), (33, 1000), (300, 300)])
+def test_long_sequences_are_streamed(ctx, case, tq, tk):
+    """More than 256 keys: chunks of 64 keys through LDS with a running maximum and sum per query."""
+    case(f"streamed attention tq {tq} tk {tk}")
+    q = RNG.standard_normal((2, 2, tq, 64)).astype(np.float32)
+    k = RNG.standard_normal((2, 2, tk, 64)).astype(np.float32)
+    v = RNG.standard_normal((2, 2, tk, 64)).astype(np.float32)
+    mask = np.where(RNG.random((2, tk)) < 0.2, -1e4, 0.0).astype(np.float32)
+    got = ctx.attention(q, k, v, 1, 0.125, mask=mask)
+    s = q.astype(np.float64) @ np.swapaxes(k.astype(np.float64), -1, -2) * 0.125 + mask[:, None, None, :]
+    e = np.exp(s - s.max(-1, keepdims=True))
+    np.testing.assert_allclose(got, (e / e.sum(-1, keepdims=True)) @ v, rtol=2e-4, atol=2e-5)
