@@ -277,19 +277,21 @@ __global__ __launch_bounds__(THREADS, 1) void gemm_bf16x3(SplitGemmArgs g) {
     }
 #undef STEP
 
-    // A tile cut along k: every block leaves its partial sums in `partials` (register r of thread t at
-    // [r][t]: coalesced), and the block that arrives last adds them up in slice order, so the result does not
+    // A tile cut along k: every block leaves its partial sums in `partials` (coalesced 16-byte stores), and the block that arrives last adds them up in slice order, so the result does not
     // depend on who was last, and goes on to the epilogue.  All slices of a tile run on one XCD (one L2).
     if (nparts > 1) {
         __shared__ int arrived;
         const uint32_t idx = xcd * (g.chunk - g.full) + (local - g.full);
-        float *mine = g.partials + ((size_t)idx * nparts + part) * (TM * TN);
+        // Four accumulator registers per 16-byte store: [register / 4][thread][4].
+        f32x4 *mine = reinterpret_cast<f32x4 *>(g.partials + ((size_t)idx * nparts + part) * (TM * TN)) + tid;
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) mine[(size_t)((i * 4 + j) * 16 + r) * THREADS + tid] = acc[i][j][r];
+                for (int r4 = 0; r4 < 4; r4++)
+                    mine[(size_t)((i * 4 + j) * 4 + r4) * THREADS] =
+                        f32x4{acc[i][j][4 * r4], acc[i][j][4 * r4 + 1], acc[i][j][4 * r4 + 2], acc[i][j][4 * r4 + 3]};
         // The partial sums only have to reach this XCD's L2, where the other slices' blocks read them: stores
         // write through the L1, and vmcnt(0) says the L2 has them.  (A device-wide release fence here would
         // write the whole L2 back, once per wavefront.)
@@ -299,8 +301,8 @@ __global__ __launch_bounds__(THREADS, 1) void gemm_bf16x3(SplitGemmArgs g) {
         if (arrived != (int)nparts - 1) return;
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // nothing stale in this CU's L1
         if (tid == 0) atomicExch(&g.counters[idx], 0);      // ready for the next launch
-        // Sum in slice order, 64 registers' worth of loads in flight at a time.
-        const float *all = g.partials + (size_t)idx * nparts * (TM * TN) + tid;
+        // Sum in slice order, 64 registers' worth of 16-byte loads in flight at a time.
+        const f32x4 *all = reinterpret_cast<const f32x4 *>(g.partials + (size_t)idx * nparts * (TM * TN)) + tid;
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -308,16 +310,19 @@ __global__ __launch_bounds__(THREADS, 1) void gemm_bf16x3(SplitGemmArgs g) {
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
         for (uint32_t q = 0; q < nparts; q++) {
-            const float *src = all + (size_t)q * (TM * TN);
+            const f32x4 *src = all + (size_t)q * (TM * TN / 4);
 #pragma unroll
             for (int i = 0; i < 2; i++) {
-                float tmp[64];
+                f32x4 tmp[16];
 #pragma unroll
-                for (int e = 0; e < 64; e++) tmp[e] = src[(size_t)(i * 64 + e) * THREADS];
+                for (int e = 0; e < 16; e++) tmp[e] = src[(size_t)(i * 16 + e) * THREADS];
 #pragma unroll
                 for (int j = 0; j < 4; j++)
 #pragma unroll
-                    for (int r = 0; r < 16; r++) acc[i][j][r] += tmp[j * 16 + r];
+                    for (int r4 = 0; r4 < 4; r4++) {
+                        const f32x4 t = tmp[j * 4 + r4];
+                        acc[i][j][4 * r4] += t.x, acc[i][j][4 * r4 + 1] += t.y, acc[i][j][4 * r4 + 2] += t.z, acc[i][j][4 * r4 + 3] += t.w;
+                    }
             }
         }
     }
