@@ -150,6 +150,8 @@ int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, c
 int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t m, size_t n, size_t k,
                       int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t c0_row_stride, size_t c0_col_stride,
                       float alpha, float beta, int a_op = 0);
+// The context's grow-only GEMM workspace, at least `bytes` large (stream-ordered use only).
+int gemm_workspace(DeviceCtx &ctx, size_t bytes, void **p);
 // Whether launch_gemm would send this single-batch product through launch_gemm_split.
 bool gemm_takes_split(const DeviceCtx &ctx, size_t m, size_t n, size_t k);
 // Large and tile-filling enough for the split kernel to win (the AHIP_GEMM_AUTO rule).

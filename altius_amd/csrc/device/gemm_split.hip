@@ -507,15 +507,19 @@ int ensure_partials(DeviceCtx &ctx, size_t bytes) {
 
 }  // namespace
 
+int gemm_workspace(DeviceCtx &ctx, size_t bytes, void **p) {
+    const int rc = ensure_workspace(ctx, bytes);
+    *p = rc ? nullptr : ctx.gemm_ws;
+    return rc;
+}
+
 bool gemm_split_worthwhile(size_t m, size_t n, size_t k) {
-    // Large products whose C fills most of its 256 x 256 tiles; also products with few rows and a long k (one image
-    // through a transformer layer: [197, 768] x [768, 2304]), where cutting the tiles along k spreads the k loop over
-    // the CUs that the few tiles leave idle: measured 3.7 against 4.7 ms for a ViT-B/16 encoder at batch 1.
-    if (m < 128 || n < 256 || k < 256) return false;
+    // Large products whose C fills most of its 256 x 256 tiles.  Products with few rows (one image through a
+    // transformer layer: [197, 768] x [768, 2304]) are faster on the fp32 kernel with k cut into batches: its
+    // tiles are smaller and nothing has to be split into planes first (30 against 49 us for that shape).
+    if (m < 1024 || n < 256 || k < 128) return false;
     const double useful = (double)m * (double)n / ((double)round_up(m, TM) * (double)round_up(n, TN));
-    const double work = (double)m * (double)n * (double)k;
-    if (m >= 1024) return useful >= 0.8 && work >= 2147483648.0;
-    return useful >= 0.5 && work >= 100e6;
+    return useful >= 0.8 && (double)m * (double)n * (double)k >= 2147483648.0;
 }
 
 int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t m, size_t n, size_t k,

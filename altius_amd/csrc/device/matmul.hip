@@ -13,6 +13,7 @@
 // one barrier per K tile.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <type_traits>
 
 #include "common.h"
@@ -221,7 +222,23 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_mfma(GemmArgs g) {
         }
 }
 
+// C = alpha * (sum over k slices, in slice order) + beta * C0: the second half of a product cut along k.
+__global__ __launch_bounds__(256) void splitk_finish(float *__restrict__ c, const float *__restrict__ partials, uint32_t slices,
+                                                     uint32_t m, uint32_t n, uint32_t ldc, const float *__restrict__ c0, uint32_t c0_rs,
+                                                     uint32_t c0_cs, float alpha, float beta) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, total = (size_t)m * n;
+    if (i >= total) return;
+    float sum = partials[i];
+    for (uint32_t s = 1; s < slices; s++) sum += partials[(size_t)s * total + i];
+    const uint32_t row = (uint32_t)(i / n), col = (uint32_t)(i % n);
+    float v = alpha * sum;
+    if (c0) v += beta * c0[(size_t)row * c0_rs + (size_t)col * c0_cs];
+    c[(size_t)row * ldc + col] = v;
+}
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+thread_local bool split_k_inner = false;  // the batched launch of the slices must not cut again
 
 }  // namespace
 
@@ -258,6 +275,32 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
     const size_t tn = narrow ? 64 : BN;
     const size_t gy = (m + BM - 1) / BM, gx = (n + tn - 1) / tn;
     if (gy > 65535 || batch > 65535) return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm: more than 65535 row tiles or batches");
+    // A single product with few tiles and a long k (one image through a transformer layer) leaves most CUs idle
+    // while each block walks all of k: cut k into slices that run as batches into a workspace, and add the
+    // slices up in order afterwards (the bias and alpha / beta go there).
+    if (batch == 1 && ctx.gemm_split_k && gx * gy <= 128 && k >= 512 && !split_k_inner) {
+        const size_t cus = ctx.cus_per_xcd ? (size_t)ctx.cus_per_xcd * 8 : 256;
+        size_t slices = std::min<size_t>(std::min<size_t>((cus + gx * gy - 1) / (gx * gy), k / 128), 16);
+        while (slices > 1 && k % (slices * 16) != 0) slices--;  // equal slices of whole k tiles
+        if (slices >= 2) {
+            void *ws = nullptr;
+            int rc = gemm_workspace(ctx, slices * m * n * sizeof(float), &ws);
+            if (rc) return rc;
+            const size_t ks = k / slices;
+            // slice z of op(A) starts ks columns (or rows, transposed) further on; likewise op(B)
+            const size_t a_bs[2] = {trans_a ? ks * lda : ks, 0}, b_bs[2] = {trans_b ? ks : ks * ldb, 0}, c_bs[2] = {m * n, 0};
+            split_k_inner = true;
+            rc = launch_gemm_batch2(ctx, static_cast<float *>(ws), a, b, nullptr, slices, 1, m, n, ks, trans_a, trans_b, lda, ldb, n, a_bs, b_bs,
+                                    c_bs, 0, 0, 1.0f, 0.0f);
+            split_k_inner = false;
+            if (rc) return rc;
+            const size_t total = m * n;
+            hipLaunchKernelGGL(splitk_finish, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx.stream, c, static_cast<const float *>(ws),
+                               (uint32_t)slices, (uint32_t)m, (uint32_t)n, (uint32_t)ldc, (c0 && beta != 0.0f) ? c0 : nullptr,
+                               (uint32_t)c0_row_stride, (uint32_t)c0_col_stride, alpha, beta);
+            return ctx.check(hipGetLastError(), "gemm split-k finish launch");
+        }
+    }
     GemmArgs g;
     g.a = a;
     g.b = b;

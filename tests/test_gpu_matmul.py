@@ -214,3 +214,23 @@ def test_transposes_folded_into_the_product(case, a_shape, b_shape, ta, tb):
     A = np.swapaxes(a, -1, -2) if ta else a
     Bm = np.swapaxes(b, -1, -2) if tb else b
     np.testing.assert_allclose(got, np.matmul(A.astype(np.float64), Bm.astype(np.float64)), rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("m,k,n", [(197, 768, 2304), (197, 3072, 768), (100, 1024, 64), (8, 4096, 130), (300, 512, 300)])
+def test_few_tiles_and_a_long_k_are_cut_along_k(ctx, case, m, k, n):
+    """Few output tiles and k >= 512: k runs as batches of slices into a workspace and a second kernel adds the slices up
+    in order (bias, alpha and beta applied there).  Exact on integers, bounded on reals, every C0 shape, both transposes."""
+    from altius_amd import device as D
+
+    case(f"split-k gemm {m}x{k}x{n}")
+    try:
+        ctx.gemm_set_algorithm(D.GEMM_FP32)
+        for ta, tb in ((False, False), (True, True), (False, True)):
+            a, b = ints(*((k, m) if ta else (m, k))), ints(*((n, k) if tb else (k, n)))
+            for c in (None, ints(n), ints(m, n), ints(m, 1)):
+                got = ctx.gemm(a, b, c, alpha=2.0, beta=3.0, trans_a=ta, trans_b=tb)
+                assert_bits_equal(got, O.gemm(a, b, c, alpha=2.0, beta=3.0, trans_a=ta, trans_b=tb), f"ta={ta} tb={tb} c={None if c is None else c.shape}")
+        a, b = RNG.standard_normal((m, k)).astype(np.float32), RNG.standard_normal((k, n)).astype(np.float32)
+        check_bound(ctx.matmul(a, b), a, b, "random operands")
+    finally:
+        ctx.gemm_set_algorithm(D.GEMM_AUTO)
