@@ -53,7 +53,10 @@ struct AttnArgs {
 
 constexpr int KC = 64;  // keys per chunk
 
-__global__ __launch_bounds__(64 * MAX_WAVES, 4) void attention_stream_d64(AttnArgs g) {
+// W: wavefronts (tiles of 32 queries) per block.  Fewer when there are few (batch, head) pairs, so that the queries of
+// one pair spread over several CUs; every block stages the keys and values it needs itself.
+template <int W>
+__global__ __launch_bounds__(64 * W, W == 8 ? 4 : 1) void attention_stream_d64(AttnArgs g) {
     __shared__ __align__(16) float ks[2][KC * K_PITCH];
     __shared__ __align__(16) float vs[2][KC * D];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -64,24 +67,25 @@ __global__ __launch_bounds__(64 * MAX_WAVES, 4) void attention_stream_d64(AttnAr
     const float *v = g.v + zo * g.v_bs[0] + zi * g.v_bs[1];
     float *o = g.o + zo * g.o_bs[0] + zi * g.o_bs[1];
     const float *mask = g.mask ? g.mask + (size_t)zo * g.mask_outer_stride : nullptr;
-    const uint32_t query = (blockIdx.y * MAX_WAVES + wave) * 32 + lr;
-    const bool active = (blockIdx.y * MAX_WAVES + wave) * 32 < g.tq;  // wavefronts without queries still help staging
+    const uint32_t query = (blockIdx.y * W + wave) * 32 + lr;
+    const bool active = (blockIdx.y * W + wave) * 32 < g.tq;  // wavefronts without queries still help staging
     const uint32_t nchunks = (g.tk + KC - 1) / KC;
 
-    // Staging: 512 threads move 32 rows of 16 float4 per pass, two passes per operand and chunk.
+    // Staging: the block's threads move 4 W rows of 16 float4 per pass, 16 / W passes per operand and chunk.
+    constexpr int PASSES = 16 / W, ROWS = 4 * W;
     const uint32_t r0 = tid >> 4, c4 = tid & 15;
-    f32x4 stage[2];
+    f32x4 stage[PASSES];
     auto fetch = [&](const float *base, uint32_t ld, uint32_t chunk) {
 #pragma unroll
-        for (int it = 0; it < 2; it++) {
-            const uint32_t row = chunk * KC + it * 32 + r0;
+        for (int it = 0; it < PASSES; it++) {
+            const uint32_t row = chunk * KC + it * ROWS + r0;
             stage[it] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
             if (row < g.tk) stage[it] = *reinterpret_cast<const f32x4 *>(base + (size_t)row * ld + c4 * 4);
         }
     };
     auto park = [&](float *dst, int pitch) {
 #pragma unroll
-        for (int it = 0; it < 2; it++) *reinterpret_cast<f32x4 *>(dst + (it * 32 + r0) * pitch + c4 * 4) = stage[it];
+        for (int it = 0; it < PASSES; it++) *reinterpret_cast<f32x4 *>(dst + (it * ROWS + r0) * pitch + c4 * 4) = stage[it];
     };
     fetch(k, g.ldk, 0);
     park(ks[0], K_PITCH);
@@ -217,12 +221,17 @@ int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, c
     g.scale = scale;
     g.mask = mask;
     g.mask_outer_stride = (uint32_t)mask_outer_stride;
-    const size_t q_tiles = (tq + 31) / 32;
-    const size_t gy = (q_tiles + MAX_WAVES - 1) / MAX_WAVES;
+    // As many query tiles per block as still leave a block for most CUs.
+    const size_t q_tiles = (tq + 31) / 32, cus = ctx.cus_per_xcd ? (size_t)ctx.cus_per_xcd * 8 : 256;
+    size_t w = MAX_WAVES;
+    while (w > 1 && batch * ((q_tiles + w - 1) / w) < cus) w /= 2;
+    const size_t gy = (q_tiles + w - 1) / w;
     if (gy > 65535) return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: too many queries");
-    const unsigned threads = 64 * MAX_WAVES;
     const dim3 grid((unsigned)batch, (unsigned)gy);
-    hipLaunchKernelGGL(attention_stream_d64, grid, dim3(threads), 0, ctx.stream, g);
+    if (w == 8) hipLaunchKernelGGL(attention_stream_d64<8>, grid, dim3(512), 0, ctx.stream, g);
+    else if (w == 4) hipLaunchKernelGGL(attention_stream_d64<4>, grid, dim3(256), 0, ctx.stream, g);
+    else if (w == 2) hipLaunchKernelGGL(attention_stream_d64<2>, grid, dim3(128), 0, ctx.stream, g);
+    else hipLaunchKernelGGL(attention_stream_d64<1>, grid, dim3(64), 0, ctx.stream, g);
     return ctx.check(hipGetLastError(), "attention launch");
 }
 

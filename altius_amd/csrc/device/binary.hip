@@ -275,6 +275,39 @@ __global__ __launch_bounds__(BLOCK) void binary_rowbcast(float *__restrict__ out
     }
 }
 
+// ---------------------------------------------------------------------------
+// Two-axis kernel for rows that are whole float4s: out[r][c] = full[r][c] op small[c]
+// (a bias or scale vector on rows longer than the row-broadcast kernel stages) or
+// out[r][c] = full[r][c] op small[r] (a per-row mean or deviation).  A lane's four
+// elements lie in one row, so the dense 16-byte load goes out before any index
+// arithmetic and the small operand costs one more load: 16 bytes that hit in L1, or
+// one dword that most lanes of the wavefront share.
+// ---------------------------------------------------------------------------
+enum { SMALL_VECTOR = 0, SMALL_COLUMN = 1 };
+
+template <class OP, int KIND, bool SMALL_IS_A, bool NT>
+__global__ __launch_bounds__(BLOCK) void binary_rows4(float *__restrict__ out, const float *__restrict__ full,
+                                                      const float *__restrict__ small, uint32_t total,
+                                                      const FastDiv c) {
+    const uint32_t i0 = (blockIdx.x * BLOCK + threadIdx.x) * 4;
+    if (i0 >= total) return;  // total is a multiple of 4
+    const float4 x = load4<NT>(full + i0);
+    const uint32_t row = c.div(i0);
+    float4 y;
+    if (KIND == SMALL_VECTOR) {
+        y = *reinterpret_cast<const float4 *>(small + (i0 - row * c.d));
+    } else {
+        const float v = small[row];
+        y = make_float4(v, v, v, v);
+    }
+    float4 r;
+    r.x = SMALL_IS_A ? OP::f(y.x, x.x) : OP::f(x.x, y.x);
+    r.y = SMALL_IS_A ? OP::f(y.y, x.y) : OP::f(x.y, y.y);
+    r.z = SMALL_IS_A ? OP::f(y.z, x.z) : OP::f(x.z, y.z);
+    r.w = SMALL_IS_A ? OP::f(y.w, x.w) : OP::f(x.w, y.w);
+    store4<NT>(out + i0, r);
+}
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <class OP, int MA, int MB>
@@ -341,6 +374,22 @@ void rowbcast_launch(hipStream_t s, bool small_is_a, bool nt, float *out, const 
         if (nt) hipLaunchKernelGGL((binary_rowbcast<OP, false, true>), grid, dim3(BLOCK), shmem, s, out, full, small, g);
         else hipLaunchKernelGGL((binary_rowbcast<OP, false, false>), grid, dim3(BLOCK), shmem, s, out, full, small, g);
     }
+}
+
+template <class OP>
+void rows4_launch(hipStream_t s, int kind, bool small_is_a, bool nt, float *out, const float *full, const float *small,
+                  uint32_t total, const FastDiv &c) {
+    const dim3 grid((total / 4 + BLOCK - 1) / BLOCK);
+#define ALTIUS_ROWS4(K, A, N) \
+    hipLaunchKernelGGL((binary_rows4<OP, K, A, N>), grid, dim3(BLOCK), 0, s, out, full, small, total, c)
+    if (kind == SMALL_VECTOR) {
+        if (small_is_a) { if (nt) ALTIUS_ROWS4(SMALL_VECTOR, true, true); else ALTIUS_ROWS4(SMALL_VECTOR, true, false); }
+        else { if (nt) ALTIUS_ROWS4(SMALL_VECTOR, false, true); else ALTIUS_ROWS4(SMALL_VECTOR, false, false); }
+    } else {
+        if (small_is_a) { if (nt) ALTIUS_ROWS4(SMALL_COLUMN, true, true); else ALTIUS_ROWS4(SMALL_COLUMN, true, false); }
+        else { if (nt) ALTIUS_ROWS4(SMALL_COLUMN, false, true); else ALTIUS_ROWS4(SMALL_COLUMN, false, false); }
+    }
+#undef ALTIUS_ROWS4
 }
 
 }  // namespace
@@ -458,6 +507,30 @@ int launch_binary(DeviceCtx &ctx, int op, float *out, const float *a, const floa
             case AHIP_POW: rowbcast_launch<OpPow>(s, small_is_a, nt, out, full, small, rb); break;
             }
             return ctx.check(hipGetLastError(), "binary row-broadcast launch");
+        }
+    }
+
+    // Two axes, rows of whole float4s, one operand dense and the other a vector along the row
+    // (strides [0,1]) or one value per row (strides [1,0]).
+    {
+        const int64_t *ss = ma == STRIDED ? as : bs;
+        const int other = ma == STRIDED ? mb : ma;
+        const bool small_is_a = ma == STRIDED;
+        const float *full = small_is_a ? b : a;
+        const float *small = small_is_a ? a : b;
+        const bool vector = r == 2 && ss[0] == 0 && ss[1] == 1, column = r == 2 && ss[0] == 1 && ss[1] == 0;
+        if (other == FULL && (vector || column) && dims[1] % 4 == 0 && total < LIMIT && aligned16(out) &&
+            aligned16(full) && (column || aligned16(small))) {
+            const FastDiv c = make_fastdiv((uint32_t)dims[1]);
+            const int kind = vector ? SMALL_VECTOR : SMALL_COLUMN;
+            switch (op) {
+            case AHIP_ADD: rows4_launch<OpAdd>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c); break;
+            case AHIP_SUB: rows4_launch<OpSub>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c); break;
+            case AHIP_MUL: rows4_launch<OpMul>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c); break;
+            case AHIP_DIV: rows4_launch<OpDiv>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c); break;
+            case AHIP_POW: rows4_launch<OpPow>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c); break;
+            }
+            return ctx.check(hipGetLastError(), "binary two-axis launch");
         }
     }
 

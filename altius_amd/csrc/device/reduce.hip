@@ -42,7 +42,7 @@ template <class OP> __device__ __forceinline__ float fold4(float acc, const floa
 
 // Accumulates x[begin..end) strided over `nthreads` lanes starting at `tid`.
 // VEC == 4 requires x + begin 16-byte aligned; the range length may be ragged.
-template <class OP, int VEC>
+template <class OP, int VEC, bool NT = false>
 __device__ __forceinline__ float strided_fold(const float *__restrict__ x, size_t begin, size_t end, int tid,
                                               int nthreads) {
     float acc0 = OP::identity(), acc1 = OP::identity(), acc2 = OP::identity(), acc3 = OP::identity();
@@ -51,16 +51,27 @@ __device__ __forceinline__ float strided_fold(const float *__restrict__ x, size_
         const size_t n4 = (end - begin) >> 2;
         size_t i = tid;
         for (; i + 3 * (size_t)nthreads < n4; i += 4 * (size_t)nthreads) {
-            const float4 a = x4[i];
-            const float4 b = x4[i + nthreads];
-            const float4 c = x4[i + 2 * (size_t)nthreads];
-            const float4 d = x4[i + 3 * (size_t)nthreads];
+            const float4 a = load4<NT>(reinterpret_cast<const float *>(x4 + i));
+            const float4 b = load4<NT>(reinterpret_cast<const float *>(x4 + i + nthreads));
+            const float4 c = load4<NT>(reinterpret_cast<const float *>(x4 + i + 2 * (size_t)nthreads));
+            const float4 d = load4<NT>(reinterpret_cast<const float *>(x4 + i + 3 * (size_t)nthreads));
             acc0 = fold4<OP>(acc0, a);
             acc1 = fold4<OP>(acc1, b);
             acc2 = fold4<OP>(acc2, c);
             acc3 = fold4<OP>(acc3, d);
         }
-        for (; i < n4; i += nthreads) acc0 = fold4<OP>(acc0, x4[i]);
+        {
+            // Up to three more per lane: all issued before the first is folded.
+            const size_t i1 = i + nthreads, i2 = i + 2 * (size_t)nthreads;
+            const float id = OP::identity();
+            float4 a = make_float4(id, id, id, id), b = a, c = a;
+            if (i < n4) a = load4<NT>(reinterpret_cast<const float *>(x4 + i));
+            if (i1 < n4) b = load4<NT>(reinterpret_cast<const float *>(x4 + i1));
+            if (i2 < n4) c = load4<NT>(reinterpret_cast<const float *>(x4 + i2));
+            acc0 = fold4<OP>(acc0, a);
+            acc1 = fold4<OP>(acc1, b);
+            acc2 = fold4<OP>(acc2, c);
+        }
         for (size_t j = begin + (n4 << 2) + tid; j < end; j += nthreads) acc1 = OP::apply(acc1, x[j]);
     } else {
         size_t i = begin + tid;
@@ -79,14 +90,14 @@ __device__ __forceinline__ float strided_fold(const float *__restrict__ x, size_
     return OP::apply(OP::apply(acc0, acc1), OP::apply(acc2, acc3));
 }
 
-template <class OP, int VEC, bool SCALE>
+template <class OP, int VEC, bool SCALE, bool NT>
 __global__ __launch_bounds__(ROW_BLOCK) void reduce_rows_wave(float *__restrict__ out,
                                                               const float *__restrict__ in, size_t outer,
                                                               size_t red, float scale) {
     const int lane = threadIdx.x & (WAVE - 1);
     const size_t row = (size_t)blockIdx.x * ROW_WAVES + (threadIdx.x >> 6);
     if (row >= outer) return;
-    float acc = strided_fold<OP, VEC>(in + row * red, 0, red, lane, WAVE);
+    float acc = strided_fold<OP, VEC, NT>(in + row * red, 0, red, lane, WAVE);
     acc = wave_reduce<OP>(acc);
     if (lane == 0) out[row] = SCALE ? acc * scale : acc;
 }
@@ -231,7 +242,7 @@ __global__ __launch_bounds__(SPAN_BLOCK) void reduce_cols_span(float *__restrict
         }
     };
     // The loop body has no conditional loads, so the wait before each fold can allow exactly
-    // the U younger loads to stay in flight.
+    // the U younger loads to stay in flight.  (A third span in flight was measured: slower.)
     if (sp_begin < sp_end) {
         float4 va[U], vb[U];
         uint32_t sp = sp_begin;
@@ -272,14 +283,18 @@ constexpr size_t MAX_GRID_X = 0x7FFFFFFFu;
 constexpr size_t MAX_GRID_Y = 65535;
 
 template <class OP, bool SCALE>
-void rows_wave_launch(hipStream_t s, float *out, const float *in, size_t outer, size_t red, float scale) {
+void rows_wave_launch(hipStream_t s, float *out, const float *in, size_t outer, size_t red, float scale,
+                      bool nt = false) {
     const bool vec4 = (red % 4 == 0) && aligned16(in);
     const size_t blocks = (outer + ROW_WAVES - 1) / ROW_WAVES;
-    if (vec4)
-        hipLaunchKernelGGL((reduce_rows_wave<OP, 4, SCALE>), dim3((unsigned)blocks), dim3(ROW_BLOCK), 0, s, out,
+    if (vec4 && nt)
+        hipLaunchKernelGGL((reduce_rows_wave<OP, 4, SCALE, true>), dim3((unsigned)blocks), dim3(ROW_BLOCK), 0, s, out,
+                           in, outer, red, scale);
+    else if (vec4)
+        hipLaunchKernelGGL((reduce_rows_wave<OP, 4, SCALE, false>), dim3((unsigned)blocks), dim3(ROW_BLOCK), 0, s, out,
                            in, outer, red, scale);
     else
-        hipLaunchKernelGGL((reduce_rows_wave<OP, 1, SCALE>), dim3((unsigned)blocks), dim3(ROW_BLOCK), 0, s, out,
+        hipLaunchKernelGGL((reduce_rows_wave<OP, 1, SCALE, false>), dim3((unsigned)blocks), dim3(ROW_BLOCK), 0, s, out,
                            in, outer, red, scale);
 }
 
@@ -354,7 +369,7 @@ int reduce_impl(DeviceCtx &ctx, float *out, const float *in, size_t outer, size_
         if (red <= 4096 || outer >= 65536) {
             if ((outer + ROW_WAVES - 1) / ROW_WAVES > MAX_GRID_X)
                 return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: too many rows for one launch");
-            rows_wave_launch<OP, SCALE>(s, out, in, outer, red, scale);
+            rows_wave_launch<OP, SCALE>(s, out, in, outer, red, scale, ctx.streaming(outer * red * sizeof(float)));
             return ctx.check(hipGetLastError(), "reduce rows (wave) launch");
         }
         if (outer > MAX_GRID_Y) return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: too many rows for one launch");

@@ -33,14 +33,16 @@ constexpr int WAVES_PER_BLOCK = BLOCK / WAVE;
 template <int VEC, int NCH> struct RowRegs {
     float v[NCH * VEC];
 
-    // Loads the row; slots past `len` are set to `fill`.
+    // Loads the row; slots past `len` are set to `fill`.  NT: non-temporal 16-byte accesses, for tensors
+    // too large to be found in a cache by the next kernel.
+    template <bool NT = false>
     __device__ __forceinline__ void load(const float *__restrict__ row, int len, int lane, float fill) {
 #pragma unroll
         for (int k = 0; k < NCH; k++) {
             const int e = (lane + WAVE * k) * VEC;
             if (VEC == 4) {
                 if (e < len) {
-                    const float4 t = *reinterpret_cast<const float4 *>(row + e);
+                    const float4 t = load4<NT>(row + e);
                     v[k * VEC + 0] = t.x;
                     v[k * VEC + 1 % VEC] = t.y;
                     v[k * VEC + 2 % VEC] = t.z;
@@ -54,6 +56,7 @@ template <int VEC, int NCH> struct RowRegs {
             }
         }
     }
+    template <bool NT = false>
     __device__ __forceinline__ void store(float *__restrict__ row, int len, int lane) const {
 #pragma unroll
         for (int k = 0; k < NCH; k++) {
@@ -65,7 +68,7 @@ template <int VEC, int NCH> struct RowRegs {
                     t.y = v[k * VEC + 1 % VEC];
                     t.z = v[k * VEC + 2 % VEC];
                     t.w = v[k * VEC + 3 % VEC];
-                    *reinterpret_cast<float4 *>(row + e) = t;
+                    store4<NT>(row + e, t);
                 } else {
                     row[e] = v[k];
                 }
@@ -314,7 +317,7 @@ __global__ __launch_bounds__(BLOCK) void softmax_block_stream(float *__restrict_
 // ---------------------------------------------------------------------------
 // LayerNormalization
 // ---------------------------------------------------------------------------
-template <int VEC, int NCH>
+template <int VEC, int NCH, bool NT>
 __global__ __launch_bounds__(BLOCK) void layernorm_wave(float *__restrict__ out, const float *__restrict__ in,
                                                         const float *__restrict__ gamma,
                                                         const float *__restrict__ beta, size_t rows, int len,
@@ -326,7 +329,11 @@ __global__ __launch_bounds__(BLOCK) void layernorm_wave(float *__restrict__ out,
     float *o = out + row * (size_t)len;
 
     RowRegs<VEC, NCH> r;
-    r.load(x, len, lane, 0.0f);
+    r.template load<NT>(x, len, lane, 0.0f);
+    // Scale and bias are requested right behind the row, so that they arrive during the two reductions.
+    RowRegs<VEC, NCH> g, b;
+    g.load(gamma, len, lane, 0.0f);
+    b.load(beta, len, lane, 0.0f);
 
     const float inv_n = 1.0f / (float)len;
     float sum = 0.0f;
@@ -345,12 +352,9 @@ __global__ __launch_bounds__(BLOCK) void layernorm_wave(float *__restrict__ out,
     ss = wave_reduce<SumOp>(ss);
     const float inv_std = 1.0f / sqrtf(__builtin_fmaf(ss, inv_n, eps));
 
-    RowRegs<VEC, NCH> g, b;
-    g.load(gamma, len, lane, 0.0f);
-    b.load(beta, len, lane, 0.0f);
 #pragma unroll
     for (int s = 0; s < NCH * VEC; s++) r.v[s] = __builtin_fmaf(r.v[s] * inv_std, g.v[s], b.v[s]);
-    r.store(o, len, lane);
+    r.template store<NT>(o, len, lane);
 }
 
 __global__ __launch_bounds__(BLOCK) void layernorm_block_stream(float *__restrict__ out,
@@ -418,10 +422,14 @@ template <int VEC, int NCH> struct SoftmaxLauncher {
 
 template <int VEC, int NCH> struct LayerNormLauncher {
     static void go(hipStream_t s, float *out, const float *in, const float *gamma, const float *beta,
-                   size_t rows, int len, float eps) {
+                   size_t rows, int len, float eps, bool nt) {
         const size_t blocks = (rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-        hipLaunchKernelGGL((layernorm_wave<VEC, NCH>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in,
-                           gamma, beta, rows, len, eps);
+        if (nt && VEC == 4)
+            hipLaunchKernelGGL((layernorm_wave<VEC, NCH, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in,
+                               gamma, beta, rows, len, eps);
+        else
+            hipLaunchKernelGGL((layernorm_wave<VEC, NCH, false>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in,
+                               gamma, beta, rows, len, eps);
     }
 };
 
@@ -577,7 +585,7 @@ int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *g
         const bool vec4 =
             (len % 4 == 0) && aligned16(out) && aligned16(in) && aligned16(gamma) && aligned16(beta);
         if (!dispatch_wave<LayerNormLauncher>(vec4, len, ctx.stream, out, in, gamma, beta, rows, (int)len,
-                                              eps))
+                                              eps, ctx.streaming(rows * len * sizeof(float))))
             return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: no wave layout for this row length");
     } else {
         if (rows > MAX_GRID) return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: too many rows for one launch");

@@ -117,6 +117,54 @@ def build_cfg4(ctx, D, synth, batch, rotate_bytes):
     return ops, fused, c
 
 
+def build_listed_ops(ctx, D, c, batch, rotate_bytes=900e6):
+    """Every operator of the path at configs[4]-sized tensors: the operators the step itself does not hold
+    (Sub, Mul, Pow, the unary ones, ReduceMean, LayerNormalization) on the step's own arrays, so that each has a
+    bandwidth figure at the size where bandwidth is what bounds it.  Buffers rotate past the 256 MB cache."""
+    ops = []
+    y = c["div_in"]                                   # [batch,197,768] ~ N(0,1)
+    dims = list(y.shape)
+    rows_n = batch * 197
+    k = max(2, min(4, int(np.ceil(rotate_bytes / (2 * y.nbytes)))))
+    xs = [ctx.upload(y) for _ in range(k)]
+    pos = [ctx.upload(np.abs(y) + np.float32(0.5)) for _ in range(k)]
+    outs = [ctx.alloc(y.nbytes) for _ in range(k)]
+    small = [ctx.alloc(rows_n * 4) for _ in range(k)]
+    rng = np.random.default_rng(11)
+    col = ctx.upload((1.5 + rng.random((batch, 197, 1))).astype(np.float32))       # per-row operand (mean, std)
+    vec = ctx.upload((1.0 + 0.02 * rng.standard_normal(768)).astype(np.float32))   # gamma-like operand
+    vec2 = ctx.upload((0.02 * rng.standard_normal(768)).astype(np.float32))
+    two = ctx.upload(np.array([2.0], np.float32))
+    ys = D.strides_for_broadcasting(dims, dims)
+
+    def binary(name, op, other, other_shape, src=xs):
+        os_ = D.strides_for_broadcasting(other_shape, dims)
+        nbytes = 2 * y.nbytes + 4 * int(np.prod(other_shape, dtype=np.int64))
+        ops.append(Op(name, nbytes, [(lambda i=i: ctx.binary_raw(op, outs[i].ptr, src[i].ptr, other.ptr, dims, ys, os_))
+                                     for i in range(k)]))
+
+    def unary(name, op, src=xs, alpha=0.0, beta=0.0):
+        ops.append(Op(name, 2 * y.nbytes, [(lambda i=i: ctx.unary_raw(op, outs[i].ptr, src[i].ptr, y.size, alpha, beta))
+                                           for i in range(k)]))
+
+    shape = "[%d,197,768]" % batch
+    binary("Sub %s-[%d,197,1]" % (shape, batch), D.SUB, col, [batch, 197, 1])
+    binary("Mul %s*[768]" % shape, D.MUL, vec, [768])
+    binary("Div %s/[%d,197,1]" % (shape, batch), D.DIV, col, [batch, 197, 1])
+    binary("Pow(.,2) %s" % shape, D.POW, two, [])
+    unary("Sqrt %s" % shape, D.SQRT, src=pos)
+    unary("Erf %s" % shape, D.ERF)
+    unary("Gelu %s" % shape, D.GELU)
+    unary("Sigmoid %s" % shape, D.SIGMOID)
+    unary("HardSigmoid %s" % shape, D.HARDSIGMOID, alpha=1.0 / 6.0, beta=0.5)
+    unary("Relu %s" % shape, D.RELU)
+    ops.append(Op("ReduceMean(-1) %s" % shape, y.nbytes + rows_n * 4,
+                  [(lambda i=i: ctx.reduce_raw(D.REDUCE_MEAN, small[i].ptr, xs[i].ptr, rows_n, 768, 1)) for i in range(k)]))
+    ops.append(Op("LayerNormalization(-1) %s" % shape, 2 * y.nbytes + 2 * 768 * 4,
+                  [(lambda i=i: ctx.layernorm_raw(outs[i].ptr, xs[i].ptr, vec.ptr, vec2.ptr, rows_n, 768, 1e-5)) for i in range(k)]))
+    return ops
+
+
 def build_other_configs(ctx, D, synth, rotate_bytes=600e6, max_sets=48):
     """Kernels of configs[0..3] at their BASELINE.json shapes (parity-test shapes, reported as a table
     only).  Buffers are rotated over enough copies that repeated launches miss the 256 MB cache.  Each
@@ -468,6 +516,8 @@ def main():
     ap.add_argument("--only", type=str, default="", help="run only kernels whose name contains this text (profiling)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a copy-shaped Relu of known size (scales rocprof byte counters)")
+    ap.add_argument("--no-listed-ops", action="store_true",
+                    help="skip the table of the path's other operators at configs[4]-sized tensors ('listed_ops' in the JSON)")
     ap.add_argument("--all-configs", action="store_true",
                     help="also time the kernels and graphs of configs[0..3] (table on stderr, 'other_configs' in the JSON)")
     ap.add_argument("--next-rows", action="store_true",
@@ -488,7 +538,7 @@ def main():
     from altius_amd import synth
 
     ctx = D.Context(0)
-    ops, fused_ops, _ = build_cfg4(ctx, D, synth, args.batch, rotate_bytes=600e6)
+    ops, fused_ops, cfg4_arrays = build_cfg4(ctx, D, synth, args.batch, rotate_bytes=600e6)
     if args.only:
         ops = [o for o in ops if args.only.lower() in o.name.lower()]
         fused_ops = [o for o in fused_ops if args.only.lower() in o.name.lower()]
@@ -554,6 +604,17 @@ def main():
         },
         "per_kernel": [{k: (round(v, 2) if isinstance(v, float) else v) for k, v in r.items()} for r in rows],
     }
+
+    if not args.only and not args.no_listed_ops:
+        listed = []
+        log("every operator of the path at configs[4]-sized tensors:")
+        for o in build_listed_ops(ctx, D, cfg4_arrays, args.batch):
+            ms = time_kernel(ctx, o, args.kernel_iters, 5)
+            gbps = o.nbytes / (ms * 1e-3) / 1e9
+            listed.append({"kernel": o.name, "bytes": o.nbytes, "us": round(ms * 1e3, 2), "GBps": round(gbps, 1),
+                           "pct_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 1)})
+            log("%-44s %14d %10.1f %10.1f %8.1f" % (o.name, o.nbytes, ms * 1e3, gbps, 100.0 * gbps / HBM_PEAK_GBPS))
+        result["listed_ops"] = listed
 
     if args.all_configs:
         others = []

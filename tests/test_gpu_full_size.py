@@ -58,6 +58,28 @@ def test_cfg4_div_scalar(ctx, case, cfg4):
     assert_bits_equal(q, O.binary(O.DIV, x, s), "cfg4 div vs oracle")
 
 
+def test_cfg4_sized_layernorm_chain_ops(ctx, case, cfg4):
+    """The operators of the LayerNormalization chain on [256,197,768] (155 MB, so the kernels take their
+    non-temporal variants): per-row Sub and Div, Mul by a vector, ReduceMean, LayerNormalization."""
+    case("full-size chain operators on [256,197,768]")
+    x = cfg4["div_in"]
+    rows = x.shape[0] * x.shape[1]
+    mean = ctx.reduce(D.REDUCE_MEAN, x, rows, 768, 1).reshape(256, 197, 1)
+    assert_close(mean, O.reduce(O.REDUCE_MEAN, x, [-1], True), what="mean over 768")
+    # exact in any order: mean(-x) = -mean(x)
+    assert_bits_equal(ctx.reduce(D.REDUCE_MEAN, -x, rows, 768, 1).reshape(mean.shape), -mean, "mean(-x) = -mean(x)")
+    assert_bits_equal(ctx.binary(D.SUB, x, mean), x - mean, "x - mean")
+    assert_bits_equal(ctx.binary(D.SUB, mean, x), mean - x, "mean - x")
+    dev = np.abs(mean) + np.float32(0.75)
+    assert_bits_equal(ctx.binary(D.DIV, x, dev), x / dev, "x / dev")
+    gamma = synth.normal(5, (768,), mean=1.0, std=0.02)
+    beta = synth.normal(6, (768,), mean=0.0, std=0.02)
+    assert_bits_equal(ctx.binary(D.MUL, x, gamma), x * gamma, "x * gamma")
+    assert_bits_equal(ctx.binary(D.ADD, beta, x), beta + x, "beta + x")
+    y = ctx.layer_norm(x, gamma, beta, 1e-5)
+    assert_close(y, O.layer_norm(x, gamma, beta, 1e-5, threads=THREADS), what="layernorm [256,197,768]")
+
+
 def test_cfg2_layernorm_full(ctx, case):
     case("full cfg2 LayerNormalization [32,197,768]")
     c = synth.cfg2(batch=32)

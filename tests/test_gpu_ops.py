@@ -50,6 +50,16 @@ BIN_SHAPES = [
     ([5, 2, 6], [5, 1, 6]),            # row broadcast too short for the LDS kernel
     ([2, 3, 1031], [1031]),            # bias with an odd length
     ([7, 5], [5]),
+    # rows of whole float4s with a vector along the row or one value per row (two-axis kernel), both operand orders
+    ([8, 197, 768], [768]),
+    ([768], [8, 197, 768]),
+    ([8, 197, 1], [8, 197, 768]),
+    ([33, 1028], [1028]),              # last block partly filled
+    ([33, 1028], [33, 1]),
+    ([3, 5, 4], [3, 5, 1]),
+    ([1, 4], [3, 5, 4]),
+    ([64, 197, 3072], [3072]),         # above the size at which accesses become non-temporal
+    ([64, 197, 3072], [64, 197, 1]),
 ]
 
 
