@@ -97,7 +97,7 @@ struct SoftmaxPrologue {
     uint32_t mask_rows;
 };
 
-template <int VEC, int NCH, bool PRO>
+template <int VEC, int NCH, bool PRO, bool NT>
 __global__ __launch_bounds__(BLOCK) void softmax_wave(float *__restrict__ out, const float *__restrict__ in,
                                                       size_t rows, int len, const SoftmaxPrologue pro) {
     const int lane = threadIdx.x & (WAVE - 1);
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(BLOCK) void softmax_wave(float *__restrict__ out, c
 
     RowRegs<VEC, NCH> r;
     const float nan = __builtin_nanf("");
-    r.load(x, len, lane, nan);
+    r.template load<NT>(x, len, lane, nan);
     if (PRO) {
         // The mask row is shared by rows_per_mask score rows: it comes from the caches, and its load
         // is issued before the scores are looked at.
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(BLOCK) void softmax_wave(float *__restrict__ out, c
     const float recip = 1.0f / sum;
 #pragma unroll
     for (int s = 0; s < NCH * VEC; s++) r.v[s] *= recip;
-    r.store(o, len, lane);
+    r.template store<NT>(o, len, lane);
 }
 
 // Rows whose length is not a multiple of 4 (197 tokens, say) start at addresses
@@ -410,13 +410,17 @@ bool dispatch_wave(bool vec4, size_t len, Args... args) {
 }
 
 template <int VEC, int NCH> struct SoftmaxLauncher {
-    static void go(hipStream_t s, float *out, const float *in, size_t rows, int len, const SoftmaxPrologue *pro) {
-        const size_t blocks = (rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-        if (pro)
-            hipLaunchKernelGGL((softmax_wave<VEC, NCH, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, rows, len, *pro);
+    static void go(hipStream_t s, float *out, const float *in, size_t rows, int len, const SoftmaxPrologue *pro, bool nt) {
+        const dim3 grid((unsigned)((rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK));
+        const SoftmaxPrologue none{0, 0.0f, nullptr, 1, 0};
+        if (pro && nt && VEC == 4)
+            hipLaunchKernelGGL((softmax_wave<VEC, NCH, true, true>), grid, dim3(BLOCK), 0, s, out, in, rows, len, *pro);
+        else if (pro)
+            hipLaunchKernelGGL((softmax_wave<VEC, NCH, true, false>), grid, dim3(BLOCK), 0, s, out, in, rows, len, *pro);
+        else if (nt && VEC == 4)
+            hipLaunchKernelGGL((softmax_wave<VEC, NCH, false, true>), grid, dim3(BLOCK), 0, s, out, in, rows, len, none);
         else
-            hipLaunchKernelGGL((softmax_wave<VEC, NCH, false>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, rows, len,
-                               SoftmaxPrologue{0, 0.0f, nullptr, 1, 0});
+            hipLaunchKernelGGL((softmax_wave<VEC, NCH, false, false>), grid, dim3(BLOCK), 0, s, out, in, rows, len, none);
     }
 };
 
@@ -538,7 +542,8 @@ int launch_softmax(DeviceCtx &ctx, float *out, const float *in, size_t rows, siz
         if (aligned && !wave_fits) {
             if (!softmax_lds_launch(ctx.stream, out, in, rows, len, ctx.streaming(rows * len * sizeof(float))))
                 return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: too many rows for one launch");
-        } else if (!dispatch_wave<SoftmaxLauncher>(vec4, len, ctx.stream, out, in, rows, (int)len, (const SoftmaxPrologue *)nullptr)) {
+        } else if (!dispatch_wave<SoftmaxLauncher>(vec4, len, ctx.stream, out, in, rows, (int)len, (const SoftmaxPrologue *)nullptr,
+                                                    ctx.streaming(rows * len * sizeof(float)))) {
             return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: no wave layout for this row length");
         }
     } else {
@@ -567,7 +572,8 @@ int launch_softmax_prologue(DeviceCtx &ctx, float *out, const float *in, size_t 
     const bool wave_fits = len % 4 == 0 && len * 4 >= slots * 3;
     if (wave_fits) {
         if (mask && !aligned16(mask)) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax prologue: the mask must be 16-byte aligned");
-        if ((rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK > MAX_GRID || !dispatch_wave<SoftmaxLauncher>(true, len, ctx.stream, out, in, rows, (int)len, (const SoftmaxPrologue *)&pro))
+        if ((rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK > MAX_GRID || !dispatch_wave<SoftmaxLauncher>(true, len, ctx.stream, out, in, rows, (int)len, (const SoftmaxPrologue *)&pro,
+                                                                                         ctx.streaming(rows * len * sizeof(float))))
             return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax prologue: too many rows for one launch");
     } else if (!softmax_lds_launch(ctx.stream, out, in, rows, len, ctx.streaming(rows * len * sizeof(float)), &pro)) {
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax prologue: too many rows for one launch");

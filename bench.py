@@ -160,6 +160,8 @@ def build_listed_ops(ctx, D, c, batch, rotate_bytes=900e6):
     unary("Relu %s" % shape, D.RELU)
     ops.append(Op("ReduceMean(-1) %s" % shape, y.nbytes + rows_n * 4,
                   [(lambda i=i: ctx.reduce_raw(D.REDUCE_MEAN, small[i].ptr, xs[i].ptr, rows_n, 768, 1)) for i in range(k)]))
+    ops.append(Op("Softmax(-1) %s" % shape, 2 * y.nbytes,
+                  [(lambda i=i: ctx.softmax_raw(outs[i].ptr, xs[i].ptr, rows_n, 768)) for i in range(k)]))
     ops.append(Op("LayerNormalization(-1) %s" % shape, 2 * y.nbytes + 2 * 768 * 4,
                   [(lambda i=i: ctx.layernorm_raw(outs[i].ptr, xs[i].ptr, vec.ptr, vec2.ptr, rows_n, 768, 1e-5)) for i in range(k)]))
     return ops

@@ -78,6 +78,9 @@ def test_cfg4_sized_layernorm_chain_ops(ctx, case, cfg4):
     assert_bits_equal(ctx.binary(D.ADD, beta, x), beta + x, "beta + x")
     y = ctx.layer_norm(x, gamma, beta, 1e-5)
     assert_close(y, O.layer_norm(x, gamma, beta, 1e-5, threads=THREADS), what="layernorm [256,197,768]")
+    p = ctx.softmax(x)
+    assert_close(p, O.softmax(x, threads=THREADS), what="softmax [256,197,768]")
+    np.testing.assert_allclose(p.sum(-1, dtype=np.float64), 1.0, atol=2e-6)
 
 
 def test_cfg2_layernorm_full(ctx, case):
