@@ -204,7 +204,7 @@ int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, c
     if (d != (size_t)D || tk == 0) return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: needs 64-wide heads and at least one key");
     const size_t lim = (size_t)1 << 31;
     if (mask_outer_stride >= lim) return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: mask stride above 2^31");
-    if (tq >= lim || ldq >= lim || ldk >= lim || ldv >= lim || ldo >= lim || batch >= lim)
+    if (tq >= lim || tk >= lim || ldq >= lim || ldk >= lim || ldv >= lim || ldo >= lim || batch >= lim)
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: extent above 2^31");
     auto vec_ok = [](const void *p, size_t ld, const size_t bs[2]) { return aligned16(p) && ld % 4 == 0 && bs[0] % 4 == 0 && bs[1] % 4 == 0; };
     if (!vec_ok(q, ldq, q_bs) || !vec_ok(k, ldk, k_bs) || !vec_ok(v, ldv, v_bs) || !vec_ok(o, ldo, o_bs))

@@ -53,8 +53,9 @@ struct GemmArgs {
 // Loads this thread's share of a BK x 128 operand tile into registers.
 // K_CONTIG: the operand's k axis is the contiguous one (A without transA, B with transB).
 // `mn` is the tile's first row (A) or column (B), `lim` the extent of that axis.
-// INSIDE: the whole tile lies inside the operand and 16-byte loads are legal (decided per block and
-// K tile, a scalar branch): no per-lane bounds checks.
+// INSIDE: 16-byte loads are legal, the K tile is whole, and an operand whose mn axis is the contiguous one
+// has an extent that is a multiple of 4 (decided per block and K tile, a scalar branch): no per-lane bounds
+// checks, edge tiles clamp their addresses instead.
 template <bool K_CONTIG, int WIDTH, bool INSIDE>
 __device__ __forceinline__ void load_tile(float4 (&r)[WIDTH / 64], const float *__restrict__ p, uint32_t mn0, uint32_t lim,
                                           uint32_t k0, uint32_t kdim, uint32_t s_mn, uint32_t s_k, int vec, int tid) {
@@ -70,6 +71,10 @@ __device__ __forceinline__ void load_tile(float4 (&r)[WIDTH / 64], const float *
             mn = mn0 + ((f % (WIDTH / 4)) << 2);
         }
         if (INSIDE) {
+            // Rows (or float4 columns) past the operand's edge re-read its last one: in bounds, and what they
+            // contribute only reaches elements of C that are never stored.
+            const uint32_t last = K_CONTIG ? lim - 1 : (lim - 4) & ~3u;
+            if (mn > last) mn = last;
             r[u] = *reinterpret_cast<const float4 *>(K_CONTIG ? p + (size_t)mn * s_mn + kk : p + (size_t)kk * s_k + mn);
             continue;
         }
@@ -152,10 +157,10 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_mfma(GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    // Blocks whose tiles lie inside both operands run a loop without any bounds check on all K tiles
-    // but a ragged last one; the choice is made once per block (a scalar branch around the whole loop),
-    // so the interior loop is straight-line code between its barriers.
-    const bool inside = g.a_vec && g.b_vec && m0 + BM <= g.m && n0 + TN <= g.n;
+    // Operands that allow 16-byte loads everywhere run a loop without any bounds check on all K tiles but a
+    // ragged last one (edge tiles clamp their addresses); the choice is a scalar branch around the whole
+    // loop, so the loop is straight-line code between its barriers.
+    const bool inside = g.a_vec && g.b_vec && (A_KC || (g.m & 3) == 0) && (B_KC || (g.n & 3) == 0);
     const int lr = lane & 31, lk = lane >> 5;
     auto main_loop = [&](auto inside_tag) {
         constexpr bool INSIDE = decltype(inside_tag)::value;
@@ -271,16 +276,18 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
     // K loops: with half the accumulators per wavefront more blocks fit a CU and the last round of blocks
     // is fuller (measured at [50432,3072]x[3072,768]: 120.9 against 110.3 TFLOP/s; the wide tile stays ahead
     // only where K is short and the tile's fixed costs weigh more, as in attention's 64-deep products).
-    const bool narrow = n <= 64 || (n < 512 && n % 128 != 0 && n % 128 <= 64) || k >= 256;
+    // ... and when the wide tile would leave CUs without a block (the slices of a product cut along k).
+    const size_t cus = ctx.cus_per_xcd ? (size_t)ctx.cus_per_xcd * 8 : 256;
+    const bool narrow = n <= 64 || (n < 512 && n % 128 != 0 && n % 128 <= 64) || k >= 256 ||
+                        ((m + BM - 1) / BM) * ((n + BN - 1) / BN) * batch < cus;
     const size_t tn = narrow ? 64 : BN;
     const size_t gy = (m + BM - 1) / BM, gx = (n + tn - 1) / tn;
     if (gy > 65535 || batch > 65535) return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm: more than 65535 row tiles or batches");
     // A single product with few tiles and a long k (one image through a transformer layer) leaves most CUs idle
     // while each block walks all of k: cut k into slices that run as batches into a workspace, and add the
     // slices up in order afterwards (the bias and alpha / beta go there).
-    if (batch == 1 && ctx.gemm_split_k && gx * gy <= 128 && k >= 512 && !split_k_inner) {
-        const size_t cus = ctx.cus_per_xcd ? (size_t)ctx.cus_per_xcd * 8 : 256;
-        size_t slices = std::min<size_t>(std::min<size_t>((cus + gx * gy - 1) / (gx * gy), k / 128), 16);
+    if (batch == 1 && ctx.gemm_split_k && gx * gy <= cus && k >= 512 && !split_k_inner) {
+        size_t slices = std::min<size_t>(std::min<size_t>((2 * cus + gx * gy - 1) / (gx * gy), k / 128), 16);
         while (slices > 1 && k % (slices * 16) != 0) slices--;  // equal slices of whole k tiles
         if (slices >= 2) {
             void *ws = nullptr;
