@@ -53,6 +53,60 @@ struct AttnArgs {
 
 constexpr int KC = 64;  // keys per chunk
 
+// One tile of 32 keys for a wavefront's 32 queries: scores S^T = K tile x Q^T, the running maximum and sum
+// brought up to date (what was accumulated is rescaled when the maximum rises), then O^T += V tile^T x P^T.
+// ktile / vtile: the tile's first row in LDS (pitches K_PITCH and D); key_base: its first key's index.
+__device__ __forceinline__ void attend_tile(int scale_op, float scale, uint32_t tk, const float *__restrict__ mask, const float *ktile,
+                                            const float *vtile, uint32_t key_base, const float (&qf)[32], int h, int lr, float &mx,
+                                            float &sum, floatx16 (&acc)[2]) {
+    floatx16 st;
+#pragma unroll
+    for (int r = 0; r < 16; r++) st[r] = 0.0f;
+    const float *kr = ktile + lr * K_PITCH + 32 * h;
+#pragma unroll
+    for (int cc = 0; cc < 8; cc++) {
+        const f32x4 kf = *reinterpret_cast<const f32x4 *>(kr + 4 * cc);
+        st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.x, qf[4 * cc], st, 0, 0, 0);
+        st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.y, qf[4 * cc + 1], st, 0, 0, 0);
+        st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.z, qf[4 * cc + 2], st, 0, 0, 0);
+        st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.w, qf[4 * cc + 3], st, 0, 0, 0);
+    }
+    float cmax = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const uint32_t key = key_base + 8 * (r >> 2) + 4 * h + (r & 3);
+        float x = st[r];
+        if (scale_op == 1) x = x * scale;
+        else if (scale_op == 2) x = x / scale;
+        if (mask && key < tk) x = x + mask[key];
+        st[r] = x;
+        if (key < tk) cmax = dev::nanmax(cmax, x);
+    }
+    cmax = dev::nanmax(cmax, __shfl_xor(cmax, 32));
+    const float mnew = dev::nanmax(mx, cmax);
+    if (mnew != mx) {  // what has been summed so far was taken relative to the old maximum
+        const float corr = mx == -INFINITY ? 0.0f : dev::softmax_exp(mx, mnew);
+        sum *= corr;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[0][r] *= corr, acc[1][r] *= corr;
+        mx = mnew;
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const uint32_t key = key_base + 8 * (r >> 2) + 4 * h + (r & 3);
+        const float e = key < tk ? dev::softmax_exp(st[r], mx) : 0.0f;
+        st[r] = e;
+        sum += e;
+    }
+#pragma unroll
+    for (int kk = 0; kk < 16; kk++) {
+        const int key = 8 * (kk >> 2) + 4 * h + (kk & 3);
+        const float v0 = vtile[key * D + lr], v1 = vtile[key * D + 32 + lr];
+        acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(v0, st[kk], acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(v1, st[kk], acc[1], 0, 0, 0);
+    }
+}
+
 // W: wavefronts (tiles of 32 queries) per block.  Fewer when there are few (batch, head) pairs, so that the queries of
 // one pair spread over several CUs; every block stages the keys and values it needs itself.
 template <int W>
@@ -119,53 +173,7 @@ __global__ __launch_bounds__(64 * W, W == 8 ? 4 : 1) void attention_stream_d64(A
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             if (active && j < tiles) {
-                // Scores of 32 keys: S^T tile = K tile x Q^T.
-                floatx16 st;
-#pragma unroll
-                for (int r = 0; r < 16; r++) st[r] = 0.0f;
-                const float *kr = &ks[buf][(32 * j + lr) * K_PITCH + 32 * h];
-#pragma unroll
-                for (int cc = 0; cc < 8; cc++) {
-                    const f32x4 kf = *reinterpret_cast<const f32x4 *>(kr + 4 * cc);
-                    st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.x, qf[4 * cc], st, 0, 0, 0);
-                    st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.y, qf[4 * cc + 1], st, 0, 0, 0);
-                    st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.z, qf[4 * cc + 2], st, 0, 0, 0);
-                    st = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.w, qf[4 * cc + 3], st, 0, 0, 0);
-                }
-                float cmax = -INFINITY;
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const uint32_t key = key0 + 32 * j + 8 * (r >> 2) + 4 * h + (r & 3);
-                    float x = st[r];
-                    if (g.scale_op == 1) x = x * g.scale;
-                    else if (g.scale_op == 2) x = x / g.scale;
-                    if (mask && key < g.tk) x = x + mask[key];
-                    st[r] = x;
-                    if (key < g.tk) cmax = dev::nanmax(cmax, x);
-                }
-                cmax = dev::nanmax(cmax, __shfl_xor(cmax, 32));
-                const float mnew = dev::nanmax(mx, cmax);
-                if (mnew != mx) {  // what has been summed so far was taken relative to the old maximum
-                    const float corr = mx == -INFINITY ? 0.0f : dev::softmax_exp(mx, mnew);
-                    sum *= corr;
-#pragma unroll
-                    for (int r = 0; r < 16; r++) acc[0][r] *= corr, acc[1][r] *= corr;
-                    mx = mnew;
-                }
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const uint32_t key = key0 + 32 * j + 8 * (r >> 2) + 4 * h + (r & 3);
-                    const float e = key < g.tk ? dev::softmax_exp(st[r], mx) : 0.0f;
-                    st[r] = e;
-                    sum += e;
-                }
-#pragma unroll
-                for (int kk = 0; kk < 16; kk++) {
-                    const int key = 32 * j + 8 * (kk >> 2) + 4 * h + (kk & 3);
-                    const float v0 = vs[buf][key * D + lr], v1 = vs[buf][key * D + 32 + lr];
-                    acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(v0, st[kk], acc[0], 0, 0, 0);
-                    acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(v1, st[kk], acc[1], 0, 0, 0);
-                }
+                attend_tile(g.scale_op, g.scale, g.tk, mask, &ks[buf][32 * j * K_PITCH], &vs[buf][32 * j * D], key0 + 32 * j, qf, h, lr, mx, sum, acc);
             }
             if (j == 0 && more) {
                 park(ks[buf ^ 1], K_PITCH);
@@ -179,6 +187,124 @@ __global__ __launch_bounds__(64 * W, W == 8 ? 4 : 1) void attention_stream_d64(A
     if (active && query < g.tq) {
         sum += __shfl_xor(sum, 32);
         const float recip = 1.0f / sum;
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; g4++) {
+                const f32x4 out = {acc[t][4 * g4] * recip, acc[t][4 * g4 + 1] * recip, acc[t][4 * g4 + 2] * recip, acc[t][4 * g4 + 3] * recip};
+                *reinterpret_cast<f32x4 *>(o + (size_t)query * g.ldo + 32 * t + 8 * g4 + 4 * h) = out;
+            }
+    }
+}
+
+// The same for few (batch, head) pairs, where a wavefront walking all keys alone is the whole run time: a block
+// of SW wavefronts owns ONE tile of 32 queries and deals the key tiles out among its wavefronts (tile t of a
+// chunk of 32 SW keys goes to wavefront t).  Each keeps its own running maximum, sum and O^T; at the end the
+// partial results meet in LDS and wavefront 0 combines them, every part scaled by exp(its maximum - the overall
+// one), exactly the rescaling the streaming kernel applies when its maximum rises.
+constexpr int SW = 4;
+constexpr int SC = 32 * SW;  // keys per chunk
+
+__global__ __launch_bounds__(64 * SW, 1) void attention_keysplit_d64(AttnArgs g) {
+    __shared__ __align__(16) float ks[SC * K_PITCH];
+    __shared__ __align__(16) float vs[SC * D];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int h = lane >> 5, lr = lane & 31;
+    const uint32_t zo = blockIdx.x / g.batch_inner, zi = blockIdx.x % g.batch_inner;
+    const float *q = g.q + zo * g.q_bs[0] + zi * g.q_bs[1];
+    const float *k = g.k + zo * g.k_bs[0] + zi * g.k_bs[1];
+    const float *v = g.v + zo * g.v_bs[0] + zi * g.v_bs[1];
+    float *o = g.o + zo * g.o_bs[0] + zi * g.o_bs[1];
+    const float *mask = g.mask ? g.mask + (size_t)zo * g.mask_outer_stride : nullptr;
+    const uint32_t query = blockIdx.y * 32 + lr;
+    const uint32_t nchunks = (g.tk + SC - 1) / SC;
+
+    // Staging: 256 threads move 16 rows of 16 float4 per pass, 8 passes per operand and chunk.
+    constexpr int PASSES = SC / 16;
+    const uint32_t r0 = tid >> 4, c4 = tid & 15;
+    f32x4 kst[PASSES], vst[PASSES];
+    auto fetch = [&](f32x4 (&st)[PASSES], const float *base, uint32_t ld, uint32_t chunk) {
+#pragma unroll
+        for (int it = 0; it < PASSES; it++) {
+            const uint32_t row = chunk * SC + it * 16 + r0;
+            st[it] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            if (row < g.tk) st[it] = *reinterpret_cast<const f32x4 *>(base + (size_t)row * ld + c4 * 4);
+        }
+    };
+    auto park = [&](const f32x4 (&st)[PASSES], float *dst, int pitch) {
+#pragma unroll
+        for (int it = 0; it < PASSES; it++) *reinterpret_cast<f32x4 *>(dst + (it * 16 + r0) * pitch + c4 * 4) = st[it];
+    };
+    fetch(kst, k, g.ldk, 0);
+    fetch(vst, v, g.ldv, 0);
+    float qf[32];
+    if (query < g.tq) {
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            const f32x4 t = *reinterpret_cast<const f32x4 *>(q + (size_t)query * g.ldq + 32 * h + 4 * c);
+            qf[4 * c] = t.x, qf[4 * c + 1] = t.y, qf[4 * c + 2] = t.z, qf[4 * c + 3] = t.w;
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < 32; c++) qf[c] = 0.0f;
+    }
+    park(kst, ks, K_PITCH);
+    park(vst, vs, D);
+    __syncthreads();
+
+    float mx = -INFINITY, sum = 0.0f;
+    floatx16 acc[2];
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[0][r] = 0.0f, acc[1][r] = 0.0f;
+
+    for (uint32_t c = 0; c < nchunks; c++) {
+        const bool more = c + 1 < nchunks;
+        if (more) {  // in flight during this chunk's products
+            fetch(kst, k, g.ldk, c + 1);
+            fetch(vst, v, g.ldv, c + 1);
+        }
+        const uint32_t key_base = c * SC + 32 * wave;
+        if (key_base < g.tk) attend_tile(g.scale_op, g.scale, g.tk, mask, &ks[32 * wave * K_PITCH], &vs[32 * wave * D], key_base, qf, h, lr, mx, sum, acc);
+        __syncthreads();  // nobody reads this chunk any more
+        if (more) {
+            park(kst, ks, K_PITCH);
+            park(vst, vs, D);
+            __syncthreads();
+        }
+    }
+
+    // Partial results meet in LDS (the staging area is free now): per wavefront 64 lanes x 32 accumulators, laid
+    // out [register][lane] so that every access is a row of consecutive floats, then maximum and sum per query.
+    sum += __shfl_xor(sum, 32);
+    float *part = ks;                      // [SW][32][64]
+    float *stat = vs;                      // [SW][2][32]
+    if (wave > 0) {
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) part[(wave * 32 + 16 * t + r) * 64 + lane] = acc[t][r];
+        if (h == 0) stat[(wave * 2) * 32 + lr] = mx, stat[(wave * 2 + 1) * 32 + lr] = sum;
+    }
+    __syncthreads();
+    if (wave == 0 && query < g.tq) {
+        float top = mx;
+#pragma unroll
+        for (int w = 1; w < SW; w++) top = dev::nanmax(top, stat[(w * 2) * 32 + lr]);
+        const float own = mx == -INFINITY ? 0.0f : dev::softmax_exp(mx, top);
+        float total = sum * own;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[0][r] *= own, acc[1][r] *= own;
+#pragma unroll
+        for (int w = 1; w < SW; w++) {
+            const float m = stat[(w * 2) * 32 + lr];
+            const float f = m == -INFINITY ? 0.0f : dev::softmax_exp(m, top);
+            total += stat[(w * 2 + 1) * 32 + lr] * f;
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[t][r] += part[(w * 32 + 16 * t + r) * 64 + lane] * f;
+        }
+        const float recip = 1.0f / total;
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
@@ -221,17 +347,21 @@ int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, c
     g.scale = scale;
     g.mask = mask;
     g.mask_outer_stride = (uint32_t)mask_outer_stride;
-    // As many query tiles per block as still leave a block for most CUs.
     const size_t q_tiles = (tq + 31) / 32, cus = ctx.cus_per_xcd ? (size_t)ctx.cus_per_xcd * 8 : 256;
+    if (q_tiles > 65535) return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: too many queries");
+    if (batch * q_tiles < 2 * cus) {
+        // One query tile per block would still leave the GPU thin: the keys are split over a block's wavefronts
+        // as well (ViT-B/16 at batch 1: 84 tiles; measured faster up to about two tiles per CU).
+        hipLaunchKernelGGL(attention_keysplit_d64, dim3((unsigned)batch, (unsigned)q_tiles), dim3(64 * SW), 0, ctx.stream, g);
+        return ctx.check(hipGetLastError(), "attention launch");
+    }
+    // As many query tiles per block as still leave a block for most CUs.
     size_t w = MAX_WAVES;
-    while (w > 1 && batch * ((q_tiles + w - 1) / w) < cus) w /= 2;
-    const size_t gy = (q_tiles + w - 1) / w;
-    if (gy > 65535) return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: too many queries");
-    const dim3 grid((unsigned)batch, (unsigned)gy);
+    while (w > 2 && batch * ((q_tiles + w - 1) / w) < cus) w /= 2;
+    const dim3 grid((unsigned)batch, (unsigned)((q_tiles + w - 1) / w));
     if (w == 8) hipLaunchKernelGGL(attention_stream_d64<8>, grid, dim3(512), 0, ctx.stream, g);
     else if (w == 4) hipLaunchKernelGGL(attention_stream_d64<4>, grid, dim3(256), 0, ctx.stream, g);
-    else if (w == 2) hipLaunchKernelGGL(attention_stream_d64<2>, grid, dim3(128), 0, ctx.stream, g);
-    else hipLaunchKernelGGL(attention_stream_d64<1>, grid, dim3(64), 0, ctx.stream, g);
+    else hipLaunchKernelGGL(attention_stream_d64<2>, grid, dim3(128), 0, ctx.stream, g);
     return ctx.check(hipGetLastError(), "attention launch");
 }
 

@@ -102,3 +102,36 @@ def test_long_sequences_are_streamed(ctx, case, tq, tk):
     s = q.astype(np.float64) @ np.swapaxes(k.astype(np.float64), -1, -2) * 0.125 + mask[:, None, None, :]
     e = np.exp(s - s.max(-1, keepdims=True))
     np.testing.assert_allclose(got, (e / e.sum(-1, keepdims=True)) @ v, rtol=2e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize("heads,tq,tk", [(256, 40, 70), (128, 197, 197), (96, 197, 130), (600, 33, 64), (12, 197, 197), (3, 500, 77)])
+def test_every_block_shape(ctx, case, heads, tq, tk):
+    """The launcher sizes its blocks to the work: 8, 4 or 2 query tiles per block when there are many (batch, head)
+    pairs (the first four cases, in that order and 8 again), one query tile per block with the keys dealt out among
+    its wavefronts when there are few (the last two)."""
+    case(f"attention block shapes: {heads} heads, tq {tq}, tk {tk}")
+    q = RNG.standard_normal((heads, tq, 64)).astype(np.float32)
+    k = RNG.standard_normal((heads, tk, 64)).astype(np.float32)
+    v = RNG.standard_normal((heads, tk, 64)).astype(np.float32)
+    mask = np.where(RNG.random(tk) < 0.2, -1e4, 0.0).astype(np.float32)
+    got = ctx.attention(q, k, v, 1, 0.125, mask=mask)
+    s = q.astype(np.float64) @ np.swapaxes(k.astype(np.float64), -1, -2) * 0.125 + mask
+    e = np.exp(s - s.max(-1, keepdims=True))
+    np.testing.assert_allclose(got, (e / e.sum(-1, keepdims=True)) @ v, rtol=2e-4, atol=2e-5)
+
+
+def test_keys_split_over_wavefronts_with_empty_and_masked_parts(ctx, case):
+    """Few heads: the keys of a chunk of 128 go to four wavefronts.  Fewer keys than wavefronts' tiles (some wavefronts
+    have nothing to add), and a mask that removes every key of one wavefront's tile."""
+    case("attention, keys split over wavefronts: idle and fully masked parts")
+    for tk in (1, 31, 33, 64, 65, 127, 129, 200):
+        q = RNG.standard_normal((2, 37, 64)).astype(np.float32)
+        k = RNG.standard_normal((2, tk, 64)).astype(np.float32)
+        v = RNG.standard_normal((2, tk, 64)).astype(np.float32)
+        mask = np.zeros(tk, np.float32)
+        if tk > 64:
+            mask[32:64] = -1e4  # the second wavefront's whole tile
+        got = ctx.attention(q, k, v, 2, 8.0, mask=mask)
+        s = q.astype(np.float64) @ np.swapaxes(k.astype(np.float64), -1, -2) / 8.0 + mask
+        e = np.exp(s - s.max(-1, keepdims=True))
+        np.testing.assert_allclose(got, (e / e.sum(-1, keepdims=True)) @ v, rtol=2e-4, atol=2e-5, err_msg=f"tk {tk}")
