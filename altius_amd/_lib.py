@@ -93,6 +93,7 @@ def _declare(L):
       + [P(c_size_t)] * 3 + [c_size_t, c_size_t, c_float, c_float])
     f("ahip_gemm_activated", [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p] + [c_size_t] * 3 + [c_int, c_int]
       + [c_size_t] * 5 + [c_float, c_float])
+    f("ahip_gemm_post", [c_void_p] * 5 + [c_size_t] * 3 + [c_int, c_int] + [c_size_t] * 5 + [c_float, c_float, c_int, c_void_p])
     f("ahip_attention", [c_void_p] * 5 + [c_size_t] * 9 + [P(c_size_t)] * 4 + [c_int, c_float, c_void_p, c_size_t])
     f("ahip_gemm_set_algorithm", [c_void_p, c_int])
     f("ahip_gemm_register_constant", [c_void_p, c_void_p, c_size_t])

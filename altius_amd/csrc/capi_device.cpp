@@ -403,6 +403,19 @@ int ahip_gemm_activated(ahip_ctx *ctx, int a_op, float *c, const float *a, const
                                      alpha, beta, a_op);
 }
 
+int ahip_gemm_post(ahip_ctx *ctx, float *c, const float *a, const float *b, const float *c0, size_t m, size_t n, size_t k,
+                   int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t c0_row_stride, size_t c0_col_stride,
+                   float alpha, float beta, int act, const float *residual) {
+    REQUIRE_CTX(ctx, "ahip_gemm_post");
+    if (act != 0 && act != AHIP_GELU && act != AHIP_RELU) return ctx->d.fail(AHIP_ERR_ARG, "ahip_gemm_post: act must be 0, AHIP_GELU or AHIP_RELU");
+    altius::GemmPost post;
+    post.act = act;
+    post.residual = residual;
+    const size_t none[2] = {0, 0};
+    return altius::launch_gemm_batch2(ctx->d, c, a, b, c0, 1, 1, m, n, k, trans_a, trans_b, lda, ldb, ldc, none, none, none, c0_row_stride,
+                                      c0_col_stride, alpha, beta, &post);
+}
+
 int ahip_attention(ahip_ctx *ctx, float *o, const float *q, const float *k, const float *v, size_t batch_outer,
                    size_t batch_inner, size_t tq, size_t tk, size_t d, size_t ldq, size_t ldk, size_t ldv, size_t ldo,
                    const size_t q_batch_strides[2], const size_t k_batch_strides[2], const size_t v_batch_strides[2],

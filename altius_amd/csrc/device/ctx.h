@@ -129,10 +129,17 @@ int launch_gemm(DeviceCtx &ctx, float *c, const float *a, const float *b, const 
 // The same with the batch index split in two, z = (z / batch_inner, z % batch_inner), each part with its own
 // stride per operand: operands that are strided views of a larger tensor (the heads of a [b, t, h, d] tensor
 // read in place as b x h matrices of t x d with row pitch h * d) need no copy.
+// post (may be null): what the operators behind the product would do to its result, done while it is written, single
+// batch only and always on the fp32 kernel: C = act(alpha * op(A) op(B) + beta * C0) + residual, act 0 or AHIP_GELU /
+// AHIP_RELU, residual null or a matrix laid out like C (same pitch).  Each step rounds as its own kernel would.
+struct GemmPost {
+    int act = 0;
+    const float *residual = nullptr;
+};
 int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t batch_outer,
                        size_t batch_inner, size_t m, size_t n, size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc,
                        const size_t a_batch_strides[2], const size_t b_batch_strides[2], const size_t c_batch_strides[2],
-                       size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta);
+                       size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta, const GemmPost *post = nullptr);
 
 // O = Softmax(scale(Q K^T) + mask) V per batch, scores kept in registers (attention.hip).  Q [tq, d], K [tk, d], V [tk, d],
 // O [tq, d] with row pitches ld*; batches as in launch_gemm_batch2; scale_op 0 none / 1 multiply / 2 divide; mask (may be

@@ -18,6 +18,7 @@
 
 #include "common.h"
 #include "ctx.h"
+#include "math.h"
 
 namespace altius {
 
@@ -49,6 +50,13 @@ struct GemmArgs {
     float alpha, beta;
     int a_vec, b_vec;  // 16-byte loads are legal for this operand (alignment of base, strides, batch stride)
 };
+
+__device__ __forceinline__ float post_ops(float v, int act, const float *__restrict__ residual, size_t at) {
+    if (act == AHIP_GELU) v = dev::gelu_elem(v);
+    else if (act == AHIP_RELU) v = dev::relu_elem(v);
+    if (residual) v = v + residual[at];
+    return v;
+}
 
 // Loads this thread's share of a BK x 128 operand tile into registers.
 // K_CONTIG: the operand's k axis is the contiguous one (A without transA, B with transB).
@@ -230,7 +238,8 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_mfma(GemmArgs g) {
 // C = alpha * (sum over k slices, in slice order) + beta * C0: the second half of a product cut along k.
 __global__ __launch_bounds__(256) void splitk_finish(float *__restrict__ c, const float *__restrict__ partials, uint32_t slices,
                                                      uint32_t m, uint32_t n, uint32_t ldc, const float *__restrict__ c0, uint32_t c0_rs,
-                                                     uint32_t c0_cs, float alpha, float beta) {
+                                                     uint32_t c0_cs, float alpha, float beta, int act,
+                                                     const float *__restrict__ residual) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, total = (size_t)m * n;
     if (i >= total) return;
     float sum = partials[i];
@@ -238,12 +247,22 @@ __global__ __launch_bounds__(256) void splitk_finish(float *__restrict__ c, cons
     const uint32_t row = (uint32_t)(i / n), col = (uint32_t)(i % n);
     float v = alpha * sum;
     if (c0) v += beta * c0[(size_t)row * c0_rs + (size_t)col * c0_cs];
-    c[(size_t)row * ldc + col] = v;
+    c[(size_t)row * ldc + col] = post_ops(v, act, residual, (size_t)row * ldc + col);
+}
+
+// c = act(c) + residual in place, for products that were not cut along k (their kernel's epilogue stays free of it:
+// sixty-four inlined activations per thread slowed every launch down).
+__global__ __launch_bounds__(256) void post_in_place(float *__restrict__ c, uint32_t m, uint32_t n, uint32_t ldc, int act,
+                                                     const float *__restrict__ residual) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)m * n) return;
+    const size_t at = (i / n) * ldc + i % n;
+    c[at] = post_ops(c[at], act, residual, at);
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-thread_local bool split_k_inner = false;  // the batched launch of the slices must not cut again
+thread_local int split_k_inner = 0;  // the batched launch of the slices must not cut again (1), and keeps the tile width chosen for the whole product (2: the narrow one)
 
 }  // namespace
 
@@ -263,11 +282,15 @@ int launch_gemm(DeviceCtx &ctx, float *c, const float *a, const float *b, const 
 int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t batch_outer,
                        size_t batch_inner, size_t m, size_t n, size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc,
                        const size_t a_batch_strides[2], const size_t b_batch_strides[2], const size_t c_batch_strides[2],
-                       size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta) {
+                       size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta, const GemmPost *post) {
     const size_t batch = batch_outer * batch_inner;
     if (batch == 0 || m == 0 || n == 0) return AHIP_OK;
     if (!c || (k && (!a || !b))) return ctx.fail(AHIP_ERR_ARG, "gemm: null pointer");
-    if (batch == 1 && gemm_takes_split(ctx, m, n, k))
+    const bool has_post = post && (post->act != 0 || post->residual);
+    if (has_post && batch != 1) return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm: an activation or a residual needs a single batch");
+    if (has_post && post->act != 0 && post->act != AHIP_GELU && post->act != AHIP_RELU)
+        return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm: only Gelu and Relu can follow the product in its kernel");
+    if (!has_post && batch == 1 && gemm_takes_split(ctx, m, n, k))
         return launch_gemm_split(ctx, c, a, b, c0, m, n, k, trans_a, trans_b, lda, ldb, ldc, c0_row_stride, c0_col_stride, alpha, beta);
     const size_t lim = (size_t)1 << 31;
     if (m >= lim || n >= lim || k >= lim || lda >= lim || ldb >= lim || ldc >= lim || m * ldc >= ((size_t)1 << 40))
@@ -278,8 +301,9 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
     // only where K is short and the tile's fixed costs weigh more, as in attention's 64-deep products).
     // ... and when the wide tile would leave CUs without a block (the slices of a product cut along k).
     const size_t cus = ctx.cus_per_xcd ? (size_t)ctx.cus_per_xcd * 8 : 256;
-    const bool narrow = n <= 64 || (n < 512 && n % 128 != 0 && n % 128 <= 64) || k >= 256 ||
-                        ((m + BM - 1) / BM) * ((n + BN - 1) / BN) * batch < cus;
+    const bool narrow = split_k_inner ? split_k_inner == 2
+                                      : n <= 64 || (n < 512 && n % 128 != 0 && n % 128 <= 64) || k >= 256 ||
+                                            ((m + BM - 1) / BM) * ((n + BN - 1) / BN) * batch < cus;
     const size_t tn = narrow ? 64 : BN;
     const size_t gy = (m + BM - 1) / BM, gx = (n + tn - 1) / tn;
     if (gy > 65535 || batch > 65535) return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm: more than 65535 row tiles or batches");
@@ -296,15 +320,16 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
             const size_t ks = k / slices;
             // slice z of op(A) starts ks columns (or rows, transposed) further on; likewise op(B)
             const size_t a_bs[2] = {trans_a ? ks * lda : ks, 0}, b_bs[2] = {trans_b ? ks : ks * ldb, 0}, c_bs[2] = {m * n, 0};
-            split_k_inner = true;
+            split_k_inner = narrow ? 2 : 1;
             rc = launch_gemm_batch2(ctx, static_cast<float *>(ws), a, b, nullptr, slices, 1, m, n, ks, trans_a, trans_b, lda, ldb, n, a_bs, b_bs,
                                     c_bs, 0, 0, 1.0f, 0.0f);
-            split_k_inner = false;
+            split_k_inner = 0;
             if (rc) return rc;
             const size_t total = m * n;
             hipLaunchKernelGGL(splitk_finish, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx.stream, c, static_cast<const float *>(ws),
                                (uint32_t)slices, (uint32_t)m, (uint32_t)n, (uint32_t)ldc, (c0 && beta != 0.0f) ? c0 : nullptr,
-                               (uint32_t)c0_row_stride, (uint32_t)c0_col_stride, alpha, beta);
+                               (uint32_t)c0_row_stride, (uint32_t)c0_col_stride, alpha, beta, has_post ? post->act : 0,
+                               has_post ? post->residual : nullptr);
             return ctx.check(hipGetLastError(), "gemm split-k finish launch");
         }
     }
@@ -352,6 +377,9 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
         else GEMM(false, false, 128);
     }
 #undef GEMM
+    if (has_post)
+        hipLaunchKernelGGL(post_in_place, dim3((unsigned)((m * n + 255) / 256)), dim3(256), 0, ctx.stream, c, (uint32_t)m, (uint32_t)n,
+                           (uint32_t)ldc, post->act, post->residual);
     return ctx.check(hipGetLastError(), "gemm launch");
 }
 

@@ -253,6 +253,7 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
     std::map<ValueId, DeviceTensor> values;
     copies_avoided_ = 0;
     pending_attn_.clear();
+    absorbed_add_.clear();
     std::vector<hipEvent_t> events;
     // Nothing may still read a block when it goes back to the pool for another run, and input
     // tensors must outlive their uploads: every exit path synchronises first.
@@ -355,6 +356,7 @@ bool HipSession::run_device(const std::vector<DeviceTensor> &inputs, std::vector
     std::map<ValueId, DeviceTensor> values;
     copies_avoided_ = 0;
     pending_attn_.clear();
+    absorbed_add_.clear();
     for (size_t i = 0; i < g.inputs.size(); i++) {
         if (!inputs[i].ptr && inputs[i].nbytes())
             return fail(err, SessionError::Argument, "run_device: input " + std::to_string(i) + " has no device pointer");
@@ -428,6 +430,7 @@ bool HipSession::try_capture(const std::string &key, const std::vector<Tensor> &
     std::map<ValueId, DeviceTensor> values;
     copies_avoided_ = 0;
     pending_attn_.clear();
+    absorbed_add_.clear();
     for (size_t i = 0; i < g.inputs.size(); i++) {
         DeviceTensor d;
         if (!allocate(TypedFixedShape{inputs[i].dims(), inputs[i].elem_ty()}, &d, err)) return false;
@@ -599,7 +602,24 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
     if (shapes.size() < node.outputs.size()) return fail(err, SessionError::Message, opname + ": output count mismatch");
 
     std::vector<DeviceTensor> outs;
+    values_ = &values;
 
+    auto absorbed = absorbed_add_.find(id);
+    if (absorbed != absorbed_add_.end() && absorbed->second < in.size() && in[absorbed->second]) {
+        // The MatMul that produced one operand has added the other one already.
+        DeviceTensor o = *in[absorbed->second];
+        absorbed_add_.erase(absorbed);
+        o.dims = shapes[0].dims;
+        copies_avoided_++;
+        outs.push_back(std::move(o));
+    } else if ((op.kind == OpKind::Gelu || op.kind == OpKind::ReLU) && in[0] && in[0]->applied_op == (op.kind == OpKind::Gelu ? AHIP_GELU : AHIP_RELU)) {
+        // The MatMul that produced the operand has applied this activation already.
+        DeviceTensor o = *in[0];
+        o.dims = shapes[0].dims;
+        o.applied_op = -1;
+        copies_avoided_++;
+        outs.push_back(std::move(o));
+    } else
     // Reshape family: the output is the input's memory under another shape.
     if (is_alias_op(op.kind) && in[0]) {
         std::vector<int64_t> view_strides;
@@ -1358,6 +1378,30 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
         const bool plain = in[0]->strides.empty() && in[1]->strides.empty() && out.strides.empty();
         if (plain && B.batch == 1 && A.batch == batch && !ta) {
             // [.., m, k] x [k, n]: one tall sgemm, as the reference does (session.rs:653-660)
+            // On the fp32 kernel, the activation or the residual Add behind the product is done as it is written.
+            auto mp = matmul_post_.find(current_node_);
+            if (!a_op && mp != matmul_post_.end() && !gemm_takes_split(ctx_, batch * m, n, k)) {
+                GemmPost post;
+                if (mp->second.act) {
+                    post.act = mp->second.act;
+                } else if (mp->second.has_add && values_) {
+                    const DeviceTensor *x = nullptr;
+                    auto xv = values_->find(mp->second.residual);
+                    if (xv != values_->end()) x = &xv->second;
+                    else if (auto xi = inits_.find(mp->second.residual); xi != inits_.end()) x = &xi->second;
+                    if (x && x->ptr && x->elem_ty == TensorElemType::F32 && x->strides.empty() && x->pending_op < 0 && x->applied_op < 0 &&
+                        x->dims == out.dims)
+                        post.residual = static_cast<const float *>(x->ptr);
+                }
+                if (post.act || post.residual) {
+                    const size_t none[2] = {0, 0};
+                    rc = launch_gemm_batch2(ctx_, o, f(in[0]), f(in[1]), bias, 1, 1, batch * m, n, k, 0, tb, A.ld, B.ld, n, none, none, none, 0, 1, 1.0f,
+                                            beta, &post);
+                    if (!rc && post.act) out.applied_op = post.act;
+                    if (!rc && post.residual) absorbed_add_[mp->second.add_node] = mp->second.add_input;
+                    break;
+                }
+            }
             if (a_op) rc = launch_gemm_split(ctx_, o, f(in[0]), f(in[1]), bias, batch * m, n, k, 0, tb, A.ld, B.ld, n, 0, 1, 1.0f, beta, a_op);
             else rc = launch_gemm(ctx_, o, f(in[0]), f(in[1]), bias, 1, batch * m, n, k, 0, tb, A.ld, B.ld, n, 0, 0, 0, 0, 1, 1.0f, beta);
             break;

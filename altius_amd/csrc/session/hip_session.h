@@ -89,6 +89,9 @@ struct DeviceTensor {
     // An activation (AHIP_GELU / AHIP_RELU) that has not been applied yet: the tensor holds the
     // activation's input, and its one reader, a MatMul, applies it while splitting the operand.
     int pending_op = -1;
+    // An activation (AHIP_GELU / AHIP_RELU) that the MatMul which produced the tensor has already applied while
+    // writing it: the activation node that follows passes the tensor on.
+    int applied_op = -1;
     size_t nbytes() const { return dims.total_elems() * elem_size(elem_ty); }
 };
 
@@ -226,6 +229,18 @@ private:
     std::map<NodeId, AttentionPlan> attn_head_;                  // first MatMul of a fusable attention -> the rest
     std::set<NodeId> attn_softmax_, attn_tail_;
     std::map<ValueId, PendingAttention> pending_attn_;
+    // What follows a MatMul whose result has one reader and can be done while the product is written (fp32 kernel):
+    // a Gelu / Relu node, or an Add of a tensor of the result's shape (a residual connection).
+    struct MatMulPost {
+        int act = 0;            // AHIP_GELU / AHIP_RELU, 0: none
+        bool has_add = false;
+        NodeId add_node = 0;
+        size_t add_input = 0;   // which input of the Add is the product
+        ValueId residual = 0;   // the Add's other input
+    };
+    std::map<NodeId, MatMulPost> matmul_post_;
+    std::map<NodeId, size_t> absorbed_add_;                     // Add nodes whose sum a MatMul wrote in this run -> input holding it
+    const std::map<ValueId, DeviceTensor> *values_ = nullptr;   // the running call's values, for run_device_op
     std::set<NodeId> deferred_unary_;                           // Gelu / Relu nodes folded into the MatMul that reads them
     std::set<NodeId> lazy_views_;                               // Split / Transpose nodes whose outputs are views
     std::map<NodeId, std::vector<int64_t>> matmul_out_perm_;    // MatMul nodes -> perm of the Transpose they feed  // recorded launches hold the GEMM workspace's address

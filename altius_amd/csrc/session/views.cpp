@@ -275,6 +275,22 @@ void HipSession::plan_views() {
         } else if (n.op.kind == OpKind::MatMul && n.outputs.size() == 1 && !is_output(n.outputs[0])) {
             auto it = users.find(n.outputs[0]);
             if (it == users.end() || it->second.size() != 1) continue;
+            // MatMul -> Gelu / Relu, or MatMul -> Add(residual): done by the product's own kernel when it is the fp32 one.
+            {
+                const NodeId uid = *it->second.begin();
+                const Node &u = g.nodes[uid];
+                MatMulPost mp;
+                if ((u.op.kind == OpKind::Gelu || u.op.kind == OpKind::ReLU) && u.inputs.size() == 1 && u.outputs.size() == 1) {
+                    mp.act = u.op.kind == OpKind::Gelu ? AHIP_GELU : AHIP_RELU;
+                    matmul_post_[id] = mp;
+                } else if (u.op.kind == OpKind::Add && u.inputs.size() == 2 && u.outputs.size() == 1 && u.inputs[0] != u.inputs[1]) {
+                    mp.has_add = true;
+                    mp.add_node = uid;
+                    mp.add_input = u.inputs[0] == n.outputs[0] ? 0 : 1;
+                    mp.residual = u.inputs[1 - mp.add_input];
+                    matmul_post_[id] = mp;
+                }
+            }
             // MatMul -> Softmax(last axis, optional scalar scale, no mask) -> MatMul(first operand): one attention kernel.
             {
                 const NodeId sid = *it->second.begin();

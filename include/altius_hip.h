@@ -279,6 +279,16 @@ int ahip_gemm_activated(ahip_ctx *ctx, int a_op, float *c, const float *a, const
                         size_t n, size_t k, int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc,
                         size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta);
 
+/* C = act(alpha * op(A) * op(B) + beta * C0) + residual for one batch, always on the fp32 kernel: the operators that
+ * follow a product in a transformer block (Gelu after the MLP's first MatMul; the residual Add after its second one
+ * and after attention's projection: compute_gelu session.rs:823-838, compute_add session.rs:537) done while C is
+ * written, so that neither costs a pass or a launch of its own.  act: 0 (none), AHIP_GELU or AHIP_RELU; residual: NULL
+ * or a matrix laid out like C (same pitch ldc).  Every step rounds as its own kernel would: the result has the bits
+ * of ahip_gemm (with AHIP_GEMM_FP32) -> ahip_unary -> ahip_binary(AHIP_ADD).  No counterpart in the reference. */
+int ahip_gemm_post(ahip_ctx *ctx, float *c, const float *a, const float *b, const float *c0, size_t m, size_t n, size_t k,
+                   int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t c0_row_stride, size_t c0_col_stride,
+                   float alpha, float beta, int act, const float *residual);
+
 /* O = Softmax(scale(Q K^T) + mask) V for batch_outer * batch_inner independent (batch, head) pairs in one kernel: the
  * MatMul -> (Mul | Div by a scalar) -> (Add of a per-key mask) -> Softmax(last axis) -> MatMul chain of an attention block
  * (session.rs:621-684, 990-1026) without the [tq, tk] score tensor ever reaching memory.  Q is [tq, d] with row

@@ -221,7 +221,7 @@ def test_matmul_writes_the_layout_of_the_transpose_behind_it(case):
 # ---- the activation between two products, folded into the second one's operand split ----
 
 from altius_amd import device as D  # noqa: E402
-from altius_amd._lib import ERR_UNSUPPORTED, AltiusHipError, check  # noqa: E402
+from altius_amd._lib import ERR_ARG, ERR_UNSUPPORTED, AltiusHipError, check  # noqa: E402
 
 
 def mlp(rows, hidden, inner, act, second_reader=False):
@@ -262,12 +262,21 @@ def test_activation_between_two_products(case, act, algo):
     np.testing.assert_allclose(outs[0], a @ w2, rtol=2e-3, atol=2e-3)      # the reference's Gelu is the tanh form (fast_gelu)
 
 
-def test_activation_with_a_second_reader_runs_on_its_own(case):
+def test_activation_with_a_second_reader_is_never_left_pending(case):
+    """A Gelu that a MatMul and an element-wise operator both read cannot wait for the second product's operand split.
+    On the fp32 kernel the product in front of it applies it (one node served per run); on the bf16 route it runs as
+    its own kernel."""
     case("Gelu read by a MatMul and by an element-wise operator")
     m, _ = mlp((20,), 16, 24, Op.Gelu, second_reader=True)
     x = RNG.standard_normal((20, 16)).astype(np.float32)
     (y, z), avoided = run_both(m, [x])
-    assert avoided == 0
+    assert avoided == 1
+    sess = HipSessionBuilder(m.clone()).with_gemm_algorithm(D.GEMM_BF16X3).build()
+    y2, z2 = (np.array(t) for t in sess.run([Tensor.from_numpy(x)]))
+    assert sess.copies_avoided() == 0
+    sess.close()
+    np.testing.assert_allclose(y2, y, rtol=1e-5, atol=1e-5)  # the first product's sums are rounded in another order
+    np.testing.assert_allclose(z2, z, rtol=1e-5, atol=1e-5)
 
 
 def test_gemm_activated_through_the_c_abi(ctx, case):
@@ -289,6 +298,87 @@ def test_gemm_activated_through_the_c_abi(ctx, case):
     finally:
         ctx.gemm_set_algorithm(D.GEMM_AUTO)
         for x in (da, db, dc):
+            ctx.free(x)
+
+
+def transformer_mlp(rows, hidden, inner, residual_first):
+    """x -> MatMul + bias -> Gelu -> MatMul + bias -> Add(x): the second half of a transformer block."""
+    m = Model(opset_version=13)
+    x = m.new_val_named_and_shaped("x", list(rows) + [hidden])
+    m.add_input(x)
+    w1 = (RNG.standard_normal((hidden, inner)) * 0.2).astype(np.float32)
+    w2 = (RNG.standard_normal((inner, hidden)) * 0.2).astype(np.float32)
+    b1 = RNG.standard_normal(inner).astype(np.float32)
+    b2 = RNG.standard_normal(hidden).astype(np.float32)
+    h = node(m, Op.Add, [node(m, Op.MatMul, [x, m.new_initializer(w1)]), m.new_initializer(b1)])
+    y = node(m, Op.Add, [node(m, Op.MatMul, [node(m, Op.Gelu, [h]), m.new_initializer(w2)]), m.new_initializer(b2)])
+    m.add_output(node(m, Op.Add, [x, y] if residual_first else [y, x]))
+    m.fuse_matmul_bias()
+    return m
+
+
+@pytest.mark.parametrize("rows,hidden,inner", [((197,), 768, 3072), ((3, 50), 40, 72), ((1,), 16, 8)])
+@pytest.mark.parametrize("residual_first", [True, False])
+def test_gelu_and_residual_add_ride_on_the_fp32_products(case, rows, hidden, inner, residual_first):
+    """On the fp32 kernel the Gelu behind the first product and the residual Add behind the second are done while the
+    products are written (the first shape through the k cut's finishing kernel): two nodes served without a kernel, and the
+    bits of the separate operators."""
+    case(f"MatMul -> Gelu -> MatMul -> Add(residual), rows {rows}, {hidden} -> {inner}")
+    m = transformer_mlp(rows, hidden, inner, residual_first)
+    x = RNG.standard_normal(tuple(rows) + (hidden,)).astype(np.float32)
+    outs = []
+    for views in (True, False):
+        sess = HipSessionBuilder(m.clone()).with_gemm_algorithm(D.GEMM_FP32).with_strided_views(views).build()
+        for _ in range(2):
+            got = np.array(sess.run([Tensor.from_numpy(x)])[0])
+        assert sess.copies_avoided() == (2 if views else 0)  # the Gelu node and the Add node
+        sess.close()
+        outs.append(got)
+    assert_bits_equal(outs[0], outs[1], "done by the products vs separate operators")
+
+
+def test_residual_that_is_not_the_products_shape_stays_an_add(case):
+    """Add(product, row vector) broadcasts: not a residual the product can absorb."""
+    case("MatMul -> Add(broadcast operand)")
+    m = Model(opset_version=13)
+    x = m.new_val_named_and_shaped("x", [20, 16])
+    r = m.new_val_named_and_shaped("r", [1, 24])
+    m.add_input(x)
+    m.add_input(r)
+    w = (RNG.standard_normal((16, 24)) * 0.2).astype(np.float32)
+    m.add_output(node(m, Op.Add, [node(m, Op.MatMul, [x, m.new_initializer(w)]), r]))
+    xs = RNG.standard_normal((20, 16)).astype(np.float32)
+    rs = RNG.standard_normal((1, 24)).astype(np.float32)
+    (y,), avoided = run_both(m, [xs, rs])
+    assert avoided == 0
+    np.testing.assert_allclose(y, xs.astype(np.float64) @ w + rs, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("m,k,n", [(197, 768, 3072), (130, 70, 90), (300, 1024, 96), (1, 16, 5)])
+def test_gemm_post_through_the_c_abi(ctx, case, m, k, n):
+    case(f"ahip_gemm_post vs ahip_gemm + ahip_unary + ahip_binary, [{m},{k}]x[{k},{n}]")
+    a = RNG.standard_normal((m, k)).astype(np.float32)
+    b = (RNG.standard_normal((k, n)) * 0.1).astype(np.float32)
+    bias = RNG.standard_normal(n).astype(np.float32)
+    res = RNG.standard_normal((m, n)).astype(np.float32)
+    da, db, dbias, dres, dc = ctx.upload(a), ctx.upload(b), ctx.upload(bias), ctx.upload(res), ctx.alloc(m * n * 4)
+    try:
+        ctx.gemm_set_algorithm(D.GEMM_FP32)
+        plain = ctx.matmul(a, b) + bias     # the kernel's own 1 * acc + 1 * bias rounds like this Add
+        for act in (0, D.GELU, D.RELU):
+            for with_res in (False, True):
+                check(ctx.L.ahip_gemm_post(ctx.handle, dc.ptr, da.ptr, db.ptr, dbias.ptr, m, n, k, 0, 0, k, n, n, 0, 1, 1.0, 1.0, act,
+                                           dres.ptr if with_res else None), ctx.handle)
+                want = plain if act == 0 else ctx.unary(act, plain)
+                if with_res:
+                    want = want + res
+                assert_bits_equal(ctx.download(dc, (m, n)), want, f"act {act}, residual {with_res}")
+        with pytest.raises(AltiusHipError) as e:
+            check(ctx.L.ahip_gemm_post(ctx.handle, dc.ptr, da.ptr, db.ptr, None, m, n, k, 0, 0, k, n, n, 0, 0, 1.0, 0.0, D.SIGMOID, None), ctx.handle)
+        assert e.value.code == ERR_ARG
+    finally:
+        ctx.gemm_set_algorithm(D.GEMM_AUTO)
+        for x in (da, db, dbias, dres, dc):
             ctx.free(x)
 
 
