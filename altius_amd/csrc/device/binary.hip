@@ -276,19 +276,22 @@ __global__ __launch_bounds__(BLOCK) void binary_rowbcast(float *__restrict__ out
 }
 
 // ---------------------------------------------------------------------------
-// Two-axis kernel for rows that are whole float4s: out[r][c] = full[r][c] op small[c]
-// (a bias or scale vector on rows longer than the row-broadcast kernel stages) or
-// out[r][c] = full[r][c] op small[r] (a per-row mean or deviation).  A lane's four
-// elements lie in one row, so the dense 16-byte load goes out before any index
-// arithmetic and the small operand costs one more load: 16 bytes that hit in L1, or
-// one dword that most lanes of the wavefront share.
+// Kernel for rows that are whole float4s with a small operand that is constant along or across the row:
+//   out[r][c] = full[r][c] op small[c]            a bias or scale vector on rows longer than the row-broadcast kernel stages
+//   out[n][r][c] = full[n][r][c] op small[n][c]   the same with one vector per outer index (an attention mask on long rows)
+//   out[r][c] = full[r][c] op small[r]            a per-row mean or deviation, a squeeze-excite gate [N,C,1,1] on [N,C,H,W]
+//   out[n][k][c] = full[n][k][c] op small[k]      a per-channel scale or bias [C,1,1] on [N,C,H,W]
+// A lane's four elements lie in one row, so the dense 16-byte load goes out before any index arithmetic and the small
+// operand costs one more load: 16 bytes that hit in L1, or one dword that most lanes of the wavefront share.
 // ---------------------------------------------------------------------------
-enum { SMALL_VECTOR = 0, SMALL_COLUMN = 1 };
+enum { SMALL_VECTOR = 0, SMALL_VECTOR_OUTER = 1, SMALL_COLUMN = 2, SMALL_COLUMN_MOD = 3 };
 
+// c: the row length.  o: elements per outer index (SMALL_VECTOR_OUTER) or the number of values the rows cycle
+// through (SMALL_COLUMN_MOD); unused otherwise.
 template <class OP, int KIND, bool SMALL_IS_A, bool NT>
 __global__ __launch_bounds__(BLOCK) void binary_rows4(float *__restrict__ out, const float *__restrict__ full,
                                                       const float *__restrict__ small, uint32_t total,
-                                                      const FastDiv c) {
+                                                      const FastDiv c, const FastDiv o) {
     const uint32_t i0 = (blockIdx.x * BLOCK + threadIdx.x) * 4;
     if (i0 >= total) return;  // total is a multiple of 4
     const float4 x = load4<NT>(full + i0);
@@ -296,8 +299,10 @@ __global__ __launch_bounds__(BLOCK) void binary_rows4(float *__restrict__ out, c
     float4 y;
     if (KIND == SMALL_VECTOR) {
         y = *reinterpret_cast<const float4 *>(small + (i0 - row * c.d));
+    } else if (KIND == SMALL_VECTOR_OUTER) {
+        y = *reinterpret_cast<const float4 *>(small + (o.div(i0) * c.d + (i0 - row * c.d)));
     } else {
-        const float v = small[row];
+        const float v = small[KIND == SMALL_COLUMN ? row : row - o.div(row) * o.d];
         y = make_float4(v, v, v, v);
     }
     float4 r;
@@ -306,6 +311,42 @@ __global__ __launch_bounds__(BLOCK) void binary_rows4(float *__restrict__ out, c
     r.z = SMALL_IS_A ? OP::f(y.z, x.z) : OP::f(x.z, y.z);
     r.w = SMALL_IS_A ? OP::f(y.w, x.w) : OP::f(x.w, y.w);
     store4<NT>(out + i0, r);
+}
+
+// One value per row (or per channel) on rows of any length from 4 up (7 x 7 feature maps): a lane's four elements
+// lie in at most two rows, so it reads this row's value and, only if its elements reach into it, the next row's.
+// MOD: the rows cycle through o.d values.
+template <class OP, bool MOD, bool SMALL_IS_A, bool NT>
+__global__ __launch_bounds__(BLOCK) void binary_rows_any(float *__restrict__ out, const float *__restrict__ full,
+                                                         const float *__restrict__ small, uint32_t total,
+                                                         const FastDiv c, const FastDiv o) {
+    const uint32_t i0 = (blockIdx.x * BLOCK + threadIdx.x) * 4;
+    if (i0 >= total) return;
+    const bool whole = i0 + 4 <= total;
+    float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (whole) x = load4<NT>(full + i0);
+    const uint32_t row = c.div(i0), c0 = i0 - row * c.d;
+    const uint32_t in_row = c.d - c0;  // elements of this lane that still belong to `row` (if < 4)
+    const float v0 = small[MOD ? row - o.div(row) * o.d : row];
+    float v1 = v0;
+    if (in_row < 4 && i0 + in_row < total) {
+        const uint32_t next = row + 1;
+        v1 = small[MOD ? next - o.div(next) * o.d : next];
+    }
+    const float y[4] = {v0, in_row > 1 ? v0 : v1, in_row > 2 ? v0 : v1, in_row > 3 ? v0 : v1};
+    if (whole) {
+        float4 r;
+        r.x = SMALL_IS_A ? OP::f(y[0], x.x) : OP::f(x.x, y[0]);
+        r.y = SMALL_IS_A ? OP::f(y[1], x.y) : OP::f(x.y, y[1]);
+        r.z = SMALL_IS_A ? OP::f(y[2], x.z) : OP::f(x.z, y[2]);
+        r.w = SMALL_IS_A ? OP::f(y[3], x.w) : OP::f(x.w, y[3]);
+        store4<NT>(out + i0, r);
+    } else {
+        for (int j = 0; j < 4 && i0 + j < total; j++) {
+            const float xs = full[i0 + j];
+            out[i0 + j] = SMALL_IS_A ? OP::f(y[j], xs) : OP::f(xs, y[j]);
+        }
+    }
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -376,20 +417,48 @@ void rowbcast_launch(hipStream_t s, bool small_is_a, bool nt, float *out, const 
     }
 }
 
-template <class OP>
-void rows4_launch(hipStream_t s, int kind, bool small_is_a, bool nt, float *out, const float *full, const float *small,
-                  uint32_t total, const FastDiv &c) {
+template <class OP, int KIND>
+void rows4_launch_kind(hipStream_t s, bool small_is_a, bool nt, float *out, const float *full, const float *small, uint32_t total,
+                       const FastDiv &c, const FastDiv &o) {
     const dim3 grid((total / 4 + BLOCK - 1) / BLOCK);
-#define ALTIUS_ROWS4(K, A, N) \
-    hipLaunchKernelGGL((binary_rows4<OP, K, A, N>), grid, dim3(BLOCK), 0, s, out, full, small, total, c)
-    if (kind == SMALL_VECTOR) {
-        if (small_is_a) { if (nt) ALTIUS_ROWS4(SMALL_VECTOR, true, true); else ALTIUS_ROWS4(SMALL_VECTOR, true, false); }
-        else { if (nt) ALTIUS_ROWS4(SMALL_VECTOR, false, true); else ALTIUS_ROWS4(SMALL_VECTOR, false, false); }
+#define ALTIUS_ROWS4(A, N) hipLaunchKernelGGL((binary_rows4<OP, KIND, A, N>), grid, dim3(BLOCK), 0, s, out, full, small, total, c, o)
+    if (small_is_a) {
+        if (nt) ALTIUS_ROWS4(true, true);
+        else ALTIUS_ROWS4(true, false);
     } else {
-        if (small_is_a) { if (nt) ALTIUS_ROWS4(SMALL_COLUMN, true, true); else ALTIUS_ROWS4(SMALL_COLUMN, true, false); }
-        else { if (nt) ALTIUS_ROWS4(SMALL_COLUMN, false, true); else ALTIUS_ROWS4(SMALL_COLUMN, false, false); }
+        if (nt) ALTIUS_ROWS4(false, true);
+        else ALTIUS_ROWS4(false, false);
     }
 #undef ALTIUS_ROWS4
+}
+
+template <class OP>
+void rows_any_launch(hipStream_t s, bool mod, bool small_is_a, bool nt, float *out, const float *full, const float *small,
+                     uint32_t total, const FastDiv &c, const FastDiv &o) {
+    const dim3 grid(((total + 3) / 4 + BLOCK - 1) / BLOCK);
+#define ALTIUS_ROWS_ANY(M, A, N) hipLaunchKernelGGL((binary_rows_any<OP, M, A, N>), grid, dim3(BLOCK), 0, s, out, full, small, total, c, o)
+#define ALTIUS_ROWS_ANY_M(M)                                  \
+    if (small_is_a) {                                         \
+        if (nt) ALTIUS_ROWS_ANY(M, true, true);               \
+        else ALTIUS_ROWS_ANY(M, true, false);                 \
+    } else {                                                  \
+        if (nt) ALTIUS_ROWS_ANY(M, false, true);              \
+        else ALTIUS_ROWS_ANY(M, false, false);                \
+    }
+    if (mod) { ALTIUS_ROWS_ANY_M(true) } else { ALTIUS_ROWS_ANY_M(false) }
+#undef ALTIUS_ROWS_ANY_M
+#undef ALTIUS_ROWS_ANY
+}
+
+template <class OP>
+void rows4_launch(hipStream_t s, int kind, bool small_is_a, bool nt, float *out, const float *full, const float *small,
+                  uint32_t total, const FastDiv &c, const FastDiv &o) {
+    switch (kind) {
+    case SMALL_VECTOR: rows4_launch_kind<OP, SMALL_VECTOR>(s, small_is_a, nt, out, full, small, total, c, o); break;
+    case SMALL_VECTOR_OUTER: rows4_launch_kind<OP, SMALL_VECTOR_OUTER>(s, small_is_a, nt, out, full, small, total, c, o); break;
+    case SMALL_COLUMN: rows4_launch_kind<OP, SMALL_COLUMN>(s, small_is_a, nt, out, full, small, total, c, o); break;
+    default: rows4_launch_kind<OP, SMALL_COLUMN_MOD>(s, small_is_a, nt, out, full, small, total, c, o); break;
+    }
 }
 
 }  // namespace
@@ -510,27 +579,45 @@ int launch_binary(DeviceCtx &ctx, int op, float *out, const float *a, const floa
         }
     }
 
-    // Two axes, rows of whole float4s, one operand dense and the other a vector along the row
-    // (strides [0,1]) or one value per row (strides [1,0]).
+    // Rows of whole float4s, one operand dense and the other constant along or across the row (see binary_rows4).
     {
         const int64_t *ss = ma == STRIDED ? as : bs;
         const int other = ma == STRIDED ? mb : ma;
         const bool small_is_a = ma == STRIDED;
         const float *full = small_is_a ? b : a;
         const float *small = small_is_a ? a : b;
-        const bool vector = r == 2 && ss[0] == 0 && ss[1] == 1, column = r == 2 && ss[0] == 1 && ss[1] == 0;
-        if (other == FULL && (vector || column) && dims[1] % 4 == 0 && total < LIMIT && aligned16(out) &&
-            aligned16(full) && (column || aligned16(small))) {
-            const FastDiv c = make_fastdiv((uint32_t)dims[1]);
-            const int kind = vector ? SMALL_VECTOR : SMALL_COLUMN;
+        int kind = -1;
+        uint32_t second = 1;
+        if (r == 2 && ss[0] == 0 && ss[1] == 1) kind = SMALL_VECTOR;
+        else if (r == 2 && ss[0] == 1 && ss[1] == 0) kind = SMALL_COLUMN;
+        else if (r == 3 && ss[0] == dims[2] && ss[1] == 0 && ss[2] == 1) kind = SMALL_VECTOR_OUTER, second = (uint32_t)(dims[1] * dims[2]);
+        else if (r == 3 && ss[0] == 0 && ss[1] == 1 && ss[2] == 0) kind = SMALL_COLUMN_MOD, second = (uint32_t)dims[1];
+        const bool vector = kind == SMALL_VECTOR || kind == SMALL_VECTOR_OUTER;
+        if (other == FULL && kind >= 0 && dims[r - 1] % 4 == 0 && total < LIMIT && aligned16(out) && aligned16(full) &&
+            (!vector || aligned16(small))) {
+            const FastDiv c = make_fastdiv((uint32_t)dims[r - 1]), o = make_fastdiv(second);
             switch (op) {
-            case AHIP_ADD: rows4_launch<OpAdd>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c); break;
-            case AHIP_SUB: rows4_launch<OpSub>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c); break;
-            case AHIP_MUL: rows4_launch<OpMul>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c); break;
-            case AHIP_DIV: rows4_launch<OpDiv>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c); break;
-            case AHIP_POW: rows4_launch<OpPow>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c); break;
+            case AHIP_ADD: rows4_launch<OpAdd>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
+            case AHIP_SUB: rows4_launch<OpSub>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
+            case AHIP_MUL: rows4_launch<OpMul>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
+            case AHIP_DIV: rows4_launch<OpDiv>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
+            case AHIP_POW: rows4_launch<OpPow>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
             }
-            return ctx.check(hipGetLastError(), "binary two-axis launch");
+            return ctx.check(hipGetLastError(), "binary row-aligned broadcast launch");
+        }
+        // One value per row or per channel on rows of any other length from 4 up.
+        if (other == FULL && (kind == SMALL_COLUMN || kind == SMALL_COLUMN_MOD) && dims[r - 1] >= 4 && total < LIMIT && aligned16(out) &&
+            aligned16(full)) {
+            const FastDiv c = make_fastdiv((uint32_t)dims[r - 1]), o = make_fastdiv(second);
+            const bool mod = kind == SMALL_COLUMN_MOD;
+            switch (op) {
+            case AHIP_ADD: rows_any_launch<OpAdd>(s, mod, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
+            case AHIP_SUB: rows_any_launch<OpSub>(s, mod, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
+            case AHIP_MUL: rows_any_launch<OpMul>(s, mod, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
+            case AHIP_DIV: rows_any_launch<OpDiv>(s, mod, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
+            case AHIP_POW: rows_any_launch<OpPow>(s, mod, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
+            }
+            return ctx.check(hipGetLastError(), "binary per-row broadcast launch");
         }
     }
 

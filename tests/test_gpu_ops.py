@@ -60,6 +60,23 @@ BIN_SHAPES = [
     ([1, 4], [3, 5, 4]),
     ([64, 197, 3072], [3072]),         # above the size at which accesses become non-temporal
     ([64, 197, 3072], [64, 197, 1]),
+    # the same kernel's three-axis forms: one vector per outer index, one value per channel
+    ([2, 4, 10, 1028], [2, 1, 1, 1028]),  # a mask on rows too long for the kernel that stages it in LDS
+    ([2, 1, 1, 1028], [2, 4, 10, 1028]),
+    ([2, 3, 8, 8], [3, 1, 1]),           # per-channel bias on NCHW
+    ([1, 3, 1, 1], [2, 3, 8, 8]),
+    ([4, 6, 4, 4], [4, 6, 1, 1]),        # squeeze-excite gate
+    ([5, 7, 2, 6], [7, 1, 1]),
+    ([128, 96, 56, 56], [96, 1, 1]),     # non-temporal variant
+    # one value per row or channel on rows that are not whole float4s (lanes straddling two rows, ragged end)
+    ([5, 7, 3, 3], [7, 1, 1]),
+    ([7, 1, 1], [5, 7, 3, 3]),
+    ([3, 5, 7], [3, 5, 1]),
+    ([2, 3, 5], [3, 1]),
+    ([3, 5, 1], [3, 5, 7]),
+    ([9, 4], [9, 1]),
+    ([64, 576, 7, 7], [576, 1, 1]),
+    ([768, 1024, 7, 7], [768, 1024, 1, 1]),  # non-temporal variant
 ]
 
 
