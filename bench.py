@@ -473,16 +473,16 @@ def time_kernel(ctx, op, iters, warmup):
     return ms
 
 
-def cpu_baseline(synth, batch_full, sample_batch, threads):
-    """Times the oracle on a reduced batch of the same step; returns GB/s and per-op seconds."""
+def cpu_baseline(synth, batch_full, sample_batch, threads, arrays=None):
+    """Times the oracle on the same step (the whole batch, or a reduced one); returns GB/s and per-op seconds."""
     import oracle as O
 
     O.lib()
-    c = synth.cfg4(batch=sample_batch)
+    c = arrays if arrays is not None and sample_batch == batch_full else synth.cfg4(batch=sample_batch)
     times = {}
     total_bytes = 0
 
-    def timed(name, nbytes, fn, reps=2):
+    def timed(name, nbytes, fn, reps=3):
         nonlocal total_bytes
         best = float("inf")
         for _ in range(reps):
@@ -513,7 +513,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=256, help="batch of configs[4] (256 = the named workload)")
     ap.add_argument("--kernel-iters", type=int, default=50, help="launches per kernel for the per-kernel timing")
-    ap.add_argument("--cpu-sample-batch", type=int, default=32, help="batch of the CPU baseline sample")
+    ap.add_argument("--cpu-sample-batch", type=int, default=0,
+                    help="batch of the CPU baseline sample (0: the whole batch, about 2 s of CPU time)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", type=str, default="", help="run only kernels whose name contains this text (profiling)")
     ap.add_argument("--calibrate", action="store_true",
@@ -676,11 +677,12 @@ def main():
 
     if not args.no_cpu:
         threads = min(16, os.cpu_count() or 1)
-        gbps_n, t_n = cpu_baseline(synth, args.batch, args.cpu_sample_batch, threads)
-        gbps_1, t_1 = cpu_baseline(synth, args.batch, args.cpu_sample_batch, 1)
-        scale = args.batch / args.cpu_sample_batch
+        sample = args.cpu_sample_batch or args.batch
+        gbps_n, t_n = cpu_baseline(synth, args.batch, sample, threads, cfg4_arrays)
+        gbps_1, t_1 = cpu_baseline(synth, args.batch, sample, 1, cfg4_arrays)
+        scale = args.batch / sample
         log("CPU oracle, batch %d sample (x%.0f for the full step): %d threads %.2f GB/s, 1 thread %.2f GB/s"
-            % (args.cpu_sample_batch, scale, threads, gbps_n, gbps_1))
+            % (sample, scale, threads, gbps_n, gbps_1))
         for k in t_n:
             log("  %-10s %d threads %9.1f us   1 thread %9.1f us  (scaled to batch %d)"
                 % (k, threads, t_n[k] * scale * 1e6, t_1[k] * scale * 1e6, args.batch))
@@ -689,8 +691,8 @@ def main():
             "unit": "GB/s",
             "cores": threads,
             "kind": "port",
-            "sample": "same four kernels at batch %d of %d (1/%d of the step), best of 2 runs; "
-                      "1 thread: %.2f GB/s" % (args.cpu_sample_batch, args.batch, int(scale), gbps_1),
+            "sample": "same four kernels at batch %d of %d (1/%d of the step), best of 3 runs; "
+                      "1 thread: %.2f GB/s" % (sample, args.batch, int(scale), gbps_1),
             "single_thread_value": round(gbps_1, 2),
             "us_per_kernel_scaled": {k: round(v * scale * 1e6, 1) for k, v in t_n.items()},
         }
