@@ -291,3 +291,39 @@ def test_gpt2_style_decoder_block(case):
     ops = set(sess.profile())
     assert {"LayerNormalization", "Gemm", "Where", "Softmax", "Gather", "MatMul", "Gelu"} <= ops
     assert not ops & {"Tanh", "Pow", "Sqrt", "ReduceMean"}      # the tanh chain became Gelu, the LayerNorm chains one node each
+
+
+@pytest.mark.parametrize("batch", [1, 8, 24])
+def test_full_width_vit_encoder_every_fast_path_agrees_with_the_plain_one(case, batch):
+    """A ViT-B/16-shaped encoder at full width (12 layers, 768 wide, 12 heads of 64, 197 tokens) after the reference's own
+    rewrites, run the plain way (fp32 kernels only, every operator its own kernel, no views) and with everything this
+    backend adds (softmax prologue, MatMul bias, element-wise chains, views, one-kernel attention, the activation and
+    the residual Add done by the products, the k cut at batch 1, the bf16 route from batch 8 on, graph replay): the
+    logits agree to 2e-4 of their range, and replaying gives the eager run's bits."""
+    from altius_amd import device as D
+    from altius_amd import graphs
+    from altius_amd.graph import Tensor
+
+    case(f"full-width ViT-B/16-shaped encoder, batch {batch}")
+    base = graphs.vit_encoder(batch, layers=12)
+    assert base.fuse_layer_norm() == 25 and base.fuse_gelu() == 12
+    base.eliminate_identity()
+    x = Tensor.from_numpy(np.random.default_rng(5).standard_normal((batch, 197, 768)).astype(np.float32))
+
+    plain = HipSessionBuilder(base.clone()).with_gemm_algorithm(D.GEMM_FP32).with_strided_views(False).build()
+    want = np.array(plain.run([x])[0])
+    assert plain.copies_avoided() == 0
+    plain.close()
+
+    fast = base.clone()
+    fast.fuse_softmax_prologue(), fast.fuse_matmul_bias(), fast.fuse_transpose_matmul(), fast.fuse_elemwise_ops(extended=True)
+    sess = HipSessionBuilder(fast).with_graph_replay().build()
+    got = np.array(sess.run([x])[0])
+    assert sess.copies_avoided() > 0
+    scale = float(np.abs(want).max())
+    np.testing.assert_allclose(got, want, rtol=0, atol=2e-4 * scale)
+    for _ in range(3):  # the second run records, later ones replay
+        again = np.array(sess.run([x])[0])
+        assert np.array_equal(again, got)
+    assert sess.graph_replays() >= 1
+    sess.close()
