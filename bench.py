@@ -337,7 +337,7 @@ def vit_table(batch, layers=12):
     ours.fuse_softmax_prologue(), ours.fuse_matmul_bias(), ours.fuse_transpose_matmul(), ours.fuse_elemwise_ops(extended=True)
     versions.append(("+ softmax prologue, matmul bias / transposes, element-wise chains", ours))
     versions.append(("+ large products on the bf16 matrix cores (three planes per operand)", ours))
-    versions.append(("+ strided views, one-kernel attention, Gelu folded into fc2's operand split", ours))
+    versions.append(("+ strided views, one-kernel attention, Gelu and residual Add done by the products around them", ours))
     rows = []
     for i, (name, model) in enumerate(versions):
         algo = D.GEMM_AUTO if i >= 3 else D.GEMM_FP32
