@@ -45,6 +45,39 @@ def test_binary_operators_on_random_broadcasts(case, ctx):
         assert_bits_equal(got, O.binary(o, a, b), f"#{i} {sa} {sb}")
 
 
+def test_binary_operators_on_the_patterns_with_kernels_of_their_own(case, ctx):
+    """The broadcast patterns that models produce (a trailing vector, one value per row, one value per channel, one
+    vector per outer index, either operand order), over extents on both sides of every kernel's conditions (rows that
+    are and are not whole float4s, short and long rows), against NumPy's IEEE results bit for bit."""
+    rng = np.random.default_rng(515)
+    ops = [(D.ADD, np.add), (D.SUB, np.subtract), (D.MUL, np.multiply), (D.DIV, np.divide)]
+    extents = [1, 2, 3, 4, 5, 7, 8, 12, 16, 33, 49, 64, 100, 197, 256, 516, 1028]
+    for i in range(500):
+        rank = int(rng.integers(2, 5))
+        dims = [int(rng.choice(extents)) for _ in range(rank)]
+        while np.prod(dims) > 1_500_000:
+            dims[int(rng.integers(0, rank))] = 2
+        kind = int(rng.integers(0, 4))
+        small = list(dims)
+        if kind == 0:
+            small = dims[-1:]                                   # trailing vector
+        elif kind == 1:
+            small[-1] = 1                                       # one value per row
+        elif kind == 2:
+            j = int(rng.integers(0, rank - 1))
+            small = [dims[j]] + [1] * (rank - 1 - j)            # one value per channel
+        else:
+            for ax in range(1, rank - 1):
+                small[ax] = 1                                   # one vector per outer index
+        x = rng.standard_normal(dims).astype(np.float32)
+        y = (rng.standard_normal(small) + 3.0).astype(np.float32)
+        if rng.random() < 0.3:
+            x, y = y, x
+        op, f = ops[int(rng.integers(0, 4))]
+        case(f"pattern {i}: op {op} {list(x.shape)} {list(y.shape)}")
+        assert_bits_equal(ctx.binary(op, x, y), f(x, y), f"case {i}: {list(x.shape)} op {list(y.shape)}")
+
+
 def test_row_kernels_on_random_lengths(case, ctx):
     rng = np.random.default_rng(7)
     lengths = list(rng.integers(1, 1100, size=40)) + [255, 256, 257, 511, 512, 513, 767, 768, 1023, 1024, 1025, 1400, 2049]
