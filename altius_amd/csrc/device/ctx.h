@@ -159,6 +159,9 @@ int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, 
                       float alpha, float beta, int a_op = 0);
 // The context's grow-only GEMM workspace, at least `bytes` large (stream-ordered use only).
 int gemm_workspace(DeviceCtx &ctx, size_t bytes, void **p);
+// Row sums (optionally times `scale`) or maxima of a [rows, len] matrix through LDS-staged groups of rows (rows.hip): for
+// rows that are short or not whole float4s.  Returns -1 without launching when the shape is not one it is meant for.
+int launch_reduce_rows_lds(DeviceCtx &ctx, bool is_max, float *out, const float *in, size_t rows, size_t len, float scale, bool scaled);
 // Whether launch_gemm would send this single-batch product through launch_gemm_split.
 bool gemm_takes_split(const DeviceCtx &ctx, size_t m, size_t n, size_t k);
 // Large and tile-filling enough for the split kernel to win (the AHIP_GEMM_AUTO rule).

@@ -366,6 +366,11 @@ int reduce_impl(DeviceCtx &ctx, float *out, const float *in, size_t outer, size_
                 float scale) {
     hipStream_t s = ctx.stream;
     if (inner == 1) {
+        // Short rows and rows that are not whole float4s: groups of rows staged through LDS, a few lanes per row.
+        if (red <= 1024 && (red % 4 != 0 || red < 256)) {
+            const int rc = launch_reduce_rows_lds(ctx, std::is_same<OP, MaxOp>::value, out, in, outer, red, scale, SCALE);
+            if (rc >= 0) return rc;
+        }
         if (red <= 4096 || outer >= 65536) {
             if ((outer + ROW_WAVES - 1) / ROW_WAVES > MAX_GRID_X)
                 return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: too many rows for one launch");

@@ -294,6 +294,57 @@ __global__ __launch_bounds__(LDS_BLOCK) void softmax_lds(float *__restrict__ out
     for (int i = (n4 << 2) + tid; i < n; i += LDS_BLOCK) dst[i] = lds[i];
 }
 
+// Sum or maximum of every row, for rows that are short or not whole float4s (7 x 7 feature maps, 197 tokens): a
+// wavefront per row would leave most lanes idle and read 4 bytes per lane.  Same staging as softmax_lds: a
+// line-aligned group of rows goes to LDS with 16-byte loads, then SUB lanes fold each row and lane 0 of the group
+// writes out[row] (times `scale` for a mean).
+template <class OP, int SUB, bool SCALE, bool NT>
+__global__ __launch_bounds__(LDS_BLOCK) void reduce_rows_lds(float *__restrict__ out, const float *__restrict__ in, size_t rows,
+                                                             int len, int group_rows, float scale) {
+    extern __shared__ __align__(16) float lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1);
+    const int wave = tid >> 6;
+    const size_t row0 = (size_t)blockIdx.x * group_rows;
+    const int nrows = rows - row0 < (size_t)group_rows ? (int)(rows - row0) : group_rows;
+    const int n = nrows * len;
+    const int n4 = n >> 2;
+    const float *src = in + row0 * (size_t)len;
+    float4 stage[STAGE_LDS];
+#pragma unroll
+    for (int u = 0; u < STAGE_LDS; u++) {
+        const float *p = src + 4 * (tid + LDS_BLOCK * u);
+        if (LDS_BLOCK * (u + 1) <= n4) {
+            stage[u] = load4<NT>(p);
+        } else if (LDS_BLOCK * u < n4) {
+            if (tid + LDS_BLOCK * u < n4) stage[u] = load4<NT>(p);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < STAGE_LDS; u++) {
+        float *q = lds + 4 * (tid + LDS_BLOCK * u);
+        if (LDS_BLOCK * (u + 1) <= n4) {
+            *reinterpret_cast<float4 *>(q) = stage[u];
+        } else if (LDS_BLOCK * u < n4) {
+            if (tid + LDS_BLOCK * u < n4) *reinterpret_cast<float4 *>(q) = stage[u];
+        }
+    }
+    for (int i = (n4 << 2) + tid; i < n; i += LDS_BLOCK) lds[i] = src[i];  // ragged end of the last group
+    __syncthreads();
+
+    constexpr int RPP = WAVE / SUB;  // rows per wave pass
+    const int s = lane & (SUB - 1);
+    const int rr = lane / SUB;
+    for (int r0 = wave * RPP; r0 < nrows; r0 += LDS_WAVES * RPP) {
+        const int r = r0 + rr < nrows ? r0 + rr : nrows - 1;  // lane groups past the end redo the last row and write nothing
+        const float *row = lds + r * len;
+        float acc = OP::identity();
+        for (int k = s; k < len; k += SUB) acc = OP::apply(acc, row[k]);
+        acc = subwave_allreduce<OP, SUB>(acc);
+        if (s == 0 && r0 + rr < nrows) out[row0 + r] = SCALE ? acc * scale : acc;
+    }
+}
+
 // One block per row, any length: max pass, sum pass, write pass.
 __global__ __launch_bounds__(BLOCK) void softmax_block_stream(float *__restrict__ out,
                                                               const float *__restrict__ in, size_t len) {
@@ -599,6 +650,36 @@ int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *g
                            gamma, beta, len, eps);
     }
     return ctx.check(hipGetLastError(), "layernorm launch");
+}
+
+// Row sums / maxima through reduce_rows_lds; -1 (nothing launched) when the shape is not one it is meant for.
+int launch_reduce_rows_lds(DeviceCtx &ctx, bool is_max, float *out, const float *in, size_t rows, size_t len, float scale, bool scaled) {
+    if (len == 0 || len > 1024 || rows < 64 || !aligned16(in)) return -1;
+    const size_t g = softmax_lds_group_rows(len);
+    if ((g * len) % 4 != 0) return -1;  // groups must start 16-byte aligned
+    const size_t groups = (rows + g - 1) / g;
+    if (groups > 0x7FFFFFFFu) return -1;
+    const bool nt = ctx.streaming(rows * len * sizeof(float));
+    const dim3 grid((unsigned)groups);
+    const size_t shmem = g * len * sizeof(float);
+    const int L = (int)len, G = (int)g;
+#define ALTIUS_RED(OP, SUB, SC)                                                                                                   \
+    do {                                                                                                                          \
+        if (nt) hipLaunchKernelGGL((reduce_rows_lds<OP, SUB, SC, true>), grid, dim3(LDS_BLOCK), shmem, ctx.stream, out, in, rows, L, G, scale);  \
+        else hipLaunchKernelGGL((reduce_rows_lds<OP, SUB, SC, false>), grid, dim3(LDS_BLOCK), shmem, ctx.stream, out, in, rows, L, G, scale);    \
+    } while (0)
+#define ALTIUS_RED_SUB(SUB)                                   \
+    do {                                                      \
+        if (is_max) ALTIUS_RED(MaxOp, SUB, false);            \
+        else if (scaled) ALTIUS_RED(SumOp, SUB, true);        \
+        else ALTIUS_RED(SumOp, SUB, false);                   \
+    } while (0)
+    if (len <= 256) ALTIUS_RED_SUB(16);
+    else if (len <= 512) ALTIUS_RED_SUB(32);
+    else ALTIUS_RED_SUB(64);
+#undef ALTIUS_RED_SUB
+#undef ALTIUS_RED
+    return ctx.check(hipGetLastError(), "reduce rows (LDS groups) launch");
 }
 
 }  // namespace altius

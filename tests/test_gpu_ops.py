@@ -286,6 +286,12 @@ REDUCE_CASES = [
     ([2, 100, 300], [1], False),       # several column tiles
     ([2, 4000, 64], [1], False),       # split columns through scratch
     ([7, 1, 9], [1], True),
+    ([70, 197], [1], False),           # short / unaligned rows staged through LDS in groups: a ragged last group
+    ([3000, 1], [1], True),            # rows of one element
+    ([100, 1001], [1], False),         # 64 lanes per row
+    ([500, 333], [1], True),           # 32 lanes per row
+    ([2, 999, 7, 7], [2, 3], True),    # 16 lanes per row, several groups
+    ([4096, 64], [1], False),          # short aligned rows
     ([6, 5], [0], False),
     ([1, 18, 197], [1], False),        # 16-byte flat column kernel with two left-over rows
     ([1, 17, 5], [1], False),          # the same, one left-over row, one wave of columns
