@@ -381,10 +381,14 @@ __global__ __launch_bounds__(BLOCK) void layernorm_wave(float *__restrict__ out,
 
     RowRegs<VEC, NCH> r;
     r.template load<NT>(x, len, lane, 0.0f);
-    // Scale and bias are requested right behind the row, so that they arrive during the two reductions.
-    RowRegs<VEC, NCH> g, b;
-    g.load(gamma, len, lane, 0.0f);
-    b.load(beta, len, lane, 0.0f);
+    // Scale and bias are requested right behind the row, so that they arrive during the two reductions; for rows
+    // of more than four chunks per lane they would not fit the registers and are fetched chunk by chunk at the end.
+    constexpr bool EARLY = NCH <= 4;
+    RowRegs<VEC, EARLY ? NCH : 1> g, b;
+    if (EARLY) {
+        g.load(gamma, len, lane, 0.0f);
+        b.load(beta, len, lane, 0.0f);
+    }
 
     const float inv_n = 1.0f / (float)len;
     float sum = 0.0f;
@@ -403,8 +407,19 @@ __global__ __launch_bounds__(BLOCK) void layernorm_wave(float *__restrict__ out,
     ss = wave_reduce<SumOp>(ss);
     const float inv_std = 1.0f / sqrtf(__builtin_fmaf(ss, inv_n, eps));
 
+    if (EARLY) {
 #pragma unroll
-    for (int s = 0; s < NCH * VEC; s++) r.v[s] = __builtin_fmaf(r.v[s] * inv_std, g.v[s], b.v[s]);
+        for (int s = 0; s < NCH * VEC; s++) r.v[s] = __builtin_fmaf(r.v[s] * inv_std, g.v[EARLY ? s : 0], b.v[EARLY ? s : 0]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            const int e = (lane + WAVE * k) * VEC;
+            if (e < len) {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) r.v[k * VEC + j] = __builtin_fmaf(r.v[k * VEC + j] * inv_std, gamma[e + j], beta[e + j]);
+            }
+        }
+    }
     r.template store<NT>(o, len, lane);
 }
 
@@ -457,6 +472,18 @@ bool dispatch_wave(bool vec4, size_t len, Args... args) {
     if (chunks <= 8) { Launcher<1, 8>::go(args...); return true; }
     if (chunks <= 12) { Launcher<1, 12>::go(args...); return true; }
     if (chunks <= 16) { Launcher<1, 16>::go(args...); return true; }
+    return false;
+}
+
+// Rows of 1025 to 4096 elements that are whole float4s: still a wavefront per row with the row in registers
+// (6, 8, 12 or 16 float4 per lane), read once.
+template <template <int, int> class Launcher, class... Args>
+bool dispatch_wave_long(size_t len, Args... args) {
+    const size_t chunks = (len / 4 + WAVE - 1) / WAVE;
+    if (chunks <= 6) { Launcher<4, 6>::go(args...); return true; }
+    if (chunks <= 8) { Launcher<4, 8>::go(args...); return true; }
+    if (chunks <= 12) { Launcher<4, 12>::go(args...); return true; }
+    if (chunks <= 16) { Launcher<4, 16>::go(args...); return true; }
     return false;
 }
 
@@ -574,6 +601,7 @@ bool softmax_lds_launch(hipStream_t s, float *out, const float *in, size_t rows,
 }
 
 constexpr size_t MAX_WAVE_ROW = 1024;
+constexpr size_t MAX_LONG_ROW = 4096;  // rows kept in a wavefront's registers when they are whole float4s
 constexpr size_t MAX_GRID = 0x7FFFFFFFu;
 
 }  // namespace
@@ -597,6 +625,10 @@ int launch_softmax(DeviceCtx &ctx, float *out, const float *in, size_t rows, siz
                                                     ctx.streaming(rows * len * sizeof(float)))) {
             return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: no wave layout for this row length");
         }
+    } else if (len <= MAX_LONG_ROW && len % 4 == 0 && aligned16(out) && aligned16(in) &&
+               (rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK <= MAX_GRID) {
+        dispatch_wave_long<SoftmaxLauncher>(len, ctx.stream, out, in, rows, (int)len, (const SoftmaxPrologue *)nullptr,
+                                            ctx.streaming(rows * len * sizeof(float)));
     } else {
         if (rows > MAX_GRID) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: too many rows for one launch");
         hipLaunchKernelGGL(softmax_block_stream, dim3((unsigned)rows), dim3(BLOCK), 0, ctx.stream, out, in,
@@ -644,6 +676,10 @@ int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *g
         if (!dispatch_wave<LayerNormLauncher>(vec4, len, ctx.stream, out, in, gamma, beta, rows, (int)len,
                                               eps, ctx.streaming(rows * len * sizeof(float))))
             return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: no wave layout for this row length");
+    } else if (len <= MAX_LONG_ROW && len % 4 == 0 && aligned16(out) && aligned16(in) &&
+               (rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK <= MAX_GRID) {
+        dispatch_wave_long<LayerNormLauncher>(len, ctx.stream, out, in, gamma, beta, rows, (int)len, eps,
+                                              ctx.streaming(rows * len * sizeof(float)));
     } else {
         if (rows > MAX_GRID) return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: too many rows for one launch");
         hipLaunchKernelGGL(layernorm_block_stream, dim3((unsigned)rows), dim3(BLOCK), 0, ctx.stream, out, in,
