@@ -255,7 +255,8 @@ def test_softmax_masked_rows(ctx, oracle, case):
 
 
 LN_SHAPES = [[1, 20, 10], [2, 197, 768], [3, 5, 197], [4, 1], [5, 64], [3, 1024], [2, 1028], [2, 4100], [3, 3072],
-             [5, 1280], [9, 1536], [3, 2048], [2, 2560], [2, 4092], [7, 4096], [2, 1026]]
+             [5, 1280], [9, 1536], [3, 2048], [2, 2560], [2, 4092], [7, 4096], [2, 1026],
+             [100, 49], [70, 197], [300, 64], [1000, 10], [64, 255], [65, 1], [200, 130], [4, 700, 192]]  # short rows in groups through LDS
 
 
 @pytest.mark.parametrize("shape", LN_SHAPES)
