@@ -533,6 +533,78 @@ __global__ __launch_bounds__(BLOCK) void layernorm_block_stream(float *__restric
         o[i] = __builtin_fmaf((x[i] - mean) * inv_std, gamma[i], beta[i]);
 }
 
+// Rows of 4097 to 16384 elements that are whole float4s (hidden sizes 5120, 8192; 16 K): a block per row with the
+// row in registers (8 or 16 float4 per thread), read once; the two reductions go through LDS.
+template <int NCH, bool NT>
+__global__ __launch_bounds__(BLOCK) void softmax_block_regs(float *__restrict__ out, const float *__restrict__ in, size_t len) {
+    __shared__ float lds[WAVES_PER_BLOCK];
+    const float *x = in + (size_t)blockIdx.x * len;
+    float *o = out + (size_t)blockIdx.x * len;
+    const float nan = __builtin_nanf("");
+    float4 r[NCH];
+#pragma unroll
+    for (int k = 0; k < NCH; k++) {
+        const size_t e = ((size_t)threadIdx.x + (size_t)BLOCK * k) * 4;
+        r[k] = e < len ? load4<NT>(x + e) : make_float4(nan, nan, nan, nan);
+    }
+    float mx = nan;  // NaN elements (and the slots past the row) are ignored by the maximum
+#pragma unroll
+    for (int k = 0; k < NCH; k++) mx = nanmax(nanmax(r[k].x, r[k].y), nanmax(nanmax(r[k].z, r[k].w), mx));
+    mx = block_reduce<MaxOp, WAVES_PER_BLOCK>(mx, lds);
+    float sum = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NCH; k++) {
+        const bool valid = ((size_t)threadIdx.x + (size_t)BLOCK * k) * 4 < len;
+        r[k].x = softmax_exp(r[k].x, mx), r[k].y = softmax_exp(r[k].y, mx), r[k].z = softmax_exp(r[k].z, mx), r[k].w = softmax_exp(r[k].w, mx);
+        if (valid) sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
+    }
+    sum = block_reduce<SumOp, WAVES_PER_BLOCK>(sum, lds);
+    const float recip = 1.0f / sum;
+#pragma unroll
+    for (int k = 0; k < NCH; k++) {
+        const size_t e = ((size_t)threadIdx.x + (size_t)BLOCK * k) * 4;
+        if (e < len) store4<NT>(o + e, make_float4(r[k].x * recip, r[k].y * recip, r[k].z * recip, r[k].w * recip));
+    }
+}
+
+template <int NCH, bool NT>
+__global__ __launch_bounds__(BLOCK) void layernorm_block_regs(float *__restrict__ out, const float *__restrict__ in,
+                                                              const float *__restrict__ gamma, const float *__restrict__ beta, size_t len,
+                                                              float eps) {
+    __shared__ float lds[WAVES_PER_BLOCK];
+    const float *x = in + (size_t)blockIdx.x * len;
+    float *o = out + (size_t)blockIdx.x * len;
+    const float inv_n = 1.0f / (float)len;
+    float4 r[NCH];
+    float sum = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NCH; k++) {
+        const size_t e = ((size_t)threadIdx.x + (size_t)BLOCK * k) * 4;
+        r[k] = e < len ? load4<NT>(x + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int k = 0; k < NCH; k++) sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
+    const float mean = block_reduce<SumOp, WAVES_PER_BLOCK>(sum, lds) * inv_n;
+    float ss = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NCH; k++) {
+        const bool valid = ((size_t)threadIdx.x + (size_t)BLOCK * k) * 4 < len;
+        r[k].x -= mean, r[k].y -= mean, r[k].z -= mean, r[k].w -= mean;
+        if (valid) ss += (r[k].x * r[k].x + r[k].y * r[k].y) + (r[k].z * r[k].z + r[k].w * r[k].w);
+    }
+    ss = block_reduce<SumOp, WAVES_PER_BLOCK>(ss, lds);
+    const float inv_std = 1.0f / sqrtf(__builtin_fmaf(ss, inv_n, eps));
+#pragma unroll
+    for (int k = 0; k < NCH; k++) {
+        const size_t e = ((size_t)threadIdx.x + (size_t)BLOCK * k) * 4;
+        if (e < len) {
+            const float4 g = *reinterpret_cast<const float4 *>(gamma + e), b = *reinterpret_cast<const float4 *>(beta + e);
+            store4<NT>(o + e, make_float4(__builtin_fmaf(r[k].x * inv_std, g.x, b.x), __builtin_fmaf(r[k].y * inv_std, g.y, b.y),
+                                          __builtin_fmaf(r[k].z * inv_std, g.z, b.z), __builtin_fmaf(r[k].w * inv_std, g.w, b.w)));
+        }
+    }
+}
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // Picks the register layout for a wave-per-row kernel: VEC=4 when rows stay
@@ -686,6 +758,7 @@ bool softmax_lds_launch(hipStream_t s, float *out, const float *in, size_t rows,
 
 constexpr size_t MAX_WAVE_ROW = 1024;
 constexpr size_t MAX_LONG_ROW = 4096;  // rows kept in a wavefront's registers when they are whole float4s
+constexpr size_t MAX_BLOCK_REG_ROW = 16384;  // ... and in a block's registers
 constexpr size_t MAX_GRID = 0x7FFFFFFFu;
 
 }  // namespace
@@ -713,6 +786,16 @@ int launch_softmax(DeviceCtx &ctx, float *out, const float *in, size_t rows, siz
                (rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK <= MAX_GRID) {
         dispatch_wave_long<SoftmaxLauncher>(len, ctx.stream, out, in, rows, (int)len, (const SoftmaxPrologue *)nullptr,
                                             ctx.streaming(rows * len * sizeof(float)));
+    } else if (len <= MAX_BLOCK_REG_ROW && len % 4 == 0 && aligned16(out) && aligned16(in) && rows <= MAX_GRID) {
+        const bool nt = ctx.streaming(rows * len * sizeof(float));
+        const dim3 grid((unsigned)rows);
+        if (len <= 8192) {
+            if (nt) hipLaunchKernelGGL((softmax_block_regs<8, true>), grid, dim3(BLOCK), 0, ctx.stream, out, in, len);
+            else hipLaunchKernelGGL((softmax_block_regs<8, false>), grid, dim3(BLOCK), 0, ctx.stream, out, in, len);
+        } else {
+            if (nt) hipLaunchKernelGGL((softmax_block_regs<16, true>), grid, dim3(BLOCK), 0, ctx.stream, out, in, len);
+            else hipLaunchKernelGGL((softmax_block_regs<16, false>), grid, dim3(BLOCK), 0, ctx.stream, out, in, len);
+        }
     } else {
         if (rows > MAX_GRID) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: too many rows for one launch");
         hipLaunchKernelGGL(softmax_block_stream, dim3((unsigned)rows), dim3(BLOCK), 0, ctx.stream, out, in,
@@ -786,6 +869,17 @@ int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *g
                (rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK <= MAX_GRID) {
         dispatch_wave_long<LayerNormLauncher>(len, ctx.stream, out, in, gamma, beta, rows, (int)len, eps,
                                               ctx.streaming(rows * len * sizeof(float)));
+    } else if (len <= MAX_BLOCK_REG_ROW && len % 4 == 0 && aligned16(out) && aligned16(in) && aligned16(gamma) && aligned16(beta) &&
+               rows <= MAX_GRID) {
+        const bool nt = ctx.streaming(rows * len * sizeof(float));
+        const dim3 grid((unsigned)rows);
+        if (len <= 8192) {
+            if (nt) hipLaunchKernelGGL((layernorm_block_regs<8, true>), grid, dim3(BLOCK), 0, ctx.stream, out, in, gamma, beta, len, eps);
+            else hipLaunchKernelGGL((layernorm_block_regs<8, false>), grid, dim3(BLOCK), 0, ctx.stream, out, in, gamma, beta, len, eps);
+        } else {
+            if (nt) hipLaunchKernelGGL((layernorm_block_regs<16, true>), grid, dim3(BLOCK), 0, ctx.stream, out, in, gamma, beta, len, eps);
+            else hipLaunchKernelGGL((layernorm_block_regs<16, false>), grid, dim3(BLOCK), 0, ctx.stream, out, in, gamma, beta, len, eps);
+        }
     } else {
         if (rows > MAX_GRID) return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: too many rows for one launch");
         hipLaunchKernelGGL(layernorm_block_stream, dim3((unsigned)rows), dim3(BLOCK), 0, ctx.stream, out, in,
