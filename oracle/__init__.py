@@ -199,6 +199,14 @@ def fast_sum_squares(x):
     return np.float32(lib().orc_fast_sum_squares(_fptr(x), ctypes.c_size_t(x.size)))
 
 
+def faster_pow2(p):
+    """fastapprox::faster::pow2 element by element (the helper inside Erf)."""
+    p = _f32(p)
+    out = np.empty_like(p)
+    lib().orc_faster_pow2(_fptr(p), _fptr(out), ctypes.c_size_t(p.size))
+    return out
+
+
 # ---- data movement and the remaining element-wise kernels ---------------------------------------
 
 _TYPE_OF = {np.dtype(np.bool_): 0, np.dtype(np.float32): 1, np.dtype(np.int32): 2, np.dtype(np.int64): 3}

@@ -320,7 +320,7 @@ void fast_gelu(float *out, const float *in, size_t len) {
 }
 
 // fastapprox 0.3.1, module `faster` (not vendored in the reference; restated
-// from the crate's published algorithm -- PARITY UNPINNED, see oracle.h):
+// from the crate's published algorithm; only the fitted constant K stays unconfirmed, see oracle.h):
 //   pow2(p) = from_bits(((1 << 23) as f32 * (max(p, -126) + 126.94269504)) as u32)
 //   erfc(x) = 2 / (1 + pow2(3.3509633149424609 * x));  erf(x) = 1 - erfc(x)
 // Rust's `as u32` saturates and maps NaN to 0.
@@ -1172,5 +1172,8 @@ int orc_resize(const float *x, float *out, size_t planes, size_t ih, size_t iw, 
 
 float orc_fast_sum(const float *x, size_t n) { return fast_sum(x, n); }
 float orc_fast_sum_squares(const float *x, size_t n) { return fast_sum_squares(x, n); }
+void orc_faster_pow2(const float *p, float *out, size_t n) {
+    for (size_t i = 0; i < n; i++) out[i] = faster_pow2(p[i]);
+}
 
 }  // extern "C"

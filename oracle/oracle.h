@@ -27,13 +27,18 @@
  *     and by known-answer vectors whose result depends on the 8-lane strided
  *     accumulation order (crates/session_interpreter/src/session.rs:1028-1055).
  *   - ReduceMax: order-independent, pinned by brute force.
- *   - orc_unary(ORC_ERF): PARITY UNPINNED.  The reference calls
- *     fastapprox::faster::erf from the crate fastapprox 0.3.1 (Cargo.lock:978),
- *     whose source is not vendored.  The restatement follows the published
- *     algorithm of that crate (a port of Paul Mineiro's fastapprox "fasterpow2"
- *     / "fastererfc"); only the loose bounds the reference's own test states
- *     (|erf - exact| <= 1e-1, crates/altius_py/tests/test_ops_elemwise.py:129-152)
- *     are checked.
+ *   - orc_unary(ORC_ERF): the reference calls fastapprox::faster::erf from the
+ *     crate fastapprox 0.3.1 (Cargo.lock:978), whose source is not vendored.
+ *     The restatement follows the published algorithm of that crate (a port of
+ *     Paul Mineiro's fastapprox "fasterpow2" / "fastererfc").  Pinned without
+ *     the crate: pow2 equals, bit for bit, the exact piecewise-linear
+ *     interpolant of 2^t evaluated in rational arithmetic; the knots give exact
+ *     powers of two; the clip at -126 and Rust's saturating `as u32` (NaN -> 0)
+ *     have known answers; the offset 126.94269504 is 127 - (3/2 - 1/ln 2) to
+ *     every printed digit.  PARITY UNPINNED for one number only: the fitted
+ *     constant K = 3.3509633149424609 has no closed form; the mathematics only
+ *     brackets it to a few per cent (the reference's own test allows 1e-1,
+ *     crates/altius_py/tests/test_ops_elemwise.py:129-152).
  *   - Shapes the reference interpreter has no kernel for (axis ReduceMax,
  *     multi-axis / non-rank-3 ReduceMean, general-broadcast Pow) are computed
  *     per the ONNX definition with the same accumulation primitives; the
@@ -195,6 +200,9 @@ int orc_resize(const float *x, float *out, size_t planes, size_t ih, size_t iw, 
 
 float orc_fast_sum(const float *x, size_t n);
 float orc_fast_sum_squares(const float *x, size_t n);
+/* fastapprox::faster::pow2, the helper inside Erf (session.rs:929), exposed so that tests can
+ * check it on its own against the exact piecewise-linear interpolant of 2^p. */
+void orc_faster_pow2(const float *p, float *out, size_t n);
 
 #ifdef __cplusplus
 }

@@ -207,6 +207,22 @@ def test_unary_special_values(ctx, oracle, case, name):
     assert_bits_equal(actual, expected, f"special {name}", zero_sign_free=(name == "Relu"))
 
 
+def test_erf_against_the_exact_interpolant(ctx, case):
+    """Op::Erf without the oracle: fastapprox::faster::erf (session.rs:929) restated as the exact
+    piecewise-linear interpolant of 2^t in rational arithmetic (tests/erf_exact.py), over every
+    branch of the bit trick: the clip, subnormals, the exponent-255 segment, the wrap into the sign
+    bit, the saturated cast, NaN and infinities."""
+    import erf_exact
+
+    case("erf vs exact interpolant")
+    x = erf_exact.erf_vectors()
+    want = erf_exact.erf_expected(x)
+    got = ctx.unary(D.ERF, x)
+    assert_bits_equal(got, want, "erf vs interpolant")
+    assert ctx.unary(D.ERF, np.float32([np.nan]))[0] == -1.0  # Rust's `as u32` turns NaN into 0
+    assert ctx.unary(D.ERF, np.float32([50.0]))[0] == -1.0    # the exponent field wraps into the sign bit
+
+
 def test_hardsigmoid_default_attributes(ctx, oracle, case):
     """ONNX defaults alpha=0.2, beta=0.5 (crates/core/src/onnx/load.rs:321-324)."""
     case("hardsigmoid defaults")

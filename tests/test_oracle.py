@@ -10,6 +10,7 @@ import numpy as np
 import pytest
 from scipy.special import erf as exact_erf
 
+import erf_exact
 from altius_amd import synth
 from conftest import assert_bits_equal
 
@@ -216,14 +217,106 @@ def test_tanh_rational(oracle):
 
 
 def test_erf_loose_bounds(oracle):
-    """PARITY UNPINNED at the bit level (fastapprox is not vendored); only the reference's own
-    bound is checked: |erf - exact| <= 1e-1 (test_ops_elemwise.py:129-152)."""
+    """The reference's own bound at this boundary: |erf - exact| <= 1e-1
+    (crates/altius_py/tests/test_ops_elemwise.py:129-152)."""
     x = np.linspace(-4, 4, 4001, dtype=np.float32)
     got = oracle.unary(1, x)
     assert np.max(np.abs(got - exact_erf(x.astype(np.float64)))) < 1e-1
     assert abs(oracle.unary(1, np.zeros(1, np.float32))[0]) < 0.03
     assert np.all(np.diff(got) >= -1e-6)
     assert got[0] < -0.99 and got[-1] > 0.99
+
+
+# Erf = fastapprox::faster::erf (session.rs:929; crate not vendored).  The checks below do not go
+# through the oracle's expression: tests/erf_exact.py states what the crate's bit trick means (the
+# piecewise-linear interpolant of 2^t) in rational arithmetic, and the offset constant has a closed form.
+
+def test_erf_pow2_offset_has_a_closed_form():
+    """126.94269504 = 127 - (3/2 - 1/ln 2): the shift that gives the interpolant zero mean log2 error.
+    Every digit the crate prints follows, and so does the fp32 value the arithmetic uses."""
+    closed = erf_exact.offset_closed_form()
+    assert abs(erf_exact.OFFSET - closed) < 5e-9
+    assert np.float32(erf_exact.OFFSET) == np.float32(closed)
+    f = (np.arange(1 << 16) + 0.5) / (1 << 16)
+    assert abs(np.mean(np.log2(1 + f) - f) - (127 - closed)) < 1e-9  # the mean it cancels
+    # and the interpolant built with it is unbiased in log2, biased by a full 1e-3 if the 4th decimal moves
+    t = np.linspace(-20, 20, 400001)
+    def mean_log_err(offset):
+        u = t + offset
+        return np.mean(np.log2(2.0 ** (np.floor(u) - 127) * (1 + u - np.floor(u))) - t)
+    assert abs(mean_log_err(erf_exact.OFFSET)) < 1e-6
+    assert abs(mean_log_err(erf_exact.OFFSET + 1e-3)) > 9e-4
+
+
+def test_erf_pow2_is_the_exact_interpolant(oracle):
+    """pow2 over a dense grid, bit for bit the interpolant of 2^(t-127) in Fraction arithmetic."""
+    rng = np.random.default_rng(3)
+    p = np.concatenate([np.linspace(-126, 127.9, 8001, dtype=np.float32),
+                        (rng.uniform(-126, 128, 6000)).astype(np.float32),
+                        (rng.standard_normal(2000) * 3).astype(np.float32)])
+    want = erf_exact.pow2_interpolant(p)
+    got = oracle.faster_pow2(p)
+    assert_bits_equal(got, want, "pow2 vs interpolant")
+    # it IS an interpolant of 2^t: never below, at most (1+f)/2^f <= 1.0615 above, with t = p + OFFSET - 127
+    t = p.astype(np.float64) + (erf_exact.OFFSET - 127)
+    ratio = got.astype(np.float64) / 2.0 ** t
+    ok = np.isfinite(ratio) & (p > -125)
+    assert ratio[ok].min() > 1 - 1e-6 and ratio[ok].max() < 1.0615
+    # and relative to 2^p itself (what the crate approximates) within 3.9 %
+    rel = got.astype(np.float64)[ok] / 2.0 ** p.astype(np.float64)[ok] - 1
+    assert -0.0390 < rel.min() and rel.max() < 0.0202
+
+
+def test_erf_pow2_at_the_knots_is_a_power_of_two(oracle):
+    """Where p + OFFSET is an integer n in fp32, the significand is clear: pow2 = 2^(n-127) exactly."""
+    n = np.arange(1, 255, dtype=np.float32)
+    p = n - np.float32(erf_exact.OFFSET)
+    hit = (p + np.float32(erf_exact.OFFSET)) == n
+    assert hit.sum() > 200
+    got = oracle.faster_pow2(p[hit])
+    want = np.ldexp(np.float32(1), (n[hit] - 127).astype(np.int32)).astype(np.float32)
+    assert_bits_equal(got, want, "pow2 at integer knots")
+    # just below a knot the exponent is one lower and the significand almost full
+    g = oracle.faster_pow2(p[hit] - np.float32(0.01))
+    assert np.all(g < want) and np.all(g > want * np.float32(0.985))
+
+
+def test_erf_pow2_clip_and_saturating_cast(oracle):
+    """The clip at -126 and Rust's `as u32` (negative / zero / NaN -> 0, >= 2^32 -> all ones)."""
+    at_clip = oracle.faster_pow2(np.float32([-126.0]))[0]
+    # t = 0.94269504: exponent field 0, so a subnormal with the fraction as its significand
+    assert at_clip.view(np.uint32) == np.uint32(int((np.float32(-126.0) + np.float32(erf_exact.OFFSET)) * np.float32(2 ** 23)))
+    assert 0 < at_clip < np.finfo(np.float32).tiny
+    low = oracle.faster_pow2(np.float32([-126.5, -127.0, -200.0, -1e30, -np.inf]))
+    assert_bits_equal(low, np.full(5, at_clip, np.float32), "below the clip")  # without the clip these would be 0
+    assert oracle.faster_pow2(np.float32([np.nan]))[0].view(np.uint32) == 0  # NaN -> 0u32 -> +0.0
+    for p in (385.1, 1e6, 3e38, np.inf):
+        assert oracle.faster_pow2(np.float32([p]))[0].view(np.uint32) == 0xFFFFFFFF, p  # saturated
+    assert oracle.faster_pow2(np.float32([385.0]))[0].view(np.uint32) < 0xFFFFFFFF
+    # exponent field 255 and the wrap into the sign bit are part of the crate's behaviour too
+    assert np.isinf(oracle.faster_pow2(np.float32([255 - erf_exact.OFFSET]))[0])
+    assert np.isnan(oracle.faster_pow2(np.float32([128.5]))[0])
+    neg = oracle.faster_pow2(np.float32([130.0, 200.0]))
+    assert np.all(neg < 0) and np.all(np.isfinite(neg))
+    want = erf_exact.pow2_interpolant(np.float32([-126.0, -130.0, 128.5, 130.0, 200.0, 384.9, 385.1, np.nan]))
+    assert_bits_equal(oracle.faster_pow2(np.float32([-126.0, -130.0, 128.5, 130.0, 200.0, 384.9, 385.1, np.nan])), want, "edges")
+
+
+def test_erf_bits_from_the_interpolant(oracle):
+    """Op::Erf over every branch: 1 - 2 / (1 + interpolant(K x)) with fp32 roundings, bit for bit."""
+    x = erf_exact.erf_vectors()
+    want = erf_exact.erf_expected(x)
+    got = oracle.unary(1, x)
+    assert_bits_equal(got, want, "erf vs interpolant")
+    # consequences of the cast that a C-style conversion would not give
+    assert oracle.unary(1, np.float32([np.nan]))[0] == -1.0         # NaN -> pow2 = 0 -> 1 - 2/1
+    assert oracle.unary(1, np.float32([-np.inf, -50.0]))[1] == oracle.unary(1, np.float32([-38.0]))[0]
+    assert oracle.unary(1, np.float32([50.0]))[0] == -1.0           # sign-bit wrap: pow2 = -tiny
+    assert np.isnan(oracle.unary(1, np.float32([200.0]))[0])       # saturated cast: NaN pattern
+    # K itself has no closed form: the mathematics only brackets it.  With K the approximation stays within
+    # 0.0307 of erf on [-4, 4]; a K that is 3 % lower gives 0.040 and one 5 % higher 0.038.
+    xs = np.linspace(-4, 4, 2001, dtype=np.float32)
+    assert np.max(np.abs(oracle.unary(1, xs) - exact_erf(xs.astype(np.float64)))) < 0.032
 
 
 # ---- accumulation order ----------------------------------------------------------
