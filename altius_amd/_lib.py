@@ -115,6 +115,8 @@ def _declare(L):
     f("ahip_softmax_lastaxis_prologue", [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_float, c_void_p, c_size_t])
     f("ahip_layernorm_lastaxis", [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_float])
     f("ahip_reduce", [c_void_p, c_int, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t])
+    f("ahip_reduce_static", [c_void_p, c_int, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t])
+    f("ahip_reduce_static_capacity", [], c_size_t)
 
 
 class OpAttrs(ctypes.Structure):

@@ -325,6 +325,13 @@ int ahip_reduce(ahip_ctx *ctx, int kind, float *out, const float *in, size_t out
     return altius::launch_reduce(ctx->d, kind, out, in, outer, reduce, inner);
 }
 
+int ahip_reduce_static(ahip_ctx *ctx, int kind, float *out, const float *in, size_t outer, size_t reduce, size_t inner) {
+    REQUIRE_CTX(ctx, "ahip_reduce_static");
+    return altius::launch_reduce_static(ctx->d, kind, out, in, outer, reduce, inner);
+}
+
+size_t ahip_reduce_static_capacity(void) { return altius::reduce_static_capacity_floats(); }
+
 int ahip_copy_strided(ahip_ctx *ctx, void *out, const void *in, int elem_size, int rank, const int64_t *dims,
                       const int64_t *out_strides, const int64_t *in_strides) {
     REQUIRE_CTX(ctx, "ahip_copy_strided");

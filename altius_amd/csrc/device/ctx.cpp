@@ -38,6 +38,10 @@ int create_device_ctx(int device, hipStream_t stream, bool own_stream, DeviceCtx
     e = hipSetDevice(device);
     if (e != hipSuccess) return fail(e, "hipSetDevice");
     ctx->device = device;
+    if (reduce_static_setup(device) != AHIP_OK) {
+        if (error) *error = "hipGetSymbolAddress: the fixed partial-results array of the no-allocation reduce could not be located";
+        return AHIP_ERR_HIP;
+    }
     // AHIP_GEMM_SPLIT_K=0 keeps the bf16 GEMM from cutting an XCD's partly filled last round of tiles along k
     // (for measurements).
     if (const char *e = getenv("AHIP_GEMM_SPLIT_K")) ctx->gemm_split_k = atoi(e) != 0;

@@ -99,6 +99,13 @@ int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *g
                      const float *beta, size_t rows, size_t len, float eps);
 int launch_reduce(DeviceCtx &ctx, int kind, float *out, const float *in, size_t outer, size_t red,
                   size_t inner);
+// The same reduction for callers that may not allocate: partial results go to a fixed array in the code
+// object instead of the context's scratch buffer, and a shape whose partial results do not fit fails with
+// AHIP_ERR_UNSUPPORTED.  reduce_static_setup resolves the array's address for `device`, which must be the
+// calling thread's current device; create_device_ctx calls it.
+int launch_reduce_static(DeviceCtx &ctx, int kind, float *out, const float *in, size_t outer, size_t red, size_t inner);
+int reduce_static_setup(int device);
+size_t reduce_static_capacity_floats();
 
 
 // Data movement (movement.hip).  Strides are in elements; elem_size in bytes (1, 4 or 8).

@@ -21,6 +21,8 @@
 // sums are accumulated in a different order than the reference's 8 strided
 // accumulators.
 
+#include <mutex>
+
 #include "common.h"
 #include "ctx.h"
 
@@ -28,6 +30,17 @@ namespace altius {
 namespace {
 
 using namespace dev;
+
+// Partial results for callers that may not allocate (launch_reduce_static): a fixed array in the code
+// object, one copy per GPU for the life of the process.  Host code never uses this name as an address;
+// it asks the runtime for the array's device address once per device (reduce_static_setup) and passes
+// that pointer to the kernels like any other buffer.
+constexpr size_t STATIC_SCRATCH_FLOATS = (size_t)1 << 18;  // 1 MiB
+static __device__ __align__(256) float scratch[STATIC_SCRATCH_FLOATS];
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_static_mutex;
+float *g_static_scratch[MAX_DEVICES] = {};
 
 constexpr int ROW_BLOCK = 256;
 constexpr int ROW_WAVES = ROW_BLOCK / WAVE;
@@ -361,8 +374,22 @@ size_t gcd_size(size_t a, size_t b) {
     return a;
 }
 
+// Where the partial results of a two-stage reduction go.  fixed: the buffer cannot be replaced by a
+// one-stage launch or anything else when it is too small; the call fails instead, naming the sizes.
+struct Partials {
+    float *ptr;
+    size_t floats;
+    bool fixed;
+};
+
+int partials_too_small(DeviceCtx &ctx, size_t needed, const Partials &pt) {
+    return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: this shape needs " + std::to_string(needed) + " floats of partial results, the " +
+                                              (pt.fixed ? "fixed buffer of the no-allocation entry point" : "context's scratch buffer") + " holds " +
+                                              std::to_string(pt.floats));
+}
+
 template <class OP, bool SCALE>
-int reduce_impl(DeviceCtx &ctx, float *out, const float *in, size_t outer, size_t red, size_t inner,
+int reduce_impl(DeviceCtx &ctx, const Partials &pt, float *out, const float *in, size_t outer, size_t red, size_t inner,
                 float scale) {
     hipStream_t s = ctx.stream;
     if (inner == 1) {
@@ -393,10 +420,9 @@ int reduce_impl(DeviceCtx &ctx, float *out, const float *in, size_t outer, size_
             rows_block_launch<OP, SCALE>(s, out, in, outer, red, 1, chunk, scale);
             return ctx.check(hipGetLastError(), "reduce rows (block) launch");
         }
-        if (outer * splits > ctx.scratch_floats)
-            return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: scratch buffer too small");
-        rows_block_launch<OP, false>(s, ctx.scratch, in, outer, red, splits, chunk, 1.0f);
-        rows_wave_launch<OP, SCALE>(s, out, ctx.scratch, outer, splits, scale);
+        if (outer * splits > pt.floats) return partials_too_small(ctx, outer * splits, pt);
+        rows_block_launch<OP, false>(s, pt.ptr, in, outer, red, splits, chunk, 1.0f);
+        rows_wave_launch<OP, SCALE>(s, out, pt.ptr, outer, splits, scale);
         return ctx.check(hipGetLastError(), "reduce rows (two-stage) launch");
     }
 
@@ -424,11 +450,12 @@ int reduce_impl(DeviceCtx &ctx, float *out, const float *in, size_t outer, size_
                     cols_span_launch<OP, SCALE>(s, out, in, outer, red, inner, span_rows, 1, sps, scale, nt);
                     return ctx.check(hipGetLastError(), "reduce cols (span) launch");
                 }
-                if (outer * fsplits * inner <= ctx.scratch_floats) {
-                    cols_span_launch<OP, false>(s, ctx.scratch, in, outer, red, inner, span_rows, fsplits, sps, 1.0f, nt);
-                    cols_launch<OP, SCALE>(s, out, ctx.scratch, outer, fsplits, inner, 1, fsplits, scale);
+                if (outer * fsplits * inner <= pt.floats) {
+                    cols_span_launch<OP, false>(s, pt.ptr, in, outer, red, inner, span_rows, fsplits, sps, 1.0f, nt);
+                    cols_launch<OP, SCALE>(s, out, pt.ptr, outer, fsplits, inner, 1, fsplits, scale);
                     return ctx.check(hipGetLastError(), "reduce cols (span, two-stage) launch");
                 }
+                if (pt.fixed) return partials_too_small(ctx, outer * fsplits * inner, pt);
             }
         }
     }
@@ -452,20 +479,18 @@ int reduce_impl(DeviceCtx &ctx, float *out, const float *in, size_t outer, size_
         cols_launch<OP, SCALE>(s, out, in, outer, red, inner, 1, chunk, scale);
         return ctx.check(hipGetLastError(), "reduce cols launch");
     }
-    if (outer * splits * inner > ctx.scratch_floats) {
+    if (outer * splits * inner > pt.floats) {
+        if (pt.fixed) return partials_too_small(ctx, outer * splits * inner, pt);
         // Not enough scratch for the partials: do it in one stage.
         cols_launch<OP, SCALE>(s, out, in, outer, red, inner, 1, red, scale);
         return ctx.check(hipGetLastError(), "reduce cols launch");
     }
-    cols_launch<OP, false>(s, ctx.scratch, in, outer, red, inner, splits, chunk, 1.0f);
-    cols_launch<OP, SCALE>(s, out, ctx.scratch, outer, splits, inner, 1, splits, scale);
+    cols_launch<OP, false>(s, pt.ptr, in, outer, red, inner, splits, chunk, 1.0f);
+    cols_launch<OP, SCALE>(s, out, pt.ptr, outer, splits, inner, 1, splits, scale);
     return ctx.check(hipGetLastError(), "reduce cols (two-stage) launch");
 }
 
-}  // namespace
-
-int launch_reduce(DeviceCtx &ctx, int kind, float *out, const float *in, size_t outer, size_t red,
-                  size_t inner) {
+int reduce_with(DeviceCtx &ctx, const Partials &pt, int kind, float *out, const float *in, size_t outer, size_t red, size_t inner) {
     if (kind != AHIP_REDUCE_MEAN && kind != AHIP_REDUCE_MAX && kind != AHIP_REDUCE_SUM)
         return ctx.fail(AHIP_ERR_ARG, "reduce: unknown kind");
     if (outer == 0 || inner == 0) return AHIP_OK;
@@ -473,10 +498,43 @@ int launch_reduce(DeviceCtx &ctx, int kind, float *out, const float *in, size_t 
     if (!out || !in) return ctx.fail(AHIP_ERR_ARG, "reduce: null tensor pointer");
     if (kind == AHIP_REDUCE_MEAN) {
         const float r_axis_len = 1.0f / (float)red;
-        return reduce_impl<SumOp, true>(ctx, out, in, outer, red, inner, r_axis_len);
+        return reduce_impl<SumOp, true>(ctx, pt, out, in, outer, red, inner, r_axis_len);
     }
-    if (kind == AHIP_REDUCE_SUM) return reduce_impl<SumOp, false>(ctx, out, in, outer, red, inner, 1.0f);
-    return reduce_impl<MaxOp, false>(ctx, out, in, outer, red, inner, 1.0f);
+    if (kind == AHIP_REDUCE_SUM) return reduce_impl<SumOp, false>(ctx, pt, out, in, outer, red, inner, 1.0f);
+    return reduce_impl<MaxOp, false>(ctx, pt, out, in, outer, red, inner, 1.0f);
+}
+
+}  // namespace
+
+int launch_reduce(DeviceCtx &ctx, int kind, float *out, const float *in, size_t outer, size_t red,
+                  size_t inner) {
+    return reduce_with(ctx, Partials{ctx.scratch, ctx.scratch_floats, false}, kind, out, in, outer, red, inner);
+}
+
+int reduce_static_setup(int device) {
+    if (device < 0 || device >= MAX_DEVICES) return AHIP_ERR_ARG;
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (g_static_scratch[device]) return AHIP_OK;
+    float *ptr = nullptr;
+    // The calling thread's current device is `device`: each GPU holds its own copy of the array at its own address.
+    if (hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+        (void)hipGetLastError();
+        return AHIP_ERR_HIP;
+    }
+    g_static_scratch[device] = ptr;
+    return AHIP_OK;
+}
+
+size_t reduce_static_capacity_floats() { return STATIC_SCRATCH_FLOATS; }
+
+int launch_reduce_static(DeviceCtx &ctx, int kind, float *out, const float *in, size_t outer, size_t red, size_t inner) {
+    float *ptr = nullptr;
+    if (ctx.device >= 0 && ctx.device < MAX_DEVICES) {
+        std::lock_guard<std::mutex> lock(g_static_mutex);
+        ptr = g_static_scratch[ctx.device];
+    }
+    if (!ptr) return ctx.fail(AHIP_ERR_HIP, "reduce (no-allocation entry point): the fixed buffer's address was not resolved on this device");
+    return reduce_with(ctx, Partials{ptr, STATIC_SCRATCH_FLOATS, true}, kind, out, in, outer, red, inner);
 }
 
 }  // namespace altius

@@ -169,6 +169,10 @@ class Context:
     def reduce_raw(self, kind, out_ptr, in_ptr, outer, red, inner):
         check(self.L.ahip_reduce(self.handle, kind, out_ptr, in_ptr, outer, red, inner), self.handle)
 
+    def reduce_static_raw(self, kind, out_ptr, in_ptr, outer, red, inner):
+        """ahip_reduce_static: the reduction that allocates nothing (partial results in a fixed array)."""
+        check(self.L.ahip_reduce_static(self.handle, kind, out_ptr, in_ptr, outer, red, inner), self.handle)
+
     # --- convenience: numpy in, numpy out (upload, one kernel, download) ----
     def binary(self, op, a, b):
         a = np.asarray(a, dtype=np.float32, order="C")

@@ -215,6 +215,19 @@ enum ahip_reduce_kind {
 int ahip_reduce(ahip_ctx *ctx, int kind, float *out, const float *in, size_t outer, size_t reduce,
                 size_t inner);
 
+/* ahip_reduce for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same kernels, same launch
+ * shapes and therefore the same bits as ahip_reduce, but the partial results of a two-stage reduction go to
+ * a fixed 1 MiB array inside the library's code object (resolved once per device by ahip_init) instead of
+ * the context's scratch buffer, and the call itself performs no hipMalloc / hipFree.  A shape whose partial
+ * results exceed ahip_reduce_static_capacity() floats fails with AHIP_ERR_UNSUPPORTED and launches nothing
+ * (ahip_reduce would take its larger buffer or a one-stage kernel).  Every call on a GPU shares that GPU's
+ * array, whatever its context: calls that may overlap on one GPU (two streams, two threads) race; calls on
+ * one stream are ordered.  Nothing in the array has to start at zero. */
+int ahip_reduce_static(ahip_ctx *ctx, int kind, float *out, const float *in, size_t outer, size_t reduce,
+                       size_t inner);
+size_t ahip_reduce_static_capacity(void);
+
 /* Data movement.  Element sizes are in bytes (1 = Bool, 4 = F32 / I32, 8 = I64); strides in
  * elements.  All of these move each byte once and accept any rank up to 8.
  *
