@@ -325,6 +325,23 @@ int ahip_reduce(ahip_ctx *ctx, int kind, float *out, const float *in, size_t out
     return altius::launch_reduce(ctx->d, kind, out, in, outer, reduce, inner);
 }
 
+int ahip_xcd_round_robin_holds(int cu_count, const uint32_t *xcc_of_block, size_t n_blocks) {
+    return altius::xcd_round_robin_holds(cu_count, xcc_of_block, n_blocks) ? 1 : 0;
+}
+
+int ahip_gemm_in_kernel_k_cut(ahip_ctx *ctx, int *placement_shown, int *enabled) {
+    REQUIRE_CTX(ctx, "ahip_gemm_in_kernel_k_cut");
+    if (placement_shown) *placement_shown = ctx->d.xcd_round_robin ? 1 : 0;
+    if (enabled) *enabled = (ctx->d.gemm_in_kernel_k_cut && ctx->d.gemm_split_k) ? 1 : 0;
+    return AHIP_OK;
+}
+
+int ahip_gemm_set_in_kernel_k_cut(ahip_ctx *ctx, int enable) {
+    REQUIRE_CTX(ctx, "ahip_gemm_set_in_kernel_k_cut");
+    ctx->d.gemm_in_kernel_k_cut = enable != 0;
+    return AHIP_OK;
+}
+
 int ahip_reduce_static(ahip_ctx *ctx, int kind, float *out, const float *in, size_t outer, size_t reduce, size_t inner) {
     REQUIRE_CTX(ctx, "ahip_reduce_static");
     return altius::launch_reduce_static(ctx->d, kind, out, in, outer, reduce, inner);

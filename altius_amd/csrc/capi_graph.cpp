@@ -27,8 +27,9 @@ struct ahip_session_builder {
     bool profiling = false;
     int device = 0;
     bool graph_replay = false;
-    int gemm_algorithm = AHIP_GEMM_AUTO;
+    int gemm_algorithm = AHIP_GEMM_FP32;
     bool strided_views = true;
+    bool fused_attention = false;
 };
 struct ahip_session {
     std::shared_ptr<HipSession> s;  // shared with the device tensors the session has handed out
@@ -553,6 +554,12 @@ int ahip_session_builder_with_strided_views(ahip_session_builder *builder, int e
     return AHIP_OK;
 }
 
+int ahip_session_builder_with_fused_attention(ahip_session_builder *builder, int enable) {
+    if (!builder) return fail(AHIP_ERR_ARG, "null builder");
+    builder->fused_attention = enable != 0;
+    return AHIP_OK;
+}
+
 int ahip_session_copies_avoided(const ahip_session *session, size_t *count) {
     if (!session || !count) return fail(AHIP_ERR_ARG, "ahip_session_copies_avoided: null argument");
     *count = session->s->copies_avoided();
@@ -569,7 +576,7 @@ int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **ses
     if (!builder || !session) return fail(AHIP_ERR_ARG, "ahip_session_builder_build: null argument");
     *session = nullptr;
     HipSessionBuilder b(builder->model);
-    b.with_intra_op_num_threads(builder->threads).with_profiling_enabled(builder->profiling).with_device(builder->device).with_graph_replay(builder->graph_replay).with_gemm_algorithm(builder->gemm_algorithm).with_strided_views(builder->strided_views);
+    b.with_intra_op_num_threads(builder->threads).with_profiling_enabled(builder->profiling).with_device(builder->device).with_graph_replay(builder->graph_replay).with_gemm_algorithm(builder->gemm_algorithm).with_strided_views(builder->strided_views).with_fused_attention(builder->fused_attention);
     SessionError err;
     std::unique_ptr<HipSession> s = b.build(&err);
     if (!s) return fail(err.code(), err.to_string());

@@ -45,10 +45,8 @@ int create_device_ctx(int device, hipStream_t stream, bool own_stream, DeviceCtx
     // AHIP_GEMM_SPLIT_K=0 keeps the bf16 GEMM from cutting an XCD's partly filled last round of tiles along k
     // (for measurements).
     if (const char *e = getenv("AHIP_GEMM_SPLIT_K")) ctx->gemm_split_k = atoi(e) != 0;
-    {
-        int cus = 0;
-        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && cus >= 8) ctx->cus_per_xcd = cus / 8;
-    }
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && cus >= 8) ctx->cus_per_xcd = cus / 8;
     if (own_stream) {
         // Default priority; non-blocking with respect to the legacy default stream.
         e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
@@ -80,18 +78,28 @@ int create_device_ctx(int device, hipStream_t stream, bool own_stream, DeviceCtx
     }
     ctx->flags = static_cast<int *>(flags);
     ctx->flags_armed = false;
+    // Where do blocks run?  Decides whether the bf16 GEMM may combine the slices of a tile inside one XCD's L2.
+    // A probe that cannot run leaves the answer at "not shown", which only switches that cut off.
+    if (probe_xcd_placement(*ctx, cus) != AHIP_OK) ctx->xcd_round_robin = false;
     return AHIP_OK;
 }
 
 int check_device_flags(DeviceCtx &ctx) {
     if (!ctx.flags_armed) return AHIP_OK;
     ctx.flags_armed = false;
-    int raised = 0;
-    int rc = ctx.check(hipMemcpy(&raised, ctx.flags, sizeof(int), hipMemcpyDeviceToHost), "hipMemcpy(flags)");
+    int raised[2] = {0, 0};
+    int rc = ctx.check(hipMemcpy(raised, ctx.flags, sizeof(raised), hipMemcpyDeviceToHost), "hipMemcpy(flags)");
     if (rc) return rc;
-    if (!raised) return AHIP_OK;
-    rc = ctx.check(hipMemset(ctx.flags, 0, sizeof(int)), "hipMemset(flags)");
+    if (!raised[0] && !raised[1]) return AHIP_OK;
+    rc = ctx.check(hipMemset(ctx.flags, 0, sizeof(raised)), "hipMemset(flags)");
     if (rc) return rc;
+    if (raised[1]) {
+        // The placement the probe measured did not hold for a launch: the product just computed is not to be
+        // trusted, and the cut stays off for the rest of this context's life.
+        ctx.xcd_round_robin = false;
+        return ctx.fail(AHIP_ERR_HIP, "MatMul: the slices of a tile cut along k ran on different XCDs, so their partial sums could not be "
+                                      "combined; the in-kernel cut is now switched off for this context, run the product again");
+    }
     return ctx.fail(AHIP_ERR_ARG, "Gather: an index is outside the gathered axis");
 }
 

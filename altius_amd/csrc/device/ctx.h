@@ -37,8 +37,9 @@ struct DeviceCtx {
     // Partial results of two-stage reductions (device memory, owned).
     float *scratch = nullptr;
     size_t scratch_floats = 0;
-    // Error flags kernels raise (device memory, one int: Gather's index check); read back by
-    // check_device_flags after a synchronisation, only when a kernel that can raise one has run.
+    // Error flags kernels raise (device memory; int 0: Gather's index check, int 1: the slices of a GEMM tile
+    // cut along k did not share an XCD); read back by check_device_flags after a synchronisation, only when a
+    // kernel that can raise one has run.
     int *flags = nullptr;
     bool flags_armed = false;
     // Tensors of at least this many bytes are streamed with non-temporal accesses.
@@ -46,8 +47,9 @@ struct DeviceCtx {
     // Chains of element-wise steps that were instantiated at compile time run as straight-line code;
     // switched off, every chain takes the interpreting kernel (tests compare the two).
     bool fused_static_chains = true;
-    // Which kernel large single-batch fp32 products take (AHIP_GEMM_*).
-    int gemm_algorithm = AHIP_GEMM_AUTO;
+    // Which kernel large single-batch fp32 products take (AHIP_GEMM_*).  The default is the one whose
+    // results equal fp32 arithmetic for every operand value, infinities included.
+    int gemm_algorithm = AHIP_GEMM_FP32;
     // bf16 planes of the run-time operands of the split GEMM (device memory, owned, grows on demand;
     // the generation counts reallocations so that holders of recorded launches can tell).
     void *gemm_ws = nullptr;
@@ -59,6 +61,12 @@ struct DeviceCtx {
     int *gemm_counters = nullptr;
     bool gemm_split_k = true;
     int cus_per_xcd = 0;  // compute units / 8, read when the context is created
+    // Measured when the context is created (placement.hip): blocks whose ids agree mod 8 run on one XCD, and
+    // eight consecutive blocks on eight different ones.  The bf16 GEMM lets the slices of a tile meet in one
+    // XCD's L2 only when this holds and gemm_in_kernel_k_cut is on; otherwise it does not cut tiles inside the
+    // kernel at all.
+    bool xcd_round_robin = false;
+    bool gemm_in_kernel_k_cut = true;
     std::vector<ConstantBuffer> gemm_constants;
     std::vector<PackedOperand> gemm_packed;
     std::string last_error;
@@ -76,6 +84,12 @@ const char *global_error();
 // Creates / tears down a context (stream + scratch buffer) on `device`.
 int create_device_ctx(int device, hipStream_t stream, bool own_stream, DeviceCtx *ctx, std::string *error);
 void destroy_device_ctx(DeviceCtx *ctx);
+// The decision behind DeviceCtx::xcd_round_robin, on its own so that it can be tested without a GPU: true iff
+// the CU count is a multiple of eight, blocks 0..7 of the probe launch ran on eight different XCDs and every
+// block i ran where block i % 8 did.
+bool xcd_round_robin_holds(int cu_count, const uint32_t *xcc_of_block, size_t n_blocks);
+// Runs the probe launch on the context's stream (uses the scratch buffer) and sets ctx.xcd_round_robin.
+int probe_xcd_placement(DeviceCtx &ctx, int cu_count);
 // After the stream has been synchronised: reports and clears an error flag raised by a kernel.
 int check_device_flags(DeviceCtx &ctx);
 

@@ -146,6 +146,7 @@ struct SplitGemmArgs {
     uint32_t full, sf;
     float *partials;
     int *counters;
+    int *misplaced;  // raised when the slices of a tile did not all run on one XCD
     int c_vec;    // 16-byte stores into C are aligned
     int c_stream;  // C is large: write it with non-temporal stores
 };
@@ -296,11 +297,22 @@ __global__ __launch_bounds__(THREADS, 1) void gemm_bf16x3(SplitGemmArgs g) {
         // write through the L1, and vmcnt(0) says the L2 has them.  (A device-wide release fence here would
         // write the whole L2 back, once per wavefront.)
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        if (tid == 0) arrived = atomicAdd(&g.counters[idx], 1);
+        // The launcher cuts tiles only on a context that has measured that blocks whose ids agree mod 8 share an
+        // XCD.  Every launch checks it again per tile: a slice counts itself in with 1 in the low byte and 1 in
+        // the 3-bit field of the XCD it really ran on (at most 8 slices, so at most 7 ahead of the last one).
+        uint32_t xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        xcc &= 7u;
+        if (tid == 0) arrived = atomicAdd(&g.counters[idx], (int)(1u + (1u << (8 + 3 * xcc))));
         __syncthreads();
-        if (arrived != (int)nparts - 1) return;
+        if ((arrived & 0xff) != (int)nparts - 1) return;
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // nothing stale in this CU's L1
-        if (tid == 0) atomicExch(&g.counters[idx], 0);      // ready for the next launch
+        if (tid == 0) {
+            atomicExch(&g.counters[idx], 0);  // ready for the next launch
+            // A slice that ran on another XCD left its partial sums in another L2: say so instead of adding up
+            // whatever this L2 holds at those addresses.
+            if (((uint32_t)arrived >> 8) != ((nparts - 1) << (3 * xcc))) atomicExch(g.misplaced, 1);
+        }
         // Sum in slice order, 64 registers' worth of 16-byte loads in flight at a time.
         const f32x4 *all = reinterpret_cast<const f32x4 *>(g.partials + (size_t)idx * nparts * (TM * TN)) + tid;
 #pragma unroll
@@ -584,7 +596,8 @@ int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, 
     g.full = g.chunk / per * per;
     g.sf = 1;
     const uint32_t rem = g.chunk - g.full;
-    if (rem && ctx.gemm_split_k) {
+    // Only where the slices of a tile have been shown to share an L2 (block id mod 8 = XCD, DeviceCtx::xcd_round_robin).
+    if (rem && ctx.gemm_split_k && ctx.gemm_in_kernel_k_cut && ctx.xcd_round_robin) {
         uint32_t sf = per / rem;
         sf = std::min(sf, 8u);
         sf = std::min(sf, stages / 4);
@@ -593,7 +606,10 @@ int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, 
     if (g.sf == 1) g.full = g.chunk;
     g.partials = nullptr;
     g.counters = nullptr;
+    g.misplaced = ctx.flags ? ctx.flags + 1 : nullptr;
     if (g.sf > 1) {
+        if (!g.misplaced) return ctx.fail(AHIP_ERR_HIP, "gemm: the context has no error flags");
+        ctx.flags_armed = true;
         rc = ensure_partials(ctx, (size_t)8 * (g.chunk - g.full) * g.sf * TM * TN * sizeof(float));
         if (rc) return rc;
         g.partials = static_cast<float *>(ctx.gemm_partials);

@@ -78,6 +78,15 @@ void BufferPool::release(void *ptr, size_t bucket) {
     if (ptr) free_[bucket].push_back(ptr);
 }
 
+bool BufferPool::take(void *ptr, size_t bucket) {
+    auto it = free_.find(bucket);
+    if (it == free_.end()) return false;
+    auto pos = std::find(it->second.begin(), it->second.end(), ptr);
+    if (pos == it->second.end()) return false;
+    it->second.erase(pos);
+    return true;
+}
+
 void BufferPool::trim() {
     if (hold_) return;
     for (auto &kv : free_) {
@@ -104,7 +113,7 @@ std::unique_ptr<HipSession> HipSessionBuilder::build(SessionError *err) {
         return nullptr;
     }
     s->plan_ = create_execution_plan(s->model_);
-    if (strided_views_) s->plan_views();
+    if (strided_views_) s->plan_views(fused_attention_);
 
     std::string derr;
     int rc = create_device_ctx(device_, nullptr, true, &s->ctx_, &derr);
@@ -168,6 +177,7 @@ bool HipSession::allocate(const TypedFixedShape &shape, DeviceTensor *out, Sessi
     const int rc = pool_->acquire(out->nbytes(), &block->ptr, &block->bucket);
     if (rc) return fail_code(err, rc, ctx_.last_error);
     block->pool = pool_.get();
+    if (capturing_) capture_allocs_.emplace_back(block->ptr, block->bucket);
     out->ptr = block->ptr;
     out->block = std::move(block);
     return true;
@@ -444,6 +454,7 @@ bool HipSession::try_capture(const std::string &key, const std::vector<Tensor> &
     }
     capturing_ = true;
     capture_refused_ = false;
+    capture_allocs_.clear();
     ctx_.flags_armed = false;
     bool ok = true;
     SessionError local;
@@ -478,6 +489,22 @@ bool HipSession::try_capture(const std::string &key, const std::vector<Tensor> &
     }
     if (ok && end == hipSuccess && graph && hipGraphInstantiate(&run.exec, graph, nullptr, nullptr, 0) == hipSuccess) {
         (void)hipGraphDestroy(graph);
+        // The recorded kernels address their intermediates directly.  Those blocks went back to the pool as the
+        // plan freed them (and were reused inside the recording, which stream order allows); take every one of
+        // them out of the pool for as long as the graph lives.
+        values.clear();
+        pending_attn_.clear();
+        std::sort(capture_allocs_.begin(), capture_allocs_.end());
+        capture_allocs_.erase(std::unique(capture_allocs_.begin(), capture_allocs_.end()), capture_allocs_.end());
+        for (const auto &a : capture_allocs_)
+            if (pool_->take(a.first, a.second)) {
+                auto block = std::make_shared<DeviceBlock>();
+                block->pool = pool_.get();
+                block->ptr = a.first;
+                block->bucket = a.second;
+                run.blocks.push_back(std::move(block));
+            }
+        capture_allocs_.clear();
         graphs_[key] = std::move(run);
         pool_->hold_memory(true);
         return true;

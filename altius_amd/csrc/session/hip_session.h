@@ -41,6 +41,8 @@ public:
     ~BufferPool();
     int acquire(size_t bytes, void **ptr, size_t *bucket);
     void release(void *ptr, size_t bucket);
+    // Takes one particular cached block out of the free list (true if it was there): the caller owns it now.
+    bool take(void *ptr, size_t bucket);
     void trim();  // returns every cached block to the device (a no-op while trimming is held off)
     // Recorded HIP graphs address cached blocks directly: while one exists nothing may be freed.
     void hold_memory(bool hold) { hold_ = hold; }
@@ -157,6 +159,10 @@ private:
         hipGraphExec_t exec = nullptr;
         std::vector<DeviceTensor> inputs;   // persistent device copies of the graph inputs
         std::vector<DeviceTensor> outputs;  // where the recorded kernels leave the graph outputs
+        // Every other block the recorded kernels read or write (the run's intermediates): kept out of the pool
+        // while the graph exists, so that no later run -- a device-resident one whose outputs the caller holds
+        // included -- is handed memory that a replay overwrites.
+        std::vector<std::shared_ptr<DeviceBlock>> blocks;
         bool has_gather = false;
         bool unusable = false;              // capture was tried and refused; run eagerly from now on
     };
@@ -166,7 +172,7 @@ private:
     void drop_graphs();
     // Decides at build time which Split / Transpose nodes hand out views and which MatMul nodes
     // write their result in the layout a following Transpose would produce.
-    void plan_views();
+    void plan_views(bool fused_attention);
     // Replaces a view by a dense copy of itself.
     bool materialize(DeviceTensor *t, SessionError *err);
     // How a MatMul reads an operand that may be a strided view: its last two axes as a matrix with one unit
@@ -219,6 +225,7 @@ private:
     std::mutex mutex_;
     bool graph_replay_ = false;
     bool capturing_ = false;        // a stream capture is in progress: nothing may synchronise
+    std::vector<std::pair<void *, size_t>> capture_allocs_;  // (block, bucket) of every allocation made while recording
     bool capture_refused_ = false;  // a node needed the host during capture
     std::map<std::string, CapturedRun> graphs_;
     std::map<std::string, int> eager_runs_;  // per input signature: eager runs so far (the pool is warm after one)
@@ -266,9 +273,10 @@ public:
         graph_replay_ = enable;
         return *this;
     }
-    // Not in the reference: the kernel large single-batch MatMul / Gemm products take (AHIP_GEMM_AUTO, the
-    // default, AHIP_GEMM_FP32 or AHIP_GEMM_BF16X3).  Float initializers are declared constant to the
-    // GEMM, so a weight operand's bf16 planes are made on its first use and kept.
+    // Not in the reference: the kernel large single-batch MatMul / Gemm products take (AHIP_GEMM_FP32, the
+    // default and the reference's semantics for infinite operands, AHIP_GEMM_AUTO or AHIP_GEMM_BF16X3).
+    // Float initializers are declared constant to the GEMM, so a weight operand's bf16 planes are made on
+    // its first use and kept.
     HipSessionBuilder &with_gemm_algorithm(int algorithm) {
         gemm_algorithm_ = algorithm;
         return *this;
@@ -278,6 +286,12 @@ public:
     // that Transpose's layout directly (default on; off makes every node copy, as the reference does).
     HipSessionBuilder &with_strided_views(bool enable) {
         strided_views_ = enable;
+        return *this;
+    }
+    // Not in the reference: MatMul -> Softmax -> MatMul as one attention kernel (default off: its sums run in
+    // another order than the three operators', 2e-4 relative).  Needs strided views.
+    HipSessionBuilder &with_fused_attention(bool enable) {
+        fused_attention_ = enable;
         return *this;
     }
     // Not in the reference: which GPU to run on (default 0).
@@ -295,8 +309,9 @@ private:
     bool enable_profiling_ = false;
     int device_ = 0;
     bool graph_replay_ = false;
-    int gemm_algorithm_ = AHIP_GEMM_AUTO;
+    int gemm_algorithm_ = AHIP_GEMM_FP32;
     bool strided_views_ = true;
+    bool fused_attention_ = false;
 };
 
 }  // namespace altius

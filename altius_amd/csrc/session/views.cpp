@@ -232,7 +232,7 @@ bool HipSession::run_attention_tail(const Op &op, const std::vector<DeviceTensor
 // A Split or Transpose hands out views when everything downstream of it can read them in place:
 // MatMul operands, possibly through reshapes and further transposes.  A MatMul whose only reader is
 // a Transpose that keeps the last axis writes its result directly in that Transpose's layout.
-void HipSession::plan_views() {
+void HipSession::plan_views(bool fused_attention) {
     const auto users = model_.get_value_users();
     const Graph &g = model_.graph;
     auto is_output = [&](ValueId v) { return std::find(g.outputs.begin(), g.outputs.end(), v) != g.outputs.end(); };
@@ -292,7 +292,7 @@ void HipSession::plan_views() {
                 }
             }
             // MatMul -> Softmax(last axis, optional scalar scale, no mask) -> MatMul(first operand): one attention kernel.
-            {
+            if (fused_attention) {
                 const NodeId sid = *it->second.begin();
                 const Node &sm = g.nodes[sid];
                 if (sm.op.kind == OpKind::Softmax && n.inputs.size() == 2 && !sm.inputs.empty() && sm.inputs[0] == n.outputs[0] &&

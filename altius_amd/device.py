@@ -16,7 +16,14 @@ SQRT, ERF, GELU, SIGMOID, HARDSIGMOID, RELU, TANH, LEAKYRELU, EXP, ROUND, CLIP =
 REDUCE_MEAN, REDUCE_MAX, REDUCE_SUM = 0, 1, 2
 BOOL, F32, I32, I64 = 0, 1, 2, 3
 GEMM_AUTO, GEMM_FP32, GEMM_BF16X3 = 0, 1, 2
+GEMM_DEFAULT = GEMM_FP32  # what a new context or session uses: the reference's results for every operand value
 _ELEM_OF = {np.dtype(np.bool_): BOOL, np.dtype(np.float32): F32, np.dtype(np.int32): I32, np.dtype(np.int64): I64}
+
+
+def xcd_round_robin_holds(cu_count, xcc_of_block):
+    """The decision a context takes from its placement probe (host only): block i ran on XCD i % 8 for every i."""
+    ids = np.ascontiguousarray(xcc_of_block, dtype=np.uint32)
+    return bool(_lib.lib().ahip_xcd_round_robin_holds(int(cu_count), ids.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)), ids.size))
 
 
 def broadcast_shape(a_dims, b_dims):
@@ -443,6 +450,16 @@ class Context:
     def gemm_set_algorithm(self, algorithm):
         """GEMM_AUTO / GEMM_FP32 / GEMM_BF16X3: the kernel single-batch products take."""
         check(self.L.ahip_gemm_set_algorithm(self.handle, int(algorithm)), self.handle)
+
+    def gemm_in_kernel_k_cut(self):
+        """(placement shown, cut enabled): whether the probe at context creation found block i on XCD i % 8, and
+        whether the bf16 GEMM's in-kernel k cut is switched on.  The cut runs only when both hold."""
+        shown, enabled = ctypes.c_int(), ctypes.c_int()
+        check(self.L.ahip_gemm_in_kernel_k_cut(self.handle, ctypes.byref(shown), ctypes.byref(enabled)), self.handle)
+        return bool(shown.value), bool(enabled.value)
+
+    def gemm_set_in_kernel_k_cut(self, enable):
+        check(self.L.ahip_gemm_set_in_kernel_k_cut(self.handle, int(bool(enable))), self.handle)
 
     def gemm_register_constant(self, buf):
         """Declares a device buffer immutable: the split GEMM keeps the planes of operands inside it."""

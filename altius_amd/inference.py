@@ -39,11 +39,13 @@ class _NamedSession:
         return self._sess.profile()
 
 
-def session(model, enable_profiling=False, intra_op_num_threads=1, backend="hip", device=0, gemm_algorithm=0):
+def session(model, enable_profiling=False, intra_op_num_threads=1, backend="hip", device=0, gemm_algorithm=1,
+            fused_attention=False):
     """altius_py.session (lib.rs:44-88): the same rewrite pipeline -- fuse_layer_norm, fuse_gelu, fuse_fast_gelu,
     element-wise fusion for the backend that has a kernel for it (the reference: "cpu"; here: "hip", with the wider
     rule, after the scale and mask in front of each Softmax and the bias row behind each MatMul have been folded into them), eliminate_identity -- then the session builder.  The model object is left untouched, as in the
-    reference (it takes a clone)."""
+    reference (it takes a clone).  gemm_algorithm (default device.GEMM_FP32) and fused_attention (default off) are the
+    two switches that trade the reference's exact semantics for speed; a caller opts in."""
     if backend != "hip":
         raise RuntimeError(f"Unknown backend: {backend}")
     m = model.clone()
@@ -56,7 +58,7 @@ def session(model, enable_profiling=False, intra_op_num_threads=1, backend="hip"
     m.fuse_elemwise_ops(extended=True)
     m.eliminate_identity()
     builder = HipSessionBuilder(m).with_profiling_enabled(enable_profiling).with_intra_op_num_threads(intra_op_num_threads)
-    return _NamedSession(builder.with_device(device).with_gemm_algorithm(gemm_algorithm).build())
+    return _NamedSession(builder.with_device(device).with_gemm_algorithm(gemm_algorithm).with_fused_attention(fused_attention).build())
 
 
 class InferenceSession:

@@ -342,14 +342,14 @@ def vit_table(batch, layers=12):
     for i, (name, model) in enumerate(versions):
         algo = D.GEMM_AUTO if i >= 3 else D.GEMM_FP32
         views = i >= 4
-        sess = HipSessionBuilder(model).with_gemm_algorithm(algo).with_strided_views(views).build()
+        sess = HipSessionBuilder(model).with_gemm_algorithm(algo).with_strided_views(views).with_fused_attention(views).build()
         best = float("inf")
         for _ in range(4):
             outs = sess.run([x], copy=False)
             best = min(best, sess.last_device_ms())
             del outs
         sess.close()
-        prof = HipSessionBuilder(model).with_gemm_algorithm(algo).with_strided_views(views).with_profiling_enabled(True).build()
+        prof = HipSessionBuilder(model).with_gemm_algorithm(algo).with_strided_views(views).with_fused_attention(views).with_profiling_enabled(True).build()
         for _ in range(2):
             outs = prof.run([x], copy=False)
             del outs
@@ -406,7 +406,7 @@ def build_next_rows(ctx, D, batch=256):
             def launch(algo=algo):
                 ctx.gemm_set_algorithm(algo)
                 ctx.gemm_raw(c.ptr, a.ptr, w.ptr, None, b, m, n_, k, a_bs=a_bs, b_bs=b_bs, c_bs=m * n_)
-                ctx.gemm_set_algorithm(D.GEMM_AUTO)
+                ctx.gemm_set_algorithm(D.GEMM_DEFAULT)
 
             rows.append(("%s (%s)" % (name, label), nbytes, 2.0 * b * m * n_ * k, launch))
 

@@ -323,12 +323,32 @@ int ahip_attention(ahip_ctx *ctx, float *o, const float *q, const float *k, cons
  * AHIP_GEMM_BF16X3: every operand value is split exactly into three bf16 numbers and six bf16 MFMAs per
  * product accumulate in fp32 (the terms dropped are below 2^-23 of each product); measured against
  * float64 it is as close as a chain of fp32 multiply-adds, and about 1.6 times faster on large shapes.
- * AHIP_GEMM_AUTO (the default): BF16X3 for large products whose C fills whole 256 x 256 tiles, FP32
- * otherwise.  The reference has one sgemm (gemm.rs:3-52) and no such switch. */
+ * AHIP_GEMM_AUTO: BF16X3 for large products whose C fills whole 256 x 256 tiles, FP32 otherwise.
+ * The default is AHIP_GEMM_FP32, the only one with the reference's result for every operand value: on
+ * the BF16X3 route an infinite operand value gives NaN in most of its row (inf in the leading plane meets
+ * the lower planes of the other operand: inf * 0, or inf - inf) where fp32 arithmetic gives +-inf.  The reference has one sgemm
+ * (gemm.rs:3-52) and no such switch. */
 #define AHIP_GEMM_AUTO 0
 #define AHIP_GEMM_FP32 1
 #define AHIP_GEMM_BF16X3 2
 int ahip_gemm_set_algorithm(ahip_ctx *ctx, int algorithm);
+/* The BF16X3 kernel cuts the tiles of a partly filled last round of blocks along k and lets the slice that
+ * finishes last add the others' partial sums up out of one XCD's L2.  That needs all slices of a tile on one
+ * XCD, which the kernel arranges by block id (the slices of a tile have equal ids mod 8, and consecutive ids go
+ * to the eight XCDs in turn, starting wherever the queue's previous launch stopped).  ahip_init measures that
+ * once per context with a probe launch (every block records its XCC id); the cut is used only if the probe
+ * showed blocks 0..7 on eight different XCDs, every block i where block i % 8 ran, and a CU count that is a
+ * multiple of eight -- otherwise tiles are not cut and the results are the same.  Every launch that cuts tiles
+ * checks the XCC ids of each tile's slices again; a mismatch makes the next ahip_sync / ahip_session_run return
+ * AHIP_ERR_HIP and switches the cut off for the context.  ahip_gemm_in_kernel_k_cut reports what the probe
+ * showed and whether the cut is switched on; ahip_gemm_set_in_kernel_k_cut(ctx, 0) switches it off (it cannot
+ * switch on what the probe did not show).  ahip_xcd_round_robin_holds is the decision itself on a recorded
+ * placement (no GPU needed): 1 iff cu_count is a multiple of 8 (and >= 8), n_blocks >= 16,
+ * xcc_of_block[0..7] are eight different values below 8 and xcc_of_block[i] == xcc_of_block[i % 8] for all i.
+ * No counterpart in the reference. */
+int ahip_gemm_in_kernel_k_cut(ahip_ctx *ctx, int *placement_shown, int *enabled);
+int ahip_gemm_set_in_kernel_k_cut(ahip_ctx *ctx, int enable);
+int ahip_xcd_round_robin_holds(int cu_count, const uint32_t *xcc_of_block, size_t n_blocks);
 /* Declares the device buffer [ptr, ptr + bytes) immutable (model weights) until it is unregistered:
  * AHIP_GEMM_BF16X3 then splits an operand that lies inside it once and keeps the planes (1.5 times the
  * operand's size) instead of splitting it on every call.  Unregister before freeing or rewriting the
@@ -561,9 +581,11 @@ int ahip_session_builder_with_device(ahip_session_builder *builder, int device);
  * or operands need the host during the run, and profiled sessions, keep running node by node. */
 int ahip_session_builder_with_graph_replay(ahip_session_builder *builder, int enable);
 /* Not in the reference: the kernel the session's large single-batch MatMul / Gemm products take
- * (AHIP_GEMM_AUTO, the default, AHIP_GEMM_FP32 or AHIP_GEMM_BF16X3; see ahip_gemm_set_algorithm).  The
- * session declares its float initializers constant to the GEMM, so the bf16 planes of a weight are
- * made on its first use and kept until the session is freed. */
+ * (AHIP_GEMM_FP32, the default, AHIP_GEMM_AUTO or AHIP_GEMM_BF16X3; see ahip_gemm_set_algorithm).  The
+ * default keeps the reference's semantics for every operand value (compute_mat_mul, session.rs:621-684: an
+ * infinite operand gives +-inf); AUTO and BF16X3 are the faster route a caller opts into, where an infinite
+ * operand gives NaN.  The session declares its float initializers constant to the GEMM, so the bf16 planes
+ * of a weight are made on its first use and kept until the session is freed. */
 int ahip_session_builder_with_gemm_algorithm(ahip_session_builder *builder, int algorithm);
 /* Not in the reference, whose Split and Transpose always copy (session.rs:1179-1278, 1488-1548): with enable
  * != 0 (the default) a Split or Transpose whose result only MatMuls read, possibly through reshapes and further
@@ -572,6 +594,12 @@ int ahip_session_builder_with_gemm_algorithm(ahip_session_builder *builder, int 
  * products are the same kernels on the same values: results do not change by a bit.  A view that some other
  * reader needs, or that the GEMM's addressing cannot express, is copied as before. */
 int ahip_session_builder_with_strided_views(ahip_session_builder *builder, int enable);
+/* Not in the reference, which runs MatMul, Softmax and MatMul as three kernels (session.rs:621-684, 990-1026):
+ * with enable != 0 (default 0; needs strided views) a MatMul -> Softmax(last axis, with the scale and per-key
+ * mask that ahip_fuse_softmax_prologue absorbed) -> MatMul chain with 64-wide heads runs as one ahip_attention
+ * kernel that never writes the scores.  Its sums run in another order than the three operators': results
+ * differ from theirs by up to 2e-4 relative, which is why a caller has to ask for it. */
+int ahip_session_builder_with_fused_attention(ahip_session_builder *builder, int enable);
 /* Nodes of the last node-by-node run that were served without their copy (views taken, transposed layouts
  * written in place). */
 int ahip_session_copies_avoided(const ahip_session *session, size_t *count);

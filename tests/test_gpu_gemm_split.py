@@ -19,7 +19,7 @@ RNG = np.random.default_rng(77)
 def split(ctx):
     ctx.gemm_set_algorithm(D.GEMM_BF16X3)
     yield ctx
-    ctx.gemm_set_algorithm(D.GEMM_AUTO)
+    ctx.gemm_set_algorithm(D.GEMM_DEFAULT)
 
 
 def ints(*shape):
@@ -158,22 +158,71 @@ def test_no_less_accurate_than_the_fp32_matrix_cores(ctx, case):
         ctx.gemm_set_algorithm(D.GEMM_BF16X3)
         e16 = rel_error(ctx.matmul(a, b), a, b)
     finally:
-        ctx.gemm_set_algorithm(D.GEMM_AUTO)
+        ctx.gemm_set_algorithm(D.GEMM_DEFAULT)
     print(f"rms error / |A||B|: fp32 MFMA {np.sqrt((e32 ** 2).mean()):.3e}, bf16 x 3 {np.sqrt((e16 ** 2).mean()):.3e}; "
           f"max {e32.max():.3e} vs {e16.max():.3e}")
     assert np.sqrt((e16 ** 2).mean()) <= 1.25 * np.sqrt((e32 ** 2).mean())
     assert e16.max() <= 1.25 * e32.max()
 
 
+# Shapes whose last round of blocks per XCD is partly filled, so tiles are cut along k inside the kernel:
+# 16 tiles -> 2 per XCD -> up to 8 slices each; 48 tiles -> 6 per XCD -> 5 slices; 9 tiles (7 XCDs with 2, ragged).
+CUT_SHAPES = [(1024, 512, 1024), (1024, 2048, 1024), (2048, 640, 1536), (700, 1024, 600), (256, 4096, 256)]
+
+
+@pytest.mark.parametrize("m,k,n", CUT_SHAPES)
+def test_k_cut_inside_the_kernel_and_its_fallback_give_the_same_exact_products(split, case, m, k, n):
+    """The slices of a tile are added up inside one XCD's L2 only on a context whose probe showed that blocks with
+    equal ids mod 8 share an XCD; with the cut forced off (what such a context falls back to) every tile is computed by one block.  Both
+    must give the exact products of integer operands, bit for bit, on repeated launches (the counters and the
+    partial sums of the previous launch are still in place)."""
+    shown, enabled = split.gemm_in_kernel_k_cut()
+    case(f"bf16x3 k cut {m}x{k}x{n}; placement shown {shown}, cut enabled {enabled}")
+    assert enabled
+    a, b = ints(m, k), ints(k, n)
+    want = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+    bias = ints(n)
+    try:
+        for cut in (True, False, True):
+            split.gemm_set_in_kernel_k_cut(cut)
+            assert split.gemm_in_kernel_k_cut() == (shown, cut)
+            for _ in range(2):
+                assert_bits_equal(split.matmul(a, b), want, f"cut {cut}")
+            assert_bits_equal(split.gemm(a, b, bias, alpha=2.0, beta=3.0), 2 * want + 3 * bias, f"cut {cut}, alpha / beta / bias")
+        ar, br = RNG.standard_normal((m, k)).astype(np.float32), RNG.standard_normal((k, n)).astype(np.float32)
+        split.gemm_set_in_kernel_k_cut(True)
+        with_cut = split.matmul(ar, br)
+        split.gemm_set_in_kernel_k_cut(False)
+        without = split.matmul(ar, br)
+        for got in (with_cut, without):
+            assert rel_error(got, ar, br).max() <= (k + 2) * 2.0 ** -24
+    finally:
+        split.gemm_set_in_kernel_k_cut(True)
+
+
+def test_this_part_deals_blocks_to_xcds_in_turn(ctx, case):
+    """What the library measures at context creation on an MI355X in its default partition mode: 256 CUs, eight
+    consecutive blocks on eight XCDs, block i where block i % 8 ran.  (On a part where this does not hold the
+    library only loses the in-kernel cut.)"""
+    case("placement probe")
+    shown, enabled = ctx.gemm_in_kernel_k_cut()
+    assert enabled
+    assert shown, "the probe did not find blocks dealt to the XCDs in turn: the bf16 GEMM runs without its in-kernel k cut"
+
+
 def test_auto_takes_the_split_kernel_at_model_size(ctx, case):
-    """[12608, 768] x [768, 2304] (a quarter of the ViT-B/16 batch-256 QKV projection) under the default rule, with a
-    bias row: sampled rows against float64."""
+    """[12608, 768] x [768, 2304] (a quarter of the ViT-B/16 batch-256 QKV projection) under the AHIP_GEMM_AUTO rule,
+    with a bias row: sampled rows against float64."""
     case("auto-selected gemm 12608x768x2304")
     m, k, n = 12608, 768, 2304
     a = RNG.standard_normal((m, k)).astype(np.float32)
     b = (RNG.standard_normal((k, n)) * 0.03).astype(np.float32)
     bias = RNG.standard_normal(n).astype(np.float32)
-    got = ctx.gemm(a, b, bias)
+    try:
+        ctx.gemm_set_algorithm(D.GEMM_AUTO)
+        got = ctx.gemm(a, b, bias)
+    finally:
+        ctx.gemm_set_algorithm(D.GEMM_DEFAULT)
     rows = RNG.choice(m, 64, replace=False)
     exact = a[rows].astype(np.float64) @ b.astype(np.float64)
     scale = np.abs(a[rows]).astype(np.float64) @ np.abs(b).astype(np.float64)

@@ -159,8 +159,8 @@ def test_replay_of_an_encoder_layer_with_views_attention_and_the_bf16_route(case
         m = graphs.vit_encoder(batch, layers=1, tokens=50, classes=10)
         m.fuse_layer_norm(), m.fuse_gelu(), m.fuse_softmax_prologue(), m.fuse_matmul_bias(), m.fuse_transpose_matmul()
         m.fuse_elemwise_ops(extended=True)
-        sessions[batch] = (HipSessionBuilder(m.clone()).with_gemm_algorithm(D.GEMM_BF16X3).build(),
-                           HipSessionBuilder(m).with_gemm_algorithm(D.GEMM_BF16X3).with_graph_replay().build())
+        sessions[batch] = (HipSessionBuilder(m.clone()).with_gemm_algorithm(D.GEMM_BF16X3).with_fused_attention().build(),
+                           HipSessionBuilder(m).with_gemm_algorithm(D.GEMM_BF16X3).with_fused_attention().with_graph_replay().build())
     for i in range(4):
         for batch, (eager, replayed) in sessions.items():
             x = synth.normal(50 + i, [batch, 50, 768], std=1.0)
@@ -173,3 +173,40 @@ def test_replay_of_an_encoder_layer_with_views_attention_and_the_bf16_route(case
         eager.close()
         replayed.close()
 
+
+
+def test_device_resident_outputs_survive_replays(case, ctx):
+    """A recorded graph addresses its intermediates directly.  The blocks they lived in must stay out of the pool
+    while the graph exists: outputs of run_device() that the caller holds across replayed run() calls keep their
+    bytes.  (The pool hands blocks out last-in first-out, so outputs are freed and held in turn here: that is what
+    makes a later output land in a block an earlier run used for an intermediate.)"""
+    case("graph replay: run_device outputs held across replays")
+    c = synth.cfg2(batch=2)
+    shape = c["x"].shape
+    sess = HipSessionBuilder(chain_model(shape, c["gamma"], c["beta"])).with_graph_replay().build()
+    eager = HipSessionBuilder(chain_model(shape, c["gamma"], c["beta"])).build()
+    xs = [synth.normal(300 + i, shape, std=1.0 + i) for i in range(6)]
+    for i in range(3):                                    # eager, recorded, replayed
+        (got,) = sess.run([xs[i]])
+        assert_bits_equal(got, eager.run([xs[i]])[0], f"run {i}")
+    assert sess.graph_replays() == 2
+    want = [eager.run([xs[3 + i]])[0] for i in range(3)]
+    d_in = [ctx.upload(xs[3 + i]) for i in range(3)]
+    held = []
+    for i in range(12):
+        (out,) = sess.run_device([(d_in[i % 3].ptr, shape, np.float32)])
+        if i % 2 == 0:
+            sess.synchronize()
+            out.free()                                    # back to the pool: the next run's blocks come in another order
+        else:
+            held.append((i % 3, out))
+    sess.synchronize()
+    for i in range(4):
+        (got,) = sess.run([xs[i]])                        # replays: the recorded kernels write their intermediates again
+        assert_bits_equal(got, eager.run([xs[i]])[0], f"replay {i}")
+    assert sess.graph_replays() == 6
+    for n, (i, out) in enumerate(held):
+        assert_bits_equal(ctx.download(out, shape), want[i], f"held output {n} after the replays")
+        out.free()
+    for b in d_in:
+        ctx.free(b)

@@ -233,4 +233,4 @@ def test_few_tiles_and_a_long_k_are_cut_along_k(ctx, case, m, k, n):
         a, b = RNG.standard_normal((m, k)).astype(np.float32), RNG.standard_normal((k, n)).astype(np.float32)
         check_bound(ctx.matmul(a, b), a, b, "random operands")
     finally:
-        ctx.gemm_set_algorithm(D.GEMM_AUTO)
+        ctx.gemm_set_algorithm(D.GEMM_DEFAULT)

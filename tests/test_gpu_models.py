@@ -184,15 +184,16 @@ def oracle_bert(ids, mask, p):
     return x
 
 
-def test_bert_style_encoder_layer(case):
-    case("BERT-style encoder layer from ONNX bytes")
+@pytest.mark.parametrize("fused_attention", [False, True])
+def test_bert_style_encoder_layer(case, fused_attention):
+    case(f"BERT-style encoder layer from ONNX bytes, one-kernel attention {fused_attention}")
     data, p = make_bert()
     ids = RNG.integers(0, VOCAB, size=(B, T)).astype(np.int64)
     mask = np.ones((B, T), np.int64)
     mask[0, 17:] = 0
     mask[1, 9:] = 0
     model = Model.load_onnx_from_buffer(data)
-    sess = session(model, enable_profiling=True)
+    sess = session(model, enable_profiling=True, fused_attention=fused_attention)
     (hidden,) = sess.run({"input_ids": ids, "attention_mask": mask})
     np.testing.assert_allclose(hidden, oracle_bert(ids, mask, p), rtol=3e-4, atol=3e-4)
     ops = set(sess.profile())
@@ -317,7 +318,7 @@ def test_full_width_vit_encoder_every_fast_path_agrees_with_the_plain_one(case, 
 
     fast = base.clone()
     fast.fuse_softmax_prologue(), fast.fuse_matmul_bias(), fast.fuse_transpose_matmul(), fast.fuse_elemwise_ops(extended=True)
-    sess = HipSessionBuilder(fast).with_graph_replay().build()
+    sess = HipSessionBuilder(fast).with_gemm_algorithm(D.GEMM_AUTO).with_fused_attention().with_graph_replay().build()
     got = np.array(sess.run([x])[0])
     assert sess.copies_avoided() > 0
     scale = float(np.abs(want).max())

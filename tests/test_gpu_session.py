@@ -430,3 +430,98 @@ def test_run_from_several_threads(case):
         for t in threads:
             t.join()
     assert not errors, errors
+
+
+# ---- what a session built with no switches returns -----------------------------------------------
+
+def matmul_model(m_rows, k, n, w):
+    """x [m, k] -> MatMul with a weight initializer [k, n]."""
+    m = Model(opset_version=13)
+    x = m.new_val_named_and_shaped("x", [m_rows, k])
+    y = m.new_val_named("y")
+    m.add_input(x)
+    m.add_node(Op.MatMul, [x, m.new_initializer(w)], [y])
+    m.add_output(y)
+    return m
+
+
+def test_default_session_gives_the_reference_result_for_infinite_operands(case):
+    """compute_mat_mul (session.rs:621-684) is fp32 arithmetic: an infinite operand value gives +-inf in its
+    row.  A session built with no switches must return exactly that, also at a size where AHIP_GEMM_AUTO
+    would take the bf16 matrix cores; a session that opts in to AHIP_GEMM_BF16X3 or AHIP_GEMM_AUTO returns NaN
+    for most of those rows (the documented difference: inf in the leading plane meets the lower planes of the
+    other operand, inf * 0 or inf - inf), the reference's +-inf for the rest, and agrees everywhere else."""
+    from altius_amd import device as D
+
+    case("default session: MatMul with +-inf operands, 2048 x 1024 x 1024")
+    rng = np.random.default_rng(11)
+    rows, k, n = 2048, 1024, 1024      # 2^31 multiply-adds, whole 256 x 256 tiles: the AUTO rule picks bf16 x 3
+    a = rng.standard_normal((rows, k)).astype(np.float32)
+    w = (rng.standard_normal((k, n)) * 0.05).astype(np.float32)
+    assert not (w == 0).any()
+    a[3, 17] = np.inf
+    a[700, 1000] = -np.inf
+    a[2047, 0] = np.inf
+    want = O.matmul(a, w)
+    inf_rows = [3, 700, 2047]
+    assert np.isinf(want[inf_rows]).all() and not np.isnan(want).any()
+    assert np.array_equal(np.sign(want[3]), np.sign(w[17])) and np.array_equal(np.sign(want[700]), -np.sign(w[1000]))
+
+    (got,) = HipSessionBuilder(matmul_model(rows, k, n, w)).build().run([a])
+    finite = np.ones(rows, bool)
+    finite[inf_rows] = False
+    assert np.array_equal(got[inf_rows], want[inf_rows]), "the rows of the infinite operands"
+    assert np.isfinite(got[finite]).all()
+    np.testing.assert_allclose(got[finite], want[finite], rtol=1e-4, atol=1e-4)  # summation order only
+
+    for algo in (D.GEMM_BF16X3, D.GEMM_AUTO):
+        (fast,) = HipSessionBuilder(matmul_model(rows, k, n, w)).with_gemm_algorithm(algo).build().run([a])
+        nan = np.isnan(fast[inf_rows])
+        assert nan.mean() > 0.5, "bf16 x 3: inf in the leading plane against the other operand's lower planes"
+        assert np.array_equal(fast[inf_rows][~nan], want[inf_rows][~nan]), "where it is not NaN it is the reference's infinity"
+        assert np.isfinite(fast[finite]).all()
+        np.testing.assert_allclose(fast[finite], want[finite], rtol=1e-4, atol=1e-4)
+
+
+def test_default_session_runs_a_masked_attention_block_as_the_three_operators(case):
+    """MatMul -> Div -> Add(mask) -> Softmax -> MatMul with 64-wide heads: a session built with no switches gives,
+    bit for bit, what the session that copies everything and runs every operator on its own gives, and matches
+    the oracle's three operators at the MatMul tolerance.  Opting in to the one-kernel attention changes the
+    result by its documented 2e-4 relative and nothing more."""
+    case("default session: masked attention block")
+    rng = np.random.default_rng(12)
+    b, h, tq, tk, d = 2, 3, 50, 70, 64
+    q, k, v = (rng.standard_normal((b, h, t, d)).astype(np.float32) for t in (tq, tk, tk))
+    mask = np.where(rng.random((b, 1, 1, tk)) < 0.2, np.float32(-1e4), np.float32(0)).astype(np.float32)
+
+    def build():
+        m = Model(opset_version=13)
+        ins = [m.new_val_named_and_shaped(nm, list(x.shape)) for nm, x in (("q", q), ("k", k), ("v", v))]
+        for i in ins:
+            m.add_input(i)
+        kt, s, s2, s3, p, o = (m.new_val() for _ in range(6))
+        m.add_node(Op.Transpose, [ins[1]], [kt], perm=[0, 1, 3, 2])
+        m.add_node(Op.MatMul, [ins[0], kt], [s])
+        m.add_node(Op.Div, [s, m.new_initializer(np.array(8.0, np.float32))], [s2])
+        m.add_node(Op.Add, [s2, m.new_initializer(mask)], [s3])
+        m.add_node(Op.Softmax, [s3], [p], axis=-1)
+        m.add_node(Op.MatMul, [p, ins[2]], [o])
+        m.add_output(o)
+        m.fuse_softmax_prologue()
+        m.fuse_transpose_matmul()
+        return m
+
+    feeds = [q, k, v]
+    (default,) = HipSessionBuilder(build()).build().run(feeds)
+    (separate,) = HipSessionBuilder(build()).with_strided_views(False).build().run(feeds)
+    assert_bits_equal(default, separate, "default session vs every operator on its own")
+
+    s = O.binary(O.ADD, O.binary(O.DIV, O.matmul(q, np.ascontiguousarray(k.transpose(0, 1, 3, 2))), np.float32(8.0)), mask)
+    want = O.matmul(O.softmax(s), v)
+    assert_close(default, want, rtol=1e-4, atol=1e-5, what="default session vs the oracle's three operators")
+
+    sess = HipSessionBuilder(build()).with_fused_attention().build()
+    (fused,) = sess.run(feeds)
+    assert sess.copies_avoided() == 2  # the first product and the Softmax went into the attention kernel
+    assert not np.array_equal(fused, default)
+    np.testing.assert_allclose(fused, default, rtol=2e-4, atol=2e-5)

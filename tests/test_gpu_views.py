@@ -14,13 +14,14 @@ pytestmark = pytest.mark.gpu
 RNG = np.random.default_rng(2025)
 
 
-def run_both(model, feeds, exact=True):
-    """Outputs with views and with copies, and how many nodes the first run served without a copy.  exact=False
-    where the one-kernel attention replaces three operators (other summation orders: 2e-4 relative)."""
+def run_both(model, feeds, exact=True, attention=False):
+    """Outputs with views and with copies, and how many nodes the first run served without a copy.  attention=True
+    opts in to the one-kernel attention, and exact=False goes with it where that kernel replaces three operators
+    (other summation orders: 2e-4 relative)."""
     outs = []
     avoided = 0
     for views in (True, False):
-        sess = HipSessionBuilder(model.clone()).with_strided_views(views).build()
+        sess = HipSessionBuilder(model.clone()).with_strided_views(views).with_fused_attention(attention and views).build()
         for _ in range(2):  # the second run reuses pooled blocks: a stale view would show
             got = [np.array(t) for t in sess.run([Tensor.from_numpy(x) for x in feeds])]
         if views:
@@ -82,10 +83,14 @@ def test_attention_reads_and_writes_heads_in_place(case, batch, tokens, heads, d
     case(f"attention views b={batch} t={tokens} h={heads} d={d} fold_kt={fold_kt}")
     m, w = attention(batch, tokens, heads, d, fold_kt)
     x = (RNG.standard_normal((batch, tokens, 3 * heads * d)) * 0.3).astype(np.float32)
-    fused = d == 64     # the one-kernel attention takes 64-wide heads
-    (got,), avoided = run_both(m, [x], exact=not fused)
-    # Split, three head transposes, (the K^T transpose unless folded,) and the merge transpose behind P V;
-    # with the one-kernel attention also the first product and the Softmax
+    # A default session: views, three operators.  Split, three head transposes, (the K^T transpose unless folded,)
+    # and the merge transpose behind P V are not copied, and not a bit changes.
+    (got,), avoided = run_both(m, [x], exact=True)
+    assert avoided == (5 if fold_kt else 6), avoided
+    np.testing.assert_allclose(got, attention_numpy(x, heads, d, w), rtol=2e-4, atol=2e-5)
+    # Opted in to the one-kernel attention (it takes 64-wide heads): also the first product and the Softmax.
+    fused = d == 64
+    (got,), avoided = run_both(m, [x], exact=not fused, attention=True)
     assert avoided == (5 if fold_kt else 6) + (2 if fused else 0), avoided
     np.testing.assert_allclose(got, attention_numpy(x, heads, d, w), rtol=2e-4, atol=2e-5)
 
@@ -296,7 +301,7 @@ def test_gemm_activated_through_the_c_abi(ctx, case):
             got = ctx.download(dc, (m, n))
             assert_bits_equal(got, ctx.matmul(ctx.unary(op, a), b), f"op {op}")
     finally:
-        ctx.gemm_set_algorithm(D.GEMM_AUTO)
+        ctx.gemm_set_algorithm(D.GEMM_DEFAULT)
         for x in (da, db, dc):
             ctx.free(x)
 
@@ -377,7 +382,7 @@ def test_gemm_post_through_the_c_abi(ctx, case, m, k, n):
             check(ctx.L.ahip_gemm_post(ctx.handle, dc.ptr, da.ptr, db.ptr, None, m, n, k, 0, 0, k, n, n, 0, 0, 1.0, 0.0, D.SIGMOID, None), ctx.handle)
         assert e.value.code == ERR_ARG
     finally:
-        ctx.gemm_set_algorithm(D.GEMM_AUTO)
+        ctx.gemm_set_algorithm(D.GEMM_DEFAULT)
         for x in (da, db, dbias, dres, dc):
             ctx.free(x)
 
@@ -418,7 +423,7 @@ def test_attention_triple_becomes_one_kernel(case, batch, tq, tk, heads, scale_k
     case(f"session attention b={batch} tq={tq} tk={tk} h={heads} scale={scale_kind}")
     m = scaled_attention(batch, tq, tk, heads, 64, scale_kind)
     q, k, v = (RNG.standard_normal((batch, heads, t, 64)).astype(np.float32) for t in (tq, tk, tk))
-    (got,), avoided = run_both(m, [q, k, v], exact=False)
+    (got,), avoided = run_both(m, [q, k, v], exact=False, attention=True)
     assert avoided == 2, avoided            # the first product and the Softmax
     s = q.astype(np.float64) @ k.astype(np.float64).transpose(0, 1, 3, 2)
     s = s * np.float32(64 ** -0.5) if scale_kind == "mul" else s / np.float32(8.0) if scale_kind == "div" else s
@@ -433,7 +438,7 @@ def test_attention_with_a_per_key_mask(case, mask):
     batch, tq, tk, heads = 3, 37, 50, 2
     m = scaled_attention(batch, tq, tk, heads, 64, "div", mask=mask)
     q, k, v = (RNG.standard_normal((batch, heads, t, 64)).astype(np.float32) for t in (tq, tk, tk))
-    (got,), avoided = run_both(m, [q, k, v], exact=False)
+    (got,), avoided = run_both(m, [q, k, v], exact=False, attention=True)
     assert avoided == 2, avoided
     s = q.astype(np.float64) @ k.astype(np.float64).transpose(0, 1, 3, 2) / np.float32(8.0) + m.mask_values
     e = np.exp(s - s.max(-1, keepdims=True))
@@ -452,5 +457,5 @@ def test_attention_triples_that_stay_three_operators(case, why):
         kw["mask"] = "queries"    # found only when the Softmax runs: the deferred first product is computed after all
     m = scaled_attention(**kw)
     q, k, v = (RNG.standard_normal((kw["batch"], kw["heads"], t, kw["d"])).astype(np.float32) for t in (kw["tq"], kw["tk"], kw["tk"]))
-    outs, avoided = run_both(m, [q, k, v])          # bit for bit: nothing may have changed
+    outs, avoided = run_both(m, [q, k, v], attention=True)          # bit for bit: nothing may have changed
     assert avoided == 0, avoided

@@ -35,6 +35,42 @@ def test_no_cpu_fallback_when_library_is_missing(monkeypatch, tmp_path):
         _lib.lib()
 
 
+def test_in_kernel_k_cut_is_allowed_only_on_a_round_robin_placement():
+    """The bf16 GEMM combines the slices of a tile inside one XCD's L2 only if the probe launch showed blocks 0..7
+    on eight different XCDs, every block i where block i % 8 ran, and a CU count that is a multiple of eight;
+    anything else switches the cut off.  Where the turn starts does not matter (on the part it starts where the
+    queue's previous launch stopped)."""
+    ids = np.arange(4096, dtype=np.uint32)
+    rr = ids % 8
+    assert D.xcd_round_robin_holds(256, rr)
+    assert D.xcd_round_robin_holds(64, rr[:16])
+    for start in range(1, 8):
+        assert D.xcd_round_robin_holds(256, (ids + start) % 8), start     # the turn may start at any XCD
+    assert D.xcd_round_robin_holds(256, np.array([3, 1, 4, 0, 5, 7, 2, 6], np.uint32)[ids % 8])  # any fixed order of the eight
+    assert not D.xcd_round_robin_holds(256, rr[:8])          # one round of eight says nothing
+    assert not D.xcd_round_robin_holds(256, [])
+    for cus in (0, 4, 7, 250, 255, 257, 300, -8):             # not eight equal XCDs
+        assert not D.xcd_round_robin_holds(cus, rr), cus
+    one_off = rr.copy()
+    one_off[4095] = 0                                         # a single misplaced block, the last one
+    assert not D.xcd_round_robin_holds(256, one_off)
+    one_off = rr.copy()
+    one_off[9] = 2
+    assert not D.xcd_round_robin_holds(256, one_off)
+    assert not D.xcd_round_robin_holds(256, np.zeros(4096, np.uint32))   # one XCD for everything
+    assert not D.xcd_round_robin_holds(256, ids // 512)                  # contiguous runs per XCD
+    assert not D.xcd_round_robin_holds(256, ids % 4)                     # four XCDs
+    assert not D.xcd_round_robin_holds(256, ids % 16)                    # ids no eight-XCD part has
+    drift = (ids + ids // 1000) % 8                                      # the turn slips by one every 1000 blocks
+    assert not D.xcd_round_robin_holds(256, drift)
+    never_ran = rr.copy()
+    never_ran[100] = 0xFFFFFFFF                               # the probe's fill value: that block wrote nothing
+    assert not D.xcd_round_robin_holds(256, never_ran)
+    never_ran = rr.copy()
+    never_ran[3] = 0xFFFFFFFF
+    assert not D.xcd_round_robin_holds(256, never_ran)
+
+
 def test_broadcast_reference_unit_tests():
     """crates/core/src/fixed_dim.rs:192-245."""
     assert D.broadcast_shape([1], [1]) == [1]
