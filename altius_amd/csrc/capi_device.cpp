@@ -325,6 +325,12 @@ int ahip_reduce(ahip_ctx *ctx, int kind, float *out, const float *in, size_t out
     return altius::launch_reduce(ctx->d, kind, out, in, outer, reduce, inner);
 }
 
+int ahip_set_streaming_threshold(ahip_ctx *ctx, size_t bytes) {
+    REQUIRE_CTX(ctx, "ahip_set_streaming_threshold");
+    ctx->d.nt_threshold_bytes = bytes;
+    return AHIP_OK;
+}
+
 int ahip_xcd_round_robin_holds(int cu_count, const uint32_t *xcc_of_block, size_t n_blocks) {
     return altius::xcd_round_robin_holds(cu_count, xcc_of_block, n_blocks) ? 1 : 0;
 }

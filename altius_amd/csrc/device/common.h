@@ -76,12 +76,23 @@ template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
 }
 constexpr int DPP_ROW_ROR = 0x120;  // + n: rotate right by n lanes within a row of 16
 
-// All-reduce over aligned groups of SUB lanes (SUB = 16, 32 or 64); every lane
+constexpr int DPP_QUAD_XOR1 = 0xB1;     // quad_perm [1,0,3,2]: lane ^ 1
+constexpr int DPP_QUAD_XOR2 = 0x4E;     // quad_perm [2,3,0,1]: lane ^ 2
+constexpr int DPP_ROW_HALF_MIRROR = 0x141;  // lane i of each group of 8 reads lane 7 - i
+
+// All-reduce over aligned groups of SUB lanes (SUB = 4, 8, 16, 32 or 64); every lane
 // ends with the result of its group.  Rotation and exchange steps combine the
 // same two partial results in every lane of a pair and OP is commutative, so all
 // lanes of a group hold bit-identical values.
 template <class OP, int SUB> __device__ __forceinline__ float subwave_allreduce(float v) {
-    static_assert(SUB == 16 || SUB == 32 || SUB == 64, "group size");
+    static_assert(SUB == 4 || SUB == 8 || SUB == 16 || SUB == 32 || SUB == 64, "group size");
+    if (SUB <= 8) {
+        v = OP::apply(v, dpp_move<DPP_QUAD_XOR1>(v));
+        v = OP::apply(v, dpp_move<DPP_QUAD_XOR2>(v));
+        // every lane of a quad now holds the quad's result, so the mirror image is the other quad's
+        if (SUB == 8) v = OP::apply(v, dpp_move<DPP_ROW_HALF_MIRROR>(v));
+        return v;
+    }
     v = OP::apply(v, dpp_move<DPP_ROW_ROR + 8>(v));
     v = OP::apply(v, dpp_move<DPP_ROW_ROR + 4>(v));
     v = OP::apply(v, dpp_move<DPP_ROW_ROR + 2>(v));

@@ -294,11 +294,15 @@ __global__ __launch_bounds__(LDS_BLOCK) void softmax_lds(float *__restrict__ out
     for (int i = (n4 << 2) + tid; i < n; i += LDS_BLOCK) dst[i] = lds[i];
 }
 
-// LayerNormalization of short rows (under 160 elements), where a wavefront per row leaves most lanes idle: the same
-// staging as softmax_lds (a line-aligned group of rows through LDS, 16-byte global accesses), SUB lanes per row, three
-// walks over the row in LDS (sum, squared deviations, result), scale and bias staged in LDS once per block.
-template <int SUB, bool NT>
-__global__ __launch_bounds__(LDS_BLOCK) void layernorm_lds(float *__restrict__ out, const float *__restrict__ in,
+// LayerNormalization of rows that a wavefront per row with 16-byte accesses does not fit (not whole float4s, or
+// short): the same staging as softmax_lds (a line-aligned group of rows through LDS, 16-byte global accesses), SUB
+// lanes per row with the row in NCH registers per lane, read from LDS once and written back once.  A lane works on
+// the same columns of every row it meets, so its scale and bias values are read once per block (from LDS, where they
+// are staged with coalesced loads).
+// Two blocks of sixteen wavefronts share a CU (one loads or stores while the other computes), which leaves each lane
+// 64 registers: the second launch bound says so to the register allocator.
+template <int SUB, int NCH, bool NT>
+__global__ __launch_bounds__(LDS_BLOCK, 8) void layernorm_lds(float *__restrict__ out, const float *__restrict__ in,
                                                            const float *__restrict__ gamma, const float *__restrict__ beta, size_t rows,
                                                            int len, int group_rows, float eps) {
     extern __shared__ __align__(16) float lds[];
@@ -321,6 +325,13 @@ __global__ __launch_bounds__(LDS_BLOCK) void layernorm_lds(float *__restrict__ o
             if (tid + LDS_BLOCK * u < n4) stage[u] = load4<NT>(p);
         }
     }
+    constexpr int RPP = WAVE / SUB;  // rows per wave pass
+    constexpr int LAST = NCH - 1;    // NCH == ceil(len / SUB): only the last chunk can be partial
+    const int s = lane & (SUB - 1);
+    const int rr = lane / SUB;
+    const bool last_valid = s + SUB * LAST < len;
+    // Scale and bias go to LDS behind the rows with coalesced loads, once per block, and from there into each
+    // lane's registers.
     float *g_lds = lds + (size_t)group_rows * len, *b_lds = g_lds + len;
     for (int i = tid; i < len; i += LDS_BLOCK) g_lds[i] = gamma[i], b_lds[i] = beta[i];
 #pragma unroll
@@ -335,25 +346,50 @@ __global__ __launch_bounds__(LDS_BLOCK) void layernorm_lds(float *__restrict__ o
     for (int i = (n4 << 2) + tid; i < n; i += LDS_BLOCK) lds[i] = src[i];  // ragged end of the last group
     __syncthreads();
 
-    constexpr int RPP = WAVE / SUB;  // rows per wave pass
-    const int s = lane & (SUB - 1);
-    const int rr = lane / SUB;
+    // Up to 10 chunks the lane's scale and bias values stay in registers for all of its rows; beyond that they would
+    // not fit beside the row (64 registers per lane) and are read from LDS where they are used.
+    constexpr bool GB_REGS = NCH <= 10;
+    constexpr int NGB = GB_REGS ? NCH : 1;
+    float g[NGB], b[NGB];
+    if (GB_REGS) {
+#pragma unroll
+        for (int k = 0; k < NGB; k++) {
+            const bool valid = k < LAST || last_valid;
+            g[k] = valid ? g_lds[s + SUB * k] : 0.0f;
+            b[k] = valid ? b_lds[s + SUB * k] : 0.0f;
+        }
+    }
     const float inv_n = 1.0f / (float)len;
     for (int r0 = wave * RPP; r0 < nrows; r0 += LDS_WAVES * RPP) {
-        const bool mine = r0 + rr < nrows;  // lane groups past the end walk the last row along and write nothing
-        float *row = lds + (mine ? r0 + rr : nrows - 1) * len;
+        // Lane groups past the end of a ragged last group redo its last row: they compute and store the same
+        // values as the group that owns it.
+        const int r = r0 + rr < nrows ? r0 + rr : nrows - 1;
+        float *row = lds + r * len + s;
+        float x[NCH];
+#pragma unroll
+        for (int k = 0; k < LAST; k++) x[k] = row[SUB * k];
+        x[LAST] = last_valid ? row[SUB * LAST] : 0.0f;
         float sum = 0.0f;
-        for (int k = s; k < len; k += SUB) sum += row[k];
+#pragma unroll
+        for (int k = 0; k < NCH; k++) sum += x[k];
         const float mean = subwave_allreduce<SumOp, SUB>(sum) * inv_n;
         float ss = 0.0f;
-        for (int k = s; k < len; k += SUB) {
-            const float d = row[k] - mean;
-            ss += d * d;
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            x[k] = x[k] - mean;
+            const float d2 = x[k] * x[k];
+            ss += (k < LAST || last_valid) ? d2 : 0.0f;
         }
         ss = subwave_allreduce<SumOp, SUB>(ss);
         const float inv_std = 1.0f / sqrtf(__builtin_fmaf(ss, inv_n, eps));
-        if (mine)
-            for (int k = s; k < len; k += SUB) row[k] = __builtin_fmaf((row[k] - mean) * inv_std, g_lds[k], b_lds[k]);
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            if (k < LAST || last_valid) {
+                const float gk = GB_REGS ? g[GB_REGS ? k : 0] : g_lds[s + SUB * k];
+                const float bk = GB_REGS ? b[GB_REGS ? k : 0] : b_lds[s + SUB * k];
+                row[SUB * k] = __builtin_fmaf(x[k] * inv_std, gk, bk);
+            }
+        }
     }
     __syncthreads();
 
@@ -533,70 +569,84 @@ __global__ __launch_bounds__(BLOCK) void layernorm_block_stream(float *__restric
         o[i] = __builtin_fmaf((x[i] - mean) * inv_std, gamma[i], beta[i]);
 }
 
-// Rows of 4097 to 16384 elements that are whole float4s (hidden sizes 5120, 8192; 16 K): a block per row with the
-// row in registers (8 or 16 float4 per thread), read once; the two reductions go through LDS.
-template <int NCH, bool NT>
-__global__ __launch_bounds__(BLOCK) void softmax_block_regs(float *__restrict__ out, const float *__restrict__ in, size_t len) {
-    __shared__ float lds[WAVES_PER_BLOCK];
+// Long rows that are whole float4s: a block of THREADS threads per row with the row in registers (NCH float4 per
+// thread, read once); the two reductions go through LDS.  Few loads per thread and many threads per row: on this
+// part a wavefront that issues many 16-byte loads back to back streams more slowly than many wavefronts issuing a
+// few each.
+template <int THREADS, int NCH, bool NT>
+__global__ __launch_bounds__(THREADS) void softmax_block_regs(float *__restrict__ out, const float *__restrict__ in, size_t len) {
+    __shared__ float lds[THREADS / WAVE];
     const float *x = in + (size_t)blockIdx.x * len;
     float *o = out + (size_t)blockIdx.x * len;
     const float nan = __builtin_nanf("");
     float4 r[NCH];
-#pragma unroll
-    for (int k = 0; k < NCH; k++) {
-        const size_t e = ((size_t)threadIdx.x + (size_t)BLOCK * k) * 4;
-        r[k] = e < len ? load4<NT>(x + e) : make_float4(nan, nan, nan, nan);
-    }
     float mx = nan;  // NaN elements (and the slots past the row) are ignored by the maximum
+    // At most two 16-byte loads per thread are requested at a time; with four chunks the second pair goes out
+    // once the first has been folded into the maximum.
+    constexpr int BURST = NCH >= 4 && NCH % 2 == 0 ? NCH / 2 : NCH;
 #pragma unroll
-    for (int k = 0; k < NCH; k++) mx = nanmax(nanmax(r[k].x, r[k].y), nanmax(nanmax(r[k].z, r[k].w), mx));
-    mx = block_reduce<MaxOp, WAVES_PER_BLOCK>(mx, lds);
+    for (int k0 = 0; k0 < NCH; k0 += BURST) {
+#pragma unroll
+        for (int k = k0; k < k0 + BURST; k++) {
+            const size_t e = ((size_t)threadIdx.x + (size_t)THREADS * k) * 4;
+            r[k] = e < len ? load4<NT>(x + e) : make_float4(nan, nan, nan, nan);
+        }
+#pragma unroll
+        for (int k = k0; k < k0 + BURST; k++) mx = nanmax(nanmax(r[k].x, r[k].y), nanmax(nanmax(r[k].z, r[k].w), mx));
+        if (BURST != NCH) asm volatile("" ::: "memory");
+    }
+    mx = block_reduce<MaxOp, THREADS / WAVE>(mx, lds);
     float sum = 0.0f;
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        const bool valid = ((size_t)threadIdx.x + (size_t)BLOCK * k) * 4 < len;
+        const bool valid = ((size_t)threadIdx.x + (size_t)THREADS * k) * 4 < len;
         r[k].x = softmax_exp(r[k].x, mx), r[k].y = softmax_exp(r[k].y, mx), r[k].z = softmax_exp(r[k].z, mx), r[k].w = softmax_exp(r[k].w, mx);
         if (valid) sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
     }
-    sum = block_reduce<SumOp, WAVES_PER_BLOCK>(sum, lds);
+    sum = block_reduce<SumOp, THREADS / WAVE>(sum, lds);
     const float recip = 1.0f / sum;
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        const size_t e = ((size_t)threadIdx.x + (size_t)BLOCK * k) * 4;
+        const size_t e = ((size_t)threadIdx.x + (size_t)THREADS * k) * 4;
         if (e < len) store4<NT>(o + e, make_float4(r[k].x * recip, r[k].y * recip, r[k].z * recip, r[k].w * recip));
     }
 }
 
-template <int NCH, bool NT>
-__global__ __launch_bounds__(BLOCK) void layernorm_block_regs(float *__restrict__ out, const float *__restrict__ in,
-                                                              const float *__restrict__ gamma, const float *__restrict__ beta, size_t len,
-                                                              float eps) {
-    __shared__ float lds[WAVES_PER_BLOCK];
+template <int THREADS, int NCH, bool NT>
+__global__ __launch_bounds__(THREADS) void layernorm_block_regs(float *__restrict__ out, const float *__restrict__ in,
+                                                                const float *__restrict__ gamma, const float *__restrict__ beta, size_t len,
+                                                                float eps) {
+    __shared__ float lds[THREADS / WAVE];
     const float *x = in + (size_t)blockIdx.x * len;
     float *o = out + (size_t)blockIdx.x * len;
     const float inv_n = 1.0f / (float)len;
     float4 r[NCH];
     float sum = 0.0f;
+    constexpr int BURST = NCH >= 4 && NCH % 2 == 0 ? NCH / 2 : NCH;  // see softmax_block_regs
 #pragma unroll
-    for (int k = 0; k < NCH; k++) {
-        const size_t e = ((size_t)threadIdx.x + (size_t)BLOCK * k) * 4;
-        r[k] = e < len ? load4<NT>(x + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int k0 = 0; k0 < NCH; k0 += BURST) {
+#pragma unroll
+        for (int k = k0; k < k0 + BURST; k++) {
+            const size_t e = ((size_t)threadIdx.x + (size_t)THREADS * k) * 4;
+            r[k] = e < len ? load4<NT>(x + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int k = k0; k < k0 + BURST; k++) sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
+        if (BURST != NCH) asm volatile("" ::: "memory");
     }
-#pragma unroll
-    for (int k = 0; k < NCH; k++) sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
-    const float mean = block_reduce<SumOp, WAVES_PER_BLOCK>(sum, lds) * inv_n;
+    const float mean = block_reduce<SumOp, THREADS / WAVE>(sum, lds) * inv_n;
     float ss = 0.0f;
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        const bool valid = ((size_t)threadIdx.x + (size_t)BLOCK * k) * 4 < len;
+        const bool valid = ((size_t)threadIdx.x + (size_t)THREADS * k) * 4 < len;
         r[k].x -= mean, r[k].y -= mean, r[k].z -= mean, r[k].w -= mean;
         if (valid) ss += (r[k].x * r[k].x + r[k].y * r[k].y) + (r[k].z * r[k].z + r[k].w * r[k].w);
     }
-    ss = block_reduce<SumOp, WAVES_PER_BLOCK>(ss, lds);
+    ss = block_reduce<SumOp, THREADS / WAVE>(ss, lds);
     const float inv_std = 1.0f / sqrtf(__builtin_fmaf(ss, inv_n, eps));
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        const size_t e = ((size_t)threadIdx.x + (size_t)BLOCK * k) * 4;
+        const size_t e = ((size_t)threadIdx.x + (size_t)THREADS * k) * 4;
         if (e < len) {
             const float4 g = *reinterpret_cast<const float4 *>(gamma + e), b = *reinterpret_cast<const float4 *>(beta + e);
             store4<NT>(o + e, make_float4(__builtin_fmaf(r[k].x * inv_std, g.x, b.x), __builtin_fmaf(r[k].y * inv_std, g.y, b.y),
@@ -604,6 +654,38 @@ __global__ __launch_bounds__(BLOCK) void layernorm_block_regs(float *__restrict_
         }
     }
 }
+
+// Threads per row and float4 per thread for a row of `len` elements in the block-per-row kernels.
+struct BlockLayout {
+    int threads, nch;
+};
+// Measured over rows of 2048 to 16384 elements: two float4 per thread is the best shape (256 x 2 for 2048, 512 x 2
+// for 4096, 1024 x 2 for 8192: 77-80 % of peak for Softmax), three cost little, and a 16 K row has to take four
+// (requested two at a time).
+inline BlockLayout block_layout(size_t len) {
+    const size_t v = len / 4;  // float4 per row
+    const int threads = v <= 512 ? 256 : v <= 1536 ? 512 : 1024;
+    return BlockLayout{threads, (int)((v + threads - 1) / threads)};
+}
+
+template <int THREADS, int NCH>
+void softmax_block_go(bool nt, hipStream_t s, size_t rows, float *out, const float *in, size_t len) {
+    const dim3 grid((unsigned)rows);
+    if (nt) hipLaunchKernelGGL((softmax_block_regs<THREADS, NCH, true>), grid, dim3(THREADS), 0, s, out, in, len);
+    else hipLaunchKernelGGL((softmax_block_regs<THREADS, NCH, false>), grid, dim3(THREADS), 0, s, out, in, len);
+}
+template <int THREADS, int NCH>
+void layernorm_block_go(bool nt, hipStream_t s, size_t rows, float *out, const float *in, const float *gamma, const float *beta, size_t len,
+                        float eps) {
+    const dim3 grid((unsigned)rows);
+    if (nt) hipLaunchKernelGGL((layernorm_block_regs<THREADS, NCH, true>), grid, dim3(THREADS), 0, s, out, in, gamma, beta, len, eps);
+    else hipLaunchKernelGGL((layernorm_block_regs<THREADS, NCH, false>), grid, dim3(THREADS), 0, s, out, in, gamma, beta, len, eps);
+}
+// GO(THREADS, NCH) for the layout of a row; false if there is none.
+#define ALTIUS_BLOCK_LAYOUTS(L)                                                          \
+    switch ((L).threads * 100 + (L).nch) {                                               \
+        ALTIUS_GO(256, 2) ALTIUS_GO(512, 2) ALTIUS_GO(512, 3) ALTIUS_GO(1024, 2) ALTIUS_GO(1024, 3) ALTIUS_GO(1024, 4) \
+    }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -631,15 +713,12 @@ bool dispatch_wave(bool vec4, size_t len, Args... args) {
     return false;
 }
 
-// Rows of 1025 to 4096 elements that are whole float4s: still a wavefront per row with the row in registers
-// (6, 8, 12 or 16 float4 per lane), read once.
+// Rows of 1025 to 1536 elements that are whole float4s: still a wavefront per row with the row in registers
+// (6 float4 per lane), read once.
 template <template <int, int> class Launcher, class... Args>
 bool dispatch_wave_long(size_t len, Args... args) {
     const size_t chunks = (len / 4 + WAVE - 1) / WAVE;
     if (chunks <= 6) { Launcher<4, 6>::go(args...); return true; }
-    if (chunks <= 8) { Launcher<4, 8>::go(args...); return true; }
-    if (chunks <= 12) { Launcher<4, 12>::go(args...); return true; }
-    if (chunks <= 16) { Launcher<4, 16>::go(args...); return true; }
     return false;
 }
 
@@ -714,6 +793,41 @@ size_t softmax_lds_group_rows(size_t len) {
     return 4;  // unreachable for len <= 1024: 4 rows are at most 4096 floats
 }
 
+// Lanes per row and chunks per lane for a row of L <= 1024 elements in the LDS-staged kernels: the narrowest lane
+// group that covers the row in at most 16 chunks.  Narrow groups mean more rows per wavefront pass, and the work a
+// pass does once per row group (the two all-reduces, the division, the loop) is shared by more rows: 4 lanes up to
+// 64 elements (unless the length is a multiple of 8: the sixteen rows of a pass would then meet in the same LDS
+// banks), 8 up to 128, 16 up to 256, 32 up to 512, 64 above.
+#define ALTIUS_LDS_LAYOUTS(L)                                                                                       \
+    if ((L) <= 64 && (L) % 8 != 0) {                                                                                \
+        switch (((L) + 3) / 4) {                                                                                    \
+            ALTIUS_GO(4, 1) ALTIUS_GO(4, 2) ALTIUS_GO(4, 3) ALTIUS_GO(4, 4) ALTIUS_GO(4, 5) ALTIUS_GO(4, 6)         \
+            ALTIUS_GO(4, 7) ALTIUS_GO(4, 8) ALTIUS_GO(4, 9) ALTIUS_GO(4, 10) ALTIUS_GO(4, 11) ALTIUS_GO(4, 12)      \
+            ALTIUS_GO(4, 13) ALTIUS_GO(4, 14) ALTIUS_GO(4, 15) ALTIUS_GO(4, 16)                                     \
+        }                                                                                                           \
+    } else if ((L) <= 128) {                                                                                               \
+        switch (((L) + 7) / 8) {                                                                                    \
+            ALTIUS_GO(8, 1) ALTIUS_GO(8, 2) ALTIUS_GO(8, 3) ALTIUS_GO(8, 4) ALTIUS_GO(8, 5) ALTIUS_GO(8, 6)         \
+            ALTIUS_GO(8, 7) ALTIUS_GO(8, 8) ALTIUS_GO(8, 9) ALTIUS_GO(8, 10) ALTIUS_GO(8, 11) ALTIUS_GO(8, 12)      \
+            ALTIUS_GO(8, 13) ALTIUS_GO(8, 14) ALTIUS_GO(8, 15) ALTIUS_GO(8, 16)                                     \
+        }                                                                                                           \
+    } else if ((L) <= 256) {                                                                                        \
+        switch (((L) + 15) / 16) {                                                                                  \
+            ALTIUS_GO(16, 9) ALTIUS_GO(16, 10) ALTIUS_GO(16, 11) ALTIUS_GO(16, 12) ALTIUS_GO(16, 13)                \
+            ALTIUS_GO(16, 14) ALTIUS_GO(16, 15) ALTIUS_GO(16, 16)                                                   \
+        }                                                                                                           \
+    } else if ((L) <= 512) {                                                                                        \
+        switch (((L) + 31) / 32) {                                                                                  \
+            ALTIUS_GO(32, 9) ALTIUS_GO(32, 10) ALTIUS_GO(32, 11) ALTIUS_GO(32, 12) ALTIUS_GO(32, 13)                \
+            ALTIUS_GO(32, 14) ALTIUS_GO(32, 15) ALTIUS_GO(32, 16)                                                   \
+        }                                                                                                           \
+    } else {                                                                                                        \
+        switch (((L) + 63) / 64) {                                                                                  \
+            ALTIUS_GO(64, 9) ALTIUS_GO(64, 10) ALTIUS_GO(64, 11) ALTIUS_GO(64, 12) ALTIUS_GO(64, 13)                \
+            ALTIUS_GO(64, 14) ALTIUS_GO(64, 15) ALTIUS_GO(64, 16)                                                   \
+        }                                                                                                           \
+    }
+
 bool softmax_lds_launch(hipStream_t s, float *out, const float *in, size_t rows, size_t len, bool nt,
                         const SoftmaxPrologue *pro = nullptr) {
     static_assert(4 * 1024 <= LDS_GROUP_FLOATS, "four rows of the longest supported length must fit");
@@ -735,29 +849,37 @@ bool softmax_lds_launch(hipStream_t s, float *out, const float *in, size_t rows,
     case N:                                                                  \
         softmax_lds_go<SUB, N>(nt, grid, shmem, s, out, in, rows, L, G, pro); \
         return true;
-    if (len <= 256) {
-        switch ((L + 15) / 16) {
-            ALTIUS_GO(16, 1) ALTIUS_GO(16, 2) ALTIUS_GO(16, 3) ALTIUS_GO(16, 4) ALTIUS_GO(16, 5) ALTIUS_GO(16, 6)
-            ALTIUS_GO(16, 7) ALTIUS_GO(16, 8) ALTIUS_GO(16, 9) ALTIUS_GO(16, 10) ALTIUS_GO(16, 11)
-            ALTIUS_GO(16, 12) ALTIUS_GO(16, 13) ALTIUS_GO(16, 14) ALTIUS_GO(16, 15) ALTIUS_GO(16, 16)
-        }
-    } else if (len <= 512) {
-        switch ((L + 31) / 32) {
-            ALTIUS_GO(32, 9) ALTIUS_GO(32, 10) ALTIUS_GO(32, 11) ALTIUS_GO(32, 12) ALTIUS_GO(32, 13)
-            ALTIUS_GO(32, 14) ALTIUS_GO(32, 15) ALTIUS_GO(32, 16)
-        }
-    } else {
-        switch ((L + 63) / 64) {
-            ALTIUS_GO(64, 9) ALTIUS_GO(64, 10) ALTIUS_GO(64, 11) ALTIUS_GO(64, 12) ALTIUS_GO(64, 13)
-            ALTIUS_GO(64, 14) ALTIUS_GO(64, 15) ALTIUS_GO(64, 16)
-        }
-    }
+    ALTIUS_LDS_LAYOUTS(L)
+#undef ALTIUS_GO
+    return false;
+}
+
+template <int SUB, int NCH>
+void layernorm_lds_go(bool nt, dim3 grid, size_t shmem, hipStream_t s, float *out, const float *in, const float *gamma, const float *beta,
+                      size_t rows, int len, int g, float eps) {
+    if (nt) hipLaunchKernelGGL((layernorm_lds<SUB, NCH, true>), grid, dim3(LDS_BLOCK), shmem, s, out, in, gamma, beta, rows, len, g, eps);
+    else hipLaunchKernelGGL((layernorm_lds<SUB, NCH, false>), grid, dim3(LDS_BLOCK), shmem, s, out, in, gamma, beta, rows, len, g, eps);
+}
+
+bool layernorm_lds_launch(hipStream_t s, float *out, const float *in, const float *gamma, const float *beta, size_t rows, size_t len, float eps,
+                          bool nt) {
+    const size_t g = softmax_lds_group_rows(len);
+    const size_t groups = (rows + g - 1) / g;
+    if ((g * len) % 4 != 0 || groups > 0x7FFFFFFFu) return false;
+    const dim3 grid((unsigned)groups);
+    const size_t shmem = (g * len + 2 * len) * sizeof(float);
+    const int L = (int)len, G = (int)g;
+#define ALTIUS_GO(SUB, N)                                                                     \
+    case N:                                                                                   \
+        layernorm_lds_go<SUB, N>(nt, grid, shmem, s, out, in, gamma, beta, rows, L, G, eps);   \
+        return true;
+    ALTIUS_LDS_LAYOUTS(L)
 #undef ALTIUS_GO
     return false;
 }
 
 constexpr size_t MAX_WAVE_ROW = 1024;
-constexpr size_t MAX_LONG_ROW = 4096;  // rows kept in a wavefront's registers when they are whole float4s
+constexpr size_t MAX_LONG_ROW = 1536;  // rows kept in a wavefront's registers when they are whole float4s
 constexpr size_t MAX_BLOCK_REG_ROW = 16384;  // ... and in a block's registers
 constexpr size_t MAX_GRID = 0x7FFFFFFFu;
 
@@ -788,14 +910,16 @@ int launch_softmax(DeviceCtx &ctx, float *out, const float *in, size_t rows, siz
                                             ctx.streaming(rows * len * sizeof(float)));
     } else if (len <= MAX_BLOCK_REG_ROW && len % 4 == 0 && aligned16(out) && aligned16(in) && rows <= MAX_GRID) {
         const bool nt = ctx.streaming(rows * len * sizeof(float));
-        const dim3 grid((unsigned)rows);
-        if (len <= 8192) {
-            if (nt) hipLaunchKernelGGL((softmax_block_regs<8, true>), grid, dim3(BLOCK), 0, ctx.stream, out, in, len);
-            else hipLaunchKernelGGL((softmax_block_regs<8, false>), grid, dim3(BLOCK), 0, ctx.stream, out, in, len);
-        } else {
-            if (nt) hipLaunchKernelGGL((softmax_block_regs<16, true>), grid, dim3(BLOCK), 0, ctx.stream, out, in, len);
-            else hipLaunchKernelGGL((softmax_block_regs<16, false>), grid, dim3(BLOCK), 0, ctx.stream, out, in, len);
-        }
+        const BlockLayout lay = block_layout(len);
+        bool launched = false;
+#define ALTIUS_GO(T, N)                                                         \
+    case T * 100 + N:                                                           \
+        softmax_block_go<T, N>(nt, ctx.stream, rows, out, in, len);             \
+        launched = true;                                                        \
+        break;
+        ALTIUS_BLOCK_LAYOUTS(lay)
+#undef ALTIUS_GO
+        if (!launched) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: no block layout for this row length");
     } else {
         if (rows > MAX_GRID) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: too many rows for one launch");
         hipLaunchKernelGGL(softmax_block_stream, dim3((unsigned)rows), dim3(BLOCK), 0, ctx.stream, out, in,
@@ -835,27 +959,13 @@ int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *g
                      size_t rows, size_t len, float eps) {
     if (rows == 0 || len == 0) return AHIP_OK;
     if (!out || !in || !gamma || !beta) return ctx.fail(AHIP_ERR_ARG, "layernorm: null tensor pointer");
-    if (len < 160 && rows >= 64 && aligned16(out) && aligned16(in)) {
-        // Short rows: groups of rows through LDS, 16 or 32 lanes per row (measured ahead of the wavefront-per-row
-        // kernel up to about 160 elements: 58 against 24 % of peak at 49, 68 against 29 % at 64, even at 197).
-        const size_t g = softmax_lds_group_rows(len);
-        const size_t groups = (rows + g - 1) / g;
-        if ((g * len) % 4 == 0 && groups <= MAX_GRID) {
-            const bool nt = ctx.streaming(rows * len * sizeof(float));
-            const dim3 grid((unsigned)groups);
-            const size_t shmem = (g * len + 2 * len) * sizeof(float);
-#define ALTIUS_LN_LDS(SUB, N) \
-    hipLaunchKernelGGL((layernorm_lds<SUB, N>), grid, dim3(LDS_BLOCK), shmem, ctx.stream, out, in, gamma, beta, rows, (int)len, (int)g, eps)
-            if (len <= 128) {
-                if (nt) ALTIUS_LN_LDS(16, true);
-                else ALTIUS_LN_LDS(16, false);
-            } else {
-                if (nt) ALTIUS_LN_LDS(32, true);
-                else ALTIUS_LN_LDS(32, false);
-            }
-#undef ALTIUS_LN_LDS
+    if (len <= MAX_WAVE_ROW && rows >= 64 && aligned16(out) && aligned16(in)) {
+        // Rows that fill (most of) a wavefront's 256-element chunks with whole float4s take the wavefront-per-row
+        // kernel; every other row of up to 1024 elements goes through LDS in line-aligned groups (the rule Softmax uses).
+        const size_t slots = (len + 255) / 256 * 256;
+        const bool wave_fits = len % 32 == 0 && len * 4 >= slots * 3 && aligned16(gamma) && aligned16(beta);
+        if (!wave_fits && layernorm_lds_launch(ctx.stream, out, in, gamma, beta, rows, len, eps, ctx.streaming(rows * len * sizeof(float))))
             return ctx.check(hipGetLastError(), "layernorm (LDS groups) launch");
-        }
     }
     if (len <= MAX_WAVE_ROW) {
         if ((rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK > MAX_GRID)
@@ -872,14 +982,16 @@ int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *g
     } else if (len <= MAX_BLOCK_REG_ROW && len % 4 == 0 && aligned16(out) && aligned16(in) && aligned16(gamma) && aligned16(beta) &&
                rows <= MAX_GRID) {
         const bool nt = ctx.streaming(rows * len * sizeof(float));
-        const dim3 grid((unsigned)rows);
-        if (len <= 8192) {
-            if (nt) hipLaunchKernelGGL((layernorm_block_regs<8, true>), grid, dim3(BLOCK), 0, ctx.stream, out, in, gamma, beta, len, eps);
-            else hipLaunchKernelGGL((layernorm_block_regs<8, false>), grid, dim3(BLOCK), 0, ctx.stream, out, in, gamma, beta, len, eps);
-        } else {
-            if (nt) hipLaunchKernelGGL((layernorm_block_regs<16, true>), grid, dim3(BLOCK), 0, ctx.stream, out, in, gamma, beta, len, eps);
-            else hipLaunchKernelGGL((layernorm_block_regs<16, false>), grid, dim3(BLOCK), 0, ctx.stream, out, in, gamma, beta, len, eps);
-        }
+        const BlockLayout lay = block_layout(len);
+        bool launched = false;
+#define ALTIUS_GO(T, N)                                                                      \
+    case T * 100 + N:                                                                        \
+        layernorm_block_go<T, N>(nt, ctx.stream, rows, out, in, gamma, beta, len, eps);      \
+        launched = true;                                                                     \
+        break;
+        ALTIUS_BLOCK_LAYOUTS(lay)
+#undef ALTIUS_GO
+        if (!launched) return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: no block layout for this row length");
     } else {
         if (rows > MAX_GRID) return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: too many rows for one launch");
         hipLaunchKernelGGL(layernorm_block_stream, dim3((unsigned)rows), dim3(BLOCK), 0, ctx.stream, out, in,
@@ -910,7 +1022,9 @@ int launch_reduce_rows_lds(DeviceCtx &ctx, bool is_max, float *out, const float 
         else if (scaled) ALTIUS_RED(SumOp, SUB, true);        \
         else ALTIUS_RED(SumOp, SUB, false);                   \
     } while (0)
-    if (len <= 256) ALTIUS_RED_SUB(16);
+    if (len <= 64 && len % 8 != 0) ALTIUS_RED_SUB(4);
+    else if (len <= 128) ALTIUS_RED_SUB(8);
+    else if (len <= 256) ALTIUS_RED_SUB(16);
     else if (len <= 512) ALTIUS_RED_SUB(32);
     else ALTIUS_RED_SUB(64);
 #undef ALTIUS_RED_SUB

@@ -451,6 +451,10 @@ class Context:
         """GEMM_AUTO / GEMM_FP32 / GEMM_BF16X3: the kernel single-batch products take."""
         check(self.L.ahip_gemm_set_algorithm(self.handle, int(algorithm)), self.handle)
 
+    def set_streaming_threshold(self, nbytes):
+        """Tensors of at least this many bytes are streamed with non-temporal accesses."""
+        check(self.L.ahip_set_streaming_threshold(self.handle, int(nbytes)), self.handle)
+
     def gemm_in_kernel_k_cut(self):
         """(placement shown, cut enabled): whether the probe at context creation found block i on XCD i % 8, and
         whether the bf16 GEMM's in-kernel k cut is switched on.  The cut runs only when both hold."""

@@ -167,6 +167,49 @@ def build_listed_ops(ctx, D, c, batch, rotate_bytes=900e6):
     return ops
 
 
+ROW_SWEEP_ELEMS = 96 << 20   # 403 MB in, 403 MB out: every launch misses the 256 MB cache
+ROW_SWEEP_LENGTHS = (49, 64, 100, 128, 197, 256, 384, 512, 768, 1000, 1024, 1280, 2048, 3072, 4096, 5120, 8192, 12288, 16384)
+
+
+def build_row_sweep(ctx, D, lengths=ROW_SWEEP_LENGTHS, elems=ROW_SWEEP_ELEMS):
+    """The three row operators of the path on one ~400 MB array cut into rows of every length between a 7 x 7
+    feature map and a 16 K hidden size.  One input and one output buffer serve all lengths."""
+    rng = np.random.default_rng(21)
+    d_in = ctx.upload(rng.standard_normal(elems, dtype=np.float32))
+    d_out = ctx.alloc(elems * 4)
+    longest = max(lengths)
+    d_g = ctx.upload((1.0 + 0.02 * rng.standard_normal(longest)).astype(np.float32))
+    d_b = ctx.upload((0.02 * rng.standard_normal(longest)).astype(np.float32))
+    for length in lengths:
+        rows = elems // length
+        n = rows * length
+        yield length, [
+            Op("Softmax", 2 * n * 4, [lambda rows=rows, length=length: ctx.softmax_raw(d_out.ptr, d_in.ptr, rows, length)]),
+            Op("LayerNormalization", 2 * n * 4 + 2 * length * 4,
+               [lambda rows=rows, length=length: ctx.layernorm_raw(d_out.ptr, d_in.ptr, d_g.ptr, d_b.ptr, rows, length, 1e-5)]),
+            Op("ReduceMean", n * 4 + rows * 4,
+               [lambda rows=rows, length=length: ctx.reduce_raw(D.REDUCE_MEAN, d_out.ptr, d_in.ptr, rows, length, 1)]),
+        ]
+    for b in (d_in, d_out, d_g, d_b):
+        ctx.free(b)
+
+
+def run_row_sweep(ctx, D, args, lengths):
+    sweep = []
+    log("Softmax / LayerNormalization / ReduceMean over the last axis, %d M elements, by row length (%% of 8 TB/s):" % (ROW_SWEEP_ELEMS >> 20))
+    for length, ops_l in build_row_sweep(ctx, D, lengths):
+        entry = {"row_length": length}
+        for o in ops_l:
+            t = time_kernel(ctx, o, args.kernel_iters, args.kernel_warmup)
+            r = t.row(o.nbytes)
+            entry[o.name] = {"bytes": o.nbytes, "us": r["us"], "us_median": r["us_median"], "us_min": r["us_min"], "GBps": r["GBps"],
+                             "pct_hbm_peak": r["pct_hbm_peak"]}
+        sweep.append(entry)
+        log("  rows of %6d: %s" % (length, "   ".join("%s %6.1f us %5.1f %%" % (k, v["us"], v["pct_hbm_peak"])
+                                                        for k, v in entry.items() if k != "row_length")))
+    return sweep
+
+
 def build_other_configs(ctx, D, synth, rotate_bytes=600e6, max_sets=48):
     """Kernels of configs[0..3] at their BASELINE.json shapes (parity-test shapes, reported as a table
     only).  Buffers are rotated over enough copies that repeated launches miss the 256 MB cache.  Each
@@ -443,10 +486,13 @@ def calibration_op(ctx, D):
               [lambda: ctx.unary_raw(D.RELU, d_out.ptr, d_in.ptr, n)])
 
 
+TRAFFIC_FILE = "profiles/hbm_traffic.json"
+
+
 def measured_traffic(kernel_name):
-    """HBM bytes per launch of a kernel as derived from rocprofv3 FETCH_SIZE / WRITE_SIZE runs
-    (profiles/hbm_traffic.json, written by hand from those runs), or None."""
-    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    """HBM bytes per launch of a kernel as derived from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this program
+    (profiles/hbm_traffic.json, written from those runs; counters cannot be read from inside the timed run), or None."""
+    path = os.path.join(ROOT, TRAFFIC_FILE)
     if not os.path.exists(path):
         return None
     with open(path) as f:
@@ -457,53 +503,117 @@ def measured_traffic(kernel_name):
     return None
 
 
-def time_kernel(ctx, op, iters, warmup):
-    """Average duration of one launch, in ms, from HIP events around `iters` back-to-back launches."""
+class Timing:
+    """Launch durations of one kernel in ms: mean over all timed launches (what `roofline.achieved` uses),
+    median and minimum over the samples (one sample = the average of a short group of back-to-back launches)."""
+
+    def __init__(self, samples_ms, group):
+        self.samples = sorted(samples_ms)
+        self.group = group
+        self.launches = len(samples_ms) * group
+        self.mean = sum(samples_ms) / len(samples_ms)
+        self.median = float(np.median(samples_ms))
+        self.min = self.samples[0]
+
+    def row(self, nbytes):
+        """The figures every table of the report carries, rounded."""
+        gbps = nbytes / (self.mean * 1e-3) / 1e9
+        return {"us": round(self.mean * 1e3, 2), "us_median": round(self.median * 1e3, 2), "us_min": round(self.min * 1e3, 2),
+                "launches": self.launches, "GBps": round(gbps, 1), "pct_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 1),
+                "pct_hbm_peak_median": round(100.0 * nbytes / (self.median * 1e-3) / 1e9 / HBM_PEAK_GBPS, 1)}
+
+
+def time_kernel(ctx, op, iters=100, warmup=20):
+    """`warmup` untimed launches, then at least `iters` timed ones with a HIP event on the kernels' stream between
+    consecutive samples.  A sample is a group of back-to-back launches lasting about 0.25 ms (one launch for the longest
+    kernels, dozens for the few-microsecond ones), so that the event between samples does not weigh on the figure."""
     for _ in range(warmup):
         op.launch()
-    start, stop = ctx.event(), ctx.event()
+    probe = [ctx.event(), ctx.event()]
     ctx.sync()
-    ctx.record(start)
-    for _ in range(iters):
+    ctx.record(probe[0])
+    for _ in range(5):
         op.launch()
-    ctx.record(stop)
-    ms = ctx.elapsed_ms(start, stop) / iters
-    ctx.destroy_event(start)
-    ctx.destroy_event(stop)
-    return ms
+    ctx.record(probe[1])
+    est_ms = ctx.elapsed_ms(probe[0], probe[1]) / 5
+    for e in probe:
+        ctx.destroy_event(e)
+    group = max(1, min(64, int(round(0.25 / max(est_ms, 1e-4)))))
+    n = max(25, (iters + group - 1) // group)
+    events = [ctx.event() for _ in range(n + 1)]
+    ctx.sync()
+    ctx.record(events[0])
+    for i in range(n):
+        for _ in range(group):
+            op.launch()
+        ctx.record(events[i + 1])
+    ctx.sync()
+    samples = [ctx.elapsed_ms(events[i], events[i + 1]) / group for i in range(n)]
+    for e in events:
+        ctx.destroy_event(e)
+    return Timing(samples, group)
+
+
+def time_interleaved(ctx, ops, steps, warmup):
+    """The step's kernels in step order, an event between every two launches: the duration of each kernel while the
+    others run around it (sustained mixed load), as opposed to the same kernel launched back to back."""
+    for _ in range(warmup):
+        for o in ops:
+            o.launch()
+    events = [[ctx.event() for _ in range(len(ops) + 1)] for _ in range(steps)]
+    ctx.sync()
+    for s in range(steps):
+        ctx.record(events[s][0])
+        for i, o in enumerate(ops):
+            o.launch()
+            ctx.record(events[s][i + 1])
+    ctx.sync()
+    out = []
+    for i in range(len(ops)):
+        out.append(Timing([ctx.elapsed_ms(events[s][i], events[s][i + 1]) for s in range(steps)], 1))
+    for row in events:
+        for e in row:
+            ctx.destroy_event(e)
+    return out
 
 
 def cpu_baseline(synth, batch_full, sample_batch, threads, arrays=None):
-    """Times the oracle on the same step (the whole batch, or a reduced one); returns GB/s and per-op seconds."""
+    """Times the oracle on the same step (the whole batch, or a reduced one).  Every operator is timed twice: writing
+    into a fresh output array per call, which is what the reference's run_node does (session.rs:95-110: one allocation
+    per node output, whose pages fault in while the kernel writes), and writing into an output that already exists.
+    Returns GB/s of the step (fresh outputs, the reference's behaviour), per-op seconds of both variants."""
     import oracle as O
 
     O.lib()
     c = arrays if arrays is not None and sample_batch == batch_full else synth.cfg4(batch=sample_batch)
-    times = {}
+    fresh, reused = {}, {}
     total_bytes = 0
 
-    def timed(name, nbytes, fn, reps=3):
-        nonlocal total_bytes
+    def best_of(fn, reps=3):
         best = float("inf")
         for _ in range(reps):
             t0 = time.perf_counter()
             fn()
             best = min(best, time.perf_counter() - t0)
-        times[name] = best
+        return best
+
+    def timed(name, nbytes, fn, out_shape):
+        nonlocal total_bytes
+        fresh[name] = best_of(lambda: fn(np.empty(out_shape, np.float32)))
+        out = np.zeros(out_shape, np.float32)    # exists and is mapped
+        reused[name] = best_of(lambda: fn(out))
         total_bytes += nbytes
+        return out
 
     scores, mask = c["scores"], c["mask"]
-    z = {}
-    timed("Add", 2 * scores.nbytes + mask.nbytes, lambda: z.__setitem__("z", O.binary(O.ADD, scores, mask, threads=threads)))
-    out = np.empty_like(scores)
-    timed("Softmax", 2 * scores.nbytes, lambda: O.softmax(z["z"], threads=threads, out=out))
+    z = timed("Add", 2 * scores.nbytes + mask.nbytes, lambda out: O.binary(O.ADD, scores, mask, threads=threads, out=out), scores.shape)
+    timed("Softmax", 2 * scores.nbytes, lambda out: O.softmax(z, threads=threads, out=out), scores.shape)
     x = c["rmax_in"]
-    timed("ReduceMax", x.nbytes + sample_batch * 197 * 4, lambda: O.reduce(O.REDUCE_MAX, x, [1], False))
+    timed("ReduceMax", x.nbytes + sample_batch * 197 * 4, lambda out: O.reduce(O.REDUCE_MAX, x, [1], False, out=out), (sample_batch, 197))
     y = c["div_in"]
     s = np.array(c["div_scalar"], np.float32)
-    timed("Div", 2 * y.nbytes + 4, lambda: O.binary(O.DIV, y, s, threads=threads))
-    total_s = sum(times.values())
-    return total_bytes / total_s / 1e9, times
+    timed("Div", 2 * y.nbytes + 4, lambda out: O.binary(O.DIV, y, s, threads=threads, out=out), y.shape)
+    return total_bytes / sum(fresh.values()) / 1e9, fresh, total_bytes / sum(reused.values()) / 1e9, reused
 
 
 def main():
@@ -512,7 +622,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=256, help="batch of configs[4] (256 = the named workload)")
-    ap.add_argument("--kernel-iters", type=int, default=50, help="launches per kernel for the per-kernel timing")
+    ap.add_argument("--kernel-iters", type=int, default=100, help="timed launches per kernel for the per-kernel timing")
+    ap.add_argument("--kernel-warmup", type=int, default=20, help="untimed launches per kernel ahead of them")
     ap.add_argument("--cpu-sample-batch", type=int, default=0,
                     help="batch of the CPU baseline sample (0: the whole batch, about 2 s of CPU time)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -521,8 +632,14 @@ def main():
                     help="also run a copy-shaped Relu of known size (scales rocprof byte counters)")
     ap.add_argument("--no-listed-ops", action="store_true",
                     help="skip the table of the path's other operators at configs[4]-sized tensors ('listed_ops' in the JSON)")
-    ap.add_argument("--all-configs", action="store_true",
-                    help="also time the kernels and graphs of configs[0..3] (table on stderr, 'other_configs' in the JSON)")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the kernels and graphs of configs[0..3] (table on stderr, 'other_configs' in the JSON: us, GB/s and "
+                         "the CPU oracle's us at 16 threads and at 1 thread beside each)")
+    ap.add_argument("--all-configs", action="store_true", help="accepted for compatibility: configs[0..3] are part of the default run")
+    ap.add_argument("--no-row-sweep", action="store_true",
+                    help="skip Softmax / LayerNormalization / ReduceMean by row length ('row_sweep' in the JSON)")
+    ap.add_argument("--sweep-lengths", type=str, default="", help="comma-separated row lengths for the sweep (default: 49 ... 16384)")
+    ap.add_argument("--sweep-only", action="store_true", help="run the row sweep and nothing else (profiling)")
     ap.add_argument("--next-rows", action="store_true",
                     help="also time the data-movement and MatMul kernels at ViT-B/16 shapes ('next_rows' in the JSON)")
     ap.add_argument("--vit", type=int, default=0, metavar="BATCH",
@@ -541,6 +658,11 @@ def main():
     from altius_amd import synth
 
     ctx = D.Context(0)
+    sweep_lengths = tuple(int(v) for v in args.sweep_lengths.split(",") if v) or ROW_SWEEP_LENGTHS
+    if args.sweep_only:
+        print(json.dumps({"row_sweep": run_row_sweep(ctx, D, args, sweep_lengths)}), flush=True)
+        ctx.close()
+        return
     ops, fused_ops, cfg4_arrays = build_cfg4(ctx, D, synth, args.batch, rotate_bytes=600e6)
     if args.only:
         ops = [o for o in ops if args.only.lower() in o.name.lower()]
@@ -566,13 +688,18 @@ def main():
     # --- per kernel, HIP events on the kernels' stream -----------------------------------------
     rows = []
     for o in ops + extra_ops:
-        ms = time_kernel(ctx, o, args.kernel_iters, 5)
-        gbps = o.nbytes / (ms * 1e-3) / 1e9
-        rows.append({"kernel": o.name, "bytes": o.nbytes, "us": ms * 1e3, "GBps": gbps,
-                     "pct_hbm_peak": 100.0 * gbps / HBM_PEAK_GBPS})
-    log("%-44s %14s %10s %10s %8s" % ("kernel", "alg. bytes", "us/call", "GB/s", "% peak"))
+        t = time_kernel(ctx, o, args.kernel_iters, args.kernel_warmup)
+        rows.append(dict({"kernel": o.name, "bytes": o.nbytes}, **t.row(o.nbytes)))
+    # ... and each of the step's kernels while the others run around it
+    if len(ops) > 1:
+        for r, t in zip(rows, time_interleaved(ctx, ops, max(args.steps, 25), args.warmup)):
+            r["us_interleaved"] = round(t.mean * 1e3, 2)
+            r["us_interleaved_median"] = round(t.median * 1e3, 2)
+            r["pct_hbm_peak_interleaved"] = round(100.0 * r["bytes"] / (t.mean * 1e-3) / 1e9 / HBM_PEAK_GBPS, 1)
+    log("%-44s %14s %9s %9s %9s %9s %8s %12s" % ("kernel", "alg. bytes", "us mean", "us median", "us min", "GB/s", "% peak", "us in step"))
     for r in rows:
-        log("%-44s %14d %10.1f %10.1f %8.1f" % (r["kernel"], r["bytes"], r["us"], r["GBps"], r["pct_hbm_peak"]))
+        log("%-44s %14d %9.1f %9.1f %9.1f %9.1f %8.1f %12s" % (r["kernel"], r["bytes"], r["us"], r["us_median"], r["us_min"], r["GBps"],
+                                                            r["pct_hbm_peak"], "%.1f" % r["us_interleaved"] if "us_interleaved" in r else "-"))
     dom = max(rows[:len(ops)], key=lambda r: r["us"])
 
     result = {
@@ -602,31 +729,41 @@ def main():
             "unit": "GB/s",
             "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
             "traffic": measured_traffic(dom["kernel"]),
+            "traffic_source": TRAFFIC_FILE + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by a copy kernel of known "
+                              "size; a constant read from that file, not measured in this run)",
             "us_per_launch": round(dom["us"], 2),
+            "us_per_launch_median": dom["us_median"],
+            "us_per_launch_min": dom["us_min"],
+            "us_per_launch_in_step": dom.get("us_interleaved"),
+            "frac_in_step": round(dom["bytes"] / (dom["us_interleaved"] * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4) if "us_interleaved" in dom else None,
+            "launches": dom["launches"],
             "algorithmic_bytes": dom["bytes"],
         },
-        "per_kernel": [{k: (round(v, 2) if isinstance(v, float) else v) for k, v in r.items()} for r in rows],
+        "timing": "per kernel: %d warm-up launches, then >= %d launches with a HIP event between samples on the kernels' stream; "
+                  "us = mean, us_median, us_min; us_interleaved = the same kernel inside the step (an event between every two "
+                  "kernels of the step)" % (args.kernel_warmup, args.kernel_iters),
+        "per_kernel": rows,
     }
 
     if not args.only and not args.no_listed_ops:
         listed = []
         log("every operator of the path at configs[4]-sized tensors:")
         for o in build_listed_ops(ctx, D, cfg4_arrays, args.batch):
-            ms = time_kernel(ctx, o, args.kernel_iters, 5)
-            gbps = o.nbytes / (ms * 1e-3) / 1e9
-            listed.append({"kernel": o.name, "bytes": o.nbytes, "us": round(ms * 1e3, 2), "GBps": round(gbps, 1),
-                           "pct_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 1)})
-            log("%-44s %14d %10.1f %10.1f %8.1f" % (o.name, o.nbytes, ms * 1e3, gbps, 100.0 * gbps / HBM_PEAK_GBPS))
+            t = time_kernel(ctx, o, args.kernel_iters, args.kernel_warmup)
+            r = dict({"kernel": o.name, "bytes": o.nbytes}, **t.row(o.nbytes))
+            listed.append(r)
+            log("%-44s %14d %9.1f %9.1f %9.1f %9.1f %8.1f" % (o.name, o.nbytes, r["us"], r["us_median"], r["us_min"], r["GBps"], r["pct_hbm_peak"]))
         result["listed_ops"] = listed
 
-    if args.all_configs:
+    if not args.only and not args.no_row_sweep:
+        result["row_sweep"] = run_row_sweep(ctx, D, args, sweep_lengths)
+
+    if not args.only and not args.no_other_configs:
         others = []
-        log("%-44s %14s %10s %10s %8s %14s %14s" % ("kernel", "alg. bytes", "us/call", "GB/s", "% peak", "CPU 16 thr us", "CPU 1 thr us"))
+        log("%-44s %14s %10s %10s %10s %8s %14s %14s" % ("kernel", "alg. bytes", "us mean", "us median", "GB/s", "% peak", "CPU 16 thr us", "CPU 1 thr us"))
         for o in build_other_configs(ctx, D, synth):
-            ms = time_kernel(ctx, o, args.kernel_iters, 5)
-            gbps = o.nbytes / (ms * 1e-3) / 1e9
-            row = {"kernel": o.name, "bytes": o.nbytes, "us": round(ms * 1e3, 2), "GBps": round(gbps, 1),
-                   "pct_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 1)}
+            t = time_kernel(ctx, o, args.kernel_iters, args.kernel_warmup)
+            row = dict({"kernel": o.name, "bytes": o.nbytes}, **t.row(o.nbytes))
             cpu_us = {}
             if not args.no_cpu and o.cpu:
                 for threads in (16, 1):               # the CPU oracle on the host cores, best of 2 calls
@@ -638,8 +775,8 @@ def main():
                     cpu_us[threads] = best * 1e6
                 row["cpu_us_16_threads"], row["cpu_us_1_thread"] = round(cpu_us[16], 1), round(cpu_us[1], 1)
             others.append(row)
-            log("%-44s %14d %10.2f %10.1f %8.1f %14s %14s" % (o.name, o.nbytes, ms * 1e3, gbps, 100.0 * gbps / HBM_PEAK_GBPS,
-                                                               "%.1f" % cpu_us[16] if cpu_us else "-", "%.1f" % cpu_us[1] if cpu_us else "-"))
+            log("%-44s %14d %10.2f %10.2f %10.1f %8.1f %14s %14s" % (o.name, o.nbytes, row["us"], row["us_median"], row["GBps"], row["pct_hbm_peak"],
+                                                                     "%.1f" % cpu_us[16] if cpu_us else "-", "%.1f" % cpu_us[1] if cpu_us else "-"))
         graphs_rows = session_table(synth, ctx)
         for r in graphs_rows:
             log("%-36s kernels %7.1f us, as one HIP graph %7.1f us (%7.1f GB/s)  run_device() wall %7.1f us  run() incl. PCIe %7.3f ms"
@@ -659,7 +796,7 @@ def main():
         nxt = []
         for name, nbytes, flops, fn in build_next_rows(ctx, D, args.batch):
             o = Op(name, nbytes, [fn])
-            ms = time_kernel(ctx, o, max(10, args.kernel_iters // 2), 3)
+            ms = time_kernel(ctx, o, max(10, args.kernel_iters // 2), 3).mean
             row = {"kernel": name, "us": round(ms * 1e3, 1), "bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1)}
             if flops:
                 # six bf16 MFMAs per fp32 product: the bf16 peak (2500 TFLOP/s dense) over six
@@ -678,23 +815,32 @@ def main():
     if not args.no_cpu:
         threads = min(16, os.cpu_count() or 1)
         sample = args.cpu_sample_batch or args.batch
-        gbps_n, t_n = cpu_baseline(synth, args.batch, sample, threads, cfg4_arrays)
-        gbps_1, t_1 = cpu_baseline(synth, args.batch, sample, 1, cfg4_arrays)
+        gbps_n, t_n, gbps_n_re, t_n_re = cpu_baseline(synth, args.batch, sample, threads, cfg4_arrays)
+        gbps_1, t_1, gbps_1_re, t_1_re = cpu_baseline(synth, args.batch, sample, 1, cfg4_arrays)
         scale = args.batch / sample
-        log("CPU oracle, batch %d sample (x%.0f for the full step): %d threads %.2f GB/s, 1 thread %.2f GB/s"
-            % (sample, scale, threads, gbps_n, gbps_1))
+        log("CPU oracle, batch %d sample (x%.0f for the full step), fresh output per call as the reference allocates it: "
+            "%d threads %.2f GB/s, 1 thread %.2f GB/s; into existing outputs: %.2f and %.2f GB/s"
+            % (sample, scale, threads, gbps_n, gbps_1, gbps_n_re, gbps_1_re))
         for k in t_n:
-            log("  %-10s %d threads %9.1f us   1 thread %9.1f us  (scaled to batch %d)"
-                % (k, threads, t_n[k] * scale * 1e6, t_1[k] * scale * 1e6, args.batch))
+            log("  %-10s %d threads %9.1f us (existing output %9.1f)   1 thread %9.1f us (existing output %9.1f)  (scaled to batch %d)"
+                % (k, threads, t_n[k] * scale * 1e6, t_n_re[k] * scale * 1e6, t_1[k] * scale * 1e6, t_1_re[k] * scale * 1e6, args.batch))
+        us = lambda t: {k: round(v * scale * 1e6, 1) for k, v in t.items()}
         result["cpu_baseline"] = {
             "value": round(gbps_n, 2),
             "unit": "GB/s",
             "cores": threads,
             "kind": "port",
-            "sample": "same four kernels at batch %d of %d (1/%d of the step), best of 3 runs; "
-                      "1 thread: %.2f GB/s" % (sample, args.batch, int(scale), gbps_1),
+            "sample": "same four kernels at batch %d of %d (1/%d of the step), best of 3 runs, each output allocated per call "
+                      "as the reference's run_node does; 1 thread: %.2f GB/s; writing into existing outputs instead: %.2f GB/s "
+                      "(%d threads), %.2f GB/s (1 thread)" % (sample, args.batch, int(scale), gbps_1, gbps_n_re, threads, gbps_1_re),
             "single_thread_value": round(gbps_1, 2),
-            "us_per_kernel_scaled": {k: round(v * scale * 1e6, 1) for k, v in t_n.items()},
+            "value_existing_outputs": round(gbps_n_re, 2),
+            "single_thread_value_existing_outputs": round(gbps_1_re, 2),
+            "us_per_kernel_scaled": us(t_n),
+            "us_per_kernel_scaled_existing_outputs": us(t_n_re),
+            "us_per_kernel_scaled_1_thread": us(t_1),
+            "us_per_kernel_scaled_1_thread_existing_outputs": us(t_1_re),
+            "build": "g++ -O3 -march=x86-64-v3 -ffp-contract=off (oracle/Makefile)",
         }
 
     ctx.close()

@@ -332,6 +332,12 @@ int ahip_attention(ahip_ctx *ctx, float *o, const float *q, const float *k, cons
 #define AHIP_GEMM_FP32 1
 #define AHIP_GEMM_BF16X3 2
 int ahip_gemm_set_algorithm(ahip_ctx *ctx, int algorithm);
+/* Tensors of at least `bytes` bytes are read and written with non-temporal 16-byte accesses (they would not be
+ * found in the 256 MB Infinity Cache by the next kernel anyway); smaller ones are left to the caches.
+ * Default 128 MiB.  (size_t)-1 switches the hint off, 0 applies it to everything.  No counterpart in the
+ * reference. */
+int ahip_set_streaming_threshold(ahip_ctx *ctx, size_t bytes);
+
 /* The BF16X3 kernel cuts the tiles of a partly filled last round of blocks along k and lets the slice that
  * finishes last add the others' partial sums up out of one XCD's L2.  That needs all slices of a tile on one
  * XCD, which the kernel arranges by block id (the slices of a tile have equal ids mod 8, and consecutive ids go

@@ -112,13 +112,17 @@ def reduce_shape(kind, dims, axes, keep_dims):
     return [int(out[i]) for i in range(out_rank.value)]
 
 
-def binary(op, a, b, threads=1, strict=False, info=None):
+def binary(op, a, b, threads=1, strict=False, info=None, out=None):
+    """out: a float32 array of the broadcast shape to write into (the reference's run_node allocates a fresh
+    one per call, which is what out=None does)."""
     a = _f32(a)
     b = _f32(b)
     shape = broadcast(a.shape, b.shape)
     if shape is None:
         raise OracleError(ERR_BROADCAST, "binary")
-    out = np.empty(shape, dtype=np.float32)
+    if out is None:
+        out = np.empty(shape, dtype=np.float32)
+    assert out.dtype == np.float32 and list(out.shape) == list(shape) and out.flags.c_contiguous
     ad, ar = _dims(a.shape)
     bd, br = _dims(b.shape)
     noref = ctypes.c_int(0)
@@ -171,10 +175,12 @@ def layer_norm(x, scale, bias, eps=1e-5, threads=1, out=None):
     return out
 
 
-def reduce(kind, x, axes, keep_dims, strict=False, info=None):
+def reduce(kind, x, axes, keep_dims, strict=False, info=None, out=None):
     x = _f32(x)
     shape = reduce_shape(kind, x.shape, axes, keep_dims)
-    out = np.empty(shape, dtype=np.float32)
+    if out is None:
+        out = np.empty(shape, dtype=np.float32)
+    assert out.dtype == np.float32 and list(out.shape) == list(shape) and out.flags.c_contiguous
     d, r = _dims(x.shape)
     ax, na = _dims(axes)
     noref = ctypes.c_int(0)
