@@ -115,6 +115,35 @@ __global__ __launch_bounds__(ROW_BLOCK) void reduce_rows_wave(float *__restrict_
     if (lane == 0) out[row] = SCALE ? acc * scale : acc;
 }
 
+// Rows of 4 to 256 elements that are whole float4s: SUB = 1 to 64 lanes per row, one 16-byte load per lane, so a
+// wavefront's load is one contiguous piece of the tensor holding 64 / SUB whole rows (lanes past the row's last
+// float4 idle when the float4 count is not a power of two).  Each wavefront takes U such pieces, all loads requested
+// before the first is folded.
+template <class OP, int SUB, int U, bool SCALE, bool NT>
+__global__ __launch_bounds__(ROW_BLOCK) void reduce_rows_sub4(float *__restrict__ out, const float *__restrict__ in, size_t outer,
+                                                              uint32_t red, float scale) {
+    constexpr int RPP = WAVE / SUB;  // rows per wavefront pass
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int s = lane & (SUB - 1), rr = lane / SUB;
+    const size_t wave = (size_t)blockIdx.x * ROW_WAVES + (threadIdx.x >> 6);
+    const size_t row0 = wave * (size_t)(RPP * U) + rr;
+    const bool has = (uint32_t)(4 * s) < red;
+    float4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const size_t row = row0 + (size_t)u * RPP;
+        const float id = OP::identity();
+        v[u] = has && row < outer ? load4<NT>(in + row * red + 4 * s) : make_float4(id, id, id, id);
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const size_t row = row0 + (size_t)u * RPP;
+        float acc = OP::apply(OP::apply(v[u].x, v[u].y), OP::apply(v[u].z, v[u].w));
+        if (SUB > 1) acc = subwave_allreduce<OP, SUB < 4 ? 4 : SUB>(acc);
+        if (s == 0 && row < outer) out[row] = SCALE ? acc * scale : acc;
+    }
+}
+
 // grid = (splits, outer).  Block (s, o) folds chunk s of row o into
 // dst[o * splits + s].
 template <class OP, int VEC, bool SCALE>
@@ -393,6 +422,32 @@ int reduce_impl(DeviceCtx &ctx, const Partials &pt, float *out, const float *in,
                 float scale) {
     hipStream_t s = ctx.stream;
     if (inner == 1) {
+        // Rows of up to 256 elements that are whole float4s: a few lanes per row, straight from memory.
+        if (red % 4 == 0 && red >= 16 && red <= 256 && aligned16(in)) {
+            constexpr int U = 4;
+            const size_t v4 = red / 4;
+            const int sub = v4 <= 4 ? 4 : v4 <= 8 ? 8 : v4 <= 16 ? 16 : v4 <= 32 ? 32 : 64;
+            const size_t rows_per_wave = (size_t)(WAVE / sub) * U;
+            const size_t blocks = (outer + rows_per_wave * ROW_WAVES - 1) / (rows_per_wave * ROW_WAVES);
+            if (blocks <= MAX_GRID_X) {
+                const bool nt = ctx.streaming(outer * red * sizeof(float));
+                const dim3 grid((unsigned)blocks), block(ROW_BLOCK);
+#define ALTIUS_SUB4(SUBV)                                                                                                          \
+    do {                                                                                                                           \
+        if (nt) hipLaunchKernelGGL((reduce_rows_sub4<OP, SUBV, U, SCALE, true>), grid, block, 0, s, out, in, outer, (uint32_t)red, scale);  \
+        else hipLaunchKernelGGL((reduce_rows_sub4<OP, SUBV, U, SCALE, false>), grid, block, 0, s, out, in, outer, (uint32_t)red, scale);    \
+    } while (0)
+                switch (sub) {
+                case 4: ALTIUS_SUB4(4); break;
+                case 8: ALTIUS_SUB4(8); break;
+                case 16: ALTIUS_SUB4(16); break;
+                case 32: ALTIUS_SUB4(32); break;
+                default: ALTIUS_SUB4(64); break;
+                }
+#undef ALTIUS_SUB4
+                return ctx.check(hipGetLastError(), "reduce rows (lane groups) launch");
+            }
+        }
         // Short rows and rows that are not whole float4s: groups of rows staged through LDS, a few lanes per row.
         if (red <= 1024 && (red % 4 != 0 || red < 256)) {
             const int rc = launch_reduce_rows_lds(ctx, std::is_same<OP, MaxOp>::value, out, in, outer, red, scale, SCALE);

@@ -878,6 +878,14 @@ bool layernorm_lds_launch(hipStream_t s, float *out, const float *in, const floa
     return false;
 }
 
+// A wavefront per row with 16-byte accesses suits rows that are whole 128-byte lines (no line shared between the
+// loads of two wavefronts) and fill at least three quarters of the wavefront's 256-element chunks; every other
+// row of up to 1024 elements goes through LDS in line-aligned groups.
+inline bool wave_row_fits(size_t len) {
+    const size_t slots = (len + 255) / 256 * 256;
+    return len % 32 == 0 && len * 4 >= slots * 3;
+}
+
 constexpr size_t MAX_WAVE_ROW = 1024;
 constexpr size_t MAX_LONG_ROW = 1536;  // rows kept in a wavefront's registers when they are whole float4s
 constexpr size_t MAX_BLOCK_REG_ROW = 16384;  // ... and in a block's registers
@@ -895,8 +903,7 @@ int launch_softmax(DeviceCtx &ctx, float *out, const float *in, size_t rows, siz
         const bool vec4 = (len % 4 == 0) && aligned;
         // A wave per row with 16-byte accesses is ideal when the row fills (most of) the wave's
         // 256-element chunks; otherwise go through LDS, which needs aligned buffers only.
-        const size_t slots = (len + 255) / 256 * 256;
-        const bool wave_fits = vec4 && len * 4 >= slots * 3;
+        const bool wave_fits = vec4 && wave_row_fits(len);
         if (aligned && !wave_fits) {
             if (!softmax_lds_launch(ctx.stream, out, in, rows, len, ctx.streaming(rows * len * sizeof(float))))
                 return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: too many rows for one launch");
@@ -942,8 +949,7 @@ int launch_softmax_prologue(DeviceCtx &ctx, float *out, const float *in, size_t 
     if (len > MAX_WAVE_ROW || !aligned16(out) || !aligned16(in) || rows >= ((size_t)1 << 32) || rows_per_mask >= ((size_t)1 << 32))
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax prologue: needs 16-byte aligned tensors and rows of at most 1024 elements");
     SoftmaxPrologue pro{scale_op, scale, mask, (uint32_t)(mask ? rows_per_mask : 1), (uint32_t)(mask ? rows / rows_per_mask : 0)};
-    const size_t slots = (len + 255) / 256 * 256;
-    const bool wave_fits = len % 4 == 0 && len * 4 >= slots * 3;
+    const bool wave_fits = wave_row_fits(len);
     if (wave_fits) {
         if (mask && !aligned16(mask)) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax prologue: the mask must be 16-byte aligned");
         if ((rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK > MAX_GRID || !dispatch_wave<SoftmaxLauncher>(true, len, ctx.stream, out, in, rows, (int)len, (const SoftmaxPrologue *)&pro,
@@ -962,8 +968,7 @@ int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *g
     if (len <= MAX_WAVE_ROW && rows >= 64 && aligned16(out) && aligned16(in)) {
         // Rows that fill (most of) a wavefront's 256-element chunks with whole float4s take the wavefront-per-row
         // kernel; every other row of up to 1024 elements goes through LDS in line-aligned groups (the rule Softmax uses).
-        const size_t slots = (len + 255) / 256 * 256;
-        const bool wave_fits = len % 32 == 0 && len * 4 >= slots * 3 && aligned16(gamma) && aligned16(beta);
+        const bool wave_fits = wave_row_fits(len) && aligned16(gamma) && aligned16(beta);
         if (!wave_fits && layernorm_lds_launch(ctx.stream, out, in, gamma, beta, rows, len, eps, ctx.streaming(rows * len * sizeof(float))))
             return ctx.check(hipGetLastError(), "layernorm (LDS groups) launch");
     }
