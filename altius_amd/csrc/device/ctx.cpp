@@ -45,6 +45,9 @@ int create_device_ctx(int device, hipStream_t stream, bool own_stream, DeviceCtx
     // AHIP_GEMM_SPLIT_K=0 keeps the bf16 GEMM from cutting an XCD's partly filled last round of tiles along k
     // (for measurements).
     if (const char *e = getenv("AHIP_GEMM_SPLIT_K")) ctx->gemm_split_k = atoi(e) != 0;
+    // AHIP_STREAMING_THRESHOLD_MIB: the tensor size from which accesses are non-temporal (for measurements; see
+    // ahip_set_streaming_threshold).
+    if (const char *e = getenv("AHIP_STREAMING_THRESHOLD_MIB")) ctx->nt_threshold_bytes = (size_t)atol(e) << 20;
     int cus = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && cus >= 8) ctx->cus_per_xcd = cus / 8;
     if (own_stream) {

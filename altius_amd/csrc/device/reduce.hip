@@ -448,8 +448,9 @@ int reduce_impl(DeviceCtx &ctx, const Partials &pt, float *out, const float *in,
                 return ctx.check(hipGetLastError(), "reduce rows (lane groups) launch");
             }
         }
-        // Short rows and rows that are not whole float4s: groups of rows staged through LDS, a few lanes per row.
-        if (red <= 1024 && (red % 4 != 0 || red < 256)) {
+        // Short rows and rows that are not whole 128-byte lines (a wavefront per row would fetch the lines two rows
+        // share twice: 10 % more traffic on rows of 1000): groups of rows staged through LDS, a few lanes per row.
+        if (red <= 1024 && (red % 32 != 0 || red < 256)) {
             const int rc = launch_reduce_rows_lds(ctx, std::is_same<OP, MaxOp>::value, out, in, outer, red, scale, SCALE);
             if (rc >= 0) return rc;
         }

@@ -638,6 +638,8 @@ def main():
     ap.add_argument("--all-configs", action="store_true", help="accepted for compatibility: configs[0..3] are part of the default run")
     ap.add_argument("--no-row-sweep", action="store_true",
                     help="skip Softmax / LayerNormalization / ReduceMean by row length ('row_sweep' in the JSON)")
+    ap.add_argument("--streaming-threshold-mib", type=int, default=-1,
+                    help="tensors of at least this many MiB use non-temporal accesses (default: the library's own threshold)")
     ap.add_argument("--sweep-lengths", type=str, default="", help="comma-separated row lengths for the sweep (default: 49 ... 16384)")
     ap.add_argument("--sweep-only", action="store_true", help="run the row sweep and nothing else (profiling)")
     ap.add_argument("--next-rows", action="store_true",
@@ -658,9 +660,17 @@ def main():
     from altius_amd import synth
 
     ctx = D.Context(0)
+    if args.streaming_threshold_mib >= 0:
+        ctx.set_streaming_threshold(args.streaming_threshold_mib << 20)
     sweep_lengths = tuple(int(v) for v in args.sweep_lengths.split(",") if v) or ROW_SWEEP_LENGTHS
     if args.sweep_only:
-        print(json.dumps({"row_sweep": run_row_sweep(ctx, D, args, sweep_lengths)}), flush=True)
+        out = {}
+        if args.calibrate:  # first, so that a profile of this run finds the copy kernel of known size ahead of the sweep
+            cal = calibration_op(ctx, D)
+            out["calibration"] = dict({"kernel": cal.name, "bytes": cal.nbytes}, **time_kernel(ctx, cal, args.kernel_iters, args.kernel_warmup).row(cal.nbytes))
+            log("%-44s %14d %9.1f us %6.1f %%" % (cal.name, cal.nbytes, out["calibration"]["us"], out["calibration"]["pct_hbm_peak"]))
+        out["row_sweep"] = run_row_sweep(ctx, D, args, sweep_lengths)
+        print(json.dumps(out), flush=True)
         ctx.close()
         return
     ops, fused_ops, cfg4_arrays = build_cfg4(ctx, D, synth, args.batch, rotate_bytes=600e6)
