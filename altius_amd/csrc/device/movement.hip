@@ -37,7 +37,10 @@ struct CopyGeom {
 
 // T is the storage unit: 1, 4, 8 or 16 bytes (16 = four 4-byte elements moved together when the
 // innermost axis is contiguous on both sides and everything is 16-byte aligned).
-template <class T>
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// NT (16-byte units only): non-temporal accesses, for tensors too large to be found in a cache afterwards.
+template <class T, bool NT = false>
 __global__ __launch_bounds__(BLOCK) void copy_strided(T *__restrict__ out, const T *__restrict__ in, CopyGeom g,
                                                       uint32_t total) {
     const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
@@ -53,7 +56,13 @@ __global__ __launch_bounds__(BLOCK) void copy_strided(T *__restrict__ out, const
             rest = q;
         }
     }
-    out[dst] = in[src];
+    if (NT) {
+        static_assert(!NT || sizeof(T) == 16, "non-temporal copies move 16-byte units");
+        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(in + src));
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out + dst));
+    } else {
+        out[dst] = in[src];
+    }
 }
 
 // ---- tiled transpose -------------------------------------------------------------------------
@@ -109,18 +118,18 @@ __global__ __launch_bounds__(BLOCK) void transpose_tiled(T *__restrict__ out, co
 // matrix as one contiguous span, scatters it into LDS transposed, and writes the result as one
 // contiguous span, so both global sides run at full 16-byte width whatever the extents are.
 // The LDS row pitch is odd, which keeps the transposed stores conflict-free.
-template <class T, int VEC>
-__global__ __launch_bounds__(BLOCK) void transpose_small(T *__restrict__ out, const T *__restrict__ in, uint32_t r_len,
-                                                         uint32_t c_len, uint32_t pitch, FastDiv cdiv, FastDiv rdiv) {
+template <class T, int VEC, int TB = BLOCK, bool NT = false>
+__global__ __launch_bounds__(TB) void transpose_small(T *__restrict__ out, const T *__restrict__ in, uint32_t r_len,
+                                                      uint32_t c_len, uint32_t pitch, FastDiv cdiv, FastDiv rdiv) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T *lds = reinterpret_cast<T *>(smem_raw);  // [c_len][pitch], element (c, r) at c * pitch + r
     const uint32_t n = r_len * c_len;
     const T *src = in + (size_t)blockIdx.x * n;
     T *dst = out + (size_t)blockIdx.x * n;
-    for (uint32_t i = threadIdx.x * VEC; i < n; i += BLOCK * VEC) {
+    for (uint32_t i = threadIdx.x * VEC; i < n; i += TB * VEC) {
         T v[VEC];
         if (VEC == 4) {
-            const uint4 t = *reinterpret_cast<const uint4 *>(src + i);
+            const u32x4 t = NT ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + i)) : *reinterpret_cast<const u32x4 *>(src + i);
             v[0] = (T)t.x; v[1 % VEC] = (T)t.y; v[2 % VEC] = (T)t.z; v[3 % VEC] = (T)t.w;
         } else {
             v[0] = src[i];
@@ -136,7 +145,7 @@ __global__ __launch_bounds__(BLOCK) void transpose_small(T *__restrict__ out, co
         }
     }
     __syncthreads();
-    for (uint32_t i = threadIdx.x * VEC; i < n; i += BLOCK * VEC) {
+    for (uint32_t i = threadIdx.x * VEC; i < n; i += TB * VEC) {
         uint32_t c = rdiv.div(i), r = i - c * r_len;  // output is [c][r]
         T v[VEC];
 #pragma unroll
@@ -148,9 +157,10 @@ __global__ __launch_bounds__(BLOCK) void transpose_small(T *__restrict__ out, co
             }
         }
         if (VEC == 4) {
-            uint4 t;
+            u32x4 t;
             t.x = (uint32_t)v[0]; t.y = (uint32_t)v[1 % VEC]; t.z = (uint32_t)v[2 % VEC]; t.w = (uint32_t)v[3 % VEC];
-            *reinterpret_cast<uint4 *>(dst + i) = t;
+            if (NT) __builtin_nontemporal_store(t, reinterpret_cast<u32x4 *>(dst + i));
+            else *reinterpret_cast<u32x4 *>(dst + i) = t;
         } else {
             dst[i] = v[0];
         }
@@ -474,7 +484,13 @@ int launch_copy_strided(DeviceCtx &ctx, void *out, const void *in, int elem_size
     case 1: launch_copy<uint8_t>(ctx.stream, out, in, g, (uint32_t)total); break;
     case 4: launch_copy<uint32_t>(ctx.stream, out, in, g, (uint32_t)total); break;
     case 8: launch_copy<uint64_t>(ctx.stream, out, in, g, (uint32_t)total); break;
-    default: launch_copy<uint4>(ctx.stream, out, in, g, (uint32_t)total); break;
+    default:
+        if (ctx.streaming(total * 16))
+            hipLaunchKernelGGL((copy_strided<uint4, true>), dim3((unsigned)((total + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, ctx.stream,
+                               static_cast<uint4 *>(out), static_cast<const uint4 *>(in), g, (uint32_t)total);
+        else
+            launch_copy<uint4>(ctx.stream, out, in, g, (uint32_t)total);
+        break;
     }
     return ctx.check(hipGetLastError(), "copy_strided launch");
 }
@@ -577,7 +593,15 @@ int launch_transpose(DeviceCtx &ctx, void *out, const void *in, int elem_size, i
                 const FastDiv cdiv = make_fastdiv(g.c_len), rdiv = make_fastdiv(g.r_len);
                 const dim3 grid((unsigned)batches);
                 const bool vec = elem_size == 4 && n % 4 == 0 && aligned16(out) && aligned16(in);
-                if (elem_size == 4 && vec)
+                // Matrices of 8192 elements and more get a block of 1024 threads (one matrix's LDS image allows two or
+                // three blocks per CU: with 256 threads each the CU would be nearly empty).
+                if (elem_size == 4 && vec && n >= 8192 && ctx.streaming(total * 4))
+                    hipLaunchKernelGGL((transpose_small<uint32_t, 4, 1024, true>), grid, dim3(1024), lds_bytes, ctx.stream,
+                                       static_cast<uint32_t *>(out), static_cast<const uint32_t *>(in), g.r_len, g.c_len, pitch, cdiv, rdiv);
+                else if (elem_size == 4 && vec && n >= 8192)
+                    hipLaunchKernelGGL((transpose_small<uint32_t, 4, 1024, false>), grid, dim3(1024), lds_bytes, ctx.stream,
+                                       static_cast<uint32_t *>(out), static_cast<const uint32_t *>(in), g.r_len, g.c_len, pitch, cdiv, rdiv);
+                else if (elem_size == 4 && vec)
                     hipLaunchKernelGGL((transpose_small<uint32_t, 4>), grid, dim3(BLOCK), lds_bytes, ctx.stream,
                                        static_cast<uint32_t *>(out), static_cast<const uint32_t *>(in), g.r_len, g.c_len, pitch, cdiv, rdiv);
                 else if (elem_size == 4)
