@@ -175,9 +175,19 @@ int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, c
 // product (gemm_split.hip): as accurate as an fp32 multiply-add chain, about 1.6 times the fp32 matrix
 // cores' rate on large shapes.  launch_gemm takes this route by itself according to ctx.gemm_algorithm.
 // a_op: 0, or AHIP_GELU / AHIP_RELU applied to A's values while they are split (C = alpha f(A) B + beta C0).
+// a_planes (may be null): the first operand already as planes, as launch_layernorm_planes writes them (then a, lda
+// and a_op are not used): rows = m, k = k, gemm_planes_bytes(m, k) bytes.
 int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t m, size_t n, size_t k,
                       int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t c0_row_stride, size_t c0_col_stride,
-                      float alpha, float beta, int a_op = 0);
+                      float alpha, float beta, int a_op = 0, const void *a_planes = nullptr);
+size_t gemm_planes_bytes(size_t rows, size_t k);
+// LayerNormalization over rows of `len` elements written as the planes of the first operand of a product on the
+// bf16 route (rows = rows, k = len; gemm_planes_bytes(rows, len) bytes) instead of fp32 values: the planes that
+// launch_layernorm followed by the operand split would give, bit for bit.  in2 (may be null): the rows are in + in2
+// (a residual connection), and the sum is stored to sum_out as well.  Only for shapes layernorm_planes_fits accepts.
+int launch_layernorm_planes(DeviceCtx &ctx, void *planes, float *sum_out, const float *in, const float *in2, const float *gamma,
+                            const float *beta, size_t rows, size_t len, float eps);
+bool layernorm_planes_fits(size_t rows, size_t len);
 // The context's grow-only GEMM workspace, at least `bytes` large (stream-ordered use only).
 int gemm_workspace(DeviceCtx &ctx, size_t bytes, void **p);
 // Row sums (optionally times `scale`) or maxima of a [rows, len] matrix through LDS-staged groups of rows (rows.hip): for

@@ -120,6 +120,91 @@ __global__ __launch_bounds__(256) void split_planes_rows(const float *__restrict
     store_planes(planes, v, row, kg, rp, kgs);
 }
 
+// ---------------------------------------------------------------- LayerNormalization straight into planes
+// LayerNormalization over the last axis (crates/session_interpreter/src/session.rs:1433-1486) whose only reader is
+// the first operand of a product on this route: the normalised rows are written as that operand's planes and never
+// as fp32 (232 MB instead of 155 MB written, and the 155 MB + 232 MB of the operand split saved, on [50432, 768]).
+// A block of sixteen wavefronts takes sixteen rows, a wavefront per row with the row in registers: lane l holds
+// float4 l, l + 64, ... and the additions run in the order of the stand-alone wavefront-per-row kernel
+// (layernorm_wave in rows.hip), so mean, variance and every output value have its bits.  A lane's four values are
+// half of a 16-byte chunk of each plane; the halves go to LDS as [plane][k group][row], and from there the block
+// stores 256 contiguous bytes (sixteen rows of one k group) at a time.  ADD: the rows are a + b (a residual
+// connection); the sum is also stored as fp32 for its other readers.
+constexpr int LNP_ROWS = 16, LNP_THREADS = 1024;
+constexpr int LNP_KG_PITCH = LNP_ROWS * 4 + 4;  // 32-bit words per k group in LDS: sixteen 16-byte chunks and a pad
+
+template <int NCH, bool ADD>
+__global__ __launch_bounds__(LNP_THREADS) void layernorm_planes(u32x4 *__restrict__ planes, float *__restrict__ sum_out,
+                                                                const float *__restrict__ in, const float *__restrict__ in2,
+                                                                const float *__restrict__ gamma, const float *__restrict__ beta, uint32_t rows,
+                                                                uint32_t len, float eps, uint32_t rp, uint32_t kgs) {
+    extern __shared__ __align__(16) uint32_t lnp_lds[];  // [3][kgs][LNP_KG_PITCH]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t row0 = blockIdx.x * LNP_ROWS, grow = row0 + wave;
+    const uint32_t v4 = len / 4;  // float4 per row
+    float v[NCH * 4];
+#pragma unroll
+    for (int k = 0; k < NCH; k++) {
+        const uint32_t c = lane + 64 * k;
+        f32x4 t = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (grow < rows && c < v4) {
+            const size_t off = (size_t)grow * len + 4 * c;
+            t = *reinterpret_cast<const f32x4 *>(in + off);
+            if (ADD) {
+                const f32x4 u = *reinterpret_cast<const f32x4 *>(in2 + off);
+                t = f32x4{t.x + u.x, t.y + u.y, t.z + u.z, t.w + u.w};
+                *reinterpret_cast<f32x4 *>(sum_out + off) = t;
+            }
+        }
+        v[4 * k] = t.x, v[4 * k + 1] = t.y, v[4 * k + 2] = t.z, v[4 * k + 3] = t.w;
+    }
+    const float inv_n = 1.0f / (float)len;
+    float sum = 0.0f;
+#pragma unroll
+    for (int s = 0; s < NCH * 4; s++) sum += v[s];
+    const float mean = dev::wave_reduce<dev::SumOp>(sum) * inv_n;
+    float ss = 0.0f;
+#pragma unroll
+    for (int s = 0; s < NCH * 4; s++) {
+        const bool valid = (uint32_t)(lane + 64 * (s / 4)) < v4;
+        v[s] = v[s] - mean;
+        ss += valid ? v[s] * v[s] : 0.0f;
+    }
+    ss = dev::wave_reduce<dev::SumOp>(ss);
+    const float inv_std = 1.0f / sqrtf(__builtin_fmaf(ss, inv_n, eps));
+    // this lane's half chunks of the three planes -> LDS
+#pragma unroll
+    for (int k = 0; k < NCH; k++) {
+        const uint32_t c = lane + 64 * k;  // float4 number: k group c / 2, half c % 2
+        if (c < 2 * kgs) {
+            uint32_t h[3][4];
+            const bool live = grow < rows && c < v4;
+            f32x4 gm = {0.0f, 0.0f, 0.0f, 0.0f}, bt = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (live) gm = *reinterpret_cast<const f32x4 *>(gamma + 4 * c), bt = *reinterpret_cast<const f32x4 *>(beta + 4 * c);
+            const float g4[4] = {gm.x, gm.y, gm.z, gm.w}, b4[4] = {bt.x, bt.y, bt.z, bt.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float y = live ? __builtin_fmaf(v[4 * k + j] * inv_std, g4[j], b4[j]) : 0.0f;
+                split3(y, h[0][j], h[1][j], h[2][j]);
+            }
+#pragma unroll
+            for (int p = 0; p < 3; p++) {
+                uint32_t *dst = lnp_lds + ((size_t)p * kgs + (c >> 1)) * LNP_KG_PITCH + wave * 4 + (c & 1) * 2;
+                dst[0] = h[p][0] | (h[p][1] << 16);
+                dst[1] = h[p][2] | (h[p][3] << 16);
+            }
+        }
+    }
+    __syncthreads();
+    // LDS -> planes: consecutive threads take consecutive rows of one (plane, k group): 256 contiguous bytes
+    const uint32_t chunks = 3 * kgs * LNP_ROWS;
+    for (uint32_t i = tid; i < chunks; i += LNP_THREADS) {
+        const uint32_t r = i & (LNP_ROWS - 1), pk = i / LNP_ROWS;  // pk = plane * kgs + k group
+        const u32x4 o = *reinterpret_cast<const u32x4 *>(lnp_lds + (size_t)pk * LNP_KG_PITCH + r * 4);
+        planes[(size_t)pk * rp + row0 + r] = o;
+    }
+}
+
 // ---------------------------------------------------------------- the product
 
 constexpr int TM = 256, TN = 256, THREADS = 512;
@@ -536,11 +621,12 @@ bool gemm_split_worthwhile(size_t m, size_t n, size_t k) {
 
 int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, const float *c0, size_t m, size_t n, size_t k,
                       int trans_a, int trans_b, size_t lda, size_t ldb, size_t ldc, size_t c0_row_stride, size_t c0_col_stride,
-                      float alpha, float beta, int a_op) {
+                      float alpha, float beta, int a_op, const void *a_planes) {
     if (a_op != 0 && a_op != AHIP_GELU && a_op != AHIP_RELU)
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm (bf16 x 3): only Gelu and Relu can be folded into the operand split");
+    if (a_planes && (a_op || trans_a)) return ctx.fail(AHIP_ERR_ARG, "gemm (bf16 x 3): planes of the first operand come as they are");
     if (m == 0 || n == 0) return AHIP_OK;
-    if (!c || !a || !b || k == 0) return ctx.fail(AHIP_ERR_ARG, "gemm (bf16 x 3): null pointer or k = 0");
+    if (!c || (!a && !a_planes) || !b || k == 0) return ctx.fail(AHIP_ERR_ARG, "gemm (bf16 x 3): null pointer or k = 0");
     const size_t lim = (size_t)1 << 31;
     if (m >= lim - 256 || n >= lim - 256 || k >= lim - 16 || lda >= lim || ldb >= lim || ldc >= lim || c0_row_stride >= lim ||
         c0_col_stride >= lim)
@@ -550,7 +636,7 @@ int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, 
     if (tiles >= lim / 8 || (da.kgs + 3) / 4 > 65535) return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm (bf16 x 3): too many tiles");
     const bool a_kc = !trans_a, b_kc = trans_b != 0;
     int rc = AHIP_OK;
-    const void *pa = a_op ? nullptr : cached_planes(ctx, a, m, k, lda, a_kc, &rc);  // cached planes hold the plain values
+    const void *pa = a_planes ? a_planes : a_op ? nullptr : cached_planes(ctx, a, m, k, lda, a_kc, &rc);  // cached planes hold the plain values
     if (rc) return rc;
     const void *pb = cached_planes(ctx, b, n, k, ldb, b_kc, &rc);
     if (rc) return rc;
@@ -621,6 +707,45 @@ int launch_gemm_split(DeviceCtx &ctx, float *c, const float *a, const float *b, 
     g.c_stream = ctx.streaming(m * n * sizeof(float));
     hipLaunchKernelGGL(gemm_bf16x3, dim3(slots * 8), dim3(THREADS), 0, ctx.stream, g);
     return ctx.check(hipGetLastError(), "gemm (bf16 x 3) launch");
+}
+
+size_t gemm_planes_bytes(size_t rows, size_t k) { return plane_dims(rows, k).bytes; }
+
+int launch_layernorm_planes(DeviceCtx &ctx, void *planes, float *sum_out, const float *in, const float *in2, const float *gamma,
+                            const float *beta, size_t rows, size_t len, float eps) {
+    if (!planes || !in || !gamma || !beta || (in2 && !sum_out)) return ctx.fail(AHIP_ERR_ARG, "layernorm (planes): null pointer");
+    if (!layernorm_planes_fits(rows, len) || !aligned16(in) || !aligned16(gamma) || !aligned16(beta) ||
+        (in2 && (!aligned16(in2) || !aligned16(sum_out))))
+        return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm (planes): rows must be whole 128-byte lines of 256 to 1024 elements, 16-byte aligned");
+    const PlaneDims d = plane_dims(rows, len);
+    const dim3 grid((unsigned)(d.rp / LNP_ROWS));
+    const size_t shmem = (size_t)3 * d.kgs * LNP_KG_PITCH * sizeof(uint32_t);
+    const int nch = (int)((len / 4 + 63) / 64);
+#define ALTIUS_LNP(N)                                                                                                                   \
+    do {                                                                                                                                \
+        if (in2)                                                                                                                        \
+            hipLaunchKernelGGL((layernorm_planes<N, true>), grid, dim3(LNP_THREADS), shmem, ctx.stream, static_cast<u32x4 *>(planes), sum_out, in, \
+                               in2, gamma, beta, (uint32_t)rows, (uint32_t)len, eps, (uint32_t)d.rp, (uint32_t)d.kgs);                  \
+        else                                                                                                                            \
+            hipLaunchKernelGGL((layernorm_planes<N, false>), grid, dim3(LNP_THREADS), shmem, ctx.stream, static_cast<u32x4 *>(planes), sum_out, in, \
+                               in2, gamma, beta, (uint32_t)rows, (uint32_t)len, eps, (uint32_t)d.rp, (uint32_t)d.kgs);                  \
+    } while (0)
+    switch (nch) {
+    case 1: ALTIUS_LNP(1); break;
+    case 2: ALTIUS_LNP(2); break;
+    case 3: ALTIUS_LNP(3); break;
+    default: ALTIUS_LNP(4); break;
+    }
+#undef ALTIUS_LNP
+    return ctx.check(hipGetLastError(), "layernorm (planes) launch");
+}
+
+// The row lengths the stand-alone LayerNormalization gives to its wavefront-per-row kernel (whole 128-byte lines
+// filling three quarters of the wavefront's 256-element chunks, at most 1024 elements): only there does the planes
+// kernel reproduce its summation order.
+bool layernorm_planes_fits(size_t rows, size_t len) {
+    const size_t slots = (len + 255) / 256 * 256;
+    return rows > 0 && rows < ((size_t)1 << 31) - 256 && len >= 32 && len <= 1024 && len % 32 == 0 && len * 4 >= slots * 3;
 }
 
 int gemm_register_constant(DeviceCtx &ctx, const void *ptr, size_t bytes) {

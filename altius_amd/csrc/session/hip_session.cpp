@@ -183,6 +183,34 @@ bool HipSession::allocate(const TypedFixedShape &shape, DeviceTensor *out, Sessi
     return true;
 }
 
+// Whether this Add (planned as the residual connection in front of a planes-writing LayerNormalization) can leave its
+// sum to that kernel in this run: two dense f32 tensors of the result's shape, 16-byte aligned, nothing else owed, and
+// the LayerNormalization's own conditions (row length, the product behind it on the bf16 route).
+bool HipSession::defers_add(NodeId id, const std::vector<DeviceTensor *> &in, const std::vector<TypedFixedShape> &shapes) const {
+    if (in.size() != 2 || !in[0] || !in[1] || shapes.empty()) return false;
+    auto ln = planes_out_.find(add_into_ln_.at(id));
+    if (ln == planes_out_.end() || matmul_out_perm_.count(ln->second.consumer)) return false;
+    const FixedDimensions &d = shapes[0].dims;
+    for (const DeviceTensor *t : {in[0], in[1]})
+        if (t->elem_ty != TensorElemType::F32 || t->host || !(t->dims == d) || !t->strides.empty() || t->pending_op >= 0 || t->applied_op >= 0 ||
+            t->planes || t->owes_add() || !t->ptr || (reinterpret_cast<uintptr_t>(t->ptr) & 15u))
+            return false;
+    if (d.len() < 2) return false;
+    const size_t len = d[d.len() - 1], rows = len ? d.total_elems() / len : 0;
+    return layernorm_planes_fits(rows, len) && gemm_takes_split(ctx_, rows, ln->second.next_n, len);
+}
+
+bool HipSession::allocate_bytes(size_t nbytes, DeviceTensor *out, SessionError *err) {
+    auto block = std::make_shared<DeviceBlock>();
+    const int rc = pool_->acquire(nbytes, &block->ptr, &block->bucket);
+    if (rc) return fail_code(err, rc, ctx_.last_error);
+    block->pool = pool_.get();
+    if (capturing_) capture_allocs_.emplace_back(block->ptr, block->bucket);
+    out->ptr = block->ptr;
+    out->block = std::move(block);
+    return true;
+}
+
 bool HipSession::upload(const Tensor &t, DeviceTensor *out, SessionError *err) {
     if (!allocate(TypedFixedShape{t.dims(), t.elem_ty()}, out, err)) return false;
     if (out->nbytes()) {
@@ -591,6 +619,13 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
     if (!reads_views(node.op.kind))
         for (auto *d : in)
             if (d && !d->strides.empty() && !materialize(d, err)) return false;
+    // Operand planes have exactly one planned reader: the product behind the LayerNormalization that wrote them.
+    for (size_t i = 0; i < in.size(); i++)
+        if (in[i] && in[i]->planes && !(i == 0 && planes_consumer_.count(id)))
+            return fail(err, SessionError::Message, "internal: operand planes reached an operator that cannot read them");
+    // A deferred Add runs now unless the reader is the LayerNormalization that can compute the sum itself.
+    for (size_t i = 0; i < in.size(); i++)
+        if (in[i] && in[i]->owes_add() && !(i == 0 && planes_out_.count(id)) && !flush_add(in[i], err)) return false;
     // An activation still owed is applied by the MatMul that reads the tensor as its first operand, or here.
     for (size_t i = 0; i < in.size(); i++)
         if (in[i] && in[i]->pending_op >= 0 && !(node.op.kind == OpKind::MatMul && i == 0) &&
@@ -707,6 +742,18 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
             current_node_ = id;
             if (!run_device_op(node, op, in, shapes, &outs, err)) return false;
         }
+    } else if (add_into_ln_.count(id) && defers_add(id, in, shapes)) {
+        // A residual Add whose sum the LayerNormalization behind it computes on its way: reserve the sum's block,
+        // keep the operands, run nothing yet.
+        DeviceTensor o;
+        if (!allocate(shapes[0], &o, err)) return false;
+        auto p = std::make_shared<PendingAdd>();
+        p->a_block = in[0]->block, p->b_block = in[1]->block;
+        p->a = static_cast<const float *>(in[0]->ptr), p->b = static_cast<const float *>(in[1]->ptr);
+        p->elems = shapes[0].dims.total_elems();
+        o.pending_add = std::move(p);
+        copies_avoided_++;
+        outs.push_back(std::move(o));
     } else if (deferred_unary_.count(id) && in[0] && !in[0]->host && in[0]->elem_ty == TensorElemType::F32 && in[0]->pending_op < 0) {
         DeviceTensor o = *in[0];
         o.dims = shapes[0].dims;
@@ -1137,6 +1184,33 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
         const size_t len = in[0]->dims[rank - 1];
         if (in[1]->dims.total_elems() != len || in[2]->dims.total_elems() != len)
             return fail(err, SessionError::Shape, "LayerNormalization: scale and bias must hold one value per column");
+        {
+            // Read only by a product with a weight matrix that takes the bf16 route: write that product's operand planes.
+            auto pp = planes_out_.find(current_node_);
+            const size_t rows = len ? n_out / len : 0;
+            auto a16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+            if (pp != planes_out_.end() && in[0]->strides.empty() && layernorm_planes_fits(rows, len) && a16(in[0]->ptr) && a16(in[1]->ptr) &&
+                a16(in[2]->ptr) && matmul_out_perm_.count(pp->second.consumer) == 0 && gemm_takes_split(ctx_, rows, pp->second.next_n, len)) {
+                DeviceTensor planes;
+                if (!allocate_bytes(gemm_planes_bytes(rows, len), &planes, err)) return false;
+                if (in[0]->owes_add()) {  // the residual Add in front was left to this kernel: it writes the sum too
+                    PendingAdd &pa = *in[0]->pending_add;
+                    rc = launch_layernorm_planes(ctx_, planes.ptr, static_cast<float *>(in[0]->ptr), pa.a, pa.b, f(in[1]), f(in[2]), rows, len,
+                                                 op.epsilon);
+                    pa.done = true;
+                    pa.a_block.reset();
+                    pa.b_block.reset();
+                } else {
+                    rc = launch_layernorm_planes(ctx_, planes.ptr, nullptr, f(in[0]), nullptr, f(in[1]), f(in[2]), rows, len, op.epsilon);
+                }
+                out.block = planes.block;  // the fp32 block goes back to the pool unused
+                out.ptr = planes.ptr;
+                out.planes = true;
+                copies_avoided_++;  // the operand split of the product behind (and the fp32 tensor between them)
+                break;
+            }
+        }
+        if (!flush_add(in[0], err)) return false;
         rc = launch_layernorm(ctx_, o, f(in[0]), f(in[1]), f(in[2]), len ? n_out / len : 0, len, op.epsilon);
         break;
     }
@@ -1355,6 +1429,26 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
         if (in[0]->dims.len() < 2 || in[1]->dims.len() < 2) return fail(err, SessionError::Shape, "MatMul: operands of rank < 2");
         if (in[0]->pending_op == PENDING_ATTENTION) {  // the second product of a deferred attention: everything happens here
             if (!run_attention_tail(op, in, &out, err)) return false;
+            break;
+        }
+        if (in[0]->planes) {
+            // The first operand arrives as the planes the LayerNormalization in front wrote: [rows, k] x weights [k, n] on the bf16 route.
+            const FixedDimensions &ad = in[0]->dims, &bdm = in[1]->dims;
+            size_t rows = 1;
+            for (size_t i = 0; i + 1 < ad.len(); i++) rows *= ad[i];
+            const size_t kk = ad[ad.len() - 1];
+            if (op.trans_a || bdm.len() != 2 || !in[1]->strides.empty() || matmul_out_perm_.count(current_node_) ||
+                (op.trans_b ? bdm[1] : bdm[0]) != kk)
+                return fail(err, SessionError::Message, "internal: operand planes reached a product of another form");
+            const size_t nn = op.trans_b ? bdm[0] : bdm[1];
+            const float *bias_p = nullptr;
+            if (in.size() > 2 && in[2]) {
+                if (in[2]->elem_ty != TensorElemType::F32 || in[2]->dims.total_elems() != nn)
+                    return fail(err, SessionError::Shape, "MatMul: the absorbed bias must hold one f32 value per output column");
+                bias_p = f(in[2]);
+            }
+            rc = launch_gemm_split(ctx_, o, nullptr, f(in[1]), bias_p, rows, nn, kk, 0, op.trans_b ? 1 : 0, kk, op.trans_b ? kk : nn, nn, 0, 1, 1.0f,
+                                   bias_p ? 1.0f : 0.0f, 0, in[0]->ptr);
             break;
         }
         // The activation the first operand still owes is folded into the bf16 route's operand split when this

@@ -74,6 +74,17 @@ struct DeviceBlock {
 // DeviceTensor::pending_op of the placeholder a deferred attention product leaves behind (no memory).
 constexpr int PENDING_ATTENTION = 1000;
 
+struct DeviceTensor;
+// An Add of two tensors of one shape that has not run yet: the tensor's block is reserved for the sum, the operands
+// are kept alive, and either the LayerNormalization behind it computes the sum on its way (writing it here as well),
+// or the first other reader makes it run.  Shared by every alias of the tensor.
+struct PendingAdd {
+    std::shared_ptr<DeviceBlock> a_block, b_block;
+    const float *a = nullptr, *b = nullptr;
+    size_t elems = 0;
+    bool done = false;
+};
+
 struct DeviceTensor {
     FixedDimensions dims;
     TensorElemType elem_ty = TensorElemType::F32;
@@ -94,6 +105,13 @@ struct DeviceTensor {
     // An activation (AHIP_GELU / AHIP_RELU) that the MatMul which produced the tensor has already applied while
     // writing it: the activation node that follows passes the tensor on.
     int applied_op = -1;
+    // The block does not hold fp32 values but the tensor's three bf16 planes, laid out as the first operand of the
+    // tall bf16 product that is its only reader; the LayerNormalization that produced the tensor wrote them instead
+    // of the fp32 result.
+    bool planes = false;
+    // Set while the tensor's values are still owed by an Add that was deferred (see PendingAdd).
+    std::shared_ptr<PendingAdd> pending_add;
+    bool owes_add() const { return pending_add && !pending_add->done; }
     size_t nbytes() const { return dims.total_elems() * elem_size(elem_ty); }
 };
 
@@ -143,6 +161,9 @@ private:
     bool run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, SessionError *err);
     // A fresh pooled tensor of the given shape (contents unspecified).
     bool allocate(const TypedFixedShape &shape, DeviceTensor *out, SessionError *err);
+    // A pooled block of the given size behind a tensor whose shape the caller sets (operand planes).
+    bool allocate_bytes(size_t nbytes, DeviceTensor *out, SessionError *err);
+    bool defers_add(NodeId id, const std::vector<DeviceTensor *> &in, const std::vector<TypedFixedShape> &shapes) const;
     // Uploads a host tensor into a fresh pooled tensor that remembers its host contents.
     bool upload(const Tensor &t, DeviceTensor *out, SessionError *err);
     // Makes t.host available by reading a small tensor back (synchronises the stream).
@@ -249,6 +270,17 @@ private:
     std::map<NodeId, size_t> absorbed_add_;                     // Add nodes whose sum a MatMul wrote in this run -> input holding it
     const std::map<ValueId, DeviceTensor> *values_ = nullptr;   // the running call's values, for run_device_op
     std::set<NodeId> deferred_unary_;                           // Gelu / Relu nodes folded into the MatMul that reads them
+    // LayerNormalization -> MatMul(weights) with a single reader: where the product takes the bf16 route the
+    // normalisation writes the operand planes the product reads instead of fp32 values (next_n: columns of the weights).
+    struct PlanesPlan {
+        NodeId consumer = 0;
+        size_t next_n = 0;
+    };
+    std::map<NodeId, PlanesPlan> planes_out_;
+    std::set<NodeId> planes_consumer_;
+    std::map<NodeId, NodeId> add_into_ln_;  // Add nodes (a residual connection) -> the planes-writing LayerNormalization that reads the sum
+    // Runs a deferred Add into the tensor's block.
+    bool flush_add(DeviceTensor *t, SessionError *err);
     std::set<NodeId> lazy_views_;                               // Split / Transpose nodes whose outputs are views
     std::map<NodeId, std::vector<int64_t>> matmul_out_perm_;    // MatMul nodes -> perm of the Transpose they feed  // recorded launches hold the GEMM workspace's address
 };

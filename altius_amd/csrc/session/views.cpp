@@ -27,7 +27,20 @@ bool HipSession::materialize(DeviceTensor *t, SessionError *err) {
     return true;
 }
 
+bool HipSession::flush_add(DeviceTensor *t, SessionError *err) {
+    if (!t->owes_add()) return true;
+    PendingAdd &p = *t->pending_add;
+    const int64_t n = (int64_t)p.elems, one = 1;
+    const int rc = launch_binary(ctx_, AHIP_ADD, static_cast<float *>(t->ptr), p.a, p.b, 1, &n, &one, &one);
+    if (rc) return fail_code(err, rc, ctx_.last_error);
+    p.done = true;
+    p.a_block.reset();
+    p.b_block.reset();
+    return true;
+}
+
 bool HipSession::apply_pending(DeviceTensor *t, SessionError *err) {
+    if (!flush_add(t, err)) return false;
     if (t->pending_op < 0) return true;
     if (t->pending_op == PENDING_ATTENTION)  // callers that know the value's id flush it instead (flush_attention)
         return fail(err, SessionError::Message, "internal: a deferred attention product was read by an operator that cannot finish it");
@@ -234,6 +247,7 @@ bool HipSession::run_attention_tail(const Op &op, const std::vector<DeviceTensor
 // a Transpose that keeps the last axis writes its result directly in that Transpose's layout.
 void HipSession::plan_views(bool fused_attention) {
     const auto users = model_.get_value_users();
+    const auto parents = model_.get_value_parents();
     const Graph &g = model_.graph;
     auto is_output = [&](ValueId v) { return std::find(g.outputs.begin(), g.outputs.end(), v) != g.outputs.end(); };
     std::function<bool(ValueId, int)> view_ok = [&](ValueId v, int depth) -> bool {
@@ -272,6 +286,28 @@ void HipSession::plan_views(bool fused_attention) {
             bool elsewhere = false;
             for (size_t i = 1; i < mm.inputs.size(); i++) elsewhere = elsewhere || mm.inputs[i] == n.outputs[0];
             if (!elsewhere) deferred_unary_.insert(id);
+        } else if (n.op.kind == OpKind::LayerNormalization && n.outputs.size() == 1 && n.inputs.size() == 3 && !is_output(n.outputs[0])) {
+            // LayerNormalization read only by a product with a weight matrix: it can write that product's operand planes.
+            auto it = users.find(n.outputs[0]);
+            if (it == users.end() || it->second.size() != 1) continue;
+            const Node &mm = g.nodes[*it->second.begin()];
+            if (mm.op.kind != OpKind::MatMul || mm.inputs.size() < 2 || mm.inputs[0] != n.outputs[0] || mm.op.trans_a) continue;
+            bool elsewhere = false;
+            for (size_t i = 1; i < mm.inputs.size(); i++) elsewhere = elsewhere || mm.inputs[i] == n.outputs[0];
+            auto w = g.inits.find(mm.inputs[1]);
+            if (elsewhere || w == g.inits.end() || w->second.dims().len() != 2 || w->second.elem_ty() != TensorElemType::F32) continue;
+            PlanesPlan pp;
+            pp.consumer = *it->second.begin();
+            pp.next_n = mm.op.trans_b ? w->second.dims()[0] : w->second.dims()[1];
+            planes_out_[id] = pp;
+            planes_consumer_.insert(pp.consumer);
+            // The residual Add in front of it (two tensors of one shape) can leave its sum to this kernel.
+            auto par = parents.find(n.inputs[0]);
+            if (par != parents.end()) {
+                const Node &add = g.nodes[par->second];
+                if (add.op.kind == OpKind::Add && add.inputs.size() == 2 && add.outputs.size() == 1 && add.inputs[0] != add.inputs[1])
+                    add_into_ln_[par->second] = id;
+            }
         } else if (n.op.kind == OpKind::MatMul && n.outputs.size() == 1 && !is_output(n.outputs[0])) {
             auto it = users.find(n.outputs[0]);
             if (it == users.end() || it->second.size() != 1) continue;

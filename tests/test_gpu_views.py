@@ -459,3 +459,79 @@ def test_attention_triples_that_stay_three_operators(case, why):
     q, k, v = (RNG.standard_normal((kw["batch"], kw["heads"], t, kw["d"])).astype(np.float32) for t in (kw["tq"], kw["tk"], kw["tk"]))
     outs, avoided = run_both(m, [q, k, v], attention=True)          # bit for bit: nothing may have changed
     assert avoided == 0, avoided
+
+
+# ---- LayerNormalization (with the residual Add in front) writing the next product's operand planes ----
+
+def residual_norm_block(rows, hidden, n_out, with_add, sum_read_again, ln_second_reader=False):
+    """x (+ r) -> LayerNormalization -> MatMul(weights) [+ bias]; optionally the sum is read again behind (the next
+    residual connection of a transformer block), or the normalised tensor has a second reader."""
+    m = Model(opset_version=17)
+    shape = list(rows) + [hidden]
+    x = m.new_val_named_and_shaped("x", shape)
+    m.add_input(x)
+    s = x
+    if with_add:
+        r = m.new_val_named_and_shaped("r", shape)
+        m.add_input(r)
+        s = node(m, Op.Add, [x, r])
+    gamma = (1.0 + 0.1 * RNG.standard_normal(hidden)).astype(np.float32)
+    beta = (0.1 * RNG.standard_normal(hidden)).astype(np.float32)
+    w = (RNG.standard_normal((hidden, n_out)) * 0.1).astype(np.float32)
+    b = RNG.standard_normal(n_out).astype(np.float32)
+    y = node(m, Op.LayerNormalization, [s, m.new_initializer(gamma), m.new_initializer(beta)], axis=-1, epsilon=1e-5)
+    p = node(m, Op.Add, [node(m, Op.MatMul, [y, m.new_initializer(w)]), m.new_initializer(b)])
+    m.add_output(p)
+    if sum_read_again:
+        m.add_output(node(m, Op.Mul, [s, s]))
+    if ln_second_reader:
+        m.add_output(node(m, Op.Relu if hasattr(Op, "Relu") else Op.ReLU, [y]))
+    m.fuse_matmul_bias()
+    return m, (gamma, beta, w, b)
+
+
+@pytest.mark.parametrize("rows,hidden", [((3, 50), 768), ((300,), 256), ((2, 17), 1024), ((40,), 512), ((5, 7), 128)])
+@pytest.mark.parametrize("with_add,sum_read_again", [(False, False), (True, False), (True, True)])
+def test_layernorm_writes_the_operand_planes_of_the_product_behind_it(case, rows, hidden, with_add, sum_read_again):
+    """On the bf16 route a LayerNormalization whose only reader is a product with a weight matrix writes that
+    product's operand planes instead of fp32 values, and the residual Add in front of it leaves its sum to the same
+    kernel.  Every bit must be that of the separate operators (views off: Add, LayerNormalization, operand split)."""
+    case(f"Add {with_add} -> LayerNormalization -> MatMul, rows {rows}, hidden {hidden}, sum read again {sum_read_again}")
+    m, (gamma, beta, w, b) = residual_norm_block(rows, hidden, 96, with_add, sum_read_again)
+    feeds = [RNG.standard_normal(list(rows) + [hidden]).astype(np.float32) for _ in range(2 if with_add else 1)]
+    outs = []
+    for views in (True, False):
+        sess = HipSessionBuilder(m.clone()).with_gemm_algorithm(D.GEMM_BF16X3).with_strided_views(views).build()
+        for _ in range(2):
+            got = [np.array(t) for t in sess.run([Tensor.from_numpy(x) for x in feeds])]
+        outs.append(got)
+        # rows of 128 have no wavefront-per-row layout: the separate kernels run; otherwise the operand split is
+        # saved, and with it the Add's own pass
+        fits = hidden != 128
+        assert sess.copies_avoided() == ((1 + (1 if with_add else 0)) if views and fits else 0)
+        sess.close()
+    for a, c in zip(*outs):
+        assert_bits_equal(a, c, "planes written by LayerNormalization vs separate operators")
+    s = feeds[0].astype(np.float64) + (feeds[1] if with_add else 0)
+    mu, var = s.mean(-1, keepdims=True), s.var(-1, keepdims=True)
+    want = ((s - mu) / np.sqrt(var + 1e-5) * gamma + beta) @ w.astype(np.float64) + b
+    np.testing.assert_allclose(outs[0][0], want, rtol=1e-4, atol=1e-4)
+    if sum_read_again:
+        np.testing.assert_allclose(outs[0][1], s * s, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("why", ["row length without a wavefront layout", "second reader of the normalised tensor", "fp32 route"])
+def test_layernorm_planes_fall_back(case, why):
+    case(f"LayerNormalization -> MatMul without planes: {why}")
+    hidden = 200 if why.startswith("row length") else 256
+    m, _ = residual_norm_block((30,), hidden, 64, True, True, ln_second_reader=why.startswith("second reader"))
+    feeds = [RNG.standard_normal((30, hidden)).astype(np.float32) for _ in range(2)]
+    algo = D.GEMM_FP32 if why == "fp32 route" else D.GEMM_BF16X3
+    outs = []
+    for views in (True, False):
+        sess = HipSessionBuilder(m.clone()).with_gemm_algorithm(algo).with_strided_views(views).build()
+        outs.append([np.array(t) for t in sess.run([Tensor.from_numpy(x) for x in feeds])])
+        assert sess.copies_avoided() == 0
+        sess.close()
+    for a, c in zip(*outs):
+        assert_bits_equal(a, c, why)
