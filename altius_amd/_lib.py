@@ -204,6 +204,7 @@ def _declare_graph(L):
     f("ahip_session_builder_with_fused_attention", [c_void_p, c_int])
     f("ahip_session_builder_with_strided_views", [c_void_p, c_int])
     f("ahip_session_copies_avoided", [c_void_p, P(c_size_t)])
+    f("ahip_session_lanes", [c_void_p, P(c_size_t)])
     f("ahip_session_graph_replays", [c_void_p, P(c_size_t)])
     f("ahip_session_builder_build", [c_void_p, P(c_void_p)])
     f("ahip_session_free", [c_void_p], None)

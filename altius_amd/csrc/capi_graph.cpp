@@ -1,5 +1,7 @@
 // C ABI: graph IR, analysis, fusion passes, host tensors and the session.
+#include <condition_variable>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 
@@ -31,11 +33,79 @@ struct ahip_session_builder {
     bool strided_views = true;
     bool fused_attention = false;
 };
+// InterpreterSession::run takes &self and keeps its intermediates in a map per calling thread
+// (crates/session_interpreter/src/session.rs:56,75-78), so several threads may run one session at once.  Here a
+// HipSession is one stream, one buffer pool and one set of uploaded initializers, used by one call at a time; a
+// session therefore holds several of them ("lanes"): lane 0 is built with the session, further ones from the same
+// model and switches the first time a call finds every lane busy.
+constexpr size_t MAX_LANES = 16;
 struct ahip_session {
-    std::shared_ptr<HipSession> s;  // shared with the device tensors the session has handed out
+    std::shared_ptr<HipSession> s;  // lane 0; shared with the device tensors the session has handed out
     ahip_model view;  // what ahip_session_model hands out (a copy of the session's model)
     std::vector<std::pair<std::string, double>> profile;
+    ahip_session_builder settings;                    // to build further lanes (its model is left empty: `view` holds it)
+    std::mutex lanes_mutex;                           // guards lanes, busy, building and profile
+    std::condition_variable lane_freed;
+    std::vector<std::shared_ptr<HipSession>> lanes;   // lanes[0] == s
+    std::vector<bool> busy;
+    size_t building = 0;                              // lanes under construction
 };
+
+namespace {
+
+int fail(int code, const std::string &msg);
+
+// A lane nobody is using: a free one, a newly built one while fewer than MAX_LANES exist, else whichever frees up first.
+// The lane comes back as a pointer of its own, since another thread may grow `lanes` while this one runs.
+int acquire_lane(ahip_session *session, size_t *index, std::shared_ptr<HipSession> *lane_out) {
+    std::unique_lock<std::mutex> lock(session->lanes_mutex);
+    for (;;) {
+        for (size_t i = 0; i < session->lanes.size(); i++)
+            if (!session->busy[i]) {
+                session->busy[i] = true;
+                *index = i;
+                *lane_out = session->lanes[i];
+                return AHIP_OK;
+            }
+        if (session->lanes.size() + session->building < MAX_LANES) break;
+        session->lane_freed.wait(lock);
+    }
+    session->building++;
+    lock.unlock();
+    const ahip_session_builder &b = session->settings;
+    HipSessionBuilder hb(session->view.m);
+    hb.with_intra_op_num_threads(b.threads).with_profiling_enabled(b.profiling).with_device(b.device).with_graph_replay(b.graph_replay)
+        .with_gemm_algorithm(b.gemm_algorithm).with_strided_views(b.strided_views).with_fused_attention(b.fused_attention);
+    SessionError err;
+    std::shared_ptr<HipSession> lane = hb.build(&err);
+    lock.lock();
+    session->building--;
+    if (!lane) {
+        session->lane_freed.notify_all();
+        return fail(err.code(), "ahip_session_run: could not build another lane for a concurrent call: " + err.to_string());
+    }
+    session->lanes.push_back(lane);
+    session->busy.push_back(true);
+    *index = session->lanes.size() - 1;
+    *lane_out = std::move(lane);
+    return AHIP_OK;
+}
+
+// The device-resident calls keep their tensors in lane 0's pool and order their work on lane 0's stream.
+void acquire_first_lane(ahip_session *session) {
+    std::unique_lock<std::mutex> lock(session->lanes_mutex);
+    while (session->busy[0]) session->lane_freed.wait(lock);
+    session->busy[0] = true;
+}
+
+void release_lane(ahip_session *session, size_t index, bool keep_profile) {
+    std::lock_guard<std::mutex> lock(session->lanes_mutex);
+    if (keep_profile) session->profile.assign(session->lanes[index]->last_profile().begin(), session->lanes[index]->last_profile().end());
+    session->busy[index] = false;
+    session->lane_freed.notify_all();
+}
+
+}  // namespace
 
 struct ahip_device_tensor {
     DeviceTensor t;
@@ -584,7 +654,23 @@ int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **ses
     if (!out) return fail(AHIP_ERR_OOM, "ahip_session_builder_build: out of host memory");
     out->view.m = s->model();
     out->s = std::move(s);
+    out->settings.threads = builder->threads;
+    out->settings.profiling = builder->profiling;
+    out->settings.device = builder->device;
+    out->settings.graph_replay = builder->graph_replay;
+    out->settings.gemm_algorithm = builder->gemm_algorithm;
+    out->settings.strided_views = builder->strided_views;
+    out->settings.fused_attention = builder->fused_attention;
+    out->lanes.push_back(out->s);
+    out->busy.push_back(false);
     *session = out;
+    return AHIP_OK;
+}
+
+int ahip_session_lanes(ahip_session *session, size_t *count) {
+    if (!session || !count) return fail(AHIP_ERR_ARG, "ahip_session_lanes: null argument");
+    std::lock_guard<std::mutex> lock(session->lanes_mutex);
+    *count = session->lanes.size();
     return AHIP_OK;
 }
 
@@ -602,7 +688,12 @@ int ahip_session_run(ahip_session *session, int n_inputs, const ahip_tensor *con
     }
     std::vector<Tensor> out;
     SessionError err;
-    if (!session->s->run(in, &out, &err)) return fail(err.code(), err.to_string());
+    size_t lane_index = 0;
+    std::shared_ptr<HipSession> lane;
+    if (const int rc = acquire_lane(session, &lane_index, &lane)) return rc;
+    const bool ok = lane->run(in, &out, &err);
+    release_lane(session, lane_index, ok);
+    if (!ok) return fail(err.code(), err.to_string());
     *n_outputs = (int)out.size();
     if ((int)out.size() > output_capacity) return fail(AHIP_ERR_ARG, "ahip_session_run: output capacity too small");
     for (size_t i = 0; i < out.size(); i++) {
@@ -614,7 +705,6 @@ int ahip_session_run(ahip_session *session, int n_inputs, const ahip_tensor *con
         t->t = std::move(out[i]);
         outputs[i] = t;
     }
-    session->profile.assign(session->s->last_profile().begin(), session->s->last_profile().end());
     return AHIP_OK;
 }
 
@@ -637,7 +727,10 @@ int ahip_session_run_device(ahip_session *session, int n_inputs, const void *con
     }
     std::vector<DeviceTensor> out;
     SessionError err;
-    if (!session->s->run_device(in, &out, &err)) return fail(err.code(), err.to_string());
+    acquire_first_lane(session);
+    const bool ok = session->s->run_device(in, &out, &err);
+    release_lane(session, 0, false);
+    if (!ok) return fail(err.code(), err.to_string());
     *n_outputs = (int)out.size();
     auto drop_all = [&](size_t made) {
         for (size_t j = 0; j < made; j++) delete outputs[j];

@@ -126,6 +126,13 @@ class HipSession:
         check(self.L.ahip_session_copies_avoided(self.handle, ctypes.byref(c)))
         return c.value
 
+    def lanes(self):
+        """Streams (each with a buffer pool and a copy of the initializers) the session holds so far: 1 until two
+        run() calls have overlapped."""
+        c = ctypes.c_size_t()
+        check(self.L.ahip_session_lanes(self.handle, ctypes.byref(c)))
+        return c.value
+
     def device_allocations(self):
         c = ctypes.c_size_t()
         check(self.L.ahip_session_device_allocations(self.handle, ctypes.byref(c)))

@@ -609,6 +609,8 @@ int ahip_session_builder_with_fused_attention(ahip_session_builder *builder, int
 /* Nodes of the last node-by-node run that were served without their copy (views taken, transposed layouts
  * written in place). */
 int ahip_session_copies_avoided(const ahip_session *session, size_t *count);
+/* Lanes the session holds so far (1 until two ahip_session_run calls have overlapped). */
+int ahip_session_lanes(ahip_session *session, size_t *count);
 /* build(): shape inference (AHIP_ERR_SHAPE on failure), execution plan, device context,
  * upload of the initializers.  The builder stays valid and must still be freed. */
 int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **session);
@@ -616,8 +618,13 @@ int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **ses
 void ahip_session_free(ahip_session *session);
 /* run(inputs): inputs are bound to graph.inputs in order; outputs come back in
  * graph.outputs order as new tensors the caller frees.  *n_outputs gets their
- * number; AHIP_ERR_ARG if output_capacity is too small.  Calls on one session
- * are serialised internally. */
+ * number; AHIP_ERR_ARG if output_capacity is too small.  Like
+ * InterpreterSession::run(&self), which keeps its values in a map per calling
+ * thread (crates/session_interpreter/src/session.rs:56,75-78), it may be called
+ * from several threads at once: a session holds up to 16 lanes (a stream, a
+ * buffer pool and a copy of the initializers each), builds a further one the first
+ * time a call finds all of them busy, and queues calls beyond 16.  The profile
+ * read back afterwards is that of the call that finished last. */
 int ahip_session_run(ahip_session *session, int n_inputs, const ahip_tensor *const *inputs,
                      int output_capacity, ahip_tensor **outputs, int *n_outputs);
 /* Not in the reference (its tensors are host memory): the same run on tensors that already live on

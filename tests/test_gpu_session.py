@@ -398,12 +398,13 @@ def test_softmax_with_absorbed_scale_and_mask(case, shape, mask_shape, scale_kin
 
 def test_run_from_several_threads(case):
     """InterpreterSession::run takes &self and may be called from several threads at once (per-thread value maps,
-    session.rs:52-58).  Here concurrent calls on one session are serialised internally, and sessions of different
-    threads run side by side on their own streams; every call must return its own inputs' result."""
+    session.rs:52-58).  Here a session gives each of the calls that overlap a lane of its own (stream, buffer pool,
+    initializers), and sessions of different threads run side by side as well; every call must return its own
+    inputs' result."""
     import threading
 
     case("session: concurrent run() calls")
-    c = synth.cfg2(batch=1)
+    c = synth.cfg2(batch=16)
     m = Model()
     x = m.new_val_named_and_shaped("x", c["x"].shape)
     out, _, _ = layer_norm_chain(m, x, c["gamma"], c["beta"], eps=float(c["eps"]))
@@ -413,10 +414,13 @@ def test_run_from_several_threads(case):
     inputs = [synth.normal(300 + i, c["x"].shape, std=1.0 + i) for i in range(4)]
     want = [oracle_ln_chain(v, c["gamma"], c["beta"], c["eps"]) for v in inputs]
     errors = []
+    start = threading.Barrier(4)
+    assert shared.lanes() == 1
 
     def worker(i, own_session):
         try:
             sess = HipSessionBuilder(m.clone()).build() if own_session else shared
+            start.wait()
             for _ in range(8):
                 (got,) = sess.run([inputs[i]])
                 assert_close(got, want[i], what=f"thread {i}")
@@ -430,6 +434,11 @@ def test_run_from_several_threads(case):
         for t in threads:
             t.join()
     assert not errors, errors
+    # 32 calls of a few milliseconds each, started together from four threads, overlapped at least once
+    assert 2 <= shared.lanes() <= 4, shared.lanes()
+    (alone,) = shared.run([inputs[0]])
+    assert_close(alone, want[0], what="a call after the threads have gone")
+    assert 2 <= shared.lanes() <= 4
 
 
 # ---- what a session built with no switches returns -----------------------------------------------
