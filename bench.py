@@ -11,11 +11,16 @@ one "step" is one pass of the four kernels over device-resident fp32 inputs
 
 `value` is the whole step's algorithmic bytes (every tensor read or written once) divided by
 the step time, in GB/s.  Per-kernel times are measured with HIP events on the stream the
-kernels run on; `roofline` describes the slowest kernel of the step.  The CPU baseline is the
-oracle (a C++ restatement of the reference interpreter's kernels) timed on this machine's host
-cores on a reduced batch of the same workload.
+kernels run on (mean, median and minimum over at least 100 launches after 20 warm-ups, and once
+more inside the running step); `roofline` describes the slowest kernel of the step.  Beside the
+step the line carries every other operator of the path on the step's [256,197,768] array
+(`listed_ops`), Softmax / LayerNormalization / ReduceMean by row length (`row_sweep`) and the
+kernels and graphs of configs[0..3] (`other_configs`).  The CPU baseline is the oracle (a C++
+restatement of the reference interpreter's kernels) timed on this machine's host cores on the same
+workload, with 16 threads and with 1, allocating its outputs per call as the reference does and
+writing into existing ones.
 
-Prints one JSON line on stdout; a per-kernel table goes to stderr.
+Prints one JSON line on stdout; the tables go to stderr.
 """
 import argparse
 import json
