@@ -46,7 +46,9 @@ struct GemmArgs {
     uint32_t batch_inner;
     // Single-batch launches are one-dimensional: consecutive block ids go to the eight XCDs in turn, and
     // each XCD (one L2) is given a contiguous run of tiles, so the blocks it runs together share panels.
-    uint32_t tiles_n, tiles, chunk;  // chunk = 0: the grid is (n tiles, m tiles, batches)
+    // Within that order tiles go by groups of group_n tile columns, each group walked row of tiles by row of tiles,
+    // so that the blocks an XCD runs together cover few columns of B (they stay in its L2) and many rows of A.
+    uint32_t tiles_n, tiles_m, tiles, chunk, group_n;  // chunk = 0: the grid is (n tiles, m tiles, batches)
     float alpha, beta;
     int a_vec, b_vec;  // 16-byte loads are legal for this operand (alignment of base, strides, batch stride)
 };
@@ -148,7 +150,9 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_mfma(GemmArgs g) {
     if (g.chunk) {
         const uint32_t tile = (blockIdx.x & 7) * g.chunk + (blockIdx.x >> 3);
         if (tile >= g.tiles) return;
-        tile_m = tile / g.tiles_n, tile_n = tile % g.tiles_n;
+        const uint32_t per_group = g.tiles_m * g.group_n, grp = tile / per_group, r = tile - grp * per_group;
+        const uint32_t width = min(g.group_n, g.tiles_n - grp * g.group_n);  // the last group may be narrower
+        tile_m = r / width, tile_n = grp * g.group_n + r % width;
     }
     const uint32_t m0 = tile_m * BM, n0 = tile_n * TN;
     const uint32_t zo = blockIdx.z / g.batch_inner, zi = blockIdx.z % g.batch_inner;
@@ -360,7 +364,15 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
     g.a_vec = aligned16(a) && lda % 4 == 0 && a_batch_strides[0] % 4 == 0 && a_batch_strides[1] % 4 == 0;
     g.b_vec = aligned16(b) && ldb % 4 == 0 && b_batch_strides[0] % 4 == 0 && b_batch_strides[1] % 4 == 0;
     g.tiles_n = (uint32_t)gx;
+    g.tiles_m = (uint32_t)gy;
     g.tiles = (uint32_t)(gx * gy);
+    {
+        // Groups of about 768 columns (measured on [50432,768]x[768,2304..3072] and 4096^3 .. 8192^3: widths of
+        // 6 to 16 tile columns are within 1 % of each other and up to 3 % ahead of whole rows of tiles; a single
+        // column is 3-6 % behind), all groups equally wide.
+        const size_t group = std::max<size_t>(1, 768 / tn), groups = (gx + group - 1) / group;
+        g.group_n = (uint32_t)((gx + groups - 1) / groups);
+    }
     g.chunk = batch == 1 && gx * gy >= 64 && gx * gy < lim / 8 ? (uint32_t)((gx * gy + 7) / 8) : 0;
     const dim3 grid = g.chunk ? dim3(g.chunk * 8) : dim3((unsigned)gx, (unsigned)gy, (unsigned)batch);
     const bool a_kc = !trans_a, b_kc = trans_b != 0;
