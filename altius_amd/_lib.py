@@ -97,6 +97,7 @@ def _declare(L):
     f("ahip_attention", [c_void_p] * 5 + [c_size_t] * 9 + [P(c_size_t)] * 4 + [c_int, c_float, c_void_p, c_size_t])
     f("ahip_gemm_set_algorithm", [c_void_p, c_int])
     f("ahip_set_streaming_threshold", [c_void_p, c_size_t])
+    f("ahip_set_load_streaming_threshold", [c_void_p, c_size_t])
     f("ahip_gemm_in_kernel_k_cut", [c_void_p, P(c_int), P(c_int)])
     f("ahip_gemm_set_in_kernel_k_cut", [c_void_p, c_int])
     f("ahip_xcd_round_robin_holds", [c_int, P(ctypes.c_uint32), c_size_t])

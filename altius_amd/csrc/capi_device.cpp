@@ -331,6 +331,12 @@ int ahip_set_streaming_threshold(ahip_ctx *ctx, size_t bytes) {
     return AHIP_OK;
 }
 
+int ahip_set_load_streaming_threshold(ahip_ctx *ctx, size_t bytes) {
+    REQUIRE_CTX(ctx, "ahip_set_load_streaming_threshold");
+    ctx->d.nt_load_threshold_bytes = bytes;
+    return AHIP_OK;
+}
+
 int ahip_xcd_round_robin_holds(int cu_count, const uint32_t *xcc_of_block, size_t n_blocks) {
     return altius::xcd_round_robin_holds(cu_count, xcc_of_block, n_blocks) ? 1 : 0;
 }

@@ -43,7 +43,7 @@ constexpr int BLOCK = 256;
 // ---------------------------------------------------------------------------
 // Flat kernel: both operands are FULL or SCALAR.  One float4 per lane.
 // ---------------------------------------------------------------------------
-template <class OP, int MA, int MB, bool NT>
+template <class OP, int MA, int MB, bool NT, bool NTL = NT>
 __global__ __launch_bounds__(BLOCK) void binary_flat_vec4(float *__restrict__ out,
                                                           const float *__restrict__ a,
                                                           const float *__restrict__ b, size_t n) {
@@ -53,8 +53,8 @@ __global__ __launch_bounds__(BLOCK) void binary_flat_vec4(float *__restrict__ ou
     if (MA == SCALAR) sa = a[0];
     if (MB == SCALAR) sb = b[0];
     if (i < n4) {
-        const float4 x = MA == FULL ? load4<NT>(a + 4 * i) : make_float4(sa, sa, sa, sa);
-        const float4 y = MB == FULL ? load4<NT>(b + 4 * i) : make_float4(sb, sb, sb, sb);
+        const float4 x = MA == FULL ? load4<NTL>(a + 4 * i) : make_float4(sa, sa, sa, sa);
+        const float4 y = MB == FULL ? load4<NTL>(b + 4 * i) : make_float4(sb, sb, sb, sb);
         float4 r;
         r.x = OP::f(x.x, y.x);
         r.y = OP::f(x.y, y.y);
@@ -220,7 +220,7 @@ struct RowBcast {
     uint32_t total; // N * R * C
 };
 
-template <class OP, bool SMALL_IS_A, bool NT>
+template <class OP, bool SMALL_IS_A, bool NT, bool NTL = NT>
 __global__ __launch_bounds__(BLOCK) void binary_rowbcast(float *__restrict__ out, const float *__restrict__ full,
                                                          const float *__restrict__ small, const RowBcast g) {
     extern __shared__ float rows_lds[];  // two rows of C floats
@@ -232,7 +232,7 @@ __global__ __launch_bounds__(BLOCK) void binary_rowbcast(float *__restrict__ out
     const uint32_t i0 = block_start + threadIdx.x * 4;
     const bool whole = i0 + 4 <= g.total;
     float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (whole) x = load4<NT>(full + i0);
+    if (whole) x = load4<NTL>(full + i0);
     {
         // Row n_first, and the next one only if this block really reaches into it.
         uint32_t block_last = block_start + BLOCK * 4 - 1;
@@ -288,13 +288,13 @@ enum { SMALL_VECTOR = 0, SMALL_VECTOR_OUTER = 1, SMALL_COLUMN = 2, SMALL_COLUMN_
 
 // c: the row length.  o: elements per outer index (SMALL_VECTOR_OUTER) or the number of values the rows cycle
 // through (SMALL_COLUMN_MOD); unused otherwise.
-template <class OP, int KIND, bool SMALL_IS_A, bool NT>
+template <class OP, int KIND, bool SMALL_IS_A, bool NT, bool NTL = NT>
 __global__ __launch_bounds__(BLOCK) void binary_rows4(float *__restrict__ out, const float *__restrict__ full,
                                                       const float *__restrict__ small, uint32_t total,
                                                       const FastDiv c, const FastDiv o) {
     const uint32_t i0 = (blockIdx.x * BLOCK + threadIdx.x) * 4;
     if (i0 >= total) return;  // total is a multiple of 4
-    const float4 x = load4<NT>(full + i0);
+    const float4 x = load4<NTL>(full + i0);
     const uint32_t row = c.div(i0);
     float4 y;
     if (KIND == SMALL_VECTOR) {
@@ -352,12 +352,15 @@ __global__ __launch_bounds__(BLOCK) void binary_rows_any(float *__restrict__ out
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <class OP, int MA, int MB>
-void flat_dispatch(hipStream_t s, float *out, const float *a, const float *b, size_t n, bool vec, bool nt) {
+void flat_dispatch(hipStream_t s, float *out, const float *a, const float *b, size_t n, bool vec, bool nt, bool ntl) {
     if (vec) {
         size_t blocks = ((n >> 2) + BLOCK - 1) / BLOCK;
         if (blocks == 0) blocks = 1;
         if (nt)
             hipLaunchKernelGGL((binary_flat_vec4<OP, MA, MB, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s,
+                               out, a, b, n);
+        else if (ntl)
+            hipLaunchKernelGGL((binary_flat_vec4<OP, MA, MB, false, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s,
                                out, a, b, n);
         else
             hipLaunchKernelGGL((binary_flat_vec4<OP, MA, MB, false>), dim3((unsigned)blocks), dim3(BLOCK), 0, s,
@@ -371,11 +374,11 @@ void flat_dispatch(hipStream_t s, float *out, const float *a, const float *b, si
 
 template <class OP>
 void flat_launch(hipStream_t s, int ma, int mb, float *out, const float *a, const float *b, size_t n, bool vec,
-                 bool nt) {
-    if (ma == FULL && mb == FULL) flat_dispatch<OP, FULL, FULL>(s, out, a, b, n, vec, nt);
-    else if (ma == FULL && mb == SCALAR) flat_dispatch<OP, FULL, SCALAR>(s, out, a, b, n, vec, nt);
-    else if (ma == SCALAR && mb == FULL) flat_dispatch<OP, SCALAR, FULL>(s, out, a, b, n, vec, nt);
-    else flat_dispatch<OP, SCALAR, SCALAR>(s, out, a, b, n, vec, nt);
+                 bool nt, bool ntl) {
+    if (ma == FULL && mb == FULL) flat_dispatch<OP, FULL, FULL>(s, out, a, b, n, vec, nt, ntl);
+    else if (ma == FULL && mb == SCALAR) flat_dispatch<OP, FULL, SCALAR>(s, out, a, b, n, vec, nt, ntl);
+    else if (ma == SCALAR && mb == FULL) flat_dispatch<OP, SCALAR, FULL>(s, out, a, b, n, vec, nt, ntl);
+    else flat_dispatch<OP, SCALAR, SCALAR>(s, out, a, b, n, vec, nt, false);
 }
 
 template <class OP, int RANK>
@@ -404,30 +407,34 @@ void strided_launch(hipStream_t s, int rank, float *out, const float *a, const f
 }
 
 template <class OP>
-void rowbcast_launch(hipStream_t s, bool small_is_a, bool nt, float *out, const float *full, const float *small,
+void rowbcast_launch(hipStream_t s, bool small_is_a, bool nt, bool ntl, float *out, const float *full, const float *small,
                      const RowBcast &g) {
     const dim3 grid((g.total + BLOCK * 4 - 1) / (BLOCK * 4));
     const size_t shmem = (size_t)2 * g.c.d * sizeof(float);
     if (small_is_a) {
         if (nt) hipLaunchKernelGGL((binary_rowbcast<OP, true, true>), grid, dim3(BLOCK), shmem, s, out, full, small, g);
+        else if (ntl) hipLaunchKernelGGL((binary_rowbcast<OP, true, false, true>), grid, dim3(BLOCK), shmem, s, out, full, small, g);
         else hipLaunchKernelGGL((binary_rowbcast<OP, true, false>), grid, dim3(BLOCK), shmem, s, out, full, small, g);
     } else {
         if (nt) hipLaunchKernelGGL((binary_rowbcast<OP, false, true>), grid, dim3(BLOCK), shmem, s, out, full, small, g);
+        else if (ntl) hipLaunchKernelGGL((binary_rowbcast<OP, false, false, true>), grid, dim3(BLOCK), shmem, s, out, full, small, g);
         else hipLaunchKernelGGL((binary_rowbcast<OP, false, false>), grid, dim3(BLOCK), shmem, s, out, full, small, g);
     }
 }
 
 template <class OP, int KIND>
-void rows4_launch_kind(hipStream_t s, bool small_is_a, bool nt, float *out, const float *full, const float *small, uint32_t total,
+void rows4_launch_kind(hipStream_t s, bool small_is_a, bool nt, bool ntl, float *out, const float *full, const float *small, uint32_t total,
                        const FastDiv &c, const FastDiv &o) {
     const dim3 grid((total / 4 + BLOCK - 1) / BLOCK);
-#define ALTIUS_ROWS4(A, N) hipLaunchKernelGGL((binary_rows4<OP, KIND, A, N>), grid, dim3(BLOCK), 0, s, out, full, small, total, c, o)
+#define ALTIUS_ROWS4(A, N, L) hipLaunchKernelGGL((binary_rows4<OP, KIND, A, N, L>), grid, dim3(BLOCK), 0, s, out, full, small, total, c, o)
     if (small_is_a) {
-        if (nt) ALTIUS_ROWS4(true, true);
-        else ALTIUS_ROWS4(true, false);
+        if (nt) ALTIUS_ROWS4(true, true, true);
+        else if (ntl) ALTIUS_ROWS4(true, false, true);
+        else ALTIUS_ROWS4(true, false, false);
     } else {
-        if (nt) ALTIUS_ROWS4(false, true);
-        else ALTIUS_ROWS4(false, false);
+        if (nt) ALTIUS_ROWS4(false, true, true);
+        else if (ntl) ALTIUS_ROWS4(false, false, true);
+        else ALTIUS_ROWS4(false, false, false);
     }
 #undef ALTIUS_ROWS4
 }
@@ -451,13 +458,13 @@ void rows_any_launch(hipStream_t s, bool mod, bool small_is_a, bool nt, float *o
 }
 
 template <class OP>
-void rows4_launch(hipStream_t s, int kind, bool small_is_a, bool nt, float *out, const float *full, const float *small,
+void rows4_launch(hipStream_t s, int kind, bool small_is_a, bool nt, bool ntl, float *out, const float *full, const float *small,
                   uint32_t total, const FastDiv &c, const FastDiv &o) {
     switch (kind) {
-    case SMALL_VECTOR: rows4_launch_kind<OP, SMALL_VECTOR>(s, small_is_a, nt, out, full, small, total, c, o); break;
-    case SMALL_VECTOR_OUTER: rows4_launch_kind<OP, SMALL_VECTOR_OUTER>(s, small_is_a, nt, out, full, small, total, c, o); break;
-    case SMALL_COLUMN: rows4_launch_kind<OP, SMALL_COLUMN>(s, small_is_a, nt, out, full, small, total, c, o); break;
-    default: rows4_launch_kind<OP, SMALL_COLUMN_MOD>(s, small_is_a, nt, out, full, small, total, c, o); break;
+    case SMALL_VECTOR: rows4_launch_kind<OP, SMALL_VECTOR>(s, small_is_a, nt, ntl, out, full, small, total, c, o); break;
+    case SMALL_VECTOR_OUTER: rows4_launch_kind<OP, SMALL_VECTOR_OUTER>(s, small_is_a, nt, ntl, out, full, small, total, c, o); break;
+    case SMALL_COLUMN: rows4_launch_kind<OP, SMALL_COLUMN>(s, small_is_a, nt, ntl, out, full, small, total, c, o); break;
+    default: rows4_launch_kind<OP, SMALL_COLUMN_MOD>(s, small_is_a, nt, ntl, out, full, small, total, c, o); break;
     }
 }
 
@@ -520,17 +527,17 @@ int launch_binary(DeviceCtx &ctx, int op, float *out, const float *a, const floa
 
     hipStream_t s = ctx.stream;
     if (total > ((size_t)1 << 38)) return ctx.fail(AHIP_ERR_UNSUPPORTED, "binary: more than 2^38 elements");
-    const bool nt = ctx.streaming(total * sizeof(float));
+    const bool nt = ctx.streaming(total * sizeof(float)), ntl = ctx.streaming_loads(total * sizeof(float));
     if (ma != STRIDED && mb != STRIDED) {
         const bool vec = aligned16(out) && (ma != FULL || aligned16(a)) && (mb != FULL || aligned16(b));
         switch (op) {
-        case AHIP_ADD: flat_launch<OpAdd>(s, ma, mb, out, a, b, total, vec, nt); break;
-        case AHIP_SUB: flat_launch<OpSub>(s, ma, mb, out, a, b, total, vec, nt); break;
-        case AHIP_MUL: flat_launch<OpMul>(s, ma, mb, out, a, b, total, vec, nt); break;
-        case AHIP_DIV: flat_launch<OpDiv>(s, ma, mb, out, a, b, total, vec, nt); break;
+        case AHIP_ADD: flat_launch<OpAdd>(s, ma, mb, out, a, b, total, vec, nt, ntl); break;
+        case AHIP_SUB: flat_launch<OpSub>(s, ma, mb, out, a, b, total, vec, nt, ntl); break;
+        case AHIP_MUL: flat_launch<OpMul>(s, ma, mb, out, a, b, total, vec, nt, ntl); break;
+        case AHIP_DIV: flat_launch<OpDiv>(s, ma, mb, out, a, b, total, vec, nt, ntl); break;
         case AHIP_POW:
-            if (square) flat_launch<OpPowScalarExp>(s, ma, mb, out, a, b, total, vec, nt);
-            else flat_launch<OpPow>(s, ma, mb, out, a, b, total, vec, nt);
+            if (square) flat_launch<OpPowScalarExp>(s, ma, mb, out, a, b, total, vec, nt, ntl);
+            else flat_launch<OpPow>(s, ma, mb, out, a, b, total, vec, nt, ntl);
             break;
         }
         return ctx.check(hipGetLastError(), "binary flat launch");
@@ -569,11 +576,11 @@ int launch_binary(DeviceCtx &ctx, int op, float *out, const float *a, const floa
             const float *full = small_is_a ? b : a;
             const float *small = small_is_a ? a : b;
             switch (op) {
-            case AHIP_ADD: rowbcast_launch<OpAdd>(s, small_is_a, nt, out, full, small, rb); break;
-            case AHIP_SUB: rowbcast_launch<OpSub>(s, small_is_a, nt, out, full, small, rb); break;
-            case AHIP_MUL: rowbcast_launch<OpMul>(s, small_is_a, nt, out, full, small, rb); break;
-            case AHIP_DIV: rowbcast_launch<OpDiv>(s, small_is_a, nt, out, full, small, rb); break;
-            case AHIP_POW: rowbcast_launch<OpPow>(s, small_is_a, nt, out, full, small, rb); break;
+            case AHIP_ADD: rowbcast_launch<OpAdd>(s, small_is_a, nt, ntl, out, full, small, rb); break;
+            case AHIP_SUB: rowbcast_launch<OpSub>(s, small_is_a, nt, ntl, out, full, small, rb); break;
+            case AHIP_MUL: rowbcast_launch<OpMul>(s, small_is_a, nt, ntl, out, full, small, rb); break;
+            case AHIP_DIV: rowbcast_launch<OpDiv>(s, small_is_a, nt, ntl, out, full, small, rb); break;
+            case AHIP_POW: rowbcast_launch<OpPow>(s, small_is_a, nt, ntl, out, full, small, rb); break;
             }
             return ctx.check(hipGetLastError(), "binary row-broadcast launch");
         }
@@ -597,11 +604,11 @@ int launch_binary(DeviceCtx &ctx, int op, float *out, const float *a, const floa
             (!vector || aligned16(small))) {
             const FastDiv c = make_fastdiv((uint32_t)dims[r - 1]), o = make_fastdiv(second);
             switch (op) {
-            case AHIP_ADD: rows4_launch<OpAdd>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
-            case AHIP_SUB: rows4_launch<OpSub>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
-            case AHIP_MUL: rows4_launch<OpMul>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
-            case AHIP_DIV: rows4_launch<OpDiv>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
-            case AHIP_POW: rows4_launch<OpPow>(s, kind, small_is_a, nt, out, full, small, (uint32_t)total, c, o); break;
+            case AHIP_ADD: rows4_launch<OpAdd>(s, kind, small_is_a, nt, ntl, out, full, small, (uint32_t)total, c, o); break;
+            case AHIP_SUB: rows4_launch<OpSub>(s, kind, small_is_a, nt, ntl, out, full, small, (uint32_t)total, c, o); break;
+            case AHIP_MUL: rows4_launch<OpMul>(s, kind, small_is_a, nt, ntl, out, full, small, (uint32_t)total, c, o); break;
+            case AHIP_DIV: rows4_launch<OpDiv>(s, kind, small_is_a, nt, ntl, out, full, small, (uint32_t)total, c, o); break;
+            case AHIP_POW: rows4_launch<OpPow>(s, kind, small_is_a, nt, ntl, out, full, small, (uint32_t)total, c, o); break;
             }
             return ctx.check(hipGetLastError(), "binary row-aligned broadcast launch");
         }

@@ -660,11 +660,13 @@ struct BlockLayout {
     int threads, nch;
 };
 // Measured over rows of 2048 to 16384 elements: two float4 per thread is the best shape (256 x 2 for 2048, 512 x 2
-// for 4096, 1024 x 2 for 8192: 77-80 % of peak for Softmax), three cost little, and a 16 K row has to take four
-// (requested two at a time).
+// for 4096, 1024 x 2 for 6144 and 8192: 77-80 % of peak for Softmax), three cost little (512 x 3 for 5120, 1024 x 3
+// for 12288: 78-79 %), and a 16 K row has to take four, requested two at a time (72 %; all four at once costs
+// LayerNormalization 5 points).  Fewer threads with more float4 each (512 x 4..8, 256 x 5..16) are 3-8 points behind
+// at every length from 5120 up.
 inline BlockLayout block_layout(size_t len) {
     const size_t v = len / 4;  // float4 per row
-    const int threads = v <= 512 ? 256 : v <= 1536 ? 512 : 1024;
+    const int threads = v <= 512 ? 256 : v <= 1280 ? 512 : 1024;
     return BlockLayout{threads, (int)((v + threads - 1) / threads)};
 }
 

@@ -49,13 +49,16 @@ constexpr int BLOCK = 256;
 
 // One float4 per lane: on this part a streaming kernel is fastest with the
 // smallest per-lane footprint and the occupancy that comes with it.
-template <class F, bool NT>
+// NT: non-temporal stores (and loads) for tensors too large to be found in a cache by the next kernel.  NTL alone:
+// non-temporal loads of a mid-sized input that nobody reads again, while the result is stored the ordinary way so
+// that the next kernel finds it in the Infinity Cache.
+template <class F, bool NT, bool NTL = NT>
 __global__ __launch_bounds__(BLOCK) void unary_vec4(float *__restrict__ out, const float *__restrict__ in,
                                                     size_t n, F f) {
     const size_t n4 = n >> 2;
     const size_t i = (size_t)blockIdx.x * BLOCK + threadIdx.x;
     if (i < n4) {
-        const float4 v = load4<NT>(in + 4 * i);
+        const float4 v = load4<NTL>(in + 4 * i);
         float4 r;
         r.x = f(v.x);
         r.y = f(v.y);
@@ -76,13 +79,15 @@ __global__ __launch_bounds__(BLOCK) void unary_scalar(float *__restrict__ out, c
     if (i < n) out[i] = f(in[i]);
 }
 
-template <class F> void launch(hipStream_t s, float *out, const float *in, size_t n, F f, bool nt) {
+template <class F> void launch(hipStream_t s, float *out, const float *in, size_t n, F f, bool nt, bool ntl) {
     const bool vec = ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(in)) & 15u) == 0;
     if (vec) {
         size_t blocks = ((n >> 2) + BLOCK - 1) / BLOCK;
         if (blocks == 0) blocks = 1;
         if (nt)
             hipLaunchKernelGGL((unary_vec4<F, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, n, f);
+        else if (ntl)
+            hipLaunchKernelGGL((unary_vec4<F, false, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, n, f);
         else
             hipLaunchKernelGGL((unary_vec4<F, false>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, n, f);
     } else {
@@ -98,20 +103,20 @@ int launch_unary(DeviceCtx &ctx, int op, float *out, const float *in, size_t n, 
     if (n == 0) return AHIP_OK;
     if (!out || !in) return ctx.fail(AHIP_ERR_ARG, "unary: null tensor pointer");
     if (n > ((size_t)1 << 38)) return ctx.fail(AHIP_ERR_UNSUPPORTED, "unary: more than 2^38 elements");
-    const bool nt = ctx.streaming(n * sizeof(float));
+    const bool nt = ctx.streaming(n * sizeof(float)), ntl = ctx.streaming_loads(n * sizeof(float));
     switch (op) {
-    case AHIP_SQRT: launch(ctx.stream, out, in, n, FSqrt{}, nt); break;
-    case AHIP_ERF: launch(ctx.stream, out, in, n, FErf{}, nt); break;
-    case AHIP_GELU: launch(ctx.stream, out, in, n, FGelu{}, nt); break;
-    case AHIP_SIGMOID: launch(ctx.stream, out, in, n, FSigmoid{}, nt); break;
-    case AHIP_HARDSIGMOID: launch(ctx.stream, out, in, n, FHardSigmoid{alpha, beta}, nt); break;
-    case AHIP_RELU: launch(ctx.stream, out, in, n, FRelu{}, nt); break;
-    case AHIP_TANH: launch(ctx.stream, out, in, n, FTanh{}, nt); break;
-    case AHIP_LEAKYRELU: launch(ctx.stream, out, in, n, FLeakyRelu{alpha}, nt); break;
-    case AHIP_EXP: launch(ctx.stream, out, in, n, FExp{}, nt); break;
-    case AHIP_ROUND: launch(ctx.stream, out, in, n, FRound{}, nt); break;
-    case AHIP_CLIP: launch(ctx.stream, out, in, n, FClip{alpha, beta}, nt); break;
-    case AHIP_DIV_BY: launch(ctx.stream, out, in, n, FDivBy{alpha}, nt); break;
+    case AHIP_SQRT: launch(ctx.stream, out, in, n, FSqrt{}, nt, ntl); break;
+    case AHIP_ERF: launch(ctx.stream, out, in, n, FErf{}, nt, ntl); break;
+    case AHIP_GELU: launch(ctx.stream, out, in, n, FGelu{}, nt, ntl); break;
+    case AHIP_SIGMOID: launch(ctx.stream, out, in, n, FSigmoid{}, nt, ntl); break;
+    case AHIP_HARDSIGMOID: launch(ctx.stream, out, in, n, FHardSigmoid{alpha, beta}, nt, ntl); break;
+    case AHIP_RELU: launch(ctx.stream, out, in, n, FRelu{}, nt, ntl); break;
+    case AHIP_TANH: launch(ctx.stream, out, in, n, FTanh{}, nt, ntl); break;
+    case AHIP_LEAKYRELU: launch(ctx.stream, out, in, n, FLeakyRelu{alpha}, nt, ntl); break;
+    case AHIP_EXP: launch(ctx.stream, out, in, n, FExp{}, nt, ntl); break;
+    case AHIP_ROUND: launch(ctx.stream, out, in, n, FRound{}, nt, ntl); break;
+    case AHIP_CLIP: launch(ctx.stream, out, in, n, FClip{alpha, beta}, nt, ntl); break;
+    case AHIP_DIV_BY: launch(ctx.stream, out, in, n, FDivBy{alpha}, nt, ntl); break;
     }
     return ctx.check(hipGetLastError(), "unary launch");
 }

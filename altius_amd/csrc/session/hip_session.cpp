@@ -121,6 +121,8 @@ std::unique_ptr<HipSession> HipSessionBuilder::build(SessionError *err) {
         fail_code(err, rc, derr);
         return nullptr;
     }
+    // Every input of a node was written by the node in front and is, up to the size of the caches, still in them.
+    s->ctx_.nt_load_threshold_bytes = s->ctx_.nt_threshold_bytes;
     if (gemm_algorithm_ != AHIP_GEMM_AUTO && gemm_algorithm_ != AHIP_GEMM_FP32 && gemm_algorithm_ != AHIP_GEMM_BF16X3) {
         destroy_device_ctx(&s->ctx_);
         fail(err, SessionError::Argument, "unknown GEMM algorithm");

@@ -455,6 +455,10 @@ class Context:
         """Tensors of at least this many bytes are streamed with non-temporal accesses."""
         check(self.L.ahip_set_streaming_threshold(self.handle, int(nbytes)), self.handle)
 
+    def set_load_streaming_threshold(self, nbytes):
+        """Element-wise operators read dense operands of at least this many bytes with non-temporal loads."""
+        check(self.L.ahip_set_load_streaming_threshold(self.handle, int(nbytes)), self.handle)
+
     def gemm_in_kernel_k_cut(self):
         """(placement shown, cut enabled): whether the probe at context creation found block i on XCD i % 8, and
         whether the bf16 GEMM's in-kernel k cut is switched on.  The cut runs only when both hold."""

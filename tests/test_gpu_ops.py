@@ -95,6 +95,31 @@ def test_binary_bit_exact(ctx, oracle, case, name, sa, sb):
     assert_bits_equal(expected, ref.astype(np.float32), f"oracle vs numpy {name}")
 
 
+@pytest.mark.parametrize("threshold", [0, 2**64 - 1])
+def test_streamed_loads_change_no_bit(oracle, case, threshold):
+    """Dense operands of at least `ahip_set_load_streaming_threshold` bytes are read with non-temporal loads while the
+    result is stored the ordinary way: the same values either way, for every element-wise kernel that has the variant
+    (flat, a row staged in LDS, a vector / column beside rows of float4s, unary)."""
+    case(f"element-wise operators with the load streaming threshold at {threshold}")
+    c = D.Context(0)
+    try:
+        c.set_load_streaming_threshold(threshold)
+        for sa, sb in [([3, 1, 10], [3, 1, 10]), ([16, 3, 224, 224], [16, 3, 224, 224]), ([3, 28, 28], []), ([4, 12, 197, 197], [4, 1, 1, 197]),
+                       ([3, 1, 30], [3, 40, 30]), ([8, 197, 768], [768]), ([8, 197, 1], [8, 197, 768]), ([2, 3, 8, 8], [3, 1, 1]),
+                       ([2, 4, 10, 1028], [2, 1, 1, 1028])]:
+            a = synth.uniform(21, sa) + np.float32(0.25)
+            b = synth.uniform(22, sb) + np.float32(0.25)
+            for name, (op, oop) in BIN.items():
+                assert_bits_equal(c.binary(op, a, b), oracle.binary(oop, a, b), f"{name} {sa} {sb} threshold {threshold}")
+        x = synth.normal(23, [4, 197, 3072], std=2.0)
+        for name, (op, oop) in UNARY.items():
+            v = np.abs(x) if name == "Sqrt" else x
+            alpha, beta = (1.0 / 6.0, 0.5) if name == "HardSigmoid" else (0.0, 0.0)
+            assert_bits_equal(c.unary(op, v, alpha, beta), oracle.unary(oop, v, alpha, beta), f"{name} threshold {threshold}")
+    finally:
+        c.close()
+
+
 def test_binary_known_answer(ctx, case):
     """[1,3,...,15] + [2,4,...,16] = [3,7,...,31] (crates/session/tests/ort.rs:17-25)."""
     case("binary KAT")
