@@ -24,6 +24,7 @@
 #include "common.h"
 #include "ctx.h"
 #include "math.h"
+#include "split3.h"
 
 namespace altius {
 
@@ -181,6 +182,224 @@ __global__ __launch_bounds__(64 * W, W == 8 ? 4 : 1) void attention_stream_d64(A
             }
         }
         if (more) park(vs[buf ^ 1], D);
+        __syncthreads();  // the next chunk is in place, and nobody reads this one any more
+    }
+
+    if (active && query < g.tq) {
+        sum += __shfl_xor(sum, 32);
+        const float recip = 1.0f / sum;
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; g4++) {
+                const f32x4 out = {acc[t][4 * g4] * recip, acc[t][4 * g4 + 1] * recip, acc[t][4 * g4 + 2] * recip, acc[t][4 * g4 + 3] * recip};
+                *reinterpret_cast<f32x4 *>(o + (size_t)query * g.ldo + 32 * t + 8 * g4 + 4 * h) = out;
+            }
+    }
+}
+
+// ---------------------------------------------------------------- the same on the bf16 matrix cores
+// Both products with every fp32 operand value as the exact sum of three bf16 numbers and six
+// v_mfma_f32_32x32x16_bf16 per k step (the scheme of gemm_split.hip): 48 MFMAs of 8 passes per tile of 32 keys
+// instead of 64 fp32 MFMAs of 16 passes.  K and V are split once per block on their way into LDS, Q once per
+// wavefront into registers; the probabilities are split where they are, in the accumulator registers of S^T, whose
+// layout is again the B operand's: half-wave h supplies the 8 k slots of a 16-key step from accumulator registers
+// 8 u .. 8 u + 7, i.e. keys 16 u + 8 (i / 4) + 4 h + i % 4, and V^T is laid out in LDS in that key order.
+// Keys go through LDS 32 at a time, double-buffered: 57 KiB, two blocks per CU.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int KCB = 32;       // keys per chunk (one tile)
+constexpr int KB_PITCH = 72;  // 16-bit words per K row in LDS: 64 d and a pad that spreads 16-byte reads of 16 rows over all banks
+constexpr int VB_PITCH = 40;  // 16-bit words per V^T row (one d): 32 key slots and a pad, likewise
+
+#define ALTIUS_MFMA_BF16(A, B, C) \
+    C = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, A), __builtin_bit_cast(bf16x8, B), C, 0, 0, 0)
+
+// Smallest terms first.
+__device__ __forceinline__ void six_products(const u32x4 (&a)[3], const u32x4 &b0, const u32x4 &b1, const u32x4 &b2, floatx16 &c) {
+    ALTIUS_MFMA_BF16(a[0], b2, c);
+    ALTIUS_MFMA_BF16(a[2], b0, c);
+    ALTIUS_MFMA_BF16(a[1], b1, c);
+    ALTIUS_MFMA_BF16(a[0], b1, c);
+    ALTIUS_MFMA_BF16(a[1], b0, c);
+    ALTIUS_MFMA_BF16(a[0], b0, c);
+}
+
+// Two probabilities (in [0, 1]: no rounding up to infinity, no NaN payloads to keep) as three pairs of bf16.
+__device__ __forceinline__ void split_pair(float e0, float e1, uint32_t &p0, uint32_t &p1, uint32_t &p2) {
+    p0 = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){e0, e1}, bf16x2));
+    const float r0 = e0 - __uint_as_float(p0 << 16), r1 = e1 - __uint_as_float(p0 & 0xffff0000u);
+    p1 = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){r0, r1}, bf16x2));
+    const float s0 = r0 - __uint_as_float(p1 << 16), s1 = r1 - __uint_as_float(p1 & 0xffff0000u);
+    p2 = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){s0, s1}, bf16x2));
+}
+
+// Two operand values likewise.  The hardware conversion rounds to nearest even like dev::split3; a value that it
+// rounds up to infinity, an infinity or a NaN (exponent bits all ones in the first plane) takes split3's route, which
+// truncates the first, and keeps the other two out of the lower planes.
+__device__ __forceinline__ void split_operand_pair(float x0, float x1, uint32_t &p0, uint32_t &p1, uint32_t &p2) {
+    split_pair(x0, x1, p0, p1, p2);
+    if (__builtin_expect(((p0 & 0x7f80u) == 0x7f80u) | ((p0 & 0x7f800000u) == 0x7f800000u), 0)) {
+        uint32_t a[3], b[3];
+        dev::split3(x0, a[0], a[1], a[2]);
+        dev::split3(x1, b[0], b[1], b[2]);
+        p0 = a[0] | (b[0] << 16), p1 = a[1] | (b[1] << 16), p2 = a[2] | (b[2] << 16);
+    }
+}
+
+// kp / vp: this chunk's planes in LDS; qp[plane][k step]: the wavefront's queries.
+// FULL: every key of the tile exists.  SCALE_OP and MASK are the launch's, so that the sixteen scores of a lane go
+// through straight-line code.
+template <bool FULL, int SCALE_OP, bool MASK>
+__device__ __forceinline__ void attend_tile_bf16(float scale, uint32_t tk, const float *__restrict__ mask, const uint16_t *kp,
+                                                 const uint16_t *vp, uint32_t key_base, const u32x4 (&qp)[3][4], int h, int lr, float &mx,
+                                                 float &sum, floatx16 (&acc)[2]) {
+    floatx16 st;
+#pragma unroll
+    for (int r = 0; r < 16; r++) st[r] = 0.0f;
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        u32x4 kf[3];
+#pragma unroll
+        for (int p = 0; p < 3; p++) kf[p] = *reinterpret_cast<const u32x4 *>(kp + p * (KCB * KB_PITCH) + lr * KB_PITCH + 16 * s + 8 * h);
+        six_products(kf, qp[0][s], qp[1][s], qp[2][s], st);
+    }
+    float cmax = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const uint32_t key = key_base + 8 * (r >> 2) + 4 * h + (r & 3);
+        float x = st[r];
+        if (SCALE_OP == 1) x = x * scale;
+        else if (SCALE_OP == 2) x = x / scale;
+        if (MASK && (FULL || key < tk)) x = x + mask[key];
+        st[r] = x;
+        if (FULL || key < tk) cmax = dev::nanmax(cmax, x);
+    }
+    cmax = dev::nanmax(cmax, __shfl_xor(cmax, 32));
+    const float mnew = dev::nanmax(mx, cmax);
+    if (mnew != mx) {  // what has been summed so far was taken relative to the old maximum
+        const float corr = mx == -INFINITY ? 0.0f : dev::softmax_exp(mx, mnew);
+        sum *= corr;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[0][r] *= corr, acc[1][r] *= corr;
+        mx = mnew;
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const uint32_t key = key_base + 8 * (r >> 2) + 4 * h + (r & 3);
+        const float e = (FULL || key < tk) ? dev::softmax_exp(st[r], mx) : 0.0f;
+        st[r] = e;
+        sum += e;
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        u32x4 pf[3];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            uint32_t p0, p1, p2;
+            split_pair(st[8 * u + 2 * i], st[8 * u + 2 * i + 1], p0, p1, p2);
+            pf[0][i] = p0, pf[1][i] = p1, pf[2][i] = p2;
+        }
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            u32x4 vf[3];
+#pragma unroll
+            for (int p = 0; p < 3; p++)
+                vf[p] = *reinterpret_cast<const u32x4 *>(vp + p * (D * VB_PITCH) + (32 * t + lr) * VB_PITCH + (2 * u + h) * 8);
+            six_products(vf, pf[0], pf[1], pf[2], acc[t]);
+        }
+    }
+}
+
+template <int SCALE_OP, bool MASK>
+__global__ __launch_bounds__(512, 2) void attention_stream_d64_bf16(AttnArgs g) {
+    constexpr int W = 8;
+    __shared__ __align__(16) uint16_t kps[2][3 * KCB * KB_PITCH];
+    __shared__ __align__(16) uint16_t vps[2][3 * D * VB_PITCH];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int h = lane >> 5, lr = lane & 31;
+    const uint32_t zo = blockIdx.x / g.batch_inner, zi = blockIdx.x % g.batch_inner;
+    const float *q = g.q + zo * g.q_bs[0] + zi * g.q_bs[1];
+    const float *k = g.k + zo * g.k_bs[0] + zi * g.k_bs[1];
+    const float *v = g.v + zo * g.v_bs[0] + zi * g.v_bs[1];
+    float *o = g.o + zo * g.o_bs[0] + zi * g.o_bs[1];
+    const float *mask = g.mask ? g.mask + (size_t)zo * g.mask_outer_stride : nullptr;
+    const uint32_t query = (blockIdx.y * W + wave) * 32 + lr;
+    const bool active = (blockIdx.y * W + wave) * 32 < g.tq;  // wavefronts without queries still help staging
+    const uint32_t nchunks = (g.tk + KCB - 1) / KCB;
+
+    // Staging: thread (key r0, float4 c4) moves one float4 of K and one of V per chunk.
+    const uint32_t r0 = tid >> 4, c4 = tid & 15;
+    // Where key r0 sits in a V^T row: group (u, h) of 8 slots, slot i within it (see above).
+    const uint32_t vslot = ((r0 >> 4) * 2 + ((r0 & 7) >> 2)) * 8 + 4 * ((r0 & 15) >> 3) + (r0 & 3);
+    f32x4 kst, vst;
+    auto fetch = [&](uint32_t chunk) {
+        const uint32_t row = chunk * KCB + r0;
+        kst = vst = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        if (row < g.tk) {
+            kst = *reinterpret_cast<const f32x4 *>(k + (size_t)row * g.ldk + c4 * 4);
+            vst = *reinterpret_cast<const f32x4 *>(v + (size_t)row * g.ldv + c4 * 4);
+        }
+    };
+    auto park = [&](int buf) {
+        uint32_t hk[3][2], hv[3][2];
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            split_operand_pair(kst[2 * e], kst[2 * e + 1], hk[0][e], hk[1][e], hk[2][e]);
+            split_operand_pair(vst[2 * e], vst[2 * e + 1], hv[0][e], hv[1][e], hv[2][e]);
+        }
+#pragma unroll
+        for (int p = 0; p < 3; p++) {
+            *reinterpret_cast<u32x2 *>(&kps[buf][p * (KCB * KB_PITCH) + r0 * KB_PITCH + 4 * c4]) = u32x2{hk[p][0], hk[p][1]};
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                vps[buf][p * (D * VB_PITCH) + (4 * c4 + e) * VB_PITCH + vslot] = (uint16_t)(e & 1 ? hv[p][e >> 1] >> 16 : hv[p][e >> 1]);
+        }
+    };
+    fetch(0);
+    park(0);
+
+    u32x4 qp[3][4];
+    if (active && query < g.tq) {
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            const float *src = q + (size_t)query * g.ldq + 16 * s + 8 * h;
+            const f32x4 lo = *reinterpret_cast<const f32x4 *>(src), hi = *reinterpret_cast<const f32x4 *>(src + 4);
+            uint32_t hq[3][4];
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                split_operand_pair(lo[2 * e], lo[2 * e + 1], hq[0][e], hq[1][e], hq[2][e]);
+                split_operand_pair(hi[2 * e], hi[2 * e + 1], hq[0][2 + e], hq[1][2 + e], hq[2][2 + e]);
+            }
+#pragma unroll
+            for (int p = 0; p < 3; p++) qp[p][s] = u32x4{hq[p][0], hq[p][1], hq[p][2], hq[p][3]};
+        }
+    } else {
+#pragma unroll
+        for (int p = 0; p < 3; p++)
+#pragma unroll
+            for (int s = 0; s < 4; s++) qp[p][s] = u32x4{0u, 0u, 0u, 0u};
+    }
+    __syncthreads();
+
+    float mx = -INFINITY, sum = 0.0f;
+    floatx16 acc[2];
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[0][r] = 0.0f, acc[1][r] = 0.0f;
+
+    for (uint32_t c = 0; c < nchunks; c++) {
+        const int buf = c & 1;
+        const bool more = c + 1 < nchunks;
+        if (more) fetch(c + 1);  // in flight during the tile
+        if (active) {
+            if ((c + 1) * KCB <= g.tk) attend_tile_bf16<true, SCALE_OP, MASK>(g.scale, g.tk, mask, kps[buf], vps[buf], c * KCB, qp, h, lr, mx, sum, acc);
+            else attend_tile_bf16<false, SCALE_OP, MASK>(g.scale, g.tk, mask, kps[buf], vps[buf], c * KCB, qp, h, lr, mx, sum, acc);
+        }
+        if (more) park(buf ^ 1);
         __syncthreads();  // the next chunk is in place, and nobody reads this one any more
     }
 
@@ -359,7 +578,21 @@ int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, c
     size_t w = MAX_WAVES;
     while (w > 2 && batch * ((q_tiles + w - 1) / w) < cus) w /= 2;
     const dim3 grid((unsigned)batch, (unsigned)((q_tiles + w - 1) / w));
-    if (w == 8) hipLaunchKernelGGL(attention_stream_d64<8>, grid, dim3(512), 0, ctx.stream, g);
+    // Where products may take the bf16 matrix cores (an infinite operand then gives NaN, as in the GEMM on that
+    // route), full blocks do.
+    if (w == 8 && ctx.gemm_algorithm != AHIP_GEMM_FP32) {
+#define ALTIUS_ATT(S, M) hipLaunchKernelGGL((attention_stream_d64_bf16<S, M>), grid, dim3(512), 0, ctx.stream, g)
+        if (mask) {
+            if (scale_op == 0) ALTIUS_ATT(0, true);
+            else if (scale_op == 1) ALTIUS_ATT(1, true);
+            else ALTIUS_ATT(2, true);
+        } else {
+            if (scale_op == 0) ALTIUS_ATT(0, false);
+            else if (scale_op == 1) ALTIUS_ATT(1, false);
+            else ALTIUS_ATT(2, false);
+        }
+#undef ALTIUS_ATT
+    } else if (w == 8) hipLaunchKernelGGL(attention_stream_d64<8>, grid, dim3(512), 0, ctx.stream, g);
     else if (w == 4) hipLaunchKernelGGL(attention_stream_d64<4>, grid, dim3(256), 0, ctx.stream, g);
     else hipLaunchKernelGGL(attention_stream_d64<2>, grid, dim3(128), 0, ctx.stream, g);
     return ctx.check(hipGetLastError(), "attention launch");

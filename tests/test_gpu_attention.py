@@ -135,3 +135,83 @@ def test_keys_split_over_wavefronts_with_empty_and_masked_parts(ctx, case):
         s = q.astype(np.float64) @ np.swapaxes(k.astype(np.float64), -1, -2) / 8.0 + mask
         e = np.exp(s - s.max(-1, keepdims=True))
         np.testing.assert_allclose(got, (e / e.sum(-1, keepdims=True)) @ v, rtol=2e-4, atol=2e-5, err_msg=f"tk {tk}")
+
+
+# ---- the same kernel on the bf16 matrix cores (contexts whose products may take that route) --------------------------
+
+@pytest.fixture()
+def bf16_ctx():
+    from altius_amd import device as D
+
+    c = D.Context(0)
+    c.gemm_set_algorithm(D.GEMM_BF16X3)
+    yield c
+    c.close()
+
+
+@pytest.mark.parametrize("heads,tq,tk", [(300, 197, 197), (256, 40, 70), (600, 33, 64), (260, 300, 100), (256, 1, 1), (512, 64, 31),
+                                         (256, 257, 224), (256, 5, 33)])
+@pytest.mark.parametrize("scale_op", [0, 1, 2])
+def test_attention_on_the_bf16_matrix_cores(bf16_ctx, ctx, case, heads, tq, tk, scale_op):
+    """Enough (batch, head) pairs for full blocks: both products run as six bf16 MFMAs per k step on operands split
+    into three bf16 planes (K, V on their way into LDS, Q in registers, the probabilities where the first product
+    leaves them).  Held to the definition in float64 at the fp32 kernel's bars, and to the fp32 kernel itself."""
+    case(f"bf16 attention: {heads} heads, tq {tq}, tk {tk}, scale_op {scale_op}")
+    q = RNG.standard_normal((heads, tq, 64)).astype(np.float32)
+    k = RNG.standard_normal((heads, tk, 64)).astype(np.float32)
+    v = RNG.standard_normal((heads, tk, 64)).astype(np.float32)
+    scale = np.float32(0.125) if scale_op == 1 else np.float32(8.0)
+    mask = np.where(RNG.random(tk) < 0.2, -1e4, 0.0).astype(np.float32) if scale_op else None
+    if mask is not None:
+        mask[0] = 0.0
+    got = bf16_ctx.attention(q, k, v, scale_op, float(scale), mask=mask)
+    s = q.astype(np.float64) @ np.swapaxes(k.astype(np.float64), -1, -2)
+    s = s * scale if scale_op == 1 else s / scale if scale_op == 2 else s
+    if mask is not None:
+        s = s + mask
+    e = np.exp(s - s.max(-1, keepdims=True))
+    np.testing.assert_allclose(got, (e / e.sum(-1, keepdims=True)) @ v, rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(got, ctx.attention(q, k, v, scale_op, float(scale), mask=mask), rtol=2e-4, atol=2e-5)
+
+
+def test_bf16_attention_reads_heads_in_place_with_a_mask_per_batch(bf16_ctx, case):
+    case("bf16 attention on strided heads, one mask row per batch")
+    b, t, h, d = 24, 45, 12, 64
+    x = RNG.standard_normal((b, t, 3 * h * d)).astype(np.float32)
+    mask = np.where(RNG.random((b, t)) < 0.3, -1e4, 0.0).astype(np.float32)
+    mask[:, 0] = 0.0
+    dx, do, dm = bf16_ctx.upload(x), bf16_ctx.alloc(b * t * h * d * 4), bf16_ctx.upload(mask)
+    S = ctypes.c_size_t * 2
+    try:
+        ld = 3 * h * d
+        check(bf16_ctx.L.ahip_attention(bf16_ctx.handle, do.ptr, dx.ptr, dx.ptr + h * d * 4, dx.ptr + 2 * h * d * 4, b, h, t, t, d, ld, ld, ld,
+                                        h * d, S(t * ld, d), S(t * ld, d), S(t * ld, d), S(t * h * d, d), 1, 0.125, dm.ptr, t), bf16_ctx.handle)
+        got = bf16_ctx.download(do, (b, t, h, d))
+    finally:
+        for m in (dx, do, dm):
+            bf16_ctx.free(m)
+    q, k, v = (x[:, :, i * h * d:(i + 1) * h * d].reshape(b, t, h, d).transpose(0, 2, 1, 3) for i in range(3))
+    s = q.astype(np.float64) @ np.swapaxes(k.astype(np.float64), -1, -2) * 0.125 + mask[:, None, None, :]
+    e = np.exp(s - s.max(-1, keepdims=True))
+    np.testing.assert_allclose(got.transpose(0, 2, 1, 3), (e / e.sum(-1, keepdims=True)) @ v, rtol=2e-4, atol=2e-5)
+
+
+def test_bf16_attention_special_values(bf16_ctx, case):
+    """Values the hardware conversion would round up to infinity are truncated (the planes still add up to the value);
+    an exact representation: integer-valued operands give the exact result of the definition wherever the probabilities
+    are exact (one key: probability 1); an infinite operand gives NaN (for most elements; +inf, the fp32 result, for the rest), as in the product on this route."""
+    case("bf16 attention: huge, integer-valued and infinite operands")
+    heads, tq = 256, 40
+    q = RNG.integers(-3, 4, (heads, tq, 64)).astype(np.float32)
+    k = RNG.integers(-3, 4, (heads, 1, 64)).astype(np.float32)
+    v = (RNG.integers(-(2 ** 23), 2 ** 23, (heads, 1, 64))).astype(np.float32)
+    v[0, 0, :4] = [3.4e38, -3.4e38, 3.3895e38, 1e-30]  # (below 2^-109 the third plane runs out of exponent)
+    got = bf16_ctx.attention(q, k, v)
+    np.testing.assert_array_equal(got, np.broadcast_to(v, got.shape))  # one key: O = V, every bit of it
+    k2 = RNG.standard_normal((heads, 70, 64)).astype(np.float32)
+    v2 = RNG.standard_normal((heads, 70, 64)).astype(np.float32)
+    v2[3, 5, 7] = np.inf
+    out = bf16_ctx.attention(q, k2, v2, 1, 0.125)
+    col = out[3, :, 7]  # NaN (inf times a zero lower plane of a probability) or the fp32 kernel's +inf, never a finite number
+    assert (np.isnan(col) | (col == np.inf)).all() and np.isnan(col).mean() > 0.5
+    assert np.isfinite(out[3, :, :7]).all() and np.isfinite(np.delete(out, 3, axis=0)).all()
