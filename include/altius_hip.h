@@ -310,7 +310,9 @@ int ahip_gemm_post(ahip_ctx *ctx, float *c, const float *a, const float *b, cons
  * written into one in place.  scale_op: 0 none, 1 scores * scale, 2 scores / scale.  mask (may be NULL): one value per
  * key, added after the scale, read at mask[(z / batch_inner) * mask_outer_stride + key] (stride 0: one row for all
  * batches; tk: one row per outer batch, the [b, 1, 1, tk] padding mask of BERT-style graphs).  Same exp and
- * reciprocal-multiply normalisation as ahip_softmax_lastaxis; the two products on the fp32 matrix cores.
+ * reciprocal-multiply normalisation as ahip_softmax_lastaxis; the two products on the fp32 matrix cores, or, on a
+ * context set to AHIP_GEMM_AUTO / AHIP_GEMM_BF16X3 and with at least one full block per CU, on the bf16 matrix cores
+ * with every value as three bf16 planes (as accurate; an infinite value in Q, K or V then gives NaN).
  * AHIP_ERR_UNSUPPORTED (nothing launched) unless d == 64 and all pointers, pitches and batch strides are
  * multiples of 16 bytes: run the three operators then.  Any number of keys (they are streamed 64 at a time).  No counterpart in the reference. */
 int ahip_attention(ahip_ctx *ctx, float *o, const float *q, const float *k, const float *v, size_t batch_outer,
