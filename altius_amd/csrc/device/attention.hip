@@ -238,20 +238,6 @@ __device__ __forceinline__ void split_pair(float e0, float e1, uint32_t &p0, uin
     p2 = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){s0, s1}, bf16x2));
 }
 
-// Two operand values likewise.  The hardware conversion rounds to nearest even like dev::split3; a value that it
-// rounds up to infinity, an infinity or a NaN (exponent bits all ones in the first plane) takes split3's route, which
-// truncates the first, and keeps the other two out of the lower planes.
-__device__ __forceinline__ void split_operand_pair(float x0, float x1, uint32_t &p0, uint32_t &p1, uint32_t &p2) {
-    split_pair(x0, x1, p0, p1, p2);
-    if (__builtin_expect(((p0 & 0x7f80u) == 0x7f80u) | ((p0 & 0x7f800000u) == 0x7f800000u), 0)) {
-        uint32_t a[3], b[3];
-        dev::split3(x0, a[0], a[1], a[2]);
-        dev::split3(x1, b[0], b[1], b[2]);
-        p0 = a[0] | (b[0] << 16), p1 = a[1] | (b[1] << 16), p2 = a[2] | (b[2] << 16);
-    }
-}
-
-// kp / vp: this chunk's planes in LDS; qp[plane][k step]: the wavefront's queries.
 // FULL: every key of the tile exists.  SCALE_OP and MASK are the launch's, so that the sixteen scores of a lane go
 // through straight-line code.
 template <bool FULL, int SCALE_OP, bool MASK>
@@ -349,8 +335,8 @@ __global__ __launch_bounds__(512, 2) void attention_stream_d64_bf16(AttnArgs g) 
         uint32_t hk[3][2], hv[3][2];
 #pragma unroll
         for (int e = 0; e < 2; e++) {
-            split_operand_pair(kst[2 * e], kst[2 * e + 1], hk[0][e], hk[1][e], hk[2][e]);
-            split_operand_pair(vst[2 * e], vst[2 * e + 1], hv[0][e], hv[1][e], hv[2][e]);
+            dev::split3_pair(kst[2 * e], kst[2 * e + 1], hk[0][e], hk[1][e], hk[2][e]);
+            dev::split3_pair(vst[2 * e], vst[2 * e + 1], hv[0][e], hv[1][e], hv[2][e]);
         }
 #pragma unroll
         for (int p = 0; p < 3; p++) {
@@ -372,8 +358,8 @@ __global__ __launch_bounds__(512, 2) void attention_stream_d64_bf16(AttnArgs g) 
             uint32_t hq[3][4];
 #pragma unroll
             for (int e = 0; e < 2; e++) {
-                split_operand_pair(lo[2 * e], lo[2 * e + 1], hq[0][e], hq[1][e], hq[2][e]);
-                split_operand_pair(hi[2 * e], hi[2 * e + 1], hq[0][2 + e], hq[1][2 + e], hq[2][2 + e]);
+                dev::split3_pair(lo[2 * e], lo[2 * e + 1], hq[0][e], hq[1][e], hq[2][e]);
+                dev::split3_pair(hi[2 * e], hi[2 * e + 1], hq[0][2 + e], hq[1][2 + e], hq[2][2 + e]);
             }
 #pragma unroll
             for (int p = 0; p < 3; p++) qp[p][s] = u32x4{hq[p][0], hq[p][1], hq[p][2], hq[p][3]};

@@ -34,7 +34,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // ---------------------------------------------------------------- operand -> three bf16 planes
 
-using dev::split3;
+using dev::split3_pair;
 
 // An activation applied to the operand's values on their way into the planes (PRE: 0 none, else an AHIP_* unary
 // code): the product reads f(A) without f(A) ever being stored as fp32.
@@ -47,18 +47,11 @@ __device__ __forceinline__ float pre(float x) {
 
 __device__ __forceinline__ void store_planes(u32x4 *__restrict__ planes, const float (&v)[8], uint32_t row, uint32_t kg, uint32_t rp,
                                              uint32_t kgs) {
-    uint32_t h[3][8];
+    uint32_t h[3][4];
 #pragma unroll
-    for (int j = 0; j < 8; j++) split3(v[j], h[0][j], h[1][j], h[2][j]);
+    for (int j = 0; j < 4; j++) split3_pair(v[2 * j], v[2 * j + 1], h[0][j], h[1][j], h[2][j]);
 #pragma unroll
-    for (int p = 0; p < 3; p++) {
-        u32x4 o;
-        o.x = h[p][0] | (h[p][1] << 16);
-        o.y = h[p][2] | (h[p][3] << 16);
-        o.z = h[p][4] | (h[p][5] << 16);
-        o.w = h[p][6] | (h[p][7] << 16);
-        planes[((size_t)p * kgs + kg) * rp + row] = o;
-    }
+    for (int p = 0; p < 3; p++) planes[((size_t)p * kgs + kg) * rp + row] = u32x4{h[p][0], h[p][1], h[p][2], h[p][3]};
 }
 
 // Any strides: element (row, k) is src[row * s_r + k * s_k].  Consecutive lanes take consecutive rows,
@@ -157,21 +150,21 @@ __global__ __launch_bounds__(LNP_THREADS) void layernorm_planes(u32x4 *__restric
     for (int k = 0; k < NCH; k++) {
         const uint32_t c = lane + 64 * k;  // float4 number: k group c / 2, half c % 2
         if (c < 2 * kgs) {
-            uint32_t h[3][4];
+            uint32_t h[3][2];
+            float y[4];
             const bool live = grow < rows && c < v4;
             f32x4 gm = {0.0f, 0.0f, 0.0f, 0.0f}, bt = {0.0f, 0.0f, 0.0f, 0.0f};
             if (live) gm = *reinterpret_cast<const f32x4 *>(gamma + 4 * c), bt = *reinterpret_cast<const f32x4 *>(beta + 4 * c);
             const float g4[4] = {gm.x, gm.y, gm.z, gm.w}, b4[4] = {bt.x, bt.y, bt.z, bt.w};
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const float y = live ? __builtin_fmaf(v[4 * k + j] * inv_std, g4[j], b4[j]) : 0.0f;
-                split3(y, h[0][j], h[1][j], h[2][j]);
-            }
+            for (int j = 0; j < 4; j++) y[j] = live ? __builtin_fmaf(v[4 * k + j] * inv_std, g4[j], b4[j]) : 0.0f;
+            split3_pair(y[0], y[1], h[0][0], h[1][0], h[2][0]);
+            split3_pair(y[2], y[3], h[0][1], h[1][1], h[2][1]);
 #pragma unroll
             for (int p = 0; p < 3; p++) {
                 uint32_t *dst = lnp_lds + ((size_t)p * kgs + (c >> 1)) * LNP_KG_PITCH + wave * 4 + (c & 1) * 2;
-                dst[0] = h[p][0] | (h[p][1] << 16);
-                dst[1] = h[p][2] | (h[p][3] << 16);
+                dst[0] = h[p][0];
+                dst[1] = h[p][1];
             }
         }
     }

@@ -30,5 +30,24 @@ __device__ __forceinline__ void split3(float x, uint32_t &h0, uint32_t &h1, uint
     h2 = r2 >> 16;
 }
 
+// The same for two values at once with the hardware's float -> bf16 conversion (round to nearest even, like
+// round_bf16): the low half of p_i is x0's plane i, the high half x1's.  A value that the conversion rounds up to
+// infinity, an infinity or a NaN (exponent bits all ones in a first plane) takes split3's route.
+__device__ __forceinline__ void split3_pair(float x0, float x1, uint32_t &p0, uint32_t &p1, uint32_t &p2) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    p0 = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){x0, x1}, bf16x2));
+    const float r0 = x0 - __uint_as_float(p0 << 16), r1 = x1 - __uint_as_float(p0 & 0xffff0000u);
+    p1 = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){r0, r1}, bf16x2));
+    const float s0 = r0 - __uint_as_float(p1 << 16), s1 = r1 - __uint_as_float(p1 & 0xffff0000u);
+    p2 = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){s0, s1}, bf16x2));
+    if (__builtin_expect(((p0 & 0x7f80u) == 0x7f80u) | ((p0 & 0x7f800000u) == 0x7f800000u), 0)) {
+        uint32_t a[3], b[3];
+        split3(x0, a[0], a[1], a[2]);
+        split3(x1, b[0], b[1], b[2]);
+        p0 = a[0] | (b[0] << 16), p1 = a[1] | (b[1] << 16), p2 = a[2] | (b[2] << 16);
+    }
+}
+
 }  // namespace dev
 }  // namespace altius

@@ -464,6 +464,19 @@ def build_next_rows(ctx, D, batch=256):
     gemm("MatMul proj [%d,768]x[768,768]" % M, 1, M, H, H, 0, 0, both)
     gemm("MatMul fc1 [%d,768]x[768,3072]" % M, 1, M, 4 * H, H, 0, 0, both)
     gemm("MatMul fc2 [%d,3072]x[3072,768]" % M, 1, M, H, 4 * H, 0, 0, both)
+    # the MLP's second product with the Gelu in front of it applied while its operand is split (f(A) never stored)
+    ga = ctx.upload(rng.standard_normal((M, 4 * H), dtype=np.float32))
+    gw = ctx.upload(rng.standard_normal((4 * H, H), dtype=np.float32) * np.float32(0.03))
+    gc = ctx.alloc(M * H * 4)
+    ctx.gemm_register_constant(gw)
+
+    def gelu_fc2():
+        ctx.gemm_set_algorithm(D.GEMM_BF16X3)
+        check(L.ahip_gemm_activated(h, D.GELU, gc.ptr, ga.ptr, gw.ptr, None, M, H, 4 * H, 0, 0, 4 * H, H, H, 0, 0, 1.0, 0.0), h)
+        ctx.gemm_set_algorithm(D.GEMM_DEFAULT)
+
+    rows.append(("MatMul Gelu(A) x B, fc2 [%d,3072]x[3072,768] (bf16 x 3 incl. Gelu and split of A)" % M, 4 * (M * 4 * H + 4 * H * H + M * H),
+                 2.0 * M * H * 4 * H, gelu_fc2))
     gemm("MatMul QK^T %d x [197,64]x[64,197]" % (batch * NH), batch * NH, T, T, DH, T * DH, DH * T)
     gemm("MatMul PV %d x [197,197]x[197,64]" % (batch * NH), batch * NH, T, DH, T, T * T, T * DH)
     # QK^T -> scale -> Softmax -> PV in one kernel, heads read in place from the [b, t, 3 h d] result of the qkv product
@@ -473,10 +486,15 @@ def build_next_rows(ctx, D, batch=256):
     att = ctx.alloc(batch * T * H * 4)
     S2 = ctypes.c_size_t * 2
     ld = 3 * H
-    rows.append(("Attention %d x Softmax(QK^T/8)V [197,64], one kernel" % (batch * NH), 4 * batch * T * 4 * H,
-                 2.0 * batch * NH * (2 * T * T * DH),
-                 lambda: check(L.ahip_attention(h, att.ptr, qkv3.ptr, qkv3.ptr + H * 4, qkv3.ptr + 2 * H * 4, batch, NH, T, T, DH, ld, ld, ld, H,
-                                                S2(T * ld, DH), S2(T * ld, DH), S2(T * ld, DH), S2(T * H, DH), 1, 0.125, None, 0), h)))
+    def attention(algo):
+        ctx.gemm_set_algorithm(algo)
+        check(L.ahip_attention(h, att.ptr, qkv3.ptr, qkv3.ptr + H * 4, qkv3.ptr + 2 * H * 4, batch, NH, T, T, DH, ld, ld, ld, H,
+                               S2(T * ld, DH), S2(T * ld, DH), S2(T * ld, DH), S2(T * H, DH), 1, 0.125, None, 0), h)
+        ctx.gemm_set_algorithm(D.GEMM_DEFAULT)
+
+    for label, algo in (("fp32 MFMA", D.GEMM_FP32), ("bf16 x 3", D.GEMM_BF16X3)):
+        rows.append(("Attention %d x Softmax(QK^T/8)V [197,64], one kernel (%s)" % (batch * NH, label), 4 * batch * T * 4 * H,
+                     2.0 * batch * NH * (2 * T * T * DH), lambda algo=algo: attention(algo)))
     return rows
 
 
