@@ -12,8 +12,9 @@
 // that both the GEMM's global reads and its LDS layout are plain contiguous copies.  gemm_bf16x3
 // computes a 256 x 256 tile of C per 512-thread block (8 wavefronts, 64 x 128 each) in k steps of
 // 16 through three LDS buffers that are filled by direct global->LDS loads issued two steps ahead;
-// one barrier per step.  The epilogue transposes the accumulators through LDS so that C is written
-// in whole 512-byte row segments.
+// one barrier per step, with the block's two groups of four wavefronts half a step apart (a SIMD's two
+// wavefronts take turns at the matrix pipe).  The epilogue transposes the accumulators through LDS so that
+// C is written in whole 512-byte row segments.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -228,62 +229,45 @@ __device__ __forceinline__ void issue(Stage &s, const u32x4 *ga, const u32x4 *gb
 #define DS_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off) : "memory")
 #define MFMA(A, B, C) C = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, A), __builtin_bit_cast(bf16x8, B), C, 0, 0, 0)
 
-// Smallest terms first.
-__device__ __forceinline__ void six(const u32x4 (&a)[3], const u32x4 (&b)[3], floatx16 &c) {
-    MFMA(a[0], b[2], c);
-    MFMA(a[2], b[0], c);
-    MFMA(a[1], b[1], c);
-    MFMA(a[0], b[1], c);
-    MFMA(a[1], b[0], c);
-    MFMA(a[0], b[0], c);
+// A wavefront's operands for one stage: 64 x 16 of A and 16 x 128 of B in three planes each, 18 reads of 16 bytes per
+// lane.  They are all requested at once and the 48 MFMAs follow when they have arrived.
+struct Fragments {
+    u32x4 a[2][3], b[4][3];
+};
+
+__device__ __forceinline__ void read_fragments(Fragments &f, uint32_t a_addr, uint32_t b_addr) {
+#pragma unroll
+    for (int p = 0; p < 3; p++) {
+        DS_READ(f.a[0][p], a_addr, 0 + 0);
+        DS_READ(f.a[1][p], a_addr, 512);
+        DS_READ(f.b[0][p], b_addr, 0 + 0);
+        DS_READ(f.b[1][p], b_addr, 512);
+        DS_READ(f.b[2][p], b_addr, 1024);
+        DS_READ(f.b[3][p], b_addr, 1536);
+        a_addr += PLANE_BYTES;
+        b_addr += PLANE_BYTES;
+    }
 }
 
-// a_addr / b_addr: LDS byte addresses of this lane's first A / B fragment in the stage.
-__device__ __forceinline__ void compute(uint32_t a_addr, uint32_t b_addr, floatx16 (&acc)[2][4]) {
-    u32x4 a0[3], a1[3], b0[3], b1[3], b2[3], b3[3];
-    DS_READ(a0[0], a_addr, 0);
-    DS_READ(a0[1], a_addr, PLANE_BYTES);
-    DS_READ(a0[2], a_addr, 2 * PLANE_BYTES);
-    DS_READ(b0[0], b_addr, 0);
-    DS_READ(b0[1], b_addr, PLANE_BYTES);
-    DS_READ(b0[2], b_addr, 2 * PLANE_BYTES);
-    DS_READ(a1[0], a_addr, 512);
-    DS_READ(a1[1], a_addr, PLANE_BYTES + 512);
-    DS_READ(a1[2], a_addr, 2 * PLANE_BYTES + 512);
-    DS_READ(b1[0], b_addr, 512);
-    DS_READ(b1[1], b_addr, PLANE_BYTES + 512);
-    DS_READ(b1[2], b_addr, 2 * PLANE_BYTES + 512);
-    asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(a0[0]), "+v"(a0[1]), "+v"(a0[2]), "+v"(b0[0]), "+v"(b0[1]), "+v"(b0[2]));
-    six(a0, b0, acc[0][0]);
-    asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(a1[0]), "+v"(a1[1]), "+v"(a1[2]));
-    six(a1, b0, acc[1][0]);
-    DS_READ(b2[0], b_addr, 1024);
-    DS_READ(b2[1], b_addr, PLANE_BYTES + 1024);
-    DS_READ(b2[2], b_addr, 2 * PLANE_BYTES + 1024);
-    asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(b1[0]), "+v"(b1[1]), "+v"(b1[2]));
-    six(a0, b1, acc[0][1]);
-    six(a1, b1, acc[1][1]);
-    DS_READ(b3[0], b_addr, 1536);
-    DS_READ(b3[1], b_addr, PLANE_BYTES + 1536);
-    DS_READ(b3[2], b_addr, 2 * PLANE_BYTES + 1536);
-    asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(b2[0]), "+v"(b2[1]), "+v"(b2[2]));
-    six(a0, b2, acc[0][2]);
-    six(a1, b2, acc[1][2]);
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(b3[0]), "+v"(b3[1]), "+v"(b3[2]));
-    six(a0, b3, acc[0][3]);
-    six(a1, b3, acc[1][3]);
+// Smallest terms first for every accumulator; consecutive MFMAs go to different accumulators.
+__device__ __forceinline__ void multiply_fragments(Fragments &f, floatx16 (&acc)[2][4]) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(f.a[0][0]), "+v"(f.a[0][1]), "+v"(f.a[0][2]), "+v"(f.a[1][0]), "+v"(f.a[1][1]), "+v"(f.a[1][2]), "+v"(f.b[0][0]),
+                   "+v"(f.b[0][1]), "+v"(f.b[0][2]), "+v"(f.b[1][0]), "+v"(f.b[1][1]), "+v"(f.b[1][2]), "+v"(f.b[2][0]), "+v"(f.b[2][1]),
+                   "+v"(f.b[2][2]), "+v"(f.b[3][0]), "+v"(f.b[3][1]), "+v"(f.b[3][2]));
+    constexpr int PA[6] = {0, 2, 1, 0, 1, 0}, PB[6] = {2, 0, 1, 1, 0, 0};
+#pragma unroll
+    for (int t = 0; t < 6; t++)
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) MFMA(f.a[i][PA[t]], f.b[j][PB[t]], acc[i][j]);
 }
 
-// Stage t lives in buffer t % 3.  Before stage t is used: this wavefront's six loads of it have
-// landed (those of stage t + 1 may still be in flight), and the barrier says the same of every
-// wavefront and that all of them are done with stage t - 1, whose buffer the loads of stage
-// t + 2 then overwrite.
-__device__ __forceinline__ void step(uint32_t a_addr, uint32_t b_addr, Stage *next2, floatx16 (&acc)[2][4], bool more1, bool more2,
-                                     const u32x4 *ga, const u32x4 *gb, size_t a_plane, size_t b_plane, int sub) {
-    if (more1) asm volatile("s_waitcnt vmcnt(6)\n\ts_barrier" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    if (more2) issue(*next2, ga, gb, a_plane, b_plane, sub);
-    compute(a_addr, b_addr, acc);
+__device__ __forceinline__ void slot_barrier(bool loads_left_in_flight) {
+    // lgkmcnt(0): this wavefront's fragment reads have left LDS before anybody may overwrite the stage.
+    if (loads_left_in_flight) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
 __global__ __launch_bounds__(THREADS, 1) void gemm_bf16x3(SplitGemmArgs g) {
@@ -323,18 +307,28 @@ __global__ __launch_bounds__(THREADS, 1) void gemm_bf16x3(SplitGemmArgs g) {
     const u32x4 *gb = g.bp + first * b_step + (size_t)(wave >> 2) * g.np + n0 + (wave & 3) * 64 + lane;
     issue(S[0], ga, gb, a_plane, b_plane, sub);
     if (nst > 1) issue(S[1], ga + a_step, gb + b_step, a_plane, b_plane, sub);
-#define STEP(CUR, NEXT2)                                                                                              \
-    {                                                                                                                 \
-        step(a_addr + CUR * (uint32_t)sizeof(Stage), b_addr + CUR * (uint32_t)sizeof(Stage), &S[NEXT2], acc, t + 1 < nst, \
-             t + 2 < nst, ga + (t + 2) * a_step, gb + (t + 2) * b_step, a_plane, b_plane, sub);                          \
-        if (++t >= nst) break;                                                                                        \
+    // One barrier per stage.  Between two barriers group 0 (wavefronts 0-3) reads stage t and multiplies it, group 1
+    // multiplies stage t - 1 and reads stage t: wavefronts w and w + 4 share a SIMD, and while one waits for its
+    // fragments the other keeps the matrix pipe busy.  Before barrier t every wavefront's own loads of stage t have
+    // landed and its reads of stage t - 1 have left LDS (slot_barrier), so stage t + 2 may go where stage t - 1 was.
+    Fragments f;
+    if (wave < 4) {
+        for (uint32_t t = 0; t < nst; t++) {
+            slot_barrier(t + 1 < nst);
+            read_fragments(f, a_addr + (t % 3) * (uint32_t)sizeof(Stage), b_addr + (t % 3) * (uint32_t)sizeof(Stage));
+            if (t + 2 < nst) issue(S[(t + 2) % 3], ga + (t + 2) * a_step, gb + (t + 2) * b_step, a_plane, b_plane, sub);
+            multiply_fragments(f, acc);
+        }
+    } else {
+        slot_barrier(nst > 1);
+        for (uint32_t t = 0; t < nst; t++) {
+            if (t > 0) multiply_fragments(f, acc);
+            read_fragments(f, a_addr + (t % 3) * (uint32_t)sizeof(Stage), b_addr + (t % 3) * (uint32_t)sizeof(Stage));
+            if (t + 2 < nst) issue(S[(t + 2) % 3], ga + (t + 2) * a_step, gb + (t + 2) * b_step, a_plane, b_plane, sub);
+            if (t + 1 < nst) slot_barrier(t + 2 < nst);
+        }
+        multiply_fragments(f, acc);
     }
-    for (uint32_t t = 0;;) {
-        STEP(0, 2)
-        STEP(1, 0)
-        STEP(2, 1)
-    }
-#undef STEP
 
     // A tile cut along k: every block leaves its partial sums in `partials` (coalesced 16-byte stores), and the block that arrives last adds them up in slice order, so the result does not
     // depend on who was last, and goes on to the epilogue.  All slices of a tile run on one XCD (one L2).
