@@ -445,6 +445,38 @@ def test_attention_with_a_per_key_mask(case, mask):
     np.testing.assert_allclose(got, (e / e.sum(-1, keepdims=True)) @ v, rtol=2e-4, atol=2e-5)
 
 
+@pytest.mark.parametrize("mask", [False, "keys"])
+def test_attention_of_a_session_on_the_bf16_route(case, mask):
+    """A session whose products may use the bf16 matrix cores (AHIP_GEMM_AUTO) and that has opted in to the one-kernel
+    attention: with enough (batch, head) pairs for full blocks the kernel's two products take that route as well.
+    Compared with the definition and with a default session (fp32 products, three operators)."""
+    case(f"session attention on the bf16 route, mask {mask}")
+    from altius_amd import device as D
+
+    batch, tq, tk, heads = 24, 45, 70, 12
+    m = scaled_attention(batch, tq, tk, heads, 64, "div", mask=mask)
+    q, k, v = (RNG.standard_normal((batch, heads, t, 64)).astype(np.float32) for t in (tq, tk, tk))
+    outs = []
+    for fast in (True, False):
+        b = HipSessionBuilder(m.clone())
+        if fast:
+            b = b.with_gemm_algorithm(D.GEMM_AUTO).with_fused_attention(True)
+        sess = b.build()
+        for _ in range(2):
+            (got,) = [np.array(t) for t in sess.run([Tensor.from_numpy(x) for x in (q, k, v)])]
+        if fast:
+            assert sess.copies_avoided() == 2, sess.copies_avoided()
+        sess.close()
+        outs.append(got)
+    s_ = q.astype(np.float64) @ k.astype(np.float64).transpose(0, 1, 3, 2) / np.float32(8.0)
+    if mask:
+        s_ = s_ + m.mask_values
+    e = np.exp(s_ - s_.max(-1, keepdims=True))
+    want = (e / e.sum(-1, keepdims=True)) @ v
+    np.testing.assert_allclose(outs[0], want, rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(outs[0], outs[1], rtol=2e-4, atol=2e-5)
+
+
 @pytest.mark.parametrize("why", ["narrow heads", "second reader of the probabilities", "mask per query"])
 def test_attention_triples_that_stay_three_operators(case, why):
     case(f"attention not fused: {why}")
