@@ -37,6 +37,8 @@ constexpr int D = 64;          // head width
 constexpr int K_PITCH = 68;    // floats; 16-byte aligned rows whose b128 reads by 8 consecutive rows cover all banks
 constexpr int MAX_WAVES = 8;   // query tiles per block
 
+typedef uint32_t u32x4_attn __attribute__((ext_vector_type(4)));
+
 struct AttnArgs {
     const float *q, *k, *v;
     float *o;
@@ -50,6 +52,10 @@ struct AttnArgs {
     // Added to the scaled scores, one value per key: mask[(z / batch_inner) * mask_outer_stride + key] (null: none).
     const float *mask;
     uint32_t mask_outer_stride;
+    // attention_stream_d64_bf16<.., PLANES>: O, a [batch_outer * tq, batch_inner * 64] matrix, leaves as the three bf16
+    // planes of the first operand of the product that reads it ([plane][k / 8][row][8], o_rp rows, o_kgs k groups).
+    u32x4_attn *o_planes;
+    uint32_t o_rp, o_kgs;
 };
 
 constexpr int KC = 64;  // keys per chunk
@@ -301,7 +307,7 @@ __device__ __forceinline__ void attend_tile_bf16(float scale, uint32_t tk, const
     }
 }
 
-template <int SCALE_OP, bool MASK>
+template <int SCALE_OP, bool MASK, bool PLANES>
 __global__ __launch_bounds__(512, 2) void attention_stream_d64_bf16(AttnArgs g) {
     constexpr int W = 8;
     __shared__ __align__(16) uint16_t kps[2][3 * KCB * KB_PITCH];
@@ -397,7 +403,18 @@ __global__ __launch_bounds__(512, 2) void attention_stream_d64_bf16(AttnArgs g) 
 #pragma unroll
             for (int g4 = 0; g4 < 4; g4++) {
                 const f32x4 out = {acc[t][4 * g4] * recip, acc[t][4 * g4 + 1] * recip, acc[t][4 * g4 + 2] * recip, acc[t][4 * g4 + 3] * recip};
-                *reinterpret_cast<f32x4 *>(o + (size_t)query * g.ldo + 32 * t + 8 * g4 + 4 * h) = out;
+                if (PLANES) {
+                    // The lane's four values are half h of the 16-byte chunk (row zo tq + query, k group 8 zi + 4 t + g4).
+                    uint32_t lo[3], hi[3];
+                    dev::split3_pair(out[0], out[1], lo[0], lo[1], lo[2]);
+                    dev::split3_pair(out[2], out[3], hi[0], hi[1], hi[2]);
+                    const size_t row = (size_t)zo * g.tq + query, kg = (size_t)zi * 8 + 4 * t + g4;
+#pragma unroll
+                    for (int p = 0; p < 3; p++)
+                        reinterpret_cast<u32x2 *>(g.o_planes + ((size_t)p * g.o_kgs + kg) * g.o_rp + row)[h] = u32x2{lo[p], hi[p]};
+                } else {
+                    *reinterpret_cast<f32x4 *>(o + (size_t)query * g.ldo + 32 * t + 8 * g4 + 4 * h) = out;
+                }
             }
     }
 }
@@ -524,13 +541,23 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 }  // namespace
 
+// Whether launch_attention would run the kernel that can write O as operand planes: enough (batch, head) pairs for full
+// blocks on a context whose products may take the bf16 route.
+bool attention_writes_planes(const DeviceCtx &ctx, size_t batch_outer, size_t batch_inner, size_t tq) {
+    const size_t q_tiles = (tq + 31) / 32, cus = ctx.cus_per_xcd ? (size_t)ctx.cus_per_xcd * 8 : 256, batch = batch_outer * batch_inner;
+    return ctx.gemm_algorithm != AHIP_GEMM_FP32 && tq > 0 && batch * ((q_tiles + 7) / 8) >= cus && batch * q_tiles >= 2 * cus &&
+           batch_outer * tq < ((size_t)1 << 31) - 256;
+}
+
 int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, const float *v, size_t batch_outer, size_t batch_inner,
                      size_t tq, size_t tk, size_t d, size_t ldq, size_t ldk, size_t ldv, size_t ldo, const size_t q_bs[2],
                      const size_t k_bs[2], const size_t v_bs[2], const size_t o_bs[2], int scale_op, float scale, const float *mask,
-                     size_t mask_outer_stride) {
+                     size_t mask_outer_stride, void *o_planes) {
     const size_t batch = batch_outer * batch_inner;
     if (batch == 0 || tq == 0) return AHIP_OK;
-    if (!o || !q || !k || !v) return ctx.fail(AHIP_ERR_ARG, "attention: null pointer");
+    if ((!o && !o_planes) || !q || !k || !v) return ctx.fail(AHIP_ERR_ARG, "attention: null pointer");
+    if (o_planes && !attention_writes_planes(ctx, batch_outer, batch_inner, tq))
+        return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: operand planes are written by the bf16 kernel on full blocks only");
     if (scale_op < 0 || scale_op > 2) return ctx.fail(AHIP_ERR_ARG, "attention: scale_op must be 0, 1 or 2");
     if (d != (size_t)D || tk == 0) return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: needs 64-wide heads and at least one key");
     const size_t lim = (size_t)1 << 31;
@@ -538,7 +565,7 @@ int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, c
     if (tq >= lim || tk >= lim || ldq >= lim || ldk >= lim || ldv >= lim || ldo >= lim || batch >= lim)
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: extent above 2^31");
     auto vec_ok = [](const void *p, size_t ld, const size_t bs[2]) { return aligned16(p) && ld % 4 == 0 && bs[0] % 4 == 0 && bs[1] % 4 == 0; };
-    if (!vec_ok(q, ldq, q_bs) || !vec_ok(k, ldk, k_bs) || !vec_ok(v, ldv, v_bs) || !vec_ok(o, ldo, o_bs))
+    if (!vec_ok(q, ldq, q_bs) || !vec_ok(k, ldk, k_bs) || !vec_ok(v, ldv, v_bs) || (!o_planes && !vec_ok(o, ldo, o_bs)))
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: operands must be 16-byte aligned with pitches that are multiples of 4");
     if (ldq < (size_t)D || ldk < (size_t)D || ldv < (size_t)D || ldo < (size_t)D)
         return ctx.fail(AHIP_ERR_ARG, "attention: a row pitch is below the head width");
@@ -552,6 +579,9 @@ int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, c
     g.scale = scale;
     g.mask = mask;
     g.mask_outer_stride = (uint32_t)mask_outer_stride;
+    g.o_planes = static_cast<u32x4_attn *>(o_planes);
+    g.o_rp = (uint32_t)((batch_outer * tq + 255) / 256 * 256);
+    g.o_kgs = (uint32_t)(batch_inner * 8);
     const size_t q_tiles = (tq + 31) / 32, cus = ctx.cus_per_xcd ? (size_t)ctx.cus_per_xcd * 8 : 256;
     if (q_tiles > 65535) return ctx.fail(AHIP_ERR_UNSUPPORTED, "attention: too many queries");
     if (batch * q_tiles < 2 * cus) {
@@ -567,7 +597,11 @@ int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, c
     // Where products may take the bf16 matrix cores (an infinite operand then gives NaN, as in the GEMM on that
     // route), full blocks do.
     if (w == 8 && ctx.gemm_algorithm != AHIP_GEMM_FP32) {
-#define ALTIUS_ATT(S, M) hipLaunchKernelGGL((attention_stream_d64_bf16<S, M>), grid, dim3(512), 0, ctx.stream, g)
+#define ALTIUS_ATT(S, M)                                                                                             \
+    do {                                                                                                             \
+        if (o_planes) hipLaunchKernelGGL((attention_stream_d64_bf16<S, M, true>), grid, dim3(512), 0, ctx.stream, g);  \
+        else hipLaunchKernelGGL((attention_stream_d64_bf16<S, M, false>), grid, dim3(512), 0, ctx.stream, g);         \
+    } while (0)
         if (mask) {
             if (scale_op == 0) ALTIUS_ATT(0, true);
             else if (scale_op == 1) ALTIUS_ATT(1, true);

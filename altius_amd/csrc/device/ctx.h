@@ -175,7 +175,11 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
 int launch_attention(DeviceCtx &ctx, float *o, const float *q, const float *k, const float *v, size_t batch_outer, size_t batch_inner,
                      size_t tq, size_t tk, size_t d, size_t ldq, size_t ldk, size_t ldv, size_t ldo, const size_t q_bs[2],
                      const size_t k_bs[2], const size_t v_bs[2], const size_t o_bs[2], int scale_op, float scale, const float *mask = nullptr,
-                     size_t mask_outer_stride = 0);
+                     size_t mask_outer_stride = 0, void *o_planes = nullptr);
+// o_planes: O, taken as the matrix [batch_outer * tq, batch_inner * 64] (o is not written), leaves as the operand planes
+// of the product on the bf16 route that reads it (gemm_planes_bytes(batch_outer * tq, batch_inner * 64) bytes).  Only
+// where attention_writes_planes says so.
+bool attention_writes_planes(const DeviceCtx &ctx, size_t batch_outer, size_t batch_inner, size_t tq);
 
 // The same product for one batch through three bf16 planes per operand and six bf16 MFMAs per fp32
 // product (gemm_split.hip): as accurate as an fp32 multiply-add chain, about 1.6 times the fp32 matrix

@@ -623,7 +623,7 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
             if (d && !d->strides.empty() && !materialize(d, err)) return false;
     // Operand planes have exactly one planned reader: the product behind the LayerNormalization that wrote them.
     for (size_t i = 0; i < in.size(); i++)
-        if (in[i] && in[i]->planes && !(i == 0 && planes_consumer_.count(id)))
+        if (in[i] && in[i]->planes && !(i == 0 && (planes_consumer_.count(id) || planes_pass_.count(id))))
             return fail(err, SessionError::Message, "internal: operand planes reached an operator that cannot read them");
     // A deferred Add runs now unless the reader is the LayerNormalization that can compute the sum itself.
     for (size_t i = 0; i < in.size(); i++)

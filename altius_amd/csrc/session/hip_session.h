@@ -278,6 +278,10 @@ private:
     };
     std::map<NodeId, PlanesPlan> planes_out_;
     std::set<NodeId> planes_consumer_;
+    // The second product of an attention -> Transpose (written in place) -> Reshape -> MatMul(weights): the attention kernel
+    // writes that last product's operand planes; the two nodes between pass them on.
+    std::map<NodeId, PlanesPlan> attn_planes_;
+    std::set<NodeId> planes_pass_;
     std::map<NodeId, NodeId> add_into_ln_;  // Add nodes (a residual connection) -> the planes-writing LayerNormalization that reads the sum
     // Runs a deferred Add into the tensor's block.
     bool flush_add(DeviceTensor *t, SessionError *err);

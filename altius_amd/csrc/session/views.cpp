@@ -234,10 +234,24 @@ bool HipSession::run_attention_tail(const Op &op, const std::vector<DeviceTensor
     size_t q2[2], k2[2], v2[2], o2[2];
     two(pa.Q.bstr, q2), two(pa.K.bstr, k2), two(vs, v2), two(os, o2);
     const size_t outer = pa.bd.size() > 0 ? pa.bd[0] : 1, inner = pa.bd.size() > 1 ? pa.bd[1] : 1;
-    const int rc = launch_attention(ctx_, static_cast<float *>(out->ptr), static_cast<const float *>(pa.q.ptr),
+    // O as the operand planes of the product behind it: O is [outer, inner, tq, 64] written as [outer, tq, inner * 64]
+    // (the Transpose's layout), which that product reads as [outer * tq, inner * 64].
+    void *planes_ptr = nullptr;
+    auto ap = attn_planes_.find(current_node_);
+    if (ap != attn_planes_.end() && pa.bd.size() == 2 && rank == 4 && !out->strides.empty() && ldo == inner * 64 && o2[0] == tq * ldo && o2[1] == 64 &&
+        attention_writes_planes(ctx_, outer, inner, tq) && gemm_takes_split(ctx_, outer * tq, ap->second.next_n, inner * 64)) {
+        DeviceTensor planes;
+        if (!allocate_bytes(gemm_planes_bytes(outer * tq, inner * 64), &planes, err)) return false;
+        out->block = planes.block;  // the fp32 block goes back to the pool unused
+        out->ptr = planes.ptr;
+        out->planes = true;
+        planes_ptr = planes.ptr;
+        copies_avoided_++;  // the operand split of the product behind
+    }
+    const int rc = launch_attention(ctx_, planes_ptr ? nullptr : static_cast<float *>(out->ptr), static_cast<const float *>(pa.q.ptr),
                                     static_cast<const float *>(pa.k.ptr), static_cast<const float *>(in[1]->ptr), outer, inner, tq, tk, 64,
                                     pa.Q.ld, pa.K.ld, V.ld, ldo, q2, k2, v2, o2, plan->scale_op, plan->scale,
-                                    pa.mask.ptr ? static_cast<const float *>(pa.mask.ptr) : nullptr, pa.mask_outer_stride);
+                                    pa.mask.ptr ? static_cast<const float *>(pa.mask.ptr) : nullptr, pa.mask_outer_stride, planes_ptr);
     if (rc) return fail_code(err, rc, ctx_.last_error);
     return true;
 }
@@ -367,6 +381,39 @@ void HipSession::plan_views(bool fused_attention) {
             if (perm.size() < 3 || perm.back() != (int64_t)perm.size() - 1) continue;
             matmul_out_perm_[id] = perm;
         }
+    }
+    // An attention whose result goes, through the Transpose it is written ahead of and one Reshape, into a product with a
+    // weight matrix and nowhere else: the attention kernel can write that product's operand planes.
+    for (NodeId tid : attn_tail_) {
+        auto pv = matmul_out_perm_.find(tid);
+        if (pv == matmul_out_perm_.end() || pv->second != std::vector<int64_t>{0, 2, 1, 3}) continue;
+        auto single_user = [&](ValueId v, NodeId *u) {
+            auto it = users.find(v);
+            if (it == users.end() || it->second.size() != 1 || is_output(v)) return false;
+            *u = *it->second.begin();
+            return true;
+        };
+        NodeId tr, rs, mm;
+        if (!single_user(g.nodes[tid].outputs[0], &tr) || g.nodes[tr].op.kind != OpKind::Transpose || g.nodes[tr].outputs.size() != 1) continue;
+        if (!single_user(g.nodes[tr].outputs[0], &rs) || g.nodes[rs].op.kind != OpKind::Reshape || g.nodes[rs].outputs.size() != 1 ||
+            g.nodes[rs].inputs.empty() || g.nodes[rs].inputs[0] != g.nodes[tr].outputs[0])
+            continue;
+        if (!single_user(g.nodes[rs].outputs[0], &mm)) continue;
+        const Node &m = g.nodes[mm];
+        if (m.op.kind != OpKind::MatMul || m.inputs.size() < 2 || m.inputs[0] != g.nodes[rs].outputs[0] || m.op.trans_a ||
+            planes_consumer_.count(mm) || matmul_out_perm_.count(mm))
+            continue;
+        bool elsewhere = false;
+        for (size_t i = 1; i < m.inputs.size(); i++) elsewhere = elsewhere || m.inputs[i] == m.inputs[0];
+        auto w = g.inits.find(m.inputs[1]);
+        if (elsewhere || w == g.inits.end() || w->second.dims().len() != 2 || w->second.elem_ty() != TensorElemType::F32) continue;
+        PlanesPlan pp;
+        pp.consumer = mm;
+        pp.next_n = m.op.trans_b ? w->second.dims()[0] : w->second.dims()[1];
+        attn_planes_[tid] = pp;
+        planes_consumer_.insert(mm);
+        planes_pass_.insert(tr);
+        planes_pass_.insert(rs);
     }
 }
 

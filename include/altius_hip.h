@@ -613,7 +613,9 @@ int ahip_session_builder_with_strided_views(ahip_session_builder *builder, int e
  * with enable != 0 (default 0; needs strided views) a MatMul -> Softmax(last axis, with the scale and per-key
  * mask that ahip_fuse_softmax_prologue absorbed) -> MatMul chain with 64-wide heads runs as one ahip_attention
  * kernel that never writes the scores.  Its sums run in another order than the three operators': results
- * differ from theirs by up to 2e-4 relative, which is why a caller has to ask for it. */
+ * differ from theirs by up to 2e-4 relative, which is why a caller has to ask for it.  On the bf16 route, an
+ * attention whose output only the product behind its Transpose and Reshape reads leaves the kernel as that
+ * product's operand planes (the split of the same values). */
 int ahip_session_builder_with_fused_attention(ahip_session_builder *builder, int enable);
 /* Nodes of the last node-by-node run that were served without their copy (views taken, transposed layouts
  * written in place). */

@@ -95,6 +95,34 @@ def test_attention_reads_and_writes_heads_in_place(case, batch, tokens, heads, d
     np.testing.assert_allclose(got, attention_numpy(x, heads, d, w), rtol=2e-4, atol=2e-5)
 
 
+@pytest.mark.parametrize("batch,tokens,planes", [(24, 45, True), (22, 197, True), (4, 45, False)])
+def test_attention_writes_the_operand_planes_of_the_projection_behind_it(case, batch, tokens, planes):
+    """On the bf16 route, with the one-kernel attention and heads enough for full blocks, the attention's output is
+    read by nothing but the Transpose it is written ahead of, the Reshape and the projection: it leaves the kernel as
+    that product's three bf16 planes and the separate split is not launched (one more copy avoided than the first
+    product's and the Softmax's).  Checked against the definition and against the same session with the three
+    operators apart, to the bars of the attention kernel.  With too few heads for the bf16 kernel's blocks the fp32
+    kernel runs and the projection splits its operand itself."""
+    case(f"attention -> planes -> projection, b={batch} t={tokens}")
+    from altius_amd import device as D
+
+    heads, d = 12, 64
+    m, w = attention(batch, tokens, heads, d, True)
+    x = (RNG.standard_normal((batch, tokens, 3 * heads * d)) * 0.3).astype(np.float32)
+    outs, avoided = [], []
+    for fused in (True, False):
+        sess = HipSessionBuilder(m.clone()).with_gemm_algorithm(D.GEMM_BF16X3).with_fused_attention(fused).build()
+        for _ in range(2):
+            (got,) = [np.array(t) for t in sess.run([Tensor.from_numpy(x)])]
+        avoided.append(sess.copies_avoided())
+        sess.close()
+        outs.append(got)
+    assert avoided[0] == avoided[1] + (3 if planes else 2), avoided  # the first product's, the Softmax's, the operand split
+    want = attention_numpy(x, heads, d, w)
+    np.testing.assert_allclose(outs[0], want, rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(outs[0], outs[1], rtol=2e-4, atol=2e-5)
+
+
 def test_view_with_another_reader_is_copied(case):
     """A part that an element-wise operator also reads is not made a view; its siblings' fate follows (one Split node)."""
     case("split part read by Add as well")
