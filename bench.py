@@ -205,7 +205,7 @@ def run_row_sweep(ctx, D, args, lengths):
     for length, ops_l in build_row_sweep(ctx, D, lengths):
         entry = {"row_length": length}
         for o in ops_l:
-            t = time_kernel(ctx, o, args.kernel_iters, args.kernel_warmup)
+            t = time_kernel(ctx, o, args.kernel_iters, args.kernel_warmup, args.kernel_settle_ms)
             r = t.row(o.nbytes)
             entry[o.name] = {"bytes": o.nbytes, "us": r["us"], "us_median": r["us_median"], "us_min": r["us_min"], "GBps": r["GBps"],
                              "pct_hbm_peak": r["pct_hbm_peak"]}
@@ -546,10 +546,18 @@ class Timing:
                 "pct_hbm_peak_median": round(100.0 * nbytes / (self.median * 1e-3) / 1e9 / HBM_PEAK_GBPS, 1)}
 
 
-def time_kernel(ctx, op, iters=100, warmup=20):
-    """`warmup` untimed launches, then at least `iters` timed ones with a HIP event on the kernels' stream between
-    consecutive samples.  A sample is a group of back-to-back launches lasting about 0.25 ms (one launch for the longest
-    kernels, dozens for the few-microsecond ones), so that the event between samples does not weigh on the figure."""
+SETTLE_MS = 25.0  # warm-up of a kernel lasts at least this long
+
+
+def time_kernel(ctx, op, iters=100, warmup=20, settle_ms=SETTLE_MS):
+    """`warmup` untimed launches, and as many more as it takes to keep the GPU on this kernel for `settle_ms`; then at
+    least `iters` timed ones with a HIP event on the kernels' stream between consecutive samples.  A sample is a group
+    of back-to-back launches lasting about 0.25 ms (one launch for the longest kernels, dozens for the few-microsecond
+    ones), so that the event between samples does not weigh on the figure.
+    Why the warm-up goes by time: after an idle period, or when the load changes, the part runs the next 3 to 25 ms of
+    kernels several percent slower (a 150 us Softmax: up to 180 us between its 15th and its 100th launch, then 152 us
+    for as long as it is kept busy) while its power management settles; 20 launches of a long kernel end inside that
+    window and 100 timed ones cover it."""
     for _ in range(warmup):
         op.launch()
     probe = [ctx.event(), ctx.event()]
@@ -561,6 +569,8 @@ def time_kernel(ctx, op, iters=100, warmup=20):
     est_ms = ctx.elapsed_ms(probe[0], probe[1]) / 5
     for e in probe:
         ctx.destroy_event(e)
+    for _ in range(min(20000, max(0, int(settle_ms / max(est_ms, 1e-4)) - warmup - 5))):
+        op.launch()
     group = max(1, min(64, int(round(0.25 / max(est_ms, 1e-4)))))
     n = max(25, (iters + group - 1) // group)
     events = [ctx.event() for _ in range(n + 1)]
@@ -575,6 +585,22 @@ def time_kernel(ctx, op, iters=100, warmup=20):
     for e in events:
         ctx.destroy_event(e)
     return Timing(samples, group)
+
+
+def launch_timeline(ctx, op, n):
+    """Duration of each of n consecutive launches (a HIP event after every launch): shows how long after an idle
+    period the kernel takes to reach the time it then keeps."""
+    events = [ctx.event() for _ in range(n + 1)]
+    ctx.sync()
+    ctx.record(events[0])
+    for i in range(n):
+        op.launch()
+        ctx.record(events[i + 1])
+    ctx.sync()
+    us = [ctx.elapsed_ms(events[i], events[i + 1]) * 1e3 for i in range(n)]
+    for e in events:
+        ctx.destroy_event(e)
+    return us
 
 
 def time_interleaved(ctx, ops, steps, warmup):
@@ -646,7 +672,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=256, help="batch of configs[4] (256 = the named workload)")
     ap.add_argument("--kernel-iters", type=int, default=100, help="timed launches per kernel for the per-kernel timing")
-    ap.add_argument("--kernel-warmup", type=int, default=20, help="untimed launches per kernel ahead of them")
+    ap.add_argument("--kernel-warmup", type=int, default=20, help="untimed launches per kernel ahead of them (and as many more as %g ms take)" % SETTLE_MS)
+    ap.add_argument("--kernel-settle-ms", type=float, default=SETTLE_MS,
+                    help="least duration of a kernel's warm-up (0 for counter passes of a profiler, where every launch is slow)")
+    ap.add_argument("--settle-ms", type=float, default=250.0,
+                    help="the step is run for this long, untimed, before the W warm-up steps and the K timed ones that make 'value' "
+                         "(the K steps straight after the uploads are reported beside it as 'value_after_idle')")
     ap.add_argument("--cpu-sample-batch", type=int, default=0,
                     help="batch of the CPU baseline sample (0: the whole batch, about 2 s of CPU time)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -665,6 +696,9 @@ def main():
                     help="tensors of at least this many MiB use non-temporal accesses (default: the library's own threshold)")
     ap.add_argument("--sweep-lengths", type=str, default="", help="comma-separated row lengths for the sweep (default: 49 ... 16384)")
     ap.add_argument("--sweep-only", action="store_true", help="run the row sweep and nothing else (profiling)")
+    ap.add_argument("--timeline", type=int, default=0, metavar="N",
+                    help="print the duration of each of N consecutive launches of every kernel of the step, the first kernel after "
+                         "the uploads and one second of idle, and exit ('timeline' in the JSON)")
     ap.add_argument("--next-rows", action="store_true",
                     help="also time the data-movement and MatMul kernels at ViT-B/16 shapes ('next_rows' in the JSON)")
     ap.add_argument("--vit", type=int, default=0, metavar="BATCH",
@@ -690,7 +724,7 @@ def main():
         out = {}
         if args.calibrate:  # first, so that a profile of this run finds the copy kernel of known size ahead of the sweep
             cal = calibration_op(ctx, D)
-            out["calibration"] = dict({"kernel": cal.name, "bytes": cal.nbytes}, **time_kernel(ctx, cal, args.kernel_iters, args.kernel_warmup).row(cal.nbytes))
+            out["calibration"] = dict({"kernel": cal.name, "bytes": cal.nbytes}, **time_kernel(ctx, cal, args.kernel_iters, args.kernel_warmup, args.kernel_settle_ms).row(cal.nbytes))
             log("%-44s %14d %9.1f us %6.1f %%" % (cal.name, cal.nbytes, out["calibration"]["us"], out["calibration"]["pct_hbm_peak"]))
         out["row_sweep"] = run_row_sweep(ctx, D, args, sweep_lengths)
         print(json.dumps(out), flush=True)
@@ -704,24 +738,49 @@ def main():
     extra_ops = fused_ops + ([calibration_op(ctx, D)] if args.calibrate else [])
     ctx.sync()
 
+    if args.timeline:
+        out = {"timeline": []}
+        time.sleep(1.0)
+        for o in [ops[1], ops[0], ops[1]] if len(ops) > 1 else ops:
+            us = launch_timeline(ctx, o, args.timeline)
+            tenths = [sum(us[i:i + 10]) / len(us[i:i + 10]) for i in range(0, len(us), 10)]
+            out["timeline"].append({"kernel": o.name, "us_mean_of_each_10_launches": [round(v, 1) for v in tenths]})
+            log("%-44s %s" % (o.name, " ".join("%.0f" % v for v in tenths)))
+        print(json.dumps(out), flush=True)
+        ctx.close()
+        return
+
     # --- whole step: W warm-up steps, then exactly K timed steps --------------------------------
-    for _ in range(args.warmup):
-        for o in ops:
-            o.launch()
-    ctx.sync()
+    def timed_steps():
+        for _ in range(args.warmup):
+            for o in ops:
+                o.launch()
+        ctx.sync()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            for o in ops:
+                o.launch()
+        ctx.sync()
+        return (time.perf_counter() - t0) / args.steps
+
+    # Once straight after the uploads (the GPU has been idle for seconds: the first 3 to 25 ms of kernels run inside
+    # the window in which the part's power management settles), and once for the record after the step has kept the
+    # GPU busy for --settle-ms: the sustained rate, which is what a job of more than a few steps sees.
+    step_s_after_idle = timed_steps()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        for o in ops:
-            o.launch()
-    ctx.sync()
-    step_s = (time.perf_counter() - t0) / args.steps
+    while (time.perf_counter() - t0) * 1e3 < args.settle_ms:
+        for _ in range(8):
+            for o in ops:
+                o.launch()
+        ctx.sync()
+    step_s = timed_steps()
     step_bytes = sum(o.nbytes for o in ops)
     value = step_bytes / step_s / 1e9
 
     # --- per kernel, HIP events on the kernels' stream -----------------------------------------
     rows = []
     for o in ops + extra_ops:
-        t = time_kernel(ctx, o, args.kernel_iters, args.kernel_warmup)
+        t = time_kernel(ctx, o, args.kernel_iters, args.kernel_warmup, args.kernel_settle_ms)
         rows.append(dict({"kernel": o.name, "bytes": o.nbytes}, **t.row(o.nbytes)))
     # ... and each of the step's kernels while the others run around it
     if len(ops) > 1:
@@ -743,6 +802,9 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4),
+        "value_after_idle": round(step_bytes / step_s_after_idle / 1e9, 1),
+        "ms_per_step_after_idle": round(step_s_after_idle * 1e3, 4),
+        "settle_ms": args.settle_ms,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -772,9 +834,11 @@ def main():
             "launches": dom["launches"],
             "algorithmic_bytes": dom["bytes"],
         },
-        "timing": "per kernel: %d warm-up launches, then >= %d launches with a HIP event between samples on the kernels' stream; "
-                  "us = mean, us_median, us_min; us_interleaved = the same kernel inside the step (an event between every two "
-                  "kernels of the step)" % (args.kernel_warmup, args.kernel_iters),
+        "timing": "value: the step run untimed for settle_ms, then W warm-up steps, then K timed steps (value_after_idle: W + K steps "
+                  "straight after the uploads, while the part's power management is still settling). "
+                  "per kernel: %d warm-up launches and as many more as %g ms take, then >= %d launches with a HIP event between "
+                  "samples on the kernels' stream; us = mean, us_median, us_min; us_interleaved = the same kernel inside the step "
+                  "(an event between every two kernels of the step)" % (args.kernel_warmup, args.kernel_settle_ms, args.kernel_iters),
         "per_kernel": rows,
     }
 
@@ -782,7 +846,7 @@ def main():
         listed = []
         log("every operator of the path at configs[4]-sized tensors:")
         for o in build_listed_ops(ctx, D, cfg4_arrays, args.batch):
-            t = time_kernel(ctx, o, args.kernel_iters, args.kernel_warmup)
+            t = time_kernel(ctx, o, args.kernel_iters, args.kernel_warmup, args.kernel_settle_ms)
             r = dict({"kernel": o.name, "bytes": o.nbytes}, **t.row(o.nbytes))
             listed.append(r)
             log("%-44s %14d %9.1f %9.1f %9.1f %9.1f %8.1f" % (o.name, o.nbytes, r["us"], r["us_median"], r["us_min"], r["GBps"], r["pct_hbm_peak"]))
@@ -795,7 +859,7 @@ def main():
         others = []
         log("%-44s %14s %10s %10s %10s %8s %14s %14s" % ("kernel", "alg. bytes", "us mean", "us median", "GB/s", "% peak", "CPU 16 thr us", "CPU 1 thr us"))
         for o in build_other_configs(ctx, D, synth):
-            t = time_kernel(ctx, o, args.kernel_iters, args.kernel_warmup)
+            t = time_kernel(ctx, o, args.kernel_iters, args.kernel_warmup, args.kernel_settle_ms)
             row = dict({"kernel": o.name, "bytes": o.nbytes}, **t.row(o.nbytes))
             cpu_us = {}
             if not args.no_cpu and o.cpu:
@@ -829,7 +893,7 @@ def main():
         nxt = []
         for name, nbytes, flops, fn in build_next_rows(ctx, D, args.batch):
             o = Op(name, nbytes, [fn])
-            ms = time_kernel(ctx, o, max(10, args.kernel_iters // 2), 3).mean
+            ms = time_kernel(ctx, o, max(10, args.kernel_iters // 2), 3, args.kernel_settle_ms).mean
             row = {"kernel": name, "us": round(ms * 1e3, 1), "bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1)}
             if flops:
                 # six bf16 MFMAs per fp32 product: the bf16 peak (2500 TFLOP/s dense) over six

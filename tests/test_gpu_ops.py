@@ -317,6 +317,33 @@ def test_layernorm(ctx, oracle, case, shape):
     np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5)
 
 
+# More rows than blocks fit the device, of lengths that take 1024 threads: the kernels that request a row ahead.
+MANY_LONG_ROWS = [(1100, 5120), (1029, 6144), (1500, 8192), (1031, 8196), (1100, 12288), (1111, 16384), (1040, 16380), (2100, 5004)]
+
+
+@pytest.mark.parametrize("rows,length", MANY_LONG_ROWS)
+def test_softmax_and_layernorm_of_many_long_rows(ctx, oracle, case, rows, length):
+    """The same rows a few at a time go through the kernels that hold one row per block and launch: not a bit may
+    differ.  Against the oracle on the first, the last and some rows between, a NaN and an all-equal row among them."""
+    case(f"softmax / layernorm of {rows} rows of {length}")
+    x = synth.normal(71, (rows, length), mean=0.2, std=1.5)
+    x[3, 17] = np.nan
+    x[rows - 1] = 2.5
+    x[5, ::3] = -1e4
+    g = synth.normal(72, (length,), mean=1.0, std=0.02)
+    b = synth.normal(73, (length,), mean=0.0, std=0.02)
+    pick = np.r_[0:8, rows // 2 : rows // 2 + 4, rows - 6 : rows]
+    with np.errstate(all="ignore"):
+        got = ctx.softmax(x)
+        few = np.concatenate([ctx.softmax(x[i : i + 500]) for i in range(0, rows, 500)])
+        assert_bits_equal(got, few, "softmax: many rows vs a few at a time")
+        assert_close(got[pick], oracle.softmax(x[pick]), what="softmax of many long rows")
+        got = ctx.layer_norm(x, g, b, 1e-5)
+        few = np.concatenate([ctx.layer_norm(x[i : i + 500], g, b, 1e-5) for i in range(0, rows, 500)])
+        assert_bits_equal(got, few, "layernorm: many rows vs a few at a time")
+        assert_close(got[pick], oracle.layer_norm(x[pick], g, b, 1e-5), what="layernorm of many long rows")
+
+
 REDUCE_CASES = [
     # (shape, axes, keepdims)
     ([1, 50, 70], [-1], True),         # test_ops_reduce.py:10-18
