@@ -167,13 +167,12 @@ __global__ __launch_bounds__(BLOCK) void softmax_wave(float *__restrict__ out, c
 //   3. the span is written back with 16-byte stores.
 // With SUB*NCH just above the row length nearly every lane slot of the
 // arithmetic does useful work (197 -> 16 x 13 = 208 slots).
-constexpr int LDS_BLOCK = 1024;
-constexpr int LDS_WAVES = LDS_BLOCK / WAVE;
+constexpr int LDS_BLOCK = 1024;                                      // threads of the wide block; the narrow one has half
 constexpr int STAGE_LDS = 2;                                         // float4 per lane staged through registers
 constexpr size_t LDS_GROUP_FLOATS = (size_t)STAGE_LDS * LDS_BLOCK * 4;  // 8192 floats = 32 KiB of LDS at most
 
-template <int SUB, int NCH, bool NT, bool PRO>
-__global__ __launch_bounds__(LDS_BLOCK) void softmax_lds(float *__restrict__ out, const float *__restrict__ in,
+template <int BT, int SUB, int NCH, bool NT, bool PRO>
+__global__ __launch_bounds__(BT) void softmax_lds(float *__restrict__ out, const float *__restrict__ in,
                                                          size_t rows, int len, int group_rows, const SoftmaxPrologue pro) {
     extern __shared__ __align__(16) float lds[];
     const int tid = threadIdx.x;
@@ -191,23 +190,23 @@ __global__ __launch_bounds__(LDS_BLOCK) void softmax_lds(float *__restrict__ out
     float4 stage[STAGE_LDS];
 #pragma unroll
     for (int u = 0; u < STAGE_LDS; u++) {
-        const float *p = src + 4 * (tid + LDS_BLOCK * u);
-        if (LDS_BLOCK * (u + 1) <= n4) {
+        const float *p = src + 4 * (tid + BT * u);
+        if (BT * (u + 1) <= n4) {
             stage[u] = load4<NT>(p);
-        } else if (LDS_BLOCK * u < n4) {
-            if (tid + LDS_BLOCK * u < n4) stage[u] = load4<NT>(p);
+        } else if (BT * u < n4) {
+            if (tid + BT * u < n4) stage[u] = load4<NT>(p);
         }
     }
 #pragma unroll
     for (int u = 0; u < STAGE_LDS; u++) {
-        float *q = lds + 4 * (tid + LDS_BLOCK * u);
-        if (LDS_BLOCK * (u + 1) <= n4) {
+        float *q = lds + 4 * (tid + BT * u);
+        if (BT * (u + 1) <= n4) {
             *reinterpret_cast<float4 *>(q) = stage[u];
-        } else if (LDS_BLOCK * u < n4) {
-            if (tid + LDS_BLOCK * u < n4) *reinterpret_cast<float4 *>(q) = stage[u];
+        } else if (BT * u < n4) {
+            if (tid + BT * u < n4) *reinterpret_cast<float4 *>(q) = stage[u];
         }
     }
-    for (int i = (n4 << 2) + tid; i < n; i += LDS_BLOCK) lds[i] = src[i];  // ragged end of the last group
+    for (int i = (n4 << 2) + tid; i < n; i += BT) lds[i] = src[i];  // ragged end of the last group
     // The group's rows use at most two consecutive mask rows (the host checks rows_per_mask >=
     // group_rows); they go to LDS behind the scores, once per block.
     float *mask_lds = lds + (size_t)group_rows * len;
@@ -219,7 +218,7 @@ __global__ __launch_bounds__(LDS_BLOCK) void softmax_lds(float *__restrict__ out
         if (two) second_mask_from = (uint32_t)(boundary - row0);
         const int count = two ? 2 * len : len;
         const float *m = pro.mask + (size_t)m0 * len;
-        for (int i = tid; i < count; i += LDS_BLOCK) mask_lds[i] = m[i];
+        for (int i = tid; i < count; i += BT) mask_lds[i] = m[i];
     }
     __syncthreads();
 
@@ -229,7 +228,7 @@ __global__ __launch_bounds__(LDS_BLOCK) void softmax_lds(float *__restrict__ out
     const int rr = lane / SUB;
     const bool last_valid = s + SUB * LAST < len;
     const float nan = __builtin_nanf("");
-    for (int r0 = wave * RPP; r0 < nrows; r0 += LDS_WAVES * RPP) {
+    for (int r0 = wave * RPP; r0 < nrows; r0 += (BT / WAVE) * RPP) {
         // Lane groups past the end of a ragged last group redo its last row: they compute and
         // store the same values as the group that owns it.
         const int r = r0 + rr < nrows ? r0 + rr : nrows - 1;
@@ -275,23 +274,23 @@ __global__ __launch_bounds__(LDS_BLOCK) void softmax_lds(float *__restrict__ out
 
 #pragma unroll
     for (int u = 0; u < STAGE_LDS; u++) {
-        const float *q = lds + 4 * (tid + LDS_BLOCK * u);
-        if (LDS_BLOCK * (u + 1) <= n4) {
+        const float *q = lds + 4 * (tid + BT * u);
+        if (BT * (u + 1) <= n4) {
             stage[u] = *reinterpret_cast<const float4 *>(q);
-        } else if (LDS_BLOCK * u < n4) {
-            if (tid + LDS_BLOCK * u < n4) stage[u] = *reinterpret_cast<const float4 *>(q);
+        } else if (BT * u < n4) {
+            if (tid + BT * u < n4) stage[u] = *reinterpret_cast<const float4 *>(q);
         }
     }
 #pragma unroll
     for (int u = 0; u < STAGE_LDS; u++) {
-        float *p = dst + 4 * (tid + LDS_BLOCK * u);
-        if (LDS_BLOCK * (u + 1) <= n4) {
+        float *p = dst + 4 * (tid + BT * u);
+        if (BT * (u + 1) <= n4) {
             store4<NT>(p, stage[u]);
-        } else if (LDS_BLOCK * u < n4) {
-            if (tid + LDS_BLOCK * u < n4) store4<NT>(p, stage[u]);
+        } else if (BT * u < n4) {
+            if (tid + BT * u < n4) store4<NT>(p, stage[u]);
         }
     }
-    for (int i = (n4 << 2) + tid; i < n; i += LDS_BLOCK) dst[i] = lds[i];
+    for (int i = (n4 << 2) + tid; i < n; i += BT) dst[i] = lds[i];
 }
 
 // LayerNormalization of rows that a wavefront per row with 16-byte accesses does not fit (not whole float4s, or
@@ -301,8 +300,8 @@ __global__ __launch_bounds__(LDS_BLOCK) void softmax_lds(float *__restrict__ out
 // are staged with coalesced loads).
 // Two blocks of sixteen wavefronts share a CU (one loads or stores while the other computes), which leaves each lane
 // 64 registers: the second launch bound says so to the register allocator.
-template <int SUB, int NCH, bool NT>
-__global__ __launch_bounds__(LDS_BLOCK, 8) void layernorm_lds(float *__restrict__ out, const float *__restrict__ in,
+template <int BT, int SUB, int NCH, bool NT>
+__global__ __launch_bounds__(BT, 8) void layernorm_lds(float *__restrict__ out, const float *__restrict__ in,
                                                            const float *__restrict__ gamma, const float *__restrict__ beta, size_t rows,
                                                            int len, int group_rows, float eps) {
     extern __shared__ __align__(16) float lds[];
@@ -318,11 +317,11 @@ __global__ __launch_bounds__(LDS_BLOCK, 8) void layernorm_lds(float *__restrict_
     float4 stage[STAGE_LDS];
 #pragma unroll
     for (int u = 0; u < STAGE_LDS; u++) {
-        const float *p = src + 4 * (tid + LDS_BLOCK * u);
-        if (LDS_BLOCK * (u + 1) <= n4) {
+        const float *p = src + 4 * (tid + BT * u);
+        if (BT * (u + 1) <= n4) {
             stage[u] = load4<NT>(p);
-        } else if (LDS_BLOCK * u < n4) {
-            if (tid + LDS_BLOCK * u < n4) stage[u] = load4<NT>(p);
+        } else if (BT * u < n4) {
+            if (tid + BT * u < n4) stage[u] = load4<NT>(p);
         }
     }
     constexpr int RPP = WAVE / SUB;  // rows per wave pass
@@ -333,17 +332,17 @@ __global__ __launch_bounds__(LDS_BLOCK, 8) void layernorm_lds(float *__restrict_
     // Scale and bias go to LDS behind the rows with coalesced loads, once per block, and from there into each
     // lane's registers.
     float *g_lds = lds + (size_t)group_rows * len, *b_lds = g_lds + len;
-    for (int i = tid; i < len; i += LDS_BLOCK) g_lds[i] = gamma[i], b_lds[i] = beta[i];
+    for (int i = tid; i < len; i += BT) g_lds[i] = gamma[i], b_lds[i] = beta[i];
 #pragma unroll
     for (int u = 0; u < STAGE_LDS; u++) {
-        float *q = lds + 4 * (tid + LDS_BLOCK * u);
-        if (LDS_BLOCK * (u + 1) <= n4) {
+        float *q = lds + 4 * (tid + BT * u);
+        if (BT * (u + 1) <= n4) {
             *reinterpret_cast<float4 *>(q) = stage[u];
-        } else if (LDS_BLOCK * u < n4) {
-            if (tid + LDS_BLOCK * u < n4) *reinterpret_cast<float4 *>(q) = stage[u];
+        } else if (BT * u < n4) {
+            if (tid + BT * u < n4) *reinterpret_cast<float4 *>(q) = stage[u];
         }
     }
-    for (int i = (n4 << 2) + tid; i < n; i += LDS_BLOCK) lds[i] = src[i];  // ragged end of the last group
+    for (int i = (n4 << 2) + tid; i < n; i += BT) lds[i] = src[i];  // ragged end of the last group
     __syncthreads();
 
     // Up to 10 chunks the lane's scale and bias values stay in registers for all of its rows; beyond that they would
@@ -360,7 +359,7 @@ __global__ __launch_bounds__(LDS_BLOCK, 8) void layernorm_lds(float *__restrict_
         }
     }
     const float inv_n = 1.0f / (float)len;
-    for (int r0 = wave * RPP; r0 < nrows; r0 += LDS_WAVES * RPP) {
+    for (int r0 = wave * RPP; r0 < nrows; r0 += (BT / WAVE) * RPP) {
         // Lane groups past the end of a ragged last group redo its last row: they compute and store the same
         // values as the group that owns it.
         const int r = r0 + rr < nrows ? r0 + rr : nrows - 1;
@@ -395,31 +394,31 @@ __global__ __launch_bounds__(LDS_BLOCK, 8) void layernorm_lds(float *__restrict_
 
 #pragma unroll
     for (int u = 0; u < STAGE_LDS; u++) {
-        const float *q = lds + 4 * (tid + LDS_BLOCK * u);
-        if (LDS_BLOCK * (u + 1) <= n4) {
+        const float *q = lds + 4 * (tid + BT * u);
+        if (BT * (u + 1) <= n4) {
             stage[u] = *reinterpret_cast<const float4 *>(q);
-        } else if (LDS_BLOCK * u < n4) {
-            if (tid + LDS_BLOCK * u < n4) stage[u] = *reinterpret_cast<const float4 *>(q);
+        } else if (BT * u < n4) {
+            if (tid + BT * u < n4) stage[u] = *reinterpret_cast<const float4 *>(q);
         }
     }
 #pragma unroll
     for (int u = 0; u < STAGE_LDS; u++) {
-        float *p = dst + 4 * (tid + LDS_BLOCK * u);
-        if (LDS_BLOCK * (u + 1) <= n4) {
+        float *p = dst + 4 * (tid + BT * u);
+        if (BT * (u + 1) <= n4) {
             store4<NT>(p, stage[u]);
-        } else if (LDS_BLOCK * u < n4) {
-            if (tid + LDS_BLOCK * u < n4) store4<NT>(p, stage[u]);
+        } else if (BT * u < n4) {
+            if (tid + BT * u < n4) store4<NT>(p, stage[u]);
         }
     }
-    for (int i = (n4 << 2) + tid; i < n; i += LDS_BLOCK) dst[i] = lds[i];
+    for (int i = (n4 << 2) + tid; i < n; i += BT) dst[i] = lds[i];
 }
 
 // Sum or maximum of every row, for rows that are short or not whole float4s (7 x 7 feature maps, 197 tokens): a
 // wavefront per row would leave most lanes idle and read 4 bytes per lane.  Same staging as softmax_lds: a
 // line-aligned group of rows goes to LDS with 16-byte loads, then SUB lanes fold each row and lane 0 of the group
 // writes out[row] (times `scale` for a mean).
-template <class OP, int SUB, bool SCALE, bool NT>
-__global__ __launch_bounds__(LDS_BLOCK) void reduce_rows_lds(float *__restrict__ out, const float *__restrict__ in, size_t rows,
+template <int BT, int ST, class OP, int SUB, bool SCALE, bool NT>
+__global__ __launch_bounds__(BT) void reduce_rows_lds(float *__restrict__ out, const float *__restrict__ in, size_t rows,
                                                              int len, int group_rows, float scale) {
     extern __shared__ __align__(16) float lds[];
     const int tid = threadIdx.x;
@@ -430,32 +429,32 @@ __global__ __launch_bounds__(LDS_BLOCK) void reduce_rows_lds(float *__restrict__
     const int n = nrows * len;
     const int n4 = n >> 2;
     const float *src = in + row0 * (size_t)len;
-    float4 stage[STAGE_LDS];
+    float4 stage[ST];
 #pragma unroll
-    for (int u = 0; u < STAGE_LDS; u++) {
-        const float *p = src + 4 * (tid + LDS_BLOCK * u);
-        if (LDS_BLOCK * (u + 1) <= n4) {
+    for (int u = 0; u < ST; u++) {
+        const float *p = src + 4 * (tid + BT * u);
+        if (BT * (u + 1) <= n4) {
             stage[u] = load4<NT>(p);
-        } else if (LDS_BLOCK * u < n4) {
-            if (tid + LDS_BLOCK * u < n4) stage[u] = load4<NT>(p);
+        } else if (BT * u < n4) {
+            if (tid + BT * u < n4) stage[u] = load4<NT>(p);
         }
     }
 #pragma unroll
-    for (int u = 0; u < STAGE_LDS; u++) {
-        float *q = lds + 4 * (tid + LDS_BLOCK * u);
-        if (LDS_BLOCK * (u + 1) <= n4) {
+    for (int u = 0; u < ST; u++) {
+        float *q = lds + 4 * (tid + BT * u);
+        if (BT * (u + 1) <= n4) {
             *reinterpret_cast<float4 *>(q) = stage[u];
-        } else if (LDS_BLOCK * u < n4) {
-            if (tid + LDS_BLOCK * u < n4) *reinterpret_cast<float4 *>(q) = stage[u];
+        } else if (BT * u < n4) {
+            if (tid + BT * u < n4) *reinterpret_cast<float4 *>(q) = stage[u];
         }
     }
-    for (int i = (n4 << 2) + tid; i < n; i += LDS_BLOCK) lds[i] = src[i];  // ragged end of the last group
+    for (int i = (n4 << 2) + tid; i < n; i += BT) lds[i] = src[i];  // ragged end of the last group
     __syncthreads();
 
     constexpr int RPP = WAVE / SUB;  // rows per wave pass
     const int s = lane & (SUB - 1);
     const int rr = lane / SUB;
-    for (int r0 = wave * RPP; r0 < nrows; r0 += LDS_WAVES * RPP) {
+    for (int r0 = wave * RPP; r0 < nrows; r0 += (BT / WAVE) * RPP) {
         const int r = r0 + rr < nrows ? r0 + rr : nrows - 1;  // lane groups past the end redo the last row and write nothing
         const float *row = lds + r * len;
         float acc = OP::identity();
@@ -912,20 +911,26 @@ template <int VEC, int NCH> struct LayerNormLauncher {
 // Launches softmax_lds with the lane-group width and chunk count that waste the
 // fewest lane slots for this row length (len <= 1024): 16 lanes per row up to
 // 256 elements, 32 up to 512, 64 above.
-template <int SUB, int NCH>
-void softmax_lds_go(bool nt, dim3 grid, size_t shmem, hipStream_t s, float *out, const float *in, size_t rows,
-                    int len, int g, const SoftmaxPrologue *pro) {
+template <int BT, int SUB, int NCH>
+void softmax_lds_go_bt(bool nt, dim3 grid, size_t shmem, hipStream_t s, float *out, const float *in, size_t rows,
+                       int len, int g, const SoftmaxPrologue *pro) {
     const SoftmaxPrologue none{0, 0.0f, nullptr, 1, 0};
     if (pro) {
         if (nt)
-            hipLaunchKernelGGL((softmax_lds<SUB, NCH, true, true>), grid, dim3(LDS_BLOCK), shmem, s, out, in, rows, len, g, *pro);
+            hipLaunchKernelGGL((softmax_lds<BT, SUB, NCH, true, true>), grid, dim3(BT), shmem, s, out, in, rows, len, g, *pro);
         else
-            hipLaunchKernelGGL((softmax_lds<SUB, NCH, false, true>), grid, dim3(LDS_BLOCK), shmem, s, out, in, rows, len, g, *pro);
+            hipLaunchKernelGGL((softmax_lds<BT, SUB, NCH, false, true>), grid, dim3(BT), shmem, s, out, in, rows, len, g, *pro);
     } else if (nt) {
-        hipLaunchKernelGGL((softmax_lds<SUB, NCH, true, false>), grid, dim3(LDS_BLOCK), shmem, s, out, in, rows, len, g, none);
+        hipLaunchKernelGGL((softmax_lds<BT, SUB, NCH, true, false>), grid, dim3(BT), shmem, s, out, in, rows, len, g, none);
     } else {
-        hipLaunchKernelGGL((softmax_lds<SUB, NCH, false, false>), grid, dim3(LDS_BLOCK), shmem, s, out, in, rows, len, g, none);
+        hipLaunchKernelGGL((softmax_lds<BT, SUB, NCH, false, false>), grid, dim3(BT), shmem, s, out, in, rows, len, g, none);
     }
+}
+template <int SUB, int NCH>
+void softmax_lds_go(int threads, bool nt, dim3 grid, size_t shmem, hipStream_t s, float *out, const float *in, size_t rows,
+                    int len, int g, const SoftmaxPrologue *pro) {
+    if (threads == LDS_BLOCK) softmax_lds_go_bt<LDS_BLOCK, SUB, NCH>(nt, grid, shmem, s, out, in, rows, len, g, pro);
+    else softmax_lds_go_bt<LDS_BLOCK / 2, SUB, NCH>(nt, grid, shmem, s, out, in, rows, len, g, pro);
 }
 
 size_t gcd_size(size_t a, size_t b) {
@@ -939,17 +944,27 @@ size_t gcd_size(size_t a, size_t b) {
 
 // Rows per block: the smallest count whose span is a whole number of 128-byte lines (or of
 // 64/32/16 bytes when that would not fit), repeated up to the LDS budget.
-size_t softmax_lds_group_rows(size_t len) {
+size_t softmax_lds_group_rows(size_t len, size_t budget_floats = LDS_GROUP_FLOATS) {
     for (size_t align_floats = 32; align_floats >= 4; align_floats /= 2) {
         const size_t base = align_floats / gcd_size(len, align_floats);
-        if (base * len <= LDS_GROUP_FLOATS) {
-            size_t m = LDS_GROUP_FLOATS / (base * len);
+        if (base * len <= budget_floats) {
+            size_t m = budget_floats / (base * len);
             const size_t max_rows = 1024;
             if (base * m > max_rows) m = max_rows / base > 0 ? max_rows / base : 1;
             return base * m;
         }
     }
     return 4;  // unreachable for len <= 1024: 4 rows are at most 4096 floats
+}
+
+// Threads of a block of the LDS-staged kernels.  Half-wide blocks (512 threads, 16 KiB groups) put four blocks on a CU
+// instead of two, and every block loads, computes and stores in turn: Softmax and LayerNormalization gain 2-3 points
+// of the HBM peak at 49, 64, 100, 128 and 1000 elements.  Where the smallest line-aligned group of rows does not fit
+// 16 KiB (197: 32 rows are 25 KiB) the narrow block would have to cut groups inside a 128-byte line and loses 2-5
+// points (one point of that comes back when the two blocks that share a line are dealt to one XCD): those keep the
+// wide block.
+inline int lds_block_threads(size_t len) {
+    return 32 / gcd_size(len, 32) * len <= LDS_GROUP_FLOATS / 2 ? LDS_BLOCK / 2 : LDS_BLOCK;
 }
 
 // Lanes per row and chunks per lane for a row of L <= 1024 elements in the LDS-staged kernels: the narrowest lane
@@ -990,7 +1005,8 @@ size_t softmax_lds_group_rows(size_t len) {
 bool softmax_lds_launch(hipStream_t s, float *out, const float *in, size_t rows, size_t len, bool nt,
                         const SoftmaxPrologue *pro = nullptr) {
     static_assert(4 * 1024 <= LDS_GROUP_FLOATS, "four rows of the longest supported length must fit");
-    size_t g = softmax_lds_group_rows(len);
+    const int threads = lds_block_threads(len);
+    size_t g = softmax_lds_group_rows(len, (size_t)STAGE_LDS * threads * 4);
     // A group may straddle one boundary between mask rows, not more: with a mask, groups are cut
     // down to a line-aligned row count that does not exceed the rows of one mask row.
     if (pro && pro->mask && pro->rows_per_mask < g) {
@@ -1006,23 +1022,30 @@ bool softmax_lds_launch(hipStream_t s, float *out, const float *in, size_t rows,
     const int L = (int)len, G = (int)g;
 #define ALTIUS_GO(SUB, N)                                                    \
     case N:                                                                  \
-        softmax_lds_go<SUB, N>(nt, grid, shmem, s, out, in, rows, L, G, pro); \
+        softmax_lds_go<SUB, N>(threads, nt, grid, shmem, s, out, in, rows, L, G, pro); \
         return true;
     ALTIUS_LDS_LAYOUTS(L)
 #undef ALTIUS_GO
     return false;
 }
 
+template <int BT, int SUB, int NCH>
+void layernorm_lds_go_bt(bool nt, dim3 grid, size_t shmem, hipStream_t s, float *out, const float *in, const float *gamma, const float *beta,
+                         size_t rows, int len, int g, float eps) {
+    if (nt) hipLaunchKernelGGL((layernorm_lds<BT, SUB, NCH, true>), grid, dim3(BT), shmem, s, out, in, gamma, beta, rows, len, g, eps);
+    else hipLaunchKernelGGL((layernorm_lds<BT, SUB, NCH, false>), grid, dim3(BT), shmem, s, out, in, gamma, beta, rows, len, g, eps);
+}
 template <int SUB, int NCH>
-void layernorm_lds_go(bool nt, dim3 grid, size_t shmem, hipStream_t s, float *out, const float *in, const float *gamma, const float *beta,
-                      size_t rows, int len, int g, float eps) {
-    if (nt) hipLaunchKernelGGL((layernorm_lds<SUB, NCH, true>), grid, dim3(LDS_BLOCK), shmem, s, out, in, gamma, beta, rows, len, g, eps);
-    else hipLaunchKernelGGL((layernorm_lds<SUB, NCH, false>), grid, dim3(LDS_BLOCK), shmem, s, out, in, gamma, beta, rows, len, g, eps);
+void layernorm_lds_go(int threads, bool nt, dim3 grid, size_t shmem, hipStream_t s, float *out, const float *in, const float *gamma,
+                      const float *beta, size_t rows, int len, int g, float eps) {
+    if (threads == LDS_BLOCK) layernorm_lds_go_bt<LDS_BLOCK, SUB, NCH>(nt, grid, shmem, s, out, in, gamma, beta, rows, len, g, eps);
+    else layernorm_lds_go_bt<LDS_BLOCK / 2, SUB, NCH>(nt, grid, shmem, s, out, in, gamma, beta, rows, len, g, eps);
 }
 
 bool layernorm_lds_launch(hipStream_t s, float *out, const float *in, const float *gamma, const float *beta, size_t rows, size_t len, float eps,
                           bool nt) {
-    const size_t g = softmax_lds_group_rows(len);
+    const int threads = lds_block_threads(len);
+    const size_t g = softmax_lds_group_rows(len, (size_t)STAGE_LDS * threads * 4);
     const size_t groups = (rows + g - 1) / g;
     if ((g * len) % 4 != 0 || groups > 0x7FFFFFFFu) return false;
     const dim3 grid((unsigned)groups);
@@ -1030,7 +1053,7 @@ bool layernorm_lds_launch(hipStream_t s, float *out, const float *in, const floa
     const int L = (int)len, G = (int)g;
 #define ALTIUS_GO(SUB, N)                                                                     \
     case N:                                                                                   \
-        layernorm_lds_go<SUB, N>(nt, grid, shmem, s, out, in, gamma, beta, rows, L, G, eps);   \
+        layernorm_lds_go<SUB, N>(threads, nt, grid, shmem, s, out, in, gamma, beta, rows, L, G, eps); \
         return true;
     ALTIUS_LDS_LAYOUTS(L)
 #undef ALTIUS_GO
@@ -1169,7 +1192,11 @@ int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *g
 // Row sums / maxima through reduce_rows_lds; -1 (nothing launched) when the shape is not one it is meant for.
 int launch_reduce_rows_lds(DeviceCtx &ctx, bool is_max, float *out, const float *in, size_t rows, size_t len, float scale, bool scaled) {
     if (len == 0 || len > 1024 || rows < 64 || !aligned16(in)) return -1;
-    const size_t g = softmax_lds_group_rows(len);
+    // Read-only: blocks of 512 threads, four to a CU (72-75 % of the HBM peak with 1024 become 83-90 %); two float4 per
+    // thread where a line-aligned group of rows fits 16 KiB, four where it takes 32 KiB (197).
+    constexpr int RT = LDS_BLOCK / 2;
+    const bool deep = lds_block_threads(len) == LDS_BLOCK;
+    const size_t g = softmax_lds_group_rows(len, (size_t)(deep ? 4 : 2) * RT * 4);
     if ((g * len) % 4 != 0) return -1;  // groups must start 16-byte aligned
     const size_t groups = (rows + g - 1) / g;
     if (groups > 0x7FFFFFFFu) return -1;
@@ -1179,8 +1206,10 @@ int launch_reduce_rows_lds(DeviceCtx &ctx, bool is_max, float *out, const float 
     const int L = (int)len, G = (int)g;
 #define ALTIUS_RED(OP, SUB, SC)                                                                                                   \
     do {                                                                                                                          \
-        if (nt) hipLaunchKernelGGL((reduce_rows_lds<OP, SUB, SC, true>), grid, dim3(LDS_BLOCK), shmem, ctx.stream, out, in, rows, L, G, scale);  \
-        else hipLaunchKernelGGL((reduce_rows_lds<OP, SUB, SC, false>), grid, dim3(LDS_BLOCK), shmem, ctx.stream, out, in, rows, L, G, scale);    \
+        if (deep && nt) hipLaunchKernelGGL((reduce_rows_lds<RT, 4, OP, SUB, SC, true>), grid, dim3(RT), shmem, ctx.stream, out, in, rows, L, G, scale);  \
+        else if (deep) hipLaunchKernelGGL((reduce_rows_lds<RT, 4, OP, SUB, SC, false>), grid, dim3(RT), shmem, ctx.stream, out, in, rows, L, G, scale);  \
+        else if (nt) hipLaunchKernelGGL((reduce_rows_lds<RT, 2, OP, SUB, SC, true>), grid, dim3(RT), shmem, ctx.stream, out, in, rows, L, G, scale);     \
+        else hipLaunchKernelGGL((reduce_rows_lds<RT, 2, OP, SUB, SC, false>), grid, dim3(RT), shmem, ctx.stream, out, in, rows, L, G, scale);           \
     } while (0)
 #define ALTIUS_RED_SUB(SUB)                                   \
     do {                                                      \
