@@ -799,14 +799,15 @@ __global__ __launch_bounds__(THREADS, 2048 / THREADS * (THREADS / WAVE) / 4) voi
 struct BlockLayout {
     int threads, nch;
 };
-// Measured over rows of 2048 to 16384 elements: two float4 per thread is the best shape (256 x 2 for 2048, 512 x 2
-// for 4096, 1024 x 2 for 6144 and 8192: 77-80 % of peak for Softmax), three cost little (512 x 3 for 5120, 1024 x 3
-// for 12288: 78-79 %), and a 16 K row has to take four, requested two at a time (72 %; all four at once costs
-// LayerNormalization 5 points).  Fewer threads with more float4 each (512 x 4..8, 256 x 5..16) are 3-8 points behind
-// at every length from 5120 up.
+// Measured over rows of 1536 to 16384 elements: two float4 per thread is the best shape (256 x 2 to 2048 elements,
+// 384 x 2 to 3072, 512 x 2 to 4096, 768 x 2 to 6144, 1024 x 2 to 8192: 79-81 % of peak for Softmax, 75-78 % for
+// LayerNormalization, which then requests scale and bias behind the row; with three float4 on fewer threads
+// LayerNormalization loses 2-4 points at 2560, 4608 and 5120), 1024 x 3 for 12288, and a 16 K row has to take four
+// (the kernels that request a row ahead).  Fewer threads with more float4 each (512 x 4..8, 256 x 5..16) are 3-8
+// points behind at every length from 5120 up.
 inline BlockLayout block_layout(size_t len) {
     const size_t v = len / 4;  // float4 per row
-    const int threads = v <= 512 ? 256 : v <= 1280 ? 512 : 1024;
+    const int threads = v <= 512 ? 256 : v <= 768 ? 384 : v <= 1024 ? 512 : v <= 1536 ? 768 : 1024;
     return BlockLayout{threads, (int)((v + threads - 1) / threads)};
 }
 
@@ -842,7 +843,7 @@ void layernorm_block_go(bool nt, hipStream_t s, size_t rows, size_t resident, fl
 // GO(THREADS, NCH) for the layout of a row; false if there is none.
 #define ALTIUS_BLOCK_LAYOUTS(L)                                                          \
     switch ((L).threads * 100 + (L).nch) {                                               \
-        ALTIUS_GO(256, 2) ALTIUS_GO(512, 2) ALTIUS_GO(512, 3) ALTIUS_GO(1024, 2) ALTIUS_GO(1024, 3) ALTIUS_GO(1024, 4) \
+        ALTIUS_GO(256, 2) ALTIUS_GO(384, 2) ALTIUS_GO(512, 2) ALTIUS_GO(768, 2) ALTIUS_GO(1024, 2) ALTIUS_GO(1024, 3) ALTIUS_GO(1024, 4) \
     }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -871,12 +872,12 @@ bool dispatch_wave(bool vec4, size_t len, Args... args) {
     return false;
 }
 
-// Rows of 1025 to 1536 elements that are whole float4s: still a wavefront per row with the row in registers
-// (6 float4 per lane), read once.
+// Rows of 1025 to 1280 elements that are whole float4s: still a wavefront per row with the row in registers
+// (5 float4 per lane), read once.
 template <template <int, int> class Launcher, class... Args>
 bool dispatch_wave_long(size_t len, Args... args) {
     const size_t chunks = (len / 4 + WAVE - 1) / WAVE;
-    if (chunks <= 6) { Launcher<4, 6>::go(args...); return true; }
+    if (chunks <= 5) { Launcher<4, 5>::go(args...); return true; }
     return false;
 }
 
@@ -1069,7 +1070,7 @@ inline bool wave_row_fits(size_t len) {
 }
 
 constexpr size_t MAX_WAVE_ROW = 1024;
-constexpr size_t MAX_LONG_ROW = 1536;  // rows kept in a wavefront's registers when they are whole float4s
+constexpr size_t MAX_LONG_ROW = 1280;  // rows kept in a wavefront's registers when they are whole float4s (at 1536 a block per row is 2 points ahead)
 constexpr size_t MAX_BLOCK_REG_ROW = 16384;  // ... and in a block's registers
 constexpr size_t MAX_GRID = 0x7FFFFFFFu;
 
