@@ -344,6 +344,28 @@ def test_softmax_and_layernorm_of_many_long_rows(ctx, oracle, case, rows, length
         assert_close(got[pick], oracle.layer_norm(x[pick], g, b, 1e-5), what="layernorm of many long rows")
 
 
+@pytest.mark.parametrize("rows,length", [(40001, 197), (36 * 1100 + 7, 193), (12000, 700), (9003, 900), (33000, 205)])
+def test_softmax_of_many_rows_in_wide_groups(ctx, oracle, case, rows, length):
+    """Rows whose smallest line-aligned group takes the wide block, tens of thousands of them: not a bit may differ
+    from the same rows a few thousand at a time, with the scale and mask prologue and without; ragged last groups,
+    row counts that are not whole float4s in total."""
+    case(f"softmax of {rows} rows of {length}")
+    x = synth.normal(81, (rows, length), std=2.0)
+    x[11, 5] = np.nan
+    x[rows - 1] = -3.0
+    with np.errstate(all="ignore"):
+        got = ctx.softmax(x)
+        few = np.concatenate([ctx.softmax(x[i : i + 3000]) for i in range(0, rows, 3000)])
+        assert_bits_equal(got, few, "softmax: all rows vs a few thousand at a time")
+        pick = np.r_[0:16, rows // 2 : rows // 2 + 8, rows - 8 : rows]
+        assert_close(got[pick], oracle.softmax(x[pick]), what="softmax of many rows")
+        per_mask = 1000 if rows % 1000 == 0 else 3 if rows % 3 == 0 else 1
+        mask = np.where(synth.normal(82, (rows // per_mask, length)) > 1.2, np.float32(-1e4), np.float32(0))
+        fused = ctx.softmax_prologue(x, 2, 8.0, mask)
+        z = x / np.float32(8.0) + np.repeat(mask, per_mask, axis=0)
+        assert_bits_equal(fused, ctx.softmax(z), "prologue vs the operators")
+
+
 REDUCE_CASES = [
     # (shape, axes, keepdims)
     ([1, 50, 70], [-1], True),         # test_ops_reduce.py:10-18
