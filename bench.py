@@ -10,9 +10,12 @@ one "step" is one pass of the four kernels over device-resident fp32 inputs
     Div      [256,197,768] / scalar
 
 `value` is the whole step's algorithmic bytes (every tensor read or written once) divided by
-the step time, in GB/s.  Per-kernel times are measured with HIP events on the stream the
-kernels run on (mean, median and minimum over at least 100 launches after 20 warm-ups, and once
-more inside the running step); `roofline` describes the slowest kernel of the step.  Beside the
+the step time, in GB/s: W warm-up steps and K timed ones after the step has kept the GPU busy
+for --settle-ms; `value_after_idle` is the same W + K steps straight after the uploads, which
+leave the GPU idle for seconds (for a few milliseconds after an idle period the part runs
+slower).  Per-kernel times are measured with HIP events on the stream the kernels run on (mean,
+median and minimum over at least 100 launches after a warm-up of 20 launches and at least 25 ms,
+and once more inside the running step); `roofline` describes the slowest kernel of the step.  Beside the
 step the line carries every other operator of the path on the step's [256,197,768] array
 (`listed_ops`), Softmax / LayerNormalization / ReduceMean by row length (`row_sweep`) and the
 kernels and graphs of configs[0..3] (`other_configs`).  The CPU baseline is the oracle (a C++
