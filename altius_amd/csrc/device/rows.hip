@@ -35,13 +35,13 @@ template <int VEC, int NCH> struct RowRegs {
 
     // Loads the row; slots past `len` are set to `fill`.  NT: non-temporal 16-byte accesses, for tensors
     // too large to be found in a cache by the next kernel.
-    template <bool NT = false>
+    template <bool NT = false, bool FULL = false>
     __device__ __forceinline__ void load(const float *__restrict__ row, int len, int lane, float fill) {
 #pragma unroll
         for (int k = 0; k < NCH; k++) {
             const int e = (lane + WAVE * k) * VEC;
             if (VEC == 4) {
-                if (e < len) {
+                if (FULL || e < len) {
                     const float4 t = load4<NT>(row + e);
                     v[k * VEC + 0] = t.x;
                     v[k * VEC + 1 % VEC] = t.y;
@@ -56,12 +56,12 @@ template <int VEC, int NCH> struct RowRegs {
             }
         }
     }
-    template <bool NT = false>
+    template <bool NT = false, bool FULL = false>
     __device__ __forceinline__ void store(float *__restrict__ row, int len, int lane) const {
 #pragma unroll
         for (int k = 0; k < NCH; k++) {
             const int e = (lane + WAVE * k) * VEC;
-            if (e < len) {
+            if (FULL || e < len) {
                 if (VEC == 4) {
                     float4 t;
                     t.x = v[k * VEC + 0];
@@ -97,9 +97,12 @@ struct SoftmaxPrologue {
     uint32_t mask_rows;
 };
 
-template <int VEC, int NCH, bool PRO, bool NT>
+// FULL: the row fills every slot (len == NCH * 64 * VEC: 256, 512, 768, 1024), known when the kernel is built, so
+// that no load, store or summand is guarded: 36 of the 311 vector instructions of a 768-element row are such guards.
+template <int VEC, int NCH, bool PRO, bool NT, bool FULL = false>
 __global__ __launch_bounds__(BLOCK) void softmax_wave(float *__restrict__ out, const float *__restrict__ in,
-                                                      size_t rows, int len, const SoftmaxPrologue pro) {
+                                                      size_t rows, int len_arg, const SoftmaxPrologue pro) {
+    const int len = FULL ? NCH * WAVE * VEC : len_arg;
     const int lane = threadIdx.x & (WAVE - 1);
     const size_t row = (size_t)blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
     if (row >= rows) return;
@@ -108,12 +111,12 @@ __global__ __launch_bounds__(BLOCK) void softmax_wave(float *__restrict__ out, c
 
     RowRegs<VEC, NCH> r;
     const float nan = __builtin_nanf("");
-    r.template load<NT>(x, len, lane, nan);
+    r.template load<NT, FULL>(x, len, lane, nan);
     if (PRO) {
         // The mask row is shared by rows_per_mask score rows: it comes from the caches, and its load
         // is issued before the scores are looked at.
         RowRegs<VEC, NCH> m;
-        if (pro.mask) m.load(pro.mask + (size_t)((uint32_t)row / pro.rows_per_mask) * len, len, lane, 0.0f);
+        if (pro.mask) m.template load<false, FULL>(pro.mask + (size_t)((uint32_t)row / pro.rows_per_mask) * len, len, lane, 0.0f);
         if (pro.scale_code == 1) {
 #pragma unroll
             for (int s = 0; s < NCH * VEC; s++) r.v[s] = r.v[s] * pro.scale;
@@ -135,7 +138,7 @@ __global__ __launch_bounds__(BLOCK) void softmax_wave(float *__restrict__ out, c
     float sum = 0.0f;
 #pragma unroll
     for (int s = 0; s < NCH * VEC; s++) {
-        const bool valid = RowRegs<VEC, NCH>::index(lane, s) < len;
+        const bool valid = FULL || RowRegs<VEC, NCH>::index(lane, s) < len;
         const float e = softmax_exp(r.v[s], mx);
         r.v[s] = e;
         sum += valid ? e : 0.0f;
@@ -144,7 +147,7 @@ __global__ __launch_bounds__(BLOCK) void softmax_wave(float *__restrict__ out, c
     const float recip = 1.0f / sum;
 #pragma unroll
     for (int s = 0; s < NCH * VEC; s++) r.v[s] *= recip;
-    r.template store<NT>(o, len, lane);
+    r.template store<NT, FULL>(o, len, lane);
 }
 
 // Rows whose length is not a multiple of 4 (197 tokens, say) start at addresses
@@ -487,11 +490,12 @@ __global__ __launch_bounds__(BLOCK) void softmax_block_stream(float *__restrict_
 // ---------------------------------------------------------------------------
 // LayerNormalization
 // ---------------------------------------------------------------------------
-template <int VEC, int NCH, bool NT>
+template <int VEC, int NCH, bool NT, bool FULL = false>
 __global__ __launch_bounds__(BLOCK) void layernorm_wave(float *__restrict__ out, const float *__restrict__ in,
                                                         const float *__restrict__ gamma,
-                                                        const float *__restrict__ beta, size_t rows, int len,
+                                                        const float *__restrict__ beta, size_t rows, int len_arg,
                                                         float eps) {
+    const int len = FULL ? NCH * WAVE * VEC : len_arg;  // see softmax_wave
     const int lane = threadIdx.x & (WAVE - 1);
     const size_t row = (size_t)blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
     if (row >= rows) return;
@@ -499,14 +503,14 @@ __global__ __launch_bounds__(BLOCK) void layernorm_wave(float *__restrict__ out,
     float *o = out + row * (size_t)len;
 
     RowRegs<VEC, NCH> r;
-    r.template load<NT>(x, len, lane, 0.0f);
+    r.template load<NT, FULL>(x, len, lane, 0.0f);
     // Scale and bias are requested right behind the row, so that they arrive during the two reductions; for rows
     // of more than four chunks per lane they would not fit the registers and are fetched chunk by chunk at the end.
     constexpr bool EARLY = NCH <= 4;
     RowRegs<VEC, EARLY ? NCH : 1> g, b;
     if (EARLY) {
-        g.load(gamma, len, lane, 0.0f);
-        b.load(beta, len, lane, 0.0f);
+        g.template load<false, FULL>(gamma, len, lane, 0.0f);
+        b.template load<false, FULL>(beta, len, lane, 0.0f);
     }
 
     const float inv_n = 1.0f / (float)len;
@@ -518,7 +522,7 @@ __global__ __launch_bounds__(BLOCK) void layernorm_wave(float *__restrict__ out,
     float ss = 0.0f;
 #pragma unroll
     for (int s = 0; s < NCH * VEC; s++) {
-        const bool valid = RowRegs<VEC, NCH>::index(lane, s) < len;
+        const bool valid = FULL || RowRegs<VEC, NCH>::index(lane, s) < len;
         const float d = r.v[s] - mean;
         r.v[s] = d;
         ss += valid ? d * d : 0.0f;
@@ -533,13 +537,13 @@ __global__ __launch_bounds__(BLOCK) void layernorm_wave(float *__restrict__ out,
 #pragma unroll
         for (int k = 0; k < NCH; k++) {
             const int e = (lane + WAVE * k) * VEC;
-            if (e < len) {
+            if (FULL || e < len) {
 #pragma unroll
                 for (int j = 0; j < VEC; j++) r.v[k * VEC + j] = __builtin_fmaf(r.v[k * VEC + j] * inv_std, gamma[e + j], beta[e + j]);
             }
         }
     }
-    r.template store<NT>(o, len, lane);
+    r.template store<NT, FULL>(o, len, lane);
 }
 
 __global__ __launch_bounds__(BLOCK) void layernorm_block_stream(float *__restrict__ out,
@@ -885,6 +889,15 @@ template <int VEC, int NCH> struct SoftmaxLauncher {
     static void go(hipStream_t s, float *out, const float *in, size_t rows, int len, const SoftmaxPrologue *pro, bool nt) {
         const dim3 grid((unsigned)((rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK));
         const SoftmaxPrologue none{0, 0.0f, nullptr, 1, 0};
+        if constexpr (VEC == 4 && NCH <= 4) {
+            if (len == NCH * WAVE * VEC) {  // every slot of the wavefront's chunks is an element
+                if (pro && nt) hipLaunchKernelGGL((softmax_wave<VEC, NCH, true, true, true>), grid, dim3(BLOCK), 0, s, out, in, rows, len, *pro);
+                else if (pro) hipLaunchKernelGGL((softmax_wave<VEC, NCH, true, false, true>), grid, dim3(BLOCK), 0, s, out, in, rows, len, *pro);
+                else if (nt) hipLaunchKernelGGL((softmax_wave<VEC, NCH, false, true, true>), grid, dim3(BLOCK), 0, s, out, in, rows, len, none);
+                else hipLaunchKernelGGL((softmax_wave<VEC, NCH, false, false, true>), grid, dim3(BLOCK), 0, s, out, in, rows, len, none);
+                return;
+            }
+        }
         if (pro && nt && VEC == 4)
             hipLaunchKernelGGL((softmax_wave<VEC, NCH, true, true>), grid, dim3(BLOCK), 0, s, out, in, rows, len, *pro);
         else if (pro)
@@ -900,6 +913,13 @@ template <int VEC, int NCH> struct LayerNormLauncher {
     static void go(hipStream_t s, float *out, const float *in, const float *gamma, const float *beta,
                    size_t rows, int len, float eps, bool nt) {
         const size_t blocks = (rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+        if constexpr (VEC == 4 && NCH <= 4) {
+            if (len == NCH * WAVE * VEC) {
+                if (nt) hipLaunchKernelGGL((layernorm_wave<VEC, NCH, true, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, gamma, beta, rows, len, eps);
+                else hipLaunchKernelGGL((layernorm_wave<VEC, NCH, false, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, gamma, beta, rows, len, eps);
+                return;
+            }
+        }
         if (nt && VEC == 4)
             hipLaunchKernelGGL((layernorm_wave<VEC, NCH, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in,
                                gamma, beta, rows, len, eps);
