@@ -889,7 +889,7 @@ template <int VEC, int NCH> struct SoftmaxLauncher {
     static void go(hipStream_t s, float *out, const float *in, size_t rows, int len, const SoftmaxPrologue *pro, bool nt) {
         const dim3 grid((unsigned)((rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK));
         const SoftmaxPrologue none{0, 0.0f, nullptr, 1, 0};
-        if constexpr (VEC == 4 && NCH <= 4) {
+        if constexpr (VEC == 4 && NCH <= 4) {  // with five chunks the five unguarded loads in a row cost 3 points
             if (len == NCH * WAVE * VEC) {  // every slot of the wavefront's chunks is an element
                 if (pro && nt) hipLaunchKernelGGL((softmax_wave<VEC, NCH, true, true, true>), grid, dim3(BLOCK), 0, s, out, in, rows, len, *pro);
                 else if (pro) hipLaunchKernelGGL((softmax_wave<VEC, NCH, true, false, true>), grid, dim3(BLOCK), 0, s, out, in, rows, len, *pro);
@@ -913,7 +913,7 @@ template <int VEC, int NCH> struct LayerNormLauncher {
     static void go(hipStream_t s, float *out, const float *in, const float *gamma, const float *beta,
                    size_t rows, int len, float eps, bool nt) {
         const size_t blocks = (rows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-        if constexpr (VEC == 4 && NCH <= 4) {
+        if constexpr (VEC == 4 && NCH <= 5) {
             if (len == NCH * WAVE * VEC) {
                 if (nt) hipLaunchKernelGGL((layernorm_wave<VEC, NCH, true, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, gamma, beta, rows, len, eps);
                 else hipLaunchKernelGGL((layernorm_wave<VEC, NCH, false, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, gamma, beta, rows, len, eps);
