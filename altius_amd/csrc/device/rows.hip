@@ -499,25 +499,33 @@ __global__ __launch_bounds__(BLOCK) void layernorm_wave(float *__restrict__ out,
     const int lane = threadIdx.x & (WAVE - 1);
     size_t row = (size_t)blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
     constexpr bool EARLY = NCH <= 4;
-    // Rows that fill every slot of two to four chunks: the block's four wavefronts fetch scale and bias once between
-    // them and pass them on through LDS (a wavefront of its own reads 2 x the row's bytes of them from the caches per
-    // row): 512 / 768 / 1024 elements gain about one point of the HBM peak; with one chunk (256) the barrier costs 3.
-    constexpr bool SHARE = FULL && EARLY && VEC == 4 && NCH >= 2;
+    // Rows of two chunks and more (whole float4s): the block's four wavefronts fetch scale and bias once between them
+    // and pass them on through LDS (a wavefront of its own reads 2 x the row's bytes of them from the caches per
+    // row): 512 / 768 / 1024 elements gain about one point of the HBM peak, 384 two; with one chunk (256) the barrier
+    // costs 3.  Up to four chunks they are read back into registers at once (SHARE); with five they wait in the
+    // requesting thread's registers during the reductions and go through LDS just before they are used (LATE).
+    constexpr bool SHARE = EARLY && VEC == 4 && NCH >= 2;
+    constexpr bool LATE = !EARLY && VEC == 4;
+    constexpr int GB = 2 * NCH * WAVE;  // float4s of scale and bias
+    __shared__ float4 gb_lds[SHARE || LATE ? GB : 1];
+    auto fetch_gb = [&](int i) {
+        const int e = 4 * (i < NCH * WAVE ? i : i - NCH * WAVE);
+        return FULL || e < len ? *reinterpret_cast<const float4 *>((i < NCH * WAVE ? gamma : beta) + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+    };
     const bool active = row < rows;
-    if (!SHARE && !active) return;
+    if (!SHARE && !LATE && !active) return;
     if (!active) row = rows - 1;  // keeps the block's barrier company; stores nothing
     const float *x = in + row * (size_t)len;
     float *o = out + row * (size_t)len;
 
     RowRegs<VEC, NCH> r;
     r.template load<NT, FULL>(x, len, lane, 0.0f);
-    // Scale and bias are requested right behind the row, so that they arrive during the two reductions; for rows
-    // of more than four chunks per lane they would not fit the registers and are fetched chunk by chunk at the end.
+    // Scale and bias are requested right behind the row, so that they arrive during the two reductions.
     RowRegs<VEC, EARLY ? NCH : 1> g, b;
+    constexpr int STAGED = LATE ? (GB + BLOCK - 1) / BLOCK : 1;
+    float4 staged[STAGED];
     if (SHARE) {
-        __shared__ float4 gb_lds[SHARE ? 2 * NCH * WAVE : 1];
-        for (int i = threadIdx.x; i < 2 * NCH * WAVE; i += BLOCK)
-            gb_lds[i] = *reinterpret_cast<const float4 *>((i < NCH * WAVE ? gamma : beta - 4 * NCH * WAVE) + 4 * i);
+        for (int i = threadIdx.x; i < GB; i += BLOCK) gb_lds[i] = fetch_gb(i);
         __syncthreads();
 #pragma unroll
         for (int k = 0; k < NCH; k++) {
@@ -528,6 +536,12 @@ __global__ __launch_bounds__(BLOCK) void layernorm_wave(float *__restrict__ out,
             b.v[(k * 4 + 2) % (EARLY ? NCH * VEC : 1)] = bv.z, b.v[(k * 4 + 3) % (EARLY ? NCH * VEC : 1)] = bv.w;
         }
         if (!active) return;
+    } else if (LATE) {
+#pragma unroll
+        for (int u = 0; u < STAGED; u++) {
+            const int i = threadIdx.x + u * BLOCK;
+            if (i < GB) staged[u] = fetch_gb(i);
+        }
     } else if (EARLY) {
         g.template load<false, FULL>(gamma, len, lane, 0.0f);
         b.template load<false, FULL>(beta, len, lane, 0.0f);
@@ -553,6 +567,22 @@ __global__ __launch_bounds__(BLOCK) void layernorm_wave(float *__restrict__ out,
     if (EARLY) {
 #pragma unroll
         for (int s = 0; s < NCH * VEC; s++) r.v[s] = __builtin_fmaf(r.v[s] * inv_std, g.v[EARLY ? s : 0], b.v[EARLY ? s : 0]);
+    } else if (LATE) {
+#pragma unroll
+        for (int u = 0; u < STAGED; u++) {
+            const int i = threadIdx.x + u * BLOCK;
+            if (i < GB) gb_lds[i] = staged[u];
+        }
+        __syncthreads();
+        if (!active) return;
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            const float4 gv = gb_lds[lane + WAVE * k], bv = gb_lds[NCH * WAVE + lane + WAVE * k];
+            r.v[(k * 4 + 0) % (NCH * VEC)] = __builtin_fmaf(r.v[(k * 4 + 0) % (NCH * VEC)] * inv_std, gv.x, bv.x);
+            r.v[(k * 4 + 1) % (NCH * VEC)] = __builtin_fmaf(r.v[(k * 4 + 1) % (NCH * VEC)] * inv_std, gv.y, bv.y);
+            r.v[(k * 4 + 2) % (NCH * VEC)] = __builtin_fmaf(r.v[(k * 4 + 2) % (NCH * VEC)] * inv_std, gv.z, bv.z);
+            r.v[(k * 4 + 3) % (NCH * VEC)] = __builtin_fmaf(r.v[(k * 4 + 3) % (NCH * VEC)] * inv_std, gv.w, bv.w);
+        }
     } else {
 #pragma unroll
         for (int k = 0; k < NCH; k++) {

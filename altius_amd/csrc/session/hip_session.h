@@ -147,9 +147,9 @@ public:
     // events on the session's stream.
     double last_device_ms() const { return last_device_ms_; }
     size_t device_allocations() const { return pool_->device_allocations(); }
-    // Runs served by replaying a captured HIP graph since the session was built.
     // Nodes of the last node-by-node run that produced a view or wrote a following Transpose's layout.
     size_t copies_avoided() const { return copies_avoided_; }
+    // Runs served by replaying a captured HIP graph since the session was built.
     size_t graph_replays() const { return graph_replays_; }
     const std::vector<NodeExecutionPlan> &execution_plan() const { return plan_; }
     const InferredShapes &inferred_shapes() const { return inferred_; }
@@ -251,7 +251,7 @@ private:
     std::map<std::string, CapturedRun> graphs_;
     std::map<std::string, int> eager_runs_;  // per input signature: eager runs so far (the pool is warm after one)
     size_t graph_replays_ = 0;
-    uint64_t seen_ws_generation_ = 0;
+    uint64_t seen_ws_generation_ = 0;  // recorded launches hold the GEMM workspace's address: graphs are dropped when it moves
     size_t copies_avoided_ = 0;
     NodeId current_node_ = 0;  // the node run_device_op is working on
     std::map<NodeId, AttentionPlan> attn_head_;                  // first MatMul of a fusable attention -> the rest
@@ -286,7 +286,7 @@ private:
     // Runs a deferred Add into the tensor's block.
     bool flush_add(DeviceTensor *t, SessionError *err);
     std::set<NodeId> lazy_views_;                               // Split / Transpose nodes whose outputs are views
-    std::map<NodeId, std::vector<int64_t>> matmul_out_perm_;    // MatMul nodes -> perm of the Transpose they feed  // recorded launches hold the GEMM workspace's address
+    std::map<NodeId, std::vector<int64_t>> matmul_out_perm_;    // MatMul nodes -> perm of the Transpose they feed
 };
 
 class HipSessionBuilder {

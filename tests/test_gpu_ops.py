@@ -262,7 +262,8 @@ SOFTMAX_SHAPES = [[1, 2, 3], [3, 28, 28], [16, 512, 512], [2, 12, 197, 197], [5,
                   [3, 1000], [2, 1024], [3, 1025], [2, 4096], [2, 5000], [1, 70001],
                   [3, 1028], [5, 1280], [9, 1536], [3, 2048], [2, 2560], [4, 3072], [2, 4092], [2, 4100],  # rows of 1025..4096 whole float4s stay in registers
                   [2, 5120], [3, 8192], [2, 8196], [2, 16384], [1, 12000], [2, 16388], [2, 5001],  # up to 16384: in a block's registers
-                  [3, 1284], [3, 2052], [2, 3076], [2, 4608], [2, 6144], [2, 6148], [2, 12288]]  # either side of every block width
+                  [3, 1284], [3, 2052], [2, 3076], [2, 4608], [2, 6144], [2, 6148], [2, 12288],  # either side of every block width
+                  [5, 384], [7, 640], [6, 896], [3, 1088], [9, 1152], [13, 320]]  # a wavefront per row, last chunk partly filled
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
@@ -301,7 +302,8 @@ LN_SHAPES = [[1, 20, 10], [2, 197, 768], [3, 5, 197], [4, 1], [5, 64], [3, 1024]
              [5, 1280], [9, 1536], [3, 2048], [2, 2560], [2, 4092], [7, 4096], [2, 1026],
              [100, 49], [70, 197], [300, 64], [1000, 10], [64, 255], [65, 1], [200, 130], [4, 700, 192],  # short rows in groups through LDS
              [2, 5120], [3, 8192], [2, 8196], [2, 16384], [1, 12000], [2, 16388], [2, 5001],  # rows up to 16384 in a block's registers
-             [3, 1284], [3, 2052], [2, 3076], [2, 4608], [2, 6144], [2, 6148], [2, 12288]]  # either side of every block width
+             [3, 1284], [3, 2052], [2, 3076], [2, 4608], [2, 6144], [2, 6148], [2, 12288],  # either side of every block width
+             [5, 384], [7, 640], [6, 896], [3, 1088], [9, 1152], [1, 512], [13, 320]]  # a wavefront per row, last chunk partly filled, rows not a multiple of the block's four
 
 
 @pytest.mark.parametrize("shape", LN_SHAPES)
