@@ -321,6 +321,39 @@ def test_layernorm(ctx, oracle, case, shape):
     np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5)
 
 
+UNALIGNED_ROWS = [(7, 768), (5, 197), (3, 1280), (2, 4096), (2, 8192), (3, 1000), (9, 64)]
+
+
+@pytest.mark.parametrize("rows,length", UNALIGNED_ROWS)
+@pytest.mark.parametrize("in_off,out_off", [(1, 0), (0, 3), (2, 2)])
+def test_row_and_unary_operators_on_unaligned_pointers(ctx, oracle, case, rows, length, in_off, out_off):
+    """The reference's tensors are plain slices of floats: nothing promises 16-byte alignment.  Input and output start
+    in_off / out_off floats past an aligned address (other kernels take such calls, with their own order of summation,
+    so the sums are checked against the oracle, not against the aligned call's bits)."""
+    case(f"Softmax / LayerNormalization / ReduceMean / ReduceMax / Gelu on [{rows},{length}], input +{in_off} floats, output +{out_off}")
+    x = synth.normal(71, (rows, length), mean=0.2, std=1.5)
+    g = synth.normal(72, (length,), mean=1.0, std=0.05)
+    b = synth.normal(73, (length,), mean=0.0, std=0.05)
+    n = rows * length
+    pad = np.zeros(in_off, np.float32)
+    dx = ctx.upload(np.concatenate([pad, x.ravel()]))
+    dg, db = ctx.upload(np.concatenate([pad, g])), ctx.upload(np.concatenate([pad, b]))
+    do = ctx.alloc((n + 4) * 4)
+    px, pg, pb, po = dx.ptr + 4 * in_off, dg.ptr + 4 * in_off, db.ptr + 4 * in_off, do.ptr + 4 * out_off
+    ctx.softmax_raw(po, px, rows, length)
+    assert_close(ctx.download(do, (rows, length), offset_bytes=4 * out_off), oracle.softmax(x), what="Softmax")
+    ctx.layernorm_raw(po, px, pg, pb, rows, length, 1e-5)
+    assert_close(ctx.download(do, (rows, length), offset_bytes=4 * out_off), oracle.layer_norm(x, g, b, 1e-5), what="LayerNormalization")
+    ctx.reduce_raw(D.REDUCE_MEAN, po, px, rows, length, 1)
+    assert_close(ctx.download(do, (rows, 1), offset_bytes=4 * out_off), oracle.reduce(oracle.REDUCE_MEAN, x, [1], True), what="ReduceMean")
+    ctx.reduce_raw(D.REDUCE_MAX, po, px, 1, rows, length)
+    assert_bits_equal(ctx.download(do, (1, length), offset_bytes=4 * out_off), x.max(0, keepdims=True), "ReduceMax over rows")
+    ctx.unary_raw(D.GELU, po, px, n)
+    assert_bits_equal(ctx.download(do, (rows, length), offset_bytes=4 * out_off), oracle.unary(oracle.GELU, x), "Gelu")
+    for t in (dx, dg, db, do):
+        ctx.free(t)
+
+
 # More rows than blocks fit the device, of lengths that take 1024 threads: the kernels that request a row ahead.
 MANY_LONG_ROWS = [(1100, 5120), (1029, 6144), (1500, 8192), (1031, 8196), (1100, 12288), (1111, 16384), (1040, 16380), (2100, 5004)]
 
