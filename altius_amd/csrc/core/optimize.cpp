@@ -46,6 +46,17 @@ void replace_value(Model &m, const Users &users, ValueId from, ValueId to) {
         if (out == from) out = to;
 }
 
+// Matches are collected on the graph as it was, and rewritten one after the other in topological order: where one
+// pattern starts at the value another one ends in (two chains back to back), the later one has to read what the
+// earlier rewrite put in that value's place.
+struct Renamed {
+    std::map<ValueId, ValueId> to;
+    ValueId operator()(ValueId v) const {
+        auto it = to.find(v);
+        return it == to.end() ? v : it->second;
+    }
+};
+
 }  // namespace
 
 size_t fuse_layer_norm(Model &model) {
@@ -85,12 +96,14 @@ size_t fuse_layer_norm(Model &model) {
         doomed.insert(doomed.end(), ids.begin(), ids.end());
     }
 
+    Renamed now;
     for (const Match &m : matches) {
         const ValueId ln_out = model.graph.values.new_val();
         Node ln(Op::layer_normalization(-1, m.epsilon, 1));
-        ln.with_in(m.data).with_in(m.scale).with_in(m.bias).with_out(ln_out);
+        ln.with_in(now(m.data)).with_in(now(m.scale)).with_in(now(m.bias)).with_out(ln_out);
         model.graph.add_node(std::move(ln));
         replace_value(model, users, m.end, ln_out);
+        now.to[m.end] = ln_out;
     }
     for (NodeId id : doomed) model.graph.nodes[id].deleted = true;
     model.remove_unnecessary_nodes();
@@ -140,12 +153,14 @@ size_t fuse_gelu(Model &model) {
         for (NodeId id : {div_id, *erf_id, *add_id, *mul1_id, *mul2_id}) doomed.push_back(id);
     }
 
+    Renamed now;
     for (const Match &m : matches) {
         const ValueId gelu_out = model.graph.values.new_val();
         Node gelu{Op(OpKind::Gelu)};
-        gelu.with_in(m.start).with_out(gelu_out);
+        gelu.with_in(now(m.start)).with_out(gelu_out);
         model.graph.add_node(std::move(gelu));
         replace_value(model, users, m.end, gelu_out);
+        now.to[m.end] = gelu_out;
     }
     for (NodeId id : doomed) model.graph.nodes[id].deleted = true;
     model.remove_unnecessary_nodes();
@@ -223,12 +238,14 @@ size_t fuse_fast_gelu(Model &model) {
             doomed.push_back(id);
     }
 
+    Renamed now;
     for (const Match &m : matches) {
         const ValueId gelu_out = model.graph.values.new_val();
         Node gelu{Op(OpKind::Gelu)};
-        gelu.with_in(m.start).with_out(gelu_out);
+        gelu.with_in(now(m.start)).with_out(gelu_out);
         model.graph.add_node(std::move(gelu));
         replace_value(model, users, m.end, gelu_out);
+        now.to[m.end] = gelu_out;
     }
     for (NodeId id : doomed) model.graph.nodes[id].deleted = true;
     model.remove_unnecessary_nodes();

@@ -253,6 +253,39 @@ def test_fuse_layer_norm():
     assert m.fuse_layer_norm() == 0 and len(m.nodes()) == 2
 
 
+def test_fused_chains_back_to_back_read_each_other():
+    """Two patterns where the second starts at the value the first ends in (the matches are collected before any of
+    them is rewritten, layer_norm_fusion.rs:24-139, gelu_fusion.rs:12-74): the second fused node must read the first
+    one's new output, also where that value is a graph output as well."""
+    for middle_is_output in (False, True):
+        m = Model()
+        x = m.new_val_named_and_shaped("x", [2, 8])
+        a, _, _ = layer_norm_chain(m, x, np.ones(8, np.float32), np.zeros(8, np.float32))
+        b, _, _ = layer_norm_chain(m, a, np.ones(8, np.float32), np.zeros(8, np.float32))
+        m.add_input(x)
+        if middle_is_output:
+            m.add_output(a)
+        m.add_output(b)
+        assert m.fuse_layer_norm() == 2
+        first, second = m.nodes()
+        assert first["inputs"][0] == x and second["inputs"][0] == first["outputs"][0]
+        assert m.outputs == ([first["outputs"][0]] if middle_is_output else []) + second["outputs"]
+        m.infer_value_shape(m.outputs[-1])  # every value has a producer
+
+        m = Model()
+        x = m.new_val_named_and_shaped("x", [1, 2, 3])
+        a = erf_gelu_chain(m, x)
+        b = erf_gelu_chain(m, a)
+        m.add_input(x)
+        if middle_is_output:
+            m.add_output(a)
+        m.add_output(b)
+        assert m.fuse_gelu() == 2
+        first, second = m.nodes()
+        assert first["inputs"] == [x] and second["inputs"] == first["outputs"]
+        assert m.outputs == ([first["outputs"][0]] if middle_is_output else []) + second["outputs"]
+
+
 def test_fuse_gelu():
     """crates/core/src/optimize/gelu_fusion.rs:12-82."""
     m = Model()
