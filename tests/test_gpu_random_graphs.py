@@ -35,14 +35,15 @@ def softmax(x):
 class RandomGraph:
     """A model under construction together with every value's float64 definition."""
 
-    def __init__(self, rng):
+    def __init__(self, rng, open_batch=False):
         self.rng = rng
+        self.open_batch = open_batch  # the input is declared without a shape and no node spells the batch out
         self.b = int(rng.choice([1, 2, 3, 8]))
         self.t = int(rng.choice([5, 16, 33, 45, 64, 197]))
         self.c = int(rng.choice([64, 128, 192, 256, 384]))
         self.m = Model(opset_version=13)
         self.ref, self.ops = {}, []
-        x = self.m.new_val_named_and_shaped("x", [self.b, self.t, self.c])
+        x = self.m.new_val_named("x") if open_batch else self.m.new_val_named_and_shaped("x", [self.b, self.t, self.c])
         self.m.add_input(x)
         self.feed = (rng.standard_normal((self.b, self.t, self.c)) * 0.5).astype(np.float32)
         self.ref[x] = self.feed.astype(np.float64)
@@ -123,7 +124,7 @@ class RandomGraph:
         qkv = self.linear(v, 3 * hd, bias=self.flip(0.7))
         sizes = self.init(np.array([hd, hd, hd], np.int64))
         parts = self.node(Op.Split, [qkv, sizes], lambda: [ref[qkv][..., i * hd:(i + 1) * hd] for i in range(3)], 3, axis=2)
-        heads = self.init(np.array([b, t, h, d], np.int64))
+        heads = self.init(np.array([0, 0, h, d] if self.open_batch else [b, t, h, d], np.int64))
 
         def head(p):
             r = self.node(Op.Reshape, [p, heads], lambda: ref[p].reshape(b, t, h, d))
@@ -151,6 +152,8 @@ class RandomGraph:
             s = self.node(Op.Mul, [s, sc], lambda s=s: ref[s] * sc_v)
         if self.flip(0.3):
             shape = [(b, 1, 1, t), (b, 1, 1, t), (1, 1, t, t), (b, 1, t, t), (t,)][int(rng.integers(0, 5))]
+            if self.open_batch and len(shape) == 4:
+                shape = (1, 1) + shape[2:]
             mask = np.where(rng.random(shape) < 0.2, -10000.0, 0.0).astype(np.float32)
             s = self.node(Op.Add, [s, self.init(mask)], lambda s=s: ref[s] + mask)
         if self.flip(0.1):
@@ -162,7 +165,7 @@ class RandomGraph:
         ot = self.node(Op.Transpose, [o], lambda: ref[o].transpose(0, 2, 1, 3), perm=[0, 2, 1, 3])
         if self.flip(0.1):
             extra.append(ot)
-        merged = self.init(np.array([b, t, hd], np.int64))
+        merged = self.init(np.array([0, 0, hd] if self.open_batch else [b, t, hd], np.int64))
         a = self.node(Op.Reshape, [ot, merged], lambda: ref[ot].reshape(b, t, hd))
         return self.linear(a, c, bias=self.flip(0.7)), extra
 
@@ -199,7 +202,8 @@ class RandomGraph:
                 cur = self.node(Op.Transpose, [tr], lambda: ref[tr].transpose(0, 2, 1), perm=[0, 2, 1])
             elif r < 0.98:
                 b, t, c = ref[z].shape
-                flat, back = self.init(np.array([b * t, c], np.int64)), self.init(np.array([b, t, c], np.int64))
+                flat = self.init(np.array([-1 if self.open_batch else b * t, c], np.int64))
+                back = self.init(np.array([-1 if self.open_batch else b, t, c], np.int64))
                 f = self.node(Op.Reshape, [cur, flat], lambda: ref[z].reshape(b * t, c))
                 y = self.linear(f, c, bias=self.flip(0.5), act=[None, "gelu"][int(rng.integers(0, 2))])
                 cur = self.node(Op.Reshape, [y, back], lambda: ref[y].reshape(b, t, c))
@@ -286,3 +290,45 @@ def test_random_encoder_graphs_in_every_session_configuration(case, seed):
                 else:
                     tol = 1e-3 * max(1.0, float(np.abs(plain[i]).max()))
                     np.testing.assert_allclose(got[i], plain[i], rtol=1e-3, atol=tol, err_msg=what)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_one_session_fed_batches_of_changing_size(case, seed):
+    """The input is declared without a shape (shapes are then inferred at every run, crates/core/src/analysis/
+    shape.rs:704-706) and no node spells the batch out (Reshape targets use 0 and -1): one session of every
+    configuration is fed six batches of four sizes in turn, and each result is held to a fresh plain session's on the
+    same feed -- what a run leaves behind (pooled blocks, recorded graphs, plans made for another size) must not show."""
+    rng = np.random.default_rng(9000 + seed)
+    g = RandomGraph(rng, open_batch=True)
+    outs = g.grow()
+    case(f"random graph {seed}, open batch: [{g.b},{g.t},{g.c}], {len(g.ops)} nodes, {len(outs)} outputs: {' '.join(g.ops)}")
+    if not g.ops:
+        pytest.skip("the draw added no node")
+    batches = [g.b, 1, g.b + 2, g.b, 2, g.b + 2]
+    feeds = {b: (rng.standard_normal((b, g.t, g.c)) * 0.5).astype(np.float32) for b in set(batches)}
+    plain = {b: run(g.m.clone(), feed) for b, feed in feeds.items()}
+    first = run(g.m.clone(), g.feed)
+    for i, o in enumerate(outs):
+        tol = 2e-3 * max(1.0, float(np.abs(g.ref[o]).max()))
+        np.testing.assert_allclose(first[i], g.ref[o], rtol=2e-3, atol=tol, err_msg=f"plain session, output {i}")
+    for rewrites, apply in REWRITES:
+        model = g.m.clone()
+        apply(model)
+        for name, options, same_kernels in SESSIONS:
+            builder = HipSessionBuilder(model.clone()).with_strided_views(options.get("views", False))
+            builder = builder.with_gemm_algorithm(options.get("algorithm", D.GEMM_FP32))
+            builder = builder.with_fused_attention(options.get("attention", False)).with_graph_replay(options.get("replay", False))
+            session = builder.build()
+            try:
+                for j, b in enumerate(batches):
+                    got = [np.array(t) for t in session.run([Tensor.from_numpy(feeds[b])])]
+                    for i in range(len(outs)):
+                        what = f"{rewrites}, {name}, run {j} (batch {b}), output {i}"
+                        want = plain[b][i]
+                        if same_kernels and rewrites == "as built":
+                            assert got[i].tobytes() == want.tobytes(), what
+                        else:
+                            tol = 1e-3 * max(1.0, float(np.abs(want).max()))
+                            np.testing.assert_allclose(got[i], want, rtol=1e-3, atol=tol, err_msg=what)
+            finally:
+                session.close()
