@@ -9,6 +9,7 @@
 #include "core/model.h"
 #include "core/optimize.h"
 #include "core/shape.h"
+#include "capi_guard.h"
 #include "device/ctx.h"
 #include "device/host_pool.h"
 #include "onnx/load.h"
@@ -77,7 +78,15 @@ int acquire_lane(ahip_session *session, size_t *index, std::shared_ptr<HipSessio
     hb.with_intra_op_num_threads(b.threads).with_profiling_enabled(b.profiling).with_device(b.device).with_graph_replay(b.graph_replay)
         .with_gemm_algorithm(b.gemm_algorithm).with_strided_views(b.strided_views).with_fused_attention(b.fused_attention);
     SessionError err;
-    std::shared_ptr<HipSession> lane = hb.build(&err);
+    std::shared_ptr<HipSession> lane;
+    try {
+        lane = hb.build(&err);
+    } catch (...) {
+        lock.lock();
+        session->building--;
+        session->lane_freed.notify_all();
+        throw;
+    }
     lock.lock();
     session->building--;
     if (!lane) {
@@ -157,11 +166,13 @@ void op_to_c(const Op &op, ahip_op_attrs *a) {
 
 bool valid_value(const ahip_model *m, int64_t id) { return id >= 0 && (size_t)id < m->m.graph.values.size(); }
 
-template <class F> int run_pass(ahip_model *model, int *count, F pass, const char *name) {
+template <class F> int run_pass(ahip_model *model, int *count, F pass, const char *name) try {
     if (!model) return fail(AHIP_ERR_ARG, std::string(name) + ": null model");
     const size_t n = pass(model->m);
     if (count) *count = (int)n;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary(name);
 }
 
 }  // namespace
@@ -182,31 +193,37 @@ void ahip_op_attrs_default(ahip_op_attrs *a) {
 
 const char *ahip_op_name(int op_kind) { return op_kind_name(static_cast<OpKind>(op_kind)); }
 
-int ahip_model_new(int64_t opset_version, ahip_model **model) {
+int ahip_model_new(int64_t opset_version, ahip_model **model) try {
     if (!model) return fail(AHIP_ERR_ARG, "ahip_model_new: null output pointer");
     *model = new (std::nothrow) ahip_model();
     if (!*model) return fail(AHIP_ERR_OOM, "ahip_model_new: out of host memory");
     (*model)->m.opset_version = opset_version;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_new");
 }
 
-int ahip_model_clone(const ahip_model *model, ahip_model **copy) {
+int ahip_model_clone(const ahip_model *model, ahip_model **copy) try {
     if (!model || !copy) return fail(AHIP_ERR_ARG, "ahip_model_clone: null argument");
     *copy = new (std::nothrow) ahip_model(*model);
     if (!*copy) return fail(AHIP_ERR_OOM, "ahip_model_clone: out of host memory");
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_clone");
 }
 
 void ahip_model_free(ahip_model *model) { delete model; }
 
-int ahip_model_new_value(ahip_model *model, const char *name, int64_t *value_id) {
+int ahip_model_new_value(ahip_model *model, const char *name, int64_t *value_id) try {
     if (!model || !value_id) return fail(AHIP_ERR_ARG, "ahip_model_new_value: null argument");
     *value_id = (int64_t)(name ? model->m.graph.values.new_val_named(name) : model->m.graph.values.new_val());
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_new_value");
 }
 
 int ahip_model_new_value_shaped(ahip_model *model, const char *name, int elem_type, int rank, const int64_t *dims,
-                                int64_t *value_id) {
+                                int64_t *value_id) try {
     if (!model || !value_id || rank < 0 || (rank && !dims) || !valid_elem_type(elem_type))
         return fail(AHIP_ERR_ARG, "ahip_model_new_value_shaped: invalid argument");
     std::vector<Dimension> d;
@@ -215,10 +232,12 @@ int ahip_model_new_value_shaped(ahip_model *model, const char *name, int elem_ty
     TypedShape ts{Dimensions(std::move(d)), static_cast<TensorElemType>(elem_type)};
     *value_id = (int64_t)model->m.graph.values.new_val_named_and_shaped(name ? name : "", std::move(ts));
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_new_value_shaped");
 }
 
 int ahip_model_add_initializer(ahip_model *model, int64_t value_id, int elem_type, int rank, const int64_t *dims,
-                               const void *data, size_t nbytes) {
+                               const void *data, size_t nbytes) try {
     if (!model || rank < 0 || (rank && !dims) || !valid_elem_type(elem_type) || !valid_value(model, value_id))
         return fail(AHIP_ERR_ARG, "ahip_model_add_initializer: invalid argument");
     for (int i = 0; i < rank; i++)
@@ -229,10 +248,12 @@ int ahip_model_add_initializer(ahip_model *model, int64_t value_id, int elem_typ
         return fail(AHIP_ERR_ARG, "ahip_model_add_initializer: data size does not match the shape");
     model->m.graph.inits[(ValueId)value_id] = Tensor::from_raw(std::move(fd), ty, data, nbytes);
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_add_initializer");
 }
 
 int ahip_model_add_node(ahip_model *model, int op_kind, const ahip_op_attrs *attrs, const char *name, int n_inputs,
-                        const int64_t *inputs, int n_outputs, const int64_t *outputs, int64_t *node_id) {
+                        const int64_t *inputs, int n_outputs, const int64_t *outputs, int64_t *node_id) try {
     if (!model || op_kind < 0 || op_kind >= AHIP_OP_COUNT || n_inputs < 0 || n_outputs < 0 ||
         (n_inputs && !inputs) || (n_outputs && !outputs))
         return fail(AHIP_ERR_ARG, "ahip_model_add_node: invalid argument");
@@ -249,48 +270,60 @@ int ahip_model_add_node(ahip_model *model, int op_kind, const ahip_op_attrs *att
     const NodeId id = model->m.graph.add_node(std::move(node));
     if (node_id) *node_id = (int64_t)id;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_add_node");
 }
 
-int ahip_model_add_input(ahip_model *model, int64_t value_id) {
+int ahip_model_add_input(ahip_model *model, int64_t value_id) try {
     if (!model || !valid_value(model, value_id)) return fail(AHIP_ERR_ARG, "ahip_model_add_input: invalid argument");
     model->m.graph.inputs.push_back((ValueId)value_id);
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_add_input");
 }
 
-int ahip_model_add_output(ahip_model *model, int64_t value_id) {
+int ahip_model_add_output(ahip_model *model, int64_t value_id) try {
     if (!model || !valid_value(model, value_id)) return fail(AHIP_ERR_ARG, "ahip_model_add_output: invalid argument");
     model->m.graph.outputs.push_back((ValueId)value_id);
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_add_output");
 }
 
-int ahip_model_lookup_named_value(const ahip_model *model, const char *name, int64_t *value_id) {
+int ahip_model_lookup_named_value(const ahip_model *model, const char *name, int64_t *value_id) try {
     if (!model || !name || !value_id) return fail(AHIP_ERR_ARG, "ahip_model_lookup_named_value: null argument");
     auto id = model->m.lookup_named_value(name);
     if (!id) return fail(AHIP_ERR_ARG, std::string("no value named '") + name + "'");
     *value_id = (int64_t)*id;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_lookup_named_value");
 }
 
-int ahip_model_graph_io(const ahip_model *model, int which, int64_t *value_ids, int capacity, int *n) {
+int ahip_model_graph_io(const ahip_model *model, int which, int64_t *value_ids, int capacity, int *n) try {
     if (!model || !n || (which != 0 && which != 1) || capacity < 0 || (capacity && !value_ids))
         return fail(AHIP_ERR_ARG, "ahip_model_graph_io: invalid argument");
     const auto &v = which == 0 ? model->m.graph.inputs : model->m.graph.outputs;
     *n = (int)v.size();
     for (int i = 0; i < capacity && i < (int)v.size(); i++) value_ids[i] = (int64_t)v[i];
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_graph_io");
 }
 
-int ahip_model_topo_sort(const ahip_model *model, int64_t *node_ids, int capacity, int *n) {
+int ahip_model_topo_sort(const ahip_model *model, int64_t *node_ids, int capacity, int *n) try {
     if (!model || !n || capacity < 0 || (capacity && !node_ids))
         return fail(AHIP_ERR_ARG, "ahip_model_topo_sort: invalid argument");
     const auto order = model->m.topo_sort_nodes();
     *n = (int)order.size();
     for (int i = 0; i < capacity && i < (int)order.size(); i++) node_ids[i] = (int64_t)order[i];
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_topo_sort");
 }
 
 int ahip_model_node_info(const ahip_model *model, int64_t node_id, int *op_kind, ahip_op_attrs *attrs, int *n_inputs,
-                         int64_t *inputs, int *n_outputs, int64_t *outputs, int io_capacity) {
+                         int64_t *inputs, int *n_outputs, int64_t *outputs, int io_capacity) try {
     if (!model || node_id < 0 || (size_t)node_id >= model->m.graph.nodes.size() || io_capacity < 0)
         return fail(AHIP_ERR_ARG, "ahip_model_node_info: invalid argument");
     const Node &node = model->m.graph.nodes[(size_t)node_id];
@@ -303,10 +336,12 @@ int ahip_model_node_info(const ahip_model *model, int64_t node_id, int *op_kind,
     if (outputs)
         for (int i = 0; i < io_capacity && i < (int)node.outputs.size(); i++) outputs[i] = (int64_t)node.outputs[i];
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_node_info");
 }
 
 int ahip_model_infer_value_shape(const ahip_model *model, int64_t value_id, int *elem_type, int *rank,
-                                 int64_t *dims) {
+                                 int64_t *dims) try {
     if (!model || !rank || !dims || !valid_value(model, value_id))
         return fail(AHIP_ERR_ARG, "ahip_model_infer_value_shape: invalid argument");
     std::map<ValueId, TypedFixedShape> shapes;
@@ -319,10 +354,12 @@ int ahip_model_infer_value_shape(const ahip_model *model, int64_t value_id, int 
     *rank = (int)it->second.dims.len();
     for (size_t i = 0; i < it->second.dims.len(); i++) dims[i] = (int64_t)it->second.dims[i];
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_infer_value_shape");
 }
 
 int ahip_model_execution_plan(const ahip_model *model, int64_t *node_ids, int *free_offsets, int node_capacity,
-                              int64_t *free_vals, int free_capacity, int *n_nodes, int *n_free) {
+                              int64_t *free_vals, int free_capacity, int *n_nodes, int *n_free) try {
     if (!model || !n_nodes || !n_free || node_capacity < 0 || free_capacity < 0)
         return fail(AHIP_ERR_ARG, "ahip_model_execution_plan: invalid argument");
     const auto plan = create_execution_plan(model->m);
@@ -341,6 +378,8 @@ int ahip_model_execution_plan(const ahip_model *model, int64_t *node_ids, int *f
     *n_nodes = (int)plan.size();
     *n_free = nf;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_execution_plan");
 }
 
 // ---- ONNX loader, value / node inspection, attributes by name ------------------------------
@@ -367,7 +406,7 @@ int no_attr(const char *fn, const Node &n, const char *name) {
 
 }  // namespace
 
-int ahip_model_load_onnx(const char *path, ahip_model **model) {
+int ahip_model_load_onnx(const char *path, ahip_model **model) try {
     if (!path || !model) return fail(AHIP_ERR_ARG, "ahip_model_load_onnx: null argument");
     *model = nullptr;
     ahip_model *m = new (std::nothrow) ahip_model();
@@ -379,9 +418,11 @@ int ahip_model_load_onnx(const char *path, ahip_model **model) {
     }
     *model = m;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_load_onnx");
 }
 
-int ahip_model_load_onnx_buffer(const void *data, size_t bytes, ahip_model **model) {
+int ahip_model_load_onnx_buffer(const void *data, size_t bytes, ahip_model **model) try {
     if (!model || (!data && bytes)) return fail(AHIP_ERR_ARG, "ahip_model_load_onnx_buffer: null argument");
     *model = nullptr;
     ahip_model *m = new (std::nothrow) ahip_model();
@@ -393,6 +434,8 @@ int ahip_model_load_onnx_buffer(const void *data, size_t bytes, ahip_model **mod
     }
     *model = m;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_load_onnx_buffer");
 }
 
 int64_t ahip_model_opset_version(const ahip_model *model) { return model ? model->m.opset_version : -1; }
@@ -400,7 +443,7 @@ int64_t ahip_model_num_values(const ahip_model *model) { return model ? (int64_t
 int64_t ahip_model_num_nodes(const ahip_model *model) { return model ? (int64_t)model->m.graph.nodes.size() : -1; }
 
 int ahip_model_value_info(const ahip_model *model, int64_t value_id, const char **name, int *elem_type, int *rank,
-                          int64_t *dims, int dims_capacity) {
+                          int64_t *dims, int dims_capacity) try {
     if (!model || !valid_value(model, value_id) || dims_capacity < 0 || (dims_capacity && !dims))
         return fail(AHIP_ERR_ARG, "ahip_model_value_info: invalid argument");
     const Value &v = model->m.graph.values[(ValueId)value_id];
@@ -414,9 +457,11 @@ int ahip_model_value_info(const ahip_model *model, int64_t value_id, const char 
     if (rank) *rank = (int)dv.size();
     for (int i = 0; i < dims_capacity && i < (int)dv.size(); i++) dims[i] = dv[(size_t)i].fixed ? (int64_t)dv[(size_t)i].value : -1;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_value_info");
 }
 
-int ahip_model_initializer(const ahip_model *model, int64_t value_id, ahip_tensor **tensor) {
+int ahip_model_initializer(const ahip_model *model, int64_t value_id, ahip_tensor **tensor) try {
     if (!model || !tensor || !valid_value(model, value_id)) return fail(AHIP_ERR_ARG, "ahip_model_initializer: invalid argument");
     auto it = model->m.graph.inits.find((ValueId)value_id);
     if (it == model->m.graph.inits.end()) return fail(AHIP_ERR_ARG, "ahip_model_initializer: the value has no initializer");
@@ -425,6 +470,8 @@ int ahip_model_initializer(const ahip_model *model, int64_t value_id, ahip_tenso
     t->t = it->second;  // shares the bytes
     *tensor = t;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_model_initializer");
 }
 
 const char *ahip_model_node_name(const ahip_model *model, int64_t node_id) {
@@ -432,46 +479,60 @@ const char *ahip_model_node_name(const ahip_model *model, int64_t node_id) {
     return n && n->name ? n->name->c_str() : nullptr;
 }
 
-int ahip_node_set_attr_int(ahip_model *model, int64_t node_id, const char *name, int64_t value) {
+int ahip_node_set_attr_int(ahip_model *model, int64_t node_id, const char *name, int64_t value) try {
     Node *n = live_node(model, node_id);
     if (!n || !name) return fail(AHIP_ERR_ARG, "ahip_node_set_attr_int: invalid argument");
     return n->op.set_int(name, value) ? AHIP_OK : no_attr("ahip_node_set_attr_int", *n, name);
+} catch (...) {
+    return altius::caught_at_boundary("ahip_node_set_attr_int");
 }
-int ahip_node_set_attr_float(ahip_model *model, int64_t node_id, const char *name, float value) {
+int ahip_node_set_attr_float(ahip_model *model, int64_t node_id, const char *name, float value) try {
     Node *n = live_node(model, node_id);
     if (!n || !name) return fail(AHIP_ERR_ARG, "ahip_node_set_attr_float: invalid argument");
     return n->op.set_float(name, value) ? AHIP_OK : no_attr("ahip_node_set_attr_float", *n, name);
+} catch (...) {
+    return altius::caught_at_boundary("ahip_node_set_attr_float");
 }
-int ahip_node_set_attr_ints(ahip_model *model, int64_t node_id, const char *name, const int64_t *values, int count) {
+int ahip_node_set_attr_ints(ahip_model *model, int64_t node_id, const char *name, const int64_t *values, int count) try {
     Node *n = live_node(model, node_id);
     if (!n || !name || count < 0 || (count && !values)) return fail(AHIP_ERR_ARG, "ahip_node_set_attr_ints: invalid argument");
     return n->op.set_ints(name, std::vector<int64_t>(values, values + count)) ? AHIP_OK
                                                                                : no_attr("ahip_node_set_attr_ints", *n, name);
+} catch (...) {
+    return altius::caught_at_boundary("ahip_node_set_attr_ints");
 }
-int ahip_node_set_attr_string(ahip_model *model, int64_t node_id, const char *name, const char *value) {
+int ahip_node_set_attr_string(ahip_model *model, int64_t node_id, const char *name, const char *value) try {
     Node *n = live_node(model, node_id);
     if (!n || !name || !value) return fail(AHIP_ERR_ARG, "ahip_node_set_attr_string: invalid argument");
     return n->op.set_string(name, value) ? AHIP_OK : no_attr("ahip_node_set_attr_string", *n, name);
+} catch (...) {
+    return altius::caught_at_boundary("ahip_node_set_attr_string");
 }
-int ahip_node_set_attr_tensor(ahip_model *model, int64_t node_id, const char *name, const ahip_tensor *value) {
+int ahip_node_set_attr_tensor(ahip_model *model, int64_t node_id, const char *name, const ahip_tensor *value) try {
     Node *n = live_node(model, node_id);
     if (!n || !name || !value) return fail(AHIP_ERR_ARG, "ahip_node_set_attr_tensor: invalid argument");
     if (n->op.kind != OpKind::Constant || std::string(name) != "value") return no_attr("ahip_node_set_attr_tensor", *n, name);
     n->op.value = std::make_shared<Tensor>(value->t);
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_node_set_attr_tensor");
 }
-int ahip_node_get_attr_int(const ahip_model *model, int64_t node_id, const char *name, int64_t *value) {
+int ahip_node_get_attr_int(const ahip_model *model, int64_t node_id, const char *name, int64_t *value) try {
     const Node *n = live_node_c(model, node_id);
     if (!n || !name || !value) return fail(AHIP_ERR_ARG, "ahip_node_get_attr_int: invalid argument");
     return n->op.get_int(name, value) ? AHIP_OK : no_attr("ahip_node_get_attr_int", *n, name);
+} catch (...) {
+    return altius::caught_at_boundary("ahip_node_get_attr_int");
 }
-int ahip_node_get_attr_float(const ahip_model *model, int64_t node_id, const char *name, float *value) {
+int ahip_node_get_attr_float(const ahip_model *model, int64_t node_id, const char *name, float *value) try {
     const Node *n = live_node_c(model, node_id);
     if (!n || !name || !value) return fail(AHIP_ERR_ARG, "ahip_node_get_attr_float: invalid argument");
     return n->op.get_float(name, value) ? AHIP_OK : no_attr("ahip_node_get_attr_float", *n, name);
+} catch (...) {
+    return altius::caught_at_boundary("ahip_node_get_attr_float");
 }
 int ahip_node_get_attr_ints(const ahip_model *model, int64_t node_id, const char *name, int64_t *values, int capacity,
-                            int *count) {
+                            int *count) try {
     const Node *n = live_node_c(model, node_id);
     if (!n || !name || capacity < 0 || (capacity && !values)) return fail(AHIP_ERR_ARG, "ahip_node_get_attr_ints: invalid argument");
     std::vector<int64_t> v;
@@ -479,9 +540,11 @@ int ahip_node_get_attr_ints(const ahip_model *model, int64_t node_id, const char
     for (int i = 0; i < capacity && i < (int)v.size(); i++) values[i] = v[(size_t)i];
     if (count) *count = (int)v.size();
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_node_get_attr_ints");
 }
 int ahip_node_get_attr_string(const ahip_model *model, int64_t node_id, const char *name, char *value, int capacity,
-                              int *length) {
+                              int *length) try {
     const Node *n = live_node_c(model, node_id);
     if (!n || !name || capacity < 0 || (capacity && !value)) return fail(AHIP_ERR_ARG, "ahip_node_get_attr_string: invalid argument");
     std::string v;
@@ -493,8 +556,10 @@ int ahip_node_get_attr_string(const ahip_model *model, int64_t node_id, const ch
     }
     if (length) *length = (int)v.size();
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_node_get_attr_string");
 }
-int ahip_node_get_attr_tensor(const ahip_model *model, int64_t node_id, const char *name, ahip_tensor **value) {
+int ahip_node_get_attr_tensor(const ahip_model *model, int64_t node_id, const char *name, ahip_tensor **value) try {
     const Node *n = live_node_c(model, node_id);
     if (!n || !name || !value) return fail(AHIP_ERR_ARG, "ahip_node_get_attr_tensor: invalid argument");
     if (n->op.kind != OpKind::Constant || std::string(name) != "value" || !n->op.value)
@@ -504,6 +569,8 @@ int ahip_node_get_attr_tensor(const ahip_model *model, int64_t node_id, const ch
     t->t = *n->op.value;
     *value = t;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_node_get_attr_tensor");
 }
 
 int ahip_fuse_layer_norm(ahip_model *model, int *count) { return run_pass(model, count, fuse_layer_norm, "ahip_fuse_layer_norm"); }
@@ -513,7 +580,7 @@ int ahip_eliminate_identity(ahip_model *model, int *count) { return run_pass(mod
 int ahip_fuse_transpose_matmul(ahip_model *model, int *count) { return run_pass(model, count, fuse_transpose_matmul, "ahip_fuse_transpose_matmul"); }
 int ahip_fuse_matmul_bias(ahip_model *model, int *count) { return run_pass(model, count, fuse_matmul_bias, "ahip_fuse_matmul_bias"); }
 int ahip_fuse_softmax_prologue(ahip_model *model, int *count) { return run_pass(model, count, fuse_softmax_prologue, "ahip_fuse_softmax_prologue"); }
-int ahip_fuse_elemwise_ops(ahip_model *model, int rule, int *count) {
+int ahip_fuse_elemwise_ops(ahip_model *model, int rule, int *count) try {
     if (!model) return fail(AHIP_ERR_ARG, "ahip_fuse_elemwise_ops: null model");
     if (rule != AHIP_FUSE_REFERENCE_RULE && rule != AHIP_FUSE_EXTENDED_RULE) return fail(AHIP_ERR_ARG, "ahip_fuse_elemwise_ops: unknown rule");
     size_t n = 0;
@@ -521,12 +588,14 @@ int ahip_fuse_elemwise_ops(ahip_model *model, int rule, int *count) {
     if (!fuse_elemwise_ops(model->m, static_cast<ElemwiseFusionRule>(rule), &n, &msg)) return fail(AHIP_ERR_SHAPE, msg);
     if (count) *count = (int)n;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_fuse_elemwise_ops");
 }
 
 // ---- tensors -----------------------------------------------------------------------
 
 int ahip_tensor_new(int elem_type, int rank, const int64_t *dims, const void *data, size_t nbytes,
-                    ahip_tensor **tensor) {
+                    ahip_tensor **tensor) try {
     if (!tensor || rank < 0 || (rank && !dims) || !valid_elem_type(elem_type))
         return fail(AHIP_ERR_ARG, "ahip_tensor_new: invalid argument");
     for (int i = 0; i < rank; i++)
@@ -546,17 +615,21 @@ int ahip_tensor_new(int elem_type, int rank, const int64_t *dims, const void *da
     }
     *tensor = t;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_tensor_new");
 }
 
 void *ahip_tensor_data_mut(ahip_tensor *tensor) { return tensor ? tensor->t.data_as_bytes_mut() : nullptr; }
 
-int ahip_host_pool_stats(size_t *live_bytes, size_t *cached_bytes, size_t *pinned_allocations, size_t *reuses) {
+int ahip_host_pool_stats(size_t *live_bytes, size_t *cached_bytes, size_t *pinned_allocations, size_t *reuses) try {
     const altius::HostPoolStats st = altius::host_pool_stats();
     if (live_bytes) *live_bytes = st.live_bytes;
     if (cached_bytes) *cached_bytes = st.cached_bytes;
     if (pinned_allocations) *pinned_allocations = st.pinned_allocations;
     if (reuses) *reuses = st.reuses;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_host_pool_stats");
 }
 
 size_t ahip_host_pool_trim(void) { return altius::host_pool_trim(); }
@@ -564,85 +637,107 @@ size_t ahip_host_pool_trim(void) { return altius::host_pool_trim(); }
 void ahip_tensor_free(ahip_tensor *tensor) { delete tensor; }
 int ahip_tensor_elem_type(const ahip_tensor *tensor) { return tensor ? (int)tensor->t.elem_ty() : -1; }
 int ahip_tensor_rank(const ahip_tensor *tensor) { return tensor ? (int)tensor->t.dims().len() : -1; }
-int ahip_tensor_dims(const ahip_tensor *tensor, int64_t *dims, int capacity) {
+int ahip_tensor_dims(const ahip_tensor *tensor, int64_t *dims, int capacity) try {
     if (!tensor || capacity < 0 || (capacity && !dims)) return fail(AHIP_ERR_ARG, "ahip_tensor_dims: invalid argument");
     const auto &d = tensor->t.dims();
     for (int i = 0; i < capacity && i < (int)d.len(); i++) dims[i] = (int64_t)d[i];
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_tensor_dims");
 }
 size_t ahip_tensor_nbytes(const ahip_tensor *tensor) { return tensor ? tensor->t.nbytes() : 0; }
 const void *ahip_tensor_data(const ahip_tensor *tensor) { return tensor ? tensor->t.data_as_bytes() : nullptr; }
 
 // ---- session ---------------------------------------------------------------------------
 
-int ahip_session_builder_new(const ahip_model *model, ahip_session_builder **builder) {
+int ahip_session_builder_new(const ahip_model *model, ahip_session_builder **builder) try {
     if (!model || !builder) return fail(AHIP_ERR_ARG, "ahip_session_builder_new: null argument");
     ahip_session_builder *b = new (std::nothrow) ahip_session_builder();
     if (!b) return fail(AHIP_ERR_OOM, "ahip_session_builder_new: out of host memory");
     b->model = model->m;
     *builder = b;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_builder_new");
 }
 
 void ahip_session_builder_free(ahip_session_builder *builder) { delete builder; }
 
-int ahip_session_builder_with_intra_op_num_threads(ahip_session_builder *builder, size_t n) {
+int ahip_session_builder_with_intra_op_num_threads(ahip_session_builder *builder, size_t n) try {
     if (!builder) return fail(AHIP_ERR_ARG, "null builder");
     builder->threads = n;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_builder_with_intra_op_num_threads");
 }
 
-int ahip_session_builder_with_profiling_enabled(ahip_session_builder *builder, int enable) {
+int ahip_session_builder_with_profiling_enabled(ahip_session_builder *builder, int enable) try {
     if (!builder) return fail(AHIP_ERR_ARG, "null builder");
     builder->profiling = enable != 0;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_builder_with_profiling_enabled");
 }
 
-int ahip_session_builder_with_device(ahip_session_builder *builder, int device) {
+int ahip_session_builder_with_device(ahip_session_builder *builder, int device) try {
     if (!builder) return fail(AHIP_ERR_ARG, "null builder");
     builder->device = device;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_builder_with_device");
 }
 
-int ahip_session_builder_with_graph_replay(ahip_session_builder *builder, int enable) {
+int ahip_session_builder_with_graph_replay(ahip_session_builder *builder, int enable) try {
     if (!builder) return fail(AHIP_ERR_ARG, "null builder");
     builder->graph_replay = enable != 0;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_builder_with_graph_replay");
 }
 
-int ahip_session_builder_with_gemm_algorithm(ahip_session_builder *builder, int algorithm) {
+int ahip_session_builder_with_gemm_algorithm(ahip_session_builder *builder, int algorithm) try {
     if (!builder) return fail(AHIP_ERR_ARG, "null builder");
     if (algorithm != AHIP_GEMM_AUTO && algorithm != AHIP_GEMM_FP32 && algorithm != AHIP_GEMM_BF16X3)
         return fail(AHIP_ERR_ARG, "ahip_session_builder_with_gemm_algorithm: unknown algorithm");
     builder->gemm_algorithm = algorithm;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_builder_with_gemm_algorithm");
 }
 
-int ahip_session_builder_with_strided_views(ahip_session_builder *builder, int enable) {
+int ahip_session_builder_with_strided_views(ahip_session_builder *builder, int enable) try {
     if (!builder) return fail(AHIP_ERR_ARG, "null builder");
     builder->strided_views = enable != 0;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_builder_with_strided_views");
 }
 
-int ahip_session_builder_with_fused_attention(ahip_session_builder *builder, int enable) {
+int ahip_session_builder_with_fused_attention(ahip_session_builder *builder, int enable) try {
     if (!builder) return fail(AHIP_ERR_ARG, "null builder");
     builder->fused_attention = enable != 0;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_builder_with_fused_attention");
 }
 
-int ahip_session_copies_avoided(const ahip_session *session, size_t *count) {
+int ahip_session_copies_avoided(const ahip_session *session, size_t *count) try {
     if (!session || !count) return fail(AHIP_ERR_ARG, "ahip_session_copies_avoided: null argument");
     *count = session->s->copies_avoided();
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_copies_avoided");
 }
 
-int ahip_session_graph_replays(const ahip_session *session, size_t *count) {
+int ahip_session_graph_replays(const ahip_session *session, size_t *count) try {
     if (!session || !count) return fail(AHIP_ERR_ARG, "ahip_session_graph_replays: null argument");
     *count = session->s->graph_replays();
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_graph_replays");
 }
 
-int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **session) {
+int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **session) try {
     if (!builder || !session) return fail(AHIP_ERR_ARG, "ahip_session_builder_build: null argument");
     *session = nullptr;
     HipSessionBuilder b(builder->model);
@@ -665,19 +760,23 @@ int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **ses
     out->busy.push_back(false);
     *session = out;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_builder_build");
 }
 
-int ahip_session_lanes(ahip_session *session, size_t *count) {
+int ahip_session_lanes(ahip_session *session, size_t *count) try {
     if (!session || !count) return fail(AHIP_ERR_ARG, "ahip_session_lanes: null argument");
     std::lock_guard<std::mutex> lock(session->lanes_mutex);
     *count = session->lanes.size();
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_lanes");
 }
 
 void ahip_session_free(ahip_session *session) { delete session; }
 
 int ahip_session_run(ahip_session *session, int n_inputs, const ahip_tensor *const *inputs, int output_capacity,
-                     ahip_tensor **outputs, int *n_outputs) {
+                     ahip_tensor **outputs, int *n_outputs) try {
     if (!session || n_inputs < 0 || (n_inputs && !inputs) || output_capacity < 0 || (output_capacity && !outputs) ||
         !n_outputs)
         return fail(AHIP_ERR_ARG, "ahip_session_run: invalid argument");
@@ -691,7 +790,13 @@ int ahip_session_run(ahip_session *session, int n_inputs, const ahip_tensor *con
     size_t lane_index = 0;
     std::shared_ptr<HipSession> lane;
     if (const int rc = acquire_lane(session, &lane_index, &lane)) return rc;
-    const bool ok = lane->run(in, &out, &err);
+    bool ok = false;
+    try {
+        ok = lane->run(in, &out, &err);
+    } catch (...) {
+        release_lane(session, lane_index, false);
+        throw;
+    }
     release_lane(session, lane_index, ok);
     if (!ok) return fail(err.code(), err.to_string());
     *n_outputs = (int)out.size();
@@ -706,11 +811,13 @@ int ahip_session_run(ahip_session *session, int n_inputs, const ahip_tensor *con
         outputs[i] = t;
     }
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_run");
 }
 
 int ahip_session_run_device(ahip_session *session, int n_inputs, const void *const *device_ptrs, const int *elem_types,
                             const int *ranks, const int64_t *const *dims, int output_capacity,
-                            ahip_device_tensor **outputs, int *n_outputs) {
+                            ahip_device_tensor **outputs, int *n_outputs) try {
     if (!session || n_inputs < 0 || (n_inputs && (!device_ptrs || !elem_types || !ranks || !dims)) || output_capacity < 0 ||
         (output_capacity && !outputs) || !n_outputs)
         return fail(AHIP_ERR_ARG, "ahip_session_run_device: invalid argument");
@@ -728,7 +835,13 @@ int ahip_session_run_device(ahip_session *session, int n_inputs, const void *con
     std::vector<DeviceTensor> out;
     SessionError err;
     acquire_first_lane(session);
-    const bool ok = session->s->run_device(in, &out, &err);
+    bool ok = false;
+    try {
+        ok = session->s->run_device(in, &out, &err);
+    } catch (...) {
+        release_lane(session, 0, false);
+        throw;
+    }
     release_lane(session, 0, false);
     if (!ok) return fail(err.code(), err.to_string());
     *n_outputs = (int)out.size();
@@ -751,13 +864,17 @@ int ahip_session_run_device(ahip_session *session, int n_inputs, const void *con
         outputs[i] = t;
     }
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_run_device");
 }
 
-int ahip_session_synchronize(ahip_session *session) {
+int ahip_session_synchronize(ahip_session *session) try {
     if (!session) return fail(AHIP_ERR_ARG, "ahip_session_synchronize: null session");
     SessionError err;
     if (!session->s->synchronize(&err)) return fail(err.code(), err.to_string());
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_synchronize");
 }
 
 void ahip_device_tensor_free(ahip_device_tensor *tensor) { delete tensor; }
@@ -765,15 +882,17 @@ void *ahip_device_tensor_ptr(const ahip_device_tensor *tensor) { return tensor ?
 int ahip_device_tensor_elem_type(const ahip_device_tensor *tensor) { return tensor ? (int)tensor->t.elem_ty : -1; }
 int ahip_device_tensor_rank(const ahip_device_tensor *tensor) { return tensor ? (int)tensor->t.dims.len() : -1; }
 size_t ahip_device_tensor_nbytes(const ahip_device_tensor *tensor) { return tensor ? tensor->t.nbytes() : 0; }
-int ahip_device_tensor_dims(const ahip_device_tensor *tensor, int64_t *dims, int capacity) {
+int ahip_device_tensor_dims(const ahip_device_tensor *tensor, int64_t *dims, int capacity) try {
     if (!tensor || capacity < 0 || (capacity && !dims)) return fail(AHIP_ERR_ARG, "ahip_device_tensor_dims: invalid argument");
     for (int i = 0; i < capacity && i < (int)tensor->t.dims.len(); i++) dims[i] = (int64_t)tensor->t.dims[i];
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_device_tensor_dims");
 }
 
 const ahip_model *ahip_session_model(const ahip_session *session) { return session ? &session->view : nullptr; }
 
-int ahip_session_profile(const ahip_session *session, int index, const char **op_name, double *ms, int *count) {
+int ahip_session_profile(const ahip_session *session, int index, const char **op_name, double *ms, int *count) try {
     if (!session) return fail(AHIP_ERR_ARG, "ahip_session_profile: null session");
     if (count) *count = (int)session->profile.size();
     if (index < 0 || index >= (int)session->profile.size()) {
@@ -783,24 +902,32 @@ int ahip_session_profile(const ahip_session *session, int index, const char **op
     if (op_name) *op_name = session->profile[index].first.c_str();
     if (ms) *ms = session->profile[index].second;
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_profile");
 }
 
-int ahip_session_last_device_ms(const ahip_session *session, double *ms) {
+int ahip_session_last_device_ms(const ahip_session *session, double *ms) try {
     if (!session || !ms) return fail(AHIP_ERR_ARG, "ahip_session_last_device_ms: null argument");
     *ms = session->s->last_device_ms();
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_last_device_ms");
 }
 
-int ahip_session_last_run_ms(const ahip_session *session, double *ms) {
+int ahip_session_last_run_ms(const ahip_session *session, double *ms) try {
     if (!session || !ms) return fail(AHIP_ERR_ARG, "ahip_session_last_run_ms: null argument");
     *ms = session->s->last_run_ms();
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_last_run_ms");
 }
 
-int ahip_session_device_allocations(const ahip_session *session, size_t *count) {
+int ahip_session_device_allocations(const ahip_session *session, size_t *count) try {
     if (!session || !count) return fail(AHIP_ERR_ARG, "ahip_session_device_allocations: null argument");
     *count = session->s->device_allocations();
     return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_device_allocations");
 }
 
 }  // extern "C"

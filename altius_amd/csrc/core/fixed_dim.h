@@ -31,9 +31,17 @@ public:
     bool is_empty() const { return d_.empty(); }
     // Rank 0, or rank 1 with extent 0 or 1 (fixed_dim.rs:26-28).
     bool is_scalar() const { return d_.empty() || (d_.size() == 1 && (d_[0] == 0 || d_[0] == 1)); }
+    // The product of the extents.  A product that does not fit comes back as SATURATED instead of wrapped: no tensor
+    // is that large, so every allocation sized from it fails cleanly (times an element size it still does not wrap).
+    static constexpr size_t SATURATED = ~size_t(0) / 16;
     size_t total_elems() const {
         size_t n = 1;
-        for (auto x : d_) n *= x;
+        for (auto x : d_)
+            if (x == 0) return 0;
+        for (auto x : d_) {
+            if (n > SATURATED / x) return SATURATED;
+            n *= x;
+        }
         return n;
     }
     const std::vector<FixedDimension> &as_vec() const { return d_; }

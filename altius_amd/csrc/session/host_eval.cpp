@@ -111,6 +111,10 @@ bool evaluate_on_host(const Model &model, const Op &op, const std::vector<const 
     outputs->clear();
     if (shapes.empty()) return fail(error, std::string(op.name()) + ": no output shape");
     const TypedFixedShape &os = shapes[0];
+    // What runs here is the integer arithmetic on shapes and indices that exporters leave in a graph: small tensors.
+    // A result of 2^26 elements and more (a Range whose limit is a mistake) is refused instead of filling host memory.
+    if (os.dims.total_elems() >= ((size_t)1 << 26))
+        return fail(error, std::string(op.name()) + ": a result of " + std::to_string(os.dims.total_elems()) + " elements is too large to evaluate on the host");
     auto input = [&](size_t i) -> const Tensor * { return i < in.size() ? in[i] : nullptr; };
     auto ints = [&](size_t i, std::vector<int64_t> *v) {
         const Tensor *t = input(i);

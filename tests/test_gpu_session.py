@@ -7,7 +7,7 @@ import pytest
 
 import oracle as O
 from altius_amd import synth
-from altius_amd._lib import ERR_ARG, ERR_SHAPE, ERR_UNSUPPORTED, AltiusHipError
+from altius_amd._lib import ERR_ARG, ERR_OOM, ERR_SHAPE, ERR_UNSUPPORTED, AltiusHipError
 from altius_amd.graph import F32, I64, Model, Op, Tensor, host_pool_stats, host_pool_trim
 from altius_amd.graphs import erf_gelu_chain, layer_norm_chain
 from altius_amd.session import HipSessionBuilder
@@ -305,6 +305,70 @@ def test_errors_come_back_as_values(case):
 
     with pytest.raises(AltiusHipError):        # no such GPU
         HipSessionBuilder(binary_model(Op.Add)).with_device(99).build()
+
+
+def test_graphs_that_make_no_sense_come_back_as_errors(case):
+    """Tensors no device holds, values nobody produces, cycles: the reference unwraps and panics; here each is an
+    error code, the process lives and the next session works."""
+    case("session: nonsense graphs")
+    one = np.ones(4, np.float32)
+
+    def outcome(m, feeds):
+        sess = HipSessionBuilder(m).build()
+        try:
+            sess.run(feeds)
+        except AltiusHipError as e:
+            return e.code
+        finally:
+            sess.close()
+        return 0
+
+    def start():
+        m = Model()
+        x = m.new_val_named_and_shaped("x", [4])
+        m.add_input(x)
+        return m, x
+
+    m, x = start()  # an index range of 2^40 values
+    lo, hi, step = (m.new_initializer(np.array(v, np.int64)) for v in (0, 1 << 40, 1))
+    r = m.new_val()
+    m.add_node(Op.Range, [lo, hi, step], [r])
+    m.add_output(r)
+    assert outcome(m, [one]) == ERR_OOM
+    for extents in ([1 << 33, 1 << 33], [1 << 20, 1 << 20]):  # 2^66 elements (wraps to 4 in 64 bits) and 4 TB
+        m = Model()
+        x = m.new_val_named_and_shaped("x", [1])
+        m.add_input(x)
+        y = m.new_val()
+        m.add_node(Op.Expand, [x, m.new_initializer(np.array(extents, np.int64))], [y])
+        m.add_output(y)
+        assert outcome(m, [np.ones(1, np.float32)]) == ERR_OOM
+    m, x = start()  # a cycle
+    y, z = m.new_val(), m.new_val()
+    m.add_node(Op.ReLU, [z], [y])
+    m.add_node(Op.Sqrt, [y], [z])
+    m.add_output(z)
+    assert outcome(m, [one]) == ERR_UNSUPPORTED
+    m, x = start()  # a node that reads its own output
+    y = m.new_val()
+    m.add_node(Op.Add, [x, y], [y])
+    m.add_output(y)
+    assert outcome(m, [one]) == ERR_UNSUPPORTED
+    m, x = start()  # a value nobody produces
+    y, orphan = m.new_val(), m.new_val()
+    m.add_node(Op.ReLU, [orphan], [y])
+    m.add_output(y)
+    assert outcome(m, [one]) == ERR_UNSUPPORTED
+    m, x = start()  # nothing to compute: the input is the output, or there is no output
+    m.add_output(x)
+    sess = HipSessionBuilder(m).build()
+    (got,) = sess.run([one])
+    assert got.tolist() == one.tolist()
+    m, x = start()
+    assert HipSessionBuilder(m).build().run([one]) == []
+    sess = HipSessionBuilder(binary_model(Op.Add)).build()
+    (z,) = sess.run([one, one])
+    assert z.tolist() == [2.0] * 4
 
 
 def test_session_model_accessor_and_threads_option(case):

@@ -5,13 +5,15 @@ tests and from the documented behaviour of its functions (cited per test)."""
 import ctypes
 import os
 import re
+import subprocess
+import sys
 
 import numpy as np
 import pytest
 
 from altius_amd import _lib
 from altius_amd import device as D
-from altius_amd._lib import ERR_ARG, ERR_SHAPE, AltiusHipError
+from altius_amd._lib import ERR_ARG, ERR_OOM, ERR_SHAPE, AltiusHipError
 from altius_amd.graph import F32, I64, Model, Op, Tensor, host_pool_stats, host_pool_trim
 from altius_amd.graphs import erf_gelu_chain, layer_norm_chain
 
@@ -350,6 +352,59 @@ def test_eliminate_identity():
     assert m.eliminate_identity() == 1
     nodes = m.nodes()
     assert [n["op_name"] for n in nodes] == ["ReLU", "Identity"] and nodes[0]["inputs"] == [x]
+
+
+def test_extents_whose_product_does_not_fit_are_refused():
+    """usize arithmetic wraps in the reference's release build (tensor.rs:116-132 multiplies the extents); here a
+    product past 2^60 saturates, so the allocation sized from it fails instead of succeeding at the wrapped size
+    (2^33 x 2^33 elements would wrap to 4)."""
+    for dims in ([1 << 40, 1 << 40], [1 << 33, 1 << 33], [1 << 62, 4], [3, 1 << 31, 1 << 31]):
+        with pytest.raises(AltiusHipError) as e:
+            Tensor.zeros(dims)
+        assert e.value.code == ERR_OOM, dims
+    assert Tensor.zeros([0, 1 << 62, 1 << 62]).dims == [0, 1 << 62, 1 << 62]  # an empty tensor is empty whatever its other extents
+    m = Model()
+    x = m.new_val_named_and_shaped("x", [1 << 33, 1 << 33])
+    y = m.new_val()
+    m.add_node(Op.ReLU, [x], [y])
+    m.add_input(x)
+    assert m.infer_value_shape(y)[0] == [1 << 33, 1 << 33]  # shapes are only numbers until something is allocated
+
+
+OUT_OF_MEMORY_INSIDE_THE_LIBRARY = """
+import resource, sys
+from altius_amd.graph import Model, Op
+from altius_amd._lib import AltiusHipError, ERR_OOM
+m = Model()
+cur = m.new_val_named_and_shaped("x", [4])
+m.add_input(cur)
+for _ in range(60000):
+    nxt = m.new_val()
+    m.add_node(Op.ReLU, [cur], [nxt])
+    cur = nxt
+m.add_output(cur)
+size = next(int(line.split()[1]) * 1024 for line in open("/proc/self/status") if line.startswith("VmSize"))
+resource.setrlimit(resource.RLIMIT_AS, (size + (24 << 20), size + (24 << 20)))
+try:
+    copies = [m.clone() for _ in range(2000)]
+except AltiusHipError as e:
+    print("code", e.code, e.message)
+    sys.exit(0 if e.code == ERR_OOM else 4)
+except MemoryError:
+    print("the interpreter ran out first")
+    sys.exit(3)
+sys.exit(5)
+"""
+
+
+def test_running_out_of_memory_inside_the_library_is_an_error_code():
+    """No exception may unwind through the C boundary (the reference panics; a C++ exception escaping an extern "C"
+    function ends the caller's process).  A child process copies a 60 000-node model under an address-space limit a
+    few MB above what it already uses: the copy constructor's allocation fails inside ahip_model_clone, and the call
+    must return AHIP_ERR_OOM with the process alive."""
+    r = subprocess.run([sys.executable, "-c", OUT_OF_MEMORY_INSIDE_THE_LIBRARY], cwd=ROOT, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, (r.returncode, r.stdout[-300:], r.stderr[-300:])
+    assert "out of host memory" in r.stdout
 
 
 def test_argument_errors():
