@@ -1,19 +1,27 @@
 // ReduceMean / ReduceMax for gfx950 over an [outer, reduce, inner] view.
 //
 //   inner == 1 (reduced axes are the trailing ones):
-//     short or many rows  -> one wavefront per row, lanes stride through the
+//     rows under 4096     -> one wavefront per row, lanes stride through the
 //                            row (16-byte loads when rows stay aligned), lane
-//                            butterfly at the end;
-//     long rows           -> a grid of 256-thread blocks per row, each block
-//                            reducing a contiguous chunk through LDS; with more
+//                            butterfly at the end (short rows: a few lanes per
+//                            row, or groups of rows through LDS);
+//     longer rows         -> 256-thread blocks, each reducing a row or a
+//                            contiguous chunk of one through LDS; with more
 //                            than one chunk per row the partials go to the
 //                            context's scratch buffer and a second, tiny launch
 //                            folds them.
-//   inner > 1 (e.g. axis 1 of [256,768,197]):
-//     lanes own output columns, so a wave reads whole contiguous input rows;
-//     the 8 waves of a block interleave over the reduced axis and combine
-//     through LDS; the reduced axis can additionally be split over blocks,
-//     again through the scratch buffer.
+//   inner > 1 (e.g. axis 1 of [256,768,197], the tokens of [N,197,768]):
+//     rows of whole float4s -> lanes own float4 columns, the four wavefronts
+//                            of a block deal the rows between them and combine
+//                            through LDS (reduce_cols_vec4); a thread per
+//                            column for up to four rows (reduce_cols_few_rows);
+//     other widths to 1024 -> spans of rows that make whole 128-byte lines,
+//                            16-byte loads (reduce_cols_span);
+//     slabs of a few KB   -> groups of slabs through LDS, a thread per output
+//                            (reduce_small_slabs);
+//     anything else       -> lanes own single columns (reduce_cols).
+//     The reduced axis can additionally be split over blocks, again through
+//     the scratch buffer.
 //
 // Reference: crates/session_interpreter/src/session.rs:1292-1340.  ReduceMean
 // multiplies the sum by the f32 reciprocal of the reduced length, as the
@@ -21,6 +29,7 @@
 // sums are accumulated in a different order than the reference's 8 strided
 // accumulators.
 
+#include <algorithm>
 #include <mutex>
 
 #include "common.h"
@@ -146,7 +155,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void reduce_rows_sub4(float *__restrict_
 
 // grid = (splits, outer).  Block (s, o) folds chunk s of row o into
 // dst[o * splits + s].
-template <class OP, int VEC, bool SCALE>
+template <class OP, int VEC, bool SCALE, bool NT = false>
 __global__ __launch_bounds__(ROW_BLOCK) void reduce_rows_block(float *__restrict__ dst,
                                                                const float *__restrict__ in, size_t red,
                                                                size_t chunk, float scale) {
@@ -156,7 +165,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void reduce_rows_block(float *__restrict
     size_t end = begin + chunk;
     if (end > red) end = red;
     float acc = OP::identity();
-    if (begin < end) acc = strided_fold<OP, VEC>(in + o * red, begin, end, threadIdx.x, ROW_BLOCK);
+    if (begin < end) acc = strided_fold<OP, VEC, NT>(in + o * red, begin, end, threadIdx.x, ROW_BLOCK);
     acc = block_reduce<OP, ROW_WAVES>(acc, lds);
     if (threadIdx.x == 0) dst[o * gridDim.x + s] = SCALE ? acc * scale : acc;
 }
@@ -224,6 +233,133 @@ __global__ __launch_bounds__(COL_BLOCK) void reduce_cols(float *__restrict__ dst
         for (int w = 0; w < COL_WAVES; w++) a = OP::apply(a, lds[w][t]);
         const uint32_t c = blockIdx.y * (CPL * WAVE) + t;
         if (c < inner) dst[(size_t)blockIdx.x * inner + c] = SCALE ? a * scale : a;
+    }
+}
+
+// inner a multiple of 4 (rows of whole float4s, 16-byte aligned): lanes own float4 columns.  A block takes a tile of
+// tile4 = min(inner / 4, 64) float4 columns; where a row of the tile is narrower than a wavefront, the wavefront's
+// lanes cover rpp = 64 / tile4 consecutive rows of it at once (inner = 8: 32 rows, one contiguous KiB per load), so
+// the four wavefronts step through the reduced axis 4 * rpp rows at a time, CV_U loads in flight each.  The lanes'
+// float4 accumulators meet in LDS, where the first tile4 threads fold the 4 * rpp partial results of their column.
+// grid = (outer * splits * tiles of 64 float4 columns).
+constexpr int CV_BLOCK = 256, CV_WAVES = CV_BLOCK / WAVE, CV_U = 4;
+
+template <class OP> __device__ __forceinline__ float4 apply4(const float4 &a, const float4 &b) {
+    return make_float4(OP::apply(a.x, b.x), OP::apply(a.y, b.y), OP::apply(a.z, b.z), OP::apply(a.w, b.w));
+}
+
+template <class OP, bool SCALE, bool NT>
+__global__ __launch_bounds__(CV_BLOCK) void reduce_cols_vec4(float *__restrict__ dst, const float *__restrict__ in, uint32_t red,
+                                                             uint32_t inner, uint32_t splits, uint32_t chunk, uint32_t tile4,
+                                                             uint32_t rpp, uint32_t tiles, float scale) {
+    __shared__ float4 lds[CV_WAVES][WAVE];
+    const uint32_t lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x >> 6;
+    // Consecutive blocks take the column tiles of one (slab, split): together they read whole rows.
+    const uint32_t part = blockIdx.x / tiles, tile = blockIdx.x - part * tiles;
+    const uint32_t o = part / splits, s = part % splits;
+    const uint32_t lr = lane / tile4, lc = lane - lr * tile4;
+    const uint32_t v4 = inner >> 2, c4 = tile * WAVE + lc;
+    const uint32_t r_begin = s * chunk;
+    uint32_t r_end = r_begin + chunk;
+    if (r_end > red) r_end = red;
+    const uint32_t step = CV_WAVES * rpp;  // rows per pass of the block
+    const float id = OP::identity();
+    float4 acc = make_float4(id, id, id, id);
+    if (lr < rpp && c4 < v4) {
+        const float *col = in + (size_t)o * red * inner + 4 * (size_t)c4;
+        uint32_t r = r_begin + wave * rpp + lr;
+        for (; r + (CV_U - 1) * step < r_end; r += CV_U * step) {
+            float4 v[CV_U];
+#pragma unroll
+            for (int u = 0; u < CV_U; u++) v[u] = load4<NT>(col + (size_t)(r + u * step) * inner);
+#pragma unroll
+            for (int u = 0; u < CV_U; u++) acc = apply4<OP>(acc, v[u]);
+        }
+        {
+            // Up to CV_U - 1 more rows: all requested before the first is folded.
+            float4 v[CV_U - 1];
+#pragma unroll
+            for (int u = 0; u < CV_U - 1; u++)
+                v[u] = r + u * step < r_end ? load4<NT>(col + (size_t)(r + u * step) * inner) : make_float4(id, id, id, id);
+#pragma unroll
+            for (int u = 0; u < CV_U - 1; u++) acc = apply4<OP>(acc, v[u]);
+        }
+    }
+    lds[wave][lane] = acc;
+    __syncthreads();
+    const uint32_t t = threadIdx.x, out4 = tile * WAVE + t;
+    if (t < tile4 && out4 < v4) {
+        float4 a = make_float4(id, id, id, id);
+        for (uint32_t w = 0; w < CV_WAVES; w++)
+            for (uint32_t q = 0; q < rpp; q++) a = apply4<OP>(a, lds[w][q * tile4 + t]);
+        if (SCALE) a = make_float4(a.x * scale, a.y * scale, a.z * scale, a.w * scale);
+        *reinterpret_cast<float4 *>(dst + (size_t)part * inner + 4 * (size_t)out4) = a;
+    }
+}
+
+// Very few rows of many float4 columns ([768, 2, 65536]): a thread owns one float4 column of one slab and
+// walks all of its rows, CV_U loads in flight; nothing to combine.  Threads number the (slab, column) pairs, so a slab
+// narrower than a block leaves no thread idle.  grid = (outer * columns / 256 float4).
+template <class OP, bool SCALE, bool NT>
+__global__ __launch_bounds__(CV_BLOCK) void reduce_cols_few_rows(float *__restrict__ dst, const float *__restrict__ in, size_t outer,
+                                                                 uint32_t red, uint32_t inner, float scale) {
+    const uint32_t v4 = inner >> 2;
+    const size_t g = (size_t)blockIdx.x * CV_BLOCK + threadIdx.x;
+    const size_t o = g / v4;
+    if (o >= outer) return;
+    const uint32_t c4 = (uint32_t)(g - o * v4);
+    const float *col = in + o * red * inner + 4 * (size_t)c4;
+    const float id = OP::identity();
+    float4 acc = make_float4(id, id, id, id);
+    uint32_t r = 0;
+    for (; r + CV_U <= red; r += CV_U) {
+        float4 v[CV_U];
+#pragma unroll
+        for (int u = 0; u < CV_U; u++) v[u] = load4<NT>(col + (size_t)(r + u) * inner);
+#pragma unroll
+        for (int u = 0; u < CV_U; u++) acc = apply4<OP>(acc, v[u]);
+    }
+    for (; r < red; r++) acc = apply4<OP>(acc, load4<NT>(col + (size_t)r * inner));
+    if (SCALE) acc = make_float4(acc.x * scale, acc.y * scale, acc.z * scale, acc.w * scale);
+    *reinterpret_cast<float4 *>(dst + o * inner + 4 * (size_t)c4) = acc;
+}
+
+// Slabs of a few KB at most ([N, 7, 7] over axis 1, [N, 196, 3]): a block takes `group` consecutive slabs -- one
+// contiguous, 16-byte aligned piece of the tensor (group is a multiple of 4) -- into LDS with 16-byte loads, and then a
+// thread per output value walks its column there.  A block or a wavefront per slab would leave most lanes idle on 49
+// values, and lanes reading single columns from memory would fetch every 128-byte line many times.
+// grid = (outer / group); dynamic LDS = group * red * inner floats.
+constexpr int SS_BLOCK = 256;
+constexpr size_t SS_MAX_SLAB = 2048, SS_GROUP_FLOATS = 8192;
+
+template <class OP, bool SCALE, bool NT>
+__global__ __launch_bounds__(SS_BLOCK) void reduce_small_slabs(float *__restrict__ dst, const float *__restrict__ in, size_t outer,
+                                                               uint32_t red, uint32_t inner, uint32_t group, float scale) {
+    extern __shared__ __align__(16) float ss_lds[];
+    const uint32_t slab = red * inner;
+    const size_t o0 = (size_t)blockIdx.x * group;
+    const uint32_t n_slabs = outer - o0 < group ? (uint32_t)(outer - o0) : group;
+    const uint32_t floats = n_slabs * slab, n4 = floats >> 2;
+    const float *src = in + o0 * slab;
+#pragma unroll 4
+    for (uint32_t i = threadIdx.x; i < n4; i += SS_BLOCK) reinterpret_cast<float4 *>(ss_lds)[i] = load4<NT>(src + 4 * (size_t)i);
+    for (uint32_t i = (n4 << 2) + threadIdx.x; i < floats; i += SS_BLOCK) ss_lds[i] = src[i];  // the tensor's ragged end
+    __syncthreads();
+    const uint32_t outs = n_slabs * inner;
+    for (uint32_t j = threadIdx.x; j < outs; j += SS_BLOCK) {
+        const uint32_t ol = j / inner, c = j - ol * inner;
+        const float *p = ss_lds + ol * slab + c;
+        float a0 = OP::identity(), a1 = a0, a2 = a0, a3 = a0;
+        uint32_t r = 0;
+        for (; r + 4 <= red; r += 4) {
+            a0 = OP::apply(a0, p[r * inner]);
+            a1 = OP::apply(a1, p[(r + 1) * inner]);
+            a2 = OP::apply(a2, p[(r + 2) * inner]);
+            a3 = OP::apply(a3, p[(r + 3) * inner]);
+        }
+        for (; r < red; r++) a0 = OP::apply(a0, p[r * inner]);
+        const float acc = OP::apply(OP::apply(a0, a1), OP::apply(a2, a3));
+        dst[o0 * inner + j] = SCALE ? acc * scale : acc;
     }
 }
 
@@ -342,11 +478,14 @@ void rows_wave_launch(hipStream_t s, float *out, const float *in, size_t outer, 
 
 template <class OP, bool SCALE>
 void rows_block_launch(hipStream_t s, float *dst, const float *in, size_t outer, size_t red, size_t splits,
-                       size_t chunk, float scale) {
+                       size_t chunk, float scale, bool nt = false) {
     // Chunks start 16-byte aligned when the row pitch and the chunk length are multiples of 4.
     const bool vec4 = aligned16(in) && (red % 4 == 0 || outer == 1) && (chunk % 4 == 0);
     const dim3 grid((unsigned)splits, (unsigned)outer);
-    if (vec4)
+    if (vec4 && nt)
+        hipLaunchKernelGGL((reduce_rows_block<OP, 4, SCALE, true>), grid, dim3(ROW_BLOCK), 0, s, dst, in, red, chunk,
+                           scale);
+    else if (vec4)
         hipLaunchKernelGGL((reduce_rows_block<OP, 4, SCALE>), grid, dim3(ROW_BLOCK), 0, s, dst, in, red, chunk,
                            scale);
     else
@@ -354,9 +493,27 @@ void rows_block_launch(hipStream_t s, float *dst, const float *in, size_t outer,
                            scale);
 }
 
+// Whether reduce_cols_vec4 takes this geometry, and its grid's second extent.
+inline bool cols_vec4_fits(const float *dst, const float *in, size_t inner) {
+    return inner % 4 == 0 && aligned16(in) && aligned16(dst);
+}
+inline size_t cols_vec4_tiles(size_t inner) { return (inner / 4 + WAVE - 1) / WAVE; }
+
 template <class OP, bool SCALE>
 void cols_launch(hipStream_t s, float *dst, const float *in, size_t outer, size_t red, size_t inner,
-                 size_t splits, size_t chunk, float scale) {
+                 size_t splits, size_t chunk, float scale, bool nt = false) {
+    if (cols_vec4_fits(dst, in, inner)) {
+        const size_t v4 = inner / 4, tile4 = v4 < (size_t)WAVE ? v4 : (size_t)WAVE, rpp = WAVE / tile4;
+        const size_t tiles = cols_vec4_tiles(inner);
+        const dim3 grid((unsigned)(outer * splits * tiles));
+        if (nt)
+            hipLaunchKernelGGL((reduce_cols_vec4<OP, SCALE, true>), grid, dim3(CV_BLOCK), 0, s, dst, in, (uint32_t)red, (uint32_t)inner,
+                               (uint32_t)splits, (uint32_t)chunk, (uint32_t)tile4, (uint32_t)rpp, (uint32_t)tiles, scale);
+        else
+            hipLaunchKernelGGL((reduce_cols_vec4<OP, SCALE, false>), grid, dim3(CV_BLOCK), 0, s, dst, in, (uint32_t)red, (uint32_t)inner,
+                               (uint32_t)splits, (uint32_t)chunk, (uint32_t)tile4, (uint32_t)rpp, (uint32_t)tiles, scale);
+        return;
+    }
     const size_t cpl = inner <= 64 ? 1 : inner <= 128 ? 2 : 4;
     const size_t tiles = (inner + cpl * WAVE - 1) / (cpl * WAVE);
     const dim3 grid((unsigned)(outer * splits), (unsigned)tiles);
@@ -454,7 +611,9 @@ int reduce_impl(DeviceCtx &ctx, const Partials &pt, float *out, const float *in,
             const int rc = launch_reduce_rows_lds(ctx, std::is_same<OP, MaxOp>::value, out, in, outer, red, scale, SCALE);
             if (rc >= 0) return rc;
         }
-        if (red <= 4096 || outer >= 65536) {
+        // A wavefront per row below 4096 elements, a block of four above (measured over 96 M elements, non-temporal loads
+        // in both: 4096: 84 against 88 % of the HBM peak, 8192: 82 / 88, 16384: 77 / 87; 3072: 86.5 / 85.5).
+        if (red < 4096 || outer >= 65536) {
             if ((outer + ROW_WAVES - 1) / ROW_WAVES > MAX_GRID_X)
                 return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: too many rows for one launch");
             rows_wave_launch<OP, SCALE>(s, out, in, outer, red, scale, ctx.streaming(outer * red * sizeof(float)));
@@ -472,12 +631,13 @@ int reduce_impl(DeviceCtx &ctx, const Partials &pt, float *out, const float *in,
         size_t chunk = (red + splits - 1) / splits;
         chunk = (chunk + 1023) / 1024 * 1024;
         splits = (red + chunk - 1) / chunk;
+        const bool nt = ctx.streaming(outer * red * sizeof(float));
         if (splits == 1) {
-            rows_block_launch<OP, SCALE>(s, out, in, outer, red, 1, chunk, scale);
+            rows_block_launch<OP, SCALE>(s, out, in, outer, red, 1, chunk, scale, nt);
             return ctx.check(hipGetLastError(), "reduce rows (block) launch");
         }
         if (outer * splits > pt.floats) return partials_too_small(ctx, outer * splits, pt);
-        rows_block_launch<OP, false>(s, pt.ptr, in, outer, red, splits, chunk, 1.0f);
+        rows_block_launch<OP, false>(s, pt.ptr, in, outer, red, splits, chunk, 1.0f, nt);
         rows_wave_launch<OP, SCALE>(s, out, pt.ptr, outer, splits, scale);
         return ctx.check(hipGetLastError(), "reduce rows (two-stage) launch");
     }
@@ -485,6 +645,21 @@ int reduce_impl(DeviceCtx &ctx, const Partials &pt, float *out, const float *in,
     // inner > 1
     if (red >= ((size_t)1 << 32) || inner >= ((size_t)1 << 31))
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: axis extent exceeds 32-bit index range");
+    // Small slabs whose rows are not whole float4s, or too few and too narrow to keep half of reduce_cols_vec4's lanes busy.
+    if (red * inner <= SS_MAX_SLAB && aligned16(in) && (inner % 4 != 0 || red * std::min<size_t>(inner / 4, WAVE) < CV_BLOCK / 2)) {
+        const size_t slab = red * inner;
+        size_t group = SS_GROUP_FLOATS / slab / 4 * 4;  // SS_MAX_SLAB * 4 <= SS_GROUP_FLOATS: at least 4
+        while (group > 4 && (outer + group - 1) / group < 2048) group -= 4;  // rather more blocks than fuller ones
+        const size_t blocks = (outer + group - 1) / group;
+        if (blocks <= MAX_GRID_X) {
+            const bool nt = ctx.streaming(outer * slab * sizeof(float));
+            const dim3 grid((unsigned)blocks), block(SS_BLOCK);
+            const size_t shmem = group * slab * sizeof(float);
+            if (nt) hipLaunchKernelGGL((reduce_small_slabs<OP, SCALE, true>), grid, block, shmem, s, out, in, outer, (uint32_t)red, (uint32_t)inner, (uint32_t)group, scale);
+            else hipLaunchKernelGGL((reduce_small_slabs<OP, SCALE, false>), grid, block, shmem, s, out, in, outer, (uint32_t)red, (uint32_t)inner, (uint32_t)group, scale);
+            return ctx.check(hipGetLastError(), "reduce (small slabs) launch");
+        }
+    }
     // Rows that are not multiples of 16 bytes, moderate width: the span variant with 16-byte loads.
     if (inner % 4 != 0 && inner <= 1024 && aligned16(in) && (outer == 1 || (red * inner) % 4 == 0)) {
         const size_t span_rows = 32 / gcd_size(inner, 32);  // smallest P with P * inner * 4 bytes a multiple of 128
@@ -516,32 +691,46 @@ int reduce_impl(DeviceCtx &ctx, const Partials &pt, float *out, const float *in,
         }
     }
 
+    const bool nt = ctx.streaming(outer * red * inner * sizeof(float));
+    const bool vec4 = cols_vec4_fits(out, in, inner);
+    // Up to four rows (fewer than reduce_cols_vec4's wavefronts could share) of at least a wavefront's worth of float4
+    // columns: a thread per column, no partial results ([768,2,65536]: 84 % of the HBM peak against 53 %; from eight
+    // rows on the other kernel is ahead, [12288,8,1024]: 78 against 83 %).
+    if (vec4 && red <= 4 && inner >= 4 * (size_t)WAVE && (outer * (inner / 4) + CV_BLOCK - 1) / CV_BLOCK <= MAX_GRID_X) {
+        const dim3 grid((unsigned)((outer * (inner / 4) + CV_BLOCK - 1) / CV_BLOCK));
+        if (nt) hipLaunchKernelGGL((reduce_cols_few_rows<OP, SCALE, true>), grid, dim3(CV_BLOCK), 0, s, out, in, outer, (uint32_t)red, (uint32_t)inner, scale);
+        else hipLaunchKernelGGL((reduce_cols_few_rows<OP, SCALE, false>), grid, dim3(CV_BLOCK), 0, s, out, in, outer, (uint32_t)red, (uint32_t)inner, scale);
+        return ctx.check(hipGetLastError(), "reduce cols (few rows) launch");
+    }
     const size_t cpl = inner <= 64 ? 1 : inner <= 128 ? 2 : 4;
-    const size_t tiles = (inner + cpl * WAVE - 1) / (cpl * WAVE);
-    if (tiles > MAX_GRID_Y) return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: inner extent too large");
+    const size_t tiles = vec4 ? cols_vec4_tiles(inner) : (inner + cpl * WAVE - 1) / (cpl * WAVE);
+    if (!vec4 && tiles > MAX_GRID_Y) return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: inner extent too large");
     size_t splits = 1;
     const size_t blocks = outer * tiles;
-    if (blocks < 1024 && red >= 64) {
+    // Rows one pass of a block covers (its wavefronts take different rows; a wavefront of reduce_cols_vec4 covers
+    // several where a row is narrower than its 64 lanes): a block keeps at least eight passes.
+    const size_t rows_per_pass = vec4 ? (size_t)CV_WAVES * (WAVE / std::min<size_t>(inner / 4, WAVE)) : 4;
+    if (blocks < 1024 && red >= 16 * rows_per_pass) {
         splits = (1024 + blocks - 1) / blocks;
-        const size_t max_splits = red / 32;  // at least 32 rows (4 per wave) per block
+        const size_t max_splits = red / (8 * rows_per_pass);
         if (splits > max_splits) splits = max_splits;
         if (splits < 1) splits = 1;
     }
     size_t chunk = (red + splits - 1) / splits;
     splits = (red + chunk - 1) / chunk;
-    if (outer * splits > MAX_GRID_X)
+    if (outer * splits * (vec4 ? tiles : 1) > MAX_GRID_X)
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce: outer extent too large for one launch");
     if (splits == 1) {
-        cols_launch<OP, SCALE>(s, out, in, outer, red, inner, 1, chunk, scale);
+        cols_launch<OP, SCALE>(s, out, in, outer, red, inner, 1, chunk, scale, nt);
         return ctx.check(hipGetLastError(), "reduce cols launch");
     }
     if (outer * splits * inner > pt.floats) {
         if (pt.fixed) return partials_too_small(ctx, outer * splits * inner, pt);
         // Not enough scratch for the partials: do it in one stage.
-        cols_launch<OP, SCALE>(s, out, in, outer, red, inner, 1, red, scale);
+        cols_launch<OP, SCALE>(s, out, in, outer, red, inner, 1, red, scale, nt);
         return ctx.check(hipGetLastError(), "reduce cols launch");
     }
-    cols_launch<OP, false>(s, pt.ptr, in, outer, red, inner, splits, chunk, 1.0f);
+    cols_launch<OP, false>(s, pt.ptr, in, outer, red, inner, splits, chunk, 1.0f, nt);
     cols_launch<OP, SCALE>(s, out, pt.ptr, outer, splits, inner, 1, splits, scale);
     return ctx.check(hipGetLastError(), "reduce cols (two-stage) launch");
 }

@@ -434,6 +434,20 @@ REDUCE_CASES = [
     ([3, 640, 7], [1], False),         # span kernel, one float4 step per thread
     ([1, 4099, 33], [1], False),       # span kernel split over blocks, three left-over rows
     ([2, 130, 1023], [1], True),       # span kernel at its widest (four float4 steps per thread)
+    ([5, 197, 768], [1], False),       # float4 columns, three tiles of 64 per slab (mean over tokens)
+    ([9, 49, 1024], [1], True),        # the same, few rows per wavefront
+    ([3, 1000, 8], [1], False),        # float4 columns, 32 rows per wavefront pass
+    ([7, 333, 100], [1], False),       # 25 float4 per row: two rows per pass, 14 lanes idle
+    ([2, 70, 260], [1], False),        # a second tile of one float4 column
+    ([1, 5000, 256], [1], False),      # float4 columns, the reduced axis split over blocks through scratch
+    ([11, 2, 4096], [1], False),       # two to four rows of many columns: a thread per float4 column
+    ([5, 3, 260], [1], True),
+    ([40, 4, 256], [1], False),
+    ([1000, 7, 7], [1], False),        # small slabs staged through LDS in groups, a thread per output value
+    ([333, 196, 3], [1], True),
+    ([4099, 3, 4], [1], False),        # whole float4s, but too few rows for the float4-column kernel
+    ([10001, 2, 3], [1], False),       # groups of 1364 slabs, a ragged last group
+    ([3, 100, 20], [1], False),        # slabs of 2000 values: groups of four, the last one of three
 ]
 
 
