@@ -112,6 +112,17 @@ __device__ __forceinline__ float strided_fold(const float *__restrict__ x, size_
     return OP::apply(OP::apply(acc0, acc1), OP::apply(acc2, acc3));
 }
 
+// The same for a range that starts anywhere: single elements up to the first 16-byte boundary, then float4s.
+template <class OP, bool NT>
+__device__ __forceinline__ float peeled_fold(const float *__restrict__ x, size_t begin, size_t end, int tid, int nthreads) {
+    const size_t lead = (4 - ((reinterpret_cast<uintptr_t>(x + begin) >> 2) & 3)) & 3;
+    const size_t head = lead < end - begin ? lead : end - begin;
+    float acc = OP::identity();
+    if ((size_t)tid < head) acc = x[begin + tid];
+    return OP::apply(acc, strided_fold<OP, 4, NT>(x, begin + head, end, tid, nthreads));
+}
+
+// VEC: 4 = rows of whole float4s on 16-byte boundaries, 0 = rows that start anywhere (peeled_fold), 1 = single elements.
 template <class OP, int VEC, bool SCALE, bool NT>
 __global__ __launch_bounds__(ROW_BLOCK) void reduce_rows_wave(float *__restrict__ out,
                                                               const float *__restrict__ in, size_t outer,
@@ -119,7 +130,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void reduce_rows_wave(float *__restrict_
     const int lane = threadIdx.x & (WAVE - 1);
     const size_t row = (size_t)blockIdx.x * ROW_WAVES + (threadIdx.x >> 6);
     if (row >= outer) return;
-    float acc = strided_fold<OP, VEC, NT>(in + row * red, 0, red, lane, WAVE);
+    float acc = VEC == 0 ? peeled_fold<OP, NT>(in + row * red, 0, red, lane, WAVE) : strided_fold<OP, VEC == 0 ? 1 : VEC, NT>(in + row * red, 0, red, lane, WAVE);
     acc = wave_reduce<OP>(acc);
     if (lane == 0) out[row] = SCALE ? acc * scale : acc;
 }
@@ -165,7 +176,9 @@ __global__ __launch_bounds__(ROW_BLOCK) void reduce_rows_block(float *__restrict
     size_t end = begin + chunk;
     if (end > red) end = red;
     float acc = OP::identity();
-    if (begin < end) acc = strided_fold<OP, VEC, NT>(in + o * red, begin, end, threadIdx.x, ROW_BLOCK);
+    if (begin < end)
+        acc = VEC == 0 ? peeled_fold<OP, NT>(in + o * red, begin, end, threadIdx.x, ROW_BLOCK)
+                       : strided_fold<OP, VEC == 0 ? 1 : VEC, NT>(in + o * red, begin, end, threadIdx.x, ROW_BLOCK);
     acc = block_reduce<OP, ROW_WAVES>(acc, lds);
     if (threadIdx.x == 0) dst[o * gridDim.x + s] = SCALE ? acc * scale : acc;
 }
@@ -471,6 +484,12 @@ void rows_wave_launch(hipStream_t s, float *out, const float *in, size_t outer, 
     else if (vec4)
         hipLaunchKernelGGL((reduce_rows_wave<OP, 4, SCALE, false>), dim3((unsigned)blocks), dim3(ROW_BLOCK), 0, s, out,
                            in, outer, red, scale);
+    else if (red >= 64 && nt)  // long enough for a body of float4s behind the row's first elements
+        hipLaunchKernelGGL((reduce_rows_wave<OP, 0, SCALE, true>), dim3((unsigned)blocks), dim3(ROW_BLOCK), 0, s, out,
+                           in, outer, red, scale);
+    else if (red >= 64)
+        hipLaunchKernelGGL((reduce_rows_wave<OP, 0, SCALE, false>), dim3((unsigned)blocks), dim3(ROW_BLOCK), 0, s, out,
+                           in, outer, red, scale);
     else
         hipLaunchKernelGGL((reduce_rows_wave<OP, 1, SCALE, false>), dim3((unsigned)blocks), dim3(ROW_BLOCK), 0, s, out,
                            in, outer, red, scale);
@@ -488,8 +507,11 @@ void rows_block_launch(hipStream_t s, float *dst, const float *in, size_t outer,
     else if (vec4)
         hipLaunchKernelGGL((reduce_rows_block<OP, 4, SCALE>), grid, dim3(ROW_BLOCK), 0, s, dst, in, red, chunk,
                            scale);
+    else if (nt)
+        hipLaunchKernelGGL((reduce_rows_block<OP, 0, SCALE, true>), grid, dim3(ROW_BLOCK), 0, s, dst, in, red, chunk,
+                           scale);
     else
-        hipLaunchKernelGGL((reduce_rows_block<OP, 1, SCALE>), grid, dim3(ROW_BLOCK), 0, s, dst, in, red, chunk,
+        hipLaunchKernelGGL((reduce_rows_block<OP, 0, SCALE, false>), grid, dim3(ROW_BLOCK), 0, s, dst, in, red, chunk,
                            scale);
 }
 

@@ -467,24 +467,75 @@ __global__ __launch_bounds__(BT) void reduce_rows_lds(float *__restrict__ out, c
     }
 }
 
-// One block per row, any length: max pass, sum pass, write pass.
-__global__ __launch_bounds__(BLOCK) void softmax_block_stream(float *__restrict__ out,
-                                                              const float *__restrict__ in, size_t len) {
-    __shared__ float lds[WAVES_PER_BLOCK];
+// One block per row, any length and any 4-byte alignment: max pass, sum pass, write pass.  Every pass walks the row as
+// `head` single elements up to the first 16-byte boundary, a body of whole float4s with four loads in flight per thread,
+// and up to three single elements at the end; the second and third pass find the row in the caches (a row that does
+// not fit them would have to be read three times by any kernel that cannot hold it).  SAME: the output row starts at
+// the same offset from a 16-byte boundary as the input row, so the body is stored as float4s too.
+// The shape of a row as the streaming kernels walk it.
+struct RowWalk {
+    uint32_t head, tail;
+    size_t body4;
+    __device__ __forceinline__ RowWalk(const float *x, size_t len) {
+        const size_t lead = (4 - ((reinterpret_cast<uintptr_t>(x) >> 2) & 3)) & 3;
+        head = (uint32_t)(lead < len ? lead : len);
+        body4 = (len - head) >> 2;
+        tail = (uint32_t)(len - head - (body4 << 2));
+    }
+};
+
+// Folds f(element) over the row into `acc` with `join`; f4 handles a float4 of the body.
+template <int THREADS, class F1, class F4>
+__device__ __forceinline__ void walk_row(const float *__restrict__ x, const RowWalk &w, F1 one, F4 four) {
+    const uint32_t tid = threadIdx.x;
+    if (tid < w.head) one(x[tid], (size_t)tid);
+    const float *body = x + w.head;
+    size_t i = tid;
+    for (; i + 3 * (size_t)THREADS < w.body4; i += 4 * (size_t)THREADS) {
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) v[u] = *reinterpret_cast<const float4 *>(body + 4 * (i + u * (size_t)THREADS));
+#pragma unroll
+        for (int u = 0; u < 4; u++) four(v[u], w.head + 4 * (i + u * (size_t)THREADS));
+    }
+    for (; i < w.body4; i += THREADS) four(*reinterpret_cast<const float4 *>(body + 4 * i), w.head + 4 * i);
+    if (tid < w.tail) {
+        const size_t at = w.head + (w.body4 << 2) + tid;
+        one(x[at], at);
+    }
+}
+
+template <int THREADS, bool NT>
+__global__ __launch_bounds__(THREADS) void softmax_block_stream(float *__restrict__ out, const float *__restrict__ in, size_t len) {
+    __shared__ float lds[THREADS / WAVE];
     const float *x = in + (size_t)blockIdx.x * len;
     float *o = out + (size_t)blockIdx.x * len;
-    const float nan = __builtin_nanf("");
+    const RowWalk w(x, len);
+    const bool same = ((reinterpret_cast<uintptr_t>(x) ^ reinterpret_cast<uintptr_t>(o)) & 15u) == 0;
 
-    float mx = nan;
-    for (size_t i = threadIdx.x; i < len; i += BLOCK) mx = nanmax(x[i], mx);
-    mx = block_reduce<MaxOp, WAVES_PER_BLOCK>(mx, lds);
+    float mx = __builtin_nanf("");
+    walk_row<THREADS>(x, w, [&](float v, size_t) { mx = nanmax(v, mx); },
+                      [&](const float4 &v, size_t) { mx = nanmax(nanmax(v.x, v.y), nanmax(nanmax(v.z, v.w), mx)); });
+    mx = block_reduce<MaxOp, THREADS / WAVE>(mx, lds);
 
     float sum = 0.0f;
-    for (size_t i = threadIdx.x; i < len; i += BLOCK) sum += softmax_exp(x[i], mx);
-    sum = block_reduce<SumOp, WAVES_PER_BLOCK>(sum, lds);
+    walk_row<THREADS>(x, w, [&](float v, size_t) { sum += softmax_exp(v, mx); },
+                      [&](const float4 &v, size_t) {
+                          sum += (softmax_exp(v.x, mx) + softmax_exp(v.y, mx)) + (softmax_exp(v.z, mx) + softmax_exp(v.w, mx));
+                      });
+    sum = block_reduce<SumOp, THREADS / WAVE>(sum, lds);
     const float recip = 1.0f / sum;
 
-    for (size_t i = threadIdx.x; i < len; i += BLOCK) o[i] = softmax_exp(x[i], mx) * recip;
+    walk_row<THREADS>(x, w, [&](float v, size_t at) { o[at] = softmax_exp(v, mx) * recip; },
+                      [&](const float4 &v, size_t at) {
+                          const float4 e = make_float4(softmax_exp(v.x, mx) * recip, softmax_exp(v.y, mx) * recip,
+                                                       softmax_exp(v.z, mx) * recip, softmax_exp(v.w, mx) * recip);
+                          if (same) {
+                              store4<NT>(o + at, e);
+                          } else {
+                              o[at] = e.x, o[at + 1] = e.y, o[at + 2] = e.z, o[at + 3] = e.w;
+                          }
+                      });
 }
 
 // ---------------------------------------------------------------------------
@@ -596,42 +647,73 @@ __global__ __launch_bounds__(BLOCK) void layernorm_wave(float *__restrict__ out,
     r.template store<NT, FULL>(o, len, lane);
 }
 
-__global__ __launch_bounds__(BLOCK) void layernorm_block_stream(float *__restrict__ out,
-                                                                const float *__restrict__ in,
-                                                                const float *__restrict__ gamma,
-                                                                const float *__restrict__ beta, size_t len,
-                                                                float eps) {
-    __shared__ float lds[WAVES_PER_BLOCK];
+// One block per row, any length and alignment: sum pass, squared-deviation pass, write pass (see softmax_block_stream).
+// Scale and bias are read as float4s where the row's body lines up with theirs.
+template <int THREADS, bool NT>
+__global__ __launch_bounds__(THREADS) void layernorm_block_stream(float *__restrict__ out, const float *__restrict__ in,
+                                                                  const float *__restrict__ gamma, const float *__restrict__ beta,
+                                                                  size_t len, float eps) {
+    __shared__ float lds[THREADS / WAVE];
     const float *x = in + (size_t)blockIdx.x * len;
     float *o = out + (size_t)blockIdx.x * len;
+    const RowWalk w(x, len);
+    const bool same = ((reinterpret_cast<uintptr_t>(x) ^ reinterpret_cast<uintptr_t>(o)) & 15u) == 0;
+    // gamma + head and beta + head are 16-byte aligned
+    const bool gb4 = ((reinterpret_cast<uintptr_t>(gamma + w.head) | reinterpret_cast<uintptr_t>(beta + w.head)) & 15u) == 0;
     const float inv_n = 1.0f / (float)len;
 
     float sum = 0.0f;
-    for (size_t i = threadIdx.x; i < len; i += BLOCK) sum += x[i];
-    const float mean = block_reduce<SumOp, WAVES_PER_BLOCK>(sum, lds) * inv_n;
+    walk_row<THREADS>(x, w, [&](float v, size_t) { sum += v; }, [&](const float4 &v, size_t) { sum += (v.x + v.y) + (v.z + v.w); });
+    const float mean = block_reduce<SumOp, THREADS / WAVE>(sum, lds) * inv_n;
 
     float ss = 0.0f;
-    for (size_t i = threadIdx.x; i < len; i += BLOCK) {
-        const float d = x[i] - mean;
-        ss += d * d;
-    }
-    ss = block_reduce<SumOp, WAVES_PER_BLOCK>(ss, lds);
+    walk_row<THREADS>(x, w,
+                      [&](float v, size_t) {
+                          const float d = v - mean;
+                          ss += d * d;
+                      },
+                      [&](const float4 &v, size_t) {
+                          const float a = v.x - mean, b = v.y - mean, c = v.z - mean, d = v.w - mean;
+                          ss += (a * a + b * b) + (c * c + d * d);
+                      });
+    ss = block_reduce<SumOp, THREADS / WAVE>(ss, lds);
     const float inv_std = 1.0f / sqrtf(__builtin_fmaf(ss, inv_n, eps));
 
-    for (size_t i = threadIdx.x; i < len; i += BLOCK)
-        o[i] = __builtin_fmaf((x[i] - mean) * inv_std, gamma[i], beta[i]);
+    walk_row<THREADS>(x, w, [&](float v, size_t at) { o[at] = __builtin_fmaf((v - mean) * inv_std, gamma[at], beta[at]); },
+                      [&](const float4 &v, size_t at) {
+                          float4 g, b;
+                          if (gb4) {
+                              g = *reinterpret_cast<const float4 *>(gamma + at), b = *reinterpret_cast<const float4 *>(beta + at);
+                          } else {
+                              g = make_float4(gamma[at], gamma[at + 1], gamma[at + 2], gamma[at + 3]);
+                              b = make_float4(beta[at], beta[at + 1], beta[at + 2], beta[at + 3]);
+                          }
+                          const float4 e = make_float4(__builtin_fmaf((v.x - mean) * inv_std, g.x, b.x), __builtin_fmaf((v.y - mean) * inv_std, g.y, b.y),
+                                                       __builtin_fmaf((v.z - mean) * inv_std, g.z, b.z), __builtin_fmaf((v.w - mean) * inv_std, g.w, b.w));
+                          if (same) {
+                              store4<NT>(o + at, e);
+                          } else {
+                              o[at] = e.x, o[at + 1] = e.y, o[at + 2] = e.z, o[at + 3] = e.w;
+                          }
+                      });
 }
 
 // Long rows that are whole float4s: a block of THREADS threads per row with the row in registers (NCH float4 per
 // thread, read once); the two reductions go through LDS.  Few loads per thread and many threads per row: on this
 // part a wavefront that issues many 16-byte loads back to back streams more slowly than many wavefronts issuing a
 // few each.
-template <int THREADS, int NCH, bool NT>
+// SHIFT: rows that do not start on 16-byte boundaries (a length that is not a multiple of 4, or a base pointer that
+// is not aligned; input and output rows equally far past a boundary).  The block then holds the aligned float4s that
+// cover the row: float4 f holds row elements 4 f - m .. 4 f - m + 3, m = 0 .. 3 the elements by which the row starts
+// past a boundary.  All of them are aligned 16-byte accesses but the first and the last, which straddle the row's ends
+// and are read and written element by element.
+template <int THREADS, int NCH, bool NT, bool SHIFT = false>
 __global__ __launch_bounds__(THREADS) void softmax_block_regs(float *__restrict__ out, const float *__restrict__ in, size_t len) {
     __shared__ float lds[THREADS / WAVE];
     const float *x = in + (size_t)blockIdx.x * len;
     float *o = out + (size_t)blockIdx.x * len;
     const float nan = __builtin_nanf("");
+    const ptrdiff_t m = SHIFT ? (ptrdiff_t)((reinterpret_cast<uintptr_t>(x) >> 2) & 3) : 0, n = (ptrdiff_t)len;
     float4 r[NCH];
     float mx = nan;  // NaN elements (and the slots past the row) are ignored by the maximum
     // At most two 16-byte loads per thread are requested at a time; with four chunks the second pair goes out
@@ -641,8 +723,17 @@ __global__ __launch_bounds__(THREADS) void softmax_block_regs(float *__restrict_
     for (int k0 = 0; k0 < NCH; k0 += BURST) {
 #pragma unroll
         for (int k = k0; k < k0 + BURST; k++) {
-            const size_t e = ((size_t)threadIdx.x + (size_t)THREADS * k) * 4;
-            r[k] = e < len ? load4<NT>(x + e) : make_float4(nan, nan, nan, nan);
+            const ptrdiff_t e = ((ptrdiff_t)threadIdx.x + (ptrdiff_t)THREADS * k) * 4 - m;
+            if (!SHIFT) {
+                r[k] = e < n ? load4<NT>(x + e) : make_float4(nan, nan, nan, nan);
+            } else if (e >= 0 && e + 4 <= n) {
+                r[k] = load4<NT>(x + e);
+            } else {
+                r[k].x = e >= 0 && e < n ? x[e] : nan;
+                r[k].y = e + 1 >= 0 && e + 1 < n ? x[e + 1] : nan;
+                r[k].z = e + 2 >= 0 && e + 2 < n ? x[e + 2] : nan;
+                r[k].w = e + 3 >= 0 && e + 3 < n ? x[e + 3] : nan;
+            }
         }
 #pragma unroll
         for (int k = k0; k < k0 + BURST; k++) mx = nanmax(nanmax(r[k].x, r[k].y), nanmax(nanmax(r[k].z, r[k].w), mx));
@@ -652,16 +743,32 @@ __global__ __launch_bounds__(THREADS) void softmax_block_regs(float *__restrict_
     float sum = 0.0f;
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        const bool valid = ((size_t)threadIdx.x + (size_t)THREADS * k) * 4 < len;
+        const ptrdiff_t e = ((ptrdiff_t)threadIdx.x + (ptrdiff_t)THREADS * k) * 4 - m;
         r[k].x = softmax_exp(r[k].x, mx), r[k].y = softmax_exp(r[k].y, mx), r[k].z = softmax_exp(r[k].z, mx), r[k].w = softmax_exp(r[k].w, mx);
-        if (valid) sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
+        if (!SHIFT) {
+            if (e < n) sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
+        } else if (e >= 0 && e + 4 <= n) {
+            sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
+        } else {
+            sum += ((e >= 0 && e < n ? r[k].x : 0.0f) + (e + 1 >= 0 && e + 1 < n ? r[k].y : 0.0f)) +
+                   ((e + 2 >= 0 && e + 2 < n ? r[k].z : 0.0f) + (e + 3 >= 0 && e + 3 < n ? r[k].w : 0.0f));
+        }
     }
     sum = block_reduce<SumOp, THREADS / WAVE>(sum, lds);
     const float recip = 1.0f / sum;
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        const size_t e = ((size_t)threadIdx.x + (size_t)THREADS * k) * 4;
-        if (e < len) store4<NT>(o + e, make_float4(r[k].x * recip, r[k].y * recip, r[k].z * recip, r[k].w * recip));
+        const ptrdiff_t e = ((ptrdiff_t)threadIdx.x + (ptrdiff_t)THREADS * k) * 4 - m;
+        if (!SHIFT) {
+            if (e < n) store4<NT>(o + e, make_float4(r[k].x * recip, r[k].y * recip, r[k].z * recip, r[k].w * recip));
+        } else if (e >= 0 && e + 4 <= n) {
+            store4<NT>(o + e, make_float4(r[k].x * recip, r[k].y * recip, r[k].z * recip, r[k].w * recip));
+        } else {
+            if (e >= 0 && e < n) o[e] = r[k].x * recip;
+            if (e + 1 >= 0 && e + 1 < n) o[e + 1] = r[k].y * recip;
+            if (e + 2 >= 0 && e + 2 < n) o[e + 2] = r[k].z * recip;
+            if (e + 3 >= 0 && e + 3 < n) o[e + 3] = r[k].w * recip;
+        }
     }
 }
 
@@ -880,6 +987,12 @@ void softmax_block_go(bool nt, hipStream_t s, size_t rows, size_t resident, floa
     const dim3 grid((unsigned)rows);
     if (nt) hipLaunchKernelGGL((softmax_block_regs<THREADS, NCH, true>), grid, dim3(THREADS), 0, s, out, in, len);
     else hipLaunchKernelGGL((softmax_block_regs<THREADS, NCH, false>), grid, dim3(THREADS), 0, s, out, in, len);
+}
+template <int THREADS, int NCH>
+void softmax_block_shift_go(bool nt, hipStream_t s, size_t rows, float *out, const float *in, size_t len) {
+    const dim3 grid((unsigned)rows);
+    if (nt) hipLaunchKernelGGL((softmax_block_regs<THREADS, NCH, true, true>), grid, dim3(THREADS), 0, s, out, in, len);
+    else hipLaunchKernelGGL((softmax_block_regs<THREADS, NCH, false, true>), grid, dim3(THREADS), 0, s, out, in, len);
 }
 template <int THREADS, int NCH>
 void layernorm_block_go(bool nt, hipStream_t s, size_t rows, size_t resident, float *out, const float *in, const float *gamma, const float *beta,
@@ -1152,6 +1265,9 @@ constexpr size_t MAX_GRID = 0x7FFFFFFFu;
 
 }  // namespace
 
+// Threads of the streaming kernels' block: two float4 per thread and pass up to 8192 elements, then the widest block.
+inline int stream_block_threads(size_t len) { return len <= 2048 ? 256 : len <= 4096 ? 512 : 1024; }
+
 int launch_softmax(DeviceCtx &ctx, float *out, const float *in, size_t rows, size_t len) {
     if (rows == 0 || len == 0) return AHIP_OK;
     if (!out || !in) return ctx.fail(AHIP_ERR_ARG, "softmax: null tensor pointer");
@@ -1187,10 +1303,33 @@ int launch_softmax(DeviceCtx &ctx, float *out, const float *in, size_t rows, siz
         ALTIUS_BLOCK_LAYOUTS(lay)
 #undef ALTIUS_GO
         if (!launched) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: no block layout for this row length");
+    } else if (len > MAX_WAVE_ROW && len + 3 <= MAX_BLOCK_REG_ROW && rows <= MAX_GRID &&
+               ((reinterpret_cast<uintptr_t>(in) ^ reinterpret_cast<uintptr_t>(out)) & 15u) == 0) {
+        // Rows that start anywhere: the aligned float4s covering a row (up to three elements more than the row).
+        const bool nt = ctx.streaming(rows * len * sizeof(float));
+        const BlockLayout lay = block_layout(len + 6);
+        bool launched = false;
+#define ALTIUS_GO(T, N)                                                      \
+    case T * 100 + N:                                                        \
+        softmax_block_shift_go<T, N>(nt, ctx.stream, rows, out, in, len);    \
+        launched = true;                                                     \
+        break;
+        ALTIUS_BLOCK_LAYOUTS(lay)
+#undef ALTIUS_GO
+        if (!launched) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: no block layout for this row length");
     } else {
         if (rows > MAX_GRID) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: too many rows for one launch");
-        hipLaunchKernelGGL(softmax_block_stream, dim3((unsigned)rows), dim3(BLOCK), 0, ctx.stream, out, in,
-                           len);
+        const bool nt = ctx.streaming(rows * len * sizeof(float));
+        const int threads = stream_block_threads(len);
+#define ALTIUS_GO(T)                                                                                                          \
+    do {                                                                                                                      \
+        if (nt) hipLaunchKernelGGL((softmax_block_stream<T, true>), dim3((unsigned)rows), dim3(T), 0, ctx.stream, out, in, len);  \
+        else hipLaunchKernelGGL((softmax_block_stream<T, false>), dim3((unsigned)rows), dim3(T), 0, ctx.stream, out, in, len);    \
+    } while (0)
+        if (threads == 256) ALTIUS_GO(256);
+        else if (threads == 512) ALTIUS_GO(512);
+        else ALTIUS_GO(1024);
+#undef ALTIUS_GO
     }
     return ctx.check(hipGetLastError(), "softmax launch");
 }
@@ -1260,8 +1399,17 @@ int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *g
         if (!launched) return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: no block layout for this row length");
     } else {
         if (rows > MAX_GRID) return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: too many rows for one launch");
-        hipLaunchKernelGGL(layernorm_block_stream, dim3((unsigned)rows), dim3(BLOCK), 0, ctx.stream, out, in,
-                           gamma, beta, len, eps);
+        const bool nt = ctx.streaming(rows * len * sizeof(float));
+        const int threads = stream_block_threads(len);
+#define ALTIUS_GO(T)                                                                                                                          \
+    do {                                                                                                                                      \
+        if (nt) hipLaunchKernelGGL((layernorm_block_stream<T, true>), dim3((unsigned)rows), dim3(T), 0, ctx.stream, out, in, gamma, beta, len, eps);  \
+        else hipLaunchKernelGGL((layernorm_block_stream<T, false>), dim3((unsigned)rows), dim3(T), 0, ctx.stream, out, in, gamma, beta, len, eps);    \
+    } while (0)
+        if (threads == 256) ALTIUS_GO(256);
+        else if (threads == 512) ALTIUS_GO(512);
+        else ALTIUS_GO(1024);
+#undef ALTIUS_GO
     }
     return ctx.check(hipGetLastError(), "layernorm launch");
 }

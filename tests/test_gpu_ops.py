@@ -263,7 +263,8 @@ SOFTMAX_SHAPES = [[1, 2, 3], [3, 28, 28], [16, 512, 512], [2, 12, 197, 197], [5,
                   [3, 1028], [5, 1280], [9, 1536], [3, 2048], [2, 2560], [4, 3072], [2, 4092], [2, 4100],  # rows of 1025..4096 whole float4s stay in registers
                   [2, 5120], [3, 8192], [2, 8196], [2, 16384], [1, 12000], [2, 16388], [2, 5001],  # up to 16384: in a block's registers
                   [3, 1284], [3, 2052], [2, 3076], [2, 4608], [2, 6144], [2, 6148], [2, 12288],  # either side of every block width
-                  [5, 384], [7, 640], [6, 896], [3, 1088], [9, 1152], [13, 320]]  # a wavefront per row, last chunk partly filled
+                  [5, 384], [7, 640], [6, 896], [3, 1088], [9, 1152], [13, 320],  # a wavefront per row, last chunk partly filled
+                  [7, 1030], [5, 2049], [3, 4097], [3, 9999], [2, 16381], [2, 16383], [2, 50257]]  # rows that start anywhere: the aligned cover in registers to 16381, three passes above
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
@@ -303,7 +304,8 @@ LN_SHAPES = [[1, 20, 10], [2, 197, 768], [3, 5, 197], [4, 1], [5, 64], [3, 1024]
              [100, 49], [70, 197], [300, 64], [1000, 10], [64, 255], [65, 1], [200, 130], [4, 700, 192],  # short rows in groups through LDS
              [2, 5120], [3, 8192], [2, 8196], [2, 16384], [1, 12000], [2, 16388], [2, 5001],  # rows up to 16384 in a block's registers
              [3, 1284], [3, 2052], [2, 3076], [2, 4608], [2, 6144], [2, 6148], [2, 12288],  # either side of every block width
-             [5, 384], [7, 640], [6, 896], [3, 1088], [9, 1152], [1, 512], [13, 320]]  # a wavefront per row, last chunk partly filled, rows not a multiple of the block's four
+             [5, 384], [7, 640], [6, 896], [3, 1088], [9, 1152], [1, 512], [13, 320],  # a wavefront per row, last chunk partly filled, rows not a multiple of the block's four
+             [7, 1030], [5, 2049], [3, 4097], [3, 9999], [2, 16383], [2, 50257]]  # three passes with float4 bodies, rows that start anywhere
 
 
 @pytest.mark.parametrize("shape", LN_SHAPES)
@@ -448,6 +450,11 @@ REDUCE_CASES = [
     ([4099, 3, 4], [1], False),        # whole float4s, but too few rows for the float4-column kernel
     ([10001, 2, 3], [1], False),       # groups of 1364 slabs, a ragged last group
     ([3, 100, 20], [1], False),        # slabs of 2000 values: groups of four, the last one of three
+    ([7, 1030], [1], False),           # rows that start anywhere: single elements to the first 16-byte boundary, then float4s
+    ([5, 2049], [1], True),
+    ([3, 5001], [1], False),           # the same in the block kernel
+    ([2, 50257], [1], False),
+    ([1, 3, 70001], [2], False),
 ]
 
 
