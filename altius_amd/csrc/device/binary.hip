@@ -275,6 +275,40 @@ __global__ __launch_bounds__(BLOCK) void binary_rowbcast(float *__restrict__ out
     }
 }
 
+// A vector of two or three values on the innermost axis ([N,H,W,3] op [3]): shorter than a lane's four elements, which
+// therefore cycle through it more than once; the vector lives in three registers.
+template <class OP, bool SMALL_IS_A, bool NT>
+__global__ __launch_bounds__(BLOCK) void binary_short_vector(float *__restrict__ out, const float *__restrict__ full,
+                                                             const float *__restrict__ small, const FastDiv c, uint32_t total) {
+    const uint32_t i0 = (blockIdx.x * BLOCK + threadIdx.x) * 4;
+    if (i0 >= total) return;
+    const bool whole = i0 + 4 <= total;
+    float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (whole) x = load4<NT>(full + i0);
+    const uint32_t C = c.d;
+    const float v0 = small[0], v1 = small[1], v2 = small[C > 2 ? 2 : 0];
+    uint32_t idx = i0 - c.div(i0) * C;
+    float y[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        y[j] = idx == 0 ? v0 : idx == 1 ? v1 : v2;
+        idx = idx + 1 == C ? 0 : idx + 1;
+    }
+    if (whole) {
+        float4 r;
+        r.x = SMALL_IS_A ? OP::f(y[0], x.x) : OP::f(x.x, y[0]);
+        r.y = SMALL_IS_A ? OP::f(y[1], x.y) : OP::f(x.y, y[1]);
+        r.z = SMALL_IS_A ? OP::f(y[2], x.z) : OP::f(x.z, y[2]);
+        r.w = SMALL_IS_A ? OP::f(y[3], x.w) : OP::f(x.w, y[3]);
+        store4<NT>(out + i0, r);
+    } else {
+        for (int j = 0; j < 4 && i0 + j < total; j++) {
+            const float xs = full[i0 + j];
+            out[i0 + j] = SMALL_IS_A ? OP::f(y[j], xs) : OP::f(xs, y[j]);
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Kernel for rows that are whole float4s with a small operand that is constant along or across the row:
 //   out[r][c] = full[r][c] op small[c]            a bias or scale vector on rows longer than the row-broadcast kernel stages
@@ -422,6 +456,19 @@ void rowbcast_launch(hipStream_t s, bool small_is_a, bool nt, bool ntl, float *o
     }
 }
 
+template <class OP>
+void short_vector_launch(hipStream_t s, bool small_is_a, bool nt, float *out, const float *full, const float *small, uint32_t c, uint32_t total) {
+    const dim3 grid((total + BLOCK * 4 - 1) / (BLOCK * 4));
+    const FastDiv fd = make_fastdiv(c);
+    if (small_is_a) {
+        if (nt) hipLaunchKernelGGL((binary_short_vector<OP, true, true>), grid, dim3(BLOCK), 0, s, out, full, small, fd, total);
+        else hipLaunchKernelGGL((binary_short_vector<OP, true, false>), grid, dim3(BLOCK), 0, s, out, full, small, fd, total);
+    } else {
+        if (nt) hipLaunchKernelGGL((binary_short_vector<OP, false, true>), grid, dim3(BLOCK), 0, s, out, full, small, fd, total);
+        else hipLaunchKernelGGL((binary_short_vector<OP, false, false>), grid, dim3(BLOCK), 0, s, out, full, small, fd, total);
+    }
+}
+
 template <class OP, int KIND>
 void rows4_launch_kind(hipStream_t s, bool small_is_a, bool nt, bool ntl, float *out, const float *full, const float *small, uint32_t total,
                        const FastDiv &c, const FastDiv &o) {
@@ -563,6 +610,19 @@ int launch_binary(DeviceCtx &ctx, int op, float *out, const float *a, const floa
         const int64_t C = dims[r - 1];
         // A block covers BLOCK*4 consecutive elements and stages two rows of the small operand, so
         // an outer index must span at least that many elements.
+        if (other == FULL && pattern2 && (C == 2 || C == 3) && total < LIMIT && aligned16(out) && aligned16(ma == STRIDED ? b : a)) {
+            const bool small_is_a = ma == STRIDED;
+            const float *full = small_is_a ? b : a;
+            const float *small = small_is_a ? a : b;
+            switch (op) {
+            case AHIP_ADD: short_vector_launch<OpAdd>(s, small_is_a, nt, out, full, small, (uint32_t)C, (uint32_t)total); break;
+            case AHIP_SUB: short_vector_launch<OpSub>(s, small_is_a, nt, out, full, small, (uint32_t)C, (uint32_t)total); break;
+            case AHIP_MUL: short_vector_launch<OpMul>(s, small_is_a, nt, out, full, small, (uint32_t)C, (uint32_t)total); break;
+            case AHIP_DIV: short_vector_launch<OpDiv>(s, small_is_a, nt, out, full, small, (uint32_t)C, (uint32_t)total); break;
+            case AHIP_POW: short_vector_launch<OpPow>(s, small_is_a, nt, out, full, small, (uint32_t)C, (uint32_t)total); break;
+            }
+            return ctx.check(hipGetLastError(), "binary short-vector launch");
+        }
         const bool two_rows_suffice = pattern2 || (r == 3 && dims[1] * dims[2] >= BLOCK * 4);
         if (other == FULL && (pattern3 || pattern2) && two_rows_suffice && C >= 4 && C <= 512 && total < LIMIT &&
             aligned16(out) &&

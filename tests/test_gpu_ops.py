@@ -77,6 +77,11 @@ BIN_SHAPES = [
     ([9, 4], [9, 1]),
     ([64, 576, 7, 7], [576, 1, 1]),
     ([768, 1024, 7, 7], [768, 1024, 1, 1]),  # non-temporal variant
+    # a vector of two or three values (an RGB mean on NHWC): a lane's four elements cycle through it
+    ([5, 67, 3], [3]),
+    ([3], [2, 224, 224, 3]),
+    ([333, 2], [2]),
+    ([4096, 4096, 3], [3]),              # non-temporal variant
 ]
 
 
