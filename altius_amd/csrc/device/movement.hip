@@ -113,6 +113,59 @@ __global__ __launch_bounds__(BLOCK) void transpose_tiled(T *__restrict__ out, co
     }
 }
 
+// The same patch with 16-byte accesses on both sides, for 4-byte elements when both extents, both strides and every
+// batch offset are multiples of 4 and the tensors are 16-byte aligned: a thread reads four float4 along C and writes
+// four float4 along R (each gathered from four LDS rows).  The pitch of 65 words keeps both the row-wise stores and
+// the column-wise gathers of a wavefront on 64 different banks.
+template <bool NT>
+__global__ __launch_bounds__(BLOCK) void transpose_tiled_vec4(uint32_t *__restrict__ out, const uint32_t *__restrict__ in, TransGeom g) {
+    __shared__ uint32_t tile[TILE][TILE + 1];
+    uint32_t rest = blockIdx.z, src0 = 0, dst0 = 0;
+#pragma unroll
+    for (int d = 0; d < MAX_RANK; d++) {
+        if (d < g.brank) {
+            const uint32_t q = g.bdims[d].div(rest);
+            const uint32_t r = rest - q * g.bdims[d].d;
+            src0 += r * g.b_in_str[d];
+            dst0 += r * g.b_out_str[d];
+            rest = q;
+        }
+    }
+    // Tiles are dealt diagonally: blocks that run together (consecutive blockIdx.x) then differ in R as well as in C, so
+    // with a pitch that is a large power of two their rows do not all fall on the same memory channels.
+    uint32_t by = blockIdx.y + blockIdx.x;
+    by = by >= gridDim.y ? by % gridDim.y : by;
+    const uint32_t c0 = blockIdx.x * TILE, r0 = by * TILE;
+    const uint32_t q4 = threadIdx.x & 15, line = threadIdx.x >> 4;  // 16 float4 per 64-wide line, 16 lines per pass
+    u32x4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const uint32_t r = r0 + line + 16 * k, c = c0 + 4 * q4;
+        v[k] = u32x4{0, 0, 0, 0};
+        if (r < g.r_len && c < g.c_len) {
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(in + src0 + (size_t)r * g.r_in_str + c);
+            v[k] = NT ? __builtin_nontemporal_load(p) : *p;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        uint32_t *row = &tile[line + 16 * k][4 * q4];
+        row[0] = v[k].x, row[1] = v[k].y, row[2] = v[k].z, row[3] = v[k].w;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const uint32_t c = c0 + line + 16 * k, r = r0 + 4 * q4;
+        if (r < g.r_len && c < g.c_len) {
+            const uint32_t col = line + 16 * k;
+            const u32x4 w = {tile[4 * q4][col], tile[4 * q4 + 1][col], tile[4 * q4 + 2][col], tile[4 * q4 + 3][col]};
+            u32x4 *p = reinterpret_cast<u32x4 *>(out + dst0 + (size_t)c * g.c_out_str + r);
+            if (NT) __builtin_nontemporal_store(w, p);
+            else *p = w;
+        }
+    }
+}
+
 // Batched transpose of small matrices that are contiguous on both sides (attention's K^T:
 // [.., 197, 64] -> [.., 64, 197]).  One block moves one whole r_len x c_len matrix: it reads the
 // matrix as one contiguous span, scatters it into LDS transposed, and writes the result as one
@@ -623,6 +676,20 @@ int launch_transpose(DeviceCtx &ctx, void *out, const void *in, int elem_size, i
         return launch_copy_strided(ctx, out, in, elem_size, (int)d.size(), d.data(), so.data(), si.data());
     }
     const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batches);
+    if (elem_size == 4 && g.r_len % 4 == 0 && g.c_len % 4 == 0 && g.r_in_str % 4 == 0 && g.c_out_str % 4 == 0 &&
+        (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && (reinterpret_cast<uintptr_t>(in) & 15u) == 0) {
+        bool batches_line_up = true;
+        for (int i = 0; i < g.brank; i++) batches_line_up = batches_line_up && g.b_in_str[i] % 4 == 0 && g.b_out_str[i] % 4 == 0;
+        if (batches_line_up) {
+            if (ctx.streaming(total * 4))
+                hipLaunchKernelGGL((transpose_tiled_vec4<true>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint32_t *>(out),
+                                   static_cast<const uint32_t *>(in), g);
+            else
+                hipLaunchKernelGGL((transpose_tiled_vec4<false>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint32_t *>(out),
+                                   static_cast<const uint32_t *>(in), g);
+            return ctx.check(hipGetLastError(), "transpose_tiled (16-byte) launch");
+        }
+    }
     switch (elem_size) {
     case 1:
         hipLaunchKernelGGL((transpose_tiled<uint8_t>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint8_t *>(out),

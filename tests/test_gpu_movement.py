@@ -32,6 +32,9 @@ TRANSPOSES = [
     ((5, 1, 7, 1, 3), (4, 3, 2, 1, 0)), ((2, 3, 4, 5, 6, 2), (5, 0, 3, 1, 4, 2)),
     ((8, 3, 14, 14), (0, 2, 3, 1)),        # NCHW -> NHWC
     ((7,), (0,)), ((0, 5), (1, 0)), ((4, 0, 3), (2, 0, 1)),
+    # both extents and pitches whole float4s: 16-byte accesses on both sides, tiles dealt diagonally
+    ((256, 320), (1, 0)), ((3, 64, 28, 28), (0, 2, 3, 1)), ((3, 28, 28, 64), (0, 3, 1, 2)), ((68, 132), (1, 0)),
+    ((5, 100, 72), (0, 2, 1)), ((100, 5, 72), (2, 1, 0)), ((24, 16, 20, 32), (3, 2, 1, 0)), ((1000, 16), (1, 0)),
 ]
 
 
