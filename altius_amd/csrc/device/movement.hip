@@ -65,6 +65,36 @@ __global__ __launch_bounds__(BLOCK) void copy_strided(T *__restrict__ out, const
     }
 }
 
+// The element-wise copy with four elements per thread, BLOCK apart (each access of a wavefront stays as coalesced as
+// it was): the four loads are requested before the first store, and a block's index arithmetic overlaps them.
+template <class T>
+__global__ __launch_bounds__(BLOCK) void copy_strided_x4(T *__restrict__ out, const T *__restrict__ in, CopyGeom g, uint32_t total) {
+    const uint32_t first = blockIdx.x * (4 * BLOCK) + threadIdx.x;
+    uint32_t src[4], dst[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        uint32_t rest = first + k * BLOCK;
+        src[k] = dst[k] = 0;
+#pragma unroll
+        for (int d = 0; d < MAX_RANK; d++) {
+            if (d < g.rank) {
+                const uint32_t q = g.dims[d].div(rest);
+                const uint32_t r = rest - q * g.dims[d].d;
+                src[k] += r * g.in_str[d];
+                dst[k] += r * g.out_str[d];
+                rest = q;
+            }
+        }
+    }
+    T v[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        if (first + k * BLOCK < total) v[k] = in[src[k]];
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        if (first + k * BLOCK < total) out[dst[k]] = v[k];
+}
+
 // ---- tiled transpose -------------------------------------------------------------------------
 // For permutations whose output-innermost axis is not the input-innermost axis.  View the tensor
 // as [batch..., R, ..., C, ...] where C is the input's contiguous axis and R the axis that becomes
@@ -459,6 +489,11 @@ int fits32(DeviceCtx &ctx, size_t total, const char *what) {
 
 template <class T>
 void launch_copy(hipStream_t s, void *out, const void *in, const CopyGeom &g, uint32_t total) {
+    if (sizeof(T) < 16 && total >= 16 * BLOCK) {  // elements past `total` are decomposed too (and dropped): no address is formed from them
+        hipLaunchKernelGGL((copy_strided_x4<T>), dim3((total + 4 * BLOCK - 1) / (4 * BLOCK)), dim3(BLOCK), 0, s, static_cast<T *>(out),
+                           static_cast<const T *>(in), g, total);
+        return;
+    }
     hipLaunchKernelGGL((copy_strided<T>), dim3((total + BLOCK - 1) / BLOCK), dim3(BLOCK), 0, s, static_cast<T *>(out),
                        static_cast<const T *>(in), g, total);
 }
