@@ -828,6 +828,71 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_regs(float *__restric
     }
 }
 
+// LayerNormalization over rows that start anywhere (see softmax_block_regs' SHIFT): the block holds the aligned float4s
+// covering the row; scale and bias, which do not share the row's shift, are read element by element at the end (cache
+// hits), or as float4s where the row happens to start on a boundary.
+template <int THREADS, int NCH, bool NT>
+__global__ __launch_bounds__(THREADS) void layernorm_block_shift(float *__restrict__ out, const float *__restrict__ in,
+                                                                 const float *__restrict__ gamma, const float *__restrict__ beta, size_t len,
+                                                                 float eps) {
+    __shared__ float lds[THREADS / WAVE];
+    const float *x = in + (size_t)blockIdx.x * len;
+    float *o = out + (size_t)blockIdx.x * len;
+    const ptrdiff_t m = (ptrdiff_t)((reinterpret_cast<uintptr_t>(x) >> 2) & 3), n = (ptrdiff_t)len;
+    const bool gb4 = m == 0 && ((reinterpret_cast<uintptr_t>(gamma) | reinterpret_cast<uintptr_t>(beta)) & 15u) == 0;
+    const float inv_n = 1.0f / (float)len;
+    float4 r[NCH];
+    float sum = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NCH; k++) {
+        const ptrdiff_t e = ((ptrdiff_t)threadIdx.x + (ptrdiff_t)THREADS * k) * 4 - m;
+        if (e >= 0 && e + 4 <= n) {
+            r[k] = load4<NT>(x + e);
+        } else {  // slots outside the row hold zero: they add nothing to the sum
+            r[k].x = e >= 0 && e < n ? x[e] : 0.0f;
+            r[k].y = e + 1 >= 0 && e + 1 < n ? x[e + 1] : 0.0f;
+            r[k].z = e + 2 >= 0 && e + 2 < n ? x[e + 2] : 0.0f;
+            r[k].w = e + 3 >= 0 && e + 3 < n ? x[e + 3] : 0.0f;
+        }
+        sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
+    }
+    const float mean = block_reduce<SumOp, THREADS / WAVE>(sum, lds) * inv_n;
+    float ss = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NCH; k++) {
+        const ptrdiff_t e = ((ptrdiff_t)threadIdx.x + (ptrdiff_t)THREADS * k) * 4 - m;
+        r[k].x -= mean, r[k].y -= mean, r[k].z -= mean, r[k].w -= mean;
+        if (e >= 0 && e + 4 <= n) {
+            ss += (r[k].x * r[k].x + r[k].y * r[k].y) + (r[k].z * r[k].z + r[k].w * r[k].w);
+        } else {
+            ss += ((e >= 0 && e < n ? r[k].x * r[k].x : 0.0f) + (e + 1 >= 0 && e + 1 < n ? r[k].y * r[k].y : 0.0f)) +
+                  ((e + 2 >= 0 && e + 2 < n ? r[k].z * r[k].z : 0.0f) + (e + 3 >= 0 && e + 3 < n ? r[k].w * r[k].w : 0.0f));
+        }
+    }
+    ss = block_reduce<SumOp, THREADS / WAVE>(ss, lds);
+    const float inv_std = 1.0f / sqrtf(__builtin_fmaf(ss, inv_n, eps));
+#pragma unroll
+    for (int k = 0; k < NCH; k++) {
+        const ptrdiff_t e = ((ptrdiff_t)threadIdx.x + (ptrdiff_t)THREADS * k) * 4 - m;
+        if (e >= 0 && e + 4 <= n) {
+            float4 g, b;
+            if (gb4) {
+                g = *reinterpret_cast<const float4 *>(gamma + e), b = *reinterpret_cast<const float4 *>(beta + e);
+            } else {
+                g = make_float4(gamma[e], gamma[e + 1], gamma[e + 2], gamma[e + 3]);
+                b = make_float4(beta[e], beta[e + 1], beta[e + 2], beta[e + 3]);
+            }
+            store4<NT>(o + e, make_float4(__builtin_fmaf(r[k].x * inv_std, g.x, b.x), __builtin_fmaf(r[k].y * inv_std, g.y, b.y),
+                                          __builtin_fmaf(r[k].z * inv_std, g.z, b.z), __builtin_fmaf(r[k].w * inv_std, g.w, b.w)));
+        } else {
+            if (e >= 0 && e < n) o[e] = __builtin_fmaf(r[k].x * inv_std, gamma[e], beta[e]);
+            if (e + 1 >= 0 && e + 1 < n) o[e + 1] = __builtin_fmaf(r[k].y * inv_std, gamma[e + 1], beta[e + 1]);
+            if (e + 2 >= 0 && e + 2 < n) o[e + 2] = __builtin_fmaf(r[k].z * inv_std, gamma[e + 2], beta[e + 2]);
+            if (e + 3 >= 0 && e + 3 < n) o[e + 3] = __builtin_fmaf(r[k].w * inv_std, gamma[e + 3], beta[e + 3]);
+        }
+    }
+}
+
 // The block-per-row kernels again for rows that take 1024 threads: two such blocks are all a CU holds, and a block
 // that loads its row, reduces, reduces again and stores leaves the memory pipeline idle while it reduces.  Here a
 // block walks rows blockIdx.x, blockIdx.x + gridDim.x, ... and requests the next row before it works on the one it
@@ -993,6 +1058,13 @@ void softmax_block_shift_go(bool nt, hipStream_t s, size_t rows, float *out, con
     const dim3 grid((unsigned)rows);
     if (nt) hipLaunchKernelGGL((softmax_block_regs<THREADS, NCH, true, true>), grid, dim3(THREADS), 0, s, out, in, len);
     else hipLaunchKernelGGL((softmax_block_regs<THREADS, NCH, false, true>), grid, dim3(THREADS), 0, s, out, in, len);
+}
+template <int THREADS, int NCH>
+void layernorm_block_shift_go(bool nt, hipStream_t s, size_t rows, float *out, const float *in, const float *gamma, const float *beta, size_t len,
+                              float eps) {
+    const dim3 grid((unsigned)rows);
+    if (nt) hipLaunchKernelGGL((layernorm_block_shift<THREADS, NCH, true>), grid, dim3(THREADS), 0, s, out, in, gamma, beta, len, eps);
+    else hipLaunchKernelGGL((layernorm_block_shift<THREADS, NCH, false>), grid, dim3(THREADS), 0, s, out, in, gamma, beta, len, eps);
 }
 template <int THREADS, int NCH>
 void layernorm_block_go(bool nt, hipStream_t s, size_t rows, size_t resident, float *out, const float *in, const float *gamma, const float *beta,
@@ -1393,6 +1465,20 @@ int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *g
     case T * 100 + N:                                                                        \
         layernorm_block_go<T, N>(nt, ctx.stream, rows, resident, out, in, gamma, beta, len, eps); \
         launched = true;                                                                     \
+        break;
+        ALTIUS_BLOCK_LAYOUTS(lay)
+#undef ALTIUS_GO
+        if (!launched) return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: no block layout for this row length");
+    } else if (len > MAX_WAVE_ROW && len + 3 <= MAX_BLOCK_REG_ROW && rows <= MAX_GRID &&
+               ((reinterpret_cast<uintptr_t>(in) ^ reinterpret_cast<uintptr_t>(out)) & 15u) == 0) {
+        // Rows that start anywhere: the aligned float4s covering a row (see launch_softmax).
+        const bool nt = ctx.streaming(rows * len * sizeof(float));
+        const BlockLayout lay = block_layout(len + 6);
+        bool launched = false;
+#define ALTIUS_GO(T, N)                                                                            \
+    case T * 100 + N:                                                                              \
+        layernorm_block_shift_go<T, N>(nt, ctx.stream, rows, out, in, gamma, beta, len, eps);      \
+        launched = true;                                                                           \
         break;
         ALTIUS_BLOCK_LAYOUTS(lay)
 #undef ALTIUS_GO
