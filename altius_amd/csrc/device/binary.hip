@@ -577,6 +577,17 @@ int launch_binary(DeviceCtx &ctx, int op, float *out, const float *a, const floa
     const bool nt = ctx.streaming(total * sizeof(float)), ntl = ctx.streaming_loads(total * sizeof(float));
     if (ma != STRIDED && mb != STRIDED) {
         const bool vec = aligned16(out) && (ma != FULL || aligned16(a)) && (mb != FULL || aligned16(b));
+        // Every dense tensor equally far past a 16-byte boundary (views into the middle of buffers), and large enough
+        // for a second launch not to matter: the one to three elements up to the boundary on their own, the rest as float4s.
+        const uintptr_t off = reinterpret_cast<uintptr_t>(out) & 15u;
+        auto same_off = [&](int mode, const float *p) { return mode != FULL || (reinterpret_cast<uintptr_t>(p) & 15u) == off; };
+        if (!vec && off != 0 && off % 4 == 0 && same_off(ma, a) && same_off(mb, b) && total >= ((size_t)1 << 16)) {
+            const size_t head = (16 - off) / 4;
+            const int64_t head_dims[1] = {(int64_t)head}, rest_dims[1] = {(int64_t)(total - head)};
+            const int64_t sa[1] = {ma == FULL ? 1 : 0}, sb[1] = {mb == FULL ? 1 : 0};
+            if (int rc = launch_binary(ctx, op, out, a, b, 1, head_dims, sa, sb)) return rc;
+            return launch_binary(ctx, op, out + head, ma == FULL ? a + head : a, mb == FULL ? b + head : b, 1, rest_dims, sa, sb);
+        }
         switch (op) {
         case AHIP_ADD: flat_launch<OpAdd>(s, ma, mb, out, a, b, total, vec, nt, ntl); break;
         case AHIP_SUB: flat_launch<OpSub>(s, ma, mb, out, a, b, total, vec, nt, ntl); break;

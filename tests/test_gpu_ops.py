@@ -328,6 +328,29 @@ def test_layernorm(ctx, oracle, case, shape):
     np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("off", [1, 2, 3])
+def test_flat_operators_on_large_views_that_start_off_a_boundary(ctx, oracle, case, off):
+    """Every tensor `off` floats past a 16-byte boundary and large enough for two launches: the elements up to the
+    boundary go on their own and the rest as float4s; not a bit may differ from the aligned call."""
+    case(f"Gelu / Add / Mul by a scalar / Sub from a scalar on 70001 elements, every tensor +{off} floats")
+    n = 70001
+    a, b = synth.normal(81, (n + off,)), synth.normal(82, (n + off,), mean=2.0)
+    da, db = ctx.upload(a), ctx.upload(b)
+    do = ctx.alloc((n + 4) * 4)
+    ds = ctx.upload(np.array([1.7], np.float32))
+    pa, pb, po = da.ptr + 4 * off, db.ptr + 4 * off, do.ptr + 4 * off
+    ctx.unary_raw(D.GELU, po, pa, n)
+    assert_bits_equal(ctx.download(do, (n,), offset_bytes=4 * off), oracle.unary(oracle.GELU, a[off:]), "Gelu")
+    ctx.binary_raw(D.ADD, po, pa, pb, [n], [1], [1])
+    assert_bits_equal(ctx.download(do, (n,), offset_bytes=4 * off), a[off:] + b[off:], "Add")
+    ctx.binary_raw(D.MUL, po, pa, ds.ptr, [n], [1], [0])
+    assert_bits_equal(ctx.download(do, (n,), offset_bytes=4 * off), a[off:] * np.float32(1.7), "Mul by a scalar")
+    ctx.binary_raw(D.SUB, po, ds.ptr, pb, [n], [0], [1])
+    assert_bits_equal(ctx.download(do, (n,), offset_bytes=4 * off), np.float32(1.7) - b[off:], "Sub from a scalar")
+    for t in (da, db, do, ds):
+        ctx.free(t)
+
+
 UNALIGNED_ROWS = [(7, 768), (5, 197), (3, 1280), (2, 4096), (2, 8192), (3, 1000), (9, 64)]
 
 
