@@ -128,12 +128,15 @@ __global__ __launch_bounds__(BLOCK) void transpose_tiled(T *__restrict__ out, co
     }
     const uint32_t c0 = blockIdx.x * TILE, r0 = blockIdx.y * TILE;
     const uint32_t tx = threadIdx.x & (TILE - 1), ty = threadIdx.x / TILE;  // 64 x 4
-    // read: lane tx walks C, ty (+4k) walks R
-#pragma unroll 4
+    // read: lane tx walks C, ty (+4k) walks R; all sixteen loads are requested before the first goes to LDS
+    T v[TILE / (BLOCK / TILE)];
+#pragma unroll
     for (int k = 0; k < TILE; k += BLOCK / TILE) {
         const uint32_t r = r0 + ty + k, c = c0 + tx;
-        if (r < g.r_len && c < g.c_len) tile[ty + k][tx] = in[src0 + r * g.r_in_str + c];
+        if (r < g.r_len && c < g.c_len) v[k / (BLOCK / TILE)] = in[src0 + r * g.r_in_str + c];
     }
+#pragma unroll
+    for (int k = 0; k < TILE; k += BLOCK / TILE) tile[ty + k][tx] = v[k / (BLOCK / TILE)];
     __syncthreads();
     // write: lane tx walks R, ty (+4k) walks C
 #pragma unroll 4
