@@ -212,21 +212,36 @@ __global__ __launch_bounds__(TB) void transpose_small(T *__restrict__ out, const
     const uint32_t n = r_len * c_len;
     const T *src = in + (size_t)blockIdx.x * n;
     T *dst = out + (size_t)blockIdx.x * n;
-    for (uint32_t i = threadIdx.x * VEC; i < n; i += TB * VEC) {
-        T v[VEC];
-        if (VEC == 4) {
-            const u32x4 t = NT ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + i)) : *reinterpret_cast<const u32x4 *>(src + i);
-            v[0] = (T)t.x; v[1 % VEC] = (T)t.y; v[2 % VEC] = (T)t.z; v[3 % VEC] = (T)t.w;
-        } else {
-            v[0] = src[i];
-        }
-        uint32_t r = cdiv.div(i), c = i - r * c_len;  // input is [r][c]
+    // Four loads per thread are requested before the first is scattered into LDS (the trip count is not known at
+    // compile time, so the loop would otherwise wait for every load in turn).
+    constexpr int U = 4;
+    for (uint32_t i0 = threadIdx.x * VEC; i0 < n; i0 += U * TB * VEC) {
+        T v[U][VEC];
 #pragma unroll
-        for (int k = 0; k < VEC; k++) {
-            lds[c * pitch + r] = v[k];
-            if (++c == c_len) {
-                c = 0;
-                r++;
+        for (int u = 0; u < U; u++) {
+            const uint32_t i = i0 + u * TB * VEC;
+            if (i < n) {
+                if (VEC == 4) {
+                    const u32x4 t = NT ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + i)) : *reinterpret_cast<const u32x4 *>(src + i);
+                    v[u][0] = (T)t.x; v[u][1 % VEC] = (T)t.y; v[u][2 % VEC] = (T)t.z; v[u][3 % VEC] = (T)t.w;
+                } else {
+                    v[u][0] = src[i];
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t i = i0 + u * TB * VEC;
+            if (i < n) {
+                uint32_t r = cdiv.div(i), c = i - r * c_len;  // input is [r][c]
+#pragma unroll
+                for (int k = 0; k < VEC; k++) {
+                    lds[c * pitch + r] = v[u][k];
+                    if (++c == c_len) {
+                        c = 0;
+                        r++;
+                    }
+                }
             }
         }
     }
