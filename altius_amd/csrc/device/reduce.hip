@@ -354,8 +354,15 @@ __global__ __launch_bounds__(SS_BLOCK) void reduce_small_slabs(float *__restrict
     const uint32_t n_slabs = outer - o0 < group ? (uint32_t)(outer - o0) : group;
     const uint32_t floats = n_slabs * slab, n4 = floats >> 2;
     const float *src = in + o0 * slab;
-#pragma unroll 4
-    for (uint32_t i = threadIdx.x; i < n4; i += SS_BLOCK) reinterpret_cast<float4 *>(ss_lds)[i] = load4<NT>(src + 4 * (size_t)i);
+    for (uint32_t i0 = threadIdx.x; i0 < n4; i0 += 4 * SS_BLOCK) {  // four loads requested before the first goes to LDS
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (i0 + u * SS_BLOCK < n4) v[u] = load4<NT>(src + 4 * (size_t)(i0 + u * SS_BLOCK));
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (i0 + u * SS_BLOCK < n4) reinterpret_cast<float4 *>(ss_lds)[i0 + u * SS_BLOCK] = v[u];
+    }
     for (uint32_t i = (n4 << 2) + threadIdx.x; i < floats; i += SS_BLOCK) ss_lds[i] = src[i];  // the tensor's ragged end
     __syncthreads();
     const uint32_t outs = n_slabs * inner;
