@@ -17,7 +17,8 @@ slower).  Per-kernel times are measured with HIP events on the stream the kernel
 median and minimum over at least 100 launches after a warm-up of 20 launches and at least 25 ms,
 and once more inside the running step); `roofline` describes the slowest kernel of the step.  Beside the
 step the line carries every other operator of the path on the step's [256,197,768] array
-(`listed_ops`), Softmax / LayerNormalization / ReduceMean by row length (`row_sweep`) and the
+(`listed_ops`), Softmax / LayerNormalization / ReduceMean by row length (`row_sweep`), the same operators on
+shapes away from the configs' own (`shape_sweep`) and the
 kernels and graphs of configs[0..3] (`other_configs`).  The CPU baseline is the oracle (a C++
 restatement of the reference interpreter's kernels) timed on this machine's host cores on the same
 workload, with 16 threads and with 1, allocating its outputs per call as the reference does and
@@ -216,6 +217,45 @@ def run_row_sweep(ctx, D, args, lengths):
         log("  rows of %6d: %s" % (length, "   ".join("%s %6.1f us %5.1f %%" % (k, v["us"], v["pct_hbm_peak"])
                                                         for k, v in entry.items() if k != "row_length")))
     return sweep
+
+
+SHAPE_SWEEP_ELEMS = 96 << 20
+
+
+def build_shape_sweep(ctx, D, elems=SHAPE_SWEEP_ELEMS):
+    """The listed operators on shapes away from the configs' own: reductions over a middle axis, rows that are not whole
+    float4s (lengths above 1024, a vocabulary), a broadcast vector of three values, transposes that change the
+    innermost axis.  One ~400 MB input, cut to each shape."""
+    from altius_amd._lib import check, i64_array
+    rng = np.random.default_rng(22)
+    d_in = ctx.upload(rng.standard_normal(elems, dtype=np.float32))
+    d_out = ctx.alloc(elems * 4)
+    d_g = ctx.upload((1.0 + 0.02 * rng.standard_normal(65536)).astype(np.float32))
+    d_b = ctx.upload((0.02 * rng.standard_normal(65536)).astype(np.float32))
+    ops = []
+    for red, inner in ((197, 768), (49, 1024), (12, 4096), (1024, 8), (2, 65536), (196, 3), (7, 7)):
+        outer = elems // (red * inner)
+        for kind, name in ((D.REDUCE_MEAN, "ReduceMean"), (D.REDUCE_MAX, "ReduceMax")):
+            ops.append(Op("%s(axis=1) [%d,%d,%d]" % (name, outer, red, inner), (outer * red * inner + outer * inner) * 4,
+                          [lambda k=kind, o=outer, r=red, i=inner: ctx.reduce_raw(k, d_out.ptr, d_in.ptr, o, r, i)]))
+    for length in (1025, 2049, 5001, 9999, 50257):
+        rows = elems // length
+        n = rows * length
+        ops.append(Op("Softmax(-1) [%d,%d]" % (rows, length), 2 * n * 4, [lambda r=rows, l=length: ctx.softmax_raw(d_out.ptr, d_in.ptr, r, l)]))
+        ops.append(Op("LayerNormalization(-1) [%d,%d]" % (rows, length), 2 * n * 4 + 2 * length * 4,
+                      [lambda r=rows, l=length: ctx.layernorm_raw(d_out.ptr, d_in.ptr, d_g.ptr, d_b.ptr, r, l, 1e-5)]))
+        ops.append(Op("ReduceMean(-1) [%d,%d]" % (rows, length), (n + rows) * 4, [lambda r=rows, l=length: ctx.reduce_raw(D.REDUCE_MEAN, d_out.ptr, d_in.ptr, r, l, 1)]))
+    rgb = [4096, 4096, 3]
+    ops.append(Op("Sub [4096,4096,3] - [3]", (2 * 4096 * 4096 * 3 + 3) * 4,
+                  [lambda: ctx.binary_raw(D.SUB, d_out.ptr, d_in.ptr, d_g.ptr, rgb, D.strides_for_broadcasting(rgb, rgb), D.strides_for_broadcasting([3], rgb))]))
+    for shape, perm in (([64, 256, 56, 56], [0, 2, 3, 1]), ([8192, 8192], [1, 0]), ([256, 197, 768], [0, 2, 1]), ([50257, 768], [1, 0])):
+        n = int(np.prod(shape))
+        ops.append(Op("Transpose %s -> %s" % (shape, tuple(perm)), 2 * n * 4,
+                      [lambda sh=shape, pm=perm: check(ctx.L.ahip_transpose(ctx.handle, d_out.ptr, d_in.ptr, 4, len(sh), i64_array(sh), i64_array(pm)), ctx.handle)]))
+    for o in ops:
+        yield o
+    for b in (d_in, d_out, d_g, d_b):
+        ctx.free(b)
 
 
 def build_other_configs(ctx, D, synth, rotate_bytes=600e6, max_sets=48):
@@ -857,6 +897,14 @@ def main():
 
     if not args.only and not args.no_row_sweep:
         result["row_sweep"] = run_row_sweep(ctx, D, args, sweep_lengths)
+        shapes = []
+        log("the same operators on other shapes (a middle axis, rows that are not whole float4s, innermost-axis transposes):")
+        for o in build_shape_sweep(ctx, D):
+            t = time_kernel(ctx, o, min(args.kernel_iters, 40), min(args.kernel_warmup, 10), args.kernel_settle_ms)
+            r = dict({"kernel": o.name, "bytes": o.nbytes}, **t.row(o.nbytes))
+            shapes.append(r)
+            log("%-52s %14d %9.1f us %8.1f GB/s %6.1f %%" % (o.name, o.nbytes, r["us"], r["GBps"], r["pct_hbm_peak"]))
+        result["shape_sweep"] = shapes
 
     if not args.only and not args.no_other_configs:
         others = []
