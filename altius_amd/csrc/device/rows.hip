@@ -21,6 +21,8 @@
 
 #include <math.h>
 
+#include <type_traits>
+
 namespace altius {
 namespace {
 
@@ -713,7 +715,11 @@ __global__ __launch_bounds__(THREADS) void softmax_block_regs(float *__restrict_
     const float *x = in + (size_t)blockIdx.x * len;
     float *o = out + (size_t)blockIdx.x * len;
     const float nan = __builtin_nanf("");
-    const ptrdiff_t m = SHIFT ? (ptrdiff_t)((reinterpret_cast<uintptr_t>(x) >> 2) & 3) : 0, n = (ptrdiff_t)len;
+    // Element indices inside a row (at most 65536 elements): 32-bit from four float4 per thread on -- with 64-bit ones
+    // the SHIFT build of twelve and sixteen spills, and from four on it is 3 to 13 points of the HBM peak slower;
+    // below that the 64-bit ones, which the compiler folds into the addresses, are 5 points ahead.
+    using idx_t = std::conditional_t<(NCH >= 4), int, ptrdiff_t>;
+    const idx_t m = SHIFT ? (idx_t)((reinterpret_cast<uintptr_t>(x) >> 2) & 3) : 0, n = (idx_t)len;
     float4 r[NCH];
     float mx = nan;  // NaN elements (and the slots past the row) are ignored by the maximum
     // At most two 16-byte loads per thread are requested at a time; with four chunks the second pair goes out
@@ -723,7 +729,7 @@ __global__ __launch_bounds__(THREADS) void softmax_block_regs(float *__restrict_
     for (int k0 = 0; k0 < NCH; k0 += BURST) {
 #pragma unroll
         for (int k = k0; k < k0 + BURST; k++) {
-            const ptrdiff_t e = ((ptrdiff_t)threadIdx.x + (ptrdiff_t)THREADS * k) * 4 - m;
+            const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4 - m;
             if (!SHIFT) {
                 r[k] = e < n ? load4<NT>(x + e) : make_float4(nan, nan, nan, nan);
             } else if (e >= 0 && e + 4 <= n) {
@@ -743,7 +749,7 @@ __global__ __launch_bounds__(THREADS) void softmax_block_regs(float *__restrict_
     float sum = 0.0f;
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        const ptrdiff_t e = ((ptrdiff_t)threadIdx.x + (ptrdiff_t)THREADS * k) * 4 - m;
+        const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4 - m;
         r[k].x = softmax_exp(r[k].x, mx), r[k].y = softmax_exp(r[k].y, mx), r[k].z = softmax_exp(r[k].z, mx), r[k].w = softmax_exp(r[k].w, mx);
         if (!SHIFT) {
             if (e < n) sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
@@ -758,7 +764,7 @@ __global__ __launch_bounds__(THREADS) void softmax_block_regs(float *__restrict_
     const float recip = 1.0f / sum;
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        const ptrdiff_t e = ((ptrdiff_t)threadIdx.x + (ptrdiff_t)THREADS * k) * 4 - m;
+        const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4 - m;
         if (!SHIFT) {
             if (e < n) store4<NT>(o + e, make_float4(r[k].x * recip, r[k].y * recip, r[k].z * recip, r[k].w * recip));
         } else if (e >= 0 && e + 4 <= n) {
@@ -838,14 +844,15 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_shift(float *__restri
     __shared__ float lds[THREADS / WAVE];
     const float *x = in + (size_t)blockIdx.x * len;
     float *o = out + (size_t)blockIdx.x * len;
-    const ptrdiff_t m = (ptrdiff_t)((reinterpret_cast<uintptr_t>(x) >> 2) & 3), n = (ptrdiff_t)len;
+    using idx_t = std::conditional_t<(NCH > 8), int, ptrdiff_t>;  // see softmax_block_regs; here 64-bit indices are ahead up to eight float4 per thread
+    const idx_t m = (idx_t)((reinterpret_cast<uintptr_t>(x) >> 2) & 3), n = (idx_t)len;
     const bool gb4 = m == 0 && ((reinterpret_cast<uintptr_t>(gamma) | reinterpret_cast<uintptr_t>(beta)) & 15u) == 0;
     const float inv_n = 1.0f / (float)len;
     float4 r[NCH];
     float sum = 0.0f;
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        const ptrdiff_t e = ((ptrdiff_t)threadIdx.x + (ptrdiff_t)THREADS * k) * 4 - m;
+        const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4 - m;
         if (e >= 0 && e + 4 <= n) {
             r[k] = load4<NT>(x + e);
         } else {  // slots outside the row hold zero: they add nothing to the sum
@@ -860,7 +867,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_shift(float *__restri
     float ss = 0.0f;
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        const ptrdiff_t e = ((ptrdiff_t)threadIdx.x + (ptrdiff_t)THREADS * k) * 4 - m;
+        const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4 - m;
         r[k].x -= mean, r[k].y -= mean, r[k].z -= mean, r[k].w -= mean;
         if (e >= 0 && e + 4 <= n) {
             ss += (r[k].x * r[k].x + r[k].y * r[k].y) + (r[k].z * r[k].z + r[k].w * r[k].w);
@@ -873,7 +880,7 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_shift(float *__restri
     const float inv_std = 1.0f / sqrtf(__builtin_fmaf(ss, inv_n, eps));
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        const ptrdiff_t e = ((ptrdiff_t)threadIdx.x + (ptrdiff_t)THREADS * k) * 4 - m;
+        const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4 - m;
         if (e >= 0 && e + 4 <= n) {
             float4 g, b;
             if (gb4) {
@@ -1034,7 +1041,9 @@ struct BlockLayout {
 inline BlockLayout block_layout(size_t len) {
     const size_t v = len / 4;  // float4 per row
     const int threads = v <= 512 ? 256 : v <= 768 ? 384 : v <= 1024 ? 512 : v <= 1536 ? 768 : 1024;
-    return BlockLayout{threads, (int)((v + threads - 1) / threads)};
+    int nch = (int)((v + threads - 1) / threads);
+    if (nch > 4 && nch <= 16) nch = nch <= 6 ? 6 : nch <= 8 ? 8 : nch <= 12 ? 12 : 16;  // rows beyond 16 K: the layouts that exist
+    return BlockLayout{threads, nch};
 }
 
 // Blocks of 1024 threads and four float4 per thread (rows of more than 12288 elements) with more than two rows each to
@@ -1043,7 +1052,7 @@ inline BlockLayout block_layout(size_t len) {
 // float4 per thread the plain kernels are 2-5 points ahead of it.
 template <int THREADS, int NCH>
 void softmax_block_go(bool nt, hipStream_t s, size_t rows, size_t resident, float *out, const float *in, size_t len) {
-    if constexpr (THREADS == 1024 && NCH >= 4) if (rows > 2 * resident) {
+    if constexpr (THREADS == 1024 && NCH == 4) if (rows > 2 * resident) {
         const dim3 grid((unsigned)resident);
         if (nt) hipLaunchKernelGGL((softmax_block_pipe<THREADS, NCH, true>), grid, dim3(THREADS), 0, s, out, in, (uint32_t)len, rows);
         else hipLaunchKernelGGL((softmax_block_pipe<THREADS, NCH, false>), grid, dim3(THREADS), 0, s, out, in, (uint32_t)len, rows);
@@ -1069,7 +1078,7 @@ void layernorm_block_shift_go(bool nt, hipStream_t s, size_t rows, float *out, c
 template <int THREADS, int NCH>
 void layernorm_block_go(bool nt, hipStream_t s, size_t rows, size_t resident, float *out, const float *in, const float *gamma, const float *beta,
                         size_t len, float eps) {
-    if constexpr (THREADS == 1024 && NCH >= 4) if (rows > 2 * resident) {
+    if constexpr (THREADS == 1024 && NCH == 4) if (rows > 2 * resident) {
         const dim3 grid((unsigned)resident);
         if (nt) hipLaunchKernelGGL((layernorm_block_pipe<THREADS, NCH, true>), grid, dim3(THREADS), 0, s, out, in, gamma, beta, (uint32_t)len, rows, eps);
         else hipLaunchKernelGGL((layernorm_block_pipe<THREADS, NCH, false>), grid, dim3(THREADS), 0, s, out, in, gamma, beta, (uint32_t)len, rows, eps);
@@ -1083,6 +1092,7 @@ void layernorm_block_go(bool nt, hipStream_t s, size_t rows, size_t resident, fl
 #define ALTIUS_BLOCK_LAYOUTS(L)                                                          \
     switch ((L).threads * 100 + (L).nch) {                                               \
         ALTIUS_GO(256, 2) ALTIUS_GO(384, 2) ALTIUS_GO(512, 2) ALTIUS_GO(768, 2) ALTIUS_GO(1024, 2) ALTIUS_GO(1024, 3) ALTIUS_GO(1024, 4) \
+        ALTIUS_GO(1024, 6) ALTIUS_GO(1024, 8) ALTIUS_GO(1024, 12) ALTIUS_GO(1024, 16)                                                      \
     }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -1332,7 +1342,7 @@ inline bool wave_row_fits(size_t len) {
 
 constexpr size_t MAX_WAVE_ROW = 1024;
 constexpr size_t MAX_LONG_ROW = 1280;  // rows kept in a wavefront's registers when they are whole float4s (at 1536 a block per row is 2 points ahead)
-constexpr size_t MAX_BLOCK_REG_ROW = 16384;  // ... and in a block's registers
+constexpr size_t MAX_BLOCK_REG_ROW = 65536;  // ... and in a block's registers
 constexpr size_t MAX_GRID = 0x7FFFFFFFu;
 
 }  // namespace

@@ -269,7 +269,8 @@ SOFTMAX_SHAPES = [[1, 2, 3], [3, 28, 28], [16, 512, 512], [2, 12, 197, 197], [5,
                   [2, 5120], [3, 8192], [2, 8196], [2, 16384], [1, 12000], [2, 16388], [2, 5001],  # up to 16384: in a block's registers
                   [3, 1284], [3, 2052], [2, 3076], [2, 4608], [2, 6144], [2, 6148], [2, 12288],  # either side of every block width
                   [5, 384], [7, 640], [6, 896], [3, 1088], [9, 1152], [13, 320],  # a wavefront per row, last chunk partly filled
-                  [7, 1030], [5, 2049], [3, 4097], [3, 9999], [2, 16381], [2, 16383], [2, 50257]]  # rows that start anywhere: the aligned cover in registers to 16381, three passes above
+                  [7, 1030], [5, 2049], [3, 4097], [3, 9999], [2, 16381], [2, 16383], [2, 50257],  # rows that start anywhere: the aligned cover of a row in registers
+                  [2, 20000], [2, 32768], [1, 49152], [2, 65536], [2, 30522], [1, 65533], [1, 65540]]  # 6 to 16 float4 per thread up to 65536 elements, three passes above
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
@@ -310,7 +311,8 @@ LN_SHAPES = [[1, 20, 10], [2, 197, 768], [3, 5, 197], [4, 1], [5, 64], [3, 1024]
              [2, 5120], [3, 8192], [2, 8196], [2, 16384], [1, 12000], [2, 16388], [2, 5001],  # rows up to 16384 in a block's registers
              [3, 1284], [3, 2052], [2, 3076], [2, 4608], [2, 6144], [2, 6148], [2, 12288],  # either side of every block width
              [5, 384], [7, 640], [6, 896], [3, 1088], [9, 1152], [1, 512], [13, 320],  # a wavefront per row, last chunk partly filled, rows not a multiple of the block's four
-             [7, 1030], [5, 2049], [3, 4097], [3, 9999], [2, 16383], [2, 50257]]  # three passes with float4 bodies, rows that start anywhere
+             [7, 1030], [5, 2049], [3, 4097], [3, 9999], [2, 16383], [2, 50257],  # rows that start anywhere: the aligned cover of a row in registers
+             [2, 20000], [2, 32768], [1, 49152], [2, 65536], [2, 30522], [1, 65533], [1, 65540]]  # 6 to 16 float4 per thread up to 65536 elements, three passes above
 
 
 @pytest.mark.parametrize("shape", LN_SHAPES)
