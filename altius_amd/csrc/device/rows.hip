@@ -4,8 +4,15 @@
 // registers (read once, written once), max / sum reductions as lane butterflies.
 // Lane l owns elements (l + 64*k)*VEC .. +VEC-1, so every load instruction of
 // the wave covers one contiguous 256-byte (VEC=1) or 1-KiB (VEC=4) span.
-// Longer rows: one 256-thread block per row, streaming the row from memory
-// (L2-resident after the first pass) with LDS-staged block reductions.
+// Rows that are not whole 128-byte lines, and short rows: groups of rows staged
+// through LDS, a few lanes per row.
+// Rows of up to 65536 elements: one block of 256 to 1024 threads per row, the row
+// in the block's registers (2 to 16 float4 per thread), the two reductions
+// through LDS; rows that do not start on 16-byte boundaries are held as the
+// aligned float4s that cover them.
+// Longer rows, and input and output that are differently aligned: one block per
+// row walking it three times (from the caches after the first pass), single
+// elements up to the first 16-byte boundary and float4s from there.
 //
 // Reference arithmetic:
 //   Softmax  crates/session_interpreter/src/session.rs:990-1026,
