@@ -25,6 +25,18 @@ template <bool NT> __device__ __forceinline__ float4 load4(const float *p) {
     }
     return *reinterpret_cast<const float4 *>(p);
 }
+// The same for addresses that are only 4-byte aligned: the part's 16-byte global accesses need no more than that, and
+// the compiler emits them for a vector type declared with that alignment.
+typedef float v4f_dword __attribute__((ext_vector_type(4), aligned(4)));
+template <bool NT> __device__ __forceinline__ float4 load4_dword_aligned(const float *p) {
+    const v4f_dword t = NT ? __builtin_nontemporal_load(reinterpret_cast<const v4f_dword *>(p)) : *reinterpret_cast<const v4f_dword *>(p);
+    return make_float4(t.x, t.y, t.z, t.w);
+}
+template <bool NT> __device__ __forceinline__ void store4_dword_aligned(float *p, const float4 &v) {
+    const v4f_dword t = {v.x, v.y, v.z, v.w};
+    if (NT) __builtin_nontemporal_store(t, reinterpret_cast<v4f_dword *>(p));
+    else *reinterpret_cast<v4f_dword *>(p) = t;
+}
 template <bool NT> __device__ __forceinline__ void store4(float *p, const float4 &v) {
     if (NT) {
         v4f t;

@@ -72,6 +72,21 @@ __global__ __launch_bounds__(BLOCK) void unary_vec4(float *__restrict__ out, con
     }
 }
 
+// Tensors on 4-byte boundaries only: the same four elements per lane through 16-byte accesses that are not aligned.
+template <class F, bool NT>
+__global__ __launch_bounds__(BLOCK) void unary_vec4_any(float *__restrict__ out, const float *__restrict__ in, size_t n, F f) {
+    const size_t i = (size_t)blockIdx.x * BLOCK + threadIdx.x;
+    const size_t n4 = n >> 2;
+    if (i < n4) {
+        const float4 v = load4_dword_aligned<NT>(in + 4 * i);
+        store4_dword_aligned<NT>(out + 4 * i, make_float4(f(v.x), f(v.y), f(v.z), f(v.w)));
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const size_t j = (n4 << 2) + threadIdx.x;
+        out[j] = f(in[j]);
+    }
+}
+
 template <class F>
 __global__ __launch_bounds__(BLOCK) void unary_scalar(float *__restrict__ out, const float *__restrict__ in,
                                                       size_t n, F f) {
@@ -99,6 +114,10 @@ template <class F> void launch(hipStream_t s, float *out, const float *in, size_
             hipLaunchKernelGGL((unary_vec4<F, false, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, n, f);
         else
             hipLaunchKernelGGL((unary_vec4<F, false>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, n, f);
+    } else if (n >= 4 * BLOCK && ((off_in | off_out) & 3u) == 0) {
+        const size_t blocks = ((n >> 2) + BLOCK - 1) / BLOCK;
+        if (nt) hipLaunchKernelGGL((unary_vec4_any<F, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, n, f);
+        else hipLaunchKernelGGL((unary_vec4_any<F, false>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, in, n, f);
     } else {
         hipLaunchKernelGGL((unary_scalar<F>), dim3((unsigned)((n + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, s,
                            out, in, n, f);
