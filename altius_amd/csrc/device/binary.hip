@@ -69,7 +69,27 @@ __global__ __launch_bounds__(BLOCK) void binary_flat_vec4(float *__restrict__ ou
     }
 }
 
-// Same, one element per lane, for buffers that are not 16-byte aligned.
+// The same on tensors that lie on 4-byte boundaries only: this part's 16-byte global accesses need no more.
+template <class OP, int MA, int MB, bool NT>
+__global__ __launch_bounds__(BLOCK) void binary_flat_vec4_any(float *__restrict__ out, const float *__restrict__ a,
+                                                              const float *__restrict__ b, size_t n) {
+    const size_t n4 = n >> 2;
+    const size_t i = (size_t)blockIdx.x * BLOCK + threadIdx.x;
+    float sa = 0.f, sb = 0.f;
+    if (MA == SCALAR) sa = a[0];
+    if (MB == SCALAR) sb = b[0];
+    if (i < n4) {
+        const float4 x = MA == FULL ? load4_dword_aligned<NT>(a + 4 * i) : make_float4(sa, sa, sa, sa);
+        const float4 y = MB == FULL ? load4_dword_aligned<NT>(b + 4 * i) : make_float4(sb, sb, sb, sb);
+        store4_dword_aligned<NT>(out + 4 * i, make_float4(OP::f(x.x, y.x), OP::f(x.y, y.y), OP::f(x.z, y.z), OP::f(x.w, y.w)));
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const size_t j = (n4 << 2) + threadIdx.x;
+        out[j] = OP::f(MA == FULL ? a[j] : sa, MB == FULL ? b[j] : sb);
+    }
+}
+
+// Same, one element per lane, for the smallest tensors that are not 16-byte aligned.
 template <class OP, int MA, int MB>
 __global__ __launch_bounds__(BLOCK) void binary_flat_scalar(float *__restrict__ out,
                                                             const float *__restrict__ a,
@@ -399,6 +419,10 @@ void flat_dispatch(hipStream_t s, float *out, const float *a, const float *b, si
         else
             hipLaunchKernelGGL((binary_flat_vec4<OP, MA, MB, false>), dim3((unsigned)blocks), dim3(BLOCK), 0, s,
                                out, a, b, n);
+    } else if (n >= 4 * BLOCK) {
+        const size_t blocks = ((n >> 2) + BLOCK - 1) / BLOCK;
+        if (nt) hipLaunchKernelGGL((binary_flat_vec4_any<OP, MA, MB, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, a, b, n);
+        else hipLaunchKernelGGL((binary_flat_vec4_any<OP, MA, MB, false>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, a, b, n);
     } else {
         const size_t blocks = (n + BLOCK - 1) / BLOCK;
         hipLaunchKernelGGL((binary_flat_scalar<OP, MA, MB>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, a,
@@ -577,17 +601,6 @@ int launch_binary(DeviceCtx &ctx, int op, float *out, const float *a, const floa
     const bool nt = ctx.streaming(total * sizeof(float)), ntl = ctx.streaming_loads(total * sizeof(float));
     if (ma != STRIDED && mb != STRIDED) {
         const bool vec = aligned16(out) && (ma != FULL || aligned16(a)) && (mb != FULL || aligned16(b));
-        // Every dense tensor equally far past a 16-byte boundary (views into the middle of buffers), and large enough
-        // for a second launch not to matter: the one to three elements up to the boundary on their own, the rest as float4s.
-        const uintptr_t off = reinterpret_cast<uintptr_t>(out) & 15u;
-        auto same_off = [&](int mode, const float *p) { return mode != FULL || (reinterpret_cast<uintptr_t>(p) & 15u) == off; };
-        if (!vec && off != 0 && off % 4 == 0 && same_off(ma, a) && same_off(mb, b) && total >= ((size_t)1 << 16)) {
-            const size_t head = (16 - off) / 4;
-            const int64_t head_dims[1] = {(int64_t)head}, rest_dims[1] = {(int64_t)(total - head)};
-            const int64_t sa[1] = {ma == FULL ? 1 : 0}, sb[1] = {mb == FULL ? 1 : 0};
-            if (int rc = launch_binary(ctx, op, out, a, b, 1, head_dims, sa, sb)) return rc;
-            return launch_binary(ctx, op, out + head, ma == FULL ? a + head : a, mb == FULL ? b + head : b, 1, rest_dims, sa, sb);
-        }
         switch (op) {
         case AHIP_ADD: flat_launch<OpAdd>(s, ma, mb, out, a, b, total, vec, nt, ntl); break;
         case AHIP_SUB: flat_launch<OpSub>(s, ma, mb, out, a, b, total, vec, nt, ntl); break;

@@ -96,14 +96,6 @@ __global__ __launch_bounds__(BLOCK) void unary_scalar(float *__restrict__ out, c
 
 template <class F> void launch(hipStream_t s, float *out, const float *in, size_t n, F f, bool nt, bool ntl) {
     const uintptr_t off_in = reinterpret_cast<uintptr_t>(in) & 15u, off_out = reinterpret_cast<uintptr_t>(out) & 15u;
-    // Both tensors equally far past a 16-byte boundary (a view into the middle of a buffer), and large enough for a
-    // second launch not to matter: the one to three elements up to the boundary on their own, the rest as float4s.
-    if (off_in != 0 && off_in == off_out && off_in % 4 == 0 && n >= ((size_t)1 << 16)) {
-        const size_t head = (16 - off_in) / 4;
-        hipLaunchKernelGGL((unary_scalar<F>), dim3(1), dim3(BLOCK), 0, s, out, in, head, f);
-        launch(s, out + head, in + head, n - head, f, nt, ntl);
-        return;
-    }
     const bool vec = (off_in | off_out) == 0;
     if (vec) {
         size_t blocks = ((n >> 2) + BLOCK - 1) / BLOCK;

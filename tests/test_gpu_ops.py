@@ -332,8 +332,8 @@ def test_layernorm(ctx, oracle, case, shape):
 
 @pytest.mark.parametrize("off", [1, 2, 3])
 def test_flat_operators_on_large_views_that_start_off_a_boundary(ctx, oracle, case, off):
-    """Every tensor `off` floats past a 16-byte boundary and large enough for two launches: the elements up to the
-    boundary go on their own and the rest as float4s; not a bit may differ from the aligned call."""
+    """Every tensor `off` floats past a 16-byte boundary: four elements per lane through 16-byte accesses that are only
+    4-byte aligned; not a bit may differ from the aligned call."""
     case(f"Gelu / Add / Mul by a scalar / Sub from a scalar on 70001 elements, every tensor +{off} floats")
     n = 70001
     a, b = synth.normal(81, (n + off,)), synth.normal(82, (n + off,), mean=2.0)
