@@ -24,7 +24,9 @@ restatement of the reference interpreter's kernels) timed on this machine's host
 workload, with 16 threads and with 1, allocating its outputs per call as the reference does and
 writing into existing ones.
 
-Prints one JSON line on stdout; the tables go to stderr.
+Prints one JSON line of less than 6000 characters on stdout, last: the headline, `roofline` and `cpu_baseline` in full and
+every table as rows of numbers under a `cols` legend.  stderr carries one short line per section; --verbose prints the
+tables there, --full-json PATH writes every figure to a file.
 """
 import argparse
 import json
@@ -40,8 +42,85 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 
 
+VERBOSE = False
+
+
 def log(*a):
+    """The wide tables: stderr, only with --verbose."""
+    if VERBOSE:
+        print(*a, file=sys.stderr, flush=True)
+
+
+def note(*a):
+    """One short progress line per section: stderr, always (a few hundred characters over the whole run)."""
     print(*a, file=sys.stderr, flush=True)
+
+
+LINE_LIMIT = 6000  # the JSON line on stdout stays below this many characters
+
+
+def _strip(name):
+    return name.replace(", ", ",").replace(" -> ", ">").replace(" ", "")
+
+
+def compact_line(result, limit=LINE_LIMIT):
+    """The one line for stdout: the headline fields, `config`, `roofline` and `cpu_baseline` in full, and every table
+    of the run as rows of numbers under a `cols` legend (us = mean HIP-event time per launch, pct = algorithmic bytes
+    / us as a percentage of 8 TB/s).  Tables are dropped, last first, if the line would pass `limit`, and named
+    under `dropped`; the full record goes to the file --full-json names."""
+    head = ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline",
+            "dtype", "data", "config", "value_after_idle", "ms_per_step_after_idle", "settle_ms")
+    line = {k: result[k] for k in head if k in result}
+    if "roofline" in result:
+        line["roofline"] = result["roofline"]
+    if "cpu_baseline" in result:
+        keep = ("value", "unit", "cores", "kind", "sample", "single_thread_value", "value_existing_outputs",
+                "single_thread_value_existing_outputs", "us_per_kernel_scaled", "us_per_kernel_scaled_1_thread")
+        line["cpu_baseline"] = {k: v for k, v in result["cpu_baseline"].items() if k in keep}
+    tables = []
+    if result.get("per_kernel"):
+        tables.append(("per_kernel", {"cols": ["kernel", "bytes", "us", "us_median", "pct", "us_in_step"],
+                                      "rows": [[_strip(r["kernel"]), r["bytes"], r["us"], r["us_median"], r["pct_hbm_peak"], r.get("us_interleaved")]
+                                               for r in result["per_kernel"]]}))
+    if result.get("listed_ops"):
+        tables.append(("listed_ops", {"cols": ["kernel", "us", "pct"],
+                                      "rows": [[_strip(r["kernel"]), r["us"], r["pct_hbm_peak"]] for r in result["listed_ops"]]}))
+    if result.get("other_configs"):
+        oc = result["other_configs"]
+        tables.append(("other_configs", {
+            "cols": ["kernel", "us", "pct", "cpu_us_16_threads", "cpu_us_1_thread"],
+            "rows": [[_strip(r["kernel"]), r["us"], r["pct_hbm_peak"], r.get("cpu_us_16_threads"), r.get("cpu_us_1_thread")] for r in oc["kernels"]],
+            "graph_cols": ["graph", "kernels_us", "kernels_us_graph_replay", "run_device_us", "run_ms_with_pcie"],
+            "graphs": [[r["graph"], r["kernels_us"], r["kernels_us_graph_replay"], r["run_device_us"], r["run_ms_with_pcie"]] for r in oc["graphs"]]}))
+    if result.get("row_sweep"):
+        names = [k for k in result["row_sweep"][0] if k != "row_length"]
+        tables.append(("row_sweep", {"cols": ["row_length"] + [n + "_pct" for n in names],
+                                     "rows": [[e["row_length"]] + [e[n]["pct_hbm_peak"] for n in names] for e in result["row_sweep"]]}))
+    if result.get("shape_sweep"):
+        # operators that share a shape share a row: [shape, pct of each operator of the group]
+        groups = {}
+        for r in result["shape_sweep"]:
+            op, _, shape = r["kernel"].partition(" ")
+            g = groups.setdefault("Transpose" if op == "Transpose" else "middle_axis" if "axis=1" in op else "odd_rows" if "(-1)" in op else "other",
+                                  {"ops": [], "shapes": {}})
+            if op not in g["ops"]:
+                g["ops"].append(op)
+            g["shapes"].setdefault(_strip(shape), {})[op] = r["pct_hbm_peak"]
+        tables.append(("shape_sweep", {name: {"cols": ["shape"] + [o + "_pct" for o in g["ops"]],
+                                              "rows": [[sh] + [v.get(o) for o in g["ops"]] for sh, v in g["shapes"].items()]}
+                                       for name, g in groups.items()}))
+    for k in ("vit", "next_rows", "timeline", "calibration"):
+        if k in result:
+            tables.append((k, result[k]))
+    for name, t in tables:
+        line[name] = t
+    dropped = []
+    while len(json.dumps(line, separators=(",", ":"))) >= limit and tables:
+        name, _ = tables.pop()
+        del line[name]
+        dropped.append(name)
+        line["dropped"] = dropped
+    return json.dumps(line, separators=(",", ":"))
 
 
 def ensure_built():
@@ -50,7 +129,7 @@ def ensure_built():
     if not os.path.exists(_lib.LIB_PATH):
         from altius_amd import build
 
-        log("libaltius_hip.so missing: building")
+        note("libaltius_hip.so missing: building")
         build.build()
 
 
@@ -220,6 +299,9 @@ def run_row_sweep(ctx, D, args, lengths):
 
 
 SHAPE_SWEEP_ELEMS = 96 << 20
+SHAPE_SWEEP_MIDDLE = ((197, 768), (49, 1024), (12, 4096), (1024, 8), (2, 65536), (196, 3), (7, 7))   # (reduced, inner) extents
+SHAPE_SWEEP_ODD_ROWS = (1025, 2049, 5001, 9999, 50257)
+SHAPE_SWEEP_TRANSPOSES = (([64, 256, 56, 56], [0, 2, 3, 1]), ([8192, 8192], [1, 0]), ([256, 197, 768], [0, 2, 1]), ([50257, 768], [1, 0]))
 
 
 def build_shape_sweep(ctx, D, elems=SHAPE_SWEEP_ELEMS):
@@ -233,12 +315,12 @@ def build_shape_sweep(ctx, D, elems=SHAPE_SWEEP_ELEMS):
     d_g = ctx.upload((1.0 + 0.02 * rng.standard_normal(65536)).astype(np.float32))
     d_b = ctx.upload((0.02 * rng.standard_normal(65536)).astype(np.float32))
     ops = []
-    for red, inner in ((197, 768), (49, 1024), (12, 4096), (1024, 8), (2, 65536), (196, 3), (7, 7)):
+    for red, inner in SHAPE_SWEEP_MIDDLE:
         outer = elems // (red * inner)
         for kind, name in ((D.REDUCE_MEAN, "ReduceMean"), (D.REDUCE_MAX, "ReduceMax")):
             ops.append(Op("%s(axis=1) [%d,%d,%d]" % (name, outer, red, inner), (outer * red * inner + outer * inner) * 4,
                           [lambda k=kind, o=outer, r=red, i=inner: ctx.reduce_raw(k, d_out.ptr, d_in.ptr, o, r, i)]))
-    for length in (1025, 2049, 5001, 9999, 50257):
+    for length in SHAPE_SWEEP_ODD_ROWS:
         rows = elems // length
         n = rows * length
         ops.append(Op("Softmax(-1) [%d,%d]" % (rows, length), 2 * n * 4, [lambda r=rows, l=length: ctx.softmax_raw(d_out.ptr, d_in.ptr, r, l)]))
@@ -248,7 +330,7 @@ def build_shape_sweep(ctx, D, elems=SHAPE_SWEEP_ELEMS):
     rgb = [4096, 4096, 3]
     ops.append(Op("Sub [4096,4096,3] - [3]", (2 * 4096 * 4096 * 3 + 3) * 4,
                   [lambda: ctx.binary_raw(D.SUB, d_out.ptr, d_in.ptr, d_g.ptr, rgb, D.strides_for_broadcasting(rgb, rgb), D.strides_for_broadcasting([3], rgb))]))
-    for shape, perm in (([64, 256, 56, 56], [0, 2, 3, 1]), ([8192, 8192], [1, 0]), ([256, 197, 768], [0, 2, 1]), ([50257, 768], [1, 0])):
+    for shape, perm in SHAPE_SWEEP_TRANSPOSES:
         n = int(np.prod(shape))
         ops.append(Op("Transpose %s -> %s" % (shape, tuple(perm)), 2 * n * 4,
                       [lambda sh=shape, pm=perm: check(ctx.L.ahip_transpose(ctx.handle, d_out.ptr, d_in.ptr, 4, len(sh), i64_array(sh), i64_array(pm)), ctx.handle)]))
@@ -747,10 +829,15 @@ def main():
     ap.add_argument("--vit", type=int, default=0, metavar="BATCH",
                     help="also run a ViT-B/16-shaped encoder (12 layers, exporter-style graph, random weights) at this batch: "
                          "device time per forward as exported, after the reference's rewrites, and after this backend's ('vit' in the JSON)")
+    ap.add_argument("--verbose", action="store_true", help="print the tables of every section on stderr (default: one short line per section)")
+    ap.add_argument("--full-json", type=str, default="", metavar="PATH",
+                    help="also write the full record (every figure of every table, as one JSON document) to this file")
     args = ap.parse_args()
+    global VERBOSE
+    VERBOSE = args.verbose
 
     if args.gpus != 1:
-        log("bench.py: this build runs on one GPU only (every operator on the path is independent along the batch "
+        note("bench.py: this build runs on one GPU only (every operator on the path is independent along the batch "
             "axis, so more GPUs would each run the same kernels on a slice of the batch, without communication); "
             "run with --gpus 1")
         sys.exit(2)
@@ -836,6 +923,8 @@ def main():
         log("%-44s %14d %9.1f %9.1f %9.1f %9.1f %8.1f %12s" % (r["kernel"], r["bytes"], r["us"], r["us_median"], r["us_min"], r["GBps"],
                                                             r["pct_hbm_peak"], "%.1f" % r["us_interleaved"] if "us_interleaved" in r else "-"))
     dom = max(rows[:len(ops)], key=lambda r: r["us"])
+    note("step %.4f ms, %.1f GB/s; per kernel: %s" % (step_s * 1e3, value, "; ".join(
+        "%s %.1f us %.1f %%" % (r["kernel"].split(" ")[0], r["us"], r["pct_hbm_peak"]) for r in rows)))
 
     result = {
         "metric": "per-op HBM GB/s and % of MI355X peak; us/call vs CPU interpreter",
@@ -867,8 +956,8 @@ def main():
             "unit": "GB/s",
             "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
             "traffic": measured_traffic(dom["kernel"]),
-            "traffic_source": TRAFFIC_FILE + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by a copy kernel of known "
-                              "size; a constant read from that file, not measured in this run)",
+            "traffic_source": TRAFFIC_FILE + ": rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command scaled by a copy kernel of known "
+                              "size; read from that file, not measured in this run",
             "us_per_launch": round(dom["us"], 2),
             "us_per_launch_median": dom["us_median"],
             "us_per_launch_min": dom["us_min"],
@@ -894,6 +983,7 @@ def main():
             listed.append(r)
             log("%-44s %14d %9.1f %9.1f %9.1f %9.1f %8.1f" % (o.name, o.nbytes, r["us"], r["us_median"], r["us_min"], r["GBps"], r["pct_hbm_peak"]))
         result["listed_ops"] = listed
+        note("listed_ops: %d kernels, %.1f to %.1f %% of 8 TB/s" % (len(listed), min(r["pct_hbm_peak"] for r in listed), max(r["pct_hbm_peak"] for r in listed)))
 
     if not args.only and not args.no_row_sweep:
         result["row_sweep"] = run_row_sweep(ctx, D, args, sweep_lengths)
@@ -905,6 +995,8 @@ def main():
             shapes.append(r)
             log("%-52s %14d %9.1f us %8.1f GB/s %6.1f %%" % (o.name, o.nbytes, r["us"], r["GBps"], r["pct_hbm_peak"]))
         result["shape_sweep"] = shapes
+        note("row_sweep: %d row lengths; shape_sweep: %d kernels, lowest %s" % (
+            len(result["row_sweep"]), len(shapes), ", ".join("%s %.1f %%" % (r["kernel"], r["pct_hbm_peak"]) for r in sorted(shapes, key=lambda r: r["pct_hbm_peak"])[:3])))
 
     if not args.only and not args.no_other_configs:
         others = []
@@ -931,6 +1023,7 @@ def main():
                 % (r["graph"], r["kernels_us"], r["kernels_us_graph_replay"], r["kernels_GBps"], r["run_device_us"],
                    r["run_ms_with_pcie"]))
         result["other_configs"] = {"kernels": others, "graphs": graphs_rows}
+        note("other_configs: %d kernels, %d graphs" % (len(others), len(graphs_rows)))
 
     if args.vit:
         vit_rows = vit_table(args.vit)
@@ -966,7 +1059,7 @@ def main():
         gbps_n, t_n, gbps_n_re, t_n_re = cpu_baseline(synth, args.batch, sample, threads, cfg4_arrays)
         gbps_1, t_1, gbps_1_re, t_1_re = cpu_baseline(synth, args.batch, sample, 1, cfg4_arrays)
         scale = args.batch / sample
-        log("CPU oracle, batch %d sample (x%.0f for the full step), fresh output per call as the reference allocates it: "
+        note("CPU oracle, batch %d sample (x%.0f for the full step), fresh output per call as the reference allocates it: "
             "%d threads %.2f GB/s, 1 thread %.2f GB/s; into existing outputs: %.2f and %.2f GB/s"
             % (sample, scale, threads, gbps_n, gbps_1, gbps_n_re, gbps_1_re))
         for k in t_n:
@@ -992,7 +1085,12 @@ def main():
         }
 
     ctx.close()
-    print(json.dumps(result), flush=True)
+    if args.full_json:
+        os.makedirs(os.path.dirname(os.path.abspath(args.full_json)), exist_ok=True)
+        with open(args.full_json, "w") as f:
+            json.dump(result, f)
+    sys.stderr.flush()
+    print(compact_line(result), flush=True)
 
 
 if __name__ == "__main__":
