@@ -6,10 +6,10 @@
 // the wave covers one contiguous 256-byte (VEC=1) or 1-KiB (VEC=4) span.
 // Rows that are not whole 128-byte lines, and short rows: groups of rows staged
 // through LDS, a few lanes per row.
-// Rows of up to 65536 elements: one block of 256 to 1024 threads per row, the row
-// in the block's registers (2 to 16 float4 per thread), the two reductions
-// through LDS; rows that do not start on 16-byte boundaries use 16-byte
-// accesses on 4-byte boundaries.
+// Rows of up to 65536 elements: one block of 192 to 1024 threads per row, the row
+// in the block's registers (2 to 20 float4 per thread), the two reductions
+// through LDS; rows that start anywhere are addressed as buffers from their
+// first 128-byte boundary on.
 // Longer rows: one block per row walking it three times (from the caches after
 // the first pass), single elements up to the first 16-byte boundary and float4s
 // from there.
@@ -711,21 +711,16 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_stream(float *__restr
 // thread, read once); the two reductions go through LDS.  Few loads per thread and many threads per row: on this
 // part a wavefront that issues many 16-byte loads back to back streams more slowly than many wavefronts issuing a
 // few each.
-// ANYWHERE: rows that do not start on 16-byte boundaries (a length that is not a multiple of 4, or a base pointer that
-// is not aligned).  The part's 16-byte global accesses need 4-byte alignment only, so a thread's float4s are read and
-// written where they lie (75 % of the HBM peak on rows of 5001 against 67 % with the aligned float4s that cover the row
-// and two edges handled apart, which this build did first); the row's last, partial float4 goes element by element.
-template <int THREADS, int NCH, bool NT, bool ANYWHERE = false>
+template <int THREADS, int NCH, bool NT>
 __global__ __launch_bounds__(THREADS) void softmax_block_regs(float *__restrict__ out, const float *__restrict__ in, size_t len) {
     __shared__ float lds[THREADS / WAVE];
     const float *x = in + (size_t)blockIdx.x * len;
     float *o = out + (size_t)blockIdx.x * len;
     const float nan = __builtin_nanf("");
-    // Element indices inside a row (at most 65536 elements): 32-bit from four float4 per thread on -- with 64-bit ones
-    // the ANYWHERE build of twelve and sixteen spills, and from four on it is 3 to 13 points of the HBM peak slower;
-    // below that the 64-bit ones, which the compiler folds into the addresses, are 5 points ahead.
+    // Element indices inside a row (at most 65536 elements): 32-bit from four float4 per thread on; below that the
+    // 64-bit ones, which the compiler folds into the addresses, are 5 points of the HBM peak ahead.
     using idx_t = std::conditional_t<(NCH >= 4), int, ptrdiff_t>;
-    const idx_t m = 0, n = (idx_t)len;
+    const idx_t n = (idx_t)len;
     float4 r[NCH];
     float mx = nan;  // NaN elements (and the slots past the row) are ignored by the maximum
     // At most two 16-byte loads per thread are requested at a time; with four chunks the second pair goes out
@@ -735,17 +730,8 @@ __global__ __launch_bounds__(THREADS) void softmax_block_regs(float *__restrict_
     for (int k0 = 0; k0 < NCH; k0 += BURST) {
 #pragma unroll
         for (int k = k0; k < k0 + BURST; k++) {
-            const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4 - m;
-            if (!ANYWHERE) {
-                r[k] = e < n ? load4<NT>(x + e) : make_float4(nan, nan, nan, nan);
-            } else if (e >= 0 && e + 4 <= n) {
-                r[k] = load4_dword_aligned<NT>(x + e);
-            } else {
-                r[k].x = e >= 0 && e < n ? x[e] : nan;
-                r[k].y = e + 1 >= 0 && e + 1 < n ? x[e + 1] : nan;
-                r[k].z = e + 2 >= 0 && e + 2 < n ? x[e + 2] : nan;
-                r[k].w = e + 3 >= 0 && e + 3 < n ? x[e + 3] : nan;
-            }
+            const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4;
+            r[k] = e < n ? load4<NT>(x + e) : make_float4(nan, nan, nan, nan);
         }
 #pragma unroll
         for (int k = k0; k < k0 + BURST; k++) mx = nanmax(nanmax(r[k].x, r[k].y), nanmax(nanmax(r[k].z, r[k].w), mx));
@@ -755,32 +741,16 @@ __global__ __launch_bounds__(THREADS) void softmax_block_regs(float *__restrict_
     float sum = 0.0f;
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4 - m;
+        const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4;
         r[k].x = softmax_exp(r[k].x, mx), r[k].y = softmax_exp(r[k].y, mx), r[k].z = softmax_exp(r[k].z, mx), r[k].w = softmax_exp(r[k].w, mx);
-        if (!ANYWHERE) {
-            if (e < n) sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
-        } else if (e >= 0 && e + 4 <= n) {
-            sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
-        } else {
-            sum += ((e >= 0 && e < n ? r[k].x : 0.0f) + (e + 1 >= 0 && e + 1 < n ? r[k].y : 0.0f)) +
-                   ((e + 2 >= 0 && e + 2 < n ? r[k].z : 0.0f) + (e + 3 >= 0 && e + 3 < n ? r[k].w : 0.0f));
-        }
+        if (e < n) sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
     }
     sum = block_reduce<SumOp, THREADS / WAVE>(sum, lds);
     const float recip = 1.0f / sum;
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4 - m;
-        if (!ANYWHERE) {
-            if (e < n) store4<NT>(o + e, make_float4(r[k].x * recip, r[k].y * recip, r[k].z * recip, r[k].w * recip));
-        } else if (e >= 0 && e + 4 <= n) {
-            store4_dword_aligned<NT>(o + e, make_float4(r[k].x * recip, r[k].y * recip, r[k].z * recip, r[k].w * recip));
-        } else {
-            if (e >= 0 && e < n) o[e] = r[k].x * recip;
-            if (e + 1 >= 0 && e + 1 < n) o[e + 1] = r[k].y * recip;
-            if (e + 2 >= 0 && e + 2 < n) o[e + 2] = r[k].z * recip;
-            if (e + 3 >= 0 && e + 3 < n) o[e + 3] = r[k].w * recip;
-        }
+        const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4;
+        if (e < n) store4<NT>(o + e, make_float4(r[k].x * recip, r[k].y * recip, r[k].z * recip, r[k].w * recip));
     }
 }
 
@@ -840,169 +810,250 @@ __global__ __launch_bounds__(THREADS) void layernorm_block_regs(float *__restric
     }
 }
 
-// LayerNormalization over rows that start anywhere (see softmax_block_regs' ANYWHERE): 16-byte accesses on 4-byte
-// boundaries for the row, scale and bias alike; the last, partial float4 element by element.
-template <int THREADS, int NCH, bool NT>
-__global__ __launch_bounds__(THREADS) void layernorm_block_anywhere(float *__restrict__ out, const float *__restrict__ in,
-                                                                 const float *__restrict__ gamma, const float *__restrict__ beta, size_t len,
-                                                                 float eps) {
-    __shared__ float lds[THREADS / WAVE];
-    const float *x = in + (size_t)blockIdx.x * len;
-    float *o = out + (size_t)blockIdx.x * len;
-    using idx_t = std::conditional_t<(NCH > 8), int, ptrdiff_t>;  // see softmax_block_regs; here 64-bit indices are ahead up to eight float4 per thread
-    const idx_t m = 0, n = (idx_t)len;
-    const float inv_n = 1.0f / (float)len;
-    float4 r[NCH];
-    float sum = 0.0f;
-#pragma unroll
-    for (int k = 0; k < NCH; k++) {
-        const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4 - m;
-        if (e >= 0 && e + 4 <= n) {
-            r[k] = load4_dword_aligned<NT>(x + e);
-        } else {  // slots outside the row hold zero: they add nothing to the sum
-            r[k].x = e >= 0 && e < n ? x[e] : 0.0f;
-            r[k].y = e + 1 >= 0 && e + 1 < n ? x[e + 1] : 0.0f;
-            r[k].z = e + 2 >= 0 && e + 2 < n ? x[e + 2] : 0.0f;
-            r[k].w = e + 3 >= 0 && e + 3 < n ? x[e + 3] : 0.0f;
-        }
-        sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
-    }
-    const float mean = block_reduce<SumOp, THREADS / WAVE>(sum, lds) * inv_n;
-    float ss = 0.0f;
-#pragma unroll
-    for (int k = 0; k < NCH; k++) {
-        const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4 - m;
-        r[k].x -= mean, r[k].y -= mean, r[k].z -= mean, r[k].w -= mean;
-        if (e >= 0 && e + 4 <= n) {
-            ss += (r[k].x * r[k].x + r[k].y * r[k].y) + (r[k].z * r[k].z + r[k].w * r[k].w);
-        } else {
-            ss += ((e >= 0 && e < n ? r[k].x * r[k].x : 0.0f) + (e + 1 >= 0 && e + 1 < n ? r[k].y * r[k].y : 0.0f)) +
-                  ((e + 2 >= 0 && e + 2 < n ? r[k].z * r[k].z : 0.0f) + (e + 3 >= 0 && e + 3 < n ? r[k].w * r[k].w : 0.0f));
-        }
-    }
-    ss = block_reduce<SumOp, THREADS / WAVE>(ss, lds);
-    const float inv_std = 1.0f / sqrtf(__builtin_fmaf(ss, inv_n, eps));
-#pragma unroll
-    for (int k = 0; k < NCH; k++) {
-        const idx_t e = ((idx_t)threadIdx.x + (idx_t)THREADS * k) * 4 - m;
-        if (e >= 0 && e + 4 <= n) {
-            float4 g, b;
-            g = load4_dword_aligned<false>(gamma + e), b = load4_dword_aligned<false>(beta + e);
-            store4_dword_aligned<NT>(o + e, make_float4(__builtin_fmaf(r[k].x * inv_std, g.x, b.x), __builtin_fmaf(r[k].y * inv_std, g.y, b.y),
-                                          __builtin_fmaf(r[k].z * inv_std, g.z, b.z), __builtin_fmaf(r[k].w * inv_std, g.w, b.w)));
-        } else {
-            if (e >= 0 && e < n) o[e] = __builtin_fmaf(r[k].x * inv_std, gamma[e], beta[e]);
-            if (e + 1 >= 0 && e + 1 < n) o[e + 1] = __builtin_fmaf(r[k].y * inv_std, gamma[e + 1], beta[e + 1]);
-            if (e + 2 >= 0 && e + 2 < n) o[e + 2] = __builtin_fmaf(r[k].z * inv_std, gamma[e + 2], beta[e + 2]);
-            if (e + 3 >= 0 && e + 3 < n) o[e + 3] = __builtin_fmaf(r[k].w * inv_std, gamma[e + 3], beta[e + 3]);
-        }
-    }
-}
-
-// The block-per-row kernels again for rows that take 1024 threads: two such blocks are all a CU holds, and a block
-// that loads its row, reduces, reduces again and stores leaves the memory pipeline idle while it reduces.  Here a
-// block walks rows blockIdx.x, blockIdx.x + gridDim.x, ... and requests the next row before it works on the one it
-// holds.  Which thread holds which elements and the order of every sum are those of the kernels above: same bits.
-// Both rows have to fit 64 registers per thread together with everything else, so rows, scale and bias are
-// addressed as buffers: a descriptor in scalar registers and one 32-bit vector offset per chunk, the same for every
-// buffer, and slots past the row's end read zero and store nothing without a branch.
+// ---------------------------------------------------------------------------
+// Rows addressed as buffers
+// ---------------------------------------------------------------------------
+// A raw buffer's 16-byte accesses need 4-byte alignment only and are checked against the buffer's size in hardware:
+// what lies past the end reads as zero and is not stored, without a branch, and one 32-bit offset per thread
+// addresses the input row, the output row, scale and bias alike (the descriptors sit in scalar registers).  That is
+// what rows that start anywhere need (a length that is not a multiple of 4, or a base pointer that is only 4-byte
+// aligned), and what lets a thread hold two rows, or 26 float4 of one, in its registers.
+//
+// A row of `len` elements as its block holds it (EDGES): a head of up to 31 elements that ends at the row's first
+// 128-byte boundary, one each in the block's first threads; the body, whole float4s from that boundary on, float4
+// number tid + stride * k in chunk k of thread tid, so that every load and store instruction of a wavefront covers
+// eight whole 128-byte lines (rows of 36 K and 50 K elements: 3 to 5 points of the HBM peak over float4s taken where
+// the row starts); and a tail of up to three elements behind the body, again in the first threads.  The body's
+// descriptor ends with the body, so a float4 is in range or out of range as a whole.  Without EDGES the row is all
+// body: whole float4s, and 128-byte lines when its tensor is a stack of them.
 typedef uint32_t u32x4_row __attribute__((ext_vector_type(4)));
 typedef float f32x4_row __attribute__((ext_vector_type(4)));
 
-// The chunk's offset goes into the vector offset: that one is checked against the buffer's size, the scalar offset
-// of the instruction is not.
 template <bool NT>
-__device__ __forceinline__ float4 load_chunk(__amdgpu_buffer_rsrc_t row, uint32_t byte_offset) {
-    const f32x4_row f = __builtin_bit_cast(f32x4_row, __builtin_amdgcn_raw_buffer_load_b128(row, threadIdx.x * 16u + byte_offset, 0, NT ? 2 : 0));
+__device__ __forceinline__ float4 load_at(__amdgpu_buffer_rsrc_t row, uint32_t byte_offset) {
+    const f32x4_row f = __builtin_bit_cast(f32x4_row, __builtin_amdgcn_raw_buffer_load_b128(row, byte_offset, 0, NT ? 2 : 0));
     return make_float4(f[0], f[1], f[2], f[3]);
+}
+template <bool NT>
+__device__ __forceinline__ void store_at(__amdgpu_buffer_rsrc_t row, uint32_t byte_offset, float4 v) {
+    const f32x4_row f = {v.x, v.y, v.z, v.w};
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_row, f), row, byte_offset, 0, NT ? 2 : 0);
 }
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t row_buffer(const float *row, uint32_t len) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(row), 0, (int)(len * 4u), 0x00020000);  // raw buffer of 32-bit words
 }
 
-template <int THREADS, int NCH, bool NT>
-__device__ __forceinline__ void request_row(float4 (&r)[NCH], __amdgpu_buffer_rsrc_t row) {
+struct RowBuf {
+    const float *p;
+    uint32_t len;
+    uint32_t head;  // elements ahead of the body
+    __device__ __forceinline__ uint32_t body() const { return (len - head) & ~3u; }
+    __device__ __forceinline__ uint32_t tail() const { return (len - head) & 3u; }
+    __device__ __forceinline__ __amdgpu_buffer_rsrc_t body_rsrc() const { return row_buffer(p + head, body()); }
+    __device__ __forceinline__ __amdgpu_buffer_rsrc_t head_rsrc() const { return row_buffer(p, head); }
+    __device__ __forceinline__ __amdgpu_buffer_rsrc_t tail_rsrc() const { return row_buffer(p + head + body(), tail()); }
+};
+
+// Elements of the row that starts at `row` ahead of its first 128-byte boundary (0 to 31).
+__device__ __forceinline__ uint32_t elements_to_line(const float *row) {
+    return ((128u - ((uint32_t)reinterpret_cast<uintptr_t>(row) & 127u)) & 127u) >> 2;
+}
+
+// One element of a row's head or tail per thread: element tid of the piece, zero (and nothing stored) past its end.
+__device__ __forceinline__ float load_edge(__amdgpu_buffer_rsrc_t piece, uint32_t tid) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(piece, tid * 4u, 0, 0));
+}
+__device__ __forceinline__ void store_edge(__amdgpu_buffer_rsrc_t piece, uint32_t tid, float v) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), piece, tid * 4u, 0, 0);
+}
+
+// Byte offset of a thread's float4 in chunk k; `stride` threads share the row.  The thread's own offset is hidden from
+// the compiler's value numbering at every use: left to itself it keeps one register per chunk alive from the row's
+// load to its store (18 to 26 registers of a long row) instead of an addition per access.
+__device__ __forceinline__ uint32_t chunk_offset(uint32_t tid, uint32_t stride, int k) {
+    uint32_t own = tid * 16u;
+    asm volatile("" : "+v"(own));
+    return own + (uint32_t)k * stride * 16u;
+}
+
+// `stride` threads share the row (a block's, or a wavefront's 64); tid is the thread's number among them.
+template <int NCH, bool NT, bool EDGES>
+__device__ __forceinline__ void request_row(float4 (&r)[NCH], float &h, float &t, const RowBuf &row, uint32_t tid, uint32_t stride) {
+    const __amdgpu_buffer_rsrc_t body = row.body_rsrc();
 #pragma unroll
-    for (int k = 0; k < NCH; k++) {
-        r[k] = load_chunk<NT>(row, k * THREADS * 16);
-    }
+    for (int k = 0; k < NCH; k++) r[k] = load_at<NT>(body, chunk_offset(tid, stride, k));
+    h = EDGES ? load_edge(row.head_rsrc(), tid) : 0.0f;
+    t = EDGES ? load_edge(row.tail_rsrc(), tid) : 0.0f;
 }
 
-template <int THREADS, bool NT>
-__device__ __forceinline__ void store_chunk(__amdgpu_buffer_rsrc_t row, int k, float4 v) {
-    const f32x4_row f = {v.x, v.y, v.z, v.w};
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_row, f), row, threadIdx.x * 16u + (uint32_t)(k * THREADS * 16), 0, NT ? 2 : 0);
+template <int NCH, bool NT, bool EDGES>
+__device__ __forceinline__ void store_row(const float4 (&r)[NCH], float h, float t, const RowBuf &row, uint32_t tid, uint32_t stride) {
+    const __amdgpu_buffer_rsrc_t body = row.body_rsrc();
+#pragma unroll
+    for (int k = 0; k < NCH; k++) store_at<NT>(body, chunk_offset(tid, stride, k), r[k]);
+    if (EDGES) store_edge(row.head_rsrc(), tid, h), store_edge(row.tail_rsrc(), tid, t);
 }
 
-template <int THREADS, int NCH, bool NT>
-__device__ __forceinline__ void softmax_row_in_regs(float4 (&r)[NCH], __amdgpu_buffer_rsrc_t o, uint32_t len, float *lds) {
+// Reduction over a block of any whole number of wavefronts (at most 16); `lds` holds 16 floats.
+template <class OP> __device__ __forceinline__ float block_reduce_any(float v, float *lds) {
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    v = wave_reduce<OP>(v);
+    __syncthreads();  // protects lds against a previous use
+    if (lane == 0) lds[wave] = v;
+    __syncthreads();
+    float r = OP::identity();
+    for (int w = 0; w < nwaves; w++) r = OP::apply(r, lds[w]);
+    return r;
+}
+
+// The two reductions of a row: over the wavefront, or over the block through LDS.
+template <class OP, bool WAVE_ROW> __device__ __forceinline__ float row_reduce(float v, float *lds) {
+    if constexpr (WAVE_ROW) return wave_reduce<OP>(v);
+    else return block_reduce_any<OP>(v, lds);
+}
+
+// Softmax of the row in r (and h, t), written to o.
+template <int NCH, bool NT, bool EDGES, bool WAVE_ROW>
+__device__ __forceinline__ void softmax_row_in_regs(float4 (&r)[NCH], float h, float t, const RowBuf &o, uint32_t tid, uint32_t stride, float *lds) {
     const float nan = __builtin_nanf("");
-    float mx = nan;
+    const uint32_t body = o.body();
+    float mx = nan;  // NaN elements (and the slots past the row) are ignored by the maximum
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        if ((threadIdx.x + THREADS * k) * 4u >= len) r[k] = make_float4(nan, nan, nan, nan);
+        if ((tid + stride * k) * 4u >= body) r[k] = make_float4(nan, nan, nan, nan);
         mx = nanmax(nanmax(r[k].x, r[k].y), nanmax(nanmax(r[k].z, r[k].w), mx));
     }
-    mx = block_reduce<MaxOp, THREADS / WAVE>(mx, lds);
+    if (EDGES) {
+        h = tid < o.head ? h : nan, t = tid < o.tail() ? t : nan;
+        mx = nanmax(nanmax(h, t), mx);
+    }
+    mx = row_reduce<MaxOp, WAVE_ROW>(mx, lds);
     float sum = 0.0f;
 #pragma unroll
     for (int k = 0; k < NCH; k++) {
-        const bool valid = (threadIdx.x + THREADS * k) * 4u < len;
         r[k].x = softmax_exp(r[k].x, mx), r[k].y = softmax_exp(r[k].y, mx), r[k].z = softmax_exp(r[k].z, mx), r[k].w = softmax_exp(r[k].w, mx);
-        if (valid) sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
+        if ((tid + stride * k) * 4u < body) sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
         __builtin_amdgcn_sched_barrier(0);  // one chunk's temporaries at a time
     }
-    sum = block_reduce<SumOp, THREADS / WAVE>(sum, lds);
+    if (EDGES) {
+        h = softmax_exp(h, mx), t = softmax_exp(t, mx);
+        sum += (tid < o.head ? h : 0.0f) + (tid < o.tail() ? t : 0.0f);
+    }
+    sum = row_reduce<SumOp, WAVE_ROW>(sum, lds);
     const float recip = 1.0f / sum;
 #pragma unroll
-    for (int k = 0; k < NCH; k++)
-        store_chunk<THREADS, NT>(o, k, make_float4(r[k].x * recip, r[k].y * recip, r[k].z * recip, r[k].w * recip));
+    for (int k = 0; k < NCH; k++) r[k] = make_float4(r[k].x * recip, r[k].y * recip, r[k].z * recip, r[k].w * recip);
+    store_row<NCH, NT, EDGES>(r, h * recip, t * recip, o, tid, stride);
 }
 
+// LayerNormalization of the row in r (and h, t), written to o; scale and bias are cut into head, body and tail as the
+// row is.  GB: when scale and bias are requested: 0 chunk by chunk behind the reductions, 1 between the two reductions
+// (they then wait in registers during the second).
+template <int NCH, bool NT, bool EDGES, bool WAVE_ROW, int GB>
+__device__ __forceinline__ void layernorm_row_in_regs(float4 (&r)[NCH], float h, float t, const RowBuf &o, const RowBuf &gamma, const RowBuf &beta,
+                                                      float eps, uint32_t tid, uint32_t stride, float *lds) {
+    const uint32_t body = o.body();
+    const float inv_n = 1.0f / (float)o.len;
+    const __amdgpu_buffer_rsrc_t ob = o.body_rsrc(), gb = gamma.body_rsrc(), bb = beta.body_rsrc();
+    float4 g[GB ? NCH : 1], b[GB ? NCH : 1];
+    float gh = 0.0f, bh = 0.0f, gt = 0.0f, bt = 0.0f;
+    auto request_gb = [&]() {
+#pragma unroll
+        for (int k = 0; k < (GB ? NCH : 0); k++)
+            g[GB ? k : 0] = load_at<false>(gb, chunk_offset(tid, stride, k)), b[GB ? k : 0] = load_at<false>(bb, chunk_offset(tid, stride, k));
+        if (EDGES) {
+            gh = load_edge(gamma.head_rsrc(), tid), bh = load_edge(beta.head_rsrc(), tid);
+            gt = load_edge(gamma.tail_rsrc(), tid), bt = load_edge(beta.tail_rsrc(), tid);
+        }
+    };
+    float sum = 0.0f;  // slots past the row hold zeros
+#pragma unroll
+    for (int k = 0; k < NCH; k++) sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
+    if (EDGES) sum += h + t;
+    const float mean = row_reduce<SumOp, WAVE_ROW>(sum, lds) * inv_n;
+    if (GB == 1) request_gb();
+    float ss = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NCH; k++) {
+        r[k].x -= mean, r[k].y -= mean, r[k].z -= mean, r[k].w -= mean;
+        if ((tid + stride * k) * 4u < body) ss += (r[k].x * r[k].x + r[k].y * r[k].y) + (r[k].z * r[k].z + r[k].w * r[k].w);
+    }
+    if (EDGES) {
+        h -= mean, t -= mean;
+        ss += (tid < o.head ? h * h : 0.0f) + (tid < o.tail() ? t * t : 0.0f);
+    }
+    ss = row_reduce<SumOp, WAVE_ROW>(ss, lds);
+    const float inv_std = 1.0f / sqrtf(__builtin_fmaf(ss, inv_n, eps));
+    if (GB == 0) request_gb();  // the edges' scale and bias only
+#pragma unroll
+    for (int k = 0; k < NCH; k++) {
+        const float4 gk = GB ? g[GB ? k : 0] : load_at<false>(gb, chunk_offset(tid, stride, k));
+        const float4 bk = GB ? b[GB ? k : 0] : load_at<false>(bb, chunk_offset(tid, stride, k));
+        store_at<NT>(ob, chunk_offset(tid, stride, k),
+                     make_float4(__builtin_fmaf(r[k].x * inv_std, gk.x, bk.x), __builtin_fmaf(r[k].y * inv_std, gk.y, bk.y),
+                                 __builtin_fmaf(r[k].z * inv_std, gk.z, bk.z), __builtin_fmaf(r[k].w * inv_std, gk.w, bk.w)));
+        if (!GB && k % 2 == 1) __builtin_amdgcn_sched_barrier(0);  // scale and bias of two chunks at a time
+    }
+    if (EDGES) {
+        store_edge(o.head_rsrc(), tid, __builtin_fmaf(h * inv_std, gh, bh));
+        store_edge(o.tail_rsrc(), tid, __builtin_fmaf(t * inv_std, gt, bt));
+    }
+}
+
+// One block per row, the row wherever it starts; the block is any whole number of wavefronts (its threads share the
+// row's float4s NCH each, so a row of 1025 float4 takes 576 threads and not the next power of two).
+// MINW: wavefronts per SIMD to leave room for: 8 (64 registers a thread: blocks of 1024 threads fit a CU two at a time,
+// and one loads or stores while the other reduces) up to eight float4 per thread; 4 (128 registers) beyond, where a row
+// takes blocks of 512 threads with 18 or 20 float4 each, two to a CU, or of 1024 threads, one to a CU.
+template <int NCH, bool NT, bool EDGES, int MINW>
+__global__ __launch_bounds__(1024, MINW) void softmax_block_anywhere(float *__restrict__ out, const float *__restrict__ in, uint32_t len) {
+    __shared__ float lds[16];
+    const float *x = in + (size_t)blockIdx.x * len;
+    const uint32_t head = EDGES ? elements_to_line(x) : 0;
+    float4 r[NCH];
+    float h, t;
+    request_row<NCH, NT, EDGES>(r, h, t, RowBuf{x, len, head}, threadIdx.x, blockDim.x);
+    softmax_row_in_regs<NCH, NT, EDGES, false>(r, h, t, RowBuf{out + (size_t)blockIdx.x * len, len, head}, threadIdx.x, blockDim.x, lds);
+}
+
+template <int NCH, bool NT, bool EDGES, int MINW, int GB>
+__global__ __launch_bounds__(1024, MINW) void layernorm_block_anywhere(float *__restrict__ out, const float *__restrict__ in,
+                                                                       const float *__restrict__ gamma, const float *__restrict__ beta, uint32_t len,
+                                                                       float eps) {
+    __shared__ float lds[16];
+    const float *x = in + (size_t)blockIdx.x * len;
+    const uint32_t head = EDGES ? elements_to_line(x) : 0;
+    float4 r[NCH];
+    float h, t;
+    request_row<NCH, NT, EDGES>(r, h, t, RowBuf{x, len, head}, threadIdx.x, blockDim.x);
+    layernorm_row_in_regs<NCH, NT, EDGES, false, GB>(r, h, t, RowBuf{out + (size_t)blockIdx.x * len, len, head}, RowBuf{gamma, len, head},
+                                                     RowBuf{beta, len, head}, eps, threadIdx.x, blockDim.x, lds);
+}
+
+// The block-per-row kernels for rows that take 1024 threads and four float4 each: two such blocks are all a CU holds,
+// and a block that loads its row, reduces, reduces again and stores leaves the memory pipeline idle while it reduces.
+// Here a block walks rows blockIdx.x, blockIdx.x + gridDim.x, ... and requests the next row before it works on the one
+// it holds; both rows fit 64 registers per thread together with everything else.  Which thread holds which elements
+// and the order of every sum are those of softmax_block_regs / layernorm_block_regs: same bits.
 template <int THREADS, int NCH, bool NT>
 __global__ __launch_bounds__(THREADS, 2048 / THREADS * (THREADS / WAVE) / 4) void softmax_block_pipe(float *__restrict__ out, const float *__restrict__ in,
                                                                                                       uint32_t len, size_t rows) {
-    __shared__ float lds[THREADS / WAVE];
+    __shared__ float lds[16];
     size_t row = blockIdx.x;
     const size_t step = gridDim.x;
     float4 next[NCH];
-    request_row<THREADS, NCH, NT>(next, row_buffer(in + row * len, len));
+    float h, t;  // unused: these rows are whole float4s
+    request_row<NCH, NT, false>(next, h, t, RowBuf{in + row * len, len, 0}, threadIdx.x, THREADS);
     while (row + step < rows) {
         float4 r[NCH];
 #pragma unroll
         for (int k = 0; k < NCH; k++) r[k] = next[k];
-        request_row<THREADS, NCH, NT>(next, row_buffer(in + (row + step) * len, len));
-        softmax_row_in_regs<THREADS, NCH, NT>(r, row_buffer(out + row * len, len), len, lds);
+        request_row<NCH, NT, false>(next, h, t, RowBuf{in + (row + step) * len, len, 0}, threadIdx.x, THREADS);
+        softmax_row_in_regs<NCH, NT, false, false>(r, 0.0f, 0.0f, RowBuf{out + row * len, len, 0}, threadIdx.x, THREADS, lds);
         row += step;
     }
-    softmax_row_in_regs<THREADS, NCH, NT>(next, row_buffer(out + row * len, len), len, lds);
-}
-
-template <int THREADS, int NCH, bool NT>
-__device__ __forceinline__ void layernorm_row_in_regs(float4 (&r)[NCH], __amdgpu_buffer_rsrc_t o, __amdgpu_buffer_rsrc_t gamma,
-                                                      __amdgpu_buffer_rsrc_t beta, uint32_t len, float eps, float *lds) {
-    const float inv_n = 1.0f / (float)len;
-    float sum = 0.0f;  // slots past the row hold zeros
-#pragma unroll
-    for (int k = 0; k < NCH; k++) sum += (r[k].x + r[k].y) + (r[k].z + r[k].w);
-    const float mean = block_reduce<SumOp, THREADS / WAVE>(sum, lds) * inv_n;
-    float ss = 0.0f;
-#pragma unroll
-    for (int k = 0; k < NCH; k++) {
-        const bool valid = (threadIdx.x + THREADS * k) * 4u < len;
-        r[k].x -= mean, r[k].y -= mean, r[k].z -= mean, r[k].w -= mean;
-        if (valid) ss += (r[k].x * r[k].x + r[k].y * r[k].y) + (r[k].z * r[k].z + r[k].w * r[k].w);
-    }
-    ss = block_reduce<SumOp, THREADS / WAVE>(ss, lds);
-    const float inv_std = 1.0f / sqrtf(__builtin_fmaf(ss, inv_n, eps));
-#pragma unroll
-    for (int k = 0; k < NCH; k++) {
-        const float4 g = load_chunk<false>(gamma, k * THREADS * 16), b = load_chunk<false>(beta, k * THREADS * 16);
-        store_chunk<THREADS, NT>(o, k, make_float4(__builtin_fmaf(r[k].x * inv_std, g.x, b.x), __builtin_fmaf(r[k].y * inv_std, g.y, b.y),
-                                                   __builtin_fmaf(r[k].z * inv_std, g.z, b.z), __builtin_fmaf(r[k].w * inv_std, g.w, b.w)));
-        if (k % 2 == 1) __builtin_amdgcn_sched_barrier(0);  // scale and bias of two chunks at a time
-    }
+    softmax_row_in_regs<NCH, NT, false, false>(next, 0.0f, 0.0f, RowBuf{out + row * len, len, 0}, threadIdx.x, THREADS, lds);
 }
 
 template <int THREADS, int NCH, bool NT>
@@ -1010,21 +1061,22 @@ __global__ __launch_bounds__(THREADS, 2048 / THREADS * (THREADS / WAVE) / 4) voi
                                                                                                         const float *__restrict__ gamma,
                                                                                                         const float *__restrict__ beta, uint32_t len,
                                                                                                         size_t rows, float eps) {
-    __shared__ float lds[THREADS / WAVE];
+    __shared__ float lds[16];
     size_t row = blockIdx.x;
     const size_t step = gridDim.x;
-    const __amdgpu_buffer_rsrc_t g = row_buffer(gamma, len), b = row_buffer(beta, len);
+    const RowBuf g{gamma, len, 0}, b{beta, len, 0};
     float4 next[NCH];
-    request_row<THREADS, NCH, NT>(next, row_buffer(in + row * len, len));
+    float h, t;
+    request_row<NCH, NT, false>(next, h, t, RowBuf{in + row * len, len, 0}, threadIdx.x, THREADS);
     while (row + step < rows) {
         float4 r[NCH];
 #pragma unroll
         for (int k = 0; k < NCH; k++) r[k] = next[k];
-        request_row<THREADS, NCH, NT>(next, row_buffer(in + (row + step) * len, len));
-        layernorm_row_in_regs<THREADS, NCH, NT>(r, row_buffer(out + row * len, len), g, b, len, eps, lds);
+        request_row<NCH, NT, false>(next, h, t, RowBuf{in + (row + step) * len, len, 0}, threadIdx.x, THREADS);
+        layernorm_row_in_regs<NCH, NT, false, false, 0>(r, 0.0f, 0.0f, RowBuf{out + row * len, len, 0}, g, b, eps, threadIdx.x, THREADS, lds);
         row += step;
     }
-    layernorm_row_in_regs<THREADS, NCH, NT>(next, row_buffer(out + row * len, len), g, b, len, eps, lds);
+    layernorm_row_in_regs<NCH, NT, false, false, 0>(next, 0.0f, 0.0f, RowBuf{out + row * len, len, 0}, g, b, eps, threadIdx.x, THREADS, lds);
 }
 
 // Threads per row and float4 per thread for a row of `len` elements in the block-per-row kernels.
@@ -1061,18 +1113,70 @@ void softmax_block_go(bool nt, hipStream_t s, size_t rows, size_t resident, floa
     if (nt) hipLaunchKernelGGL((softmax_block_regs<THREADS, NCH, true>), grid, dim3(THREADS), 0, s, out, in, len);
     else hipLaunchKernelGGL((softmax_block_regs<THREADS, NCH, false>), grid, dim3(THREADS), 0, s, out, in, len);
 }
-template <int THREADS, int NCH>
-void softmax_block_anywhere_go(bool nt, hipStream_t s, size_t rows, float *out, const float *in, size_t len) {
-    const dim3 grid((unsigned)rows);
-    if (nt) hipLaunchKernelGGL((softmax_block_regs<THREADS, NCH, true, true>), grid, dim3(THREADS), 0, s, out, in, len);
-    else hipLaunchKernelGGL((softmax_block_regs<THREADS, NCH, false, true>), grid, dim3(THREADS), 0, s, out, in, len);
+// Threads of a block and float4 per thread for a row that starts anywhere: two float4 per thread up to 2048 float4 in
+// the row, then the fewest that 1024 threads cover it with; the threads are the whole wavefronts that hold the row's
+// at most len / 4 whole float4s (the elements ahead of them and behind them ride along in the first threads).  From 8 K float4 on
+// blocks of 512 threads with 18 or 20 each, then blocks of 1024 threads, one to a CU.
+struct AnyLayout {
+    int threads, nch;
+};
+inline AnyLayout any_layout(size_t len) {
+    const size_t v = len / 4;
+    const int nch = v <= 2048 ? 2 : v <= 3072 ? 3 : v <= 4096 ? 4 : v <= 6144 ? 6 : v <= 8192 ? 8 : 0;
+    if (nch) return AnyLayout{(int)(((v + nch - 1) / nch + WAVE - 1) / WAVE * WAVE), nch};
+    if (v <= 512 * 18) return AnyLayout{512, 18};
+    if (v <= 512 * 20) return AnyLayout{512, 20};
+    return AnyLayout{1024, v <= 12288 ? 12 : v <= 13312 ? 13 : 16};
 }
-template <int THREADS, int NCH>
-void layernorm_block_anywhere_go(bool nt, hipStream_t s, size_t rows, float *out, const float *in, const float *gamma, const float *beta, size_t len,
-                              float eps) {
-    const dim3 grid((unsigned)rows);
-    if (nt) hipLaunchKernelGGL((layernorm_block_anywhere<THREADS, NCH, true>), grid, dim3(THREADS), 0, s, out, in, gamma, beta, len, eps);
-    else hipLaunchKernelGGL((layernorm_block_anywhere<THREADS, NCH, false>), grid, dim3(THREADS), 0, s, out, in, gamma, beta, len, eps);
+#define ALTIUS_ANY_LAYOUTS(L)                                                                                       \
+    switch ((L).nch) {                                                                                              \
+        ALTIUS_GO(2, 8) ALTIUS_GO(3, 8) ALTIUS_GO(4, 8) ALTIUS_GO(6, 8) ALTIUS_GO(8, 8)                             \
+        ALTIUS_GO(12, 4) ALTIUS_GO(13, 4) ALTIUS_GO(16, 4) ALTIUS_GO(18, 4) ALTIUS_GO(20, 4)                        \
+    }
+
+// A launch with the template's flags NT and EDGES taken from run-time values; AFTER: the template arguments behind them.
+#define ALTIUS_NT_EDGES(KERNEL, NCH, AFTER, ...)                                                            \
+    do {                                                                                                    \
+        if (nt && edges) hipLaunchKernelGGL((KERNEL<NCH, true, true, AFTER>), __VA_ARGS__);                 \
+        else if (nt) hipLaunchKernelGGL((KERNEL<NCH, true, false, AFTER>), __VA_ARGS__);                    \
+        else if (edges) hipLaunchKernelGGL((KERNEL<NCH, false, true, AFTER>), __VA_ARGS__);                 \
+        else hipLaunchKernelGGL((KERNEL<NCH, false, false, AFTER>), __VA_ARGS__);                           \
+    } while (0)
+#define ALTIUS_COMMA ,
+
+inline bool aligned128(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 127u) == 0; }
+
+// Softmax / LayerNormalization over rows of more than 1024 and at most 65536 elements that start anywhere.
+bool softmax_anywhere_launch(bool nt, hipStream_t s, size_t rows, float *out, const float *in, size_t len) {
+    const bool edges = !(len % 32 == 0 && aligned128(in) && aligned128(out));  // not a stack of whole 128-byte lines
+    const AnyLayout lay = any_layout(len);
+    const dim3 grid((unsigned)rows), block((unsigned)lay.threads);
+#define ALTIUS_GO(N, W)                                                                              \
+    case N:                                                                                          \
+        ALTIUS_NT_EDGES(softmax_block_anywhere, N, W, grid, block, 0, s, out, in, (uint32_t)len);    \
+        return true;
+    ALTIUS_ANY_LAYOUTS(lay)
+#undef ALTIUS_GO
+    return false;
+}
+bool layernorm_anywhere_launch(bool nt, hipStream_t s, size_t rows, float *out, const float *in, const float *gamma, const float *beta, size_t len,
+                               float eps) {
+    const bool edges = !(len % 32 == 0 && aligned128(in) && aligned128(out));
+    const AnyLayout lay = any_layout(len);
+    const dim3 grid((unsigned)rows), block((unsigned)lay.threads);
+    // Scale and bias between the two reductions: 2 to 3.5 points of the HBM peak for blocks of up to 512 threads with
+    // two float4 each (rows of up to 4 K elements), 5 lost with 640 and 768 threads; behind the reductions otherwise.
+    if (lay.nch == 2 && lay.threads <= 512) {
+        ALTIUS_NT_EDGES(layernorm_block_anywhere, 2, 8 ALTIUS_COMMA 1, grid, block, 0, s, out, in, gamma, beta, (uint32_t)len, eps);
+        return true;
+    }
+#define ALTIUS_GO(N, W)                                                                                                                 \
+    case N:                                                                                                                             \
+        ALTIUS_NT_EDGES(layernorm_block_anywhere, N, W ALTIUS_COMMA 0, grid, block, 0, s, out, in, gamma, beta, (uint32_t)len, eps);     \
+        return true;
+    ALTIUS_ANY_LAYOUTS(lay)
+#undef ALTIUS_GO
+    return false;
 }
 template <int THREADS, int NCH>
 void layernorm_block_go(bool nt, hipStream_t s, size_t rows, size_t resident, float *out, const float *in, const float *gamma, const float *beta,
@@ -1091,7 +1195,7 @@ void layernorm_block_go(bool nt, hipStream_t s, size_t rows, size_t resident, fl
 #define ALTIUS_BLOCK_LAYOUTS(L)                                                          \
     switch ((L).threads * 100 + (L).nch) {                                               \
         ALTIUS_GO(256, 2) ALTIUS_GO(384, 2) ALTIUS_GO(512, 2) ALTIUS_GO(768, 2) ALTIUS_GO(1024, 2) ALTIUS_GO(1024, 3) ALTIUS_GO(1024, 4) \
-        ALTIUS_GO(1024, 6) ALTIUS_GO(1024, 8) ALTIUS_GO(1024, 12) ALTIUS_GO(1024, 16)                                                      \
+        ALTIUS_GO(1024, 6) ALTIUS_GO(1024, 8) ALTIUS_GO(1024, 12) ALTIUS_GO(1024, 16)                                                                       \
     }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -1343,7 +1447,6 @@ constexpr size_t MAX_WAVE_ROW = 1024;
 constexpr size_t MAX_LONG_ROW = 1280;  // rows kept in a wavefront's registers when they are whole float4s (at 1536 a block per row is 2 points ahead)
 constexpr size_t MAX_BLOCK_REG_ROW = 65536;  // ... and in a block's registers
 constexpr size_t MAX_GRID = 0x7FFFFFFFu;
-
 }  // namespace
 
 // Threads of the streaming kernels' block: two float4 per thread and pass up to 8192 elements, then the widest block.
@@ -1384,19 +1487,10 @@ int launch_softmax(DeviceCtx &ctx, float *out, const float *in, size_t rows, siz
         ALTIUS_BLOCK_LAYOUTS(lay)
 #undef ALTIUS_GO
         if (!launched) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: no block layout for this row length");
-    } else if (len > MAX_WAVE_ROW && len + 3 <= MAX_BLOCK_REG_ROW && rows <= MAX_GRID) {
+    } else if (len > MAX_WAVE_ROW && len <= MAX_BLOCK_REG_ROW && rows <= MAX_GRID) {
         // Rows that start anywhere, input and output each where it lies.
-        const bool nt = ctx.streaming(rows * len * sizeof(float));
-        const BlockLayout lay = block_layout(len + 6);
-        bool launched = false;
-#define ALTIUS_GO(T, N)                                                      \
-    case T * 100 + N:                                                        \
-        softmax_block_anywhere_go<T, N>(nt, ctx.stream, rows, out, in, len);    \
-        launched = true;                                                     \
-        break;
-        ALTIUS_BLOCK_LAYOUTS(lay)
-#undef ALTIUS_GO
-        if (!launched) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: no block layout for this row length");
+        if (!softmax_anywhere_launch(ctx.streaming(rows * len * sizeof(float)), ctx.stream, rows, out, in, len))
+            return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: no block layout for this row length");
     } else {
         if (rows > MAX_GRID) return ctx.fail(AHIP_ERR_UNSUPPORTED, "softmax: too many rows for one launch");
         const bool nt = ctx.streaming(rows * len * sizeof(float));
@@ -1477,19 +1571,10 @@ int launch_layernorm(DeviceCtx &ctx, float *out, const float *in, const float *g
         ALTIUS_BLOCK_LAYOUTS(lay)
 #undef ALTIUS_GO
         if (!launched) return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: no block layout for this row length");
-    } else if (len > MAX_WAVE_ROW && len + 3 <= MAX_BLOCK_REG_ROW && rows <= MAX_GRID) {
+    } else if (len > MAX_WAVE_ROW && len <= MAX_BLOCK_REG_ROW && rows <= MAX_GRID) {
         // Rows that start anywhere (see launch_softmax).
-        const bool nt = ctx.streaming(rows * len * sizeof(float));
-        const BlockLayout lay = block_layout(len + 6);
-        bool launched = false;
-#define ALTIUS_GO(T, N)                                                                            \
-    case T * 100 + N:                                                                              \
-        layernorm_block_anywhere_go<T, N>(nt, ctx.stream, rows, out, in, gamma, beta, len, eps);      \
-        launched = true;                                                                           \
-        break;
-        ALTIUS_BLOCK_LAYOUTS(lay)
-#undef ALTIUS_GO
-        if (!launched) return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: no block layout for this row length");
+        if (!layernorm_anywhere_launch(ctx.streaming(rows * len * sizeof(float)), ctx.stream, rows, out, in, gamma, beta, len, eps))
+            return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: no block layout for this row length");
     } else {
         if (rows > MAX_GRID) return ctx.fail(AHIP_ERR_UNSUPPORTED, "layernorm: too many rows for one launch");
         const bool nt = ctx.streaming(rows * len * sizeof(float));

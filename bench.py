@@ -821,6 +821,9 @@ def main():
                     help="tensors of at least this many MiB use non-temporal accesses (default: the library's own threshold)")
     ap.add_argument("--sweep-lengths", type=str, default="", help="comma-separated row lengths for the sweep (default: 49 ... 16384)")
     ap.add_argument("--sweep-only", action="store_true", help="run the row sweep and nothing else (profiling)")
+    ap.add_argument("--section", type=str, default="", choices=("", "row_sweep", "shape_sweep", "other_configs"),
+                    help="run this table and nothing else, behind the calibration kernel if --calibrate is given (profiling); "
+                         "prints the table's full records as one JSON line")
     ap.add_argument("--timeline", type=int, default=0, metavar="N",
                     help="print the duration of each of N consecutive launches of every kernel of the step, the first kernel after "
                          "the uploads and one second of idle, and exit ('timeline' in the JSON)")
@@ -851,12 +854,27 @@ def main():
         ctx.set_streaming_threshold(args.streaming_threshold_mib << 20)
     sweep_lengths = tuple(int(v) for v in args.sweep_lengths.split(",") if v) or ROW_SWEEP_LENGTHS
     if args.sweep_only:
+        args.section = "row_sweep"
+    if args.section:
         out = {}
-        if args.calibrate:  # first, so that a profile of this run finds the copy kernel of known size ahead of the sweep
+        if args.calibrate:  # first, so that a profile of this run finds the copy kernel of known size ahead of the table
             cal = calibration_op(ctx, D)
             out["calibration"] = dict({"kernel": cal.name, "bytes": cal.nbytes}, **time_kernel(ctx, cal, args.kernel_iters, args.kernel_warmup, args.kernel_settle_ms).row(cal.nbytes))
             log("%-44s %14d %9.1f us %6.1f %%" % (cal.name, cal.nbytes, out["calibration"]["us"], out["calibration"]["pct_hbm_peak"]))
-        out["row_sweep"] = run_row_sweep(ctx, D, args, sweep_lengths)
+        if args.section == "row_sweep":
+            out["row_sweep"] = run_row_sweep(ctx, D, args, sweep_lengths)
+        else:
+            build = build_shape_sweep(ctx, D) if args.section == "shape_sweep" else build_other_configs(ctx, D, synth)
+            rows = []
+            mark = ctx.alloc(256)
+            for o in build:
+                if args.only and args.only.lower() not in o.name.lower():
+                    continue
+                ctx.memset(mark, 0)  # a fill kernel between two tables' rows: a profile of this run can tell them apart
+                t = time_kernel(ctx, o, args.kernel_iters, args.kernel_warmup, args.kernel_settle_ms)
+                rows.append(dict({"kernel": o.name, "bytes": o.nbytes}, **t.row(o.nbytes)))
+                log("%-52s %14d %9.2f us %8.1f GB/s %6.1f %%" % (o.name, o.nbytes, rows[-1]["us"], rows[-1]["GBps"], rows[-1]["pct_hbm_peak"]))
+            out[args.section] = rows
         print(json.dumps(out), flush=True)
         ctx.close()
         return

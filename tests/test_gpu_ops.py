@@ -270,7 +270,9 @@ SOFTMAX_SHAPES = [[1, 2, 3], [3, 28, 28], [16, 512, 512], [2, 12, 197, 197], [5,
                   [3, 1284], [3, 2052], [2, 3076], [2, 4608], [2, 6144], [2, 6148], [2, 12288],  # either side of every block width
                   [5, 384], [7, 640], [6, 896], [3, 1088], [9, 1152], [13, 320],  # a wavefront per row, last chunk partly filled
                   [7, 1030], [5, 2049], [3, 4097], [3, 9999], [2, 16381], [2, 16383], [2, 50257],  # rows that start anywhere: the aligned cover of a row in registers
-                  [2, 20000], [2, 32768], [1, 49152], [2, 65536], [2, 30522], [1, 65533], [1, 65540]]  # 6 to 16 float4 per thread up to 65536 elements, three passes above
+                  [2, 20000], [2, 32768], [1, 49152], [2, 65536], [2, 30522], [1, 65533], [1, 65540],  # 6 to 16 float4 per thread up to 65536 elements, three passes above
+                  [9, 1026], [6, 1281], [7, 1535], [5, 1537], [5, 1793], [4, 2047], [3, 2050],  # rows that start anywhere, a wavefront per row: 5 to 8 float4 per lane
+                  [2, 49156], [1, 52000], [2, 53248], [1, 53245], [1, 53249]]  # thirteen float4 per thread, and just past them
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
@@ -312,7 +314,9 @@ LN_SHAPES = [[1, 20, 10], [2, 197, 768], [3, 5, 197], [4, 1], [5, 64], [3, 1024]
              [3, 1284], [3, 2052], [2, 3076], [2, 4608], [2, 6144], [2, 6148], [2, 12288],  # either side of every block width
              [5, 384], [7, 640], [6, 896], [3, 1088], [9, 1152], [1, 512], [13, 320],  # a wavefront per row, last chunk partly filled, rows not a multiple of the block's four
              [7, 1030], [5, 2049], [3, 4097], [3, 9999], [2, 16383], [2, 50257],  # rows that start anywhere: the aligned cover of a row in registers
-             [2, 20000], [2, 32768], [1, 49152], [2, 65536], [2, 30522], [1, 65533], [1, 65540]]  # 6 to 16 float4 per thread up to 65536 elements, three passes above
+             [2, 20000], [2, 32768], [1, 49152], [2, 65536], [2, 30522], [1, 65533], [1, 65540],  # 6 to 16 float4 per thread up to 65536 elements, three passes above
+             [9, 1025], [6, 1281], [7, 1535], [5, 1537], [5, 1793], [4, 2047], [3, 2050],  # rows that start anywhere, a wavefront per row: 5 to 8 float4 per lane
+             [2, 49156], [1, 52000], [2, 53248], [1, 53245], [1, 53249]]  # thirteen float4 per thread, and just past them
 
 
 @pytest.mark.parametrize("shape", LN_SHAPES)
@@ -353,7 +357,7 @@ def test_flat_operators_on_large_views_that_start_off_a_boundary(ctx, oracle, ca
         ctx.free(t)
 
 
-UNALIGNED_ROWS = [(7, 768), (5, 197), (3, 1280), (2, 4096), (2, 8192), (3, 1000), (9, 64)]
+UNALIGNED_ROWS = [(7, 768), (5, 197), (3, 1280), (2, 4096), (2, 8192), (3, 1000), (9, 64), (5, 2048), (6, 1500), (2, 51200)]
 
 
 @pytest.mark.parametrize("rows,length", UNALIGNED_ROWS)
