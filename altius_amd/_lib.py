@@ -201,6 +201,7 @@ def _declare_graph(L):
     f("ahip_session_builder_with_profiling_enabled", [c_void_p, c_int])
     f("ahip_session_builder_with_device", [c_void_p, c_int])
     f("ahip_session_builder_with_graph_replay", [c_void_p, c_int])
+    f("ahip_session_builder_with_device_timing", [c_void_p, c_int])
     f("ahip_session_builder_with_gemm_algorithm", [c_void_p, c_int])
     f("ahip_session_builder_with_fused_attention", [c_void_p, c_int])
     f("ahip_session_builder_with_strided_views", [c_void_p, c_int])

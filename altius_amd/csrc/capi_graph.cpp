@@ -33,6 +33,7 @@ struct ahip_session_builder {
     int gemm_algorithm = AHIP_GEMM_FP32;
     bool strided_views = true;
     bool fused_attention = false;
+    bool device_timing = true;
 };
 // InterpreterSession::run takes &self and keeps its intermediates in a map per calling thread
 // (crates/session_interpreter/src/session.rs:56,75-78), so several threads may run one session at once.  Here a
@@ -75,7 +76,7 @@ int acquire_lane(ahip_session *session, size_t *index, std::shared_ptr<HipSessio
     lock.unlock();
     const ahip_session_builder &b = session->settings;
     HipSessionBuilder hb(session->view.m);
-    hb.with_intra_op_num_threads(b.threads).with_profiling_enabled(b.profiling).with_device(b.device).with_graph_replay(b.graph_replay)
+    hb.with_intra_op_num_threads(b.threads).with_profiling_enabled(b.profiling).with_device(b.device).with_graph_replay(b.graph_replay).with_device_timing(b.device_timing)
         .with_gemm_algorithm(b.gemm_algorithm).with_strided_views(b.strided_views).with_fused_attention(b.fused_attention);
     SessionError err;
     std::shared_ptr<HipSession> lane;
@@ -687,6 +688,14 @@ int ahip_session_builder_with_device(ahip_session_builder *builder, int device) 
     return altius::caught_at_boundary("ahip_session_builder_with_device");
 }
 
+int ahip_session_builder_with_device_timing(ahip_session_builder *builder, int enable) try {
+    if (!builder) return fail(AHIP_ERR_ARG, "ahip_session_builder_with_device_timing: null builder");
+    builder->device_timing = enable != 0;
+    return AHIP_OK;
+} catch (...) {
+    return altius::caught_at_boundary("ahip_session_builder_with_device_timing");
+}
+
 int ahip_session_builder_with_graph_replay(ahip_session_builder *builder, int enable) try {
     if (!builder) return fail(AHIP_ERR_ARG, "null builder");
     builder->graph_replay = enable != 0;
@@ -741,7 +750,7 @@ int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **ses
     if (!builder || !session) return fail(AHIP_ERR_ARG, "ahip_session_builder_build: null argument");
     *session = nullptr;
     HipSessionBuilder b(builder->model);
-    b.with_intra_op_num_threads(builder->threads).with_profiling_enabled(builder->profiling).with_device(builder->device).with_graph_replay(builder->graph_replay).with_gemm_algorithm(builder->gemm_algorithm).with_strided_views(builder->strided_views).with_fused_attention(builder->fused_attention);
+    b.with_intra_op_num_threads(builder->threads).with_profiling_enabled(builder->profiling).with_device(builder->device).with_graph_replay(builder->graph_replay).with_gemm_algorithm(builder->gemm_algorithm).with_strided_views(builder->strided_views).with_fused_attention(builder->fused_attention).with_device_timing(builder->device_timing);
     SessionError err;
     std::unique_ptr<HipSession> s = b.build(&err);
     if (!s) return fail(err.code(), err.to_string());
@@ -753,6 +762,7 @@ int ahip_session_builder_build(ahip_session_builder *builder, ahip_session **ses
     out->settings.profiling = builder->profiling;
     out->settings.device = builder->device;
     out->settings.graph_replay = builder->graph_replay;
+    out->settings.device_timing = builder->device_timing;
     out->settings.gemm_algorithm = builder->gemm_algorithm;
     out->settings.strided_views = builder->strided_views;
     out->settings.fused_attention = builder->fused_attention;

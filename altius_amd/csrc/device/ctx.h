@@ -28,6 +28,9 @@ struct PackedOperand {
     size_t bytes;
 };
 
+// The streaming threshold of a session's context (see DeviceCtx::nt_threshold_bytes).
+constexpr size_t SESSION_NT_THRESHOLD_BYTES = (size_t)128 << 20;
+
 // One context = one device + one stream.  All work issued through a context is
 // ordered on that stream.  A context is not thread-safe; use one per thread.
 struct DeviceCtx {
@@ -42,8 +45,9 @@ struct DeviceCtx {
     // kernel that can raise one has run.
     int *flags = nullptr;
     bool flags_armed = false;
-    // Tensors of at least this many bytes are streamed with non-temporal accesses.
-    size_t nt_threshold_bytes = (size_t)128 << 20;
+    // Tensors of at least this many bytes are streamed with non-temporal accesses (a session raises it to
+    // SESSION_NT_THRESHOLD_BYTES: its results are read by the node behind, out of the Infinity Cache if they fit).
+    size_t nt_threshold_bytes = (size_t)64 << 20;
     size_t nt_load_threshold_bytes = (size_t)16 << 20;
     // Chains of element-wise steps that were instantiated at compile time run as straight-line code;
     // switched off, every chain takes the interpreting kernel (tests compare the two).

@@ -199,6 +199,144 @@ __global__ __launch_bounds__(BLOCK) void transpose_tiled_vec4(uint32_t *__restri
     }
 }
 
+// The 64 x 64 patch of 4-byte elements when only one side lines up for 16-byte accesses (an odd R extent:
+// [50257, 768] -> [768, 50257]; or an odd C extent the other way round): that side moves float4s as in
+// transpose_tiled_vec4, the other single elements as in transpose_tiled.  (16-byte accesses on 4-byte boundaries are
+// no way out here: a wavefront's store is four separate 256-byte pieces, and cut at odd addresses they run at half
+// the speed of the single elements.)
+template <bool LOAD4, bool NT>
+__global__ __launch_bounds__(BLOCK) void transpose_tiled_mixed(uint32_t *__restrict__ out, const uint32_t *__restrict__ in, TransGeom g) {
+    __shared__ uint32_t tile[TILE][TILE + 1];
+    uint32_t rest = blockIdx.z, src0 = 0, dst0 = 0;
+#pragma unroll
+    for (int d = 0; d < MAX_RANK; d++) {
+        if (d < g.brank) {
+            const uint32_t q = g.bdims[d].div(rest);
+            const uint32_t r = rest - q * g.bdims[d].d;
+            src0 += r * g.b_in_str[d];
+            dst0 += r * g.b_out_str[d];
+            rest = q;
+        }
+    }
+    uint32_t by = blockIdx.y + blockIdx.x;  // tiles dealt diagonally, see transpose_tiled_vec4
+    by = by >= gridDim.y ? by % gridDim.y : by;
+    const uint32_t c0 = blockIdx.x * TILE, r0 = by * TILE;
+    const uint32_t q4 = threadIdx.x & 15, line = threadIdx.x >> 4;           // the float4 side: 16 float4 per line, 16 lines per pass
+    const uint32_t tx = threadIdx.x & (TILE - 1), ty = threadIdx.x / TILE;  // the element side: 64 x 4
+    if (LOAD4) {
+        u32x4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t r = r0 + line + 16 * k, c = c0 + 4 * q4;
+            v[k] = u32x4{0, 0, 0, 0};
+            if (r < g.r_len && c < g.c_len) {
+                const u32x4 *p = reinterpret_cast<const u32x4 *>(in + src0 + (size_t)r * g.r_in_str + c);
+                v[k] = NT ? __builtin_nontemporal_load(p) : *p;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            uint32_t *row = &tile[line + 16 * k][4 * q4];
+            row[0] = v[k].x, row[1] = v[k].y, row[2] = v[k].z, row[3] = v[k].w;
+        }
+    } else {
+        uint32_t v[TILE / (BLOCK / TILE)];
+#pragma unroll
+        for (int k = 0; k < TILE; k += BLOCK / TILE) {
+            const uint32_t r = r0 + ty + k, c = c0 + tx;
+            if (r < g.r_len && c < g.c_len) v[k / (BLOCK / TILE)] = in[src0 + (size_t)r * g.r_in_str + c];
+        }
+#pragma unroll
+        for (int k = 0; k < TILE; k += BLOCK / TILE) tile[ty + k][tx] = v[k / (BLOCK / TILE)];
+    }
+    __syncthreads();
+    if (LOAD4) {
+#pragma unroll 4
+        for (int k = 0; k < TILE; k += BLOCK / TILE) {
+            const uint32_t c = c0 + ty + k, r = r0 + tx;
+            if (r < g.r_len && c < g.c_len) out[dst0 + (size_t)c * g.c_out_str + r] = tile[tx][ty + k];
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t c = c0 + line + 16 * k, r = r0 + 4 * q4;
+            if (r < g.r_len && c < g.c_len) {
+                const uint32_t col = line + 16 * k;
+                const u32x4 w = {tile[4 * q4][col], tile[4 * q4 + 1][col], tile[4 * q4 + 2][col], tile[4 * q4 + 3][col]};
+                u32x4 *p = reinterpret_cast<u32x4 *>(out + dst0 + (size_t)c * g.c_out_str + r);
+                if (NT) __builtin_nontemporal_store(w, p);
+                else *p = w;
+            }
+        }
+    }
+}
+
+// Matrices whose transposed image is dense ([.., R, C] -> [.., C, R] with R of up to a thousand elements: 197 tokens x
+// 768 channels) but too large for one block: a block takes a panel of TC columns, all R rows of them.  It reads R
+// segments of TC elements (whole 128-byte lines with TC = 32) and writes one dense span of TC x R elements, which
+// starts and ends on a 128-byte boundary whatever R is: 16-byte accesses on both sides and no line written by two
+// blocks, where 64 x 64 patches leave 5 of the last patch's 64 rows in use and cut every output row at odd addresses.
+// LDS holds the panel transposed, [TC][pitch] with an odd pitch.
+constexpr int PANEL = 32;
+template <int TC, bool NT>
+__global__ __launch_bounds__(BLOCK) void transpose_panel(uint32_t *__restrict__ out, const uint32_t *__restrict__ in, TransGeom g, uint32_t pitch,
+                                                         FastDiv rdiv) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    uint32_t *lds = reinterpret_cast<uint32_t *>(smem_raw);  // element (c, r) of the panel at c * pitch + r
+    uint32_t rest = blockIdx.y, src0 = 0, dst0 = 0;
+#pragma unroll
+    for (int d = 0; d < MAX_RANK; d++) {
+        if (d < g.brank) {
+            const uint32_t q = g.bdims[d].div(rest);
+            const uint32_t r = rest - q * g.bdims[d].d;
+            src0 += r * g.b_in_str[d];
+            dst0 += r * g.b_out_str[d];
+            rest = q;
+        }
+    }
+    const uint32_t c0 = blockIdx.x * TC;
+    constexpr uint32_t Q = TC / 4;                 // float4 per row segment
+    const uint32_t n4 = g.r_len * Q;               // float4 of the panel, on either side
+    const uint32_t *src = in + src0 + c0;
+    uint32_t *dst = out + dst0 + (size_t)c0 * g.r_len;
+    constexpr int U = 4;  // loads requested before the first is scattered into LDS
+    for (uint32_t i0 = threadIdx.x; i0 < n4; i0 += U * BLOCK) {
+        u32x4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t i = i0 + u * BLOCK;
+            if (i < n4) {
+                const u32x4 *p = reinterpret_cast<const u32x4 *>(src + (size_t)(i / Q) * g.r_in_str + 4 * (i % Q));
+                v[u] = NT ? __builtin_nontemporal_load(p) : *p;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t i = i0 + u * BLOCK;
+            if (i < n4) {
+                const uint32_t r = i / Q, c = 4 * (i % Q);
+                lds[c * pitch + r] = v[u].x, lds[(c + 1) * pitch + r] = v[u].y, lds[(c + 2) * pitch + r] = v[u].z, lds[(c + 3) * pitch + r] = v[u].w;
+            }
+        }
+    }
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < n4; i += BLOCK) {
+        uint32_t c = rdiv.div(4 * i), r = 4 * i - c * g.r_len;  // the span is [c][r]
+        uint32_t w[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            w[k] = lds[c * pitch + r];
+            if (++r == g.r_len) {
+                r = 0;
+                c++;
+            }
+        }
+        const u32x4 t = {w[0], w[1], w[2], w[3]};
+        if (NT) __builtin_nontemporal_store(t, reinterpret_cast<u32x4 *>(dst + 4 * (size_t)i));
+        else *reinterpret_cast<u32x4 *>(dst + 4 * (size_t)i) = t;
+    }
+}
+
 // Batched transpose of small matrices that are contiguous on both sides (attention's K^T:
 // [.., 197, 64] -> [.., 64, 197]).  One block moves one whole r_len x c_len matrix: it reads the
 // matrix as one contiguous span, scatters it into LDS transposed, and writes the result as one
@@ -723,6 +861,24 @@ int launch_transpose(DeviceCtx &ctx, void *out, const void *in, int elem_size, i
             }
         }
     }
+    // Dense transposed matrices with a short R axis, too large for one block: panels of 32 columns (with 16, which a
+    // longer R axis would need to fit LDS, the segments read are half lines and the 64 x 64 patches are ahead).
+    if (elem_size == 4 && g.c_out_str == g.r_len && g.c_len % PANEL == 0 && g.r_in_str % 4 == 0 && aligned16(out) && aligned16(in) && batches <= 65535 &&
+        (size_t)PANEL * (g.r_len | 1u) * 4 <= 64 * 1024) {
+        bool lines_up = true;
+        for (int i = 0; i < g.brank; i++) lines_up = lines_up && g.b_in_str[i] % 4 == 0 && g.b_out_str[i] % 4 == 0;
+        if (lines_up) {
+            const uint32_t pitch = g.r_len | 1u;
+            const dim3 grid((unsigned)(g.c_len / PANEL), (unsigned)batches);
+            const size_t lds_bytes = (size_t)PANEL * pitch * 4;
+            const FastDiv rdiv = make_fastdiv(g.r_len);
+            uint32_t *o = static_cast<uint32_t *>(out);
+            const uint32_t *x = static_cast<const uint32_t *>(in);
+            if (ctx.streaming(total * 4)) hipLaunchKernelGGL((transpose_panel<PANEL, true>), grid, dim3(BLOCK), lds_bytes, ctx.stream, o, x, g, pitch, rdiv);
+            else hipLaunchKernelGGL((transpose_panel<PANEL, false>), grid, dim3(BLOCK), lds_bytes, ctx.stream, o, x, g, pitch, rdiv);
+            return ctx.check(hipGetLastError(), "transpose_panel launch");
+        }
+    }
     const size_t gx = (g.c_len + TILE - 1) / TILE, gy = (g.r_len + TILE - 1) / TILE;
     if (gy > 65535 || batches > 65535) {
         // Grid limits: fall back to the one-element-per-thread copy (still correct, reads uncoalesced).
@@ -748,10 +904,19 @@ int launch_transpose(DeviceCtx &ctx, void *out, const void *in, int elem_size, i
         hipLaunchKernelGGL((transpose_tiled<uint8_t>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint8_t *>(out),
                            static_cast<const uint8_t *>(in), g);
         break;
-    case 4:
-        hipLaunchKernelGGL((transpose_tiled<uint32_t>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint32_t *>(out),
-                           static_cast<const uint32_t *>(in), g);
+    case 4: {
+        bool in4 = g.c_len % 4 == 0 && g.r_in_str % 4 == 0 && aligned16(in), out4 = g.r_len % 4 == 0 && g.c_out_str % 4 == 0 && aligned16(out);
+        for (int i = 0; i < g.brank; i++) in4 = in4 && g.b_in_str[i] % 4 == 0, out4 = out4 && g.b_out_str[i] % 4 == 0;
+        uint32_t *o = static_cast<uint32_t *>(out);
+        const uint32_t *x = static_cast<const uint32_t *>(in);
+        const bool nt = ctx.streaming(total * 4);
+        if (in4 && nt) hipLaunchKernelGGL((transpose_tiled_mixed<true, true>), grid, dim3(BLOCK), 0, ctx.stream, o, x, g);
+        else if (in4) hipLaunchKernelGGL((transpose_tiled_mixed<true, false>), grid, dim3(BLOCK), 0, ctx.stream, o, x, g);
+        else if (out4 && nt) hipLaunchKernelGGL((transpose_tiled_mixed<false, true>), grid, dim3(BLOCK), 0, ctx.stream, o, x, g);
+        else if (out4) hipLaunchKernelGGL((transpose_tiled_mixed<false, false>), grid, dim3(BLOCK), 0, ctx.stream, o, x, g);
+        else hipLaunchKernelGGL((transpose_tiled<uint32_t>), grid, dim3(BLOCK), 0, ctx.stream, o, x, g);
         break;
+    }
     default:
         hipLaunchKernelGGL((transpose_tiled<uint64_t>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint64_t *>(out),
                            static_cast<const uint64_t *>(in), g);

@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <chrono>
+#include <cstdlib>
 #include <functional>
 #include <limits>
 
@@ -106,6 +107,7 @@ std::unique_ptr<HipSession> HipSessionBuilder::build(SessionError *err) {
     s->enable_profiling_ = enable_profiling_;
     s->intra_op_num_threads_ = intra_op_num_threads_;
     s->graph_replay_ = graph_replay_ && !enable_profiling_;
+    s->device_timing_ = device_timing_;
 
     ShapeError serr;
     if (!infer_shapes(s->model_, &s->inferred_, nullptr, &serr)) {
@@ -122,6 +124,7 @@ std::unique_ptr<HipSession> HipSessionBuilder::build(SessionError *err) {
         return nullptr;
     }
     // Every input of a node was written by the node in front and is, up to the size of the caches, still in them.
+    if (!getenv("AHIP_STREAMING_THRESHOLD_MIB")) s->ctx_.nt_threshold_bytes = SESSION_NT_THRESHOLD_BYTES;
     s->ctx_.nt_load_threshold_bytes = s->ctx_.nt_threshold_bytes;
     if (gemm_algorithm_ != AHIP_GEMM_AUTO && gemm_algorithm_ != AHIP_GEMM_FP32 && gemm_algorithm_ != AHIP_GEMM_BF16X3) {
         destroy_device_ctx(&s->ctx_);
@@ -328,7 +331,7 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
     }
 
     // The hot loop (session.rs:86-92).
-    (void)hipEventRecord(span_begin_, ctx_.stream);
+    if (device_timing_) (void)hipEventRecord(span_begin_, ctx_.stream);
     for (size_t i = 0; i < plan_.size(); i++) {
         if (!run_node(plan_[i].node_id, values, err)) return finish(false);
         if (enable_profiling_) (void)hipEventRecord(events[i + 1], ctx_.stream);
@@ -338,7 +341,7 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
             if (std::find(g.outputs.begin(), g.outputs.end(), v) == g.outputs.end()) values.erase(v);
     }
 
-    (void)hipEventRecord(span_end_, ctx_.stream);
+    if (device_timing_) (void)hipEventRecord(span_end_, ctx_.stream);
 
     // Download the outputs (session.rs:127-133).
     for (ValueId v : g.outputs) {
@@ -367,7 +370,7 @@ bool HipSession::run(const std::vector<Tensor> &inputs, std::vector<Tensor> *out
         return finish(fail_code(err, rc, ctx_.last_error));
     }
     float span_ms = 0;
-    last_device_ms_ = hipEventElapsedTime(&span_ms, span_begin_, span_end_) == hipSuccess ? span_ms : 0;
+    last_device_ms_ = device_timing_ && hipEventElapsedTime(&span_ms, span_begin_, span_end_) == hipSuccess ? span_ms : 0;
     if (enable_profiling_) {
         for (size_t i = 0; i < plan_.size(); i++) {
             float ms = 0;
@@ -409,13 +412,13 @@ bool HipSession::run_device(const std::vector<DeviceTensor> &inputs, std::vector
     }
     // A failed run leaves nothing behind; blocks released while kernels are still queued are only
     // handed to later work on the same stream.
-    (void)hipEventRecord(span_begin_, ctx_.stream);
+    if (device_timing_) (void)hipEventRecord(span_begin_, ctx_.stream);
     for (size_t i = 0; i < plan_.size(); i++) {
         if (!run_node(plan_[i].node_id, values, err)) return false;
         for (ValueId v : plan_[i].free_vals)
             if (std::find(g.outputs.begin(), g.outputs.end(), v) == g.outputs.end()) values.erase(v);
     }
-    (void)hipEventRecord(span_end_, ctx_.stream);
+    if (device_timing_) (void)hipEventRecord(span_end_, ctx_.stream);
     for (ValueId v : g.outputs) {
         const DeviceTensor *d = nullptr;
         auto it = values.find(v);
@@ -431,7 +434,7 @@ bool HipSession::run_device(const std::vector<DeviceTensor> &inputs, std::vector
         }
         outputs->push_back(*d);
     }
-    span_pending_ = true;
+    span_pending_ = device_timing_;
     last_run_ms_ = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     return true;
 }
@@ -558,9 +561,9 @@ bool HipSession::replay(CapturedRun &run, const std::vector<Tensor> &inputs, std
             rc = ctx_.check(hipMemcpyAsync(run.inputs[i].ptr, inputs[i].data_as_bytes(), run.inputs[i].nbytes(), hipMemcpyHostToDevice,
                                            ctx_.stream),
                             "hipMemcpyAsync(input)");
-    (void)hipEventRecord(span_begin_, ctx_.stream);
+    if (device_timing_) (void)hipEventRecord(span_begin_, ctx_.stream);
     if (!rc) rc = ctx_.check(hipGraphLaunch(run.exec, ctx_.stream), "hipGraphLaunch");
-    (void)hipEventRecord(span_end_, ctx_.stream);
+    if (device_timing_) (void)hipEventRecord(span_end_, ctx_.stream);
     for (size_t i = 0; i < run.outputs.size() && !rc; i++) {
         Tensor t = Tensor::uninit_of_type(run.outputs[i].elem_ty, run.outputs[i].dims, pinned_host_block);
         if (!t.has_data()) {
@@ -585,14 +588,14 @@ bool HipSession::replay(CapturedRun &run, const std::vector<Tensor> &inputs, std
         return fail_code(err, rc, ctx_.last_error);
     }
     float span_ms = 0;
-    last_device_ms_ = hipEventElapsedTime(&span_ms, span_begin_, span_end_) == hipSuccess ? span_ms : 0;
+    last_device_ms_ = device_timing_ && hipEventElapsedTime(&span_ms, span_begin_, span_end_) == hipSuccess ? span_ms : 0;
     graph_replays_++;
     return true;
 }
 
 bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, SessionError *err) {
     const Node &node = model_.graph.nodes[id];
-    const std::string opname = node.op.name();
+    auto opname = [&]() { return std::string(node.op.name()); };  // for messages only
 
     // Inputs: run-time values first, then initializers.  An input whose value is never produced
     // and carries the empty name is an omitted optional input (the reference binds a dummy tensor).
@@ -613,9 +616,9 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
             in.push_back(nullptr);
             continue;
         }
-        return fail(err, SessionError::Message, opname + ": an input value is missing");
+        return fail(err, SessionError::Message, opname() + ": an input value is missing");
     }
-    if (node.outputs.empty()) return fail(err, SessionError::Message, opname + ": node without outputs");
+    if (node.outputs.empty()) return fail(err, SessionError::Message, opname() + ": node without outputs");
     // Strided views are read in place by the operators that can; every other reader gets a dense
     // copy, which also replaces the view for whoever reads the value later.
     if (!reads_views(node.op.kind))
@@ -637,12 +640,14 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
 
     // Output shapes: inferred at build time if possible, else now (session.rs:149-158).  Operands
     // whose contents decide a shape are read from their host copy, fetched on demand.
-    Op op = node.op;
-    std::vector<TypedFixedShape> shapes;
+    Op inferred_op;
+    std::vector<TypedFixedShape> inferred_shapes;
+    const Op *op_used = &inferred_op;
+    const std::vector<TypedFixedShape> *shapes_used = &inferred_shapes;
     auto cached = inferred_.find(id);
-    if (cached != inferred_.end()) {
-        op = cached->second.first;
-        shapes = cached->second.second;
+    if (cached != inferred_.end()) {  // no copies on this path: it is the one every node of a planned graph takes
+        op_used = &cached->second.first;
+        shapes_used = &cached->second.second;
     } else if (capturing_) {
         capture_refused_ = true;
         return fail(err, SessionError::Message, "graph capture: a node's shape is not known before the run");
@@ -655,15 +660,17 @@ bool HipSession::run_node(NodeId id, std::map<ValueId, DeviceTensor> &values, Se
             std::vector<const Tensor *> ptrs;
             for (auto &m : meta) ptrs.push_back(&m);
             ShapeError serr;
-            op = node.op;
-            if (compute_output_shapes(model_, op, ptrs, node.outputs.size(), &shapes, &serr)) break;
+            inferred_op = node.op;
+            if (compute_output_shapes(model_, inferred_op, ptrs, node.outputs.size(), &inferred_shapes, &serr)) break;
             if (!serr.needs_data || attempt > 0) return fail(err, SessionError::Shape, serr.message);
             // Read back the small operands (shape vectors, Resize scales) and try once more.
             for (size_t i = 1; i < in.size(); i++)
                 if (in[i] && !in[i]->host && in[i]->dims.total_elems() <= 4096 && !fetch_host(in[i], err)) return false;
         }
     }
-    if (shapes.size() < node.outputs.size()) return fail(err, SessionError::Message, opname + ": output count mismatch");
+    const Op &op = *op_used;
+    const std::vector<TypedFixedShape> &shapes = *shapes_used;
+    if (shapes.size() < node.outputs.size()) return fail(err, SessionError::Message, opname() + ": output count mismatch");
 
     std::vector<DeviceTensor> outs;
     values_ = &values;
@@ -997,7 +1004,11 @@ bool HipSession::run_fused_elemwise(const Node &node, const Op &op, const std::v
 
 bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector<DeviceTensor *> &in,
                                const std::vector<TypedFixedShape> &shapes, std::vector<DeviceTensor> *outs, SessionError *err) {
-    const std::string opname = op.name();
+    struct LazyName {  // the operator's name, made where a message needs it
+        const Op &op;
+        std::string operator+(const char *rest) const { return std::string(op.name()) + rest; }
+        std::string operator+(const std::string &rest) const { return std::string(op.name()) + rest; }
+    } opname{op};
     auto need = [&](size_t n) {
         if (in.size() >= n) {
             bool all = true;

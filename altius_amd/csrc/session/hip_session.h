@@ -242,6 +242,7 @@ private:
     double last_run_ms_ = 0;
     double last_device_ms_ = 0;
     bool span_pending_ = false;  // run_device() recorded the span; synchronize() reads it
+    bool device_timing_ = true;  // record the span at all
     hipEvent_t span_begin_ = nullptr, span_end_ = nullptr;  // bracket the kernels of a run
     std::mutex mutex_;
     bool graph_replay_ = false;
@@ -330,6 +331,13 @@ public:
         fused_attention_ = enable;
         return *this;
     }
+    // Not in the reference: whether a run is bracketed by two events on the session's stream, which is what
+    // last_device_ms() reports (default on).  Off saves two event records per run, on the host and in the queue: a
+    // caller that runs small graphs back to back and does not ask for the device time turns it off.
+    HipSessionBuilder &with_device_timing(bool enable) {
+        device_timing_ = enable;
+        return *this;
+    }
     // Not in the reference: which GPU to run on (default 0).
     HipSessionBuilder &with_device(int device) {
         device_ = device;
@@ -348,6 +356,7 @@ private:
     int gemm_algorithm_ = AHIP_GEMM_FP32;
     bool strided_views_ = true;
     bool fused_attention_ = false;
+    bool device_timing_ = true;
 };
 
 }  // namespace altius

@@ -74,10 +74,9 @@ class HipSession:
         tensors_out = [Tensor(ctypes.c_void_p(outs[i])) for i in range(n.value)]
         return [t.numpy() if copy else t.view() for t in tensors_out]
 
-    def run_device(self, inputs):
-        """inputs: (device pointer, shape, numpy dtype) triples, positional in graph.inputs order, on the
-        session's GPU.  Enqueues the plan and returns DeviceTensors without waiting for the GPU; call
-        synchronize() before reading them from another stream or copying them out."""
+    def prepare_device_inputs(self, inputs):
+        """The C arguments of run_device for these (device pointer, shape, numpy dtype) triples, built once: a loop that
+        calls the same graph on the same buffers passes them to run_device_prepared and pays for the call alone."""
         n_in = len(inputs)
         ptrs = (ctypes.c_void_p * max(n_in, 1))(*[int(p) for p, _, _ in inputs])
         elem = (ctypes.c_int * max(n_in, 1))(*[_ELEM_OF[np.dtype(dt)] for _, _, dt in inputs])
@@ -85,10 +84,18 @@ class HipSession:
         dim_arrays = [(ctypes.c_int64 * max(len(shape), 1))(*[int(d) for d in shape]) for _, shape, _ in inputs]
         dims = (ctypes.POINTER(ctypes.c_int64) * max(n_in, 1))(*[ctypes.cast(a, ctypes.POINTER(ctypes.c_int64)) for a in dim_arrays])
         cap = 16
-        outs = (ctypes.c_void_p * cap)()
-        n = ctypes.c_int()
+        return (n_in, ptrs, elem, ranks, dims, cap, (ctypes.c_void_p * cap)(), ctypes.c_int(), dim_arrays)
+
+    def run_device_prepared(self, prepared):
+        n_in, ptrs, elem, ranks, dims, cap, outs, n, _ = prepared
         check(self.L.ahip_session_run_device(self.handle, n_in, ptrs, elem, ranks, dims, cap, outs, ctypes.byref(n)))
         return [DeviceTensor(ctypes.c_void_p(outs[i])) for i in range(n.value)]
+
+    def run_device(self, inputs):
+        """inputs: (device pointer, shape, numpy dtype) triples, positional in graph.inputs order, on the
+        session's GPU.  Enqueues the plan and returns DeviceTensors without waiting for the GPU; call
+        synchronize() before reading them from another stream or copying them out."""
+        return self.run_device_prepared(self.prepare_device_inputs(inputs))
 
     def synchronize(self):
         check(self.L.ahip_session_synchronize(self.handle))
@@ -159,6 +166,11 @@ class HipSessionBuilder:
 
     def with_profiling_enabled(self, enable):
         check(self.L.ahip_session_builder_with_profiling_enabled(self.handle, int(bool(enable))))
+        return self
+
+    def with_device_timing(self, enable=True):
+        """Bracket every run by two events so that last_device_ms() can report the kernels' time (default on)."""
+        check(self.L.ahip_session_builder_with_device_timing(self.handle, int(bool(enable))))
         return self
 
     def with_graph_replay(self, enable=True):

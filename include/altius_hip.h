@@ -334,10 +334,12 @@ int ahip_attention(ahip_ctx *ctx, float *o, const float *q, const float *k, cons
 #define AHIP_GEMM_FP32 1
 #define AHIP_GEMM_BF16X3 2
 int ahip_gemm_set_algorithm(ahip_ctx *ctx, int algorithm);
-/* Tensors of at least `bytes` bytes are read and written with non-temporal 16-byte accesses (they would not be
- * found in the 256 MB Infinity Cache by the next kernel anyway); smaller ones are left to the caches.
- * Default 128 MiB.  (size_t)-1 switches the hint off, 0 applies it to everything.  No counterpart in the
- * reference. */
+/* Tensors of at least `bytes` bytes are read and written with non-temporal 16-byte accesses; smaller ones are
+ * left to the caches.  Default 64 MiB for a context of its own, whose caller hands over tensors from elsewhere
+ * and reads results nobody knows when (Gelu over 77 MB in, 77 MB out: 70 % of the HBM peak become 73.5 %); a
+ * session keeps 128 MiB for its context, because the node behind finds a smaller result in the 256 MB Infinity
+ * Cache (a chain of five element-wise nodes over 77 MB tensors: 127 us against 140 us).  (size_t)-1 switches the
+ * hint off, 0 applies it to everything.  No counterpart in the reference. */
 int ahip_set_streaming_threshold(ahip_ctx *ctx, size_t bytes);
 /* The element-wise operators (ahip_unary, ahip_binary) read a dense operand of at least `bytes` bytes with
  * non-temporal loads while storing the result the ordinary way, so that the next kernel finds it in the caches:
@@ -595,6 +597,12 @@ int ahip_session_builder_with_device(ahip_session_builder *builder, int device);
  * run instead of one per node).  Results are those of the node-by-node run.  Graphs whose shapes
  * or operands need the host during the run, and profiled sessions, keep running node by node. */
 int ahip_session_builder_with_graph_replay(ahip_session_builder *builder, int enable);
+/* Not in the reference (its run() times itself with Instant::now() only when profiling is on,
+ * crates/session_interpreter/src/session.rs:74,117-125): with enable == 0 a run is no longer bracketed by
+ * two events on the session's stream, and ahip_session_last_device_ms reports 0.  Default on.  Two event
+ * records per run cost a few microseconds on the host and in the queue, which a caller of small graphs
+ * that does not read the device time can do without. */
+int ahip_session_builder_with_device_timing(ahip_session_builder *builder, int enable);
 /* Not in the reference: the kernel the session's large single-batch MatMul / Gemm products take
  * (AHIP_GEMM_FP32, the default, AHIP_GEMM_AUTO or AHIP_GEMM_BF16X3; see ahip_gemm_set_algorithm).  The
  * default keeps the reference's semantics for every operand value (compute_mat_mul, session.rs:621-684: an

@@ -50,7 +50,7 @@ def canned_result(batch=256, us=12345.67):
     for sh, perm in bench.SHAPE_SWEEP_TRANSPOSES:
         shape_names.append("Transpose %s -> %s" % (sh, tuple(perm)))
     shapes = [dict({"kernel": k, "bytes": n}, **_timing(n, us)) for k in shape_names]
-    other_names = ["cfg0 Add [1,197,768]+[768]", "cfg1 Softmax [8,12,197,197]", "cfg1 LayerNorm [8,197,768]",
+    other_names = ["floor Relu [64]", "cfg0 Add [1,197,768]+[768]", "cfg1 Softmax [8,12,197,197]", "cfg1 LayerNorm [8,197,768]",
                    "cfg2 LayerNorm (fused) [32,197,768]", "cfg2 ReduceMean(-1) [32,197,768]", "cfg2 Sub [32,197,768]-[32,197,1]",
                    "cfg2 Pow(.,2) [32,197,768]", "cfg2 Div [32,197,768]/[32,197,1]", "cfg2 Mul gamma [32,197,768]*[768]",
                    "cfg3 Gelu [32,197,3072]", "cfg3 Erf [32,197,3072]", "cfg3 Mul [32,197,3072]*[32,197,3072]",
@@ -60,7 +60,7 @@ def canned_result(batch=256, us=12345.67):
                    "cfg3 erf-GELU chain, 5 nodes", "cfg3 after fuse_gelu, 1 node", "cfg3 chain after fuse_elemwise_ops, 1 node",
                    "cfg3 squeeze-excite, 3 nodes"]
     graphs = [{"graph": g, "algorithmic_bytes": n, "kernels_us": 1234.5, "run_ms_with_pcie": 12.345, "kernels_us_graph_replay": 1234.5,
-               "run_ms_with_pcie_graph_replay": 12.345, "kernels_GBps": 4283.6, "run_device_us": 1234.5} for g in graph_names]
+               "run_ms_with_pcie_graph_replay": 12.345, "kernels_GBps": 4283.6, "run_device_us": 1234.5, "run_device_enqueue_us": 123.4} for g in graph_names]
     per = {"Add": 32184.7, "Softmax": 12438.1, "ReduceMax": 82546.8, "Div": 10542.4}
     return {
         "metric": "per-op HBM GB/s and % of MI355X peak; us/call vs CPU interpreter", "value": 6421.3, "unit": "GB/s", "n_gpus": 1,
@@ -97,7 +97,7 @@ def test_default_line_fits_and_keeps_every_section():
     assert len(out["per_kernel"]["rows"]) == 5 and len(out["per_kernel"]["cols"]) == len(out["per_kernel"]["rows"][0])
     assert len(out["listed_ops"]["rows"]) == 13
     assert len(out["row_sweep"]["rows"]) == len(bench.ROW_SWEEP_LENGTHS) and len(out["row_sweep"]["cols"]) == 4
-    assert len(out["other_configs"]["rows"]) == 15 and len(out["other_configs"]["graphs"]) == 7
+    assert len(out["other_configs"]["rows"]) == 16 and len(out["other_configs"]["graphs"]) == 7
     n_shapes = sum(len(g["rows"]) * (len(g["cols"]) - 1) for g in out["shape_sweep"].values())
     assert n_shapes == 2 * len(bench.SHAPE_SWEEP_MIDDLE) + 3 * len(bench.SHAPE_SWEEP_ODD_ROWS) + 1 + len(bench.SHAPE_SWEEP_TRANSPOSES)
 
