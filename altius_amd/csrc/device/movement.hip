@@ -278,8 +278,9 @@ __global__ __launch_bounds__(BLOCK) void transpose_tiled_mixed(uint32_t *__restr
 // blocks, where 64 x 64 patches leave 5 of the last patch's 64 rows in use and cut every output row at odd addresses.
 // LDS holds the panel transposed, [TC][pitch] with an odd pitch.
 constexpr int PANEL = 32;
+constexpr int PANEL_BLOCK = 512;  // 197 rows of 8 float4: one round of four loads per thread
 template <int TC, bool NT>
-__global__ __launch_bounds__(BLOCK) void transpose_panel(uint32_t *__restrict__ out, const uint32_t *__restrict__ in, TransGeom g, uint32_t pitch,
+__global__ __launch_bounds__(PANEL_BLOCK) void transpose_panel(uint32_t *__restrict__ out, const uint32_t *__restrict__ in, TransGeom g, uint32_t pitch,
                                                          FastDiv rdiv) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     uint32_t *lds = reinterpret_cast<uint32_t *>(smem_raw);  // element (c, r) of the panel at c * pitch + r
@@ -300,11 +301,11 @@ __global__ __launch_bounds__(BLOCK) void transpose_panel(uint32_t *__restrict__ 
     const uint32_t *src = in + src0 + c0;
     uint32_t *dst = out + dst0 + (size_t)c0 * g.r_len;
     constexpr int U = 4;  // loads requested before the first is scattered into LDS
-    for (uint32_t i0 = threadIdx.x; i0 < n4; i0 += U * BLOCK) {
+    for (uint32_t i0 = threadIdx.x; i0 < n4; i0 += U * PANEL_BLOCK) {
         u32x4 v[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const uint32_t i = i0 + u * BLOCK;
+            const uint32_t i = i0 + u * PANEL_BLOCK;
             if (i < n4) {
                 const u32x4 *p = reinterpret_cast<const u32x4 *>(src + (size_t)(i / Q) * g.r_in_str + 4 * (i % Q));
                 v[u] = NT ? __builtin_nontemporal_load(p) : *p;
@@ -312,7 +313,7 @@ __global__ __launch_bounds__(BLOCK) void transpose_panel(uint32_t *__restrict__ 
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const uint32_t i = i0 + u * BLOCK;
+            const uint32_t i = i0 + u * PANEL_BLOCK;
             if (i < n4) {
                 const uint32_t r = i / Q, c = 4 * (i % Q);
                 lds[c * pitch + r] = v[u].x, lds[(c + 1) * pitch + r] = v[u].y, lds[(c + 2) * pitch + r] = v[u].z, lds[(c + 3) * pitch + r] = v[u].w;
@@ -320,18 +321,24 @@ __global__ __launch_bounds__(BLOCK) void transpose_panel(uint32_t *__restrict__ 
         }
     }
     __syncthreads();
-    for (uint32_t i = threadIdx.x; i < n4; i += BLOCK) {
-        uint32_t c = rdiv.div(4 * i), r = 4 * i - c * g.r_len;  // the span is [c][r]
-        uint32_t w[4];
+    const bool image = pitch == g.r_len;  // an odd R: LDS holds the span as it goes out, 16 bytes at a time
+    for (uint32_t i = threadIdx.x; i < n4; i += PANEL_BLOCK) {
+        u32x4 t;
+        if (image) {
+            t = *reinterpret_cast<const u32x4 *>(lds + 4 * i);
+        } else {
+            uint32_t c = rdiv.div(4 * i), r = 4 * i - c * g.r_len;  // the span is [c][r]
+            uint32_t w[4];
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            w[k] = lds[c * pitch + r];
-            if (++r == g.r_len) {
-                r = 0;
-                c++;
+            for (int k = 0; k < 4; k++) {
+                w[k] = lds[c * pitch + r];
+                if (++r == g.r_len) {
+                    r = 0;
+                    c++;
+                }
             }
+            t = u32x4{w[0], w[1], w[2], w[3]};
         }
-        const u32x4 t = {w[0], w[1], w[2], w[3]};
         if (NT) __builtin_nontemporal_store(t, reinterpret_cast<u32x4 *>(dst + 4 * (size_t)i));
         else *reinterpret_cast<u32x4 *>(dst + 4 * (size_t)i) = t;
     }
@@ -874,8 +881,8 @@ int launch_transpose(DeviceCtx &ctx, void *out, const void *in, int elem_size, i
             const FastDiv rdiv = make_fastdiv(g.r_len);
             uint32_t *o = static_cast<uint32_t *>(out);
             const uint32_t *x = static_cast<const uint32_t *>(in);
-            if (ctx.streaming(total * 4)) hipLaunchKernelGGL((transpose_panel<PANEL, true>), grid, dim3(BLOCK), lds_bytes, ctx.stream, o, x, g, pitch, rdiv);
-            else hipLaunchKernelGGL((transpose_panel<PANEL, false>), grid, dim3(BLOCK), lds_bytes, ctx.stream, o, x, g, pitch, rdiv);
+            if (ctx.streaming(total * 4)) hipLaunchKernelGGL((transpose_panel<PANEL, true>), grid, dim3(PANEL_BLOCK), lds_bytes, ctx.stream, o, x, g, pitch, rdiv);
+            else hipLaunchKernelGGL((transpose_panel<PANEL, false>), grid, dim3(PANEL_BLOCK), lds_bytes, ctx.stream, o, x, g, pitch, rdiv);
             return ctx.check(hipGetLastError(), "transpose_panel launch");
         }
     }
