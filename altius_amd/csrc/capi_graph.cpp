@@ -50,6 +50,8 @@ struct ahip_session {
     std::condition_variable lane_freed;
     std::vector<std::shared_ptr<HipSession>> lanes;   // lanes[0] == s
     std::vector<bool> busy;
+    size_t last_lane = 0;                             // the lane that served the call that finished last: the statistics read it
+    bool lanes_full = false;                          // a further lane could not be built (memory): concurrent calls wait instead
     size_t building = 0;                              // lanes under construction
 };
 
@@ -69,7 +71,7 @@ int acquire_lane(ahip_session *session, size_t *index, std::shared_ptr<HipSessio
                 *lane_out = session->lanes[i];
                 return AHIP_OK;
             }
-        if (session->lanes.size() + session->building < MAX_LANES) break;
+        if (!session->lanes_full && session->lanes.size() + session->building < MAX_LANES) break;
         session->lane_freed.wait(lock);
     }
     session->building++;
@@ -91,14 +93,35 @@ int acquire_lane(ahip_session *session, size_t *index, std::shared_ptr<HipSessio
     lock.lock();
     session->building--;
     if (!lane) {
+        // Every lane holds its own copy of the weights: the GPU may simply have no room for another.  The lanes that
+        // exist still serve every call, one after the other.
+        session->lanes_full = true;
         session->lane_freed.notify_all();
-        return fail(err.code(), "ahip_session_run: could not build another lane for a concurrent call: " + err.to_string());
+        for (;;) {
+            for (size_t i = 0; i < session->lanes.size(); i++)
+                if (!session->busy[i]) {
+                    session->busy[i] = true;
+                    *index = i;
+                    *lane_out = session->lanes[i];
+                    return AHIP_OK;
+                }
+            session->lane_freed.wait(lock);
+        }
     }
     session->lanes.push_back(lane);
     session->busy.push_back(true);
     *index = session->lanes.size() - 1;
     *lane_out = std::move(lane);
     return AHIP_OK;
+}
+
+// The lane whose run finished last, for the statistics calls.  A lane that is running is waited for: its counters
+// are written by the run.
+std::shared_ptr<HipSession> last_lane_idle(const ahip_session *session_c) {
+    ahip_session *session = const_cast<ahip_session *>(session_c);
+    std::unique_lock<std::mutex> lock(session->lanes_mutex);
+    while (session->busy[session->last_lane]) session->lane_freed.wait(lock);
+    return session->lanes[session->last_lane];
 }
 
 // The device-resident calls keep their tensors in lane 0's pool and order their work on lane 0's stream.
@@ -112,6 +135,7 @@ void release_lane(ahip_session *session, size_t index, bool keep_profile) {
     std::lock_guard<std::mutex> lock(session->lanes_mutex);
     if (keep_profile) session->profile.assign(session->lanes[index]->last_profile().begin(), session->lanes[index]->last_profile().end());
     session->busy[index] = false;
+    session->last_lane = index;
     session->lane_freed.notify_all();
 }
 
@@ -732,7 +756,7 @@ int ahip_session_builder_with_fused_attention(ahip_session_builder *builder, int
 
 int ahip_session_copies_avoided(const ahip_session *session, size_t *count) try {
     if (!session || !count) return fail(AHIP_ERR_ARG, "ahip_session_copies_avoided: null argument");
-    *count = session->s->copies_avoided();
+    *count = last_lane_idle(session)->copies_avoided();
     return AHIP_OK;
 } catch (...) {
     return altius::caught_at_boundary("ahip_session_copies_avoided");
@@ -740,7 +764,7 @@ int ahip_session_copies_avoided(const ahip_session *session, size_t *count) try 
 
 int ahip_session_graph_replays(const ahip_session *session, size_t *count) try {
     if (!session || !count) return fail(AHIP_ERR_ARG, "ahip_session_graph_replays: null argument");
-    *count = session->s->graph_replays();
+    *count = last_lane_idle(session)->graph_replays();
     return AHIP_OK;
 } catch (...) {
     return altius::caught_at_boundary("ahip_session_graph_replays");
@@ -880,8 +904,16 @@ int ahip_session_run_device(ahip_session *session, int n_inputs, const void *con
 
 int ahip_session_synchronize(ahip_session *session) try {
     if (!session) return fail(AHIP_ERR_ARG, "ahip_session_synchronize: null session");
-    SessionError err;
-    if (!session->s->synchronize(&err)) return fail(err.code(), err.to_string());
+    // Every lane's stream: a call that another thread made on a lane of its own is waited for as well.
+    std::vector<std::shared_ptr<HipSession>> lanes;
+    {
+        std::lock_guard<std::mutex> lock(session->lanes_mutex);
+        lanes = session->lanes;
+    }
+    for (auto &lane : lanes) {
+        SessionError err;
+        if (!lane->synchronize(&err)) return fail(err.code(), err.to_string());
+    }
     return AHIP_OK;
 } catch (...) {
     return altius::caught_at_boundary("ahip_session_synchronize");
@@ -904,6 +936,9 @@ const ahip_model *ahip_session_model(const ahip_session *session) { return sessi
 
 int ahip_session_profile(const ahip_session *session, int index, const char **op_name, double *ms, int *count) try {
     if (!session) return fail(AHIP_ERR_ARG, "ahip_session_profile: null session");
+    // The names handed out point into `profile`, which the next profiled run replaces: as before, the caller reads
+    // them before it runs again; the lock keeps a run on another thread from replacing it in mid-read.
+    std::lock_guard<std::mutex> lock(const_cast<ahip_session *>(session)->lanes_mutex);
     if (count) *count = (int)session->profile.size();
     if (index < 0 || index >= (int)session->profile.size()) {
         if (op_name || ms) return fail(AHIP_ERR_ARG, "ahip_session_profile: index out of range");
@@ -918,7 +953,7 @@ int ahip_session_profile(const ahip_session *session, int index, const char **op
 
 int ahip_session_last_device_ms(const ahip_session *session, double *ms) try {
     if (!session || !ms) return fail(AHIP_ERR_ARG, "ahip_session_last_device_ms: null argument");
-    *ms = session->s->last_device_ms();
+    *ms = last_lane_idle(session)->last_device_ms();
     return AHIP_OK;
 } catch (...) {
     return altius::caught_at_boundary("ahip_session_last_device_ms");
@@ -926,7 +961,7 @@ int ahip_session_last_device_ms(const ahip_session *session, double *ms) try {
 
 int ahip_session_last_run_ms(const ahip_session *session, double *ms) try {
     if (!session || !ms) return fail(AHIP_ERR_ARG, "ahip_session_last_run_ms: null argument");
-    *ms = session->s->last_run_ms();
+    *ms = last_lane_idle(session)->last_run_ms();
     return AHIP_OK;
 } catch (...) {
     return altius::caught_at_boundary("ahip_session_last_run_ms");
@@ -934,7 +969,7 @@ int ahip_session_last_run_ms(const ahip_session *session, double *ms) try {
 
 int ahip_session_device_allocations(const ahip_session *session, size_t *count) try {
     if (!session || !count) return fail(AHIP_ERR_ARG, "ahip_session_device_allocations: null argument");
-    *count = session->s->device_allocations();
+    *count = last_lane_idle(session)->device_allocations();
     return AHIP_OK;
 } catch (...) {
     return altius::caught_at_boundary("ahip_session_device_allocations");

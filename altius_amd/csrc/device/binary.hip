@@ -419,7 +419,10 @@ void flat_dispatch(hipStream_t s, float *out, const float *a, const float *b, si
         else
             hipLaunchKernelGGL((binary_flat_vec4<OP, MA, MB, false>), dim3((unsigned)blocks), dim3(BLOCK), 0, s,
                                out, a, b, n);
-    } else if (n >= 4 * BLOCK) {
+    } else if (n >= 4 * BLOCK && ((reinterpret_cast<uintptr_t>(out) | (MA == FULL ? reinterpret_cast<uintptr_t>(a) : 0) |
+                                   (MB == FULL ? reinterpret_cast<uintptr_t>(b) : 0)) & 3u) == 0) {
+        // 16-byte accesses on 4-byte boundaries: the output and every full operand must at least be float-aligned
+        // (a pointer at a byte offset takes the single-element kernel below)
         const size_t blocks = ((n >> 2) + BLOCK - 1) / BLOCK;
         if (nt) hipLaunchKernelGGL((binary_flat_vec4_any<OP, MA, MB, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, a, b, n);
         else hipLaunchKernelGGL((binary_flat_vec4_any<OP, MA, MB, false>), dim3((unsigned)blocks), dim3(BLOCK), 0, s, out, a, b, n);

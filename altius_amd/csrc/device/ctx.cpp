@@ -38,10 +38,9 @@ int create_device_ctx(int device, hipStream_t stream, bool own_stream, DeviceCtx
     e = hipSetDevice(device);
     if (e != hipSuccess) return fail(e, "hipSetDevice");
     ctx->device = device;
-    if (reduce_static_setup(device) != AHIP_OK) {
-        if (error) *error = "hipGetSymbolAddress: the fixed partial-results array of the no-allocation reduce could not be located";
-        return AHIP_ERR_HIP;
-    }
+    // Only ahip_reduce_static needs the fixed array's address: without it that entry point reports the failure, and
+    // everything else works.
+    (void)reduce_static_setup(device);
     // AHIP_GEMM_SPLIT_K=0 keeps the bf16 GEMM from cutting an XCD's partly filled last round of tiles along k
     // (for measurements).
     if (const char *e = getenv("AHIP_GEMM_SPLIT_K")) ctx->gemm_split_k = atoi(e) != 0;
@@ -83,7 +82,18 @@ int create_device_ctx(int device, hipStream_t stream, bool own_stream, DeviceCtx
     ctx->flags_armed = false;
     // Where do blocks run?  Decides whether the bf16 GEMM may combine the slices of a tile inside one XCD's L2.
     // A probe that cannot run leaves the answer at "not shown", which only switches that cut off.
+    // On a stream of the library's own: a caller's stream may be capturing, or busy with work the probe's
+    // synchronisation would wait for.
+    hipStream_t given = ctx->stream, probe_stream = nullptr;
+    if (!ctx->owns_stream && hipStreamCreateWithFlags(&probe_stream, hipStreamNonBlocking) != hipSuccess) {
+        (void)hipGetLastError();
+        ctx->xcd_round_robin = false;
+        return AHIP_OK;
+    }
+    if (probe_stream) ctx->stream = probe_stream;
     if (probe_xcd_placement(*ctx, cus) != AHIP_OK) ctx->xcd_round_robin = false;
+    ctx->stream = given;
+    if (probe_stream) (void)hipStreamDestroy(probe_stream);
     return AHIP_OK;
 }
 
@@ -109,6 +119,7 @@ int check_device_flags(DeviceCtx &ctx) {
 void destroy_device_ctx(DeviceCtx *ctx) {
     if (hipSetDevice(ctx->device) != hipSuccess) return;
     (void)hipStreamSynchronize(ctx->stream);
+    reduce_static_forget_stream(ctx->device, ctx->stream);
     gemm_release_all(*ctx);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     ctx->scratch = nullptr;

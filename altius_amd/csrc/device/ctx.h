@@ -129,6 +129,8 @@ int launch_reduce(DeviceCtx &ctx, int kind, float *out, const float *in, size_t 
 // calling thread's current device; create_device_ctx calls it.
 int launch_reduce_static(DeviceCtx &ctx, int kind, float *out, const float *in, size_t outer, size_t red, size_t inner);
 int reduce_static_setup(int device);
+// A stream that is about to be destroyed (its work has been waited for) no longer owns the fixed array.
+void reduce_static_forget_stream(int device, hipStream_t stream);
 size_t reduce_static_capacity_floats();
 
 

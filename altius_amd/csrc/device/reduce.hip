@@ -50,6 +50,10 @@ static __device__ __align__(256) float scratch[STATIC_SCRATCH_FLOATS];
 constexpr int MAX_DEVICES = 64;
 std::mutex g_static_mutex;
 float *g_static_scratch[MAX_DEVICES] = {};
+// The stream whose launch last used each device's fixed array (guarded by g_static_mutex).  Calls on one stream are
+// ordered; a call on another stream may take the array over only once everything queued on that stream has finished.
+hipStream_t g_static_owner[MAX_DEVICES] = {};
+bool g_static_owned[MAX_DEVICES] = {};
 
 constexpr int ROW_BLOCK = 256;
 constexpr int ROW_WAVES = ROW_BLOCK / WAVE;
@@ -603,6 +607,24 @@ int partials_too_small(DeviceCtx &ctx, size_t needed, const Partials &pt) {
                                               std::to_string(pt.floats));
 }
 
+// Before a launch writes partial results: the context's own buffer is its own business; the fixed array of the
+// no-allocation entry point is shared by every context and stream of the GPU, and a second stream gets it only when
+// the first has drained (hipStreamQuery: no allocation, no wait).  Otherwise the call fails instead of racing.
+int claim_partials(DeviceCtx &ctx, const Partials &pt) {
+    if (!pt.fixed || ctx.device < 0 || ctx.device >= MAX_DEVICES) return AHIP_OK;
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (g_static_owned[ctx.device] && g_static_owner[ctx.device] != ctx.stream) {
+        const hipError_t e = hipStreamQuery(g_static_owner[ctx.device]);
+        if (e == hipErrorNotReady)
+            return ctx.fail(AHIP_ERR_UNSUPPORTED, "reduce (no-allocation entry point): the fixed buffer is still in use by work queued on "
+                                                  "another stream of this GPU; synchronize that stream first, or use ahip_reduce");
+        (void)hipGetLastError();  // finished, or a stream that no longer exists: the array is free either way
+    }
+    g_static_owner[ctx.device] = ctx.stream;
+    g_static_owned[ctx.device] = true;
+    return AHIP_OK;
+}
+
 template <class OP, bool SCALE>
 int reduce_impl(DeviceCtx &ctx, const Partials &pt, float *out, const float *in, size_t outer, size_t red, size_t inner,
                 float scale) {
@@ -666,6 +688,7 @@ int reduce_impl(DeviceCtx &ctx, const Partials &pt, float *out, const float *in,
             return ctx.check(hipGetLastError(), "reduce rows (block) launch");
         }
         if (outer * splits > pt.floats) return partials_too_small(ctx, outer * splits, pt);
+        if (int rc = claim_partials(ctx, pt)) return rc;
         rows_block_launch<OP, false>(s, pt.ptr, in, outer, red, splits, chunk, 1.0f, nt);
         rows_wave_launch<OP, SCALE>(s, out, pt.ptr, outer, splits, scale);
         return ctx.check(hipGetLastError(), "reduce rows (two-stage) launch");
@@ -711,6 +734,7 @@ int reduce_impl(DeviceCtx &ctx, const Partials &pt, float *out, const float *in,
                     return ctx.check(hipGetLastError(), "reduce cols (span) launch");
                 }
                 if (outer * fsplits * inner <= pt.floats) {
+                    if (int rc = claim_partials(ctx, pt)) return rc;
                     cols_span_launch<OP, false>(s, pt.ptr, in, outer, red, inner, span_rows, fsplits, sps, 1.0f, nt);
                     cols_launch<OP, SCALE>(s, out, pt.ptr, outer, fsplits, inner, 1, fsplits, scale);
                     return ctx.check(hipGetLastError(), "reduce cols (span, two-stage) launch");
@@ -759,6 +783,7 @@ int reduce_impl(DeviceCtx &ctx, const Partials &pt, float *out, const float *in,
         cols_launch<OP, SCALE>(s, out, in, outer, red, inner, 1, red, scale, nt);
         return ctx.check(hipGetLastError(), "reduce cols launch");
     }
+    if (int rc = claim_partials(ctx, pt)) return rc;
     cols_launch<OP, false>(s, pt.ptr, in, outer, red, inner, splits, chunk, 1.0f, nt);
     cols_launch<OP, SCALE>(s, out, pt.ptr, outer, splits, inner, 1, splits, scale);
     return ctx.check(hipGetLastError(), "reduce cols (two-stage) launch");
@@ -800,6 +825,12 @@ int reduce_static_setup(int device) {
 }
 
 size_t reduce_static_capacity_floats() { return STATIC_SCRATCH_FLOATS; }
+
+void reduce_static_forget_stream(int device, hipStream_t stream) {
+    if (device < 0 || device >= MAX_DEVICES) return;
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (g_static_owned[device] && g_static_owner[device] == stream) g_static_owned[device] = false;
+}
 
 int launch_reduce_static(DeviceCtx &ctx, int kind, float *out, const float *in, size_t outer, size_t red, size_t inner) {
     float *ptr = nullptr;

@@ -1219,6 +1219,7 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
                 out.block = planes.block;  // the fp32 block goes back to the pool unused
                 out.ptr = planes.ptr;
                 out.planes = true;
+                out.planes_rows = rows, out.planes_k = len;
                 copies_avoided_++;  // the operand split of the product behind (and the fp32 tensor between them)
                 break;
             }
@@ -1451,7 +1452,7 @@ bool HipSession::run_device_op(const Node &node, const Op &op, const std::vector
             for (size_t i = 0; i + 1 < ad.len(); i++) rows *= ad[i];
             const size_t kk = ad[ad.len() - 1];
             if (op.trans_a || bdm.len() != 2 || !in[1]->strides.empty() || matmul_out_perm_.count(current_node_) ||
-                (op.trans_b ? bdm[1] : bdm[0]) != kk)
+                (op.trans_b ? bdm[1] : bdm[0]) != kk || in[0]->planes_rows != rows || in[0]->planes_k != kk)
                 return fail(err, SessionError::Message, "internal: operand planes reached a product of another form");
             const size_t nn = op.trans_b ? bdm[0] : bdm[1];
             const float *bias_p = nullptr;

@@ -109,6 +109,7 @@ struct DeviceTensor {
     // tall bf16 product that is its only reader; the LayerNormalization that produced the tensor wrote them instead
     // of the fp32 result.
     bool planes = false;
+    size_t planes_rows = 0, planes_k = 0;  // the [rows, k] operand the planes were written for
     // Set while the tensor's values are still owed by an Add that was deferred (see PendingAdd).
     std::shared_ptr<PendingAdd> pending_add;
     bool owes_add() const { return pending_add && !pending_add->done; }

@@ -245,6 +245,7 @@ bool HipSession::run_attention_tail(const Op &op, const std::vector<DeviceTensor
         out->block = planes.block;  // the fp32 block goes back to the pool unused
         out->ptr = planes.ptr;
         out->planes = true;
+        out->planes_rows = outer * tq, out->planes_k = inner * 64;
         planes_ptr = planes.ptr;
         copies_avoided_++;  // the operand split of the product behind
     }
@@ -407,6 +408,18 @@ void HipSession::plan_views(bool fused_attention) {
         for (size_t i = 1; i < m.inputs.size(); i++) elsewhere = elsewhere || m.inputs[i] == m.inputs[0];
         auto w = g.inits.find(m.inputs[1]);
         if (elsewhere || w == g.inits.end() || w->second.dims().len() != 2 || w->second.elem_ty() != TensorElemType::F32) continue;
+        // The planes are laid out for [b * t, h * 64] x weights [h * 64, n]: the attention's result must be [b, h, t, 64],
+        // the Reshape must merge exactly the heads into the last axis (any other valid reshape, [b, t * h, 64] say, would
+        // read the planes with another geometry), and the weights must have h * 64 rows.  Shapes that are not known
+        // before the run leave the plan out.
+        auto at = inferred_.find(tid), rt = inferred_.find(rs);
+        if (at == inferred_.end() || rt == inferred_.end() || at->second.second.empty() || rt->second.second.empty()) continue;
+        const FixedDimensions &ad = at->second.second[0].dims, &rd = rt->second.second[0].dims;
+        if (ad.len() != 4 || ad[3] != 64 || rd.len() < 2) continue;
+        const size_t merged = ad[1] * 64, rows = ad[0] * ad[2];
+        size_t lead = 1;
+        for (size_t i = 0; i + 1 < rd.len(); i++) lead *= rd[i];
+        if (rd[rd.len() - 1] != merged || lead != rows || (m.op.trans_b ? w->second.dims()[1] : w->second.dims()[0]) != merged) continue;
         PlanesPlan pp;
         pp.consumer = mm;
         pp.next_n = m.op.trans_b ? w->second.dims()[0] : w->second.dims()[1];

@@ -222,8 +222,11 @@ int ahip_reduce(ahip_ctx *ctx, int kind, float *out, const float *in, size_t out
  * the context's scratch buffer, and the call itself performs no hipMalloc / hipFree.  A shape whose partial
  * results exceed ahip_reduce_static_capacity() floats fails with AHIP_ERR_UNSUPPORTED and launches nothing
  * (ahip_reduce would take its larger buffer or a one-stage kernel).  Every call on a GPU shares that GPU's
- * array, whatever its context: calls that may overlap on one GPU (two streams, two threads) race; calls on
- * one stream are ordered.  Nothing in the array has to start at zero. */
+ * array, whatever its context.  Calls on one stream are ordered.  A two-stage call on another stream takes the
+ * array over only if everything queued on the stream that used it last has finished (hipStreamQuery, no wait);
+ * otherwise it fails with AHIP_ERR_UNSUPPORTED and launches nothing -- synchronize the other stream first.  Two
+ * threads that call on different streams without such a handover would race: the library's record of the
+ * last stream is what turns that into the error above.  Nothing in the array has to start at zero. */
 int ahip_reduce_static(ahip_ctx *ctx, int kind, float *out, const float *in, size_t outer, size_t reduce,
                        size_t inner);
 size_t ahip_reduce_static_capacity(void);

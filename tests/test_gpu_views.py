@@ -123,6 +123,38 @@ def test_attention_writes_the_operand_planes_of_the_projection_behind_it(case, b
     np.testing.assert_allclose(outs[0], outs[1], rtol=2e-4, atol=2e-5)
 
 
+def test_attention_planes_are_not_planned_for_a_reshape_that_keeps_the_heads_apart(case):
+    """The same chain with the Reshape behind the merge Transpose giving [b, t * h, 64] and weights of 64 rows: a
+    valid graph whose last product has another geometry than the planes would be written for.  The plan must leave
+    it to the ordinary route (one copy avoided fewer than with the merging Reshape) and the result must be right."""
+    case("attention -> Transpose -> Reshape [b, t*h, 64] -> MatMul [64, n]")
+    from altius_amd import device as D
+
+    batch, tokens, heads, d = 24, 45, 12, 64
+    hd = heads * d
+    m = Model(opset_version=13)
+    x = m.new_val_named_and_shaped("qkv", [batch, tokens, 3 * hd])
+    m.add_input(x)
+    parts = node(m, Op.Split, [x, i64(m, hd, hd, hd)], 3, axis=2)
+    q, k, v = (node(m, Op.Transpose, [node(m, Op.Reshape, [p, i64(m, batch, tokens, heads, d)])], perm=[0, 2, 1, 3]) for p in parts)
+    s = node(m, Op.Softmax, [node(m, Op.MatMul, [q, node(m, Op.Transpose, [k], perm=[0, 1, 3, 2])])], axis=-1)
+    a = node(m, Op.Reshape, [node(m, Op.Transpose, [node(m, Op.MatMul, [s, v])], perm=[0, 2, 1, 3]), i64(m, batch, tokens * heads, d)])
+    w = (RNG.standard_normal((d, 96)) * 0.1).astype(np.float32)
+    m.add_output(node(m, Op.MatMul, [a, m.new_initializer(w)]))
+    m.fuse_transpose_matmul()
+    feed = (RNG.standard_normal((batch, tokens, 3 * hd)) * 0.3).astype(np.float32)
+    sess = HipSessionBuilder(m.clone()).with_gemm_algorithm(D.GEMM_BF16X3).with_fused_attention(True).build()
+    for _ in range(2):
+        (got,) = [np.array(t) for t in sess.run([Tensor.from_numpy(feed)])]
+    sess.close()
+    qn, kn, vn = (feed[:, :, i * hd:(i + 1) * hd].reshape(batch, tokens, heads, d).transpose(0, 2, 1, 3).astype(np.float64) for i in range(3))
+    p = qn @ kn.transpose(0, 1, 3, 2)
+    p = np.exp(p - p.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    want = (p @ vn).transpose(0, 2, 1, 3).reshape(batch, tokens * heads, d) @ w.astype(np.float64)
+    np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-5)
+
+
 def test_view_with_another_reader_is_copied(case):
     """A part that an element-wise operator also reads is not made a view; its siblings' fate follows (one Split node)."""
     case("split part read by Add as well")
