@@ -174,6 +174,12 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
                        const size_t a_batch_strides[2], const size_t b_batch_strides[2], const size_t c_batch_strides[2],
                        size_t c0_row_stride, size_t c0_col_stride, float alpha, float beta, const GemmPost *post = nullptr);
 
+// Many small products at once (matmul_small.hip): one block per matrix.  C = A B, A with unit stride along k.
+bool gemm_small_batched_fits(size_t batch, size_t m, size_t n, size_t k);
+int launch_gemm_small_batched(DeviceCtx &ctx, float *c, const float *a, const float *b, size_t batch_outer, size_t batch_inner, size_t m, size_t n,
+                              size_t k, int trans_b, size_t lda, size_t ldb, size_t ldc, const size_t a_bs[2], const size_t b_bs[2],
+                              const size_t c_bs[2]);
+
 // O = Softmax(scale(Q K^T) + mask) V per batch, scores kept in registers (attention.hip).  Q [tq, d], K [tk, d], V [tk, d],
 // O [tq, d] with row pitches ld*; batches as in launch_gemm_batch2; scale_op 0 none / 1 multiply / 2 divide; mask (may be
 // null) one value per key, read at mask[outer batch * mask_outer_stride + key].

@@ -299,6 +299,10 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
     const size_t lim = (size_t)1 << 31;
     if (m >= lim || n >= lim || k >= lim || lda >= lim || ldb >= lim || ldc >= lim || m * ldc >= ((size_t)1 << 40))
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm: extent above 2^31");
+    // Hundreds of small matrices (attention's two products per head): one block per matrix.
+    if (!has_post && !trans_a && alpha == 1.0f && (!c0 || beta == 0.0f) && !split_k_inner && gemm_small_batched_fits(batch, m, n, k))
+        return launch_gemm_small_batched(ctx, c, a, b, batch_outer, batch_inner, m, n, k, trans_b, lda, ldb, ldc, a_batch_strides, b_batch_strides,
+                                         c_batch_strides);
     // The 128 x 64 tile when it leaves fewer idle columns (n = 64: 64 instead of 128 computed), and for long
     // K loops: with half the accumulators per wavefront more blocks fit a CU and the last round of blocks
     // is fuller (measured at [50432,3072]x[3072,768]: 120.9 against 110.3 TFLOP/s; the wide tile stays ahead
