@@ -3,24 +3,34 @@
 // (compute_mat_mul, crates/session_interpreter/src/session.rs:621-684, one sgemm per batch entry).
 //
 // The 128 x 128 tiles of matmul.hip fit such matrices badly: four tiles per head of which 59 % is
-// padding, every operand fetched twice.  Here one block takes one whole matrix product, cut into
-// 16 x 16 tiles of v_mfma_f32_16x16x4_f32 (197 rows pad to 208, where 32 x 32 tiles pad to 224):
-// wavefront w owns rows 16 w .. 16 w + 15 of C, thirteen wavefronts for 197 rows.
+// padding, every operand fetched twice.  Here one block of 16 wavefronts per compute unit walks the
+// heads blockIdx.x, blockIdx.x + gridDim.x, ... and takes each product whole, cut into 16 x 16 tiles
+// of v_mfma_f32_16x16x4_f32 (197 rows pad to 208, where 32 x 32 tiles pad to 224).
+//
+// Twelve wavefronts multiply (three per SIMD) and four fetch (one per SIMD).  The fetchers bring the
+// operands from global memory into LDS a step ahead of the multipliers, which read LDS only and store
+// results.  The two kinds of work are kept in different wavefronts because the hardware counts a
+// wavefront's loads and stores in one counter: a wavefront that waits for a load it issued before
+// storing results waits for those stores too, and stores take microseconds to drain.  (One block per
+// matrix, loading and then multiplying, leaves the matrix unit idle while it loads, and two such
+// blocks on a compute unit do not fill each other's gaps: loads issued while the other block stores
+// queue behind those stores in the compute unit's L1, which serves requests in order.)
 //
 // The instruction adds four values of k per step, one from each quarter of the wavefront (lane / 16),
-// and a sum does not care which four: both kernels hand the quarters the values of k that make their
-// loads cheap, the same way for A and B and whichever way round B is stored, so that a product and the
-// same product through a view of its second operand add the same numbers in the same order.
+// and a sum does not care which four: quarter q takes k = 16 q .. 16 q + 15 of a chunk of 64, so that
+// a lane reads its 16 values as four 16-byte pieces of a row of LDS.  The assignment is the same for A
+// and B and whichever way round B is stored, so that a product and the same product through a view of
+// its second operand add the same numbers in the same order.  Tiles are computed transposed (B's
+// fragment as the instruction's first operand), so that a lane's four results lie next to each other
+// in a row of C.
 //
-//   k <= 64 (Q K^T), gemm_small_k64: quarter q takes k = 16 q .. 16 q + 15.  A lane's 16 values of A lie
-//     next to each other in memory and go from there to registers; all of B goes through LDS once per
-//     block, stored the way it lies in memory, and every wavefront meets its column tiles one after the
-//     other and stores a finished 16 x 16 tile of C per column tile.
-//   n <= 64 (P V), gemm_small_n64: up to four column tiles, whose accumulators stay in registers while k
-//     goes by in chunks of 32; in a chunk step s gives quarter q the value k = 4 s + q.  Per chunk a
-//     wavefront stages its own rows of A (lanes along k, so that its loads are whole runs of a row) and
-//     the block stages the chunk's part of B.
-// C = A B only (no alpha, beta or third operand), A with unit stride along k; B either way round.
+//   k <= 64 (Q K^T), gemm_small_k64: all of A and all of B of a head in LDS (B twice, for this head and
+//     the next); a multiplier keeps its rows of A in registers and sweeps its row of tiles of C from
+//     left to right, a tile stored as soon as it is finished.
+//   n <= 64 (P V), gemm_small_n64: k goes by in chunks of 64, each chunk of A and of B in LDS twice; a
+//     multiplier keeps the (up to five) tiles of C it owns in registers until the head is done.
+// C = A B only (no alpha, beta or third operand), A with unit stride along k; B either way round;
+// m <= 208.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -39,12 +49,6 @@ constexpr int WAVE = 64;
 constexpr int TILE = 16;        // rows / columns of an MFMA tile
 constexpr int CHUNK = 64;       // values of k in a chunk: 16 steps of 4
 constexpr int STEPS = CHUNK / 4;
-constexpr int MAX_WAVES = 16;   // wavefronts per block: up to 256 rows of C
-constexpr int MIN_WAVES = 4;    // at least four, so that the staging of B is shared by enough threads
-constexpr int N64_CHUNK = 32;       // gemm_small_n64 takes k 32 at a time: two groups of four steps
-constexpr int N64_K_PITCH = N64_CHUNK + 4;
-constexpr int J_PITCH_N64 = 64 + 16; // floats per LDS row of a chunk of B stored [k][column], columns <= 64: quarters
-                                     // q and q + 1 of a wavefront land on different halves of the banks
 
 struct SmallGemm {
     const float *a, *b;
@@ -53,15 +57,13 @@ struct SmallGemm {
     uint32_t lda, ldb, ldc;  // A(i, kk) = a[i * lda + kk]; B(kk, j) = b[j * ldb + kk] (k contiguous) or b[kk * ldb + j]
     uint64_t a_bs, b_bs, c_bs, a_bs2, b_bs2, c_bs2;
     uint32_t batch_inner;
-    uint32_t batch;  // gemm_small_k64: heads
+    uint32_t batch;  // heads
 };
 
-__device__ __forceinline__ void batch_offsets(const SmallGemm &g, const float *&a, const float *&b, float *&c) {
-    const uint32_t z = blockIdx.x, zo = z / g.batch_inner, zi = z - zo * g.batch_inner;
-    a = g.a + zo * g.a_bs + zi * g.a_bs2;
-    b = g.b + zo * g.b_bs + zi * g.b_bs2;
-    c = g.c + zo * g.c_bs + zi * g.c_bs2;
-}
+// A barrier that orders the block's LDS traffic only.  __syncthreads() also waits for the wavefront's global loads and
+// stores (one counter for both), which is what the fetchers' loads in flight and the multipliers' draining stores must
+// not be made to do: nothing here hands data from wavefront to wavefront through global memory.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // The tiles are computed transposed (B's fragment as the instruction's first operand), so that a lane's four results
 // lie next to each other in a row of C: element r of a lane's accumulator is C(row0 + lane % 16, col0 + 4 (lane / 16) + r).
@@ -221,14 +223,14 @@ __global__ __launch_bounds__(PB_WAVES * WAVE) void gemm_small_k64(SmallGemm args
         uint32_t parity = 0;
         for (uint32_t head = head0; head < batch; head += head_step) {
             write_rows<0, NA>(pa, lds_a, ftid);
-            __syncthreads();  // this head's A and B are in LDS
+            lds_barrier();  // this head's A and B are in LDS
             parity ^= 1;
             if (head + head_step < batch) {
                 operands(head + head_step, A, B);
                 copy_operand<B_K_CONTIGUOUS, B_VEC>(lds_b + parity * b_floats, B, ldb, n, k, ftid);
                 load_rows<0, NA>(pa, operand_buffer(A, (m - 1) * lda + k), lda, k, ftid);
             }
-            __syncthreads();  // the multipliers are done with this head's A
+            lds_barrier();  // the multipliers are done with this head's A
         }
         return;
     }
@@ -267,7 +269,7 @@ __global__ __launch_bounds__(PB_WAVES * WAVE) void gemm_small_k64(SmallGemm args
         }
     };
     for (uint32_t head = head0; head < batch; head += head_step) {
-        __syncthreads();  // this head's A and B are in LDS
+        lds_barrier();  // this head's A and B are in LDS
         const uint32_t zo = head / batch_inner, zi = head - zo * batch_inner;
         float *C = args.c + zo * args.c_bs + zi * args.c_bs2;
         float a[STEPS], b[STEPS];
@@ -294,75 +296,190 @@ __global__ __launch_bounds__(PB_WAVES * WAVE) void gemm_small_k64(SmallGemm args
             }
             store_tile(acc, m, n, ldc, C, row0, col0, lane);
         }
-        __syncthreads();  // done with this head's A and B
+        lds_barrier();  // done with this head's A and B
         b_now = b_now == lds_b ? lds_b + b_floats : lds_b;
     }
 }
 
-// n <= 16 NT, k in chunks of 32.  LDS: [16][N64_K_PITCH] per wavefront for its rows of A, then the chunk's part of B,
-// [k][J_PITCH_N64] when B's columns are contiguous and [column][N64_K_PITCH] when its k axis is.
-// B_VEC (columns contiguous only): B's rows are whole, 16-byte aligned float4s.
-template <bool B_K_CONTIGUOUS, bool B_VEC, int NT>
-__global__ __launch_bounds__(MAX_WAVES * WAVE) void gemm_small_n64(SmallGemm g) {
-    extern __shared__ __align__(16) float lds[];
-    const uint32_t tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid >> 6, nthreads = blockDim.x, nwaves = nthreads >> 6;
-    const uint32_t j = lane & 15, quarter = lane >> 4;
-    const uint32_t half = lane >> 5, kk32 = lane & 31;  // staging: two rows of 32 values of k per wavefront and load
-    float *a_tile = lds + wave * (TILE * N64_K_PITCH);
-    float *b_tile = lds + nwaves * (TILE * N64_K_PITCH);
-    const float *A, *B;
-    float *C;
-    batch_offsets(g, A, B, C);
-    const uint32_t row0 = wave * TILE;
-    const bool active = row0 < g.m;
-    floatx4 acc[NT];
-#pragma unroll
-    for (int t = 0; t < NT; t++) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+// n <= 64, m <= 208, any k.  LDS: a chunk of A, [208][64] with exchanged pieces, and the same chunk of B, [64][64]
+// with exchanged pieces when B's k axis is contiguous or [64][N64_J_PITCH] when its columns are; both twice.  While the
+// multipliers work on chunk g out of one copy, the fetchers fill the other with chunk g + 1 (of the same head or the
+// first of the next), and one barrier per chunk separates the two.
+//
+// A multiplier owns a row of 16 rows of C (up to four tiles); with 13 rows of tiles the last row's tiles go to
+// wavefronts 0 .. 3 as a fifth tile (13 tiles per SIMD).  A's rows are whole 16-byte pieces only by accident (197
+// floats per row of P), so the fetchers read them with buffer loads, which need no more than 4-byte alignment, and
+// zero what lies past k themselves: a row's last piece reaches into the next row.
+constexpr int N64_J_PITCH = 65;
+constexpr int N64_B_PIECES = CHUNK * 64 / (FETCHERS * WAVE);  // single values per fetching lane of a [64][64] chunk of B: 16
 
-    for (uint32_t k0 = 0; k0 < g.k; k0 += N64_CHUNK) {
-        if (k0) __syncthreads();  // everyone has read the previous chunk's part of B
-        const bool in = k0 + kk32 < g.k;
-        if (active) {
+// What a fetching lane holds of a chunk between asking for it and writing it to LDS.
+template <bool B_K_CONTIGUOUS>
+struct N64Pieces {
+    float4 a[VEC_PIECES];
+    typename std::conditional<B_K_CONTIGUOUS, float4, float>::type b[B_K_CONTIGUOUS ? 4 : N64_B_PIECES];
+};
+
+// Ask for values k0 .. k0 + 63 of A (13 float4s per lane, 16 rows apart; rows past m lie past the buffer's end and read
+// as zero) and of B.
+template <bool B_K_CONTIGUOUS>
+__device__ __forceinline__ void n64_ask(N64Pieces<B_K_CONTIGUOUS> &v, const float *A, const float *B, uint32_t m, uint32_t n, uint32_t k, uint32_t lda,
+                                        uint32_t ldb, uint32_t k0, uint32_t ftid) {
+    const uint32_t q = ftid & 15;
+    const __amdgpu_buffer_rsrc_t abuf = operand_buffer(A, (m - 1) * lda + k);
+    const uint32_t a_offset = ((ftid >> 4) * lda + 4 * q) * 4;
 #pragma unroll
-            for (int r = 0; r < TILE; r += 2)
-                a_tile[(r + half) * N64_K_PITCH + kk32] = in ? A[(size_t)min(row0 + r + half, g.m - 1) * g.lda + k0 + kk32] : 0.0f;
-        }
-        if (B_K_CONTIGUOUS) {
-            for (uint32_t jj = 2 * wave + half; jj < g.n; jj += 2 * nwaves) b_tile[jj * N64_K_PITCH + kk32] = in ? B[(size_t)jj * g.ldb + k0 + kk32] : 0.0f;
-        } else if (B_VEC) {
-            const uint32_t q = tid & 15;
-            if (4 * q < g.n)
-                for (uint32_t kk = tid >> 4; kk < N64_CHUNK; kk += nthreads >> 4)
-                    *reinterpret_cast<float4 *>(b_tile + kk * J_PITCH_N64 + 4 * q) =
-                        k0 + kk < g.k ? *reinterpret_cast<const float4 *>(B + (size_t)(k0 + kk) * g.ldb + 4 * q) : make_float4(0.f, 0.f, 0.f, 0.f);
-        } else {
-            if (lane < g.n)
-                for (uint32_t kk = wave; kk < N64_CHUNK; kk += nwaves) b_tile[kk * J_PITCH_N64 + lane] = k0 + kk < g.k ? B[(size_t)(k0 + kk) * g.ldb + lane] : 0.0f;
-        }
-        __syncthreads();
-        if (!active) continue;
-        // four steps (16 values of k) at a time, as many as the chunk holds
-        const uint32_t groups = (min((uint32_t)N64_CHUNK, g.k - k0) + 15) / 16;
-        const float *ap = a_tile + j * N64_K_PITCH + quarter;
-        const float *bp = B_K_CONTIGUOUS ? b_tile + j * N64_K_PITCH + quarter : b_tile + quarter * J_PITCH_N64 + j;
-        for (uint32_t grp = 0; grp < groups; grp++) {
-            float a4[4], b4[NT][4];
-#pragma unroll
-            for (int s = 0; s < 4; s++) a4[s] = ap[16 * grp + 4 * s];
-#pragma unroll
-            for (int t = 0; t < NT; t++)
-#pragma unroll
-                for (int s = 0; s < 4; s++)
-                    b4[t][s] = B_K_CONTIGUOUS ? bp[t * TILE * N64_K_PITCH + 16 * grp + 4 * s] : bp[(16 * grp + 4 * s) * J_PITCH_N64 + t * TILE];
-#pragma unroll
-            for (int s = 0; s < 4; s++)
-#pragma unroll
-                for (int t = 0; t < NT; t++) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b4[t][s], a4[s], acc[t], 0, 0, 0);
-        }
+    for (int u = 0; u < VEC_PIECES; u++) {
+        const f32x4_raw f = __builtin_bit_cast(f32x4_raw, __builtin_amdgcn_raw_buffer_load_b128(abuf, a_offset, (16 * u * lda + k0) * 4, 0));
+        v.a[u] = make_float4(f.x, f.y, f.z, f.w);
     }
-    if (active) {
+    if constexpr (B_K_CONTIGUOUS) {  // B as [column][k]: 4 float4s per lane, 16 columns apart
+        const __amdgpu_buffer_rsrc_t bbuf = operand_buffer(B, (n - 1) * ldb + k);
+        const uint32_t b_offset = ((ftid >> 4) * ldb + 4 * q) * 4;
 #pragma unroll
-        for (int t = 0; t < NT; t++) store_tile(acc[t], g.m, g.n, g.ldc, C, row0, t * TILE, lane);
+        for (int u = 0; u < 4; u++) {
+            const f32x4_raw f = __builtin_bit_cast(f32x4_raw, __builtin_amdgcn_raw_buffer_load_b128(bbuf, b_offset, (16 * u * ldb + k0) * 4, 0));
+            v.b[u] = make_float4(f.x, f.y, f.z, f.w);
+        }
+    } else {  // B as [k][column]: 16 values per lane, 4 rows of k apart; rows past k lie past the buffer's end
+        const __amdgpu_buffer_rsrc_t bbuf = operand_buffer(B, (k - 1) * ldb + n);
+        const uint32_t b_offset = ((ftid >> 6) * ldb + (ftid & 63)) * 4;
+#pragma unroll
+        for (int u = 0; u < N64_B_PIECES; u++)
+            v.b[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(bbuf, b_offset, (k0 + 4 * u) * ldb * 4, 0));
+    }
+}
+
+// ... and write them to LDS; what lies past k (a row's last float4 reaches into the next row) and past n becomes zero.
+template <bool B_K_CONTIGUOUS>
+__device__ __forceinline__ void n64_write(const N64Pieces<B_K_CONTIGUOUS> &v, float *dst_a, float *dst_b, uint32_t n, uint32_t k, uint32_t k0, uint32_t ftid) {
+    const uint32_t q = ftid & 15, kk = k0 + 4 * q;
+    auto within_k = [&](float4 f) {
+        f.x = kk < k ? f.x : 0.f, f.y = kk + 1 < k ? f.y : 0.f, f.z = kk + 2 < k ? f.z : 0.f, f.w = kk + 3 < k ? f.w : 0.f;
+        return f;
+    };
+#pragma unroll
+    for (int u = 0; u < VEC_PIECES; u++) *reinterpret_cast<float4 *>(dst_a + swizzled((ftid >> 4) + 16 * u, 4 * q)) = within_k(v.a[u]);
+    if constexpr (B_K_CONTIGUOUS) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) *reinterpret_cast<float4 *>(dst_b + swizzled((ftid >> 4) + 16 * u, 4 * q)) = within_k(v.b[u]);
+    } else {
+        const uint32_t jj = ftid & 63;
+#pragma unroll
+        for (int u = 0; u < N64_B_PIECES; u++) dst_b[((ftid >> 6) + 4 * u) * N64_J_PITCH + jj] = jj < n ? v.b[u] : 0.f;
+    }
+}
+
+template <bool B_K_CONTIGUOUS>
+__global__ __launch_bounds__(PB_WAVES * WAVE) void gemm_small_n64(SmallGemm args) {
+    extern __shared__ __align__(16) float lds[];
+    const uint32_t tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid >> 6;
+    constexpr uint32_t a_floats = MAX_MN * CHUNK, b_floats = B_K_CONTIGUOUS ? 64 * CHUNK : CHUNK * N64_J_PITCH;
+    float *lds_a = lds, *lds_b = lds + 2 * a_floats;
+    const uint32_t batch = args.batch, batch_inner = args.batch_inner, k = args.k;
+    const uint32_t chunks = (k + CHUNK - 1) / CHUNK;
+    const uint32_t my_heads = (batch - blockIdx.x + gridDim.x - 1) / gridDim.x;  // the grid has at most as many blocks as there are heads
+    const uint32_t steps_total = my_heads * chunks;
+
+    if (wave >= MULTIPLIERS) {
+        // ---- a fetching wavefront: chunk g + 1 is written to LDS while the multipliers work on chunk g, and chunk g + 2 is
+        // asked for right after, so that its way from memory has two chunks' time
+        const uint32_t ftid = tid - MULTIPLIERS * WAVE;
+        const uint32_t m = args.m, n = args.n, lda = args.lda, ldb = args.ldb;
+        N64Pieces<B_K_CONTIGUOUS> pieces;
+        auto ask = [&](uint32_t g) {  // chunk g of this block's heads
+            const uint32_t hi = g / chunks, c = g - hi * chunks, head = blockIdx.x + hi * gridDim.x;
+            const uint32_t zo = head / batch_inner, zi = head - zo * batch_inner;
+            n64_ask<B_K_CONTIGUOUS>(pieces, args.a + zo * args.a_bs + zi * args.a_bs2, args.b + zo * args.b_bs + zi * args.b_bs2, m, n, k, lda, ldb, c * CHUNK, ftid);
+        };
+        auto write = [&](uint32_t g) {  // -> copy g % 2
+            n64_write<B_K_CONTIGUOUS>(pieces, lds_a + (g & 1) * a_floats, lds_b + (g & 1) * b_floats, n, k, (g % chunks) * CHUNK, ftid);
+        };
+        ask(0);
+        write(0);
+        for (uint32_t g = 0; g < steps_total; g++) {
+            lds_barrier();  // chunk g is in LDS, and the multipliers are done with chunk g - 1
+            if (g + 1 < steps_total) { ask(g + 1); write(g + 1); }
+        }
+        return;
+    }
+
+    // ---- a multiplying wavefront
+    const uint32_t m = args.m, n = args.n, ldc = args.ldc;
+    const uint32_t j = lane & 15, quarter = lane >> 4;
+    const uint32_t col_tiles = (n + TILE - 1) / TILE, row_tiles = (m + TILE - 1) / TILE;
+    const bool owner = wave < row_tiles;
+    // the tiles of the rows past the twelfth: tile e of them belongs to wavefront e
+    const uint32_t extras = row_tiles > (uint32_t)MULTIPLIERS ? (row_tiles - MULTIPLIERS) * col_tiles : 0;
+    const bool extra = wave < extras;
+    const uint32_t extra_it = MULTIPLIERS + wave / col_tiles, extra_jt = wave % col_tiles;
+    auto fragment = [&](float (&f)[STEPS], const float *operand, uint32_t tile) {
+#pragma unroll
+        for (int i = 0; i < STEPS / 4; i++) {
+            const float4 v = *reinterpret_cast<const float4 *>(operand + swizzled(tile * TILE + j, STEPS * quarter + 4 * i));
+            f[4 * i] = v.x, f[4 * i + 1] = v.y, f[4 * i + 2] = v.z, f[4 * i + 3] = v.w;
+        }
+    };
+    floatx4 acc[4], acc_x;
+    uint32_t head = blockIdx.x, c = 0;
+    for (uint32_t g = 0; g < steps_total; g++) {
+        lds_barrier();  // chunk g is in LDS
+        if (c == 0) {
+#pragma unroll
+            for (int t = 0; t < 4; t++) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+            acc_x = floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+        const float *a_now = lds_a + (g & 1) * a_floats, *b_now = lds_b + (g & 1) * b_floats;
+        // steps of this chunk that hold values of k at all: quarter 0 has the chunk's first 16
+        const uint32_t steps = min((uint32_t)STEPS, k - c * CHUNK);
+        float a[STEPS], ax[STEPS];
+        if (owner) fragment(a, a_now, wave);
+        if (extra) fragment(ax, a_now, extra_it);
+        auto fragment_b = [&](float (&f)[STEPS], uint32_t t) {
+            if constexpr (B_K_CONTIGUOUS) {
+                fragment(f, b_now, t);
+            } else {
+                const float *p = b_now + STEPS * quarter * N64_J_PITCH + t * TILE + j;
+#pragma unroll
+                for (int s = 0; s < STEPS; s++) f[s] = p[s * N64_J_PITCH];
+            }
+        };
+        // transposed (B's fragment first): a lane's four results are C(16 row of tiles + j, 16 t + 4 quarter + r)
+        auto multiply = [&](auto whole) {  // whole: all 16 steps, without a test per step
+            constexpr bool WHOLE = decltype(whole)::value;
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                if ((uint32_t)t < col_tiles) {
+                    float b[STEPS];
+                    fragment_b(b, t);
+                    if (owner) {
+#pragma unroll
+                        for (int s = 0; s < STEPS; s++)
+                            if (WHOLE || (uint32_t)s < steps) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[s], a[s], acc[t], 0, 0, 0);
+                    }
+                    if (extra && extra_jt == (uint32_t)t) {
+#pragma unroll
+                        for (int s = 0; s < STEPS; s++)
+                            if (WHOLE || (uint32_t)s < steps) acc_x = __builtin_amdgcn_mfma_f32_16x16x4f32(b[s], ax[s], acc_x, 0, 0, 0);
+                    }
+                }
+            }
+        };
+        if (owner || extra) {
+            if (steps == STEPS) multiply(std::true_type{});
+            else multiply(std::false_type{});
+        }
+        if (++c == chunks) {
+            const uint32_t zo = head / batch_inner, zi = head - zo * batch_inner;
+            float *C = args.c + zo * args.c_bs + zi * args.c_bs2;
+            if (owner) {
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+                    if ((uint32_t)t < col_tiles) store_tile(acc[t], m, n, ldc, C, wave * TILE, t * TILE, lane);
+            }
+            if (extra) store_tile(acc_x, m, n, ldc, C, extra_it * TILE, extra_jt * TILE, lane);
+            c = 0, head += gridDim.x;
+        }
     }
 }
 
@@ -375,8 +492,8 @@ inline bool float4_rows(const void *p, size_t ld, const size_t bs[2]) {
 // Whether launch_gemm_small_batched takes this product; decided by the shape alone, so that a product and the same
 // product with an operand stored the other way round (a view of K against a materialised K^T) run the same arithmetic.
 bool gemm_small_batched_fits(size_t batch, size_t m, size_t n, size_t k) {
-    return batch >= 64 && batch < ((size_t)1 << 31) && m >= 1 && m <= (size_t)MAX_WAVES * TILE && k >= 1 &&
-           ((k <= CHUNK && n <= (size_t)MAX_MN && m <= (size_t)MAX_MN) || (n <= 64 && k <= 4096));
+    return batch >= 64 && batch < ((size_t)1 << 31) && m >= 1 && m <= (size_t)MAX_MN && k >= 1 &&
+           ((k <= CHUNK && n <= (size_t)MAX_MN) || (n <= 64 && k <= 4096));
 }
 
 int launch_gemm_small_batched(DeviceCtx &ctx, float *c, const float *a, const float *b, size_t batch_outer, size_t batch_inner, size_t m, size_t n,
@@ -388,17 +505,14 @@ int launch_gemm_small_batched(DeviceCtx &ctx, float *c, const float *a, const fl
     g.lda = (uint32_t)lda, g.ldb = (uint32_t)ldb, g.ldc = (uint32_t)ldc;
     g.a_bs = a_bs[0], g.b_bs = b_bs[0], g.c_bs = c_bs[0], g.a_bs2 = a_bs[1], g.b_bs2 = b_bs[1], g.c_bs2 = c_bs[1];
     g.batch_inner = (uint32_t)batch_inner;
-    const dim3 grid((unsigned)(batch_outer * batch_inner));
-    const size_t waves = std::max<size_t>(MIN_WAVES, (m + TILE - 1) / TILE);
-    const dim3 block((unsigned)(waves * WAVE));
+    g.batch = (uint32_t)(batch_outer * batch_inner);
+    const size_t cus = ctx.cus_per_xcd ? (size_t)ctx.cus_per_xcd * 8 : 256;
+    const dim3 grid((unsigned)std::min<size_t>(g.batch, cus)), block(PB_WAVES * WAVE);
     if (k <= CHUNK) {
         const bool a_vec = k % 4 == 0 && float4_rows(a, lda, a_bs);
         const bool b_vec = trans_b && k % 4 == 0 && float4_rows(b, ldb, b_bs);
-        g.batch = (uint32_t)(batch_outer * batch_inner);
         const size_t shmem = ((size_t)MAX_MN * CHUNK + 2 * (trans_b ? (size_t)MAX_MN * CHUNK : (size_t)CHUNK * J_PITCH)) * sizeof(float);
-        const size_t cus = ctx.cus_per_xcd ? (size_t)ctx.cus_per_xcd * 8 : 256;
-        const dim3 pgrid((unsigned)std::min<size_t>(g.batch, cus)), pblock(PB_WAVES * WAVE);
-#define GO(KC, AV, BV) hipLaunchKernelGGL((gemm_small_k64<KC, AV, BV>), pgrid, pblock, shmem, ctx.stream, g)
+#define GO(KC, AV, BV) hipLaunchKernelGGL((gemm_small_k64<KC, AV, BV>), grid, block, shmem, ctx.stream, g)
         if (trans_b) {
             if (a_vec && b_vec) GO(true, true, true);
             else if (a_vec) GO(true, true, false);
@@ -410,23 +524,9 @@ int launch_gemm_small_batched(DeviceCtx &ctx, float *c, const float *a, const fl
         }
 #undef GO
     } else {
-        const int nt = n <= 16 ? 1 : n <= 32 ? 2 : 4;
-        const bool b_vec = !trans_b && n % 4 == 0 && float4_rows(b, ldb, b_bs);
-        const size_t shmem = (waves * TILE * N64_K_PITCH + (trans_b ? (size_t)nt * TILE * N64_K_PITCH : (size_t)N64_CHUNK * J_PITCH_N64)) * sizeof(float);
-#define GO(KC, BV, NT) hipLaunchKernelGGL((gemm_small_n64<KC, BV, NT>), grid, block, shmem, ctx.stream, g)
-#define GO_NT(KC, BV)          \
-    if (nt == 1) GO(KC, BV, 1); \
-    else if (nt == 2) GO(KC, BV, 2); \
-    else GO(KC, BV, 4)
-        if (trans_b) {
-            GO_NT(true, false);
-        } else if (b_vec) {
-            GO_NT(false, true);
-        } else {
-            GO_NT(false, false);
-        }
-#undef GO_NT
-#undef GO
+        const size_t shmem = 2 * ((size_t)MAX_MN * CHUNK + (trans_b ? (size_t)64 * CHUNK : (size_t)CHUNK * N64_J_PITCH)) * sizeof(float);
+        if (trans_b) hipLaunchKernelGGL((gemm_small_n64<true>), grid, block, shmem, ctx.stream, g);
+        else hipLaunchKernelGGL((gemm_small_n64<false>), grid, block, shmem, ctx.stream, g);
     }
     return ctx.check(hipGetLastError(), "gemm (small batched) launch");
 }

@@ -234,3 +234,77 @@ def test_few_tiles_and_a_long_k_are_cut_along_k(ctx, case, m, k, n):
         check_bound(ctx.matmul(a, b), a, b, "random operands")
     finally:
         ctx.gemm_set_algorithm(D.GEMM_DEFAULT)
+
+
+def _laid_out(x, pad, offset):
+    """x [batch, rows, cols] as a flat array with `pad` unused floats behind every row and `offset` in front."""
+    batch, rows, cols = x.shape
+    full = np.zeros((batch, rows, cols + pad), np.float32)
+    full[:, :, :cols] = x
+    return np.concatenate([np.zeros(offset, np.float32), full.ravel()]), cols + pad
+
+
+def _many_small(ctx, a, b, trans_b=False, pad=(0, 0), offset=(0, 0), shared_b=False):
+    """C[z] = A[z] B[z] for a [batch, m, k] and b [batch, k, n] through one ahip_gemm call; B is handed over as
+    [batch, n, k] when trans_b, rows are `pad` floats longer than their contents, bases `offset` floats past 16-byte
+    boundaries.  Every extent handed to the library is taken from the arrays that were uploaded."""
+    batch, m, k = a.shape
+    n = b.shape[-1]
+    flat_a, lda = _laid_out(a, pad[0], offset[0])
+    bb = b[:1] if shared_b else b
+    flat_b, ldb = _laid_out(np.ascontiguousarray(bb.transpose(0, 2, 1)) if trans_b else bb, pad[1], offset[1])
+    da, db, dc = ctx.upload(flat_a), ctx.upload(flat_b), ctx.alloc(batch * m * n * 4)
+    try:
+        assert flat_a.size >= offset[0] + (batch - 1) * m * lda + (m - 1) * lda + k
+        rows_b = n if trans_b else k
+        assert flat_b.size >= offset[1] + ((0 if shared_b else batch - 1) * rows_b + rows_b - 1) * ldb + (k if trans_b else n)
+        ctx.gemm_raw(dc.ptr, da.ptr + 4 * offset[0], db.ptr + 4 * offset[1], None, batch, m, n, k, trans_b=trans_b, lda=lda, ldb=ldb,
+                     a_bs=m * lda, b_bs=0 if shared_b else rows_b * ldb, c_bs=m * n)
+        return ctx.download(dc, (batch, m, n))
+    finally:
+        for x in (da, db, dc):
+            ctx.free(x)
+
+
+# batch, m, n, k: the shapes that take the kernels of many small products (64 or more products, m <= 208 and either
+# k <= 64 and n <= 208 or n <= 64), at their limits, and their neighbours that do not
+MANY_SMALL = [(96, 197, 197, 64), (96, 197, 64, 197), (64, 208, 208, 64), (300, 197, 197, 64), (300, 197, 64, 197), (64, 1, 1, 1),
+              (65, 33, 7, 3), (70, 193, 190, 33), (64, 100, 17, 64), (64, 208, 64, 300), (64, 30, 64, 65), (70, 16, 16, 1000),
+              (64, 192, 48, 128), (64, 209, 64, 64), (64, 197, 209, 64), (63, 197, 197, 64), (64, 64, 65, 65)]
+
+
+@pytest.mark.parametrize("batch,m,n,k", MANY_SMALL)
+def test_many_small_products(ctx, case, batch, m, n, k):
+    case(f"{batch} products [{m},{k}] x [{k},{n}]")
+    a, b = ints(batch, m, k), ints(batch, k, n)
+    want = np.matmul(a.astype(np.float64), b.astype(np.float64)).astype(np.float32)
+    got = {}
+    for trans_b in (False, True):
+        got[trans_b] = _many_small(ctx, a, b, trans_b)
+        assert_bits_equal(got[trans_b], want, f"integer operands, trans_b={trans_b}")
+    # rows that are no whole float4s and bases off the 16-byte grid: the single-value loads
+    assert_bits_equal(_many_small(ctx, a, b, False, pad=(1, 3), offset=(1, 2)), want, "odd pitches and bases")
+    assert_bits_equal(_many_small(ctx, a, b, True, pad=(3, 1), offset=(3, 1)), want, "odd pitches and bases, trans_b")
+    assert_bits_equal(_many_small(ctx, a, b[:1].repeat(batch, 0), False, shared_b=True),
+                      np.matmul(a.astype(np.float64), b[:1].astype(np.float64)).astype(np.float32), "one B for every product")
+    a, b = RNG.standard_normal(a.shape).astype(np.float32), RNG.standard_normal(b.shape).astype(np.float32)
+    r0, r1 = _many_small(ctx, a, b, False), _many_small(ctx, a, b, True)
+    check_bound(r0, a, b, "random operands")
+    # a product and the same product through the other layout of B add the same numbers in the same order
+    assert_bits_equal(r1, r0, "B stored [n, k] against B stored [k, n]")
+    assert_bits_equal(_many_small(ctx, a, b, True, pad=(1, 2), offset=(2, 3)), r0, "padded, offset operands against dense ones")
+
+
+def test_many_small_products_land_in_their_places(ctx, case):
+    """Every (head, row, column) gets its own value: a tile written to the wrong head, row or column shows."""
+    case("placement of 300 x [197,64] x [64,197] and 300 x [197,197] x [197,64]")
+    batch, m = 300, 197
+    for n, k in ((197, 64), (64, 197)):
+        a = np.zeros((batch, m, k), np.float32)
+        b = np.zeros((batch, k, n), np.float32)
+        p = np.arange(batch) % k                      # head z multiplies through k = z % k only
+        a[np.arange(batch), :, p] = np.arange(1, m + 1)[None, :] + 256.0 * (np.arange(batch) % 7)[:, None]
+        b[np.arange(batch), p, :] = np.arange(1, n + 1)[None, :] * 2048.0
+        want = a[np.arange(batch), :, p][:, :, None] * b[np.arange(batch), p, :][:, None, :]
+        for trans_b in (False, True):
+            assert_bits_equal(_many_small(ctx, a, b, trans_b), want.astype(np.float32), f"n={n} k={k} trans_b={trans_b}")
