@@ -82,9 +82,8 @@ __device__ __forceinline__ void store_tile(const floatx4 &acc, uint32_t m, uint3
 
 // k <= 64, m and n <= 208.  One block of 16 wavefronts per compute unit walks the heads blockIdx.x, blockIdx.x + gridDim.x, ...
 //
-// LDS (160 KB): all of A as [208][64] and all of B, [208][64] when B's k axis is contiguous (both with the 16-byte pieces of a
-// row exchanged by piece ^= row % 16, which spreads a column of pieces over the banks without padding) or [64][209] when
-// B's columns are.
+// LDS (156 KB): all of A as [208][64] and all of B as [column][64], whichever way round B lies in memory, both with the
+// 16-byte pieces of a row exchanged by piece ^= row % 16, which spreads a column of pieces over the banks without padding.
 //
 // Twelve wavefronts multiply (three per SIMD) and four fetch (one per SIMD).  B is in LDS twice: while the multipliers
 // read one copy the fetchers fill the other with the next head's; the next head's A waits in the fetchers' registers (52
@@ -99,7 +98,6 @@ __device__ __forceinline__ void store_tile(const floatx4 &acc, uint32_t m, uint3
 constexpr int PB_WAVES = 16;
 constexpr int FETCHERS = 4, MULTIPLIERS = PB_WAVES - FETCHERS;
 constexpr int MAX_MN = 208;                                  // rows of A and columns of B
-constexpr int J_PITCH = MAX_MN + 1;                          // floats per LDS row of B stored [k][column]
 constexpr int VEC_PIECES = MAX_MN * (CHUNK / 4) / (FETCHERS * WAVE);   // float4s per fetching lane and operand: 13
 constexpr int PIECES = MAX_MN * CHUNK / (FETCHERS * WAVE);   // single values per fetching lane and operand: 52
 
@@ -158,11 +156,13 @@ __device__ __forceinline__ void load_columns(float (&v)[COUNT], __amdgpu_buffer_
         v[u] = in ? f : 0.0f;
     }
 }
+// ... written as [column][64] with exchanged pieces like an operand stored that way: the multipliers read B the same way
+// whichever way round it came (eight lanes of a wavefront meet in a bank here; the fetchers have the time).
 template <int FIRST, int COUNT>
 __device__ __forceinline__ void write_columns(const float (&v)[COUNT], float *dst, uint32_t ftid) {
     if (ftid >= MAX_MN) return;
 #pragma unroll
-    for (int u = 0; u < COUNT; u++) dst[(FIRST + u) * J_PITCH + ftid] = v[u];
+    for (int u = 0; u < COUNT; u++) dst[swizzled(ftid, FIRST + u)] = v[u];
 }
 // One operand of a head, global memory -> LDS, in two rounds of loads that are all asked for before the first is
 // written (the rounds of the float4 kind hold 7 and 6 pieces, of the others 26 and 26 or 32 and 32).  `extent` is the
@@ -200,7 +200,7 @@ template <bool B_K_CONTIGUOUS, bool A_VEC, bool B_VEC>
 __global__ __launch_bounds__(PB_WAVES * WAVE) void gemm_small_k64(SmallGemm args) {
     extern __shared__ __align__(16) float lds[];
     const uint32_t tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid >> 6;
-    constexpr uint32_t b_floats = B_K_CONTIGUOUS ? MAX_MN * CHUNK : CHUNK * J_PITCH;  // B is there twice, for this head and the next
+    constexpr uint32_t b_floats = MAX_MN * CHUNK;  // B is there twice, for this head and the next
     float *lds_a = lds, *lds_b = lds + MAX_MN * CHUNK;
     const uint32_t batch = args.batch, batch_inner = args.batch_inner;
     const uint32_t head0 = blockIdx.x, head_step = gridDim.x;  // the grid has at most as many blocks as there are heads
@@ -259,15 +259,7 @@ __global__ __launch_bounds__(PB_WAVES * WAVE) void gemm_small_k64(SmallGemm args
             f[4 * i] = v.x, f[4 * i + 1] = v.y, f[4 * i + 2] = v.z, f[4 * i + 3] = v.w;
         }
     };
-    auto fragment_b = [&](float (&f)[STEPS], uint32_t jt) {
-        if constexpr (B_K_CONTIGUOUS) {
-            fragment(f, b_now, jt);
-        } else {
-            const float *p = b_now + STEPS * quarter * J_PITCH + jt * TILE + j;
-#pragma unroll
-            for (int s = 0; s < STEPS; s++) f[s] = p[s * J_PITCH];
-        }
-    };
+    auto fragment_b = [&](float (&f)[STEPS], uint32_t jt) { fragment(f, b_now, jt); };
     for (uint32_t head = head0; head < batch; head += head_step) {
         lds_barrier();  // this head's A and B are in LDS
         const uint32_t zo = head / batch_inner, zi = head - zo * batch_inner;
@@ -301,8 +293,8 @@ __global__ __launch_bounds__(PB_WAVES * WAVE) void gemm_small_k64(SmallGemm args
     }
 }
 
-// n <= 64, m <= 208, any k.  LDS: a chunk of A, [208][64] with exchanged pieces, and the same chunk of B, [64][64]
-// with exchanged pieces when B's k axis is contiguous or [64][N64_J_PITCH] when its columns are; both twice.  While the
+// n <= 64, m <= 208, any k.  LDS: a chunk of A, [208][64] with exchanged pieces, and the same chunk of B as
+// [column][64] with exchanged pieces; both twice.  While the
 // multipliers work on chunk g out of one copy, the fetchers fill the other with chunk g + 1 (of the same head or the
 // first of the next), and one barrier per chunk separates the two.
 //
@@ -310,7 +302,6 @@ __global__ __launch_bounds__(PB_WAVES * WAVE) void gemm_small_k64(SmallGemm args
 // wavefronts 0 .. 3 as a fifth tile (13 tiles per SIMD).  A's rows are whole 16-byte pieces only by accident (197
 // floats per row of P), so the fetchers read them with buffer loads, which need no more than 4-byte alignment, and
 // zero what lies past k themselves: a row's last piece reaches into the next row.
-constexpr int N64_J_PITCH = 65;
 constexpr int N64_B_PIECES = CHUNK * 64 / (FETCHERS * WAVE);  // single values per fetching lane of a [64][64] chunk of B: 16
 
 // What a fetching lane holds of a chunk between asking for it and writing it to LDS.
@@ -364,9 +355,9 @@ __device__ __forceinline__ void n64_write(const N64Pieces<B_K_CONTIGUOUS> &v, fl
 #pragma unroll
         for (int u = 0; u < 4; u++) *reinterpret_cast<float4 *>(dst_b + swizzled((ftid >> 4) + 16 * u, 4 * q)) = within_k(v.b[u]);
     } else {
-        const uint32_t jj = ftid & 63;
+        const uint32_t jj = ftid & 63;  // [column][64] like an operand stored that way (eight lanes meet in a bank)
 #pragma unroll
-        for (int u = 0; u < N64_B_PIECES; u++) dst_b[((ftid >> 6) + 4 * u) * N64_J_PITCH + jj] = jj < n ? v.b[u] : 0.f;
+        for (int u = 0; u < N64_B_PIECES; u++) dst_b[swizzled(jj, (ftid >> 6) + 4 * u)] = jj < n ? v.b[u] : 0.f;
     }
 }
 
@@ -374,7 +365,7 @@ template <bool B_K_CONTIGUOUS>
 __global__ __launch_bounds__(PB_WAVES * WAVE) void gemm_small_n64(SmallGemm args) {
     extern __shared__ __align__(16) float lds[];
     const uint32_t tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid >> 6;
-    constexpr uint32_t a_floats = MAX_MN * CHUNK, b_floats = B_K_CONTIGUOUS ? 64 * CHUNK : CHUNK * N64_J_PITCH;
+    constexpr uint32_t a_floats = MAX_MN * CHUNK, b_floats = 64 * CHUNK;
     float *lds_a = lds, *lds_b = lds + 2 * a_floats;
     const uint32_t batch = args.batch, batch_inner = args.batch_inner, k = args.k;
     const uint32_t chunks = (k + CHUNK - 1) / CHUNK;
@@ -435,15 +426,7 @@ __global__ __launch_bounds__(PB_WAVES * WAVE) void gemm_small_n64(SmallGemm args
         float a[STEPS], ax[STEPS];
         if (owner) fragment(a, a_now, wave);
         if (extra) fragment(ax, a_now, extra_it);
-        auto fragment_b = [&](float (&f)[STEPS], uint32_t t) {
-            if constexpr (B_K_CONTIGUOUS) {
-                fragment(f, b_now, t);
-            } else {
-                const float *p = b_now + STEPS * quarter * N64_J_PITCH + t * TILE + j;
-#pragma unroll
-                for (int s = 0; s < STEPS; s++) f[s] = p[s * N64_J_PITCH];
-            }
-        };
+        auto fragment_b = [&](float (&f)[STEPS], uint32_t t) { fragment(f, b_now, t); };
         // transposed (B's fragment first): a lane's four results are C(16 row of tiles + j, 16 t + 4 quarter + r)
         auto multiply = [&](auto whole) {  // whole: all 16 steps, without a test per step
             constexpr bool WHOLE = decltype(whole)::value;
@@ -511,7 +494,7 @@ int launch_gemm_small_batched(DeviceCtx &ctx, float *c, const float *a, const fl
     if (k <= CHUNK) {
         const bool a_vec = k % 4 == 0 && float4_rows(a, lda, a_bs);
         const bool b_vec = trans_b && k % 4 == 0 && float4_rows(b, ldb, b_bs);
-        const size_t shmem = ((size_t)MAX_MN * CHUNK + 2 * (trans_b ? (size_t)MAX_MN * CHUNK : (size_t)CHUNK * J_PITCH)) * sizeof(float);
+        const size_t shmem = 3 * (size_t)MAX_MN * CHUNK * sizeof(float);
 #define GO(KC, AV, BV) hipLaunchKernelGGL((gemm_small_k64<KC, AV, BV>), grid, block, shmem, ctx.stream, g)
         if (trans_b) {
             if (a_vec && b_vec) GO(true, true, true);
@@ -524,7 +507,7 @@ int launch_gemm_small_batched(DeviceCtx &ctx, float *c, const float *a, const fl
         }
 #undef GO
     } else {
-        const size_t shmem = 2 * ((size_t)MAX_MN * CHUNK + (trans_b ? (size_t)64 * CHUNK : (size_t)CHUNK * N64_J_PITCH)) * sizeof(float);
+        const size_t shmem = 2 * ((size_t)MAX_MN * CHUNK + (size_t)64 * CHUNK) * sizeof(float);
         if (trans_b) hipLaunchKernelGGL((gemm_small_n64<true>), grid, block, shmem, ctx.stream, g);
         else hipLaunchKernelGGL((gemm_small_n64<false>), grid, block, shmem, ctx.stream, g);
     }

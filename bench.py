@@ -573,7 +573,7 @@ def build_next_rows(ctx, D, batch=256):
 
     rng = np.random.default_rng(5)
 
-    def gemm(name, b, m, n_, k, a_bs, b_bs, algorithms=(("fp32 MFMA", D.GEMM_FP32),)):
+    def gemm(name, b, m, n_, k, a_bs, b_bs, algorithms=(("fp32 MFMA", D.GEMM_FP32),), trans_b=False):
         # random operands: constant ones toggle fewer bits in the matrix cores and run at a higher clock
         a = ctx.upload(rng.standard_normal(((b if a_bs else 1) * m, k), dtype=np.float32))
         w = ctx.upload(rng.standard_normal(((b if b_bs else 1) * k, n_), dtype=np.float32) * np.float32(0.03))
@@ -585,7 +585,7 @@ def build_next_rows(ctx, D, batch=256):
 
             def launch(algo=algo):
                 ctx.gemm_set_algorithm(algo)
-                ctx.gemm_raw(c.ptr, a.ptr, w.ptr, None, b, m, n_, k, a_bs=a_bs, b_bs=b_bs, c_bs=m * n_)
+                ctx.gemm_raw(c.ptr, a.ptr, w.ptr, None, b, m, n_, k, trans_b=trans_b, a_bs=a_bs, b_bs=b_bs, c_bs=m * n_)
                 ctx.gemm_set_algorithm(D.GEMM_DEFAULT)
 
             rows.append(("%s (%s)" % (name, label), nbytes, 2.0 * b * m * n_ * k, launch))
@@ -610,6 +610,9 @@ def build_next_rows(ctx, D, batch=256):
     rows.append(("MatMul Gelu(A) x B, fc2 [%d,3072]x[3072,768] (bf16 x 3 incl. Gelu and split of A)" % M, 4 * (M * 4 * H + 4 * H * H + M * H),
                  2.0 * M * H * 4 * H, gelu_fc2))
     gemm("MatMul QK^T %d x [197,64]x[64,197]" % (batch * NH), batch * NH, T, T, DH, T * DH, DH * T)
+    # the same product with K where it lies, [197,64] per head, as a session that plans views hands it over (the operand has
+    # the same number of values either way round, so the upload above serves)
+    gemm("MatMul QK^T %d x [197,64]x[197,64]^T, K in place" % (batch * NH), batch * NH, T, T, DH, T * DH, DH * T, trans_b=True)
     gemm("MatMul PV %d x [197,197]x[197,64]" % (batch * NH), batch * NH, T, DH, T, T * T, T * DH)
     # QK^T -> scale -> Softmax -> PV in one kernel, heads read in place from the [b, t, 3 h d] result of the qkv product
     # and written as [b, t, h d]
