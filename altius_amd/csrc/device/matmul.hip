@@ -300,7 +300,10 @@ int launch_gemm_batch2(DeviceCtx &ctx, float *c, const float *a, const float *b,
     if (m >= lim || n >= lim || k >= lim || lda >= lim || ldb >= lim || ldc >= lim || m * ldc >= ((size_t)1 << 40))
         return ctx.fail(AHIP_ERR_UNSUPPORTED, "gemm: extent above 2^31");
     // Hundreds of small matrices (attention's two products per head): one block per matrix.
-    if (!has_post && !trans_a && alpha == 1.0f && (!c0 || beta == 0.0f) && !split_k_inner && gemm_small_batched_fits(batch, m, n, k))
+    // (its fetchers address a head's operand with 32-bit byte offsets: 2^29 floats per head at most)
+    const size_t a_extent = (m - 1) * lda + k, b_extent = trans_b ? (n - 1) * ldb + k : (k ? k - 1 : 0) * ldb + n;
+    if (!has_post && !trans_a && alpha == 1.0f && (!c0 || beta == 0.0f) && !split_k_inner && gemm_small_batched_fits(batch, m, n, k) &&
+        a_extent < ((size_t)1 << 29) && b_extent < ((size_t)1 << 29))
         return launch_gemm_small_batched(ctx, c, a, b, batch_outer, batch_inner, m, n, k, trans_b, lda, ldb, ldc, a_batch_strides, b_batch_strides,
                                          c_batch_strides);
     // The 128 x 64 tile when it leaves fewer idle columns (n = 64: 64 instead of 128 computed), and for long

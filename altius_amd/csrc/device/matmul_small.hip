@@ -104,9 +104,17 @@ constexpr int PIECES = MAX_MN * CHUNK / (FETCHERS * WAVE);   // single values pe
 // The float offset of k (a multiple of 4 for float4s) in row `row` of an operand stored [row][64] with exchanged pieces.
 __device__ __forceinline__ uint32_t swizzled(uint32_t row, uint32_t k) { return row * CHUNK + ((((k >> 2) ^ row) & 15) << 2) + (k & 3); }
 
-// The fetchers address an operand of a head as a buffer of its own: a thread's pieces differ by a multiple of the row
-// stride that is the same for all threads (the instruction's scalar offset), so that one vector register of offsets
-// serves them all, and pieces past the operand's last value read as zero without a test.
+// The fetchers address an operand of a head as a buffer of its own, so that pieces past the operand's last value (rows
+// past m, columns past n, values of k past the end in an operand stored [k][column]) read as zero without a test and,
+// for the last head of a tensor, without touching memory behind it.  The whole offset of a piece goes into the
+// instruction's vector offset: the scalar offset takes no part in the comparison with the buffer's size on this part.
+// (The launcher sends operands of 2^29 floats and more per head to the general kernel: offsets are 32 bits.)
+// One running offset per thread: without the empty asm the compiler keeps an offset register per piece and spills.
+__device__ __forceinline__ uint32_t next_piece(uint32_t offset, uint32_t step) {
+    offset += step;
+    asm volatile("" : "+v"(offset));
+    return offset;
+}
 typedef float f32x4_raw __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_raw __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t operand_buffer(const float *p, uint32_t floats) {
@@ -117,21 +125,23 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t operand_buffer(const float *p,
 // thread's pieces are 16 (float4s) or 4 (single values) rows apart at the same k; k past `k` reads as zero.
 template <int FIRST, int COUNT>
 __device__ __forceinline__ void load_rows(float4 (&v)[COUNT], __amdgpu_buffer_rsrc_t src, uint32_t ld, uint32_t k, uint32_t ftid) {
-    const uint32_t q = ftid & 15, offset = ((ftid >> 4) * ld + 4 * q) * 4;
+    const uint32_t q = ftid & 15;
+    uint32_t offset = (((ftid >> 4) + 16 * FIRST) * ld + 4 * q) * 4;
     const bool in = 4 * q < k;
 #pragma unroll
-    for (int u = 0; u < COUNT; u++) {
-        const f32x4_raw f = __builtin_bit_cast(f32x4_raw, __builtin_amdgcn_raw_buffer_load_b128(src, offset, 16 * (FIRST + u) * ld * 4, 0));
+    for (int u = 0; u < COUNT; u++, offset = next_piece(offset, 16 * ld * 4)) {
+        const f32x4_raw f = __builtin_bit_cast(f32x4_raw, __builtin_amdgcn_raw_buffer_load_b128(src, offset, 0, 0));
         v[u] = in ? make_float4(f.x, f.y, f.z, f.w) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 }
 template <int FIRST, int COUNT>
 __device__ __forceinline__ void load_rows(float (&v)[COUNT], __amdgpu_buffer_rsrc_t src, uint32_t ld, uint32_t k, uint32_t ftid) {
-    const uint32_t kk = ftid & 63, offset = ((ftid >> 6) * ld + kk) * 4;
+    const uint32_t kk = ftid & 63;
+    uint32_t offset = (((ftid >> 6) + 4 * FIRST) * ld + kk) * 4;
     const bool in = kk < k;
 #pragma unroll
-    for (int u = 0; u < COUNT; u++) {
-        const float f = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(src, offset, 4 * (FIRST + u) * ld * 4, 0));
+    for (int u = 0; u < COUNT; u++, offset = next_piece(offset, 4 * ld * 4)) {
+        const float f = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(src, offset, 0, 0));
         v[u] = in ? f : 0.0f;
     }
 }
@@ -150,9 +160,10 @@ __device__ __forceinline__ void write_rows(const float (&v)[COUNT], float *dst, 
 template <int FIRST, int COUNT>
 __device__ __forceinline__ void load_columns(float (&v)[COUNT], __amdgpu_buffer_rsrc_t src, uint32_t ld, uint32_t cols, uint32_t ftid) {
     const bool in = ftid < cols;
+    uint32_t offset = (FIRST * ld + ftid) * 4;
 #pragma unroll
-    for (int u = 0; u < COUNT; u++) {
-        const float f = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(src, ftid * 4, (FIRST + u) * ld * 4, 0));
+    for (int u = 0; u < COUNT; u++, offset = next_piece(offset, ld * 4)) {
+        const float f = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(src, offset, 0, 0));
         v[u] = in ? f : 0.0f;
     }
 }
@@ -164,36 +175,48 @@ __device__ __forceinline__ void write_columns(const float (&v)[COUNT], float *ds
 #pragma unroll
     for (int u = 0; u < COUNT; u++) dst[swizzled(ftid, FIRST + u)] = v[u];
 }
-// One operand of a head, global memory -> LDS, in two rounds of loads that are all asked for before the first is
-// written (the rounds of the float4 kind hold 7 and 6 pieces, of the others 26 and 26 or 32 and 32).  `extent` is the
+// One operand of a head, global memory -> LDS, in rounds of loads that are all asked for before the first is written
+// (two rounds of 7 and 6 float4s; four of 13 single values for rows, two of 32 for columns).  `extent` is the
 // operand's number of rows (ROWS) or columns.
 template <bool ROWS, bool VEC>
 __device__ __forceinline__ void copy_operand(float *dst, const float *src, uint32_t ld, uint32_t extent, uint32_t k, uint32_t ftid) {
+    // between rounds: keeps the compiler from asking for the next round before this one is written (registers)
+    auto round_done = [] { asm volatile("" ::: "memory"); };
     if constexpr (ROWS && VEC) {
         const __amdgpu_buffer_rsrc_t buf = operand_buffer(src, (extent - 1) * ld + k);
         constexpr int H = (VEC_PIECES + 1) / 2;
         float4 v0[H], v1[VEC_PIECES - H];
         load_rows<0, H>(v0, buf, ld, k, ftid);
         write_rows<0, H>(v0, dst, ftid);
+        round_done();
         load_rows<H, VEC_PIECES - H>(v1, buf, ld, k, ftid);
         write_rows<H, VEC_PIECES - H>(v1, dst, ftid);
     } else if constexpr (ROWS) {
         const __amdgpu_buffer_rsrc_t buf = operand_buffer(src, (extent - 1) * ld + k);
-        constexpr int H = PIECES / 2;
-        float v0[H], v1[PIECES - H];
+        constexpr int H = PIECES / 4;
+        float v0[H], v1[H], v2[H], v3[H];
         load_rows<0, H>(v0, buf, ld, k, ftid);
         write_rows<0, H>(v0, dst, ftid);
-        load_rows<H, PIECES - H>(v1, buf, ld, k, ftid);
-        write_rows<H, PIECES - H>(v1, dst, ftid);
+        round_done();
+        load_rows<H, H>(v1, buf, ld, k, ftid);
+        write_rows<H, H>(v1, dst, ftid);
+        round_done();
+        load_rows<2 * H, H>(v2, buf, ld, k, ftid);
+        write_rows<2 * H, H>(v2, dst, ftid);
+        round_done();
+        load_rows<3 * H, H>(v3, buf, ld, k, ftid);
+        write_rows<3 * H, H>(v3, dst, ftid);
     } else {
         const __amdgpu_buffer_rsrc_t buf = operand_buffer(src, (k - 1) * ld + extent);
         constexpr int H = CHUNK / 2;
         float v0[H], v1[CHUNK - H];
         load_columns<0, H>(v0, buf, ld, extent, ftid);
         write_columns<0, H>(v0, dst, ftid);
+        round_done();
         load_columns<H, CHUNK - H>(v1, buf, ld, extent, ftid);
         write_columns<H, CHUNK - H>(v1, dst, ftid);
     }
+    round_done();
 }
 
 template <bool B_K_CONTIGUOUS, bool A_VEC, bool B_VEC>
@@ -318,26 +341,26 @@ __device__ __forceinline__ void n64_ask(N64Pieces<B_K_CONTIGUOUS> &v, const floa
                                         uint32_t ldb, uint32_t k0, uint32_t ftid) {
     const uint32_t q = ftid & 15;
     const __amdgpu_buffer_rsrc_t abuf = operand_buffer(A, (m - 1) * lda + k);
-    const uint32_t a_offset = ((ftid >> 4) * lda + 4 * q) * 4;
+    uint32_t a_offset = ((ftid >> 4) * lda + k0 + 4 * q) * 4;
 #pragma unroll
-    for (int u = 0; u < VEC_PIECES; u++) {
-        const f32x4_raw f = __builtin_bit_cast(f32x4_raw, __builtin_amdgcn_raw_buffer_load_b128(abuf, a_offset, (16 * u * lda + k0) * 4, 0));
+    for (int u = 0; u < VEC_PIECES; u++, a_offset = next_piece(a_offset, 16 * lda * 4)) {
+        const f32x4_raw f = __builtin_bit_cast(f32x4_raw, __builtin_amdgcn_raw_buffer_load_b128(abuf, a_offset, 0, 0));
         v.a[u] = make_float4(f.x, f.y, f.z, f.w);
     }
     if constexpr (B_K_CONTIGUOUS) {  // B as [column][k]: 4 float4s per lane, 16 columns apart
         const __amdgpu_buffer_rsrc_t bbuf = operand_buffer(B, (n - 1) * ldb + k);
-        const uint32_t b_offset = ((ftid >> 4) * ldb + 4 * q) * 4;
+        uint32_t b_offset = ((ftid >> 4) * ldb + k0 + 4 * q) * 4;
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const f32x4_raw f = __builtin_bit_cast(f32x4_raw, __builtin_amdgcn_raw_buffer_load_b128(bbuf, b_offset, (16 * u * ldb + k0) * 4, 0));
+        for (int u = 0; u < 4; u++, b_offset = next_piece(b_offset, 16 * ldb * 4)) {
+            const f32x4_raw f = __builtin_bit_cast(f32x4_raw, __builtin_amdgcn_raw_buffer_load_b128(bbuf, b_offset, 0, 0));
             v.b[u] = make_float4(f.x, f.y, f.z, f.w);
         }
     } else {  // B as [k][column]: 16 values per lane, 4 rows of k apart; rows past k lie past the buffer's end
         const __amdgpu_buffer_rsrc_t bbuf = operand_buffer(B, (k - 1) * ldb + n);
-        const uint32_t b_offset = ((ftid >> 6) * ldb + (ftid & 63)) * 4;
+        uint32_t b_offset = ((k0 + (ftid >> 6)) * ldb + (ftid & 63)) * 4;
 #pragma unroll
-        for (int u = 0; u < N64_B_PIECES; u++)
-            v.b[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(bbuf, b_offset, (k0 + 4 * u) * ldb * 4, 0));
+        for (int u = 0; u < N64_B_PIECES; u++, b_offset = next_piece(b_offset, 4 * ldb * 4))
+            v.b[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(bbuf, b_offset, 0, 0));
     }
 }
 
