@@ -38,6 +38,28 @@ def test_device_run_equals_host_run(case, ctx):
     ctx.free(d_x)
 
 
+def test_a_session_without_its_timing_events_runs_the_same(case, ctx):
+    """with_device_timing(False): no pair of events around a run, last_device_ms() reports 0, results and the
+    prepared-arguments route unchanged."""
+    case("run_device without device timing")
+    c = synth.cfg2(batch=2)
+    timed = HipSessionBuilder(chain_model(c)).build()
+    plain = HipSessionBuilder(chain_model(c)).with_device_timing(False).build()
+    (want,) = timed.run([c["x"]])
+    (got,) = plain.run([c["x"]])
+    assert_bits_equal(got, want, "run() without timing events")
+    assert timed.last_device_ms() > 0 and plain.last_device_ms() == 0
+    d_x = ctx.upload(c["x"])
+    prepared = plain.prepare_device_inputs([(d_x.ptr, c["x"].shape, np.float32)])
+    for i in range(3):
+        (out,) = plain.run_device_prepared(prepared)
+        plain.synchronize()
+        assert plain.last_device_ms() == 0
+        assert_bits_equal(ctx.download(out, out.shape), want, f"prepared device run {i}")
+        out.free()
+    ctx.free(d_x)
+
+
 def test_outputs_feed_another_session_and_outlive_theirs(case, ctx):
     """LayerNorm chain on one session, erf-GELU chain on another, device to device; the first session
     is closed before its output is read or freed."""
