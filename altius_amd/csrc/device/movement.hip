@@ -868,7 +868,7 @@ int launch_transpose(DeviceCtx &ctx, void *out, const void *in, int elem_size, i
             }
         }
     }
-    // Dense transposed matrices with a short R axis, too large for one block: panels of 32 columns (with 16, which a
+    // Dense transposed matrices with a short R axis, too large for one block: panels of 32 or 64 columns (with 16, which a
     // longer R axis would need to fit LDS, the segments read are half lines and the 64 x 64 patches are ahead).
     if (elem_size == 4 && g.c_out_str == g.r_len && g.c_len % PANEL == 0 && g.r_in_str % 4 == 0 && aligned16(out) && aligned16(in) && batches <= 65535 &&
         (size_t)PANEL * (g.r_len | 1u) * 4 <= 64 * 1024) {
@@ -876,12 +876,18 @@ int launch_transpose(DeviceCtx &ctx, void *out, const void *in, int elem_size, i
         for (int i = 0; i < g.brank; i++) lines_up = lines_up && g.b_in_str[i] % 4 == 0 && g.b_out_str[i] % 4 == 0;
         if (lines_up) {
             const uint32_t pitch = g.r_len | 1u;
-            const dim3 grid((unsigned)(g.c_len / PANEL), (unsigned)batches);
-            const size_t lds_bytes = (size_t)PANEL * pitch * 4;
+            // twice as wide where that still fits LDS: the segments read are two whole lines
+            const bool wide = g.c_len % (2 * PANEL) == 0 && (size_t)2 * PANEL * pitch * 4 <= 64 * 1024;
+            const uint32_t tc = wide ? 2 * PANEL : PANEL;
+            const dim3 grid((unsigned)(g.c_len / tc), (unsigned)batches);
+            const size_t lds_bytes = (size_t)tc * pitch * 4;
             const FastDiv rdiv = make_fastdiv(g.r_len);
             uint32_t *o = static_cast<uint32_t *>(out);
             const uint32_t *x = static_cast<const uint32_t *>(in);
-            if (ctx.streaming(total * 4)) hipLaunchKernelGGL((transpose_panel<PANEL, true>), grid, dim3(PANEL_BLOCK), lds_bytes, ctx.stream, o, x, g, pitch, rdiv);
+            const bool nt = ctx.streaming(total * 4);
+            if (wide && nt) hipLaunchKernelGGL((transpose_panel<2 * PANEL, true>), grid, dim3(PANEL_BLOCK), lds_bytes, ctx.stream, o, x, g, pitch, rdiv);
+            else if (wide) hipLaunchKernelGGL((transpose_panel<2 * PANEL, false>), grid, dim3(PANEL_BLOCK), lds_bytes, ctx.stream, o, x, g, pitch, rdiv);
+            else if (nt) hipLaunchKernelGGL((transpose_panel<PANEL, true>), grid, dim3(PANEL_BLOCK), lds_bytes, ctx.stream, o, x, g, pitch, rdiv);
             else hipLaunchKernelGGL((transpose_panel<PANEL, false>), grid, dim3(PANEL_BLOCK), lds_bytes, ctx.stream, o, x, g, pitch, rdiv);
             return ctx.check(hipGetLastError(), "transpose_panel launch");
         }

@@ -35,8 +35,10 @@ TRANSPOSES = [
     # both extents and pitches whole float4s: 16-byte accesses on both sides, tiles dealt diagonally
     ((256, 320), (1, 0)), ((3, 64, 28, 28), (0, 2, 3, 1)), ((3, 28, 28, 64), (0, 3, 1, 2)), ((68, 132), (1, 0)),
     ((5, 100, 72), (0, 2, 1)), ((100, 5, 72), (2, 1, 0)), ((24, 16, 20, 32), (3, 2, 1, 0)), ((1000, 16), (1, 0)),
-    # dense transposed matrices too large for one block: panels of 32 and of 16 columns, odd and even row counts
+    # dense transposed matrices too large for one block: panels of 64 columns where 64 rows of LDS hold the row axis, of 32
+    # otherwise; odd and even row counts, either side of both limits
     ((3, 197, 768), (0, 2, 1)), ((2, 600, 112), (0, 2, 1)), ((1001, 64), (1, 0)), ((2, 3, 500, 96), (0, 1, 3, 2)), ((510, 160), (1, 0)),
+    ((3, 100, 128), (0, 2, 1)), ((2, 255, 192), (0, 2, 1)), ((2, 257, 192), (0, 2, 1)), ((2, 511, 64), (0, 2, 1)),
     # 4-byte elements in 64 x 64 patches with 16-byte accesses wherever the rows start: odd extents on either side
     ((5000, 70), (1, 0)), ((70, 5000), (1, 0)), ((2001, 129), (1, 0)), ((3, 1029, 67), (0, 2, 1)), ((4099, 68), (1, 0)), ((3, 130, 5, 66), (0, 3, 2, 1)),
 ]
