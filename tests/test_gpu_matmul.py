@@ -266,11 +266,11 @@ def _many_small(ctx, a, b, trans_b=False, pad=(0, 0), offset=(0, 0), shared_b=Fa
             ctx.free(x)
 
 
-# batch, m, n, k: the shapes that take the kernels of many small products (64 or more products, m <= 208 and either
+# batch, m, n, k: the shapes that take the kernels of many small products (128 or more products, m <= 208 and either
 # k <= 64 and n <= 208 or n <= 64), at their limits, and their neighbours that do not
-MANY_SMALL = [(96, 197, 197, 64), (96, 197, 64, 197), (64, 208, 208, 64), (300, 197, 197, 64), (300, 197, 64, 197), (64, 1, 1, 1),
-              (65, 33, 7, 3), (70, 193, 190, 33), (64, 100, 17, 64), (64, 208, 64, 300), (64, 30, 64, 65), (70, 16, 16, 1000),
-              (64, 192, 48, 128), (64, 209, 64, 64), (64, 197, 209, 64), (63, 197, 197, 64), (64, 64, 65, 65)]
+MANY_SMALL = [(144, 197, 197, 64), (144, 197, 64, 197), (128, 208, 208, 64), (300, 197, 197, 64), (300, 197, 64, 197), (128, 1, 1, 1),
+              (129, 33, 7, 3), (130, 193, 190, 33), (128, 100, 17, 64), (128, 208, 64, 300), (128, 30, 64, 65), (130, 16, 16, 1000),
+              (128, 192, 48, 128), (128, 209, 64, 64), (128, 197, 209, 64), (127, 197, 197, 64), (128, 64, 65, 65)]
 
 
 @pytest.mark.parametrize("batch,m,n,k", MANY_SMALL)
