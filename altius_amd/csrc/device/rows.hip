@@ -1113,16 +1113,22 @@ void softmax_block_go(bool nt, hipStream_t s, size_t rows, size_t resident, floa
     if (nt) hipLaunchKernelGGL((softmax_block_regs<THREADS, NCH, true>), grid, dim3(THREADS), 0, s, out, in, len);
     else hipLaunchKernelGGL((softmax_block_regs<THREADS, NCH, false>), grid, dim3(THREADS), 0, s, out, in, len);
 }
-// Threads of a block and float4 per thread for a row that starts anywhere: two float4 per thread up to 2048 float4 in
-// the row, then the fewest that 1024 threads cover it with; the threads are the whole wavefronts that hold the row's
-// at most len / 4 whole float4s (the elements ahead of them and behind them ride along in the first threads).  From 8 K float4 on
-// blocks of 512 threads with 18 or 20 each, then blocks of 1024 threads, one to a CU.
+// Threads of a block and float4 per thread for a row of len / 4 whole float4s that starts anywhere (the elements ahead
+// of them and behind them ride along in the first threads).  The threads are the whole wavefronts that hold the row at
+// the chosen float4 per thread.  Blocks of 640 to 768 threads run 2 to 4 points of the HBM peak ahead of blocks of 896
+// to 1024 with fewer float4 each (three of them fit a CU where two of the larger do): Softmax takes two float4 per thread
+// up to 768 threads, then the fewest that 1024 threads cover the row with; LayerNormalization, which also waits for its
+// scale and bias, keeps to 768 threads (832 with four float4) up to eight float4 per thread and takes sixteen on at most
+// 512 threads from there to 8 K float4.  Beyond 8 K float4 both take blocks of 512 threads with 18 or 20 each, then
+// blocks of 1024 threads, one to a CU.
 struct AnyLayout {
     int threads, nch;
 };
-inline AnyLayout any_layout(size_t len) {
+inline AnyLayout any_layout(size_t len, bool layer_norm) {
     const size_t v = len / 4;
-    const int nch = v <= 2048 ? 2 : v <= 3072 ? 3 : v <= 4096 ? 4 : v <= 6144 ? 6 : v <= 8192 ? 8 : 0;
+    int nch;
+    if (layer_norm) nch = v <= 1536 ? 2 : v <= 2304 ? 3 : v <= 3328 ? 4 : v <= 4608 ? 6 : v <= 6144 ? 8 : v <= 8192 ? 16 : 0;
+    else nch = v <= 1536 ? 2 : v <= 3072 ? 3 : v <= 4096 ? 4 : v <= 6144 ? 6 : v <= 8192 ? 8 : 0;
     if (nch) return AnyLayout{(int)(((v + nch - 1) / nch + WAVE - 1) / WAVE * WAVE), nch};
     if (v <= 512 * 18) return AnyLayout{512, 18};
     if (v <= 512 * 20) return AnyLayout{512, 20};
@@ -1149,7 +1155,7 @@ inline bool aligned128(const void *p) { return (reinterpret_cast<uintptr_t>(p) &
 // Softmax / LayerNormalization over rows of more than 1024 and at most 65536 elements that start anywhere.
 bool softmax_anywhere_launch(bool nt, hipStream_t s, size_t rows, float *out, const float *in, size_t len) {
     const bool edges = !(len % 32 == 0 && aligned128(in) && aligned128(out));  // not a stack of whole 128-byte lines
-    const AnyLayout lay = any_layout(len);
+    const AnyLayout lay = any_layout(len, false);
     const dim3 grid((unsigned)rows), block((unsigned)lay.threads);
 #define ALTIUS_GO(N, W)                                                                              \
     case N:                                                                                          \
@@ -1162,7 +1168,7 @@ bool softmax_anywhere_launch(bool nt, hipStream_t s, size_t rows, float *out, co
 bool layernorm_anywhere_launch(bool nt, hipStream_t s, size_t rows, float *out, const float *in, const float *gamma, const float *beta, size_t len,
                                float eps) {
     const bool edges = !(len % 32 == 0 && aligned128(in) && aligned128(out));
-    const AnyLayout lay = any_layout(len);
+    const AnyLayout lay = any_layout(len, true);
     const dim3 grid((unsigned)rows), block((unsigned)lay.threads);
     // Scale and bias between the two reductions: 2 to 3.5 points of the HBM peak for blocks of up to 512 threads with
     // two float4 each (rows of up to 4 K elements), 5 lost with 640 and 768 threads; behind the reductions otherwise.

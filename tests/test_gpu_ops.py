@@ -270,6 +270,7 @@ SOFTMAX_SHAPES = [[1, 2, 3], [3, 28, 28], [16, 512, 512], [2, 12, 197, 197], [5,
                   [3, 1284], [3, 2052], [2, 3076], [2, 4608], [2, 6144], [2, 6148], [2, 12288],  # either side of every block width
                   [5, 384], [7, 640], [6, 896], [3, 1088], [9, 1152], [13, 320],  # a wavefront per row, last chunk partly filled
                   [7, 1030], [5, 2049], [3, 4097], [3, 9999], [2, 16381], [2, 16383], [2, 50257],  # rows that start anywhere: the aligned cover of a row in registers
+                  [2, 6147], [2, 6149], [2, 7001], [2, 12291], [2, 12293], [2, 24579], [1, 32771], [1, 36001], [1, 40961],  # either side of each step in its float4 per thread
                   [2, 20000], [2, 32768], [1, 49152], [2, 65536], [2, 30522], [1, 65533], [1, 65540],  # 6 to 16 float4 per thread up to 65536 elements, three passes above
                   [9, 1026], [6, 1281], [7, 1535], [5, 1537], [5, 1793], [4, 2047], [3, 2050],  # rows that start anywhere, a wavefront per row: 5 to 8 float4 per lane
                   [2, 49156], [1, 52000], [2, 53248], [1, 53245], [1, 53249]]  # thirteen float4 per thread, and just past them
@@ -314,6 +315,8 @@ LN_SHAPES = [[1, 20, 10], [2, 197, 768], [3, 5, 197], [4, 1], [5, 64], [3, 1024]
              [3, 1284], [3, 2052], [2, 3076], [2, 4608], [2, 6144], [2, 6148], [2, 12288],  # either side of every block width
              [5, 384], [7, 640], [6, 896], [3, 1088], [9, 1152], [1, 512], [13, 320],  # a wavefront per row, last chunk partly filled, rows not a multiple of the block's four
              [7, 1030], [5, 2049], [3, 4097], [3, 9999], [2, 16383], [2, 50257],  # rows that start anywhere: the aligned cover of a row in registers
+             [2, 6147], [2, 6149], [2, 9219], [2, 9221], [2, 13315], [2, 13317], [2, 18435], [2, 18437],  # either side of each step in its float4 per thread
+             [2, 24579], [2, 24581], [1, 32771], [1, 32773], [1, 36001], [1, 40961],
              [2, 20000], [2, 32768], [1, 49152], [2, 65536], [2, 30522], [1, 65533], [1, 65540],  # 6 to 16 float4 per thread up to 65536 elements, three passes above
              [9, 1025], [6, 1281], [7, 1535], [5, 1537], [5, 1793], [4, 2047], [3, 2050],  # rows that start anywhere, a wavefront per row: 5 to 8 float4 per lane
              [2, 49156], [1, 52000], [2, 53248], [1, 53245], [1, 53249]]  # thirteen float4 per thread, and just past them
