@@ -87,9 +87,10 @@ __device__ __forceinline__ void store_tile(const floatx4 &acc, uint32_t m, uint3
 //
 // Twelve wavefronts multiply (three per SIMD) and four fetch (one per SIMD).  B is in LDS twice: while the multipliers
 // read one copy the fetchers fill the other with the next head's; the next head's A waits in the fetchers' registers (52
-// per lane) and is written between two barriers when the multipliers are done.  The two kinds of work are kept in different wavefronts because the hardware
-// counts a wavefront's loads and stores in one counter: a wavefront that waits for a load it issued before storing results
-// waits for the stores too, and the head's last stores take several microseconds to drain.
+// per lane) and is written between two barriers when the multipliers are done.  The two kinds of work are kept in
+// different wavefronts because the hardware counts a wavefront's loads and stores in one counter: a wavefront that waits
+// for a load it issued before storing results waits for the stores too, and the head's last stores take several
+// microseconds to drain.
 //
 // A multiplier sweeps a row of tiles of C from left to right, so that the 64-byte pieces it stores complete each other's
 // cache lines while those are still on their way out (pieces that meet a half-written line much later cost twice the
