@@ -23,6 +23,7 @@ using dev::make_fastdiv;
 constexpr int BLOCK = 256;
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool aligned128(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 127u) == 0; }
 
 // ---- generic strided copy --------------------------------------------------------------------
 // Logical index space dims[0..rank) (axis 0 innermost here); element `idx` is read at
@@ -112,6 +113,33 @@ struct TransGeom {
     int brank;
 };
 
+// Which patch a block takes where pieces of a patch start and end inside cache lines (single elements at odd
+// addresses; 16-byte accesses along rows whose pitch is not a whole number of 128-byte lines).  The patch next door
+// completes such a line.  Blocks i, i + 8, i + 16, ... of a launch run on one XCD, under one L2: each of the eight takes
+// a run of consecutive patches (in the order of its blocks), so that the parts of a line meet in one L2 while it is
+// still there, instead of being fetched twice and going out to memory as two partial lines from two XCDs
+// ([50257, 768] -> [768, 50257]: 11 % more bytes written than the result holds and 65 % of the HBM peak with patches
+// dealt out row by row, 72 % this way; the other way round 69 -> 84 %).  A run goes along one axis in a band of `band`
+// patches across: neighbours along the run's axis are `band` blocks apart, neighbours across it follow each other.
+// Where blocks land is a matter of speed only: any order of the patches gives the same result.
+// along_r: runs go along R (whose pieces are written), else along C (whose pieces are read).
+__device__ __forceinline__ void patch_of_block(bool along_r, uint32_t band, uint32_t &bx, uint32_t &by) {
+    const uint32_t nx = gridDim.x, ny = gridDim.y, patches = nx * ny;
+    const uint32_t id = blockIdx.y * nx + blockIdx.x, xcd = id & 7u, each = patches >> 3, more = patches & 7u;
+    const uint32_t turn = xcd * each + (xcd < more ? xcd : more) + (id >> 3);  // a bijection of 0 .. patches - 1
+    const uint32_t n_run = along_r ? ny : nx, n_across = along_r ? nx : ny;
+    const uint32_t whole = n_across / band * band, in_whole = whole * n_run;  // patches in bands of full width
+    uint32_t run, across;
+    if (turn < in_whole) {
+        const uint32_t b = turn / (band * n_run), rest = turn - b * band * n_run;
+        run = rest / band, across = b * band + rest - run * band;
+    } else {
+        const uint32_t w = n_across - whole, rest = turn - in_whole;  // the last, narrower band
+        run = rest / w, across = whole + rest - run * w;
+    }
+    bx = along_r ? across : run, by = along_r ? run : across;
+}
+
 template <class T>
 __global__ __launch_bounds__(BLOCK) void transpose_tiled(T *__restrict__ out, const T *__restrict__ in, TransGeom g) {
     __shared__ T tile[TILE][TILE + 1];
@@ -126,7 +154,9 @@ __global__ __launch_bounds__(BLOCK) void transpose_tiled(T *__restrict__ out, co
             rest = q;
         }
     }
-    const uint32_t c0 = blockIdx.x * TILE, r0 = blockIdx.y * TILE;
+    uint32_t bx, by;
+    patch_of_block(true, 8, bx, by);  // both sides move single elements
+    const uint32_t c0 = bx * TILE, r0 = by * TILE;
     const uint32_t tx = threadIdx.x & (TILE - 1), ty = threadIdx.x / TILE;  // 64 x 4
     // read: lane tx walks C, ty (+4k) walks R; all sixteen loads are requested before the first goes to LDS
     T v[TILE / (BLOCK / TILE)];
@@ -147,10 +177,11 @@ __global__ __launch_bounds__(BLOCK) void transpose_tiled(T *__restrict__ out, co
 }
 
 // The same patch with 16-byte accesses on both sides, for 4-byte elements when both extents, both strides and every
-// batch offset are multiples of 4 and the tensors are 16-byte aligned: a thread reads four float4 along C and writes
-// four float4 along R (each gathered from four LDS rows).  The pitch of 65 words keeps both the row-wise stores and
-// the column-wise gathers of a wavefront on 64 different banks.
-template <bool NT>
+// batch offset are multiples of 4, the tensors are 16-byte aligned and the rows written start on 128-byte boundaries:
+// a thread reads four float4 along C and writes four float4 along R (each gathered from four LDS rows).  The pitch
+// of 65 words keeps both the row-wise stores and the column-wise gathers of a wavefront on 64 different banks.
+// LINES: the rows read start on 128-byte boundaries too.
+template <bool NT, bool LINES>
 __global__ __launch_bounds__(BLOCK) void transpose_tiled_vec4(uint32_t *__restrict__ out, const uint32_t *__restrict__ in, TransGeom g) {
     __shared__ uint32_t tile[TILE][TILE + 1];
     uint32_t rest = blockIdx.z, src0 = 0, dst0 = 0;
@@ -164,11 +195,17 @@ __global__ __launch_bounds__(BLOCK) void transpose_tiled_vec4(uint32_t *__restri
             rest = q;
         }
     }
-    // Tiles are dealt diagonally: blocks that run together (consecutive blockIdx.x) then differ in R as well as in C, so
-    // with a pitch that is a large power of two their rows do not all fall on the same memory channels.
-    uint32_t by = blockIdx.y + blockIdx.x;
-    by = by >= gridDim.y ? by % gridDim.y : by;
-    const uint32_t c0 = blockIdx.x * TILE, r0 = by * TILE;
+    uint32_t bx, by;
+    if (LINES) {
+        // Pitches of whole lines: tiles are dealt diagonally.  Blocks that run together (consecutive blockIdx.x) then differ
+        // in R as well as in C, so with a pitch that is a large power of two their rows do not all fall on the same memory
+        // channels.
+        bx = blockIdx.x, by = blockIdx.y + blockIdx.x;
+        by = by >= gridDim.y ? by % gridDim.y : by;
+    } else {
+        patch_of_block(true, 8, bx, by);
+    }
+    const uint32_t c0 = bx * TILE, r0 = by * TILE;
     const uint32_t q4 = threadIdx.x & 15, line = threadIdx.x >> 4;  // 16 float4 per 64-wide line, 16 lines per pass
     u32x4 v[4];
 #pragma unroll
@@ -200,10 +237,10 @@ __global__ __launch_bounds__(BLOCK) void transpose_tiled_vec4(uint32_t *__restri
 }
 
 // The 64 x 64 patch of 4-byte elements when only one side lines up for 16-byte accesses (an odd R extent:
-// [50257, 768] -> [768, 50257]; or an odd C extent the other way round): that side moves float4s as in
-// transpose_tiled_vec4, the other single elements as in transpose_tiled.  (16-byte accesses on 4-byte boundaries are
-// no way out here: a wavefront's store is four separate 256-byte pieces, and cut at odd addresses they run at half
-// the speed of the single elements.)
+// [50257, 768] -> [768, 50257], or rows written that do not start on 128-byte boundaries; or an odd C extent the
+// other way round): that side moves float4s as in transpose_tiled_vec4, the other single elements as in
+// transpose_tiled.  (16-byte stores are no way out on the written side: a wavefront's store is four separate 256-byte
+// pieces, and where those straddle cache lines they run at half the speed of the single elements.)
 template <bool LOAD4, bool NT>
 __global__ __launch_bounds__(BLOCK) void transpose_tiled_mixed(uint32_t *__restrict__ out, const uint32_t *__restrict__ in, TransGeom g) {
     __shared__ uint32_t tile[TILE][TILE + 1];
@@ -218,9 +255,9 @@ __global__ __launch_bounds__(BLOCK) void transpose_tiled_mixed(uint32_t *__restr
             rest = q;
         }
     }
-    uint32_t by = blockIdx.y + blockIdx.x;  // tiles dealt diagonally, see transpose_tiled_vec4
-    by = by >= gridDim.y ? by % gridDim.y : by;
-    const uint32_t c0 = blockIdx.x * TILE, r0 = by * TILE;
+    uint32_t bx, by;
+    patch_of_block(LOAD4, 8, bx, by);  // runs along the axis that moves single elements
+    const uint32_t c0 = bx * TILE, r0 = by * TILE;
     const uint32_t q4 = threadIdx.x & 15, line = threadIdx.x >> 4;           // the float4 side: 16 float4 per line, 16 lines per pass
     const uint32_t tx = threadIdx.x & (TILE - 1), ty = threadIdx.x / TILE;  // the element side: 64 x 4
     if (LOAD4) {
@@ -898,32 +935,30 @@ int launch_transpose(DeviceCtx &ctx, void *out, const void *in, int elem_size, i
         return launch_copy_strided(ctx, out, in, elem_size, (int)d.size(), d.data(), so.data(), si.data());
     }
     const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batches);
-    if (elem_size == 4 && g.r_len % 4 == 0 && g.c_len % 4 == 0 && g.r_in_str % 4 == 0 && g.c_out_str % 4 == 0 &&
-        (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && (reinterpret_cast<uintptr_t>(in) & 15u) == 0) {
-        bool batches_line_up = true;
-        for (int i = 0; i < g.brank; i++) batches_line_up = batches_line_up && g.b_in_str[i] % 4 == 0 && g.b_out_str[i] % 4 == 0;
-        if (batches_line_up) {
-            if (ctx.streaming(total * 4))
-                hipLaunchKernelGGL((transpose_tiled_vec4<true>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint32_t *>(out),
-                                   static_cast<const uint32_t *>(in), g);
-            else
-                hipLaunchKernelGGL((transpose_tiled_vec4<false>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint32_t *>(out),
-                                   static_cast<const uint32_t *>(in), g);
-            return ctx.check(hipGetLastError(), "transpose_tiled (16-byte) launch");
-        }
-    }
     switch (elem_size) {
     case 1:
         hipLaunchKernelGGL((transpose_tiled<uint8_t>), grid, dim3(BLOCK), 0, ctx.stream, static_cast<uint8_t *>(out),
                            static_cast<const uint8_t *>(in), g);
         break;
     case 4: {
-        bool in4 = g.c_len % 4 == 0 && g.r_in_str % 4 == 0 && aligned16(in), out4 = g.r_len % 4 == 0 && g.c_out_str % 4 == 0 && aligned16(out);
-        for (int i = 0; i < g.brank; i++) in4 = in4 && g.b_in_str[i] % 4 == 0, out4 = out4 && g.b_out_str[i] % 4 == 0;
+        // 16-byte loads along C where every row of a patch starts on a 16-byte boundary.  16-byte stores along R only where
+        // every row of a patch starts on a 128-byte boundary as well: a wavefront's store is four 256-byte pieces, and pieces
+        // that straddle lines run at half the rate of single elements ([8196, 8196]: 38 % of the HBM peak against 74 %);
+        // loads do not mind.
+        const bool in_lines = g.r_in_str % 32 == 0 && aligned128(in), out_lines = g.c_out_str % 32 == 0 && aligned128(out);
+        bool in4 = g.c_len % 4 == 0 && g.r_in_str % 4 == 0 && aligned16(in), out4 = g.r_len % 4 == 0 && out_lines, lines = in_lines && out_lines;
+        for (int i = 0; i < g.brank; i++) {
+            in4 = in4 && g.b_in_str[i] % 4 == 0, out4 = out4 && g.b_out_str[i] % 32 == 0;
+            lines = lines && g.b_in_str[i] % 32 == 0 && g.b_out_str[i] % 32 == 0;
+        }
         uint32_t *o = static_cast<uint32_t *>(out);
         const uint32_t *x = static_cast<const uint32_t *>(in);
         const bool nt = ctx.streaming(total * 4);
-        if (in4 && nt) hipLaunchKernelGGL((transpose_tiled_mixed<true, true>), grid, dim3(BLOCK), 0, ctx.stream, o, x, g);
+        if (in4 && out4 && nt && lines) hipLaunchKernelGGL((transpose_tiled_vec4<true, true>), grid, dim3(BLOCK), 0, ctx.stream, o, x, g);
+        else if (in4 && out4 && nt) hipLaunchKernelGGL((transpose_tiled_vec4<true, false>), grid, dim3(BLOCK), 0, ctx.stream, o, x, g);
+        else if (in4 && out4 && lines) hipLaunchKernelGGL((transpose_tiled_vec4<false, true>), grid, dim3(BLOCK), 0, ctx.stream, o, x, g);
+        else if (in4 && out4) hipLaunchKernelGGL((transpose_tiled_vec4<false, false>), grid, dim3(BLOCK), 0, ctx.stream, o, x, g);
+        else if (in4 && nt) hipLaunchKernelGGL((transpose_tiled_mixed<true, true>), grid, dim3(BLOCK), 0, ctx.stream, o, x, g);
         else if (in4) hipLaunchKernelGGL((transpose_tiled_mixed<true, false>), grid, dim3(BLOCK), 0, ctx.stream, o, x, g);
         else if (out4 && nt) hipLaunchKernelGGL((transpose_tiled_mixed<false, true>), grid, dim3(BLOCK), 0, ctx.stream, o, x, g);
         else if (out4) hipLaunchKernelGGL((transpose_tiled_mixed<false, false>), grid, dim3(BLOCK), 0, ctx.stream, o, x, g);

@@ -41,6 +41,10 @@ TRANSPOSES = [
     ((3, 100, 128), (0, 2, 1)), ((2, 255, 192), (0, 2, 1)), ((2, 257, 192), (0, 2, 1)), ((2, 511, 64), (0, 2, 1)),
     # 4-byte elements in 64 x 64 patches with 16-byte accesses wherever the rows start: odd extents on either side
     ((5000, 70), (1, 0)), ((70, 5000), (1, 0)), ((2001, 129), (1, 0)), ((3, 1029, 67), (0, 2, 1)), ((4099, 68), (1, 0)), ((3, 130, 5, 66), (0, 3, 2, 1)),
+    # which side of a patch moves 16 bytes at a time: reads where rows start on 16-byte boundaries, writes only where they
+    # start on 128-byte boundaries; more patches than the eight XCDs take in one turn, with and without a batch axis
+    ((4096, 68), (1, 0)), ((3, 4096, 68), (0, 2, 1)), ((2052, 132), (1, 0)), ((2, 2052, 132), (0, 2, 1)), ((2052, 131), (1, 0)),
+    ((2048, 131), (1, 0)), ((2, 1024, 67), (0, 2, 1)), ((1100, 1028), (1, 0)), ((1031, 1033), (1, 0)), ((9, 577, 129), (0, 2, 1)),
 ]
 
 
