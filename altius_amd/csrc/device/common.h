@@ -10,6 +10,17 @@ namespace dev {
 
 constexpr int WAVE = 64;
 
+// Neighbouring pieces of work under one L2.  Blocks i, i + 8, i + 16, ... of a launch run on one of the part's eight
+// XCDs, each with an L2 of its own, so blocks that take pieces i and i + 1 of a tensor never share one: a cache line
+// that two neighbouring pieces both touch (rows, slabs or patches that do not end on a 128-byte boundary) is fetched
+// twice and goes out to memory as two partial lines.  This maps block `id` of `n` to a piece such that each XCD takes
+// a run of consecutive pieces, in the order of its blocks: the parts of such a line then meet in one L2 while it is
+// still there.  A bijection of 0 .. n - 1; where blocks really land is a matter of speed only.
+__device__ __forceinline__ uint32_t piece_of_block(uint32_t id, uint32_t n) {
+    const uint32_t xcd = id & 7u, each = n >> 3, more = n & 7u;
+    return xcd * each + (xcd < more ? xcd : more) + (id >> 3);
+}
+
 __device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
 __device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
 

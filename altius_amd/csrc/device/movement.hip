@@ -115,18 +115,14 @@ struct TransGeom {
 
 // Which patch a block takes where pieces of a patch start and end inside cache lines (single elements at odd
 // addresses; 16-byte accesses along rows whose pitch is not a whole number of 128-byte lines).  The patch next door
-// completes such a line.  Blocks i, i + 8, i + 16, ... of a launch run on one XCD, under one L2: each of the eight takes
-// a run of consecutive patches (in the order of its blocks), so that the parts of a line meet in one L2 while it is
-// still there, instead of being fetched twice and going out to memory as two partial lines from two XCDs
-// ([50257, 768] -> [768, 50257]: 11 % more bytes written than the result holds and 65 % of the HBM peak with patches
-// dealt out row by row, 72 % this way; the other way round 69 -> 84 %).  A run goes along one axis in a band of `band`
-// patches across: neighbours along the run's axis are `band` blocks apart, neighbours across it follow each other.
-// Where blocks land is a matter of speed only: any order of the patches gives the same result.
+// completes such a line, so each XCD takes a run of neighbouring patches (dev::piece_of_block): [50257, 768] ->
+// [768, 50257] wrote 11 % more bytes than the result holds and ran at 65 % of the HBM peak with patches dealt out row by
+// row, 74 % this way; the other way round 69 -> 85 %.  A run goes along one axis in a band of `band` patches across:
+// neighbours along the run's axis are `band` blocks apart, neighbours across it follow each other.
 // along_r: runs go along R (whose pieces are written), else along C (whose pieces are read).
 __device__ __forceinline__ void patch_of_block(bool along_r, uint32_t band, uint32_t &bx, uint32_t &by) {
-    const uint32_t nx = gridDim.x, ny = gridDim.y, patches = nx * ny;
-    const uint32_t id = blockIdx.y * nx + blockIdx.x, xcd = id & 7u, each = patches >> 3, more = patches & 7u;
-    const uint32_t turn = xcd * each + (xcd < more ? xcd : more) + (id >> 3);  // a bijection of 0 .. patches - 1
+    const uint32_t nx = gridDim.x, ny = gridDim.y;
+    const uint32_t turn = dev::piece_of_block(blockIdx.y * nx + blockIdx.x, nx * ny);
     const uint32_t n_run = along_r ? ny : nx, n_across = along_r ? nx : ny;
     const uint32_t whole = n_across / band * band, in_whole = whole * n_run;  // patches in bands of full width
     uint32_t run, across;

@@ -302,7 +302,8 @@ def run_row_sweep(ctx, D, args, lengths):
 SHAPE_SWEEP_ELEMS = 96 << 20
 SHAPE_SWEEP_MIDDLE = ((197, 768), (49, 1024), (12, 4096), (1024, 8), (2, 65536), (196, 3), (7, 7))   # (reduced, inner) extents
 SHAPE_SWEEP_ODD_ROWS = (1025, 2049, 5001, 9999, 50257)
-SHAPE_SWEEP_TRANSPOSES = (([64, 256, 56, 56], [0, 2, 3, 1]), ([8192, 8192], [1, 0]), ([256, 197, 768], [0, 2, 1]), ([50257, 768], [1, 0]))
+SHAPE_SWEEP_TRANSPOSES = (([64, 256, 56, 56], [0, 2, 3, 1]), ([8192, 8192], [1, 0]), ([8196, 8196], [1, 0]), ([256, 197, 768], [0, 2, 1]), ([50257, 768], [1, 0]),
+                          ([768, 50257], [1, 0]))
 
 
 def build_shape_sweep(ctx, D, elems=SHAPE_SWEEP_ELEMS):
