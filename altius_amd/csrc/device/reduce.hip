@@ -30,6 +30,7 @@
 // accumulators.
 
 #include <algorithm>
+#include <numeric>
 #include <mutex>
 
 #include "common.h"
@@ -351,7 +352,7 @@ constexpr size_t SS_MAX_SLAB = 2048, SS_GROUP_FLOATS = 8192;
 
 template <class OP, bool SCALE, bool NT>
 __global__ __launch_bounds__(SS_BLOCK) void reduce_small_slabs(float *__restrict__ dst, const float *__restrict__ in, size_t outer,
-                                                               uint32_t red, uint32_t inner, uint32_t group, float scale) {
+                                                               uint32_t red, uint32_t inner, uint32_t group, uint32_t parts, float scale) {
     extern __shared__ __align__(16) float ss_lds[];
     const uint32_t slab = red * inner;
     const size_t o0 = (size_t)blockIdx.x * group;
@@ -370,6 +371,34 @@ __global__ __launch_bounds__(SS_BLOCK) void reduce_small_slabs(float *__restrict
     for (uint32_t i = (n4 << 2) + threadIdx.x; i < floats; i += SS_BLOCK) ss_lds[i] = src[i];  // the tensor's ragged end
     __syncthreads();
     const uint32_t outs = n_slabs * inner;
+    if (parts > 1) {
+        // Few outputs per block (a group of [196, 3] slabs has 36): `parts` threads share an output's column, thread p of
+        // them taking rows p, p + parts, ..., so that most of the block walks LDS instead of a seventh of it 196 rows each.
+        // The partial results go through LDS (the slabs are done with by then) and are combined in a fixed order.
+        const uint32_t j = threadIdx.x / parts, p = threadIdx.x - j * parts;  // outs * parts <= SS_BLOCK
+        float acc = OP::identity();
+        if (j < outs) {
+            const uint32_t ol = j / inner, c = j - ol * inner;
+            const float *q = ss_lds + ol * slab + c;
+            float a0 = OP::identity(), a1 = a0;
+            uint32_t r = p;
+            for (; r + parts < red; r += 2 * parts) {
+                a0 = OP::apply(a0, q[r * inner]);
+                a1 = OP::apply(a1, q[(r + parts) * inner]);
+            }
+            if (r < red) a0 = OP::apply(a0, q[r * inner]);
+            acc = OP::apply(a0, a1);
+        }
+        __syncthreads();
+        if (j < outs) ss_lds[threadIdx.x] = acc;  // parts <= red: the partial results fit where the group's slabs were
+        __syncthreads();
+        if (threadIdx.x < outs) {
+            float a = ss_lds[threadIdx.x * parts];
+            for (uint32_t k = 1; k < parts; k++) a = OP::apply(a, ss_lds[threadIdx.x * parts + k]);
+            dst[o0 * inner + threadIdx.x] = SCALE ? a * scale : a;
+        }
+        return;
+    }
     for (uint32_t j = threadIdx.x; j < outs; j += SS_BLOCK) {
         const uint32_t ol = j / inner, c = j - ol * inner;
         const float *p = ss_lds + ol * slab + c;
@@ -700,15 +729,25 @@ int reduce_impl(DeviceCtx &ctx, const Partials &pt, float *out, const float *in,
     // Small slabs whose rows are not whole float4s, or too few and too narrow to keep half of reduce_cols_vec4's lanes busy.
     if (red * inner <= SS_MAX_SLAB && aligned16(in) && (inner % 4 != 0 || red * std::min<size_t>(inner / 4, WAVE) < CV_BLOCK / 2)) {
         const size_t slab = red * inner;
-        size_t group = SS_GROUP_FLOATS / slab / 4 * 4;  // SS_MAX_SLAB * 4 <= SS_GROUP_FLOATS: at least 4
-        while (group > 4 && (outer + group - 1) / group < 2048) group -= 4;  // rather more blocks than fuller ones
+        // Slabs per group: a multiple of 4 (16-byte loads), and of as many slabs as have whole 128-byte lines of results where
+        // a group holds that many (32 slabs of 7 x 7: 68 -> 72 % of the HBM peak), so that no line of the output is written
+        // in part by two blocks.  (Lines of the input shared by two groups cost nothing measurable: [196, 3] slabs run
+        // a point better in groups of 12 than in groups of 8, which end on line boundaries.)
+        const size_t limit = SS_GROUP_FLOATS / slab;  // SS_MAX_SLAB * 4 <= SS_GROUP_FLOATS: at least 4
+        const size_t whole_lines = 32 / std::gcd<size_t>(inner, 32);
+        const size_t step = whole_lines >= 4 && whole_lines <= limit ? whole_lines : 4;
+        size_t group = limit / step * step;
+        while (group > step && (outer + group - 1) / group < 2048) group -= step;  // rather more blocks than fuller ones
         const size_t blocks = (outer + group - 1) / group;
         if (blocks <= MAX_GRID_X) {
             const bool nt = ctx.streaming(outer * slab * sizeof(float));
             const dim3 grid((unsigned)blocks), block(SS_BLOCK);
             const size_t shmem = group * slab * sizeof(float);
-            if (nt) hipLaunchKernelGGL((reduce_small_slabs<OP, SCALE, true>), grid, block, shmem, s, out, in, outer, (uint32_t)red, (uint32_t)inner, (uint32_t)group, scale);
-            else hipLaunchKernelGGL((reduce_small_slabs<OP, SCALE, false>), grid, block, shmem, s, out, in, outer, (uint32_t)red, (uint32_t)inner, (uint32_t)group, scale);
+            // threads per output where a group has few of them: as many as the block has, at most 8, rows for each
+            const size_t per_output = std::min<size_t>({(size_t)SS_BLOCK / (group * inner), (size_t)8, red / 4});
+            const uint32_t parts = per_output >= 2 ? (uint32_t)per_output : 1u;
+            if (nt) hipLaunchKernelGGL((reduce_small_slabs<OP, SCALE, true>), grid, block, shmem, s, out, in, outer, (uint32_t)red, (uint32_t)inner, (uint32_t)group, parts, scale);
+            else hipLaunchKernelGGL((reduce_small_slabs<OP, SCALE, false>), grid, block, shmem, s, out, in, outer, (uint32_t)red, (uint32_t)inner, (uint32_t)group, parts, scale);
             return ctx.check(hipGetLastError(), "reduce (small slabs) launch");
         }
     }

@@ -487,6 +487,10 @@ REDUCE_CASES = [
     ([4099, 3, 4], [1], False),        # whole float4s, but too few rows for the float4-column kernel
     ([10001, 2, 3], [1], False),       # groups of 1364 slabs, a ragged last group
     ([3, 100, 20], [1], False),        # slabs of 2000 values: groups of four, the last one of three
+    ([50, 64, 5], [1], False),         # few outputs per group: eight threads share a column, then three, then two
+    ([7, 131, 20], [1], True),
+    ([9, 9, 6], [1], False),
+    ([3000, 196, 3], [1], False),      # groups of twelve slabs, seven threads per output
     ([7, 1030], [1], False),           # rows that start anywhere: single elements to the first 16-byte boundary, then float4s
     ([5, 2049], [1], True),
     ([3, 5001], [1], False),           # the same in the block kernel
