@@ -270,7 +270,8 @@ def _many_small(ctx, a, b, trans_b=False, pad=(0, 0), offset=(0, 0), shared_b=Fa
 # k <= 64 and n <= 208 or n <= 64), at their limits, and their neighbours that do not
 MANY_SMALL = [(144, 197, 197, 64), (144, 197, 64, 197), (128, 208, 208, 64), (300, 197, 197, 64), (300, 197, 64, 197), (128, 1, 1, 1),
               (129, 33, 7, 3), (130, 193, 190, 33), (128, 100, 17, 64), (128, 208, 64, 300), (128, 30, 64, 65), (130, 16, 16, 1000),
-              (128, 192, 48, 128), (128, 209, 64, 64), (128, 197, 209, 64), (127, 197, 197, 64), (128, 64, 65, 65)]
+              (128, 192, 48, 128), (128, 209, 64, 64), (128, 197, 209, 64), (127, 197, 197, 64), (128, 64, 65, 65),
+              (128, 50, 20, 97), (128, 197, 64, 130), (128, 17, 33, 81), (128, 40, 64, 113)]  # k cut into chunks of 64+48, 48+48+48, 48+48, 64+64
 
 
 @pytest.mark.parametrize("batch,m,n,k", MANY_SMALL)
